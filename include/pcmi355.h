@@ -1,0 +1,200 @@
+/*
+ * pcmi355 -- C ABI of the MI355X probabilistic-circuit engine.
+ *
+ * Every entry point returns 0 on success and a negative pcm_status on failure;
+ * pcm_last_error() then holds a message for the calling thread.  No exception crosses
+ * this boundary.  Pointers named d_* are DEVICE pointers (hipMalloc'd or owned by any
+ * framework on the current device); all other pointers are host memory owned by the
+ * caller and only touched during the call.  Calls on one circuit are serialised by the
+ * caller; distinct circuits are independent.  Work is queued on the circuit's stream
+ * (default: the null stream) and entry points that return host data synchronise it.
+ *
+ * Citations name the reference interface each entry replaces; paths are relative to
+ * VariationalJuice.jl/ in the reference tree.
+ */
+#ifndef PCMI355_H
+#define PCMI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct pcm_circuit pcm_circuit;
+
+enum pcm_status {
+  PCM_OK = 0,
+  PCM_ERR_ARG = -1,       /* null pointer, bad size, bad handle */
+  PCM_ERR_SHAPE = -2,     /* tree / circuit description is malformed */
+  PCM_ERR_UNSUPPORTED = -3,
+  PCM_ERR_HIP = -4,       /* a HIP call failed; message names it */
+  PCM_ERR_STATE = -5      /* call order violated (e.g. update before flows) */
+};
+
+/* Message of the last failure on this thread (never NULL). */
+const char* pcm_last_error(void);
+int pcm_version(void);
+
+/* ---- compilation -------------------------------------------------------------- */
+
+/*
+ * Build the hidden Chow-Liu tree circuit of src/structures/hclts.jl:100-145
+ * (`hclt_from_clt` with one observed variable per tree node and Categorical leaves) and
+ * flatten it as ProbabilisticCircuits.jl `BitsProbCircuit` + src/bits_circuit.jl:39-113
+ * (`CuMetaBitsProbCircuit`) do, into the dense per-tree-node block form the kernels use.
+ * clt_parent[v] is the tree parent of variable v (-1 for the single root).
+ * Parameters start uniform; set them with pcm_hclt_set_params or pcm_update_parameters.
+ */
+int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats,
+                    int32_t num_cats, pcm_circuit** out);
+
+/*
+ * Compile a general circuit given as a DAG in topological order (children before
+ * parents, root last), the flat form a binding obtains by walking a `ProbCircuit`:
+ * replaces `CuMetaBitsProbCircuit(pc)` (src/bits_circuit.jl:39) and, with num_heads > 0,
+ * `CuMultiHeadBitsProbCircuit(pcs)` (src-jl/multi_head_pc/bit_circuit.jl:14-56; the last
+ * num_heads nodes are the heads and no fake root is needed).
+ * node_type: 0 input, 1 sum, 2 product.  child_ptr[n..n+1] delimits node n's children in
+ * child_idx; sum_logp is parallel to child_idx (ignored under products).  Input node n
+ * reads variable input_var[n] and owns num_cats log-probabilities, given in creation order
+ * in input_logp.
+ */
+int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
+                       const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
+                       const float* input_logp, int32_t num_vars, int32_t num_cats,
+                       int32_t num_heads, pcm_circuit** out);
+
+/* Releases the circuit and all device memory it owns. */
+int pcm_free(pcm_circuit* c);
+
+/* Queue this circuit's work on the given hipStream_t (NULL = null stream). */
+int pcm_set_stream(pcm_circuit* c, void* hip_stream);
+
+/* ---- sizes and index tables --------------------------------------------------- */
+
+/* `num_parameters(mbpc)`, `num_nodes`, `num_edges`, `num_input_params`
+ * (src/bits_circuit.jl:119-131).  what: 0 parameters, 1 sum parameters, 2 nodes,
+ * 3 edges, 4 input parameters, 5 variables, 6 categories, 7 hidden categories (0 if not an
+ * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes. */
+int64_t pcm_size(const pcm_circuit* c, int32_t what);
+
+/* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.
+ * which: 0 edge2param [edges], 1 param2edge [sum parameters], 2 param2group [sum
+ * parameters], 3 pargroup_sizes [groups], 4 innode2ncumparam [input nodes],
+ * 5 up-layer ends [layers], 6 edge parent ids, 7 edge prime ids, 8 edge sub ids (0: none)
+ * [edges, up order].  n must equal the table length. */
+int pcm_index_table(const pcm_circuit* c, int32_t which, int64_t* out, int64_t n);
+
+/* ---- parameters --------------------------------------------------------------- */
+
+/* `vectorize_parameters(mbpc, params)` (src/misc.jl:5-40): sum-edge log-parameters in
+ * up-edge order, then every input node's log-probabilities in creation order. */
+int pcm_vectorize_parameters(pcm_circuit* c, float* out, int64_t n);
+/* `update_parameters(mbpc, params)` (src/misc.jl:73-102). */
+int pcm_update_parameters(pcm_circuit* c, const float* params, int64_t n);
+
+/* HCLT block form.  theta is [num_vars][K][K] log-parameters (row k: sum node k of the
+ * tree node, column j: hidden state j; rows of leaf tree nodes are ignored and only row 0
+ * of the root is used, hclts.jl:137); leaf is [num_vars][K][num_cats] log-probabilities of
+ * `joined_leaves[v, j]` (hclts.jl:147-156).  Either pointer may be NULL to skip it. */
+int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf);
+int pcm_hclt_get_params(pcm_circuit* c, float* theta, float* leaf);
+/* Sufficient statistics of the last pcm_flows / pcm_em_step in the same block form:
+ * edge_aggr [num_vars][K][K] (the reference's `edge_aggr`, src/queries/flow.jl:73-81) and
+ * leaf_flow [num_vars][K][num_cats] (the heap's flow slots,
+ * src/nodes/fixable_categorical_dist.jl:121-130). */
+int pcm_hclt_get_flows(pcm_circuit* c, float* edge_aggr, float* leaf_flow);
+
+/* ---- queries ------------------------------------------------------------------ */
+
+/*
+ * Forward pass: `loglikelihoods(bpc, data; batch_size)` / `loglikelihoods_probcat`
+ * (src/regularization/reg_likelihood.jl:139-162) for one batch.  d_data holds uint8
+ * categories; element (example e, variable v) is d_data[e*stride_ex + v*stride_var].
+ * d_example_ids (may be NULL = 0..batch-1) selects the batch rows, 0-based, like the
+ * reference's `example_ids`.  d_ll_out receives `batch` floats (mars[:, end]).
+ * For a multi-head circuit d_ll_out receives [num_heads][batch]
+ * (src-jl/multi_head_pc/likelihood.jl:3-18 with head_mask = nothing).
+ */
+int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex,
+                       int64_t stride_var, const int32_t* d_example_ids, int32_t batch,
+                       float* d_ll_out);
+
+/*
+ * Forward + backward + leaf flows: `probs_flows_circuit_with_reg` with soft_reg = 0
+ * (src/regularization/reg_flow.jl:276-282) == `probs_flows_circuit`
+ * (src/queries/flow.jl:228-234).  The circuit's edge_aggr and leaf flow accumulators are
+ * first scaled by `rate` (0 clears them; src/regularization/reg_em.jl:276-284) and then
+ * receive this batch.  d_head_mask (multi-head circuits only, else NULL) is
+ * [num_heads][batch] and seeds the head flows (src-jl/multi_head_pc/flow.jl:141-176).
+ */
+int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
+              const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask,
+              float* d_ll_out);
+
+/*
+ * Parameter update from the accumulated flows, the four calls of
+ * src/regularization/reg_em.jl:292-299: add_pseudocount, aggr_node_flows,
+ * update_params(inertia), update_input_node_params(pseudocount, inertia).
+ */
+int pcm_em_update(pcm_circuit* c, float pseudocount, float inertia);
+
+/* pcm_flows followed by pcm_em_update: one iteration of the batch loop of
+ * `mini_batch_em_with_reg` (src/regularization/reg_em.jl:272-300). */
+int pcm_em_step(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
+                const int32_t* d_example_ids, int32_t batch, float rate, float pseudocount,
+                float inertia, float* d_ll_out);
+
+/* General circuits: host copies of per-batch node values / flows of the last pcm_flows,
+ * [num_nodes][batch] (the reference's `mars` / `flows`, transposed), and of the
+ * accumulators: edge_aggr [edges, up order], leaf_flow [input parameters]. */
+int pcm_get_node_values(pcm_circuit* c, float* mars, float* flows, int64_t n);
+int pcm_get_aggregates(pcm_circuit* c, float* edge_aggr, int64_t n_edges, float* leaf_flow,
+                       int64_t n_leaf);
+
+/*
+ * KL(p || q) of two parameterisations of one structure: `kld(mbpc, params1, params2)`
+ * with norm_params = false (src/queries/kld.jl:177-206).  p and q must have been compiled
+ * from the same description.  *out receives klds[:, end].
+ */
+int pcm_kld(pcm_circuit* p, pcm_circuit* q, float* out);
+/* `kld_backward(mbpc, params1, params2; grad_wrt_logparams = true)`
+ * (src/queries/kld.jl:593-649): gradients in parameter-vector order. */
+int pcm_kld_backward(pcm_circuit* p, pcm_circuit* q, float* grad_p, float* grad_q, int64_t n);
+
+/*
+ * Gumbel-max ancestral sampling from supplied noise: the temperature -> 0 limit of
+ * `gumbel_sample` (src/queries/sample.jl:338-383), which itself draws its noise in-kernel
+ * (:45) and has no counterpart taking a noise tensor.  d_node_noise is
+ * [batch][pcm_sample_noise_size()] (HCLT: [batch][inner tree nodes in bottom-up
+ * order][K], indexed by the hidden state chosen; general: one float per sum parameter),
+ * d_leaf_noise is [batch][num_vars][num_cats], d_out [batch][num_vars] uint8.
+ */
+int64_t pcm_sample_noise_size(const pcm_circuit* c);
+int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_noise,
+               int32_t batch, uint8_t* d_out);
+
+/*
+ * Adam ascent step on the sum parameters followed by per-sum-node normalisation
+ * (src/sgd/adam.jl:63-86, :88-127, :318-319).  d_grad, d_params (unnormalised
+ * log-parameters), d_m, d_v are device vectors in parameter-vector order over the sum
+ * parameters; the circuit's log-parameters become params - log(sum exp(params)) per node.
+ */
+int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d_m, float* d_v,
+                  float lr, float beta1, float beta2, float eps, int32_t t);
+
+/* ---- instrumentation ----------------------------------------------------------- */
+
+/* Per-kernel timing, the role of `debug = true` -> `CUDA.@time` around each launch
+ * (src/queries/likelihood.jl:86-92, src/queries/flow.jl:127-133).  When on, pcm_flows
+ * brackets its forward / backward / statistics launches with events on the circuit's
+ * stream and synchronises; pcm_get_timing returns the last milliseconds of each
+ * (n <= 4 values: forward, backward, statistics, reserved). */
+int pcm_set_timing(pcm_circuit* c, int32_t on);
+int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,178 @@
+// C ABI of pcmi355: argument checks, exception -> status translation.
+#include <new>
+
+#include "common.hpp"
+#include "hclt_engine.hpp"
+
+namespace {
+thread_local std::string g_last_error;
+
+template <typename F>
+int guarded(F&& f) {
+  try {
+    f();
+    return PCM_OK;
+  } catch (const pcm::Error& e) {
+    g_last_error = e.what();
+    return e.status;
+  } catch (const std::bad_alloc&) {
+    g_last_error = "out of host memory";
+    return PCM_ERR_ARG;
+  } catch (const std::exception& e) {
+    g_last_error = e.what();
+    return PCM_ERR_ARG;
+  }
+}
+
+pcm_circuit* need(pcm_circuit* c) {
+  if (!c) pcm::fail(PCM_ERR_ARG, "circuit handle is null");
+  return c;
+}
+
+pcm::HcltCircuit* need_hclt(pcm_circuit* c) {
+  auto* h = dynamic_cast<pcm::HcltCircuit*>(need(c));
+  if (!h) pcm::fail(PCM_ERR_ARG, "circuit was not created by pcm_hclt_create");
+  return h;
+}
+
+pcm::BatchRef batch_ref(const uint8_t* d, int64_t se, int64_t sv, const int32_t* idx, int32_t b) {
+  return pcm::BatchRef{d, se, sv, idx, b};
+}
+}  // namespace
+
+extern "C" {
+
+const char* pcm_last_error(void) { return g_last_error.c_str(); }
+int pcm_version(void) { return 1; }
+
+int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
+                    pcm_circuit** out) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    *out = nullptr;
+    *out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats);
+  });
+}
+
+int pcm_circuit_create(int32_t, const uint8_t*, const int32_t*, const int32_t*, const float*, const int32_t*,
+                       const float*, int32_t, int32_t, int32_t, pcm_circuit** out) {
+  return guarded([&] {
+    if (out) *out = nullptr;
+    pcm::fail(PCM_ERR_UNSUPPORTED, "pcm_circuit_create: general circuits are not built yet");
+  });
+}
+
+int pcm_free(pcm_circuit* c) {
+  return guarded([&] { delete need(c); });
+}
+
+int pcm_set_stream(pcm_circuit* c, void* s) {
+  return guarded([&] { need(c)->stream = reinterpret_cast<hipStream_t>(s); });
+}
+
+int64_t pcm_size(const pcm_circuit* c, int32_t what) {
+  int64_t r = -1;
+  guarded([&] { r = need(const_cast<pcm_circuit*>(c))->size(what); });
+  return r;
+}
+
+int pcm_index_table(const pcm_circuit* c, int32_t which, int64_t* out, int64_t n) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    need(const_cast<pcm_circuit*>(c))->index_table(which, out, n);
+  });
+}
+
+int pcm_vectorize_parameters(pcm_circuit* c, float* out, int64_t n) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    need(c)->vectorize(out, n);
+  });
+}
+
+int pcm_update_parameters(pcm_circuit* c, const float* p, int64_t n) {
+  return guarded([&] {
+    if (!p) pcm::fail(PCM_ERR_ARG, "params is null");
+    need(c)->update_parameters(p, n);
+  });
+}
+
+int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf) {
+  return guarded([&] { need_hclt(c)->set_block_params(theta, leaf); });
+}
+int pcm_hclt_get_params(pcm_circuit* c, float* theta, float* leaf) {
+  return guarded([&] { need_hclt(c)->get_block_params(theta, leaf); });
+}
+int pcm_hclt_get_flows(pcm_circuit* c, float* edge_aggr, float* leaf_flow) {
+  return guarded([&] { need_hclt(c)->get_block_flows(edge_aggr, leaf_flow); });
+}
+
+int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t se, int64_t sv, const int32_t* idx,
+                       int32_t batch, float* d_ll) {
+  return guarded([&] { need(c)->loglikelihoods(batch_ref(d_data, se, sv, idx, batch), d_ll); });
+}
+
+int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t se, int64_t sv, const int32_t* idx, int32_t batch,
+              float rate, const float* d_head_mask, float* d_ll) {
+  return guarded([&] { need(c)->flows(batch_ref(d_data, se, sv, idx, batch), rate, d_head_mask, d_ll); });
+}
+
+int pcm_em_update(pcm_circuit* c, float pseudocount, float inertia) {
+  return guarded([&] { need(c)->em_update(pseudocount, inertia); });
+}
+
+int pcm_em_step(pcm_circuit* c, const uint8_t* d_data, int64_t se, int64_t sv, const int32_t* idx, int32_t batch,
+                float rate, float pseudocount, float inertia, float* d_ll) {
+  return guarded([&] {
+    need(c)->flows(batch_ref(d_data, se, sv, idx, batch), rate, nullptr, d_ll);
+    c->em_update(pseudocount, inertia);
+  });
+}
+
+int pcm_get_node_values(pcm_circuit* c, float*, float*, int64_t) {
+  return guarded([&] { need(c); pcm::fail(PCM_ERR_UNSUPPORTED, "node values are kept only by general circuits"); });
+}
+int pcm_get_aggregates(pcm_circuit* c, float*, int64_t, float*, int64_t) {
+  return guarded([&] { need(c); pcm::fail(PCM_ERR_UNSUPPORTED, "use pcm_hclt_get_flows on an HCLT circuit"); });
+}
+
+int pcm_kld(pcm_circuit* p, pcm_circuit* q, float* out) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    need(q);
+    need(p)->kld(q, out);
+  });
+}
+int pcm_kld_backward(pcm_circuit* p, pcm_circuit* q, float* gp, float* gq, int64_t n) {
+  return guarded([&] {
+    need(q);
+    need(p)->kld_backward(q, gp, gq, n);
+  });
+}
+
+int64_t pcm_sample_noise_size(const pcm_circuit* c) {
+  int64_t r = -1;
+  guarded([&] { r = need(const_cast<pcm_circuit*>(c))->sample_noise_size(); });
+  return r;
+}
+int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
+  return guarded([&] { need(c)->sample(d_node_noise, d_leaf_noise, batch, d_out); });
+}
+
+int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
+                  float b1, float b2, float eps, int32_t t) {
+  return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });
+}
+
+int pcm_set_timing(pcm_circuit* c, int32_t on) {
+  return guarded([&] { need_hclt(c)->timing = on != 0; });
+}
+int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n) {
+  return guarded([&] {
+    if (!ms || n < 0 || n > 4) pcm::fail(PCM_ERR_ARG, "ms is null or n outside 0..4");
+    auto* h = need_hclt(c);
+    for (int i = 0; i < n; ++i) ms[i] = h->last_ms[i];
+  });
+}
+
+}  // extern "C"

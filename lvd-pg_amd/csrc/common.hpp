@@ -1,0 +1,105 @@
+// Shared host-side plumbing of the pcmi355 library: error reporting, device buffers,
+// and the abstract engine every compiled circuit implements.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/pcmi355.h"
+
+namespace pcm {
+
+// Error carried from anywhere below the C ABI to the entry point that reports it.
+struct Error : std::runtime_error {
+  int status;
+  Error(int s, const std::string& m) : std::runtime_error(m), status(s) {}
+};
+
+[[noreturn]] inline void fail(int status, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  throw Error(status, buf);
+}
+
+#define PCM_HIP(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t e__ = (expr);                                                            \
+    if (e__ != hipSuccess)                                                              \
+      ::pcm::fail(PCM_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(e__),  \
+                  __FILE__, __LINE__);                                                  \
+  } while (0)
+
+// Owning device array.
+template <typename T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  DevBuf() = default;
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+  ~DevBuf() { release(); }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+  void alloc(size_t count) {
+    release();
+    if (count) PCM_HIP(hipMalloc((void**)&p, count * sizeof(T)));
+    n = count;
+  }
+  void ensure(size_t count) {
+    if (count > n) alloc(count);
+  }
+  void upload(const std::vector<T>& h, hipStream_t s = nullptr) {
+    alloc(h.size());
+    if (!h.empty()) {
+      PCM_HIP(hipMemcpyAsync(p, h.data(), h.size() * sizeof(T), hipMemcpyHostToDevice, s));
+      PCM_HIP(hipStreamSynchronize(s));
+    }
+  }
+  void zero(hipStream_t s = nullptr) {
+    if (n) PCM_HIP(hipMemsetAsync(p, 0, n * sizeof(T), s));
+  }
+};
+
+inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
+
+struct BatchRef {
+  const uint8_t* d_data;
+  int64_t stride_ex, stride_var;
+  const int32_t* d_idx;
+  int32_t batch;
+};
+
+}  // namespace pcm
+
+// The opaque handle of the C ABI.
+struct pcm_circuit {
+  hipStream_t stream = nullptr;
+  virtual ~pcm_circuit() {}
+  virtual int64_t size(int what) const = 0;
+  virtual void index_table(int which, int64_t* out, int64_t n) const = 0;
+  virtual void vectorize(float* out, int64_t n) = 0;
+  virtual void update_parameters(const float* in, int64_t n) = 0;
+  virtual void loglikelihoods(const pcm::BatchRef& b, float* d_ll) = 0;
+  virtual void flows(const pcm::BatchRef& b, float rate, const float* d_head_mask, float* d_ll) = 0;
+  virtual void em_update(float pseudocount, float inertia) = 0;
+  virtual void kld(pcm_circuit* q, float* out) = 0;
+  virtual void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) = 0;
+  virtual int64_t sample_noise_size() const = 0;
+  virtual void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
+                      uint8_t* d_out) = 0;
+  virtual void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
+                         float b1, float b2, float eps, int t) = 0;
+};

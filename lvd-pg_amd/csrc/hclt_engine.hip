@@ -1,0 +1,537 @@
+// Host side of the dense-block HCLT engine: structure, schedules, parameter order,
+// launches.
+#include "hclt_engine.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <functional>
+#include <numeric>
+
+#include "hclt_kernels.hip.hpp"
+
+namespace pcm {
+
+#define PCM_DISPATCH_K(K_, ...)                         \
+  switch (K_) {                                         \
+    case 16: { constexpr int KK = 16; __VA_ARGS__; break; } \
+    case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
+    case 64: { constexpr int KK = 64; __VA_ARGS__; break; } \
+    default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
+  }
+
+static void check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C) : V_(V), K_(K), C_(C) {
+  if (!parent) fail(PCM_ERR_ARG, "clt_parent is null");
+  if (V < 2) fail(PCM_ERR_SHAPE, "an HCLT needs at least 2 variables, got %d", V);
+  if (K != 16 && K != 32 && K != 64)
+    fail(PCM_ERR_UNSUPPORTED, "num_hidden_cats must be 16, 32 or 64 for the block engine, got %d", K);
+  if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
+  parent_.assign(parent, parent + V);
+  build_structure();
+  build_param_order();
+
+  // uniform parameters
+  std::vector<float> theta((size_t)V_ * K_ * K_, -std::log((float)K_));
+  std::vector<float> leaf((size_t)V_ * K_ * C_, -std::log((float)C_));
+  d_leaf_.alloc((size_t)V_ * C_ * K_);
+  d_logtheta_.alloc((size_t)n_inner_ * K_ * K_);
+  d_Wf_.alloc((size_t)n_inner_ * K_ * K_);
+  d_Wb_.alloc((size_t)n_inner_ * K_ * K_);
+  d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_);
+  d_leaf_flow_.alloc((size_t)V_ * C_ * K_);
+  d_edge_aggr_.zero();
+  d_leaf_flow_.zero();
+  set_block_params(theta.data(), leaf.data());
+}
+
+void HcltCircuit::build_structure() {
+  children_.assign(V_, {});
+  root_ = -1;
+  for (int v = 0; v < V_; ++v) {
+    int p = parent_[v];
+    if (p < 0) {
+      if (root_ >= 0) fail(PCM_ERR_SHAPE, "clt_parent has more than one root (%d and %d)", root_, v);
+      root_ = v;
+    } else {
+      if (p >= V_ || p == v) fail(PCM_ERR_SHAPE, "clt_parent[%d] = %d is out of range", v, p);
+      children_[p].push_back(v);
+    }
+  }
+  if (root_ < 0) fail(PCM_ERR_SHAPE, "clt_parent has no root (-1 entry)");
+  // bottom-up order by iterative post-order; detects cycles / unreachable nodes
+  std::vector<int32_t> order;
+  order.reserve(V_);
+  std::vector<std::pair<int32_t, int32_t>> st;
+  st.push_back({root_, 0});
+  depth_.assign(V_, -1);
+  depth_[root_] = 0;
+  while (!st.empty()) {
+    auto& top = st.back();
+    int v = top.first;
+    if (top.second < (int)children_[v].size()) {
+      int c = children_[v][top.second++];
+      depth_[c] = depth_[v] + 1;
+      st.push_back({c, 0});
+    } else {
+      order.push_back(v);
+      st.pop_back();
+    }
+  }
+  if ((int)order.size() != V_) fail(PCM_ERR_SHAPE, "clt_parent is not a tree: %d of %d variables reach the root",
+                                    (int)order.size(), V_);
+  inner_of_var_.assign(V_, -1);
+  var_of_inner_.clear();
+  height_.assign(V_, 0);
+  for (int v : order) {
+    if (children_[v].empty()) continue;
+    inner_of_var_[v] = (int)var_of_inner_.size();
+    var_of_inner_.push_back(v);
+    int h = 0;
+    for (int c : children_[v]) h = std::max(h, height_[c]);
+    height_[v] = h + 1;
+  }
+  n_inner_ = (int)var_of_inner_.size();
+
+  std::vector<HcltNode> nodes(n_inner_);
+  std::vector<int32_t> ci, cl;
+  for (int n = 0; n < n_inner_; ++n) {
+    int v = var_of_inner_[n];
+    HcltNode& nd = nodes[n];
+    nd.var = v;
+    nd.parent = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+    nd.is_root = v == root_;
+    nd.ic_off = (int)ci.size();
+    nd.lc_off = (int)cl.size();
+    for (int c : children_[v]) {
+      if (children_[c].empty()) cl.push_back(c); else ci.push_back(inner_of_var_[c]);
+    }
+    nd.ic_cnt = (int)ci.size() - nd.ic_off;
+    nd.lc_cnt = (int)cl.size() - nd.lc_off;
+    nd.has_inner_child = nd.ic_cnt > 0;
+  }
+  if (ci.empty()) ci.push_back(0);
+  if (cl.empty()) cl.push_back(0);
+  d_nodes_.upload(nodes);
+  d_child_inner_.upload(ci);
+  d_child_leaf_.upload(cl);
+
+  // forward levels: by height (1..H); backward levels: by depth (0..D)
+  auto make_levels = [&](const std::vector<int32_t>& key, int& n_levels, DevBuf<int32_t>& dptr,
+                         DevBuf<int32_t>& ditems) {
+    int maxk = 0;
+    for (int n = 0; n < n_inner_; ++n) maxk = std::max(maxk, key[n]);
+    n_levels = maxk + 1;
+    std::vector<int32_t> ptr(n_levels + 1, 0), items(n_inner_);
+    for (int n = 0; n < n_inner_; ++n) ptr[key[n] + 1]++;
+    for (int l = 0; l < n_levels; ++l) ptr[l + 1] += ptr[l];
+    std::vector<int32_t> fill(ptr.begin(), ptr.end() - 1);
+    for (int n = 0; n < n_inner_; ++n) items[fill[key[n]]++] = n;
+    dptr.upload(ptr);
+    ditems.upload(items);
+  };
+  std::vector<int32_t> hk(n_inner_), dk(n_inner_);
+  for (int n = 0; n < n_inner_; ++n) {
+    hk[n] = height_[var_of_inner_[n]] - 1;
+    dk[n] = depth_[var_of_inner_[n]];
+  }
+  make_levels(hk, n_fwd_levels_, d_fwd_ptr_, d_fwd_items_);
+  // compact the depth keys of inner nodes (a depth with only leaf tree nodes has no items,
+  // which is fine: an empty level costs one barrier)
+  make_levels(dk, n_bwd_levels_, d_bwd_ptr_, d_bwd_items_);
+}
+
+// Numbering the reference would give this circuit.  Nodes are created in depth-first
+// post-order from the root sum node (children in order, prime before sub); the sum node
+// (v, k) is reached from its tree parent's edge j = k, so the first visit of tree node v is
+// through (v, 0), which creates, for j = 0..K-1: [children circuits at state j], [the
+// K-ary product if v has several children], input leaf_v[j]; then sum (v, 0); later visits
+// create only (v, k).  Up edges are ordered by layer, then by parent id
+// (reference: test/bits_circuit_tests.jl:13-24, test/misc_tests.jl:39-62 for the pinned
+// part; src/bits_circuit.jl:46-70 for the tables).
+void HcltCircuit::build_param_order() {
+  const int K = K_;
+  std::vector<int64_t> sum_id((size_t)V_ * K, -1), mul_id((size_t)V_ * K, -1), in_id((size_t)V_ * K, -1);
+  int64_t next = 0;
+  input_order_.clear();
+  // explicit stack machine for visit(v, k)
+  struct Frame { int v, k, j, c; };
+  std::vector<Frame> st;
+  auto create_input = [&](int v, int j) {
+    if (in_id[(size_t)v * K + j] < 0) {
+      in_id[(size_t)v * K + j] = next++;
+      input_order_.push_back(v * K + j);
+    }
+  };
+  st.push_back({root_, 0, 0, 0});
+  std::vector<char> expanded(V_, 0);
+  while (!st.empty()) {
+    Frame& f = st.back();
+    const int v = f.v;
+    if (sum_id[(size_t)v * K + f.k] >= 0) { st.pop_back(); continue; }
+    if (expanded[v] == 2) {   // subtree already created: only this sum node is new
+      sum_id[(size_t)v * K + f.k] = next++;
+      st.pop_back();
+      continue;
+    }
+    expanded[v] = 1;
+    if (f.j < K) {
+      if (f.c < (int)children_[v].size()) {
+        int c = children_[v][f.c++];
+        if (children_[c].empty()) create_input(c, f.j);
+        else if (sum_id[(size_t)c * K + f.j] < 0) st.push_back({c, f.j, 0, 0});
+        continue;
+      }
+      if (children_[v].size() > 1) mul_id[(size_t)v * K + f.j] = next++;
+      create_input(v, f.j);
+      f.j++;
+      f.c = 0;
+      continue;
+    }
+    expanded[v] = 2;
+    sum_id[(size_t)v * K + f.k] = next++;
+    st.pop_back();
+  }
+  n_nodes_ = next;
+
+  // layers
+  std::vector<int> vlayer(V_, 0);   // layer of the sum nodes of v (0 for leaves = inputs)
+  std::vector<int> mlayer(V_, 0);
+  for (int n = 0; n < n_inner_; ++n) {
+    int v = var_of_inner_[n];
+    int lc = 0;
+    for (int c : children_[v]) lc = std::max(lc, vlayer[c]);
+    if (children_[v].size() > 1) { mlayer[v] = lc + 1; lc = lc + 1; }
+    vlayer[v] = lc + 1;
+  }
+  // edge records (parent id, layer) -> sorted
+  struct Rec { int layer; int64_t parent; int kind; int v, k; };   // kind 0 mul, 1 sum
+  std::vector<Rec> recs;
+  for (int n = 0; n < n_inner_; ++n) {
+    int v = var_of_inner_[n];
+    if (children_[v].size() > 1)
+      for (int j = 0; j < K; ++j) recs.push_back({mlayer[v], mul_id[(size_t)v * K + j], 0, v, j});
+    int nk = v == root_ ? 1 : K;
+    for (int k = 0; k < nk; ++k) recs.push_back({vlayer[v], sum_id[(size_t)v * K + k], 1, v, k});
+  }
+  std::sort(recs.begin(), recs.end(), [](const Rec& a, const Rec& b) {
+    return a.layer != b.layer ? a.layer < b.layer : a.parent < b.parent;
+  });
+  sum_param_src_.clear();
+  sum_group_size_.clear();
+  edge2param_.clear(); edge_parent_.clear(); edge_prime_.clear(); edge_sub_.clear(); layer_ends_.clear();
+  auto circ_id = [&](int c, int j) -> int64_t {
+    return children_[c].empty() ? in_id[(size_t)c * K + j] : sum_id[(size_t)c * K + j];
+  };
+  int cur_layer = recs.empty() ? 0 : recs[0].layer;
+  for (const Rec& r : recs) {
+    if (r.layer != cur_layer) { layer_ends_.push_back((int64_t)edge_parent_.size()); cur_layer = r.layer; }
+    const auto& ch = children_[r.v];
+    if (r.kind == 0) {
+      for (size_t q = 0; q < ch.size(); q += 2) {
+        edge_parent_.push_back(r.parent + 1);
+        edge_prime_.push_back(circ_id(ch[q], r.k) + 1);
+        edge_sub_.push_back(q + 1 < ch.size() ? circ_id(ch[q + 1], r.k) + 1 : 0);
+        edge2param_.push_back(0);
+      }
+    } else {
+      const int n = inner_of_var_[r.v];
+      for (int j = 0; j < K; ++j) {
+        edge_parent_.push_back(r.parent + 1);
+        int64_t prime = ch.size() > 1 ? mul_id[(size_t)r.v * K + j] : circ_id(ch[0], j);
+        edge_prime_.push_back(prime + 1);
+        edge_sub_.push_back(in_id[(size_t)r.v * K + j] + 1);
+        sum_param_src_.push_back(((int64_t)n * K + r.k) * K + j);
+        edge2param_.push_back((int64_t)sum_param_src_.size());
+      }
+      sum_group_size_.push_back(K);
+    }
+  }
+  layer_ends_.push_back((int64_t)edge_parent_.size());
+  n_edges_ = (int64_t)edge_parent_.size();
+  d_sum_param_src_.upload(sum_param_src_);
+}
+
+int64_t HcltCircuit::size(int what) const {
+  switch (what) {
+    case 0: return (int64_t)sum_param_src_.size() + (int64_t)V_ * K_ * C_;
+    case 1: return (int64_t)sum_param_src_.size();
+    case 2: return n_nodes_;
+    case 3: return n_edges_;
+    case 4: return (int64_t)V_ * K_ * C_;
+    case 5: return V_;
+    case 6: return C_;
+    case 7: return K_;
+    case 8: return n_inner_;
+    case 9: return (int64_t)layer_ends_.size();
+    case 10: return (int64_t)sum_group_size_.size();
+    case 11: return (int64_t)V_ * K_;
+    default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
+  }
+}
+
+void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
+  auto copy = [&](const std::vector<int64_t>& v) {
+    if ((int64_t)v.size() != n) fail(PCM_ERR_ARG, "index table %d has %lld entries, caller gave %lld",
+                                     which, (long long)v.size(), (long long)n);
+    std::copy(v.begin(), v.end(), out);
+  };
+  switch (which) {
+    case 0: copy(edge2param_); break;
+    case 1: {
+      std::vector<int64_t> p2e;
+      for (size_t e = 0; e < edge2param_.size(); ++e) if (edge2param_[e]) p2e.push_back((int64_t)e + 1);
+      copy(p2e); break;
+    }
+    case 2: {
+      std::vector<int64_t> p2g;
+      for (size_t gi = 0; gi < sum_group_size_.size(); ++gi)
+        for (int i = 0; i < sum_group_size_[gi]; ++i) p2g.push_back((int64_t)gi + 1);
+      copy(p2g); break;
+    }
+    case 3: copy(std::vector<int64_t>(sum_group_size_.begin(), sum_group_size_.end())); break;
+    case 4: {
+      std::vector<int64_t> cum((size_t)V_ * K_);
+      for (size_t i = 0; i < cum.size(); ++i) cum[i] = (int64_t)(i + 1) * C_;
+      copy(cum); break;
+    }
+    case 5: copy(layer_ends_); break;
+    case 6: copy(edge_parent_); break;
+    case 7: copy(edge_prime_); break;
+    case 8: copy(edge_sub_); break;
+    default: fail(PCM_ERR_ARG, "unknown index table %d", which);
+  }
+}
+
+// ---- parameters -------------------------------------------------------------------
+
+void HcltCircuit::rebuild_w() {
+  const int64_t tot = (int64_t)n_inner_ * K_ * K_;
+  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_rebuild_w_kernel<KK>, dim3(ceil_div(tot, 256)), dim3(256), 0,
+                                        stream, d_logtheta_.p, d_Wf_.p, d_Wb_.p, n_inner_));
+  check_launch("rebuild_w");
+}
+
+void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
+  const int K = K_, C = C_;
+  if (theta) {
+    std::vector<float> lt((size_t)n_inner_ * K * K);
+    for (int n = 0; n < n_inner_; ++n) {
+      const float* src = theta + (size_t)var_of_inner_[n] * K * K;
+      float* dst = lt.data() + (size_t)n * K * K;
+      std::copy(src, src + (size_t)K * K, dst);
+      if (var_of_inner_[n] == root_)
+        for (int i = K; i < K * K; ++i) dst[i] = -INFINITY;   // the root keeps one sum node
+    }
+    PCM_HIP(hipMemcpyAsync(d_logtheta_.p, lt.data(), lt.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+    PCM_HIP(hipStreamSynchronize(stream));
+    rebuild_w();
+  }
+  if (leaf) {
+    std::vector<float> t((size_t)V_ * C * K);
+    for (int v = 0; v < V_; ++v)
+      for (int j = 0; j < K; ++j)
+        for (int c = 0; c < C; ++c) t[((size_t)v * C + c) * K + j] = leaf[((size_t)v * K + j) * C + c];
+    PCM_HIP(hipMemcpyAsync(d_leaf_.p, t.data(), t.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+    PCM_HIP(hipStreamSynchronize(stream));
+  }
+}
+
+static void fetch(std::vector<float>& h, const float* d, size_t n, hipStream_t s) {
+  h.resize(n);
+  PCM_HIP(hipMemcpyAsync(h.data(), d, n * sizeof(float), hipMemcpyDeviceToHost, s));
+  PCM_HIP(hipStreamSynchronize(s));
+}
+
+void HcltCircuit::get_block_params(float* theta, float* leaf) {
+  const int K = K_, C = C_;
+  std::vector<float> h;
+  if (theta) {
+    fetch(h, d_logtheta_.p, d_logtheta_.n, stream);
+    std::fill(theta, theta + (size_t)V_ * K * K, 0.f);
+    for (int n = 0; n < n_inner_; ++n)
+      std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
+                theta + (size_t)var_of_inner_[n] * K * K);
+  }
+  if (leaf) {
+    fetch(h, d_leaf_.p, d_leaf_.n, stream);
+    for (int v = 0; v < V_; ++v)
+      for (int j = 0; j < K; ++j)
+        for (int c = 0; c < C; ++c) leaf[((size_t)v * K + j) * C + c] = h[((size_t)v * C + c) * K + j];
+  }
+}
+
+void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
+  const int K = K_, C = C_;
+  std::vector<float> h;
+  if (edge_aggr) {
+    fetch(h, d_edge_aggr_.p, d_edge_aggr_.n, stream);
+    std::fill(edge_aggr, edge_aggr + (size_t)V_ * K * K, 0.f);
+    for (int n = 0; n < n_inner_; ++n)
+      std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
+                edge_aggr + (size_t)var_of_inner_[n] * K * K);
+  }
+  if (leaf_flow) {
+    fetch(h, d_leaf_flow_.p, d_leaf_flow_.n, stream);
+    for (int v = 0; v < V_; ++v)
+      for (int j = 0; j < K; ++j)
+        for (int c = 0; c < C; ++c) leaf_flow[((size_t)v * K + j) * C + c] = h[((size_t)v * C + c) * K + j];
+  }
+}
+
+void HcltCircuit::vectorize(float* out, int64_t n) {
+  if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
+                         (long long)size(0));
+  std::vector<float> lt, lf;
+  fetch(lt, d_logtheta_.p, d_logtheta_.n, stream);
+  fetch(lf, d_leaf_.p, d_leaf_.n, stream);
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  for (int64_t i = 0; i < ns; ++i) out[i] = lt[sum_param_src_[i]];
+  float* o = out + ns;
+  for (size_t q = 0; q < input_order_.size(); ++q) {
+    const int v = input_order_[q] / K_, j = input_order_[q] % K_;
+    for (int c = 0; c < C_; ++c) o[q * C_ + c] = lf[((size_t)v * C_ + c) * K_ + j];
+  }
+}
+
+void HcltCircuit::update_parameters(const float* in, int64_t n) {
+  if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
+                         (long long)size(0));
+  std::vector<float> lt;
+  fetch(lt, d_logtheta_.p, d_logtheta_.n, stream);
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  for (int64_t i = 0; i < ns; ++i) lt[sum_param_src_[i]] = in[i];
+  std::vector<float> lf((size_t)V_ * C_ * K_);
+  const float* o = in + ns;
+  for (size_t q = 0; q < input_order_.size(); ++q) {
+    const int v = input_order_[q] / K_, j = input_order_[q] % K_;
+    for (int c = 0; c < C_; ++c) lf[((size_t)v * C_ + c) * K_ + j] = o[q * C_ + c];
+  }
+  PCM_HIP(hipMemcpyAsync(d_logtheta_.p, lt.data(), lt.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+  PCM_HIP(hipMemcpyAsync(d_leaf_.p, lf.data(), lf.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+  rebuild_w();
+}
+
+// ---- batches ------------------------------------------------------------------------
+
+void HcltCircuit::ensure_batch(int batch) {
+  const int ns = ceil_div(batch, kSlice);
+  if (ns <= cap_slices_) return;
+  d_O_.alloc((size_t)n_inner_ * ns * kSlice * K_);
+  d_G_.alloc((size_t)n_inner_ * ns * kSlice * K_);
+  d_xb_.alloc((size_t)V_ * ns * kSlice);
+  cap_slices_ = ns;
+}
+
+HcltDev HcltCircuit::dev(int batch) const {
+  HcltDev d;
+  d.nodes = d_nodes_.p;
+  d.child_inner = d_child_inner_.p;
+  d.child_leaf = d_child_leaf_.p;
+  d.leaf = d_leaf_.p;
+  d.logtheta = d_logtheta_.p;
+  d.Wf = d_Wf_.p;
+  d.Wb = d_Wb_.p;
+  d.xb = d_xb_.p;
+  d.O = d_O_.p;
+  d.G = d_G_.p;
+  d.B = batch;
+  d.nslices = ceil_div(batch, kSlice);
+  d.Bp = d.nslices * kSlice;
+  d.C = C_;
+  d.n_inner = n_inner_;
+  d.V = V_;
+  return d;
+}
+
+void HcltCircuit::stage_batch(const BatchRef& b) {
+  if (!b.d_data) fail(PCM_ERR_ARG, "data pointer is null");
+  if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
+  ensure_batch(b.batch);
+  const int Bp = ceil_div(b.batch, kSlice) * kSlice;
+  hipLaunchKernelGGL(hclt_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
+                     b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
+  check_launch("stage_batch");
+}
+
+void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
+  if (timing) PCM_HIP(hipEventRecord(ev_[0], stream));
+  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_forward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
+                                        stream, d, d_fwd_ptr_.p, d_fwd_items_.p, n_fwd_levels_, d_ll));
+  check_launch("hclt_forward");
+  if (timing) PCM_HIP(hipEventRecord(ev_[1], stream));
+}
+
+void HcltCircuit::run_backward(const HcltDev& d) {
+  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_backward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
+                                        stream, d, d_bwd_ptr_.p, d_bwd_items_.p, n_bwd_levels_));
+  check_launch("hclt_backward");
+  if (timing) PCM_HIP(hipEventRecord(ev_[2], stream));
+}
+
+void HcltCircuit::run_stats(const HcltDev& d, float rate) {
+  int dev_id = 0, max_lds = 0;
+  PCM_HIP(hipGetDevice(&dev_id));
+  PCM_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev_id));
+  const size_t hist = (size_t)C_ * (K_ + 1) * sizeof(float);
+  const size_t amin = std::max(hist, (size_t)K_ * K_ * sizeof(float));
+  int waves = kStatWaves;
+  auto pads_of = [&](int w) { return (size_t)w * 2 * kSlice * (K_ + 16) * sizeof(float); };
+  while (waves > 1 && pads_of(waves) + amin > (size_t)max_lds) waves /= 2;
+  const size_t pads = pads_of(waves);
+  if (pads + amin > (size_t)max_lds)
+    fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", pads + amin, max_lds);
+  int nh = std::min(4, (int)(((size_t)max_lds - pads) / hist));
+  size_t hist_floats = ((size_t)nh * C_ * (K_ + 1) + 3) & ~(size_t)3;
+  hist_floats = std::max(hist_floats, (size_t)K_ * K_);
+  const size_t lds = hist_floats * sizeof(float) + pads;
+  PCM_DISPATCH_K(K_, {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_kernel<KK>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(hclt_stats_kernel<KK>, dim3(n_inner_), dim3(waves * 64), lds, stream, d,
+                       d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_floats);
+  });
+  check_launch("hclt_stats");
+  if (timing) PCM_HIP(hipEventRecord(ev_[3], stream));
+}
+
+void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (timing && !ev_[0]) for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
+  stage_batch(b);
+  run_forward(dev(b.batch), d_ll);
+}
+
+void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
+  if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (timing && !ev_[0]) for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
+  stage_batch(b);
+  HcltDev d = dev(b.batch);
+  run_forward(d, d_ll);
+  run_backward(d);
+  run_stats(d, rate);
+  have_flows_ = true;
+  if (timing) {
+    PCM_HIP(hipStreamSynchronize(stream));
+    for (int i = 0; i < 3; ++i) PCM_HIP(hipEventElapsedTime(&last_ms[i], ev_[i], ev_[i + 1]));
+  }
+}
+
+void HcltCircuit::em_update(float pseudocount, float inertia) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
+  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)),
+                                        dim3(128), 0, stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p,
+                                        d_edge_aggr_.p, n_inner_, pseudocount, inertia));
+  check_launch("theta_update");
+  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(ceil_div((int64_t)V_ * K_, 128)), dim3(128), 0, stream,
+                     d_leaf_.p, d_leaf_flow_.p, V_, C_, K_, pseudocount, inertia);
+  check_launch("leaf_update");
+}
+
+}  // namespace pcm

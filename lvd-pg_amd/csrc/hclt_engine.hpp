@@ -1,0 +1,102 @@
+// Dense-block engine for hidden Chow-Liu tree circuits.
+//
+// An HCLT (reference: src/structures/hclts.jl:100-145) has one K x K block of sum edges
+// per non-leaf tree node v:  O_v[b,k] = logsumexp_j(theta_v[k,j] + Z_v[b,j]) with
+// Z_v[b,j] = leaf_v[j][x_b,v] + sum over tree children c of (O_c[b,j] or leaf_c[j][x_b,c]).
+// The engine never materialises the K^2 product nodes per block; it keeps one K-vector of
+// node values (and one of flows) per tree node and example.
+#pragma once
+
+#include "common.hpp"
+
+namespace pcm {
+
+struct HcltNode {     // one non-leaf tree node, device-resident
+  int32_t var;        // its observed variable
+  int32_t parent;     // inner id of the tree parent, -1 for the root
+  int32_t ic_off, ic_cnt;  // non-leaf tree children (inner ids) in child_inner
+  int32_t lc_off, lc_cnt;  // leaf tree children (variable ids) in child_leaf
+  int32_t is_root;
+  int32_t has_inner_child;
+};
+
+// Everything the kernels need, passed by value.
+struct HcltDev {
+  const HcltNode* nodes;
+  const int32_t* child_inner;
+  const int32_t* child_leaf;
+  const float* leaf;      // [V][C][K] log-probabilities, hidden state fastest
+  const float* logtheta;  // [n_inner][K][K]
+  const float* Wf;        // exp(theta) laid out per MFMA operand, forward contraction
+  const float* Wb;        // same values, operand layout of the backward contraction
+  const uint8_t* xb;      // [V][Bp] batch categories, example fastest
+  float* O;               // [n_inner][nslices][16*K] node values, tile-native layout
+  float* G;               // [n_inner][nslices][16*K] child flows, same layout
+  int32_t B, Bp, nslices, C, n_inner, V;
+};
+
+class HcltCircuit : public pcm_circuit {
+ public:
+  HcltCircuit(const int32_t* parent, int V, int K, int C);
+  ~HcltCircuit() override {}
+
+  int64_t size(int what) const override;
+  void index_table(int which, int64_t* out, int64_t n) const override;
+  void vectorize(float* out, int64_t n) override;
+  void update_parameters(const float* in, int64_t n) override;
+  void loglikelihoods(const BatchRef& b, float* d_ll) override;
+  void flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) override;
+  void em_update(float pseudocount, float inertia) override;
+  void kld(pcm_circuit* q, float* out) override;
+  void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
+  int64_t sample_noise_size() const override { return (int64_t)n_inner_ * K_; }
+  void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
+              uint8_t* d_out) override;
+  void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
+                 float b2, float eps, int t) override;
+
+  void set_block_params(const float* theta, const float* leaf);
+  void get_block_params(float* theta, float* leaf);
+  void get_block_flows(float* edge_aggr, float* leaf_flow);
+
+  // Kernel timing hooks for the benchmark: ms of the last forward / backward / statistics
+  // launches measured with events on the circuit's stream (0 if timing is off).
+  bool timing = false;
+  float last_ms[4] = {0, 0, 0, 0};
+
+ private:
+  int V_, K_, C_, n_inner_, root_;
+  std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;
+  std::vector<std::vector<int32_t>> children_;
+  int n_fwd_levels_ = 0, n_bwd_levels_ = 0;
+  // parameter-vector order (reference numbering, see build_param_order)
+  std::vector<int64_t> sum_param_src_;   // param i -> index into logtheta [n_inner][K][K]
+  std::vector<int32_t> sum_group_size_;  // sizes of the normalisation groups, in order
+  std::vector<int32_t> input_order_;     // i-th input node -> v*K + j
+  std::vector<int64_t> edge2param_, edge_parent_, edge_prime_, edge_sub_, layer_ends_;
+  int64_t n_nodes_ = 0, n_edges_ = 0;
+
+  DevBuf<HcltNode> d_nodes_;
+  DevBuf<int32_t> d_child_inner_, d_child_leaf_, d_fwd_ptr_, d_fwd_items_, d_bwd_ptr_, d_bwd_items_;
+  DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_G_;
+  DevBuf<uint8_t> d_xb_;
+  DevBuf<float> d_leaf_kc_;      // [V][K][C] copy for sampling
+  DevBuf<float> d_kld_;          // scratch of the KL recursion
+  DevBuf<uint8_t> d_state_;
+  DevBuf<int64_t> d_sum_param_src_;
+  int cap_slices_ = 0;
+  bool have_flows_ = false;
+  hipEvent_t ev_[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+
+  void build_structure();
+  void build_param_order();
+  void ensure_batch(int batch);
+  HcltDev dev(int batch) const;
+  void stage_batch(const BatchRef& b);
+  void rebuild_w();
+  void run_forward(const HcltDev& d, float* d_ll);
+  void run_backward(const HcltDev& d);
+  void run_stats(const HcltDev& d, float rate);
+};
+
+}  // namespace pcm

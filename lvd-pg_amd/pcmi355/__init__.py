@@ -1,0 +1,12 @@
+"""Host-side mirror of the reference's probabilistic-circuit API over libpcmi355.so.
+
+The reference's host language (Julia) is not available where this package is built, so
+the host side is Python; names, argument meaning and error behaviour follow the Julia
+functions cited in each docstring (paths relative to VariationalJuice.jl/).  Device
+memory and streams come from torch; everything numeric happens in the HIP library.
+"""
+from .circuits import BitsCircuit, HcltCircuit, hclt_from_clt, compile_circuit, compile_multihead  # noqa: F401
+from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
+                      vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
+                      mini_batch_em_for_multihead_pc)
+from ._lib import PcmError, LIB_PATH  # noqa: F401

@@ -1,0 +1,141 @@
+"""Compiled circuits: thin owners of a `pcm_circuit*` handle."""
+import ctypes
+
+import numpy as np
+
+from ._lib import lib, check, np_ptr, H, c_i64
+
+_SIZE = dict(parameters=0, sum_parameters=1, nodes=2, edges=3, input_parameters=4, variables=5,
+             categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11)
+_TABLE = dict(edge2param=(0, "edges"), param2edge=(1, "sum_parameters"), param2group=(2, "sum_parameters"),
+              pargroup_sizes=(3, "groups"), innode2ncumparam=(4, "input_nodes"), layer_ends=(5, "layers"),
+              edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"))
+
+
+class BitsCircuit:
+    """Counterpart of `CuMetaBitsProbCircuit` (src/bits_circuit.jl:5-37): the flattened
+    circuit lives on the device inside the library; index tables are served on request."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            lib.pcm_free(h)
+
+    @property
+    def handle(self):
+        if not self._h:
+            raise ValueError("circuit has been freed")
+        return self._h
+
+    def size(self, what):
+        r = lib.pcm_size(self.handle, _SIZE[what])
+        if r < 0:
+            check(-1)
+        return int(r)
+
+    # src/bits_circuit.jl:119-131
+    def num_parameters(self):
+        return self.size("parameters")
+
+    def num_nodes(self):
+        return self.size("nodes")
+
+    def num_edges(self):
+        return self.size("edges")
+
+    def num_input_params(self):
+        return self.size("input_parameters")
+
+    def num_inner_params(self):
+        return self.size("sum_parameters")
+
+    def table(self, name):
+        """1-based index tables named as the fields of `CuMetaBitsProbCircuit`."""
+        which, length = _TABLE[name]
+        out = np.empty(self.size(length), dtype=np.int64)
+        check(lib.pcm_index_table(self.handle, which, np_ptr(out), c_i64(len(out))))
+        return out
+
+    def set_stream(self, stream):
+        check(lib.pcm_set_stream(self.handle, ctypes.c_void_p(stream)))
+
+
+class HcltCircuit(BitsCircuit):
+    def __init__(self, handle, clt_parent, num_cats, num_hidden_cats):
+        super().__init__(handle)
+        self.clt_parent = np.asarray(clt_parent, dtype=np.int32).copy()
+        self.num_vars = len(self.clt_parent)
+        self.num_cats = num_cats
+        self.num_hidden_cats = num_hidden_cats
+
+    def set_params(self, theta=None, leaf=None):
+        """theta [V, K, K], leaf [V, K, C] log-parameters (block form)."""
+        V, K, C = self.num_vars, self.num_hidden_cats, self.num_cats
+        if theta is not None:
+            theta = np.ascontiguousarray(theta, dtype=np.float32)
+            assert theta.shape == (V, K, K), theta.shape
+        if leaf is not None:
+            leaf = np.ascontiguousarray(leaf, dtype=np.float32)
+            assert leaf.shape == (V, K, C), leaf.shape
+        check(lib.pcm_hclt_set_params(self.handle, np_ptr(theta), np_ptr(leaf)))
+
+    def get_params(self):
+        V, K, C = self.num_vars, self.num_hidden_cats, self.num_cats
+        theta = np.empty((V, K, K), np.float32)
+        leaf = np.empty((V, K, C), np.float32)
+        check(lib.pcm_hclt_get_params(self.handle, np_ptr(theta), np_ptr(leaf)))
+        return theta, leaf
+
+    def get_flows(self):
+        V, K, C = self.num_vars, self.num_hidden_cats, self.num_cats
+        ea = np.empty((V, K, K), np.float32)
+        lf = np.empty((V, K, C), np.float32)
+        check(lib.pcm_hclt_get_flows(self.handle, np_ptr(ea), np_ptr(lf)))
+        return ea, lf
+
+    def set_timing(self, on):
+        check(lib.pcm_set_timing(self.handle, int(on)))
+
+    def get_timing(self):
+        ms = np.zeros(4, np.float32)
+        check(lib.pcm_get_timing(self.handle, np_ptr(ms), 4))
+        return dict(forward=float(ms[0]), backward=float(ms[1]), statistics=float(ms[2]))
+
+
+def hclt_from_clt(clt_parent, num_cats, num_hidden_cats):
+    """`hclt_from_clt(clt, num_cats, num_hidden_cats, variable_groups; input_type = Categorical)`
+    (src/structures/hclts.jl:100-145) followed by `CuMetaBitsProbCircuit(pc)`; the tree is
+    given as a parent array (root: -1), one observed variable per tree node."""
+    par = np.ascontiguousarray(clt_parent, dtype=np.int32)
+    h = H()
+    check(lib.pcm_hclt_create(np_ptr(par), len(par), int(num_hidden_cats), int(num_cats), ctypes.byref(h)))
+    return HcltCircuit(h, par, int(num_cats), int(num_hidden_cats))
+
+
+def compile_circuit(node_type, child_ptr, child_idx, sum_logp, input_var, input_logp, num_vars, num_cats,
+                    num_heads=0):
+    """`CuMetaBitsProbCircuit(pc)` (src/bits_circuit.jl:39) for a DAG in flat form."""
+    node_type = np.ascontiguousarray(node_type, np.uint8)
+    child_ptr = np.ascontiguousarray(child_ptr, np.int32)
+    child_idx = np.ascontiguousarray(child_idx, np.int32)
+    sum_logp = np.ascontiguousarray(sum_logp, np.float32)
+    input_var = np.ascontiguousarray(input_var, np.int32)
+    input_logp = np.ascontiguousarray(input_logp, np.float32)
+    h = H()
+    check(lib.pcm_circuit_create(len(node_type), np_ptr(node_type), np_ptr(child_ptr), np_ptr(child_idx),
+                                 np_ptr(sum_logp), np_ptr(input_var), np_ptr(input_logp), int(num_vars),
+                                 int(num_cats), int(num_heads), ctypes.byref(h)))
+    c = BitsCircuit(h)
+    c.num_vars, c.num_cats, c.num_heads = int(num_vars), int(num_cats), int(num_heads)
+    return c
+
+
+def compile_multihead(node_type, child_ptr, child_idx, sum_logp, input_var, input_logp, num_vars, num_cats,
+                      num_heads):
+    """`CuMultiHeadBitsProbCircuit(pcs)` (src-jl/multi_head_pc/bit_circuit.jl:14-56): the
+    last `num_heads` nodes of the description are the heads."""
+    return compile_circuit(node_type, child_ptr, child_idx, sum_logp, input_var, input_logp, num_vars,
+                           num_cats, num_heads)

@@ -1,0 +1,194 @@
+"""Queries and learning loops, named after the reference functions they replace."""
+import numpy as np
+import torch
+
+from ._lib import lib, check, np_ptr, c_i64
+
+
+def _dev_ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _check_data(bpc, data):
+    if not (isinstance(data, torch.Tensor) and data.is_cuda and data.dtype == torch.uint8 and data.dim() == 2):
+        raise ValueError("data must be a 2-D uint8 tensor on the GPU (examples x variables)")
+    nv = bpc.size("variables")
+    if data.shape[1] != nv:
+        raise ValueError(f"data has {data.shape[1]} variables, circuit has {nv}")
+
+
+def _ids(example_ids, device):
+    if example_ids is None:
+        return None
+    if isinstance(example_ids, torch.Tensor):
+        return example_ids.to(device=device, dtype=torch.int32).contiguous()
+    return torch.as_tensor(np.asarray(example_ids), dtype=torch.int32, device=device)
+
+
+def loglikelihoods(bpc, data, batch_size=None, example_ids=None):
+    """`loglikelihoods(bpc, data; batch_size)` / `loglikelihoods_probcat`
+    (src/regularization/reg_likelihood.jl:139-162): per-example log-likelihoods as a device
+    vector.  A multi-head circuit returns [num_examples, num_heads]
+    (src-jl/multi_head_pc/likelihood.jl:37-71 with head_mask = nothing)."""
+    _check_data(bpc, data)
+    ids = _ids(example_ids, data.device)
+    n = data.shape[0] if ids is None else len(ids)
+    batch_size = n if batch_size is None else batch_size
+    heads = getattr(bpc, "num_heads", 0)
+    out = torch.empty((max(heads, 1), n), dtype=torch.float32, device=data.device)
+    for s in range(0, n, batch_size):
+        b = min(batch_size, n - s)
+        if ids is None:
+            d_ptr, i_ptr = data[s:s + b].data_ptr(), None
+        else:
+            d_ptr, i_ptr = data.data_ptr(), ids[s:s + b].data_ptr()
+        if heads:
+            tmp = torch.empty((heads, b), dtype=torch.float32, device=data.device)
+            check(lib.pcm_loglikelihoods(bpc.handle, d_ptr, data.stride(0), data.stride(1), i_ptr, b, tmp.data_ptr()))
+            out[:, s:s + b] = tmp
+        else:
+            check(lib.pcm_loglikelihoods(bpc.handle, d_ptr, data.stride(0), data.stride(1), i_ptr, b,
+                                         out[0, s:s + b].data_ptr()))
+    return out.t().contiguous() if heads else out[0]
+
+
+def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
+    """`probs_flows_circuit` (src/queries/flow.jl:228-234) /
+    `probs_flows_circuit_with_reg` with soft_reg = 0 (src/regularization/reg_flow.jl:276-282):
+    forward, backward and leaf flows for one batch; the aggregates stay in the circuit.
+    Returns the batch's log-likelihoods (`mars[:, end]`)."""
+    _check_data(bpc, data)
+    ids = _ids(example_ids, data.device)
+    b = data.shape[0] if ids is None else len(ids)
+    ll = torch.empty(b, dtype=torch.float32, device=data.device)
+    hm = None
+    if head_mask is not None:
+        hm = head_mask.to(device=data.device, dtype=torch.float32)
+        if ids is not None:
+            hm = hm[ids.long()]
+        hm = hm.t().contiguous()   # [heads, batch]
+    check(lib.pcm_flows(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), _dev_ptr(ids), b,
+                        float(rate), _dev_ptr(hm), ll.data_ptr()))
+    return ll
+
+
+def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
+                           ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
+                           shuffle="each_epoch", verbose=False, generator=None, head_mask=None):
+    """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
+    of per-epoch mean log-likelihoods.  soft_reg and ent_reg must be 0 (the reference's
+    entropy regulariser is commented out at :294-296; soft evidence is not built)."""
+    if soft_reg != 0.0 or ent_reg != 0.0:
+        raise NotImplementedError("soft_reg / ent_reg other than 0 are not supported")
+    _check_data(bpc, data)
+    n = data.shape[0]
+    if batch_size > n:
+        raise ValueError("batch_size must not exceed the number of examples")   # reg_em.jl:219
+    num_batches = n // batch_size   # drop last incomplete batch (:217)
+    if param_inertia_end is None:
+        param_inertia_end = param_inertia
+    d_inertia = (param_inertia_end - param_inertia) / num_epochs
+    perm = torch.arange(n, dtype=torch.int32, device=data.device)
+
+    def do_shuffle():
+        nonlocal perm
+        perm = torch.randperm(n, generator=generator).to(device=data.device, dtype=torch.int32)
+
+    if shuffle == "once":
+        do_shuffle()
+    lls = []
+    ll = torch.empty(batch_size, dtype=torch.float32, device=data.device)
+    hm_t = None if head_mask is None else head_mask.to(device=data.device, dtype=torch.float32)
+    for _ in range(num_epochs):
+        if shuffle == "each_epoch":
+            do_shuffle()
+        acc = torch.zeros((), dtype=torch.float64, device=data.device)
+        for bi in range(num_batches):
+            if shuffle == "each_batch":
+                do_shuffle()
+            ids = perm[bi * batch_size:(bi + 1) * batch_size]
+            rate = 0.0 if flow_memory == 0 else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
+            if hm_t is None:
+                check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
+                                      batch_size, rate, float(pseudocount), float(param_inertia), ll.data_ptr()))
+            else:
+                hm = hm_t[ids.long()].t().contiguous()
+                check(lib.pcm_flows(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
+                                    batch_size, rate, hm.data_ptr(), ll.data_ptr()))
+                check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
+            acc += ll.sum(dtype=torch.float64)
+        lls.append(float(acc.item()) / batch_size / num_batches)
+        param_inertia += d_inertia
+        if verbose:
+            print(f"Mini-batch EM epoch {len(lls)}/{num_epochs}; train LL {lls[-1]}")
+    return lls
+
+
+def mini_batch_em(bpc, data, num_epochs, *, batch_size, pseudocount, param_inertia, param_inertia_end=None,
+                  flow_memory=0.0, shuffle="each_epoch", **kw):
+    """`PCs.mini_batch_em` as called by test/sgd/adam_tests.jl:20: the same loop without
+    regularisers."""
+    return mini_batch_em_with_reg(bpc, data, num_epochs, batch_size=batch_size, pseudocount=pseudocount,
+                                  param_inertia=param_inertia, param_inertia_end=param_inertia_end,
+                                  flow_memory=flow_memory, shuffle=shuffle, **kw)
+
+
+def mini_batch_em_for_multihead_pc(mhbpc, data, head_mask, num_epochs, **kw):
+    """`mini_batch_em_for_multihead_pc` (src-jl/multi_head_pc/em.jl:1-99)."""
+    return mini_batch_em_with_reg(mhbpc, data, num_epochs, head_mask=head_mask, **kw)
+
+
+def vectorize_parameters(bpc):
+    """`vectorize_parameters(mbpc)` (src/misc.jl:33-40) -> host float32 vector."""
+    out = np.empty(bpc.num_parameters(), np.float32)
+    check(lib.pcm_vectorize_parameters(bpc.handle, np_ptr(out), c_i64(len(out))))
+    return out
+
+
+def update_parameters(bpc, params):
+    """`update_parameters(mbpc, params)` (src/misc.jl:73-102)."""
+    p = np.ascontiguousarray(params, np.float32)
+    if len(p) != bpc.num_parameters():   # the reference asserts the same (:75)
+        raise ValueError(f"{bpc.num_parameters()} != {len(p)}")
+    check(lib.pcm_update_parameters(bpc.handle, np_ptr(p), c_i64(len(p))))
+
+
+def kld(bpc_p, bpc_q):
+    """`kld(mbpc, params1, params2)` (src/queries/kld.jl:177-206), one parameter row:
+    the two parameter sets are the two circuits' own parameters."""
+    out = np.zeros(1, np.float32)
+    check(lib.pcm_kld(bpc_p.handle, bpc_q.handle, np_ptr(out)))
+    return float(out[0])
+
+
+def kld_backward(bpc_p, bpc_q):
+    """`kld_backward(mbpc, params1, params2; grad_wrt_logparams = true)`
+    (src/queries/kld.jl:593-649) -> (grads1, grads2) in parameter-vector order."""
+    n = bpc_p.num_parameters()
+    g1 = np.empty(n, np.float32)
+    g2 = np.empty(n, np.float32)
+    check(lib.pcm_kld_backward(bpc_p.handle, bpc_q.handle, np_ptr(g1), np_ptr(g2), c_i64(n)))
+    return g1, g2
+
+
+def sample(bpc, node_noise, leaf_noise):
+    """Gumbel-max samples from supplied noise (temperature -> 0 limit of `gumbel_sample`,
+    src/queries/sample.jl:338-383).  node_noise [B, sample_noise_size], leaf_noise
+    [B, V, C], float32 on the GPU.  Returns uint8 [B, V] on the GPU."""
+    b = node_noise.shape[0]
+    need = int(lib.pcm_sample_noise_size(bpc.handle))
+    nv, nc = bpc.size("variables"), bpc.size("categories")
+    if tuple(node_noise.shape) != (b, need) or tuple(leaf_noise.shape) != (b, nv, nc):
+        raise ValueError(f"noise shapes must be ({b}, {need}) and ({b}, {nv}, {nc})")
+    node_noise = node_noise.contiguous().float()
+    leaf_noise = leaf_noise.contiguous().float()
+    out = torch.empty((b, nv), dtype=torch.uint8, device=node_noise.device)
+    check(lib.pcm_sample(bpc.handle, node_noise.data_ptr(), leaf_noise.data_ptr(), b, out.data_ptr()))
+    return out
+
+
+def adam_step(bpc, grad, params, m, v, *, lr, beta1=0.9, beta2=0.999, eps=1e-8, t=1):
+    """One optimiser step of `adam` (src/sgd/adam.jl:318-325): moving averages, ascent
+    update of the unnormalised sum parameters, per-node normalisation into the circuit."""
+    check(lib.pcm_adam_step(bpc.handle, grad.data_ptr(), params.data_ptr(), m.data_ptr(), v.data_ptr(),
+                            float(lr), float(beta1), float(beta2), float(eps), int(t)))

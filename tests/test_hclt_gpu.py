@@ -1,0 +1,118 @@
+"""GPU parity of the dense-block HCLT engine against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+LL_RTOL = 1e-4      # relative, per-example log-likelihoods (fp32)
+PARAM_RTOL = 1e-4   # relative, updated parameters compared as probabilities
+FLOW_RTOL = 2e-4    # relative to the largest entry of the block, aggregated flows
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    import pcmi355
+    return torch, pcmi355
+
+
+def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None):
+    torch, P = gpu
+    from helpers import make_hclt, correlated_data, oracle_em_reference, block_theta, rel_err
+    parent, theta, leaf, fc = make_hclt(V, K, C, seed)
+    N = N or B
+    data = correlated_data(N, V, C, seed + 1, parent)
+    ids = np.arange(B, dtype=np.int32) if idx is None else idx
+    ll_ref, th_ref, leaf_ref, ea_ref, lf_ref = oracle_em_reference(fc, data, ids, 0.1, 0.9)
+
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    d = torch.from_numpy(data).cuda()
+    ll = P.loglikelihoods(bpc, d, example_ids=None if idx is None else idx)
+    ll = ll.cpu().numpy()
+    assert rel_err(ll, ll_ref).max() < LL_RTOL
+
+    ll2 = P.probs_flows_circuit(bpc, d, example_ids=None if idx is None else idx).cpu().numpy()
+    assert np.array_equal(ll, ll2)
+    ea, lf = bpc.get_flows()
+    for v, blk in ea_ref.items():
+        nk = blk.shape[0]
+        assert np.abs(ea[v][:nk] - blk).max() < FLOW_RTOL * max(blk.max(), 1e-3), f"edge_aggr block {v}"
+        # invariant: flows into the K sum nodes sum to the batch size (root: row 0 only)
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * max(lf_ref.max(), 1e-3)
+    np.testing.assert_allclose(lf.sum(axis=(1, 2)), B, rtol=1e-4)   # every example passes every variable once
+
+    import pcmi355._lib as L
+    L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+    th, lf_new = bpc.get_params()
+    for v, blk in th_ref.items():
+        nk = blk.shape[0]
+        assert rel_err(np.exp(th[v][:nk]), np.exp(blk)).max() < PARAM_RTOL, f"theta block {v}"
+    assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < PARAM_RTOL
+    return bpc
+
+
+@pytest.mark.parametrize("V,K,C,B", [(2, 16, 5, 16), (7, 16, 8, 48), (12, 32, 256, 64), (9, 64, 17, 32)])
+def test_em_step_matches_oracle(gpu, oracle, V, K, C, B):
+    _compare_step(gpu, oracle, V, K, C, B, seed=100 + V)
+
+
+def test_ragged_batch_and_example_ids(gpu, oracle):
+    rng = np.random.default_rng(5)
+    idx = rng.permutation(200)[:37].astype(np.int32)
+    _compare_step(gpu, oracle, 10, 32, 11, 37, seed=7, idx=idx, N=200)
+
+
+def test_config1_shape(gpu, oracle):
+    """64 variables, K=16, 256 categories, batch 1024 (the reference's CPU-runnable case)."""
+    _compare_step(gpu, oracle, 64, 16, 256, 1024, seed=11)
+
+
+def test_param_vector_roundtrip(gpu, oracle):
+    torch, P = gpu
+    from helpers import make_hclt, block_theta
+    parent, theta, leaf, fc = make_hclt(9, 16, 6, 3)
+    bpc = P.hclt_from_clt(parent, 6, 16)
+    bpc.set_params(block_theta(parent, 16, theta), leaf)
+    dag = oracle.bits_compile(oracle.hclt_dag(parent, 16, 6, theta, leaf), 6, 9)
+    ref = dag.vectorize_parameters()
+    got = P.vectorize_parameters(bpc)
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got, ref)
+    P.update_parameters(bpc, got[::-1].copy() * 0 + got)   # write back the same vector
+    np.testing.assert_array_equal(P.vectorize_parameters(bpc), ref)
+    t = dag.param_tables()
+    assert bpc.num_nodes() == dag.n_nodes and bpc.num_edges() == dag.n_edges
+    np.testing.assert_array_equal(bpc.table("edge2param"), t["edge2param"])
+    np.testing.assert_array_equal(bpc.table("param2edge"), t["param2edge"])
+    np.testing.assert_array_equal(bpc.table("param2group"), t["param2group"])
+    np.testing.assert_array_equal(bpc.table("pargroup_sizes"), t["pargroup_sizes"])
+
+
+def test_ten_em_steps_track_oracle(gpu, oracle):
+    """Ten mini-batch EM steps (step size 0.1 == inertia 0.9, pseudocount 0.1) stay on the
+    oracle's trajectory."""
+    torch, P = gpu
+    from helpers import make_hclt, correlated_data, block_theta, rel_err
+    V, K, C, B = 12, 16, 32, 256
+    parent, theta, leaf, fc = make_hclt(V, K, C, 21)
+    data = correlated_data(B, V, C, 22, parent)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    d = torch.from_numpy(data).cuda()
+    import pcmi355._lib as L
+    ll = torch.empty(B, device="cuda")
+    cur = fc
+    for step in range(10):
+        ll_ref, logp, lf, _, _ = oracle.em_step(cur, data, np.arange(B, dtype=np.int32), 0.1, 0.9)
+        cur = cur.copy()
+        cur.logp, cur.leaf_logp = logp, lf
+        L.check(L.lib.pcm_em_step(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, 0.1, 0.9,
+                                  ll.data_ptr()))
+        assert rel_err(ll.cpu().numpy(), ll_ref).max() < LL_RTOL, step
+    th_ref, leaf_ref = oracle.hclt_block_params(cur)
+    th, lf_new = bpc.get_params()
+    for v, blk in th_ref.items():
+        assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
+    assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
