@@ -1,0 +1,145 @@
+#!/usr/bin/env python3
+"""Headline benchmark: examples/sec of forward + backward + EM on the 3072-variable HCLT
+(K = 32, 256 categories, batch 4096) on one MI355X, with the dominant kernel's roofline
+fraction and the CPU oracle timed beside it.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3_hclt3072_k32]
+
+A step is one mini-batch EM iteration (pcm_em_step: stage batch, forward, backward,
+statistics, parameter update) on a batch already resident in HBM.  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "lvd-pg_amd"))
+
+HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
+
+
+def algorithmic_bytes(n_int, V, K, C, B):
+    """Bytes the algorithm has to move per launch, per kernel.  A node-value or flow vector
+    is K*4 bytes per (tree node, example).  Forward writes each node's value vector once and
+    reads it once as a child (2 vectors).  Backward + statistics together need the value
+    vector as child and as parent, and the flow vector written once and read once (4
+    vectors); all of that is booked on the backward kernel, so the statistics kernel, which
+    re-reads three of those vectors, is credited only with the data, parameters and
+    accumulators it alone touches."""
+    vec = K * 4 * B
+    n_sum_edges = (n_int - 1) * K * K + K
+    theta = 4 * n_sum_edges
+    leaf = 4 * V * K * C
+    fwd = n_int * 2 * vec + V * B + theta + leaf
+    bwd = n_int * 4 * vec + V * B + theta + leaf
+    stats = V * B + 2 * theta + 2 * leaf          # read params, write both accumulators
+    update = 2 * theta + 3 * leaf                 # read accumulators, read+write parameters
+    return dict(forward=fwd, backward=bwd, statistics=stats, update=update,
+                step=n_int * 6 * vec + V * B + 3 * theta + 5 * leaf)
+
+
+def cpu_baseline(cfg, sample):
+    """The oracle (a C port of the reference arithmetic, OpenMP over examples) on the
+    first `sample` examples of the same batch: one full EM step."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import numpy as np
+    import pc_oracle as O
+    parent, K, C = cfg["parent"], cfg["K"], cfg["C"]
+    ch, _ = O.clt_children(parent)
+    theta = {v: cfg["theta"][v] for v in range(len(parent)) if ch[v]}
+    fc = O.hclt_flat(parent, K, C, theta, cfg["leaf"])
+    data = np.ascontiguousarray(cfg["data"][:sample])
+    idx = np.arange(sample, dtype=np.int32)
+    t0 = time.perf_counter()
+    ll, *_ = O.em_step(fc, data, idx, 0.1, 0.9)
+    dt = time.perf_counter() - t0
+    return dict(value=sample / dt, unit="examples/s", cores=int(O.lib().orc_max_threads()), kind="port",
+                sample=f"one EM step on the first {sample} examples of the batch, {dt:.1f} s"), ll
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3_hclt3072_k32")
+    ap.add_argument("--cpu-sample", type=int, default=128)
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    import pcmi355
+    from pcmi355 import workloads
+    from pcmi355._lib import lib, check
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+
+    cfg = workloads.make_config(args.workload)
+    stats = workloads.tree_stats(cfg["parent"])
+    V, K, C, B = cfg["V"], cfg["K"], cfg["C"], cfg["B"]
+    bpc = pcmi355.hclt_from_clt(cfg["parent"], C, K)
+    bpc.set_params(cfg["theta"], cfg["leaf"])
+    data = torch.from_numpy(cfg["data"]).cuda()
+    ll = torch.empty(B, dtype=torch.float32, device="cuda")
+
+    def step():
+        check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), None, B, 0.0, 0.1, 0.9,
+                              ll.data_ptr()))
+
+    for _ in range(args.warmup):
+        step()
+    bpc.set_timing(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    kernel_ms = bpc.get_timing()          # mean over the timed steps, events on the launch stream
+    bpc.set_timing(False)
+    ll_first = ll[:args.cpu_sample].cpu().numpy()
+
+    ab = algorithmic_bytes(stats["n_inner"], V, K, C, B)
+    dominant = max(kernel_ms, key=kernel_ms.get)
+    achieved = ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9
+    ms_per_step = dt / args.steps * 1e3
+    out = {
+        "metric": "examples/sec fwd+bwd+EM, 3072-var HCLT K=32; % of HBM/MFMA roofline",
+        "value": B * args.steps / dt,
+        "unit": "examples/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
+                   "tree_inner_nodes": stats["n_inner"], "tree_depth": stats["depth"]},
+        "roofline": {"bound": "hbm", "kernel": f"hclt_{dominant}_kernel", "achieved": achieved,
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+        "kernels_ms": kernel_ms,
+        "step_roofline_frac": ab["step"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+    }
+    if not args.no_cpu:
+        # LL after `warmup + steps` parameter updates differs from the oracle's first step, so
+        # the baseline is only timed here; parity lives in tests/.
+        cb, _ = cpu_baseline(cfg, args.cpu_sample)
+        out["cpu_baseline"] = cb
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

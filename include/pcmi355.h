@@ -189,7 +189,8 @@ int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d
 /* Per-kernel timing, the role of `debug = true` -> `CUDA.@time` around each launch
  * (src/queries/likelihood.jl:86-92, src/queries/flow.jl:127-133).  When on, pcm_flows
  * brackets its forward / backward / statistics launches with events on the circuit's
- * stream and synchronises; pcm_get_timing returns the last milliseconds of each
+ * stream (no synchronisation); pcm_get_timing synchronises and returns the mean
+ * milliseconds over the calls since the previous read of each
  * (n <= 4 values: forward, backward, statistics, reserved). */
 int pcm_set_timing(pcm_circuit* c, int32_t on);
 int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n);

@@ -170,8 +170,7 @@ int pcm_set_timing(pcm_circuit* c, int32_t on) {
 int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n) {
   return guarded([&] {
     if (!ms || n < 0 || n > 4) pcm::fail(PCM_ERR_ARG, "ms is null or n outside 0..4");
-    auto* h = need_hclt(c);
-    for (int i = 0; i < n; ++i) ms[i] = h->last_ms[i];
+    need_hclt(c)->read_timing(ms, n);
   });
 }
 

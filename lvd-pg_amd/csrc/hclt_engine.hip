@@ -460,18 +460,18 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
 }
 
 void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
-  if (timing) PCM_HIP(hipEventRecord(ev_[0], stream));
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
   PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_forward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
                                         stream, d, d_fwd_ptr_.p, d_fwd_items_.p, n_fwd_levels_, d_ll));
   check_launch("hclt_forward");
-  if (timing) PCM_HIP(hipEventRecord(ev_[1], stream));
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
 
 void HcltCircuit::run_backward(const HcltDev& d) {
   PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_backward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
                                         stream, d, d_bwd_ptr_.p, d_bwd_items_.p, n_bwd_levels_));
   check_launch("hclt_backward");
-  if (timing) PCM_HIP(hipEventRecord(ev_[2], stream));
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
@@ -497,12 +497,11 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
                        d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_floats);
   });
   check_launch("hclt_stats");
-  if (timing) PCM_HIP(hipEventRecord(ev_[3], stream));
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
 }
 
 void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (timing && !ev_[0]) for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
   stage_batch(b);
   run_forward(dev(b.batch), d_ll);
 }
@@ -510,17 +509,39 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (timing && !ev_[0]) for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
   stage_batch(b);
   HcltDev d = dev(b.batch);
   run_forward(d, d_ll);
   run_backward(d);
   run_stats(d, rate);
   have_flows_ = true;
-  if (timing) {
-    PCM_HIP(hipStreamSynchronize(stream));
-    for (int i = 0; i < 3; ++i) PCM_HIP(hipEventElapsedTime(&last_ms[i], ev_[i], ev_[i + 1]));
+  if (timing) ++n_timed_;
+}
+
+HcltCircuit::~HcltCircuit() {
+  for (hipEvent_t e : ev_) (void)hipEventDestroy(e);
+}
+
+hipEvent_t* HcltCircuit::ev_set() {
+  if (ev_.empty()) {
+    ev_.resize((size_t)kTimingRing * 4, nullptr);
+    for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
   }
+  return ev_.data() + (size_t)(n_timed_ % kTimingRing) * 4;
+}
+
+void HcltCircuit::read_timing(float* ms, int n) {
+  for (int i = 0; i < n; ++i) ms[i] = 0.f;
+  const int cnt = std::min(n_timed_, (int)kTimingRing);
+  if (cnt == 0) return;
+  PCM_HIP(hipStreamSynchronize(stream));
+  for (int s = 0; s < cnt; ++s)
+    for (int i = 0; i < std::min(n, 3); ++i) {
+      float t = 0.f;
+      PCM_HIP(hipEventElapsedTime(&t, ev_[(size_t)s * 4 + i], ev_[(size_t)s * 4 + i + 1]));
+      ms[i] += t / cnt;
+    }
+  n_timed_ = 0;
 }
 
 void HcltCircuit::em_update(float pseudocount, float inertia) {

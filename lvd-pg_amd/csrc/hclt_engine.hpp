@@ -38,7 +38,7 @@ struct HcltDev {
 class HcltCircuit : public pcm_circuit {
  public:
   HcltCircuit(const int32_t* parent, int V, int K, int C);
-  ~HcltCircuit() override {}
+  ~HcltCircuit() override;
 
   int64_t size(int what) const override;
   void index_table(int which, int64_t* out, int64_t n) const override;
@@ -59,10 +59,12 @@ class HcltCircuit : public pcm_circuit {
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 
-  // Kernel timing hooks for the benchmark: ms of the last forward / backward / statistics
-  // launches measured with events on the circuit's stream (0 if timing is off).
+  // Kernel timing: when on, pcm_flows brackets its forward / backward / statistics launches
+  // with events on the circuit's stream (no synchronisation); read_timing synchronises and
+  // averages the calls recorded since the previous read (at most kTimingRing of them).
+  static constexpr int kTimingRing = 64;
   bool timing = false;
-  float last_ms[4] = {0, 0, 0, 0};
+  void read_timing(float* ms, int n);
 
  private:
   int V_, K_, C_, n_inner_, root_;
@@ -86,7 +88,9 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int64_t> d_sum_param_src_;
   int cap_slices_ = 0;
   bool have_flows_ = false;
-  hipEvent_t ev_[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  std::vector<hipEvent_t> ev_;   // kTimingRing sets of 4 events
+  int n_timed_ = 0;
+  hipEvent_t* ev_set();
 
   void build_structure();
   void build_param_order();

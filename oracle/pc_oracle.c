@@ -29,6 +29,8 @@
 #define NODE_SUM 1
 #define NODE_MUL 2
 
+int orc_max_threads(void);
+
 #if defined(_OPENMP)
 #include <omp.h>
 #endif
@@ -106,38 +108,51 @@ void orc_backward(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
                   REAL* edge_aggr, int n_roots, const int32_t* root_ids,
                   const REAL* root_flow) {
   int n_edges = edge_ptr[n_nodes];
-  double* aggr = (double*)calloc((size_t)n_edges, sizeof(double));
-  memset(flows, 0, sizeof(REAL) * (size_t)n_nodes * B);
-  if (n_roots == 0) {
-    for (int b = 0; b < B; ++b) flows[(int64_t)(n_nodes - 1) * B + b] = 1;
-  } else {
-    for (int h = 0; h < n_roots; ++h)
-      for (int b = 0; b < B; ++b)
-        flows[(int64_t)root_ids[h] * B + b] = root_flow[(int64_t)h * B + b];
-  }
-  for (int n = n_nodes - 1; n >= 0; --n) {
-    if (type[n] == NODE_INPUT) continue;
-    int issum = type[n] == NODE_SUM;
-    for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
-      if (skip && skip[e]) continue;
-      double s = 0;
-      for (int b = 0; b < B; ++b) {
-        REAL ef = flows[(int64_t)n * B + b];
-        if (issum) {
-          REAL child = mars[(int64_t)prime[e] * B + b] + logp[e];
-          if (sub[e] >= 0) child += mars[(int64_t)sub[e] * B + b];
-          REAL d = child - mars[(int64_t)n * B + b];
-          ef = ef * (sizeof(REAL) == 4 ? (REAL)expf((float)d) : (REAL)exp((double)d));
+  int nthreads = orc_max_threads();
+  if (nthreads > B) nthreads = B;
+  double* aggr = (double*)calloc((size_t)n_edges * nthreads, sizeof(double));
+  /* examples are independent: each thread owns a contiguous range of them */
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+  for (int t = 0; t < nthreads; ++t) {
+    int b0 = (int)((int64_t)B * t / nthreads), b1 = (int)((int64_t)B * (t + 1) / nthreads);
+    double* my = aggr + (size_t)t * n_edges;
+    for (int n = 0; n < n_nodes; ++n)
+      for (int b = b0; b < b1; ++b) flows[(int64_t)n * B + b] = 0;
+    if (n_roots == 0) {
+      for (int b = b0; b < b1; ++b) flows[(int64_t)(n_nodes - 1) * B + b] = 1;
+    } else {
+      for (int h = 0; h < n_roots; ++h)
+        for (int b = b0; b < b1; ++b)
+          flows[(int64_t)root_ids[h] * B + b] = root_flow[(int64_t)h * B + b];
+    }
+    for (int n = n_nodes - 1; n >= 0; --n) {
+      if (type[n] == NODE_INPUT) continue;
+      int issum = type[n] == NODE_SUM;
+      for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
+        if (skip && skip[e]) continue;
+        double s = 0;
+        for (int b = b0; b < b1; ++b) {
+          REAL ef = flows[(int64_t)n * B + b];
+          if (issum) {
+            REAL child = mars[(int64_t)prime[e] * B + b] + logp[e];
+            if (sub[e] >= 0) child += mars[(int64_t)sub[e] * B + b];
+            REAL d = child - mars[(int64_t)n * B + b];
+            ef = ef * (sizeof(REAL) == 4 ? (REAL)expf((float)d) : (REAL)exp((double)d));
+          }
+          flows[(int64_t)prime[e] * B + b] += ef;
+          if (sub[e] >= 0) flows[(int64_t)sub[e] * B + b] += ef;
+          s += ef;
         }
-        flows[(int64_t)prime[e] * B + b] += ef;
-        if (sub[e] >= 0) flows[(int64_t)sub[e] * B + b] += ef;
-        s += ef;
+        my[e] += s;
       }
-      aggr[e] += s;
     }
   }
   if (edge_aggr)
-    for (int e = 0; e < n_edges; ++e) edge_aggr[e] += (REAL)aggr[e];
+    for (int e = 0; e < n_edges; ++e) {
+      double s = 0;
+      for (int t = 0; t < nthreads; ++t) s += aggr[(size_t)t * n_edges + e];
+      edge_aggr[e] += (REAL)s;
+    }
   free(aggr);
 }
 
