@@ -119,29 +119,246 @@ void HcltCircuit::build_structure() {
   d_child_inner_.upload(ci);
   d_child_leaf_.upload(cl);
 
-  // forward levels: by height (1..H); backward levels: by depth (0..D)
-  auto make_levels = [&](const std::vector<int32_t>& key, int& n_levels, DevBuf<int32_t>& dptr,
-                         DevBuf<int32_t>& ditems) {
-    int maxk = 0;
-    for (int n = 0; n < n_inner_; ++n) maxk = std::max(maxk, key[n]);
-    n_levels = maxk + 1;
-    std::vector<int32_t> ptr(n_levels + 1, 0), items(n_inner_);
-    for (int n = 0; n < n_inner_; ++n) ptr[key[n] + 1]++;
-    for (int l = 0; l < n_levels; ++l) ptr[l + 1] += ptr[l];
-    std::vector<int32_t> fill(ptr.begin(), ptr.end() - 1);
-    for (int n = 0; n < n_inner_; ++n) items[fill[key[n]]++] = n;
-    dptr.upload(ptr);
-    ditems.upload(items);
-  };
-  std::vector<int32_t> hk(n_inner_), dk(n_inner_);
+  build_schedules();
+}
+
+// Step schedules of the two tree walks.  Every step holds at most kWalkWaves nodes whose
+// dependencies were produced in earlier steps; among the ready nodes those with the longest
+// remaining chain go first (for unit-time tasks on a tree this greedy rule gives the fewest
+// steps).  The host also places every produced tile into one of the LDS slots, for as long
+// as a later step still reads it.
+void HcltCircuit::build_schedules() {
+  int dev_id = 0;
+  PCM_HIP(hipGetDevice(&dev_id));
+  PCM_HIP(hipDeviceGetAttribute(&max_lds_, hipDeviceAttributeMaxSharedMemoryPerBlock, dev_id));
+  const int tile_bytes = kSlice * K_ * (int)sizeof(float);
+  lds_slots_ = std::min(max_lds_ / tile_bytes, (1 << (31 - kSlotShift)) - 2);
+  if (lds_slots_ < 3) fail(PCM_ERR_UNSUPPORTED, "device offers %d bytes of LDS, a value tile needs %d", max_lds_, tile_bytes);
+  const int trash_slot = lds_slots_ - 1;          // idle waves and childless nodes write here
+  const int zero_tile = n_inner_, trash_tile = n_inner_ + 1;
+
+  std::vector<std::vector<int32_t>> ic(n_inner_), lc(n_inner_);
+  std::vector<int32_t> par(n_inner_, -1), hin(n_inner_, 0);   // hin: longest chain of inner nodes below
   for (int n = 0; n < n_inner_; ++n) {
-    hk[n] = height_[var_of_inner_[n]] - 1;
-    dk[n] = depth_[var_of_inner_[n]];
+    const int v = var_of_inner_[n];
+    if (parent_[v] >= 0) par[n] = inner_of_var_[parent_[v]];
+    for (int c : children_[v]) {
+      if (children_[c].empty()) lc[n].push_back(c);
+      else { ic[n].push_back(inner_of_var_[c]); hin[n] = std::max(hin[n], hin[inner_of_var_[c]] + 1); }
+    }
   }
-  make_levels(hk, n_fwd_levels_, d_fwd_ptr_, d_fwd_items_);
-  // compact the depth keys of inner nodes (a depth with only leaf tree nodes has no items,
-  // which is fine: an empty level costs one barrier)
-  make_levels(dk, n_bwd_levels_, d_bwd_ptr_, d_bwd_items_);
+  std::vector<uint32_t> ext;
+  auto fill_ops = [&](StepItem& it, PreItem& q, const std::vector<uint32_t>& ops) {
+    it.n_g = (int32_t)std::min<size_t>(ops.size(), kInlineOps);
+    for (int i = 0; i < kInlineOps; ++i) it.g[i] = i < it.n_g ? ops[i] : 0;
+    for (int i = 0; i < kPre; ++i) q.g[i] = i < (int)ops.size() ? ops[i] : (uint32_t)zero_tile;
+    it.ext_off = (int32_t)ext.size();
+    it.ext_cnt = 0;
+    if (ops.size() > (size_t)kPre) it.flags |= kItemOverflow;
+    if (ops.size() > (size_t)kInlineOps) {
+      it.ext_cnt = (int32_t)(ops.size() - kInlineOps);
+      ext.insert(ext.end(), ops.begin() + kInlineOps, ops.end());
+    }
+  };
+  auto blank = [&](int n) {
+    StepItem it;
+    std::memset(&it, 0, sizeof it);
+    it.node = n >= 0 ? n : trash_tile;
+    it.out_slot = trash_slot; it.in_slot = trash_slot; it.parent = n >= 0 ? par[n] : -1;
+    if (n >= 0) it.flags = (par[n] < 0 ? kItemRoot : 0) | (ic[n].empty() ? 0 : kItemHasInnerChild);
+    return it;
+  };
+  auto blank_pre = [&](int n) {
+    PreItem q;
+    std::memset(&q, 0, sizeof q);
+    q.node = n >= 0 ? n : zero_tile;
+    q.wnode = n >= 0 ? n : 0;
+    for (int i = 0; i < kPre; ++i) q.g[i] = (uint32_t)zero_tile;
+    return q;
+  };
+  const int dbg = getenv("PCM_DBG") ? atoi(getenv("PCM_DBG")) : 0;   // TEMP experiment knob
+  auto dbg_fix = [&](std::vector<PreItem>& pre) {
+    for (auto& q : pre) {
+      if (dbg & 1) for (int i = 0; i < kPre; ++i) q.g[i] = (uint32_t)zero_tile;
+      if (dbg & 2) q.wnode = 0;
+      if (dbg & 4) for (int i = 0; i < kPre; ++i) if (q.g[i] & kOpLeaf) q.g[i] = kOpLeaf | 0u;
+    }
+  };
+  // field rows [field][wave][stride] with 64 idle steps of padding (a chunk refill reads
+  // 64 steps starting anywhere below n_steps)
+  auto make_fields = [&](std::vector<StepItem>& sched, std::vector<PreItem>& pre, bool forward, int& stride,
+                         DevBuf<int32_t>& dst) {
+    dbg_fix(pre);
+    const int n_steps = (int)sched.size() / kWalkWaves;
+    for (int i = 0; i < 64 * kWalkWaves; ++i) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); }
+    stride = n_steps + 64;
+    std::vector<int32_t> f((size_t)kSchedFields * kWalkWaves * stride, 0);
+    for (int s = 0; s < stride; ++s)
+      for (int w = 0; w < kWalkWaves; ++w) {
+        const StepItem& it = sched[(size_t)s * kWalkWaves + w];
+        const PreItem& q = pre[(size_t)s * kWalkWaves + w];
+        auto put = [&](int field, int32_t v) { f[((size_t)field * kWalkWaves + w) * stride + s] = v; };
+        put(kFNode, q.node); put(kFWnode, q.wnode);
+        put(kFG0, (int32_t)q.g[0]); put(kFG1, (int32_t)q.g[1]); put(kFG2, (int32_t)q.g[2]);
+        put(kFStore, it.node); put(kFOutSlot, it.out_slot);
+        put(kFFlags, it.flags | (it.n_l << 8));
+        if (forward) { put(kFL0, (int32_t)it.l[0]); put(kFL1, (int32_t)it.l[1]); put(kFL2, (int32_t)it.l[2]); }
+        else { put(kFL0, it.in_slot); put(kFL1, it.parent < 0 ? 0 : it.parent); put(kFL2, 0); }
+      }
+    dst.upload(f);
+  };
+  auto depth_of = [&](int n) { return depth_[var_of_inner_[n]]; };
+
+  // ---- forward -----------------------------------------------------------------------
+  {
+    std::vector<int32_t> pending(n_inner_), slot(n_inner_, -1), free_slots;
+    for (int s = trash_slot - 1; s >= 0; --s) free_slots.push_back(s);
+    auto cmp = [&](int a, int b) {   // max-heap: deeper first, then lower id (post-order)
+      return depth_of(a) != depth_of(b) ? depth_of(a) < depth_of(b) : a > b;
+    };
+    std::vector<int32_t> ready;
+    for (int n = 0; n < n_inner_; ++n) { pending[n] = (int)ic[n].size(); if (!pending[n]) ready.push_back(n); }
+    std::make_heap(ready.begin(), ready.end(), cmp);
+    std::vector<StepItem> sched;
+    std::vector<PreItem> pre;
+    fwd_spill_ = false;
+    int done = 0;
+    while (done < n_inner_) {
+      // nodes whose flow tile needs an LDS slot wait while none is free (their turn comes
+      // when children of earlier nodes have drained); only if nothing else is ready does a
+      // tile go through HBM instead
+      std::vector<int32_t> step, deferred;
+      int slots_left = (int)free_slots.size();
+      while (!ready.empty() && (int)step.size() < kWalkWaves) {
+        std::pop_heap(ready.begin(), ready.end(), cmp);
+        const int n = ready.back();
+        ready.pop_back();
+        if (!ic[n].empty()) {
+          if (slots_left == 0) { deferred.push_back(n); continue; }
+          --slots_left;
+        }
+        step.push_back(n);
+      }
+      if (step.empty() && !deferred.empty()) { step.push_back(deferred.back()); deferred.pop_back(); }
+      for (int n : deferred) { ready.push_back(n); std::push_heap(ready.begin(), ready.end(), cmp); }
+      if (step.empty()) fail(PCM_ERR_SHAPE, "forward schedule stalled (tree is inconsistent)");
+      for (int w = 0; w < kWalkWaves; ++w) {
+        if (w >= (int)step.size()) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); continue; }
+        const int n = step[w];
+        StepItem it = blank(n);
+        PreItem q = blank_pre(n);
+        std::vector<uint32_t> ops;
+        ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
+        for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+        it.n_l = 0;
+        for (int c : ic[n]) {
+          if (it.n_l < kInlineLds) it.l[it.n_l++] = ((uint32_t)(slot[c] + 1) << kSlotShift) | (uint32_t)c;
+          else { ops.push_back((uint32_t)c); fwd_spill_ = true; }   // read back from HBM
+          if (slot[c] < 0) fwd_spill_ = true;
+        }
+        fill_ops(it, q, ops);
+        if (par[n] >= 0 && !free_slots.empty()) { slot[n] = free_slots.back(); free_slots.pop_back(); }
+        if (slot[n] >= 0) it.out_slot = slot[n];
+        sched.push_back(it);
+        pre.push_back(q);
+      }
+      for (int n : step) {
+        for (int c : ic[n]) if (slot[c] >= 0) free_slots.push_back(slot[c]);
+        if (par[n] >= 0 && --pending[par[n]] == 0) { ready.push_back(par[n]); std::push_heap(ready.begin(), ready.end(), cmp); }
+        ++done;
+      }
+    }
+    n_fwd_steps_ = (int)sched.size() / kWalkWaves;
+    make_fields(sched, pre, true, fwd_stride_, d_fwd_fields_);
+    d_fwd_sched_.upload(sched);
+  }
+  // ---- backward ----------------------------------------------------------------------
+  // Oldest-ready first (ties: longest chain below first): a parent's flow tile then leaves
+  // its LDS slot a few steps after it was produced, so the number of live tiles stays near
+  // the width of the tree instead of growing with every postponed short subtree.
+  {
+    std::vector<int32_t> remaining(n_inner_), slot(n_inner_, -1), ready_at(n_inner_, 0), free_slots;
+    for (int s = trash_slot - 1; s >= 0; --s) free_slots.push_back(s);
+    std::vector<int32_t> ready;
+    for (int n = 0; n < n_inner_; ++n) { remaining[n] = (int)ic[n].size(); if (par[n] < 0) ready.push_back(n); }
+    std::vector<StepItem> sched;
+    std::vector<PreItem> pre;
+    bwd_spill_ = false;
+    int done = 0, step_no = 0;
+    while (done < n_inner_) {
+      std::sort(ready.begin(), ready.end(), [&](int a, int b) {
+        if (ready_at[a] != ready_at[b]) return ready_at[a] < ready_at[b];
+        return hin[a] != hin[b] ? hin[a] > hin[b] : a > b;
+      });
+      // a node whose flow tile needs a slot waits while none is free; only if nothing else
+      // is ready does a tile go through HBM instead
+      std::vector<int32_t> step, rest;
+      int slots_left = (int)free_slots.size();
+      for (int n : ready) {
+        if ((int)step.size() < kWalkWaves && (ic[n].empty() || slots_left > 0)) {
+          step.push_back(n);
+          if (!ic[n].empty()) --slots_left;
+        } else {
+          rest.push_back(n);
+        }
+      }
+      if (step.empty()) {
+        if (rest.empty()) fail(PCM_ERR_SHAPE, "backward schedule stalled (tree is inconsistent)");
+        step.push_back(rest.front());
+        rest.erase(rest.begin());
+      }
+      ready.swap(rest);
+      for (int w = 0; w < kWalkWaves; ++w) {
+        if (w >= (int)step.size()) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); continue; }
+        const int n = step[w];
+        StepItem it = blank(n);
+        PreItem q = blank_pre(n);
+        std::vector<uint32_t> ops;
+        ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
+        for (int c : ic[n]) ops.push_back((uint32_t)c);
+        for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+        fill_ops(it, q, ops);
+        if (par[n] >= 0) it.in_slot = slot[par[n]];   // -1: the parent's tile went to HBM
+        if (!ic[n].empty()) {
+          if (!free_slots.empty()) { slot[n] = free_slots.back(); free_slots.pop_back(); it.out_slot = slot[n]; }
+          else { bwd_spill_ = true; it.flags |= kItemSpillOut; }
+        }
+        sched.push_back(it);
+        pre.push_back(q);
+      }
+      ++step_no;
+      for (int n : step) {
+        if (par[n] >= 0 && --remaining[par[n]] == 0 && slot[par[n]] >= 0) free_slots.push_back(slot[par[n]]);
+        for (int c : ic[n]) { ready.push_back(c); ready_at[c] = step_no; }
+        ++done;
+      }
+    }
+    n_bwd_steps_ = (int)sched.size() / kWalkWaves;
+    make_fields(sched, pre, false, bwd_stride_, d_bwd_fields_);
+    d_bwd_sched_.upload(sched);
+  }
+  // ---- statistics: the static operands of every node ------------------------------------
+  {
+    std::vector<StepItem> items;
+    for (int n = 0; n < n_inner_; ++n) {
+      StepItem it = blank(n);
+      PreItem q = blank_pre(n);
+      std::vector<uint32_t> ops;
+      ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
+      for (int c : ic[n]) ops.push_back((uint32_t)c);
+      for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+      fill_ops(it, q, ops);
+      for (int i = 0; i < kPre; ++i) it.g[i] = q.g[i];   // absent operands name the zero tile
+      items.push_back(it);
+    }
+    d_stat_items_.upload(items);
+  }
+  if (ext.empty()) ext.push_back(0);
+  d_ext_ops_.upload(ext);
+  if (getenv("PCM_VERBOSE"))
+    fprintf(stderr, "[pcmi355] hclt V=%d K=%d C=%d inner=%d: forward %d steps%s, backward %d steps%s, %d LDS slots\n",
+            V_, K_, C_, n_inner_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", n_bwd_steps_,
+            bwd_spill_ ? " (spills)" : "", lds_slots_);
 }
 
 // Numbering the reference would give this circuit.  Nodes are created in depth-first
@@ -422,8 +639,13 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
 void HcltCircuit::ensure_batch(int batch) {
   const int ns = ceil_div(batch, kSlice);
   if (ns <= cap_slices_) return;
-  d_O_.alloc((size_t)n_inner_ * ns * kSlice * K_);
-  d_G_.alloc((size_t)n_inner_ * ns * kSlice * K_);
+  // two extra tiles per slice: index n_inner is all zeros (absent operands read it),
+  // index n_inner + 1 receives the stores of idle waves
+  const size_t tile = (size_t)ns * kSlice * K_;
+  d_O_.alloc((size_t)(n_inner_ + 2) * tile);
+  d_R_.alloc((size_t)(n_inner_ + 2) * tile);
+  PCM_HIP(hipMemsetAsync(d_O_.p + (size_t)n_inner_ * tile, 0, 2 * tile * sizeof(float), stream));
+  if (bwd_spill_) d_G_.alloc((size_t)(n_inner_ + 2) * tile);
   d_xb_.alloc((size_t)V_ * ns * kSlice);
   cap_slices_ = ns;
 }
@@ -439,13 +661,18 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.Wb = d_Wb_.p;
   d.xb = d_xb_.p;
   d.O = d_O_.p;
+  d.R = d_R_.p;
   d.G = d_G_.p;
+  d.ext_ops = d_ext_ops_.p;
   d.B = batch;
   d.nslices = ceil_div(batch, kSlice);
   d.Bp = d.nslices * kSlice;
   d.C = C_;
   d.n_inner = n_inner_;
   d.V = V_;
+  d.dbg = getenv("PCM_DBG") ? atoi(getenv("PCM_DBG")) : 0;
+  d.leaf_stride = (uint32_t)C_ * K_ * 4;
+  d.tile_stride = (uint32_t)d.nslices * kSlice * K_ * 4;
   return d;
 }
 
@@ -461,40 +688,53 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
 
 void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
   if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
-  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_forward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
-                                        stream, d, d_fwd_ptr_.p, d_fwd_items_.p, n_fwd_levels_, d_ll));
+  const size_t lds = (size_t)lds_slots_ * kSlice * K_ * sizeof(float);
+  auto launch = [&](auto kernel) {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_fwd_fields_.p,
+                       fwd_stride_, d_fwd_sched_.p, n_fwd_steps_, d_ll);
+  };
+  PCM_DISPATCH_K(K_, {
+    if (fwd_spill_) launch(&hclt_forward_kernel<KK, true>); else launch(&hclt_forward_kernel<KK, false>);
+  });
   check_launch("hclt_forward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
 
 void HcltCircuit::run_backward(const HcltDev& d) {
-  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_backward_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), 0,
-                                        stream, d, d_bwd_ptr_.p, d_bwd_items_.p, n_bwd_levels_));
+  const size_t lds = (size_t)lds_slots_ * kSlice * K_ * sizeof(float);
+  auto launch = [&](auto kernel) {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_fields_.p,
+                       bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
+  };
+  PCM_DISPATCH_K(K_, {
+    if (bwd_spill_) launch(&hclt_backward_kernel<KK, true>); else launch(&hclt_backward_kernel<KK, false>);
+  });
   check_launch("hclt_backward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
-  int dev_id = 0, max_lds = 0;
-  PCM_HIP(hipGetDevice(&dev_id));
-  PCM_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev_id));
+  const int max_lds = max_lds_;
   const size_t hist = (size_t)C_ * (K_ + 1) * sizeof(float);
   const size_t amin = std::max(hist, (size_t)K_ * K_ * sizeof(float));
   int waves = kStatWaves;
-  auto pads_of = [&](int w) { return (size_t)w * 2 * kSlice * (K_ + 16) * sizeof(float); };
+  auto pads_of = [&](int w) { return (size_t)w * kSlice * (K_ + 16) * sizeof(float); };
   while (waves > 1 && pads_of(waves) + amin > (size_t)max_lds) waves /= 2;
   const size_t pads = pads_of(waves);
   if (pads + amin > (size_t)max_lds)
     fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", pads + amin, max_lds);
-  int nh = std::min(4, (int)(((size_t)max_lds - pads) / hist));
+  int nh = std::min(3, (int)(((size_t)max_lds - pads) / hist));
   size_t hist_floats = ((size_t)nh * C_ * (K_ + 1) + 3) & ~(size_t)3;
   hist_floats = std::max(hist_floats, (size_t)K_ * K_);
   const size_t lds = hist_floats * sizeof(float) + pads;
+  if (d.dbg & 64) d_leaf_flow_.zero(stream);
   PCM_DISPATCH_K(K_, {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(hclt_stats_kernel<KK>, dim3(n_inner_), dim3(waves * 64), lds, stream, d,
-                       d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_floats);
+                       d_stat_items_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_floats);
   });
   check_launch("hclt_stats");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));

@@ -11,6 +11,16 @@
 
 namespace pcm {
 
+constexpr int kSlice = 16;       // examples per tile
+constexpr int kWalkWaves = 16;   // waves per workgroup (= items per step) in the tree-walk kernels
+constexpr int kInlineOps = 4;    // static operands held in a step item
+constexpr int kInlineLds = 3;    // LDS-resident operands held in a step item
+constexpr uint32_t kOpLeaf = 0x80000000u;    // operand is a leaf-table row of variable id
+constexpr uint32_t kOpIdMask = 0x003fffffu;  // else: value tile of inner node id
+constexpr int kSlotShift = 22;               // LDS operand: (slot + 1) << kSlotShift | inner id
+constexpr int kItemRoot = 1, kItemHasInnerChild = 2, kItemOverflow = 4, kItemSpillOut = 8;
+constexpr int kPre = 3;          // static operand tiles a wave requests one step ahead
+
 struct HcltNode {     // one non-leaf tree node, device-resident
   int32_t var;        // its observed variable
   int32_t parent;     // inner id of the tree parent, -1 for the root
@@ -20,19 +30,57 @@ struct HcltNode {     // one non-leaf tree node, device-resident
   int32_t has_inner_child;
 };
 
+// What one wave does in one step of a tree walk (or, for the statistics kernel, what a
+// workgroup needs to know about its node).  64 bytes, read with scalar loads.
+struct StepItem {
+  int32_t node;       // inner id (tile index); idle waves get the trash tile
+  int32_t out_slot;   // LDS slot receiving the produced tile (trash slot if nobody reads it)
+  int32_t in_slot;    // backward: LDS slot of the parent's flow tile, -1: read it from HBM
+  int32_t parent;     // inner id of the tree parent
+  int32_t flags;      // kItemRoot | kItemHasInnerChild | kItemOverflow | kItemSpillOut
+  int32_t n_g, n_l;   // inline static operands / inline LDS operands
+  int32_t ext_off;    // static operands beyond the inline list: ext_ops[ext_off .. +ext_cnt)
+  int32_t ext_cnt;
+  uint32_t g[kInlineOps];   // static operands, most urgent first
+  uint32_t l[kInlineLds];   // forward: inner children as (slot + 1) << kSlotShift | inner id
+};
+static_assert(sizeof(StepItem) == 64, "StepItem is read as 16 dwords");
+
+// Field rows of a walk schedule (see SchedChunk in the kernels).  kFNode is the tile whose
+// value the item reads ahead (backward: its own O tile; idle: the zero tile), kFStore the
+// tile index it writes (idle: the trash tile).  kFL0..2: forward: the inner children's
+// (slot + 1) << kSlotShift | id; backward: kFL0 = LDS slot of the parent's flow tile (-1:
+// in HBM), kFL1 = inner id of the parent.  kFFlags = item flags | n_l << 8.
+enum { kFNode = 0, kFWnode, kFG0, kFG1, kFG2, kFStore, kFOutSlot, kFFlags, kFL0, kFL1, kFL2, kSchedFields };
+
+// What a wave has to request ahead for an item: its value tile / parameter block ids and
+// its first kPre static operands (absent ones name the zero tile).
+struct PreItem {
+  int32_t node;    // tile index of the item's own node (idle: the zero tile)
+  int32_t wnode;   // parameter block to fetch (idle: block 0)
+  uint32_t g[kPre];
+  int32_t pad[3];
+};
+static_assert(sizeof(PreItem) == 32, "PreItem is read as 8 dwords");
+
 // Everything the kernels need, passed by value.
 struct HcltDev {
   const HcltNode* nodes;
   const int32_t* child_inner;
   const int32_t* child_leaf;
+  const uint32_t* ext_ops;
   const float* leaf;      // [V][C][K] log-probabilities, hidden state fastest
   const float* logtheta;  // [n_inner][K][K]
   const float* Wf;        // exp(theta) laid out per MFMA operand, forward contraction
   const float* Wb;        // same values, operand layout of the backward contraction
   const uint8_t* xb;      // [V][Bp] batch categories, example fastest
   float* O;               // [n_inner][nslices][16*K] node values, tile-native layout
-  float* G;               // [n_inner][nslices][16*K] child flows, same layout
+  float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
+  float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   int32_t B, Bp, nslices, C, n_inner, V;
+  int32_t dbg;            // TEMP experiment knob
+  uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
+  uint32_t tile_stride;   // bytes per node in O / R / G (nslices*16*K*4)
 };
 
 class HcltCircuit : public pcm_circuit {
@@ -70,7 +118,8 @@ class HcltCircuit : public pcm_circuit {
   int V_, K_, C_, n_inner_, root_;
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;
   std::vector<std::vector<int32_t>> children_;
-  int n_fwd_levels_ = 0, n_bwd_levels_ = 0;
+  int n_fwd_steps_ = 0, n_bwd_steps_ = 0, lds_slots_ = 0, max_lds_ = 0;
+  bool fwd_spill_ = false, bwd_spill_ = false;
   // parameter-vector order (reference numbering, see build_param_order)
   std::vector<int64_t> sum_param_src_;   // param i -> index into logtheta [n_inner][K][K]
   std::vector<int32_t> sum_group_size_;  // sizes of the normalisation groups, in order
@@ -79,8 +128,12 @@ class HcltCircuit : public pcm_circuit {
   int64_t n_nodes_ = 0, n_edges_ = 0;
 
   DevBuf<HcltNode> d_nodes_;
-  DevBuf<int32_t> d_child_inner_, d_child_leaf_, d_fwd_ptr_, d_fwd_items_, d_bwd_ptr_, d_bwd_items_;
-  DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_G_;
+  DevBuf<int32_t> d_child_inner_, d_child_leaf_;
+  DevBuf<StepItem> d_fwd_sched_, d_bwd_sched_, d_stat_items_;
+  DevBuf<int32_t> d_fwd_fields_, d_bwd_fields_;
+  int fwd_stride_ = 0, bwd_stride_ = 0;
+  DevBuf<uint32_t> d_ext_ops_;
+  DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_R_, d_G_;
   DevBuf<uint8_t> d_xb_;
   DevBuf<float> d_leaf_kc_;      // [V][K][C] copy for sampling
   DevBuf<float> d_kld_;          // scratch of the KL recursion
@@ -93,6 +146,7 @@ class HcltCircuit : public pcm_circuit {
   hipEvent_t* ev_set();
 
   void build_structure();
+  void build_schedules();
   void build_param_order();
   void ensure_batch(int batch);
   HcltDev dev(int batch) const;

@@ -3,17 +3,20 @@
 // Work decomposition.  Examples are independent, tree nodes are not: a node's value needs
 // its children's values (forward) and its parent's flows (backward).  The forward and
 // backward kernels therefore give each workgroup ONE slice of 16 examples and let it walk
-// the whole tree, level by level, its waves taking the nodes of a level in turn and
-// meeting at a workgroup barrier -- no grid-wide synchronisation exists anywhere.  The
-// sufficient statistics (edge flows summed over the batch, leaf histograms) need the whole
-// batch per node instead, so a third kernel gives each workgroup one tree node and all
-// slices, recomputing the node's flows from the stored node values.
+// the whole tree in host-scheduled steps: in every step each of the 16 waves takes at most
+// one tree node whose dependencies were produced in earlier steps, and the waves meet at a
+// workgroup barrier -- no grid-wide synchronisation exists anywhere.  The tile a step
+// produces for later steps (a node's values going up, the flow handed to its children
+// going down) stays in LDS in a slot the host allocated; everything else a step needs is
+// static, so it is requested from HBM one step ahead.  The sufficient statistics (edge
+// flows summed over the batch, leaf histograms) need the whole batch per node instead, so
+// a third kernel gives each workgroup one tree node and all slices.
 //
 // Register tile.  A wave holds a [16 examples x K states] tile as K/16 float4 per lane:
 // lane = 16*g + b owns example b and states kt*16 + 4*g + i (kt < K/16, i < 4).  This is
 // both the B-operand layout and the accumulator layout of v_mfma_f32_16x16x4_f32 with the
 // parameter block as A-operand (rows = output states), so the output tile of one
-// contraction feeds the next one, and HBM, unchanged.  Tiles are stored as K/16 runs of
+// contraction feeds the next one, LDS and HBM unchanged.  Tiles are stored as K/16 runs of
 // 64 float4 (1 KiB, fully coalesced).
 #pragma once
 
@@ -25,9 +28,7 @@ namespace pcm {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kSlice = 16;       // examples per tile
-constexpr int kWalkWaves = 16;   // waves per workgroup in the tree-walk kernels
-constexpr int kStatWaves = 8;    // most waves per workgroup in the statistics kernel
+constexpr int kStatWaves = 8;    // most waves per workgroup in the statistics kernel (256 registers each)
 
 template <int K>
 struct Tile {
@@ -35,181 +36,430 @@ struct Tile {
 };
 
 template <int K>
-__device__ __forceinline__ void tile_load(const float* base, int node, int nslices, int slice,
-                                          int lane, Tile<K>& t) {
-  const v4f* p = reinterpret_cast<const v4f*>(base + ((size_t)node * nslices + slice) * (kSlice * K));
+__device__ __forceinline__ void tile_zero(Tile<K>& t) {
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = v4f{0.f, 0.f, 0.f, 0.f};
+}
+
+template <int K>
+__device__ __forceinline__ void tile_add(Tile<K>& a, const Tile<K>& b) {
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt) a.v[kt] += b.v[kt];
+}
+
+// Per-thread constants of the address arithmetic.  Every global access is "uniform 64-bit
+// base + 32-bit per-lane byte offset", so the per-lane cost is one or two integer adds.
+struct LaneOffs {
+  uint32_t tile;   // byte offset of this lane's first float4 inside a node's [nslices] tile row
+  uint32_t leaf;   // byte offset of this lane's first float4 inside a leaf-table row
+  int bcol;        // batch column of this lane's example
+};
+
+template <int K>
+__device__ __forceinline__ LaneOffs lane_offs(int slice, int lane) {
+  LaneOffs o;
+  o.tile = (uint32_t)slice * (kSlice * K * 4) + (uint32_t)lane * 16;
+  o.leaf = (uint32_t)(lane >> 4) * 16;
+  o.bcol = slice * kSlice + (lane & 15);
+  return o;
+}
+
+template <int K>
+__device__ __forceinline__ void tile_load(const float* base, int node, size_t node_stride_bytes,
+                                          uint32_t voff, Tile<K>& t) {
+  const char* p = reinterpret_cast<const char*>(base) + (size_t)node * node_stride_bytes;
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = *reinterpret_cast<const v4f*>(p + voff + kt * 1024);
+}
+
+template <int K>
+__device__ __forceinline__ void tile_store(float* base, int node, size_t node_stride_bytes, uint32_t voff,
+                                           const Tile<K>& t) {
+  char* p = reinterpret_cast<char*>(base) + (size_t)node * node_stride_bytes;
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt) *reinterpret_cast<v4f*>(p + voff + kt * 1024) = t.v[kt];
+}
+
+template <int K>
+__device__ __forceinline__ void lds_tile_load(const float* lds, int slot, int lane, Tile<K>& t) {
+  const v4f* p = reinterpret_cast<const v4f*>(lds + (size_t)slot * (kSlice * K));
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = p[kt * 64 + lane];
 }
 
 template <int K>
-__device__ __forceinline__ void tile_store(float* base, int node, int nslices, int slice, int lane,
-                                           const Tile<K>& t) {
-  v4f* p = reinterpret_cast<v4f*>(base + ((size_t)node * nslices + slice) * (kSlice * K));
+__device__ __forceinline__ void lds_tile_store(float* lds, int slot, int lane, const Tile<K>& t) {
+  v4f* p = reinterpret_cast<v4f*>(lds + (size_t)slot * (kSlice * K));
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt) p[kt * 64 + lane] = t.v[kt];
 }
 
-// Row of the leaf table for this lane's example: log p(x_b,var | hidden state).
-template <int K, bool kFirst>
-__device__ __forceinline__ void leaf_row(const HcltDev& d, int var, int bcol, int g, Tile<K>& z) {
-  int x = d.xb[(size_t)var * d.Bp + bcol];
-  const v4f* row = reinterpret_cast<const v4f*>(d.leaf + ((size_t)var * d.C + x) * K);
-#pragma unroll
-  for (int kt = 0; kt < K / 16; ++kt) {
-    v4f t = row[kt * 4 + g];
-    if (kFirst) z.v[kt] = t; else z.v[kt] += t;
-  }
+__device__ __forceinline__ int load_x(const HcltDev& d, int var, int bcol) {
+  return d.xb[(size_t)var * d.Bp + bcol];
 }
 
-// Z = own leaf row + leaf rows of leaf children + value tiles of inner children;
-// returns E = exp(Z - m) and the per-example maximum m.
+// One static operand of a step: a leaf-table row (needs the category x) or a value tile.
+// Branch-free: the same load instructions serve both kinds, only the address differs, so
+// the number of loads in flight at any point of a kernel is the same on every path.
 template <int K>
-__device__ __forceinline__ float gather_exp(const HcltDev& d, const HcltNode& nd, int slice,
-                                            int lane, Tile<K>& e) {
-  const int b = lane & 15, g = lane >> 4;
-  const int bcol = slice * kSlice + b;
-  leaf_row<K, true>(d, nd.var, bcol, g, e);
-  for (int c = 0; c < nd.lc_cnt; ++c) leaf_row<K, false>(d, d.child_leaf[nd.lc_off + c], bcol, g, e);
-  for (int c = 0; c < nd.ic_cnt; ++c) {
-    Tile<K> o;
-    tile_load<K>(d.O, d.child_inner[nd.ic_off + c], d.nslices, slice, lane, o);
+__device__ __forceinline__ void operand_load(const HcltDev& d, uint32_t op, int x, const LaneOffs& lo,
+                                             Tile<K>& t) {
+  const bool leaf = (op & kOpLeaf) != 0;
+  const uint32_t id = op & kOpIdMask;
+  const char* base = leaf ? reinterpret_cast<const char*>(d.leaf) + (size_t)id * d.leaf_stride
+                          : reinterpret_cast<const char*>(d.O) + (size_t)id * d.tile_stride;
+  const uint32_t voff = leaf ? (uint32_t)x * (K * 4) + lo.leaf : lo.tile;
+  const uint32_t step = leaf ? 64u : 1024u;
 #pragma unroll
-    for (int kt = 0; kt < K / 16; ++kt) e.v[kt] += o.v[kt];
-  }
+  for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = *reinterpret_cast<const v4f*>(base + (voff + kt * step));
+}
+
+// Category of this lane's example for a leaf-row operand (variable 0 for the others, whose
+// loads ignore it).
+__device__ __forceinline__ int operand_x(const HcltDev& d, uint32_t op, int bcol) {
+  const uint32_t var = (op & kOpLeaf) ? (op & kOpIdMask) : 0u;
+  const uint8_t* base = d.xb + (size_t)var * d.Bp;
+  return base[(uint32_t)bcol];
+}
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// Per-example maximum over the K states (the lanes b, b+16, b+32, b+48 share an example).
+template <int K>
+__device__ __forceinline__ float tile_rowmax(const Tile<K>& z) {
   float m = -INFINITY;
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) m = fmaxf(m, e.v[kt][i]);
+    for (int i = 0; i < 4; ++i) m = fmaxf(m, z.v[kt][i]);
   m = fmaxf(m, __shfl_xor(m, 16));
   m = fmaxf(m, __shfl_xor(m, 32));
-  if (m == -INFINITY) m = 0.f;
+  return m == -INFINITY ? 0.f : m;
+}
+
+template <int K>
+__device__ __forceinline__ void tile_exp_sub(Tile<K>& z, float m) {
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) e.v[kt][i] = __expf(e.v[kt][i] - m);
-  return m;
+    for (int i = 0; i < 4; ++i) z.v[kt][i] = __builtin_amdgcn_exp2f(fmaf(z.v[kt][i], kLog2e, -m * kLog2e));
 }
 
-// out[b, r] = sum_c W[r, c] * in[b, c] on the matrix cores; Wop is the node's block already
-// laid out as A-operands: float4 (row tile rt, column tile ct, lane) holds
-// W[rt*16 + lane%16][ct*16 + 4*(lane/16) + 0..3].
+// A node's parameter block as MFMA A-operands: float4 (row tile rt, column tile ct, lane)
+// holds W[rt*16 + lane%16][ct*16 + 4*(lane/16) + 0..3].
 template <int K>
-__device__ __forceinline__ void contract(const float* Wop, int lane, const Tile<K>& in, Tile<K>& out) {
+struct WTile {
+  v4f a[(K / 16) * (K / 16)];
+};
+
+template <int K>
+__device__ __forceinline__ void w_load(const float* Wop, int lane, WTile<K>& w) {
+  const v4f* p = reinterpret_cast<const v4f*>(Wop);
+#pragma unroll
+  for (int i = 0; i < (K / 16) * (K / 16); ++i) w.a[i] = p[i * 64 + lane];
+}
+
+// out[b, r] = sum_c W[r, c] * in[b, c] on the matrix cores.
+template <int K>
+__device__ __forceinline__ void contract(const WTile<K>& w, const Tile<K>& in, Tile<K>& out) {
   constexpr int KT = K / 16;
-  const v4f* w = reinterpret_cast<const v4f*>(Wop);
 #pragma unroll
   for (int rt = 0; rt < KT; ++rt) {
     v4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ct = 0; ct < KT; ++ct) {
-      v4f a = w[(rt * KT + ct) * 64 + lane];
+    for (int ct = 0; ct < KT; ++ct)
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[i], in.v[ct][i], acc, 0, 0, 0);
-    }
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w.a[rt * KT + ct][i], in.v[ct][i], acc, 0, 0, 0);
     out.v[rt] = acc;
   }
 }
 
-// ---- forward: O_v = m + log(E W^T) --------------------------------------------------
-template <int K>
-__global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
-    HcltDev d, const int32_t* __restrict__ level_ptr, const int32_t* __restrict__ items,
-    int n_levels, float* __restrict__ ll_out) {
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int slice = blockIdx.x;
-  for (int L = 0; L < n_levels; ++L) {
-    const int beg = level_ptr[L], end = level_ptr[L + 1];
-    for (int it = beg + wave; it < end; it += kWalkWaves) {
-      const int n = items[it];
-      const HcltNode nd = d.nodes[n];
-      Tile<K> e, s;
-      const float m = gather_exp<K>(d, nd, slice, lane, e);
-      contract<K>(d.Wf + (size_t)n * K * K, lane, e, s);
-#pragma unroll
-      for (int kt = 0; kt < K / 16; ++kt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) s.v[kt][i] = m + __logf(s.v[kt][i]);
-      tile_store<K>(d.O, n, d.nslices, slice, lane, s);
-      if (nd.is_root && lane < 16 && slice * kSlice + lane < d.B) ll_out[slice * kSlice + lane] = s.v[0][0];
-    }
+// Barrier that orders LDS only: HBM stores of a step keep draining behind it.  kFull is
+// used when some dependency tile had to go through HBM.
+template <bool kFull>
+__device__ __forceinline__ void step_barrier() {
+  if (kFull) {
     __syncthreads();
+  } else {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
   }
 }
 
-// Flows arriving at the node's K sum nodes divided by their values: R = F / S, S = exp(O - m).
+// Static operands beyond the kPre requested ahead (nodes with many children): fetched at
+// the point of use, with the stall that implies.
 template <int K>
-__device__ __forceinline__ void flow_ratio(const HcltDev& d, const HcltNode& nd, int n, int slice,
-                                           int lane, float m, Tile<K>& r) {
-  Tile<K> o;
-  tile_load<K>(d.O, n, d.nslices, slice, lane, o);
-  if (nd.is_root) {
-    const bool live = lane < 16 && slice * kSlice + lane < d.B;
+__device__ __forceinline__ void operands_extra(const HcltDev& d, const StepItem* __restrict__ it, int n_g,
+                                               int ext_off, int ext_cnt, const LaneOffs& lo, Tile<K>& z) {
+  const int bcol = lo.bcol;
+  for (int i = kPre; i < n_g; ++i) {
+    Tile<K> t;
+    const uint32_t op = it->g[i];
+    operand_load<K>(d, op, operand_x(d, op, bcol), lo, t);
+    tile_add<K>(z, t);
+  }
+  const uint32_t* ext = d.ext_ops + ext_off;
+  for (int i = 0; i < ext_cnt; ++i) {
+    Tile<K> t;
+    const uint32_t op = ext[i];
+    operand_load<K>(d, op, operand_x(d, op, bcol), lo, t);
+    tile_add<K>(z, t);
+  }
+}
+
+// What the statistics kernel keeps of its node's item in scalar registers.
+struct PreRegs {
+  int node, wnode;
+  uint32_t g0, g1, g2;
+};
+static_assert(kPre == 3, "PreRegs holds three operands");
+
+template <int K>
+__device__ __forceinline__ void pre_request_x(const HcltDev& d, const PreRegs& q, int bcol, int (&x)[kPre]) {
+  x[0] = operand_x(d, q.g0, bcol);
+  x[1] = operand_x(d, q.g1, bcol);
+  x[2] = operand_x(d, q.g2, bcol);
+}
+
+template <int K>
+__device__ __forceinline__ void pre_request_ops(const HcltDev& d, const PreRegs& q, const int (&x)[kPre],
+                                                const LaneOffs& lo, Tile<K> (&P)[kPre]) {
+  operand_load<K>(d, q.g0, x[0], lo, P[0]);
+  operand_load<K>(d, q.g1, x[1], lo, P[1]);
+  operand_load<K>(d, q.g2, x[2], lo, P[2]);
+}
+
+// The step schedule of a walk is stored field by field, one row of n_steps entries per wave
+// (kSchedFields rows per wave).  A wave keeps 64 consecutive steps of every field in
+// registers, one step per lane, and reads the entry of a step with v_readlane: the inner
+// loop does no scalar memory loads (whose latency a step is too short to hide).
+struct SchedChunk {
+  int v[kSchedFields];
+  int base;
+};
+
+__device__ __forceinline__ void sched_refill(const int32_t* __restrict__ fields, int stride, int wave, int lane,
+                                             int base, SchedChunk& c) {
 #pragma unroll
-    for (int kt = 0; kt < K / 16; ++kt) r.v[kt] = v4f{0.f, 0.f, 0.f, 0.f};
-    r.v[0][0] = live ? __expf(m - o.v[0][0]) : 0.f;
-  } else {
-    tile_load<K>(d.G, nd.parent, d.nslices, slice, lane, r);
+  for (int f = 0; f < kSchedFields; ++f) c.v[f] = fields[((size_t)f * kWalkWaves + wave) * stride + base + lane];
+  c.base = base;
+}
+
+__device__ __forceinline__ int sched_get(const SchedChunk& c, int field, int step) {
+  return __builtin_amdgcn_readlane(c.v[field], step - c.base);
+}
+
+__device__ __forceinline__ PreRegs sched_pre(const SchedChunk& c, int step) {
+  PreRegs q;
+  q.node = sched_get(c, kFNode, step);
+  q.wnode = sched_get(c, kFWnode, step);
+  q.g0 = (uint32_t)sched_get(c, kFG0, step);
+  q.g1 = (uint32_t)sched_get(c, kFG1, step);
+  q.g2 = (uint32_t)sched_get(c, kFG2, step);
+  return q;
+}
+
+// The walk kernels run a three-stage software pipeline over the steps.  At the top of
+// step s a wave (1) consumes what it requested during step s-1 -- the static operands and
+// parameter block of its item of step s and the categories for step s+1 --, (2) requests
+// the operands and parameters of step s+1 and the categories of step s+2, (3) computes
+// step s.  Every wave issues the same loads and stores in every step (an idle wave works
+// on the zero tile and writes to the trash tile), so the waits the compiler places count
+// exactly the requests that must have landed and never the ones just issued.
+//
+// ---- forward: O_v = m + log(E W^T), E = exp(Z - m) ------------------------------------
+// Static operands: the node's own leaf row and its leaf children's rows.  Dependencies:
+// the value tiles of its inner children, read from their LDS slots (kSpill: or from HBM).
+template <int K, bool kSpill>
+__global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
+    HcltDev d, const int32_t* __restrict__ fields, int stride, const StepItem* __restrict__ sched,
+    int n_steps, float* __restrict__ ll_out) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slice = blockIdx.x;
+  const LaneOffs lo = lane_offs<K>(slice, lane);
+  const int bcol = lo.bcol;
+
+  // prologue: the rows carry 64 idle steps past n_steps, so no index needs a guard
+  SchedChunk sc;
+  sched_refill(fields, stride, wave, lane, 0, sc);
+  Tile<K> P[kPre];
+  WTile<K> wn;
+  int xs[kPre];
+  {
+    const PreRegs q0 = sched_pre(sc, 0), q1 = sched_pre(sc, 1);
+    int x0[kPre];
+    pre_request_x<K>(d, q0, bcol, x0);
+    pre_request_ops<K>(d, q0, x0, lo, P);
+    w_load<K>(d.Wf + (size_t)q0.wnode * K * K, lane, wn);
+    pre_request_x<K>(d, q1, bcol, xs);
+  }
+  float ll = 0.f;
+
+  for (int s = 0; s < n_steps; ++s) {
+    if (s - sc.base >= 61) sched_refill(fields, stride, wave, lane, s, sc);
+    // (1) consume
+    Tile<K> z = P[0];
+#pragma unroll
+    for (int i = 1; i < kPre; ++i) tile_add<K>(z, P[i]);
+    const WTile<K> w = wn;
+    int xc[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) xc[i] = xs[i];
+    // (2) request
+    const PreRegs qa = sched_pre(sc, s + 1);
+    pre_request_ops<K>(d, qa, xc, lo, P);
+    w_load<K>(d.Wf + (size_t)qa.wnode * K * K, lane, wn);
+    const PreRegs qb = sched_pre(sc, s + 2);
+    pre_request_x<K>(d, qb, bcol, xs);
+    // (3) compute
+    const int node = sched_get(sc, kFStore, s), out_slot = sched_get(sc, kFOutSlot, s);
+    const int flags = sched_get(sc, kFFlags, s);
+    const int n_l = flags >> 8;
+    if (flags & kItemOverflow) {
+      const StepItem* itp = sched + (size_t)s * kWalkWaves + wave;
+      operands_extra<K>(d, itp, itp->n_g, itp->ext_off, itp->ext_cnt, lo, z);
+    }
+#pragma unroll
+    for (int c = 0; c < kInlineLds; ++c) {
+      if (c < n_l) {
+        const uint32_t l = (uint32_t)sched_get(sc, kFL0 + c, s);
+        const int slot = (int)(l >> kSlotShift) - 1;
+        Tile<K> t;
+        if (!kSpill || slot >= 0) lds_tile_load<K>(lds, slot, lane, t);
+        else tile_load<K>(d.O, (int)(l & kOpIdMask), d.tile_stride, lo.tile, t);
+        tile_add<K>(z, t);
+      }
+    }
+    const float m = tile_rowmax<K>(z);
+    tile_exp_sub<K>(z, m);
+    Tile<K> o;
+    contract<K>(w, z, o);
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) r.v[kt][i] = r.v[kt][i] * __expf(m - o.v[kt][i]);
+      for (int i = 0; i < 4; ++i) o.v[kt][i] = fmaf(__builtin_amdgcn_logf(o.v[kt][i]), kLn2, m);
+    tile_store<K>(d.O, node, d.tile_stride, lo.tile, o);
+    lds_tile_store<K>(lds, out_slot, lane, o);
+    if (flags & kItemRoot) ll = o.v[0][0];
+    step_barrier<kSpill>();
   }
+  if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
 }
 
-// ---- backward: G_v = E .* (R W), the flow every child of v (and v's own leaf) receives ---
-template <int K>
+// ---- backward: R_v = F_v / S_v, G_v = E_v .* (R_v W_v) ----------------------------------
+// Static operands: own leaf row, children's value tiles, leaf children's rows (-> E_v), and
+// the node's own value tile O_v (-> S_v = exp(O_v - m)).  Dependency: F_v = G_parent from
+// its LDS slot.  R_v goes to HBM for the statistics kernel, G_v to an LDS slot for the
+// children (kSpill: to HBM when no slot was free).
+template <int K, bool kSpill>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
-    HcltDev d, const int32_t* __restrict__ level_ptr, const int32_t* __restrict__ items,
-    int n_levels) {
+    HcltDev d, const int32_t* __restrict__ fields, int stride, const StepItem* __restrict__ sched,
+    int n_steps) {
+  extern __shared__ float lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slice = blockIdx.x;
-  for (int L = 0; L < n_levels; ++L) {
-    const int beg = level_ptr[L], end = level_ptr[L + 1];
-    for (int it = beg + wave; it < end; it += kWalkWaves) {
-      const int n = items[it];
-      const HcltNode nd = d.nodes[n];
-      if (!nd.has_inner_child) continue;   // nobody reads this node's G
-      Tile<K> e, r, t;
-      const float m = gather_exp<K>(d, nd, slice, lane, e);
-      flow_ratio<K>(d, nd, n, slice, lane, m, r);
-      contract<K>(d.Wb + (size_t)n * K * K, lane, r, t);
+  const LaneOffs lo = lane_offs<K>(slice, lane);
+  const int bcol = lo.bcol;
+
+  SchedChunk sc;
+  sched_refill(fields, stride, wave, lane, 0, sc);
+  Tile<K> P[kPre], ovn;
+  WTile<K> wn;
+  int xs[kPre];
+  {
+    const PreRegs q0 = sched_pre(sc, 0), q1 = sched_pre(sc, 1);
+    int x0[kPre];
+    pre_request_x<K>(d, q0, bcol, x0);
+    pre_request_ops<K>(d, q0, x0, lo, P);
+    tile_load<K>(d.O, q0.node, d.tile_stride, lo.tile, ovn);
+    w_load<K>(d.Wb + (size_t)q0.wnode * K * K, lane, wn);
+    pre_request_x<K>(d, q1, bcol, xs);
+  }
+
+  for (int s = 0; s < n_steps; ++s) {
+    if (s - sc.base >= 61) sched_refill(fields, stride, wave, lane, s, sc);
+    Tile<K> e = P[0];
 #pragma unroll
-      for (int kt = 0; kt < K / 16; ++kt) t.v[kt] *= e.v[kt];
-      tile_store<K>(d.G, n, d.nslices, slice, lane, t);
+    for (int i = 1; i < kPre; ++i) tile_add<K>(e, P[i]);
+    const Tile<K> ov = ovn;
+    const WTile<K> w = wn;
+    int xc[kPre];
+#pragma unroll
+    for (int i = 0; i < kPre; ++i) xc[i] = xs[i];
+    const PreRegs qa = sched_pre(sc, s + 1);
+    pre_request_ops<K>(d, qa, xc, lo, P);
+    tile_load<K>(d.O, qa.node, d.tile_stride, lo.tile, ovn);
+    w_load<K>(d.Wb + (size_t)qa.wnode * K * K, lane, wn);
+    const PreRegs qb = sched_pre(sc, s + 2);
+    pre_request_x<K>(d, qb, bcol, xs);
+
+    const int node = sched_get(sc, kFStore, s), out_slot = sched_get(sc, kFOutSlot, s);
+    const int in_slot = sched_get(sc, kFL0, s), flags = sched_get(sc, kFFlags, s);
+    if (flags & kItemOverflow) {
+      const StepItem* itp = sched + (size_t)s * kWalkWaves + wave;
+      operands_extra<K>(d, itp, itp->n_g, itp->ext_off, itp->ext_cnt, lo, e);
     }
-    __syncthreads();
+    const float m = tile_rowmax<K>(e);
+    tile_exp_sub<K>(e, m);
+    Tile<K> r, t;
+    if (!kSpill || in_slot >= 0) lds_tile_load<K>(lds, in_slot, lane, r);
+    else tile_load<K>(d.G, sched_get(sc, kFL1, s), d.tile_stride, lo.tile, r);
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) r.v[kt][i] *= __builtin_amdgcn_exp2f(fmaf(ov.v[kt][i], -kLog2e, m * kLog2e));
+    if (flags & kItemRoot) {   // flow 1 into the single root sum node of every live example
+      tile_zero<K>(r);
+      r.v[0][0] = (lane < 16 && bcol < d.B) ? __builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e) : 0.f;
+    }
+    tile_store<K>(d.R, node, d.tile_stride, lo.tile, r);
+    contract<K>(w, r, t);
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt) t.v[kt] *= e.v[kt];
+    lds_tile_store<K>(lds, out_slot, lane, t);
+    if (kSpill && (flags & kItemSpillOut)) tile_store<K>(d.G, node, d.tile_stride, lo.tile, t);
+    step_barrier<kSpill>();
   }
 }
 
 // ---- statistics: one workgroup per tree node, all slices ------------------------------
 //   edge_aggr[v][k][j] = rate*old + W[k][j] * sum_b R[b,k] E[b,j]
 //   leaf_flow[u][c][j] = rate*old + sum_b [x_b,u = c] G_v[b,j]   for u = v and v's leaf children
-// LDS: hist_floats floats holding nh histograms of C x (K+1), then per wave two [16][K+16]
-// transposition pads.
+// with G_v = E .* (R W) recomputed from R_v (stored by the backward kernel) and the node's
+// static operands.  Same request-ahead pipeline as the walks, over the wave's slices.
+// LDS: hist_floats floats holding nh histograms of C x (K+1), then per wave one
+// [16][K+16] transposition pad.
 template <int K>
 __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
-    HcltDev d, float* __restrict__ edge_aggr, float* __restrict__ leaf_flow, float rate, int nh,
-    int hist_floats) {
+    HcltDev d, const StepItem* __restrict__ items, float* __restrict__ edge_aggr,
+    float* __restrict__ leaf_flow, float rate, int nh, int hist_floats) {
   constexpr int KT = K / 16;
-  constexpr int LD = K + 16;   // row stride of the transposition pads: conflict-free column reads
+  constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
   extern __shared__ float smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = lane & 15, g = lane >> 4;
   const int nwaves = blockDim.x >> 6;
   const int n = blockIdx.x;
+  const StepItem* itp = items + n;
+  PreRegs q;
+  q.node = n; q.wnode = n; q.g0 = itp->g[0]; q.g1 = itp->g[1]; q.g2 = itp->g[2];
+  const int it_flags = itp->flags, it_ng = itp->n_g, it_eo = itp->ext_off, it_ec = itp->ext_cnt;
   const HcltNode nd = d.nodes[n];
   const int hist_sz = d.C * (K + 1);
   float* hist = smem;
-  float* Rl = smem + hist_floats + (size_t)wave * (2 * kSlice * LD);
-  float* El = Rl + kSlice * LD;
+  float* pad = smem + hist_floats + (size_t)wave * (kSlice * LD);
   const int nu = 1 + nd.lc_cnt;
+  const int last = d.nslices - 1;
 
+  WTile<K> w;
+  w_load<K>(d.Wb + (size_t)n * K * K, lane, w);
   v4f accA[KT][KT];
 #pragma unroll
   for (int a = 0; a < KT; ++a)
@@ -220,44 +470,89 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     const int nhere = min(nh, nu - u0);
     for (int i = threadIdx.x; i < nhere * hist_sz; i += blockDim.x) hist[i] = 0.f;
     __syncthreads();
-    for (int slice = wave; slice < d.nslices; slice += nwaves) {
-      Tile<K> e, r, t;
-      const float m = gather_exp<K>(d, nd, slice, lane, e);
-      flow_ratio<K>(d, nd, n, slice, lane, m, r);
-      contract<K>(d.Wb + (size_t)n * K * K, lane, r, t);
+
+    // prologue (slices past the end are clamped: harmless repeated loads)
+    Tile<K> P[kPre], rn;
+    int xs[kPre], xc[kPre];   // categories of the next-but-one / next slice (after the top: next / current)
+    {
+      const int sa = min(wave, last), sb = min(wave + nwaves, last);
+      const LaneOffs la = lane_offs<K>(sa, lane);
+      pre_request_x<K>(d, q, la.bcol, xc);
+      pre_request_ops<K>(d, q, xc, la, P);
+      tile_load<K>(d.R, n, d.tile_stride, la.tile, rn);
+      pre_request_x<K>(d, q, sb * kSlice + b, xs);
+    }
+    for (int s0 = wave; s0 < d.nslices; s0 += nwaves) {
+      const int s1 = min(s0 + nwaves, last), s2 = min(s0 + 2 * nwaves, last);
+      Tile<K> e = P[0];
+#pragma unroll
+      for (int i = 1; i < kPre; ++i) tile_add<K>(e, P[i]);
+      const Tile<K> r0 = rn;
+      int xh[kPre];   // categories of the slice computed now
+#pragma unroll
+      for (int i = 0; i < kPre; ++i) { xh[i] = xc[i]; xc[i] = xs[i]; }
+      const LaneOffs l1 = lane_offs<K>(s1, lane);
+      pre_request_ops<K>(d, q, xc, l1, P);
+      tile_load<K>(d.R, n, d.tile_stride, l1.tile, rn);
+      pre_request_x<K>(d, q, s2 * kSlice + b, xs);
+
+      if (it_flags & kItemOverflow) operands_extra<K>(d, itp, it_ng, it_eo, it_ec, lane_offs<K>(s0, lane), e);
+      const float m = tile_rowmax<K>(e);
+      tile_exp_sub<K>(e, m);
+      Tile<K> t;
+      if (!(d.dbg & 32)) contract<K>(w, r0, t); else t = r0;
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
-      const int bcol = slice * kSlice + b;
-      if (u0 == 0) {
-        // A += R^T E over the 16 examples of the tile (contraction over examples)
+      const int bcol = s0 * kSlice + b;
+      if (u0 == 0 && !(d.dbg & 16)) {
+        // A += R^T E over the 16 examples of the tile (contraction over examples): both
+        // operands go through the wave's pad to reach the [state][example] operand layout
+        float ra[4][KT];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) {
-          *reinterpret_cast<v4f*>(&Rl[b * LD + kt * 16 + 4 * g]) = r.v[kt];
-          *reinterpret_cast<v4f*>(&El[b * LD + kt * 16 + 4 * g]) = e.v[kt];
-        }
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = r0.v[kt];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt) ra[s][kt] = pad[(4 * s + g) * LD + kt * 16 + b];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = e.v[kt];
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-          float ra[KT], eb[KT];
+          float eb[KT];
 #pragma unroll
-          for (int kt = 0; kt < KT; ++kt) {
-            ra[kt] = Rl[(4 * s + g) * LD + kt * 16 + b];
-            eb[kt] = El[(4 * s + g) * LD + kt * 16 + b];
-          }
+          for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[(4 * s + g) * LD + jt * 16 + b];
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int jt = 0; jt < KT; ++jt)
-              accA[kt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[kt], eb[jt], accA[kt][jt], 0, 0, 0);
+              accA[kt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[s][kt], eb[jt], accA[kt][jt], 0, 0, 0);
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
-      if (bcol < d.B) {
+      if (bcol < d.B && !(d.dbg & 8)) {
         for (int h = 0; h < nhere; ++h) {
+          // operand position of histogram variable u0+h: 0 is the node's own row, leaf
+          // children follow the inner children; the first kPre categories are in registers
+          const int pos = (u0 + h == 0) ? 0 : nd.ic_cnt + u0 + h;
           const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
-          const int x = d.xb[(size_t)u * d.Bp + bcol];
+          const int x = pos == 0 ? xh[0] : pos == 1 ? xh[1] : pos == 2 ? xh[2] : load_x(d, u, bcol);
+          if (d.dbg & 64) {
+            float* grow = leaf_flow + ((size_t)u * d.C + x) * K;
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                __hip_atomic_fetch_add(&grow[kt * 16 + 4 * g + i], t.v[kt][i], __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+            continue;
+          }
           float* hrow = hist + (size_t)h * hist_sz + x * (K + 1);
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
@@ -269,7 +564,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
       }
     }
     __syncthreads();
-    for (int h = 0; h < nhere; ++h) {
+    for (int h = 0; h < nhere && !(d.dbg & 64); ++h) {
       const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
       float* dst = leaf_flow + (size_t)u * d.C * K;
       const float* src = hist + (size_t)h * hist_sz;
