@@ -716,25 +716,25 @@ void HcltCircuit::run_backward(const HcltDev& d) {
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
-  const int max_lds = max_lds_;
-  const size_t hist = (size_t)C_ * (K_ + 1) * sizeof(float);
-  const size_t amin = std::max(hist, (size_t)K_ * K_ * sizeof(float));
-  int waves = kStatWaves;
-  auto pads_of = [&](int w) { return (size_t)w * kSlice * (K_ + 16) * sizeof(float); };
-  while (waves > 1 && pads_of(waves) + amin > (size_t)max_lds) waves /= 2;
-  const size_t pads = pads_of(waves);
-  if (pads + amin > (size_t)max_lds)
-    fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", pads + amin, max_lds);
-  int nh = std::min(3, (int)(((size_t)max_lds - pads) / hist));
-  size_t hist_floats = ((size_t)nh * C_ * (K_ + 1) + 3) & ~(size_t)3;
-  hist_floats = std::max(hist_floats, (size_t)K_ * K_);
-  const size_t lds = hist_floats * sizeof(float) + pads;
-  if (d.dbg & 64) d_leaf_flow_.zero(stream);
+  // LDS layout of hclt_stats_kernel
+  const size_t hist = 2 * (size_t)C_ * (K_ + 1);                    // words per histogram (two limbs)
+  const size_t pads = (size_t)kStatWaves * kSlice * (K_ + 16);
+  auto hist_words = [&](int nh) { return std::max((((size_t)nh * hist + 3) & ~(size_t)3), (size_t)K_ * K_); };
+  int nh = 3;
+  while (nh > 1 && (hist_words(nh) + pads) * 4 > (size_t)max_lds_) --nh;
+  const size_t lds = (hist_words(nh) + pads) * 4;
+  if (lds > (size_t)max_lds_)
+    fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", lds, max_lds_);
+  // fixed-point split of the flows: limb sums over the padded batch must stay below 2^32
+  int bits = 0;
+  while ((1 << bits) < d.Bp) ++bits;
+  const int limb = std::min(24, 32 - bits);
+  if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   PCM_DISPATCH_K(K_, {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(hclt_stats_kernel<KK>, dim3(n_inner_), dim3(waves * 64), lds, stream, d,
-                       d_stat_items_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_floats);
+    hipLaunchKernelGGL(hclt_stats_kernel<KK>, dim3(n_inner_), dim3(kStatWaves * 64), lds, stream, d,
+                       d_stat_items_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb);
   });
   check_launch("hclt_stats");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));

@@ -28,7 +28,7 @@ namespace pcm {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kStatWaves = 8;    // most waves per workgroup in the statistics kernel (256 registers each)
+constexpr int kStatWaves = 12;   // waves per workgroup in the statistics kernel (168 registers each)
 
 template <int K>
 struct Tile {
@@ -432,15 +432,25 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
 //   edge_aggr[v][k][j] = rate*old + W[k][j] * sum_b R[b,k] E[b,j]
 //   leaf_flow[u][c][j] = rate*old + sum_b [x_b,u = c] G_v[b,j]   for u = v and v's leaf children
 // with G_v = E .* (R W) recomputed from R_v (stored by the backward kernel) and the node's
-// static operands.  Same request-ahead pipeline as the walks, over the wave's slices.
-// LDS: hist_floats floats holding nh histograms of C x (K+1), then per wave one
-// [16][K+16] transposition pad.
+// static operands; same request-ahead pipeline as the walks, over the wave's slices.
+//
+// Leaf histograms.  The scatter-add of every example's K flows into row x_b of a C x K table
+// is done with LDS atomics, but not floating-point ones: ds_add_f32 retires about one lane
+// per three cycles on this hardware, integer LDS atomics a whole wave in under ten.  Flows
+// are non-negative and at most 1, so each is added as a fixed-point number split into two
+// integer limbs of `limb` bits (hi + lo, 2*limb fractional bits in total); with
+// limb = 32 - ceil(log2(batch)) neither limb sum can overflow, and 2*limb >= 32 bits keep the
+// quantisation below fp32 rounding of the result.  The sum is also independent of the order
+// in which the waves arrive.
+//
+// LDS (32-bit words): [nh][2][C][K+1] limb histograms | [waves][16][K+16] transposition pads.
 template <int K>
 __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     HcltDev d, const StepItem* __restrict__ items, float* __restrict__ edge_aggr,
-    float* __restrict__ leaf_flow, float rate, int nh, int hist_floats) {
+    float* __restrict__ leaf_flow, float rate, int nh, int hist_words, int limb) {
   constexpr int KT = K / 16;
   constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
+  constexpr int HS = K + 1;    // row stride of a histogram: spreads equal states over banks
   extern __shared__ float smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -452,11 +462,12 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
   q.node = n; q.wnode = n; q.g0 = itp->g[0]; q.g1 = itp->g[1]; q.g2 = itp->g[2];
   const int it_flags = itp->flags, it_ng = itp->n_g, it_eo = itp->ext_off, it_ec = itp->ext_cnt;
   const HcltNode nd = d.nodes[n];
-  const int hist_sz = d.C * (K + 1);
-  float* hist = smem;
-  float* pad = smem + hist_floats + (size_t)wave * (kSlice * LD);
+  const int hist_sz = d.C * HS;                     // words per limb table
+  unsigned* hist = reinterpret_cast<unsigned*>(smem);
+  float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
   const int nu = 1 + nd.lc_cnt;
   const int last = d.nslices - 1;
+  const float hi_scale = __builtin_ldexpf(1.f, limb), lo_scale = hi_scale;
 
   WTile<K> w;
   w_load<K>(d.Wb + (size_t)n * K * K, lane, w);
@@ -468,7 +479,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
 
   for (int u0 = 0; u0 < nu; u0 += nh) {
     const int nhere = min(nh, nu - u0);
-    for (int i = threadIdx.x; i < nhere * hist_sz; i += blockDim.x) hist[i] = 0.f;
+    for (int i = threadIdx.x; i < nhere * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
     __syncthreads();
 
     // prologue (slices past the end are clamped: harmless repeated loads)
@@ -500,11 +511,11 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
       const float m = tile_rowmax<K>(e);
       tile_exp_sub<K>(e, m);
       Tile<K> t;
-      if (!(d.dbg & 32)) contract<K>(w, r0, t); else t = r0;
+      contract<K>(w, r0, t);
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
       const int bcol = s0 * kSlice + b;
-      if (u0 == 0 && !(d.dbg & 16)) {
+      if (u0 == 0) {
         // A += R^T E over the 16 examples of the tile (contraction over examples): both
         // operands go through the wave's pad to reach the [state][example] operand layout
         float ra[4][KT];
@@ -536,48 +547,55 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
-      if (bcol < d.B && !(d.dbg & 8)) {
+      if (bcol < d.B) {
+        // fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
+        unsigned hi[KT][4], lo[KT][4];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float v = fminf(fmaxf(t.v[kt][i], 0.f), 1.f) * hi_scale;
+            const float fl = floorf(v);
+            hi[kt][i] = (unsigned)fl;
+            lo[kt][i] = (unsigned)((v - fl) * lo_scale);
+          }
         for (int h = 0; h < nhere; ++h) {
           // operand position of histogram variable u0+h: 0 is the node's own row, leaf
           // children follow the inner children; the first kPre categories are in registers
           const int pos = (u0 + h == 0) ? 0 : nd.ic_cnt + u0 + h;
           const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
           const int x = pos == 0 ? xh[0] : pos == 1 ? xh[1] : pos == 2 ? xh[2] : load_x(d, u, bcol);
-          if (d.dbg & 64) {
-            float* grow = leaf_flow + ((size_t)u * d.C + x) * K;
-#pragma unroll
-            for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-              for (int i = 0; i < 4; ++i)
-                __hip_atomic_fetch_add(&grow[kt * 16 + 4 * g + i], t.v[kt][i], __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_WORKGROUP);
-            continue;
-          }
-          float* hrow = hist + (size_t)h * hist_sz + x * (K + 1);
+          unsigned* hrow = hist + (size_t)h * 2 * hist_sz + x * HS;
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              __hip_atomic_fetch_add(&hrow[kt * 16 + 4 * g + i], t.v[kt][i], __ATOMIC_RELAXED,
+            for (int i = 0; i < 4; ++i) {
+              __hip_atomic_fetch_add(&hrow[kt * 16 + 4 * g + i], hi[kt][i], __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_WORKGROUP);
+              __hip_atomic_fetch_add(&hrow[hist_sz + kt * 16 + 4 * g + i], lo[kt][i], __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
         }
       }
     }
     __syncthreads();
-    for (int h = 0; h < nhere && !(d.dbg & 64); ++h) {
+    const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+    for (int h = 0; h < nhere; ++h) {
       const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
       float* dst = leaf_flow + (size_t)u * d.C * K;
-      const float* src = hist + (size_t)h * hist_sz;
+      const unsigned* src = hist + (size_t)h * 2 * hist_sz;
       for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
         const int c = i / K, j = i % K;
+        const float val = (float)src[c * HS + j] * hi_inv + (float)src[hist_sz + c * HS + j] * lo_inv;
         const float old = rate != 0.f ? rate * dst[i] : 0.f;
-        dst[i] = old + src[c * (K + 1) + j];
+        dst[i] = old + val;
       }
     }
     __syncthreads();
   }
 
   // combine the waves' partial A through LDS, scale by W, write the node's block once
+  // (floating-point LDS atomics: K*K per wave per node, negligible)
   float* abuf = smem;
   for (int i = threadIdx.x; i < K * K; i += blockDim.x) abuf[i] = 0.f;
   __syncthreads();
