@@ -135,7 +135,6 @@ void HcltCircuit::build_schedules() {
   lds_slots_ = std::min(max_lds_ / tile_bytes, (1 << (31 - kSlotShift)) - 2);
   if (lds_slots_ < 3) fail(PCM_ERR_UNSUPPORTED, "device offers %d bytes of LDS, a value tile needs %d", max_lds_, tile_bytes);
   const int trash_slot = lds_slots_ - 1;          // idle waves and childless nodes write here
-  const int zero_tile = n_inner_, trash_tile = n_inner_ + 1;
 
   std::vector<std::vector<int32_t>> ic(n_inner_), lc(n_inner_);
   std::vector<int32_t> par(n_inner_, -1), hin(n_inner_, 0);   // hin: longest chain of inner nodes below
@@ -148,10 +147,16 @@ void HcltCircuit::build_schedules() {
     }
   }
   std::vector<uint32_t> ext;
+  // a leaf child's row operand: its category is byte 1 + i of the node's packed word (the
+  // word holds the first three leaf children; later ones only occur beyond the kPre
+  // requested-ahead operands, where the category is fetched on the spot)
+  auto leaf_child_op = [&](int var, size_t i) {
+    return kOpLeaf | (uint32_t)var | ((uint32_t)std::min<size_t>(i + 1, 3) << kXSelShift);
+  };
   auto fill_ops = [&](StepItem& it, PreItem& q, const std::vector<uint32_t>& ops) {
     it.n_g = (int32_t)std::min<size_t>(ops.size(), kInlineOps);
     for (int i = 0; i < kInlineOps; ++i) it.g[i] = i < it.n_g ? ops[i] : 0;
-    for (int i = 0; i < kPre; ++i) q.g[i] = i < (int)ops.size() ? ops[i] : (uint32_t)zero_tile;
+    for (int i = 0; i < kPre; ++i) q.g[i] = i < (int)ops.size() ? ops[i] : kOpNone;
     it.ext_off = (int32_t)ext.size();
     it.ext_cnt = 0;
     if (ops.size() > (size_t)kPre) it.flags |= kItemOverflow;
@@ -163,7 +168,7 @@ void HcltCircuit::build_schedules() {
   auto blank = [&](int n) {
     StepItem it;
     std::memset(&it, 0, sizeof it);
-    it.node = n >= 0 ? n : trash_tile;
+    it.node = n;
     it.out_slot = trash_slot; it.in_slot = trash_slot; it.parent = n >= 0 ? par[n] : -1;
     if (n >= 0) it.flags = (par[n] < 0 ? kItemRoot : 0) | (ic[n].empty() ? 0 : kItemHasInnerChild);
     return it;
@@ -171,15 +176,15 @@ void HcltCircuit::build_schedules() {
   auto blank_pre = [&](int n) {
     PreItem q;
     std::memset(&q, 0, sizeof q);
-    q.node = n >= 0 ? n : zero_tile;
-    q.wnode = n >= 0 ? n : 0;
-    for (int i = 0; i < kPre; ++i) q.g[i] = (uint32_t)zero_tile;
+    q.node = n;
+    q.wnode = n;
+    for (int i = 0; i < kPre; ++i) q.g[i] = kOpNone;
     return q;
   };
   const int dbg = getenv("PCM_DBG") ? atoi(getenv("PCM_DBG")) : 0;   // TEMP experiment knob
   auto dbg_fix = [&](std::vector<PreItem>& pre) {
     for (auto& q : pre) {
-      if (dbg & 1) for (int i = 0; i < kPre; ++i) q.g[i] = (uint32_t)zero_tile;
+      if (dbg & 1) for (int i = 0; i < kPre; ++i) q.g[i] = kOpNone;
       if (dbg & 2) q.wnode = 0;
       if (dbg & 4) for (int i = 0; i < kPre; ++i) if (q.g[i] & kOpLeaf) q.g[i] = kOpLeaf | 0u;
     }
@@ -249,7 +254,7 @@ void HcltCircuit::build_schedules() {
         PreItem q = blank_pre(n);
         std::vector<uint32_t> ops;
         ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
-        for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+        for (size_t i = 0; i < lc[n].size(); ++i) ops.push_back(leaf_child_op(lc[n][i], i));
         it.n_l = 0;
         for (int c : ic[n]) {
           if (it.n_l < kInlineLds) it.l[it.n_l++] = ((uint32_t)(slot[c] + 1) << kSlotShift) | (uint32_t)c;
@@ -316,7 +321,7 @@ void HcltCircuit::build_schedules() {
         std::vector<uint32_t> ops;
         ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
         for (int c : ic[n]) ops.push_back((uint32_t)c);
-        for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+        for (size_t i = 0; i < lc[n].size(); ++i) ops.push_back(leaf_child_op(lc[n][i], i));
         fill_ops(it, q, ops);
         if (par[n] >= 0) it.in_slot = slot[par[n]];   // -1: the parent's tile went to HBM
         if (!ic[n].empty()) {
@@ -346,7 +351,7 @@ void HcltCircuit::build_schedules() {
       std::vector<uint32_t> ops;
       ops.push_back(kOpLeaf | (uint32_t)var_of_inner_[n]);
       for (int c : ic[n]) ops.push_back((uint32_t)c);
-      for (int c : lc[n]) ops.push_back(kOpLeaf | (uint32_t)c);
+      for (size_t i = 0; i < lc[n].size(); ++i) ops.push_back(leaf_child_op(lc[n][i], i));
       fill_ops(it, q, ops);
       for (int i = 0; i < kPre; ++i) it.g[i] = q.g[i];   // absent operands name the zero tile
       items.push_back(it);
@@ -639,14 +644,12 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
 void HcltCircuit::ensure_batch(int batch) {
   const int ns = ceil_div(batch, kSlice);
   if (ns <= cap_slices_) return;
-  // two extra tiles per slice: index n_inner is all zeros (absent operands read it),
-  // index n_inner + 1 receives the stores of idle waves
   const size_t tile = (size_t)ns * kSlice * K_;
-  d_O_.alloc((size_t)(n_inner_ + 2) * tile);
-  d_R_.alloc((size_t)(n_inner_ + 2) * tile);
-  PCM_HIP(hipMemsetAsync(d_O_.p + (size_t)n_inner_ * tile, 0, 2 * tile * sizeof(float), stream));
-  if (bwd_spill_) d_G_.alloc((size_t)(n_inner_ + 2) * tile);
+  d_O_.alloc((size_t)n_inner_ * tile);
+  d_R_.alloc((size_t)n_inner_ * tile);
+  if (bwd_spill_) d_G_.alloc((size_t)n_inner_ * tile);
   d_xb_.alloc((size_t)V_ * ns * kSlice);
+  d_xn_.alloc((size_t)n_inner_ * ns * kSlice);
   cap_slices_ = ns;
 }
 
@@ -660,6 +663,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.Wf = d_Wf_.p;
   d.Wb = d_Wb_.p;
   d.xb = d_xb_.p;
+  d.xn = d_xn_.p;
   d.O = d_O_.p;
   d.R = d_R_.p;
   d.G = d_G_.p;
@@ -684,6 +688,9 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   hipLaunchKernelGGL(hclt_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
                      b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
   check_launch("stage_batch");
+  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
+                     d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
+  check_launch("pack_x");
 }
 
 void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {

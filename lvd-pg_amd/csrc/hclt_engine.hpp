@@ -17,6 +17,8 @@ constexpr int kInlineOps = 4;    // static operands held in a step item
 constexpr int kInlineLds = 3;    // LDS-resident operands held in a step item
 constexpr uint32_t kOpLeaf = 0x80000000u;    // operand is a leaf-table row of variable id
 constexpr uint32_t kOpIdMask = 0x003fffffu;  // else: value tile of inner node id
+constexpr uint32_t kOpNone = 0x40000000u;    // absent operand: reads as zeros
+constexpr int kXSelShift = 28;               // leaf operand: which byte of the packed categories (2 bits)
 constexpr int kSlotShift = 22;               // LDS operand: (slot + 1) << kSlotShift | inner id
 constexpr int kItemRoot = 1, kItemHasInnerChild = 2, kItemOverflow = 4, kItemSpillOut = 8;
 constexpr int kPre = 3;          // static operand tiles a wave requests one step ahead
@@ -74,6 +76,7 @@ struct HcltDev {
   const float* Wf;        // exp(theta) laid out per MFMA operand, forward contraction
   const float* Wb;        // same values, operand layout of the backward contraction
   const uint8_t* xb;      // [V][Bp] batch categories, example fastest
+  const uint32_t* xn;     // [n_inner][Bp] packed categories of a node's own variable and leaf children
   float* O;               // [n_inner][nslices][16*K] node values, tile-native layout
   float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
@@ -135,6 +138,7 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<uint32_t> d_ext_ops_;
   DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_R_, d_G_;
   DevBuf<uint8_t> d_xb_;
+  DevBuf<uint32_t> d_xn_;
   DevBuf<float> d_leaf_kc_;      // [V][K][C] copy for sampling
   DevBuf<float> d_kld_;          // scratch of the KL recursion
   DevBuf<uint8_t> d_state_;

@@ -64,20 +64,37 @@ __device__ __forceinline__ LaneOffs lane_offs(int slice, int lane) {
   return o;
 }
 
-template <int K>
-__device__ __forceinline__ void tile_load(const float* base, int node, size_t node_stride_bytes,
-                                          uint32_t voff, Tile<K>& t) {
-  const char* p = reinterpret_cast<const char*>(base) + (size_t)node * node_stride_bytes;
-#pragma unroll
-  for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = *reinterpret_cast<const v4f*>(p + voff + kt * 1024);
+// All HBM traffic of the hot kernels goes through raw buffer descriptors (uniform base +
+// size in scalar registers, 32-bit per-lane byte offset).  A descriptor of size 0 makes the
+// access a no-op that still counts as issued: loads return zeros, stores are dropped, and
+// nothing reaches the memory system.  That is how absent operands and idle waves are handled
+// without branches, which keeps the number of requests in flight the same on every path.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
 }
 
 template <int K>
-__device__ __forceinline__ void tile_store(float* base, int node, size_t node_stride_bytes, uint32_t voff,
-                                           const Tile<K>& t) {
-  char* p = reinterpret_cast<char*>(base) + (size_t)node * node_stride_bytes;
+__device__ __forceinline__ void tile_load(const float* base, int node, uint32_t node_stride_bytes,
+                                          uint32_t voff, Tile<K>& t) {
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<const char*>(base) + (size_t)max(node, 0) * node_stride_bytes,
+                                             node >= 0 ? node_stride_bytes : 0u);
+  const uint32_t v = node >= 0 ? voff : 0u, step = node >= 0 ? 1024u : 0u;
 #pragma unroll
-  for (int kt = 0; kt < K / 16; ++kt) *reinterpret_cast<v4f*>(p + voff + kt * 1024) = t.v[kt];
+  for (int kt = 0; kt < K / 16; ++kt)
+    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(v + kt * step), 0, 0));
+}
+
+template <int K>
+__device__ __forceinline__ void tile_store(float* base, int node, uint32_t node_stride_bytes, uint32_t voff,
+                                           const Tile<K>& t) {
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(reinterpret_cast<char*>(base) + (size_t)max(node, 0) * node_stride_bytes,
+                                             node >= 0 ? node_stride_bytes : 0u);
+  const uint32_t v = node >= 0 ? voff : 0u, step = node >= 0 ? 1024u : 0u;
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt)
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(v + kt * step), 0, 0);
 }
 
 template <int K>
@@ -98,28 +115,33 @@ __device__ __forceinline__ int load_x(const HcltDev& d, int var, int bcol) {
   return d.xb[(size_t)var * d.Bp + bcol];
 }
 
-// One static operand of a step: a leaf-table row (needs the category x) or a value tile.
-// Branch-free: the same load instructions serve both kinds, only the address differs, so
-// the number of loads in flight at any point of a kernel is the same on every path.
+// One static operand of a step: a leaf-table row (needs the category x), a value tile, or
+// nothing (kOpNone).  An absent operand is still requested -- the number of requests in
+// flight must not depend on the item -- but through an empty descriptor and with every lane
+// on the same address: such a request returns zeros and costs the memory pipeline a few
+// cycles instead of the ~17 of a real one.
 template <int K>
-__device__ __forceinline__ void operand_load(const HcltDev& d, uint32_t op, int x, const LaneOffs& lo,
+__device__ __forceinline__ void operand_load(const HcltDev& d, uint32_t op, uint32_t xpack, const LaneOffs& lo,
                                              Tile<K>& t) {
   const bool leaf = (op & kOpLeaf) != 0;
-  const uint32_t id = op & kOpIdMask;
+  const bool none = op == kOpNone;
+  const uint32_t id = none ? 0u : op & kOpIdMask;
   const char* base = leaf ? reinterpret_cast<const char*>(d.leaf) + (size_t)id * d.leaf_stride
                           : reinterpret_cast<const char*>(d.O) + (size_t)id * d.tile_stride;
-  const uint32_t voff = leaf ? (uint32_t)x * (K * 4) + lo.leaf : lo.tile;
-  const uint32_t step = leaf ? 64u : 1024u;
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(base, none ? 0u : leaf ? d.leaf_stride : d.tile_stride);
+  const uint32_t x = (xpack >> (((op >> kXSelShift) & 3u) * 8u)) & 0xffu;
+  const uint32_t voff = none ? 0u : leaf ? x * (K * 4) + lo.leaf : lo.tile;
+  const uint32_t step = none ? 0u : leaf ? 64u : 1024u;
 #pragma unroll
-  for (int kt = 0; kt < K / 16; ++kt) t.v[kt] = *reinterpret_cast<const v4f*>(base + (voff + kt * step));
+  for (int kt = 0; kt < K / 16; ++kt)
+    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * step), 0, 0));
 }
 
-// Category of this lane's example for a leaf-row operand (variable 0 for the others, whose
-// loads ignore it).
-__device__ __forceinline__ int operand_x(const HcltDev& d, uint32_t op, int bcol) {
-  const uint32_t var = (op & kOpLeaf) ? (op & kOpIdMask) : 0u;
-  const uint8_t* base = d.xb + (size_t)var * d.Bp;
-  return base[(uint32_t)bcol];
+// Categories of this lane's example for the leaf-row operands of a node, four bytes packed
+// into one word (byte i: the operand whose selector is i); one request per item.
+__device__ __forceinline__ uint32_t xpack_load(const HcltDev& d, int node, int bcol) {
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(d.xn + (size_t)max(node, 0) * d.Bp, node >= 0 ? (uint32_t)d.Bp * 4u : 0u);
+  return __builtin_amdgcn_raw_buffer_load_b32(r, node >= 0 ? bcol * 4 : 0, 0, 0);
 }
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -154,10 +176,12 @@ struct WTile {
 };
 
 template <int K>
-__device__ __forceinline__ void w_load(const float* Wop, int lane, WTile<K>& w) {
-  const v4f* p = reinterpret_cast<const v4f*>(Wop);
+__device__ __forceinline__ void w_load(const float* Wops, int node, int lane, WTile<K>& w) {
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(Wops + (size_t)max(node, 0) * K * K, node >= 0 ? K * K * 4u : 0u);
+  const int v = node >= 0 ? lane * 16 : 0, step = node >= 0 ? 1024 : 0;
 #pragma unroll
-  for (int i = 0; i < (K / 16) * (K / 16); ++i) w.a[i] = p[i * 64 + lane];
+  for (int i = 0; i < (K / 16) * (K / 16); ++i)
+    w.a[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, v + i * step, 0, 0));
 }
 
 // out[b, r] = sum_c W[r, c] * in[b, c] on the matrix cores.
@@ -198,14 +222,14 @@ __device__ __forceinline__ void operands_extra(const HcltDev& d, const StepItem*
   for (int i = kPre; i < n_g; ++i) {
     Tile<K> t;
     const uint32_t op = it->g[i];
-    operand_load<K>(d, op, operand_x(d, op, bcol), lo, t);
+    operand_load<K>(d, op & ~(3u << kXSelShift), (op & kOpLeaf) ? (uint32_t)load_x(d, (int)(op & kOpIdMask), bcol) : 0u, lo, t);
     tile_add<K>(z, t);
   }
   const uint32_t* ext = d.ext_ops + ext_off;
   for (int i = 0; i < ext_cnt; ++i) {
     Tile<K> t;
     const uint32_t op = ext[i];
-    operand_load<K>(d, op, operand_x(d, op, bcol), lo, t);
+    operand_load<K>(d, op & ~(3u << kXSelShift), (op & kOpLeaf) ? (uint32_t)load_x(d, (int)(op & kOpIdMask), bcol) : 0u, lo, t);
     tile_add<K>(z, t);
   }
 }
@@ -218,18 +242,11 @@ struct PreRegs {
 static_assert(kPre == 3, "PreRegs holds three operands");
 
 template <int K>
-__device__ __forceinline__ void pre_request_x(const HcltDev& d, const PreRegs& q, int bcol, int (&x)[kPre]) {
-  x[0] = operand_x(d, q.g0, bcol);
-  x[1] = operand_x(d, q.g1, bcol);
-  x[2] = operand_x(d, q.g2, bcol);
-}
-
-template <int K>
-__device__ __forceinline__ void pre_request_ops(const HcltDev& d, const PreRegs& q, const int (&x)[kPre],
+__device__ __forceinline__ void pre_request_ops(const HcltDev& d, const PreRegs& q, uint32_t xpack,
                                                 const LaneOffs& lo, Tile<K> (&P)[kPre]) {
-  operand_load<K>(d, q.g0, x[0], lo, P[0]);
-  operand_load<K>(d, q.g1, x[1], lo, P[1]);
-  operand_load<K>(d, q.g2, x[2], lo, P[2]);
+  operand_load<K>(d, q.g0, xpack, lo, P[0]);
+  operand_load<K>(d, q.g1, xpack, lo, P[1]);
+  operand_load<K>(d, q.g2, xpack, lo, P[2]);
 }
 
 // The step schedule of a walk is stored field by field, one row of n_steps entries per wave
@@ -266,9 +283,9 @@ __device__ __forceinline__ PreRegs sched_pre(const SchedChunk& c, int step) {
 // step s a wave (1) consumes what it requested during step s-1 -- the static operands and
 // parameter block of its item of step s and the categories for step s+1 --, (2) requests
 // the operands and parameters of step s+1 and the categories of step s+2, (3) computes
-// step s.  Every wave issues the same loads and stores in every step (an idle wave works
-// on the zero tile and writes to the trash tile), so the waits the compiler places count
-// exactly the requests that must have landed and never the ones just issued.
+// step s.  Every wave issues the same loads and stores in every step (an idle wave through
+// empty buffer descriptors), so the waits the compiler places count exactly the requests
+// that must have landed and never the ones just issued.
 //
 // ---- forward: O_v = m + log(E W^T), E = exp(Z - m) ------------------------------------
 // Static operands: the node's own leaf row and its leaf children's rows.  Dependencies:
@@ -289,14 +306,13 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
   sched_refill(fields, stride, wave, lane, 0, sc);
   Tile<K> P[kPre];
   WTile<K> wn;
-  int xs[kPre];
+  uint32_t xs;
   {
     const PreRegs q0 = sched_pre(sc, 0), q1 = sched_pre(sc, 1);
-    int x0[kPre];
-    pre_request_x<K>(d, q0, bcol, x0);
+    const uint32_t x0 = xpack_load(d, q0.wnode, bcol);
     pre_request_ops<K>(d, q0, x0, lo, P);
-    w_load<K>(d.Wf + (size_t)q0.wnode * K * K, lane, wn);
-    pre_request_x<K>(d, q1, bcol, xs);
+    w_load<K>(d.Wf, q0.wnode, lane, wn);
+    xs = xpack_load(d, q1.wnode, bcol);
   }
   float ll = 0.f;
 
@@ -307,15 +323,12 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
 #pragma unroll
     for (int i = 1; i < kPre; ++i) tile_add<K>(z, P[i]);
     const WTile<K> w = wn;
-    int xc[kPre];
-#pragma unroll
-    for (int i = 0; i < kPre; ++i) xc[i] = xs[i];
+    const uint32_t xc = xs;
     // (2) request
     const PreRegs qa = sched_pre(sc, s + 1);
     pre_request_ops<K>(d, qa, xc, lo, P);
-    w_load<K>(d.Wf + (size_t)qa.wnode * K * K, lane, wn);
-    const PreRegs qb = sched_pre(sc, s + 2);
-    pre_request_x<K>(d, qb, bcol, xs);
+    w_load<K>(d.Wf, qa.wnode, lane, wn);
+    xs = xpack_load(d, sched_get(sc, kFWnode, s + 2), bcol);
     // (3) compute
     const int node = sched_get(sc, kFStore, s), out_slot = sched_get(sc, kFOutSlot, s);
     const int flags = sched_get(sc, kFFlags, s);
@@ -371,15 +384,14 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
   sched_refill(fields, stride, wave, lane, 0, sc);
   Tile<K> P[kPre], ovn;
   WTile<K> wn;
-  int xs[kPre];
+  uint32_t xs;
   {
     const PreRegs q0 = sched_pre(sc, 0), q1 = sched_pre(sc, 1);
-    int x0[kPre];
-    pre_request_x<K>(d, q0, bcol, x0);
+    const uint32_t x0 = xpack_load(d, q0.wnode, bcol);
     pre_request_ops<K>(d, q0, x0, lo, P);
     tile_load<K>(d.O, q0.node, d.tile_stride, lo.tile, ovn);
-    w_load<K>(d.Wb + (size_t)q0.wnode * K * K, lane, wn);
-    pre_request_x<K>(d, q1, bcol, xs);
+    w_load<K>(d.Wb, q0.wnode, lane, wn);
+    xs = xpack_load(d, q1.wnode, bcol);
   }
 
   for (int s = 0; s < n_steps; ++s) {
@@ -389,15 +401,12 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
     for (int i = 1; i < kPre; ++i) tile_add<K>(e, P[i]);
     const Tile<K> ov = ovn;
     const WTile<K> w = wn;
-    int xc[kPre];
-#pragma unroll
-    for (int i = 0; i < kPre; ++i) xc[i] = xs[i];
+    const uint32_t xc = xs;
     const PreRegs qa = sched_pre(sc, s + 1);
     pre_request_ops<K>(d, qa, xc, lo, P);
     tile_load<K>(d.O, qa.node, d.tile_stride, lo.tile, ovn);
-    w_load<K>(d.Wb + (size_t)qa.wnode * K * K, lane, wn);
-    const PreRegs qb = sched_pre(sc, s + 2);
-    pre_request_x<K>(d, qb, bcol, xs);
+    w_load<K>(d.Wb, qa.wnode, lane, wn);
+    xs = xpack_load(d, sched_get(sc, kFWnode, s + 2), bcol);
 
     const int node = sched_get(sc, kFStore, s), out_slot = sched_get(sc, kFOutSlot, s);
     const int in_slot = sched_get(sc, kFL0, s), flags = sched_get(sc, kFFlags, s);
@@ -470,7 +479,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
   const float hi_scale = __builtin_ldexpf(1.f, limb), lo_scale = hi_scale;
 
   WTile<K> w;
-  w_load<K>(d.Wb + (size_t)n * K * K, lane, w);
+  w_load<K>(d.Wb, n, lane, w);
   v4f accA[KT][KT];
 #pragma unroll
   for (int a = 0; a < KT; ++a)
@@ -484,14 +493,14 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
 
     // prologue (slices past the end are clamped: harmless repeated loads)
     Tile<K> P[kPre], rn;
-    int xs[kPre], xc[kPre];   // categories of the next-but-one / next slice (after the top: next / current)
+    uint32_t xs, xc;   // packed categories of the next-but-one / next slice (after the top: next / current)
     {
       const int sa = min(wave, last), sb = min(wave + nwaves, last);
       const LaneOffs la = lane_offs<K>(sa, lane);
-      pre_request_x<K>(d, q, la.bcol, xc);
+      xc = xpack_load(d, n, la.bcol);
       pre_request_ops<K>(d, q, xc, la, P);
       tile_load<K>(d.R, n, d.tile_stride, la.tile, rn);
-      pre_request_x<K>(d, q, sb * kSlice + b, xs);
+      xs = xpack_load(d, n, sb * kSlice + b);
     }
     for (int s0 = wave; s0 < d.nslices; s0 += nwaves) {
       const int s1 = min(s0 + nwaves, last), s2 = min(s0 + 2 * nwaves, last);
@@ -499,13 +508,12 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
 #pragma unroll
       for (int i = 1; i < kPre; ++i) tile_add<K>(e, P[i]);
       const Tile<K> r0 = rn;
-      int xh[kPre];   // categories of the slice computed now
-#pragma unroll
-      for (int i = 0; i < kPre; ++i) { xh[i] = xc[i]; xc[i] = xs[i]; }
+      const uint32_t xh = xc;   // packed categories of the slice computed now
+      xc = xs;
       const LaneOffs l1 = lane_offs<K>(s1, lane);
       pre_request_ops<K>(d, q, xc, l1, P);
       tile_load<K>(d.R, n, d.tile_stride, l1.tile, rn);
-      pre_request_x<K>(d, q, s2 * kSlice + b, xs);
+      xs = xpack_load(d, n, s2 * kSlice + b);
 
       if (it_flags & kItemOverflow) operands_extra<K>(d, itp, it_ng, it_eo, it_ec, lane_offs<K>(s0, lane), e);
       const float m = tile_rowmax<K>(e);
@@ -560,11 +568,11 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
             lo[kt][i] = (unsigned)((v - fl) * lo_scale);
           }
         for (int h = 0; h < nhere; ++h) {
-          // operand position of histogram variable u0+h: 0 is the node's own row, leaf
-          // children follow the inner children; the first kPre categories are in registers
-          const int pos = (u0 + h == 0) ? 0 : nd.ic_cnt + u0 + h;
-          const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
-          const int x = pos == 0 ? xh[0] : pos == 1 ? xh[1] : pos == 2 ? xh[2] : load_x(d, u, bcol);
+          // histogram variable u0+h: 0 is the node's own variable, then its leaf children;
+          // the categories of the first four are in the packed word
+          const int sel = u0 + h;
+          const int u = sel == 0 ? nd.var : d.child_leaf[nd.lc_off + sel - 1];
+          const int x = sel < 4 ? (int)((xh >> (8 * sel)) & 0xffu) : load_x(d, u, bcol);
           unsigned* hrow = hist + (size_t)h * 2 * hist_sz + x * HS;
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
@@ -680,6 +688,20 @@ __global__ void hclt_leaf_update_kernel(float* __restrict__ leaf, const float* _
     const float newv = (1.f - inertia) * (fl[(size_t)c * K] + cat_pc) / node_flow;
     lp[(size_t)c * K] = logf(oldv + newv);
   }
+}
+
+// xn[node][example] = categories of the node's own variable (byte 0) and of its first three
+// leaf children (bytes 1..3), so that a wave fetches all of them with one request.
+__global__ void hclt_pack_x_kernel(const HcltNode* __restrict__ nodes, const int32_t* __restrict__ child_leaf,
+                                   const uint8_t* __restrict__ xb, int n_inner, int Bp,
+                                   uint32_t* __restrict__ xn) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  const int n = blockIdx.y;
+  if (b >= Bp) return;
+  const HcltNode nd = nodes[n];
+  uint32_t v = xb[(size_t)nd.var * Bp + b];
+  for (int i = 0; i < nd.lc_cnt && i < 3; ++i) v |= (uint32_t)xb[(size_t)child_leaf[nd.lc_off + i] * Bp + b] << (8 * (i + 1));
+  xn[(size_t)n * Bp + b] = v;
 }
 
 // Batch rows -> xb[var][example] (example fastest), through a 64 x 64 LDS tile.
