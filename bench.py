@@ -22,21 +22,21 @@ HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 
 def algorithmic_bytes(n_int, V, K, C, B):
     """Bytes the algorithm has to move per launch, per kernel.  A node-value or flow vector
-    is K*4 bytes per (tree node, example).  Forward writes each node's value vector once and
-    reads it once as a child (2 vectors).  Backward + statistics together need the value
-    vector as child and as parent, and the flow vector written once and read once (4
-    vectors); all of that is booked on the backward kernel, so the statistics kernel, which
-    re-reads three of those vectors, is credited only with the data, parameters and
-    accumulators it alone touches."""
+    is K*4 bytes per (tree node, example); the whole step needs six of them per tree node:
+    the value vector written and read as a child going up, read again as a child and as a
+    parent going down, the flow vector written once and read once.  They are booked where
+    this implementation's kernels touch them: forward 2 (value written, value read as a
+    child), backward 3 (value as child, value as parent, flow written), statistics 1 (flow
+    read).  Each kernel also reads the batch (V*B bytes), the sum parameters (4 bytes per
+    edge) and the leaf tables (4*V*K*C); statistics additionally writes both accumulators."""
     vec = K * 4 * B
     n_sum_edges = (n_int - 1) * K * K + K
     theta = 4 * n_sum_edges
     leaf = 4 * V * K * C
     fwd = n_int * 2 * vec + V * B + theta + leaf
-    bwd = n_int * 4 * vec + V * B + theta + leaf
-    stats = V * B + 2 * theta + 2 * leaf          # read params, write both accumulators
-    update = 2 * theta + 3 * leaf                 # read accumulators, read+write parameters
-    return dict(forward=fwd, backward=bwd, statistics=stats, update=update,
+    bwd = n_int * 3 * vec + V * B + theta + leaf
+    stats = n_int * 1 * vec + V * B + 2 * theta + 2 * leaf
+    return dict(forward=fwd, backward=bwd, statistics=stats,
                 step=n_int * 6 * vec + V * B + 3 * theta + 5 * leaf)
 
 
@@ -65,7 +65,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3_hclt3072_k32")
-    ap.add_argument("--cpu-sample", type=int, default=128)
+    ap.add_argument("--cpu-sample", type=int, default=4096)
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:

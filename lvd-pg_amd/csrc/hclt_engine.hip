@@ -797,8 +797,8 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
                                         dim3(128), 0, stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p,
                                         d_edge_aggr_.p, n_inner_, pseudocount, inertia));
   check_launch("theta_update");
-  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(ceil_div((int64_t)V_ * K_, 128)), dim3(128), 0, stream,
-                     d_leaf_.p, d_leaf_flow_.p, V_, C_, K_, pseudocount, inertia);
+  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
+                     pseudocount, inertia);
   check_launch("leaf_update");
 }
 

@@ -116,22 +116,25 @@ __device__ __forceinline__ int load_x(const HcltDev& d, int var, int bcol) {
 }
 
 // One static operand of a step: a leaf-table row (needs the category x), a value tile, or
-// nothing (kOpNone).  An absent operand is still requested -- the number of requests in
-// flight must not depend on the item -- but through an empty descriptor and with every lane
-// on the same address: such a request returns zeros and costs the memory pipeline a few
-// cycles instead of the ~17 of a real one.
+// nothing (kOpNone: zeros, no request).  Skipping a request is safe for the request-ahead
+// pipeline because everything issued AFTER the operands of a step (parameter block,
+// categories, stores) is issued unconditionally: waiting until only those remain in flight
+// always covers the operands, however many of them there were.
 template <int K>
 __device__ __forceinline__ void operand_load(const HcltDev& d, uint32_t op, uint32_t xpack, const LaneOffs& lo,
                                              Tile<K>& t) {
+  if (op == kOpNone) {
+    tile_zero<K>(t);
+    return;
+  }
   const bool leaf = (op & kOpLeaf) != 0;
-  const bool none = op == kOpNone;
-  const uint32_t id = none ? 0u : op & kOpIdMask;
+  const uint32_t id = op & kOpIdMask;
   const char* base = leaf ? reinterpret_cast<const char*>(d.leaf) + (size_t)id * d.leaf_stride
                           : reinterpret_cast<const char*>(d.O) + (size_t)id * d.tile_stride;
-  const __amdgpu_buffer_rsrc_t r = make_rsrc(base, none ? 0u : leaf ? d.leaf_stride : d.tile_stride);
+  const __amdgpu_buffer_rsrc_t r = make_rsrc(base, leaf ? d.leaf_stride : d.tile_stride);
   const uint32_t x = (xpack >> (((op >> kXSelShift) & 3u) * 8u)) & 0xffu;
-  const uint32_t voff = none ? 0u : leaf ? x * (K * 4) + lo.leaf : lo.tile;
-  const uint32_t step = none ? 0u : leaf ? 64u : 1024u;
+  const uint32_t voff = leaf ? x * (K * 4) + lo.leaf : lo.tile;
+  const uint32_t step = leaf ? 64u : 1024u;
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
     t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * step), 0, 0));
@@ -670,23 +673,30 @@ __global__ void hclt_theta_update_kernel(const HcltNode* __restrict__ nodes, flo
   }
 }
 
-// Leaf update, one thread per (variable, hidden state); categories are strided by K so
-// consecutive threads touch consecutive addresses.
-__global__ void hclt_leaf_update_kernel(float* __restrict__ leaf, const float* __restrict__ leaf_flow,
-                                        int V, int C, int K, float pseudocount, float inertia) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= V * K) return;
-  const int u = i / K, j = i % K;
-  float* lp = leaf + (size_t)u * C * K + j;
-  const float* fl = leaf_flow + (size_t)u * C * K + j;
-  float node_flow = 0.f;
-  for (int c = 0; c < C; ++c) node_flow += fl[(size_t)c * K];
-  node_flow += pseudocount;
+// Leaf update (the reference's per-input-node update with missing_flow = 0), one workgroup
+// per variable: thread (category group cg, hidden state j) first sums the flows of its
+// categories, the groups are combined through LDS, then every thread rewrites its
+// categories.  Consecutive threads touch consecutive addresses in both passes.
+__global__ __launch_bounds__(256) void hclt_leaf_update_kernel(float* __restrict__ leaf,
+                                                               const float* __restrict__ leaf_flow, int C, int K,
+                                                               float pseudocount, float inertia) {
+  __shared__ float part[256];
+  const int u = blockIdx.x;
+  const int j = threadIdx.x % K, cg = threadIdx.x / K, ncg = blockDim.x / K;
+  float* lp = leaf + (size_t)u * C * K;
+  const float* fl = leaf_flow + (size_t)u * C * K;
+  float s = 0.f;
+  for (int c = cg; c < C; c += ncg) s += fl[(size_t)c * K + j];
+  part[threadIdx.x] = s;
+  __syncthreads();
+  float node_flow = pseudocount;
+  for (int q = 0; q < ncg; ++q) node_flow += part[q * K + j];
   const float cat_pc = pseudocount / (float)C;
-  for (int c = 0; c < C; ++c) {
-    const float oldv = inertia * expf(lp[(size_t)c * K]);
-    const float newv = (1.f - inertia) * (fl[(size_t)c * K] + cat_pc) / node_flow;
-    lp[(size_t)c * K] = logf(oldv + newv);
+  for (int c = cg; c < C; c += ncg) {
+    const size_t i = (size_t)c * K + j;
+    const float oldv = inertia * expf(lp[i]);
+    const float newv = (1.f - inertia) * (fl[i] + cat_pc) / node_flow;
+    lp[i] = logf(oldv + newv);
   }
 }
 
