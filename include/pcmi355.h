@@ -57,8 +57,11 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
  * num_heads nodes are the heads and no fake root is needed).
  * node_type: 0 input, 1 sum, 2 product.  child_ptr[n..n+1] delimits node n's children in
  * child_idx; sum_logp is parallel to child_idx (ignored under products).  Input node n
- * reads variable input_var[n] and owns num_cats log-probabilities, given in creation order
- * in input_logp.
+ * reads variable input_var[n] (0-based) and owns num_cats log-probabilities; input_logp holds
+ * them for the input nodes in the order they appear in the description.  The compiled
+ * circuit numbers its nodes, edges and parameters as the reference's flattening does
+ * (depth-first from the root, children in order); nodes unreachable from the root or the
+ * heads are dropped.
  */
 int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
                        const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
@@ -76,14 +79,16 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
 /* `num_parameters(mbpc)`, `num_nodes`, `num_edges`, `num_input_params`
  * (src/bits_circuit.jl:119-131).  what: 0 parameters, 1 sum parameters, 2 nodes,
  * 3 edges, 4 input parameters, 5 variables, 6 categories, 7 hidden categories (0 if not an
- * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes. */
+ * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes,
+ * 12 heads (0 for a single-root circuit). */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.
  * which: 0 edge2param [edges], 1 param2edge [sum parameters], 2 param2group [sum
  * parameters], 3 pargroup_sizes [groups], 4 innode2ncumparam [input nodes],
  * 5 up-layer ends [layers], 6 edge parent ids, 7 edge prime ids, 8 edge sub ids (0: none)
- * [edges, up order].  n must equal the table length. */
+ * [edges, up order], 9 head node ids (`root_ids`, src-jl/multi_head_pc/bit_circuit.jl:38-51)
+ * [heads].  n must equal the table length. */
 int pcm_index_table(const pcm_circuit* c, int32_t which, int64_t* out, int64_t n);
 
 /* ---- parameters --------------------------------------------------------------- */
@@ -127,7 +132,10 @@ int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex,
  * (src/queries/flow.jl:228-234).  The circuit's edge_aggr and leaf flow accumulators are
  * first scaled by `rate` (0 clears them; src/regularization/reg_em.jl:276-284) and then
  * receive this batch.  d_head_mask (multi-head circuits only, else NULL) is
- * [num_heads][batch] and seeds the head flows (src-jl/multi_head_pc/flow.jl:141-176).
+ * [num_heads][batch] and seeds the head flows (src-jl/multi_head_pc/flow.jl:141-176);
+ * d_ll_out then receives `batch` floats, the mask-weighted mixture
+ * logsumexp_h(mars[head_h] + log mask_h) - log sum_h mask_h
+ * (src-jl/multi_head_pc/likelihood.jl:3-12).
  */
 int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
               const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask,

@@ -3,6 +3,7 @@
 
 #include "common.hpp"
 #include "hclt_engine.hpp"
+#include "sparse_engine.hpp"
 
 namespace {
 thread_local std::string g_last_error;
@@ -54,11 +55,15 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
   });
 }
 
-int pcm_circuit_create(int32_t, const uint8_t*, const int32_t*, const int32_t*, const float*, const int32_t*,
-                       const float*, int32_t, int32_t, int32_t, pcm_circuit** out) {
+int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
+                       const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
+                       const float* input_logp, int32_t num_vars, int32_t num_cats, int32_t num_heads,
+                       pcm_circuit** out) {
   return guarded([&] {
-    if (out) *out = nullptr;
-    pcm::fail(PCM_ERR_UNSUPPORTED, "pcm_circuit_create: general circuits are not built yet");
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    *out = nullptr;
+    *out = new pcm::SparseCircuit(pcm::flatten_dag(num_nodes, node_type, child_ptr, child_idx, sum_logp, input_var,
+                                                   input_logp, num_vars, num_cats, num_heads));
   });
 }
 
@@ -129,11 +134,19 @@ int pcm_em_step(pcm_circuit* c, const uint8_t* d_data, int64_t se, int64_t sv, c
   });
 }
 
-int pcm_get_node_values(pcm_circuit* c, float*, float*, int64_t) {
-  return guarded([&] { need(c); pcm::fail(PCM_ERR_UNSUPPORTED, "node values are kept only by general circuits"); });
+int pcm_get_node_values(pcm_circuit* c, float* mars, float* flows, int64_t n) {
+  return guarded([&] {
+    auto* s = dynamic_cast<pcm::SparseCircuit*>(need(c));
+    if (!s) pcm::fail(PCM_ERR_UNSUPPORTED, "node values are kept only by circuits from pcm_circuit_create");
+    s->get_node_values(mars, flows, n);
+  });
 }
-int pcm_get_aggregates(pcm_circuit* c, float*, int64_t, float*, int64_t) {
-  return guarded([&] { need(c); pcm::fail(PCM_ERR_UNSUPPORTED, "use pcm_hclt_get_flows on an HCLT circuit"); });
+int pcm_get_aggregates(pcm_circuit* c, float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf) {
+  return guarded([&] {
+    auto* s = dynamic_cast<pcm::SparseCircuit*>(need(c));
+    if (!s) pcm::fail(PCM_ERR_UNSUPPORTED, "use pcm_hclt_get_flows on an HCLT circuit");
+    s->get_aggregates(edge_aggr, n_edges, leaf_flow, n_leaf);
+  });
 }
 
 int pcm_kld(pcm_circuit* p, pcm_circuit* q, float* out) {

@@ -407,8 +407,11 @@ void HcltCircuit::build_param_order() {
         else if (sum_id[(size_t)c * K + f.j] < 0) st.push_back({c, f.j, 0, 0});
         continue;
       }
-      if (children_[v].size() > 1) mul_id[(size_t)v * K + f.j] = next++;
+      // a product of exactly two circuits stays an unnumbered (prime, sub) pair until the
+      // product above it (with leaf_v[j]) needs it as a node, i.e. after the leaf
+      if (children_[v].size() > 2) mul_id[(size_t)v * K + f.j] = next++;
       create_input(v, f.j);
+      if (children_[v].size() == 2) mul_id[(size_t)v * K + f.j] = next++;
       f.j++;
       f.c = 0;
       continue;
@@ -475,6 +478,42 @@ void HcltCircuit::build_param_order() {
   layer_ends_.push_back((int64_t)edge_parent_.size());
   n_edges_ = (int64_t)edge_parent_.size();
   d_sum_param_src_.upload(sum_param_src_);
+
+  // the same circuit in general form, for the queries that run on the general engine
+  flat_ = FlatCircuit();
+  flat_.num_vars = V_; flat_.num_cats = C_; flat_.num_heads = 0;
+  flat_.type.assign(n_nodes_, kInput);
+  flat_.layer.assign(n_nodes_, 0);
+  flat_.in_var.assign(n_nodes_, -1);
+  flat_.in_off.assign(n_nodes_, -1);
+  flat_.input_nodes.resize(input_order_.size());
+  for (size_t q = 0; q < input_order_.size(); ++q) {
+    const int v = input_order_[q] / K, j = input_order_[q] % K;
+    const int64_t id = in_id[(size_t)v * K + j];
+    flat_.input_nodes[q] = (int32_t)id;
+    flat_.in_var[id] = v;
+    flat_.in_off[id] = (int64_t)q * C_;
+  }
+  for (int n = 0; n < n_inner_; ++n) {
+    const int v = var_of_inner_[n];
+    for (int k = 0; k < K; ++k) {
+      if (mul_id[(size_t)v * K + k] >= 0) { flat_.type[mul_id[(size_t)v * K + k]] = kMul; flat_.layer[mul_id[(size_t)v * K + k]] = mlayer[v]; }
+      if (sum_id[(size_t)v * K + k] >= 0) { flat_.type[sum_id[(size_t)v * K + k]] = kSum; flat_.layer[sum_id[(size_t)v * K + k]] = vlayer[v]; }
+    }
+  }
+  flat_.leaf_logp.assign((size_t)V_ * K * C_, 0.f);
+  noise_slot_.assign(n_edges_, 0);
+  for (int64_t ed = 0; ed < n_edges_; ++ed) {
+    flat_.e_parent.push_back((int32_t)(edge_parent_[ed] - 1));
+    flat_.e_prime.push_back((int32_t)(edge_prime_[ed] - 1));
+    flat_.e_sub.push_back((int32_t)(edge_sub_[ed] - 1));
+    flat_.e_logp.push_back(0.f);
+    if (edge2param_[ed]) {
+      const int64_t src = sum_param_src_[edge2param_[ed] - 1];
+      noise_slot_[ed] = (int32_t)((src / ((int64_t)K * K)) * K + src % K);
+    }
+  }
+  flat_.finish();
 }
 
 int64_t HcltCircuit::size(int what) const {
@@ -491,6 +530,7 @@ int64_t HcltCircuit::size(int what) const {
     case 9: return (int64_t)layer_ends_.size();
     case 10: return (int64_t)sum_group_size_.size();
     case 11: return (int64_t)V_ * K_;
+    case 12: return 0;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -524,6 +564,7 @@ void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
     case 6: copy(edge_parent_); break;
     case 7: copy(edge_prime_); break;
     case 8: copy(edge_sub_); break;
+    case 9: copy(std::vector<int64_t>()); break;
     default: fail(PCM_ERR_ARG, "unknown index table %d", which);
   }
 }
@@ -552,6 +593,7 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
     PCM_HIP(hipStreamSynchronize(stream));
     rebuild_w();
   }
+  general_stale_ = true;
   if (leaf) {
     std::vector<float> t((size_t)V_ * C * K);
     for (int v = 0; v < V_; ++v)
@@ -637,6 +679,7 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
   PCM_HIP(hipMemcpyAsync(d_leaf_.p, lf.data(), lf.size() * sizeof(float), hipMemcpyHostToDevice, stream));
   PCM_HIP(hipStreamSynchronize(stream));
   rebuild_w();
+  general_stale_ = true;
 }
 
 // ---- batches ------------------------------------------------------------------------
@@ -685,7 +728,7 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
   ensure_batch(b.batch);
   const int Bp = ceil_div(b.batch, kSlice) * kSlice;
-  hipLaunchKernelGGL(hclt_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
+  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
                      b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
   check_launch("stage_batch");
   hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
@@ -800,6 +843,7 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
   hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
                      pseudocount, inertia);
   check_launch("leaf_update");
+  general_stale_ = true;
 }
 
 }  // namespace pcm

@@ -7,7 +7,10 @@
 // node values (and one of flows) per tree node and example.
 #pragma once
 
+#include <memory>
+
 #include "common.hpp"
+#include "sparse_engine.hpp"
 
 namespace pcm {
 
@@ -149,6 +152,12 @@ class HcltCircuit : public pcm_circuit {
   int n_timed_ = 0;
   hipEvent_t* ev_set();
 
+  FlatCircuit flat_;                       // the same circuit in general form (structure only)
+  std::vector<int32_t> noise_slot_;       // per up edge: column of the compact sampling noise
+  std::unique_ptr<SparseCircuit> general_; // built on first use by the KL / sampling / Adam queries
+  bool general_stale_ = true;
+  SparseCircuit* general();
+  void pull_from_general();
   void build_structure();
   void build_schedules();
   void build_param_order();

@@ -1,0 +1,848 @@
+// General engine: flattening of circuit DAGs and layered kernels for any circuit.
+#include "sparse_engine.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <numeric>
+
+#include "stage_kernel.hip.hpp"
+
+namespace pcm {
+
+static void check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+// ---------------------------------------------------------------------------------------
+// flattening
+// ---------------------------------------------------------------------------------------
+
+// Restates ProbabilisticCircuits.jl `BitsProbCircuit(pc)` (un-vendored; behaviour pinned by
+// the reference's test/bits_circuit_tests.jl:13-24, test/misc_tests.jl:39-62 and
+// test/queries/likelihood_tests.jl:24-37 on the 3-variable fixture): nodes are created in
+// depth-first post-order from the root, children in order; a node with a single child is
+// passed through; a product of exactly two plain nodes that has a single parent becomes a
+// (prime, sub) edge of that parent; other products pair their children up into edges;
+// up edges are grouped by layer (height), then by parent id.
+FlatCircuit flatten_dag(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
+                        const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
+                        const float* input_logp, int32_t num_vars, int32_t num_cats, int32_t num_heads) {
+  if (num_nodes < 1) fail(PCM_ERR_SHAPE, "circuit has no nodes");
+  if (!node_type || !child_ptr || !input_var || !input_logp) fail(PCM_ERR_ARG, "null description array");
+  if (num_cats < 1 || num_cats > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256, got %d", num_cats);
+  if (num_heads < 0 || num_heads > num_nodes) fail(PCM_ERR_SHAPE, "num_heads %d out of range", num_heads);
+  const int n_edges_in = child_ptr[num_nodes];
+  if (n_edges_in > 0 && (!child_idx || !sum_logp)) fail(PCM_ERR_ARG, "null child arrays");
+  std::vector<int64_t> in_rank(num_nodes, -1);
+  int64_t n_in = 0;
+  for (int n = 0; n < num_nodes; ++n) {
+    if (node_type[n] > kMul) fail(PCM_ERR_SHAPE, "node %d has unknown type %d", n, node_type[n]);
+    const int c0 = child_ptr[n], c1 = child_ptr[n + 1];
+    if (c1 < c0) fail(PCM_ERR_SHAPE, "child_ptr decreases at node %d", n);
+    if (node_type[n] == kInput) {
+      if (c1 != c0) fail(PCM_ERR_SHAPE, "input node %d has children", n);
+      if (input_var[n] < 0 || input_var[n] >= num_vars) fail(PCM_ERR_SHAPE, "input node %d reads variable %d", n, input_var[n]);
+      in_rank[n] = n_in++;
+    } else {
+      if (c1 == c0) fail(PCM_ERR_SHAPE, "inner node %d has no children", n);
+      for (int c = c0; c < c1; ++c)
+        if (child_idx[c] < 0 || child_idx[c] >= n) fail(PCM_ERR_SHAPE, "node %d: child %d is not an earlier node", n, child_idx[c]);
+    }
+  }
+  std::vector<int32_t> roots;
+  if (num_heads == 0) roots.push_back(num_nodes - 1);
+  else for (int h = 0; h < num_heads; ++h) roots.push_back(num_nodes - num_heads + h);
+
+  // parents of reachable nodes
+  std::vector<int32_t> nparents(num_nodes, 0);
+  {
+    std::vector<char> seen(num_nodes, 0);
+    std::vector<int32_t> st(roots.begin(), roots.end());
+    while (!st.empty()) {
+      int n = st.back(); st.pop_back();
+      if (seen[n]) continue;
+      seen[n] = 1;
+      for (int c = child_ptr[n]; c < child_ptr[n + 1]; ++c) { nparents[child_idx[c]]++; st.push_back(child_idx[c]); }
+    }
+  }
+
+  FlatCircuit fc;
+  fc.num_vars = num_vars; fc.num_cats = num_cats; fc.num_heads = num_heads;
+  struct Info { int kind = -1; int32_t a = -1, b = -1; };   // kind 0: node a; 1: element (a, b)
+  std::vector<Info> memo(num_nodes);
+  struct Edge { int32_t prime, sub; float logp; };
+  std::vector<std::vector<Edge>> edges;
+  auto new_node = [&](uint8_t t, int32_t var, int64_t off) {
+    fc.type.push_back(t); fc.in_var.push_back(var); fc.in_off.push_back(off);
+    edges.emplace_back();
+    return (int32_t)fc.type.size() - 1;
+  };
+  auto materialize = [&](Info& i) {
+    if (i.kind == 1) {
+      const int32_t id = new_node(kMul, -1, -1);
+      edges[id].push_back({i.a, i.b, 0.f});
+      i = Info{0, id, -1};
+    }
+    return i.a;
+  };
+  struct Frame { int32_t n, c; };
+  for (int32_t root : roots) {
+    std::vector<Frame> st;
+    st.push_back({root, child_ptr[root]});
+    while (!st.empty()) {
+      Frame& f = st.back();
+      const int n = f.n;
+      if (memo[n].kind >= 0) { st.pop_back(); continue; }
+      if (f.c < child_ptr[n + 1]) {
+        const int c = child_idx[f.c++];
+        if (memo[c].kind < 0) st.push_back({c, child_ptr[c]});
+        continue;
+      }
+      Info info;
+      const int c0 = child_ptr[n], c1 = child_ptr[n + 1];
+      if (node_type[n] == kInput) {
+        const int64_t off = (int64_t)fc.input_nodes.size() * num_cats;
+        const int32_t id = new_node(kInput, input_var[n], off);
+        fc.input_nodes.push_back(id);
+        fc.leaf_logp.insert(fc.leaf_logp.end(), input_logp + in_rank[n] * num_cats, input_logp + (in_rank[n] + 1) * num_cats);
+        info = Info{0, id, -1};
+      } else if (c1 - c0 == 1) {
+        info = memo[child_idx[c0]];
+      } else if (node_type[n] == kSum) {
+        std::vector<Edge> es;
+        for (int c = c0; c < c1; ++c) {
+          const Info& ci = memo[child_idx[c]];
+          es.push_back({ci.a, ci.kind == 1 ? ci.b : -1, sum_logp[c]});
+        }
+        const int32_t id = new_node(kSum, -1, -1);
+        edges[id] = es;
+        info = Info{0, id, -1};
+      } else {
+        std::vector<int32_t> ids;
+        for (int c = c0; c < c1; ++c) ids.push_back(materialize(memo[child_idx[c]]));
+        if (ids.size() == 2 && nparents[n] <= 1) {
+          info = Info{1, ids[0], ids[1]};
+        } else {
+          const int32_t id = new_node(kMul, -1, -1);
+          for (size_t q = 0; q < ids.size(); q += 2)
+            edges[id].push_back({ids[q], q + 1 < ids.size() ? ids[q + 1] : -1, 0.f});
+          info = Info{0, id, -1};
+        }
+      }
+      memo[n] = info;
+      st.pop_back();
+    }
+    fc.heads.push_back(materialize(memo[root]));
+  }
+  if (num_heads == 0) fc.heads.clear();
+
+  // layers and up-edge order
+  const int64_t nn = fc.n_nodes();
+  fc.layer.assign(nn, 0);
+  for (int64_t n = 0; n < nn; ++n)
+    for (const Edge& e : edges[n]) {
+      fc.layer[n] = std::max(fc.layer[n], fc.layer[e.prime] + 1);
+      if (e.sub >= 0) fc.layer[n] = std::max(fc.layer[n], fc.layer[e.sub] + 1);
+    }
+  std::vector<int32_t> parents;
+  for (int64_t n = 0; n < nn; ++n) if (!edges[n].empty()) parents.push_back((int32_t)n);
+  std::stable_sort(parents.begin(), parents.end(), [&](int32_t a, int32_t b) { return fc.layer[a] < fc.layer[b]; });
+  for (int32_t p : parents)
+    for (const Edge& e : edges[p]) {
+      fc.e_parent.push_back(p); fc.e_prime.push_back(e.prime); fc.e_sub.push_back(e.sub); fc.e_logp.push_back(e.logp);
+    }
+  fc.finish();
+  return fc;
+}
+
+void FlatCircuit::finish() {
+  const int64_t nn = n_nodes(), ne = n_edges();
+  node_e0.assign(nn, 0); node_e1.assign(nn, 0);
+  layer_ends.clear();
+  edge2param.assign(ne, 0); param2edge.clear(); param2group.clear(); pargroup_sizes.clear();
+  int64_t group = 0;
+  for (int64_t e = 0; e < ne; ++e) {
+    const int32_t p = e_parent[e];
+    const bool first = e == 0 || e_parent[e - 1] != p, last = e + 1 == ne || e_parent[e + 1] != p;
+    if (first) node_e0[p] = (int32_t)e;
+    if (last) node_e1[p] = (int32_t)e + 1;
+    if (e > 0 && layer[e_parent[e - 1]] != layer[p]) layer_ends.push_back(e);
+    if (type[p] == kSum) {
+      if (first) { ++group; pargroup_sizes.push_back(0); }
+      param2edge.push_back(e + 1);
+      edge2param[e] = (int64_t)param2edge.size();
+      param2group.push_back(group);
+      pargroup_sizes.back()++;
+    }
+  }
+  if (ne) layer_ends.push_back(ne);
+}
+
+// ---------------------------------------------------------------------------------------
+// kernels
+// ---------------------------------------------------------------------------------------
+
+struct SparseDev {
+  const uint8_t* type;
+  const int32_t* order;      // node ids sorted by layer
+  const int32_t *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_var, *in_ptr, *in_edge;
+  const int64_t* in_off;
+  const float* logp;
+  const float* leaf;
+  const uint8_t* xb;         // [V][Bp]
+  float* mars;               // [n_nodes][Bp]
+  float* flows;
+  int32_t B, Bp, C;
+};
+
+// ProbabilisticCircuits.jl logsumexp(x, y) as used by src/queries/likelihood.jl:101-102.
+__device__ __forceinline__ float lse2(float x, float y) {
+  if (isfinite(x) && isfinite(y)) return fmaxf(x, y) + log1pf(expf(-fabsf(x - y)));
+  return fmaxf(x, y);
+}
+
+// Forward, one layer: thread = (node of the layer, example).  Restates
+// src/regularization/reg_likelihood.jl:16-49 (inputs) and src/queries/likelihood.jl:29-48
+// (edges folded in up-edge order with pairwise logsumexp / +).
+__global__ void sparse_forward_kernel(SparseDev d, int n0) {
+  const int n = d.order[n0 + blockIdx.x];
+  const int b = blockIdx.y * blockDim.x + threadIdx.x;
+  if (b >= d.Bp) return;
+  float acc;
+  if (d.type[n] == kInput) {
+    acc = d.leaf[d.in_off[n] + d.xb[(size_t)d.in_var[n] * d.Bp + b]];
+  } else {
+    const bool issum = d.type[n] == kSum;
+    const int e0 = d.node_e0[n], e1 = d.node_e1[n];
+    acc = 0.f;
+    for (int e = e0; e < e1; ++e) {
+      float child = d.mars[(size_t)d.e_prime[e] * d.Bp + b];
+      const int s = d.e_sub[e];
+      if (s >= 0) child += d.mars[(size_t)s * d.Bp + b];
+      if (issum) child += d.logp[e];
+      acc = e == e0 ? child : issum ? lse2(acc, child) : acc + child;
+    }
+  }
+  d.mars[(size_t)n * d.Bp + b] = acc;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+  return v;
+}
+
+// Backward, one layer (top-down): thread = (node, example) adds up the flows of the node's
+// incoming edges, src/queries/flow.jl:49-60: edge_flow = flows[parent] (product edge) or
+// flows[parent] * exp(mars[prime] + logp (+ mars[sub]) - mars[parent]) (sum edge).  Each
+// edge's flow is summed over the batch where the node is the edge's prime (:73-81); input
+// nodes add their flow to the leaf counters (src/nodes/fixable_categorical_dist.jl:121-130).
+__global__ void sparse_backward_kernel(SparseDev d, int n0, const int32_t* __restrict__ seed_of,
+                                       const float* __restrict__ seed, float* __restrict__ edge_aggr,
+                                       float* __restrict__ leaf_flow) {
+  const int n = d.order[n0 + blockIdx.x];
+  const int b = blockIdx.y * blockDim.x + threadIdx.x;
+  const bool live = b < d.B;
+  const int bb = min(b, d.Bp - 1);
+  float acc = 0.f;
+  const int sd = seed_of[n];
+  if (sd >= 0) acc = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
+  for (int i = d.in_ptr[n]; i < d.in_ptr[n + 1]; ++i) {
+    const int ie = d.in_edge[i];
+    const int e = ie >> 1;
+    const int p = d.e_parent[e];
+    float ef = d.flows[(size_t)p * d.Bp + bb];
+    if (d.type[p] == kSum) {
+      float child = d.mars[(size_t)d.e_prime[e] * d.Bp + bb] + d.logp[e];
+      const int s = d.e_sub[e];
+      if (s >= 0) child += d.mars[(size_t)s * d.Bp + bb];
+      ef *= expf(child - d.mars[(size_t)p * d.Bp + bb]);
+    }
+    if (!live) ef = 0.f;
+    acc += ef;
+    if (!(ie & 1) && edge_aggr) {
+      const float tot = wave_sum(ef);
+      if ((threadIdx.x & 63) == 0) atomicAdd(&edge_aggr[e], tot);
+    }
+  }
+  if (b < d.Bp) d.flows[(size_t)n * d.Bp + b] = live ? acc : 0.f;
+  if (live && leaf_flow && d.type[n] == kInput)
+    atomicAdd(&leaf_flow[d.in_off[n] + d.xb[(size_t)d.in_var[n] * d.Bp + b]], acc);
+}
+
+__global__ void sparse_scale_kernel(float* p, int64_t n, float rate) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = rate != 0.f ? p[i] * rate : 0.f;
+}
+
+// EM update, one thread per node: add_pseudocount, aggr_node_flows, update_params
+// (src/pretrain/mini_batch_warmup.jl:4-17, :54-70 without the 1e-8 guards) and the leaf
+// update (src/nodes/fixable_categorical_dist.jl:223-248, missing_flow = 0).
+__global__ void sparse_update_kernel(SparseDev d, int n_nodes, float* __restrict__ logp, float* __restrict__ leaf,
+                                     float* __restrict__ edge_aggr, const float* __restrict__ leaf_flow,
+                                     float pseudocount, float inertia) {
+  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+  if (n >= n_nodes) return;
+  if (d.type[n] == kSum) {
+    const int e0 = d.node_e0[n], e1 = d.node_e1[n];
+    const float share = pseudocount / (float)(e1 - e0);
+    float tot = 0.f;
+    for (int e = e0; e < e1; ++e) { edge_aggr[e] += share; tot += edge_aggr[e]; }
+    if (e1 - e0 == 1) return;
+    for (int e = e0; e < e1; ++e)
+      logp[e] = logf(inertia * expf(logp[e]) + (1.f - inertia) * edge_aggr[e] / tot);
+  } else if (d.type[n] == kInput) {
+    float* lp = leaf + d.in_off[n];
+    const float* fl = leaf_flow + d.in_off[n];
+    float node_flow = 0.f;
+    for (int c = 0; c < d.C; ++c) node_flow += fl[c];
+    node_flow += pseudocount;
+    const float cat_pc = pseudocount / (float)d.C;
+    for (int c = 0; c < d.C; ++c)
+      lp[c] = logf(inertia * expf(lp[c]) + (1.f - inertia) * (fl[c] + cat_pc) / node_flow);
+  }
+}
+
+// KL recursion, one layer, one thread per node: src/queries/kld.jl:95-128 and the leaf term
+// of src/nodes/fixable_categorical_dist.jl:187-192 (log-parameter form).
+__global__ void sparse_kld_up_kernel(SparseDev d, int n0, int n1, const float* __restrict__ logp2,
+                                     const float* __restrict__ leaf2, float* __restrict__ klds,
+                                     float* __restrict__ edge_klds) {
+  const int i = n0 + blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n1) return;
+  const int n = d.order[i];
+  float acc = 0.f;
+  if (d.type[n] == kInput) {
+    for (int c = 0; c < d.C; ++c) {
+      const float a = d.leaf[d.in_off[n] + c], q = leaf2[d.in_off[n] + c];
+      acc += expf(a) * (a - q);
+    }
+  } else {
+    for (int e = d.node_e0[n]; e < d.node_e1[n]; ++e) {
+      float k = klds[d.e_prime[e]];
+      if (d.e_sub[e] >= 0) k += klds[d.e_sub[e]];
+      if (d.type[n] == kSum) k = expf(d.logp[e]) * (k + d.logp[e] - logp2[e]);
+      edge_klds[e] = k;
+      acc = e == d.node_e0[n] ? k : acc + k;
+    }
+  }
+  klds[n] = acc;
+}
+
+// Reverse pass of the KL recursion, node gradients of one layer (top-down):
+// src/queries/kld.jl:262-300: a child receives g_parent * exp(p1) over a sum edge,
+// g_parent over a product edge.
+__global__ void sparse_kld_down_kernel(SparseDev d, int n0, int n1, int root, float* __restrict__ grads) {
+  const int i = n0 + blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n1) return;
+  const int n = d.order[i];
+  float acc = n == root ? 1.f : 0.f;
+  for (int q = d.in_ptr[n]; q < d.in_ptr[n + 1]; ++q) {
+    const int e = d.in_edge[q] >> 1;
+    const int p = d.e_parent[e];
+    acc += grads[p] * (d.type[p] == kSum ? expf(d.logp[e]) : 1.f);
+  }
+  grads[n] = acc;
+}
+
+// Edge and leaf gradients, src/queries/kld.jl:271-272 and, written as the source has them,
+// src/nodes/fixable_categorical_dist.jl:219.
+__global__ void sparse_kld_edge_grad_kernel(SparseDev d, int64_t n_edges, const float* __restrict__ grads,
+                                            const float* __restrict__ edge_klds, float* __restrict__ g1,
+                                            float* __restrict__ g2) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n_edges) return;
+  const int p = d.e_parent[e];
+  if (d.type[p] == kSum) {
+    const float g = grads[p], p1 = expf(d.logp[e]);
+    g1[e] = g * (edge_klds[e] + p1);
+    g2[e] = -g * p1;
+  } else {
+    g1[e] = 0.f;
+    g2[e] = 0.f;
+  }
+}
+
+__global__ void sparse_kld_leaf_grad_kernel(SparseDev d, const int32_t* __restrict__ input_nodes, int n_inputs,
+                                            const float* __restrict__ leaf2, const float* __restrict__ grads,
+                                            float* __restrict__ g1, float* __restrict__ g2) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)n_inputs * d.C) return;
+  const int n = input_nodes[i / d.C];
+  const float g = grads[n], a = d.leaf[i], q = leaf2[i];
+  g1[i] = g * (a - q + 1.f);
+  g2[i] = g * expf(a - q);
+}
+
+// Gumbel-max sampling, one layer (top-down), thread = (node, example): a visited sum node
+// keeps the edge maximising logp + noise (first maximum wins), a visited product visits all
+// its edges, a visited input emits argmax_c(logp_c + noise_c).
+__global__ void sparse_sample_kernel(SparseDev d, int n0, const int32_t* __restrict__ noise_slot,
+                                     const int64_t* __restrict__ edge2param, int64_t noise_stride,
+                                     const float* __restrict__ node_noise, const float* __restrict__ leaf_noise,
+                                     int V, uint8_t* __restrict__ visit, uint8_t* __restrict__ out) {
+  const int n = d.order[n0 + blockIdx.x];
+  const int b = blockIdx.y * blockDim.x + threadIdx.x;
+  if (b >= d.B || !visit[(size_t)n * d.Bp + b]) return;
+  if (d.type[n] == kInput) {
+    const float* lp = d.leaf + d.in_off[n];
+    const float* g = leaf_noise + ((size_t)b * V + d.in_var[n]) * d.C;
+    int best = 0;
+    float bv = lp[0] + g[0];
+    for (int c = 1; c < d.C; ++c) {
+      const float v = lp[c] + g[c];
+      if (v > bv) { bv = v; best = c; }
+    }
+    out[(size_t)b * V + d.in_var[n]] = (uint8_t)best;
+  } else if (d.type[n] == kSum) {
+    const float* en = node_noise + (size_t)b * noise_stride;
+    const int e0 = d.node_e0[n], e1 = d.node_e1[n];
+    int best = e0;
+    float bv = -INFINITY;
+    for (int e = e0; e < e1; ++e) {
+      const int64_t slot = noise_slot ? noise_slot[e] : edge2param[e] - 1;
+      const float v = d.logp[e] + en[slot];
+      if (e == e0 || v > bv) { bv = v; best = e; }
+    }
+    visit[(size_t)d.e_prime[best] * d.Bp + b] = 1;
+    if (d.e_sub[best] >= 0) visit[(size_t)d.e_sub[best] * d.Bp + b] = 1;
+  } else {
+    for (int e = d.node_e0[n]; e < d.node_e1[n]; ++e) {
+      visit[(size_t)d.e_prime[e] * d.Bp + b] = 1;
+      if (d.e_sub[e] >= 0) visit[(size_t)d.e_sub[e] * d.Bp + b] = 1;
+    }
+  }
+}
+
+// Adam on the sum parameters: src/sgd/adam.jl:318-319 (moments), :63-76 (ascent step).
+__global__ void sparse_adam_kernel(int64_t n, const float* __restrict__ grad, float* __restrict__ params,
+                                   float* __restrict__ m, float* __restrict__ v, float lr, float b1, float b2,
+                                   float eps, float c1, float c2) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float g = grad[i];
+  m[i] = b1 * m[i] + (1.f - b1) * g;
+  v[i] = b2 * v[i] + (1.f - b2) * g * g;
+  params[i] += lr * ((m[i] / c1) / (sqrtf(v[i] / c2) + eps));
+}
+
+// Per-sum-node normalisation into the circuit: src/sgd/adam.jl:88-127.
+__global__ void sparse_normalize_kernel(int n_groups, const int32_t* __restrict__ group_ptr,
+                                        const int32_t* __restrict__ param2edge, const float* __restrict__ params,
+                                        float* __restrict__ logp) {
+  const int gi = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gi >= n_groups) return;
+  const int p0 = group_ptr[gi], p1 = group_ptr[gi + 1];
+  if (p1 - p0 == 1) return;
+  float s = 0.f;
+  for (int p = p0; p < p1; ++p) s += expf(params[p]);
+  const float l = logf(s);
+  for (int p = p0; p < p1; ++p) logp[param2edge[p]] = params[p] - l;
+}
+
+__global__ void sparse_fill_u8_kernel(uint8_t* p, int64_t n, uint8_t v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+__global__ void sparse_set_row_u8_kernel(uint8_t* p, int B, uint8_t v) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < B) p[i] = v;
+}
+
+__global__ void sparse_copy_rows_kernel(const float* __restrict__ mars, int Bp, int B, const int32_t* __restrict__ nodes,
+                                        int n_rows, float* __restrict__ out) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  const int r = blockIdx.y;
+  if (b < B && r < n_rows) out[(size_t)r * B + b] = mars[(size_t)nodes[r] * Bp + b];
+}
+
+// Mask-weighted mixture over the heads, src-jl/multi_head_pc/likelihood.jl:3-12:
+// ll = logsumexp_h(mars[head_h] + log mask[h]) - log sum_h mask[h], folded head by head
+// from -inf with the pairwise logsumexp.
+__global__ void sparse_head_mixture_kernel(const float* __restrict__ mars, int Bp, int B, const int32_t* __restrict__ heads,
+                                           int n_heads, const float* __restrict__ mask, float* __restrict__ out) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  float acc = -INFINITY, tot = 0.f;
+  for (int h = 0; h < n_heads; ++h) {
+    const float m = mask[(size_t)h * B + b];
+    acc = lse2(acc, mars[(size_t)heads[h] * Bp + b] + logf(m));
+    tot += m;
+  }
+  out[b] = acc - logf(tot);
+}
+
+// ---------------------------------------------------------------------------------------
+// host
+// ---------------------------------------------------------------------------------------
+
+SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
+  const int64_t nn = fc_.n_nodes(), ne = fc_.n_edges();
+  if (nn == 0) fail(PCM_ERR_SHAPE, "empty circuit");
+  // nodes by layer
+  std::vector<int32_t> order(nn);
+  std::iota(order.begin(), order.end(), 0);
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return fc_.layer[a] < fc_.layer[b]; });
+  n_layers_ = fc_.layer[order.back()] + 1;
+  layer_node0_.assign(n_layers_ + 1, 0);
+  for (int64_t i = 0; i < nn; ++i) layer_node0_[fc_.layer[order[i]] + 1]++;
+  for (int l = 0; l < n_layers_; ++l) layer_node0_[l + 1] += layer_node0_[l];
+  // incoming edges per node: entry = edge << 1 | as_sub
+  std::vector<int32_t> in_ptr(nn + 1, 0), in_edge;
+  for (int64_t e = 0; e < ne; ++e) { in_ptr[fc_.e_prime[e] + 1]++; if (fc_.e_sub[e] >= 0) in_ptr[fc_.e_sub[e] + 1]++; }
+  for (int64_t n = 0; n < nn; ++n) in_ptr[n + 1] += in_ptr[n];
+  in_edge.resize(in_ptr[nn]);
+  {
+    std::vector<int32_t> fill(in_ptr.begin(), in_ptr.end() - 1);
+    for (int64_t e = 0; e < ne; ++e) {
+      in_edge[fill[fc_.e_prime[e]]++] = (int32_t)(e << 1);
+      if (fc_.e_sub[e] >= 0) in_edge[fill[fc_.e_sub[e]]++] = (int32_t)(e << 1 | 1);
+    }
+  }
+  if (in_edge.empty()) in_edge.push_back(0);
+  d_type_.upload(fc_.type);
+  d_order_.upload(order);
+  d_node_e0_.upload(fc_.node_e0); d_node_e1_.upload(fc_.node_e1);
+  auto up = [&](DevBuf<int32_t>& dst, std::vector<int32_t> v) { if (v.empty()) v.push_back(0); dst.upload(v); };
+  up(d_e_parent_, fc_.e_parent); up(d_e_prime_, fc_.e_prime); up(d_e_sub_, fc_.e_sub);
+  d_in_var_.upload(fc_.in_var);
+  d_in_off_.upload(fc_.in_off);
+  { std::vector<float> lp = fc_.e_logp; if (lp.empty()) lp.push_back(0.f); d_logp_.upload(lp); }
+  d_leaf_.upload(fc_.leaf_logp);
+  d_in_ptr_.upload(in_ptr); d_in_edge_.upload(in_edge);
+  d_edge_aggr_.alloc(std::max<int64_t>(ne, 1)); d_edge_aggr_.zero();
+  d_leaf_flow_.alloc(fc_.leaf_logp.size()); d_leaf_flow_.zero();
+  // seed table: which root / head a node is (-1: none)
+  std::vector<int32_t> seed_of(nn, -1);
+  if (fc_.heads.empty()) seed_of[nn - 1] = 0;
+  else for (size_t h = 0; h < fc_.heads.size(); ++h) seed_of[fc_.heads[h]] = (int32_t)h;
+  d_heads_.upload(seed_of);
+  // normalisation groups over the sum parameters
+  std::vector<int32_t> gp(1, 0), p2e;
+  for (int64_t s : fc_.pargroup_sizes) gp.push_back(gp.back() + (int32_t)s);
+  for (int64_t e : fc_.param2edge) p2e.push_back((int32_t)(e - 1));
+  if (p2e.empty()) p2e.push_back(0);
+  d_group_ptr_.upload(gp);
+  d_param2edge_.upload(p2e);
+}
+
+int64_t SparseCircuit::size(int what) const {
+  switch (what) {
+    case 0: return (int64_t)fc_.param2edge.size() + (int64_t)fc_.leaf_logp.size();
+    case 1: return (int64_t)fc_.param2edge.size();
+    case 2: return fc_.n_nodes();
+    case 3: return fc_.n_edges();
+    case 4: return (int64_t)fc_.leaf_logp.size();
+    case 5: return fc_.num_vars;
+    case 6: return fc_.num_cats;
+    case 7: return 0;
+    case 8: return 0;
+    case 9: return (int64_t)fc_.layer_ends.size();
+    case 10: return (int64_t)fc_.pargroup_sizes.size();
+    case 11: return (int64_t)fc_.input_nodes.size();
+    case 12: return fc_.num_heads;
+    default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
+  }
+}
+
+void SparseCircuit::index_table(int which, int64_t* out, int64_t n) const {
+  auto copy = [&](const std::vector<int64_t>& v) {
+    if ((int64_t)v.size() != n) fail(PCM_ERR_ARG, "index table %d has %lld entries, caller gave %lld", which,
+                                     (long long)v.size(), (long long)n);
+    std::copy(v.begin(), v.end(), out);
+  };
+  auto plus1 = [&](const std::vector<int32_t>& v) { std::vector<int64_t> r(v.size()); for (size_t i = 0; i < v.size(); ++i) r[i] = v[i] + 1; return r; };
+  switch (which) {
+    case 0: copy(fc_.edge2param); break;
+    case 1: copy(fc_.param2edge); break;
+    case 2: copy(fc_.param2group); break;
+    case 3: copy(fc_.pargroup_sizes); break;
+    case 4: { std::vector<int64_t> c(fc_.input_nodes.size()); for (size_t i = 0; i < c.size(); ++i) c[i] = (int64_t)(i + 1) * fc_.num_cats; copy(c); break; }
+    case 5: copy(fc_.layer_ends); break;
+    case 6: copy(plus1(fc_.e_parent)); break;
+    case 7: copy(plus1(fc_.e_prime)); break;
+    case 8: copy(plus1(fc_.e_sub)); break;
+    case 9: copy(plus1(fc_.heads)); break;
+    default: fail(PCM_ERR_ARG, "unknown index table %d", which);
+  }
+}
+
+static void fetch(std::vector<float>& h, const float* d, size_t n, hipStream_t s) {
+  h.resize(n);
+  if (!n) return;
+  PCM_HIP(hipMemcpyAsync(h.data(), d, n * sizeof(float), hipMemcpyDeviceToHost, s));
+  PCM_HIP(hipStreamSynchronize(s));
+}
+
+void SparseCircuit::vectorize(float* out, int64_t n) {
+  if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n, (long long)size(0));
+  std::vector<float> lp, lf;
+  fetch(lp, d_logp_.p, fc_.n_edges(), stream);
+  fetch(lf, d_leaf_.p, fc_.leaf_logp.size(), stream);
+  const size_t ns = fc_.param2edge.size();
+  for (size_t i = 0; i < ns; ++i) out[i] = lp[fc_.param2edge[i] - 1];
+  std::copy(lf.begin(), lf.end(), out + ns);
+}
+
+void SparseCircuit::update_parameters(const float* in, int64_t n) {
+  if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n, (long long)size(0));
+  std::vector<float> lp;
+  fetch(lp, d_logp_.p, fc_.n_edges(), stream);
+  const size_t ns = fc_.param2edge.size();
+  for (size_t i = 0; i < ns; ++i) lp[fc_.param2edge[i] - 1] = in[i];
+  if (!lp.empty()) PCM_HIP(hipMemcpyAsync(d_logp_.p, lp.data(), lp.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+  if (!fc_.leaf_logp.empty())
+    PCM_HIP(hipMemcpyAsync(d_leaf_.p, in + ns, fc_.leaf_logp.size() * sizeof(float), hipMemcpyHostToDevice, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void SparseCircuit::ensure_batch(int batch) {
+  if (batch <= cap_batch_) return;
+  const int Bp = ceil_div(batch, 64) * 64;
+  d_mars_.alloc((size_t)fc_.n_nodes() * Bp);
+  d_flows_.alloc((size_t)fc_.n_nodes() * Bp);
+  cap_batch_ = Bp;
+}
+
+static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32_t* e0, const int32_t* e1,
+                          const int32_t* ep, const int32_t* epr, const int32_t* es, const int32_t* in_var,
+                          const int32_t* in_ptr, const int32_t* in_edge, const int64_t* in_off, const float* logp,
+                          const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C) {
+  SparseDev d;
+  d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
+  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
+  d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C;
+  return d;
+}
+
+#define SPARSE_DEV(B_, Bp_, xb_) \
+  make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
+           d_in_ptr_.p, d_in_edge_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
+
+void SparseCircuit::run_forward(const BatchRef& b) {
+  if (!b.d_data) fail(PCM_ERR_ARG, "data pointer is null");
+  if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
+  ensure_batch(b.batch);
+  const int Bp = ceil_div(b.batch, 64) * 64;
+  // staged categories live at the head of the flows buffer's tail: use a dedicated buffer
+  d_visit_.ensure((size_t)std::max<int64_t>((int64_t)fc_.num_vars, fc_.n_nodes()) * Bp);
+  uint8_t* xb = d_visit_.p;
+  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(fc_.num_vars, 64)), dim3(256), 0, stream,
+                     b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, fc_.num_vars, fc_.num_cats, xb);
+  check_launch("stage_batch");
+  SparseDev d = SPARSE_DEV(b.batch, Bp, xb);
+  for (int l = 0; l < n_layers_; ++l) {
+    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
+    hipLaunchKernelGGL(sparse_forward_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
+  }
+  check_launch("sparse_forward");
+  last_batch_ = b.batch;
+}
+
+void SparseCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  run_forward(b);
+  const int Bp = ceil_div(b.batch, 64) * 64;
+  // root (or head) rows -> output; the root is the last node
+  if (fc_.heads.empty()) {
+    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)b.batch * sizeof(float),
+                           hipMemcpyDeviceToDevice, stream));
+  } else {
+    DevBuf<int32_t> hn;
+    hn.upload(fc_.heads, stream);
+    hipLaunchKernelGGL(sparse_copy_rows_kernel, dim3(ceil_div(b.batch, 256), (int)fc_.heads.size()), dim3(256), 0, stream,
+                       d_mars_.p, Bp, b.batch, hn.p, (int)fc_.heads.size(), d_ll);
+    check_launch("copy_rows");
+    PCM_HIP(hipStreamSynchronize(stream));
+  }
+}
+
+void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (fc_.heads.empty() && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (!fc_.heads.empty() && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
+  run_forward(b);
+  const int Bp = ceil_div(b.batch, 64) * 64;
+  const int64_t ne = fc_.n_edges();
+  hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div(std::max<int64_t>(ne, 1), 256)), dim3(256), 0, stream, d_edge_aggr_.p, ne, rate);
+  hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)fc_.leaf_logp.size(), 256)), dim3(256), 0, stream,
+                     d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
+  SparseDev d = SPARSE_DEV(b.batch, Bp, d_visit_.p);
+  for (int l = n_layers_ - 1; l >= 0; --l) {
+    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
+    hipLaunchKernelGGL(sparse_backward_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0, d_heads_.p, d_head_mask,
+                       d_edge_aggr_.p, d_leaf_flow_.p);
+  }
+  check_launch("sparse_backward");
+  if (fc_.heads.empty()) {
+    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)b.batch * sizeof(float),
+                           hipMemcpyDeviceToDevice, stream));
+  } else {
+    DevBuf<int32_t> hn;
+    hn.upload(fc_.heads, stream);
+    hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(b.batch, 256)), dim3(256), 0, stream, d_mars_.p, Bp, b.batch,
+                       hn.p, (int)fc_.heads.size(), d_head_mask, d_ll);
+    check_launch("head_mixture");
+    PCM_HIP(hipStreamSynchronize(stream));
+  }
+  have_flows_ = true;
+}
+
+void SparseCircuit::em_update(float pseudocount, float inertia) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
+  SparseDev d = SPARSE_DEV(0, 64, nullptr);
+  hipLaunchKernelGGL(sparse_update_kernel, dim3(ceil_div(fc_.n_nodes(), 128)), dim3(128), 0, stream, d, (int)fc_.n_nodes(),
+                     d_logp_.p, d_leaf_.p, d_edge_aggr_.p, d_leaf_flow_.p, pseudocount, inertia);
+  check_launch("sparse_update");
+}
+
+void SparseCircuit::get_node_values(float* mars, float* flows, int64_t n) {
+  if (!last_batch_) fail(PCM_ERR_STATE, "no batch has been evaluated yet");
+  const int B = last_batch_, Bp = ceil_div(B, 64) * 64;
+  if (n != fc_.n_nodes() * B) fail(PCM_ERR_ARG, "expected %lld values (nodes x batch), caller gave %lld",
+                                   (long long)(fc_.n_nodes() * B), (long long)n);
+  std::vector<float> h;
+  for (int pass = 0; pass < 2; ++pass) {
+    float* dst = pass ? flows : mars;
+    if (!dst) continue;
+    if (pass && !have_flows_) fail(PCM_ERR_STATE, "no flows have been computed yet");
+    fetch(h, pass ? d_flows_.p : d_mars_.p, (size_t)fc_.n_nodes() * Bp, stream);
+    for (int64_t i = 0; i < fc_.n_nodes(); ++i) std::copy(h.begin() + i * Bp, h.begin() + i * Bp + B, dst + i * B);
+  }
+}
+
+void SparseCircuit::get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed yet");
+  if (edge_aggr) {
+    if (n_edges != fc_.n_edges()) fail(PCM_ERR_ARG, "circuit has %lld edges, caller gave %lld", (long long)fc_.n_edges(), (long long)n_edges);
+    if (n_edges) { PCM_HIP(hipMemcpyAsync(edge_aggr, d_edge_aggr_.p, n_edges * sizeof(float), hipMemcpyDeviceToHost, stream)); }
+  }
+  if (leaf_flow) {
+    if (n_leaf != (int64_t)fc_.leaf_logp.size()) fail(PCM_ERR_ARG, "circuit has %zu input parameters, caller gave %lld", fc_.leaf_logp.size(), (long long)n_leaf);
+    PCM_HIP(hipMemcpyAsync(leaf_flow, d_leaf_flow_.p, n_leaf * sizeof(float), hipMemcpyDeviceToHost, stream));
+  }
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+// ---- KL ---------------------------------------------------------------------------------
+
+static SparseCircuit* same_structure(SparseCircuit* p, pcm_circuit* q) {
+  auto* s = dynamic_cast<SparseCircuit*>(q);
+  if (!s) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
+  if (s->flat().n_nodes() != p->flat().n_nodes() || s->flat().n_edges() != p->flat().n_edges() ||
+      s->flat().e_prime != p->flat().e_prime || s->flat().e_sub != p->flat().e_sub || s->flat().num_cats != p->flat().num_cats)
+    fail(PCM_ERR_SHAPE, "the two circuits of a KL query must share one structure");
+  return s;
+}
+
+void SparseCircuit::kld_forward_device(SparseCircuit* q) {
+  if (!fc_.heads.empty()) fail(PCM_ERR_UNSUPPORTED, "KL of multi-head circuits is not defined");
+  d_kld_.ensure(fc_.n_nodes());
+  d_edge_kld_.ensure(std::max<int64_t>(fc_.n_edges(), 1));
+  SparseDev d = SPARSE_DEV(0, 64, nullptr);
+  for (int l = 0; l < n_layers_; ++l) {
+    const int n0 = layer_node0_[l], n1 = layer_node0_[l + 1];
+    hipLaunchKernelGGL(sparse_kld_up_kernel, dim3(ceil_div(n1 - n0, 128)), dim3(128), 0, stream, d, n0, n1, q->d_logp_.p,
+                       q->d_leaf_.p, d_kld_.p, d_edge_kld_.p);
+  }
+  check_launch("sparse_kld_up");
+}
+
+void SparseCircuit::kld(pcm_circuit* q, float* out) {
+  SparseCircuit* s = same_structure(this, q);
+  kld_forward_device(s);
+  PCM_HIP(hipMemcpyAsync(out, d_kld_.p + fc_.n_nodes() - 1, sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void SparseCircuit::kld_backward_device(SparseCircuit* q, float* g1, float* g2, float* lg1, float* lg2) {
+  kld_forward_device(q);
+  d_grad_.ensure(fc_.n_nodes());
+  SparseDev d = SPARSE_DEV(0, 64, nullptr);
+  for (int l = n_layers_ - 1; l >= 0; --l) {
+    const int n0 = layer_node0_[l], n1 = layer_node0_[l + 1];
+    hipLaunchKernelGGL(sparse_kld_down_kernel, dim3(ceil_div(n1 - n0, 128)), dim3(128), 0, stream, d, n0, n1,
+                       (int)fc_.n_nodes() - 1, d_grad_.p);
+  }
+  const int64_t ne = fc_.n_edges();
+  if (ne) hipLaunchKernelGGL(sparse_kld_edge_grad_kernel, dim3(ceil_div(ne, 256)), dim3(256), 0, stream, d, ne, d_grad_.p,
+                             d_edge_kld_.p, g1, g2);
+  DevBuf<int32_t> inn;
+  inn.upload(fc_.input_nodes, stream);
+  const int64_t nl = (int64_t)fc_.leaf_logp.size();
+  hipLaunchKernelGGL(sparse_kld_leaf_grad_kernel, dim3(ceil_div(nl, 256)), dim3(256), 0, stream, d, inn.p,
+                     (int)fc_.input_nodes.size(), q->d_leaf_.p, d_grad_.p, lg1, lg2);
+  check_launch("sparse_kld_backward");
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void SparseCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) {
+  SparseCircuit* s = same_structure(this, q);
+  if (n != size(0)) fail(PCM_ERR_ARG, "gradient vectors have %lld entries, circuit has %lld parameters", (long long)n, (long long)size(0));
+  if (!gp || !gq) fail(PCM_ERR_ARG, "gradient pointer is null");
+  const int64_t ne = std::max<int64_t>(fc_.n_edges(), 1), nl = (int64_t)fc_.leaf_logp.size();
+  DevBuf<float> g1, g2, l1, l2;
+  g1.alloc(ne); g2.alloc(ne); l1.alloc(nl); l2.alloc(nl);
+  kld_backward_device(s, g1.p, g2.p, l1.p, l2.p);
+  std::vector<float> h1, h2;
+  fetch(h1, g1.p, ne, stream); fetch(h2, g2.p, ne, stream);
+  const size_t ns = fc_.param2edge.size();
+  for (size_t i = 0; i < ns; ++i) { gp[i] = h1[fc_.param2edge[i] - 1]; gq[i] = h2[fc_.param2edge[i] - 1]; }
+  fetch(h1, l1.p, nl, stream); fetch(h2, l2.p, nl, stream);
+  std::copy(h1.begin(), h1.end(), gp + ns);
+  std::copy(h2.begin(), h2.end(), gq + ns);
+}
+
+// ---- sampling ---------------------------------------------------------------------------
+
+void SparseCircuit::sample_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
+                                      const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
+  if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
+  if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  if (!fc_.heads.empty()) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
+  const int Bp = ceil_div(batch, 64) * 64;
+  d_visit_.ensure((size_t)std::max<int64_t>((int64_t)fc_.num_vars, fc_.n_nodes()) * Bp);
+  const int64_t nv = fc_.n_nodes() * Bp;
+  hipLaunchKernelGGL(sparse_fill_u8_kernel, dim3(ceil_div(nv, 256)), dim3(256), 0, stream, d_visit_.p, nv, (uint8_t)0);
+  hipLaunchKernelGGL(sparse_set_row_u8_kernel, dim3(ceil_div(Bp, 256)), dim3(256), 0, stream,
+                     d_visit_.p + (size_t)(fc_.n_nodes() - 1) * Bp, Bp, (uint8_t)1);
+  hipLaunchKernelGGL(sparse_fill_u8_kernel, dim3(ceil_div((int64_t)batch * fc_.num_vars, 256)), dim3(256), 0, stream, d_out,
+                     (int64_t)batch * fc_.num_vars, (uint8_t)255);
+  DevBuf<int64_t> e2p;
+  std::vector<int64_t> e2pv = fc_.edge2param;
+  if (e2pv.empty()) e2pv.push_back(0);
+  e2p.upload(e2pv, stream);
+  SparseDev d = SPARSE_DEV(batch, Bp, nullptr);
+  for (int l = n_layers_ - 1; l >= 0; --l) {
+    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
+    hipLaunchKernelGGL(sparse_sample_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0, d_noise_slot, e2p.p,
+                       noise_stride, d_node_noise, d_leaf_noise, fc_.num_vars, d_visit_.p, d_out);
+  }
+  check_launch("sparse_sample");
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void SparseCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
+  sample_with_slots(d_node_noise, nullptr, sample_noise_size(), d_leaf_noise, batch, d_out);
+}
+
+// ---- Adam ---------------------------------------------------------------------------------
+
+void SparseCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
+                              float b2, float eps, int t) {
+  if (!d_grad || !d_params || !d_m || !d_v) fail(PCM_ERR_ARG, "null optimiser array");
+  if (t < 1) fail(PCM_ERR_ARG, "step count must start at 1, got %d", t);
+  const int64_t ns = (int64_t)fc_.param2edge.size();
+  if (!ns) return;
+  const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
+  hipLaunchKernelGGL(sparse_adam_kernel, dim3(ceil_div(ns, 256)), dim3(256), 0, stream, ns, d_grad, d_params, d_m, d_v, lr,
+                     b1, b2, eps, c1, c2);
+  const int ng = (int)fc_.pargroup_sizes.size();
+  hipLaunchKernelGGL(sparse_normalize_kernel, dim3(ceil_div(ng, 128)), dim3(128), 0, stream, ng, d_group_ptr_.p,
+                     d_param2edge_.p, d_params, d_logp_.p);
+  check_launch("sparse_adam");
+}
+
+}  // namespace pcm

@@ -1,0 +1,96 @@
+// General engine: any circuit DAG, flattened into nodes + (prime, sub) edges and evaluated
+// layer by layer.  It restates what the reference gets from ProbabilisticCircuits.jl
+// `BitsProbCircuit` (un-vendored) plus src/bits_circuit.jl:39-113, with two layout changes
+// for the GPU: node values are kept node-major with the example index fastest (coalesced
+// over a wave), and every node owns a contiguous run of up-edges and a contiguous run of
+// incoming (down) edges, so that a thread folds one node's edges sequentially and writes
+// its result once -- no atomics on node values or flows.
+#pragma once
+
+#include "common.hpp"
+
+namespace pcm {
+
+enum : uint8_t { kInput = 0, kSum = 1, kMul = 2 };
+
+// Host-side flat circuit (also used by the HCLT engine to expose its general form).
+struct FlatCircuit {
+  int32_t num_vars = 0, num_cats = 0, num_heads = 0;
+  std::vector<uint8_t> type;          // per node
+  std::vector<int32_t> layer;         // per node: inputs 0, inner 1 + max over children
+  std::vector<int32_t> in_var;        // per node (inputs)
+  std::vector<int64_t> in_off;        // per node (inputs): offset into leaf arrays
+  std::vector<int32_t> input_nodes;   // input node ids in creation order
+  // up edges in the reference's order: by layer, then by parent id
+  std::vector<int32_t> e_parent, e_prime, e_sub;   // sub = -1: none
+  std::vector<float> e_logp;                         // 0 on product edges
+  std::vector<int32_t> node_e0, node_e1;             // a node's run of up edges
+  std::vector<int64_t> layer_ends;                   // edge count at the end of each up layer
+  std::vector<float> leaf_logp;                      // [inputs * C]
+  std::vector<int32_t> heads;                        // node ids of the heads (multi-head)
+  // parameter tables (1-based, src/bits_circuit.jl:46-70)
+  std::vector<int64_t> edge2param, param2edge, param2group, pargroup_sizes;
+  int64_t n_nodes() const { return (int64_t)type.size(); }
+  int64_t n_edges() const { return (int64_t)e_parent.size(); }
+  void finish();   // derives node_e0/e1, layer_ends and the parameter tables from the edges
+};
+
+// Flattening of a DAG description (see pcm_circuit_create for the format).
+FlatCircuit flatten_dag(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
+                        const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
+                        const float* input_logp, int32_t num_vars, int32_t num_cats, int32_t num_heads);
+
+class SparseCircuit : public pcm_circuit {
+ public:
+  explicit SparseCircuit(FlatCircuit fc);
+  ~SparseCircuit() override {}
+
+  int64_t size(int what) const override;
+  void index_table(int which, int64_t* out, int64_t n) const override;
+  void vectorize(float* out, int64_t n) override;
+  void update_parameters(const float* in, int64_t n) override;
+  void loglikelihoods(const BatchRef& b, float* d_ll) override;
+  void flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) override;
+  void em_update(float pseudocount, float inertia) override;
+  void kld(pcm_circuit* q, float* out) override;
+  void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
+  int64_t sample_noise_size() const override { return (int64_t)fc_.param2edge.size(); }
+  void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) override;
+  void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1, float b2,
+                 float eps, int t) override;
+
+  void get_node_values(float* mars, float* flows, int64_t n);
+  void get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf);
+
+  // device views for engines that embed a general circuit (the HCLT engine's KL / sampling)
+  float* d_logp() { return d_logp_.p; }
+  float* d_leaf() { return d_leaf_.p; }
+  const FlatCircuit& flat() const { return fc_; }
+  // noise_slot: optional device table (one entry per edge, up order) mapping a sum edge to its
+  // column in the node-noise matrix; noise_stride: columns of that matrix
+  void sample_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
+                         const float* d_leaf_noise, int32_t batch, uint8_t* d_out);
+  void kld_forward_device(SparseCircuit* q);          // leaves the result in d_kld_ (root last)
+  void kld_backward_device(SparseCircuit* q, float* d_edge_g1, float* d_edge_g2, float* d_leaf_g1, float* d_leaf_g2);
+  float* d_kld() { return d_kld_.p; }
+
+ private:
+  FlatCircuit fc_;
+  int n_layers_ = 0;
+  std::vector<int32_t> layer_node0_;   // nodes sorted by layer: ranges per layer
+  DevBuf<uint8_t> d_type_;
+  DevBuf<int32_t> d_order_, d_node_e0_, d_node_e1_, d_e_parent_, d_e_prime_, d_e_sub_, d_in_var_;
+  DevBuf<int64_t> d_in_off_;
+  DevBuf<float> d_logp_, d_leaf_, d_edge_aggr_, d_leaf_flow_, d_mars_, d_flows_, d_kld_, d_edge_kld_, d_grad_;
+  // incoming edges per node (down direction)
+  DevBuf<int32_t> d_in_ptr_, d_in_edge_;
+  DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_;
+  DevBuf<uint8_t> d_visit_;
+  int cap_batch_ = 0, last_batch_ = 0;
+  bool have_flows_ = false;
+
+  void ensure_batch(int batch);
+  void run_forward(const BatchRef& b);
+};
+
+}  // namespace pcm

@@ -6,10 +6,10 @@ import numpy as np
 from ._lib import lib, check, np_ptr, H, c_i64
 
 _SIZE = dict(parameters=0, sum_parameters=1, nodes=2, edges=3, input_parameters=4, variables=5,
-             categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11)
+             categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11, heads=12)
 _TABLE = dict(edge2param=(0, "edges"), param2edge=(1, "sum_parameters"), param2group=(2, "sum_parameters"),
               pargroup_sizes=(3, "groups"), innode2ncumparam=(4, "input_nodes"), layer_ends=(5, "layers"),
-              edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"))
+              edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"), heads=(9, "heads"))
 
 
 class BitsCircuit:
@@ -61,6 +61,22 @@ class BitsCircuit:
 
     def set_stream(self, stream):
         check(lib.pcm_set_stream(self.handle, ctypes.c_void_p(stream)))
+
+    def get_node_values(self, batch, flows=True):
+        """Host copies of `mars` (and `flows`) of the last batch, [num_nodes, batch]
+        (circuits from compile_circuit only)."""
+        n = self.num_nodes()
+        mars = np.empty((n, batch), np.float32)
+        fl = np.empty((n, batch), np.float32) if flows else None
+        check(lib.pcm_get_node_values(self.handle, np_ptr(mars), np_ptr(fl), c_i64(n * batch)))
+        return (mars, fl) if flows else mars
+
+    def get_aggregates(self):
+        """(edge_aggr [edges, up order], leaf flows [input parameters]) accumulated so far."""
+        ea = np.empty(self.num_edges(), np.float32)
+        lf = np.empty(self.num_input_params(), np.float32)
+        check(lib.pcm_get_aggregates(self.handle, np_ptr(ea), c_i64(len(ea)), np_ptr(lf), c_i64(len(lf))))
+        return ea, lf
 
 
 class HcltCircuit(BitsCircuit):

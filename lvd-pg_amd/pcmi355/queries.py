@@ -52,6 +52,17 @@ def loglikelihoods(bpc, data, batch_size=None, example_ids=None):
     return out.t().contiguous() if heads else out[0]
 
 
+def multihead_loglikelihoods(mhbpc, data, head_mask, batch_size=None, example_ids=None):
+    """`loglikelihoods(mhbpc, data, head_mask; batch_size)`
+    (src-jl/multi_head_pc/likelihood.jl:37-71) with a head mask [num_examples, num_heads]:
+    logsumexp_h(ll_h + log mask_h) - log sum_h mask_h (:3-12), from the per-head values."""
+    per_head = loglikelihoods(mhbpc, data, batch_size=batch_size, example_ids=example_ids)
+    hm = head_mask.to(device=data.device, dtype=torch.float32)
+    if example_ids is not None:
+        hm = hm[_ids(example_ids, data.device).long()]
+    return torch.logsumexp(per_head + torch.log(hm), dim=1) - torch.log(hm.sum(dim=1))
+
+
 def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
     """`probs_flows_circuit` (src/queries/flow.jl:228-234) /
     `probs_flows_circuit_with_reg` with soft_reg = 0 (src/regularization/reg_flow.jl:276-282):

@@ -54,3 +54,90 @@ def rel_err(a, b, floor=1e-30):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return np.abs(a - b) / np.maximum(np.abs(b), floor)
+
+
+def describe_dag(roots):
+    """Oracle DAG (pc_oracle.Node) -> the flat description pcm_circuit_create takes:
+    children before parents, the given roots last (several roots = heads of a multi-head
+    circuit).  Returns a dict of numpy arrays."""
+    roots = list(roots)
+    root_ids = {id(r) for r in roots}
+    order, seen = [], set()
+
+    def visit(n):
+        if id(n) in seen:
+            return
+        seen.add(id(n))
+        for c in n.children:
+            visit(c)
+        if id(n) not in root_ids:
+            order.append(n)
+
+    for r in roots:
+        visit(r)
+    order += roots
+    index = {id(n): i for i, n in enumerate(order)}
+    node_type = np.array([n.kind for n in order], np.uint8)
+    child_ptr = np.zeros(len(order) + 1, np.int32)
+    child_idx, sum_logp, input_var, input_logp = [], [], [], []
+    for i, n in enumerate(order):
+        for q, c in enumerate(n.children):
+            child_idx.append(index[id(c)])
+            sum_logp.append(float(n.logps[q]) if n.kind == O.SUM else 0.0)
+        child_ptr[i + 1] = len(child_idx)
+        input_var.append(n.var if n.kind == O.INPUT else -1)
+        if n.kind == O.INPUT:
+            input_logp.append(np.asarray(n.logps, np.float32))
+    return dict(node_type=node_type, child_ptr=child_ptr, child_idx=np.array(child_idx, np.int32),
+                sum_logp=np.array(sum_logp, np.float32), input_var=np.array(input_var, np.int32),
+                input_logp=np.concatenate(input_logp).astype(np.float32))
+
+
+def log_dirichlet(rng, n):
+    x = rng.exponential(size=n) + 1e-3
+    return np.log(x / x.sum()).astype(np.float32)
+
+
+def simple_3vars_circuit(C, rng=None, weights=None):
+    """test/helpers/simple_circuits.jl:4-14: summate(multiply(n11, n21, n31), multiply(n12, n22, n32))."""
+    def leaf(v):
+        lp = np.full(C, -np.log(C), np.float32) if rng is None else log_dirichlet(rng, C)
+        return O.input_node(v, lp)
+    n11, n21, n31 = leaf(0), leaf(1), leaf(2)
+    n12, n22, n32 = leaf(0), leaf(1), leaf(2)
+    w = None if weights is None else np.log(np.asarray(weights, np.float32))
+    return O.summate(O.multiply(n11, n21, n31), O.multiply(n12, n22, n32), logps=w)
+
+
+def simple_multihead_circuit(C, rng=None):
+    """test/helpers/simple_circuits.jl:54-66: two sum heads over the same two 3-way products."""
+    def leaf(v):
+        lp = np.full(C, -np.log(C), np.float32) if rng is None else log_dirichlet(rng, C)
+        return O.input_node(v, lp)
+    n11, n21, n31 = leaf(0), leaf(1), leaf(2)
+    n12, n22, n32 = leaf(0), leaf(1), leaf(2)
+    n1, n2 = O.multiply(n11, n21, n31), O.multiply(n12, n22, n32)
+    return [O.summate(n1, n2), O.summate(n1, n2)]
+
+
+def random_dag(V, C, rng, width=4, depth=3):
+    """A random smooth & decomposable circuit with shared sub-circuits: a balanced
+    variable-partition tree; each region holds `width` sum nodes over products that pair
+    (or triple) children regions' nodes; region nodes are reused by several parents."""
+    def region(vars_, d):
+        if len(vars_) == 1:
+            return [O.input_node(int(vars_[0]), log_dirichlet(rng, C)) for _ in range(width)]
+        nparts = 3 if (len(vars_) >= 3 and rng.random() < 0.4) else 2
+        parts = np.array_split(vars_, nparts)
+        kids = [region(p, d + 1) for p in parts]
+        outs = []
+        nsum = 1 if d == 0 else width
+        prods = []
+        for _ in range(width + 1):
+            prods.append(O.multiply(*[k[rng.integers(len(k))] for k in kids]))
+        for _ in range(nsum):
+            m = int(rng.integers(1, len(prods) + 1))
+            sel = rng.choice(len(prods), size=m, replace=False)
+            outs.append(O.summate(*[prods[q] for q in sel], logps=log_dirichlet(rng, m)))
+        return outs
+    return region(np.arange(V), 0)[0]

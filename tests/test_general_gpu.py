@@ -1,0 +1,263 @@
+"""GPU parity of the general (layered) engine against the CPU oracle, through the C ABI:
+the reference's fixture circuits, random DAGs with shared sub-circuits, multi-head circuits,
+and the HCLT in its general form against the dense-block engine."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+LL_RTOL = 1e-4
+PARAM_RTOL = 1e-4
+FLOW_RTOL = 2e-4
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    import pcmi355
+    return torch, pcmi355
+
+
+def _compile(P, roots, V, C, heads=0):
+    from helpers import describe_dag
+    d = describe_dag(roots)
+    return P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"],
+                             d["input_logp"], V, C, heads)
+
+
+def _check_tables(bpc, fc):
+    """Index tables and parameter vector of the compiled circuit against the oracle's flattening."""
+    import pcmi355 as P
+    t = fc.param_tables()
+    order = fc.up_order()
+    assert bpc.num_nodes() == fc.n_nodes and bpc.num_edges() == fc.n_edges
+    for name in ("edge2param", "param2edge", "param2group", "pargroup_sizes", "innode2ncumparam"):
+        assert np.array_equal(bpc.table(name), t[name]), name
+    assert np.array_equal(bpc.table("edge_parent") - 1, fc.edge_parent()[order])
+    assert np.array_equal(bpc.table("edge_prime") - 1, fc.prime[order])
+    assert np.array_equal(bpc.table("edge_sub") - 1, fc.sub[order])
+    assert np.array_equal(P.vectorize_parameters(bpc), fc.vectorize_parameters())
+    return order
+
+
+def _check_em_step(gpu, O, root, V, C, B, seed, pseudocount=0.1, inertia=0.9):
+    torch, P = gpu
+    from helpers import rel_err
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, [root], V, C)
+    order = _check_tables(bpc, fc)
+    rng = np.random.default_rng(seed)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+
+    mars_ref = O.forward(fc, data)
+    ll = P.loglikelihoods(bpc, d).cpu().numpy()
+    assert rel_err(ll, mars_ref[-1]).max() < LL_RTOL
+    ll2 = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    assert np.array_equal(ll, ll2)
+
+    flows_ref, ea_ref = O.backward(fc, mars_ref)
+    lf_ref = O.input_flows(fc, data, flows_ref)
+    mars, flows = bpc.get_node_values(B)
+    assert np.abs(mars - mars_ref).max() < LL_RTOL * np.abs(mars_ref).max()
+    assert np.abs(flows - flows_ref).max() < FLOW_RTOL
+    ea, lf = bpc.get_aggregates()
+    assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * max(ea_ref.max(), 1.0)
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * max(lf_ref.max(), 1.0)
+
+    import pcmi355._lib as L
+    L.check(L.lib.pcm_em_update(bpc.handle, pseudocount, inertia))
+    logp, leaf = O.em_update(fc, ea_ref, lf_ref, pseudocount, inertia)
+    new = fc.copy()
+    new.logp, new.leaf_logp = logp, leaf
+    got = P.vectorize_parameters(bpc)
+    assert rel_err(np.exp(got), np.exp(new.vectorize_parameters())).max() < PARAM_RTOL
+    return bpc, fc
+
+
+def test_three_var_fixture_known_answers(gpu, oracle):
+    """test/bits_circuit_tests.jl:13-24 and test/misc_tests.jl:39-62 on simple_3vars_circuit."""
+    torch, P = gpu
+    from helpers import simple_3vars_circuit
+    root = simple_3vars_circuit(5, np.random.default_rng(3))
+    bpc = _compile(P, [root], 3, 5)
+    assert bpc.num_nodes() == 9 and bpc.num_edges() == 6
+    assert bpc.num_parameters() == 32 and bpc.num_input_params() == 30
+    assert bpc.table("edge2param").tolist() == [0, 0, 0, 0, 1, 2]
+    assert bpc.table("param2edge").tolist() == [5, 6]
+    assert bpc.table("param2group").tolist() == [1, 1]
+    assert bpc.table("pargroup_sizes").tolist() == [2]
+    assert bpc.table("innode2ncumparam").tolist() == [5, 10, 15, 20, 25, 30]
+
+
+@pytest.mark.parametrize("B", [1, 7, 64, 200])
+def test_three_var_fixture_em_step(gpu, oracle, B):
+    from helpers import simple_3vars_circuit
+    root = simple_3vars_circuit(5, np.random.default_rng(11), weights=[0.3, 0.7])
+    _check_em_step(gpu, oracle, root, 3, 5, B, seed=B)
+
+
+@pytest.mark.parametrize("V,C,width,seed", [(4, 3, 2, 0), (9, 6, 4, 1), (17, 11, 5, 2), (6, 256, 3, 3)])
+def test_random_dag_em_step(gpu, oracle, V, C, width, seed):
+    from helpers import random_dag
+    root = random_dag(V, C, np.random.default_rng(seed), width=width)
+    _check_em_step(gpu, oracle, root, V, C, 96, seed=seed + 50)
+
+
+def test_example_ids_and_flow_memory(gpu, oracle):
+    """Batches picked by example ids; accumulators scaled by `rate` before a batch
+    (src/regularization/reg_em.jl:276-284)."""
+    torch, P = gpu
+    O = oracle
+    from helpers import random_dag
+    V, C = 7, 5
+    root = random_dag(V, C, np.random.default_rng(5), width=3)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, [root], V, C)
+    order = fc.up_order()
+    rng = np.random.default_rng(6)
+    data = rng.integers(0, C, size=(300, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+    ids1 = rng.permutation(300)[:70].astype(np.int32)
+    ids2 = rng.permutation(300)[:33].astype(np.int32)
+    P.probs_flows_circuit(bpc, d, example_ids=ids1)
+    P.probs_flows_circuit(bpc, d, example_ids=ids2, rate=0.25)
+    ea, lf = bpc.get_aggregates()
+    m1 = O.forward(fc, data, ids1)
+    f1, ea1 = O.backward(fc, m1)
+    lf1 = O.input_flows(fc, data, f1, ids1)
+    m2 = O.forward(fc, data, ids2)
+    f2, ea2 = O.backward(fc, m2)
+    lf2 = O.input_flows(fc, data, f2, ids2)
+    ea_ref = 0.25 * ea1 + ea2
+    lf_ref = 0.25 * lf1 + lf2
+    assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
+
+
+def test_multihead_closed_forms(gpu, oracle):
+    """test/multi_head_pc/multi_head_pc_learning_tests.jl:11-47."""
+    torch, P = gpu
+    from helpers import simple_multihead_circuit
+    heads = simple_multihead_circuit(5)
+    heads[0].children[0].children[0].logps = np.log(np.array([0.1, 0.2, 0.3, 0.3, 0.1], np.float32))
+    heads[0].logps = np.log(np.array([0.2, 0.8], np.float32))
+    heads[1].logps = np.log(np.array([0.6, 0.4], np.float32))
+    bpc = _compile(P, heads, 3, 5, heads=2)
+    assert bpc.size("heads") == 2
+    assert bpc.table("heads").tolist() == [9, 10]          # the reference's root_ids (fake root would be 11)
+    data = torch.tensor([[0, 0, 0], [2, 0, 0]], dtype=torch.uint8).cuda()
+    head_mask = torch.tensor([[1.0, 0.0], [0.0, 1.0]]).cuda()
+    want = [np.log(0.1 * 0.2 * 0.2 * 0.2 + 0.2 ** 3 * 0.8), np.log(0.3 * 0.2 * 0.2 * 0.6 + 0.2 ** 3 * 0.4)]
+    lls = P.multihead_loglikelihoods(bpc, data, head_mask).cpu().numpy()
+    np.testing.assert_allclose(lls, want, rtol=1e-5)
+    per_head = P.loglikelihoods(bpc, data).cpu().numpy()
+    assert per_head.shape == (2, 2)
+    np.testing.assert_allclose([per_head[0, 0], per_head[1, 1]], want, rtol=1e-5)
+
+    ll = P.probs_flows_circuit(bpc, data, head_mask=head_mask).cpu().numpy()
+    np.testing.assert_allclose(ll, want, rtol=1e-5)
+    mars, flows = bpc.get_node_values(2)
+    mars, flows = mars.T, flows.T        # [example, node] like the reference
+    n = lambda i: i - 1                  # the reference's 1-based node ids
+    assert flows[0, n(9)] == 1.0 and flows[0, n(10)] == 0.0
+    assert flows[1, n(9)] == 0.0 and flows[1, n(10)] == 1.0
+    f32 = np.float32
+    np.testing.assert_allclose(flows[0, n(4)], np.exp(mars[0, 0] + mars[0, 1] + mars[0, 2] + np.log(f32(0.2)) - mars[0, n(9)]), rtol=1e-5)
+    np.testing.assert_allclose(flows[0, n(8)], np.exp(mars[0, 4] + mars[0, 5] + mars[0, 6] + np.log(f32(0.8)) - mars[0, n(9)]), rtol=1e-5)
+    np.testing.assert_allclose(flows[1, n(4)], np.exp(mars[1, 0] + mars[1, 1] + mars[1, 2] + np.log(f32(0.6)) - mars[1, n(10)]), rtol=1e-5)
+    np.testing.assert_allclose(flows[1, n(8)], np.exp(mars[1, 4] + mars[1, 5] + mars[1, 6] + np.log(f32(0.4)) - mars[1, n(10)]), rtol=1e-5)
+
+
+def test_multihead_soft_mask_em_matches_oracle(gpu, oracle):
+    """Soft head masks: flows seeded by head_mask[b, h] (src-jl/multi_head_pc/flow.jl:141-176),
+    mixture LL (likelihood.jl:3-12), then the four update calls (em.jl:77-81).  The oracle
+    runs the reference's construction: a fake root over the heads whose edges are skipped."""
+    torch, P = gpu
+    O = oracle
+    from helpers import random_dag, rel_err
+    V, C, H, B = 6, 4, 3, 80
+    rng = np.random.default_rng(21)
+    body = random_dag(V, C, rng, width=3)
+    # heads: H sums over the products feeding the body's root
+    prods = body.children
+    heads = [O.summate(*prods, logps=np.log(rng.dirichlet(np.ones(len(prods)))).astype(np.float32)) for _ in range(H)]
+    bpc = _compile(P, heads, V, C, heads=H)
+    fake = O.summate(*heads)
+    fc = O.bits_compile(fake, C, V)
+    n_real = fc.n_nodes - 1
+    assert bpc.num_nodes() == n_real
+    root_ids = (bpc.table("heads") - 1).astype(np.int32)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    mask = rng.random((B, H)).astype(np.float32) + 0.05
+    mask[::7, 1] = 0.0     # hard zeros: log(0) = -inf must fold away
+    d = torch.from_numpy(data).cuda()
+    hm = torch.from_numpy(mask).cuda()
+
+    ll = P.probs_flows_circuit(bpc, d, head_mask=hm).cpu().numpy()
+    mars_ref = O.forward(fc, data)
+    with np.errstate(divide="ignore"):
+        mix = np.logaddexp.reduce(mars_ref[root_ids].astype(np.float64) + np.log(mask.T.astype(np.float64)), axis=0) \
+            - np.log(mask.sum(axis=1, dtype=np.float64))
+    assert rel_err(ll, mix).max() < LL_RTOL
+    skip = (fc.edge_parent() == fc.n_nodes - 1).astype(np.uint8)
+    flows_ref, ea_ref = O.backward(fc, mars_ref, skip=skip, root_ids=root_ids, root_flow=np.ascontiguousarray(mask.T))
+    lf_ref = O.input_flows(fc, data, flows_ref)
+    mars, flows = bpc.get_node_values(B)
+    assert np.abs(flows - flows_ref[:n_real]).max() < FLOW_RTOL
+    ea, lf = bpc.get_aggregates()
+    order = fc.up_order()
+    order = order[fc.edge_parent()[order] != fc.n_nodes - 1]
+    assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
+
+    lls = P.mini_batch_em_for_multihead_pc(bpc, d, hm, 2, batch_size=40, pseudocount=0.1, param_inertia=0.5,
+                                           shuffle="none")
+    assert len(lls) == 2 and lls[1] > lls[0]
+
+
+def test_hclt_general_form_matches_block_engine(gpu, oracle):
+    """The same HCLT through both engines: LL, parameter vector after an EM step."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, correlated_data, block_theta, rel_err
+    V, K, C, B = 11, 16, 9, 128
+    parent, theta, leaf, fc = make_hclt(V, K, C, 77)
+    dense = P.hclt_from_clt(parent, C, K)
+    dense.set_params(block_theta(parent, K, theta), leaf)
+    general = _compile(P, [O.hclt_dag(parent, K, C, theta, leaf)], V, C)
+    for name in ("edge2param", "param2edge", "param2group", "pargroup_sizes", "edge_parent", "edge_prime", "edge_sub"):
+        assert np.array_equal(dense.table(name), general.table(name)), name
+    p0 = P.vectorize_parameters(dense)
+    assert np.array_equal(p0, P.vectorize_parameters(general))
+    data = correlated_data(B, V, C, 78, parent)
+    d = torch.from_numpy(data).cuda()
+    import pcmi355._lib as L
+    lls = []
+    for bpc in (dense, general):
+        ll = torch.empty(B, device="cuda")
+        L.check(L.lib.pcm_em_step(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, 0.1, 0.9, ll.data_ptr()))
+        lls.append(ll.cpu().numpy())
+    assert rel_err(lls[0], lls[1]).max() < LL_RTOL
+    assert rel_err(np.exp(P.vectorize_parameters(dense)), np.exp(P.vectorize_parameters(general))).max() < PARAM_RTOL
+
+
+def test_error_paths(gpu):
+    torch, P = gpu
+    import pcmi355._lib as L
+    nt = np.array([0, 0, 1], np.uint8)
+    ok = dict(child_ptr=[0, 0, 0, 2], child_idx=[0, 1], sum_logp=np.log([0.5, 0.5]), input_var=[0, 0, -1],
+              input_logp=np.log(np.full(8, 0.25)))
+    P.compile_circuit(nt, ok["child_ptr"], ok["child_idx"], ok["sum_logp"], ok["input_var"], ok["input_logp"], 1, 4)
+    with pytest.raises(L.PcmError):      # child that is not an earlier node
+        P.compile_circuit(nt, ok["child_ptr"], [0, 2], ok["sum_logp"], ok["input_var"], ok["input_logp"], 1, 4)
+    with pytest.raises(L.PcmError):      # variable out of range
+        P.compile_circuit(nt, ok["child_ptr"], ok["child_idx"], ok["sum_logp"], [0, 3, -1], ok["input_logp"], 1, 4)
+    with pytest.raises(L.PcmError):      # inner node without children
+        P.compile_circuit(nt, [0, 0, 0, 0], [], [], ok["input_var"], ok["input_logp"], 1, 4)
+    bpc = P.compile_circuit(nt, ok["child_ptr"], ok["child_idx"], ok["sum_logp"], ok["input_var"], ok["input_logp"], 1, 4)
+    with pytest.raises(L.PcmError):      # update before any flows
+        L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+    with pytest.raises(ValueError):      # wrong number of variables
+        P.loglikelihoods(bpc, torch.zeros((4, 2), dtype=torch.uint8, device="cuda"))

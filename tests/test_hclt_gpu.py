@@ -69,13 +69,18 @@ def test_config1_shape(gpu, oracle):
     _compare_step(gpu, oracle, 64, 16, 256, 1024, seed=11)
 
 
-def test_param_vector_roundtrip(gpu, oracle):
+@pytest.mark.parametrize("tree", [None, [-1, 0, 0], [-1, 0, 1, 1], [-1, 0, 0, 0, 0], [1, -1, 1, 2, 2, 0, 0, 3],
+                                  [-1, 0, 0, 2, 2, 2, 4, 1, 6, 3, 9]])
+def test_param_vector_roundtrip(gpu, oracle, tree):
+    """Parameter vector and index tables follow the numbering of the flattened DAG, on
+    trees whose nodes have one, two, three and four children."""
     torch, P = gpu
     from helpers import make_hclt, block_theta
-    parent, theta, leaf, fc = make_hclt(9, 16, 6, 3)
+    V = 9 if tree is None else len(tree)
+    parent, theta, leaf, fc = make_hclt(V, 16, 6, 3, parent=None if tree is None else np.array(tree, np.int32))
     bpc = P.hclt_from_clt(parent, 6, 16)
     bpc.set_params(block_theta(parent, 16, theta), leaf)
-    dag = oracle.bits_compile(oracle.hclt_dag(parent, 16, 6, theta, leaf), 6, 9)
+    dag = oracle.bits_compile(oracle.hclt_dag(parent, 16, 6, theta, leaf), 6, V)
     ref = dag.vectorize_parameters()
     got = P.vectorize_parameters(bpc)
     assert got.shape == ref.shape
@@ -88,6 +93,10 @@ def test_param_vector_roundtrip(gpu, oracle):
     np.testing.assert_array_equal(bpc.table("param2edge"), t["param2edge"])
     np.testing.assert_array_equal(bpc.table("param2group"), t["param2group"])
     np.testing.assert_array_equal(bpc.table("pargroup_sizes"), t["pargroup_sizes"])
+    order = dag.up_order()
+    np.testing.assert_array_equal(bpc.table("edge_parent") - 1, dag.edge_parent()[order])
+    np.testing.assert_array_equal(bpc.table("edge_prime") - 1, dag.prime[order])
+    np.testing.assert_array_equal(bpc.table("edge_sub") - 1, dag.sub[order])
 
 
 def test_ten_em_steps_track_oracle(gpu, oracle):

@@ -1,0 +1,266 @@
+"""GPU parity of the parameter-space queries (KL recursion and its gradient, Gumbel-max
+sampling from supplied noise, Adam) against the CPU oracle and the reference tests' closed
+forms, through the C ABI, on general circuits and on HCLTs."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+KLD_RTOL = 1e-4
+GRAD_RTOL = 1e-4
+ADAM_RTOL = 1e-5
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    import pcmi355
+    return torch, pcmi355
+
+
+def _compile(P, root, V, C):
+    from helpers import describe_dag
+    d = describe_dag([root])
+    return P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"],
+                             d["input_logp"], V, C)
+
+
+def _perturbed(params, C, n_sum, rng):
+    """Another normalised parameter vector for the same structure (sum groups are passed in
+    by the caller as whole-vector renormalisation is wrong: only the leaves are redrawn here)."""
+    out = params.copy()
+    leaves = out[n_sum:].reshape(-1, C)
+    x = np.exp(leaves) * rng.uniform(0.5, 1.5, size=leaves.shape)
+    out[n_sum:] = np.log(x / x.sum(axis=1, keepdims=True)).reshape(-1)
+    return out.astype(np.float32)
+
+
+def _grads_in_param_order(fc, eg, lg):
+    pe = fc.sum_param_edges()
+    leaf = [lg[fc.in_off[n]:fc.in_off[n] + fc.C] for n in fc.input_nodes()]
+    return np.concatenate([eg[pe]] + leaf)
+
+
+def test_kld_closed_forms_three_var_fixture(gpu):
+    """test/queries/kld_tests.jl:9-70 and :106-131, one parameter row at a time."""
+    torch, P = gpu
+    from helpers import simple_3vars_circuit
+    rng = np.random.default_rng(0)
+    root = simple_3vars_circuit(5, rng, weights=[0.45, 0.55])
+    p = _compile(P, root, 3, 5)
+    q = _compile(P, root, 3, 5)
+    pars = P.vectorize_parameters(p)
+    assert len(pars) == 32
+    assert abs(P.kld(p, q)) < 1e-7
+
+    for (a, b) in [((0.2, 0.8), (0.4, 0.6)), ((0.5, 0.5), (0.9, 0.1))]:
+        p1, p2 = pars.copy(), pars.copy()
+        p1[:2] = np.log(np.float32(a))
+        p2[:2] = np.log(np.float32(b))
+        P.update_parameters(p, p1)
+        P.update_parameters(q, p2)
+        want = a[0] * np.log(a[0] / b[0]) + a[1] * np.log(a[1] / b[1])
+        np.testing.assert_allclose(P.kld(p, q), want, rtol=1e-5)
+        g1, g2 = P.kld_backward(p, q)
+        np.testing.assert_allclose(g1[:2], [a[0] * (np.log(a[0]) - np.log(b[0]) + 1), a[1] * (np.log(a[1]) - np.log(b[1]) + 1)], rtol=1e-5)
+        np.testing.assert_allclose(g2[:2], [-a[0], -a[1]], rtol=1e-6)
+
+    for w, l1, l2 in [(0.2, [0.1, 0.2, 0.3, 0.2, 0.2], [0.2, 0.1, 0.1, 0.3, 0.3]),
+                      (0.5, [0.1, 0.2, 0.3, 0.2, 0.2], [0.2, 0.1, 0.2, 0.3, 0.2])]:
+        p1, p2 = pars.copy(), pars.copy()
+        p1[:2] = p2[:2] = np.log(np.float32([w, 1 - w]))
+        p1[2:7] = np.log(np.float32(l1))
+        p2[2:7] = np.log(np.float32(l2))
+        P.update_parameters(p, p1)
+        P.update_parameters(q, p2)
+        want = float(np.sum(np.exp(p1[2:7]) * (p1[2:7] - p2[2:7])) * w)
+        np.testing.assert_allclose(P.kld(p, q), want, rtol=1e-4)
+
+    # equal parameters: the gradient of the sum edges is +-exp(logp) (kld_tests.jl:101-108)
+    P.update_parameters(p, pars)
+    P.update_parameters(q, pars)
+    g1, g2 = P.kld_backward(p, q)
+    np.testing.assert_allclose(g1[:2], np.exp(pars[:2]), rtol=1e-6)
+    np.testing.assert_allclose(g2[:2], -np.exp(pars[:2]), rtol=1e-6)
+
+
+@pytest.mark.parametrize("V,C,width,seed", [(5, 4, 3, 0), (12, 7, 4, 1)])
+def test_kld_and_gradient_match_oracle_random_dag(gpu, oracle, V, C, width, seed):
+    torch, P = gpu
+    O = oracle
+    from helpers import random_dag, rel_err
+    rng = np.random.default_rng(seed)
+    root = random_dag(V, C, rng, width=width)
+    fc1 = O.bits_compile(root, C, V)
+    p = _compile(P, root, V, C)
+    q = _compile(P, root, V, C)
+    pars = P.vectorize_parameters(p)
+    n_sum = p.num_inner_params()
+    # second parameterisation: perturbed leaves, re-drawn sum weights per group
+    p2 = _perturbed(pars, C, n_sum, rng)
+    sizes = p.table("pargroup_sizes")
+    pos = 0
+    for s in sizes:
+        w = rng.dirichlet(np.ones(s)) if s > 1 else np.ones(1)
+        p2[pos:pos + s] = np.log(w)
+        pos += s
+    P.update_parameters(q, p2)
+    fc2 = fc1.copy()
+    fc2.update_parameters(p2)
+    klds, ek = O.kld(fc1, fc2, double=True)
+    got = P.kld(p, q)
+    assert abs(got - klds[-1]) < KLD_RTOL * abs(klds[-1])
+    _, eg1, eg2, lg1, lg2 = O.kld_backward(fc1, fc2, ek, double=True)
+    g1, g2 = P.kld_backward(p, q)
+    w1, w2 = _grads_in_param_order(fc1, eg1, lg1), _grads_in_param_order(fc1, eg2, lg2)
+    assert np.abs(g1 - w1).max() < GRAD_RTOL * np.abs(w1).max()
+    assert np.abs(g2 - w2).max() < GRAD_RTOL * np.abs(w2).max()
+
+
+def _hclt_pair(P, O, V, K, C, seed):
+    from helpers import make_hclt, block_theta
+    parent, theta, leaf, fc = make_hclt(V, K, C, seed)
+    rng = np.random.default_rng(seed + 1)
+    theta2, leaf2 = O.random_hclt_params(parent, K, C, rng)
+    a = P.hclt_from_clt(parent, C, K)
+    a.set_params(block_theta(parent, K, theta), leaf)
+    b = P.hclt_from_clt(parent, C, K)
+    b.set_params(block_theta(parent, K, theta2), leaf2)
+    return parent, (theta, leaf), (theta2, leaf2), a, b
+
+
+def test_hclt_kld_and_gradient_match_oracle(gpu, oracle):
+    torch, P = gpu
+    O = oracle
+    V, K, C = 9, 16, 6
+    parent, (t1, l1), (t2, l2), a, b = _hclt_pair(P, O, V, K, C, 31)
+    fc1 = O.bits_compile(O.hclt_dag(parent, K, C, t1, l1), C, V)
+    fc2 = O.bits_compile(O.hclt_dag(parent, K, C, t2, l2), C, V)
+    klds, ek = O.kld(fc1, fc2, double=True)
+    got = P.kld(a, b)
+    assert got > 0 and abs(got - klds[-1]) < KLD_RTOL * abs(klds[-1])
+    assert abs(P.kld(a, a)) < 1e-5
+    _, eg1, eg2, lg1, lg2 = O.kld_backward(fc1, fc2, ek, double=True)
+    g1, g2 = P.kld_backward(a, b)
+    w1, w2 = _grads_in_param_order(fc1, eg1, lg1), _grads_in_param_order(fc1, eg2, lg2)
+    assert np.abs(g1 - w1).max() < GRAD_RTOL * np.abs(w1).max()
+    assert np.abs(g2 - w2).max() < GRAD_RTOL * np.abs(w2).max()
+
+
+def _gumbel(rng, shape):
+    u = rng.random(shape)
+    return (-np.log(-np.log(np.clip(u, 1e-12, 1 - 1e-12)))).astype(np.float32)
+
+
+@pytest.mark.parametrize("V,C,width,B,seed", [(5, 4, 3, 100, 0), (12, 7, 4, 257, 1), (6, 256, 3, 64, 2)])
+def test_sampling_bit_exact_random_dag(gpu, oracle, V, C, width, B, seed):
+    torch, P = gpu
+    O = oracle
+    from helpers import random_dag
+    rng = np.random.default_rng(seed)
+    root = random_dag(V, C, rng, width=width)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, root, V, C)
+    n_sum = bpc.num_inner_params()
+    node_noise = _gumbel(rng, (B, n_sum))
+    leaf_noise = _gumbel(rng, (B, V, C))
+    # oracle edges are in CSR order: slot of an edge = its parameter index
+    slot = np.zeros(fc.n_edges, np.int64)
+    slot[fc.sum_param_edges()] = np.arange(n_sum)
+    want = O.sample(fc, node_noise, leaf_noise, noise_slot=slot)
+    got = P.sample(bpc, torch.from_numpy(node_noise).cuda(), torch.from_numpy(leaf_noise).cuda()).cpu().numpy()
+    assert got.dtype == np.uint8 and got.shape == (B, V)
+    assert np.array_equal(got, want)
+    assert (got < C).all()
+
+
+@pytest.mark.parametrize("V,K,C,B", [(7, 16, 8, 130), (12, 32, 256, 64)])
+def test_sampling_bit_exact_hclt(gpu, oracle, V, K, C, B):
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta
+    parent, theta, leaf, fc = make_hclt(V, K, C, 5 + V)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    ch, root = O.clt_children(parent)
+    inner = [v for v in O.clt_bottom_up(parent) if ch[v]]
+    rng = np.random.default_rng(V)
+    node_noise = _gumbel(rng, (B, len(inner) * K))
+    leaf_noise = _gumbel(rng, (B, V, C))
+    slot = np.zeros(fc.n_edges, np.int64)
+    for r, v in enumerate(inner):
+        nk = len(fc.meta["sum_node"][v])
+        e0 = fc.meta["edge_of"][v]
+        slot[e0:e0 + nk * K] = np.tile(r * K + np.arange(K), nk)
+    want = O.sample(fc, node_noise, leaf_noise, noise_slot=slot)
+    got = P.sample(bpc, torch.from_numpy(node_noise).cuda(), torch.from_numpy(leaf_noise).cuda()).cpu().numpy()
+    assert np.array_equal(got, want)
+
+
+def test_sampling_follows_the_circuit_distribution(gpu, oracle):
+    """With Gumbel noise the samples are exact draws: empirical frequencies of the joint on a
+    tiny circuit approach the circuit's probabilities."""
+    torch, P = gpu
+    O = oracle
+    import itertools
+    from helpers import random_dag
+    V, C, B = 3, 3, 60000
+    rng = np.random.default_rng(9)
+    root = random_dag(V, C, rng, width=2)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, root, V, C)
+    allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    prob = np.exp(O.forward(fc, allx, double=True)[-1])
+    g = torch.Generator(device="cuda").manual_seed(1)
+    u1 = torch.rand((B, bpc.num_inner_params()), device="cuda", generator=g).clamp_(1e-10, 1 - 1e-7)
+    u2 = torch.rand((B, V, C), device="cuda", generator=g).clamp_(1e-10, 1 - 1e-7)
+    s = P.sample(bpc, -torch.log(-torch.log(u1)), -torch.log(-torch.log(u2))).cpu().numpy().astype(np.int64)
+    code = (s * (C ** np.arange(V - 1, -1, -1))).sum(axis=1)
+    freq = np.bincount(code, minlength=C ** V) / B
+    assert np.abs(freq - prob).max() < 5 * np.sqrt(prob.max() / B) + 1e-3
+
+
+def test_adam_step_matches_oracle(gpu, oracle):
+    """src/sgd/adam.jl:318-319, :63-76, :88-127 on an HCLT and on a general circuit."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, random_dag, rel_err
+    V, K, C = 6, 16, 5
+    parent, theta, leaf, fc = make_hclt(V, K, C, 41)
+    hc = P.hclt_from_clt(parent, C, K)
+    hc.set_params(block_theta(parent, K, theta), leaf)
+    gc = _compile(P, random_dag(8, 4, np.random.default_rng(3), width=4), 8, 4)
+    for bpc in (hc, gc):
+        n_sum = bpc.num_inner_params()
+        rng = np.random.default_rng(n_sum)
+        before = P.vectorize_parameters(bpc)
+        params = before[:n_sum].copy() + rng.normal(0, 0.1, n_sum).astype(np.float32)
+        m = rng.normal(0, 0.01, n_sum).astype(np.float32)
+        v = (rng.random(n_sum) * 1e-3).astype(np.float32)
+        sizes = bpc.table("pargroup_sizes")
+        group_ptr = np.concatenate([[0], np.cumsum(sizes)])
+        dp, dm, dv = (torch.from_numpy(x.copy()).cuda() for x in (params, m, v))
+        rp, rm, rv = params.copy(), m.copy(), v.copy()
+        logp_ref = before[:n_sum].copy()
+        for t in (1, 2, 3):
+            grad = rng.normal(0, 1, n_sum).astype(np.float32)
+            P.adam_step(bpc, torch.from_numpy(grad).cuda(), dp, dm, dv, lr=1e-2, t=t)
+            O.adam_step(rp, grad, rm, rv, 1e-2, 0.9, 0.999, 1e-8, t, group_ptr, logp_ref)
+        np.testing.assert_allclose(dp.cpu().numpy(), rp, rtol=ADAM_RTOL, atol=1e-6)
+        np.testing.assert_allclose(dm.cpu().numpy(), rm, rtol=ADAM_RTOL, atol=1e-8)
+        np.testing.assert_allclose(dv.cpu().numpy(), rv, rtol=ADAM_RTOL, atol=1e-10)
+        after = P.vectorize_parameters(bpc)
+        assert rel_err(np.exp(after[:n_sum]), np.exp(logp_ref)).max() < 1e-5
+        assert np.array_equal(after[n_sum:], before[n_sum:])        # leaves untouched
+        # every sum node with more than one edge is normalised
+        pos = 0
+        for s in sizes:
+            if s > 1:
+                assert abs(np.exp(after[pos:pos + s].astype(np.float64)).sum() - 1) < 1e-5
+            pos += s
+    # the dense engine sees the new parameters too
+    th, _ = hc.get_params()
+    ch, root = O.clt_children(parent)
+    v0 = next(v for v in range(V) if ch[v] and v != root)
+    assert np.abs(np.exp(th[v0].astype(np.float64)).sum(axis=1) - 1).max() < 1e-5
