@@ -1,0 +1,124 @@
+"""CPU-side checks: the C-ABI library loads and exports every symbol the header declares,
+argument errors are reported as status codes without touching a GPU, and the host-side
+workload builders are deterministic and well-formed."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pcmi355.h")
+LIB = os.path.join(ROOT, "lvd-pg_amd", "libpcmi355.so")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pcm_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def cdll():
+    assert os.path.exists(LIB), "build the library first: python lvd-pg_amd/build.py"
+    return ctypes.CDLL(LIB)
+
+
+def test_header_declares_the_whole_path():
+    names = declared_symbols()
+    for must in ("pcm_hclt_create", "pcm_circuit_create", "pcm_loglikelihoods", "pcm_flows", "pcm_em_update",
+                 "pcm_em_step", "pcm_kld", "pcm_kld_backward", "pcm_sample", "pcm_adam_step",
+                 "pcm_vectorize_parameters", "pcm_update_parameters", "pcm_index_table", "pcm_free"):
+        assert must in names
+    assert len(names) >= 25
+
+
+def test_library_exports_every_declared_symbol(cdll):
+    missing = [n for n in declared_symbols() if not hasattr(cdll, n)]
+    assert not missing, missing
+
+
+def test_version_and_error_reporting_without_a_gpu(cdll):
+    cdll.pcm_last_error.restype = ctypes.c_char_p
+    assert cdll.pcm_version() >= 1
+    out = ctypes.c_void_p()
+    # null tree
+    rc = cdll.pcm_hclt_create(None, 4, 16, 8, ctypes.byref(out))
+    assert rc == -1 and out.value is None
+    assert b"null" in cdll.pcm_last_error().lower() or len(cdll.pcm_last_error()) > 0
+    # unsupported hidden size and a malformed tree are rejected before any device work
+    par = (ctypes.c_int32 * 3)(-1, 0, 0)
+    assert cdll.pcm_hclt_create(par, 3, 7, 8, ctypes.byref(out)) in (-1, -2, -3)
+    two_roots = (ctypes.c_int32 * 3)(-1, -1, 0)
+    assert cdll.pcm_hclt_create(two_roots, 3, 16, 8, ctypes.byref(out)) == -2
+    cycle = (ctypes.c_int32 * 3)(-1, 2, 1)
+    assert cdll.pcm_hclt_create(cycle, 3, 16, 8, ctypes.byref(out)) == -2
+    # null handles
+    cdll.pcm_size.restype = ctypes.c_int64
+    assert cdll.pcm_size(None, 0) < 0
+    assert cdll.pcm_em_update(None, ctypes.c_float(0.1), ctypes.c_float(0.9)) == -1
+    assert cdll.pcm_free(None) in (0, -1)
+
+
+def test_python_mirror_binds_every_symbol():
+    import pcmi355._lib as L
+    for n in declared_symbols():
+        assert hasattr(L.lib, n), n
+
+
+def test_workload_builders():
+    from pcmi355 import workloads as W
+    a = W.grf_images(64, 8, 8, 3, 2.0, 0.8, seed=5)
+    b = W.grf_images(64, 8, 8, 3, 2.0, 0.8, seed=5)
+    assert a.dtype == np.uint8 and a.shape == (64, 192) and np.array_equal(a, b)
+    assert a.min() == 0 and a.max() == 255
+    # neighbouring pixels are correlated, distant channels share the base field
+    x = a.astype(np.float64)
+    assert np.corrcoef(x[:, 0], x[:, 1])[0, 1] > 0.5
+    parent = W.chow_liu_parent(a)
+    assert (parent < 0).sum() == 1 and len(parent) == 192
+    # a tree: every node reaches the root without cycles
+    root = int(np.nonzero(parent < 0)[0][0])
+    for v in range(192):
+        seen, u = 0, v
+        while u != root:
+            u = parent[u]
+            seen += 1
+            assert seen <= 192
+    st = W.tree_stats(parent)
+    assert st["n_inner"] + st["n_leaf"] == 192 and st["depth"] >= 1
+    th, lf = W.init_params(parent, 4, 6, 1)
+    np.testing.assert_allclose(np.exp(th.astype(np.float64)).sum(-1), 1, rtol=1e-5)
+    np.testing.assert_allclose(np.exp(lf.astype(np.float64)).sum(-1), 1, rtol=1e-5)
+    ratio = np.exp(th.max(-1) - th.min(-1))
+    assert ratio.max() <= 1.4 / 0.6 + 1e-3      # init_parameters(perturbation = 0.4)
+
+
+def test_algorithmic_bytes_formula():
+    """Per-kernel bookings add up to the step formula: 6 vectors of K floats per (inner tree
+    node, example), the batch once, the sum parameters three times, the leaf tables five."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    n_int, V, K, C, B = 2505, 3072, 32, 256, 4096
+    ab = bench.algorithmic_bytes(n_int, V, K, C, B)
+    edges = (n_int - 1) * K * K + K
+    assert ab["step"] == n_int * 6 * K * 4 * B + V * B + 3 * 4 * edges + 5 * 4 * V * K * C
+    assert ab["forward"] == n_int * 2 * K * 4 * B + V * B + 4 * edges + 4 * V * K * C
+
+
+def test_describe_dag_is_topological():
+    from helpers import describe_dag, random_dag, simple_multihead_circuit
+    import pc_oracle as O
+    d = describe_dag([random_dag(7, 3, np.random.default_rng(0), width=3)])
+    n = len(d["node_type"])
+    for i in range(n):
+        kids = d["child_idx"][d["child_ptr"][i]:d["child_ptr"][i + 1]]
+        assert (kids < i).all()
+        assert (d["node_type"][i] == O.INPUT) == (len(kids) == 0)
+    assert len(d["input_logp"]) == 3 * (d["node_type"] == O.INPUT).sum()
+    heads = simple_multihead_circuit(5)
+    d = describe_dag(heads)
+    assert d["node_type"][-2:].tolist() == [O.SUM, O.SUM] and len(d["node_type"]) == 10

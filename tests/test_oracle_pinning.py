@@ -1,0 +1,492 @@
+"""Pins the CPU oracle (test infrastructure) against facts that do not depend on it:
+brute-force enumeration of latent states, closed forms and known answers quoted from the
+reference's own tests, finite differences in float64, textbook EM properties, and the
+statistics of exact samples.  A dropped term, a transposed parameter block, a wrong child
+or a wrong sign fails at least one of these."""
+import itertools
+
+import numpy as np
+import pytest
+from scipy.special import logsumexp
+
+import pc_oracle as O
+from helpers import (make_hclt, correlated_data, simple_3vars_circuit, simple_multihead_circuit, random_dag,
+                     log_dirichlet)
+
+
+# ------------------------------------------------------------------------------------
+# forward
+# ------------------------------------------------------------------------------------
+
+def brute_force_hclt_ll(parent, K, theta, leaf, x):
+    """log p(x) of the HCLT of src/structures/hclts.jl:100-145 by summing the joint over
+    every assignment of the inner tree nodes' hidden states (float64).  Hidden state of
+    tree node v: j_v; its sum parameters are theta_v[j_parent(v), j_v] (the root's parent
+    state is 0, :137 keeps circuits[1]); observed leaf of v: leaf[v, j_v, x_v]; a leaf
+    tree node c has no state of its own and contributes leaf[c, j_parent(c), x_c]."""
+    ch, root = O.clt_children(parent)
+    inner = [v for v in range(len(parent)) if ch[v]]
+    total = -np.inf
+    for states in itertools.product(range(K), repeat=len(inner)):
+        j = dict(zip(inner, states))
+        lp = 0.0
+        for v in inner:
+            jp = 0 if v == root else j[parent[v]]
+            lp += float(theta[v][jp, j[v]]) + float(leaf[v, j[v], x[v]])
+            for c in ch[v]:
+                if not ch[c]:
+                    lp += float(leaf[c, j[v], x[c]])
+        total = np.logaddexp(total, lp)
+    return total
+
+
+@pytest.mark.parametrize("tree,K,C", [([-1, 0], 3, 4), ([-1, 0, 0], 2, 3), ([-1, 0, 1, 1], 3, 2), ([1, -1, 1, 0, 0, 0], 2, 3),
+                                      ([-1, 0, 1, 2, 3], 3, 3), ([-1, 0, 0, 1, 1, 2], 2, 2)])
+def test_forward_equals_latent_enumeration(tree, K, C):
+    parent = np.array(tree, np.int32)
+    V = len(parent)
+    rng = np.random.default_rng(V * 10 + K)
+    theta, leaf = O.random_hclt_params(parent, K, C, rng)
+    data = rng.integers(0, C, size=(12, V)).astype(np.uint8)
+    want = np.array([brute_force_hclt_ll(parent, K, theta, leaf, x) for x in data])
+    for fc in (O.hclt_flat(parent, K, C, theta, leaf), O.bits_compile(O.hclt_dag(parent, K, C, theta, leaf), C, V)):
+        got64 = O.forward(fc, data, double=True)[-1]
+        np.testing.assert_allclose(got64, want, rtol=1e-6)          # parameters are float32 draws
+        got32 = O.forward(fc, data)[-1]
+        np.testing.assert_allclose(got32, want, rtol=2e-6)
+
+
+def test_forward_is_a_normalised_distribution():
+    for parent, K, C in [([-1, 0, 0, 1], 3, 3), ([-1, 0, 1, 1, 3], 2, 2)]:
+        parent = np.array(parent, np.int32)
+        V = len(parent)
+        _, _, _, fc = make_hclt(V, K, C, 4, parent=parent)
+        allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+        assert abs(np.exp(O.forward(fc, allx, double=True)[-1]).sum() - 1) < 1e-6
+    root = random_dag(5, 3, np.random.default_rng(1), width=3)
+    fc = O.bits_compile(root, 3, 5)
+    allx = np.array(list(itertools.product(range(3), repeat=5)), np.uint8)
+    assert abs(np.exp(O.forward(fc, allx, double=True)[-1]).sum() - 1) < 1e-6
+
+
+def test_pairwise_logsumexp_matches_scipy():
+    """Sum nodes fold their edges with the pairwise logsumexp (src/queries/likelihood.jl:101-102)."""
+    rng = np.random.default_rng(0)
+    C = 2
+    for m in (2, 3, 9):
+        w = log_dirichlet(rng, m)
+        leaves = [O.input_node(0, log_dirichlet(rng, C)) for _ in range(m)]
+        fc = O.bits_compile(O.summate(*leaves, logps=w), C, 1)
+        data = np.array([[0], [1]], np.uint8)
+        got = O.forward(fc, data)[-1]
+        for b in range(2):
+            want = logsumexp([w[i] + leaves[i].logps[data[b, 0]] for i in range(m)])
+            assert abs(got[b] - want) < 1e-6
+
+
+def test_three_var_fixture_likelihood():
+    """test/queries/likelihood_tests.jl:24-37: with uniform leaves over 5 categories the
+    product nodes evaluate to 3*log(1/5) and the root to logsumexp of the two branches."""
+    root = simple_3vars_circuit(5, weights=[0.25, 0.75])
+    fc = O.bits_compile(root, 5, 3)
+    data = np.array([[0, 1, 2], [4, 4, 4]], np.uint8)
+    mars = O.forward(fc, data)
+    np.testing.assert_allclose(mars[-1], 3 * np.log(0.2), rtol=1e-6)
+    assert fc.n_nodes == 9 and (fc.type == O.MUL).sum() == 2
+    for n in np.nonzero(fc.type == O.MUL)[0]:
+        np.testing.assert_allclose(mars[n], 3 * np.log(0.2), rtol=1e-6)
+
+
+# ------------------------------------------------------------------------------------
+# flattening and index tables: known answers held by the reference's tests
+# ------------------------------------------------------------------------------------
+
+def test_three_var_fixture_index_tables():
+    """test/bits_circuit_tests.jl:13-24 and test/misc_tests.jl:39-62."""
+    fc = O.bits_compile(simple_3vars_circuit(5), 5, 3)
+    t = fc.param_tables()
+    assert fc.n_nodes == 9 and fc.n_edges == 6
+    assert t["edge2param"].tolist() == [0, 0, 0, 0, 1, 2]
+    assert t["param2edge"].tolist() == [5, 6]
+    assert t["param2group"].tolist() == [1, 1]
+    assert t["pargroup_sizes"].tolist() == [2]
+    assert t["innode2ncumparam"].tolist() == [5, 10, 15, 20, 25, 30]
+    assert t["num_input_params"] == 30
+    assert len(fc.vectorize_parameters()) == 32
+
+
+def test_vectorize_update_roundtrip():
+    """test/misc_tests.jl:14-36: update_parameters(vectorize_parameters()) is the identity and
+    a changed vector lands in the circuit."""
+    rng = np.random.default_rng(2)
+    fc = O.bits_compile(random_dag(6, 4, rng, width=3), 4, 6)
+    p = fc.vectorize_parameters()
+    q = rng.normal(size=len(p)).astype(np.float32)
+    g = fc.copy()
+    g.update_parameters(q)
+    assert np.array_equal(g.vectorize_parameters(), q)
+    g.update_parameters(p)
+    assert np.array_equal(g.logp, fc.logp) and np.array_equal(g.leaf_logp, fc.leaf_logp)
+
+
+def test_multihead_node_numbering_and_closed_forms():
+    """test/multi_head_pc/multi_head_pc_learning_tests.jl:11-47: shared products become nodes
+    4 and 8, heads 9 and 10, fake root 11 (1-based); LL closed forms."""
+    heads = simple_multihead_circuit(5)
+    heads[0].children[0].children[0].logps = np.log(np.array([0.1, 0.2, 0.3, 0.3, 0.1], np.float32))
+    heads[0].logps = np.log(np.array([0.2, 0.8], np.float32))
+    heads[1].logps = np.log(np.array([0.6, 0.4], np.float32))
+    fc = O.bits_compile(O.summate(*heads), 5, 3)
+    assert fc.n_nodes == 11
+    assert fc.type.tolist() == [0, 0, 0, 2, 0, 0, 0, 2, 1, 1, 1]
+    data = np.array([[0, 0, 0], [2, 0, 0]], np.uint8)
+    mars = O.forward(fc, data)
+    np.testing.assert_allclose(mars[8, 0], np.log(0.1 * 0.2 * 0.2 * 0.2 + 0.2 ** 3 * 0.8), rtol=1e-6)
+    np.testing.assert_allclose(mars[9, 1], np.log(0.3 * 0.2 * 0.2 * 0.6 + 0.2 ** 3 * 0.4), rtol=1e-6)
+    skip = (fc.edge_parent() == 10).astype(np.uint8)
+    mask = np.array([[1.0, 0.0], [0.0, 1.0]], np.float32)       # [head, example]
+    flows, _ = O.backward(fc, mars, skip=skip, root_ids=np.array([8, 9], np.int32), root_flow=mask)
+    assert flows[8, 0] == 1 and flows[9, 0] == 0 and flows[8, 1] == 0 and flows[9, 1] == 1
+    assert (flows[10] == 0).all()
+    f32 = np.float32
+    np.testing.assert_allclose(flows[3, 0], np.exp(mars[0, 0] + mars[1, 0] + mars[2, 0] + np.log(f32(0.2)) - mars[8, 0]), rtol=1e-5)
+    np.testing.assert_allclose(flows[7, 0], np.exp(mars[4, 0] + mars[5, 0] + mars[6, 0] + np.log(f32(0.8)) - mars[8, 0]), rtol=1e-5)
+    np.testing.assert_allclose(flows[3, 1], np.exp(mars[0, 1] + mars[1, 1] + mars[2, 1] + np.log(f32(0.6)) - mars[9, 1]), rtol=1e-5)
+    np.testing.assert_allclose(flows[7, 1], np.exp(mars[4, 1] + mars[5, 1] + mars[6, 1] + np.log(f32(0.4)) - mars[9, 1]), rtol=1e-5)
+
+
+def test_hclt_flat_is_the_flattened_dag():
+    """The direct HCLT builder and the generic flattening give the same function and the
+    same multiset of parameters (node numbering differs)."""
+    parent, theta, leaf, flat = make_hclt(7, 3, 4, 8)
+    dag = O.bits_compile(O.hclt_dag(parent, 3, 4, theta, leaf), 4, 7)
+    assert flat.n_nodes == dag.n_nodes and flat.n_edges == dag.n_edges
+    data = correlated_data(40, 7, 4, 9, parent)
+    np.testing.assert_allclose(O.forward(flat, data)[-1], O.forward(dag, data)[-1], rtol=1e-6)
+    assert np.array_equal(np.sort(flat.vectorize_parameters()), np.sort(dag.vectorize_parameters()))
+
+
+# ------------------------------------------------------------------------------------
+# flows
+# ------------------------------------------------------------------------------------
+
+def _total_ll(fc, data):
+    return O.forward(fc, data, double=True)[-1].sum()
+
+
+@pytest.mark.parametrize("kind", ["hclt", "dag"])
+def test_flows_are_the_gradient_of_the_log_likelihood(kind):
+    """edge_aggr[e] = sum_b d log p(x_b) / d logp_e and leaf_flow[n, c] = sum_b d log p(x_b) /
+    d leaf_logp[n, c], checked by central differences in float64 on every parameter."""
+    if kind == "hclt":
+        parent, theta, leaf, fc = make_hclt(5, 3, 3, 12)
+        data = correlated_data(9, 5, 3, 13, parent)
+    else:
+        fc = O.bits_compile(random_dag(5, 3, np.random.default_rng(3), width=2), 3, 5)
+        data = np.random.default_rng(4).integers(0, 3, size=(9, 5)).astype(np.uint8)
+    fc.logp = fc.logp.astype(np.float64)
+    fc.leaf_logp = fc.leaf_logp.astype(np.float64)
+    mars = O.forward(fc, data, double=True)
+    flows, ea = O.backward(fc, mars, double=True)
+    lf = O.input_flows(fc, data, flows, double=True)
+    h = 1e-6
+    par = fc.edge_parent()
+    for e in range(fc.n_edges):
+        if fc.type[par[e]] != O.SUM:
+            continue
+        g = fc.copy()
+        g.logp[e] += h
+        up = _total_ll(g, data)
+        g.logp[e] -= 2 * h
+        fd = (up - _total_ll(g, data)) / (2 * h)
+        assert abs(fd - ea[e]) < 1e-6 * max(1.0, abs(ea[e])), e
+    for i in range(len(fc.leaf_logp)):
+        g = fc.copy()
+        g.leaf_logp[i] += h
+        up = _total_ll(g, data)
+        g.leaf_logp[i] -= 2 * h
+        fd = (up - _total_ll(g, data)) / (2 * h)
+        assert abs(fd - lf[i]) < 1e-6 * max(1.0, abs(lf[i])), i
+
+
+def test_flow_invariants():
+    """test/queries/flow_tests.jl:44-64, 97-114: the root's flow is 1, a sum node's edge flows
+    are flow * exp(edge_mar - node_mar) and add up to the node's flow; in an HCLT the K sum
+    nodes of a tree node share one unit of flow per example; edge_aggr is the batch sum."""
+    parent, theta, leaf, fc = make_hclt(8, 4, 5, 15)
+    data = correlated_data(30, 8, 5, 16, parent)
+    mars = O.forward(fc, data)
+    flows, ea = O.backward(fc, mars)
+    assert np.all(flows[-1] == 1)
+    for v, ids in fc.meta["sum_node"].items():
+        np.testing.assert_allclose(flows[ids].sum(axis=0), 1.0, rtol=2e-5)
+    par = fc.edge_parent()
+    for n in np.nonzero(fc.type == O.SUM)[0]:
+        tot = np.zeros(30)
+        for e in range(fc.edge_ptr[n], fc.edge_ptr[n + 1]):
+            em = mars[fc.prime[e]] + (mars[fc.sub[e]] if fc.sub[e] >= 0 else 0) + fc.logp[e]
+            ef = flows[n] * np.exp(em - mars[n])
+            np.testing.assert_allclose(ea[e], ef.sum(), rtol=1e-4, atol=1e-6)
+            tot += ef
+        np.testing.assert_allclose(tot, flows[n], rtol=1e-4, atol=1e-7)
+    lf = O.input_flows(fc, data, flows)
+    np.testing.assert_allclose(lf.reshape(8, -1).sum(axis=1), 30.0, rtol=1e-4)
+
+
+# ------------------------------------------------------------------------------------
+# EM update
+# ------------------------------------------------------------------------------------
+
+def test_em_update_formulas_by_hand():
+    """add_pseudocount / aggr_node_flows / update_params (src/pretrain/mini_batch_warmup.jl:4-17,
+    :54-70) and the leaf update (src/nodes/fixable_categorical_dist.jl:223-248) on one sum
+    node over three leaves, computed by hand."""
+    C = 4
+    w = np.array([0.5, 0.3, 0.2], np.float32)
+    lps = [np.log(np.array(p, np.float32)) for p in ([0.1, 0.2, 0.3, 0.4], [0.25, 0.25, 0.25, 0.25], [0.7, 0.1, 0.1, 0.1])]
+    fc = O.bits_compile(O.summate(*[O.input_node(0, lp) for lp in lps], logps=np.log(w)), C, 1)
+    ea = np.array([3.0, 1.0, 0.5], np.float32)
+    lf = np.array([[1, 0, 2, 0], [0, 0.5, 0, 0.5], [0.25, 0.25, 0, 0]], np.float32)
+    pc, inertia = 0.6, 0.3
+    logp, leaf = O.em_update(fc, ea, lf.reshape(-1), pc, inertia)
+    e = ea.astype(np.float64) + pc / 3
+    want = inertia * w + (1 - inertia) * e / e.sum()
+    np.testing.assert_allclose(np.exp(logp), want, rtol=1e-6)
+    for i in range(3):
+        nf = lf[i].sum() + pc
+        want = inertia * np.exp(lps[i]) + (1 - inertia) * (lf[i] + pc / C) / nf
+        np.testing.assert_allclose(np.exp(leaf[i * C:(i + 1) * C]), want, rtol=1e-6)
+
+
+def test_em_is_convex_mix_and_exact_m_step():
+    """test/regularization custom_em_tests.jl:207 (new = inertia*old + (1-inertia)*target);
+    with pseudocount 0 and inertia 0 the step is the exact M-step: the full-batch
+    log-likelihood never decreases and parameters stay normalised."""
+    parent, theta, leaf, fc = make_hclt(6, 3, 4, 18)
+    data = correlated_data(200, 6, 4, 19, parent)
+    idx = np.arange(200, dtype=np.int32)
+    _, logp0, leaf0, ea, lf = O.em_step(fc, data, idx, 0.1, 0.0, double=True)
+    _, logp3, leaf3, _, _ = O.em_step(fc, data, idx, 0.1, 0.3, double=True)
+    par = fc.edge_parent()
+    issum = fc.type[par] == O.SUM
+    np.testing.assert_allclose(np.exp(logp3[issum]), 0.3 * np.exp(fc.logp[issum].astype(np.float64)) + 0.7 * np.exp(logp0[issum]), rtol=1e-9)
+    np.testing.assert_allclose(np.exp(leaf3), 0.3 * np.exp(fc.leaf_logp.astype(np.float64)) + 0.7 * np.exp(leaf0), rtol=1e-9)
+    cur = fc.copy()
+    cur.logp = cur.logp.astype(np.float64)
+    cur.leaf_logp = cur.leaf_logp.astype(np.float64)
+    prev = -np.inf
+    for _ in range(6):
+        ll, logp, lf_new, _, _ = O.em_step(cur, data, idx, 0.0, 0.0, double=True)
+        assert ll.sum() >= prev - 1e-9
+        prev = ll.sum()
+        cur.logp, cur.leaf_logp = logp, lf_new
+    for n in np.nonzero(fc.type == O.SUM)[0]:
+        s = np.exp(cur.logp[fc.edge_ptr[n]:fc.edge_ptr[n + 1]]).sum()
+        assert abs(s - 1) < 1e-9
+    assert np.abs(np.exp(cur.leaf_logp).reshape(-1, 4).sum(axis=1) - 1).max() < 1e-9
+
+
+# ------------------------------------------------------------------------------------
+# KL recursion
+# ------------------------------------------------------------------------------------
+
+def _three_var_pair(seed=0):
+    root = simple_3vars_circuit(5, np.random.default_rng(seed), weights=[0.45, 0.55])
+    fc = O.bits_compile(root, 5, 3)
+    return fc, fc.vectorize_parameters()
+
+
+def test_kld_closed_forms():
+    """test/queries/kld_tests.jl:9-70."""
+    fc, pars = _three_var_pair()
+    klds, ek = O.kld(fc, fc.copy())
+    assert np.allclose(klds, 0) and np.allclose(ek, 0)
+    for a, b in [((0.2, 0.8), (0.4, 0.6)), ((0.5, 0.5), (0.9, 0.1))]:
+        f1, f2 = fc.copy(), fc.copy()
+        p1, p2 = pars.copy(), pars.copy()
+        p1[:2], p2[:2] = np.log(np.float32(a)), np.log(np.float32(b))
+        f1.update_parameters(p1)
+        f2.update_parameters(p2)
+        want = a[0] * np.log(a[0] / b[0]) + a[1] * np.log(a[1] / b[1])
+        np.testing.assert_allclose(O.kld(f1, f2)[0][-1], want, rtol=1e-5)
+    for w, l1, l2 in [(0.2, [0.1, 0.2, 0.3, 0.2, 0.2], [0.2, 0.1, 0.1, 0.3, 0.3]),
+                      (0.5, [0.1, 0.2, 0.3, 0.2, 0.2], [0.2, 0.1, 0.2, 0.3, 0.2])]:
+        f1, f2 = fc.copy(), fc.copy()
+        p1, p2 = pars.copy(), pars.copy()
+        p1[:2] = p2[:2] = np.log(np.float32([w, 1 - w]))
+        p1[2:7], p2[2:7] = np.log(np.float32(l1)), np.log(np.float32(l2))
+        f1.update_parameters(p1)
+        f2.update_parameters(p2)
+        want = np.sum(np.exp(p1[2:7]) * (p1[2:7] - p2[2:7])) * w
+        np.testing.assert_allclose(O.kld(f1, f2)[0][-1], want, rtol=1e-5)
+
+
+def test_kld_backward_closed_forms():
+    """test/queries/kld_tests.jl:101-131 (edges 5 and 6 are the root's sum edges)."""
+    fc, pars = _three_var_pair(1)
+    klds, ek = O.kld(fc, fc.copy())
+    _, eg1, eg2, _, _ = O.kld_backward(fc, fc.copy(), ek)
+    order = fc.up_order()
+    eg1, eg2 = eg1[order], eg2[order]
+    np.testing.assert_allclose(eg1[4:6], np.exp(pars[:2]), rtol=1e-6)
+    np.testing.assert_allclose(eg2[4:6], -eg1[4:6], rtol=1e-6)
+    assert np.all(eg1[:4] == 0) and np.all(eg2[:4] == 0)
+    f1, f2 = fc.copy(), fc.copy()
+    p1, p2 = pars.copy(), pars.copy()
+    p1[:2], p2[:2] = np.log(np.float32([0.2, 0.8])), np.log(np.float32([0.4, 0.6]))
+    f1.update_parameters(p1)
+    f2.update_parameters(p2)
+    klds, ek = O.kld(f1, f2)
+    _, eg1, eg2, _, _ = O.kld_backward(f1, f2, ek)
+    eg1, eg2 = eg1[order], eg2[order]
+    np.testing.assert_allclose(eg1[4], 0.2 * (np.log(0.2) - np.log(0.4) + 1), rtol=1e-5)
+    np.testing.assert_allclose(eg2[4], -0.2, rtol=1e-6)
+    np.testing.assert_allclose(eg1[5], 0.8 * (np.log(0.8) - np.log(0.6) + 1), rtol=1e-5)
+    np.testing.assert_allclose(eg2[5], -0.8, rtol=1e-6)
+
+
+def test_kld_equals_brute_force_on_a_deterministic_circuit():
+    """A fully factorised circuit: KL is the sum of the per-variable KLs; and a mixture whose
+    branches have disjoint support (deterministic): KL = sum_x p log(p/q) by enumeration."""
+    rng = np.random.default_rng(6)
+    C, V = 3, 3
+    # deterministic mixture: branch i puts variable 0 on category i only
+    def circuit():
+        branches = []
+        for i in range(C):
+            lp0 = np.full(C, -80.0, np.float32)
+            lp0[i] = 0.0
+            branches.append(O.multiply(O.input_node(0, lp0), O.input_node(1, log_dirichlet(rng, C)),
+                                       O.input_node(2, log_dirichlet(rng, C))))
+        return O.summate(*branches, logps=log_dirichlet(rng, C))
+    f1 = O.bits_compile(circuit(), C, V)
+    f2 = O.bits_compile(circuit(), C, V)
+    allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    lp = O.forward(f1, allx, double=True)[-1]
+    lq = O.forward(f2, allx, double=True)[-1]
+    want = np.sum(np.exp(lp) * (lp - lq))
+    got = O.kld(f1, f2, double=True)[0][-1]
+    np.testing.assert_allclose(got, want, rtol=1e-6)
+
+
+def test_kld_gradient_by_finite_differences():
+    """The recursion's reverse pass against central differences of the forward recursion in
+    float64 (sum edges; leaves with the analytic leaf derivative)."""
+    rng = np.random.default_rng(7)
+    root = random_dag(4, 3, rng, width=2)
+    f1 = O.bits_compile(root, 3, 4)
+    f2 = f1.copy()
+    f2.update_parameters((f1.vectorize_parameters() + rng.normal(0, 0.3, len(f1.vectorize_parameters()))).astype(np.float32))
+    for f in (f1, f2):
+        f.logp = f.logp.astype(np.float64)
+        f.leaf_logp = f.leaf_logp.astype(np.float64)
+    klds, ek = O.kld(f1, f2, double=True)
+    _, eg1, eg2, lg1, lg2 = O.kld_backward(f1, f2, ek, analytic=True, double=True)
+    h = 1e-6
+    par = f1.edge_parent()
+
+    def val(a, b):
+        return O.kld(a, b, double=True)[0][-1]
+
+    for e in range(f1.n_edges):
+        if f1.type[par[e]] != O.SUM:
+            assert eg1[e] == 0 and eg2[e] == 0
+            continue
+        for which, want in ((0, eg1[e]), (1, eg2[e])):
+            a, b = f1.copy(), f2.copy()
+            t = (a, b)[which]
+            t.logp[e] += h
+            up = val(a, b)
+            t.logp[e] -= 2 * h
+            fd = (up - val(a, b)) / (2 * h)
+            assert abs(fd - want) < 1e-6 * max(1, abs(want)), (e, which)
+    for i in range(len(f1.leaf_logp)):
+        for which, want in ((0, lg1[i]), (1, lg2[i])):
+            a, b = f1.copy(), f2.copy()
+            t = (a, b)[which]
+            t.leaf_logp[i] += h
+            up = val(a, b)
+            t.leaf_logp[i] -= 2 * h
+            fd = (up - val(a, b)) / (2 * h)
+            assert abs(fd - want) < 1e-6 * max(1, abs(want)), (i, which)
+
+
+# ------------------------------------------------------------------------------------
+# sampling
+# ------------------------------------------------------------------------------------
+
+def _gumbel(rng, shape):
+    return -np.log(-np.log(rng.random(shape).clip(1e-12, 1 - 1e-12)))
+
+
+def test_gumbel_max_samples_follow_the_circuit():
+    rng = np.random.default_rng(8)
+    V, C, B = 3, 3, 40000
+    fc = O.bits_compile(random_dag(V, C, rng, width=2), C, V)
+    allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    prob = np.exp(O.forward(fc, allx, double=True)[-1])
+    s = O.sample(fc, _gumbel(rng, (B, fc.n_edges)), _gumbel(rng, (B, V, C))).astype(np.int64)
+    assert (s < C).all()
+    code = (s * (C ** np.arange(V - 1, -1, -1))).sum(axis=1)
+    freq = np.bincount(code, minlength=C ** V) / B
+    assert np.abs(freq - prob).max() < 5 * np.sqrt(prob.max() / B) + 1e-3
+
+
+def test_zero_noise_sampling_is_greedy_descent():
+    """Without noise each sum node takes its heaviest edge and each leaf its mode."""
+    w = np.log(np.array([0.2, 0.5, 0.3], np.float32))
+    leaves = [O.input_node(0, np.log(np.array(p, np.float32))) for p in ([0.9, 0.1], [0.3, 0.7], [0.5, 0.5])]
+    fc = O.bits_compile(O.summate(*leaves, logps=w), 2, 1)
+    out = O.sample(fc, np.zeros((1, fc.n_edges), np.float32), np.zeros((1, 1, 2), np.float32))
+    assert out.tolist() == [[1]]
+    # ties: the first maximum wins
+    fc2 = O.bits_compile(O.summate(*leaves, logps=np.log(np.array([0.4, 0.4, 0.2], np.float32))), 2, 1)
+    assert O.sample(fc2, np.zeros((1, 3), np.float32), np.zeros((1, 1, 2), np.float32)).tolist() == [[0]]
+
+
+def test_soft_sampling_invariants():
+    """test/queries/sample_tests.jl:34-53: top-down probabilities of a sum node's children add
+    up to the node's; per variable the soft output is a distribution; at temperature 1 without
+    noise the output is the circuit's marginal."""
+    rng = np.random.default_rng(10)
+    V, C = 4, 3
+    parent, theta, leaf, fc = make_hclt(V, 3, C, 11)
+    td, out = O.gumbel_soft(fc, None, 1.0, double=True)
+    assert abs(td[-1] - 1) < 1e-12
+    np.testing.assert_allclose(out.sum(axis=1), 1.0, rtol=1e-6)
+    allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    p = np.exp(O.forward(fc, allx, double=True)[-1])
+    for v in range(V):
+        marg = np.array([p[allx[:, v] == c].sum() for c in range(C)])
+        np.testing.assert_allclose(out[v], marg, rtol=1e-5)
+    g = _gumbel(rng, fc.n_edges)
+    td, out = O.gumbel_soft(fc, g, 0.5, double=True)
+    np.testing.assert_allclose(out.sum(axis=1), 1.0, rtol=1e-6)
+    for ids in fc.meta["sum_node"].values():
+        assert abs(td[ids].sum() - 1) < 1e-9
+
+
+# ------------------------------------------------------------------------------------
+# Adam
+# ------------------------------------------------------------------------------------
+
+def test_adam_first_step_closed_form():
+    """At t = 1 with zero moments mhat = g and vhat = g^2, so params move by
+    lr * g / (|g| + eps); groups are normalised into logp_out, params stay unnormalised."""
+    rng = np.random.default_rng(12)
+    n = 10
+    params = rng.normal(size=n).astype(np.float32)
+    p0 = params.copy()
+    grad = rng.normal(size=n).astype(np.float32)
+    m = np.zeros(n, np.float32)
+    v = np.zeros(n, np.float32)
+    logp = np.full(n, 7.0, np.float32)
+    gp = np.array([0, 4, 5, 10])
+    O.adam_step(params, grad, m, v, 1e-2, 0.9, 0.999, 1e-8, 1, gp, logp)
+    np.testing.assert_allclose(params, p0 + 1e-2 * grad / (np.abs(grad) + 1e-8), rtol=1e-5)
+    np.testing.assert_allclose(m, 0.1 * grad, rtol=1e-6)
+    np.testing.assert_allclose(v, 0.001 * grad * grad, rtol=5e-5)     # 1 - 0.999 in float32
+    for a, b in ((0, 4), (5, 10)):
+        np.testing.assert_allclose(np.exp(logp[a:b].astype(np.float64)).sum(), 1.0, rtol=1e-6)
+        np.testing.assert_allclose(logp[a:b] - params[a:b], (logp[a] - params[a]), rtol=1e-5)
+    assert logp[4] == 7.0          # a sum node with one edge keeps its parameter
