@@ -40,6 +40,20 @@ def algorithmic_bytes(n_int, V, K, C, B):
                 step=n_int * 6 * vec + V * B + 3 * theta + 5 * leaf)
 
 
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the committed hardware-counter summary
+    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a copy of known size), or None."""
+    path = os.path.join(ROOT, "profiles", f"hclt_em_step_{workload}_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) == 4 and f[0] == "traffic_bytes" and f[1] == workload and f[2] == kernel:
+                return float(f[3])
+    except OSError:
+        pass
+    return None
+
+
 def cpu_baseline(cfg, sample):
     """The oracle (a C port of the reference arithmetic, OpenMP over examples) on the
     first `sample` examples of the same batch: one full EM step."""
@@ -67,6 +81,9 @@ def main():
     ap.add_argument("--workload", default="c3_hclt3072_k32")
     ap.add_argument("--cpu-sample", type=int, default=4096)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
+                    help="also launch one plain device copy of this many MiB before the timed region "
+                         "(a known-size kernel to scale hardware byte counters against)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (--gpus must be 1)", file=sys.stderr)
@@ -94,6 +111,13 @@ def main():
         check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), None, B, 0.0, 0.1, 0.9,
                               ll.data_ptr()))
 
+    if args.calibrate_copy:
+        src = torch.full((args.calibrate_copy << 20,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     for _ in range(args.warmup):
         step()
     bpc.set_timing(True)
@@ -127,7 +151,8 @@ def main():
         "config": {"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
                    "tree_inner_nodes": stats["n_inner"], "tree_depth": stats["depth"]},
         "roofline": {"bound": "hbm", "kernel": f"hclt_{dominant}_kernel", "achieved": achieved,
-                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS, "traffic": None},
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": measured_traffic(args.workload, dominant)},
         "kernels_ms": kernel_ms,
         "step_roofline_frac": ab["step"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
     }

@@ -181,19 +181,10 @@ void HcltCircuit::build_schedules() {
     for (int i = 0; i < kPre; ++i) q.g[i] = kOpNone;
     return q;
   };
-  const int dbg = getenv("PCM_DBG") ? atoi(getenv("PCM_DBG")) : 0;   // TEMP experiment knob
-  auto dbg_fix = [&](std::vector<PreItem>& pre) {
-    for (auto& q : pre) {
-      if (dbg & 1) for (int i = 0; i < kPre; ++i) q.g[i] = kOpNone;
-      if (dbg & 2) q.wnode = 0;
-      if (dbg & 4) for (int i = 0; i < kPre; ++i) if (q.g[i] & kOpLeaf) q.g[i] = kOpLeaf | 0u;
-    }
-  };
   // field rows [field][wave][stride] with 64 idle steps of padding (a chunk refill reads
   // 64 steps starting anywhere below n_steps)
   auto make_fields = [&](std::vector<StepItem>& sched, std::vector<PreItem>& pre, bool forward, int& stride,
                          DevBuf<int32_t>& dst) {
-    dbg_fix(pre);
     const int n_steps = (int)sched.size() / kWalkWaves;
     for (int i = 0; i < 64 * kWalkWaves; ++i) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); }
     stride = n_steps + 64;
@@ -717,7 +708,6 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.C = C_;
   d.n_inner = n_inner_;
   d.V = V_;
-  d.dbg = getenv("PCM_DBG") ? atoi(getenv("PCM_DBG")) : 0;
   d.leaf_stride = (uint32_t)C_ * K_ * 4;
   d.tile_stride = (uint32_t)d.nslices * kSlice * K_ * 4;
   return d;

@@ -84,7 +84,6 @@ struct HcltDev {
   float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   int32_t B, Bp, nslices, C, n_inner, V;
-  int32_t dbg;            // TEMP experiment knob
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
   uint32_t tile_stride;   // bytes per node in O / R / G (nslices*16*K*4)
 };
