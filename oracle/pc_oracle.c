@@ -12,9 +12,14 @@
  * reference's type; build with -DREAL=double for the high-precision twin used to pin
  * the float build by finite differences and closed forms).
  *
- * Pinned by tests/test_oracle_*.py: brute-force latent enumeration on tiny HCLTs,
+ * Pinned by tests/test_oracle_pinning.py: brute-force latent enumeration on tiny HCLTs,
  * closed forms quoted from the reference's own tests, finite-difference checks of the
- * flows (= dLL/dlogtheta) and of the KL gradient, exact M-step properties.
+ * flows (= dLL/dlogtheta) and of the KL gradient, exact M-step properties, statistics
+ * of exact samples.
+ * PARITY UNPINNED: the two leaf lines of orc_kld_backward in their as-written form
+ * (analytic == 0), which are not the analytic derivative and which no test or fixture
+ * of the reference exercises; they are restated by reading
+ * nodes/fixable_categorical_dist.jl:215-221 only.
  */
 #include <math.h>
 #include <stdint.h>
