@@ -29,6 +29,13 @@ namespace pcm {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
+// Cache policy of the tile stores (gfx950 buffer "aux" bits: sc0 = 1, nt = 2, sc1 = 16).
+// Value and flow tiles are written once and read next by another kernel, long after far
+// more than the caches' capacity has gone by: written through, non-temporal.  On the
+// 3072-variable benchmark this alone takes 20 % off the forward kernel (the default policy
+// makes every store burst wait on L2 allocation).
+constexpr int kStreamStore = 1 | 2 | 16;
+
 constexpr int kStatWaves = 12;   // waves per workgroup in the statistics kernel (168 registers each)
 
 template <int K>
@@ -95,7 +102,7 @@ __device__ __forceinline__ void tile_store(float* base, int node, uint32_t node_
   const uint32_t v = node >= 0 ? voff : 0u, step = node >= 0 ? 1024u : 0u;
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(v + kt * step), 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(v + kt * step), 0, kStreamStore);
 }
 
 template <int K>
