@@ -7,7 +7,7 @@
 #include <functional>
 #include <numeric>
 
-#include "hclt_kernels.hip.hpp"
+#include "hclt_walk_lean.hip.hpp"
 
 namespace pcm {
 
@@ -17,6 +17,14 @@ namespace pcm {
     case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
     case 64: { constexpr int KK = 64; __VA_ARGS__; break; } \
     default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
+  }
+
+// the lean walk kernels exist for the hidden sizes whose blocks fit the register file
+#define PCM_DISPATCH_LEAN_K(K_, ...)                    \
+  switch (K_) {                                         \
+    case 16: { constexpr int KK = 16; __VA_ARGS__; break; } \
+    case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
+    default: fail(PCM_ERR_STATE, "no lean walk kernel for hidden size %d", K_); \
   }
 
 static void check_launch(const char* what) {
@@ -203,6 +211,49 @@ void HcltCircuit::build_schedules() {
       }
     dst.upload(f);
   };
+  // lean schedule rows (see hclt_walk_lean.hip.hpp) from the padded items of a walk, or none
+  // if some node has more operands than the lean kernels hold
+  const size_t leaf_stride = (size_t)C_ * K_ * sizeof(float);
+  auto make_lean = [&](const std::vector<StepItem>& sched, bool forward, int stride, DevBuf<int32_t>& dst) -> bool {
+    if (K_ > 32 || lds_slots_ > 255 || (size_t)V_ * leaf_stride >= ((size_t)1 << 31)) return false;
+    std::vector<int32_t> f((size_t)kLeanFields * kWalkWaves * stride, 0);
+    for (int s = 0; s < stride; ++s)
+      for (int w = 0; w < kWalkWaves; ++w) {
+        const StepItem& it = sched[(size_t)s * kWalkWaves + w];
+        auto put = [&](int field, int32_t v) { f[((size_t)field * kWalkWaves + w) * stride + s] = v; };
+        const int n = it.node;
+        put(kLA1, -1); put(kLA2, -1); put(kLA3, -1);
+        if (n < 0) {   // idle: trash tile, trash slot, block and leaf rows of node / variable 0
+          put(kLNode, n_inner_);
+          put(kLSlots, forward ? (int32_t)(0xffffff00u | (uint32_t)trash_slot) : (trash_slot | trash_slot << 8));
+          continue;
+        }
+        put(kLW, (int32_t)((size_t)n * K_ * K_ * sizeof(float)));
+        put(kLA0, (int32_t)((size_t)var_of_inner_[n] * leaf_stride));
+        put(kLNode, n);
+        put(kLFlags, par[n] < 0 ? 1 : 0);
+        if (forward) {
+          if (lc[n].size() > 3 || ic[n].size() > 3) return false;
+          for (size_t i = 0; i < lc[n].size(); ++i) put(kLA1 + (int)i, (int32_t)((size_t)lc[n][i] * leaf_stride));
+          uint32_t slots = (uint32_t)it.out_slot | 0xffffff00u;
+          for (int c = 0; c < it.n_l; ++c) {
+            const int sl = (int)(it.l[c] >> kSlotShift) - 1;
+            if (sl < 0) return false;
+            slots = (slots & ~(0xffu << (8 * (c + 1)))) | ((uint32_t)sl << (8 * (c + 1)));
+          }
+          put(kLSlots, (int32_t)slots);
+        } else {
+          if (lc[n].size() + ic[n].size() > 3 || it.in_slot < 0 || (it.flags & kItemSpillOut)) return false;
+          int q = 0;
+          for (int c : ic[n]) put(kLA1 + q++, c << 3);
+          for (size_t i = 0; i < lc[n].size(); ++i)
+            put(kLA1 + q++, (int32_t)((size_t)lc[n][i] * leaf_stride) | 1 | (int32_t)((i + 1) << 1));
+          put(kLSlots, it.out_slot | it.in_slot << 8);
+        }
+      }
+    dst.upload(f);
+    return true;
+  };
   auto depth_of = [&](int n) { return depth_[var_of_inner_[n]]; };
 
   // ---- forward -----------------------------------------------------------------------
@@ -266,6 +317,7 @@ void HcltCircuit::build_schedules() {
     }
     n_fwd_steps_ = (int)sched.size() / kWalkWaves;
     make_fields(sched, pre, true, fwd_stride_, d_fwd_fields_);
+    fwd_lean_ = !fwd_spill_ && make_lean(sched, true, fwd_stride_, d_fwd_lean_);
     d_fwd_sched_.upload(sched);
   }
   // ---- backward ----------------------------------------------------------------------
@@ -331,6 +383,7 @@ void HcltCircuit::build_schedules() {
     }
     n_bwd_steps_ = (int)sched.size() / kWalkWaves;
     make_fields(sched, pre, false, bwd_stride_, d_bwd_fields_);
+    bwd_lean_ = !bwd_spill_ && make_lean(sched, false, bwd_stride_, d_bwd_lean_);
     d_bwd_sched_.upload(sched);
   }
   // ---- statistics: the static operands of every node ------------------------------------
@@ -352,9 +405,9 @@ void HcltCircuit::build_schedules() {
   if (ext.empty()) ext.push_back(0);
   d_ext_ops_.upload(ext);
   if (getenv("PCM_VERBOSE"))
-    fprintf(stderr, "[pcmi355] hclt V=%d K=%d C=%d inner=%d: forward %d steps%s, backward %d steps%s, %d LDS slots\n",
-            V_, K_, C_, n_inner_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", n_bwd_steps_,
-            bwd_spill_ ? " (spills)" : "", lds_slots_);
+    fprintf(stderr, "[pcmi355] hclt V=%d K=%d C=%d inner=%d: forward %d steps%s%s, backward %d steps%s%s, %d LDS slots\n",
+            V_, K_, C_, n_inner_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", fwd_lean_ ? " (lean)" : "", n_bwd_steps_,
+            bwd_spill_ ? " (spills)" : "", bwd_lean_ ? " (lean)" : "", lds_slots_);
 }
 
 // Numbering the reference would give this circuit.  Nodes are created in depth-first
@@ -679,11 +732,12 @@ void HcltCircuit::ensure_batch(int batch) {
   const int ns = ceil_div(batch, kSlice);
   if (ns <= cap_slices_) return;
   const size_t tile = (size_t)ns * kSlice * K_;
-  d_O_.alloc((size_t)n_inner_ * tile);
-  d_R_.alloc((size_t)n_inner_ * tile);
+  d_O_.alloc((size_t)(n_inner_ + 1) * tile);   // row n_inner: trash tile of idle waves
+  d_R_.alloc((size_t)(n_inner_ + 1) * tile);
   if (bwd_spill_) d_G_.alloc((size_t)n_inner_ * tile);
   d_xb_.alloc((size_t)V_ * ns * kSlice);
-  d_xn_.alloc((size_t)n_inner_ * ns * kSlice);
+  d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
+  d_xn_.zero();
   cap_slices_ = ns;
 }
 
@@ -734,9 +788,20 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
     hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_fwd_fields_.p,
                        fwd_stride_, d_fwd_sched_.p, n_fwd_steps_, d_ll);
   };
-  PCM_DISPATCH_K(K_, {
-    if (fwd_spill_) launch(&hclt_forward_kernel<KK, true>); else launch(&hclt_forward_kernel<KK, false>);
-  });
+  // the lean kernels address every array with 32-bit offsets from one descriptor
+  const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
+  if (fwd_lean_ && small) {
+    PCM_DISPATCH_LEAN_K(K_, {
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d,
+                         d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll);
+    });
+  } else {
+    PCM_DISPATCH_K(K_, {
+      if (fwd_spill_) launch(&hclt_forward_kernel<KK, true>); else launch(&hclt_forward_kernel<KK, false>);
+    });
+  }
   check_launch("hclt_forward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
@@ -748,9 +813,19 @@ void HcltCircuit::run_backward(const HcltDev& d) {
     hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_fields_.p,
                        bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
   };
-  PCM_DISPATCH_K(K_, {
-    if (bwd_spill_) launch(&hclt_backward_kernel<KK, true>); else launch(&hclt_backward_kernel<KK, false>);
-  });
+  const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
+  if (bwd_lean_ && small) {
+    PCM_DISPATCH_LEAN_K(K_, {
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_backward_lean_kernel<KK>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(hclt_backward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d,
+                         d_bwd_lean_.p, bwd_stride_, n_bwd_steps_);
+    });
+  } else {
+    PCM_DISPATCH_K(K_, {
+      if (bwd_spill_) launch(&hclt_backward_kernel<KK, true>); else launch(&hclt_backward_kernel<KK, false>);
+    });
+  }
   check_launch("hclt_backward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
 }

@@ -135,7 +135,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<HcltNode> d_nodes_;
   DevBuf<int32_t> d_child_inner_, d_child_leaf_;
   DevBuf<StepItem> d_fwd_sched_, d_bwd_sched_, d_stat_items_;
-  DevBuf<int32_t> d_fwd_fields_, d_bwd_fields_;
+  DevBuf<int32_t> d_fwd_fields_, d_bwd_fields_, d_fwd_lean_, d_bwd_lean_;
+  bool fwd_lean_ = false, bwd_lean_ = false;   // the lean walk kernels can run this tree
   int fwd_stride_ = 0, bwd_stride_ = 0;
   DevBuf<uint32_t> d_ext_ops_;
   DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_R_, d_G_;

@@ -1,0 +1,302 @@
+// Lean tree-walk kernels: the same slice-persistent forward / backward walks as in
+// hclt_kernels.hip.hpp, for the common case (no tile ever leaves LDS, at most three children
+// per tree node, every array below 4 GiB), written for the fewest instructions per step.
+//
+// Why a second pair of kernels.  With one 16-example tile per wave and step, a step is only
+// ~100 useful vector instructions (8 exp, 8 log, 16 MFMA, a few adds), and four waves share a
+// SIMD: measured on gfx950 the general walk kernels are bound by instruction issue, not by
+// memory -- their schedule decoding and 64-bit address arithmetic cost more instructions
+// than the arithmetic.  Here
+//   * every array is addressed through ONE buffer descriptor built before the loop; a node's
+//     byte offset comes precomputed from the schedule and goes into the instruction's scalar
+//     offset, the lane part is a per-thread constant, the tile row an immediate;
+//   * operands are typed by position (own leaf row, own value tile, up to three children), so
+//     an absent operand is a scalar branch around its loads and its adds -- nothing is
+//     zero-filled, selected or copied;
+//   * the parameter block is requested right after the contraction that used its
+//     predecessor, into the same registers, so nothing rotates between steps.
+// Idle waves work on a trash tile (row n_inner of the value arrays) and the trash LDS slot.
+#pragma once
+
+#include "hclt_kernels.hip.hpp"
+
+namespace pcm {
+
+// Field rows of a lean schedule, [field][wave][stride] like the general one.
+//   kLW     byte offset of the node's parameter block
+//   kLA0    byte offset of the node's own leaf rows (variable * leaf_stride)
+//   kLA1..3 forward: leaf children's rows (-1: none; their categories are bytes 1..3 of the
+//           packed word).  backward: children, -1: none, leaf child: row offset | 1 | category
+//           byte << 1, inner child: node index << 3 (its value tile)
+//   kLNode  node index (value / flow tile, packed-category row); idle waves: n_inner, the
+//           trash tile (its category row is out of range and reads as zero)
+//   kLSlots forward: out slot | child slots << 8, 16, 24 (0xff: none); backward: out slot |
+//           slot of the parent's flow tile << 8
+//   kLFlags bit 0: root
+enum { kLW = 0, kLA0, kLA1, kLA2, kLA3, kLNode, kLSlots, kLFlags, kLeanFields };
+
+constexpr int kLeanChunk = 62;   // steps per refill: 64 lanes minus two steps of look-ahead
+
+struct LeanChunk {
+  int v[kLeanFields];
+  int base;
+};
+
+__device__ __forceinline__ void lean_refill(const int32_t* __restrict__ fields, int stride, int wave, int lane, int base,
+                                            LeanChunk& c) {
+#pragma unroll
+  for (int f = 0; f < kLeanFields; ++f) c.v[f] = fields[((size_t)f * kWalkWaves + wave) * stride + base + lane];
+  // the rows are used as landed from here on: no step waits for them (a step's own waits
+  // then count only the requests of the steps)
+#pragma unroll
+  for (int f = 0; f < kLeanFields; ++f) asm volatile("" : "+v"(c.v[f]));
+  c.base = base;
+}
+
+__device__ __forceinline__ int lean_get(const LeanChunk& c, int field, int step) {
+  return __builtin_amdgcn_readlane(c.v[field], step - c.base);
+}
+
+template <int K>
+__device__ __forceinline__ void lean_row_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, Tile<K>& t) {
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt)
+    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * 64), soff, 0));
+}
+
+template <int K>
+__device__ __forceinline__ void lean_tile_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, Tile<K>& t) {
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt)
+    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * 1024), soff, 0));
+}
+
+template <int K>
+__device__ __forceinline__ void lean_tile_store(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, const Tile<K>& t) {
+#pragma unroll
+  for (int kt = 0; kt < K / 16; ++kt)
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(voff + kt * 1024), soff, kStreamStore);
+}
+
+template <int K>
+__device__ __forceinline__ void lean_w_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, WTile<K>& w) {
+#pragma unroll
+  for (int i = 0; i < (K / 16) * (K / 16); ++i)
+    w.a[i] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + (i & 3) * 1024), soff + (i >> 2) * 4096, 0));
+}
+
+// byte offset of this lane's part of leaf row x (byte `sel` of the packed word)
+template <int K>
+__device__ __forceinline__ uint32_t lean_row_off(uint32_t xpack, int sel, uint32_t vleaf) {
+  return ((xpack >> (8 * sel)) & 0xffu) * (K * 4) + vleaf;
+}
+
+__device__ __forceinline__ void lean_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// ---- forward ------------------------------------------------------------------------------
+template <int K>
+__global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
+    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps, float* __restrict__ ll_out) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slice = blockIdx.x;
+  const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)(lane >> 4) * 16, vx = (uint32_t)(lane & 15) * 4;
+  const int bcol = slice * kSlice + (lane & 15);
+  const uint32_t slice_bytes = (uint32_t)slice * (kSlice * K * 4);
+  const __amdgpu_buffer_rsrc_t rO =
+      make_rsrc(reinterpret_cast<const char*>(d.O) + slice_bytes, (uint32_t)(d.n_inner + 1) * d.tile_stride - slice_bytes);
+  const __amdgpu_buffer_rsrc_t rW = make_rsrc(d.Wf, (uint32_t)d.n_inner * (K * K * 4));
+  const __amdgpu_buffer_rsrc_t rL = make_rsrc(d.leaf, (uint32_t)d.V * d.leaf_stride);
+  const __amdgpu_buffer_rsrc_t rX =
+      make_rsrc(d.xn + (size_t)slice * kSlice, (uint32_t)d.n_inner * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
+  const int xrow = d.Bp * 4;
+
+  LeanChunk sc;
+  lean_refill(fields, stride, wave, lane, 0, sc);
+  Tile<K> P0, P1, P2, P3;
+  WTile<K> wA, wB;   // parameter blocks of the even / odd steps
+  uint32_t xs;
+  int a1, a2, a3;   // leaf children of the step whose operands are in flight
+  {
+    const uint32_t x0 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0);
+    xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 1) * xrow, 0);
+    lean_row_load<K>(rL, lean_row_off<K>(x0, 0, vleaf), lean_get(sc, kLA0, 0), P0);
+    a1 = lean_get(sc, kLA1, 0); a2 = lean_get(sc, kLA2, 0); a3 = lean_get(sc, kLA3, 0);
+    if (a1 >= 0) lean_row_load<K>(rL, lean_row_off<K>(x0, 1, vleaf), a1, P1);
+    if (a2 >= 0) lean_row_load<K>(rL, lean_row_off<K>(x0, 2, vleaf), a2, P2);
+    if (a3 >= 0) lean_row_load<K>(rL, lean_row_off<K>(x0, 3, vleaf), a3, P3);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 0), wA);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
+  }
+  float ll = 0.f;
+  Tile<K> o_prev;   // the value tile of the previous step, stored at the top of the next one
+  tile_zero<K>(o_prev);
+  int store_prev = d.n_inner * (int)d.tile_stride;
+
+  // the schedule is consumed in chunks of kLeanChunk steps (a chunk's registers also serve
+  // the two steps of look-ahead past its end)
+  auto step = [&](const int s, WTile<K>& w) {
+    // (1) the static operands of this step have landed
+    Tile<K> z = P0;
+    if (a1 >= 0) tile_add<K>(z, P1);
+    if (a2 >= 0) tile_add<K>(z, P2);
+    if (a3 >= 0) tile_add<K>(z, P3);
+    // the previous step's value tile goes out now
+    lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+    // (2) request the leaf rows of step s+1 and the categories of step s+2
+    {
+      // (the categories first: everything that later waits for a leaf row then covers them)
+      const uint32_t xc = xs;
+      xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, s + 2) * xrow, 0);
+      lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), lean_get(sc, kLA0, s + 1), P0);
+      a1 = lean_get(sc, kLA1, s + 1); a2 = lean_get(sc, kLA2, s + 1); a3 = lean_get(sc, kLA3, s + 1);
+      if (a1 >= 0) lean_row_load<K>(rL, lean_row_off<K>(xc, 1, vleaf), a1, P1);
+      if (a2 >= 0) lean_row_load<K>(rL, lean_row_off<K>(xc, 2, vleaf), a2, P2);
+      if (a3 >= 0) lean_row_load<K>(rL, lean_row_off<K>(xc, 3, vleaf), a3, P3);
+    }
+    // (3) children from LDS, logsumexp through the matrix cores
+    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
+#pragma unroll
+    for (int c = 1; c <= 3; ++c) {
+      const uint32_t sl = (slots >> (8 * c)) & 0xffu;
+      if (sl != 0xffu) {
+        Tile<K> t;
+        lds_tile_load<K>(lds, (int)sl, lane, t);
+        tile_add<K>(z, t);
+      }
+    }
+    const float m = tile_rowmax<K>(z);
+    tile_exp_sub<K>(z, m);
+    Tile<K> o;
+    contract<K>(w, z, o);
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o.v[kt][i] = fmaf(__builtin_amdgcn_logf(o.v[kt][i]), kLn2, m);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);   // the block of step s+2, same registers
+    o_prev = o;
+    store_prev = lean_get(sc, kLNode, s) * (int)d.tile_stride;
+    lds_tile_store<K>(lds, (int)(slots & 0xffu), lane, o);
+    if (lean_get(sc, kLFlags, s) & 1) ll = o.v[0][0];
+    lean_barrier();
+  };
+  // The schedule is consumed in chunks of kLeanChunk steps (a chunk's registers also serve the
+  // two steps of look-ahead past its end), two steps per trip: the parameter blocks alternate
+  // between two register sets, each reloaded two steps ahead right after its use.  An odd
+  // step count runs one idle step of the padding.
+  for (int base = 0; base < n_steps; base += kLeanChunk) {
+    if (base) lean_refill(fields, stride, wave, lane, base, sc);
+    const int s_end = min(base + kLeanChunk, n_steps);
+    for (int s = base; s < s_end; s += 2) {
+      step(s, wA);
+      step(s + 1, wB);
+    }
+  }
+  lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+  if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
+}
+
+// ---- backward -----------------------------------------------------------------------------
+template <int K>
+__global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
+    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps) {
+  extern __shared__ float lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int slice = blockIdx.x;
+  const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)(lane >> 4) * 16, vx = (uint32_t)(lane & 15) * 4;
+  const int bcol = slice * kSlice + (lane & 15);
+  const uint32_t slice_bytes = (uint32_t)slice * (kSlice * K * 4);
+  const uint32_t arr_bytes = (uint32_t)(d.n_inner + 1) * d.tile_stride - slice_bytes;
+  const __amdgpu_buffer_rsrc_t rO = make_rsrc(reinterpret_cast<const char*>(d.O) + slice_bytes, arr_bytes);
+  const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + slice_bytes, arr_bytes);
+  const __amdgpu_buffer_rsrc_t rW = make_rsrc(d.Wb, (uint32_t)d.n_inner * (K * K * 4));
+  const __amdgpu_buffer_rsrc_t rL = make_rsrc(d.leaf, (uint32_t)d.V * d.leaf_stride);
+  const __amdgpu_buffer_rsrc_t rX =
+      make_rsrc(d.xn + (size_t)slice * kSlice, (uint32_t)d.n_inner * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
+  const int xrow = d.Bp * 4;
+
+  // a child operand: value tile of an inner child, or leaf row of a leaf child
+  auto child_load = [&](int c, uint32_t xpack, Tile<K>& t) {
+    if (c & 1) lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), c & ~7, t);
+    else lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride, t);
+  };
+
+  LeanChunk sc;
+  lean_refill(fields, stride, wave, lane, 0, sc);
+  Tile<K> P0, OV, C1, C2, C3;
+  WTile<K> wA, wB;
+  uint32_t xs;
+  int c1, c2, c3;
+  {
+    const uint32_t x0 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0);
+    xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 1) * xrow, 0);
+    lean_row_load<K>(rL, lean_row_off<K>(x0, 0, vleaf), lean_get(sc, kLA0, 0), P0);
+    lean_tile_load<K>(rO, vtile, lean_get(sc, kLNode, 0) * (int)d.tile_stride, OV);
+    c1 = lean_get(sc, kLA1, 0); c2 = lean_get(sc, kLA2, 0); c3 = lean_get(sc, kLA3, 0);
+    if (c1 >= 0) child_load(c1, x0, C1);
+    if (c2 >= 0) child_load(c2, x0, C2);
+    if (c3 >= 0) child_load(c3, x0, C3);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 0), wA);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
+  }
+
+  auto step = [&](const int s, WTile<K>& w) {
+    // (1) E_v (unnormalised) and the factor 1/S_v = exp(m - O_v) from the landed operands
+    Tile<K> e = P0;
+    if (c1 >= 0) tile_add<K>(e, C1);
+    if (c2 >= 0) tile_add<K>(e, C2);
+    if (c3 >= 0) tile_add<K>(e, C3);
+    const float m = tile_rowmax<K>(e);
+    Tile<K> sinv;
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sinv.v[kt][i] = __builtin_amdgcn_exp2f(fmaf(OV.v[kt][i], -kLog2e, m * kLog2e));
+    // (2) request the operands of step s+1 and the categories of step s+2
+    {
+      const uint32_t xc = xs;
+      xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, s + 2) * xrow, 0);
+      lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), lean_get(sc, kLA0, s + 1), P0);
+      lean_tile_load<K>(rO, vtile, lean_get(sc, kLNode, s + 1) * (int)d.tile_stride, OV);
+      c1 = lean_get(sc, kLA1, s + 1); c2 = lean_get(sc, kLA2, s + 1); c3 = lean_get(sc, kLA3, s + 1);
+      if (c1 >= 0) child_load(c1, xc, C1);
+      if (c2 >= 0) child_load(c2, xc, C2);
+      if (c3 >= 0) child_load(c3, xc, C3);
+    }
+    // (3) R_v = F_v / S_v, G_v = E_v .* (R_v W_v)
+    tile_exp_sub<K>(e, m);
+    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
+    Tile<K> r, t;
+    lds_tile_load<K>(lds, (int)((slots >> 8) & 0xffu), lane, r);
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt) r.v[kt] *= sinv.v[kt];
+    if (lean_get(sc, kLFlags, s) & 1) {   // flow 1 into the single root sum node of every live example
+      const float r00 = (lane < 16 && bcol < d.B) ? sinv.v[0][0] : 0.f;
+      tile_zero<K>(r);
+      r.v[0][0] = r00;
+    }
+    lean_tile_store<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
+    contract<K>(w, r, t);
+    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);
+#pragma unroll
+    for (int kt = 0; kt < K / 16; ++kt) t.v[kt] *= e.v[kt];
+    lds_tile_store<K>(lds, (int)(slots & 0xffu), lane, t);
+    lean_barrier();
+  };
+  for (int base = 0; base < n_steps; base += kLeanChunk) {
+    if (base) lean_refill(fields, stride, wave, lane, base, sc);
+    const int s_end = min(base + kLeanChunk, n_steps);
+    for (int s = base; s < s_end; s += 2) {
+      step(s, wA);
+      step(s + 1, wB);
+    }
+  }
+}
+
+}  // namespace pcm
