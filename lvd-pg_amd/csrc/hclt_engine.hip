@@ -299,8 +299,15 @@ void HcltCircuit::build_schedules() {
         for (size_t i = 0; i < lc[n].size(); ++i) ops.push_back(leaf_child_op(lc[n][i], i));
         it.n_l = 0;
         for (int c : ic[n]) {
-          if (it.n_l < kInlineLds) it.l[it.n_l++] = ((uint32_t)(slot[c] + 1) << kSlotShift) | (uint32_t)c;
-          else { ops.push_back((uint32_t)c); fwd_spill_ = true; }   // read back from HBM
+          if (it.n_l < kInlineLds) {
+            it.l[it.n_l++] = ((uint32_t)(slot[c] + 1) << kSlotShift) | (uint32_t)c;
+          } else {
+            // read back from HBM, and only at the point of use: the child may have been
+            // produced in the step before this one, when the requests ahead were already out
+            while (ops.size() < (size_t)kPre) ops.push_back(kOpNone);
+            ops.push_back((uint32_t)c);
+            fwd_spill_ = true;
+          }
           if (slot[c] < 0) fwd_spill_ = true;
         }
         fill_ops(it, q, ops);

@@ -17,10 +17,10 @@ def gpu():
     return torch, pcmi355
 
 
-def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None):
+def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None, tree=None):
     torch, P = gpu
     from helpers import make_hclt, correlated_data, oracle_em_reference, block_theta, rel_err
-    parent, theta, leaf, fc = make_hclt(V, K, C, seed)
+    parent, theta, leaf, fc = make_hclt(V, K, C, seed, parent=None if tree is None else np.array(tree, np.int32))
     N = N or B
     data = correlated_data(N, V, C, seed + 1, parent)
     ids = np.arange(B, dtype=np.int32) if idx is None else idx
@@ -56,6 +56,16 @@ def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None):
 @pytest.mark.parametrize("V,K,C,B", [(2, 16, 5, 16), (7, 16, 8, 48), (12, 32, 256, 64), (9, 64, 17, 32)])
 def test_em_step_matches_oracle(gpu, oracle, V, K, C, B):
     _compare_step(gpu, oracle, V, K, C, B, seed=100 + V)
+
+
+@pytest.mark.parametrize("tree", [[-1, 0, 0, 0, 0, 0, 0],                      # star: six leaf children
+                                  [-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5],        # five inner children
+                                  [-1, 0, 1, 1, 1, 1, 2, 3, 0, 8, 8, 8, 8]])  # mixed, four children twice
+def test_em_step_on_wide_trees(gpu, oracle, tree):
+    """Nodes with more than three children take the general walk kernels (operands beyond the
+    inline ones, schedule items read from memory)."""
+    _compare_step(gpu, oracle, len(tree), 16, 7, 40, seed=len(tree), tree=tree)
+    _compare_step(gpu, oracle, len(tree), 32, 12, 33, seed=len(tree) + 1, tree=tree)
 
 
 def test_ragged_batch_and_example_ids(gpu, oracle):
