@@ -408,6 +408,25 @@ void HcltCircuit::build_schedules() {
       items.push_back(it);
     }
     d_stat_items_.upload(items);
+    // the same for the lean statistics kernel (nodes with at most three children)
+    stat_lean_ = K_ <= 32;
+    std::vector<StatNode> sn(n_inner_);
+    for (int n = 0; n < n_inner_ && stat_lean_; ++n) {
+      StatNode& q = sn[n];
+      std::memset(&q, 0, sizeof q);
+      if (ic[n].size() + lc[n].size() > 3) { stat_lean_ = false; break; }
+      q.var = var_of_inner_[n];
+      q.c[0] = q.c[1] = q.c[2] = -1;
+      int k = 0;
+      for (int c : ic[n]) q.c[k++] = c << 3;
+      q.n_hist = 1;
+      q.hvar[0] = q.var;
+      for (size_t i = 0; i < lc[n].size(); ++i) {
+        q.c[k++] = (lc[n][i] << 3) | 1 | (int32_t)((i + 1) << 1);
+        q.hvar[q.n_hist++] = lc[n][i];
+      }
+    }
+    if (stat_lean_) d_stat_lean_.upload(sn);
   }
   if (ext.empty()) ext.push_back(0);
   d_ext_ops_.upload(ext);
@@ -838,8 +857,30 @@ void HcltCircuit::run_backward(const HcltDev& d) {
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
-  // LDS layout of hclt_stats_kernel
+  // fixed-point split of the flows: limb sums over the padded batch must stay below 2^32
+  int bits = 0;
+  while ((1 << bits) < d.Bp) ++bits;
+  const int limb = std::min(24, 32 - bits);
+  if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   const size_t hist = 2 * (size_t)C_ * (K_ + 1);                    // words per histogram (two limbs)
+  if (stat_lean_) {
+    // LDS: one histogram (or the parked edge-flow blocks, whichever is larger) | per-wave pads
+    const size_t park = (size_t)kStatLeanWaves * K_ * K_;
+    const size_t hw = (std::max(hist, park) + 3) & ~(size_t)3;
+    const size_t lds = (hw + (size_t)kStatLeanWaves * kSlice * (K_ + 16)) * 4;
+    if (lds <= (size_t)max_lds_) {
+      PCM_DISPATCH_LEAN_K(K_, {
+        PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_lean_kernel<KK>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(n_inner_), dim3(kStatLeanWaves * 64), lds, stream, d,
+                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, limb);
+      });
+      check_launch("hclt_stats_lean");
+      if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
+      return;
+    }
+  }
+  // LDS layout of hclt_stats_kernel
   const size_t pads = (size_t)kStatWaves * kSlice * (K_ + 16);
   auto hist_words = [&](int nh) { return std::max((((size_t)nh * hist + 3) & ~(size_t)3), (size_t)K_ * K_); };
   int nh = 3;
@@ -847,11 +888,6 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   const size_t lds = (hist_words(nh) + pads) * 4;
   if (lds > (size_t)max_lds_)
     fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", lds, max_lds_);
-  // fixed-point split of the flows: limb sums over the padded batch must stay below 2^32
-  int bits = 0;
-  while ((1 << bits) < d.Bp) ++bits;
-  const int limb = std::min(24, 32 - bits);
-  if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   PCM_DISPATCH_K(K_, {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

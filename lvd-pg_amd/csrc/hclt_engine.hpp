@@ -68,6 +68,16 @@ struct PreItem {
 };
 static_assert(sizeof(PreItem) == 32, "PreItem is read as 8 dwords");
 
+// A node as the lean statistics kernel sees it.
+struct StatNode {
+  int32_t var;        // the node's own variable
+  int32_t c[3];       // children: -1 none, leaf child: variable << 3 | 1 | category byte << 1, inner child: node << 3
+  int32_t n_hist;     // variables to histogram: own + leaf children
+  int32_t hvar[4];    // ... their ids; entry i uses category byte i
+  int32_t pad[7];
+};
+static_assert(sizeof(StatNode) == 64, "StatNode is read with scalar loads");
+
 // Everything the kernels need, passed by value.
 struct HcltDev {
   const HcltNode* nodes;
@@ -136,7 +146,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int32_t> d_child_inner_, d_child_leaf_;
   DevBuf<StepItem> d_fwd_sched_, d_bwd_sched_, d_stat_items_;
   DevBuf<int32_t> d_fwd_fields_, d_bwd_fields_, d_fwd_lean_, d_bwd_lean_;
-  bool fwd_lean_ = false, bwd_lean_ = false;   // the lean walk kernels can run this tree
+  bool fwd_lean_ = false, bwd_lean_ = false, stat_lean_ = false;   // the lean kernels can run this tree
+  DevBuf<StatNode> d_stat_lean_;
   int fwd_stride_ = 0, bwd_stride_ = 0;
   DevBuf<uint32_t> d_ext_ops_;
   DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_R_, d_G_;

@@ -299,4 +299,179 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
   }
 }
 
+// ---- statistics -----------------------------------------------------------------------------
+// Same job as hclt_stats_kernel (one workgroup per tree node, all slices; edge flows summed
+// over the batch with the matrix cores, leaf histograms with integer LDS atomics), for nodes
+// with at most three children, written like the lean walks: per-operand descriptors built once
+// (the node is fixed, only the slice moves), typed operands behind scalar branches, every
+// register reloaded right after its last use, the waves' partial edge-flow blocks combined by
+// a plain LDS sum.  A node with leaf children runs one pass over the batch per variable it has
+// to histogram (the LDS holds one histogram); the edge flows are accumulated in pass 0.
+constexpr int kStatLeanWaves = 16;
+
+template <int K>
+__global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
+    HcltDev d, const StatNode* __restrict__ nodes, float* __restrict__ edge_aggr, float* __restrict__ leaf_flow,
+    float rate, int hist_words, int limb) {
+  constexpr int KT = K / 16;
+  constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
+  constexpr int HS = K + 1;    // row stride of a histogram: spreads equal states over banks
+  extern __shared__ float smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int b = lane & 15, g = lane >> 4;
+  const int n = blockIdx.x;
+  const StatNode nd = nodes[n];
+  const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)g * 16, vx = (uint32_t)b * 4;
+  const int hist_sz = d.C * HS;
+  unsigned* hist = reinterpret_cast<unsigned*>(smem);
+  float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
+  const float scale = __builtin_ldexpf(1.f, limb);
+
+  const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + (size_t)n * d.tile_stride, d.tile_stride);
+  const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);
+  const __amdgpu_buffer_rsrc_t rL0 = make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)nd.var * d.leaf_stride, d.leaf_stride);
+  auto child_rsrc = [&](int c) {
+    return (c & 1) ? make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)(c >> 3) * d.leaf_stride, d.leaf_stride)
+                   : make_rsrc(reinterpret_cast<const char*>(d.O) + (size_t)(max(c, 0) >> 3) * d.tile_stride, d.tile_stride);
+  };
+  const __amdgpu_buffer_rsrc_t rC1 = child_rsrc(nd.c[0]), rC2 = child_rsrc(nd.c[1]), rC3 = child_rsrc(nd.c[2]);
+  const int c1 = nd.c[0], c2 = nd.c[1], c3 = nd.c[2];
+  auto child_load = [&](__amdgpu_buffer_rsrc_t r, int c, uint32_t xpack, uint32_t slice_off, Tile<K>& t) {
+    if (c & 1) lean_row_load<K>(r, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), 0, t);
+    else lean_tile_load<K>(r, vtile, (int)slice_off, t);
+  };
+
+  WTile<K> w;
+  lean_w_load<K>(make_rsrc(d.Wb + (size_t)n * K * K, K * K * 4u), vtile, 0, w);
+  v4f accA[KT][KT];
+#pragma unroll
+  for (int a = 0; a < KT; ++a)
+#pragma unroll
+    for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  const int last = d.nslices - 1;
+  for (int pass = 0; pass < nd.n_hist; ++pass) {
+    for (int i = threadIdx.x; i < 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
+    __syncthreads();
+    const int sel = pass;   // category byte of the variable histogrammed in this pass
+
+    // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
+    // repeated loads), categories of the second
+    Tile<K> P0, R, C1, C2, C3;
+    uint32_t xc, xn;
+    {
+      const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
+      xc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sa * (kSlice * 4), 0);
+      xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sb * (kSlice * 4), 0);
+      const uint32_t so = (uint32_t)sa * (kSlice * K * 4);
+      lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
+      if (c1 >= 0) child_load(rC1, c1, xc, so, C1);
+      if (c2 >= 0) child_load(rC2, c2, xc, so, C2);
+      if (c3 >= 0) child_load(rC3, c3, xc, so, C3);
+      lean_tile_load<K>(rR, vtile, (int)so, R);
+    }
+    for (int s0 = wave; s0 < d.nslices; s0 += kStatLeanWaves) {
+      const int s1 = min(s0 + kStatLeanWaves, last), s2 = min(s0 + 2 * kStatLeanWaves, last);
+      const uint32_t so1 = (uint32_t)s1 * (kSlice * K * 4);
+      // (1) E (unnormalised) from the landed operands; request the next slice's
+      Tile<K> e = P0;
+      if (c1 >= 0) tile_add<K>(e, C1);
+      if (c2 >= 0) tile_add<K>(e, C2);
+      if (c3 >= 0) tile_add<K>(e, C3);
+      const uint32_t xh = xc;   // categories of the slice computed now
+      xc = xn;
+      xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
+      lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
+      if (c1 >= 0) child_load(rC1, c1, xc, so1, C1);
+      if (c2 >= 0) child_load(rC2, c2, xc, so1, C2);
+      if (c3 >= 0) child_load(rC3, c3, xc, so1, C3);
+      // (2) G = E .* (R W)
+      const float m = tile_rowmax<K>(e);
+      tile_exp_sub<K>(e, m);
+      Tile<K> t;
+      contract<K>(w, R, t);
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
+      if (pass == 0) {
+        // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
+        // go through the wave's pad to reach the [state][example] operand layout.  A wave's LDS
+        // accesses execute in order, so the pad needs no barrier between its phases.
+        float ra[4][KT];
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = R.v[kt];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt) ra[q][kt] = pad[(4 * q + g) * LD + kt * 16 + b];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = e.v[kt];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float eb[KT];
+#pragma unroll
+          for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[(4 * q + g) * LD + jt * 16 + b];
+#pragma unroll
+          for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+            for (int jt = 0; jt < KT; ++jt)
+              accA[kt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[q][kt], eb[jt], accA[kt][jt], 0, 0, 0);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      }
+      lean_tile_load<K>(rR, vtile, (int)so1, R);   // next slice's ratios, after the last use of these
+      // (3) histogram: fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
+      if (s0 * kSlice + b < d.B) {
+        const uint32_t x = (xh >> (8 * sel)) & 0xffu;
+        unsigned* hrow = hist + x * HS + 4 * g;
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale, 0.f, scale);
+            const unsigned hi = (unsigned)v;
+            const unsigned lo = (unsigned)(__builtin_amdgcn_fractf(v) * scale);
+            __hip_atomic_fetch_add(&hrow[kt * 16 + i], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            __hip_atomic_fetch_add(&hrow[hist_sz + kt * 16 + i], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+          }
+      }
+    }
+    __syncthreads();
+    {
+      const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+      float* dst = leaf_flow + (size_t)nd.hvar[pass] * d.C * K;
+      for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
+        const int c = i / K, j = i % K;
+        const float val = (float)hist[c * HS + j] * hi_inv + (float)hist[hist_sz + c * HS + j] * lo_inv;
+        const float old = rate != 0.f ? rate * dst[i] : 0.f;
+        dst[i] = old + val;
+      }
+    }
+    __syncthreads();
+  }
+
+  // combine the waves' partial blocks: every wave parks its accumulators in LDS (the histogram
+  // area is free now), then each thread adds up the waves' copies of its elements
+  v4f* park = reinterpret_cast<v4f*>(smem);
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt) park[((size_t)wave * KT * KT + kt * KT + jt) * 64 + lane] = accA[kt][jt];
+  __syncthreads();
+  float* dst = edge_aggr + (size_t)n * K * K;
+  const float* lt = d.logtheta + (size_t)n * K * K;
+  for (int q = threadIdx.x; q < KT * KT * 64; q += blockDim.x) {
+    v4f sum = park[q];
+    for (int wv = 1; wv < kStatLeanWaves; ++wv) sum += park[(size_t)wv * KT * KT * 64 + q];
+    const int kt = q / (KT * 64), jt = (q / 64) % KT, l = q % 64;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int idx = (kt * 16 + 4 * (l >> 4) + v) * K + jt * 16 + (l & 15);
+      const float old = rate != 0.f ? rate * dst[idx] : 0.f;
+      dst[idx] = old + __expf(lt[idx]) * sum[v];
+    }
+  }
+}
+
 }  // namespace pcm
