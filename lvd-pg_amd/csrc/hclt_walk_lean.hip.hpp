@@ -358,7 +358,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 
     // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
     // repeated loads), categories of the second
-    Tile<K> P0, R, C1, C2, C3;
+    Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
     uint32_t xc, xn;
     {
       const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
@@ -368,7 +368,6 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
       lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
       if (c1 >= 0) child_load(rC1, c1, xc, so, C1);
       if (c2 >= 0) child_load(rC2, c2, xc, so, C2);
-      if (c3 >= 0) child_load(rC3, c3, xc, so, C3);
       lean_tile_load<K>(rR, vtile, (int)so, R);
     }
     for (int s0 = wave; s0 < d.nslices; s0 += kStatLeanWaves) {
@@ -378,21 +377,20 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
       Tile<K> e = P0;
       if (c1 >= 0) tile_add<K>(e, C1);
       if (c2 >= 0) tile_add<K>(e, C2);
-      if (c3 >= 0) tile_add<K>(e, C3);
       const uint32_t xh = xc;   // categories of the slice computed now
+      if (c3 >= 0) {
+        Tile<K> t3;
+        child_load(rC3, c3, xh, (uint32_t)s0 * (kSlice * K * 4), t3);
+        tile_add<K>(e, t3);
+      }
       xc = xn;
       xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
       lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
       if (c1 >= 0) child_load(rC1, c1, xc, so1, C1);
       if (c2 >= 0) child_load(rC2, c2, xc, so1, C2);
-      if (c3 >= 0) child_load(rC3, c3, xc, so1, C3);
-      // (2) G = E .* (R W)
+      // (2) E, the edge flows, then G = E .* (R W)
       const float m = tile_rowmax<K>(e);
       tile_exp_sub<K>(e, m);
-      Tile<K> t;
-      contract<K>(w, R, t);
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
       if (pass == 0) {
         // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
         // go through the wave's pad to reach the [state][example] operand layout.  A wave's LDS
@@ -420,6 +418,10 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
         }
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
       }
+      Tile<K> t;
+      contract<K>(w, R, t);
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
       lean_tile_load<K>(rR, vtile, (int)so1, R);   // next slice's ratios, after the last use of these
       // (3) histogram: fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
       if (s0 * kSlice + b < d.B) {
