@@ -35,8 +35,10 @@ static void check_launch(const char* what) {
 HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C) : V_(V), K_(K), C_(C) {
   if (!parent) fail(PCM_ERR_ARG, "clt_parent is null");
   if (V < 2) fail(PCM_ERR_SHAPE, "an HCLT needs at least 2 variables, got %d", V);
-  if (K != 16 && K != 32 && K != 64)
-    fail(PCM_ERR_UNSUPPORTED, "num_hidden_cats must be 16, 32 or 64 for the block engine, got %d", K);
+  if (K < 1 || K > 1024) fail(PCM_ERR_SHAPE, "num_hidden_cats must be in 1..1024, got %d", K);
+  // hidden sizes without block kernels run every query on the layered engine over the
+  // circuit's general form; the block-form parameter interface stays the same
+  block_ = K == 16 || K == 32 || K == 64;
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
   build_structure();
@@ -127,7 +129,7 @@ void HcltCircuit::build_structure() {
   d_child_inner_.upload(ci);
   d_child_leaf_.upload(cl);
 
-  build_schedules();
+  if (block_) build_schedules();
 }
 
 // Step schedules of the two tree walks.  Every step holds at most kWalkWaves nodes whose
@@ -642,6 +644,7 @@ void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
 // ---- parameters -------------------------------------------------------------------
 
 void HcltCircuit::rebuild_w() {
+  if (!block_) return;
   const int64_t tot = (int64_t)n_inner_ * K_ * K_;
   PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_rebuild_w_kernel<KK>, dim3(ceil_div(tot, 256)), dim3(256), 0,
                                         stream, d_logtheta_.p, d_Wf_.p, d_Wb_.p, n_inner_));
@@ -702,6 +705,22 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   const int K = K_, C = C_;
   std::vector<float> h;
+  if (!block_) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
+    std::vector<float> ea((size_t)n_edges_), lf((size_t)V_ * K * C);
+    general_->get_aggregates(ea.data(), n_edges_, lf.data(), (int64_t)lf.size());
+    if (edge_aggr) {
+      std::fill(edge_aggr, edge_aggr + (size_t)V_ * K * K, 0.f);
+      for (int64_t e = 0; e < n_edges_; ++e)
+        if (edge2param_[e]) {
+          const int64_t src = sum_param_src_[edge2param_[e] - 1];
+          edge_aggr[(size_t)var_of_inner_[src / ((int64_t)K * K)] * K * K + src % ((int64_t)K * K)] = ea[e];
+        }
+    }
+    if (leaf_flow)
+      for (size_t q = 0; q < input_order_.size(); ++q)
+        std::copy(lf.begin() + q * C, lf.begin() + (q + 1) * C, leaf_flow + (size_t)input_order_[q] * C);
+    return;
+  }
   if (edge_aggr) {
     fetch(h, d_edge_aggr_.p, d_edge_aggr_.n, stream);
     std::fill(edge_aggr, edge_aggr + (size_t)V_ * K * K, 0.f);
@@ -900,6 +919,7 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
 
 void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (!block_) return general()->loglikelihoods(b, d_ll);
   stage_batch(b);
   run_forward(dev(b.batch), d_ll);
 }
@@ -907,6 +927,11 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (!block_) {
+    general()->flows(b, rate, nullptr, d_ll);
+    have_flows_ = true;
+    return;
+  }
   stage_batch(b);
   HcltDev d = dev(b.batch);
   run_forward(d, d_ll);
@@ -944,6 +969,12 @@ void HcltCircuit::read_timing(float* ms, int n) {
 
 void HcltCircuit::em_update(float pseudocount, float inertia) {
   if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
+  if (!block_) {
+    general_->em_update(pseudocount, inertia);
+    PCM_HIP(hipStreamSynchronize(stream));
+    pull_from_general();
+    return;
+  }
   PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)),
                                         dim3(128), 0, stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p,
                                         d_edge_aggr_.p, n_inner_, pseudocount, inertia));

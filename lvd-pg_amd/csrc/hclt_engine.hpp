@@ -131,6 +131,7 @@ class HcltCircuit : public pcm_circuit {
 
  private:
   int V_, K_, C_, n_inner_, root_;
+  bool block_ = true;   // the hidden size has block kernels; else everything runs on the layered engine
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;
   std::vector<std::vector<int32_t>> children_;
   int n_fwd_steps_ = 0, n_bwd_steps_ = 0, lds_slots_ = 0, max_lds_ = 0;

@@ -47,9 +47,10 @@ def test_version_and_error_reporting_without_a_gpu(cdll):
     rc = cdll.pcm_hclt_create(None, 4, 16, 8, ctypes.byref(out))
     assert rc == -1 and out.value is None
     assert b"null" in cdll.pcm_last_error().lower() or len(cdll.pcm_last_error()) > 0
-    # unsupported hidden size and a malformed tree are rejected before any device work
+    # bad sizes and a malformed tree are rejected before any device work
     par = (ctypes.c_int32 * 3)(-1, 0, 0)
-    assert cdll.pcm_hclt_create(par, 3, 7, 8, ctypes.byref(out)) in (-1, -2, -3)
+    assert cdll.pcm_hclt_create(par, 3, 0, 8, ctypes.byref(out)) == -2
+    assert cdll.pcm_hclt_create(par, 3, 16, 300, ctypes.byref(out)) == -2
     two_roots = (ctypes.c_int32 * 3)(-1, -1, 0)
     assert cdll.pcm_hclt_create(two_roots, 3, 16, 8, ctypes.byref(out)) == -2
     cycle = (ctypes.c_int32 * 3)(-1, 2, 1)

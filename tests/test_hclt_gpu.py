@@ -135,3 +135,48 @@ def test_ten_em_steps_track_oracle(gpu, oracle):
     for v, blk in th_ref.items():
         assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
     assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
+
+
+@pytest.mark.parametrize("V,K,C,B", [(6, 8, 5, 40), (5, 128, 7, 33), (9, 3, 4, 70)])
+def test_hidden_sizes_without_block_kernels(gpu, oracle, V, K, C, B):
+    """Hidden sizes other than 16 / 32 / 64 run on the layered engine behind the same HCLT
+    interface (block-form parameters and flows, EM step, KL, sampling)."""
+    torch, P = gpu
+    bpc = _compare_step(gpu, oracle, V, K, C, B, seed=7 * K + V)
+    assert bpc.size("hidden_categories") == K
+    theta, leaf = bpc.get_params()
+    q = P.hclt_from_clt(bpc.clt_parent, C, K)          # uniform parameters
+    assert P.kld(bpc, bpc) < 1e-5 and P.kld(bpc, q) > 0
+    n_inner = bpc.size("inner_tree_nodes")
+    g = torch.Generator(device="cuda").manual_seed(K)
+    u1 = torch.rand((16, n_inner * K), device="cuda", generator=g).clamp_(1e-9, 1 - 1e-7)
+    u2 = torch.rand((16, V, C), device="cuda", generator=g).clamp_(1e-9, 1 - 1e-7)
+    s = P.sample(bpc, -torch.log(-torch.log(u1)), -torch.log(-torch.log(u2))).cpu().numpy()
+    assert s.shape == (16, V) and (s < C).all()
+
+
+def test_config_hclt48_k128(gpu, oracle):
+    """Benchmark configuration with K = 128 (48 variables = one 4x4x3 patch, 256 categories,
+    Dirichlet(1) parameters, batch 4096): ten mini-batch EM steps with step size 0.1 and
+    pseudocount 0.1; the first step is checked against the oracle on a subset, the run for a
+    rising likelihood."""
+    torch, P = gpu
+    O = oracle
+    from pcmi355 import workloads
+    from helpers import rel_err
+    V, K, C, B = 48, 128, 256, 4096
+    data = workloads.grf_images(B, 4, 4, 3, 2.0, 0.8, seed=1002)
+    parent = workloads.chow_liu_parent(data)
+    theta, leaf = workloads.init_params(parent, K, C, 1102, kind="dirichlet")
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(theta, leaf)
+    d = torch.from_numpy(data).cuda()
+    sub = 48
+    ch, _ = O.clt_children(parent)
+    fc = O.hclt_flat(parent, K, C, {v: theta[v] for v in range(V) if ch[v]}, leaf)
+    ll_ref = O.forward(fc, data[:sub])[-1]
+    ll = P.loglikelihoods(bpc, d).cpu().numpy()
+    assert rel_err(ll[:sub], ll_ref).max() < LL_RTOL
+    lls = P.mini_batch_em_with_reg(bpc, d, 10, batch_size=B, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert all(b > a for a, b in zip(lls, lls[1:])), lls
+    np.testing.assert_allclose(lls[0], ll.mean(), rtol=1e-5)
