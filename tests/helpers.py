@@ -141,3 +141,15 @@ def random_dag(V, C, rng, width=4, depth=3):
             outs.append(O.summate(*[prods[q] for q in sel], logps=log_dirichlet(rng, m)))
         return outs
     return region(np.arange(V), 0)[0]
+
+
+def multihead_hclt(parent, K, C, H, rng):
+    """A multi-head HCLT as the patch circuits of the progressive-growing experiments use it:
+    one HCLT body, H head sum nodes over the K products under the root
+    (exps/progressive_growing/parallel_PG.jl:214-225 builds such circuits for
+    CuMultiHeadBitsProbCircuit).  Returns (heads, body root)."""
+    theta, leaf = O.random_hclt_params(parent, K, C, rng)
+    root = O.hclt_dag(parent, K, C, theta, leaf)
+    prods = root.children
+    heads = [O.summate(*prods, logps=log_dirichlet(rng, len(prods))) for _ in range(H)]
+    return heads, root

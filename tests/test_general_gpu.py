@@ -217,6 +217,61 @@ def test_multihead_soft_mask_em_matches_oracle(gpu, oracle):
     assert len(lls) == 2 and lls[1] > lls[0]
 
 
+def test_config_patch_circuit_with_128_heads_and_top_hclt(gpu, oracle):
+    """Patch-clustered configuration at its real shape: one 8x8x3 patch circuit (192 variables,
+    K = 32) with 128 heads selected by a cluster id, and the top HCLT over 64 cluster indices
+    (K = 64, 128 categories), batch 1024.  Oracle on a subset; on the whole batch the flows
+    obey conservation and EM raises the likelihood."""
+    torch, P = gpu
+    O = oracle
+    import sys
+    from pcmi355 import workloads
+    from helpers import multihead_hclt, rel_err
+    sys.setrecursionlimit(20000)
+    V, K, C, H, B = 192, 32, 256, 128, 1024
+    rng = np.random.default_rng(1004)
+    data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
+    parent = workloads.chow_liu_parent(data)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    bpc = _compile(P, heads, V, C, heads=H)
+    assert bpc.size("heads") == H
+    cluster = rng.integers(0, H, size=B)
+    mask = np.zeros((B, H), np.float32)
+    mask[np.arange(B), cluster] = 1.0
+    d = torch.from_numpy(data).cuda()
+    hm = torch.from_numpy(mask).cuda()
+    ll = P.probs_flows_circuit(bpc, d, head_mask=hm).cpu().numpy()
+    sub = 24
+    fc = O.bits_compile(O.summate(*heads), C, V)
+    root_ids = (bpc.table("heads") - 1).astype(np.int32)
+    mars = O.forward(fc, data[:sub])
+    want = mars[root_ids[cluster[:sub]], np.arange(sub)]
+    assert rel_err(ll[:sub], want).max() < LL_RTOL
+    per_head = P.loglikelihoods(bpc, d[:sub].contiguous()).cpu().numpy()
+    assert per_head.shape == (sub, H)
+    assert rel_err(per_head, mars[root_ids].T).max() < LL_RTOL
+    ea, lf = bpc.get_aggregates()
+    np.testing.assert_allclose(lf.sum(), B * V, rtol=1e-4)     # one unit of flow per example and variable
+    lls = P.mini_batch_em_for_multihead_pc(bpc, d, hm, 3, batch_size=B, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert lls[2] > lls[1] > lls[0]
+
+    # top circuit: hard cluster ids of the 64 patches as uint8 data with 128 categories
+    Vt, Kt, Ct = 64, 64, 128
+    ids = rng.integers(0, Ct, size=(B, Vt)).astype(np.uint8)
+    ids[:, 1:] = (ids[:, :-1] + rng.integers(0, 3, size=(B, Vt - 1))) % Ct      # some dependence
+    tp = workloads.chow_liu_parent(ids)
+    theta, leaf = workloads.init_params(tp, Kt, Ct, 2004)
+    top = P.hclt_from_clt(tp, Ct, Kt)
+    top.set_params(theta, leaf)
+    dt = torch.from_numpy(ids).cuda()
+    ch, _ = O.clt_children(tp)
+    ft = O.hclt_flat(tp, Kt, Ct, {v: theta[v] for v in range(Vt) if ch[v]}, leaf)
+    llt = P.loglikelihoods(top, dt).cpu().numpy()
+    assert rel_err(llt[:sub], O.forward(ft, ids[:sub])[-1]).max() < LL_RTOL
+    lls = P.mini_batch_em_with_reg(top, dt, 3, batch_size=B, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert lls[2] > lls[1] > lls[0]
+
+
 def test_hclt_general_form_matches_block_engine(gpu, oracle):
     """The same HCLT through both engines: LL, parameter vector after an EM step."""
     torch, P = gpu
