@@ -321,7 +321,8 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = lane & 15, g = lane >> 4;
   const int n = blockIdx.x;
-  const StatNode nd = nodes[n];
+  const StatNode* __restrict__ np = nodes + n;   // fields are read where needed (a local copy indexed by the pass would live in scratch)
+  const int own_var = np->var, n_hist = np->n_hist;
   const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)g * 16, vx = (uint32_t)b * 4;
   const int hist_sz = d.C * HS;
   unsigned* hist = reinterpret_cast<unsigned*>(smem);
@@ -330,13 +331,13 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 
   const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + (size_t)n * d.tile_stride, d.tile_stride);
   const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);
-  const __amdgpu_buffer_rsrc_t rL0 = make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)nd.var * d.leaf_stride, d.leaf_stride);
+  const __amdgpu_buffer_rsrc_t rL0 = make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)own_var * d.leaf_stride, d.leaf_stride);
   auto child_rsrc = [&](int c) {
     return (c & 1) ? make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)(c >> 3) * d.leaf_stride, d.leaf_stride)
                    : make_rsrc(reinterpret_cast<const char*>(d.O) + (size_t)(max(c, 0) >> 3) * d.tile_stride, d.tile_stride);
   };
-  const __amdgpu_buffer_rsrc_t rC1 = child_rsrc(nd.c[0]), rC2 = child_rsrc(nd.c[1]), rC3 = child_rsrc(nd.c[2]);
-  const int c1 = nd.c[0], c2 = nd.c[1], c3 = nd.c[2];
+  const int c1 = np->c[0], c2 = np->c[1], c3 = np->c[2];
+  const __amdgpu_buffer_rsrc_t rC1 = child_rsrc(c1), rC2 = child_rsrc(c2), rC3 = child_rsrc(c3);
   auto child_load = [&](__amdgpu_buffer_rsrc_t r, int c, uint32_t xpack, uint32_t slice_off, Tile<K>& t) {
     if (c & 1) lean_row_load<K>(r, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), 0, t);
     else lean_tile_load<K>(r, vtile, (int)slice_off, t);
@@ -351,7 +352,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
 
   const int last = d.nslices - 1;
-  for (int pass = 0; pass < nd.n_hist; ++pass) {
+  for (int pass = 0; pass < n_hist; ++pass) {
     for (int i = threadIdx.x; i < 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
     __syncthreads();
     const int sel = pass;   // category byte of the variable histogrammed in this pass
@@ -442,7 +443,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     __syncthreads();
     {
       const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
-      float* dst = leaf_flow + (size_t)nd.hvar[pass] * d.C * K;
+      float* dst = leaf_flow + (size_t)np->hvar[pass] * d.C * K;
       for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
         const int c = i / K, j = i % K;
         const float val = (float)hist[c * HS + j] * hi_inv + (float)hist[hist_sz + c * HS + j] * lo_inv;
