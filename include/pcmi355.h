@@ -184,6 +184,19 @@ int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_no
                int32_t batch, uint8_t* d_out);
 
 /*
+ * Relaxed sampling at a positive temperature: `gumbel_sample(mbpc, params, ...; temperature,
+ * no_gumbel)` (src/queries/sample.jl:338-383) for one parameter row per circuit, with the
+ * noise supplied instead of drawn in the kernel (:45).  d_node_noise is laid out as for
+ * pcm_sample, or NULL for no_gumbel = true; d_out receives the soft assignment
+ * [batch][num_vars][num_cats]: every variable's top-down probabilities times its input
+ * nodes' distributions (:262-284).  On an HCLT the sum nodes of one tree node share their
+ * noise column per hidden state; compile the circuit with pcm_circuit_create for one
+ * independent draw per sum edge.
+ */
+int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature, int32_t batch,
+                    float* d_out);
+
+/*
  * Adam ascent step on the sum parameters followed by per-sum-node normalisation
  * (src/sgd/adam.jl:63-86, :88-127, :318-319).  d_grad, d_params (unnormalised
  * log-parameters), d_m, d_v are device vectors in parameter-vector order over the sum

@@ -172,6 +172,10 @@ int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_no
   return guarded([&] { need(c)->sample(d_node_noise, d_leaf_noise, batch, d_out); });
 }
 
+int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  return guarded([&] { need(c)->sample_soft(d_node_noise, temperature, batch, d_out); });
+}
+
 int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
                   float b1, float b2, float eps, int32_t t) {
   return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });

@@ -100,6 +100,7 @@ struct pcm_circuit {
   virtual int64_t sample_noise_size() const = 0;
   virtual void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
                       uint8_t* d_out) = 0;
+  virtual void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) = 0;
   virtual void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
                          float b1, float b2, float eps, int t) = 0;
 };

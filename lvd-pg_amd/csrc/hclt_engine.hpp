@@ -117,6 +117,7 @@ class HcltCircuit : public pcm_circuit {
               uint8_t* d_out) override;
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
                  float b2, float eps, int t) override;
+  void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
 
   void set_block_params(const float* theta, const float* leaf);
   void get_block_params(float* theta, float* leaf);

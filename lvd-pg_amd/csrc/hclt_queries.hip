@@ -48,6 +48,13 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   g->sample_with_slots(d_node_noise, slots.p, sample_noise_size(), d_leaf_noise, batch, d_out);
 }
 
+void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  SparseCircuit* g = general();
+  DevBuf<int32_t> slots;
+  slots.upload(noise_slot_, stream);
+  g->sample_soft_with_slots(d_node_noise, slots.p, sample_noise_size(), temperature, batch, d_out);
+}
+
 void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
                             float b2, float eps, int t) {
   general()->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t);

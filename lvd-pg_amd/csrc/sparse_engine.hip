@@ -415,6 +415,73 @@ __global__ void sparse_sample_kernel(SparseDev d, int n0, const int32_t* __restr
   }
 }
 
+// Relaxed (Gumbel-softmax) sampling at temperature T, src/queries/sample.jl:8-148.  Pass 1,
+// thread = (sum node, example): the normaliser of the node's edge weights exp((logp + g)/T)
+// (sample.jl:37-51), kept as (max, sum of exp relative to the max) so that small temperatures
+// cannot overflow -- after normalisation identical to the reference's plain sum.
+__global__ void sparse_soft_norm_kernel(SparseDev d, int n_nodes, const int32_t* __restrict__ noise_slot,
+                                        const int64_t* __restrict__ edge2param, int64_t noise_stride,
+                                        const float* __restrict__ noise, float inv_t, float* __restrict__ emax,
+                                        float* __restrict__ esum) {
+  const int n = blockIdx.x;
+  const int b = blockIdx.y * blockDim.x + threadIdx.x;
+  if (n >= n_nodes || b >= d.B || d.type[n] != kSum) return;
+  const float* g = noise ? noise + (size_t)b * noise_stride : nullptr;
+  float m = -INFINITY;
+  for (int e = d.node_e0[n]; e < d.node_e1[n]; ++e) {
+    const float v = (d.logp[e] + (g ? g[noise_slot ? noise_slot[e] : edge2param[e] - 1] : 0.f)) * inv_t;
+    m = fmaxf(m, v);
+  }
+  float s = 0.f;
+  for (int e = d.node_e0[n]; e < d.node_e1[n]; ++e) {
+    const float v = (d.logp[e] + (g ? g[noise_slot ? noise_slot[e] : edge2param[e] - 1] : 0.f)) * inv_t;
+    s += expf(v - m);
+  }
+  emax[(size_t)n * d.Bp + b] = m;
+  esum[(size_t)n * d.Bp + b] = s;
+}
+
+// Pass 2, one layer top-down, thread = (node, example): top-down probability gathered over
+// the incoming edges (sample.jl:105-140): a sum edge hands on td[parent] * w / normaliser, a
+// product edge td[parent], to prime and sub alike.
+__global__ void sparse_soft_down_kernel(SparseDev d, int n0, int root, const int32_t* __restrict__ noise_slot,
+                                        const int64_t* __restrict__ edge2param, int64_t noise_stride,
+                                        const float* __restrict__ noise, float inv_t, const float* __restrict__ emax,
+                                        const float* __restrict__ esum, float* __restrict__ td) {
+  const int n = d.order[n0 + blockIdx.x];
+  const int b = blockIdx.y * blockDim.x + threadIdx.x;
+  if (b >= d.B) return;
+  const float* g = noise ? noise + (size_t)b * noise_stride : nullptr;
+  float acc = n == root ? 1.f : 0.f;
+  for (int i = d.in_ptr[n]; i < d.in_ptr[n + 1]; ++i) {
+    const int e = d.in_edge[i] >> 1;
+    const int p = d.e_parent[e];
+    float f = td[(size_t)p * d.Bp + b];
+    if (d.type[p] == kSum) {
+      const float v = (d.logp[e] + (g ? g[noise_slot ? noise_slot[e] : edge2param[e] - 1] : 0.f)) * inv_t;
+      f *= expf(v - emax[(size_t)p * d.Bp + b]) / esum[(size_t)p * d.Bp + b];
+    }
+    acc += f;
+  }
+  td[(size_t)n * d.Bp + b] = acc;
+}
+
+// Pass 3, thread = (variable, example, category): out[b][v][c] = sum over the variable's input
+// nodes of td * exp(leaf_logp[c]) (sample.jl:262-284).
+__global__ void sparse_soft_leaf_kernel(SparseDev d, const int32_t* __restrict__ var_ptr,
+                                        const int32_t* __restrict__ var_nodes, int V, const float* __restrict__ td,
+                                        float* __restrict__ out) {
+  const int v = blockIdx.x, b = blockIdx.y;
+  for (int c = threadIdx.x; c < d.C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int i = var_ptr[v]; i < var_ptr[v + 1]; ++i) {
+      const int n = var_nodes[i];
+      acc += td[(size_t)n * d.Bp + b] * expf(d.leaf[d.in_off[n] + c]);
+    }
+    out[((size_t)b * V + v) * d.C + c] = acc;
+  }
+}
+
 // Adam on the sum parameters: src/sgd/adam.jl:318-319 (moments), :63-76 (ascent step).
 __global__ void sparse_adam_kernel(int64_t n, const float* __restrict__ grad, float* __restrict__ params,
                                    float* __restrict__ m, float* __restrict__ v, float lr, float b1, float b2,
@@ -826,6 +893,49 @@ void SparseCircuit::sample_with_slots(const float* d_node_noise, const int32_t* 
 
 void SparseCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
   sample_with_slots(d_node_noise, nullptr, sample_noise_size(), d_leaf_noise, batch, d_out);
+}
+
+void SparseCircuit::sample_soft_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
+                                           float temperature, int32_t batch, float* d_out) {
+  if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
+  if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  if (!(temperature > 0.f)) fail(PCM_ERR_ARG, "temperature must be positive");
+  if (!fc_.heads.empty()) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
+  ensure_batch(batch);
+  const int Bp = ceil_div(batch, 64) * 64;
+  d_grad_.ensure((size_t)fc_.n_nodes() * Bp);   // normaliser sums; maxima go to the value array, td to the flow array
+  if (d_var_ptr_.n == 0) {
+    std::vector<int32_t> vp(fc_.num_vars + 1, 0), vn(fc_.input_nodes.size());
+    for (int32_t n : fc_.input_nodes) vp[fc_.in_var[n] + 1]++;
+    for (int v = 0; v < fc_.num_vars; ++v) vp[v + 1] += vp[v];
+    std::vector<int32_t> fill(vp.begin(), vp.end() - 1);
+    for (int32_t n : fc_.input_nodes) vn[fill[fc_.in_var[n]]++] = n;
+    d_var_ptr_.upload(vp, stream);
+    d_var_nodes_.upload(vn, stream);
+  }
+  DevBuf<int64_t> e2p;
+  std::vector<int64_t> e2pv = fc_.edge2param;
+  if (e2pv.empty()) e2pv.push_back(0);
+  e2p.upload(e2pv, stream);
+  SparseDev d = SPARSE_DEV(batch, Bp, nullptr);
+  const float inv_t = 1.f / temperature;
+  hipLaunchKernelGGL(sparse_soft_norm_kernel, dim3((unsigned)fc_.n_nodes(), Bp / 64), dim3(64), 0, stream, d,
+                     (int)fc_.n_nodes(), d_noise_slot, e2p.p, noise_stride, d_node_noise, inv_t, d_mars_.p, d_grad_.p);
+  for (int l = n_layers_ - 1; l >= 0; --l) {
+    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
+    hipLaunchKernelGGL(sparse_soft_down_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0, (int)fc_.n_nodes() - 1,
+                       d_noise_slot, e2p.p, noise_stride, d_node_noise, inv_t, d_mars_.p, d_grad_.p, d_flows_.p);
+  }
+  hipLaunchKernelGGL(sparse_soft_leaf_kernel, dim3(fc_.num_vars, batch), dim3(std::min(256, ceil_div(fc_.num_cats, 64) * 64)),
+                     0, stream, d, d_var_ptr_.p, d_var_nodes_.p, fc_.num_vars, d_flows_.p, d_out);
+  check_launch("sparse_sample_soft");
+  PCM_HIP(hipStreamSynchronize(stream));
+  last_batch_ = 0;       // the value / flow arrays no longer hold a batch
+  have_flows_ = false;
+}
+
+void SparseCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  sample_soft_with_slots(d_node_noise, nullptr, sample_noise_size(), temperature, batch, d_out);
 }
 
 // ---- Adam ---------------------------------------------------------------------------------

@@ -58,6 +58,9 @@ class SparseCircuit : public pcm_circuit {
   void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) override;
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1, float b2,
                  float eps, int t) override;
+  void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
+  void sample_soft_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
+                              float temperature, int32_t batch, float* d_out);
 
   void get_node_values(float* mars, float* flows, int64_t n);
   void get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf);
@@ -84,7 +87,7 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_logp_, d_leaf_, d_edge_aggr_, d_leaf_flow_, d_mars_, d_flows_, d_kld_, d_edge_kld_, d_grad_;
   // incoming edges per node (down direction)
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
-  DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_;
+  DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
   int cap_batch_ = 0, last_batch_ = 0;
   bool have_flows_ = false;

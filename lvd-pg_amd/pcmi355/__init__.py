@@ -8,5 +8,5 @@ memory and streams come from torch; everything numeric happens in the HIP librar
 from .circuits import BitsCircuit, HcltCircuit, hclt_from_clt, compile_circuit, compile_multihead  # noqa: F401
 from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
-                      mini_batch_em_for_multihead_pc, multihead_loglikelihoods)
+                      mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample)
 from ._lib import PcmError, LIB_PATH  # noqa: F401

@@ -198,6 +198,25 @@ def sample(bpc, node_noise, leaf_noise):
     return out
 
 
+def gumbel_sample(bpc, num_samples, *, temperature, node_noise=None):
+    """`gumbel_sample(mbpc, params, num_vars, par_buffer_size; temperature, no_gumbel)`
+    (src/queries/sample.jl:338-383): relaxed top-down sampling.  node_noise
+    [num_samples, sample_noise_size] float32 on the GPU, or None for no_gumbel = true.
+    Returns the soft assignment [num_samples, V, C] (float32, GPU)."""
+    nv, nc = bpc.size("variables"), bpc.size("categories")
+    need = int(lib.pcm_sample_noise_size(bpc.handle))
+    if node_noise is not None:
+        if tuple(node_noise.shape) != (num_samples, need):
+            raise ValueError(f"noise shape must be ({num_samples}, {need})")
+        node_noise = node_noise.contiguous().float()
+        dev = node_noise.device
+    else:
+        dev = torch.device("cuda")
+    out = torch.empty((num_samples, nv, nc), dtype=torch.float32, device=dev)
+    check(lib.pcm_sample_soft(bpc.handle, _dev_ptr(node_noise), float(temperature), int(num_samples), out.data_ptr()))
+    return out
+
+
 def adam_step(bpc, grad, params, m, v, *, lr, beta1=0.9, beta2=0.999, eps=1e-8, t=1):
     """One optimiser step of `adam` (src/sgd/adam.jl:318-325): moving averages, ascent
     update of the unnormalised sum parameters, per-node normalisation into the circuit."""

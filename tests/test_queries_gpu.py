@@ -264,3 +264,56 @@ def test_adam_step_matches_oracle(gpu, oracle):
     ch, root = O.clt_children(parent)
     v0 = next(v for v in range(V) if ch[v] and v != root)
     assert np.abs(np.exp(th[v0].astype(np.float64)).sum(axis=1) - 1).max() < 1e-5
+
+
+@pytest.mark.parametrize("temperature", [1.0, 0.4])
+def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
+    """Soft top-down pass (src/queries/sample.jl:37-51, :105-140, :262-284) with supplied noise
+    on a DAG with shared sub-circuits and on an HCLT, row by row against the oracle; invariants
+    of test/queries/sample_tests.jl:34-53."""
+    torch, P = gpu
+    O = oracle
+    from helpers import random_dag, make_hclt, block_theta
+    rng = np.random.default_rng(17)
+    V, C, B = 7, 5, 6
+    root = random_dag(V, C, rng, width=3)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, root, V, C)
+    n_sum = bpc.num_inner_params()
+    noise = _gumbel(rng, (B, n_sum))
+    out = P.gumbel_sample(bpc, B, temperature=temperature, node_noise=torch.from_numpy(noise).cuda()).cpu().numpy()
+    assert out.shape == (B, V, C)
+    np.testing.assert_allclose(out.sum(axis=2), 1.0, rtol=1e-4)
+    pe = fc.sum_param_edges()
+    for b in range(B):
+        g = np.zeros(fc.n_edges, np.float64)
+        g[pe] = noise[b]
+        _, want = O.gumbel_soft(fc, g, temperature, double=True)
+        np.testing.assert_allclose(out[b], want, rtol=1e-4, atol=1e-7)
+    # no noise, temperature 1: the circuit's marginals
+    import itertools
+    allx = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    p = np.exp(O.forward(fc, allx, double=True)[-1])
+    plain = P.gumbel_sample(bpc, 2, temperature=1.0).cpu().numpy()
+    for v in range(V):
+        marg = np.array([p[allx[:, v] == c].sum() for c in range(C)])
+        np.testing.assert_allclose(plain[0, v], marg, rtol=1e-4)
+    assert np.array_equal(plain[0], plain[1])
+
+    # HCLT: the K sum nodes of a tree node share the noise column of each hidden state
+    Vh, K, Ch = 6, 16, 4
+    parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23)
+    h = P.hclt_from_clt(parent, Ch, K)
+    h.set_params(block_theta(parent, K, theta), leaf)
+    ch, _ = O.clt_children(parent)
+    inner = [v for v in O.clt_bottom_up(parent) if ch[v]]
+    hn = _gumbel(rng, (3, len(inner) * K))
+    got = P.gumbel_sample(h, 3, temperature=temperature, node_noise=torch.from_numpy(hn).cuda()).cpu().numpy()
+    for b in range(3):
+        g = np.zeros(flat.n_edges, np.float64)
+        for r, v in enumerate(inner):
+            nk = len(flat.meta["sum_node"][v])
+            e0 = flat.meta["edge_of"][v]
+            g[e0:e0 + nk * K] = np.tile(hn[b, r * K:(r + 1) * K], nk)
+        _, want = O.gumbel_soft(flat, g, temperature, double=True)
+        np.testing.assert_allclose(got[b], want, rtol=1e-4, atol=1e-7)
