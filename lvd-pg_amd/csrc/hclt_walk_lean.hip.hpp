@@ -306,7 +306,8 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
 // (the node is fixed, only the slice moves), typed operands behind scalar branches, every
 // register reloaded right after its last use, the waves' partial edge-flow blocks combined by
 // a plain LDS sum.  A node with leaf children runs one pass over the batch per variable it has
-// to histogram (the LDS holds one histogram); the edge flows are accumulated in pass 0.
+// to histogram (the LDS holds one histogram): pass 0 does all the arithmetic and leaves the
+// child-flow tiles G where it read R from; the passes of the leaf children re-read G only.
 constexpr int kStatLeanWaves = 16;
 
 template <int K>
@@ -351,12 +352,27 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 #pragma unroll
     for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
 
+  // fixed-point limbs of this lane's K/4 flows (clamped to [0, 1]) into row x of the histogram
+  auto histogram = [&](const Tile<K>& t, uint32_t xpack, int sel) {
+    const uint32_t x = (xpack >> (8 * sel)) & 0xffu;
+    unsigned* hrow = hist + x * HS + 4 * g;
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale, 0.f, scale);
+        const unsigned hi = (unsigned)v;
+        const unsigned lo = (unsigned)(__builtin_amdgcn_fractf(v) * scale);
+        __hip_atomic_fetch_add(&hrow[kt * 16 + i], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_fetch_add(&hrow[hist_sz + kt * 16 + i], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+  };
+
   const int last = d.nslices - 1;
   for (int pass = 0; pass < n_hist; ++pass) {
     for (int i = threadIdx.x; i < 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
     __syncthreads();
-    const int sel = pass;   // category byte of the variable histogrammed in this pass
-
+    if (pass == 0) {
     // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
     // repeated loads), categories of the second
     Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
@@ -392,7 +408,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
       // (2) E, the edge flows, then G = E .* (R W)
       const float m = tile_rowmax<K>(e);
       tile_exp_sub<K>(e, m);
-      if (pass == 0) {
+      {
         // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
         // go through the wave's pad to reach the [state][example] operand layout.  A wave's LDS
         // accesses execute in order, so the pad needs no barrier between its phases.
@@ -424,20 +440,33 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
       lean_tile_load<K>(rR, vtile, (int)so1, R);   // next slice's ratios, after the last use of these
-      // (3) histogram: fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
-      if (s0 * kSlice + b < d.B) {
-        const uint32_t x = (xh >> (8 * sel)) & 0xffu;
-        unsigned* hrow = hist + x * HS + 4 * g;
+      if (n_hist > 1) {
+        // the later passes (one per leaf child) only need G: it replaces the tile of R just consumed
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale, 0.f, scale);
-            const unsigned hi = (unsigned)v;
-            const unsigned lo = (unsigned)(__builtin_amdgcn_fractf(v) * scale);
-            __hip_atomic_fetch_add(&hrow[kt * 16 + i], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            __hip_atomic_fetch_add(&hrow[hist_sz + kt * 16 + i], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-          }
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), rR, (int)(vtile + kt * 1024),
+                                                 (int)((uint32_t)s0 * (kSlice * K * 4)), 0);
+      }
+      // (3) histogram
+      if (s0 * kSlice + b < d.B) histogram(t, xh, 0);
+    }
+    } else {
+      // leaf child `pass`: G comes back from where pass 0 left it; only the categories differ
+      Tile<K> T;
+      uint32_t xc, xn;
+      {
+        const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
+        xc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sa * (kSlice * 4), 0);
+        xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sb * (kSlice * 4), 0);
+        lean_tile_load<K>(rR, vtile, (int)((uint32_t)sa * (kSlice * K * 4)), T);
+      }
+      for (int s0 = wave; s0 < d.nslices; s0 += kStatLeanWaves) {
+        const int s1 = min(s0 + kStatLeanWaves, last), s2 = min(s0 + 2 * kStatLeanWaves, last);
+        const uint32_t xh = xc;
+        xc = xn;
+        xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
+        if (s0 * kSlice + b < d.B) histogram(T, xh, pass);
+        lean_tile_load<K>(rR, vtile, (int)((uint32_t)s1 * (kSlice * K * 4)), T);
       }
     }
     __syncthreads();
