@@ -76,6 +76,106 @@ def cpu_baseline(cfg, sample):
                 sample=f"one EM step on the first {sample} examples of the batch, {dt:.1f} s"), ll
 
 
+def _timed(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def secondary(args):
+    """The other configurations, all on the layered engine (not the headline; same JSON shape).
+    Their byte counts are the layered engine's own minimum: per example 4 bytes written per node
+    and 8 read per edge going up; going down 4 written per node and 16 read per incoming edge."""
+    import numpy as np
+    import torch
+    import pcmi355 as P
+    from pcmi355 import workloads
+    from pcmi355._lib import lib, check
+    rng = np.random.default_rng(0)
+    out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic", "cpu_baseline": None}
+    if args.workload == "c2_hclt48_k128":
+        V, K, C, B = 48, 128, 256, 4096
+        data = workloads.grf_images(B, 4, 4, 3, 2.0, 0.8, seed=1002)
+        parent = workloads.chow_liu_parent(data)
+        theta, leaf = workloads.init_params(parent, K, C, 1102, kind="dirichlet")
+        bpc = P.hclt_from_clt(parent, C, K)
+        bpc.set_params(theta, leaf)
+        d = torch.from_numpy(data).cuda()
+        ll = torch.empty(B, device="cuda")
+        dt = _timed(torch, lambda: check(lib.pcm_em_step(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B,
+                                                          0.0, 0.1, 0.9, ll.data_ptr())), args.steps, args.warmup)
+        nn, ne = bpc.num_nodes(), bpc.num_edges()
+        algo = B * (8 * nn + 24 * ne)
+        out.update(metric="examples/sec fwd+bwd+EM, 48-var HCLT K=128 (layered engine)", value=B / dt, unit="examples/s",
+                   config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
+                           "nodes": nn, "edges": ne})
+    elif args.workload == "c4_patch_multihead":
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        sys.setrecursionlimit(20000)
+        from helpers import multihead_hclt, describe_dag      # DAG builders shared with the tests
+        V, K, C, H, B = 192, 32, 256, 128, 1024
+        data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
+        parent = workloads.chow_liu_parent(data)
+        heads, _ = multihead_hclt(parent, K, C, H, rng)
+        g = describe_dag(heads)
+        bpc = P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"],
+                                g["input_logp"], V, C, H)
+        mask = np.zeros((B, H), np.float32)
+        mask[np.arange(B), rng.integers(0, H, size=B)] = 1.0
+        d = torch.from_numpy(data).cuda()
+        hm = torch.from_numpy(mask).cuda().t().contiguous()
+        ll = torch.empty(B, device="cuda")
+
+        def step():
+            check(lib.pcm_flows(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(), ll.data_ptr()))
+            check(lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+        dt = _timed(torch, step, args.steps, args.warmup)
+        nn, ne = bpc.num_nodes(), bpc.num_edges()
+        algo = B * (8 * nn + 24 * ne)
+        out.update(metric="examples/sec fwd+bwd+EM, 192-var patch circuit K=32 with 128 heads (layered engine)",
+                   value=B / dt, unit="examples/s",
+                   config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "heads": H,
+                           "batch": B, "nodes": nn, "edges": ne})
+    elif args.workload == "c5_variational":
+        cfg = workloads.make_config("c3_hclt3072_k32")
+        V, K, C, B = cfg["V"], cfg["K"], cfg["C"], cfg["B"]
+        p = P.hclt_from_clt(cfg["parent"], C, K)
+        p.set_params(cfg["theta"], cfg["leaf"])
+        q = P.hclt_from_clt(cfg["parent"], C, K)
+        q.set_params(*workloads.init_params(cfg["parent"], K, C, 4243, kind="dirichlet"))
+        n_inner = p.size("inner_tree_nodes")
+        gen = torch.Generator(device="cuda").manual_seed(5)
+        node_noise = -torch.log(-torch.log(torch.rand((B, n_inner * K), device="cuda", generator=gen).clamp_(1e-10, 1 - 1e-7)))
+        leaf_noise = torch.empty((B, V, C), device="cuda")
+        for s0 in range(0, B, 512):
+            leaf_noise[s0:s0 + 512] = -torch.log(-torch.log(torch.rand((512, V, C), device="cuda", generator=gen).clamp_(1e-10, 1 - 1e-7)))
+        P.kld(p, q)                                                   # builds both general forms
+        t_kld = _timed(torch, lambda: P.kld(p, q), args.steps, 1)
+        t_grad = _timed(torch, lambda: P.kld_backward(p, q, device=True), args.steps, 1)
+        t_samp = _timed(torch, lambda: P.sample(p, node_noise, leaf_noise), max(1, args.steps // 4), 1)
+        dt = t_samp
+        algo = 4 * B * (n_inner * K + V * C)                           # the noise tensors, read once
+        out.update(metric="samples/sec Gumbel-max from supplied noise, 3072-var HCLT K=32",
+                   value=B / t_samp, unit="samples/s",
+                   config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
+                   queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "sample": t_samp * 1e3})
+    else:
+        print(f"unknown workload {args.workload}", file=sys.stderr)
+        sys.exit(2)
+    out["ms_per_step"] = dt * 1e3
+    ach = algo / dt / 1e9
+    out["roofline"] = {"bound": "hbm", "kernel": "whole step", "achieved": ach, "peak": HBM_PEAK_GBS,
+                       "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -101,6 +201,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
+    if args.workload not in workloads.CONFIGS:
+        return secondary(args)
 
     cfg = workloads.make_config(args.workload)
     stats = workloads.tree_stats(cfg["parent"])

@@ -170,6 +170,10 @@ int pcm_kld(pcm_circuit* p, pcm_circuit* q, float* out);
 /* `kld_backward(mbpc, params1, params2; grad_wrt_logparams = true)`
  * (src/queries/kld.jl:593-649): gradients in parameter-vector order. */
 int pcm_kld_backward(pcm_circuit* p, pcm_circuit* q, float* grad_p, float* grad_q, int64_t n);
+/* The same with the two gradient vectors left in device memory (the reference copies them to
+ * the host, src/queries/kld.jl:640-648, and its optimiser takes them back to the device,
+ * src/sgd/adam.jl:318): the form pcm_adam_step consumes.  Queued on the circuit's stream. */
+int pcm_kld_backward_dev(pcm_circuit* p, pcm_circuit* q, float* d_grad_p, float* d_grad_q, int64_t n);
 
 /*
  * Gumbel-max ancestral sampling from supplied noise: the temperature -> 0 limit of

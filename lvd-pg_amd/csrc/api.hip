@@ -163,6 +163,10 @@ int pcm_kld_backward(pcm_circuit* p, pcm_circuit* q, float* gp, float* gq, int64
   });
 }
 
+int pcm_kld_backward_dev(pcm_circuit* p, pcm_circuit* q, float* d_grad_p, float* d_grad_q, int64_t n) {
+  return guarded([&] { need(p)->kld_backward_dev(need(q), d_grad_p, d_grad_q, n); });
+}
+
 int64_t pcm_sample_noise_size(const pcm_circuit* c) {
   int64_t r = -1;
   guarded([&] { r = need(const_cast<pcm_circuit*>(c))->sample_noise_size(); });

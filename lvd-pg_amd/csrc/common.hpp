@@ -97,6 +97,7 @@ struct pcm_circuit {
   virtual void em_update(float pseudocount, float inertia) = 0;
   virtual void kld(pcm_circuit* q, float* out) = 0;
   virtual void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) = 0;
+  virtual void kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) = 0;
   virtual int64_t sample_noise_size() const = 0;
   virtual void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
                       uint8_t* d_out) = 0;

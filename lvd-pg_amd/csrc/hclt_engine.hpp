@@ -112,6 +112,7 @@ class HcltCircuit : public pcm_circuit {
   void em_update(float pseudocount, float inertia) override;
   void kld(pcm_circuit* q, float* out) override;
   void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
+  void kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) override;
   int64_t sample_noise_size() const override { return (int64_t)n_inner_ * K_; }
   void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
               uint8_t* d_out) override;
@@ -157,7 +158,9 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<uint32_t> d_xn_;
   DevBuf<float> d_leaf_kc_;      // [V][K][C] copy for sampling
   DevBuf<float> d_kld_;          // scratch of the KL recursion
-  DevBuf<uint8_t> d_state_;
+  DevBuf<uint8_t> d_state_;      // [batch][n_inner] hidden states of a batch of samples
+  DevBuf<int32_t> d_sample_tabs_;   // sampler tables: parent of every inner node | state-giving node of every variable | level order
+  int sample_groups_ = 0;
   DevBuf<int64_t> d_sum_param_src_;
   int cap_slices_ = 0;
   bool have_flows_ = false;

@@ -1,10 +1,143 @@
-// KL recursion, Gumbel-max sampling and Adam for HCLT circuits.  These queries have no batch
-// of examples to slice (KL: one parameter row; sampling: a top-down choice per example), so
-// they run on the general engine over the circuit's general form; parameters are exchanged
-// in parameter-vector order, which both forms share.
+// KL recursion, sampling and Adam for HCLT circuits.  Gumbel-max sampling has its own kernels
+// on the block form (below); the KL recursion, the relaxed sampler and Adam run on the layered
+// engine over the circuit's general form, with parameters exchanged in parameter-vector order,
+// which both forms share.
 #include "hclt_engine.hpp"
 
+#include <hip/hip_runtime.h>
+
 namespace pcm {
+
+static void check_launch_q(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+// ---- Gumbel-max sampling on the block form -------------------------------------------------
+// A sample is a top-down walk: the root's single sum node picks hidden state
+// j* = argmax_j(theta_root[0][j] + g[b][root][j]); a tree node whose parent picked k picks
+// j* = argmax_j(theta_v[k][j] + g[b][v][j]) (first maximum wins); every variable then emits
+// argmax_c(leaf[v][j*][c] + g_leaf[b][v][c]) with j* the state of its own tree node (inner
+// nodes) or of its parent (leaf tree nodes).  Same additions and comparisons, in the same
+// order, as the layered engine's sampler on the circuit's general form.
+
+// States of the inner tree nodes.  K lanes per example (64/K examples per wave), one wave per
+// group for the whole tree.  Nodes come level by level from the root (`order`, padded with -1
+// to groups of four that never straddle a level), so the four nodes of a group are
+// independent and their parameter rows are fetched together: the walk is a chain of memory
+// latencies, one per group.  The chosen states live in LDS (one byte per node and example) and
+// leave through a coalesced copy at the end.  No barriers: a wave only reads its own examples.
+template <int K>
+__global__ __launch_bounds__(256) void hclt_sample_states_kernel(const float* __restrict__ logtheta,
+                                                                 const int32_t* __restrict__ parent_of,
+                                                                 const int32_t* __restrict__ order, int n_groups,
+                                                                 const float* __restrict__ node_noise, int n_inner,
+                                                                 int batch, uint8_t* __restrict__ states) {
+  constexpr int EPW = 64 / K;   // examples per wave
+  extern __shared__ uint8_t st[];   // [examples of the block][n_inner]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane % K, sub = lane / K;
+  const int ex_in_block = wave * EPW + sub;
+  const int b = blockIdx.x * (4 * EPW) + ex_in_block;
+  const bool live = b < batch;
+  uint8_t* mine = st + (size_t)ex_in_block * n_inner;
+  const float* g = node_noise + (size_t)(live ? b : 0) * n_inner * K;
+  for (int q = 0; q < n_groups; ++q) {
+    int nd[4];
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      nd[i] = order[q * 4 + i];
+      const int n = max(nd[i], 0);
+      const int p = parent_of[n];
+      const int k = p < 0 ? 0 : mine[p];
+      v[i] = logtheta[((size_t)n * K + k) * K + j] + g[(size_t)n * K + j];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int idx = j;
+      float x = v[i];
+#pragma unroll
+      for (int o = K / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(x, o, K);
+        const int oi = __shfl_xor(idx, o, K);
+        if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
+      }
+      if (j == 0 && nd[i] >= 0) mine[nd[i]] = (uint8_t)idx;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the bytes are read by the K lanes of this example
+  }
+  __syncthreads();
+  // [block examples][n_inner] -> states[b][n]
+  const int first = blockIdx.x * (4 * EPW);
+  const int count = min(4 * EPW, batch - first);
+  for (int i = threadIdx.x; i < count * n_inner; i += blockDim.x) states[(size_t)first * n_inner + i] = st[i];
+}
+
+// Categories.  A wave takes kVarsPerWave consecutive variables of one example, 64 lanes x 4
+// categories each (more categories: further rounds), requests all their rows first and then
+// reduces them one by one: per variable the wave keeps the largest value and, among equal
+// values, the lowest category.
+constexpr int kVarsPerWave = 8;
+
+__global__ __launch_bounds__(256) void hclt_sample_leaves_kernel(const float* __restrict__ leaf_kc,
+                                                                 const int32_t* __restrict__ state_node,
+                                                                 const uint8_t* __restrict__ states,
+                                                                 const float* __restrict__ leaf_noise, int V, int K,
+                                                                 int C, int n_inner, int batch,
+                                                                 uint8_t* __restrict__ out) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.x;
+  const int v0 = (blockIdx.y * 4 + wave) * kVarsPerWave;
+  if (v0 >= V) return;
+  const uint8_t* sb = states + (size_t)b * n_inner;
+  const bool vec = (C & 3) == 0;
+  float best[kVarsPerWave];
+  int bi[kVarsPerWave];
+#pragma unroll
+  for (int q = 0; q < kVarsPerWave; ++q) { best[q] = -INFINITY; bi[q] = 0x7fffffff; }
+  for (int c0 = lane * 4; c0 < C; c0 += 256) {
+    float x[kVarsPerWave][4];
+#pragma unroll
+    for (int q = 0; q < kVarsPerWave; ++q) {
+      const int v = min(v0 + q, V - 1);
+      const float* lp = leaf_kc + ((size_t)v * K + sb[state_node[v]]) * C;
+      const float* g = leaf_noise + ((size_t)b * V + v) * C;
+      if (vec) {
+        const float4 a = *reinterpret_cast<const float4*>(lp + c0), n4 = *reinterpret_cast<const float4*>(g + c0);
+        x[q][0] = a.x + n4.x; x[q][1] = a.y + n4.y; x[q][2] = a.z + n4.z; x[q][3] = a.w + n4.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[q][i] = c0 + i < C ? lp[c0 + i] + g[c0 + i] : -INFINITY;
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < kVarsPerWave; ++q)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (c0 + i < C && (x[q][i] > best[q] || bi[q] == 0x7fffffff)) { best[q] = x[q][i]; bi[q] = c0 + i; }
+  }
+#pragma unroll
+  for (int q = 0; q < kVarsPerWave; ++q) {
+    float bv = best[q];
+    int bx = bi[q];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o);
+      const int oi = __shfl_xor(bx, o);
+      if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
+    }
+    if (lane == 0 && v0 + q < V) out[(size_t)b * V + v0 + q] = (uint8_t)bx;
+  }
+}
+
+// leaf tables [V][C][K] -> [V][K][C] (a variable's categories contiguous per hidden state)
+__global__ void hclt_leaf_kc_kernel(const float* __restrict__ leaf, float* __restrict__ leaf_kc, int V, int K, int C) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)V * K * C) return;
+  const int c = (int)(i % C), jj = (int)((i / C) % K), v = (int)(i / ((int64_t)C * K));
+  leaf_kc[i] = leaf[((size_t)v * C + c) * K + jj];
+}
 
 SparseCircuit* HcltCircuit::general() {
   if (!general_) {
@@ -41,11 +174,67 @@ void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) 
   general()->kld_backward(as_hclt(q)->general(), gp, gq, n);
 }
 
+void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
+  general()->kld_backward_dev(as_hclt(q)->general(), d_gp, d_gq, n);
+}
+
 void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
-  SparseCircuit* g = general();
-  DevBuf<int32_t> slots;
-  slots.upload(noise_slot_, stream);
-  g->sample_with_slots(d_node_noise, slots.p, sample_noise_size(), d_leaf_noise, batch, d_out);
+  if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
+  if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  const bool lanes_fit = K_ >= 2 && K_ <= 64 && (K_ & (K_ - 1)) == 0;
+  const size_t st_bytes = (size_t)(4 * (64 / std::max(K_, 1))) * n_inner_;
+  if (!lanes_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
+    SparseCircuit* g = general();
+    DevBuf<int32_t> slots;
+    slots.upload(noise_slot_, stream);
+    g->sample_with_slots(d_node_noise, slots.p, sample_noise_size(), d_leaf_noise, batch, d_out);
+    return;
+  }
+  if (d_sample_tabs_.n == 0) {
+    // per inner node: its parent | per variable: the node whose state picks its leaf row | inner
+    // nodes level by level from the root in groups of four (-1: padding)
+    std::vector<int32_t> t((size_t)n_inner_ + V_);
+    for (int n = 0; n < n_inner_; ++n) {
+      const int v = var_of_inner_[n];
+      t[n] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+    }
+    for (int v = 0; v < V_; ++v) t[(size_t)n_inner_ + v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
+    std::vector<std::vector<int32_t>> by_depth;
+    for (int n = 0; n < n_inner_; ++n) {
+      const size_t dep = (size_t)depth_[var_of_inner_[n]];
+      if (by_depth.size() <= dep) by_depth.resize(dep + 1);
+      by_depth[dep].push_back(n);
+    }
+    sample_groups_ = 0;
+    for (const auto& lvl : by_depth) {
+      for (int32_t n : lvl) t.push_back(n);
+      while ((t.size() - (size_t)n_inner_ - V_) % 4) t.push_back(-1);
+    }
+    sample_groups_ = (int)((t.size() - (size_t)n_inner_ - V_) / 4);
+    d_sample_tabs_.upload(t, stream);
+  }
+  d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
+  const int64_t tot = (int64_t)V_ * K_ * C_;
+  hipLaunchKernelGGL(hclt_leaf_kc_kernel, dim3((unsigned)ceil_div(tot, 256)), dim3(256), 0, stream, d_leaf_.p, d_leaf_kc_.p,
+                     V_, K_, C_);
+  d_state_.ensure((size_t)batch * n_inner_);
+  const int epb = 4 * (64 / K_);
+  auto states = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, epb)), dim3(256), st_bytes, stream, d_logtheta_.p, d_sample_tabs_.p,
+                       d_sample_tabs_.p + n_inner_ + V_, sample_groups_, d_node_noise, n_inner_, batch, d_state_.p);
+  };
+  switch (K_) {
+    case 2: states(&hclt_sample_states_kernel<2>); break;
+    case 4: states(&hclt_sample_states_kernel<4>); break;
+    case 8: states(&hclt_sample_states_kernel<8>); break;
+    case 16: states(&hclt_sample_states_kernel<16>); break;
+    case 32: states(&hclt_sample_states_kernel<32>); break;
+    default: states(&hclt_sample_states_kernel<64>); break;
+  }
+  hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(V_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
+                     d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch, d_out);
+  check_launch_q("hclt_sample");
+  PCM_HIP(hipStreamSynchronize(stream));
 }
 
 void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {

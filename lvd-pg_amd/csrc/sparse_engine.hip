@@ -862,6 +862,28 @@ void SparseCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n
   std::copy(h2.begin(), h2.end(), gq + ns);
 }
 
+__global__ void sparse_gather_params_kernel(const int32_t* __restrict__ param2edge, int64_t n_sum,
+                                            const float* __restrict__ edge_vals, const float* __restrict__ leaf_vals,
+                                            int64_t n_leaf, float* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n_sum) out[i] = edge_vals[param2edge[i]];
+  else if (i < n_sum + n_leaf) out[i] = leaf_vals[i - n_sum];
+}
+
+void SparseCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
+  SparseCircuit* s = same_structure(this, q);
+  if (n != size(0)) fail(PCM_ERR_ARG, "gradient vectors have %lld entries, circuit has %lld parameters", (long long)n, (long long)size(0));
+  if (!d_gp || !d_gq) fail(PCM_ERR_ARG, "gradient pointer is null");
+  const int64_t ne = std::max<int64_t>(fc_.n_edges(), 1), nl = (int64_t)fc_.leaf_logp.size();
+  d_g1_.ensure(ne); d_g2_.ensure(ne); d_l1_.ensure(nl); d_l2_.ensure(nl);
+  kld_backward_device(s, d_g1_.p, d_g2_.p, d_l1_.p, d_l2_.p);
+  const int64_t ns = (int64_t)fc_.param2edge.size();
+  const unsigned blocks = (unsigned)ceil_div(ns + nl, 256);
+  hipLaunchKernelGGL(sparse_gather_params_kernel, dim3(blocks), dim3(256), 0, stream, d_param2edge_.p, ns, d_g1_.p, d_l1_.p, nl, d_gp);
+  hipLaunchKernelGGL(sparse_gather_params_kernel, dim3(blocks), dim3(256), 0, stream, d_param2edge_.p, ns, d_g2_.p, d_l2_.p, nl, d_gq);
+  check_launch("gather_params");
+}
+
 // ---- sampling ---------------------------------------------------------------------------
 
 void SparseCircuit::sample_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,

@@ -54,6 +54,7 @@ class SparseCircuit : public pcm_circuit {
   void em_update(float pseudocount, float inertia) override;
   void kld(pcm_circuit* q, float* out) override;
   void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
+  void kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) override;
   int64_t sample_noise_size() const override { return (int64_t)fc_.param2edge.size(); }
   void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) override;
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1, float b2,
@@ -89,6 +90,7 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
+  DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
   int cap_batch_ = 0, last_batch_ = 0;
   bool have_flows_ = false;
 

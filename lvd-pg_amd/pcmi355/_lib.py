@@ -41,6 +41,7 @@ _SIGS = {
     "pcm_get_aggregates": [H, vp, c_i64, vp, c_i64],
     "pcm_kld": [H, H, vp],
     "pcm_kld_backward": [H, H, vp, vp, c_i64],
+    "pcm_kld_backward_dev": [H, H, vp, vp, c_i64],
     "pcm_sample": [H, vp, vp, c_i32, vp],
     "pcm_sample_soft": [H, vp, ctypes.c_float, c_i32, vp],
     "pcm_adam_step": [H, vp, vp, vp, vp, c_f32, c_f32, c_f32, c_f32, c_i32],

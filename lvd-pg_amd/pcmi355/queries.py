@@ -172,10 +172,17 @@ def kld(bpc_p, bpc_q):
     return float(out[0])
 
 
-def kld_backward(bpc_p, bpc_q):
+def kld_backward(bpc_p, bpc_q, device=False):
     """`kld_backward(mbpc, params1, params2; grad_wrt_logparams = true)`
-    (src/queries/kld.jl:593-649) -> (grads1, grads2) in parameter-vector order."""
+    (src/queries/kld.jl:593-649) -> (grads1, grads2) in parameter-vector order: host numpy
+    vectors like the reference, or with device=True float32 tensors on the GPU (what
+    adam_step takes)."""
     n = bpc_p.num_parameters()
+    if device:
+        g1 = torch.empty(n, dtype=torch.float32, device="cuda")
+        g2 = torch.empty(n, dtype=torch.float32, device="cuda")
+        check(lib.pcm_kld_backward_dev(bpc_p.handle, bpc_q.handle, g1.data_ptr(), g2.data_ptr(), c_i64(n)))
+        return g1, g2
     g1 = np.empty(n, np.float32)
     g2 = np.empty(n, np.float32)
     check(lib.pcm_kld_backward(bpc_p.handle, bpc_q.handle, np_ptr(g1), np_ptr(g2), c_i64(n)))

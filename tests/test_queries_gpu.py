@@ -146,6 +146,8 @@ def test_hclt_kld_and_gradient_match_oracle(gpu, oracle):
     w1, w2 = _grads_in_param_order(fc1, eg1, lg1), _grads_in_param_order(fc1, eg2, lg2)
     assert np.abs(g1 - w1).max() < GRAD_RTOL * np.abs(w1).max()
     assert np.abs(g2 - w2).max() < GRAD_RTOL * np.abs(w2).max()
+    d1, d2 = P.kld_backward(a, b, device=True)       # the same vectors left on the device
+    assert np.array_equal(d1.cpu().numpy(), g1) and np.array_equal(d2.cpu().numpy(), g2)
 
 
 def _gumbel(rng, shape):
