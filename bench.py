@@ -156,16 +156,27 @@ def secondary(args):
         leaf_noise = torch.empty((B, V, C), device="cuda")
         for s0 in range(0, B, 512):
             leaf_noise[s0:s0 + 512] = -torch.log(-torch.log(torch.rand((512, V, C), device="cuda", generator=gen).clamp_(1e-10, 1 - 1e-7)))
-        P.kld(p, q)                                                   # builds both general forms
+        P.kld(p, q)                                                   # builds the tables
         t_kld = _timed(torch, lambda: P.kld(p, q), args.steps, 1)
         t_grad = _timed(torch, lambda: P.kld_backward(p, q, device=True), args.steps, 1)
         t_samp = _timed(torch, lambda: P.sample(p, node_noise, leaf_noise), max(1, args.steps // 4), 1)
+        n_sum = p.num_inner_params()
+        g1, _ = P.kld_backward(p, q, device=True)
+        dp = torch.from_numpy(P.vectorize_parameters(p)[:n_sum].copy()).cuda()
+        dm, dv = torch.zeros_like(dp), torch.zeros_like(dp)
+        tt = [0]
+
+        def adam():
+            tt[0] += 1
+            P.adam_step(p, g1, dp, dm, dv, lr=1e-4, t=tt[0])
+        t_adam = _timed(torch, adam, args.steps, 1)
         dt = t_samp
         algo = 4 * B * (n_inner * K + V * C)                           # the noise tensors, read once
         out.update(metric="samples/sec Gumbel-max from supplied noise, 3072-var HCLT K=32",
                    value=B / t_samp, unit="samples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
-                   queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "sample": t_samp * 1e3})
+                   queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
+                               "sample": t_samp * 1e3})
     else:
         print(f"unknown workload {args.workload}", file=sys.stderr)
         sys.exit(2)

@@ -11,14 +11,6 @@
 
 namespace pcm {
 
-#define PCM_DISPATCH_K(K_, ...)                         \
-  switch (K_) {                                         \
-    case 16: { constexpr int KK = 16; __VA_ARGS__; break; } \
-    case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
-    case 64: { constexpr int KK = 64; __VA_ARGS__; break; } \
-    default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
-  }
-
 // the lean walk kernels exist for the hidden sizes whose blocks fit the register file
 #define PCM_DISPATCH_LEAN_K(K_, ...)                    \
   switch (K_) {                                         \

@@ -98,6 +98,14 @@ struct HcltDev {
   uint32_t tile_stride;   // bytes per node in O / R / G (nslices*16*K*4)
 };
 
+#define PCM_DISPATCH_K(K_, ...)                         \
+  switch (K_) {                                         \
+    case 16: { constexpr int KK = 16; __VA_ARGS__; break; } \
+    case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
+    case 64: { constexpr int KK = 64; __VA_ARGS__; break; } \
+    default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
+  }
+
 class HcltCircuit : public pcm_circuit {
  public:
   HcltCircuit(const int32_t* parent, int V, int K, int C);
@@ -173,6 +181,15 @@ class HcltCircuit : public pcm_circuit {
   std::unique_ptr<SparseCircuit> general_; // built on first use by the KL / sampling / Adam queries
   bool general_stale_ = true;
   SparseCircuit* general();
+  // KL recursion on the block form
+  DevBuf<int32_t> d_kl_up_, d_kl_down_;   // chain steps (KlItem records) bottom-up / top-down
+  DevBuf<int32_t> d_kl_tabs_;             // parent of every inner node | h-giving node of every variable | input-node positions
+  DevBuf<int32_t> d_kl_pos_;              // chain slot of every inner node: upward | downward
+  DevBuf<float> d_kl_leaf_, d_kl_vec_, d_kl_par_;
+  int kl_up_steps_ = 0, kl_down_steps_ = 0;
+  HcltCircuit* same_tree(pcm_circuit* q);
+  void build_kld_tables();
+  void kld_device(HcltCircuit* q, bool with_down);
   void pull_from_general();
   void build_structure();
   void build_schedules();

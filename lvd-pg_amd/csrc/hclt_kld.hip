@@ -1,0 +1,448 @@
+// KL divergence between two HCLTs of one structure, its gradient, and the Adam step, on the
+// block form.
+//
+// With P_v = exp(theta1_v) (K x K, row k = state of the tree parent), D_v = theta1_v - theta2_v,
+// l_v[j] = KL of the leaf distributions of v's own variable and of its leaf tree children at
+// hidden state j, the recursion of the reference (src/queries/kld.jl:95-128: a sum edge gives
+// p1 * (kld(children) + logp1 - logp2), a product adds its children) reads
+//   Z_v[j]  = l_v[j] + sum over non-leaf tree children c of KL_c[j]
+//   KL_v[k] = sum_j P_v[k,j] * (Z_v[j] + D_v[k,j])
+// and its reverse pass (src/queries/kld.jl:262-300, root gradient 1)
+//   h_v[j]  = sum_k g_v[k] * P_v[k,j],   g_c = h_v for every tree child c, g_root = e_0
+//   d/dtheta1_v[k,j] = g_v[k] * (P_v[k,j] * (Z_v[j] + D_v[k,j]) + P_v[k,j]),  d/dtheta2 = -g_v[k] * P_v[k,j]
+// with the leaf lines written as the reference has them (src/queries/kld.jl:528-535,
+// src/nodes/fixable_categorical_dist.jl:219): g * (a - b + 1) and g * exp(a - b).
+//
+// Only the two K-vector chains (KL_v up the tree, h_v down the tree) are sequential; one
+// workgroup walks each of them level by level, sixteen tree nodes (one per wave) between
+// barriers.  Everything else is a data-parallel kernel.
+#include "hclt_engine.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+namespace pcm {
+
+static void check_launch_k(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+// kl_leaf[v][j] = sum_c exp(a) * (a - b), a = leaf1[v][c][j], b = leaf2[v][c][j]
+// (src/nodes/fixable_categorical_dist.jl:187-192 in log-parameter form).
+__global__ __launch_bounds__(256) void hclt_kld_leaf_kernel(const float* __restrict__ leaf1,
+                                                            const float* __restrict__ leaf2, int K, int C,
+                                                            float* __restrict__ kl_leaf) {
+  __shared__ float part[256];
+  const int v = blockIdx.x, t = threadIdx.x;
+  const int j = t % K, cc = t / K, P = 256 / K;
+  float acc = 0.f;
+  if (cc < P) {
+    const float* a = leaf1 + (size_t)v * C * K + j;
+    const float* b = leaf2 + (size_t)v * C * K + j;
+    for (int c = cc; c < C; c += P) {
+      const float x = a[(size_t)c * K], y = b[(size_t)c * K];
+      acc += expf(x) * (x - y);
+    }
+  }
+  part[t] = acc;
+  __syncthreads();
+  if (t < K) {
+    float s = 0.f;
+    for (int q = 0; q < P; ++q) s += part[q * K + t];
+    kl_leaf[(size_t)v * K + t] = s;
+  }
+}
+
+// Per tree node, everything of the recursion that does not wait for other nodes, stored where
+// the chains will look for it: slot su = pos[n] of the upward chain's steps, slot sd =
+// pos[n_inner + n] of the downward chain's.
+//   ell[su][j]  = l_v[j]
+//   base[su][k] = sum_j P[k,j] * (D[k,j] + ell[j])
+//   pu[su][j][k] = P[k,j]   (operand layout of the upward chain: lane = k)
+//   pd[sd][k][j] = P[k,j]   (of the downward chain: lane = j)
+template <int K>
+__global__ __launch_bounds__(256) void hclt_kld_base_kernel(const HcltNode* __restrict__ nodes,
+                                                            const int32_t* __restrict__ child_leaf,
+                                                            const int32_t* __restrict__ pos, int n_inner,
+                                                            const float* __restrict__ theta1,
+                                                            const float* __restrict__ theta2,
+                                                            const float* __restrict__ kl_leaf, float* __restrict__ ell,
+                                                            float* __restrict__ base, float* __restrict__ pu,
+                                                            float* __restrict__ pd) {
+  __shared__ float tile[K][K + 1];
+  __shared__ float l[K];
+  const int n = blockIdx.x, t = threadIdx.x;
+  const HcltNode nd = nodes[n];
+  const size_t su = (size_t)pos[n], sd = (size_t)pos[n_inner + n];
+  if (t < K) {
+    float s = kl_leaf[(size_t)nd.var * K + t];
+    for (int q = 0; q < nd.lc_cnt; ++q) s += kl_leaf[(size_t)child_leaf[nd.lc_off + q] * K + t];
+    l[t] = s;
+    ell[su * K + t] = s;
+  }
+  __syncthreads();
+  const int j = t % K;
+  for (int k = t / K; k < K; k += 256 / K) {
+    const float x = theta1[((size_t)n * K + k) * K + j], y = theta2[((size_t)n * K + k) * K + j];
+    const float p = expf(x);
+    tile[k][j] = p;
+    pd[(sd * K + k) * K + j] = p;
+    float term = p > 0.f ? p * (x - y + l[j]) : 0.f;   // absent edges (the root's rows past the first) carry -inf
+#pragma unroll
+    for (int o = K / 2; o > 0; o >>= 1) term += __shfl_xor(term, o, K);
+    if (j == 0) base[su * K + k] = term;
+  }
+  __syncthreads();
+  for (int i = t; i < K * K; i += 256) pu[su * K * K + i] = tile[i % K][i / K];
+}
+
+// One tree node of a chain step.
+struct KlItem {
+  int32_t n;            // inner id, -1: this wave idles
+  int32_t c[3];         // up: first non-leaf tree children (-1 none); down: c[0] = parent (-1 root)
+  int32_t ext_off, ext_cnt;   // up: further children at child_inner[ext_off .. +ext_cnt)
+  int32_t pad[2];
+};
+static_assert(sizeof(KlItem) == 32, "KlItem is read as two 16-byte words");
+
+// Waves (= nodes per step) of a chain workgroup: as many as leave each lane the registers for two
+// steps' worth of its node's parameters.
+constexpr int kl_waves(int K) { return K > 32 ? 8 : 16; }
+
+// The two chains.  Workgroup 0 walks up (KL_v, Z_v), workgroup 1 walks down (h_v); launched
+// with one workgroup when only the divergence is wanted.  A step is kl_waves(K) independent
+// nodes (same level); the vectors a step reads were stored by earlier steps of the same
+// workgroup, so a barrier orders them.  A step first requests the vectors it waits for, then
+// the next step's item and parameters (found by step and wave alone), so that those are under
+// way while the step computes.
+template <int K>
+__global__ __launch_bounds__(kl_waves(K) * 64) void hclt_kld_chain_kernel(
+    const KlItem* __restrict__ up_items, int up_steps, const KlItem* __restrict__ down_items, int down_steps,
+    const int32_t* __restrict__ child_inner, const float* __restrict__ pu, const float* __restrict__ base,
+    const float* __restrict__ ell, const float* __restrict__ pd, float* klv, float* z, float* h) {
+  constexpr int PARTS = 64 / K, JP = K / PARTS, W = kl_waves(K);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane % K, part = lane / K;
+  const bool up = blockIdx.x == 0;
+  const int steps = up ? up_steps : down_steps;
+  const KlItem* __restrict__ items = up ? up_items : down_items;
+  const float* __restrict__ par = up ? pu : pd;   // [slot][K][K], this lane reads rows part*JP.. at column r
+  KlItem it = items[wave];
+  float p[JP];
+#pragma unroll
+  for (int i = 0; i < JP; ++i) p[i] = par[((size_t)wave * K + part * JP + i) * K + r];
+  for (int q = 0; q < steps; ++q) {
+    const size_t slot = (size_t)q * W + wave;
+    float s = 0.f, bs = 0.f, el = 0.f;
+    if (it.n >= 0) {
+      if (up) {
+#pragma unroll
+        for (int i = 0; i < 3; ++i)
+          if (it.c[i] >= 0) s += klv[(size_t)it.c[i] * K + r];
+        for (int i = 0; i < it.ext_cnt; ++i) s += klv[(size_t)child_inner[it.ext_off + i] * K + r];
+        bs = base[slot * K + r];
+        el = ell[slot * K + r];
+      } else {
+        s = it.c[0] >= 0 ? h[(size_t)it.c[0] * K + r] : (r == 0 ? 1.f : 0.f);
+      }
+    }
+    const bool more = q + 1 < steps;
+    KlItem nx = it;
+    float pn[JP];
+    if (more) nx = items[slot + W];
+#pragma unroll
+    for (int i = 0; i < JP; ++i) pn[i] = more ? par[((slot + W) * K + part * JP + i) * K + r] : 0.f;
+    if (it.n >= 0) {
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < JP; ++i) acc += p[i] * __shfl(s, part * JP + i);
+#pragma unroll
+      for (int o = K; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
+      if (part == 0) {
+        if (up) {
+          klv[(size_t)it.n * K + r] = bs + acc;
+          z[(size_t)it.n * K + r] = el + s;
+        } else {
+          h[(size_t)it.n * K + r] = acc;
+        }
+      }
+    }
+    it = nx;
+#pragma unroll
+    for (int i = 0; i < JP; ++i) p[i] = pn[i];
+    __syncthreads();
+  }
+}
+
+// Gradients of the sum parameters, in parameter-vector order (src/queries/kld.jl:271-272).
+__global__ void hclt_kld_edge_grad_kernel(int64_t ns, int K, const int64_t* __restrict__ src,
+                                          const int32_t* __restrict__ parent_of, const float* __restrict__ theta1,
+                                          const float* __restrict__ theta2, const float* __restrict__ z,
+                                          const float* __restrict__ h, float* __restrict__ gp,
+                                          float* __restrict__ gq) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= ns) return;
+  const int64_t s = src[i];
+  const int j = (int)(s % K), k = (int)((s / K) % K);
+  const int n = (int)(s / ((int64_t)K * K));
+  const int par = parent_of[n];
+  const float g = par < 0 ? 1.f : h[(size_t)par * K + k];
+  const float a = theta1[s], b = theta2[s], p1 = expf(a);
+  const float ek = p1 * (z[(size_t)n * K + j] + a - b);
+  gp[i] = g * (ek + p1);
+  gq[i] = -g * p1;
+}
+
+// Gradients of the leaf parameters: [V][C][K] tables in, parameter-vector order out (the C
+// categories of input node (v, j) contiguous at in_pos[v][j] * C), 64 categories of one
+// variable per workgroup, turned around in LDS.
+constexpr int kLeafGradCats = 64;
+
+__global__ __launch_bounds__(256) void hclt_kld_leaf_grad_kernel(const float* __restrict__ leaf1,
+                                                                 const float* __restrict__ leaf2,
+                                                                 const int32_t* __restrict__ state_node,
+                                                                 const int32_t* __restrict__ in_pos,
+                                                                 const float* __restrict__ h, int K, int C,
+                                                                 float* __restrict__ gp, float* __restrict__ gq) {
+  extern __shared__ float lg[];   // two tiles [kLeafGradCats][K + 1]
+  const int v = blockIdx.x, c0 = blockIdx.y * kLeafGradCats, t = threadIdx.x;
+  const int nc = min(kLeafGradCats, C - c0);
+  float* t1 = lg;
+  float* t2 = lg + kLeafGradCats * (K + 1);
+  {
+    const int j = t % K;
+    const float g = h[(size_t)state_node[v] * K + j];
+    for (int cc = t / K; cc < nc; cc += 256 / K) {
+      const size_t at = ((size_t)v * C + c0 + cc) * K + j;
+      const float a = leaf1[at], b = leaf2[at];
+      t1[cc * (K + 1) + j] = g * (a - b + 1.f);
+      t2[cc * (K + 1) + j] = g * expf(a - b);
+    }
+  }
+  __syncthreads();
+  const int cc = t % kLeafGradCats;
+  if (cc < nc)
+    for (int j = t / kLeafGradCats; j < K; j += 256 / kLeafGradCats) {
+      const size_t at = (size_t)in_pos[(size_t)v * K + j] * C + c0 + cc;
+      gp[at] = t1[cc * (K + 1) + j];
+      gq[at] = t2[cc * (K + 1) + j];
+    }
+}
+
+// Adam on the sum parameters (src/sgd/adam.jl:318-319 moments, :63-76 ascent step) and the
+// per-sum-node normalisation into the circuit (:88-127), in one pass: every normalisation
+// group of an HCLT is K consecutive entries of the parameter vector.
+template <int K>
+__global__ __launch_bounds__(256) void hclt_adam_kernel(int64_t ns, const float* __restrict__ grad,
+                                                        float* __restrict__ params, float* __restrict__ m,
+                                                        float* __restrict__ v, float lr, float b1, float b2, float eps,
+                                                        float c1, float c2, const int64_t* __restrict__ src,
+                                                        float* __restrict__ logtheta) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const bool live = i < ns;
+  float p = -INFINITY;
+  if (live) {
+    const float g = grad[i];
+    const float mi = b1 * m[i] + (1.f - b1) * g;
+    const float vi = b2 * v[i] + (1.f - b2) * g * g;
+    m[i] = mi;
+    v[i] = vi;
+    p = params[i] + lr * ((mi / c1) / (sqrtf(vi / c2) + eps));
+    params[i] = p;
+  }
+  float s = expf(p);
+#pragma unroll
+  for (int o = K / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, K);
+  if (live) logtheta[src[i]] = p - logf(s);
+}
+
+// ---- host --------------------------------------------------------------------------------
+
+HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
+  auto* o = dynamic_cast<HcltCircuit*>(q);
+  if (!o) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
+  if (o->K_ != K_ || o->C_ != C_ || o->parent_ != parent_)
+    fail(PCM_ERR_SHAPE, "the two circuits of a KL query must share one structure");
+  return o;
+}
+
+void HcltCircuit::build_kld_tables() {
+  if (d_kl_up_.n) return;
+  const int W = kl_waves(K_);
+  // offsets of the nodes' non-leaf children in the device's child_inner list
+  std::vector<int32_t> ic_off(n_inner_ + 1, 0);
+  for (int n = 0; n < n_inner_; ++n) {
+    int cnt = 0;
+    for (int c : children_[var_of_inner_[n]]) cnt += !children_[c].empty();
+    ic_off[n + 1] = ic_off[n] + cnt;
+  }
+  std::vector<int32_t> pos((size_t)2 * n_inner_, 0);
+  auto chain = [&](bool up) {
+    // nodes level by level (up: by height from the bottom, down: by depth from the root), each
+    // level padded to whole steps
+    std::vector<std::vector<int32_t>> lv;
+    for (int n = 0; n < n_inner_; ++n) {
+      const int v = var_of_inner_[n];
+      const size_t at = (size_t)(up ? height_[v] : depth_[v]);
+      if (lv.size() <= at) lv.resize(at + 1);
+      lv[at].push_back(n);
+    }
+    std::vector<KlItem> items;
+    for (const auto& level : lv) {
+      for (int32_t n : level) {
+        KlItem it;
+        std::memset(&it, 0, sizeof it);
+        it.n = n;
+        it.c[0] = it.c[1] = it.c[2] = -1;
+        const int v = var_of_inner_[n];
+        if (up) {
+          int seen = 0;
+          for (int c : children_[v]) {
+            if (children_[c].empty()) continue;
+            if (seen < 3) it.c[seen] = inner_of_var_[c];
+            ++seen;
+          }
+          if (seen > 3) { it.ext_off = ic_off[n] + 3; it.ext_cnt = seen - 3; }
+        } else {
+          it.c[0] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+        }
+        pos[(up ? 0 : n_inner_) + n] = (int32_t)items.size();
+        items.push_back(it);
+      }
+      while (items.size() % W) {
+        KlItem idle;
+        std::memset(&idle, 0, sizeof idle);
+        idle.n = -1;
+        idle.c[0] = idle.c[1] = idle.c[2] = -1;
+        items.push_back(idle);
+      }
+    }
+    return items;
+  };
+  std::vector<KlItem> up = chain(true), down = chain(false);
+  kl_up_steps_ = (int)(up.size() / W);
+  kl_down_steps_ = (int)(down.size() / W);
+  std::vector<int32_t> raw(up.size() * 8), rawd(down.size() * 8);
+  std::memcpy(raw.data(), up.data(), up.size() * sizeof(KlItem));
+  std::memcpy(rawd.data(), down.data(), down.size() * sizeof(KlItem));
+  d_kl_down_.upload(rawd, stream);
+  d_kl_pos_.upload(pos, stream);
+  // per inner node: its parent | per variable: the inner node whose h reaches its leaf |
+  // per input node (v, j): its position among the input nodes of the parameter vector
+  std::vector<int32_t> t((size_t)n_inner_ + V_ + (size_t)V_ * K_, 0);
+  for (int n = 0; n < n_inner_; ++n) {
+    const int v = var_of_inner_[n];
+    t[n] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+  }
+  for (int v = 0; v < V_; ++v)
+    t[(size_t)n_inner_ + v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
+  for (size_t q = 0; q < input_order_.size(); ++q) t[(size_t)n_inner_ + V_ + input_order_[q]] = (int32_t)q;
+  d_kl_tabs_.upload(t, stream);
+  d_kl_up_.upload(raw, stream);   // last: marks the tables as built
+}
+
+// Runs the recursion of this circuit (p) against q; with_down also leaves h.
+void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
+  build_kld_tables();
+  const int W = kl_waves(K_);
+  const size_t nk = (size_t)n_inner_ * K_;
+  const size_t su = (size_t)kl_up_steps_ * W, sd = (size_t)kl_down_steps_ * W;   // chain slots, idle ones included
+  d_kl_leaf_.ensure((size_t)V_ * K_);
+  if (!d_kl_vec_.n) {
+    d_kl_vec_.alloc(3 * nk + 2 * su * K_);   // klv | z | h | ell | base
+    d_kl_par_.alloc((su + sd) * K_ * K_);    // pu | pd; idle slots are read (and ignored) by idle waves
+    d_kl_vec_.zero(stream);
+    d_kl_par_.zero(stream);
+  }
+  float* klv = d_kl_vec_.p;
+  float* z = klv + nk;
+  float* h = z + nk;
+  float* ell = h + nk;
+  float* base = ell + su * K_;
+  float* pu = d_kl_par_.p;
+  float* pd = pu + su * K_ * K_;
+  hipLaunchKernelGGL(hclt_kld_leaf_kernel, dim3(V_), dim3(256), 0, stream, d_leaf_.p, q->d_leaf_.p, K_, C_, d_kl_leaf_.p);
+  PCM_DISPATCH_K(K_, {
+    hipLaunchKernelGGL(hclt_kld_base_kernel<KK>, dim3(n_inner_), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
+                       d_kl_pos_.p, n_inner_, d_logtheta_.p, q->d_logtheta_.p, d_kl_leaf_.p, ell, base, pu, pd);
+    hipLaunchKernelGGL(hclt_kld_chain_kernel<KK>, dim3(with_down ? 2 : 1), dim3(kl_waves(KK) * 64), 0, stream,
+                       reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                       reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_child_inner_.p, pu, base, ell, pd,
+                       klv, z, h);
+  });
+  check_launch_k("hclt_kld");
+}
+
+void HcltCircuit::kld(pcm_circuit* q, float* out) {
+  HcltCircuit* o = same_tree(q);
+  if (!block_) {
+    general()->kld(o->general(), out);
+    return;
+  }
+  kld_device(o, false);
+  const float* klv = d_kl_vec_.p;
+  PCM_HIP(hipMemcpyAsync(out, klv + (size_t)inner_of_var_[root_] * K_, sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
+  HcltCircuit* o = same_tree(q);
+  if (!block_) {
+    general()->kld_backward_dev(o->general(), d_gp, d_gq, n);
+    return;
+  }
+  if (n != size(0)) fail(PCM_ERR_ARG, "gradient vectors have %lld entries, circuit has %lld parameters", (long long)n, (long long)size(0));
+  if (!d_gp || !d_gq) fail(PCM_ERR_ARG, "gradient pointer is null");
+  kld_device(o, true);
+  const size_t nk = (size_t)n_inner_ * K_;
+  const float* z = d_kl_vec_.p + nk;
+  const float* h = d_kl_vec_.p + 2 * nk;
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  hipLaunchKernelGGL(hclt_kld_edge_grad_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns, K_,
+                     d_sum_param_src_.p, d_kl_tabs_.p, d_logtheta_.p, o->d_logtheta_.p, z, h, d_gp, d_gq);
+  hipLaunchKernelGGL(hclt_kld_leaf_grad_kernel, dim3(V_, ceil_div(C_, kLeafGradCats)), dim3(256),
+                     2 * kLeafGradCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, o->d_leaf_.p, d_kl_tabs_.p + n_inner_,
+                     d_kl_tabs_.p + n_inner_ + V_, h, K_, C_, d_gp + ns, d_gq + ns);
+  check_launch_k("hclt_kld_backward");
+}
+
+void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) {
+  HcltCircuit* o = same_tree(q);
+  if (!block_) {
+    general()->kld_backward(o->general(), gp, gq, n);
+    return;
+  }
+  if (!gp || !gq) fail(PCM_ERR_ARG, "gradient pointer is null");
+  DevBuf<float> d1, d2;
+  d1.alloc((size_t)std::max<int64_t>(n, 1));
+  d2.alloc((size_t)std::max<int64_t>(n, 1));
+  kld_backward_dev(q, d1.p, d2.p, n);
+  PCM_HIP(hipMemcpyAsync(gp, d1.p, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipMemcpyAsync(gq, d2.p, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
+                            float b2, float eps, int t) {
+  if (!block_) {
+    general()->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t);
+    PCM_HIP(hipStreamSynchronize(stream));
+    pull_from_general();
+    return;
+  }
+  if (!d_grad || !d_params || !d_m || !d_v) fail(PCM_ERR_ARG, "null optimiser array");
+  if (t < 1) fail(PCM_ERR_ARG, "step count must start at 1, got %d", t);
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
+  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_adam_kernel<KK>, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
+                                        d_grad, d_params, d_m, d_v, lr, b1, b2, eps, c1, c2, d_sum_param_src_.p,
+                                        d_logtheta_.p));
+  check_launch_k("hclt_adam");
+  rebuild_w();
+  general_stale_ = true;
+  PCM_HIP(hipStreamSynchronize(stream));
+}
+
+}  // namespace pcm

@@ -1,7 +1,6 @@
-// KL recursion, sampling and Adam for HCLT circuits.  Gumbel-max sampling has its own kernels
-// on the block form (below); the KL recursion, the relaxed sampler and Adam run on the layered
-// engine over the circuit's general form, with parameters exchanged in parameter-vector order,
-// which both forms share.
+// Sampling from HCLT circuits.  Gumbel-max sampling has its own kernels on the block form
+// (below); the relaxed sampler runs on the layered engine over the circuit's general form, with
+// parameters exchanged in parameter-vector order, which both forms share.
 #include "hclt_engine.hpp"
 
 #include <hip/hip_runtime.h>
@@ -162,22 +161,6 @@ void HcltCircuit::pull_from_general() {
   general_stale_ = false;
 }
 
-static HcltCircuit* as_hclt(pcm_circuit* q) {
-  auto* h = dynamic_cast<HcltCircuit*>(q);
-  if (!h) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
-  return h;
-}
-
-void HcltCircuit::kld(pcm_circuit* q, float* out) { general()->kld(as_hclt(q)->general(), out); }
-
-void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) {
-  general()->kld_backward(as_hclt(q)->general(), gp, gq, n);
-}
-
-void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
-  general()->kld_backward_dev(as_hclt(q)->general(), d_gp, d_gq, n);
-}
-
 void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
   if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
@@ -242,13 +225,6 @@ void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int3
   DevBuf<int32_t> slots;
   slots.upload(noise_slot_, stream);
   g->sample_soft_with_slots(d_node_noise, slots.p, sample_noise_size(), temperature, batch, d_out);
-}
-
-void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
-                            float b2, float eps, int t) {
-  general()->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t);
-  PCM_HIP(hipStreamSynchronize(stream));
-  pull_from_general();
 }
 
 }  // namespace pcm
