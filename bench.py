@@ -88,9 +88,10 @@ def _timed(torch, fn, steps, warmup):
 
 
 def secondary(args):
-    """The other configurations, all on the layered engine (not the headline; same JSON shape).
-    Their byte counts are the layered engine's own minimum: per example 4 bytes written per node
-    and 8 read per edge going up; going down 4 written per node and 16 read per incoming edge."""
+    """The other configurations (not the headline; same JSON shape).  c2: wide block kernels,
+    priced against the fp32 matrix peak.  c4: layered engine, whose byte count is its own minimum:
+    per example 4 bytes written per node and 8 read per edge going up; going down 4 written per
+    node and 16 read per incoming edge.  c5: block-form queries."""
     import numpy as np
     import torch
     import pcmi355 as P
@@ -110,11 +111,17 @@ def secondary(args):
         ll = torch.empty(B, device="cuda")
         dt = _timed(torch, lambda: check(lib.pcm_em_step(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B,
                                                           0.0, 0.1, 0.9, ll.data_ptr())), args.steps, args.warmup)
-        nn, ne = bpc.num_nodes(), bpc.num_edges()
-        algo = B * (8 * nn + 24 * ne)
-        out.update(metric="examples/sec fwd+bwd+EM, 48-var HCLT K=128 (layered engine)", value=B / dt, unit="examples/s",
+        n_int = bpc.size("inner_tree_nodes")
+        flops = 6.0 * K * K * B * n_int                      # three K x K contractions per (tree node, example)
+        out.update(metric="examples/sec fwd+bwd+EM, 48-var HCLT K=128 (wide block kernels)", value=B / dt, unit="examples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
-                           "nodes": nn, "edges": ne})
+                           "tree_inner_nodes": n_int})
+        out["ms_per_step"] = dt * 1e3
+        ach = flops / dt / 1e12
+        out["roofline"] = {"bound": "mfma", "kernel": "whole step", "achieved": ach, "peak": 157.3, "unit": "TFLOP/s",
+                           "frac": ach / 157.3, "traffic": None}
+        print(json.dumps(out))
+        return
     elif args.workload == "c4_patch_multihead":
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         sys.path.insert(0, os.path.join(ROOT, "oracle"))

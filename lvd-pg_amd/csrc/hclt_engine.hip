@@ -31,6 +31,7 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C) : V_(V), K_
   // hidden sizes without block kernels run every query on the layered engine over the
   // circuit's general form; the block-form parameter interface stays the same
   block_ = K == 16 || K == 32 || K == 64;
+  wide_ = K == 128;
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
   build_structure();
@@ -636,9 +637,9 @@ void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
 // ---- parameters -------------------------------------------------------------------
 
 void HcltCircuit::rebuild_w() {
-  if (!block_) return;
+  if (!block_ && !wide_) return;
   const int64_t tot = (int64_t)n_inner_ * K_ * K_;
-  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_rebuild_w_kernel<KK>, dim3(ceil_div(tot, 256)), dim3(256), 0,
+  PCM_DISPATCH_PARAM_K(K_, hipLaunchKernelGGL(hclt_rebuild_w_kernel<KK>, dim3(ceil_div(tot, 256)), dim3(256), 0,
                                         stream, d_logtheta_.p, d_Wf_.p, d_Wb_.p, n_inner_));
   check_launch("rebuild_w");
 }
@@ -697,7 +698,7 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   const int K = K_, C = C_;
   std::vector<float> h;
-  if (!block_) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
+  if (!block_ && !wide_) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
     std::vector<float> ea((size_t)n_edges_), lf((size_t)V_ * K * C);
     general_->get_aggregates(ea.data(), n_edges_, lf.data(), (int64_t)lf.size());
     if (edge_aggr) {
@@ -769,6 +770,15 @@ void HcltCircuit::ensure_batch(int batch) {
   const int ns = ceil_div(batch, kSlice);
   if (ns <= cap_slices_) return;
   const size_t tile = (size_t)ns * kSlice * K_;
+  if (wide_) {
+    d_O_.alloc((size_t)n_inner_ * tile);
+    d_G_.alloc((size_t)n_inner_ * tile);
+    d_wide_rs_.alloc((size_t)n_inner_ * tile);
+    d_wide_es_.alloc((size_t)n_inner_ * tile);
+    d_xb_.alloc((size_t)V_ * ns * kSlice);
+    cap_slices_ = ns;
+    return;
+  }
   d_O_.alloc((size_t)(n_inner_ + 1) * tile);   // row n_inner: trash tile of idle waves
   d_R_.alloc((size_t)(n_inner_ + 1) * tile);
   if (bwd_spill_) d_G_.alloc((size_t)n_inner_ * tile);
@@ -812,6 +822,7 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
                      b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
   check_launch("stage_batch");
+  if (wide_) return;
   hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
   check_launch("pack_x");
@@ -911,21 +922,29 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
 
 void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (!block_) return general()->loglikelihoods(b, d_ll);
+  if (!block_ && !wide_) return general()->loglikelihoods(b, d_ll);
   stage_batch(b);
+  if (wide_) return wide_forward(dev(b.batch), d_ll);
   run_forward(dev(b.batch), d_ll);
 }
 
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (!block_) {
+  if (!block_ && !wide_) {
     general()->flows(b, rate, nullptr, d_ll);
     have_flows_ = true;
     return;
   }
   stage_batch(b);
   HcltDev d = dev(b.batch);
+  if (wide_) {
+    wide_forward(d, d_ll);
+    wide_backward_stats(d, rate);
+    have_flows_ = true;
+    if (timing) ++n_timed_;
+    return;
+  }
   run_forward(d, d_ll);
   run_backward(d);
   run_stats(d, rate);
@@ -961,13 +980,13 @@ void HcltCircuit::read_timing(float* ms, int n) {
 
 void HcltCircuit::em_update(float pseudocount, float inertia) {
   if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
-  if (!block_) {
+  if (!block_ && !wide_) {
     general_->em_update(pseudocount, inertia);
     PCM_HIP(hipStreamSynchronize(stream));
     pull_from_general();
     return;
   }
-  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)),
+  PCM_DISPATCH_PARAM_K(K_, hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)),
                                         dim3(128), 0, stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p,
                                         d_edge_aggr_.p, n_inner_, pseudocount, inertia));
   check_launch("theta_update");

@@ -106,6 +106,16 @@ struct HcltDev {
     default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
   }
 
+// the parameter kernels also serve the wide block sizes
+#define PCM_DISPATCH_PARAM_K(K_, ...)                   \
+  switch (K_) {                                         \
+    case 16: { constexpr int KK = 16; __VA_ARGS__; break; } \
+    case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
+    case 64: { constexpr int KK = 64; __VA_ARGS__; break; } \
+    case 128: { constexpr int KK = 128; __VA_ARGS__; break; } \
+    default: fail(PCM_ERR_UNSUPPORTED, "hidden size %d not supported by the block engine", K_); \
+  }
+
 class HcltCircuit : public pcm_circuit {
  public:
   HcltCircuit(const int32_t* parent, int V, int K, int C);
@@ -141,7 +151,8 @@ class HcltCircuit : public pcm_circuit {
 
  private:
   int V_, K_, C_, n_inner_, root_;
-  bool block_ = true;   // the hidden size has block kernels; else everything runs on the layered engine
+  bool block_ = true;   // the hidden size has walk kernels (block tiles in registers)
+  bool wide_ = false;   // the hidden size has the wide block kernels (likelihoods, flows, EM); neither: layered engine
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;
   std::vector<std::vector<int32_t>> children_;
   int n_fwd_steps_ = 0, n_bwd_steps_ = 0, lds_slots_ = 0, max_lds_ = 0;
@@ -201,6 +212,11 @@ class HcltCircuit : public pcm_circuit {
   void run_forward(const HcltDev& d, float* d_ll);
   void run_backward(const HcltDev& d);
   void run_stats(const HcltDev& d, float rate);
+  // wide block kernels
+  DevBuf<float> d_wide_rs_, d_wide_es_;   // R and E of every node in the operand layout of the statistics contraction
+  DevBuf<int32_t> d_wide_state_node_;     // per variable: the inner node whose flow tile feeds its leaf histogram
+  void wide_forward(const HcltDev& d, float* d_ll);
+  void wide_backward_stats(const HcltDev& d, float rate);
 };
 
 }  // namespace pcm

@@ -1,0 +1,347 @@
+// Block kernels for wide hidden sizes (K = 128): a K x K parameter block no longer fits a
+// wave's registers, so a 16-example tile is shared by the four waves of a workgroup, each
+// producing a quarter of the output states and streaming its quarter of the block (64 KB per
+// node at K = 128, shared by all workgroups through L2) as MFMA A-operands.  Trees with wide
+// blocks are small (tens of nodes), so a workgroup simply walks the nodes in post-order
+// (forward) or reverse post-order (backward) with a barrier between nodes; tiles travel
+// through memory.
+//
+// Tile layout (same as the walk kernels'): lane = 16*g + b owns example b and states
+// kt*16 + 4*g + i (kt < K/16, i < 4); a tile is K/16 runs of 64 float4.  This is both the
+// B-operand and the accumulator layout of v_mfma_f32_16x16x4_f32 with the parameter block
+// (Wf / Wb, pre-swizzled) as A-operand.
+//
+// Algebra per tree node (reference: src/queries/likelihood.jl:4-68, src/queries/flow.jl:8-106,
+// :165-195 on the K^2 sum edges of src/structures/hclts.jl:133):
+//   Z = leaf rows + children's values, m = max_j Z, E = exp(Z - m)
+//   O[k] = m + log(sum_j W[k,j] E[j])                              forward
+//   R[k] = F[k] / exp(O[k] - m),  G[j] = E[j] * sum_k W[k,j] R[k]   backward (F = parent's G, root: e_0)
+//   edge_aggr[k,j] += W[k,j] * sum_b R[b,k] E[b,j];  leaf_flow[u][x_b,u][j] += G[b,j]
+#include "hclt_engine.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+
+namespace pcm {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kWideWaves = 4;
+
+static void check_launch_w(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+template <int K>
+struct WideLds {
+  v4f e[K / 16][64];   // E tile of the node
+  v4f r[K / 16][64];   // R tile (backward)
+  float mx[kWideWaves][16];
+};
+
+// Builds the node's E tile: every wave sums its quarter of Z, the row maxima are combined
+// through LDS, E goes to LDS and comes back whole to every wave.  Returns m of the lane's
+// example.  Two workgroup barriers.
+template <int K>
+__device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& nd, int s, int lane, int wave,
+                                              WideLds<K>& L, v4f (&e)[K / 16]) {
+  constexpr int KT = K / 16, Q = KT / kWideWaves;
+  const int b = lane & 15, g = lane >> 4;
+  const int col = s * kSlice + b;
+  v4f z[Q];
+#pragma unroll
+  for (int q = 0; q < Q; ++q) z[q] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int u = -1; u < nd.lc_cnt; ++u) {
+    const int var = u < 0 ? nd.var : d.child_leaf[nd.lc_off + u];
+    const int x = d.xb[(size_t)var * d.Bp + col];
+    const float* row = d.leaf + ((size_t)var * d.C + x) * K;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) z[q] += *reinterpret_cast<const v4f*>(row + (wave * Q + q) * 16 + 4 * g);
+  }
+  for (int c = 0; c < nd.ic_cnt; ++c) {
+    const int cn = d.child_inner[nd.ic_off + c];
+    const v4f* t = reinterpret_cast<const v4f*>(d.O + ((size_t)cn * d.nslices + s) * kSlice * K);
+#pragma unroll
+    for (int q = 0; q < Q; ++q) z[q] += t[(wave * Q + q) * 64 + lane];
+  }
+  float m = -INFINITY;
+#pragma unroll
+  for (int q = 0; q < Q; ++q)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) m = fmaxf(m, z[q][i]);
+  m = fmaxf(m, __shfl_xor(m, 16));
+  m = fmaxf(m, __shfl_xor(m, 32));
+  if (g == 0) L.mx[wave][b] = m;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < kWideWaves; ++w) m = fmaxf(m, L.mx[w][b]);
+#pragma unroll
+  for (int q = 0; q < Q; ++q) {
+    v4f x;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) x[i] = __expf(z[q][i] - m);
+    L.e[wave * Q + q][lane] = x;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int kt = 0; kt < KT; ++kt) e[kt] = L.e[kt][lane];
+  return m;
+}
+
+// Forward: one workgroup per 16-example slice walks the nodes children-first.
+template <int K>
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_forward_kernel(HcltDev d, float* __restrict__ ll) {
+  constexpr int KT = K / 16, Q = KT / kWideWaves;
+  __shared__ WideLds<K> L;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
+  const int b = lane & 15, g = lane >> 4;
+  for (int n = 0; n < d.n_inner; ++n) {
+    const HcltNode nd = d.nodes[n];
+    // this wave's rows of the parameter block: they wait for nothing computed here
+    v4f w[Q][KT];
+    const v4f* wf = reinterpret_cast<const v4f*>(d.Wf + (size_t)n * K * K);
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+#pragma unroll
+      for (int jt = 0; jt < KT; ++jt) w[q][jt] = wf[((wave * Q + q) * KT + jt) * 64 + lane];
+    v4f e[KT];
+    const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
+    v4f* out = reinterpret_cast<v4f*>(d.O + ((size_t)n * d.nslices + s) * kSlice * K);
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int jt = 0; jt < KT; ++jt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][jt][i], e[jt][i], acc, 0, 0, 0);
+      v4f o;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = m + __logf(acc[i]);
+      out[(wave * Q + q) * 64 + lane] = o;
+      if (nd.is_root && wave == 0 && q == 0 && g == 0 && s * kSlice + b < d.B) ll[s * kSlice + b] = o[0];
+    }
+    __syncthreads();   // the tile is read by the parent's step; LDS is reused
+  }
+}
+
+// Backward: the same workgroups walk the nodes parents-first.  Besides the flow tile G handed
+// to the children, every node leaves R and E in the operand layout of the statistics
+// contraction: lane 16*g' + r holds, for t < 4, the value of example 4*t + g' at state
+// kt*16 + r (the contraction runs over examples).
+template <int K>
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_backward_kernel(HcltDev d, float* G, float* __restrict__ RS,
+                                                                             float* __restrict__ ES) {
+  constexpr int KT = K / 16, Q = KT / kWideWaves;
+  __shared__ WideLds<K> L;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
+  const int b = lane & 15, g = lane >> 4;
+  const bool live = s * kSlice + b < d.B;
+  for (int n = d.n_inner - 1; n >= 0; --n) {
+    const HcltNode nd = d.nodes[n];
+    v4f w[Q][KT];
+    const v4f* wb = reinterpret_cast<const v4f*>(d.Wb + (size_t)n * K * K);
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) w[q][kt] = wb[((wave * Q + q) * KT + kt) * 64 + lane];
+    v4f e[KT];
+    const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
+    const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
+    const v4f* on = reinterpret_cast<const v4f*>(d.O + tile);
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      const int kt = wave * Q + q;
+      const v4f o = on[kt * 64 + lane];
+      v4f f;
+      if (nd.parent < 0) {
+        f = v4f{kt == 0 && g == 0 && live ? 1.f : 0.f, 0.f, 0.f, 0.f};
+      } else {
+        f = reinterpret_cast<const v4f*>(G + ((size_t)nd.parent * d.nslices + s) * kSlice * K)[kt * 64 + lane];
+      }
+      v4f r;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float sc = __expf(o[i] - m);
+        r[i] = (sc > 0.f && f[i] > 0.f) ? f[i] / sc : 0.f;
+      }
+      L.r[kt][lane] = r;
+    }
+    __syncthreads();
+    v4f r[KT];
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) r[kt] = L.r[kt][lane];
+    v4f* gout = reinterpret_cast<v4f*>(G + tile);
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      const int jt = wave * Q + q;
+      v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][kt][i], r[kt][i], acc, 0, 0, 0);
+      gout[jt * 64 + lane] = e[jt] * acc;
+    }
+    // statistics operands: lane = 16*g' + row reads example 4*t + g', state kt*16 + row
+    {
+      const int row = lane & 15, gp = lane >> 4;
+      const int src = 16 * (row >> 2) + gp, comp = row & 3;
+#pragma unroll
+      for (int q = 0; q < Q; ++q) {
+        const int kt = wave * Q + q;
+        v4f rs, es;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          rs[t] = reinterpret_cast<const float*>(&L.r[kt][src + 4 * t])[comp];
+          es[t] = reinterpret_cast<const float*>(&L.e[kt][src + 4 * t])[comp];
+        }
+        reinterpret_cast<v4f*>(RS + tile)[kt * 64 + lane] = rs;
+        reinterpret_cast<v4f*>(ES + tile)[kt * 64 + lane] = es;
+      }
+    }
+    __syncthreads();   // G is read by the children's steps; LDS is reused
+  }
+}
+
+// Edge statistics: workgroup (node n, row tile kt) contracts R^T E over all examples.
+template <int K>
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_edge_kernel(HcltDev d, const float* __restrict__ RS,
+                                                                         const float* __restrict__ ES,
+                                                                         float* __restrict__ edge_aggr, float rate) {
+  constexpr int KT = K / 16;
+  __shared__ v4f red[kWideWaves][KT][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = blockIdx.x, kt = blockIdx.y;
+  v4f acc[KT];
+#pragma unroll
+  for (int jt = 0; jt < KT; ++jt) acc[jt] = v4f{0.f, 0.f, 0.f, 0.f};
+  const v4f* rs = reinterpret_cast<const v4f*>(RS + (size_t)n * d.nslices * kSlice * K);
+  const v4f* es = reinterpret_cast<const v4f*>(ES + (size_t)n * d.nslices * kSlice * K);
+  v4f a, e[KT];
+  if (wave < d.nslices) {
+    a = rs[((size_t)wave * KT + kt) * 64 + lane];
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt) e[jt] = es[((size_t)wave * KT + jt) * 64 + lane];
+  }
+  for (int s = wave; s < d.nslices; s += kWideWaves) {
+    const v4f a0 = a;
+    v4f e0[KT];
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt) e0[jt] = e[jt];
+    const int sn = s + kWideWaves;
+    if (sn < d.nslices) {
+      a = rs[((size_t)sn * KT + kt) * 64 + lane];
+#pragma unroll
+      for (int jt = 0; jt < KT; ++jt) e[jt] = es[((size_t)sn * KT + jt) * 64 + lane];
+    }
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt)
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[t], e0[jt][t], acc[jt], 0, 0, 0);
+  }
+#pragma unroll
+  for (int jt = 0; jt < KT; ++jt) red[wave][jt][lane] = acc[jt];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < KT * 64; idx += blockDim.x) {
+    const int jt = idx >> 6, l = idx & 63;
+    v4f sum = red[0][jt][l];
+#pragma unroll
+    for (int w = 1; w < kWideWaves; ++w) sum += red[w][jt][l];
+    const int g = l >> 4, j = jt * 16 + (l & 15);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const size_t at = ((size_t)n * K + kt * 16 + 4 * g + i) * K + j;
+      const float old = rate != 0.f ? rate * edge_aggr[at] : 0.f;
+      edge_aggr[at] = old + __expf(d.logtheta[at]) * sum[i];
+    }
+  }
+}
+
+// Leaf histograms: workgroup (variable u, state tile kt) adds, for every example, the 16 flows
+// of the tile to row x_b of a [C][16] table in LDS, as two-limb fixed-point integers (integer
+// LDS atomics are more than ten times cheaper than floating-point ones here and make the sum
+// independent of the order of arrival); flows are in [0, 1].
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev d, const float* __restrict__ G,
+                                                                         const int32_t* __restrict__ state_node, int K,
+                                                                         float* __restrict__ leaf_flow, float rate,
+                                                                         int limb) {
+  extern __shared__ unsigned hist[];   // [2][C][17]
+  constexpr int HS = 17;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = lane & 15, g = lane >> 4;
+  const int u = blockIdx.x, kt = blockIdx.y, KT = K / 16;
+  const int n = state_node[u];
+  const int hw = d.C * HS;
+  for (int i = threadIdx.x; i < 2 * hw; i += blockDim.x) hist[i] = 0u;
+  __syncthreads();
+  const float scale = __builtin_ldexpf(1.f, limb);
+  const v4f* gt = reinterpret_cast<const v4f*>(G + (size_t)n * d.nslices * kSlice * K);
+  for (int s = wave; s < d.nslices; s += kWideWaves) {
+    const int col = s * kSlice + b;
+    const int x = d.xb[(size_t)u * d.Bp + col];
+    const v4f f = gt[((size_t)s * KT + kt) * 64 + lane];
+    if (col < d.B) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float v = fminf(fmaxf(f[i], 0.f), 1.f) * scale;
+        const float fl = floorf(v);
+        __hip_atomic_fetch_add(&hist[x * HS + 4 * g + i], (unsigned)fl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_fetch_add(&hist[hw + x * HS + 4 * g + i], (unsigned)((v - fl) * scale), __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+  }
+  __syncthreads();
+  const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+  for (int i = threadIdx.x; i < d.C * 16; i += blockDim.x) {
+    const int c = i >> 4, jj = i & 15;
+    const float val = (float)hist[c * HS + jj] * hi_inv + (float)hist[hw + c * HS + jj] * lo_inv;
+    const size_t at = ((size_t)u * d.C + c) * K + kt * 16 + jj;
+    const float old = rate != 0.f ? rate * leaf_flow[at] : 0.f;
+    leaf_flow[at] = old + val;
+  }
+}
+
+// ---- host --------------------------------------------------------------------------------
+
+#define PCM_DISPATCH_WIDE_K(K_, ...)                                                         \
+  switch (K_) {                                                                              \
+    case 128: { constexpr int KK = 128; __VA_ARGS__; break; }                                \
+    default: fail(PCM_ERR_STATE, "no wide block kernel for hidden size %d", K_);             \
+  }
+
+void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
+  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(kWideWaves * 64), 0, stream,
+                                             d, d_ll));
+  check_launch_w("hclt_wide_forward");
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
+}
+
+void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate) {
+  if (d_wide_state_node_.n == 0) {
+    std::vector<int32_t> t(V_);
+    for (int v = 0; v < V_; ++v) t[v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
+    d_wide_state_node_.upload(t, stream);
+  }
+  int bits = 0;
+  while ((1 << bits) < d.Bp) ++bits;
+  const int limb = std::min(24, 32 - bits);
+  if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
+  PCM_DISPATCH_WIDE_K(K_, {
+    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(kWideWaves * 64), 0, stream, d, d_G_.p,
+                       d_wide_rs_.p, d_wide_es_.p);
+    check_launch_w("hclt_wide_backward");
+    if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
+    hipLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream, d,
+                       d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p, rate);
+  });
+  const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
+  hipLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), lds, stream, d, d_G_.p,
+                     d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
+  check_launch_w("hclt_wide_stats");
+  if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
+}
+
+}  // namespace pcm

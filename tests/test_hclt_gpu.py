@@ -53,7 +53,8 @@ def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None, tree=None):
     return bpc
 
 
-@pytest.mark.parametrize("V,K,C,B", [(2, 16, 5, 16), (7, 16, 8, 48), (12, 32, 256, 64), (9, 64, 17, 32)])
+@pytest.mark.parametrize("V,K,C,B", [(2, 16, 5, 16), (7, 16, 8, 48), (12, 32, 256, 64), (9, 64, 17, 32),
+                                     (2, 128, 5, 16), (10, 128, 256, 70)])
 def test_em_step_matches_oracle(gpu, oracle, V, K, C, B):
     _compare_step(gpu, oracle, V, K, C, B, seed=100 + V)
 
@@ -66,6 +67,7 @@ def test_em_step_on_wide_trees(gpu, oracle, tree):
     inline ones, schedule items read from memory)."""
     _compare_step(gpu, oracle, len(tree), 16, 7, 40, seed=len(tree), tree=tree)
     _compare_step(gpu, oracle, len(tree), 32, 12, 33, seed=len(tree) + 1, tree=tree)
+    _compare_step(gpu, oracle, len(tree), 128, 9, 21, seed=len(tree) + 2, tree=tree)   # the wide block kernels
 
 
 def test_ragged_batch_and_example_ids(gpu, oracle):
@@ -139,8 +141,10 @@ def test_ten_em_steps_track_oracle(gpu, oracle):
 
 @pytest.mark.parametrize("V,K,C,B", [(6, 8, 5, 40), (5, 128, 7, 33), (9, 3, 4, 70)])
 def test_hidden_sizes_without_block_kernels(gpu, oracle, V, K, C, B):
-    """Hidden sizes other than 16 / 32 / 64 run on the layered engine behind the same HCLT
-    interface (block-form parameters and flows, EM step, KL, sampling)."""
+    """Hidden sizes without walk kernels: 128 has the wide block kernels for likelihoods, flows
+    and EM and the layered engine for the other queries, the rest run entirely on the layered
+    engine, all behind the same HCLT interface (block-form parameters and flows, EM step, KL,
+    sampling)."""
     torch, P = gpu
     bpc = _compare_step(gpu, oracle, V, K, C, B, seed=7 * K + V)
     assert bpc.size("hidden_categories") == K
