@@ -986,12 +986,14 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     pull_from_general();
     return;
   }
-  PCM_DISPATCH_PARAM_K(K_, hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)),
-                                        dim3(128), 0, stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p,
-                                        d_edge_aggr_.p, n_inner_, pseudocount, inertia));
+  PCM_DISPATCH_PARAM_K(K_, {
+    constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
+    hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,
+                       stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia);
+  });
   check_launch("theta_update");
-  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
-                     pseudocount, inertia);
+  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_, ceil_div(K_, 32)), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_,
+                     K_, pseudocount, inertia);
   check_launch("leaf_update");
   general_stale_ = true;
 }

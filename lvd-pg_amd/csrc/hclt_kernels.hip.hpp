@@ -653,52 +653,64 @@ __global__ void hclt_rebuild_w_kernel(const float* __restrict__ logtheta, float*
   put_w<K>(Wf + (size_t)n * K * K, Wb + (size_t)n * K * K, k, j, __expf(logtheta[i]));
 }
 
-// Sum-edge update, one thread per sum node (tree node n, state k):
-// add_pseudocount, aggr_node_flows, update_params of the reference's EM step.
+// Sum-edge update (add_pseudocount, aggr_node_flows, update_params of the reference's EM
+// step): a group of min(K, 64) lanes per sum node (tree node n, state k), so that a row of K
+// edges is read and written in whole cache lines.
 template <int K>
-__global__ void hclt_theta_update_kernel(const HcltNode* __restrict__ nodes, float* __restrict__ logtheta,
-                                         float* __restrict__ Wf, float* __restrict__ Wb,
-                                         float* __restrict__ edge_aggr, int n_inner,
-                                         float pseudocount, float inertia) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n_inner * K) return;
-  const int n = i / K, k = i % K;
+__global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* __restrict__ nodes,
+                                                                float* __restrict__ logtheta, float* __restrict__ Wf,
+                                                                float* __restrict__ Wb, float* __restrict__ edge_aggr,
+                                                                int n_inner, float pseudocount, float inertia) {
+  constexpr int G = K < 64 ? K : 64, E = K / G, RPB = 256 / G;
+  const int row = blockIdx.x * RPB + threadIdx.x / G, l = threadIdx.x % G;
+  if (row >= n_inner * K) return;
+  const int n = row / K, k = row % K;
   if (nodes[n].is_root && k > 0) return;
-  float* a = edge_aggr + ((size_t)n * K + k) * K;
-  float* lt = logtheta + ((size_t)n * K + k) * K;
+  float* a = edge_aggr + (size_t)row * K;
+  float* lt = logtheta + (size_t)row * K;
   const float share = pseudocount / (float)K;
-  float tot = 0.f;
-  for (int j = 0; j < K; ++j) {
-    a[j] += share;
-    tot += a[j];
+  float av[E], tot = 0.f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    av[e] = a[l + e * G] + share;
+    a[l + e * G] = av[e];
+    tot += av[e];
   }
-  for (int j = 0; j < K; ++j) {
+#pragma unroll
+  for (int o = G / 2; o > 0; o >>= 1) tot += __shfl_xor(tot, o, G);
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    const int j = l + e * G;
     const float oldv = inertia * expf(lt[j]);
-    const float newv = (1.f - inertia) * a[j] / tot;
-    const float l = logf(oldv + newv);
-    lt[j] = l;
-    put_w<K>(Wf + (size_t)n * K * K, Wb + (size_t)n * K * K, k, j, expf(l));
+    const float newv = (1.f - inertia) * av[e] / tot;
+    const float lg = logf(oldv + newv);
+    lt[j] = lg;
+    put_w<K>(Wf + (size_t)n * K * K, Wb + (size_t)n * K * K, k, j, expf(lg));
   }
 }
 
 // Leaf update (the reference's per-input-node update with missing_flow = 0), one workgroup
-// per variable: thread (category group cg, hidden state j) first sums the flows of its
-// categories, the groups are combined through LDS, then every thread rewrites its
-// categories.  Consecutive threads touch consecutive addresses in both passes.
+// per (variable, run of 32 hidden states): thread (category group cg, hidden state j) first
+// sums the flows of its categories, the groups are combined through LDS, then every thread
+// rewrites its categories.  Consecutive threads touch consecutive addresses in both passes.
 __global__ __launch_bounds__(256) void hclt_leaf_update_kernel(float* __restrict__ leaf,
                                                                const float* __restrict__ leaf_flow, int C, int K,
                                                                float pseudocount, float inertia) {
   __shared__ float part[256];
   const int u = blockIdx.x;
-  const int j = threadIdx.x % K, cg = threadIdx.x / K, ncg = blockDim.x / K;
+  const int jl = threadIdx.x & 31, cg = threadIdx.x >> 5, ncg = 8;
+  const int j = blockIdx.y * 32 + jl;
+  const bool valid = j < K;
   float* lp = leaf + (size_t)u * C * K;
   const float* fl = leaf_flow + (size_t)u * C * K;
   float s = 0.f;
-  for (int c = cg; c < C; c += ncg) s += fl[(size_t)c * K + j];
+  if (valid)
+    for (int c = cg; c < C; c += ncg) s += fl[(size_t)c * K + j];
   part[threadIdx.x] = s;
   __syncthreads();
+  if (!valid) return;
   float node_flow = pseudocount;
-  for (int q = 0; q < ncg; ++q) node_flow += part[q * K + j];
+  for (int q = 0; q < ncg; ++q) node_flow += part[q * 32 + jl];
   const float cat_pc = pseudocount / (float)C;
   for (int c = cg; c < C; c += ncg) {
     const size_t i = (size_t)c * K + j;
