@@ -4,6 +4,7 @@
 #include <algorithm>
 #include <cmath>
 #include <numeric>
+#include <type_traits>
 
 #include "stage_kernel.hip.hpp"
 
@@ -187,6 +188,7 @@ struct SparseDev {
   const uint8_t* type;
   const int32_t* order;      // node ids sorted by layer
   const int32_t *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_var, *in_ptr, *in_edge;
+  const int4* in_rec;        // per incoming edge: {edge << 1 | role, parent (~parent: product), prime, sub}
   const int64_t* in_off;
   const float* logp;
   const float* leaf;
@@ -202,73 +204,213 @@ __device__ __forceinline__ float lse2(float x, float y) {
   return fmaxf(x, y);
 }
 
-// Forward, one layer: thread = (node of the layer, example).  Restates
-// src/regularization/reg_likelihood.jl:16-49 (inputs) and src/queries/likelihood.jl:29-48
-// (edges folded in up-edge order with pairwise logsumexp / +).
-__global__ void sparse_forward_kernel(SparseDev d, int n0) {
+// Forward, one layer: a wave takes one node of the layer and 64 * EX examples (thread t:
+// examples t, t + 64, ...).  Restates src/regularization/reg_likelihood.jl:16-49 (inputs) and
+// src/queries/likelihood.jl:29-48: a product adds its children, a sum node is the logsumexp of
+// its edges in up-edge order -- kept as a running maximum and a sum of exponentials relative to
+// it (one exponential per edge; the reference folds pairwise, the two agree to rounding).
+#ifndef PCM_SPARSE_EX
+#define PCM_SPARSE_EX 1
+#endif
+constexpr int kSparseEx = PCM_SPARSE_EX;   // examples per thread in the layer kernels
+
+// The layer kernels are chains of memory round trips (edge records, then the rows they
+// name), not arithmetic: a wave therefore takes its node's edges in runs of 16, then 4, then
+// single ones, and requests all operands of a run before it uses the first.
+
+// x where keep is all ones, +0 where it is zero: a select the compiler cannot turn into a branch
+// around the load that produced x (a branch per edge would serialise the run's requests)
+__device__ __forceinline__ float keep_bits(float x, unsigned keep) {
+  return __builtin_bit_cast(float, __builtin_bit_cast(unsigned, x) & keep);
+}
+
+template <int U, int EX>
+__device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int c0, int e0, const int (&bb)[EX],
+                                            float (&m)[EX], float (&sum)[EX]) {
+  float child[U][EX];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int e = c0 + u;
+    const float* pr = d.mars + (size_t)d.e_prime[e] * d.Bp;
+    const int s = d.e_sub[e];
+    const float* sr = d.mars + (size_t)max(s, 0) * d.Bp;
+    const unsigned has_sub = s >= 0 ? ~0u : 0u;
+    const float lp = d.logp[e];   // 0 on product edges
+#pragma unroll
+    for (int x = 0; x < EX; ++x) child[u][x] = pr[bb[x]] + keep_bits(sr[bb[x]], has_sub) + lp;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int x = 0; x < EX; ++x) {
+      const float c = child[u][x];
+      if (c0 + u == e0) {
+        m[x] = c;
+      } else if (!issum) {
+        m[x] += c;
+      } else if (c > m[x]) {
+        sum[x] = sum[x] * __expf(m[x] - c) + 1.f;
+        m[x] = c;
+      } else if (c != -INFINITY) {
+        sum[x] += __expf(c - m[x]);
+      }
+    }
+}
+
+// Forward, one layer: a wave takes one node of the layer and 64 * EX examples (thread t:
+// examples t, t + 64, ...).  Restates src/regularization/reg_likelihood.jl:16-49 (inputs) and
+// src/queries/likelihood.jl:29-48: a product adds its children, a sum node is the logsumexp of
+// its edges in up-edge order -- kept as a running maximum and a sum of exponentials relative to
+// it (one exponential per edge; the reference folds pairwise, the two agree to rounding).
+template <int EX>
+__global__ __launch_bounds__(64) void sparse_forward_kernel(SparseDev d, int n0) {
   const int n = d.order[n0 + blockIdx.x];
-  const int b = blockIdx.y * blockDim.x + threadIdx.x;
-  if (b >= d.Bp) return;
-  float acc;
+  const int b0 = blockIdx.y * (64 * EX) + threadIdx.x;
+  int bb[EX];
+#pragma unroll
+  for (int x = 0; x < EX; ++x) bb[x] = min(b0 + 64 * x, d.Bp - 1);
+  float m[EX], sum[EX];
   if (d.type[n] == kInput) {
-    acc = d.leaf[d.in_off[n] + d.xb[(size_t)d.in_var[n] * d.Bp + b]];
+    const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
+#pragma unroll
+    for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
   } else {
     const bool issum = d.type[n] == kSum;
     const int e0 = d.node_e0[n], e1 = d.node_e1[n];
-    acc = 0.f;
-    for (int e = e0; e < e1; ++e) {
-      float child = d.mars[(size_t)d.e_prime[e] * d.Bp + b];
-      const int s = d.e_sub[e];
-      if (s >= 0) child += d.mars[(size_t)s * d.Bp + b];
-      if (issum) child += d.logp[e];
-      acc = e == e0 ? child : issum ? lse2(acc, child) : acc + child;
-    }
-  }
-  d.mars[(size_t)n * d.Bp + b] = acc;
-}
-
-__device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-  return v;
+    for (int x = 0; x < EX; ++x) { m[x] = 0.f; sum[x] = 1.f; }
+    int c0 = e0;
+    for (; c0 + 16 <= e1; c0 += 16) forward_run<16, EX>(d, issum, c0, e0, bb, m, sum);
+    for (; c0 + 4 <= e1; c0 += 4) forward_run<4, EX>(d, issum, c0, e0, bb, m, sum);
+    for (; c0 < e1; ++c0) forward_run<1, EX>(d, issum, c0, e0, bb, m, sum);
+  }
+#pragma unroll
+  for (int x = 0; x < EX; ++x)
+    if (b0 + 64 * x < d.Bp) d.mars[(size_t)n * d.Bp + b0 + 64 * x] = sum[x] == 1.f ? m[x] : m[x] + __logf(sum[x]);
 }
 
-// Backward, one layer (top-down): thread = (node, example) adds up the flows of the node's
-// incoming edges, src/queries/flow.jl:49-60: edge_flow = flows[parent] (product edge) or
-// flows[parent] * exp(mars[prime] + logp (+ mars[sub]) - mars[parent]) (sum edge).  Each
-// edge's flow is summed over the batch where the node is the edge's prime (:73-81); input
-// nodes add their flow to the leaf counters (src/nodes/fixable_categorical_dist.jl:121-130).
-__global__ void sparse_backward_kernel(SparseDev d, int n0, const int32_t* __restrict__ seed_of,
-                                       const float* __restrict__ seed, float* __restrict__ edge_aggr,
-                                       float* __restrict__ leaf_flow) {
-  const int n = d.order[n0 + blockIdx.x];
-  const int b = blockIdx.y * blockDim.x + threadIdx.x;
-  const bool live = b < d.B;
-  const int bb = min(b, d.Bp - 1);
-  float acc = 0.f;
-  const int sd = seed_of[n];
-  if (sd >= 0) acc = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
-  for (int i = d.in_ptr[n]; i < d.in_ptr[n + 1]; ++i) {
-    const int ie = d.in_edge[i];
-    const int e = ie >> 1;
-    const int p = d.e_parent[e];
-    float ef = d.flows[(size_t)p * d.Bp + bb];
-    if (d.type[p] == kSum) {
-      float child = d.mars[(size_t)d.e_prime[e] * d.Bp + bb] + d.logp[e];
-      const int s = d.e_sub[e];
-      if (s >= 0) child += d.mars[(size_t)s * d.Bp + bb];
-      ef *= expf(child - d.mars[(size_t)p * d.Bp + bb]);
-    }
-    if (!live) ef = 0.f;
-    acc += ef;
-    if (!(ie & 1) && edge_aggr) {
-      const float tot = wave_sum(ef);
-      if ((threadIdx.x & 63) == 0) atomicAdd(&edge_aggr[e], tot);
+// Sum over the 64 lanes of a wave, valid in every lane: butterflies inside rows of 16 lanes
+// with data-parallel-primitive moves (lane ^ 1, lane ^ 2, mirror of 8, mirror of 16), then the
+// four row sums through scalar registers.
+__device__ __forceinline__ float wave_sum(float v) {
+  auto dpp = [](float x, auto ctrl) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                 0xf, 0xf, true));
+  };
+  v += dpp(v, std::integral_constant<int, 0xB1>{});    // quad_perm [1,0,3,2]
+  v += dpp(v, std::integral_constant<int, 0x4E>{});    // quad_perm [2,3,0,1]
+  v += dpp(v, std::integral_constant<int, 0x141>{});   // row_half_mirror
+  v += dpp(v, std::integral_constant<int, 0x140>{});   // row_mirror
+  const int iv = __builtin_bit_cast(int, v);
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32)) +
+         __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+}
+
+template <int U, int EX>
+__device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const int (&bb)[EX], const bool (&live)[EX],
+                                             float (&acc)[EX], float* __restrict__ edge_aggr) {
+  float fl[U][EX], ex[U][EX];
+  int ies[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int4 rec = d.in_rec[c0 + u];   // one scalar record per edge instead of a chain of four index fetches
+    ies[u] = rec.x;
+    const bool issum = rec.y >= 0;
+    const int p = issum ? rec.y : ~rec.y;
+    const int s = rec.w;
+    const float* fr = d.flows + (size_t)p * d.Bp;
+    const float* mp = d.mars + (size_t)p * d.Bp;
+    const float* pr = d.mars + (size_t)rec.z * d.Bp;
+    const float* sr = d.mars + (size_t)max(s, 0) * d.Bp;
+    const float lp = d.logp[rec.x >> 1];
+    const unsigned has_sub = s >= 0 ? ~0u : 0u, sum_edge = issum ? ~0u : 0u;
+#pragma unroll
+    for (int x = 0; x < EX; ++x) {
+      fl[u][x] = fr[bb[x]];
+      ex[u][x] = keep_bits(pr[bb[x]] + lp + keep_bits(sr[bb[x]], has_sub) - mp[bb[x]], sum_edge);
     }
   }
-  if (b < d.Bp) d.flows[(size_t)n * d.Bp + b] = live ? acc : 0.f;
-  if (live && leaf_flow && d.type[n] == kInput)
-    atomicAdd(&leaf_flow[d.in_off[n] + d.xb[(size_t)d.in_var[n] * d.Bp + b]], acc);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    float part = 0.f;
+#pragma unroll
+    for (int x = 0; x < EX; ++x) {
+      float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * expf(ex[u][x]);   // product edges carry exponent 0
+      if (!live[x]) ef = 0.f;
+      acc[x] += ef;
+      part += ef;
+    }
+    if (!(ies[u] & 1) && edge_aggr) {
+      const float tot = wave_sum(part);
+      if (threadIdx.x == 0) atomicAdd(&edge_aggr[ies[u] >> 1], tot);
+    }
+  }
+}
+
+// Backward, one layer (top-down): a wave takes one node and 64 * EX examples and adds up the
+// flows of the node's incoming edges, src/queries/flow.jl:49-60: edge_flow = flows[parent]
+// (product edge) or flows[parent] * exp(mars[prime] + logp (+ mars[sub]) - mars[parent]) (sum
+// edge).  Each edge's flow is summed over the batch where the node is the edge's prime
+// (:73-81): over the thread's examples, then over the wave, then one atomic.
+template <int EX>
+__global__ __launch_bounds__(64) void sparse_backward_kernel(SparseDev d, int n0, const int32_t* __restrict__ seed_of,
+                                                             const float* __restrict__ seed,
+                                                             float* __restrict__ edge_aggr,
+                                                             const int32_t* __restrict__ alias_ptr,
+                                                             const int32_t* __restrict__ alias_list) {
+  const int n = d.order[n0 + blockIdx.x];
+  const int b0 = blockIdx.y * (64 * EX) + threadIdx.x;
+  int bb[EX];
+  bool live[EX];
+  float acc[EX];
+  const int sd = seed_of[n];
+#pragma unroll
+  for (int x = 0; x < EX; ++x) {
+    const int b = b0 + 64 * x;
+    live[x] = b < d.B;
+    bb[x] = min(b, d.Bp - 1);
+    acc[x] = 0.f;
+    if (sd >= 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
+  }
+  const int i1 = d.in_ptr[n + 1];
+  int c0 = d.in_ptr[n];
+  for (; c0 + 16 <= i1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 + 4 <= i1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 < i1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_aggr);
+#pragma unroll
+  for (int x = 0; x < EX; ++x) {
+    const int b = b0 + 64 * x;
+    if (b < d.Bp) d.flows[(size_t)n * d.Bp + b] = live[x] ? acc[x] : 0.f;
+  }
+  // input nodes that receive exactly this node's edge flows (the other factor of the same
+  // two-child products) are not computed again: their rows are copies
+  for (int q = alias_ptr[n]; q < alias_ptr[n + 1]; ++q) {
+    const int t = alias_list[q];
+#pragma unroll
+    for (int x = 0; x < EX; ++x) {
+      const int b = b0 + 64 * x;
+      if (b < d.Bp) d.flows[(size_t)t * d.Bp + b] = live[x] ? acc[x] : 0.f;
+    }
+  }
+}
+
+// Leaf counters, src/nodes/fixable_categorical_dist.jl:121-130: an input node's flow goes to the
+// counter of the example's category.  One workgroup per input node over the whole batch: the
+// node owns its C counters, so they are summed in LDS and added to memory without atomics.
+__global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, const int32_t* __restrict__ input_nodes,
+                                                               float* __restrict__ leaf_flow) {
+  __shared__ float hist[256];
+  const int n = input_nodes[blockIdx.x];
+  for (int c = threadIdx.x; c < d.C; c += blockDim.x) hist[c] = 0.f;
+  __syncthreads();
+  const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
+  const float* fr = d.flows + (size_t)n * d.Bp;
+  for (int b = threadIdx.x; b < d.B; b += blockDim.x) atomicAdd(&hist[xr[b]], fr[b]);
+  __syncthreads();
+  float* dst = leaf_flow + d.in_off[n];
+  for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += hist[c];
 }
 
 __global__ void sparse_scale_kernel(float* p, int64_t n, float rate) {
@@ -569,6 +711,12 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
     }
   }
   if (in_edge.empty()) in_edge.push_back(0);
+  std::vector<int4> in_rec(in_edge.size());
+  for (size_t i = 0; i < in_edge.size() && ne; ++i) {
+    const int32_t e = in_edge[i] >> 1, p = fc_.e_parent[e];
+    in_rec[i] = int4{in_edge[i], fc_.type[p] == kSum ? p : ~p, fc_.e_prime[e], fc_.e_sub[e]};
+  }
+  d_in_rec_.upload(in_rec);
   d_type_.upload(fc_.type);
   d_order_.upload(order);
   d_node_e0_.upload(fc_.node_e0); d_node_e1_.upload(fc_.node_e1);
@@ -586,6 +734,39 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   if (fc_.heads.empty()) seed_of[nn - 1] = 0;
   else for (size_t h = 0; h < fc_.heads.size(); ++h) seed_of[fc_.heads[h]] = (int32_t)h;
   d_heads_.upload(seed_of);
+  // An input node that is the second factor of two-child products and sees exactly the edges its
+  // first factor (the prime) sees gets the same flow as the prime: it is dropped from the backward
+  // layers and the prime's wave writes its row too (in an HCLT: every leaf).
+  std::vector<int32_t> alias_of(nn, -1);
+  for (int64_t b = 0; b < nn && ne; ++b) {
+    const int i0 = in_ptr[b], i1 = in_ptr[b + 1];
+    if (fc_.type[b] != kInput || seed_of[b] >= 0 || i0 == i1 || !(in_edge[i0] & 1)) continue;
+    const int32_t a = fc_.e_prime[in_edge[i0] >> 1];
+    if (a == b || in_ptr[a + 1] - in_ptr[a] != i1 - i0) continue;
+    bool same = true;
+    for (int q = 0; q < i1 - i0 && same; ++q)
+      same = (in_edge[i0 + q] & 1) && in_edge[in_ptr[a] + q] == (in_edge[i0 + q] & ~1);
+    if (same) alias_of[b] = a;
+  }
+  std::vector<int32_t> alias_ptr(nn + 1, 0), alias_list;
+  for (int64_t b = 0; b < nn; ++b) if (alias_of[b] >= 0) alias_ptr[alias_of[b] + 1]++;
+  for (int64_t n = 0; n < nn; ++n) alias_ptr[n + 1] += alias_ptr[n];
+  alias_list.resize(alias_ptr[nn]);
+  {
+    std::vector<int32_t> fill(alias_ptr.begin(), alias_ptr.end() - 1);
+    for (int64_t b = 0; b < nn; ++b) if (alias_of[b] >= 0) alias_list[fill[alias_of[b]]++] = (int32_t)b;
+  }
+  if (alias_list.empty()) alias_list.push_back(0);
+  std::vector<int32_t> bwd_order;
+  bwd_layer0_.assign(n_layers_ + 1, 0);
+  for (int l = 0; l < n_layers_; ++l) {
+    for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i)
+      if (alias_of[order[i]] < 0) bwd_order.push_back(order[i]);
+    bwd_layer0_[l + 1] = (int)bwd_order.size();
+  }
+  d_alias_ptr_.upload(alias_ptr);
+  d_alias_list_.upload(alias_list);
+  d_bwd_order_.upload(bwd_order);
   // normalisation groups over the sum parameters
   std::vector<int32_t> gp(1, 0), p2e;
   for (int64_t s : fc_.pargroup_sizes) gp.push_back(gp.back() + (int32_t)s);
@@ -675,18 +856,18 @@ void SparseCircuit::ensure_batch(int batch) {
 
 static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32_t* e0, const int32_t* e1,
                           const int32_t* ep, const int32_t* epr, const int32_t* es, const int32_t* in_var,
-                          const int32_t* in_ptr, const int32_t* in_edge, const int64_t* in_off, const float* logp,
+                          const int32_t* in_ptr, const int32_t* in_edge, const int4* in_rec, const int64_t* in_off, const float* logp,
                           const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C) {
   SparseDev d;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
-  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
+  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
   d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C;
   return d;
 }
 
 #define SPARSE_DEV(B_, Bp_, xb_) \
   make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
-           d_in_ptr_.p, d_in_edge_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
+           d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
 
 void SparseCircuit::run_forward(const BatchRef& b) {
   if (!b.d_data) fail(PCM_ERR_ARG, "data pointer is null");
@@ -702,7 +883,9 @@ void SparseCircuit::run_forward(const BatchRef& b) {
   SparseDev d = SPARSE_DEV(b.batch, Bp, xb);
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
-    hipLaunchKernelGGL(sparse_forward_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
+    if (Bp >= 64 * kSparseEx)
+      hipLaunchKernelGGL(sparse_forward_kernel<kSparseEx>, dim3(cnt, ceil_div(Bp, 64 * kSparseEx)), dim3(64), 0, stream, d, n0);
+    else hipLaunchKernelGGL(sparse_forward_kernel<1>, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
   }
   check_launch("sparse_forward");
   last_batch_ = b.batch;
@@ -737,10 +920,22 @@ void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mas
   hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)fc_.leaf_logp.size(), 256)), dim3(256), 0, stream,
                      d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
   SparseDev d = SPARSE_DEV(b.batch, Bp, d_visit_.p);
+  SparseDev db = d;
+  db.order = d_bwd_order_.p;   // the layers without the input nodes whose rows other nodes write
   for (int l = n_layers_ - 1; l >= 0; --l) {
-    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
-    hipLaunchKernelGGL(sparse_backward_kernel, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0, d_heads_.p, d_head_mask,
-                       d_edge_aggr_.p, d_leaf_flow_.p);
+    const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
+    if (cnt == 0) continue;
+    if (Bp >= 64 * kSparseEx)
+      hipLaunchKernelGGL(sparse_backward_kernel<kSparseEx>, dim3(cnt, ceil_div(Bp, 64 * kSparseEx)), dim3(64), 0, stream, db, n0,
+                         d_heads_.p, d_head_mask, d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
+    else
+      hipLaunchKernelGGL(sparse_backward_kernel<1>, dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p, d_head_mask,
+                         d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
+  }
+  if (!fc_.input_nodes.empty()) {
+    if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);
+    hipLaunchKernelGGL(sparse_leaf_flow_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 0, stream, d,
+                       d_input_nodes_.p, d_leaf_flow_.p);
   }
   check_launch("sparse_backward");
   if (fc_.heads.empty()) {

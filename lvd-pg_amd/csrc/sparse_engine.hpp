@@ -88,6 +88,9 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_logp_, d_leaf_, d_edge_aggr_, d_leaf_flow_, d_mars_, d_flows_, d_kld_, d_edge_kld_, d_grad_;
   // incoming edges per node (down direction)
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
+  DevBuf<int4> d_in_rec_;
+  DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
+  std::vector<int> bwd_layer0_;
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
   DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
