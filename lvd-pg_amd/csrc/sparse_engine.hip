@@ -189,6 +189,7 @@ struct SparseDev {
   const int32_t* order;      // node ids sorted by layer
   const int32_t *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_var, *in_ptr, *in_edge;
   const int4* in_rec;        // per incoming edge: {edge << 1 | role, parent (~parent: product), prime, sub}
+  const float* in_logp;      // ... and the edge's log-parameter, gathered before every backward pass
   const int64_t* in_off;
   const float* logp;
   const float* leaf;
@@ -204,15 +205,6 @@ __device__ __forceinline__ float lse2(float x, float y) {
   return fmaxf(x, y);
 }
 
-// Forward, one layer: a wave takes one node of the layer and 64 * EX examples (thread t:
-// examples t, t + 64, ...).  Restates src/regularization/reg_likelihood.jl:16-49 (inputs) and
-// src/queries/likelihood.jl:29-48: a product adds its children, a sum node is the logsumexp of
-// its edges in up-edge order -- kept as a running maximum and a sum of exponentials relative to
-// it (one exponential per edge; the reference folds pairwise, the two agree to rounding).
-#ifndef PCM_SPARSE_EX
-#define PCM_SPARSE_EX 1
-#endif
-constexpr int kSparseEx = PCM_SPARSE_EX;   // examples per thread in the layer kernels
 
 // The layer kernels are chains of memory round trips (edge records, then the rows they
 // name), not arithmetic: a wave therefore takes its node's edges in runs of 16, then 4, then
@@ -225,7 +217,7 @@ __device__ __forceinline__ float keep_bits(float x, unsigned keep) {
 }
 
 template <int U, int EX>
-__device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int c0, int e0, const int (&bb)[EX],
+__device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int c0, const int (&bb)[EX],
                                             float (&m)[EX], float (&sum)[EX]) {
   float child[U][EX];
 #pragma unroll
@@ -244,9 +236,7 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int 
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
       const float c = child[u][x];
-      if (c0 + u == e0) {
-        m[x] = c;
-      } else if (!issum) {
+      if (!issum) {
         m[x] += c;
       } else if (c > m[x]) {
         sum[x] = sum[x] * __expf(m[x] - c) + 1.f;
@@ -257,32 +247,74 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int 
     }
 }
 
-// Forward, one layer: a wave takes one node of the layer and 64 * EX examples (thread t:
+// Forward, one layer: a workgroup takes one node of the layer and 64 * EX examples (lane t:
 // examples t, t + 64, ...).  Restates src/regularization/reg_likelihood.jl:16-49 (inputs) and
 // src/queries/likelihood.jl:29-48: a product adds its children, a sum node is the logsumexp of
 // its edges in up-edge order -- kept as a running maximum and a sum of exponentials relative to
 // it (one exponential per edge; the reference folds pairwise, the two agree to rounding).
-template <int EX>
-__global__ __launch_bounds__(64) void sparse_forward_kernel(SparseDev d, int n0) {
+// kLayerWaves waves share a node's edges: the kernels are chains of dependent memory round
+// trips, so a layer too small to fill the machine finishes sooner when a node's chain is cut in
+// four; layers with plenty of (node, 64 examples) pairs give each pair one wave.
+constexpr int kSplitWaves = 4;
+constexpr int kSplitBelow = 1024;   // (node, 64 examples) pairs in a layer below which its nodes are split
+
+template <int EX, int kLayerWaves>
+__global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(SparseDev d, int n0) {
+  __shared__ float xm[kLayerWaves][EX][64], xs[kLayerWaves][EX][64];
   const int n = d.order[n0 + blockIdx.x];
-  const int b0 = blockIdx.y * (64 * EX) + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b0 = blockIdx.y * (64 * EX) + lane;
   int bb[EX];
 #pragma unroll
   for (int x = 0; x < EX; ++x) bb[x] = min(b0 + 64 * x, d.Bp - 1);
   float m[EX], sum[EX];
   if (d.type[n] == kInput) {
+    if (wave) return;
     const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
 #pragma unroll
     for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
   } else {
+    // the node's edges in kLayerWaves contiguous shares, one per wave; a share is folded as a
+    // running maximum and a sum of exponentials (products: a plain sum), the shares are then
+    // combined through LDS by the first wave
     const bool issum = d.type[n] == kSum;
     const int e0 = d.node_e0[n], e1 = d.node_e1[n];
+    const int per = (e1 - e0 + kLayerWaves - 1) / kLayerWaves;
+    const int my0 = min(e0 + wave * per, e1), my1 = min(my0 + per, e1);
 #pragma unroll
-    for (int x = 0; x < EX; ++x) { m[x] = 0.f; sum[x] = 1.f; }
-    int c0 = e0;
-    for (; c0 + 16 <= e1; c0 += 16) forward_run<16, EX>(d, issum, c0, e0, bb, m, sum);
-    for (; c0 + 4 <= e1; c0 += 4) forward_run<4, EX>(d, issum, c0, e0, bb, m, sum);
-    for (; c0 < e1; ++c0) forward_run<1, EX>(d, issum, c0, e0, bb, m, sum);
+    for (int x = 0; x < EX; ++x) { m[x] = issum ? -INFINITY : 0.f; sum[x] = issum ? 0.f : 1.f; }
+    int c0 = my0;
+    for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX>(d, issum, c0, bb, m, sum);
+    for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX>(d, issum, c0, bb, m, sum);
+    for (; c0 + 4 <= my1; c0 += 4) forward_run<4, EX>(d, issum, c0, bb, m, sum);
+    for (; c0 < my1; ++c0) forward_run<1, EX>(d, issum, c0, bb, m, sum);
+    if (e1 - e0 > per) {   // more than one share is in use (uniform over the workgroup)
+#pragma unroll
+      for (int x = 0; x < EX; ++x) { xm[wave][x][lane] = m[x]; xs[wave][x][lane] = sum[x]; }
+      __syncthreads();
+      if (wave) return;
+#pragma unroll
+      for (int x = 0; x < EX; ++x) {
+        if (issum) {
+          float mm = m[x];
+#pragma unroll
+          for (int w = 1; w < kLayerWaves; ++w) mm = fmaxf(mm, xm[w][x][lane]);
+          float ss = 0.f;
+#pragma unroll
+          for (int w = 0; w < kLayerWaves; ++w) {
+            const float mw = xm[w][x][lane];
+            if (mw != -INFINITY) ss += xs[w][x][lane] * __expf(mw - mm);
+          }
+          m[x] = mm;
+          sum[x] = mm == -INFINITY ? 1.f : ss;
+        } else {
+#pragma unroll
+          for (int w = 1; w < kLayerWaves; ++w) m[x] += xm[w][x][lane];
+        }
+      }
+    } else if (wave) {
+      return;
+    }
   }
 #pragma unroll
   for (int x = 0; x < EX; ++x)
@@ -324,7 +356,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
     const float* mp = d.mars + (size_t)p * d.Bp;
     const float* pr = d.mars + (size_t)rec.z * d.Bp;
     const float* sr = d.mars + (size_t)max(s, 0) * d.Bp;
-    const float lp = d.logp[rec.x >> 1];
+    const float lp = d.in_logp[c0 + u];
     const unsigned has_sub = s >= 0 ? ~0u : 0u, sum_edge = issum ? ~0u : 0u;
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
@@ -344,24 +376,27 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
     }
     if (!(ies[u] & 1) && edge_aggr) {
       const float tot = wave_sum(part);
-      if (threadIdx.x == 0) atomicAdd(&edge_aggr[ies[u] >> 1], tot);
+      if ((threadIdx.x & 63) == 0) atomicAdd(&edge_aggr[ies[u] >> 1], tot);
     }
   }
 }
 
-// Backward, one layer (top-down): a wave takes one node and 64 * EX examples and adds up the
+// Backward, one layer (top-down): a workgroup takes one node and 64 * EX examples and adds up the
 // flows of the node's incoming edges, src/queries/flow.jl:49-60: edge_flow = flows[parent]
 // (product edge) or flows[parent] * exp(mars[prime] + logp (+ mars[sub]) - mars[parent]) (sum
 // edge).  Each edge's flow is summed over the batch where the node is the edge's prime
 // (:73-81): over the thread's examples, then over the wave, then one atomic.
-template <int EX>
-__global__ __launch_bounds__(64) void sparse_backward_kernel(SparseDev d, int n0, const int32_t* __restrict__ seed_of,
-                                                             const float* __restrict__ seed,
-                                                             float* __restrict__ edge_aggr,
-                                                             const int32_t* __restrict__ alias_ptr,
-                                                             const int32_t* __restrict__ alias_list) {
+template <int EX, int kLayerWaves>
+__global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
+                                                                           const int32_t* __restrict__ seed_of,
+                                                                           const float* __restrict__ seed,
+                                                                           float* __restrict__ edge_aggr,
+                                                                           const int32_t* __restrict__ alias_ptr,
+                                                                           const int32_t* __restrict__ alias_list) {
+  __shared__ float xa[kLayerWaves][EX][64];
   const int n = d.order[n0 + blockIdx.x];
-  const int b0 = blockIdx.y * (64 * EX) + threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b0 = blockIdx.y * (64 * EX) + lane;
   int bb[EX];
   bool live[EX];
   float acc[EX];
@@ -372,13 +407,29 @@ __global__ __launch_bounds__(64) void sparse_backward_kernel(SparseDev d, int n0
     live[x] = b < d.B;
     bb[x] = min(b, d.Bp - 1);
     acc[x] = 0.f;
-    if (sd >= 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
+    if (sd >= 0 && wave == 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
   }
-  const int i1 = d.in_ptr[n + 1];
-  int c0 = d.in_ptr[n];
-  for (; c0 + 16 <= i1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_aggr);
-  for (; c0 + 4 <= i1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_aggr);
-  for (; c0 < i1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_aggr);
+  // the node's incoming edges in kLayerWaves contiguous shares, one per wave
+  const int i0 = d.in_ptr[n], i1 = d.in_ptr[n + 1];
+  const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
+  const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
+  int c0 = my0;
+  for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 < my1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_aggr);
+  if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
+#pragma unroll
+    for (int x = 0; x < EX; ++x) xa[wave][x][lane] = acc[x];
+    __syncthreads();
+    if (wave) return;
+#pragma unroll
+    for (int x = 0; x < EX; ++x)
+#pragma unroll
+      for (int w = 1; w < kLayerWaves; ++w) acc[x] += xa[w][x][lane];
+  } else if (wave) {
+    return;
+  }
 #pragma unroll
   for (int x = 0; x < EX; ++x) {
     const int b = b0 + 64 * x;
@@ -411,6 +462,12 @@ __global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, cons
   __syncthreads();
   float* dst = leaf_flow + d.in_off[n];
   for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += hist[c];
+}
+
+__global__ void sparse_gather_in_logp_kernel(const int4* __restrict__ in_rec, const float* __restrict__ logp, int64_t n,
+                                             float* __restrict__ in_logp) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) in_logp[i] = logp[in_rec[i].x >> 1];
 }
 
 __global__ void sparse_scale_kernel(float* p, int64_t n, float rate) {
@@ -860,7 +917,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
                           const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C) {
   SparseDev d;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
-  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
+  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
   d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C;
   return d;
 }
@@ -883,9 +940,10 @@ void SparseCircuit::run_forward(const BatchRef& b) {
   SparseDev d = SPARSE_DEV(b.batch, Bp, xb);
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
-    if (Bp >= 64 * kSparseEx)
-      hipLaunchKernelGGL(sparse_forward_kernel<kSparseEx>, dim3(cnt, ceil_div(Bp, 64 * kSparseEx)), dim3(64), 0, stream, d, n0);
-    else hipLaunchKernelGGL(sparse_forward_kernel<1>, dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
+    if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
+      hipLaunchKernelGGL((sparse_forward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, d, n0);
+    else
+      hipLaunchKernelGGL((sparse_forward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
   }
   check_launch("sparse_forward");
   last_batch_ = b.batch;
@@ -921,16 +979,22 @@ void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mas
                      d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
   SparseDev d = SPARSE_DEV(b.batch, Bp, d_visit_.p);
   SparseDev db = d;
+  if (ne) {
+    d_in_logp_.ensure(d_in_rec_.n);
+    hipLaunchKernelGGL(sparse_gather_in_logp_kernel, dim3(ceil_div((int64_t)d_in_rec_.n, 256)), dim3(256), 0, stream,
+                       d_in_rec_.p, d_logp_.p, (int64_t)d_in_rec_.n, d_in_logp_.p);
+    db.in_logp = d_in_logp_.p;
+  }
   db.order = d_bwd_order_.p;   // the layers without the input nodes whose rows other nodes write
   for (int l = n_layers_ - 1; l >= 0; --l) {
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     if (cnt == 0) continue;
-    if (Bp >= 64 * kSparseEx)
-      hipLaunchKernelGGL(sparse_backward_kernel<kSparseEx>, dim3(cnt, ceil_div(Bp, 64 * kSparseEx)), dim3(64), 0, stream, db, n0,
+    if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
+      hipLaunchKernelGGL((sparse_backward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, db, n0,
                          d_heads_.p, d_head_mask, d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
     else
-      hipLaunchKernelGGL(sparse_backward_kernel<1>, dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p, d_head_mask,
-                         d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
+      hipLaunchKernelGGL((sparse_backward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
+                         d_head_mask, d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
   }
   if (!fc_.input_nodes.empty()) {
     if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);

@@ -89,6 +89,7 @@ class SparseCircuit : public pcm_circuit {
   // incoming edges per node (down direction)
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
   DevBuf<int4> d_in_rec_;
+  DevBuf<float> d_in_logp_;
   DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
