@@ -184,6 +184,25 @@ def secondary(args):
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
                                "sample": t_samp * 1e3})
+    elif args.workload == "chow_liu_c3":
+        cfg = workloads.make_config("c3_hclt3072_k32")
+        V, C, B = cfg["V"], cfg["C"], cfg["B"]
+        d = torch.from_numpy(cfg["data"]).cuda()
+        P.pairwise_MI(d[:, :64], C, 0.1)
+        t_mi = _timed(torch, lambda: P.pairwise_MI(d, C, 0.1), max(1, args.steps // 4), 1)
+        mi = P.pairwise_MI(d, C, 0.1).cpu().numpy()
+        t0 = time.perf_counter()
+        parent = P.chow_liu_tree(mi)
+        t_tree = time.perf_counter() - t0
+        pairs = V * (V + 1) // 2
+        dt = t_mi
+        algo = pairs * 2 * B                                            # two rows of categories per pair (L2-served)
+        out["dtype"] = "u16 counts, f64 sums"
+        out.update(metric="variable pairs/sec, pairwise mutual information of 4096 x 3072 uint8 data, 256 categories",
+                   value=pairs / t_mi, unit="pairs/s",
+                   config={"workload": args.workload, "num_vars": V, "categories": C, "examples": B},
+                   structure_ms={"pairwise_mi": t_mi * 1e3, "spanning_tree_host": t_tree * 1e3},
+                   tree={"depth": workloads.tree_stats(parent)["depth"]})
     else:
         print(f"unknown workload {args.workload}", file=sys.stderr)
         sys.exit(2)

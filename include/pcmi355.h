@@ -201,6 +201,24 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
                     float* d_out);
 
 /*
+ * Structure learning, the step before pcm_hclt_create: what `hclt(data, num_hidden_cats; pseudocount)`
+ * (src/structures/hclts.jl:7-24) obtains from `learn_chow_liu_tree` and `clt_edges2graphs`.
+ *
+ * pcm_pairwise_mi: `pairwise_MI_chunked` (src/utils/information.jl:97-141 with the marginals of
+ * :43-95): mutual information of every pair of variables of a device-resident uint8 data set
+ * (element strides as in pcm_loglikelihoods, at most 65535 examples), counts smoothed with
+ * pseudocount/C per category and pseudocount/C^2 per cell.  d_mi: device, [num_vars][num_vars],
+ * symmetric, diagonal included.  Synchronous on `stream` (NULL: the default stream).
+ *
+ * pcm_chow_liu_tree: host matrix [num_vars][num_vars] -> maximum spanning tree (ties: lowest
+ * index), directed away from the lowest-numbered centre of the tree; clt_parent[v] = parent
+ * of v, -1 at the root: the argument of pcm_hclt_create.
+ */
+int pcm_pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
+                    int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream);
+int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent);
+
+/*
  * Adam ascent step on the sum parameters followed by per-sum-node normalisation
  * (src/sgd/adam.jl:63-86, :88-127, :318-319).  d_grad, d_params (unnormalised
  * log-parameters), d_m, d_v are device vectors in parameter-vector order over the sum

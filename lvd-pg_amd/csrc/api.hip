@@ -185,6 +185,18 @@ int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d
   return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });
 }
 
+int pcm_pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
+                    int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream) {
+  return guarded([&] {
+    pcm::pairwise_mi(d_data, stride_ex, stride_var, num_examples, num_vars, num_cats, pseudocount, d_mi,
+                     static_cast<hipStream_t>(stream));
+  });
+}
+
+int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent) {
+  return guarded([&] { pcm::chow_liu_tree(mi, num_vars, clt_parent); });
+}
+
 int pcm_set_timing(pcm_circuit* c, int32_t on) {
   return guarded([&] { need_hclt(c)->timing = on != 0; });
 }

@@ -1,0 +1,235 @@
+// Chow-Liu structure learning: pairwise mutual information of categorical data on the device,
+// maximum spanning tree and rooting on the host.
+//
+// Reference: src/utils/information.jl:3-95 (pairwise and single marginals with a pseudocount
+// spread as pc/C per category and pc/C^2 per cell, normalised by Z = N + pc) and :97-141
+//   MI[u,v] = sum_{a,b} ( xlogx(P_uv[a,b]) - xlogy(P_uv[a,b], P_u[a] * P_v[b]) ).
+// The tree is what src/structures/hclts.jl:17-18 asks ChowLiuTrees.jl / ProbabilisticCircuits.jl
+// for: a maximum spanning tree of MI, directed away from the centre of the tree.
+//
+// The reference fills a dense [V][V][C][C] table with float atomics and reduces it on the host.
+// Here a pair never leaves the workgroup.  With c(a,b) the count of a cell, s = pc/C^2,
+// p(c) = (c + s)/Z, la[u][a] = log P_u[a]:
+//   MI[u,v] = sum over examples e of f(c(cell of e))  -  M_u - M_v  +  C^2 * xlogx(p(0))  -  p(0) * C * (L_u + L_v)
+//   f(c) = (xlogx(p(c)) - xlogx(p(0))) / c,   M_u = (1/Z) sum_e la[u][x_eu],   L_u = sum_a la[u][a]
+// (each non-empty cell's term is shared out among its c examples; the empty cells' terms are the
+// closed-form remainder), so a pair costs three passes over its N examples against a C x C table
+// of 16-bit counters in LDS -- count, look up f, clear -- and no pass over the table itself.
+#include "common.hpp"
+#include "stage_kernel.hip.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <queue>
+
+namespace pcm {
+
+static void check_launch_c(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
+}
+
+// Single marginals of one variable per workgroup:
+//   la[v][a] = log((count + pc/C)/Z),  stat[v] = {M_v, L_v}
+__global__ __launch_bounds__(256) void mi_single_kernel(const uint8_t* __restrict__ xb, int N, int Np, int C, float pc,
+                                                        float* __restrict__ la, double* __restrict__ stat) {
+  __shared__ unsigned cnt[256];
+  __shared__ double red[256];
+  const int v = blockIdx.x, t = threadIdx.x;
+  cnt[t] = 0u;
+  __syncthreads();
+  const uint8_t* row = xb + (size_t)v * Np;
+  for (int b = t; b < N; b += 256) atomicAdd(&cnt[row[b]], 1u);
+  __syncthreads();
+  const double Z = (double)N + (double)pc;
+  double l = 0.0, m = 0.0;
+  if (t < C) {
+    const double p = ((double)cnt[t] + (double)pc / C) / Z;
+    const double lg = p > 0.0 ? log(p) : -INFINITY;
+    la[(size_t)v * C + t] = (float)lg;
+    l = lg;                                        // -inf if a category is empty and pc = 0: only used with pc > 0
+    m = cnt[t] ? (double)cnt[t] * lg / Z : 0.0;
+  }
+  red[t] = m;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) { if (t < o) red[t] += red[t + o]; __syncthreads(); }
+  const double M = red[0];
+  __syncthreads();
+  red[t] = l;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) { if (t < o) red[t] += red[t + o]; __syncthreads(); }
+  if (t == 0) { stat[2 * v] = M; stat[2 * v + 1] = red[0]; }
+}
+
+// f(c) for c = 0 .. N (f(0) unused).
+__global__ void mi_table_kernel(int N, int C, float pc, double* __restrict__ f) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  if (c > N) return;
+  const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
+  const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
+  const double p = ((double)c + s) / Z;
+  f[c] = c ? (p * log(p) - x0) / (double)c : 0.0;
+}
+
+constexpr int kMiThreads = 1024;
+
+// Pairs (u <= v) in row-major order of the upper triangle, dealt round-robin to persistent
+// workgroups.  Thread t owns examples 4t .. 4t+3 (+ 4096 per further round).
+__global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int Np, int V, int C,
+                                                             float pc, const double* __restrict__ f,
+                                                             const double* __restrict__ stat, float* __restrict__ mi) {
+  extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 doubles
+  const int t = threadIdx.x;
+  const int words = (C * C + 1) / 2;
+  double* red = reinterpret_cast<double*>(cells + ((words + 1) & ~1));
+  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;
+  __syncthreads();
+  const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
+  const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
+  const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
+  // row u of the triangle starts at pair u*V - u*(u-1)/2
+  int u = 0;
+  int64_t row0 = 0;
+  for (int64_t p = blockIdx.x; p < n_pairs; p += gridDim.x) {
+    while (p >= row0 + (V - u)) { row0 += V - u; ++u; }
+    const int v = u + (int)(p - row0);
+    const uint8_t* xu = xb + (size_t)u * Np;
+    const uint8_t* xv = xb + (size_t)v * Np;
+    double acc = 0.0;
+    // the three passes keep their keys in registers when the batch fits one round
+    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
+      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (b4 + i < N) {
+          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
+          atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
+        }
+    }
+    __syncthreads();
+    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
+      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (b4 + i < N) {
+          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
+          acc += f[(cells[key >> 1] >> (16 * (key & 1))) & 0xffffu];
+        }
+    }
+    __syncthreads();
+    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
+      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (b4 + i < N) {
+          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
+          cells[key >> 1] = 0u;
+        }
+    }
+    // sum over the workgroup
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+    if ((t & 63) == 0) red[t >> 6] = acc;
+    __syncthreads();
+    if (t == 0) {
+      double tot = 0.0;
+      for (int w = 0; w < kMiThreads / 64; ++w) tot += red[w];
+      double val = tot - stat[2 * u] - stat[2 * v] + (double)C * C * x0;
+      if (p0 > 0.0) val -= p0 * C * (stat[2 * u + 1] + stat[2 * v + 1]);
+      mi[(size_t)u * V + v] = (float)val;
+      mi[(size_t)v * V + u] = (float)val;
+    }
+    __syncthreads();
+  }
+}
+
+void pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t n_examples, int num_vars,
+                 int num_cats, float pseudocount, float* d_mi, hipStream_t stream) {
+  if (!d_data || !d_mi) fail(PCM_ERR_ARG, "data or output pointer is null");
+  if (n_examples < 1 || n_examples > 65535)
+    fail(PCM_ERR_UNSUPPORTED, "pairwise MI counts cells in 16 bits: 1..65535 examples per call, got %lld", (long long)n_examples);
+  if (num_vars < 1) fail(PCM_ERR_SHAPE, "num_vars must be positive, got %d", num_vars);
+  if (num_cats < 1 || num_cats > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", num_cats);
+  if (pseudocount < 0.f) fail(PCM_ERR_ARG, "pseudocount must not be negative");
+  const int N = (int)n_examples, Np = ceil_div(N, 64) * 64, V = num_vars, C = num_cats;
+  DevBuf<uint8_t> xb;
+  DevBuf<float> la;
+  DevBuf<double> stat, f;
+  xb.alloc((size_t)V * Np);
+  la.alloc((size_t)V * C);
+  stat.alloc((size_t)2 * V);
+  f.alloc((size_t)N + 1);
+  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Np, 64), ceil_div(V, 64)), dim3(256), 0, stream, d_data, stride_ex,
+                     stride_var, (const int32_t*)nullptr, N, Np, V, C, xb.p);
+  hipLaunchKernelGGL(mi_single_kernel, dim3(V), dim3(256), 0, stream, xb.p, N, Np, C, pseudocount, la.p, stat.p);
+  hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div(N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, f.p);
+  const int words = (C * C + 1) / 2;
+  const size_t lds = ((size_t)((words + 1) & ~1)) * 4 + (kMiThreads / 64) * sizeof(double);
+  int dev = 0, cus = 0, max_lds = 0;
+  PCM_HIP(hipGetDevice(&dev));
+  PCM_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  PCM_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+  if (lds > (size_t)max_lds) fail(PCM_ERR_UNSUPPORTED, "pair table needs %zu bytes of LDS, device offers %d", lds, max_lds);
+  PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)lds));
+  const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
+  const int per_cu = std::max<int>(1, (int)(std::min<size_t>((size_t)max_lds, 160 * 1024) / lds));
+  const int grid = (int)std::min<int64_t>(n_pairs, (int64_t)cus * std::min(per_cu, 2));
+  hipLaunchKernelGGL(mi_pair_kernel, dim3(grid), dim3(kMiThreads), lds, stream, xb.p, N, Np, V, C, pseudocount, f.p, stat.p,
+                     d_mi);
+  check_launch_c("pairwise_mi");
+  PCM_HIP(hipStreamSynchronize(stream));   // the scratch arrays die with this call
+}
+
+// Maximum spanning tree of a dense symmetric weight matrix (Prim; among equal weights the
+// lowest vertex index wins), rooted at the lowest-numbered centre of the tree (the vertex of
+// least eccentricity), as a parent array with -1 at the root.
+void chow_liu_tree(const float* mi, int V, int32_t* parent_out) {
+  if (!mi || !parent_out) fail(PCM_ERR_ARG, "matrix or output pointer is null");
+  if (V < 1) fail(PCM_ERR_SHAPE, "num_vars must be positive, got %d", V);
+  std::vector<float> best(V, -INFINITY);
+  std::vector<int32_t> link(V, -1);
+  std::vector<char> in(V, 0);
+  std::vector<std::vector<int32_t>> adj(V);
+  in[0] = 1;
+  for (int v = 1; v < V; ++v) { best[v] = mi[v]; link[v] = 0; }
+  for (int it = 1; it < V; ++it) {
+    int pick = -1;
+    for (int v = 0; v < V; ++v)
+      if (!in[v] && (pick < 0 || best[v] > best[pick])) pick = v;
+    if (!(best[pick] > -INFINITY)) fail(PCM_ERR_ARG, "mutual information matrix holds NaN or -inf in row %d", pick);
+    in[pick] = 1;
+    adj[pick].push_back(link[pick]);
+    adj[link[pick]].push_back(pick);
+    const float* row = mi + (size_t)pick * V;
+    for (int v = 0; v < V; ++v)
+      if (!in[v] && row[v] > best[v]) { best[v] = row[v]; link[v] = pick; }
+  }
+  for (auto& a : adj) std::sort(a.begin(), a.end());
+  // centre: peel leaves layer by layer; the last one or two vertices are the centres
+  std::vector<int> deg(V);
+  std::vector<int32_t> layer, next;
+  int left = V;
+  for (int v = 0; v < V; ++v) { deg[v] = (int)adj[v].size(); if (deg[v] <= 1) layer.push_back(v); }
+  while (left > 2) {
+    left -= (int)layer.size();
+    next.clear();
+    for (int32_t v : layer)
+      for (int32_t w : adj[v])
+        if (--deg[w] == 1) next.push_back(w);
+    layer.swap(next);
+  }
+  const int root = *std::min_element(layer.begin(), layer.end());
+  std::fill(parent_out, parent_out + V, -2);
+  std::queue<int32_t> q;
+  parent_out[root] = -1;
+  q.push(root);
+  while (!q.empty()) {
+    const int32_t v = q.front();
+    q.pop();
+    for (int32_t w : adj[v])
+      if (parent_out[w] == -2) { parent_out[w] = v; q.push(w); }
+  }
+}
+
+}  // namespace pcm

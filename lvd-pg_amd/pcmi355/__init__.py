@@ -9,4 +9,5 @@ from .circuits import BitsCircuit, HcltCircuit, hclt_from_clt, compile_circuit, 
 from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample)
+from .structures import pairwise_MI, chow_liu_tree, learn_chow_liu_tree, hclt  # noqa: F401
 from ._lib import PcmError, LIB_PATH  # noqa: F401

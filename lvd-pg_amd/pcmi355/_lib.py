@@ -3,6 +3,8 @@ import fails with the command that builds it."""
 import ctypes
 import os
 
+import torch  # noqa: F401  -- first, so that the library binds to the HIP runtime torch has loaded (one runtime per process)
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(_HERE), "libpcmi355.so")
 
@@ -45,6 +47,8 @@ _SIGS = {
     "pcm_sample": [H, vp, vp, c_i32, vp],
     "pcm_sample_soft": [H, vp, ctypes.c_float, c_i32, vp],
     "pcm_adam_step": [H, vp, vp, vp, vp, c_f32, c_f32, c_f32, c_f32, c_i32],
+    "pcm_pairwise_mi": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],
+    "pcm_chow_liu_tree": [vp, c_i32, vp],
     "pcm_set_timing": [H, c_i32],
     "pcm_get_timing": [H, vp, c_i32],
 }
