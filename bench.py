@@ -184,6 +184,28 @@ def secondary(args):
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
                                "sample": t_samp * 1e3})
+    elif args.workload == "c4_top_soft":
+        # the top-level circuit of C4: 64 patch variables, 128 cluster categories, K = 64, trained on soft evidence
+        V, K, C, B = 64, 64, 128, 1024
+        data = workloads.grf_images(B, 8, 8, 1, 3.0, 0.8, seed=1005)
+        parent = workloads.chow_liu_parent(data)
+        theta, leaf = workloads.init_params(parent, K, C, 1105, kind="dirichlet")
+        bpc = P.hclt_from_clt(parent, C, K)
+        bpc.set_params(theta, leaf)
+        ev = torch.from_numpy((rng.normal(-600, 30, (B, V, 1)) + rng.gumbel(0, 8, (B, V, C))).astype(np.float32)).cuda()
+        ll = torch.empty(B, device="cuda")
+
+        def step():
+            check(lib.pcm_flows_soft(bpc.handle, ev.data_ptr(), ev.stride(0), ev.stride(1), ev.stride(2), None, B, 0.0, None,
+                                     ll.data_ptr()))
+            check(lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+        dt = _timed(torch, step, args.steps, args.warmup)
+        nn, ne = bpc.num_nodes(), bpc.num_edges()
+        algo = B * (8 * nn + 24 * ne) + 2 * 4 * B * V * C * K       # + the evidence, read once per input node going up and down
+        out.update(metric="examples/sec fwd+bwd+EM on soft evidence, 64-var HCLT K=64, 128 categories (layered engine)",
+                   value=B / dt, unit="examples/s",
+                   config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
+                           "nodes": nn, "edges": ne})
     elif args.workload == "chow_liu_c3":
         cfg = workloads.make_config("c3_hclt3072_k32")
         V, C, B = cfg["V"], cfg["C"], cfg["B"]

@@ -201,6 +201,22 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
                     float* d_out);
 
 /*
+ * Soft evidence: the same two queries with a three-dimensional data argument, as the reference
+ * dispatches on `data isa CuArray{Float32,3}` (`init_mar!_with_reg_cat_kernel`
+ * src/regularization/reg_likelihood.jl:51-91, `input_flows_circuit_with_reg_cat_kernel`
+ * src/regularization/reg_flow.jl:50-82; the top-level circuits of
+ * exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl are trained on per-cluster patch
+ * log-likelihoods this way).  d_evidence[row * stride_ex + var * stride_var + cat * stride_cat]
+ * is the log-evidence of category `cat` (element strides; Julia's [N, V, C] array: 1, N, N*V).
+ * A leaf's value is logsumexp_c(evidence_c + logp_c) and its flow is shared among the categories
+ * in proportion to exp(evidence_c + logp_c - value).  pcm_em_update afterwards as usual.
+ */
+int pcm_loglikelihoods_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var,
+                            int64_t stride_cat, const int32_t* d_example_ids, int32_t batch, float* d_ll);
+int pcm_flows_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var, int64_t stride_cat,
+                   const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask, float* d_ll);
+
+/*
  * Structure learning, the step before pcm_hclt_create: what `hclt(data, num_hidden_cats; pseudocount)`
  * (src/structures/hclts.jl:7-24) obtains from `learn_chow_liu_tree` and `clt_edges2graphs`.
  *

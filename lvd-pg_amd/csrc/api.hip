@@ -185,6 +185,21 @@ int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d
   return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });
 }
 
+int pcm_loglikelihoods_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var,
+                            int64_t stride_cat, const int32_t* d_example_ids, int32_t batch, float* d_ll) {
+  return guarded([&] {
+    need(c)->loglikelihoods_soft(pcm::SoftRef{d_evidence, stride_ex, stride_var, stride_cat, d_example_ids, batch}, d_ll);
+  });
+}
+
+int pcm_flows_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var, int64_t stride_cat,
+                   const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask, float* d_ll) {
+  return guarded([&] {
+    need(c)->flows_soft(pcm::SoftRef{d_evidence, stride_ex, stride_var, stride_cat, d_example_ids, batch}, rate,
+                        d_head_mask, d_ll);
+  });
+}
+
 int pcm_pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
                     int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream) {
   return guarded([&] {

@@ -73,6 +73,14 @@ struct DevBuf {
   }
 };
 
+// A batch of soft evidence: log-evidence per (example, variable, category) with element strides.
+struct SoftRef {
+  const float* d_ev;
+  int64_t stride_ex, stride_var, stride_cat;
+  const int32_t* d_idx;
+  int32_t batch;
+};
+
 inline int ceil_div(int64_t a, int64_t b) { return (int)((a + b - 1) / b); }
 
 struct BatchRef {
@@ -99,6 +107,8 @@ struct pcm_circuit {
   virtual void update_parameters(const float* in, int64_t n) = 0;
   virtual void loglikelihoods(const pcm::BatchRef& b, float* d_ll) = 0;
   virtual void flows(const pcm::BatchRef& b, float rate, const float* d_head_mask, float* d_ll) = 0;
+  virtual void loglikelihoods_soft(const pcm::SoftRef& s, float* d_ll) = 0;
+  virtual void flows_soft(const pcm::SoftRef& s, float rate, const float* d_head_mask, float* d_ll) = 0;
   virtual void em_update(float pseudocount, float inertia) = 0;
   virtual void kld(pcm_circuit* q, float* out) = 0;
   virtual void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) = 0;

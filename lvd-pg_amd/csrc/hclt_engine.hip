@@ -698,7 +698,7 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   const int K = K_, C = C_;
   std::vector<float> h;
-  if (!block_ && !wide_) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
+  if (flows_in_general_ || (!block_ && !wide_)) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
     std::vector<float> ea((size_t)n_edges_), lf((size_t)V_ * K * C);
     general_->get_aggregates(ea.data(), n_edges_, lf.data(), (int64_t)lf.size());
     if (edge_aggr) {
@@ -928,9 +928,25 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   run_forward(dev(b.batch), d_ll);
 }
 
+// Soft evidence (src/regularization/reg_likelihood.jl:51-91, reg_flow.jl:50-82) runs on the layered
+// engine over the circuit's general form for every hidden size.
+void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) { general()->loglikelihoods_soft(s, d_ll); }
+
+void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
+  if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (have_flows_ && !flows_in_general_ && rate != 0.f && (block_ || wide_))
+    fail(PCM_ERR_STATE, "flow memory cannot carry over from categorical batches to soft-evidence batches");
+  general()->flows_soft(s, rate, nullptr, d_ll);
+  have_flows_ = true;
+  flows_in_general_ = true;
+}
+
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (flows_in_general_ && rate != 0.f && (block_ || wide_))
+    fail(PCM_ERR_STATE, "flow memory cannot carry over from soft-evidence batches to categorical batches");
+  flows_in_general_ = false;
   if (!block_ && !wide_) {
     general()->flows(b, rate, nullptr, d_ll);
     have_flows_ = true;
@@ -980,7 +996,7 @@ void HcltCircuit::read_timing(float* ms, int n) {
 
 void HcltCircuit::em_update(float pseudocount, float inertia) {
   if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
-  if (!block_ && !wide_) {
+  if (flows_in_general_ || (!block_ && !wide_)) {
     general_->em_update(pseudocount, inertia);
     PCM_HIP(hipStreamSynchronize(stream));
     pull_from_general();

@@ -127,6 +127,8 @@ class HcltCircuit : public pcm_circuit {
   void update_parameters(const float* in, int64_t n) override;
   void loglikelihoods(const BatchRef& b, float* d_ll) override;
   void flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) override;
+  void loglikelihoods_soft(const SoftRef& s, float* d_ll) override;
+  void flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) override;
   void em_update(float pseudocount, float inertia) override;
   void kld(pcm_circuit* q, float* out) override;
   void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
@@ -183,6 +185,7 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int64_t> d_sum_param_src_;
   int cap_slices_ = 0;
   bool have_flows_ = false;
+  bool flows_in_general_ = false;   // the last flows were computed by the layered engine (soft evidence)
   std::vector<hipEvent_t> ev_;   // kTimingRing sets of 4 events
   int n_timed_ = 0;
   hipEvent_t* ev_set();

@@ -194,6 +194,9 @@ struct SparseDev {
   const float* logp;
   const float* leaf;
   const uint8_t* xb;         // [V][Bp]
+  const float* ev;           // soft evidence instead of xb (else null): log-evidence of (example, variable, category)
+  int64_t ev_se, ev_sv, ev_sc;   // ... at ev[row * ev_se + var * ev_sv + cat * ev_sc], row = ev_idx ? ev_idx[b] : b
+  const int32_t* ev_idx;
   float* mars;               // [n_nodes][Bp]
   float* flows;
   int32_t B, Bp, C;
@@ -270,9 +273,27 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
   float m[EX], sum[EX];
   if (d.type[n] == kInput) {
     if (wave) return;
-    const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
+    if (d.ev) {
+      // soft evidence, src/regularization/reg_likelihood.jl:51-91: logsumexp_c(evidence_c + logp_c)
+      const float* lp = d.leaf + d.in_off[n];
 #pragma unroll
-    for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
+      for (int x = 0; x < EX; ++x) {
+        const int b = min(bb[x], d.B - 1);
+        const float* e = d.ev + (int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + (int64_t)d.in_var[n] * d.ev_sv;
+        float mm = -INFINITY, ss = 0.f;
+        for (int c = 0; c < d.C; ++c) {
+          const float t = e[(int64_t)c * d.ev_sc] + lp[c];
+          if (t > mm) { ss = ss * __expf(mm - t) + 1.f; mm = t; }
+          else if (t != -INFINITY) ss += __expf(t - mm);
+        }
+        m[x] = mm == -INFINITY ? mm : mm + __logf(ss);
+        sum[x] = 1.f;
+      }
+    } else {
+      const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
+#pragma unroll
+      for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
+    }
   } else {
     // the node's edges in kLayerWaves contiguous shares, one per wave; a share is folded as a
     // running maximum and a sum of exponentials (products: a plain sum), the shares are then
@@ -462,6 +483,39 @@ __global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, cons
   __syncthreads();
   float* dst = leaf_flow + d.in_off[n];
   for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += hist[c];
+}
+
+// The same with soft evidence, src/regularization/reg_flow.jl:50-82: category c of input node n
+// receives sum_b flow[b] * exp(evidence[b][c] + logp_c - value[b]).  Thread = category, the
+// node's values and flows of the batch staged in LDS.
+__global__ __launch_bounds__(256) void sparse_leaf_flow_soft_kernel(SparseDev d, const int32_t* __restrict__ input_nodes,
+                                                                    float* __restrict__ leaf_flow) {
+  extern __shared__ float vf[];   // [2][chunk]
+  constexpr int kChunk = 2048;
+  const int n = input_nodes[blockIdx.x];
+  const float* lp = d.leaf + d.in_off[n];
+  const int64_t voff = (int64_t)d.in_var[n] * d.ev_sv;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};   // categories threadIdx.x + 256 * i (at most 256 categories: one per thread)
+  for (int b0 = 0; b0 < d.B; b0 += kChunk) {
+    const int nb = min(kChunk, d.B - b0);
+    __syncthreads();
+    for (int i = threadIdx.x; i < nb; i += blockDim.x) {
+      vf[i] = d.mars[(size_t)n * d.Bp + b0 + i];
+      vf[kChunk + i] = d.flows[(size_t)n * d.Bp + b0 + i];
+    }
+    __syncthreads();
+    for (int c = threadIdx.x, q = 0; c < d.C; c += blockDim.x, ++q) {
+      float a = 0.f;
+      for (int i = 0; i < nb; ++i) {
+        const int b = b0 + i;
+        const float t = d.ev[(int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + voff + (int64_t)c * d.ev_sc] + lp[c];
+        if (t != -INFINITY && vf[kChunk + i] != 0.f) a += __expf(t - vf[i]) * vf[kChunk + i];
+      }
+      acc[q & 3] += a;
+    }
+  }
+  float* dst = leaf_flow + d.in_off[n];
+  for (int c = threadIdx.x, q = 0; c < d.C; c += blockDim.x, ++q) dst[c] += acc[q & 3];
 }
 
 __global__ void sparse_gather_in_logp_kernel(const int4* __restrict__ in_rec, const float* __restrict__ logp, int64_t n,
@@ -917,7 +971,8 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
                           const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C) {
   SparseDev d;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
-  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off; d.logp = logp; d.leaf = leaf;
+  d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off;
+  d.ev = nullptr; d.ev_se = d.ev_sv = d.ev_sc = 0; d.ev_idx = nullptr; d.logp = logp; d.leaf = leaf;
   d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C;
   return d;
 }
@@ -926,18 +981,22 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
   make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
            d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
 
-void SparseCircuit::run_forward(const BatchRef& b) {
-  if (!b.d_data) fail(PCM_ERR_ARG, "data pointer is null");
-  if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
-  ensure_batch(b.batch);
-  const int Bp = ceil_div(b.batch, 64) * 64;
-  // staged categories live at the head of the flows buffer's tail: use a dedicated buffer
+void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
+  const int batch = b ? b->batch : s->batch;
+  if (b ? !b->d_data : !s->d_ev) fail(PCM_ERR_ARG, "data pointer is null");
+  if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  ensure_batch(batch);
+  const int Bp = ceil_div(batch, 64) * 64;
+  // the staged categories live in a dedicated buffer
   d_visit_.ensure((size_t)std::max<int64_t>((int64_t)fc_.num_vars, fc_.n_nodes()) * Bp);
   uint8_t* xb = d_visit_.p;
-  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(fc_.num_vars, 64)), dim3(256), 0, stream,
-                     b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, fc_.num_vars, fc_.num_cats, xb);
-  check_launch("stage_batch");
-  SparseDev d = SPARSE_DEV(b.batch, Bp, xb);
+  if (b) {
+    hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(fc_.num_vars, 64)), dim3(256), 0, stream,
+                       b->d_data, b->stride_ex, b->stride_var, b->d_idx, batch, Bp, fc_.num_vars, fc_.num_cats, xb);
+    check_launch("stage_batch");
+  }
+  SparseDev d = SPARSE_DEV(batch, Bp, xb);
+  if (s) { d.ev = s->d_ev; d.ev_se = s->stride_ex; d.ev_sv = s->stride_var; d.ev_sc = s->stride_cat; d.ev_idx = s->d_idx; }
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
     if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
@@ -946,38 +1005,61 @@ void SparseCircuit::run_forward(const BatchRef& b) {
       hipLaunchKernelGGL((sparse_forward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
   }
   check_launch("sparse_forward");
-  last_batch_ = b.batch;
+  last_batch_ = batch;
 }
 
-void SparseCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
-  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  run_forward(b);
-  const int Bp = ceil_div(b.batch, 64) * 64;
-  // root (or head) rows -> output; the root is the last node
+// root (or head) rows -> output; the root is the last node
+void SparseCircuit::write_ll(int batch, float* d_ll) {
+  const int Bp = ceil_div(batch, 64) * 64;
   if (fc_.heads.empty()) {
-    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)b.batch * sizeof(float),
+    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)batch * sizeof(float),
                            hipMemcpyDeviceToDevice, stream));
   } else {
     DevBuf<int32_t> hn;
     hn.upload(fc_.heads, stream);
-    hipLaunchKernelGGL(sparse_copy_rows_kernel, dim3(ceil_div(b.batch, 256), (int)fc_.heads.size()), dim3(256), 0, stream,
-                       d_mars_.p, Bp, b.batch, hn.p, (int)fc_.heads.size(), d_ll);
+    hipLaunchKernelGGL(sparse_copy_rows_kernel, dim3(ceil_div(batch, 256), (int)fc_.heads.size()), dim3(256), 0, stream,
+                       d_mars_.p, Bp, batch, hn.p, (int)fc_.heads.size(), d_ll);
     check_launch("copy_rows");
     PCM_HIP(hipStreamSynchronize(stream));
   }
+}
+
+void SparseCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  run_forward(&b, nullptr);
+  write_ll(b.batch, d_ll);
+}
+
+void SparseCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  run_forward(nullptr, &s);
+  write_ll(s.batch, d_ll);
 }
 
 void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (fc_.heads.empty() && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!fc_.heads.empty() && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
-  run_forward(b);
-  const int Bp = ceil_div(b.batch, 64) * 64;
+  run_forward(&b, nullptr);
+  run_flows(b.batch, nullptr, rate, d_head_mask, d_ll);
+}
+
+void SparseCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (fc_.heads.empty() && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (!fc_.heads.empty() && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
+  run_forward(nullptr, &s);
+  run_flows(s.batch, &s, rate, d_head_mask, d_ll);
+}
+
+void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll) {
+  const int Bp = ceil_div(batch, 64) * 64;
   const int64_t ne = fc_.n_edges();
   hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div(std::max<int64_t>(ne, 1), 256)), dim3(256), 0, stream, d_edge_aggr_.p, ne, rate);
   hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)fc_.leaf_logp.size(), 256)), dim3(256), 0, stream,
                      d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
-  SparseDev d = SPARSE_DEV(b.batch, Bp, d_visit_.p);
+  SparseDev d = SPARSE_DEV(batch, Bp, d_visit_.p);
+  if (soft) { d.ev = soft->d_ev; d.ev_se = soft->stride_ex; d.ev_sv = soft->stride_var; d.ev_sc = soft->stride_cat; d.ev_idx = soft->d_idx; }
   SparseDev db = d;
   if (ne) {
     d_in_logp_.ensure(d_in_rec_.n);
@@ -998,17 +1080,21 @@ void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mas
   }
   if (!fc_.input_nodes.empty()) {
     if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);
-    hipLaunchKernelGGL(sparse_leaf_flow_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 0, stream, d,
-                       d_input_nodes_.p, d_leaf_flow_.p);
+    if (soft)
+      hipLaunchKernelGGL(sparse_leaf_flow_soft_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 2 * 2048 * sizeof(float),
+                         stream, d, d_input_nodes_.p, d_leaf_flow_.p);
+    else
+      hipLaunchKernelGGL(sparse_leaf_flow_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 0, stream, d,
+                         d_input_nodes_.p, d_leaf_flow_.p);
   }
   check_launch("sparse_backward");
   if (fc_.heads.empty()) {
-    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)b.batch * sizeof(float),
+    PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)batch * sizeof(float),
                            hipMemcpyDeviceToDevice, stream));
   } else {
     DevBuf<int32_t> hn;
     hn.upload(fc_.heads, stream);
-    hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(b.batch, 256)), dim3(256), 0, stream, d_mars_.p, Bp, b.batch,
+    hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(batch, 256)), dim3(256), 0, stream, d_mars_.p, Bp, batch,
                        hn.p, (int)fc_.heads.size(), d_head_mask, d_ll);
     check_launch("head_mixture");
     PCM_HIP(hipStreamSynchronize(stream));

@@ -51,6 +51,8 @@ class SparseCircuit : public pcm_circuit {
   void update_parameters(const float* in, int64_t n) override;
   void loglikelihoods(const BatchRef& b, float* d_ll) override;
   void flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) override;
+  void loglikelihoods_soft(const SoftRef& s, float* d_ll) override;
+  void flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) override;
   void em_update(float pseudocount, float inertia) override;
   void kld(pcm_circuit* q, float* out) override;
   void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
@@ -99,7 +101,9 @@ class SparseCircuit : public pcm_circuit {
   bool have_flows_ = false;
 
   void ensure_batch(int batch);
-  void run_forward(const BatchRef& b);
+  void run_forward(const BatchRef* b, const SoftRef* s);
+  void write_ll(int batch, float* d_ll);
+  void run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll);
 };
 
 }  // namespace pcm

@@ -47,6 +47,8 @@ _SIGS = {
     "pcm_sample": [H, vp, vp, c_i32, vp],
     "pcm_sample_soft": [H, vp, ctypes.c_float, c_i32, vp],
     "pcm_adam_step": [H, vp, vp, vp, vp, c_f32, c_f32, c_f32, c_f32, c_i32],
+    "pcm_loglikelihoods_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, vp],
+    "pcm_flows_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, c_f32, vp, vp],
     "pcm_pairwise_mi": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],
     "pcm_chow_liu_tree": [vp, c_i32, vp],
     "pcm_set_timing": [H, c_i32],

@@ -9,12 +9,37 @@ def _dev_ptr(t):
     return None if t is None else t.data_ptr()
 
 
+def _is_soft(data):
+    """The reference dispatches on `data isa CuArray{Float32,3}`: [examples, variables, categories] log-evidence."""
+    return isinstance(data, torch.Tensor) and data.dim() == 3
+
+
 def _check_data(bpc, data):
-    if not (isinstance(data, torch.Tensor) and data.is_cuda and data.dtype == torch.uint8 and data.dim() == 2):
+    if _is_soft(data):
+        if not (data.is_cuda and data.dtype == torch.float32):
+            raise ValueError("soft evidence must be a 3-D float32 tensor on the GPU (examples x variables x categories)")
+        if data.shape[2] != bpc.size("categories"):
+            raise ValueError(f"evidence has {data.shape[2]} categories, circuit has {bpc.size('categories')}")
+    elif not (isinstance(data, torch.Tensor) and data.is_cuda and data.dtype == torch.uint8 and data.dim() == 2):
         raise ValueError("data must be a 2-D uint8 tensor on the GPU (examples x variables)")
     nv = bpc.size("variables")
     if data.shape[1] != nv:
         raise ValueError(f"data has {data.shape[1]} variables, circuit has {nv}")
+
+
+def _forward(bpc, data, d_ptr, i_ptr, b, out_ptr):
+    if _is_soft(data):
+        check(lib.pcm_loglikelihoods_soft(bpc.handle, d_ptr, data.stride(0), data.stride(1), data.stride(2), i_ptr, b, out_ptr))
+    else:
+        check(lib.pcm_loglikelihoods(bpc.handle, d_ptr, data.stride(0), data.stride(1), i_ptr, b, out_ptr))
+
+
+def _flows(bpc, data, i_ptr, b, rate, hm_ptr, ll_ptr):
+    if _is_soft(data):
+        check(lib.pcm_flows_soft(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), data.stride(2), i_ptr, b,
+                                 float(rate), hm_ptr, ll_ptr))
+    else:
+        check(lib.pcm_flows(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), i_ptr, b, float(rate), hm_ptr, ll_ptr))
 
 
 def _ids(example_ids, device):
@@ -29,7 +54,8 @@ def loglikelihoods(bpc, data, batch_size=None, example_ids=None):
     """`loglikelihoods(bpc, data; batch_size)` / `loglikelihoods_probcat`
     (src/regularization/reg_likelihood.jl:139-162): per-example log-likelihoods as a device
     vector.  A multi-head circuit returns [num_examples, num_heads]
-    (src-jl/multi_head_pc/likelihood.jl:37-71 with head_mask = nothing)."""
+    (src-jl/multi_head_pc/likelihood.jl:37-71 with head_mask = nothing).  A 3-D float32 `data`
+    [examples, variables, categories] is soft evidence (reg_likelihood.jl:51-91)."""
     _check_data(bpc, data)
     ids = _ids(example_ids, data.device)
     n = data.shape[0] if ids is None else len(ids)
@@ -44,11 +70,10 @@ def loglikelihoods(bpc, data, batch_size=None, example_ids=None):
             d_ptr, i_ptr = data.data_ptr(), ids[s:s + b].data_ptr()
         if heads:
             tmp = torch.empty((heads, b), dtype=torch.float32, device=data.device)
-            check(lib.pcm_loglikelihoods(bpc.handle, d_ptr, data.stride(0), data.stride(1), i_ptr, b, tmp.data_ptr()))
+            _forward(bpc, data, d_ptr, i_ptr, b, tmp.data_ptr())
             out[:, s:s + b] = tmp
         else:
-            check(lib.pcm_loglikelihoods(bpc.handle, d_ptr, data.stride(0), data.stride(1), i_ptr, b,
-                                         out[0, s:s + b].data_ptr()))
+            _forward(bpc, data, d_ptr, i_ptr, b, out[0, s:s + b].data_ptr())
     return out.t().contiguous() if heads else out[0]
 
 
@@ -78,8 +103,7 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
         if ids is not None:
             hm = hm[ids.long()]
         hm = hm.t().contiguous()   # [heads, batch]
-    check(lib.pcm_flows(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), _dev_ptr(ids), b,
-                        float(rate), _dev_ptr(hm), ll.data_ptr()))
+    _flows(bpc, data, _dev_ptr(ids), b, rate, _dev_ptr(hm), ll.data_ptr())
     return ll
 
 
@@ -88,7 +112,8 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
                            shuffle="each_epoch", verbose=False, generator=None, head_mask=None):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
     of per-epoch mean log-likelihoods.  soft_reg and ent_reg must be 0 (the reference's
-    entropy regulariser is commented out at :294-296; soft evidence is not built)."""
+    entropy regulariser is commented out at :294-296).  `data` may be 3-D float32 soft evidence,
+    as for the top-level circuits of exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl."""
     if soft_reg != 0.0 or ent_reg != 0.0:
         raise NotImplementedError("soft_reg / ent_reg other than 0 are not supported")
     _check_data(bpc, data)
@@ -119,13 +144,12 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
                 do_shuffle()
             ids = perm[bi * batch_size:(bi + 1) * batch_size]
             rate = 0.0 if flow_memory == 0 else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
-            if hm_t is None:
+            if hm_t is None and not _is_soft(data):
                 check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
                                       batch_size, rate, float(pseudocount), float(param_inertia), ll.data_ptr()))
             else:
-                hm = hm_t[ids.long()].t().contiguous()
-                check(lib.pcm_flows(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
-                                    batch_size, rate, hm.data_ptr(), ll.data_ptr()))
+                hm = None if hm_t is None else hm_t[ids.long()].t().contiguous()
+                _flows(bpc, data, ids.data_ptr(), batch_size, rate, _dev_ptr(hm), ll.data_ptr())
                 check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
             acc += ll.sum(dtype=torch.float64)
         lls.append(float(acc.item()) / batch_size / num_batches)

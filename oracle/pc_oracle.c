@@ -179,6 +179,59 @@ void orc_input_flows(int n_nodes, const uint8_t* type, const int32_t* in_var,
 }
 
 /*
+ * Soft evidence: data is a [B][V][C] array of log-evidence instead of one category per variable.
+ *   leaf value : regularization/reg_likelihood.jl:51-91 -- logsumexp_c(data[b,v,c] + logp_c),
+ *                folded pairwise from -inf in category order
+ *   leaf flows : regularization/reg_flow.jl:50-82 -- counts[c] += exp(data[b,v,c] + logp_c - value) * flow
+ * Inner nodes are those of orc_forward / orc_backward.
+ */
+void orc_forward_soft(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
+                      const int32_t* prime, const int32_t* sub, const REAL* logp,
+                      const int32_t* in_var, const int64_t* in_off, int C, const REAL* leaf_logp,
+                      const REAL* ev, int64_t V, int B, REAL* mars) {
+#pragma omp parallel for schedule(static)
+  for (int b = 0; b < B; ++b) {
+    for (int n = 0; n < n_nodes; ++n) {
+      REAL* out = mars + (int64_t)n * B + b;
+      if (type[n] == NODE_INPUT) {
+        const REAL* e = ev + ((int64_t)b * V + in_var[n]) * C;
+        REAL acc = (REAL)-INFINITY;
+        for (int c = 0; c < C; ++c) acc = lse2f(acc, e[c] + leaf_logp[in_off[n] + c]);
+        *out = acc;
+        continue;
+      }
+      int issum = type[n] == NODE_SUM;
+      REAL acc = issum ? (REAL)-INFINITY : (REAL)0;
+      for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
+        REAL child = mars[(int64_t)prime[e] * B + b];
+        if (sub[e] >= 0) child += mars[(int64_t)sub[e] * B + b];
+        if (issum) child += logp[e];
+        if (e == edge_ptr[n]) acc = child;
+        else if (issum) acc = lse2f(acc, child);
+        else acc += child;
+      }
+      *out = acc;
+    }
+  }
+}
+
+void orc_input_flows_soft(int n_nodes, const uint8_t* type, const int32_t* in_var,
+                          const int64_t* in_off, int C, const REAL* leaf_logp, const REAL* ev,
+                          int64_t V, int B, const REAL* mars, const REAL* flows, REAL* leaf_flow) {
+  for (int n = 0; n < n_nodes; ++n) {
+    if (type[n] != NODE_INPUT) continue;
+    for (int b = 0; b < B; ++b) {
+      const REAL* e = ev + ((int64_t)b * V + in_var[n]) * C;
+      REAL value = mars[(int64_t)n * B + b], f = flows[(int64_t)n * B + b];
+      for (int c = 0; c < C; ++c) {
+        REAL t = e[c] + leaf_logp[in_off[n] + c];
+        if (t > (REAL)-INFINITY) leaf_flow[in_off[n] + c] += (REAL)exp((double)(t - value)) * f;
+      }
+    }
+  }
+}
+
+/*
  * Mini-batch EM parameter update, in the reference's call order
  * (regularization/reg_em.jl:292-299):
  *   add_pseudocount : edge_aggr[e] += pseudocount / #sum-edges(parent)

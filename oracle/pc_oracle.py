@@ -216,6 +216,33 @@ def input_flows(fc, data, flows, idx=None, leaf_flow=None, double=False):
     return leaf_flow
 
 
+def forward_soft(fc, ev, double=False):
+    """ev [B, V, C] log-evidence -> node values [n_nodes, B]."""
+    R = _real(double)
+    ev = np.ascontiguousarray(ev, dtype=R)
+    B, V, C = ev.shape
+    assert C == fc.C
+    mars = np.empty((fc.n_nodes, B), dtype=R)
+    lib(double).orc_forward_soft(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(fc.prime), _p(fc.sub),
+                                 _p(np.ascontiguousarray(fc.logp, dtype=R)), _p(fc.in_var), _p(fc.in_off),
+                                 ctypes.c_int(C), _p(np.ascontiguousarray(fc.leaf_logp, dtype=R)), _p(ev),
+                                 ctypes.c_int64(V), ctypes.c_int(B), _p(mars))
+    return mars
+
+
+def input_flows_soft(fc, ev, mars, flows, leaf_flow=None, double=False):
+    R = _real(double)
+    ev = np.ascontiguousarray(ev, dtype=R)
+    B, V, C = ev.shape
+    if leaf_flow is None:
+        leaf_flow = np.zeros(len(fc.leaf_logp), dtype=R)
+    lib(double).orc_input_flows_soft(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.in_var), _p(fc.in_off),
+                                     ctypes.c_int(C), _p(np.ascontiguousarray(fc.leaf_logp, dtype=R)), _p(ev),
+                                     ctypes.c_int64(V), ctypes.c_int(B), _p(np.ascontiguousarray(mars, R)),
+                                     _p(np.ascontiguousarray(flows, R)), _p(leaf_flow))
+    return leaf_flow
+
+
 def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False):
     """Updates fc.logp / fc.leaf_logp in place (float circuits only when double=False)."""
     R = _real(double)

@@ -1,0 +1,167 @@
+"""Soft evidence (3-D log-evidence data): the oracle against what the mathematics fixes (CPU),
+the HIP path against the oracle (GPU).
+Reference: src/regularization/reg_likelihood.jl:51-91, src/regularization/reg_flow.jl:50-82."""
+import itertools
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "oracle"))
+sys.path.insert(0, os.path.join(ROOT, "lvd-pg_amd"))
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+import pc_oracle as O  # noqa: E402
+from helpers import make_hclt, block_theta, random_dag, describe_dag  # noqa: E402
+
+
+def _one_hot_evidence(data, C):
+    ev = np.full(data.shape + (C,), -np.inf, np.float32)
+    np.put_along_axis(ev, data[..., None].astype(np.int64), 0.0, axis=2)
+    return ev
+
+
+# ---- the oracle, pinned ------------------------------------------------------------------
+
+def test_oracle_one_hot_evidence_is_hard_evidence():
+    parent, theta, leaf, fc = make_hclt(6, 3, 4, 5)
+    data = np.random.default_rng(0).integers(0, 4, (20, 6)).astype(np.uint8)
+    ev = _one_hot_evidence(data, 4)
+    m_hard = O.forward(fc, data, double=True)
+    m_soft = O.forward_soft(fc, ev, double=True)
+    assert np.allclose(m_soft, m_hard, rtol=0, atol=1e-12)
+    fl, _ = O.backward(fc, m_hard, double=True)
+    assert np.allclose(O.input_flows_soft(fc, ev, m_soft, fl, double=True), O.input_flows(fc, data, fl, double=True), atol=1e-12)
+
+
+def test_oracle_soft_likelihood_is_the_weighted_sum_over_assignments():
+    """LL_soft = log sum_x prod_v w[v, x_v] p(x): brute force over all assignments of a tiny circuit;
+    all-zero evidence marginalises every variable: LL = 0."""
+    V, C = 4, 3
+    parent, theta, leaf, fc = make_hclt(V, 2, C, 9)
+    rng = np.random.default_rng(1)
+    ev = rng.normal(0, 1, (3, V, C))
+    xs = np.array(list(itertools.product(range(C), repeat=V)), np.uint8)
+    logp = O.forward(fc, xs, double=True)[-1]
+    want = [np.log(np.sum(np.exp(logp + ev[b][np.arange(V), xs].sum(axis=1)))) for b in range(3)]
+    got = O.forward_soft(fc, ev, double=True)[-1]
+    assert np.allclose(got, want, atol=1e-10)
+    assert np.allclose(O.forward_soft(fc, np.zeros((2, V, C)), double=True)[-1], 0, atol=1e-6)   # parameters are normalised in float32
+
+
+def test_oracle_soft_leaf_flows_are_the_gradient_of_the_likelihood():
+    """d LL / d logp_leaf[c] = the soft count of category c (central differences, float64)."""
+    V, C = 4, 3
+    parent, theta, leaf, fc = make_hclt(V, 2, C, 12)
+    ev = np.random.default_rng(2).normal(0, 1, (5, V, C))
+    mars = O.forward_soft(fc, ev, double=True)
+    fl, _ = O.backward(fc, mars, double=True)
+    counts = O.input_flows_soft(fc, ev, mars, fl, double=True)
+    base = np.asarray(fc.leaf_logp, np.float64).copy()
+    h = 1e-6
+    for i in np.random.default_rng(3).choice(len(base), 12, replace=False):
+        g = fc.copy()
+        up, dn = base.copy(), base.copy()
+        up[i] += h
+        dn[i] -= h
+        g.leaf_logp = up
+        a = O.forward_soft(g, ev, double=True)[-1].sum()
+        g.leaf_logp = dn
+        b = O.forward_soft(g, ev, double=True)[-1].sum()
+        assert abs((a - b) / (2 * h) - counts[i]) < 1e-6
+
+
+# ---- the HIP path -------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    import pcmi355
+    return torch, pcmi355
+
+
+LL_RTOL, FLOW_RTOL = 1e-5, 1e-4
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("V,K,C,B", [(7, 16, 5, 70), (9, 64, 128, 33), (6, 8, 4, 64), (5, 128, 6, 20)])
+def test_hclt_soft_evidence_matches_oracle(gpu, V, K, C, B):
+    torch, P = gpu
+    parent, theta, leaf, fc = make_hclt(V, K, C, 50 + V)
+    rng = np.random.default_rng(V)
+    ev = rng.normal(0, 2, (B, V, C)).astype(np.float32)
+    ev[rng.random((B, V, C)) < 0.1] = -np.inf                # impossible categories
+    ev[:, :, 0] = np.where(np.isinf(ev).all(axis=2), 0.0, ev[:, :, 0])
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    mars = O.forward_soft(fc, ev, double=True)
+    d = torch.from_numpy(ev).cuda()
+    ll = P.loglikelihoods(bpc, d).cpu().numpy()
+    assert np.abs(ll - mars[-1]).max() < LL_RTOL * np.abs(mars[-1]).max()
+    # Julia's layout: examples fastest
+    dj = torch.from_numpy(np.ascontiguousarray(ev.transpose(2, 1, 0))).cuda().permute(2, 1, 0)
+    assert np.array_equal(P.loglikelihoods(bpc, dj, batch_size=16).cpu().numpy(), ll)
+    # flows and the EM update
+    ll2 = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    assert np.array_equal(ll, ll2)
+    fl, ea = O.backward(fc, mars, double=True)
+    counts = O.input_flows_soft(fc, ev, mars, fl, double=True)
+    ea_blk, lf_blk = bpc.get_flows()
+    ref_ea = O.hclt_block_aggr(fc, ea)
+    for v, blk in ref_ea.items():
+        assert np.abs(ea_blk[v][:blk.shape[0]] - blk).max() < FLOW_RTOL * max(blk.max(), 1e-3)
+    want = counts.reshape(V, K, C)                                       # the oracle's HCLT holds its leaves as [V][K][C]
+    assert np.abs(lf_blk - want).max() < FLOW_RTOL * max(want.max(), 1e-3)
+    np.testing.assert_allclose(lf_blk.sum(axis=(1, 2)), B, rtol=1e-4)      # every example passes every variable once
+    import pcmi355._lib as L
+    L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+    new_logp, new_leaf = O.em_update(fc, ea, counts, 0.1, 0.9, double=True)
+    _, leaf_after = bpc.get_params()
+    assert np.abs(np.exp(leaf_after) - np.exp(new_leaf.reshape(V, K, C))).max() < 5e-4 * np.exp(new_leaf).max()
+
+
+@pytest.mark.gpu
+def test_general_circuit_soft_evidence_and_one_hot_limit(gpu):
+    torch, P = gpu
+    V, C, B = 8, 5, 90
+    rng = np.random.default_rng(4)
+    root = random_dag(V, C, rng, width=4)
+    g = describe_dag([root])
+    bpc = P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"], g["input_logp"], V, C)
+    fc = O.bits_compile(root, C, V)
+    ev = rng.normal(0, 1.5, (B, V, C)).astype(np.float32)
+    mars = O.forward_soft(fc, ev, double=True)
+    d = torch.from_numpy(ev).cuda()
+    ids = rng.permutation(B)[:37].astype(np.int32)
+    ll = P.loglikelihoods(bpc, d, example_ids=ids).cpu().numpy()
+    assert np.abs(ll - mars[-1][ids]).max() < LL_RTOL * np.abs(mars[-1]).max()
+    # one-hot evidence gives exactly the categorical answer of the same engine
+    data = rng.integers(0, C, (B, V)).astype(np.uint8)
+    hard = P.loglikelihoods(bpc, torch.from_numpy(data).cuda()).cpu().numpy()
+    soft = P.loglikelihoods(bpc, torch.from_numpy(_one_hot_evidence(data, C)).cuda()).cpu().numpy()
+    np.testing.assert_allclose(soft, hard, rtol=1e-6)
+    # EM on soft evidence raises the soft likelihood
+    lls = P.mini_batch_em_with_reg(bpc, d, 4, batch_size=45, pseudocount=0.1, param_inertia=0.5, shuffle="none")
+    assert lls[-1] > lls[0]
+
+
+@pytest.mark.gpu
+def test_top_level_circuit_shape(gpu):
+    """The top-level circuit of the patch experiments: 64 variables (patches), 128 categories
+    (clusters), K = 64, fed per-cluster patch log-likelihoods; oracle on a subset, then training."""
+    torch, P = gpu
+    V, K, C, B = 64, 64, 128, 512
+    parent, theta, leaf, fc = make_hclt(V, K, C, 3)
+    rng = np.random.default_rng(8)
+    ev = (rng.normal(-600, 30, (B, V, 1)) + rng.gumbel(0, 8, (B, V, C))).astype(np.float32)   # patch LLs per cluster
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    d = torch.from_numpy(ev).cuda()
+    ll = P.loglikelihoods(bpc, d, batch_size=256).cpu().numpy()
+    want = O.forward_soft(fc, ev[:24], double=True)[-1]
+    assert np.abs(ll[:24] - want).max() < LL_RTOL * np.abs(want).max()
+    lls = P.mini_batch_em_with_reg(bpc, d, 3, batch_size=256, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert lls[-1] > lls[0]
