@@ -273,23 +273,8 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
   float m[EX], sum[EX];
   if (d.type[n] == kInput) {
     if (wave) return;
-    if (d.ev) {
-      // soft evidence, src/regularization/reg_likelihood.jl:51-91: logsumexp_c(evidence_c + logp_c)
-      const float* lp = d.leaf + d.in_off[n];
-#pragma unroll
-      for (int x = 0; x < EX; ++x) {
-        const int b = min(bb[x], d.B - 1);
-        const float* e = d.ev + (int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + (int64_t)d.in_var[n] * d.ev_sv;
-        float mm = -INFINITY, ss = 0.f;
-        for (int c = 0; c < d.C; ++c) {
-          const float t = e[(int64_t)c * d.ev_sc] + lp[c];
-          if (t > mm) { ss = ss * __expf(mm - t) + 1.f; mm = t; }
-          else if (t != -INFINITY) ss += __expf(t - mm);
-        }
-        m[x] = mm == -INFINITY ? mm : mm + __logf(ss);
-        sum[x] = 1.f;
-      }
-    } else {
+    if (d.ev) return;   // soft evidence: sparse_soft_input_kernel has filled the input rows
+    {
       const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
 #pragma unroll
       for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
@@ -485,37 +470,120 @@ __global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, cons
   for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += hist[c];
 }
 
-// The same with soft evidence, src/regularization/reg_flow.jl:50-82: category c of input node n
-// receives sum_b flow[b] * exp(evidence[b][c] + logp_c - value[b]).  Thread = category, the
-// node's values and flows of the batch staged in LDS.
-__global__ __launch_bounds__(256) void sparse_leaf_flow_soft_kernel(SparseDev d, const int32_t* __restrict__ input_nodes,
+// Soft evidence, per variable.  All input nodes of a variable read the same evidence, so a
+// workgroup stages a [64 examples][64 categories] tile of it in LDS once and every thread folds it
+// into several nodes; the nodes' log-parameters (going up) and values / flows (going down) are
+// uniform over a wave and come through the scalar cache.
+constexpr int kSoftTile = 64;    // examples and categories per staged tile
+constexpr int kSoftNodes = 16;   // nodes a thread carries at a time (x 4 waves = 64 nodes per round)
+
+// Leaf values, src/regularization/reg_likelihood.jl:51-91: logsumexp_c(evidence_c + logp_c) as a
+// running maximum and a sum of exponentials.  Workgroup = (variable, 64 examples); thread =
+// (example, wave w): nodes w, w + 4, ... of the variable.
+__global__ __launch_bounds__(256) void sparse_soft_input_kernel(SparseDev d, const int32_t* __restrict__ var_ptr,
+                                                                const int32_t* __restrict__ var_nodes) {
+  __shared__ float tile[kSoftTile][kSoftTile + 1];
+  const int v = blockIdx.x, b0 = blockIdx.y * kSoftTile;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = var_ptr[v], nv = var_ptr[v + 1] - n0;
+  for (int q0 = 0; q0 < nv; q0 += 4 * kSoftNodes) {
+    float m[kSoftNodes], sm[kSoftNodes];
+#pragma unroll
+    for (int q = 0; q < kSoftNodes; ++q) { m[q] = -INFINITY; sm[q] = 0.f; }
+    for (int c0 = 0; c0 < d.C; c0 += kSoftTile) {
+      __syncthreads();
+      for (int i = threadIdx.x; i < kSoftTile * kSoftTile; i += 256) {
+        // the faster of the two strides goes to consecutive threads
+        const int bi = d.ev_se <= d.ev_sc ? i % kSoftTile : i / kSoftTile, ci = d.ev_se <= d.ev_sc ? i / kSoftTile : i % kSoftTile;
+        const int b = min(b0 + bi, d.B - 1), c = c0 + ci;
+        tile[bi][ci] = c < d.C ? d.ev[(int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + (int64_t)v * d.ev_sv + (int64_t)c * d.ev_sc]
+                               : -INFINITY;
+      }
+      __syncthreads();
+      const int nc = min(kSoftTile, d.C - c0);
+#pragma unroll
+      for (int q = 0; q < kSoftNodes; ++q) {
+        const int qi = q0 + wave + 4 * q;
+        if (qi >= nv) break;
+        const float* lp = d.leaf + d.in_off[var_nodes[n0 + qi]] + c0;
+        float mm = m[q], ss = sm[q];
+        for (int c = 0; c < nc; ++c) {
+          const float t = tile[lane][c] + lp[c];
+          if (t > mm) { ss = ss * __expf(mm - t) + 1.f; mm = t; }
+          else if (t != -INFINITY) ss += __expf(t - mm);
+        }
+        m[q] = mm; sm[q] = ss;
+      }
+    }
+    if (b0 + lane < d.Bp)
+#pragma unroll
+      for (int q = 0; q < kSoftNodes; ++q) {
+        const int qi = q0 + wave + 4 * q;
+        if (qi >= nv) break;
+        d.mars[(size_t)var_nodes[n0 + qi] * d.Bp + b0 + lane] = m[q] == -INFINITY ? m[q] : m[q] + __logf(sm[q]);
+      }
+  }
+}
+
+// Leaf counters, src/regularization/reg_flow.jl:50-82: category c of input node n receives
+// sum_b flow[b] * exp(evidence[b][c] + logp_c - value[b]).  Workgroup = (variable, 64 categories,
+// 16 of the variable's nodes); thread = (category, wave w): nodes w, w + 4, w + 8, w + 12 of the
+// group; the batch goes by in tiles of 64 examples, with the nodes' values and flows beside the
+// evidence tile in LDS.
+constexpr int kFlowNodes = 4;   // nodes per thread; x 4 waves = 16 nodes per workgroup
+
+__global__ __launch_bounds__(256) void sparse_leaf_flow_soft_kernel(SparseDev d, const int32_t* __restrict__ var_ptr,
+                                                                    const int32_t* __restrict__ var_nodes,
                                                                     float* __restrict__ leaf_flow) {
-  extern __shared__ float vf[];   // [2][chunk]
-  constexpr int kChunk = 2048;
-  const int n = input_nodes[blockIdx.x];
-  const float* lp = d.leaf + d.in_off[n];
-  const int64_t voff = (int64_t)d.in_var[n] * d.ev_sv;
-  float acc[4] = {0.f, 0.f, 0.f, 0.f};   // categories threadIdx.x + 256 * i (at most 256 categories: one per thread)
-  for (int b0 = 0; b0 < d.B; b0 += kChunk) {
-    const int nb = min(kChunk, d.B - b0);
+  __shared__ float tile[kSoftTile][kSoftTile + 1];   // [example][category]
+  __shared__ float vt[4 * kFlowNodes][kSoftTile], ft[4 * kFlowNodes][kSoftTile];
+  const int v = blockIdx.x, c0 = blockIdx.y * kSoftTile, q0 = blockIdx.z * (4 * kFlowNodes);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = var_ptr[v], nv = var_ptr[v + 1] - n0;
+  if (q0 >= nv) return;
+  const int c = c0 + lane;
+  float acc[kFlowNodes], lpc[kFlowNodes];
+#pragma unroll
+  for (int q = 0; q < kFlowNodes; ++q) {
+    acc[q] = 0.f;
+    const int qi = q0 + wave + 4 * q;
+    lpc[q] = (qi < nv && c < d.C) ? d.leaf[d.in_off[var_nodes[n0 + qi]] + c] : -INFINITY;
+  }
+  for (int b0 = 0; b0 < d.B; b0 += kSoftTile) {
     __syncthreads();
-    for (int i = threadIdx.x; i < nb; i += blockDim.x) {
-      vf[i] = d.mars[(size_t)n * d.Bp + b0 + i];
-      vf[kChunk + i] = d.flows[(size_t)n * d.Bp + b0 + i];
+    for (int i = threadIdx.x; i < kSoftTile * kSoftTile; i += 256) {
+      const int bi = d.ev_se <= d.ev_sc ? i % kSoftTile : i / kSoftTile, ci = d.ev_se <= d.ev_sc ? i / kSoftTile : i % kSoftTile;
+      const int b = b0 + bi, cc = c0 + ci;
+      tile[bi][ci] = (b < d.B && cc < d.C)
+                         ? d.ev[(int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + (int64_t)v * d.ev_sv + (int64_t)cc * d.ev_sc]
+                         : -INFINITY;
+    }
+    for (int i = threadIdx.x; i < 4 * kFlowNodes * kSoftTile; i += 256) {
+      const int qi = q0 + i / kSoftTile, bi = i % kSoftTile;
+      const bool ok = qi < nv && b0 + bi < d.B;
+      const size_t at = ok ? (size_t)var_nodes[n0 + qi] * d.Bp + b0 + bi : 0;
+      vt[i / kSoftTile][bi] = ok ? d.mars[at] : 0.f;
+      ft[i / kSoftTile][bi] = ok ? d.flows[at] : 0.f;
     }
     __syncthreads();
-    for (int c = threadIdx.x, q = 0; c < d.C; c += blockDim.x, ++q) {
-      float a = 0.f;
-      for (int i = 0; i < nb; ++i) {
-        const int b = b0 + i;
-        const float t = d.ev[(int64_t)(d.ev_idx ? d.ev_idx[b] : b) * d.ev_se + voff + (int64_t)c * d.ev_sc] + lp[c];
-        if (t != -INFINITY && vf[kChunk + i] != 0.f) a += __expf(t - vf[i]) * vf[kChunk + i];
+#pragma unroll
+    for (int q = 0; q < kFlowNodes; ++q) {
+      const int r = wave + 4 * q;
+      float a = acc[q];
+#pragma unroll 8
+      for (int b = 0; b < kSoftTile; ++b) {
+        const float t = tile[b][lane] + lpc[q], f = ft[r][b];
+        if (t != -INFINITY && f != 0.f) a += __expf(t - vt[r][b]) * f;
       }
-      acc[q & 3] += a;
+      acc[q] = a;
     }
   }
-  float* dst = leaf_flow + d.in_off[n];
-  for (int c = threadIdx.x, q = 0; c < d.C; c += blockDim.x, ++q) dst[c] += acc[q & 3];
+  if (c < d.C)
+#pragma unroll
+    for (int q = 0; q < kFlowNodes; ++q) {
+      const int qi = q0 + wave + 4 * q;
+      if (qi < nv) leaf_flow[d.in_off[var_nodes[n0 + qi]] + c] += acc[q];
+    }
 }
 
 __global__ void sparse_gather_in_logp_kernel(const int4* __restrict__ in_rec, const float* __restrict__ logp, int64_t n,
@@ -981,6 +1049,21 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
   make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
            d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
 
+// input nodes grouped by variable
+void SparseCircuit::ensure_var_tables() {
+  if (d_var_ptr_.n) return;
+  std::vector<int32_t> vp(fc_.num_vars + 1, 0), vn(fc_.input_nodes.size());
+  for (int32_t n : fc_.input_nodes) vp[fc_.in_var[n] + 1]++;
+  for (int v = 0; v < fc_.num_vars; ++v) vp[v + 1] += vp[v];
+  std::vector<int32_t> fill(vp.begin(), vp.end() - 1);
+  for (int32_t n : fc_.input_nodes) vn[fill[fc_.in_var[n]]++] = n;
+  if (vn.empty()) vn.push_back(0);
+  max_var_nodes_ = 1;
+  for (int v = 0; v < fc_.num_vars; ++v) max_var_nodes_ = std::max(max_var_nodes_, vp[v + 1] - vp[v]);
+  d_var_ptr_.upload(vp, stream);
+  d_var_nodes_.upload(vn, stream);
+}
+
 void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
   const int batch = b ? b->batch : s->batch;
   if (b ? !b->d_data : !s->d_ev) fail(PCM_ERR_ARG, "data pointer is null");
@@ -996,7 +1079,12 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
     check_launch("stage_batch");
   }
   SparseDev d = SPARSE_DEV(batch, Bp, xb);
-  if (s) { d.ev = s->d_ev; d.ev_se = s->stride_ex; d.ev_sv = s->stride_var; d.ev_sc = s->stride_cat; d.ev_idx = s->d_idx; }
+  if (s) {
+    d.ev = s->d_ev; d.ev_se = s->stride_ex; d.ev_sv = s->stride_var; d.ev_sc = s->stride_cat; d.ev_idx = s->d_idx;
+    ensure_var_tables();
+    hipLaunchKernelGGL(sparse_soft_input_kernel, dim3(fc_.num_vars, Bp / kSoftTile), dim3(256), 0, stream, d, d_var_ptr_.p,
+                       d_var_nodes_.p);
+  }
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
     if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
@@ -1081,8 +1169,9 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
   if (!fc_.input_nodes.empty()) {
     if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);
     if (soft)
-      hipLaunchKernelGGL(sparse_leaf_flow_soft_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 2 * 2048 * sizeof(float),
-                         stream, d, d_input_nodes_.p, d_leaf_flow_.p);
+      hipLaunchKernelGGL(sparse_leaf_flow_soft_kernel,
+                         dim3(fc_.num_vars, ceil_div(fc_.num_cats, kSoftTile), ceil_div(max_var_nodes_, 4 * kFlowNodes)), dim3(256), 0,
+                         stream, d, d_var_ptr_.p, d_var_nodes_.p, d_leaf_flow_.p);
     else
       hipLaunchKernelGGL(sparse_leaf_flow_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 0, stream, d,
                          d_input_nodes_.p, d_leaf_flow_.p);
@@ -1271,15 +1360,7 @@ void SparseCircuit::sample_soft_with_slots(const float* d_node_noise, const int3
   ensure_batch(batch);
   const int Bp = ceil_div(batch, 64) * 64;
   d_grad_.ensure((size_t)fc_.n_nodes() * Bp);   // normaliser sums; maxima go to the value array, td to the flow array
-  if (d_var_ptr_.n == 0) {
-    std::vector<int32_t> vp(fc_.num_vars + 1, 0), vn(fc_.input_nodes.size());
-    for (int32_t n : fc_.input_nodes) vp[fc_.in_var[n] + 1]++;
-    for (int v = 0; v < fc_.num_vars; ++v) vp[v + 1] += vp[v];
-    std::vector<int32_t> fill(vp.begin(), vp.end() - 1);
-    for (int32_t n : fc_.input_nodes) vn[fill[fc_.in_var[n]]++] = n;
-    d_var_ptr_.upload(vp, stream);
-    d_var_nodes_.upload(vn, stream);
-  }
+  ensure_var_tables();
   DevBuf<int64_t> e2p;
   std::vector<int64_t> e2pv = fc_.edge2param;
   if (e2pv.empty()) e2pv.push_back(0);

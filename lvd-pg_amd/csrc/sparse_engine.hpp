@@ -97,10 +97,11 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
   DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
-  int cap_batch_ = 0, last_batch_ = 0;
+  int cap_batch_ = 0, last_batch_ = 0, max_var_nodes_ = 1;
   bool have_flows_ = false;
 
   void ensure_batch(int batch);
+  void ensure_var_tables();
   void run_forward(const BatchRef* b, const SoftRef* s);
   void write_ll(int batch, float* d_ll);
   void run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll);
