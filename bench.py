@@ -177,13 +177,17 @@ def secondary(args):
             tt[0] += 1
             P.adam_step(p, g1, dp, dm, dv, lr=1e-4, t=tt[0])
         t_adam = _timed(torch, adam, args.steps, 1)
+        soft_out = torch.empty((B, V, C), device="cuda")
+        t_soft = _timed(torch, lambda: check(lib.pcm_sample_soft(p.handle, node_noise.data_ptr(), 0.5, B, soft_out.data_ptr())),
+                        max(1, args.steps // 4), 1)
+        del soft_out
         dt = t_samp
         algo = 4 * B * (n_inner * K + V * C)                           # the noise tensors, read once
         out.update(metric="samples/sec Gumbel-max from supplied noise, 3072-var HCLT K=32",
                    value=B / t_samp, unit="samples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
-                               "sample": t_samp * 1e3})
+                               "sample": t_samp * 1e3, "gumbel_sample_relaxed_T0.5": t_soft * 1e3})
     elif args.workload == "c4_top_soft":
         # the top-level circuit of C4: 64 patch variables, 128 cluster categories, K = 64, trained on soft evidence
         V, K, C, B = 64, 64, 128, 1024

@@ -8,6 +8,7 @@
 #include <numeric>
 
 #include "hclt_walk_lean.hip.hpp"
+#include "hclt_soft_sample.hip.hpp"
 
 namespace pcm {
 
@@ -966,6 +967,58 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   run_stats(d, rate);
   have_flows_ = true;
   if (timing) ++n_timed_;
+}
+
+// Relaxed sampling on the block form; false: this hidden size / temperature goes to the layered engine.
+bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  if (!block_ || !(temperature >= kSoftMinTemperature)) return false;
+  if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
+  if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  if (d_soft_tabs_.n == 0) {
+    // parent of every inner node | per variable the node whose probabilities reach its leaf |
+    // inner nodes by depth | level offsets
+    std::vector<int32_t> t((size_t)n_inner_ + V_);
+    for (int n = 0; n < n_inner_; ++n) {
+      const int v = var_of_inner_[n];
+      t[n] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+    }
+    for (int v = 0; v < V_; ++v) t[(size_t)n_inner_ + v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
+    std::vector<std::vector<int32_t>> by_depth;
+    for (int n = 0; n < n_inner_; ++n) {
+      const size_t dep = (size_t)depth_[var_of_inner_[n]];
+      if (by_depth.size() <= dep) by_depth.resize(dep + 1);
+      by_depth[dep].push_back(n);
+    }
+    std::vector<int32_t> ptr(1, 0);
+    for (const auto& lvl : by_depth) {
+      t.insert(t.end(), lvl.begin(), lvl.end());
+      ptr.push_back(ptr.back() + (int32_t)lvl.size());
+    }
+    soft_levels_ = (int)by_depth.size();
+    t.insert(t.end(), ptr.begin(), ptr.end());
+    d_soft_tabs_.upload(t, stream);
+  }
+  ensure_batch(batch);                       // the flow-ratio tiles double as the probability tiles
+  const int ns = ceil_div(batch, kSlice);
+  d_soft_w_.ensure((size_t)2 * n_inner_ * K_ * K_);
+  float* Af = d_soft_w_.p;
+  float* Ab = Af + (size_t)n_inner_ * K_ * K_;
+  const float inv_t = 1.f / temperature;
+  const int32_t* parent_of = d_soft_tabs_.p;
+  const int32_t* state_node = parent_of + n_inner_;
+  const int32_t* order = state_node + V_;
+  const int32_t* level_ptr = order + n_inner_;
+  PCM_DISPATCH_K(K_, {
+    hipLaunchKernelGGL(hclt_soft_w_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)), dim3(128), 0, stream, d_logtheta_.p,
+                       inv_t, n_inner_, Af, Ab);
+    hipLaunchKernelGGL(hclt_soft_walk_kernel<KK>, dim3(ns), dim3(kSoftWalkWaves * 64), 0, stream, Af, Ab, parent_of, order,
+                       level_ptr, soft_levels_, d_node_noise, n_inner_, batch, ns, inv_t, d_R_.p);
+    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, dim3(V_, ceil_div(batch, 4 * kSoftLeafRun)), dim3(256), 0, stream,
+                       d_leaf_.p, state_node, d_R_.p, V_, C_, batch, ns, d_out);
+  });
+  check_launch("hclt_sample_soft");
+  PCM_HIP(hipStreamSynchronize(stream));
+  return true;
 }
 
 HcltCircuit::~HcltCircuit() {

@@ -140,6 +140,7 @@ class HcltCircuit : public pcm_circuit {
                  float b2, float eps, int t) override;
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
 
+  bool sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out);
   void set_block_params(const float* theta, const float* leaf);
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
@@ -180,6 +181,9 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_leaf_kc_;      // [V][K][C] copy for sampling
   DevBuf<float> d_kld_;          // scratch of the KL recursion
   DevBuf<uint8_t> d_state_;      // [batch][n_inner] hidden states of a batch of samples
+  DevBuf<int32_t> d_soft_tabs_;     // relaxed sampler: parents | leaf-feeding nodes | nodes by depth | level offsets
+  DevBuf<float> d_soft_w_;          // ... exp(theta / T) in the two operand layouts
+  int soft_levels_ = 0;
   DevBuf<int32_t> d_sample_tabs_;   // sampler tables: parent of every inner node | state-giving node of every variable | level order
   int sample_groups_ = 0;
   DevBuf<int64_t> d_sum_param_src_;

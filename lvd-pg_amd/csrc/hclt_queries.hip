@@ -221,6 +221,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
 }
 
 void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  if (sample_soft_block(d_node_noise, temperature, batch, d_out)) return;
   SparseCircuit* g = general();
   DevBuf<int32_t> slots;
   slots.upload(noise_slot_, stream);

@@ -320,20 +320,37 @@ def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
         np.testing.assert_allclose(plain[0, v], marg, rtol=1e-4)
     assert np.array_equal(plain[0], plain[1])
 
-    # HCLT: the K sum nodes of a tree node share the noise column of each hidden state
-    Vh, K, Ch = 6, 16, 4
-    parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23)
-    h = P.hclt_from_clt(parent, Ch, K)
-    h.set_params(block_theta(parent, K, theta), leaf)
-    ch, _ = O.clt_children(parent)
-    inner = [v for v in O.clt_bottom_up(parent) if ch[v]]
-    hn = _gumbel(rng, (3, len(inner) * K))
-    got = P.gumbel_sample(h, 3, temperature=temperature, node_noise=torch.from_numpy(hn).cuda()).cpu().numpy()
-    for b in range(3):
-        g = np.zeros(flat.n_edges, np.float64)
-        for r, v in enumerate(inner):
-            nk = len(flat.meta["sum_node"][v])
-            e0 = flat.meta["edge_of"][v]
-            g[e0:e0 + nk * K] = np.tile(hn[b, r * K:(r + 1) * K], nk)
-        _, want = O.gumbel_soft(flat, g, temperature, double=True)
-        np.testing.assert_allclose(got[b], want, rtol=1e-4, atol=1e-7)
+    # HCLT: the K sum nodes of a tree node share the noise column of each hidden state.  Block
+    # sizes run on the block form (two matrix contractions per tree node and 16 examples), other
+    # sizes on the layered engine.
+    for Vh, K, Ch, Bh in ((6, 16, 4, 3), (11, 32, 256, 37), (9, 64, 10, 16), (5, 8, 4, 3)):
+        parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23 + K)
+        h = P.hclt_from_clt(parent, Ch, K)
+        h.set_params(block_theta(parent, K, theta), leaf)
+        ch, _ = O.clt_children(parent)
+        inner = [v for v in O.clt_bottom_up(parent) if ch[v]]
+        hn = _gumbel(rng, (Bh, len(inner) * K))
+        got = P.gumbel_sample(h, Bh, temperature=temperature, node_noise=torch.from_numpy(hn).cuda()).cpu().numpy()
+        np.testing.assert_allclose(got.sum(axis=2), 1.0, rtol=1e-4)
+        for b in range(Bh):
+            g = np.zeros(flat.n_edges, np.float64)
+            for r, v in enumerate(inner):
+                nk = len(flat.meta["sum_node"][v])
+                e0 = flat.meta["edge_of"][v]
+                g[e0:e0 + nk * K] = np.tile(hn[b, r * K:(r + 1) * K], nk)
+            _, want = O.gumbel_soft(flat, g, temperature, double=True)
+            np.testing.assert_allclose(got[b], want, rtol=2e-4, atol=1e-7)
+        # without noise at temperature 1: the marginals of the circuit, whatever the engine
+        _, marg = O.gumbel_soft(flat, None, 1.0, double=True)
+        plain = P.gumbel_sample(h, 2, temperature=1.0).cpu().numpy()
+        np.testing.assert_allclose(plain[0], marg, rtol=2e-4, atol=1e-7)
+        # a temperature below the block form's range takes the layered engine: same answer
+        cold = P.gumbel_sample(h, 2, temperature=0.15, node_noise=torch.from_numpy(hn[:2].copy()).cuda()).cpu().numpy()
+        for b in range(2):
+            g = np.zeros(flat.n_edges, np.float64)
+            for r, v in enumerate(inner):
+                nk = len(flat.meta["sum_node"][v])
+                e0 = flat.meta["edge_of"][v]
+                g[e0:e0 + nk * K] = np.tile(hn[b, r * K:(r + 1) * K], nk)
+            _, want = O.gumbel_soft(flat, g, 0.15, double=True)
+            np.testing.assert_allclose(cold[b], want, rtol=1e-3, atol=1e-6)
