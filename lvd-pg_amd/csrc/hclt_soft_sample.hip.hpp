@@ -121,20 +121,26 @@ __global__ __launch_bounds__(256) void hclt_soft_leaves_kernel(const float* __re
         for (int i = 0; i < 4; ++i) sv[4 * j4 + i][c] = __expf(x[i]);
       }
     const int b_end = min(b_first + kSoftLeafRun, batch);
+    // example bq = slice * 16 + bb holds state kt*16 + 4*g + i at float ((kt*64 + 16*g + bb) * 4 + i) of its tile;
+    // the next example's probabilities are requested before this one's are used
+    auto fetch = [&](int bq, v4f (&dst)[K / 4]) {
+      const float* pe = ptile + (size_t)(bq >> 4) * (kSlice * K) + (bq & 15) * 4;   // wave-uniform address
+#pragma unroll
+      for (int q = 0; q < K / 4; ++q) dst[q] = *reinterpret_cast<const v4f*>(pe + (size_t)q * 64);
+    };
+    v4f pc[K / 4], pn[K / 4];
+    fetch(b_first, pc);
     for (int bq = b_first; bq < b_end; ++bq) {
-      // example bq = slice * 16 + bb holds state kt*16 + 4*g + i at float ((kt*64 + 16*g + bb) * 4 + i) of its tile
-      const float* pe = ptile + (size_t)(bq >> 4) * (kSlice * K) + (bq & 15) * 4;
+      fetch(min(bq + 1, b_end - 1), pn);
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kt = 0; kt < K / 16; ++kt)
+      for (int q = 0; q < K / 4; ++q)   // q = kt * 4 + g: states q * 4 + i
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const v4f p4 = *reinterpret_cast<const v4f*>(pe + (kt * 64 + 16 * g) * 4);   // wave-uniform address
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
-          for (int i = 0; i < 4; ++i)
+          for (int c = 0; c < 4; ++c) acc[c] = fmaf(pc[q][i], sv[4 * q + i][c], acc[c]);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) acc[c] = fmaf(p4[i], sv[kt * 16 + 4 * g + i][c], acc[c]);
-        }
+      for (int q = 0; q < K / 4; ++q) pc[q] = pn[q];
       float* o = out + ((size_t)bq * V + u) * C + c0;
       if (c0 + 3 < C && (C & 3) == 0) {
         __builtin_nontemporal_store(v4f{acc[0], acc[1], acc[2], acc[3]}, reinterpret_cast<v4f*>(o));
