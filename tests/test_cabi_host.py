@@ -60,6 +60,16 @@ def test_version_and_error_reporting_without_a_gpu(cdll):
     assert cdll.pcm_size(None, 0) < 0
     assert cdll.pcm_em_update(None, ctypes.c_float(0.1), ctypes.c_float(0.9)) == -1
     assert cdll.pcm_free(None) in (0, -1)
+    # structure learning and soft evidence: argument errors come back as status codes
+    i64, f32 = ctypes.c_int64, ctypes.c_float
+    assert cdll.pcm_pairwise_mi(None, i64(1), i64(1), i64(10), 3, 4, f32(0.1), None, None) == -1
+    assert cdll.pcm_chow_liu_tree(None, 3, None) == -1
+    mi = (ctypes.c_float * 9)(0, 2, 1, 2, 0, 3, 1, 3, 0)
+    parent = (ctypes.c_int32 * 3)()
+    assert cdll.pcm_chow_liu_tree(mi, 3, parent) == 0
+    assert list(parent) == [1, -1, 1]                     # path 0 - 1 - 2, rooted at its centre
+    assert cdll.pcm_loglikelihoods_soft(None, None, i64(1), i64(1), i64(1), None, 4, None) == -1
+    assert cdll.pcm_flows_soft(None, None, i64(1), i64(1), i64(1), None, 4, f32(0), None, None) == -1
 
 
 def test_python_mirror_binds_every_symbol():
