@@ -22,10 +22,52 @@ static void check_launch_q(const char* what) {
 
 // States of the inner tree nodes.  K lanes per example (64/K examples per wave), one wave per
 // group for the whole tree.  Nodes come level by level from the root (`order`, padded with -1
-// to groups of four that never straddle a level), so the four nodes of a group are
+// to groups of kSampleGroup that never straddle a level), so the nodes of a group are
 // independent and their parameter rows are fetched together: the walk is a chain of memory
 // latencies, one per group.  The chosen states live in LDS (one byte per node and example) and
 // leave through a coalesced copy at the end.  No barriers: a wave only reads its own examples.
+// Largest value and, among equal values, the lowest index over groups of K consecutive lanes,
+// left in every lane of the group.  The exchange inside rows of 16 lanes uses data-parallel-
+// primitive moves (lane ^ 1, lane ^ 2, mirror of 8, mirror of 16: a few cycles each), the step
+// across neighbouring rows a lane-swap instruction; only lane ^ 32 goes through the LDS crossbar.  The rule is symmetric, so the order of the
+// exchanges does not change the result.
+template <int kCtrl>
+__device__ __forceinline__ void argmax_dpp(float& x, int& idx) {
+  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), kCtrl, 0xf, 0xf, true));
+  const int oi = __builtin_amdgcn_update_dpp(0, idx, kCtrl, 0xf, 0xf, true);
+  if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
+}
+
+template <int K>
+__device__ __forceinline__ void argmax_lanes(float& x, int& idx) {
+  if (K >= 2) argmax_dpp<0xB1>(x, idx);    // quad_perm [1,0,3,2]
+  if (K >= 4) argmax_dpp<0x4E>(x, idx);    // quad_perm [2,3,0,1]
+  if (K >= 8) argmax_dpp<0x141>(x, idx);   // row_half_mirror
+  if (K >= 16) argmax_dpp<0x140>(x, idx);  // row_mirror
+  if (K >= 32) {
+    // lane ^ 16: v_permlane16_swap exchanges the odd rows of its first operand with the even rows
+    // of its second, so with both operands equal an even row finds its partner in the second
+    // result and an odd row in the first
+    const bool even_row = ((threadIdx.x >> 4) & 1) == 0;
+    const int xi = __builtin_bit_cast(int, x);
+    const auto sx = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);
+    const auto si = __builtin_amdgcn_permlane16_swap(idx, idx, false, false);
+    const float ov = __builtin_bit_cast(float, even_row ? (int)sx[1] : (int)sx[0]);
+    const int oi = even_row ? (int)si[1] : (int)si[0];
+    if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
+  }
+  if (K >= 64) {
+    const float ov = __shfl_xor(x, 32);
+    const int oi = __shfl_xor(idx, 32);
+    if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
+  }
+}
+
+#ifndef PCM_SAMPLE_GROUP
+#define PCM_SAMPLE_GROUP 4
+#endif
+constexpr int kSampleGroup = PCM_SAMPLE_GROUP;   // independent nodes (same level) a wave handles together
+
 template <int K>
 __global__ __launch_bounds__(256) void hclt_sample_states_kernel(const float* __restrict__ logtheta,
                                                                  const int32_t* __restrict__ parent_of,
@@ -42,26 +84,21 @@ __global__ __launch_bounds__(256) void hclt_sample_states_kernel(const float* __
   uint8_t* mine = st + (size_t)ex_in_block * n_inner;
   const float* g = node_noise + (size_t)(live ? b : 0) * n_inner * K;
   for (int q = 0; q < n_groups; ++q) {
-    int nd[4];
-    float v[4];
+    int nd[kSampleGroup];
+    float v[kSampleGroup];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      nd[i] = order[q * 4 + i];
+    for (int i = 0; i < kSampleGroup; ++i) {
+      nd[i] = order[q * kSampleGroup + i];
       const int n = max(nd[i], 0);
       const int p = parent_of[n];
       const int k = p < 0 ? 0 : mine[p];
       v[i] = logtheta[((size_t)n * K + k) * K + j] + g[(size_t)n * K + j];
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < kSampleGroup; ++i) {
       int idx = j;
       float x = v[i];
-#pragma unroll
-      for (int o = K / 2; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(x, o, K);
-        const int oi = __shfl_xor(idx, o, K);
-        if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
-      }
+      argmax_lanes<K>(x, idx);
       if (j == 0 && nd[i] >= 0) mine[nd[i]] = (uint8_t)idx;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the bytes are read by the K lanes of this example
@@ -175,7 +212,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   }
   if (d_sample_tabs_.n == 0) {
     // per inner node: its parent | per variable: the node whose state picks its leaf row | inner
-    // nodes level by level from the root in groups of four (-1: padding)
+    // nodes level by level from the root in groups of kSampleGroup (-1: padding)
     std::vector<int32_t> t((size_t)n_inner_ + V_);
     for (int n = 0; n < n_inner_; ++n) {
       const int v = var_of_inner_[n];
@@ -191,9 +228,9 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     sample_groups_ = 0;
     for (const auto& lvl : by_depth) {
       for (int32_t n : lvl) t.push_back(n);
-      while ((t.size() - (size_t)n_inner_ - V_) % 4) t.push_back(-1);
+      while ((t.size() - (size_t)n_inner_ - V_) % kSampleGroup) t.push_back(-1);
     }
-    sample_groups_ = (int)((t.size() - (size_t)n_inner_ - V_) / 4);
+    sample_groups_ = (int)((t.size() - (size_t)n_inner_ - V_) / kSampleGroup);
     d_sample_tabs_.upload(t, stream);
   }
   d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
