@@ -166,8 +166,18 @@ __device__ __forceinline__ float tile_rowmax(const Tile<K>& z) {
   for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
     for (int i = 0; i < 4; ++i) m = fmaxf(m, z.v[kt][i]);
-  m = fmaxf(m, __shfl_xor(m, 16));
-  m = fmaxf(m, __shfl_xor(m, 32));
+  // lanes ^ 16 and ^ 32 with the row- and half-swap instructions (both operands equal: the two
+  // results hold the two partners), not through the LDS crossbar
+  {
+    const int mi = __builtin_bit_cast(int, m);
+    const auto r = __builtin_amdgcn_permlane16_swap(mi, mi, false, false);
+    m = fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+  }
+  {
+    const int mi = __builtin_bit_cast(int, m);
+    const auto r = __builtin_amdgcn_permlane32_swap(mi, mi, false, false);
+    m = fmaxf(__builtin_bit_cast(float, (int)r[0]), __builtin_bit_cast(float, (int)r[1]));
+  }
   return m == -INFINITY ? 0.f : m;
 }
 
