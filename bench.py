@@ -188,6 +188,41 @@ def secondary(args):
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
                                "sample": t_samp * 1e3, "gumbel_sample_relaxed_T0.5": t_soft * 1e3})
+    elif args.workload == "c4_patch_x8_streams":
+        # eight independent patch circuits (C4 has 64), each queued on one of four streams: the layered engine's
+        # per-layer launches are small, so circuits overlap on the device
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        sys.path.insert(0, os.path.join(ROOT, "oracle"))
+        sys.setrecursionlimit(20000)
+        from helpers import multihead_hclt, describe_dag
+        V, K, C, H, B, NC, NS = 192, 32, 256, 128, 1024, 8, 4
+        data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
+        parent = workloads.chow_liu_parent(data)
+        heads, _ = multihead_hclt(parent, K, C, H, rng)
+        g = describe_dag(heads)
+        circs = [P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"],
+                                   g["input_logp"], V, C, H) for _ in range(NC)]
+        mask = np.zeros((B, H), np.float32)
+        mask[np.arange(B), rng.integers(0, H, size=B)] = 1.0
+        d = torch.from_numpy(data).cuda()
+        hm = torch.from_numpy(mask).cuda().t().contiguous()
+        lls = [torch.empty(B, device="cuda") for _ in range(NC)]
+        streams = [torch.cuda.Stream() for _ in range(NS)]
+        torch.cuda.synchronize()
+        for i, c in enumerate(circs):
+            check(lib.pcm_set_stream(c.handle, streams[i % NS].cuda_stream))
+
+        def step():
+            for c, ll in zip(circs, lls):
+                check(lib.pcm_flows(c.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(), ll.data_ptr()))
+                check(lib.pcm_em_update(c.handle, 0.1, 0.9))
+        dt = _timed(torch, step, args.steps, args.warmup)
+        nn, ne = circs[0].num_nodes(), circs[0].num_edges()
+        algo = NC * B * (8 * nn + 24 * ne)
+        out.update(metric="examples/sec fwd+bwd+EM over 8 independent 192-var K=32 128-head patch circuits on 4 streams",
+                   value=NC * B / dt, unit="examples/s",
+                   config={"workload": args.workload, "circuits": NC, "streams": NS, "num_vars": V, "hidden": K,
+                           "categories": C, "heads": H, "batch": B})
     elif args.workload == "c4_top_soft":
         # the top-level circuit of C4: 64 patch variables, 128 cluster categories, K = 64, trained on soft evidence
         V, K, C, B = 64, 64, 128, 1024

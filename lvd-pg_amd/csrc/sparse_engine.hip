@@ -913,6 +913,7 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   if (fc_.heads.empty()) seed_of[nn - 1] = 0;
   else for (size_t h = 0; h < fc_.heads.size(); ++h) seed_of[fc_.heads[h]] = (int32_t)h;
   d_heads_.upload(seed_of);
+  if (!fc_.heads.empty()) d_head_nodes_.upload(fc_.heads);
   // An input node that is the second factor of two-child products and sees exactly the edges its
   // first factor (the prime) sees gets the same flow as the prime: it is dropped from the backward
   // layers and the prime's wave writes its row too (in an HCLT: every leaf).
@@ -1103,12 +1104,9 @@ void SparseCircuit::write_ll(int batch, float* d_ll) {
     PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)batch * sizeof(float),
                            hipMemcpyDeviceToDevice, stream));
   } else {
-    DevBuf<int32_t> hn;
-    hn.upload(fc_.heads, stream);
     hipLaunchKernelGGL(sparse_copy_rows_kernel, dim3(ceil_div(batch, 256), (int)fc_.heads.size()), dim3(256), 0, stream,
-                       d_mars_.p, Bp, batch, hn.p, (int)fc_.heads.size(), d_ll);
+                       d_mars_.p, Bp, batch, d_head_nodes_.p, (int)fc_.heads.size(), d_ll);
     check_launch("copy_rows");
-    PCM_HIP(hipStreamSynchronize(stream));
   }
 }
 
@@ -1181,12 +1179,9 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)batch * sizeof(float),
                            hipMemcpyDeviceToDevice, stream));
   } else {
-    DevBuf<int32_t> hn;
-    hn.upload(fc_.heads, stream);
     hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(batch, 256)), dim3(256), 0, stream, d_mars_.p, Bp, batch,
-                       hn.p, (int)fc_.heads.size(), d_head_mask, d_ll);
+                       d_head_nodes_.p, (int)fc_.heads.size(), d_head_mask, d_ll);
     check_launch("head_mixture");
-    PCM_HIP(hipStreamSynchronize(stream));
   }
   have_flows_ = true;
 }

@@ -94,6 +94,7 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_in_logp_;
   DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
+  DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
   DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
