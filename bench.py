@@ -122,7 +122,7 @@ def secondary(args):
                            "frac": ach / 157.3, "traffic": None}
         print(json.dumps(out))
         return
-    elif args.workload == "c4_patch_multihead":
+    elif args.workload in ("c4_patch_multihead", "c4_patch_multihead_block"):
         sys.path.insert(0, os.path.join(ROOT, "tests"))
         sys.path.insert(0, os.path.join(ROOT, "oracle"))
         sys.setrecursionlimit(20000)
@@ -134,6 +134,11 @@ def secondary(args):
         g = describe_dag(heads)
         bpc = P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"],
                                 g["input_logp"], V, C, H)
+        engine = "layered engine"
+        if args.workload.endswith("_block"):      # the same circuit and parameters on the block engine
+            blk = P.multihead_hclt_from_clt(parent, C, K, H)
+            P.update_parameters(blk, P.vectorize_parameters(bpc))
+            bpc, engine = blk, "block engine"
         mask = np.zeros((B, H), np.float32)
         mask[np.arange(B), rng.integers(0, H, size=B)] = 1.0
         d = torch.from_numpy(data).cuda()
@@ -146,7 +151,9 @@ def secondary(args):
         dt = _timed(torch, step, args.steps, args.warmup)
         nn, ne = bpc.num_nodes(), bpc.num_edges()
         algo = B * (8 * nn + 24 * ne)
-        out.update(metric="examples/sec fwd+bwd+EM, 192-var patch circuit K=32 with 128 heads (layered engine)",
+        if engine == "block engine":   # block form: six K-vectors per tree node and example, the mask read going up and down
+            algo = algorithmic_bytes(bpc.size("inner_tree_nodes"), V, K, C, B)["step"] + 2 * 4 * H * B
+        out.update(metric="examples/sec fwd+bwd+EM, 192-var patch circuit K=32 with 128 heads (%s)" % engine,
                    value=B / dt, unit="examples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "heads": H,
                            "batch": B, "nodes": nn, "edges": ne})

@@ -50,6 +50,20 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
                     int32_t num_cats, pcm_circuit** out);
 
 /*
+ * A multi-head HCLT: the circuits `CuMultiHeadBitsProbCircuit(pcs)` (src-jl/multi_head_pc/bit_circuit.jl:14-56)
+ * is given when the `pcs` are num_heads root sum nodes over the K products of one HCLT body (the patch
+ * circuits of exps/progressive_growing/parallel_PG.jl:214-225 before pruning).  Runs on the block engine:
+ * the body through the tree-walk kernels, the heads as an [H][K] block in two small kernels around them.
+ * Needs num_hidden_cats 16 or 32 and at most three children per tree node (PCM_ERR_UNSUPPORTED otherwise:
+ * describe the circuit to pcm_circuit_create instead).  Parameter vector: the body's sum parameters in
+ * the order of pcm_hclt_create without the root's row, then num_heads x K head parameters, then the input
+ * nodes; the same order pcm_circuit_create gives the equivalent description.  pcm_loglikelihoods returns
+ * [num_heads][batch], pcm_flows takes d_head_mask [num_heads][batch]; KL and sampling are not defined.
+ */
+int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
+                              int32_t num_heads, pcm_circuit** out);
+
+/*
  * Compile a general circuit given as a DAG in topological order (children before
  * parents, root last), the flat form a binding obtains by walking a `ProbCircuit`:
  * replaces `CuMetaBitsProbCircuit(pc)` (src/bits_circuit.jl:39) and, with num_heads > 0,

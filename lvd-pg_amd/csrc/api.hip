@@ -55,6 +55,16 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
   });
 }
 
+int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
+                              int32_t num_heads, pcm_circuit** out) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    *out = nullptr;
+    if (num_heads < 1) pcm::fail(PCM_ERR_SHAPE, "num_heads must be positive, got %d", num_heads);
+    *out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats, num_heads);
+  });
+}
+
 int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_t* child_ptr,
                        const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
                        const float* input_logp, int32_t num_vars, int32_t num_cats, int32_t num_heads,

@@ -9,6 +9,7 @@
 
 #include "hclt_walk_lean.hip.hpp"
 #include "hclt_soft_sample.hip.hpp"
+#include "hclt_heads.hip.hpp"
 
 namespace pcm {
 
@@ -25,7 +26,10 @@ static void check_launch(const char* what) {
   if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
 }
 
-HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C) : V_(V), K_(K), C_(C) {
+HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads) : V_(V), K_(K), C_(C) {
+  if (num_heads < 0 || num_heads > 4096) fail(PCM_ERR_SHAPE, "num_heads must be in 0..4096, got %d", num_heads);
+  H_ = num_heads;
+  Hp_ = ceil_div(num_heads, 16) * 16;
   if (!parent) fail(PCM_ERR_ARG, "clt_parent is null");
   if (V < 2) fail(PCM_ERR_SHAPE, "an HCLT needs at least 2 variables, got %d", V);
   if (K < 1 || K > 1024) fail(PCM_ERR_SHAPE, "num_hidden_cats must be in 1..1024, got %d", K);
@@ -36,16 +40,26 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C) : V_(V), K_
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
   build_structure();
+  if (H_ > 0 && !(block_ && fwd_lean_ && bwd_lean_ && stat_lean_))
+    fail(PCM_ERR_UNSUPPORTED, "multi-head block kernels need K = 16 or 32 and at most three children per tree node; "
+                              "compile this circuit with pcm_circuit_create");
   build_param_order();
 
   // uniform parameters
   std::vector<float> theta((size_t)V_ * K_ * K_, -std::log((float)K_));
   std::vector<float> leaf((size_t)V_ * K_ * C_, -std::log((float)C_));
   d_leaf_.alloc((size_t)V_ * C_ * K_);
-  d_logtheta_.alloc((size_t)n_inner_ * K_ * K_);
+  d_logtheta_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)H_ * K_);   // the head rows sit behind the blocks
   d_Wf_.alloc((size_t)n_inner_ * K_ * K_);
   d_Wb_.alloc((size_t)n_inner_ * K_ * K_);
-  d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_);
+  d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)H_ * K_);
+  if (H_ > 0) {
+    d_head_wf_.alloc((size_t)Hp_ * K_);
+    d_flow_shift_.alloc(1);
+    d_head_wb_.alloc((size_t)Hp_ * K_);
+    std::vector<float> hl((size_t)H_ * K_, -std::log((float)K_));
+    PCM_HIP(hipMemcpy(head_logp(), hl.data(), hl.size() * sizeof(float), hipMemcpyHostToDevice));
+  }
   d_leaf_flow_.alloc((size_t)V_ * C_ * K_);
   d_edge_aggr_.zero();
   d_leaf_flow_.zero();
@@ -227,7 +241,7 @@ void HcltCircuit::build_schedules() {
         put(kLW, (int32_t)((size_t)n * K_ * K_ * sizeof(float)));
         put(kLA0, (int32_t)((size_t)var_of_inner_[n] * leaf_stride));
         put(kLNode, n);
-        put(kLFlags, par[n] < 0 ? 1 : 0);
+        put(kLFlags, par[n] < 0 ? (H_ > 0 ? 3 : 1) : 0);
         if (forward) {
           if (lc[n].size() > 3 || ic[n].size() > 3) return false;
           for (size_t i = 0; i < lc[n].size(); ++i) put(kLA1 + (int)i, (int32_t)((size_t)lc[n][i] * leaf_stride));
@@ -443,6 +457,7 @@ void HcltCircuit::build_schedules() {
 void HcltCircuit::build_param_order() {
   const int K = K_;
   std::vector<int64_t> sum_id((size_t)V_ * K, -1), mul_id((size_t)V_ * K, -1), in_id((size_t)V_ * K, -1);
+  std::vector<int64_t> rprod_id(K, -1);
   int64_t next = 0;
   input_order_.clear();
   // explicit stack machine for visit(v, k)
@@ -478,6 +493,8 @@ void HcltCircuit::build_param_order() {
       if (children_[v].size() > 2) mul_id[(size_t)v * K + f.j] = next++;
       create_input(v, f.j);
       if (children_[v].size() == 2) mul_id[(size_t)v * K + f.j] = next++;
+      // multi-head: the root's product (children x leaf) is shared by all heads, so it is a node of its own
+      if (H_ > 0 && v == root_) rprod_id[f.j] = next++;
       f.j++;
       f.c = 0;
       continue;
@@ -486,7 +503,8 @@ void HcltCircuit::build_param_order() {
     sum_id[(size_t)v * K + f.k] = next++;
     st.pop_back();
   }
-  n_nodes_ = next;
+  n_nodes_ = next + (H_ > 0 ? H_ - 1 : 0);   // multi-head: the root's sum node is head 0, the other heads follow it
+  const int64_t head0 = next - 1;
 
   // layers
   std::vector<int> vlayer(V_, 0);   // layer of the sum nodes of v (0 for leaves = inputs)
@@ -505,8 +523,12 @@ void HcltCircuit::build_param_order() {
     int v = var_of_inner_[n];
     if (children_[v].size() > 1)
       for (int j = 0; j < K; ++j) recs.push_back({mlayer[v], mul_id[(size_t)v * K + j], 0, v, j});
-    int nk = v == root_ ? 1 : K;
+    int nk = v == root_ ? (H_ > 0 ? 0 : 1) : K;
     for (int k = 0; k < nk; ++k) recs.push_back({vlayer[v], sum_id[(size_t)v * K + k], 1, v, k});
+  }
+  if (H_ > 0) {
+    for (int j = 0; j < K; ++j) recs.push_back({vlayer[root_], rprod_id[j], 3, root_, j});   // kind 3: a root product
+    for (int h = 0; h < H_; ++h) recs.push_back({vlayer[root_] + 1, head0 + h, 2, root_, h});   // kind 2: a head
   }
   std::sort(recs.begin(), recs.end(), [](const Rec& a, const Rec& b) {
     return a.layer != b.layer ? a.layer < b.layer : a.parent < b.parent;
@@ -528,6 +550,20 @@ void HcltCircuit::build_param_order() {
         edge_sub_.push_back(q + 1 < ch.size() ? circ_id(ch[q + 1], r.k) + 1 : 0);
         edge2param_.push_back(0);
       }
+    } else if (r.kind == 3) {   // root product of a multi-head circuit: (children's circuit, leaf) at state r.k
+      edge_parent_.push_back(r.parent + 1);
+      edge_prime_.push_back((ch.size() > 1 ? mul_id[(size_t)r.v * K + r.k] : circ_id(ch[0], r.k)) + 1);
+      edge_sub_.push_back(in_id[(size_t)r.v * K + r.k] + 1);
+      edge2param_.push_back(0);
+    } else if (r.kind == 2) {   // head r.k over the K root products
+      for (int j = 0; j < K; ++j) {
+        edge_parent_.push_back(r.parent + 1);
+        edge_prime_.push_back(rprod_id[j] + 1);
+        edge_sub_.push_back(0);
+        sum_param_src_.push_back(((int64_t)n_inner_ * K + r.k) * K + j);   // head rows sit behind the blocks
+        edge2param_.push_back((int64_t)sum_param_src_.size());
+      }
+      sum_group_size_.push_back(K);
     } else {
       const int n = inner_of_var_[r.v];
       for (int j = 0; j < K; ++j) {
@@ -547,7 +583,7 @@ void HcltCircuit::build_param_order() {
 
   // the same circuit in general form, for the queries that run on the general engine
   flat_ = FlatCircuit();
-  flat_.num_vars = V_; flat_.num_cats = C_; flat_.num_heads = 0;
+  flat_.num_vars = V_; flat_.num_cats = C_; flat_.num_heads = H_;
   flat_.type.assign(n_nodes_, kInput);
   flat_.layer.assign(n_nodes_, 0);
   flat_.in_var.assign(n_nodes_, -1);
@@ -567,6 +603,13 @@ void HcltCircuit::build_param_order() {
       if (sum_id[(size_t)v * K + k] >= 0) { flat_.type[sum_id[(size_t)v * K + k]] = kSum; flat_.layer[sum_id[(size_t)v * K + k]] = vlayer[v]; }
     }
   }
+  for (int h = 0; h < H_; ++h) {
+    flat_.type[head0 + h] = kSum;
+    flat_.layer[head0 + h] = vlayer[root_] + 1;
+    flat_.heads.push_back((int32_t)(head0 + h));
+  }
+  if (H_ > 0)
+    for (int j = 0; j < K; ++j) { flat_.type[rprod_id[j]] = kMul; flat_.layer[rprod_id[j]] = vlayer[root_]; }
   flat_.leaf_logp.assign((size_t)V_ * K * C_, 0.f);
   noise_slot_.assign(n_edges_, 0);
   for (int64_t ed = 0; ed < n_edges_; ++ed) {
@@ -576,7 +619,7 @@ void HcltCircuit::build_param_order() {
     flat_.e_logp.push_back(0.f);
     if (edge2param_[ed]) {
       const int64_t src = sum_param_src_[edge2param_[ed] - 1];
-      noise_slot_[ed] = (int32_t)((src / ((int64_t)K * K)) * K + src % K);
+      if (src < (int64_t)n_inner_ * K * K) noise_slot_[ed] = (int32_t)((src / ((int64_t)K * K)) * K + src % K);
     }
   }
   flat_.finish();
@@ -596,7 +639,7 @@ int64_t HcltCircuit::size(int what) const {
     case 9: return (int64_t)layer_ends_.size();
     case 10: return (int64_t)sum_group_size_.size();
     case 11: return (int64_t)V_ * K_;
-    case 12: return 0;
+    case 12: return H_;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -630,7 +673,11 @@ void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
     case 6: copy(edge_parent_); break;
     case 7: copy(edge_prime_); break;
     case 8: copy(edge_sub_); break;
-    case 9: copy(std::vector<int64_t>()); break;
+    case 9: {
+      std::vector<int64_t> hd;
+      for (int h = 0; h < H_; ++h) hd.push_back(n_nodes_ - H_ + h + 1);
+      copy(hd); break;
+    }
     default: fail(PCM_ERR_ARG, "unknown index table %d", which);
   }
 }
@@ -643,6 +690,22 @@ void HcltCircuit::rebuild_w() {
   PCM_DISPATCH_PARAM_K(K_, hipLaunchKernelGGL(hclt_rebuild_w_kernel<KK>, dim3(ceil_div(tot, 256)), dim3(256), 0,
                                         stream, d_logtheta_.p, d_Wf_.p, d_Wb_.p, n_inner_));
   check_launch("rebuild_w");
+  rebuild_heads();
+}
+
+void HcltCircuit::rebuild_heads() {
+  if (H_ == 0) return;
+  hipLaunchKernelGGL(hclt_heads_rebuild_kernel, dim3(ceil_div((int64_t)Hp_ * K_, 256)), dim3(256), 0, stream, head_logp(), H_,
+                     Hp_, K_, d_head_wf_.p, d_head_wb_.p);
+  check_launch("rebuild_heads");
+}
+
+// head values from the root tile the forward walk has left (identity block: the root's Z)
+void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix) {
+  const float* o_root = d.O + (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
+  PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), 0, stream,
+                                             o_root, d_head_wf_.p, H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix));
+  check_launch("heads_forward");
 }
 
 void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
@@ -653,8 +716,13 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
       const float* src = theta + (size_t)var_of_inner_[n] * K * K;
       float* dst = lt.data() + (size_t)n * K * K;
       std::copy(src, src + (size_t)K * K, dst);
-      if (var_of_inner_[n] == root_)
-        for (int i = K; i < K * K; ++i) dst[i] = -INFINITY;   // the root keeps one sum node
+      if (var_of_inner_[n] == root_) {
+        if (H_ > 0) {   // multi-head: identity block, the heads have their own rows
+          for (int i = 0; i < K * K; ++i) dst[i] = (i / K == i % K) ? 0.f : -INFINITY;
+        } else {
+          for (int i = K; i < K * K; ++i) dst[i] = -INFINITY;   // the root keeps one sum node
+        }
+      }
     }
     PCM_HIP(hipMemcpyAsync(d_logtheta_.p, lt.data(), lt.size() * sizeof(float), hipMemcpyHostToDevice, stream));
     PCM_HIP(hipStreamSynchronize(stream));
@@ -896,13 +964,15 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
         PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_lean_kernel<KK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(n_inner_), dim3(kStatLeanWaves * 64), lds, stream, d,
-                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, limb);
+                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, limb,
+                           H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
       });
       check_launch("hclt_stats_lean");
       if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
       return;
     }
   }
+  if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "multi-head HCLT with %d categories: the statistics do not fit the fast kernel", C_);
   // LDS layout of hclt_stats_kernel
   const size_t pads = (size_t)kStatWaves * kSlice * (K_ + 16);
   auto hist_words = [&](int nh) { return std::max((((size_t)nh * hist + 3) & ~(size_t)3), (size_t)K_ * K_); };
@@ -926,6 +996,13 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   if (!block_ && !wide_) return general()->loglikelihoods(b, d_ll);
   stage_batch(b);
   if (wide_) return wide_forward(dev(b.batch), d_ll);
+  if (H_ > 0) {   // per-head values [H][batch]
+    d_ll_heads_.ensure((size_t)b.batch);
+    const HcltDev d = dev(b.batch);
+    run_forward(d, d_ll_heads_.p);
+    heads_forward(d, nullptr, d_ll, nullptr);
+    return;
+  }
   run_forward(dev(b.batch), d_ll);
 }
 
@@ -934,16 +1011,17 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
 void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) { general()->loglikelihoods_soft(s, d_ll); }
 
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
-  if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (have_flows_ && !flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from categorical batches to soft-evidence batches");
-  general()->flows_soft(s, rate, nullptr, d_ll);
+  general()->flows_soft(s, rate, d_head_mask, d_ll);
   have_flows_ = true;
   flows_in_general_ = true;
 }
 
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
-  if (d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (H_ > 0 && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from soft-evidence batches to categorical batches");
@@ -955,6 +1033,24 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   }
   stage_batch(b);
   HcltDev d = dev(b.batch);
+  if (H_ > 0) {
+    d_ll_heads_.ensure((size_t)b.batch);
+    run_forward(d, d_ll_heads_.p);
+    heads_forward(d, d_head_mask, nullptr, d_ll);
+    hipLaunchKernelGGL(hclt_scale_kernel, dim3(ceil_div((int64_t)H_ * K_, 256)), dim3(256), 0, stream, head_aggr(),
+                       (int64_t)H_ * K_, rate, d_flow_shift_.p);
+    const size_t root_tile = (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
+    const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_) * sizeof(float);
+    PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,
+                                               stream, d.O + root_tile, d_head_wf_.p, d_head_wb_.p, head_logp(), H_, Hp_,
+                                               d.B, d_head_mask, d.R + root_tile, head_aggr(), d_flow_shift_.p));
+    check_launch("heads_backward");
+    run_backward(d);
+    run_stats(d, rate);
+    have_flows_ = true;
+    if (timing) ++n_timed_;
+    return;
+  }
   if (wide_) {
     wide_forward(d, d_ll);
     wide_backward_stats(d, rate);
@@ -1058,9 +1154,15 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
   PCM_DISPATCH_PARAM_K(K_, {
     constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
     hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,
-                       stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia);
+                       stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia,
+                       H_ > 0 ? 1 : 0);
   });
   check_launch("theta_update");
+  if (H_ > 0) {
+    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 64)), dim3(64), 0, stream, head_logp(), head_aggr(), H_, K_,
+                       pseudocount, inertia);
+    rebuild_heads();
+  }
   hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_, ceil_div(K_, 32)), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_,
                      K_, pseudocount, inertia);
   check_launch("leaf_update");

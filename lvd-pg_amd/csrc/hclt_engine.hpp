@@ -118,7 +118,8 @@ struct HcltDev {
 
 class HcltCircuit : public pcm_circuit {
  public:
-  HcltCircuit(const int32_t* parent, int V, int K, int C);
+  // num_heads > 0: a multi-head circuit, num_heads sum nodes over the root's K products instead of one
+  HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads = 0);
   ~HcltCircuit() override;
 
   int64_t size(int what) const override;
@@ -154,6 +155,14 @@ class HcltCircuit : public pcm_circuit {
 
  private:
   int V_, K_, C_, n_inner_, root_;
+  int H_ = 0, Hp_ = 0;             // heads, and heads rounded up to whole operand tiles
+  DevBuf<float> d_head_wf_, d_head_wb_;   // head block [Hp][K] in the two operand layouts
+  DevBuf<int> d_flow_shift_;              // ceil(log2) of the largest flow one example carried in the last flow pass
+  DevBuf<float> d_ll_heads_;       // scratch: the walk's own root output, per-head values
+  float* head_logp() { return d_logtheta_.p + (size_t)n_inner_ * K_ * K_; }   // [H][K], behind the blocks
+  float* head_aggr() { return d_edge_aggr_.p + (size_t)n_inner_ * K_ * K_; }
+  void rebuild_heads();
+  void heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix);
   bool block_ = true;   // the hidden size has walk kernels (block tiles in registers)
   bool wide_ = false;   // the hidden size has the wide block kernels (likelihoods, flows, EM); neither: layered engine
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;

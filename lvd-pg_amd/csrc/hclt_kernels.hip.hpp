@@ -670,12 +670,13 @@ template <int K>
 __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* __restrict__ nodes,
                                                                 float* __restrict__ logtheta, float* __restrict__ Wf,
                                                                 float* __restrict__ Wb, float* __restrict__ edge_aggr,
-                                                                int n_inner, float pseudocount, float inertia) {
+                                                                int n_inner, float pseudocount, float inertia,
+                                                                int skip_root) {
   constexpr int G = K < 64 ? K : 64, E = K / G, RPB = 256 / G;
   const int row = blockIdx.x * RPB + threadIdx.x / G, l = threadIdx.x % G;
   if (row >= n_inner * K) return;
   const int n = row / K, k = row % K;
-  if (nodes[n].is_root && k > 0) return;
+  if (nodes[n].is_root && (k > 0 || skip_root)) return;   // multi-head circuits keep an identity block at the root
   float* a = edge_aggr + (size_t)row * K;
   float* lt = logtheta + (size_t)row * K;
   const float share = pseudocount / (float)K;

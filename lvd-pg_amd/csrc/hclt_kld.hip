@@ -261,9 +261,10 @@ __global__ __launch_bounds__(256) void hclt_adam_kernel(int64_t ns, const float*
 // ---- host --------------------------------------------------------------------------------
 
 HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
+  if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "KL of multi-head circuits is not defined");
   auto* o = dynamic_cast<HcltCircuit*>(q);
   if (!o) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
-  if (o->K_ != K_ || o->C_ != C_ || o->parent_ != parent_)
+  if (o->K_ != K_ || o->C_ != C_ || o->H_ != H_ || o->parent_ != parent_)
     fail(PCM_ERR_SHAPE, "the two circuits of a KL query must share one structure");
   return o;
 }

@@ -199,6 +199,7 @@ void HcltCircuit::pull_from_general() {
 }
 
 void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
+  if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
   if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   const bool lanes_fit = K_ >= 2 && K_ <= 64 && (K_ & (K_ - 1)) == 0;
@@ -258,6 +259,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
 }
 
 void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
+  if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
   if (sample_soft_block(d_node_noise, temperature, batch, d_out)) return;
   SparseCircuit* g = general();
   DevBuf<int32_t> slots;

@@ -276,7 +276,10 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     lds_tile_load<K>(lds, (int)((slots >> 8) & 0xffu), lane, r);
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt) r.v[kt] *= sinv.v[kt];
-    if (lean_get(sc, kLFlags, s) & 1) {   // flow 1 into the single root sum node of every live example
+    const int fl = lean_get(sc, kLFlags, s);
+    if (fl & 2) {          // multi-head circuit: the head kernel has left the root's ratio tile in memory
+      lean_tile_load<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
+    } else if (fl & 1) {   // flow 1 into the single root sum node of every live example
       const float r00 = (lane < 16 && bcol < d.B) ? sinv.v[0][0] : 0.f;
       tile_zero<K>(r);
       r.v[0][0] = r00;
@@ -313,7 +316,7 @@ constexpr int kStatLeanWaves = 16;
 template <int K>
 __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     HcltDev d, const StatNode* __restrict__ nodes, float* __restrict__ edge_aggr, float* __restrict__ leaf_flow,
-    float rate, int hist_words, int limb) {
+    float rate, int hist_words, int limb, const int* __restrict__ flow_shift) {
   constexpr int KT = K / 16;
   constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
   constexpr int HS = K + 1;    // row stride of a histogram: spreads equal states over banks
@@ -328,7 +331,10 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
   const int hist_sz = d.C * HS;
   unsigned* hist = reinterpret_cast<unsigned*>(smem);
   float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
-  const float scale = __builtin_ldexpf(1.f, limb);
+  // flows lie in [0, 2^shift]: 1 per example in a single-head circuit, the largest total head
+  // mask of an example (found on the device by the head kernel) in a multi-head one
+  const int shift = flow_shift ? __builtin_amdgcn_readfirstlane(*flow_shift) : 0;
+  const float scale = __builtin_ldexpf(1.f, limb), scale_in = __builtin_ldexpf(1.f, limb - shift);
 
   const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + (size_t)n * d.tile_stride, d.tile_stride);
   const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);
@@ -352,7 +358,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 #pragma unroll
     for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  // fixed-point limbs of this lane's K/4 flows (clamped to [0, 1]) into row x of the histogram
+  // fixed-point limbs of this lane's K/4 flows (clamped to [0, 2^shift]) into row x of the histogram
   auto histogram = [&](const Tile<K>& t, uint32_t xpack, int sel) {
     const uint32_t x = (xpack >> (8 * sel)) & 0xffu;
     unsigned* hrow = hist + x * HS + 4 * g;
@@ -360,7 +366,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale, 0.f, scale);
+        const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale_in, 0.f, scale);
         const unsigned hi = (unsigned)v;
         const unsigned lo = (unsigned)(__builtin_amdgcn_fractf(v) * scale);
         __hip_atomic_fetch_add(&hrow[kt * 16 + i], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -471,7 +477,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     }
     __syncthreads();
     {
-      const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+      const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
       float* dst = leaf_flow + (size_t)np->hvar[pass] * d.C * K;
       for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
         const int c = i / K, j = i % K;

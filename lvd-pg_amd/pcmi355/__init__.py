@@ -5,7 +5,8 @@ the host side is Python; names, argument meaning and error behaviour follow the 
 functions cited in each docstring (paths relative to VariationalJuice.jl/).  Device
 memory and streams come from torch; everything numeric happens in the HIP library.
 """
-from .circuits import BitsCircuit, HcltCircuit, hclt_from_clt, compile_circuit, compile_multihead  # noqa: F401
+from .circuits import (BitsCircuit, HcltCircuit, hclt_from_clt, multihead_hclt_from_clt, compile_circuit,  # noqa: F401
+                       compile_multihead)
 from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample)

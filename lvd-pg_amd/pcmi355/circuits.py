@@ -121,6 +121,20 @@ class HcltCircuit(BitsCircuit):
         return dict(forward=float(ms[0]), backward=float(ms[1]), statistics=float(ms[2]))
 
 
+def multihead_hclt_from_clt(clt_parent, num_cats, num_hidden_cats, num_heads):
+    """A multi-head HCLT on the block engine: `num_heads` root sum nodes over the K products of one
+    HCLT body, what `CuMultiHeadBitsProbCircuit(pcs)` (src-jl/multi_head_pc/bit_circuit.jl:14-56) is
+    given by exps/progressive_growing/parallel_PG.jl:214-225.  Raises PcmError (unsupported) for
+    hidden sizes or trees without block kernels: use `compile_multihead` then."""
+    par = np.ascontiguousarray(clt_parent, dtype=np.int32)
+    h = ctypes.c_void_p()
+    check(lib.pcm_hclt_create_multihead(np_ptr(par), len(par), int(num_hidden_cats), int(num_cats), int(num_heads),
+                                        ctypes.byref(h)))
+    c = HcltCircuit(h, par, int(num_cats), int(num_hidden_cats))
+    c.num_heads = int(num_heads)
+    return c
+
+
 def hclt_from_clt(clt_parent, num_cats, num_hidden_cats):
     """`hclt_from_clt(clt, num_cats, num_hidden_cats, variable_groups; input_type = Categorical)`
     (src/structures/hclts.jl:100-145) followed by `CuMetaBitsProbCircuit(pc)`; the tree is

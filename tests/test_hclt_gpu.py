@@ -184,3 +184,56 @@ def test_config_hclt48_k128(gpu, oracle):
     lls = P.mini_batch_em_with_reg(bpc, d, 10, batch_size=B, pseudocount=0.1, param_inertia=0.9, shuffle="none")
     assert all(b > a for a, b in zip(lls, lls[1:])), lls
     np.testing.assert_allclose(lls[0], ll.mean(), rtol=1e-5)
+
+
+@pytest.mark.parametrize("V,K,C,H,B,tree", [(7, 16, 5, 3, 40, None), (12, 32, 9, 128, 70, None), (2, 16, 4, 16, 16, [-1, 0]),
+                                            (9, 32, 256, 40, 33, [-1, 0, 0, 1, 1, 2, 2, 3, 3])])
+def test_multihead_hclt_on_the_block_engine(gpu, oracle, V, K, C, H, B, tree):
+    """H heads over the root's products (src-jl/multi_head_pc/bit_circuit.jl:14-56): the block
+    engine (body through the walk kernels, heads in two small kernels) against the layered engine
+    on the equivalent description and against the oracle: parameter order, per-head likelihoods,
+    mask-weighted mixture, flows with one-hot and soft masks, EM update."""
+    torch, P = gpu
+    O = oracle
+    from helpers import multihead_hclt, describe_dag, correlated_data
+    from pcmi355._lib import lib, check
+    rng = np.random.default_rng(V * 100 + H)
+    parent = O.random_tree(V, rng, 3) if tree is None else np.array(tree, np.int32)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    g = describe_dag(heads)
+    gen = P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"], g["input_logp"],
+                            V, C, H)
+    blk = P.multihead_hclt_from_clt(parent, C, K, H)
+    pv = P.vectorize_parameters(gen)
+    assert blk.num_parameters() == len(pv) and blk.size("heads") == H
+    P.update_parameters(blk, pv)
+    np.testing.assert_array_equal(P.vectorize_parameters(blk), pv)
+    for t in ("edge2param", "param2edge", "pargroup_sizes", "edge_parent", "edge_prime", "edge_sub", "heads"):
+        np.testing.assert_array_equal(blk.table(t), gen.table(t), err_msg=t)
+    data = correlated_data(B, V, C, 5, parent)
+    d = torch.from_numpy(data).cuda()
+    ll_g = P.loglikelihoods(gen, d).cpu().numpy()
+    ll_b = P.loglikelihoods(blk, d).cpu().numpy()
+    assert ll_b.shape == (B, H)
+    np.testing.assert_allclose(ll_b, ll_g, rtol=2e-5)
+    fc = O.bits_compile(O.summate(*heads), C, V)                      # the oracle on the same description
+    mars = O.forward(fc, data)
+    np.testing.assert_allclose(ll_b, mars[(blk.table("heads") - 1).astype(np.int64)].T, rtol=2e-5)
+    for soft in (False, True):
+        mask = np.zeros((B, H), np.float32)
+        mask[np.arange(B), rng.integers(0, H, B)] = 1.0
+        if soft:
+            mask = (mask + rng.random((B, H)).astype(np.float32) * (rng.random((B, H)) < 0.3)).astype(np.float32)
+        hm = torch.from_numpy(mask).cuda()
+        mix_g = P.probs_flows_circuit(gen, d, head_mask=hm, rate=0.25 if soft else 0.0).cpu().numpy()
+        mix_b = P.probs_flows_circuit(blk, d, head_mask=hm, rate=0.25 if soft else 0.0).cpu().numpy()
+        np.testing.assert_allclose(mix_b, mix_g, rtol=2e-5)
+        np.testing.assert_allclose(mix_b, P.multihead_loglikelihoods(blk, d, hm).cpu().numpy(), rtol=2e-5)
+        check(lib.pcm_em_update(gen.handle, 0.1, 0.7))
+        check(lib.pcm_em_update(blk.handle, 0.1, 0.7))
+        a, b = P.vectorize_parameters(gen), P.vectorize_parameters(blk)
+        assert np.abs(np.exp(a) - np.exp(b)).max() < 5e-4 * np.exp(a).max()
+    with pytest.raises(P.PcmError):
+        P.kld(blk, blk)
+    with pytest.raises(P.PcmError):                                    # a node with four children: no lean kernels
+        P.multihead_hclt_from_clt(np.array([-1, 0, 0, 0, 0, 1], np.int32), C, K, H)
