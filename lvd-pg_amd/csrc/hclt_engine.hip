@@ -701,10 +701,12 @@ void HcltCircuit::rebuild_heads() {
 }
 
 // head values from the root tile the forward walk has left (identity block: the root's Z)
-void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix) {
+void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow,
+                                float rate) {
   const float* o_root = d.O + (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
   PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), 0, stream,
-                                             o_root, d_head_wf_.p, H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix));
+                                             o_root, d_head_wf_.p, H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix,
+                                             flows_follow ? head_aggr() : (float*)nullptr, rate, d_flow_shift_.p));
   check_launch("heads_forward");
 }
 
@@ -931,12 +933,15 @@ void HcltCircuit::run_backward(const HcltDev& d) {
                        bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
+  if (H_ > 0 && !small) fail(PCM_ERR_UNSUPPORTED, "multi-head HCLT: batch of %d examples is too large for one call", d.B);
   if (bwd_lean_ && small) {
+    auto launch_lean = [&](auto kernel) {
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_lean_.p, bwd_stride_,
+                         n_bwd_steps_);
+    };
     PCM_DISPATCH_LEAN_K(K_, {
-      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_backward_lean_kernel<KK>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      hipLaunchKernelGGL(hclt_backward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d,
-                         d_bwd_lean_.p, bwd_stride_, n_bwd_steps_);
+      if (H_ > 0) launch_lean(&hclt_backward_lean_kernel<KK, true>); else launch_lean(&hclt_backward_lean_kernel<KK, false>);
     });
   } else {
     PCM_DISPATCH_K(K_, {
@@ -1036,9 +1041,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   if (H_ > 0) {
     d_ll_heads_.ensure((size_t)b.batch);
     run_forward(d, d_ll_heads_.p);
-    heads_forward(d, d_head_mask, nullptr, d_ll);
-    hipLaunchKernelGGL(hclt_scale_kernel, dim3(ceil_div((int64_t)H_ * K_, 256)), dim3(256), 0, stream, head_aggr(),
-                       (int64_t)H_ * K_, rate, d_flow_shift_.p);
+    heads_forward(d, d_head_mask, nullptr, d_ll, true, rate);
     const size_t root_tile = (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
     const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_) * sizeof(float);
     PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,
@@ -1159,12 +1162,12 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
   });
   check_launch("theta_update");
   if (H_ > 0) {
-    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 64)), dim3(64), 0, stream, head_logp(), head_aggr(), H_, K_,
-                       pseudocount, inertia);
-    rebuild_heads();
+    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4)), dim3(256), 0, stream, head_logp(), head_aggr(), H_, Hp_,
+                       K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
   }
-  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_, ceil_div(K_, 32)), dim3(256), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_,
-                     K_, pseudocount, inertia);
+  // few variables: more category groups per workgroup, for the latency of the two passes
+  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_, ceil_div(K_, 32)), dim3(V_ * ceil_div(K_, 32) < 1024 ? 1024 : 256), 0,
+                     stream, d_leaf_.p, d_leaf_flow_.p, C_, K_, pseudocount, inertia);
   check_launch("leaf_update");
   general_stale_ = true;
 }

@@ -162,7 +162,8 @@ class HcltCircuit : public pcm_circuit {
   float* head_logp() { return d_logtheta_.p + (size_t)n_inner_ * K_ * K_; }   // [H][K], behind the blocks
   float* head_aggr() { return d_edge_aggr_.p + (size_t)n_inner_ * K_ * K_; }
   void rebuild_heads();
-  void heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix);
+  void heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow = false,
+                     float rate = 0.f);
   bool block_ = true;   // the hidden size has walk kernels (block tiles in registers)
   bool wide_ = false;   // the hidden size has the wide block kernels (likelihoods, flows, EM); neither: layered engine
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;

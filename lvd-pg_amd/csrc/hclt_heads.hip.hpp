@@ -75,9 +75,16 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
                                                                              const float* __restrict__ hwf, int H, int Hp,
                                                                              int B, const float* __restrict__ mask,
                                                                              float* __restrict__ ll_heads,
-                                                                             float* __restrict__ ll_mix) {
+                                                                             float* __restrict__ ll_mix,
+                                                                             float* __restrict__ head_aggr, float rate,
+                                                                             int* __restrict__ flow_shift) {
   __shared__ float pm[kHeadWaves * 4][16], ps[kHeadWaves * 4][16], pt[kHeadWaves * 4][16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x;
+  if (head_aggr) {   // ahead of a flow pass: previous head statistics times the flow memory rate, flow bound cleared
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < H * K; i += gridDim.x * blockDim.x)
+      head_aggr[i] = rate != 0.f ? head_aggr[i] * rate : 0.f;
+    if (blockIdx.x == 0 && threadIdx.x == 0) *flow_shift = 0;
+  }
   const int b = lane & 15, g = lane >> 4, col = slice * kSlice + b;
   Tile<K> e;
   const float m = heads_load_e<K>(O_root, slice, lane, e);
@@ -184,24 +191,27 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
   }
 }
 
-// add_pseudocount / aggr_node_flows / update_params for the head sum nodes (one thread per head)
-__global__ void hclt_heads_update_kernel(float* __restrict__ head_logp, float* __restrict__ head_aggr, int H, int K,
-                                         float pseudocount, float inertia) {
-  const int h = blockIdx.x * blockDim.x + threadIdx.x;
+// add_pseudocount / aggr_node_flows / update_params for the head sum nodes (one wave per head);
+// also refreshes the two operand layouts (their padding rows stay zero)
+__global__ __launch_bounds__(256) void hclt_heads_update_kernel(float* __restrict__ head_logp, float* __restrict__ head_aggr,
+                                                                int H, int Hp, int K, float pseudocount, float inertia,
+                                                                float* __restrict__ hwf, float* __restrict__ hwb) {
+  const int lane = threadIdx.x & 63;
+  const int h = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (h >= H) return;
   float* a = head_aggr + (size_t)h * K;
   float* lt = head_logp + (size_t)h * K;
   const float share = pseudocount / (float)K;
   float tot = 0.f;
-  for (int j = 0; j < K; ++j) { a[j] += share; tot += a[j]; }
-  for (int j = 0; j < K; ++j) lt[j] = logf(inertia * expf(lt[j]) + (1.f - inertia) * a[j] / tot);
-}
-
-// previous head statistics times the flow memory rate; also clears the flow bound
-__global__ void hclt_scale_kernel(float* p, int64_t n, float rate, int* __restrict__ flow_shift) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i == 0) *flow_shift = 0;
-  if (i < n) p[i] = rate != 0.f ? p[i] * rate : 0.f;
+  for (int j = lane; j < K; j += 64) { a[j] += share; tot += a[j]; }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) tot += __shfl_xor(tot, o);
+  for (int j = lane; j < K; j += 64) {
+    const float w = inertia * expf(lt[j]) + (1.f - inertia) * a[j] / tot;
+    lt[j] = logf(w);
+    hwf[head_wf_at(h, j, K)] = w;
+    hwb[head_wb_at(h, j, Hp)] = w;
+  }
 }
 
 }  // namespace pcm

@@ -704,12 +704,12 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
 // per (variable, run of 32 hidden states): thread (category group cg, hidden state j) first
 // sums the flows of its categories, the groups are combined through LDS, then every thread
 // rewrites its categories.  Consecutive threads touch consecutive addresses in both passes.
-__global__ __launch_bounds__(256) void hclt_leaf_update_kernel(float* __restrict__ leaf,
+__global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restrict__ leaf,
                                                                const float* __restrict__ leaf_flow, int C, int K,
                                                                float pseudocount, float inertia) {
-  __shared__ float part[256];
+  __shared__ float part[1024];
   const int u = blockIdx.x;
-  const int jl = threadIdx.x & 31, cg = threadIdx.x >> 5, ncg = 8;
+  const int jl = threadIdx.x & 31, cg = threadIdx.x >> 5, ncg = blockDim.x >> 5;
   const int j = blockIdx.y * 32 + jl;
   const bool valid = j < K;
   float* lp = leaf + (size_t)u * C * K;

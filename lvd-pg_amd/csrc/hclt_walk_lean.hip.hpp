@@ -202,7 +202,9 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
 }
 
 // ---- backward -----------------------------------------------------------------------------
-template <int K>
+// kHeads: multi-head circuit, whose head kernel has left the root's ratio tile in memory (a
+// build of its own: the extra load in the root branch costs the single-head walk 5%).
+template <int K, bool kHeads>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps) {
   extern __shared__ float lds[];
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt) r.v[kt] *= sinv.v[kt];
     const int fl = lean_get(sc, kLFlags, s);
-    if (fl & 2) {          // multi-head circuit: the head kernel has left the root's ratio tile in memory
+    if (kHeads && (fl & 2)) {   // multi-head circuit: the head kernel has left the root's ratio tile in memory
       lean_tile_load<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
     } else if (fl & 1) {   // flow 1 into the single root sum node of every live example
       const float r00 = (lane < 16 && bcol < d.B) ? sinv.v[0][0] : 0.f;

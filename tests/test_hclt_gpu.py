@@ -233,6 +233,9 @@ def test_multihead_hclt_on_the_block_engine(gpu, oracle, V, K, C, H, B, tree):
         check(lib.pcm_em_update(blk.handle, 0.1, 0.7))
         a, b = P.vectorize_parameters(gen), P.vectorize_parameters(blk)
         assert np.abs(np.exp(a) - np.exp(b)).max() < 5e-4 * np.exp(a).max()
+    P.update_parameters(blk, pv)
+    lls = P.mini_batch_em_for_multihead_pc(blk, d, hm, 3, batch_size=B, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert lls[2] > lls[1] > lls[0]
     with pytest.raises(P.PcmError):
         P.kld(blk, blk)
     with pytest.raises(P.PcmError):                                    # a node with four children: no lean kernels
