@@ -94,7 +94,8 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
  * (src/bits_circuit.jl:119-131).  what: 0 parameters, 1 sum parameters, 2 nodes,
  * 3 edges, 4 input parameters, 5 variables, 6 categories, 7 hidden categories (0 if not an
  * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes,
- * 12 heads (0 for a single-root circuit). */
+ * 12 heads (0 for a single-root circuit), 13 nodes of the description the circuit was
+ * built from (0 for an HCLT built from its tree). */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.
@@ -102,7 +103,11 @@ int64_t pcm_size(const pcm_circuit* c, int32_t what);
  * parameters], 3 pargroup_sizes [groups], 4 innode2ncumparam [input nodes],
  * 5 up-layer ends [layers], 6 edge parent ids, 7 edge prime ids, 8 edge sub ids (0: none)
  * [edges, up order], 9 head node ids (`root_ids`, src-jl/multi_head_pc/bit_circuit.jl:38-51)
- * [heads].  n must equal the table length. */
+ * [heads], 10 node id of every node of the description given to pcm_circuit_create, 0 where
+ * the node was folded into an edge or cannot be reached from a root (the inverse of the
+ * reference's `bpc.nodes_map`, used by src-jl/multi_head_pc/prune.jl:38-57 and
+ * transformation.jl:132-135) [description nodes], 11 input node ids in parameter order
+ * (`bpc.input_node_ids`) [input nodes].  n must equal the table length. */
 int pcm_index_table(const pcm_circuit* c, int32_t which, int64_t* out, int64_t n);
 
 /* ---- parameters --------------------------------------------------------------- */
@@ -172,6 +177,10 @@ int pcm_em_step(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_
  * [num_nodes][batch] (the reference's `mars` / `flows`, transposed), and of the
  * accumulators: edge_aggr [edges, up order], leaf_flow [input parameters]. */
 int pcm_get_node_values(pcm_circuit* c, float* mars, float* flows, int64_t n);
+/* General circuits: out[n] = sum over the examples of the last pcm_flows batch of the flow of
+ * node n, host array [num_nodes] (`sum(flows[1:batch, :]; dims = 1)`,
+ * src-jl/multi_head_pc/transformation.jl:121). */
+int pcm_node_flow_sums(pcm_circuit* c, float* out, int64_t n);
 int pcm_get_aggregates(pcm_circuit* c, float* edge_aggr, int64_t n_edges, float* leaf_flow,
                        int64_t n_leaf);
 

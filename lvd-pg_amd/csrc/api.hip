@@ -151,6 +151,14 @@ int pcm_get_node_values(pcm_circuit* c, float* mars, float* flows, int64_t n) {
     s->get_node_values(mars, flows, n);
   });
 }
+int pcm_node_flow_sums(pcm_circuit* c, float* out, int64_t n) {
+  return guarded([&] {
+    auto* s = dynamic_cast<pcm::SparseCircuit*>(need(c));
+    if (!s) pcm::fail(PCM_ERR_UNSUPPORTED, "node flows exist only for circuits built from a description (pcm_circuit_create)");
+    s->node_flow_sums(out, n);
+  });
+}
+
 int pcm_get_aggregates(pcm_circuit* c, float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf) {
   return guarded([&] {
     auto* s = dynamic_cast<pcm::SparseCircuit*>(need(c));

@@ -137,6 +137,9 @@ FlatCircuit flatten_dag(int32_t num_nodes, const uint8_t* node_type, const int32
     fc.heads.push_back(materialize(memo[root]));
   }
   if (num_heads == 0) fc.heads.clear();
+  fc.desc_node.assign(num_nodes, -1);
+  for (int n = 0; n < num_nodes; ++n)
+    if (memo[n].kind == 0) fc.desc_node[n] = memo[n].a;
 
   // layers and up-edge order
   const int64_t nn = fc.n_nodes();
@@ -971,6 +974,7 @@ int64_t SparseCircuit::size(int what) const {
     case 10: return (int64_t)fc_.pargroup_sizes.size();
     case 11: return (int64_t)fc_.input_nodes.size();
     case 12: return fc_.num_heads;
+    case 13: return (int64_t)fc_.desc_node.size();
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -993,6 +997,8 @@ void SparseCircuit::index_table(int which, int64_t* out, int64_t n) const {
     case 7: copy(plus1(fc_.e_prime)); break;
     case 8: copy(plus1(fc_.e_sub)); break;
     case 9: copy(plus1(fc_.heads)); break;
+    case 10: copy(plus1(fc_.desc_node)); break;
+    case 11: copy(plus1(fc_.input_nodes)); break;
     default: fail(PCM_ERR_ARG, "unknown index table %d", which);
   }
 }
@@ -1095,6 +1101,7 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
   }
   check_launch("sparse_forward");
   last_batch_ = batch;
+  flow_batch_ = 0;       // the flow array belongs to an earlier batch
 }
 
 // root (or head) rows -> output; the root is the last node
@@ -1184,6 +1191,7 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     check_launch("head_mixture");
   }
   have_flows_ = true;
+  flow_batch_ = last_batch_;
 }
 
 void SparseCircuit::em_update(float pseudocount, float inertia) {
@@ -1207,6 +1215,33 @@ void SparseCircuit::get_node_values(float* mars, float* flows, int64_t n) {
     fetch(h, pass ? d_flows_.p : d_mars_.p, (size_t)fc_.n_nodes() * Bp, stream);
     for (int64_t i = 0; i < fc_.n_nodes(); ++i) std::copy(h.begin() + i * Bp, h.begin() + i * Bp + B, dst + i * B);
   }
+}
+
+// out[n] = sum over the examples of the last flow pass of flows[n][b] (one wave per node)
+__global__ __launch_bounds__(256) void sparse_node_flow_sum_kernel(const float* __restrict__ flows, int64_t n_nodes, int B, int Bp,
+                                                                   float* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t n = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (n >= n_nodes) return;
+  const float* row = flows + n * Bp;
+  float s = 0.f;
+  for (int b = lane; b < B; b += 64) s += row[b];
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) out[n] = s;
+}
+
+void SparseCircuit::node_flow_sums(float* out, int64_t n) {
+  if (!have_flows_ || !flow_batch_) fail(PCM_ERR_STATE, "the node flows of the last batch are gone (call pcm_flows first)");
+  if (!out) fail(PCM_ERR_ARG, "output pointer is null");
+  if (n != fc_.n_nodes()) fail(PCM_ERR_ARG, "circuit has %lld nodes, caller gave %lld", (long long)fc_.n_nodes(), (long long)n);
+  const int B = flow_batch_, Bp = ceil_div(B, 64) * 64;
+  d_node_sums_.ensure((size_t)n);
+  hipLaunchKernelGGL(sparse_node_flow_sum_kernel, dim3((unsigned)ceil_div(n, 4)), dim3(256), 0, stream, d_flows_.p, n, B, Bp,
+                     d_node_sums_.p);
+  check_launch("node_flow_sums");
+  PCM_HIP(hipMemcpyAsync(out, d_node_sums_.p, n * sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
 }
 
 void SparseCircuit::get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf) {
@@ -1374,6 +1409,7 @@ void SparseCircuit::sample_soft_with_slots(const float* d_node_noise, const int3
   check_launch("sparse_sample_soft");
   PCM_HIP(hipStreamSynchronize(stream));
   last_batch_ = 0;       // the value / flow arrays no longer hold a batch
+  flow_batch_ = 0;
   have_flows_ = false;
 }
 

@@ -28,6 +28,7 @@ struct FlatCircuit {
   std::vector<int64_t> layer_ends;                   // edge count at the end of each up layer
   std::vector<float> leaf_logp;                      // [inputs * C]
   std::vector<int32_t> heads;                        // node ids of the heads (multi-head)
+  std::vector<int32_t> desc_node;                    // per node of the description: its node id, -1 where it was folded into an edge or is unreachable
   // parameter tables (1-based, src/bits_circuit.jl:46-70)
   std::vector<int64_t> edge2param, param2edge, param2group, pargroup_sizes;
   int64_t n_nodes() const { return (int64_t)type.size(); }
@@ -67,6 +68,7 @@ class SparseCircuit : public pcm_circuit {
 
   void get_node_values(float* mars, float* flows, int64_t n);
   void get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf);
+  void node_flow_sums(float* out, int64_t n);
 
   // device views for engines that embed a general circuit (the HCLT engine's KL / sampling)
   float* d_logp() { return d_logp_.p; }
@@ -100,6 +102,8 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
   int cap_batch_ = 0, last_batch_ = 0, max_var_nodes_ = 1;
   bool have_flows_ = false;
+  int flow_batch_ = 0;   // examples whose node flows d_flows_ holds (0: none)
+  DevBuf<float> d_node_sums_;
 
   void ensure_batch(int batch);
   void ensure_var_tables();

@@ -42,6 +42,7 @@ _SIGS = {
     "pcm_em_step": [H, vp, c_i64, c_i64, vp, c_i32, c_f32, c_f32, c_f32, vp],
     "pcm_get_node_values": [H, vp, vp, c_i64],
     "pcm_get_aggregates": [H, vp, c_i64, vp, c_i64],
+    "pcm_node_flow_sums": [H, vp, c_i64],
     "pcm_kld": [H, H, vp],
     "pcm_kld_backward": [H, H, vp, vp, c_i64],
     "pcm_kld_backward_dev": [H, H, vp, vp, c_i64],

@@ -6,10 +6,12 @@ import numpy as np
 from ._lib import lib, check, np_ptr, H, c_i64
 
 _SIZE = dict(parameters=0, sum_parameters=1, nodes=2, edges=3, input_parameters=4, variables=5,
-             categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11, heads=12)
+             categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11, heads=12,
+             description_nodes=13)
 _TABLE = dict(edge2param=(0, "edges"), param2edge=(1, "sum_parameters"), param2group=(2, "sum_parameters"),
               pargroup_sizes=(3, "groups"), innode2ncumparam=(4, "input_nodes"), layer_ends=(5, "layers"),
-              edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"), heads=(9, "heads"))
+              edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"), heads=(9, "heads"),
+              description2node=(10, "description_nodes"), input_node_ids=(11, "input_nodes"))
 
 
 class BitsCircuit:
@@ -70,6 +72,12 @@ class BitsCircuit:
         fl = np.empty((n, batch), np.float32) if flows else None
         check(lib.pcm_get_node_values(self.handle, np_ptr(mars), np_ptr(fl), c_i64(n * batch)))
         return (mars, fl) if flows else mars
+
+    def node_flow_sums(self):
+        """Flow of every node summed over the examples of the last flow pass, [num_nodes]."""
+        out = np.empty(self.num_nodes(), np.float32)
+        check(lib.pcm_node_flow_sums(self.handle, np_ptr(out), c_i64(len(out))))
+        return out
 
     def get_aggregates(self):
         """(edge_aggr [edges, up order], leaf flows [input parameters]) accumulated so far."""
@@ -169,3 +177,72 @@ def compile_multihead(node_type, child_ptr, child_idx, sum_logp, input_var, inpu
     last `num_heads` nodes of the description are the heads."""
     return compile_circuit(node_type, child_ptr, child_idx, sum_logp, input_var, input_logp, num_vars,
                            num_cats, num_heads)
+
+
+def _compile_nodes(pcs, num_vars, heads):
+    from . import nodes as N
+    desc, order = N.describe(pcs)
+    if num_vars is None:
+        num_vars = int(desc["input_var"].max()) + 1
+    c = compile_circuit(desc["node_type"], desc["child_ptr"], desc["child_idx"], desc["sum_logp"], desc["input_var"],
+                        desc["input_logp"], num_vars, desc["num_cats"], heads)
+    c.nodes = order            # description order: c.table("description2node")[i] is the node id of c.nodes[i]
+    c.pcs = list(pcs) if heads else pcs
+    return c
+
+
+def CuBitsProbCircuit(pc, num_vars=None):
+    """`CuBitsProbCircuit(pc)` / `CuMetaBitsProbCircuit(pc)` (src/bits_circuit.jl:39) for a
+    circuit given as a DAG of `pcmi355.nodes`."""
+    return _compile_nodes(pc, num_vars, 0)
+
+
+def CuMultiHeadBitsProbCircuit(pcs, num_vars=None):
+    """`CuMultiHeadBitsProbCircuit(pcs)` (src-jl/multi_head_pc/bit_circuit.jl:14-56): the roots
+    `pcs` share one body and become the heads, in order."""
+    pcs = list(pcs)
+    if not pcs:
+        raise ValueError("no heads given")
+    return _compile_nodes(pcs, num_vars, len(pcs))
+
+
+def node_maps(bpc):
+    """(node id -> DAG node, DAG node -> node id) of a circuit compiled from `pcmi355.nodes`
+    (`bpc.nodes_map` and its inverse, src-jl/multi_head_pc/transformation.jl:132-135).  Node ids
+    are 1-based; DAG nodes that were folded into an edge have none, and of the DAG nodes that
+    share an id (a node and its only child) the map keeps the one that owns the edges."""
+    d2n = bpc.table("description2node")
+    node2id, nodes_map = {}, {}
+    for n, f in zip(bpc.nodes, d2n):
+        if f > 0:
+            node2id[id(n)] = int(f)
+            if int(f) not in nodes_map or len(n.inputs) > 1:
+                nodes_map[int(f)] = n
+    return nodes_map, node2id
+
+
+def write_back_parameters(bpc):
+    """`update_parameters(bpc)` of ProbabilisticCircuits.jl as
+    exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl:186 calls it: copies the device
+    parameters into the DAG nodes the circuit was compiled from."""
+    from .queries import vectorize_parameters
+    pv = vectorize_parameters(bpc)
+    nodes_map, _ = node_maps(bpc)
+    e2p = bpc.table("edge2param")
+    parent = bpc.table("edge_parent")
+    pos = 0
+    while pos < len(parent):
+        end = pos
+        while end < len(parent) and parent[end] == parent[pos]:
+            end += 1
+        n = nodes_map.get(int(parent[pos]))
+        if n is not None and n.kind == 1 and e2p[pos] > 0:      # a run of product edges can carry the id of a one-child sum
+            if len(n.params) != end - pos:
+                raise RuntimeError("edge run does not match the sum node's children")
+            n.params = pv[e2p[pos:end] - 1].astype(np.float32)
+        pos = end
+    ns = bpc.num_inner_params()
+    C = bpc.num_cats
+    for i, f in enumerate(bpc.table("input_node_ids")):
+        n = nodes_map[int(f)]
+        n.logps = pv[ns + i * C: ns + (i + 1) * C].astype(np.float32)

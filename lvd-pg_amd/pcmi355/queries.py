@@ -253,3 +253,26 @@ def adam_step(bpc, grad, params, m, v, *, lr, beta1=0.9, beta2=0.999, eps=1e-8, 
     update of the unnormalised sum parameters, per-node normalisation into the circuit."""
     check(lib.pcm_adam_step(bpc.handle, grad.data_ptr(), params.data_ptr(), m.data_ptr(), v.data_ptr(),
                             float(lr), float(beta1), float(beta2), float(eps), int(t)))
+
+
+def patch_level_evidence(mhbpcs, patches, batch_size=256):
+    """The pseudo dataset of the top-level circuit
+    (exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl:82-118): for every patch (a uint8
+    device tensor [N, patch variables]) the per-head log-likelihoods of every multi-head patch
+    circuit, heads of all circuits side by side.  Returns float32 [N, patches, heads in total],
+    the soft-evidence input of `mini_batch_em_with_reg` / `loglikelihoods`."""
+    mhbpcs = list(mhbpcs)
+    total = sum(max(getattr(m, "num_heads", 0), 1) for m in mhbpcs)
+    n = patches[0].shape[0]
+    out = torch.empty((n, len(patches), total), dtype=torch.float32, device=patches[0].device)
+    for p, x in enumerate(patches):
+        if x.shape[0] != n:
+            raise ValueError("every patch must hold the same examples")
+        x = x.contiguous()
+        h0 = 0
+        for m in mhbpcs:
+            ll = loglikelihoods(m, x, batch_size=min(batch_size, n))
+            ll = ll if ll.dim() == 2 else ll[:, None]
+            out[:, p, h0:h0 + ll.shape[1]] = ll
+            h0 += ll.shape[1]
+    return out

@@ -153,3 +153,34 @@ def multihead_hclt(parent, K, C, H, rng):
     prods = root.children
     heads = [O.summate(*prods, logps=log_dirichlet(rng, len(prods))) for _ in range(H)]
     return heads, root
+
+
+def to_oracle_dag(pcs):
+    """pcmi355.nodes DAG -> pc_oracle.Node DAG (shared nodes stay shared).  Returns the list of
+    converted roots and the map id(product node) -> oracle node."""
+    from pcmi355 import nodes as N
+    roots = list(pcs) if isinstance(pcs, (list, tuple)) else [pcs]
+    conv = {}
+    for n in N.linearize(roots):
+        if n.kind == N.INPUT:
+            conv[id(n)] = O.input_node(n.var, n.logps)
+        elif n.kind == N.MUL:
+            conv[id(n)] = O.multiply(*[conv[id(c)] for c in n.inputs])
+        else:
+            conv[id(n)] = O.summate(*[conv[id(c)] for c in n.inputs], logps=n.params)
+    return [conv[id(r)] for r in roots], conv
+
+
+def from_oracle_dag(roots):
+    """pc_oracle.Node DAG -> pcmi355.nodes DAG.  Returns (converted roots, map id(oracle node) -> node)."""
+    import dag_oracle
+    from pcmi355 import nodes as N
+    conv = {}
+    for n in dag_oracle.topo(list(roots)):
+        if n.kind == O.INPUT:
+            conv[id(n)] = N.input_node(n.var, n.logps)
+        elif n.kind == O.MUL:
+            conv[id(n)] = N.multiply([conv[id(c)] for c in n.children])
+        else:
+            conv[id(n)] = N.summate([conv[id(c)] for c in n.children], params=n.logps)
+    return [conv[id(r)] for r in roots], conv

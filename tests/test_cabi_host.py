@@ -70,6 +70,8 @@ def test_version_and_error_reporting_without_a_gpu(cdll):
     assert list(parent) == [1, -1, 1]                     # path 0 - 1 - 2, rooted at its centre
     assert cdll.pcm_loglikelihoods_soft(None, None, i64(1), i64(1), i64(1), None, 4, None) == -1
     assert cdll.pcm_flows_soft(None, None, i64(1), i64(1), i64(1), None, 4, f32(0), None, None) == -1
+    assert cdll.pcm_node_flow_sums(None, None, i64(0)) == -1
+    assert cdll.pcm_hclt_create_multihead(par, 2, 16, 8, 5000, ctypes.byref(out)) == -2
 
 
 def test_python_mirror_binds_every_symbol():
