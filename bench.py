@@ -247,8 +247,10 @@ def secondary(args):
             check(lib.pcm_em_update(bpc.handle, 0.1, 0.9))
         dt = _timed(torch, step, args.steps, args.warmup)
         nn, ne = bpc.num_nodes(), bpc.num_edges()
-        algo = B * (8 * nn + 24 * ne) + 2 * 4 * B * V * C * K       # + the evidence, read once per input node going up and down
-        out.update(metric="examples/sec fwd+bwd+EM on soft evidence, 64-var HCLT K=64, 128 categories (layered engine)",
+        # block form: the step's six K-vectors per tree node and example, the evidence read going up and down, the
+        # per-example value table written once and read twice (up, down) and once more for the flows
+        algo = algorithmic_bytes(bpc.size("inner_tree_nodes"), V, K, C, B)["step"] + 2 * 4 * B * V * C + 4 * 4 * B * V * K
+        out.update(metric="examples/sec fwd+bwd+EM on soft evidence, 64-var HCLT K=64, 128 categories (block engine)",
                    value=B / dt, unit="examples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
                            "nodes": nn, "edges": ne})

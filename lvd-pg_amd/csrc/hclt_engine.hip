@@ -10,6 +10,7 @@
 #include "hclt_walk_lean.hip.hpp"
 #include "hclt_soft_sample.hip.hpp"
 #include "hclt_heads.hip.hpp"
+#include "hclt_soft_evidence.hip.hpp"
 
 namespace pcm {
 
@@ -40,6 +41,10 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
   build_structure();
+  // K = 64: a parameter block and its prefetched successor do not fit the 128 registers a wave of the 16-wave
+  // walk kernels has, so those kernels spill (6 us per step); the node-at-a-time wide kernels take about
+  // kWideNodeUs per node instead and win unless the tree is bushy enough to fill the 16 waves of a step
+  wide_walk_ = wide_ || (K == 64 && (double)n_inner_ * kWideNodeUs < (double)(n_fwd_steps_ + n_bwd_steps_) * 0.5 * kWalk64StepUs);
   if (H_ > 0 && !(block_ && fwd_lean_ && bwd_lean_ && stat_lean_))
     fail(PCM_ERR_UNSUPPORTED, "multi-head block kernels need K = 16 or 32 and at most three children per tree node; "
                               "compile this circuit with pcm_circuit_create");
@@ -852,7 +857,11 @@ void HcltCircuit::ensure_batch(int batch) {
   }
   d_O_.alloc((size_t)(n_inner_ + 1) * tile);   // row n_inner: trash tile of idle waves
   d_R_.alloc((size_t)(n_inner_ + 1) * tile);
-  if (bwd_spill_) d_G_.alloc((size_t)n_inner_ * tile);
+  if (bwd_spill_ || wide_walk_) d_G_.alloc((size_t)n_inner_ * tile);
+  if (wide_walk_) {
+    d_wide_rs_.alloc((size_t)n_inner_ * tile);
+    d_wide_es_.alloc((size_t)n_inner_ * tile);
+  }
   d_xb_.alloc((size_t)V_ * ns * kSlice);
   d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
   d_xn_.zero();
@@ -881,6 +890,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.n_inner = n_inner_;
   d.V = V_;
   d.leaf_stride = (uint32_t)C_ * K_ * 4;
+  d.leaf_slice = 0;
   d.tile_stride = (uint32_t)d.nslices * kSlice * K_ * 4;
   return d;
 }
@@ -893,7 +903,7 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
                      b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
   check_launch("stage_batch");
-  if (wide_) return;
+  if (wide_walk_) return;
   hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
   check_launch("pack_x");
@@ -909,7 +919,7 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
   };
   // the lean kernels address every array with 32-bit offsets from one descriptor
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
-  if (fwd_lean_ && small) {
+  if (fwd_lean_ && small && !force_general_walks_) {
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -934,7 +944,7 @@ void HcltCircuit::run_backward(const HcltDev& d) {
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
   if (H_ > 0 && !small) fail(PCM_ERR_UNSUPPORTED, "multi-head HCLT: batch of %d examples is too large for one call", d.B);
-  if (bwd_lean_ && small) {
+  if (bwd_lean_ && small && !force_general_walks_) {
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_lean_.p, bwd_stride_,
@@ -959,7 +969,7 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   const size_t hist = 2 * (size_t)C_ * (K_ + 1);                    // words per histogram (two limbs)
-  if (stat_lean_) {
+  if (stat_lean_ && !force_general_walks_) {
     // LDS: one histogram (or the parked edge-flow blocks, whichever is larger) | per-wave pads
     const size_t park = (size_t)kStatLeanWaves * K_ * K_;
     const size_t hw = (std::max(hist, park) + 3) & ~(size_t)3;
@@ -986,11 +996,13 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   const size_t lds = (hist_words(nh) + pads) * 4;
   if (lds > (size_t)max_lds_)
     fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", lds, max_lds_);
+  auto launch = [&](auto kernel) {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, stream, d, d_stat_items_.p, d_edge_aggr_.p,
+                       d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb);
+  };
   PCM_DISPATCH_K(K_, {
-    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_kernel<KK>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(hclt_stats_kernel<KK>, dim3(n_inner_), dim3(kStatWaves * 64), lds, stream, d,
-                       d_stat_items_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb);
+    if (d.leaf_slice != 0) launch(&hclt_stats_kernel<KK, true>); else launch(&hclt_stats_kernel<KK, false>);
   });
   check_launch("hclt_stats");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
@@ -1000,7 +1012,7 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (!block_ && !wide_) return general()->loglikelihoods(b, d_ll);
   stage_batch(b);
-  if (wide_) return wide_forward(dev(b.batch), d_ll);
+  if (wide_walk_) return wide_forward(dev(b.batch), d_ll);
   if (H_ > 0) {   // per-head values [H][batch]
     d_ll_heads_.ensure((size_t)b.batch);
     const HcltDev d = dev(b.batch);
@@ -1013,10 +1025,89 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
 
 // Soft evidence (src/regularization/reg_likelihood.jl:51-91, reg_flow.jl:50-82) runs on the layered
 // engine over the circuit's general form for every hidden size.
-void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) { general()->loglikelihoods_soft(s, d_ll); }
+// Single-head circuits with K <= 64 take it on the block kernels: a value table [V][Bp][K] of the
+// batch stands in for the leaf table (hclt_soft_evidence.hip.hpp).
+HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
+  if (!s.d_ev) fail(PCM_ERR_ARG, "evidence pointer is null");
+  if (s.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", s.batch);
+  ensure_batch(s.batch);
+  HcltDev d = dev(s.batch);
+  if ((size_t)d.Bp * K_ * 4 >= ((size_t)1 << 31)) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", s.batch);
+  const int64_t nx = (int64_t)V_ * d.Bp;
+  hipLaunchKernelGGL(hclt_soft_x_kernel, dim3(ceil_div(nx, 256)), dim3(256), 0, stream, d_xb_.p, nx);
+  if (!wide_walk_)
+    hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(d.Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
+                       d_child_leaf_.p, d_xb_.p, n_inner_, d.Bp, d_xn_.p);
+  check_launch("soft pack_x");
+  const int Bp64 = ceil_div(d.Bp, kEvExamples) * kEvExamples;
+  d_soft_lv_.ensure((size_t)V_ * Bp64 * K_);
+  d_soft_m_.ensure((size_t)V_ * Bp64);
+  const int Cp = (C_ + 3) & ~3;
+  const size_t lds = ((size_t)kEvExamples * (Cp + 4) + (size_t)Cp * (K_ + 16) + kEvExamples) * sizeof(float);
+  PCM_DISPATCH_K(K_, {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_soft_leafval_kernel<KK>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(hclt_soft_leafval_kernel<KK>, dim3(V_, Bp64 / kEvExamples), dim3(256), lds, stream, s, d_leaf_.p, C_,
+                       s.batch, Bp64, d_soft_lv_.p, d_soft_m_.p);
+  });
+  check_launch("soft_leafval");
+  d.leaf = d_soft_lv_.p;
+  d.leaf_stride = (uint32_t)((size_t)Bp64 * K_ * 4);
+  d.leaf_slice = (uint32_t)kSlice * K_ * 4;
+  return d;
+}
+
+void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
+  if (!soft_block_ok()) return general()->loglikelihoods_soft(s, d_ll);
+  if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  const HcltDev d = soft_stage(s);
+  if (wide_walk_) return wide_forward(d, d_ll);
+  force_general_walks_ = true;
+  run_forward(d, d_ll);
+  force_general_walks_ = false;
+}
 
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
   if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (soft_block_ok()) {
+    if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+    if (flows_in_general_ && rate != 0.f) fail(PCM_ERR_STATE, "flow memory cannot carry over from the layered engine");
+    const HcltDev d = soft_stage(s);
+    if (d_soft_gnode_.n == 0) {   // the tile that carries the flow of a variable's leaves: its own node's, or its parent's
+      std::vector<int32_t> gn(V_);
+      for (int v = 0; v < V_; ++v)
+        for (int c : children_[v]) gn[c] = inner_of_var_[v];
+      for (int v = 0; v < V_; ++v)
+        if (inner_of_var_[v] >= 0) gn[v] = inner_of_var_[v];
+      d_soft_gnode_.upload(gn);
+    }
+    const float* g_tiles = d.R;   // where the statistics pass leaves the child-flow tiles
+    if (wide_walk_) {
+      wide_forward(d, d_ll);
+      wide_backward_stats(d, rate, true);
+      g_tiles = d_G_.p;
+    } else {
+      force_general_walks_ = true;
+      run_forward(d, d_ll);
+      run_backward(d);
+      run_stats(d, rate);
+      force_general_walks_ = false;
+    }
+    const int Bp64 = ceil_div(d.Bp, kEvExamples) * kEvExamples;
+    // the examples are split among workgroups that add into the table, so the old statistics are scaled first
+    const int64_t n_leaf = (int64_t)V_ * C_ * K_;
+    hipLaunchKernelGGL(hclt_soft_scale_kernel, dim3(ceil_div(n_leaf, 256)), dim3(256), 0, stream, d_leaf_flow_.p, n_leaf, rate);
+    const int split = 256;
+    PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_soft_leafflow_kernel<KK>, dim3(ceil_div(C_, kEvCats), V_, ceil_div(s.batch, split)),
+                                          dim3(256), 0, stream, s, d_leaf_.p, d_soft_lv_.p, d_soft_m_.p, g_tiles,
+                                          d_soft_gnode_.p, C_, s.batch, Bp64, (size_t)d.nslices * kSlice * K_, split,
+                                          d_leaf_flow_.p));
+    check_launch("soft_leafflow");
+    have_flows_ = true;
+    flows_in_general_ = false;
+    if (timing) ++n_timed_;
+    return;
+  }
   if (have_flows_ && !flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from categorical batches to soft-evidence batches");
   general()->flows_soft(s, rate, d_head_mask, d_ll);
@@ -1054,7 +1145,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     if (timing) ++n_timed_;
     return;
   }
-  if (wide_) {
+  if (wide_walk_) {
     wide_forward(d, d_ll);
     wide_backward_stats(d, rate);
     have_flows_ = true;

@@ -15,6 +15,7 @@
 namespace pcm {
 
 constexpr int kSlice = 16;       // examples per tile
+constexpr double kWideNodeUs = 1.9, kWalk64StepUs = 7.6;   // measured costs behind the choice of walk kernels at K = 64
 constexpr int kWalkWaves = 16;   // waves per workgroup (= items per step) in the tree-walk kernels
 constexpr int kInlineOps = 4;    // static operands held in a step item
 constexpr int kInlineLds = 3;    // LDS-resident operands held in a step item
@@ -95,6 +96,8 @@ struct HcltDev {
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   int32_t B, Bp, nslices, C, n_inner, V;
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
+  uint32_t leaf_slice;    // 0; soft evidence: the "leaf table" holds one row per example ([V][Bp][K], the
+                          // categories are the example's rank in its slice) and a slice's rows start this many bytes on
   uint32_t tile_stride;   // bytes per node in O / R / G (nslices*16*K*4)
 };
 
@@ -199,6 +202,13 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int64_t> d_sum_param_src_;
   int cap_slices_ = 0;
   bool have_flows_ = false;
+  // soft evidence on the block kernels (single head, K <= 64)
+  bool soft_block_ok() const { return block_ && !wide_ && H_ == 0; }
+  HcltDev soft_stage(const SoftRef& s);
+  DevBuf<float> d_soft_lv_, d_soft_m_;   // value table [V][Bp][K] and largest evidence [V][Bp] of the batch
+  DevBuf<int32_t> d_soft_gnode_;
+  bool force_general_walks_ = false;
+  bool wide_walk_ = false;            // forward / backward / statistics run on the node-at-a-time wide kernels
   bool flows_in_general_ = false;   // the last flows were computed by the layered engine (soft evidence)
   std::vector<hipEvent_t> ev_;   // kTimingRing sets of 4 events
   int n_timed_ = 0;
@@ -233,7 +243,7 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_wide_rs_, d_wide_es_;   // R and E of every node in the operand layout of the statistics contraction
   DevBuf<int32_t> d_wide_state_node_;     // per variable: the inner node whose flow tile feeds its leaf histogram
   void wide_forward(const HcltDev& d, float* d_ll);
-  void wide_backward_stats(const HcltDev& d, float rate);
+  void wide_backward_stats(const HcltDev& d, float rate, bool soft = false);
 };
 
 }  // namespace pcm

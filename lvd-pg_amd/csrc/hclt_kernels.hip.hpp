@@ -72,6 +72,13 @@ __device__ __forceinline__ LaneOffs lane_offs(int slice, int lane) {
   return o;
 }
 
+template <int K>
+__device__ __forceinline__ LaneOffs lane_offs(const HcltDev& d, int slice, int lane) {
+  LaneOffs o = lane_offs<K>(slice, lane);
+  o.leaf += (uint32_t)slice * d.leaf_slice;
+  return o;
+}
+
 // All HBM traffic of the hot kernels goes through raw buffer descriptors (uniform base +
 // size in scalar registers, 32-bit per-lane byte offset).  A descriptor of size 0 makes the
 // access a no-op that still counts as issued: loads return zeros, stores are dropped, and
@@ -319,7 +326,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slice = blockIdx.x;
-  const LaneOffs lo = lane_offs<K>(slice, lane);
+  const LaneOffs lo = lane_offs<K>(d, slice, lane);
   const int bcol = lo.bcol;
 
   // prologue: the rows carry 64 idle steps past n_steps, so no index needs a guard
@@ -398,7 +405,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slice = blockIdx.x;
-  const LaneOffs lo = lane_offs<K>(slice, lane);
+  const LaneOffs lo = lane_offs<K>(d, slice, lane);
   const int bcol = lo.bcol;
 
   SchedChunk sc;
@@ -474,7 +481,10 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
 // in which the waves arrive.
 //
 // LDS (32-bit words): [nh][2][C][K+1] limb histograms | [waves][16][K+16] transposition pads.
-template <int K>
+// kSoft (soft evidence): no histograms; the child-flow tiles G replace the ratio tiles for the
+// leaf-flow kernel.  A build of its own: the same store behind a run-time flag, never taken, was
+// enough to make the second histogram pass of the categorical build lose flow.
+template <int K, bool kSoft>
 __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     HcltDev d, const StepItem* __restrict__ items, float* __restrict__ edge_aggr,
     float* __restrict__ leaf_flow, float rate, int nh, int hist_words, int limb) {
@@ -495,7 +505,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
   const int hist_sz = d.C * HS;                     // words per limb table
   unsigned* hist = reinterpret_cast<unsigned*>(smem);
   float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
-  const int nu = 1 + nd.lc_cnt;
+  const int nu = kSoft ? 1 : 1 + nd.lc_cnt;
   const int last = d.nslices - 1;
   const float hi_scale = __builtin_ldexpf(1.f, limb), lo_scale = hi_scale;
 
@@ -509,7 +519,8 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
 
   for (int u0 = 0; u0 < nu; u0 += nh) {
     const int nhere = min(nh, nu - u0);
-    for (int i = threadIdx.x; i < nhere * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
+    if (!kSoft)
+      for (int i = threadIdx.x; i < nhere * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
     __syncthreads();
 
     // prologue (slices past the end are clamped: harmless repeated loads)
@@ -517,7 +528,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     uint32_t xs, xc;   // packed categories of the next-but-one / next slice (after the top: next / current)
     {
       const int sa = min(wave, last), sb = min(wave + nwaves, last);
-      const LaneOffs la = lane_offs<K>(sa, lane);
+      const LaneOffs la = lane_offs<K>(d, sa, lane);
       xc = xpack_load(d, n, la.bcol);
       pre_request_ops<K>(d, q, xc, la, P);
       tile_load<K>(d.R, n, d.tile_stride, la.tile, rn);
@@ -531,12 +542,12 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
       const Tile<K> r0 = rn;
       const uint32_t xh = xc;   // packed categories of the slice computed now
       xc = xs;
-      const LaneOffs l1 = lane_offs<K>(s1, lane);
+      const LaneOffs l1 = lane_offs<K>(d, s1, lane);
       pre_request_ops<K>(d, q, xc, l1, P);
       tile_load<K>(d.R, n, d.tile_stride, l1.tile, rn);
       xs = xpack_load(d, n, s2 * kSlice + b);
 
-      if (it_flags & kItemOverflow) operands_extra<K>(d, itp, it_ng, it_eo, it_ec, lane_offs<K>(s0, lane), e);
+      if (it_flags & kItemOverflow) operands_extra<K>(d, itp, it_ng, it_eo, it_ec, lane_offs<K>(d, s0, lane), e);
       const float m = tile_rowmax<K>(e);
       tile_exp_sub<K>(e, m);
       Tile<K> t;
@@ -576,7 +587,9 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
         __builtin_amdgcn_wave_barrier();
       }
-      if (bcol < d.B) {
+      if (kSoft) {
+        tile_store<K>(d.R, n, d.tile_stride, lane_offs<K>(s0, lane).tile, t);   // r0 of this slice is in registers
+      } else if (bcol < d.B) {
         // fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
         unsigned hi[KT][4], lo[KT][4];
 #pragma unroll
@@ -609,7 +622,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     }
     __syncthreads();
     const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
-    for (int h = 0; h < nhere; ++h) {
+    for (int h = 0; h < nhere && !kSoft; ++h) {
       const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
       float* dst = leaf_flow + (size_t)u * d.C * K;
       const unsigned* src = hist + (size_t)h * 2 * hist_sz;

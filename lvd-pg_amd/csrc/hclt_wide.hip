@@ -56,7 +56,7 @@ __device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& 
   for (int u = -1; u < nd.lc_cnt; ++u) {
     const int var = u < 0 ? nd.var : d.child_leaf[nd.lc_off + u];
     const int x = d.xb[(size_t)var * d.Bp + col];
-    const float* row = d.leaf + ((size_t)var * d.C + x) * K;
+    const float* row = d.leaf + (size_t)var * (d.leaf_stride / 4) + (size_t)x * K + (size_t)s * (d.leaf_slice / 4);
 #pragma unroll
     for (int q = 0; q < Q; ++q) z[q] += *reinterpret_cast<const v4f*>(row + (wave * Q + q) * 16 + 4 * g);
   }
@@ -307,6 +307,7 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev
 
 #define PCM_DISPATCH_WIDE_K(K_, ...)                                                         \
   switch (K_) {                                                                              \
+    case 64: { constexpr int KK = 64; __VA_ARGS__; break; }                                  \
     case 128: { constexpr int KK = 128; __VA_ARGS__; break; }                                \
     default: fail(PCM_ERR_STATE, "no wide block kernel for hidden size %d", K_);             \
   }
@@ -319,7 +320,8 @@ void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
 
-void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate) {
+// soft: the evidence is soft, the caller shares out the leaf flows from the G tiles itself
+void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   if (d_wide_state_node_.n == 0) {
     std::vector<int32_t> t(V_);
     for (int v = 0; v < V_; ++v) t[v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
@@ -338,7 +340,8 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate) {
                        d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p, rate);
   });
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
-  hipLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), lds, stream, d, d_G_.p,
+  if (!soft)
+    hipLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), lds, stream, d, d_G_.p,
                      d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
   check_launch_w("hclt_wide_stats");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));

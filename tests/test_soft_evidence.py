@@ -124,6 +124,43 @@ def test_hclt_soft_evidence_matches_oracle(gpu, V, K, C, B):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("K", [16, 64])
+def test_hclt_soft_evidence_far_from_the_favoured_category(gpu, K):
+    """Evidence that favours, by 150 nats, a category some leaves all but forbid (log-probability
+    -100 or -inf): the factored sums of the block kernels lose their footing there and the exact
+    paths must take over.  Also example ids and the flow memory rate."""
+    torch, P = gpu
+    V, C, B = 6, 7, 50
+    parent, theta, leaf, fc = make_hclt(V, K, C, 77)
+    rng = np.random.default_rng(K)
+    leaf = leaf.copy()
+    hard = rng.random((V, K)) < 0.4
+    leaf[hard, 0] = np.where(rng.random(hard.sum()) < 0.5, -100.0, -np.inf)
+    leaf -= np.log(np.exp(leaf.astype(np.float64)).sum(-1, keepdims=True)).astype(np.float32)
+    fc = O.hclt_flat(parent, K, C, theta, leaf)
+    ev = rng.normal(-150, 3, (B, V, C)).astype(np.float32)
+    ev[:, :, 0] = rng.normal(0, 1, (B, V))
+    ev[rng.random((B, V)) < 0.3, 0] = -160.0                          # ... and examples where it does not
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    ids = rng.permutation(B)[:37].astype(np.int32)
+    sub = np.ascontiguousarray(ev[ids])
+    mars = O.forward_soft(fc, sub, double=True)
+    d = torch.from_numpy(ev).cuda()
+    ll = P.probs_flows_circuit(bpc, d, example_ids=ids).cpu().numpy()
+    assert np.isfinite(mars[-1]).all()
+    assert np.abs(ll - mars[-1]).max() < LL_RTOL * np.abs(mars[-1]).max()
+    fl, ea = O.backward(fc, mars, double=True)
+    counts = O.input_flows_soft(fc, sub, mars, fl, double=True).reshape(V, K, C)
+    _, lf = bpc.get_flows()
+    assert np.abs(lf - counts).max() < FLOW_RTOL * counts.max()
+    np.testing.assert_allclose(lf.sum(axis=(1, 2)), len(ids), rtol=1e-4)
+    P.probs_flows_circuit(bpc, d, example_ids=ids, rate=0.5)          # flow memory: half of the old statistics stay
+    _, lf2 = bpc.get_flows()
+    assert np.abs(lf2 - 1.5 * counts).max() < FLOW_RTOL * 1.5 * counts.max()
+
+
+@pytest.mark.gpu
 def test_general_circuit_soft_evidence_and_one_hot_limit(gpu):
     torch, P = gpu
     V, C, B = 8, 5, 90
