@@ -230,6 +230,50 @@ def secondary(args):
                    value=NC * B / dt, unit="examples/s",
                    config={"workload": args.workload, "circuits": NC, "streams": NS, "num_vars": V, "hidden": K,
                            "categories": C, "heads": H, "batch": B})
+    elif args.workload == "c4_full":
+        # C4 as a whole: 64 x 64 x 3 images cut into 64 patches of 8 x 8 x 3; one 192-variable K = 32 circuit with 128
+        # cluster heads per patch (block engine, eight streams) and the K = 64 top-level HCLT over the 64 cluster ids
+        V, K, C, H, B, NP, NS = 192, 32, 256, 128, 1024, 64, 8
+        img = workloads.grf_images(B, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(B, 3, 64, 64)
+        patches = [np.ascontiguousarray(img[:, :, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8]).reshape(B, V)
+                   for p in range(NP)]
+        cluster = rng.integers(0, H, size=(B, NP)).astype(np.uint8)          # seeded uniform cluster ids
+        circs, datas, masks = [], [], []
+        for p in range(NP):
+            parent = workloads.chow_liu_parent(patches[p])
+            c = P.multihead_hclt_from_clt(parent, C, K, H)
+            th, lf = workloads.init_params(parent, K, C, 2000 + p, kind="dirichlet")
+            c.set_params(th, lf)                                             # heads stay uniform
+            circs.append(c)
+            datas.append(torch.from_numpy(patches[p]).cuda())
+            m = np.zeros((H, B), np.float32)
+            m[cluster[:, p], np.arange(B)] = 1.0
+            masks.append(torch.from_numpy(m).cuda())
+        tparent = workloads.chow_liu_parent(cluster)
+        top = P.hclt_from_clt(tparent, H, 64)
+        top.set_params(*workloads.init_params(tparent, 64, H, 2100, kind="dirichlet"))
+        dtop = torch.from_numpy(cluster).cuda()
+        lls = [torch.empty(B, device="cuda") for _ in range(NP + 1)]
+        streams = [torch.cuda.Stream() for _ in range(NS)]
+        torch.cuda.synchronize()
+        for i, c in enumerate(circs):
+            check(lib.pcm_set_stream(c.handle, streams[i % NS].cuda_stream))
+        check(lib.pcm_set_stream(top.handle, streams[0].cuda_stream))
+
+        def step():
+            for c, d, hm, ll in zip(circs, datas, masks, lls):
+                check(lib.pcm_flows(c.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(), ll.data_ptr()))
+                check(lib.pcm_em_update(c.handle, 0.1, 0.9))
+            check(lib.pcm_em_step(top.handle, dtop.data_ptr(), dtop.stride(0), dtop.stride(1), None, B, 0.0, 0.1, 0.9,
+                                  lls[NP].data_ptr()))
+        dt = _timed(torch, step, args.steps, args.warmup)
+        algo = sum(algorithmic_bytes(c.size("inner_tree_nodes"), V, K, C, B)["step"] + 2 * 4 * H * B for c in circs) \
+            + algorithmic_bytes(top.size("inner_tree_nodes"), NP, 64, H, B)["step"]
+        out.update(metric="images/sec fwd+bwd+EM, 12288-variable patch-clustered circuit: 64 patch circuits (192 vars, K=32, "
+                          "128 heads) on 8 streams + top HCLT (64 vars, K=64)",
+                   value=B / dt, unit="examples/s",
+                   config={"workload": args.workload, "patch_circuits": NP, "streams": NS, "num_vars": NP * V, "hidden": K,
+                           "top_hidden": 64, "categories": C, "heads": H, "batch": B})
     elif args.workload == "c4_top_soft":
         # the top-level circuit of C4: 64 patch variables, 128 cluster categories, K = 64, trained on soft evidence
         V, K, C, B = 64, 64, 128, 1024

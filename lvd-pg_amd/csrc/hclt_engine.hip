@@ -45,9 +45,8 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   // walk kernels has, so those kernels spill (6 us per step); the node-at-a-time wide kernels take about
   // kWideNodeUs per node instead and win unless the tree is bushy enough to fill the 16 waves of a step
   wide_walk_ = wide_ || (K == 64 && (double)n_inner_ * kWideNodeUs < (double)(n_fwd_steps_ + n_bwd_steps_) * 0.5 * kWalk64StepUs);
-  if (H_ > 0 && !(block_ && fwd_lean_ && bwd_lean_ && stat_lean_))
-    fail(PCM_ERR_UNSUPPORTED, "multi-head block kernels need K = 16 or 32 and at most three children per tree node; "
-                              "compile this circuit with pcm_circuit_create");
+  if (H_ > 0 && !(block_ && K <= 32))
+    fail(PCM_ERR_UNSUPPORTED, "multi-head block kernels need K = 16 or 32; compile this circuit with pcm_circuit_create");
   build_param_order();
 
   // uniform parameters
@@ -943,7 +942,6 @@ void HcltCircuit::run_backward(const HcltDev& d) {
                        bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
-  if (H_ > 0 && !small) fail(PCM_ERR_UNSUPPORTED, "multi-head HCLT: batch of %d examples is too large for one call", d.B);
   if (bwd_lean_ && small && !force_general_walks_) {
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -955,7 +953,11 @@ void HcltCircuit::run_backward(const HcltDev& d) {
     });
   } else {
     PCM_DISPATCH_K(K_, {
-      if (bwd_spill_) launch(&hclt_backward_kernel<KK, true>); else launch(&hclt_backward_kernel<KK, false>);
+      if (H_ > 0) {
+        if (bwd_spill_) launch(&hclt_backward_kernel<KK, true, true>); else launch(&hclt_backward_kernel<KK, false, true>);
+      } else {
+        if (bwd_spill_) launch(&hclt_backward_kernel<KK, true, false>); else launch(&hclt_backward_kernel<KK, false, false>);
+      }
     });
   }
   check_launch("hclt_backward");
@@ -987,7 +989,6 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
       return;
     }
   }
-  if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "multi-head HCLT with %d categories: the statistics do not fit the fast kernel", C_);
   // LDS layout of hclt_stats_kernel
   const size_t pads = (size_t)kStatWaves * kSlice * (K_ + 16);
   auto hist_words = [&](int nh) { return std::max((((size_t)nh * hist + 3) & ~(size_t)3), (size_t)K_ * K_); };
@@ -999,7 +1000,7 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, stream, d, d_stat_items_.p, d_edge_aggr_.p,
-                       d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb);
+                       d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   };
   PCM_DISPATCH_K(K_, {
     if (d.leaf_slice != 0) launch(&hclt_stats_kernel<KK, true>); else launch(&hclt_stats_kernel<KK, false>);

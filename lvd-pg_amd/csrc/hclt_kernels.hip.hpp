@@ -397,7 +397,8 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
 // the node's own value tile O_v (-> S_v = exp(O_v - m)).  Dependency: F_v = G_parent from
 // its LDS slot.  R_v goes to HBM for the statistics kernel, G_v to an LDS slot for the
 // children (kSpill: to HBM when no slot was free).
-template <int K, bool kSpill>
+// kHeads: multi-head circuit; the head kernel has left the root's ratio tile in memory.
+template <int K, bool kSpill, bool kHeads>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
     HcltDev d, const int32_t* __restrict__ fields, int stride, const StepItem* __restrict__ sched,
     int n_steps) {
@@ -451,9 +452,13 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) r.v[kt][i] *= __builtin_amdgcn_exp2f(fmaf(ov.v[kt][i], -kLog2e, m * kLog2e));
-    if (flags & kItemRoot) {   // flow 1 into the single root sum node of every live example
-      tile_zero<K>(r);
-      r.v[0][0] = (lane < 16 && bcol < d.B) ? __builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e) : 0.f;
+    if (flags & kItemRoot) {
+      if (kHeads) {   // the heads' flows, already divided by their sums
+        tile_load<K>(d.R, node, d.tile_stride, lo.tile, r);
+      } else {        // flow 1 into the single root sum node of every live example
+        tile_zero<K>(r);
+        r.v[0][0] = (lane < 16 && bcol < d.B) ? __builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e) : 0.f;
+      }
     }
     tile_store<K>(d.R, node, d.tile_stride, lo.tile, r);
     contract<K>(w, r, t);
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
 template <int K, bool kSoft>
 __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     HcltDev d, const StepItem* __restrict__ items, float* __restrict__ edge_aggr,
-    float* __restrict__ leaf_flow, float rate, int nh, int hist_words, int limb) {
+    float* __restrict__ leaf_flow, float rate, int nh, int hist_words, int limb, const int* __restrict__ flow_shift) {
   constexpr int KT = K / 16;
   constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
   constexpr int HS = K + 1;    // row stride of a histogram: spreads equal states over banks
@@ -496,6 +501,10 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = lane & 15, g = lane >> 4;
   const int nwaves = blockDim.x >> 6;
+  // flows lie in [0, 2^shift]: 1 per example in a single-head circuit, the largest total head mask of an
+  // example (left on the device by the head kernel) in a multi-head one
+  const int shift = flow_shift ? __builtin_amdgcn_readfirstlane(*flow_shift) : 0;
+  const float cap = __builtin_ldexpf(1.f, shift);
   const int n = blockIdx.x;
   const StepItem* itp = items + n;
   PreRegs q;
@@ -507,7 +516,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
   float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
   const int nu = kSoft ? 1 : 1 + nd.lc_cnt;
   const int last = d.nslices - 1;
-  const float hi_scale = __builtin_ldexpf(1.f, limb), lo_scale = hi_scale;
+  const float hi_scale = __builtin_ldexpf(1.f, limb - shift), lo_scale = __builtin_ldexpf(1.f, limb);
 
   WTile<K> w;
   w_load<K>(d.Wb, n, lane, w);
@@ -590,13 +599,13 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
       if (kSoft) {
         tile_store<K>(d.R, n, d.tile_stride, lane_offs<K>(s0, lane).tile, t);   // r0 of this slice is in registers
       } else if (bcol < d.B) {
-        // fixed-point limbs of this lane's K/4 flows (clamped to [0, 1])
+        // fixed-point limbs of this lane's K/4 flows (clamped to [0, 2^shift])
         unsigned hi[KT][4], lo[KT][4];
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float v = fminf(fmaxf(t.v[kt][i], 0.f), 1.f) * hi_scale;
+            const float v = fminf(fmaxf(t.v[kt][i], 0.f), cap) * hi_scale;
             const float fl = floorf(v);
             hi[kt][i] = (unsigned)fl;
             lo[kt][i] = (unsigned)((v - fl) * lo_scale);
@@ -621,7 +630,7 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
       }
     }
     __syncthreads();
-    const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+    const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
     for (int h = 0; h < nhere && !kSoft; ++h) {
       const int u = (u0 + h == 0) ? nd.var : d.child_leaf[nd.lc_off + u0 + h - 1];
       float* dst = leaf_flow + (size_t)u * d.C * K;

@@ -187,7 +187,9 @@ def test_config_hclt48_k128(gpu, oracle):
 
 
 @pytest.mark.parametrize("V,K,C,H,B,tree", [(7, 16, 5, 3, 40, None), (12, 32, 9, 128, 70, None), (2, 16, 4, 16, 16, [-1, 0]),
-                                            (9, 32, 256, 40, 33, [-1, 0, 0, 1, 1, 2, 2, 3, 3])])
+                                            (9, 32, 256, 40, 33, [-1, 0, 0, 1, 1, 2, 2, 3, 3]),
+                                            (13, 16, 7, 20, 50, [-1, 0, 1, 1, 1, 1, 2, 3, 0, 8, 8, 8, 8]),     # four children twice
+                                            (7, 32, 6, 5, 30, [-1, 0, 0, 0, 0, 0, 0])])                        # a star
 def test_multihead_hclt_on_the_block_engine(gpu, oracle, V, K, C, H, B, tree):
     """H heads over the root's products (src-jl/multi_head_pc/bit_circuit.jl:14-56): the block
     engine (body through the walk kernels, heads in two small kernels) against the layered engine
@@ -238,5 +240,5 @@ def test_multihead_hclt_on_the_block_engine(gpu, oracle, V, K, C, H, B, tree):
     assert lls[2] > lls[1] > lls[0]
     with pytest.raises(P.PcmError):
         P.kld(blk, blk)
-    with pytest.raises(P.PcmError):                                    # a node with four children: no lean kernels
-        P.multihead_hclt_from_clt(np.array([-1, 0, 0, 0, 0, 1], np.int32), C, K, H)
+    with pytest.raises(P.PcmError):                                    # no head kernels for this hidden size
+        P.multihead_hclt_from_clt(np.array([-1, 0, 0, 0, 0, 1], np.int32), C, 64, H)
