@@ -27,7 +27,11 @@ namespace pcm {
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kWideWaves = 4;
+constexpr int kWideWaves = 4;   // waves of the edge and leaf statistics kernels
+
+// waves of a walk workgroup: one 16-state row tile of the output per wave (8 at K = 128, 4 at K = 64)
+template <int K>
+constexpr int wide_walk_waves() { return K / 16 > 8 ? 8 : K / 16; }
 
 static void check_launch_w(const char* what) {
   hipError_t e = hipGetLastError();
@@ -38,7 +42,7 @@ template <int K>
 struct WideLds {
   v4f e[K / 16][64];   // E tile of the node
   v4f r[K / 16][64];   // R tile (backward)
-  float mx[kWideWaves][16];
+  float mx[wide_walk_waves<K>()][16];
 };
 
 // Builds the node's E tile: every wave sums its quarter of Z, the row maxima are combined
@@ -47,7 +51,7 @@ struct WideLds {
 template <int K>
 __device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& nd, int s, int lane, int wave,
                                               WideLds<K>& L, v4f (&e)[K / 16]) {
-  constexpr int KT = K / 16, Q = KT / kWideWaves;
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   const int b = lane & 15, g = lane >> 4;
   const int col = s * kSlice + b;
   v4f z[Q];
@@ -76,7 +80,7 @@ __device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& 
   if (g == 0) L.mx[wave][b] = m;
   __syncthreads();
 #pragma unroll
-  for (int w = 0; w < kWideWaves; ++w) m = fmaxf(m, L.mx[w][b]);
+  for (int w = 0; w < WV; ++w) m = fmaxf(m, L.mx[w][b]);
 #pragma unroll
   for (int q = 0; q < Q; ++q) {
     v4f x;
@@ -92,22 +96,32 @@ __device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& 
 
 // Forward: one workgroup per 16-example slice walks the nodes children-first.
 template <int K>
-__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_forward_kernel(HcltDev d, float* __restrict__ ll) {
-  constexpr int KT = K / 16, Q = KT / kWideWaves;
+__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_kernel(HcltDev d, float* __restrict__ ll) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
   const int b = lane & 15, g = lane >> 4;
-  for (int n = 0; n < d.n_inner; ++n) {
-    const HcltNode nd = d.nodes[n];
-    // this wave's rows of the parameter block: they wait for nothing computed here
-    v4f w[Q][KT];
+  // this wave's rows of the parameter block wait for nothing computed here: a node's rows are
+  // requested while the node before it is being computed
+  v4f wn[Q][KT];
+  auto request_w = [&](int n) {
     const v4f* wf = reinterpret_cast<const v4f*>(d.Wf + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
-      for (int jt = 0; jt < KT; ++jt) w[q][jt] = wf[((wave * Q + q) * KT + jt) * 64 + lane];
+      for (int jt = 0; jt < KT; ++jt) wn[q][jt] = wf[((wave * Q + q) * KT + jt) * 64 + lane];
+  };
+  request_w(0);
+  for (int n = 0; n < d.n_inner; ++n) {
+    const HcltNode nd = d.nodes[n];
     v4f e[KT];
     const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
+    v4f w[Q][KT];
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+#pragma unroll
+      for (int jt = 0; jt < KT; ++jt) w[q][jt] = wn[q][jt];
+    if (n + 1 < d.n_inner) request_w(n + 1);
     v4f* out = reinterpret_cast<v4f*>(d.O + ((size_t)n * d.nslices + s) * kSlice * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -131,23 +145,33 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_forward_kernel(Hclt
 // contraction: lane 16*g' + r holds, for t < 4, the value of example 4*t + g' at state
 // kt*16 + r (the contraction runs over examples).
 template <int K>
-__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_backward_kernel(HcltDev d, float* G, float* __restrict__ RS,
-                                                                             float* __restrict__ ES) {
-  constexpr int KT = K / 16, Q = KT / kWideWaves;
+__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_kernel(HcltDev d, float* G,
+                                                                                       float* __restrict__ RS,
+                                                                                       float* __restrict__ ES) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
   const int b = lane & 15, g = lane >> 4;
   const bool live = s * kSlice + b < d.B;
-  for (int n = d.n_inner - 1; n >= 0; --n) {
-    const HcltNode nd = d.nodes[n];
-    v4f w[Q][KT];
+  v4f wn[Q][KT];
+  auto request_w = [&](int n) {
     const v4f* wb = reinterpret_cast<const v4f*>(d.Wb + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
-      for (int kt = 0; kt < KT; ++kt) w[q][kt] = wb[((wave * Q + q) * KT + kt) * 64 + lane];
+      for (int kt = 0; kt < KT; ++kt) wn[q][kt] = wb[((wave * Q + q) * KT + kt) * 64 + lane];
+  };
+  request_w(d.n_inner - 1);
+  for (int n = d.n_inner - 1; n >= 0; --n) {
+    const HcltNode nd = d.nodes[n];
     v4f e[KT];
     const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
+    v4f w[Q][KT];
+#pragma unroll
+    for (int q = 0; q < Q; ++q)
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt) w[q][kt] = wn[q][kt];
+    if (n > 0) request_w(n - 1);
     const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
     const v4f* on = reinterpret_cast<const v4f*>(d.O + tile);
 #pragma unroll
@@ -314,8 +338,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev
 
 void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
   if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
-  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(kWideWaves * 64), 0, stream,
-                                             d, d_ll));
+  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0,
+                                             stream, d, d_ll));
   check_launch_w("hclt_wide_forward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
@@ -332,7 +356,7 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   PCM_DISPATCH_WIDE_K(K_, {
-    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(kWideWaves * 64), 0, stream, d, d_G_.p,
+    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0, stream, d, d_G_.p,
                        d_wide_rs_.p, d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
     if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
