@@ -289,6 +289,57 @@ def test_compiled_dag_node_maps_and_node_flow_sums(gpu, oracle):
 
 
 @pytest.mark.gpu
+def test_structure_builders_compile_and_run(gpu, oracle):
+    """hclt_pc with variable groups, customized_hclt and joined_hclt through the layered engine
+    against the DAG oracle; hclt_pc with one variable per group against the block engine."""
+    import dag_oracle as D
+    torch, P = gpu
+    N, S = P.nodes, P
+    rng = np.random.default_rng(21)
+    B = 40
+    # variable groups: 4 tree nodes over 8 observed variables
+    groups = S.group_vars_by_grid(2, 4, 1, patch_h=1, patch_w=2)
+    pc = S.hclt_pc(np.array([-1, 0, 0, 1], np.int32), 5, 4, variable_groups=groups)
+    N.init_parameters(pc, 0.4, rng)
+    data = rng.integers(0, 5, size=(B, 8)).astype(np.uint8)
+    bpc = P.CuBitsProbCircuit(pc)
+    (ro,), _ = to_oracle_dag(pc)
+    np.testing.assert_allclose(P.loglikelihoods(bpc, torch.from_numpy(data).cuda()).cpu().numpy(),
+                               D.values([ro], data)[id(ro)], rtol=2e-5)
+    # one variable per group: the same function as the block engine's HCLT with these parameters
+    parent = oracle.random_tree(7, rng, 3)
+    pc1 = S.hclt_pc(parent, 6, 16)
+    N.init_parameters(pc1, 0.4, rng)
+    gen = P.CuBitsProbCircuit(pc1)
+    blk = P.hclt_from_clt(parent, 6, 16)
+    assert blk.num_parameters() == gen.num_parameters() and blk.num_nodes() == gen.num_nodes()
+    P.update_parameters(blk, P.vectorize_parameters(gen))
+    d1 = torch.from_numpy(rng.integers(0, 6, size=(B, 7)).astype(np.uint8)).cuda()
+    np.testing.assert_allclose(P.loglikelihoods(blk, d1).cpu().numpy(), P.loglikelihoods(gen, d1).cpu().numpy(), rtol=2e-5)
+    for t in ("edge2param", "edge_parent", "edge_prime", "edge_sub"):
+        np.testing.assert_array_equal(blk.table(t), gen.table(t), err_msg=t)
+    # joined trees: K heads over the full scope; EM on the multi-head circuit raises the mixture likelihood
+    t1 = S.clt_edges2parent([(0, 1), (1, 2), (2, 3), (3, 4)])
+    t2 = S.clt_edges2parent([(0, 2), (2, 1), (1, 3), (3, 4)])
+    roots = S.joined_hclt_from_clts([t1, t2], 3, 4)
+    N.init_parameters(roots, 0.4, rng)
+    dj = rng.integers(0, 4, size=(B, 5)).astype(np.uint8)
+    mh = P.CuMultiHeadBitsProbCircuit(roots)
+    ro, _ = to_oracle_dag(roots)
+    vals = D.values(ro, dj)
+    np.testing.assert_allclose(P.loglikelihoods(mh, torch.from_numpy(dj).cuda()).cpu().numpy(),
+                               np.stack([vals[id(r)] for r in ro], 1), rtol=2e-5)
+    hm = torch.ones((B, 3), device="cuda")
+    lls = P.mini_batch_em_for_multihead_pc(mh, torch.from_numpy(dj).cuda(), hm, 3, batch_size=B, pseudocount=0.1,
+                                           param_inertia=0.5, shuffle="none")
+    assert lls[-1] > lls[0]
+    # joined_hclt end to end: trees learned on the device from two datasets
+    ds = [torch.from_numpy(rng.integers(0, 4, size=(200, 5)).astype(np.uint8)).cuda() for _ in range(2)]
+    jr = S.joined_hclt(ds, 2, num_cats=4)
+    assert len(jr) == 2 and N.variables(jr) == [0, 1, 2, 3, 4]
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("threshold", [-1.0, 0.02, 0.15])
 def test_prune_pc_matches_the_oracle(gpu, oracle, threshold):
     import dag_oracle as D
