@@ -19,8 +19,8 @@ sys.path.insert(0, os.path.join(ROOT, "lvd-pg_amd"))
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # kernels the benchmark circuit runs (three children per node at most, K = 32: the lean set)
-KERNEL_NAMES = {"forward": "hclt_forward_lean_kernel<32>", "backward": "hclt_backward_lean_kernel<32>",
-                "statistics": "hclt_stats_lean_kernel<32>"}
+KERNEL_NAMES = {"forward": "hclt_forward_lean_kernel<%d>", "backward": "hclt_backward_lean_kernel<%d, false>",
+                "statistics": "hclt_stats_lean_kernel<%d>"}
 
 
 def algorithmic_bytes(n_int, V, K, C, B):
@@ -392,7 +392,7 @@ def main():
     achieved = ab[dominant] / (kernel_ms[dominant] * 1e-3) / 1e9
     ms_per_step = dt / args.steps * 1e3
     out = {
-        "metric": "examples/sec fwd+bwd+EM, 3072-var HCLT K=32; % of HBM/MFMA roofline",
+        "metric": "examples/sec fwd+bwd+EM, %d-var HCLT K=%d; %% of HBM/MFMA roofline" % (V, K),
         "value": B * args.steps / dt,
         "unit": "examples/s",
         "n_gpus": 1,
@@ -406,7 +406,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
                    "tree_inner_nodes": stats["n_inner"], "tree_depth": stats["depth"]},
-        "roofline": {"bound": "hbm", "kernel": KERNEL_NAMES[dominant], "achieved": achieved,
+        "roofline": {"bound": "hbm", "kernel": KERNEL_NAMES[dominant] % K, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic(args.workload, dominant)},
         "kernels_ms": kernel_ms,
@@ -415,7 +415,7 @@ def main():
     if not args.no_cpu:
         # LL after `warmup + steps` parameter updates differs from the oracle's first step, so
         # the baseline is only timed here; parity lives in tests/.
-        cb, _ = cpu_baseline(cfg, args.cpu_sample)
+        cb, _ = cpu_baseline(cfg, min(args.cpu_sample, B))
         out["cpu_baseline"] = cb
     else:
         out["cpu_baseline"] = None
