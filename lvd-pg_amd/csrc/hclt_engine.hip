@@ -851,6 +851,8 @@ void HcltCircuit::ensure_batch(int batch) {
     d_wide_rs_.alloc((size_t)n_inner_ * tile);
     d_wide_es_.alloc((size_t)n_inner_ * tile);
     d_xb_.alloc((size_t)V_ * ns * kSlice);
+    d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
+    d_xn_.zero();
     cap_slices_ = ns;
     return;
   }
@@ -902,7 +904,6 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
                      b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
   check_launch("stage_batch");
-  if (wide_walk_) return;
   hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
   check_launch("pack_x");
@@ -1036,9 +1037,8 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
   if ((size_t)d.Bp * K_ * 4 >= ((size_t)1 << 31)) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", s.batch);
   const int64_t nx = (int64_t)V_ * d.Bp;
   hipLaunchKernelGGL(hclt_soft_x_kernel, dim3(ceil_div(nx, 256)), dim3(256), 0, stream, d_xb_.p, nx);
-  if (!wide_walk_)
-    hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(d.Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
-                       d_child_leaf_.p, d_xb_.p, n_inner_, d.Bp, d_xn_.p);
+  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(d.Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
+                     d_child_leaf_.p, d_xb_.p, n_inner_, d.Bp, d_xn_.p);
   check_launch("soft pack_x");
   const int Bp64 = ceil_div(d.Bp, kEvExamples) * kEvExamples;
   d_soft_lv_.ensure((size_t)V_ * Bp64 * K_);

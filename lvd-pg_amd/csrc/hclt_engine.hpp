@@ -15,7 +15,7 @@
 namespace pcm {
 
 constexpr int kSlice = 16;       // examples per tile
-constexpr double kWideNodeUs = 1.9, kWalk64StepUs = 7.6;   // measured costs behind the choice of walk kernels at K = 64
+constexpr double kWideNodeUs = 1.6, kWalk64StepUs = 7.6;   // measured costs behind the choice of walk kernels at K = 64
 constexpr int kWalkWaves = 16;   // waves per workgroup (= items per step) in the tree-walk kernels
 constexpr int kInlineOps = 4;    // static operands held in a step item
 constexpr int kInlineLds = 3;    // LDS-resident operands held in a step item
@@ -78,6 +78,13 @@ struct StatNode {
   int32_t pad[7];
 };
 static_assert(sizeof(StatNode) == 64, "StatNode is read with scalar loads");
+
+// Per tree node, what the wide walk kernels request a node ahead (hclt_wide.hip).
+struct WideOps {
+  uint32_t fwd[6], bwd[6];   // 0: none; leaf row: bit 31 | category selector << 24 | variable; value tile: bit 30 | node
+  int32_t fwd_extra_off, fwd_extra_cnt, bwd_extra_off, bwd_extra_cnt;   // operands fetched at the point of use
+  int32_t parent, is_root, prev_child, pad;   // prev_child: node - 1 is a child (its tile is still in registers going up)
+};
 
 // Everything the kernels need, passed by value.
 struct HcltDev {
@@ -242,6 +249,9 @@ class HcltCircuit : public pcm_circuit {
   // wide block kernels
   DevBuf<float> d_wide_rs_, d_wide_es_;   // R and E of every node in the operand layout of the statistics contraction
   DevBuf<int32_t> d_wide_state_node_;     // per variable: the inner node whose flow tile feeds its leaf histogram
+  DevBuf<WideOps> d_wide_ops_;
+  DevBuf<uint32_t> d_wide_extra_;
+  void build_wide_tables();
   void wide_forward(const HcltDev& d, float* d_ll);
   void wide_backward_stats(const HcltDev& d, float rate, bool soft = false);
 };

@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cstring>
 
 namespace pcm {
 
@@ -45,31 +46,63 @@ struct WideLds {
   float mx[wide_walk_waves<K>()][16];
 };
 
-// Builds the node's E tile: every wave sums its quarter of Z, the row maxima are combined
-// through LDS, E goes to LDS and comes back whole to every wave.  Returns m of the lane's
-// example.  Two workgroup barriers.
+// Operands of a node's Z that can be requested a node ahead (they do not depend on the node
+// before): its own leaf row and the rows of its first three leaf children (their categories come
+// packed in one word per example, xn), and up to two value tiles of non-leaf children.  The
+// forward walk leaves out the child that was computed just before the node (in post-order the
+// last non-leaf child is always the node before): each wave still has its 16 states of that tile
+// in registers.  Operands beyond these are fetched at the point of use.
+constexpr int kWidePre = 6;
+constexpr uint32_t kWideLeaf = 0x80000000u, kWideTile = 0x40000000u;
+
 template <int K>
-__device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& nd, int s, int lane, int wave,
-                                              WideLds<K>& L, v4f (&e)[K / 16]) {
+__device__ __forceinline__ void wide_request(const HcltDev& d, uint32_t op, uint32_t xpack, int s, int lane, int wave,
+                                             v4f (&out)[(K / 16) / wide_walk_waves<K>()]) {
   constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
-  const int b = lane & 15, g = lane >> 4;
-  const int col = s * kSlice + b;
-  v4f z[Q];
 #pragma unroll
-  for (int q = 0; q < Q; ++q) z[q] = v4f{0.f, 0.f, 0.f, 0.f};
-  for (int u = -1; u < nd.lc_cnt; ++u) {
-    const int var = u < 0 ? nd.var : d.child_leaf[nd.lc_off + u];
-    const int x = d.xb[(size_t)var * d.Bp + col];
+  for (int q = 0; q < Q; ++q) out[q] = v4f{0.f, 0.f, 0.f, 0.f};
+  if (op & kWideLeaf) {
+    const int var = (int)(op & 0xffffffu), sel = (int)((op >> 24) & 3u);
+    const uint32_t x = (xpack >> (8 * sel)) & 0xffu;
     const float* row = d.leaf + (size_t)var * (d.leaf_stride / 4) + (size_t)x * K + (size_t)s * (d.leaf_slice / 4);
 #pragma unroll
-    for (int q = 0; q < Q; ++q) z[q] += *reinterpret_cast<const v4f*>(row + (wave * Q + q) * 16 + 4 * g);
-  }
-  for (int c = 0; c < nd.ic_cnt; ++c) {
-    const int cn = d.child_inner[nd.ic_off + c];
-    const v4f* t = reinterpret_cast<const v4f*>(d.O + ((size_t)cn * d.nslices + s) * kSlice * K);
+    for (int q = 0; q < Q; ++q) out[q] = *reinterpret_cast<const v4f*>(row + (wave * Q + q) * 16 + 4 * (lane >> 4));
+  } else if (op & kWideTile) {
+    const v4f* t = reinterpret_cast<const v4f*>(d.O + ((size_t)(op & 0xffffffu) * d.nslices + s) * kSlice * K);
 #pragma unroll
-    for (int q = 0; q < Q; ++q) z[q] += t[(wave * Q + q) * 64 + lane];
+    for (int q = 0; q < Q; ++q) out[q] = t[(wave * Q + q) * 64 + lane];
   }
+}
+
+// operands beyond the prefetched ones: (variable | kWideLeaf) or (node | kWideTile), categories from xb
+template <int K>
+__device__ __forceinline__ void wide_extras(const HcltDev& d, const uint32_t* __restrict__ extra, int off, int cnt, int s,
+                                            int lane, int wave, v4f (&z)[(K / 16) / wide_walk_waves<K>()]) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
+  const int col = s * kSlice + (lane & 15);
+  for (int i = 0; i < cnt; ++i) {
+    const uint32_t op = extra[off + i];
+    v4f t[Q];
+    if (op & kWideLeaf) {
+      const int var = (int)(op & 0xffffffu);
+      const uint32_t x = d.xb[(size_t)var * d.Bp + col];
+      wide_request<K>(d, kWideLeaf | (uint32_t)var, x, s, lane, wave, t);
+    } else {
+      wide_request<K>(d, op, 0u, s, lane, wave, t);
+    }
+#pragma unroll
+    for (int q = 0; q < Q; ++q) z[q] += t[q];
+  }
+}
+
+// E tile of the node from the waves' slices of Z: the row maxima are combined through LDS, E
+// goes to LDS and comes back whole to every wave.  Returns m of the lane's example.  Two
+// workgroup barriers.
+template <int K>
+__device__ __forceinline__ float wide_e_from_z(const v4f (&z)[(K / 16) / wide_walk_waves<K>()], int lane, int wave,
+                                               WideLds<K>& L, v4f (&e)[K / 16]) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
+  const int b = lane & 15, g = lane >> 4;
   float m = -INFINITY;
 #pragma unroll
   for (int q = 0; q < Q; ++q)
@@ -94,101 +127,147 @@ __device__ __forceinline__ float wide_build_e(const HcltDev& d, const HcltNode& 
   return m;
 }
 
-// Forward: one workgroup per 16-example slice walks the nodes children-first.
+// Forward: one workgroup per 16-example slice walks the nodes children-first.  While a node is
+// computed, the rows of the next node's parameter block, its prefetchable operands and the
+// categories of the node after it are already on their way.
 template <int K>
-__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_kernel(HcltDev d, float* __restrict__ ll) {
+__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_kernel(HcltDev d,
+                                                                                      const WideOps* __restrict__ ops,
+                                                                                      const uint32_t* __restrict__ extra,
+                                                                                      float* __restrict__ ll) {
   constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
-  const int b = lane & 15, g = lane >> 4;
-  // this wave's rows of the parameter block wait for nothing computed here: a node's rows are
-  // requested while the node before it is being computed
-  v4f wn[Q][KT];
-  auto request_w = [&](int n) {
+  const int b = lane & 15, g = lane >> 4, col = s * kSlice + b;
+  v4f wn[Q][KT], pre[kWidePre][Q], prev_o[Q];
+  uint32_t xnext = 0;
+  auto request = [&](int n, uint32_t xpack) {
     const v4f* wf = reinterpret_cast<const v4f*>(d.Wf + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
       for (int jt = 0; jt < KT; ++jt) wn[q][jt] = wf[((wave * Q + q) * KT + jt) * 64 + lane];
-  };
-  request_w(0);
-  for (int n = 0; n < d.n_inner; ++n) {
-    const HcltNode nd = d.nodes[n];
-    v4f e[KT];
-    const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
-    v4f w[Q][KT];
+    xnext = n + 1 < d.n_inner ? d.xn[(size_t)(n + 1) * d.Bp + col] : 0u;
 #pragma unroll
-    for (int q = 0; q < Q; ++q)
+    for (int i = 0; i < kWidePre; ++i) wide_request<K>(d, ops[n].fwd[i], xpack, s, lane, wave, pre[i]);
+  };
+  request(0, d.xn[col]);
+#pragma unroll
+  for (int q = 0; q < Q; ++q) prev_o[q] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int n = 0; n < d.n_inner; ++n) {
+    const WideOps on = ops[n];
+    v4f z[Q], w[Q][KT];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      z[q] = pre[0][q];
+#pragma unroll
+      for (int i = 1; i < kWidePre; ++i) z[q] += pre[i][q];
 #pragma unroll
       for (int jt = 0; jt < KT; ++jt) w[q][jt] = wn[q][jt];
-    if (n + 1 < d.n_inner) request_w(n + 1);
+    }
+    const uint32_t xcur = xnext;
+    if (n + 1 < d.n_inner) request(n + 1, xcur);
+    if (on.prev_child)
+#pragma unroll
+      for (int q = 0; q < Q; ++q) z[q] += prev_o[q];
+    if (on.fwd_extra_cnt) wide_extras<K>(d, extra, on.fwd_extra_off, on.fwd_extra_cnt, s, lane, wave, z);
+    v4f e[KT];
+    const float m = wide_e_from_z<K>(z, lane, wave, L, e);
     v4f* out = reinterpret_cast<v4f*>(d.O + ((size_t)n * d.nslices + s) * kSlice * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
-      v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+      v4f part[4];   // four independent accumulation chains: a chain of KT*4 dependent MFMAs is half a microsecond
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[i] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int jt = 0; jt < KT; ++jt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][jt][i], e[jt][i], acc, 0, 0, 0);
+        for (int i = 0; i < 4; ++i) part[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][jt][i], e[jt][i], part[i], 0, 0, 0);
+      const v4f acc = (part[0] + part[1]) + (part[2] + part[3]);
       v4f o;
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[i] = m + __logf(acc[i]);
       out[(wave * Q + q) * 64 + lane] = o;
-      if (nd.is_root && wave == 0 && q == 0 && g == 0 && s * kSlice + b < d.B) ll[s * kSlice + b] = o[0];
+      prev_o[q] = o;
+      if (on.is_root && wave == 0 && q == 0 && g == 0 && col < d.B) ll[col] = o[0];
     }
-    __syncthreads();   // the tile is read by the parent's step; LDS is reused
+    // no barrier here: a wave reads from memory only what it wrote itself, and the next node's LDS
+    // writes sit behind its own barriers
   }
 }
 
 // Backward: the same workgroups walk the nodes parents-first.  Besides the flow tile G handed
 // to the children, every node leaves R and E in the operand layout of the statistics
 // contraction: lane 16*g' + r holds, for t < 4, the value of example 4*t + g' at state
-// kt*16 + r (the contraction runs over examples).
+// kt*16 + r (the contraction runs over examples).  A node's own value tile, its operands and its
+// parent's flow tile are requested a node ahead; when the parent is the node just computed (the
+// last non-leaf child comes right after its parent in this order) its flows are still in registers.
 template <int K>
-__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_kernel(HcltDev d, float* G,
-                                                                                       float* __restrict__ RS,
+__global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_kernel(HcltDev d,
+                                                                                       const WideOps* __restrict__ ops,
+                                                                                       const uint32_t* __restrict__ extra,
+                                                                                       float* G, float* __restrict__ RS,
                                                                                        float* __restrict__ ES) {
   constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
-  const int b = lane & 15, g = lane >> 4;
-  const bool live = s * kSlice + b < d.B;
-  v4f wn[Q][KT];
-  auto request_w = [&](int n) {
+  const int b = lane & 15, g = lane >> 4, col = s * kSlice + b;
+  const bool live = col < d.B;
+  v4f wn[Q][KT], pre[kWidePre][Q], on_next[Q], f_next[Q], prev_g[Q];
+  uint32_t xnext = 0;
+  auto request = [&](int n, uint32_t xpack) {
     const v4f* wb = reinterpret_cast<const v4f*>(d.Wb + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) wn[q][kt] = wb[((wave * Q + q) * KT + kt) * 64 + lane];
-  };
-  request_w(d.n_inner - 1);
-  for (int n = d.n_inner - 1; n >= 0; --n) {
-    const HcltNode nd = d.nodes[n];
-    v4f e[KT];
-    const float m = wide_build_e<K>(d, nd, s, lane, wave, L, e);
-    v4f w[Q][KT];
+    xnext = n > 0 ? d.xn[(size_t)(n - 1) * d.Bp + col] : 0u;
 #pragma unroll
-    for (int q = 0; q < Q; ++q)
+    for (int i = 0; i < kWidePre; ++i) wide_request<K>(d, ops[n].bwd[i], xpack, s, lane, wave, pre[i]);
+    const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
+    const int par = ops[n].parent;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      on_next[q] = reinterpret_cast<const v4f*>(d.O + tile)[(wave * Q + q) * 64 + lane];
+      f_next[q] = v4f{0.f, 0.f, 0.f, 0.f};
+      if (par >= 0 && par != n + 1)
+        f_next[q] = reinterpret_cast<const v4f*>(G + ((size_t)par * d.nslices + s) * kSlice * K)[(wave * Q + q) * 64 + lane];
+    }
+  };
+  request(d.n_inner - 1, d.xn[(size_t)(d.n_inner - 1) * d.Bp + col]);
+#pragma unroll
+  for (int q = 0; q < Q; ++q) prev_g[q] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int n = d.n_inner - 1; n >= 0; --n) {
+    const WideOps on = ops[n];
+    v4f z[Q], w[Q][KT], o[Q], f[Q];
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+      z[q] = pre[0][q];
+#pragma unroll
+      for (int i = 1; i < kWidePre; ++i) z[q] += pre[i][q];
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) w[q][kt] = wn[q][kt];
-    if (n > 0) request_w(n - 1);
+      o[q] = on_next[q];
+      f[q] = f_next[q];
+    }
+    const uint32_t xcur = xnext;
+    if (n > 0) request(n - 1, xcur);
+    if (on.bwd_extra_cnt) wide_extras<K>(d, extra, on.bwd_extra_off, on.bwd_extra_cnt, s, lane, wave, z);
+    v4f e[KT];
+    const float m = wide_e_from_z<K>(z, lane, wave, L, e);
     const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
-    const v4f* on = reinterpret_cast<const v4f*>(d.O + tile);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
       const int kt = wave * Q + q;
-      const v4f o = on[kt * 64 + lane];
-      v4f f;
-      if (nd.parent < 0) {
-        f = v4f{kt == 0 && g == 0 && live ? 1.f : 0.f, 0.f, 0.f, 0.f};
-      } else {
-        f = reinterpret_cast<const v4f*>(G + ((size_t)nd.parent * d.nslices + s) * kSlice * K)[kt * 64 + lane];
-      }
+      v4f fq;
+      if (on.parent < 0) fq = v4f{kt == 0 && g == 0 && live ? 1.f : 0.f, 0.f, 0.f, 0.f};
+      else if (on.parent == n + 1) fq = prev_g[q];
+      else fq = f[q];
       v4f r;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float sc = __expf(o[i] - m);
-        r[i] = (sc > 0.f && f[i] > 0.f) ? f[i] / sc : 0.f;
+        const float sc = __expf(o[q][i] - m);
+        r[i] = (sc > 0.f && fq[i] > 0.f) ? fq[i] / sc : 0.f;
       }
       L.r[kt][lane] = r;
     }
@@ -200,12 +279,16 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
       const int jt = wave * Q + q;
-      v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+      v4f part[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) part[i] = v4f{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][kt][i], r[kt][i], acc, 0, 0, 0);
-      gout[jt * 64 + lane] = e[jt] * acc;
+        for (int i = 0; i < 4; ++i) part[i] = __builtin_amdgcn_mfma_f32_16x16x4f32(w[q][kt][i], r[kt][i], part[i], 0, 0, 0);
+      const v4f acc = (part[0] + part[1]) + (part[2] + part[3]);
+      prev_g[q] = e[jt] * acc;
+      gout[jt * 64 + lane] = prev_g[q];
     }
     // statistics operands: lane = 16*g' + row reads example 4*t + g', state kt*16 + row
     {
@@ -224,7 +307,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
         reinterpret_cast<v4f*>(ES + tile)[kt * 64 + lane] = es;
       }
     }
-    __syncthreads();   // G is read by the children's steps; LDS is reused
+    // no barrier here: see the forward walk (L.r and L.e are rewritten only behind the next node's barriers)
   }
 }
 
@@ -336,10 +419,48 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev
     default: fail(PCM_ERR_STATE, "no wide block kernel for hidden size %d", K_);             \
   }
 
+// operand tables of the wide walks
+void HcltCircuit::build_wide_tables() {
+  std::vector<WideOps> t(n_inner_);
+  std::vector<uint32_t> extra;
+  std::vector<std::vector<int32_t>> ic(n_inner_), lc(n_inner_);
+  for (int n = 0; n < n_inner_; ++n)
+    for (int c : children_[var_of_inner_[n]]) {
+      if (children_[c].empty()) lc[n].push_back(c); else ic[n].push_back(inner_of_var_[c]);
+    }
+  for (int n = 0; n < n_inner_; ++n) {
+    WideOps& o = t[n];
+    std::memset(&o, 0, sizeof(o));
+    const int v = var_of_inner_[n];
+    o.parent = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+    o.is_root = v == root_;
+    o.fwd[0] = o.bwd[0] = kWideLeaf | (uint32_t)v;
+    for (size_t i = 0; i < lc[n].size() && i < 3; ++i) o.fwd[1 + i] = o.bwd[1 + i] = kWideLeaf | ((uint32_t)(i + 1) << 24) | (uint32_t)lc[n][i];
+    std::vector<uint32_t> fx, bx;
+    for (size_t i = 3; i < lc[n].size(); ++i) { fx.push_back(kWideLeaf | (uint32_t)lc[n][i]); bx.push_back(fx.back()); }
+    int nf = 0, nb = 0;
+    for (int c : ic[n]) {
+      const uint32_t op = kWideTile | (uint32_t)c;
+      if (c == n - 1) o.prev_child = 1;
+      else if (nf < 2) o.fwd[4 + nf++] = op;
+      else fx.push_back(op);
+      if (nb < 2) o.bwd[4 + nb++] = op; else bx.push_back(op);
+    }
+    o.fwd_extra_off = (int32_t)extra.size(); o.fwd_extra_cnt = (int32_t)fx.size();
+    extra.insert(extra.end(), fx.begin(), fx.end());
+    o.bwd_extra_off = (int32_t)extra.size(); o.bwd_extra_cnt = (int32_t)bx.size();
+    extra.insert(extra.end(), bx.begin(), bx.end());
+  }
+  if (extra.empty()) extra.push_back(0);
+  d_wide_ops_.upload(t);
+  d_wide_extra_.upload(extra);
+}
+
 void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
+  if (d_wide_ops_.n == 0) build_wide_tables();
   if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
   PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0,
-                                             stream, d, d_ll));
+                                             stream, d, d_wide_ops_.p, d_wide_extra_.p, d_ll));
   check_launch_w("hclt_wide_forward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
@@ -356,8 +477,8 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   PCM_DISPATCH_WIDE_K(K_, {
-    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0, stream, d, d_G_.p,
-                       d_wide_rs_.p, d_wide_es_.p);
+    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0, stream, d,
+                       d_wide_ops_.p, d_wide_extra_.p, d_G_.p, d_wide_rs_.p, d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
     if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
     hipLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream, d,
