@@ -54,8 +54,8 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
  * is given when the `pcs` are num_heads root sum nodes over the K products of one HCLT body (the patch
  * circuits of exps/progressive_growing/parallel_PG.jl:214-225 before pruning).  Runs on the block engine:
  * the body through the tree-walk kernels, the heads as an [H][K] block in two small kernels around them.
- * Needs num_hidden_cats 16 or 32 and at most three children per tree node (PCM_ERR_UNSUPPORTED otherwise:
- * describe the circuit to pcm_circuit_create instead).  Parameter vector: the body's sum parameters in
+ * Needs num_hidden_cats 16 or 32 (PCM_ERR_UNSUPPORTED otherwise: describe the circuit to pcm_circuit_create
+ * instead).  Parameter vector: the body's sum parameters in
  * the order of pcm_hclt_create without the root's row, then num_heads x K head parameters, then the input
  * nodes; the same order pcm_circuit_create gives the equivalent description.  pcm_loglikelihoods returns
  * [num_heads][batch], pcm_flows takes d_head_mask [num_heads][batch]; KL and sampling are not defined.
