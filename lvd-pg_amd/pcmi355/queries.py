@@ -109,11 +109,14 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
 
 def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
                            ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
-                           shuffle="each_epoch", verbose=False, generator=None, head_mask=None):
+                           shuffle="each_epoch", verbose=False, generator=None, head_mask=None, eval_dataset=None,
+                           eval_interval=0):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
     of per-epoch mean log-likelihoods.  soft_reg and ent_reg must be 0 (the reference's
     entropy regulariser is commented out at :294-296).  `data` may be 3-D float32 soft evidence,
-    as for the top-level circuits of exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl."""
+    as for the top-level circuits of exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl.
+    With `verbose`, every `eval_interval` epochs the mean log-likelihood of `eval_dataset` is printed
+    beside the training one (:308-327)."""
     if soft_reg != 0.0 or ent_reg != 0.0:
         raise NotImplementedError("soft_reg / ent_reg other than 0 are not supported")
     _check_data(bpc, data)
@@ -155,7 +158,12 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
         lls.append(float(acc.item()) / batch_size / num_batches)
         param_inertia += d_inertia
         if verbose:
-            print(f"Mini-batch EM epoch {len(lls)}/{num_epochs}; train LL {lls[-1]}")
+            epoch = len(lls)
+            if eval_dataset is not None and eval_interval > 0 and epoch % eval_interval == 0 and hm_t is None:
+                test_ll = float(loglikelihoods(bpc, eval_dataset, batch_size=min(batch_size, eval_dataset.shape[0])).mean().item())
+                print(f"Mini-batch EM epoch {epoch}/{num_epochs}: train LL {lls[-1]} - test LL {test_ll}")
+            else:
+                print(f"Mini-batch EM epoch {epoch}/{num_epochs}; train LL {lls[-1]}")
     return lls
 
 
