@@ -15,7 +15,7 @@
 namespace pcm {
 
 constexpr int kSlice = 16;       // examples per tile
-constexpr double kWideNodeUs = 1.6, kWalk64StepUs = 7.6;   // measured costs behind the choice of walk kernels at K = 64
+constexpr double kWideNodeUs = 1.2, kWalk64StepUs = 7.6;   // measured costs behind the choice of walk kernels at K = 64
 constexpr int kWalkWaves = 16;   // waves per workgroup (= items per step) in the tree-walk kernels
 constexpr int kInlineOps = 4;    // static operands held in a step item
 constexpr int kInlineLds = 3;    // LDS-resident operands held in a step item

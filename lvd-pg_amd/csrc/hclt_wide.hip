@@ -55,23 +55,69 @@ struct WideLds {
 constexpr int kWidePre = 6;
 constexpr uint32_t kWideLeaf = 0x80000000u, kWideTile = 0x40000000u;
 
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t wide_rsrc(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+// What a walk keeps in scalar registers for its requests: one descriptor over the whole leaf (or
+// value) table and one over the value tiles, and the strides.  Slots 0..3 of a node's operand list
+// are always leaf rows, slots 4..5 always value tiles, so a request is one multiply for the
+// offset and a raw buffer load; an absent operand is pushed out of the descriptor's range (the
+// load returns zeros and never reaches memory), so there is no control flow for the compiler to
+// place waits at and the values stay in flight until the next node consumes them.
+struct WideRsrc {
+  __amdgpu_buffer_rsrc_t leaf, tile;
+  uint32_t leaf_stride, tile_stride, leaf_lane, tile_lane;   // *_lane: this lane's byte offset inside a row / a node's tiles
+};
+
+template <int K>
+__device__ __forceinline__ WideRsrc wide_rsrcs(const HcltDev& d, int s, int lane) {
+  WideRsrc r;
+  r.leaf = wide_rsrc(d.leaf, (uint32_t)d.V * d.leaf_stride);
+  r.tile = wide_rsrc(d.O, (uint32_t)d.n_inner * d.tile_stride);
+  r.leaf_stride = d.leaf_stride;
+  r.tile_stride = d.tile_stride;
+  r.leaf_lane = (uint32_t)s * d.leaf_slice + (uint32_t)(lane >> 4) * 16;
+  r.tile_lane = (uint32_t)s * (kSlice * K * 4) + (uint32_t)lane * 16;
+  return r;
+}
+
+constexpr uint32_t kWideAbsent = 0x80000000u;   // beyond any table (the host keeps them under 2 GB), and the row-tile steps cannot wrap
+
+template <int K>
+__device__ __forceinline__ void wide_request_leaf(const WideRsrc& r, uint32_t op_, uint32_t xpack, int wave,
+                                                  v4f (&out)[(K / 16) / wide_walk_waves<K>()]) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
+  const uint32_t op = (uint32_t)__builtin_amdgcn_readfirstlane((int)op_);
+  const uint32_t x = (xpack >> (8u * ((op >> 24) & 3u))) & 0xffu;
+  const uint32_t voff = op ? x * (K * 4) + r.leaf_lane : kWideAbsent;
+  const uint32_t soff = (op & 0xffffffu) * r.leaf_stride;
+#pragma unroll
+  for (int q = 0; q < Q; ++q)
+    out[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r.leaf, (int)(voff + (wave * Q + q) * 64), (int)soff, 0));
+}
+
+template <int K>
+__device__ __forceinline__ void wide_request_tile(const WideRsrc& r, uint32_t op_, int wave,
+                                                  v4f (&out)[(K / 16) / wide_walk_waves<K>()]) {
+  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
+  const uint32_t op = (uint32_t)__builtin_amdgcn_readfirstlane((int)op_);
+  const uint32_t voff = op ? r.tile_lane : kWideAbsent;
+  const uint32_t soff = (op & 0xffffffu) * r.tile_stride;
+#pragma unroll
+  for (int q = 0; q < Q; ++q)
+    out[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r.tile, (int)(voff + (wave * Q + q) * 1024), (int)soff, 0));
+}
+
+// point-of-use form for the rare operands beyond the prefetched ones
 template <int K>
 __device__ __forceinline__ void wide_request(const HcltDev& d, uint32_t op, uint32_t xpack, int s, int lane, int wave,
                                              v4f (&out)[(K / 16) / wide_walk_waves<K>()]) {
-  constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
-#pragma unroll
-  for (int q = 0; q < Q; ++q) out[q] = v4f{0.f, 0.f, 0.f, 0.f};
-  if (op & kWideLeaf) {
-    const int var = (int)(op & 0xffffffu), sel = (int)((op >> 24) & 3u);
-    const uint32_t x = (xpack >> (8 * sel)) & 0xffu;
-    const float* row = d.leaf + (size_t)var * (d.leaf_stride / 4) + (size_t)x * K + (size_t)s * (d.leaf_slice / 4);
-#pragma unroll
-    for (int q = 0; q < Q; ++q) out[q] = *reinterpret_cast<const v4f*>(row + (wave * Q + q) * 16 + 4 * (lane >> 4));
-  } else if (op & kWideTile) {
-    const v4f* t = reinterpret_cast<const v4f*>(d.O + ((size_t)(op & 0xffffffu) * d.nslices + s) * kSlice * K);
-#pragma unroll
-    for (int q = 0; q < Q; ++q) out[q] = t[(wave * Q + q) * 64 + lane];
-  }
+  const WideRsrc r = wide_rsrcs<K>(d, s, lane);
+  if (op & kWideLeaf) wide_request_leaf<K>(r, op, xpack, wave, out);
+  else wide_request_tile<K>(r, op, wave, out);
 }
 
 // operands beyond the prefetched ones: (variable | kWideLeaf) or (node | kWideTile), categories from xb
@@ -95,6 +141,27 @@ __device__ __forceinline__ void wide_extras(const HcltDev& d, const uint32_t* __
   }
 }
 
+// The operand table of small trees is copied to LDS once: read from memory it costs every node a
+// scalar-cache round trip ahead of its requests.
+__device__ __forceinline__ void wide_stage_ops(const WideOps* __restrict__ ops_g, int n_inner, int in_lds, uint32_t* sops_mem) {
+  if (!in_lds) return;
+  const uint32_t* src = reinterpret_cast<const uint32_t*>(ops_g);
+  const int words = n_inner * (int)(sizeof(WideOps) / 4);
+  for (int i = threadIdx.x; i < words; i += blockDim.x) sops_mem[i] = src[i];
+  __syncthreads();
+}
+
+// a node's entry, from LDS (explicitly: a generic pointer would turn every read into a flat load) or memory
+__device__ __forceinline__ WideOps wide_ops_at(const WideOps* __restrict__ ops_g, int in_lds, const uint32_t* sops_mem, int n) {
+  if (!in_lds) return ops_g[n];
+  WideOps o;
+  uint32_t* dst = reinterpret_cast<uint32_t*>(&o);
+  const uint32_t* src = sops_mem + (size_t)n * (sizeof(WideOps) / 4);
+#pragma unroll
+  for (int i = 0; i < (int)(sizeof(WideOps) / 4); ++i) dst[i] = src[i];
+  return o;
+}
+
 // E tile of the node from the waves' slices of Z: the row maxima are combined through LDS, E
 // goes to LDS and comes back whole to every wave.  Returns m of the lane's example.  Two
 // workgroup barriers.
@@ -108,8 +175,14 @@ __device__ __forceinline__ float wide_e_from_z(const v4f (&z)[(K / 16) / wide_wa
   for (int q = 0; q < Q; ++q)
 #pragma unroll
     for (int i = 0; i < 4; ++i) m = fmaxf(m, z[q][i]);
-  m = fmaxf(m, __shfl_xor(m, 16));
-  m = fmaxf(m, __shfl_xor(m, 32));
+  {   // lanes ^ 16 and ^ 32 with the row- and half-swap instructions, not through the LDS crossbar
+    const int mi = __builtin_bit_cast(int, m);
+    const auto r16 = __builtin_amdgcn_permlane16_swap(mi, mi, false, false);
+    m = fmaxf(__builtin_bit_cast(float, (int)r16[0]), __builtin_bit_cast(float, (int)r16[1]));
+    const int mj = __builtin_bit_cast(int, m);
+    const auto r32 = __builtin_amdgcn_permlane32_swap(mj, mj, false, false);
+    m = fmaxf(__builtin_bit_cast(float, (int)r32[0]), __builtin_bit_cast(float, (int)r32[1]));
+  }
   if (g == 0) L.mx[wave][b] = m;
   __syncthreads();
 #pragma unroll
@@ -132,30 +205,38 @@ __device__ __forceinline__ float wide_e_from_z(const v4f (&z)[(K / 16) / wide_wa
 // categories of the node after it are already on their way.
 template <int K>
 __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_kernel(HcltDev d,
-                                                                                      const WideOps* __restrict__ ops,
+                                                                                      const WideOps* __restrict__ ops_g,
+                                                                                      int ops_in_lds,
                                                                                       const uint32_t* __restrict__ extra,
                                                                                       float* __restrict__ ll) {
   constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
+  extern __shared__ uint32_t sops_mem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
   const int b = lane & 15, g = lane >> 4, col = s * kSlice + b;
+  wide_stage_ops(ops_g, d.n_inner, ops_in_lds, sops_mem);
+  const WideRsrc rs = wide_rsrcs<K>(d, s, lane);
   v4f wn[Q][KT], pre[kWidePre][Q], prev_o[Q];
   uint32_t xnext = 0;
+  WideOps on_next;
   auto request = [&](int n, uint32_t xpack) {
     const v4f* wf = reinterpret_cast<const v4f*>(d.Wf + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
       for (int jt = 0; jt < KT; ++jt) wn[q][jt] = wf[((wave * Q + q) * KT + jt) * 64 + lane];
-    xnext = n + 1 < d.n_inner ? d.xn[(size_t)(n + 1) * d.Bp + col] : 0u;
+    xnext = d.xn[(size_t)min(n + 1, d.n_inner - 1) * d.Bp + col];
+    on_next = wide_ops_at(ops_g, ops_in_lds, sops_mem, n);
 #pragma unroll
-    for (int i = 0; i < kWidePre; ++i) wide_request<K>(d, ops[n].fwd[i], xpack, s, lane, wave, pre[i]);
+    for (int i = 0; i < 4; ++i) wide_request_leaf<K>(rs, on_next.fwd[i], xpack, wave, pre[i]);
+#pragma unroll
+    for (int i = 4; i < kWidePre; ++i) wide_request_tile<K>(rs, on_next.fwd[i], wave, pre[i]);
   };
   request(0, d.xn[col]);
 #pragma unroll
   for (int q = 0; q < Q; ++q) prev_o[q] = v4f{0.f, 0.f, 0.f, 0.f};
   for (int n = 0; n < d.n_inner; ++n) {
-    const WideOps on = ops[n];
+    const WideOps on = on_next;
     v4f z[Q], w[Q][KT];
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -166,7 +247,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_k
       for (int jt = 0; jt < KT; ++jt) w[q][jt] = wn[q][jt];
     }
     const uint32_t xcur = xnext;
-    if (n + 1 < d.n_inner) request(n + 1, xcur);
+    request(min(n + 1, d.n_inner - 1), xcur);   // past the last node: a repeat of its requests, never used
     if (on.prev_child)
 #pragma unroll
       for (int q = 0; q < Q; ++q) z[q] += prev_o[q];
@@ -204,41 +285,51 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_k
 // last non-leaf child comes right after its parent in this order) its flows are still in registers.
 template <int K>
 __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_kernel(HcltDev d,
-                                                                                       const WideOps* __restrict__ ops,
+                                                                                       const WideOps* __restrict__ ops_g,
+                                                                                       int ops_in_lds,
                                                                                        const uint32_t* __restrict__ extra,
                                                                                        float* G, float* __restrict__ RS,
                                                                                        float* __restrict__ ES) {
   constexpr int KT = K / 16, WV = wide_walk_waves<K>(), Q = KT / WV;
   __shared__ WideLds<K> L;
+  extern __shared__ uint32_t sops_mem[];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, s = blockIdx.x;
   const int b = lane & 15, g = lane >> 4, col = s * kSlice + b;
+  wide_stage_ops(ops_g, d.n_inner, ops_in_lds, sops_mem);
+  const WideRsrc rs = wide_rsrcs<K>(d, s, lane);
   const bool live = col < d.B;
-  v4f wn[Q][KT], pre[kWidePre][Q], on_next[Q], f_next[Q], prev_g[Q];
+  v4f wn[Q][KT], pre[kWidePre][Q], o_next[Q], f_next[Q], prev_g[Q];
   uint32_t xnext = 0;
+  WideOps on_next;
   auto request = [&](int n, uint32_t xpack) {
     const v4f* wb = reinterpret_cast<const v4f*>(d.Wb + (size_t)n * K * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q)
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) wn[q][kt] = wb[((wave * Q + q) * KT + kt) * 64 + lane];
-    xnext = n > 0 ? d.xn[(size_t)(n - 1) * d.Bp + col] : 0u;
+    xnext = d.xn[(size_t)max(n - 1, 0) * d.Bp + col];
+    on_next = wide_ops_at(ops_g, ops_in_lds, sops_mem, n);
 #pragma unroll
-    for (int i = 0; i < kWidePre; ++i) wide_request<K>(d, ops[n].bwd[i], xpack, s, lane, wave, pre[i]);
-    const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
-    const int par = ops[n].parent;
+    for (int i = 0; i < 4; ++i) wide_request_leaf<K>(rs, on_next.bwd[i], xpack, wave, pre[i]);
+#pragma unroll
+    for (int i = 4; i < kWidePre; ++i) wide_request_tile<K>(rs, on_next.bwd[i], wave, pre[i]);
+    const int par = __builtin_amdgcn_readfirstlane(on_next.parent);
+    const bool from_mem = par >= 0 && par != n + 1;   // otherwise: the root, or the flows are still in registers
+    const __amdgpu_buffer_rsrc_t ro = wide_rsrc(reinterpret_cast<const char*>(d.O) + (size_t)n * d.tile_stride, d.tile_stride);
+    const __amdgpu_buffer_rsrc_t rg = wide_rsrc(reinterpret_cast<const char*>(G) + (size_t)max(par, 0) * d.tile_stride,
+                                                from_mem ? d.tile_stride : 0u);
+    const uint32_t voff = (uint32_t)s * (kSlice * K * 4) + (uint32_t)lane * 16;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
-      on_next[q] = reinterpret_cast<const v4f*>(d.O + tile)[(wave * Q + q) * 64 + lane];
-      f_next[q] = v4f{0.f, 0.f, 0.f, 0.f};
-      if (par >= 0 && par != n + 1)
-        f_next[q] = reinterpret_cast<const v4f*>(G + ((size_t)par * d.nslices + s) * kSlice * K)[(wave * Q + q) * 64 + lane];
+      o_next[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(ro, (int)(voff + (wave * Q + q) * 1024), 0, 0));
+      f_next[q] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rg, (int)(voff + (wave * Q + q) * 1024), 0, 0));
     }
   };
   request(d.n_inner - 1, d.xn[(size_t)(d.n_inner - 1) * d.Bp + col]);
 #pragma unroll
   for (int q = 0; q < Q; ++q) prev_g[q] = v4f{0.f, 0.f, 0.f, 0.f};
   for (int n = d.n_inner - 1; n >= 0; --n) {
-    const WideOps on = ops[n];
+    const WideOps on = on_next;
     v4f z[Q], w[Q][KT], o[Q], f[Q];
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -247,11 +338,11 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
       for (int i = 1; i < kWidePre; ++i) z[q] += pre[i][q];
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) w[q][kt] = wn[q][kt];
-      o[q] = on_next[q];
+      o[q] = o_next[q];
       f[q] = f_next[q];
     }
     const uint32_t xcur = xnext;
-    if (n > 0) request(n - 1, xcur);
+    request(max(n - 1, 0), xcur);   // past the last node: a repeat of its requests, never used
     if (on.bwd_extra_cnt) wide_extras<K>(d, extra, on.bwd_extra_off, on.bwd_extra_cnt, s, lane, wave, z);
     v4f e[KT];
     const float m = wide_e_from_z<K>(z, lane, wave, L, e);
@@ -458,9 +549,14 @@ void HcltCircuit::build_wide_tables() {
 
 void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
   if (d_wide_ops_.n == 0) build_wide_tables();
+  if ((size_t)V_ * d.leaf_stride >= ((size_t)1 << 31) || (size_t)n_inner_ * d.tile_stride >= ((size_t)1 << 31))
+    fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call of the wide kernels", d.B);
   if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
-  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0,
-                                             stream, d, d_wide_ops_.p, d_wide_extra_.p, d_ll));
+  const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
+  const int ops_in_lds = ops_bytes <= 32768;
+  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
+                                             ops_in_lds ? ops_bytes : 0, stream, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p,
+                                             d_ll));
   check_launch_w("hclt_wide_forward");
   if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
@@ -477,8 +573,11 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   PCM_DISPATCH_WIDE_K(K_, {
-    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64), 0, stream, d,
-                       d_wide_ops_.p, d_wide_extra_.p, d_G_.p, d_wide_rs_.p, d_wide_es_.p);
+    const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
+    const int ops_in_lds = ops_bytes <= 32768;
+    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
+                       ops_in_lds ? ops_bytes : 0, stream, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_G_.p, d_wide_rs_.p,
+                       d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
     if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
     hipLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream, d,
