@@ -1048,8 +1048,8 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
   PCM_DISPATCH_K(K_, {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_soft_leafval_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(hclt_soft_leafval_kernel<KK>, dim3(V_, Bp64 / kEvExamples), dim3(256), lds, stream, s, d_leaf_.p, C_,
-                       s.batch, Bp64, d_soft_lv_.p, d_soft_m_.p);
+    hipLaunchKernelGGL(hclt_soft_leafval_kernel<KK>, dim3(ceil_div(V_, kEvVars), Bp64 / kEvExamples), dim3(4 * (KK / 16) * 64), lds,
+                       stream, s, d_leaf_.p, C_, V_, s.batch, Bp64, d_soft_lv_.p, d_soft_m_.p);
   });
   check_launch("soft_leafval");
   d.leaf = d_soft_lv_.p;

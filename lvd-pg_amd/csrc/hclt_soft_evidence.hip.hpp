@@ -24,7 +24,8 @@ namespace pcm {
 
 constexpr int kEvExamples = 64;   // examples per evidence tile
 constexpr int kEvCats = 64;       // categories per tile of the flow kernel
-constexpr int kEvBatch = 8;       // evidence requests a thread keeps in flight while staging a tile
+constexpr int kEvVars = 1;        // variables a workgroup of the value kernel takes in turn (more: longer contiguous rows, fewer workgroups; no gain measured)
+constexpr int kEvBatch = 16;      // evidence requests a thread keeps in flight while staging a tile
 constexpr float kEvTiny = 1e-26f;     // e^-60: below it the factored sum has lost its footing
 constexpr float kEvFar = 59.f;        // value more than this below the largest evidence: exact flow
 
@@ -39,100 +40,110 @@ __device__ __forceinline__ float soft_ev(const SoftRef& s, int b, int v, int c) 
   return s.d_ev[e * s.stride_ex + (int64_t)v * s.stride_var + (int64_t)c * s.stride_cat];
 }
 
-// value table and per-example maxima of one batch; grid (V, Bp / 64), 256 threads.
+// value table and per-example maxima of one batch; grid (ceil(V / kEvVars), Bp / 64), 4 * K/16 waves.
 // LDS: E tile [64][LD] | P = exp(leaf[v]) [Cp][K + 16] | row maxima [64]; Cp = C rounded up to 4.
-// Wave w contracts examples 16w..16w+15 against all K states on the matrix cores
+// Wave w contracts examples 16*(w%4).. against states 16*(w/4).. on the matrix cores
 // (v_mfma_f32_16x16x4_f32: A = E, rows examples; B = P, columns states; 4 categories a step).
+// Many short waves rather than four long ones: every phase is a chain of LDS round trips.
 template <int K>
-__global__ __launch_bounds__(256) void hclt_soft_leafval_kernel(SoftRef s, const float* __restrict__ leaf, int C, int B, int Bp,
-                                                                float* __restrict__ LV, float* __restrict__ M) {
+__global__ __launch_bounds__(4 * (K / 16) * 64) void hclt_soft_leafval_kernel(SoftRef s, const float* __restrict__ leaf, int C,
+                                                                              int V, int B, int Bp, float* __restrict__ LV,
+                                                                              float* __restrict__ M) {
   extern __shared__ __align__(16) float smem[];
-  constexpr int KT = K / 16, LDP = K + 16;
+  constexpr int KT = K / 16, LDP = K + 16, NW = 4 * KT, NT = NW * 64, TPE = NT / kEvExamples;   // threads per example
   const int Cp = (C + 3) & ~3, LD = Cp + 4;
   float* tile = smem;
   float* Pt = tile + kEvExamples * LD;
   float* rmax = Pt + (size_t)Cp * LDP;
-  const int v = blockIdx.x, b0 = blockIdx.y * kEvExamples;   // neighbouring workgroups read neighbouring segments of the same rows
+  const int b0 = blockIdx.y * kEvExamples;
   const bool cat_fast = s.stride_cat == 1;
-  // eight requests in flight per thread: one at a time the tile is a chain of memory latencies
-  for (int i0 = threadIdx.x; i0 < kEvExamples * C; i0 += 256 * kEvBatch) {
-    float tmp[kEvBatch];
+  const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // a run of kEvVars variables per workgroup: with [examples][variables][categories] evidence the
+  // rows it reads are kEvVars * C contiguous floats each, and neighbouring workgroups continue them
+  for (int v = blockIdx.x * kEvVars; v < min((int)(blockIdx.x + 1) * kEvVars, V); ++v) {
+  if (v != (int)blockIdx.x * kEvVars) __syncthreads();   // the previous variable's tiles are still being read
+  // Evidence tile: lanes run along whichever of (category, example) is contiguous in memory, waves
+  // along the other; no division by the run-time C, kEvBatch requests in flight per thread.
+  {
+    const int n_fast = cat_fast ? C : kEvExamples, n_slow = cat_fast ? kEvExamples : C;
+    for (int f0 = 0; f0 < n_fast; f0 += 64) {
+      const int f = f0 + lane;
+      for (int s0 = w; s0 < n_slow; s0 += NW * kEvBatch) {
+        float tmp[kEvBatch];
 #pragma unroll
-    for (int u = 0; u < kEvBatch; ++u) {
-      const int i = i0 + u * 256;
-      const int e = cat_fast ? i / C : i % kEvExamples, c = cat_fast ? i % C : i / kEvExamples;
-      tmp[u] = (i < kEvExamples * C && b0 + e < B) ? soft_ev(s, b0 + e, v, c) : 0.f;
-    }
+        for (int u = 0; u < kEvBatch; ++u) {
+          const int sl = s0 + NW * u;
+          const int e = cat_fast ? sl : f, c = cat_fast ? f : sl;
+          tmp[u] = (f < n_fast && sl < n_slow && b0 + e < B) ? soft_ev(s, b0 + e, v, c) : 0.f;
+        }
 #pragma unroll
-    for (int u = 0; u < kEvBatch; ++u) {
-      const int i = i0 + u * 256;
-      const int e = cat_fast ? i / C : i % kEvExamples, c = cat_fast ? i % C : i / kEvExamples;
-      if (i < kEvExamples * C) tile[e * LD + c] = tmp[u];
+        for (int u = 0; u < kEvBatch; ++u) {
+          const int sl = s0 + NW * u;
+          const int e = cat_fast ? sl : f, c = cat_fast ? f : sl;
+          if (f < n_fast && sl < n_slow) tile[e * LD + c] = tmp[u];
+        }
+      }
     }
   }
-  // P, zero rows up to Cp
-  for (int i0 = threadIdx.x; i0 < Cp * K; i0 += 256 * kEvBatch) {
-    float tmp[kEvBatch];
+  for (int i0 = threadIdx.x; i0 < Cp * K; i0 += NT * 8) {
+    float tmp[8];
 #pragma unroll
-    for (int u = 0; u < kEvBatch; ++u) {
-      const int i = i0 + u * 256;
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * NT;
       tmp[u] = i < C * K ? leaf[(size_t)v * C * K + i] : -INFINITY;
     }
 #pragma unroll
-    for (int u = 0; u < kEvBatch; ++u) {
-      const int i = i0 + u * 256;
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * NT;
       if (i < Cp * K) Pt[(i / K) * LDP + i % K] = __expf(tmp[u]);
     }
   }
   __syncthreads();
   {
-    // four threads per example: row maximum, then E = exp(ev - m) in place (columns C..Cp-1: 0)
-    const int e = threadIdx.x >> 2, sub = threadIdx.x & 3;
+    // TPE threads per example: row maximum, then E = exp(ev - m) in place (columns C..Cp-1: 0)
+    const int e = threadIdx.x / TPE, sub = threadIdx.x % TPE;
     float m = -INFINITY;
-    for (int c = sub; c < C; c += 4) m = fmaxf(m, tile[e * LD + c]);
-    m = fmaxf(m, __shfl_xor(m, 1));
-    m = fmaxf(m, __shfl_xor(m, 2));
+    for (int c = sub; c < C; c += TPE) m = fmaxf(m, tile[e * LD + c]);
+#pragma unroll
+    for (int o = 1; o < TPE; o <<= 1) m = fmaxf(m, __shfl_xor(m, o));
     if (!(m > -INFINITY)) m = 0.f;
-    for (int c = sub; c < Cp; c += 4) tile[e * LD + c] = c < C ? __expf(tile[e * LD + c] - m) : 0.f;
+    for (int c = sub; c < Cp; c += TPE) tile[e * LD + c] = c < C ? __expf(tile[e * LD + c] - m) : 0.f;
     if (sub == 0) rmax[e] = m;
   }
   __syncthreads();
-  const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int r = lane & 15, g = lane >> 4;
-  v4f acc[KT];
-#pragma unroll
-  for (int kt = 0; kt < KT; ++kt) acc[kt] = v4f{0.f, 0.f, 0.f, 0.f};
-  const float* arow = tile + (16 * w + r) * LD + g;
-  const float* brow = Pt + g * LDP + r;
-  for (int c0 = 0; c0 < Cp; c0 += 4) {
-    const float a = arow[c0];
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) acc[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, brow[c0 * LDP + kt * 16], acc[kt], 0, 0, 0);
+  const int r = lane & 15, g = lane >> 4, bt = w & 3, kt = w >> 2;
+  v4f acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0;   // two chains
+  const float* arow = tile + (16 * bt + r) * LD + g;
+  const float* brow = Pt + g * LDP + kt * 16 + r;
+  int c0 = 0;
+  for (; c0 + 8 <= Cp; c0 += 8) {
+    acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(arow[c0], brow[c0 * LDP], acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(arow[c0 + 4], brow[(c0 + 4) * LDP], acc1, 0, 0, 0);
   }
-  // accumulator element i of tile kt: example 16w + 4g + i, state kt*16 + r
+  if (c0 < Cp) acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(arow[c0], brow[c0 * LDP], acc0, 0, 0, 0);
+  const v4f acc = acc0 + acc1;
+  // accumulator element i: example 16*bt + 4g + i, state kt*16 + r
+  const int k = kt * 16 + r;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int e = 16 * w + 4 * g + i, b = b0 + e;
+    const int e = 16 * bt + 4 * g + i, b = b0 + e;
     const float m = rmax[e];
-#pragma unroll
-    for (int kt = 0; kt < KT; ++kt) {
-      const int k = kt * 16 + r;
-      float val = 0.f;
-      if (b < B) {
-        val = m + __logf(acc[kt][i]);
-        if (!(acc[kt][i] > kEvTiny)) {            // the favoured category is all but impossible under this leaf
-          float mx = -INFINITY, sm = 0.f;
-          for (int c = 0; c < C; ++c) {
-            const float t = soft_ev(s, b, v, c) + leaf[((size_t)v * C + c) * K + k];
-            if (t > mx) { sm = sm * __expf(mx - t) + 1.f; mx = t; }
-            else if (t > -INFINITY) sm += __expf(t - mx);
-          }
-          val = mx > -INFINITY ? mx + __logf(sm) : -INFINITY;
+    float val = 0.f;
+    if (b < B) {
+      val = m + __logf(acc[i]);
+      if (!(acc[i] > kEvTiny)) {            // the favoured category is all but impossible under this leaf
+        float mx = -INFINITY, sm = 0.f;
+        for (int c = 0; c < C; ++c) {
+          const float t = soft_ev(s, b, v, c) + leaf[((size_t)v * C + c) * K + k];
+          if (t > mx) { sm = sm * __expf(mx - t) + 1.f; mx = t; }
+          else if (t > -INFINITY) sm += __expf(t - mx);
         }
+        val = mx > -INFINITY ? mx + __logf(sm) : -INFINITY;
       }
-      LV[((size_t)v * Bp + b) * K + k] = val;
     }
-    if (r == 0) M[(size_t)v * Bp + b] = b < B ? m : 0.f;
+    LV[((size_t)v * Bp + b) * K + k] = val;
+    if (kt == 0 && r == 0) M[(size_t)v * Bp + b] = b < B ? m : 0.f;
+  }
   }
 }
 
