@@ -59,8 +59,10 @@ def loglikelihoods(bpc, data, batch_size=None, example_ids=None):
     _check_data(bpc, data)
     ids = _ids(example_ids, data.device)
     n = data.shape[0] if ids is None else len(ids)
-    batch_size = n if batch_size is None else batch_size
     heads = getattr(bpc, "num_heads", 0)
+    if n == 0:                                  # no examples: an empty result, no launch
+        return torch.empty((0, heads) if heads else (0,), dtype=torch.float32, device=data.device)
+    batch_size = n if batch_size is None else batch_size
     out = torch.empty((max(heads, 1), n), dtype=torch.float32, device=data.device)
     for s in range(0, n, batch_size):
         b = min(batch_size, n - s)

@@ -76,6 +76,24 @@ def test_ragged_batch_and_example_ids(gpu, oracle):
     _compare_step(gpu, oracle, 10, 32, 11, 37, seed=7, idx=idx, N=200)
 
 
+def test_degenerate_inputs(gpu, oracle):
+    """No examples, one example, the smallest tree; a tree of one variable has no sum node and is refused."""
+    torch, P = gpu
+    c = P.hclt_from_clt(np.array([-1, 0], np.int32), 5, 16)
+    empty = P.loglikelihoods(c, torch.zeros((0, 2), dtype=torch.uint8, device="cuda"))
+    assert tuple(empty.shape) == (0,)
+    one = P.loglikelihoods(c, torch.tensor([[1, 2]], dtype=torch.uint8, device="cuda")).cpu().numpy()
+    np.testing.assert_allclose(one, [np.log(1 / 25)], rtol=1e-6)          # uniform parameters
+    lls = P.mini_batch_em_with_reg(c, torch.tensor([[1, 2]], dtype=torch.uint8, device="cuda"), 2, batch_size=1,
+                                   pseudocount=0.1, param_inertia=0.5, shuffle="none")
+    assert lls[1] > lls[0]
+    with pytest.raises(P.PcmError):
+        P.hclt_from_clt(np.array([-1], np.int32), 5, 16)
+    with pytest.raises(ValueError):
+        P.mini_batch_em_with_reg(c, torch.zeros((3, 2), dtype=torch.uint8, device="cuda"), 1, batch_size=4, pseudocount=0.1,
+                                 param_inertia=0.5)
+
+
 def test_config1_shape(gpu, oracle):
     """64 variables, K=16, 256 categories, batch 1024 (the reference's CPU-runnable case)."""
     _compare_step(gpu, oracle, 64, 16, 256, 1024, seed=11)
