@@ -9,6 +9,12 @@ hclt_small.npz     an HCLT (6 variables, 16 hidden states, 5 categories), 24 exa
                    gradient, Gumbel-max samples for stored noise
 dag_small.npz      a random DAG with shared sub-circuits in the description format of
                    pcm_circuit_create, with the same expected outputs
+soft_small.npz     the HCLT of hclt_small.npz under soft evidence [24, 6, 5] (some categories ruled
+                   out): log-likelihoods, edge and leaf statistics, one EM step
+multihead_small.npz  a three-head circuit over a shared body with a soft head mask: per-head
+                   log-likelihoods, node-flow sums per description node, edge statistics, and
+                   the sum-node children that survive pruning at threshold 0.05
+(written by `python tests/golden/make_golden.py extra`, which leaves the first two files alone)
 Inputs are float32 (what the library receives); expected outputs are float64, except the
 samples, which are bit-exact integers computed in float32 like the library does.
 """
@@ -102,5 +108,65 @@ def main():
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
 
 
+def extra():
+    """soft_small.npz and multihead_small.npz (own seeds; the first two fixtures are not touched)."""
+    import dag_oracle as D
+    from helpers import log_dirichlet
+    h = dict(np.load(os.path.join(HERE, "hclt_small.npz"), allow_pickle=False))
+    parent, K, C = h["parent"], int(h["K"]), int(h["C"])
+    V, B = len(parent), 24
+    rng = np.random.default_rng(20241)
+    ev = rng.normal(0, 2, (B, V, C)).astype(np.float32)
+    ev[rng.random((B, V, C)) < 0.15] = -np.inf
+    ev[:, :, 0] = np.where(np.isinf(ev).all(axis=2), 0.0, ev[:, :, 0])
+    fc = O.bits_compile(O.hclt_dag(parent, K, C, h["theta"], h["leaf"]), C, V)
+    assert np.array_equal(fc.vectorize_parameters(), h["params_before"])
+    mars = O.forward_soft(fc, ev, double=True)
+    fl, ea = O.backward(fc, mars, double=True)
+    counts = O.input_flows_soft(fc, ev, mars, fl, double=True)
+    logp, leaf = O.em_update(fc, ea, counts, 0.1, 0.9, double=True)
+    new = fc.copy()
+    new.logp, new.leaf_logp = logp.astype(np.float32), leaf.astype(np.float32)
+    np.savez_compressed(os.path.join(HERE, "soft_small.npz"), evidence=ev, ll=mars[-1], edge_aggr=ea[fc.up_order()],
+                        leaf_flow=counts, params_after=grads_in_param_order(fc, logp, leaf), pseudocount=0.1, inertia=0.9)
+    # ---- multi-head ----
+    V, C, H, B = 6, 4, 3, 32
+    root = random_dag(V, C, rng, width=3)
+    while len(root.children) < 3:
+        root = random_dag(V, C, rng, width=3)
+    heads = [O.summate(*root.children, logps=log_dirichlet(rng, len(root.children))) for _ in range(H)]
+    d = describe_dag(heads)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    mask = np.zeros((B, H), np.float32)
+    mask[np.arange(B), rng.integers(0, H, B)] = 1.0
+    mask += (rng.random((B, H)) < 0.25) * rng.random((B, H)).astype(np.float32)
+    F, E, val = D.flows(heads, data, mask.astype(np.float64))
+    order = [n for n in D.topo(heads) if all(n is not r for r in heads)] + heads   # description order
+    node_flow = np.array([F[id(n)].sum() for n in order])
+    is_sum = np.array([n.kind == O.SUM for n in order])
+    child_ptr = d["child_ptr"]
+    edge_flow = np.zeros(child_ptr[-1])
+    for i, n in enumerate(order):
+        if n.kind == O.SUM:
+            for q in range(len(n.children)):
+                edge_flow[child_ptr[i] + q] = E[(id(n), q)].sum()
+    keep = np.zeros(child_ptr[-1], np.uint8)
+    for i, n in enumerate(order):
+        if n.kind == O.SUM and len(n.children) > 1:
+            k = edge_flow[child_ptr[i]:child_ptr[i + 1]] > 0.05 * B
+            if not k.any():
+                k[int(np.argmax(n.logps))] = True
+            keep[child_ptr[i]:child_ptr[i + 1]] = k
+    pruned = D.prune(heads, {k: v.sum() for k, v in E.items()}, 0.05 * B)
+    probe = rng.integers(0, C, size=(16, V)).astype(np.uint8)
+    pv = D.values(pruned, probe)
+    np.savez_compressed(os.path.join(HERE, "multihead_small.npz"), V=V, C=C, H=H, data=data, head_mask=mask,
+                        ll_heads=np.stack([val[id(r)] for r in heads], 1), node_flow=node_flow, is_sum=is_sum,
+                        edge_flow=edge_flow, keep=keep, prune_threshold=0.05, probe=probe,
+                        ll_pruned=np.stack([pv[id(r)] for r in pruned], 1), **d)
+    for f in ("soft_small.npz", "multihead_small.npz"):
+        print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
+
+
 if __name__ == "__main__":
-    main()
+    extra() if sys.argv[1:] == ["extra"] else main()
