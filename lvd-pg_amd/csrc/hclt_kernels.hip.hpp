@@ -162,6 +162,7 @@ __device__ __forceinline__ uint32_t xpack_load(const HcltDev& d, int node, int b
   return __builtin_amdgcn_raw_buffer_load_b32(r, node >= 0 ? bcol * 4 : 0, 0, 0);
 }
 
+constexpr float kFlowRatioCap = 3.0e38f;   // largest value of 1 / S a flow is multiplied by
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -451,13 +452,14 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) r.v[kt][i] *= __builtin_amdgcn_exp2f(fmaf(ov.v[kt][i], -kLog2e, m * kLog2e));
+      for (int i = 0; i < 4; ++i)   // capped: a state (or a whole example) of probability zero has flow 0, not 0 * inf
+        r.v[kt][i] *= fminf(__builtin_amdgcn_exp2f(fmaf(ov.v[kt][i], -kLog2e, m * kLog2e)), kFlowRatioCap);
     if (flags & kItemRoot) {
       if (kHeads) {   // the heads' flows, already divided by their sums
         tile_load<K>(d.R, node, d.tile_stride, lo.tile, r);
       } else {        // flow 1 into the single root sum node of every live example
         tile_zero<K>(r);
-        r.v[0][0] = (lane < 16 && bcol < d.B) ? __builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e) : 0.f;
+        r.v[0][0] = (lane < 16 && bcol < d.B) ? fminf(__builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e), kFlowRatioCap) : 0.f;
       }
     }
     tile_store<K>(d.R, node, d.tile_stride, lo.tile, r);

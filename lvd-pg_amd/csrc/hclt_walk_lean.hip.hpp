@@ -259,7 +259,8 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) sinv.v[kt][i] = __builtin_amdgcn_exp2f(fmaf(OV.v[kt][i], -kLog2e, m * kLog2e));
+      for (int i = 0; i < 4; ++i)   // capped: a state (or a whole example) of probability zero has flow 0, not 0 * inf
+        sinv.v[kt][i] = fminf(__builtin_amdgcn_exp2f(fmaf(OV.v[kt][i], -kLog2e, m * kLog2e)), kFlowRatioCap);
     // (2) request the operands of step s+1 and the categories of step s+2
     {
       const uint32_t xc = xs;

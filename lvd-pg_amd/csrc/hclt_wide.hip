@@ -187,6 +187,7 @@ __device__ __forceinline__ float wide_e_from_z(const v4f (&z)[(K / 16) / wide_wa
   __syncthreads();
 #pragma unroll
   for (int w = 0; w < WV; ++w) m = fmaxf(m, L.mx[w][b]);
+  if (!(m > -INFINITY)) m = 0.f;   // an example of probability zero: E = 0 and a value of -inf, not NaN
 #pragma unroll
   for (int q = 0; q < Q; ++q) {
     v4f x;

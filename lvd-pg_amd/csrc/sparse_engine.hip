@@ -379,7 +379,8 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
       float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * expf(ex[u][x]);   // product edges carry exponent 0
-      if (!live[x]) ef = 0.f;
+      // no flow stays no flow where the parent's value is -inf (an example of probability zero: -inf - -inf)
+      if (!live[x] || !(fl[u][x] > 0.f) || ex[u][x] != ex[u][x]) ef = 0.f;
       acc[x] += ef;
       part += ef;
     }

@@ -94,6 +94,34 @@ def test_degenerate_inputs(gpu, oracle):
                                  param_inertia=0.5)
 
 
+@pytest.mark.parametrize("K", [16, 32, 64, 128, 8])
+def test_examples_of_probability_zero_carry_no_flow(gpu, oracle, K):
+    """A leaf that forbids a category makes the examples showing it impossible: their value is
+    -inf and they leave no trace in the statistics (the reference's flows turn NaN there:
+    exp(-inf - -inf) in src/queries/flow.jl:49-60); every walk engine behaves the same."""
+    torch, P = gpu
+    from helpers import make_hclt, block_theta
+    V, C, B = 5, 4, 40
+    parent, theta, leaf, fc = make_hclt(V, K, C, 3)
+    leaf = leaf.copy()
+    leaf[2, :, 1] = -np.inf
+    leaf[2] -= np.log(np.exp(leaf[2].astype(np.float64)).sum(-1, keepdims=True)).astype(np.float32)
+    data = np.random.default_rng(K).integers(0, C, (B, V)).astype(np.uint8)
+    bad = data[:, 2] == 1
+    assert bad.any() and not bad.all()
+    a, b = P.hclt_from_clt(parent, C, K), P.hclt_from_clt(parent, C, K)
+    for c in (a, b):
+        c.set_params(block_theta(parent, K, theta), leaf)
+    ll = P.probs_flows_circuit(a, torch.from_numpy(data).cuda()).cpu().numpy()
+    ll_good = P.probs_flows_circuit(b, torch.from_numpy(np.ascontiguousarray(data[~bad])).cuda()).cpu().numpy()
+    assert np.isneginf(ll[bad]).all()
+    np.testing.assert_allclose(ll[~bad], ll_good, rtol=1e-6)
+    (ea, lf), (ea2, lf2) = a.get_flows(), b.get_flows()
+    assert np.isfinite(ea).all() and np.isfinite(lf).all()
+    np.testing.assert_allclose(ea, ea2, atol=2e-4 * ea2.max())
+    np.testing.assert_allclose(lf, lf2, atol=2e-4 * lf2.max())
+
+
 def test_config1_shape(gpu, oracle):
     """64 variables, K=16, 256 categories, batch 1024 (the reference's CPU-runnable case)."""
     _compare_step(gpu, oracle, 64, 16, 256, 1024, seed=11)
