@@ -354,3 +354,56 @@ def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
                 g[e0:e0 + nk * K] = np.tile(hn[b, r * K:(r + 1) * K], nk)
             _, want = O.gumbel_soft(flat, g, 0.15, double=True)
             np.testing.assert_allclose(cold[b], want, rtol=1e-3, atol=1e-6)
+
+
+def test_prealloc_wrappers_run_the_queries_row_by_row(gpu, oracle):
+    """`kld_with_prealloc`, `kld_backward_with_prealloc`, `gumbel_sample_with_prealloc`
+    (src/utils/cuda_preallocation.jl:47-78,189-203) with one parameter vector per example,
+    against the single-vector queries and the oracle."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta
+    W = P.prealloc
+    V, K, C, R = 6, 16, 5, 3
+    parent, theta, leaf, fc = make_hclt(V, K, C, 31)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    base = P.vectorize_parameters(bpc)
+    rows1, rows2, fcs = [], [], []
+    for r in range(R + 1):
+        _, th, lf, f = make_hclt(V, K, C, 40 + r, parent=parent)
+        c = P.hclt_from_clt(parent, C, K)
+        c.set_params(block_theta(parent, K, th), lf)
+        (rows2 if r == R else rows1).append(P.vectorize_parameters(c))
+        fcs.append(f)
+    p1, prior = np.stack(rows1), np.stack(rows2)
+    with pytest.raises(RuntimeError):
+        W.kld_with_prealloc(bpc, p1, prior)
+    W.kld_preallocation(bpc, num_examples=R)
+    klds = W.kld_with_prealloc(bpc, p1, prior)
+    want = [O.kld(fcs[r], fcs[R], double=True)[0][-1] for r in range(R)]
+    np.testing.assert_allclose(klds, want, rtol=KLD_RTOL)
+    np.testing.assert_array_equal(P.vectorize_parameters(bpc), base)          # the circuit's own parameters come back
+    g1, g2 = W.kld_backward_with_prealloc(bpc)
+    assert g1.shape == g2.shape == p1.shape
+    q = P.hclt_from_clt(parent, C, K)
+    P.update_parameters(q, prior[0])
+    P.update_parameters(bpc, p1[1])
+    e1, e2 = P.kld_backward(bpc, q)
+    P.update_parameters(bpc, base)
+    np.testing.assert_allclose(g1[1], e1, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(g2[1], e2, rtol=1e-6, atol=1e-7)
+    with pytest.raises(ValueError):
+        W.kld_with_prealloc(bpc, p1[:2], prior)                                # not the preallocated number of rows
+    W.kld_free_mem()
+    W.gumbel_sample_preallocation(bpc, num_examples=R, num_vars=V, par_buffer_size=C + 2)
+    soft = W.gumbel_sample_with_prealloc(bpc, p1, temperature=1.0, no_gumbel=True)
+    assert soft.shape == (R, V, C + 2) and np.all(soft[:, :, C:] == 0)
+    np.testing.assert_allclose(soft.sum(-1), 1.0, rtol=1e-4)                   # a distribution per variable
+    P.update_parameters(bpc, p1[2])
+    direct = P.gumbel_sample(bpc, 1, temperature=1.0)[0].cpu().numpy()
+    P.update_parameters(bpc, base)
+    np.testing.assert_allclose(soft[2, :, :C], direct, rtol=1e-6, atol=1e-7)
+    noisy = W.gumbel_sample_with_prealloc(bpc, p1, temperature=0.5, generator=torch.Generator(device="cuda").manual_seed(3))
+    np.testing.assert_allclose(noisy.sum(-1), 1.0, rtol=1e-4)
+    W.gumbel_sample_free_mem()
