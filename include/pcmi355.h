@@ -95,7 +95,8 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
  * 3 edges, 4 input parameters, 5 variables, 6 categories, 7 hidden categories (0 if not an
  * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes,
  * 12 heads (0 for a single-root circuit), 13 nodes of the description the circuit was
- * built from (0 for an HCLT built from its tree). */
+ * built from (0 for an HCLT built from its tree), 14 which kernels run likelihoods and flows:
+ * 0 per-layer kernels, 1 lean tree walks, 2 general tree walks, 3 wide block kernels. */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.

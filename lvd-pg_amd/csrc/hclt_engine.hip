@@ -644,6 +644,8 @@ int64_t HcltCircuit::size(int what) const {
     case 10: return (int64_t)sum_group_size_.size();
     case 11: return (int64_t)V_ * K_;
     case 12: return H_;
+    case 13: return 0;
+    case 14: return wide_walk_ ? 3 : !block_ ? 0 : (fwd_lean_ && bwd_lean_ && stat_lean_) ? 1 : 2;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }

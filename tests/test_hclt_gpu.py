@@ -70,6 +70,22 @@ def test_em_step_on_wide_trees(gpu, oracle, tree):
     _compare_step(gpu, oracle, len(tree), 128, 9, 21, seed=len(tree) + 2, tree=tree)   # the wide block kernels
 
 
+def test_every_walk_kernel_family_is_exercised(gpu, oracle):
+    """Which kernels a circuit gets: lean walks (K <= 32, at most three children per node), general
+    walks (more children; K = 64 on bushy trees), wide block kernels (K = 128; K = 64 on small
+    trees), per-layer kernels (other hidden sizes) -- and the bushy K = 64 case against the oracle."""
+    torch, P = gpu
+    rng = np.random.default_rng(1)
+    kind = lambda parent, K: P.hclt_from_clt(np.asarray(parent, np.int32), 4, K).size("walk_kernels")
+    chain = [-1] + list(range(9))
+    assert kind(chain, 32) == 1 and kind([-1, 0, 0, 0, 0, 0], 16) == 2 and kind(chain, 128) == 3 and kind(chain, 8) == 0
+    assert kind(chain, 64) == 3
+    bushy = oracle.random_tree(600, rng, 3)
+    assert kind(bushy, 64) == 2
+    bpc = _compare_step(gpu, oracle, 600, 64, 4, 16, seed=5, tree=list(bushy))
+    assert bpc.size("walk_kernels") == 2
+
+
 def test_ragged_batch_and_example_ids(gpu, oracle):
     rng = np.random.default_rng(5)
     idx = rng.permutation(200)[:37].astype(np.int32)
