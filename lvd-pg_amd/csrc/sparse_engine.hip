@@ -380,7 +380,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
     for (int x = 0; x < EX; ++x) {
       float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * expf(ex[u][x]);   // product edges carry exponent 0
       // no flow stays no flow where the parent's value is -inf (an example of probability zero: -inf - -inf)
-      if (!live[x] || !(fl[u][x] > 0.f) || ex[u][x] != ex[u][x]) ef = 0.f;
+      if (!live[x] || ex[u][x] != ex[u][x]) ef = 0.f;
       acc[x] += ef;
       part += ef;
     }
@@ -601,30 +601,34 @@ __global__ void sparse_scale_kernel(float* p, int64_t n, float rate) {
   if (i < n) p[i] = rate != 0.f ? p[i] * rate : 0.f;
 }
 
-// EM update, one thread per node: add_pseudocount, aggr_node_flows, update_params
-// (src/pretrain/mini_batch_warmup.jl:4-17, :54-70 without the 1e-8 guards) and the leaf
-// update (src/nodes/fixable_categorical_dist.jl:223-248, missing_flow = 0).
-__global__ void sparse_update_kernel(SparseDev d, int n_nodes, float* __restrict__ logp, float* __restrict__ leaf,
-                                     float* __restrict__ edge_aggr, const float* __restrict__ leaf_flow,
-                                     float pseudocount, float inertia) {
-  const int n = blockIdx.x * blockDim.x + threadIdx.x;
+// EM update, one wave per node (lanes over the node's edges / categories): add_pseudocount,
+// aggr_node_flows, update_params (src/pretrain/mini_batch_warmup.jl:4-17, :54-70 without the 1e-8
+// guards) and the leaf update (src/nodes/fixable_categorical_dist.jl:223-248, missing_flow = 0).
+__global__ __launch_bounds__(256) void sparse_update_kernel(SparseDev d, int n_nodes, float* __restrict__ logp,
+                                                            float* __restrict__ leaf, float* __restrict__ edge_aggr,
+                                                            const float* __restrict__ leaf_flow, float pseudocount,
+                                                            float inertia) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (n >= n_nodes) return;
-  if (d.type[n] == kSum) {
+  const int type = d.type[n];
+  if (type == kSum) {
     const int e0 = d.node_e0[n], e1 = d.node_e1[n];
     const float share = pseudocount / (float)(e1 - e0);
     float tot = 0.f;
-    for (int e = e0; e < e1; ++e) { edge_aggr[e] += share; tot += edge_aggr[e]; }
+    for (int e = e0 + lane; e < e1; e += 64) { edge_aggr[e] += share; tot += edge_aggr[e]; }
+    tot = wave_sum(tot);
     if (e1 - e0 == 1) return;
-    for (int e = e0; e < e1; ++e)
+    for (int e = e0 + lane; e < e1; e += 64)
       logp[e] = logf(inertia * expf(logp[e]) + (1.f - inertia) * edge_aggr[e] / tot);
-  } else if (d.type[n] == kInput) {
+  } else if (type == kInput) {
     float* lp = leaf + d.in_off[n];
     const float* fl = leaf_flow + d.in_off[n];
     float node_flow = 0.f;
-    for (int c = 0; c < d.C; ++c) node_flow += fl[c];
-    node_flow += pseudocount;
+    for (int c = lane; c < d.C; c += 64) node_flow += fl[c];
+    node_flow = wave_sum(node_flow) + pseudocount;
     const float cat_pc = pseudocount / (float)d.C;
-    for (int c = 0; c < d.C; ++c)
+    for (int c = lane; c < d.C; c += 64)
       lp[c] = logf(inertia * expf(lp[c]) + (1.f - inertia) * (fl[c] + cat_pc) / node_flow);
   }
 }
@@ -853,17 +857,33 @@ __global__ void sparse_copy_rows_kernel(const float* __restrict__ mars, int Bp, 
 // Mask-weighted mixture over the heads, src-jl/multi_head_pc/likelihood.jl:3-12:
 // ll = logsumexp_h(mars[head_h] + log mask[h]) - log sum_h mask[h], folded head by head
 // from -inf with the pairwise logsumexp.
-__global__ void sparse_head_mixture_kernel(const float* __restrict__ mars, int Bp, int B, const int32_t* __restrict__ heads,
-                                           int n_heads, const float* __restrict__ mask, float* __restrict__ out) {
-  const int b = blockIdx.x * blockDim.x + threadIdx.x;
-  if (b >= B) return;
-  float acc = -INFINITY, tot = 0.f;
-  for (int h = 0; h < n_heads; ++h) {
-    const float m = mask[(size_t)h * B + b];
-    acc = lse2(acc, mars[(size_t)heads[h] * Bp + b] + logf(m));
-    tot += m;
-  }
-  out[b] = acc - logf(tot);
+constexpr int kMixGroups = 16;   // head groups per example in the mixture kernel
+
+// workgroup = 64 examples x kMixGroups head groups: running maximum and sum per thread, combined through LDS
+__global__ __launch_bounds__(64 * kMixGroups) void sparse_head_mixture_kernel(const float* __restrict__ mars, int Bp, int B,
+                                                                              const int32_t* __restrict__ heads, int n_heads,
+                                                                              const float* __restrict__ mask,
+                                                                              float* __restrict__ out) {
+  __shared__ float pm[kMixGroups][64], ps[kMixGroups][64], pt[kMixGroups][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int b = blockIdx.x * 64 + lane;
+  float mx = -INFINITY, sm = 0.f, tot = 0.f;
+  if (b < B)
+    for (int h = g; h < n_heads; h += kMixGroups) {
+      const float m = mask[(size_t)h * B + b];
+      const float t = mars[(size_t)heads[h] * Bp + b] + logf(m);
+      tot += m;
+      if (t > mx) { sm = sm * expf(mx - t) + 1.f; mx = t; }
+      else if (t > -INFINITY) sm += expf(t - mx);
+    }
+  pm[g][lane] = mx; ps[g][lane] = sm; pt[g][lane] = tot;
+  __syncthreads();
+  if (g || b >= B) return;
+  float M = -INFINITY, T = 0.f, S = 0.f;
+  for (int q = 0; q < kMixGroups; ++q) { M = fmaxf(M, pm[q][lane]); T += pt[q][lane]; }
+  for (int q = 0; q < kMixGroups; ++q)
+    if (pm[q][lane] > -INFINITY) S += ps[q][lane] * expf(pm[q][lane] - M);
+  out[b] = M + logf(S) - logf(T);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1188,7 +1208,7 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     PCM_HIP(hipMemcpyAsync(d_ll, d_mars_.p + (size_t)(fc_.n_nodes() - 1) * Bp, (size_t)batch * sizeof(float),
                            hipMemcpyDeviceToDevice, stream));
   } else {
-    hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(batch, 256)), dim3(256), 0, stream, d_mars_.p, Bp, batch,
+    hipLaunchKernelGGL(sparse_head_mixture_kernel, dim3(ceil_div(batch, 64)), dim3(64 * kMixGroups), 0, stream, d_mars_.p, Bp, batch,
                        d_head_nodes_.p, (int)fc_.heads.size(), d_head_mask, d_ll);
     check_launch("head_mixture");
   }
@@ -1199,7 +1219,7 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
 void SparseCircuit::em_update(float pseudocount, float inertia) {
   if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
   SparseDev d = SPARSE_DEV(0, 64, nullptr);
-  hipLaunchKernelGGL(sparse_update_kernel, dim3(ceil_div(fc_.n_nodes(), 128)), dim3(128), 0, stream, d, (int)fc_.n_nodes(),
+  hipLaunchKernelGGL(sparse_update_kernel, dim3(ceil_div(fc_.n_nodes(), 4)), dim3(256), 0, stream, d, (int)fc_.n_nodes(),
                      d_logp_.p, d_leaf_.p, d_edge_aggr_.p, d_leaf_flow_.p, pseudocount, inertia);
   check_launch("sparse_update");
 }
