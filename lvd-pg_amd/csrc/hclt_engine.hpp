@@ -206,6 +206,8 @@ class HcltCircuit : public pcm_circuit {
   int soft_levels_ = 0;
   DevBuf<int32_t> d_sample_tabs_;   // sampler tables: parent of every inner node | state-giving node of every variable | level order
   int sample_groups_ = 0;
+  DevBuf<int32_t> d_sample_passes_;   // the sampler's levels from the root in records of 64 {node, parent} pairs
+  int sample_passes_ = 0;
   DevBuf<int64_t> d_sum_param_src_;
   int cap_slices_ = 0;
   bool have_flows_ = false;
@@ -231,7 +233,9 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int32_t> d_kl_tabs_;             // parent of every inner node | h-giving node of every variable | input-node positions
   DevBuf<int32_t> d_kl_pos_;              // chain slot of every inner node: upward | downward
   DevBuf<float> d_kl_leaf_, d_kl_vec_, d_kl_par_;
+  DevBuf<int32_t> d_kl_ext_;              // chain slots of the children past the second, of nodes with more than three
   int kl_up_steps_ = 0, kl_down_steps_ = 0;
+  int kl_ring_slots_ = 0;                 // slots of the chains' LDS ring; 0: levels too wide, the ring is the whole chain in device memory
   HcltCircuit* same_tree(pcm_circuit* q);
   void build_kld_tables();
   void kld_device(HcltCircuit* q, bool with_down);

@@ -14,13 +14,19 @@
 // src/nodes/fixable_categorical_dist.jl:219): g * (a - b + 1) and g * exp(a - b).
 //
 // Only the two K-vector chains (KL_v up the tree, h_v down the tree) are sequential; one
-// workgroup walks each of them level by level, sixteen tree nodes (one per wave) between
-// barriers.  Everything else is a data-parallel kernel.
+// workgroup walks each of them level by level (deepest level first / root first), sixteen tree
+// nodes (one per wave) between barriers.  A step's vectors stay in an LDS ring indexed by chain
+// slot (a node's tree neighbours sit at most two levels' widths away), and the parameters of
+// the steps to come are requested several steps ahead, so a step costs an LDS round trip and
+// the chain runs at the rate one compute unit pulls the parameters from L2.  Everything else is
+// a data-parallel kernel.
 #include "hclt_engine.hpp"
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
+#include <cstring>
 
 namespace pcm {
 
@@ -55,13 +61,32 @@ __global__ __launch_bounds__(256) void hclt_kld_leaf_kernel(const float* __restr
   }
 }
 
+// One tree node of a chain step (16 bytes, one vector load).
+struct KlItem {
+  int32_t n;      // inner id, -1: this wave idles
+  int32_t c[3];   // up: chain slots of the non-leaf tree children (-1 none); c[2] <= -2: the third and
+                  // further children are listed at ext[-(c[2] + 2)]: their number, then their slots
+                  // down: c[0] = the parent's slot (-1: the root)
+};
+static_assert(sizeof(KlItem) == 16, "KlItem is read as one 16-byte word");
+
+// Waves (= nodes per step) of a chain workgroup and the steps of parameters a lane keeps
+// requested ahead: as many as its registers hold.
+constexpr int kl_waves(int K) { return K > 32 ? 8 : 16; }
+constexpr int kl_ahead(int K) { return K > 32 ? 2 : 4; }
+
+// Operand layout of the chains: lane (part, r) of a wave, part = lane / K, r = lane % K, owns
+// rows part * JP .. + JP (JP = K * K / 64) of its node's K x K operand at column r; the JP values
+// are consecutive, so a step's operand is JP / 4 loads of 16 bytes per lane, 1 KB per wave each:
+// word ((i / 4) * 64 + lane) * 4 + i % 4 of the slot holds row part * JP + i.
+
 // Per tree node, everything of the recursion that does not wait for other nodes, stored where
 // the chains will look for it: slot su = pos[n] of the upward chain's steps, slot sd =
 // pos[n_inner + n] of the downward chain's.
 //   ell[su][j]  = l_v[j]
 //   base[su][k] = sum_j P[k,j] * (D[k,j] + ell[j])
-//   pu[su][j][k] = P[k,j]   (operand layout of the upward chain: lane = k)
-//   pd[sd][k][j] = P[k,j]   (of the downward chain: lane = j)
+//   pu[su]: operand (row j, column k) = P[k,j]   (upward chain: a lane's column is k)
+//   pd[sd]: operand (row k, column j) = P[k,j]   (downward chain: a lane's column is j)
 template <int K>
 __global__ __launch_bounds__(256) void hclt_kld_base_kernel(const HcltNode* __restrict__ nodes,
                                                             const int32_t* __restrict__ child_leaf,
@@ -88,91 +113,117 @@ __global__ __launch_bounds__(256) void hclt_kld_base_kernel(const HcltNode* __re
     const float x = theta1[((size_t)n * K + k) * K + j], y = theta2[((size_t)n * K + k) * K + j];
     const float p = expf(x);
     tile[k][j] = p;
-    pd[(sd * K + k) * K + j] = p;
     float term = p > 0.f ? p * (x - y + l[j]) : 0.f;   // absent edges (the root's rows past the first) carry -inf
 #pragma unroll
     for (int o = K / 2; o > 0; o >>= 1) term += __shfl_xor(term, o, K);
     if (j == 0) base[su * K + k] = term;
   }
   __syncthreads();
-  for (int i = t; i < K * K; i += 256) pu[su * K * K + i] = tile[i % K][i / K];
+  // consecutive threads write consecutive words of the operand: word w = ((i4 * 64) + lane) * 4 + e
+  constexpr int JP = K * K / 64;
+  for (int w = t; w < K * K; w += 256) {
+    const int e = w & 3, lane = (w >> 2) & 63, i4 = w >> 8;
+    const int row = (lane / K) * JP + i4 * 4 + e, col = lane % K;
+    pu[su * K * K + w] = tile[col][row];
+    pd[sd * K * K + w] = tile[row][col];
+  }
 }
-
-// One tree node of a chain step.
-struct KlItem {
-  int32_t n;            // inner id, -1: this wave idles
-  int32_t c[3];         // up: first non-leaf tree children (-1 none); down: c[0] = parent (-1 root)
-  int32_t ext_off, ext_cnt;   // up: further children at child_inner[ext_off .. +ext_cnt)
-  int32_t pad[2];
-};
-static_assert(sizeof(KlItem) == 32, "KlItem is read as two 16-byte words");
-
-// Waves (= nodes per step) of a chain workgroup: as many as leave each lane the registers for two
-// steps' worth of its node's parameters.
-constexpr int kl_waves(int K) { return K > 32 ? 8 : 16; }
 
 // The two chains.  Workgroup 0 walks up (KL_v, Z_v), workgroup 1 walks down (h_v); launched
 // with one workgroup when only the divergence is wanted.  A step is kl_waves(K) independent
-// nodes (same level); the vectors a step reads were stored by earlier steps of the same
-// workgroup, so a barrier orders them.  A step first requests the vectors it waits for, then
-// the next step's item and parameters (found by step and wave alone), so that those are under
-// way while the step computes.
-template <int K>
+// nodes (same level).  The vectors a step reads were left in the ring by earlier steps of the
+// same workgroup (slot & ring_mask; the host sizes the ring beyond the largest distance between
+// a node and its tree neighbours), so a barrier orders them.  kLds: the ring is in LDS;
+// otherwise (levels too wide for that) it is the whole chain in device memory.  The item,
+// operand and constants of a step are requested D = kl_ahead(K) steps before it; the chains are
+// padded to a multiple of D steps and the tables by D idle steps more, so the requests need no
+// bounds and every lane's requests complete in the order the steps use them.
+template <int K, bool kLds>
 __global__ __launch_bounds__(kl_waves(K) * 64) void hclt_kld_chain_kernel(
     const KlItem* __restrict__ up_items, int up_steps, const KlItem* __restrict__ down_items, int down_steps,
-    const int32_t* __restrict__ child_inner, const float* __restrict__ pu, const float* __restrict__ base,
-    const float* __restrict__ ell, const float* __restrict__ pd, float* klv, float* z, float* h) {
-  constexpr int PARTS = 64 / K, JP = K / PARTS, W = kl_waves(K);
+    const int32_t* __restrict__ ext, const float* __restrict__ pu, const float* __restrict__ base,
+    const float* __restrict__ ell, const float* __restrict__ pd, int ring_mask, float* ring_up, float* ring_down,
+    float* __restrict__ klv, float* __restrict__ z, float* __restrict__ h) {
+  constexpr int PARTS = 64 / K, JP = K / PARTS, Q = JP / 4, W = kl_waves(K), D = kl_ahead(K);
+  extern __shared__ float lds_ring[];   // kLds: [ring_mask + 1][K]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane % K, part = lane / K;
   const bool up = blockIdx.x == 0;
   const int steps = up ? up_steps : down_steps;
-  const KlItem* __restrict__ items = up ? up_items : down_items;
-  const float* __restrict__ par = up ? pu : pd;   // [slot][K][K], this lane reads rows part*JP.. at column r
-  KlItem it = items[wave];
-  float p[JP];
+  const int4* __restrict__ items = reinterpret_cast<const int4*>(up ? up_items : down_items);
+  const float4* __restrict__ par = reinterpret_cast<const float4*>(up ? pu : pd);
+  float* ring_dev = up ? ring_up : ring_down;
+  auto ring_at = [&](int slot) -> float* {
+    if constexpr (kLds) return lds_ring + (size_t)(slot & ring_mask) * K;
+    else return ring_dev + (size_t)slot * K;
+  };
+  // The first round (q0 = -D) computes nothing and only places the requests of steps 0 .. D-1:
+  // with every request issued from the same place in the loop, the waits the compiler counts
+  // from the order of issue let D - 1 steps of requests stay in flight.
+  int4 it[D];
+  float4 p[D][Q];
+  float bs[D], el[D];
 #pragma unroll
-  for (int i = 0; i < JP; ++i) p[i] = par[((size_t)wave * K + part * JP + i) * K + r];
-  for (int q = 0; q < steps; ++q) {
-    const size_t slot = (size_t)q * W + wave;
-    float s = 0.f, bs = 0.f, el = 0.f;
-    if (it.n >= 0) {
-      if (up) {
+  for (int d = 0; d < D; ++d) {
+    it[d] = make_int4(-1, -1, -1, -1);
 #pragma unroll
-        for (int i = 0; i < 3; ++i)
-          if (it.c[i] >= 0) s += klv[(size_t)it.c[i] * K + r];
-        for (int i = 0; i < it.ext_cnt; ++i) s += klv[(size_t)child_inner[it.ext_off + i] * K + r];
-        bs = base[slot * K + r];
-        el = ell[slot * K + r];
-      } else {
-        s = it.c[0] >= 0 ? h[(size_t)it.c[0] * K + r] : (r == 0 ? 1.f : 0.f);
-      }
-    }
-    const bool more = q + 1 < steps;
-    KlItem nx = it;
-    float pn[JP];
-    if (more) nx = items[slot + W];
+    for (int e = 0; e < Q; ++e) p[d][e] = make_float4(0.f, 0.f, 0.f, 0.f);
+    bs[d] = el[d] = 0.f;
+  }
+  for (int q0 = -D; q0 < steps; q0 += D) {
 #pragma unroll
-    for (int i = 0; i < JP; ++i) pn[i] = more ? par[((slot + W) * K + part * JP + i) * K + r] : 0.f;
-    if (it.n >= 0) {
-      float acc = 0.f;
+    for (int d = 0; d < D; ++d) {
+      const int q = q0 + d;   // steps is a multiple of D (idle steps at the end): no way round a step
+      const int64_t slot = (int64_t)q * W + wave;
+      const int n = __builtin_amdgcn_readfirstlane(it[d].x);
+      const int c0 = __builtin_amdgcn_readfirstlane(it[d].y), c1 = __builtin_amdgcn_readfirstlane(it[d].z),
+                c2 = __builtin_amdgcn_readfirstlane(it[d].w);
+      if (n >= 0) {
+        float acc = 0.f, s = 0.f;
+        auto take = [&](int cslot) {   // acc += sum_i operand[part * JP + i] * vector[part * JP + i]
+          const float* cv = ring_at(cslot);
+          if (up) s += cv[r];
 #pragma unroll
-      for (int i = 0; i < JP; ++i) acc += p[i] * __shfl(s, part * JP + i);
-#pragma unroll
-      for (int o = K; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
-      if (part == 0) {
+          for (int e = 0; e < Q; ++e) {
+            const float4 x = *reinterpret_cast<const float4*>(cv + part * JP + 4 * e);
+            acc += p[d][e].x * x.x + p[d][e].y * x.y + p[d][e].z * x.z + p[d][e].w * x.w;
+          }
+        };
         if (up) {
-          klv[(size_t)it.n * K + r] = bs + acc;
-          z[(size_t)it.n * K + r] = el + s;
+          if (c0 >= 0) take(c0);
+          if (c1 >= 0) take(c1);
+          if (c2 >= 0) take(c2);
+          if (c2 < -1) {
+            const int32_t* more = ext + (-(c2 + 2));
+            const int cnt = more[0];
+            for (int i = 0; i < cnt; ++i) take(more[1 + i]);
+          }
+        } else if (c0 >= 0) {
+          take(c0);
         } else {
-          h[(size_t)it.n * K + r] = acc;
+          acc = part == 0 ? p[d][0].x : 0.f;   // the root's incoming vector is e_0: row 0 of its operand
+        }
+#pragma unroll
+        for (int o = K; o < 64; o <<= 1) acc += __shfl_xor(acc, o);
+        if (part == 0) {
+          const float out = up ? bs[d] + acc : acc;
+          ring_at((int)slot)[r] = out;
+          if (up) {
+            klv[(size_t)n * K + r] = out;
+            z[(size_t)n * K + r] = el[d] + s;
+          } else {
+            h[(size_t)n * K + r] = out;
+          }
         }
       }
-    }
-    it = nx;
+      const size_t nx = (size_t)(slot + D * W);
+      it[d] = items[nx];
 #pragma unroll
-    for (int i = 0; i < JP; ++i) p[i] = pn[i];
-    __syncthreads();
+      for (int e = 0; e < Q; ++e) p[d][e] = par[(nx * Q + e) * 64 + lane];
+      bs[d] = base[nx * K + r];
+      el[d] = ell[nx * K + r];
+      __syncthreads();
+    }
   }
 }
 
@@ -271,65 +322,66 @@ HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
 
 void HcltCircuit::build_kld_tables() {
   if (d_kl_up_.n) return;
-  const int W = kl_waves(K_);
-  // offsets of the nodes' non-leaf children in the device's child_inner list
-  std::vector<int32_t> ic_off(n_inner_ + 1, 0);
-  for (int n = 0; n < n_inner_; ++n) {
-    int cnt = 0;
-    for (int c : children_[var_of_inner_[n]]) cnt += !children_[c].empty();
-    ic_off[n + 1] = ic_off[n] + cnt;
-  }
+  const int W = kl_waves(K_), D = kl_ahead(K_);
   std::vector<int32_t> pos((size_t)2 * n_inner_, 0);
+  std::vector<int32_t> ext;
+  int reach = 0;   // largest distance in chain slots between a node and a tree neighbour it reads
   auto chain = [&](bool up) {
-    // nodes level by level (up: by height from the bottom, down: by depth from the root), each
-    // level padded to whole steps
+    // nodes level by level (up: deepest level first, down: from the root), each level padded to
+    // whole steps; D idle steps at the end for the requests that run ahead
     std::vector<std::vector<int32_t>> lv;
     for (int n = 0; n < n_inner_; ++n) {
-      const int v = var_of_inner_[n];
-      const size_t at = (size_t)(up ? height_[v] : depth_[v]);
+      const size_t at = (size_t)depth_[var_of_inner_[n]];
       if (lv.size() <= at) lv.resize(at + 1);
       lv[at].push_back(n);
     }
+    if (up) std::reverse(lv.begin(), lv.end());
+    const KlItem idle{-1, {-1, -1, -1}};
     std::vector<KlItem> items;
     for (const auto& level : lv) {
       for (int32_t n : level) {
-        KlItem it;
-        std::memset(&it, 0, sizeof it);
+        KlItem it = idle;
         it.n = n;
-        it.c[0] = it.c[1] = it.c[2] = -1;
         const int v = var_of_inner_[n];
+        const int32_t me = (int32_t)items.size();
         if (up) {
-          int seen = 0;
-          for (int c : children_[v]) {
-            if (children_[c].empty()) continue;
-            if (seen < 3) it.c[seen] = inner_of_var_[c];
-            ++seen;
+          std::vector<int32_t> cs;
+          for (int c : children_[v])
+            if (!children_[c].empty()) cs.push_back(pos[inner_of_var_[c]]);
+          for (int32_t c : cs) reach = std::max(reach, me - c);
+          for (size_t i = 0; i < cs.size() && i < 3; ++i) it.c[i] = cs[i];
+          if (cs.size() > 3) {
+            it.c[2] = -((int32_t)ext.size() + 2);
+            ext.push_back((int32_t)cs.size() - 2);
+            ext.insert(ext.end(), cs.begin() + 2, cs.end());
           }
-          if (seen > 3) { it.ext_off = ic_off[n] + 3; it.ext_cnt = seen - 3; }
-        } else {
-          it.c[0] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
+        } else if (parent_[v] >= 0) {
+          it.c[0] = pos[n_inner_ + inner_of_var_[parent_[v]]];
+          reach = std::max(reach, me - it.c[0]);
         }
-        pos[(up ? 0 : n_inner_) + n] = (int32_t)items.size();
+        pos[(up ? 0 : n_inner_) + n] = me;
         items.push_back(it);
       }
-      while (items.size() % W) {
-        KlItem idle;
-        std::memset(&idle, 0, sizeof idle);
-        idle.n = -1;
-        idle.c[0] = idle.c[1] = idle.c[2] = -1;
-        items.push_back(idle);
-      }
+      while (items.size() % W) items.push_back(idle);
     }
+    while (items.size() % ((size_t)D * W)) items.push_back(idle);   // whole rounds of D steps
+    items.resize(items.size() + (size_t)D * W, idle);
     return items;
   };
   std::vector<KlItem> up = chain(true), down = chain(false);
-  kl_up_steps_ = (int)(up.size() / W);
-  kl_down_steps_ = (int)(down.size() / W);
-  std::vector<int32_t> raw(up.size() * 8), rawd(down.size() * 8);
+  kl_up_steps_ = (int)(up.size() / W) - D;
+  kl_down_steps_ = (int)(down.size() / W) - D;
+  // the ring: a power of two of slots beyond the reach, in LDS when 64 KB hold it
+  int ring = 1;
+  while (ring < reach + W) ring <<= 1;
+  kl_ring_slots_ = (size_t)ring * K_ * sizeof(float) <= (size_t)64 * 1024 ? ring : 0;
+  std::vector<int32_t> raw(up.size() * 4), rawd(down.size() * 4);
   std::memcpy(raw.data(), up.data(), up.size() * sizeof(KlItem));
   std::memcpy(rawd.data(), down.data(), down.size() * sizeof(KlItem));
   d_kl_down_.upload(rawd, stream);
   d_kl_pos_.upload(pos, stream);
+  if (ext.empty()) ext.push_back(0);
+  d_kl_ext_.upload(ext, stream);
   // per inner node: its parent | per variable: the inner node whose h reaches its leaf |
   // per input node (v, j): its position among the input nodes of the parameter vector
   std::vector<int32_t> t((size_t)n_inner_ + V_ + (size_t)V_ * K_, 0);
@@ -347,12 +399,14 @@ void HcltCircuit::build_kld_tables() {
 // Runs the recursion of this circuit (p) against q; with_down also leaves h.
 void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
   build_kld_tables();
-  const int W = kl_waves(K_);
+  const int W = kl_waves(K_), D = kl_ahead(K_);
   const size_t nk = (size_t)n_inner_ * K_;
-  const size_t su = (size_t)kl_up_steps_ * W, sd = (size_t)kl_down_steps_ * W;   // chain slots, idle ones included
+  // chain slots, idle ones and the idle steps at the end included
+  const size_t su = (size_t)(kl_up_steps_ + D) * W, sd = (size_t)(kl_down_steps_ + D) * W;
+  const size_t sm = std::max(su, sd);   // ell and base have a row per slot of the longer chain: both chains request them
   d_kl_leaf_.ensure((size_t)V_ * K_);
   if (!d_kl_vec_.n) {
-    d_kl_vec_.alloc(3 * nk + 2 * su * K_);   // klv | z | h | ell | base
+    d_kl_vec_.alloc(3 * nk + 2 * sm * K_ + (kl_ring_slots_ ? 0 : (su + sd) * K_));   // klv | z | h | ell | base | rings
     d_kl_par_.alloc((su + sd) * K_ * K_);    // pu | pd; idle slots are read (and ignored) by idle waves
     d_kl_vec_.zero(stream);
     d_kl_par_.zero(stream);
@@ -361,17 +415,23 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
   float* z = klv + nk;
   float* h = z + nk;
   float* ell = h + nk;
-  float* base = ell + su * K_;
+  float* base = ell + sm * K_;
+  float* ring_up = kl_ring_slots_ ? nullptr : base + sm * K_;
+  float* ring_down = kl_ring_slots_ ? nullptr : ring_up + su * K_;
   float* pu = d_kl_par_.p;
   float* pd = pu + su * K_ * K_;
   hipLaunchKernelGGL(hclt_kld_leaf_kernel, dim3(V_), dim3(256), 0, stream, d_leaf_.p, q->d_leaf_.p, K_, C_, d_kl_leaf_.p);
   PCM_DISPATCH_K(K_, {
     hipLaunchKernelGGL(hclt_kld_base_kernel<KK>, dim3(n_inner_), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
                        d_kl_pos_.p, n_inner_, d_logtheta_.p, q->d_logtheta_.p, d_kl_leaf_.p, ell, base, pu, pd);
-    hipLaunchKernelGGL(hclt_kld_chain_kernel<KK>, dim3(with_down ? 2 : 1), dim3(kl_waves(KK) * 64), 0, stream,
-                       reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
-                       reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_child_inner_.p, pu, base, ell, pd,
-                       klv, z, h);
+    auto chain = [&](auto kernel, size_t lds) {
+      hipLaunchKernelGGL(kernel, dim3(with_down ? 2 : 1), dim3(kl_waves(KK) * 64), lds, stream,
+                         reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                         reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
+                         kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h);
+    };
+    if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
+    else chain(&hclt_kld_chain_kernel<KK, false>, 0);
   });
   check_launch_k("hclt_kld");
 }

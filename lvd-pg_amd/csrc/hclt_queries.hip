@@ -110,6 +110,62 @@ __global__ __launch_bounds__(256) void hclt_sample_states_kernel(const float* __
   for (int i = threadIdx.x; i < count * n_inner; i += blockDim.x) states[(size_t)first * n_inner + i] = st[i];
 }
 
+// States of the inner tree nodes, a lane per tree node: a wave takes one example and walks the
+// levels from the root, 64 nodes of a level at a time (`passes` records of 64 {node, parent}
+// pairs, -1: no node).  A lane reads its node's K noise values and the parameter row its
+// parent's state selects (two contiguous rows of 4K bytes) and scans them in order: first
+// maximum wins, no exchange between lanes.  The noise does not depend on any state, so its
+// requests leave before the parent's state is read.  The chosen states live in LDS (one byte
+// per node) and leave through a coalesced copy at the end; no barriers, a wave only reads its
+// own example's bytes.
+template <int K>
+__global__ __launch_bounds__(256) void hclt_sample_states_node_kernel(const float* __restrict__ logtheta,
+                                                                      const int2* __restrict__ passes_tab, int passes,
+                                                                      const float* __restrict__ node_noise,
+                                                                      int n_inner, int stride, int batch,
+                                                                      uint8_t* __restrict__ states) {
+  static_assert(K % 4 == 0, "rows are read as 16-byte words");
+  constexpr int CH = K < 32 ? K : 32;   // values scanned per round: 8 words of noise and 8 of parameters in registers
+  extern __shared__ uint8_t st[];   // [4 waves][stride]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int b = blockIdx.x * 4 + wave;
+  if (b >= batch) return;
+  uint8_t* mine = st + (size_t)wave * stride;
+  const float* g = node_noise + (size_t)b * n_inner * K;
+  int2 rec = passes_tab[lane];
+  for (int ps = 0; ps < passes; ++ps) {
+    const int n = rec.x, par = rec.y;
+    if (ps + 1 < passes) rec = passes_tab[(size_t)(ps + 1) * 64 + lane];
+    if (n >= 0) {
+      const float4* gz = reinterpret_cast<const float4*>(g + (size_t)n * K);
+      float best = 0.f;
+      int idx = 0;
+#pragma unroll
+      for (int j0 = 0; j0 < K; j0 += CH) {
+        float4 z[CH / 4], a[CH / 4];
+#pragma unroll
+        for (int i = 0; i < CH / 4; ++i) z[i] = gz[j0 / 4 + i];
+        const int k = par < 0 ? 0 : mine[par];
+        const float4* row = reinterpret_cast<const float4*>(logtheta + ((size_t)n * K + k) * K);
+#pragma unroll
+        for (int i = 0; i < CH / 4; ++i) a[i] = row[j0 / 4 + i];
+#pragma unroll
+        for (int i = 0; i < CH / 4; ++i) {
+          const float x[4] = {a[i].x + z[i].x, a[i].y + z[i].y, a[i].z + z[i].z, a[i].w + z[i].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int j = j0 + 4 * i + e;
+            if (j == 0 || x[e] > best) { best = x[e]; idx = j; }
+          }
+        }
+      }
+      mine[n] = (uint8_t)idx;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the next level's lanes read these bytes
+  }
+  for (int i = lane; i < n_inner; i += 64) states[(size_t)b * n_inner + i] = mine[i];
+}
+
 // Categories.  A wave takes kVarsPerWave consecutive variables of one example, 64 lanes x 4
 // categories each (more categories: further rounds), requests all their rows first and then
 // reduces them one by one: per variable the wave keeps the largest value and, among equal
@@ -203,7 +259,9 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   const bool lanes_fit = K_ >= 2 && K_ <= 64 && (K_ & (K_ - 1)) == 0;
-  const size_t st_bytes = (size_t)(4 * (64 / std::max(K_, 1))) * n_inner_;
+  const int stride = (n_inner_ + 15) & ~15;   // bytes of one example's states in LDS
+  // K lanes per example below 4 states, a wave per example from there on
+  const size_t st_bytes = K_ >= 4 ? (size_t)4 * stride : (size_t)(4 * (64 / std::max(K_, 1))) * n_inner_;
   if (!lanes_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
     SparseCircuit* g = general();
     DevBuf<int32_t> slots;
@@ -232,6 +290,17 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
       while ((t.size() - (size_t)n_inner_ - V_) % kSampleGroup) t.push_back(-1);
     }
     sample_groups_ = (int)((t.size() - (size_t)n_inner_ - V_) / kSampleGroup);
+    // the same levels in records of 64 {node, parent} pairs for the lane-per-node walk
+    std::vector<int32_t> rec;
+    for (const auto& lvl : by_depth) {
+      for (int32_t n : lvl) {
+        rec.push_back(n);
+        rec.push_back(t[n]);
+      }
+      while (rec.size() % 128) rec.push_back(-1);
+    }
+    sample_passes_ = (int)(rec.size() / 128);
+    d_sample_passes_.upload(rec, stream);
     d_sample_tabs_.upload(t, stream);
   }
   d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
@@ -244,13 +313,18 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, epb)), dim3(256), st_bytes, stream, d_logtheta_.p, d_sample_tabs_.p,
                        d_sample_tabs_.p + n_inner_ + V_, sample_groups_, d_node_noise, n_inner_, batch, d_state_.p);
   };
+  auto node_states = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, 4)), dim3(256), st_bytes, stream, d_logtheta_.p,
+                       reinterpret_cast<const int2*>(d_sample_passes_.p), sample_passes_, d_node_noise, n_inner_, stride, batch,
+                       d_state_.p);
+  };
   switch (K_) {
     case 2: states(&hclt_sample_states_kernel<2>); break;
-    case 4: states(&hclt_sample_states_kernel<4>); break;
-    case 8: states(&hclt_sample_states_kernel<8>); break;
-    case 16: states(&hclt_sample_states_kernel<16>); break;
-    case 32: states(&hclt_sample_states_kernel<32>); break;
-    default: states(&hclt_sample_states_kernel<64>); break;
+    case 4: node_states(&hclt_sample_states_node_kernel<4>); break;
+    case 8: node_states(&hclt_sample_states_node_kernel<8>); break;
+    case 16: node_states(&hclt_sample_states_node_kernel<16>); break;
+    case 32: node_states(&hclt_sample_states_node_kernel<32>); break;
+    default: node_states(&hclt_sample_states_node_kernel<64>); break;
   }
   hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(V_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
                      d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch, d_out);

@@ -135,6 +135,7 @@ def _hclt_pair(P, O, V, K, C, seed, tree=None):
     (2, 16, 5, [-1, 0]),                                           # the root is the only tree node with a block
     (11, 16, 7, [-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5]),               # five non-leaf children under one node
     (13, 32, 12, [-1, 0, 1, 1, 1, 1, 2, 3, 0, 8, 8, 8, 8]),
+    (541, 64, 4, [-1] + [0] * 270 + list(range(1, 271))),          # a level too wide for the chains' LDS ring
     (9, 8, 6, None)])                                              # a hidden size without block kernels
 def test_hclt_kld_and_gradient_match_oracle(gpu, oracle, V, K, C, tree):
     """KL recursion and its reverse pass on the block form (chains up and down the tree plus the
@@ -184,12 +185,14 @@ def test_sampling_bit_exact_random_dag(gpu, oracle, V, C, width, B, seed):
     assert (got < C).all()
 
 
-@pytest.mark.parametrize("V,K,C,B", [(7, 16, 8, 130), (12, 32, 256, 64)])
-def test_sampling_bit_exact_hclt(gpu, oracle, V, K, C, B):
+@pytest.mark.parametrize("V,K,C,B,tree", [
+    (7, 16, 8, 130, None), (12, 32, 256, 64, None), (10, 64, 5, 70, None), (9, 4, 6, 50, None), (6, 2, 3, 40, None),
+    (141, 8, 3, 33, [-1] + [0] * 70 + list(range(1, 71)))])      # a level of more than 64 tree nodes
+def test_sampling_bit_exact_hclt(gpu, oracle, V, K, C, B, tree):
     torch, P = gpu
     O = oracle
     from helpers import make_hclt, block_theta
-    parent, theta, leaf, fc = make_hclt(V, K, C, 5 + V)
+    parent, theta, leaf, fc = make_hclt(V, K, C, 5 + V, parent=None if tree is None else np.array(tree, np.int32))
     bpc = P.hclt_from_clt(parent, C, K)
     bpc.set_params(block_theta(parent, K, theta), leaf)
     ch, root = O.clt_children(parent)
