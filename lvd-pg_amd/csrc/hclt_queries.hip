@@ -188,17 +188,31 @@ __global__ __launch_bounds__(256) void hclt_sample_leaves_kernel(const float* __
   int bi[kVarsPerWave];
 #pragma unroll
   for (int q = 0; q < kVarsPerWave; ++q) { best[q] = -INFINITY; bi[q] = 0x7fffffff; }
+  // the states pick the leaf rows: requested once, ahead of everything that waits for them
+  int row[kVarsPerWave];
+#pragma unroll
+  for (int q = 0; q < kVarsPerWave; ++q) {
+    const int v = min(v0 + q, V - 1);
+    row[q] = v * K + sb[state_node[v]];
+  }
   for (int c0 = lane * 4; c0 < C; c0 += 256) {
     float x[kVarsPerWave][4];
+    if (vec) {
+      // the noise needs no state: its requests leave first
+      float4 n4[kVarsPerWave];
 #pragma unroll
-    for (int q = 0; q < kVarsPerWave; ++q) {
-      const int v = min(v0 + q, V - 1);
-      const float* lp = leaf_kc + ((size_t)v * K + sb[state_node[v]]) * C;
-      const float* g = leaf_noise + ((size_t)b * V + v) * C;
-      if (vec) {
-        const float4 a = *reinterpret_cast<const float4*>(lp + c0), n4 = *reinterpret_cast<const float4*>(g + c0);
-        x[q][0] = a.x + n4.x; x[q][1] = a.y + n4.y; x[q][2] = a.z + n4.z; x[q][3] = a.w + n4.w;
-      } else {
+      for (int q = 0; q < kVarsPerWave; ++q)
+        n4[q] = *reinterpret_cast<const float4*>(leaf_noise + ((size_t)b * V + min(v0 + q, V - 1)) * C + c0);
+#pragma unroll
+      for (int q = 0; q < kVarsPerWave; ++q) {
+        const float4 a = *reinterpret_cast<const float4*>(leaf_kc + (size_t)row[q] * C + c0);
+        x[q][0] = a.x + n4[q].x; x[q][1] = a.y + n4[q].y; x[q][2] = a.z + n4[q].z; x[q][3] = a.w + n4[q].w;
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < kVarsPerWave; ++q) {
+        const float* lp = leaf_kc + (size_t)row[q] * C;
+        const float* g = leaf_noise + ((size_t)b * V + min(v0 + q, V - 1)) * C;
 #pragma unroll
         for (int i = 0; i < 4; ++i) x[q][i] = c0 + i < C ? lp[c0 + i] + g[c0 + i] : -INFINITY;
       }
@@ -220,6 +234,76 @@ __global__ __launch_bounds__(256) void hclt_sample_leaves_kernel(const float* __
       if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
     }
     if (lane == 0 && v0 + q < V) out[(size_t)b * V + v0 + q] = (uint8_t)bx;
+  }
+}
+
+// Categories with the leaf table in LDS.  A workgroup takes one variable and kLeafExamples
+// examples: it turns the variable's [C][K] table into [K][C + 4] in LDS (rows stay 16-byte
+// aligned, the turning stores spread over the banks) and gathers the examples' states of the
+// node that picks the row; then every wave takes kLeafUnroll examples at a time, requests
+// their noise rows (C contiguous floats) and adds the table rows from LDS, so the table
+// crosses the L2 once per workgroup instead of a row per example.  Same rule as above: largest
+// value, lowest category among equal values.
+constexpr int kLeafExamples = 512, kLeafUnroll = 4, kLeafWaves = 8;
+
+__global__ __launch_bounds__(kLeafWaves * 64) void hclt_sample_leaves_lds_kernel(
+    const float* __restrict__ leaf, const int32_t* __restrict__ state_node, const uint8_t* __restrict__ states,
+    const float* __restrict__ leaf_noise, int V, int K, int C, int n_inner, int batch, uint8_t* __restrict__ out) {
+  extern __shared__ float tab[];   // [K][C + 4] floats, then kLeafExamples state bytes
+  const int CS = C + 4;
+  uint8_t* ks = reinterpret_cast<uint8_t*>(tab + (size_t)K * CS);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int v = blockIdx.x, b0 = blockIdx.y * kLeafExamples;
+  const int nb = min(kLeafExamples, batch - b0);
+  {
+    const float4* src = reinterpret_cast<const float4*>(leaf + (size_t)v * C * K);   // K is a multiple of 4
+    for (int i = threadIdx.x; i < C * K / 4; i += kLeafWaves * 64) {
+      const float4 x = src[i];
+      const int c = (i * 4) / K, k = (i * 4) % K;
+      tab[(k + 0) * CS + c] = x.x;
+      tab[(k + 1) * CS + c] = x.y;
+      tab[(k + 2) * CS + c] = x.z;
+      tab[(k + 3) * CS + c] = x.w;
+    }
+    const int node = state_node[v];
+    for (int e = threadIdx.x; e < kLeafExamples; e += kLeafWaves * 64)
+      ks[e] = e < nb ? states[(size_t)(b0 + e) * n_inner + node] : 0;
+  }
+  __syncthreads();
+  for (int e0 = wave * kLeafUnroll; e0 < nb; e0 += kLeafWaves * kLeafUnroll) {
+    float best[kLeafUnroll];
+    int bi[kLeafUnroll];
+#pragma unroll
+    for (int u = 0; u < kLeafUnroll; ++u) { best[u] = -INFINITY; bi[u] = 0x7fffffff; }
+    for (int c0 = lane * 4; c0 < C; c0 += 256) {
+      float4 n4[kLeafUnroll];
+#pragma unroll
+      for (int u = 0; u < kLeafUnroll; ++u) {
+        const int e = min(e0 + u, nb - 1);
+        n4[u] = *reinterpret_cast<const float4*>(leaf_noise + ((size_t)(b0 + e) * V + v) * C + c0);
+      }
+#pragma unroll
+      for (int u = 0; u < kLeafUnroll; ++u) {
+        const int e = min(e0 + u, nb - 1);
+        const float4 a = *reinterpret_cast<const float4*>(tab + (size_t)ks[e] * CS + c0);
+        const float x[4] = {a.x + n4[u].x, a.y + n4[u].y, a.z + n4[u].z, a.w + n4[u].w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (x[i] > best[u] || bi[u] == 0x7fffffff) { best[u] = x[i]; bi[u] = c0 + i; }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kLeafUnroll; ++u) {
+      float bv = best[u];
+      int bx = bi[u];
+#pragma unroll
+      for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o);
+        const int oi = __shfl_xor(bx, o);
+        if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
+      }
+      if (lane == 0 && e0 + u < nb) out[(size_t)(b0 + e0 + u) * V + v] = (uint8_t)bx;
+    }
   }
 }
 
@@ -303,10 +387,6 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     d_sample_passes_.upload(rec, stream);
     d_sample_tabs_.upload(t, stream);
   }
-  d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
-  const int64_t tot = (int64_t)V_ * K_ * C_;
-  hipLaunchKernelGGL(hclt_leaf_kc_kernel, dim3((unsigned)ceil_div(tot, 256)), dim3(256), 0, stream, d_leaf_.p, d_leaf_kc_.p,
-                     V_, K_, C_);
   d_state_.ensure((size_t)batch * n_inner_);
   const int epb = 4 * (64 / K_);
   auto states = [&](auto kernel) {
@@ -326,8 +406,20 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     case 32: node_states(&hclt_sample_states_node_kernel<32>); break;
     default: node_states(&hclt_sample_states_node_kernel<64>); break;
   }
-  hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(V_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
-                     d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch, d_out);
+  // the variable's table in LDS when 64 KB hold it and its rows are whole 16-byte words
+  const size_t lds = (size_t)K_ * (C_ + 4) * sizeof(float) + kLeafExamples;
+  if ((C_ & 3) == 0 && (K_ & 3) == 0 && lds <= (size_t)64 * 1024) {
+    hipLaunchKernelGGL(hclt_sample_leaves_lds_kernel, dim3(V_, ceil_div(batch, kLeafExamples)), dim3(kLeafWaves * 64), lds,
+                       stream, d_leaf_.p, d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch,
+                       d_out);
+  } else {
+    d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
+    const int64_t tot = (int64_t)V_ * K_ * C_;
+    hipLaunchKernelGGL(hclt_leaf_kc_kernel, dim3((unsigned)ceil_div(tot, 256)), dim3(256), 0, stream, d_leaf_.p, d_leaf_kc_.p,
+                       V_, K_, C_);
+    hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(V_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
+                       d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch, d_out);
+  }
   check_launch_q("hclt_sample");
   PCM_HIP(hipStreamSynchronize(stream));
 }
