@@ -1204,10 +1204,11 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
   PCM_DISPATCH_K(K_, {
     hipLaunchKernelGGL(hclt_soft_w_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)), dim3(128), 0, stream, d_logtheta_.p,
                        inv_t, n_inner_, Af, Ab);
-    hipLaunchKernelGGL(hclt_soft_walk_kernel<KK>, dim3(ns), dim3(kSoftWalkWaves * 64), 0, stream, Af, Ab, parent_of, order,
+    hipLaunchKernelGGL(hclt_soft_walk_kernel<KK>, dim3(ns), dim3(soft_walk_waves(KK) * 64), 0, stream, Af, Ab, parent_of, order,
                        level_ptr, soft_levels_, d_node_noise, n_inner_, batch, ns, inv_t, d_R_.p);
-    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, dim3(V_, ceil_div(batch, 4 * kSoftLeafRun)), dim3(256), 0, stream,
-                       d_leaf_.p, state_node, d_R_.p, V_, C_, batch, ns, d_out);
+    const int nchunks = ceil_div(C_, kSoftLeafCats);
+    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, dim3(V_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4)), dim3(256), 0,
+                       stream, d_leaf_.p, state_node, d_R_.p, V_, C_, batch, ns, nchunks, d_out);
   });
   check_launch("hclt_sample_soft");
   PCM_HIP(hipStreamSynchronize(stream));

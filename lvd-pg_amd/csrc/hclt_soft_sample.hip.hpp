@@ -19,7 +19,9 @@
 namespace pcm {
 
 constexpr float kSoftMinTemperature = 0.2f;
-constexpr int kSoftWalkWaves = 4;
+// Waves of a walk workgroup: a level's nodes are dealt to them, and each holds a node's two
+// operand tiles in registers.
+constexpr int soft_walk_waves(int K) { return K > 32 ? 8 : 16; }
 
 // A_v in the two operand layouts of the contractions (per call: it depends on T).
 template <int K>
@@ -36,10 +38,10 @@ __global__ void hclt_soft_w_kernel(const float* __restrict__ logtheta, float inv
 }
 
 // p_v for every tree node: one workgroup per 16-example slice, nodes level by level from the
-// root, the nodes of a level dealt to the four waves, a barrier between levels (a node reads
+// root, the nodes of a level dealt to the waves, a barrier between levels (a node reads
 // its parent's tile, stored one level earlier by some wave of this workgroup).
 template <int K>
-__global__ __launch_bounds__(kSoftWalkWaves * 64) void hclt_soft_walk_kernel(
+__global__ __launch_bounds__(soft_walk_waves(K) * 64) void hclt_soft_walk_kernel(
     const float* __restrict__ Af, const float* __restrict__ Ab, const int32_t* __restrict__ parent_of,
     const int32_t* __restrict__ order, const int32_t* __restrict__ level_ptr, int n_levels, const float* __restrict__ noise,
     int n_inner, int batch, int nslices, float inv_t, float* P) {
@@ -50,7 +52,7 @@ __global__ __launch_bounds__(kSoftWalkWaves * 64) void hclt_soft_walk_kernel(
   const uint32_t tile_stride = (uint32_t)nslices * kSlice * K * 4;
   const float* grow = noise ? noise + (size_t)min(lo.bcol, batch - 1) * n_inner * K + 4 * g : nullptr;
   for (int l = 0; l < n_levels; ++l) {
-    for (int i = level_ptr[l] + wave; i < level_ptr[l + 1]; i += kSoftWalkWaves) {
+    for (int i = level_ptr[l] + wave; i < level_ptr[l + 1]; i += soft_walk_waves(K)) {
       const int n = order[i], par = parent_of[n];
       WTile<K> af, ab;
       w_load<K>(Af, n, lane, af);
@@ -91,65 +93,82 @@ __global__ __launch_bounds__(kSoftWalkWaves * 64) void hclt_soft_walk_kernel(
   }
 }
 
-// out[b][u][:] = p_{v(u)}[b][:] * exp(leaf[u])  (a [1 x K] by [K x C] product per example and
-// variable).  A wave keeps exp(leaf[u]) of four categories per lane in registers for a run of
-// examples; an example's K probabilities are wave-uniform and come through scalar registers,
-// so the inner product is one fused multiply-add per (state, category).  Write-bound: the
-// output is batch x V x C floats.
-constexpr int kSoftLeafRun = 64;   // examples per wave
+// out[b][u][:] = p_{v(u)}[b][:] * exp(leaf[u]): a [B x K] by [K x C] product per variable, on
+// the matrix cores with categories as rows and the 16 examples of a slice as columns.  A wave
+// keeps exp(leaf[u]) of kSoftLeafCats categories as A operands in registers for a run of
+// kSoftLeafSlices slices; a slice's probabilities arrive in the tile layout the walk wrote them
+// in, which is the B operand layout: with k-step (kt, i) standing for the states
+// kt*16 + 4g + i, g = 0..3, component i of a lane's 16-byte word at kt is its B value and
+// component i of the word at leaf[u][c][kt*16 + 4g] its A value.  A lane of the result holds
+// four consecutive categories of one example: one 16-byte store, four lanes side by side.
+// Write-bound: the output is batch x V x C floats.
+constexpr int kSoftLeafSlices = 8;   // slices of 16 examples per work item
+constexpr int kSoftLeafCats = 256;   // categories per work item
 
 template <int K>
 __global__ __launch_bounds__(256) void hclt_soft_leaves_kernel(const float* __restrict__ leaf,
                                                                const int32_t* __restrict__ state_node,
                                                                const float* __restrict__ P, int V, int C, int batch,
-                                                               int nslices, float* __restrict__ out) {
+                                                               int nslices, int nchunks, float* __restrict__ out) {
+  constexpr int KT = K / 16, CT = kSoftLeafCats / 16;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int u = blockIdx.x;
-  const int b_first = (blockIdx.y * 4 + wave) * kSoftLeafRun;
-  if (b_first >= batch) return;
-  const int n = state_node[u];
-  const float* ptile = P + (size_t)n * nslices * kSlice * K;
-  for (int c0 = 4 * lane; c0 < C; c0 += 256) {
-    float sv[K][4];
+  const int item = blockIdx.y * 4 + wave;
+  const int chunk = item % nchunks, run = item / nchunks;
+  const int s_first = run * kSoftLeafSlices;
+  if (s_first >= nslices) return;
+  const int s_end = min(s_first + kSoftLeafSlices, nslices);
+  const int g = lane >> 4, bb = lane & 15;
+  const int cbase = chunk * kSoftLeafCats;
+  v4f a[CT][KT];
 #pragma unroll
-    for (int j4 = 0; j4 < K / 4; ++j4)
+  for (int ct = 0; ct < CT; ++ct) {
+    const int c = cbase + 16 * ct + bb;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const v4f x = c0 + c < C ? *reinterpret_cast<const v4f*>(leaf + ((size_t)u * C + c0 + c) * K + 4 * j4)
-                                 : v4f{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) sv[4 * j4 + i][c] = __expf(x[i]);
-      }
-    const int b_end = min(b_first + kSoftLeafRun, batch);
-    // example bq = slice * 16 + bb holds state kt*16 + 4*g + i at float ((kt*64 + 16*g + bb) * 4 + i) of its tile;
-    // the next example's probabilities are requested before this one's are used
-    auto fetch = [&](int bq, v4f (&dst)[K / 4]) {
-      const float* pe = ptile + (size_t)(bq >> 4) * (kSlice * K) + (bq & 15) * 4;   // wave-uniform address
-#pragma unroll
-      for (int q = 0; q < K / 4; ++q) dst[q] = *reinterpret_cast<const v4f*>(pe + (size_t)q * 64);
-    };
-    v4f pc[K / 4], pn[K / 4];
-    fetch(b_first, pc);
-    for (int bq = b_first; bq < b_end; ++bq) {
-      fetch(min(bq + 1, b_end - 1), pn);
-      float acc[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int q = 0; q < K / 4; ++q)   // q = kt * 4 + g: states q * 4 + i
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-          for (int c = 0; c < 4; ++c) acc[c] = fmaf(pc[q][i], sv[4 * q + i][c], acc[c]);
-#pragma unroll
-      for (int q = 0; q < K / 4; ++q) pc[q] = pn[q];
-      float* o = out + ((size_t)bq * V + u) * C + c0;
-      if (c0 + 3 < C && (C & 3) == 0) {
-        __builtin_nontemporal_store(v4f{acc[0], acc[1], acc[2], acc[3]}, reinterpret_cast<v4f*>(o));
+    for (int kt = 0; kt < KT; ++kt) {
+      if (c < C) {
+        const v4f x = *reinterpret_cast<const v4f*>(leaf + ((size_t)u * C + c) * K + kt * 16 + 4 * g);
+        a[ct][kt] = v4f{__expf(x[0]), __expf(x[1]), __expf(x[2]), __expf(x[3])};
       } else {
-#pragma unroll
-        for (int c = 0; c < 4; ++c)
-          if (c0 + c < C) o[c] = acc[c];
+        a[ct][kt] = v4f{0.f, 0.f, 0.f, 0.f};
       }
     }
+  }
+  const float* ptile = P + (size_t)state_node[u] * nslices * kSlice * K;
+  // the next slice's probabilities are requested before this one's are used
+  auto fetch = [&](int s, v4f (&dst)[KT]) {
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+      dst[kt] = *reinterpret_cast<const v4f*>(ptile + (size_t)s * (kSlice * K) + (size_t)(kt * 64 + lane) * 4);
+  };
+  v4f pc[KT], pn[KT];
+  fetch(s_first, pc);
+  const bool words = (C & 3) == 0;
+  for (int s = s_first; s < s_end; ++s) {
+    fetch(min(s + 1, s_end - 1), pn);
+    const int b = s * kSlice + bb;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      if (cbase + 16 * ct >= C) break;   // the same for the whole wave
+      v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[ct][kt][i], pc[kt][i], acc, 0, 0, 0);
+      const int c = cbase + 16 * ct + 4 * g;
+      if (b < batch) {
+        float* o = out + ((size_t)b * V + u) * C + c;
+        if (words && c + 3 < C) {
+          *reinterpret_cast<v4f*>(o) = acc;   // default policy: the other half of the 128-byte line follows with the next tile
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (c + i < C) o[i] = acc[i];
+        }
+      }
+    }
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt) pc[kt] = pn[kt];
   }
 }
 

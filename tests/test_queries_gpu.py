@@ -326,7 +326,8 @@ def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
     # HCLT: the K sum nodes of a tree node share the noise column of each hidden state.  Block
     # sizes run on the block form (two matrix contractions per tree node and 16 examples), other
     # sizes on the layered engine.
-    for Vh, K, Ch, Bh in ((6, 16, 4, 3), (11, 32, 256, 37), (9, 64, 10, 16), (5, 8, 4, 3)):
+    for Vh, K, Ch, Bh in ((6, 16, 4, 3), (11, 32, 256, 37), (9, 64, 10, 16), (5, 8, 4, 3),
+                          (7, 16, 200, 20), (6, 32, 20, 33)):       # category tiles left out past C; a partial tile of whole words
         parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23 + K)
         h = P.hclt_from_clt(parent, Ch, K)
         h.set_params(block_theta(parent, K, theta), leaf)
