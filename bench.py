@@ -232,8 +232,8 @@ def secondary(args):
                            "categories": C, "heads": H, "batch": B})
     elif args.workload == "c4_full":
         # C4 as a whole: 64 x 64 x 3 images cut into 64 patches of 8 x 8 x 3; one 192-variable K = 32 circuit with 128
-        # cluster heads per patch (block engine, eight streams) and the K = 64 top-level HCLT over the 64 cluster ids
-        V, K, C, H, B, NP, NS = 192, 32, 256, 128, 1024, 64, 8
+        # cluster heads per patch (block engine, 32 streams) and the K = 64 top-level HCLT over the 64 cluster ids
+        V, K, C, H, B, NP, NS = 192, 32, 256, 128, 1024, 64, 32
         img = workloads.grf_images(B, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(B, 3, 64, 64)
         patches = [np.ascontiguousarray(img[:, :, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8]).reshape(B, V)
                    for p in range(NP)]
@@ -270,7 +270,7 @@ def secondary(args):
         algo = sum(algorithmic_bytes(c.size("inner_tree_nodes"), V, K, C, B)["step"] + 2 * 4 * H * B for c in circs) \
             + algorithmic_bytes(top.size("inner_tree_nodes"), NP, 64, H, B)["step"]
         out.update(metric="images/sec fwd+bwd+EM, 12288-variable patch-clustered circuit: 64 patch circuits (192 vars, K=32, "
-                          "128 heads) on 8 streams + top HCLT (64 vars, K=64)",
+                          "128 heads) on 32 streams + top HCLT (64 vars, K=64)",
                    value=B / dt, unit="examples/s",
                    config={"workload": args.workload, "patch_circuits": NP, "streams": NS, "num_vars": NP * V, "hidden": K,
                            "top_hidden": 64, "categories": C, "heads": H, "batch": B})
