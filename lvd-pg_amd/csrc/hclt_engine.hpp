@@ -205,7 +205,6 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_soft_w_;          // ... exp(theta / T) in the two operand layouts
   int soft_levels_ = 0;
   DevBuf<int32_t> d_sample_tabs_;   // sampler tables: parent of every inner node | state-giving node of every variable | level order
-  int sample_groups_ = 0;
   DevBuf<int32_t> d_sample_passes_;   // the sampler's levels from the root in records of 64 {node, parent} pairs
   int sample_passes_ = 0;
   DevBuf<int64_t> d_sum_param_src_;

@@ -20,96 +20,6 @@ static void check_launch_q(const char* what) {
 // nodes) or of its parent (leaf tree nodes).  Same additions and comparisons, in the same
 // order, as the layered engine's sampler on the circuit's general form.
 
-// States of the inner tree nodes.  K lanes per example (64/K examples per wave), one wave per
-// group for the whole tree.  Nodes come level by level from the root (`order`, padded with -1
-// to groups of kSampleGroup that never straddle a level), so the nodes of a group are
-// independent and their parameter rows are fetched together: the walk is a chain of memory
-// latencies, one per group.  The chosen states live in LDS (one byte per node and example) and
-// leave through a coalesced copy at the end.  No barriers: a wave only reads its own examples.
-// Largest value and, among equal values, the lowest index over groups of K consecutive lanes,
-// left in every lane of the group.  The exchange inside rows of 16 lanes uses data-parallel-
-// primitive moves (lane ^ 1, lane ^ 2, mirror of 8, mirror of 16: a few cycles each), the step
-// across neighbouring rows a lane-swap instruction; only lane ^ 32 goes through the LDS crossbar.  The rule is symmetric, so the order of the
-// exchanges does not change the result.
-template <int kCtrl>
-__device__ __forceinline__ void argmax_dpp(float& x, int& idx) {
-  const float ov = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), kCtrl, 0xf, 0xf, true));
-  const int oi = __builtin_amdgcn_update_dpp(0, idx, kCtrl, 0xf, 0xf, true);
-  if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
-}
-
-template <int K>
-__device__ __forceinline__ void argmax_lanes(float& x, int& idx) {
-  if (K >= 2) argmax_dpp<0xB1>(x, idx);    // quad_perm [1,0,3,2]
-  if (K >= 4) argmax_dpp<0x4E>(x, idx);    // quad_perm [2,3,0,1]
-  if (K >= 8) argmax_dpp<0x141>(x, idx);   // row_half_mirror
-  if (K >= 16) argmax_dpp<0x140>(x, idx);  // row_mirror
-  if (K >= 32) {
-    // lane ^ 16: v_permlane16_swap exchanges the odd rows of its first operand with the even rows
-    // of its second, so with both operands equal an even row finds its partner in the second
-    // result and an odd row in the first
-    const bool even_row = ((threadIdx.x >> 4) & 1) == 0;
-    const int xi = __builtin_bit_cast(int, x);
-    const auto sx = __builtin_amdgcn_permlane16_swap(xi, xi, false, false);
-    const auto si = __builtin_amdgcn_permlane16_swap(idx, idx, false, false);
-    const float ov = __builtin_bit_cast(float, even_row ? (int)sx[1] : (int)sx[0]);
-    const int oi = even_row ? (int)si[1] : (int)si[0];
-    if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
-  }
-  if (K >= 64) {
-    const float ov = __shfl_xor(x, 32);
-    const int oi = __shfl_xor(idx, 32);
-    if (ov > x || (ov == x && oi < idx)) { x = ov; idx = oi; }
-  }
-}
-
-#ifndef PCM_SAMPLE_GROUP
-#define PCM_SAMPLE_GROUP 4
-#endif
-constexpr int kSampleGroup = PCM_SAMPLE_GROUP;   // independent nodes (same level) a wave handles together
-
-template <int K>
-__global__ __launch_bounds__(256) void hclt_sample_states_kernel(const float* __restrict__ logtheta,
-                                                                 const int32_t* __restrict__ parent_of,
-                                                                 const int32_t* __restrict__ order, int n_groups,
-                                                                 const float* __restrict__ node_noise, int n_inner,
-                                                                 int batch, uint8_t* __restrict__ states) {
-  constexpr int EPW = 64 / K;   // examples per wave
-  extern __shared__ uint8_t st[];   // [examples of the block][n_inner]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int j = lane % K, sub = lane / K;
-  const int ex_in_block = wave * EPW + sub;
-  const int b = blockIdx.x * (4 * EPW) + ex_in_block;
-  const bool live = b < batch;
-  uint8_t* mine = st + (size_t)ex_in_block * n_inner;
-  const float* g = node_noise + (size_t)(live ? b : 0) * n_inner * K;
-  for (int q = 0; q < n_groups; ++q) {
-    int nd[kSampleGroup];
-    float v[kSampleGroup];
-#pragma unroll
-    for (int i = 0; i < kSampleGroup; ++i) {
-      nd[i] = order[q * kSampleGroup + i];
-      const int n = max(nd[i], 0);
-      const int p = parent_of[n];
-      const int k = p < 0 ? 0 : mine[p];
-      v[i] = logtheta[((size_t)n * K + k) * K + j] + g[(size_t)n * K + j];
-    }
-#pragma unroll
-    for (int i = 0; i < kSampleGroup; ++i) {
-      int idx = j;
-      float x = v[i];
-      argmax_lanes<K>(x, idx);
-      if (j == 0 && nd[i] >= 0) mine[nd[i]] = (uint8_t)idx;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the bytes are read by the K lanes of this example
-  }
-  __syncthreads();
-  // [block examples][n_inner] -> states[b][n]
-  const int first = blockIdx.x * (4 * EPW);
-  const int count = min(4 * EPW, batch - first);
-  for (int i = threadIdx.x; i < count * n_inner; i += blockDim.x) states[(size_t)first * n_inner + i] = st[i];
-}
-
 // States of the inner tree nodes, a lane per tree node: a wave takes one example and walks the
 // levels from the root, 64 nodes of a level at a time (`passes` records of 64 {node, parent}
 // pairs, -1: no node).  A lane reads its node's K noise values and the parameter row its
@@ -342,11 +252,10 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
   if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
-  const bool lanes_fit = K_ >= 2 && K_ <= 64 && (K_ & (K_ - 1)) == 0;
+  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0;   // rows of whole 16-byte words, states in a byte
   const int stride = (n_inner_ + 15) & ~15;   // bytes of one example's states in LDS
-  // K lanes per example below 4 states, a wave per example from there on
-  const size_t st_bytes = K_ >= 4 ? (size_t)4 * stride : (size_t)(4 * (64 / std::max(K_, 1))) * n_inner_;
-  if (!lanes_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
+  const size_t st_bytes = (size_t)4 * stride;
+  if (!rows_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
     SparseCircuit* g = general();
     DevBuf<int32_t> slots;
     slots.upload(noise_slot_, stream);
@@ -354,27 +263,20 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     return;
   }
   if (d_sample_tabs_.n == 0) {
-    // per inner node: its parent | per variable: the node whose state picks its leaf row | inner
-    // nodes level by level from the root in groups of kSampleGroup (-1: padding)
+    // per inner node: its parent | per variable: the node whose state picks its leaf row
     std::vector<int32_t> t((size_t)n_inner_ + V_);
     for (int n = 0; n < n_inner_; ++n) {
       const int v = var_of_inner_[n];
       t[n] = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
     }
     for (int v = 0; v < V_; ++v) t[(size_t)n_inner_ + v] = children_[v].empty() ? inner_of_var_[parent_[v]] : inner_of_var_[v];
+    // inner nodes level by level from the root in records of 64 {node, parent} pairs (-1: padding)
     std::vector<std::vector<int32_t>> by_depth;
     for (int n = 0; n < n_inner_; ++n) {
       const size_t dep = (size_t)depth_[var_of_inner_[n]];
       if (by_depth.size() <= dep) by_depth.resize(dep + 1);
       by_depth[dep].push_back(n);
     }
-    sample_groups_ = 0;
-    for (const auto& lvl : by_depth) {
-      for (int32_t n : lvl) t.push_back(n);
-      while ((t.size() - (size_t)n_inner_ - V_) % kSampleGroup) t.push_back(-1);
-    }
-    sample_groups_ = (int)((t.size() - (size_t)n_inner_ - V_) / kSampleGroup);
-    // the same levels in records of 64 {node, parent} pairs for the lane-per-node walk
     std::vector<int32_t> rec;
     for (const auto& lvl : by_depth) {
       for (int32_t n : lvl) {
@@ -388,18 +290,12 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     d_sample_tabs_.upload(t, stream);
   }
   d_state_.ensure((size_t)batch * n_inner_);
-  const int epb = 4 * (64 / K_);
-  auto states = [&](auto kernel) {
-    hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, epb)), dim3(256), st_bytes, stream, d_logtheta_.p, d_sample_tabs_.p,
-                       d_sample_tabs_.p + n_inner_ + V_, sample_groups_, d_node_noise, n_inner_, batch, d_state_.p);
-  };
   auto node_states = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, 4)), dim3(256), st_bytes, stream, d_logtheta_.p,
                        reinterpret_cast<const int2*>(d_sample_passes_.p), sample_passes_, d_node_noise, n_inner_, stride, batch,
                        d_state_.p);
   };
   switch (K_) {
-    case 2: states(&hclt_sample_states_kernel<2>); break;
     case 4: node_states(&hclt_sample_states_node_kernel<4>); break;
     case 8: node_states(&hclt_sample_states_node_kernel<8>); break;
     case 16: node_states(&hclt_sample_states_node_kernel<16>); break;
