@@ -304,3 +304,73 @@ def test_multihead_hclt_on_the_block_engine(gpu, oracle, V, K, C, H, B, tree):
         P.kld(blk, blk)
     with pytest.raises(P.PcmError):                                    # no head kernels for this hidden size
         P.multihead_hclt_from_clt(np.array([-1, 0, 0, 0, 0, 1], np.int32), C, 64, H)
+
+
+def _random_tree(rng, V):
+    """A tree over V variables in one of three shapes: uniform attachment (bushy, large fan-out
+    near the root), mostly a chain, attachment to one of the last six nodes."""
+    parent = np.full(V, -1, np.int32)
+    style = int(rng.integers(0, 3))
+    for v in range(1, V):
+        if style == 0:
+            parent[v] = rng.integers(0, v)
+        elif style == 1 and rng.random() < 0.8:
+            parent[v] = v - 1
+        else:
+            parent[v] = rng.integers(max(0, v - 6), v)
+    return parent
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_block_engine_against_layered_engine(gpu, oracle, seed):
+    """Randomly drawn trees, hidden sizes, category counts and ragged batches: the block engines
+    (lean / general / wide walks, KL chains, Gumbel-max sampler) against the layered engine on the
+    equivalent description -- two independent implementations, the second checked against the
+    oracle elsewhere -- and, for the samples, against the oracle itself.  Tolerances: 1e-4
+    relative on likelihoods, KL and its gradient, 2e-4 on updated parameters; samples equal."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, describe_dag
+    rng = np.random.default_rng(9000 + seed)
+    V = int(rng.integers(2, 70))
+    K = int(rng.choice([16, 32, 64, 128]))
+    C = int(rng.choice([2, 3, 7, 16, 33, 100, 255, 256]))
+    B = int(rng.integers(1, 200))
+    parent, theta, leaf, fc = make_hclt(V, K, C, seed, parent=_random_tree(rng, V))
+    a = P.hclt_from_clt(parent, C, K)
+    a.set_params(block_theta(parent, K, theta), leaf)
+    d = describe_dag([O.hclt_dag(parent, K, C, theta, leaf)])
+    g = P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"], d["input_logp"], V, C)
+    np.testing.assert_allclose(P.vectorize_parameters(a), P.vectorize_parameters(g), atol=1e-6)
+    data = torch.from_numpy(rng.integers(0, C, (B, V)).astype(np.uint8)).cuda()
+    np.testing.assert_allclose(P.loglikelihoods(a, data).cpu().numpy(), P.loglikelihoods(g, data).cpu().numpy(), rtol=1e-4)
+    # KL and its gradient against a second parameter set
+    _, theta2, leaf2, _ = make_hclt(V, K, C, seed + 1000, parent=parent)
+    a2 = P.hclt_from_clt(parent, C, K)
+    a2.set_params(block_theta(parent, K, theta2), leaf2)
+    g2 = P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"], d["input_logp"], V, C)
+    P.update_parameters(g2, P.vectorize_parameters(a2))
+    ka, kg = P.kld(a, a2), P.kld(g, g2)
+    assert abs(ka - kg) <= 1e-4 * abs(kg)
+    for x, y in zip(P.kld_backward(a, a2), P.kld_backward(g, g2)):
+        assert np.abs(x - y).max() <= 1e-4 * np.abs(y).max()
+    # Gumbel-max samples against the oracle (compact noise: one draw per tree node and hidden state)
+    if K <= 64 and V * K * K < 150_000:
+        ch, _ = O.clt_children(parent)
+        inner = [v for v in O.clt_bottom_up(parent) if ch[v]]
+        nb = min(B, 40)
+        u = rng.random((nb, len(inner) * K)), rng.random((nb, V, C))
+        nn, ln = [(-np.log(-np.log(np.clip(x, 1e-12, 1 - 1e-12)))).astype(np.float32) for x in u]
+        slot = np.zeros(fc.n_edges, np.int64)
+        for r, v in enumerate(inner):
+            nk = len(fc.meta["sum_node"][v])
+            e0 = fc.meta["edge_of"][v]
+            slot[e0:e0 + nk * K] = np.tile(r * K + np.arange(K), nk)
+        want = O.sample(fc, nn, ln, noise_slot=slot)
+        got = P.sample(a, torch.from_numpy(nn).cuda(), torch.from_numpy(ln).cuda()).cpu().numpy()
+        assert np.array_equal(got, want)
+    # one EM step
+    for c in (a, g):
+        P.mini_batch_em(c, data, 1, batch_size=B, pseudocount=0.1, param_inertia=0.3)
+    pa, pg = np.exp(P.vectorize_parameters(a)), np.exp(P.vectorize_parameters(g))
+    assert np.max(np.abs(pa - pg) / np.maximum(pg, 1e-6)) < 2e-4
