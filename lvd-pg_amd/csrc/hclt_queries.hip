@@ -12,6 +12,14 @@ static void check_launch_q(const char* what) {
   if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
 }
 
+// Four consecutive noise values, read once: a non-temporal request, so the stream does not push
+// the tables out of the caches.
+__device__ __forceinline__ float4 noise_word(const float* p) {
+  typedef float v4f_t __attribute__((ext_vector_type(4)));
+  const v4f_t t = __builtin_nontemporal_load(reinterpret_cast<const v4f_t*>(p));
+  return make_float4(t[0], t[1], t[2], t[3]);
+}
+
 // ---- Gumbel-max sampling on the block form -------------------------------------------------
 // A sample is a top-down walk: the root's single sum node picks hidden state
 // j* = argmax_j(theta_root[0][j] + g[b][root][j]); a tree node whose parent picked k picks
@@ -54,7 +62,7 @@ __global__ __launch_bounds__(256) void hclt_sample_states_node_kernel(const floa
       for (int j0 = 0; j0 < K; j0 += CH) {
         float4 z[CH / 4], a[CH / 4];
 #pragma unroll
-        for (int i = 0; i < CH / 4; ++i) z[i] = gz[j0 / 4 + i];
+        for (int i = 0; i < CH / 4; ++i) z[i] = gz[j0 / 4 + i];   // default policy: a lane's row is one cache line read in pieces
         const int k = par < 0 ? 0 : mine[par];
         const float4* row = reinterpret_cast<const float4*>(logtheta + ((size_t)n * K + k) * K);
 #pragma unroll
@@ -190,7 +198,7 @@ __global__ __launch_bounds__(kLeafWaves * 64) void hclt_sample_leaves_lds_kernel
 #pragma unroll
       for (int u = 0; u < kLeafUnroll; ++u) {
         const int e = min(e0 + u, nb - 1);
-        n4[u] = *reinterpret_cast<const float4*>(leaf_noise + ((size_t)(b0 + e) * V + v) * C + c0);
+        n4[u] = noise_word(leaf_noise + ((size_t)(b0 + e) * V + v) * C + c0);
       }
 #pragma unroll
       for (int u = 0; u < kLeafUnroll; ++u) {
