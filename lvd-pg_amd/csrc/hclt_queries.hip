@@ -33,7 +33,8 @@ __device__ __forceinline__ float4 noise_word(const float* p) {
 // pairs, -1: no node).  A lane reads its node's K noise values and the parameter row its
 // parent's state selects (two contiguous rows of 4K bytes) and scans them in order: first
 // maximum wins, no exchange between lanes.  The noise does not depend on any state, so its
-// requests leave before the parent's state is read.  The chosen states live in LDS (one byte
+// requests leave a pass ahead (up to K = 32, where a row fits the registers twice), or at
+// least before the parent's state is read.  The chosen states live in LDS (one byte
 // per node) and leave through a coalesced copy at the end; no barriers, a wave only reads its
 // own example's bytes.
 template <int K>
@@ -50,36 +51,85 @@ __global__ __launch_bounds__(256) void hclt_sample_states_node_kernel(const floa
   if (b >= batch) return;
   uint8_t* mine = st + (size_t)wave * stride;
   const float* g = node_noise + (size_t)b * n_inner * K;
-  int2 rec = passes_tab[lane];
-  for (int ps = 0; ps < passes; ++ps) {
-    const int n = rec.x, par = rec.y;
-    if (ps + 1 < passes) rec = passes_tab[(size_t)(ps + 1) * 64 + lane];
-    if (n >= 0) {
-      const float4* gz = reinterpret_cast<const float4*>(g + (size_t)n * K);
-      float best = 0.f;
-      int idx = 0;
+  if constexpr (K <= 32) {
+    // the noise of a pass is requested one pass ahead (the table ends with two empty records)
+    int2 rec0 = passes_tab[lane], rec1 = passes_tab[64 + lane];
+    float4 z[K / 4];
 #pragma unroll
-      for (int j0 = 0; j0 < K; j0 += CH) {
-        float4 z[CH / 4], a[CH / 4];
+    for (int i = 0; i < K / 4; ++i) z[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (rec0.x >= 0) {
 #pragma unroll
-        for (int i = 0; i < CH / 4; ++i) z[i] = gz[j0 / 4 + i];   // default policy: a lane's row is one cache line read in pieces
-        const int k = par < 0 ? 0 : mine[par];
+      for (int i = 0; i < K / 4; ++i) z[i] = reinterpret_cast<const float4*>(g + (size_t)rec0.x * K)[i];
+    }
+    for (int ps = 0; ps < passes; ++ps) {
+      const int n = rec0.x, par = rec0.y;
+      const int2 rec2 = passes_tab[(size_t)(ps + 2) * 64 + lane];
+      const int k = (n >= 0 && par >= 0) ? mine[par] : 0;
+      float4 a[K / 4], zn[K / 4];
+      if (n >= 0) {
         const float4* row = reinterpret_cast<const float4*>(logtheta + ((size_t)n * K + k) * K);
 #pragma unroll
-        for (int i = 0; i < CH / 4; ++i) a[i] = row[j0 / 4 + i];
+        for (int i = 0; i < K / 4; ++i) a[i] = row[i];
+      }
 #pragma unroll
-        for (int i = 0; i < CH / 4; ++i) {
+      for (int i = 0; i < K / 4; ++i) zn[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (rec1.x >= 0) {
+#pragma unroll
+        for (int i = 0; i < K / 4; ++i) zn[i] = reinterpret_cast<const float4*>(g + (size_t)rec1.x * K)[i];
+      }
+      if (n >= 0) {
+        float best = 0.f;
+        int idx = 0;
+#pragma unroll
+        for (int i = 0; i < K / 4; ++i) {
           const float x[4] = {a[i].x + z[i].x, a[i].y + z[i].y, a[i].z + z[i].z, a[i].w + z[i].w};
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            const int j = j0 + 4 * i + e;
+            const int j = 4 * i + e;
             if (j == 0 || x[e] > best) { best = x[e]; idx = j; }
           }
         }
+        mine[n] = (uint8_t)idx;
       }
-      mine[n] = (uint8_t)idx;
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+#pragma unroll
+      for (int i = 0; i < K / 4; ++i) z[i] = zn[i];
+      rec0 = rec1;
+      rec1 = rec2;
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the next level's lanes read these bytes
+  } else {
+    // K = 64: a row is scanned in two rounds of 32 values, its noise requested with it
+  int2 rec = passes_tab[lane];
+    for (int ps = 0; ps < passes; ++ps) {
+      const int n = rec.x, par = rec.y;
+      if (ps + 1 < passes) rec = passes_tab[(size_t)(ps + 1) * 64 + lane];
+      if (n >= 0) {
+        const float4* gz = reinterpret_cast<const float4*>(g + (size_t)n * K);
+        float best = 0.f;
+        int idx = 0;
+  #pragma unroll
+        for (int j0 = 0; j0 < K; j0 += CH) {
+          float4 z[CH / 4], a[CH / 4];
+  #pragma unroll
+          for (int i = 0; i < CH / 4; ++i) z[i] = gz[j0 / 4 + i];   // default policy: a lane's row is one cache line read in pieces
+          const int k = par < 0 ? 0 : mine[par];
+          const float4* row = reinterpret_cast<const float4*>(logtheta + ((size_t)n * K + k) * K);
+  #pragma unroll
+          for (int i = 0; i < CH / 4; ++i) a[i] = row[j0 / 4 + i];
+  #pragma unroll
+          for (int i = 0; i < CH / 4; ++i) {
+            const float x[4] = {a[i].x + z[i].x, a[i].y + z[i].y, a[i].z + z[i].z, a[i].w + z[i].w};
+  #pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int j = j0 + 4 * i + e;
+              if (j == 0 || x[e] > best) { best = x[e]; idx = j; }
+            }
+          }
+        }
+        mine[n] = (uint8_t)idx;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");   // the next level's lanes read these bytes
+    }
   }
   for (int i = lane; i < n_inner; i += 64) states[(size_t)b * n_inner + i] = mine[i];
 }
@@ -294,6 +344,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
       while (rec.size() % 128) rec.push_back(-1);
     }
     sample_passes_ = (int)(rec.size() / 128);
+    rec.resize(rec.size() + 256, -1);   // two empty records: the walk requests records two passes ahead
     d_sample_passes_.upload(rec, stream);
     d_sample_tabs_.upload(t, stream);
   }
