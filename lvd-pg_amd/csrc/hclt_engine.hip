@@ -584,6 +584,11 @@ void HcltCircuit::build_param_order() {
   layer_ends_.push_back((int64_t)edge_parent_.size());
   n_edges_ = (int64_t)edge_parent_.size();
   d_sum_param_src_.upload(sum_param_src_);
+  {
+    std::vector<int32_t> pos((size_t)V_ * K_, 0);
+    for (size_t q = 0; q < input_order_.size(); ++q) pos[(size_t)input_order_[q]] = (int32_t)q;
+    d_in_pos_.upload(pos);
+  }
 
   // the same circuit in general form, for the queries that run on the general engine
   flat_ = FlatCircuit();
@@ -809,34 +814,35 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
 void HcltCircuit::vectorize(float* out, int64_t n) {
   if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
                          (long long)size(0));
-  std::vector<float> lt, lf;
-  fetch(lt, d_logtheta_.p, d_logtheta_.n, stream);
-  fetch(lf, d_leaf_.p, d_leaf_.n, stream);
+  if (!out) fail(PCM_ERR_ARG, "parameter vector is null");
   const int64_t ns = (int64_t)sum_param_src_.size();
-  for (int64_t i = 0; i < ns; ++i) out[i] = lt[sum_param_src_[i]];
-  float* o = out + ns;
-  for (size_t q = 0; q < input_order_.size(); ++q) {
-    const int v = input_order_[q] / K_, j = input_order_[q] % K_;
-    for (int c = 0; c < C_; ++c) o[q * C_ + c] = lf[((size_t)v * C_ + c) * K_ + j];
-  }
+  d_param_vec_.ensure((size_t)n);
+  if (ns > 0)
+    hipLaunchKernelGGL(hclt_params_gather_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
+                       d_sum_param_src_.p, d_logtheta_.p, d_param_vec_.p);
+  hipLaunchKernelGGL(hclt_leaf_vector_kernel<true>, dim3(V_, ceil_div(C_, kLeafVecCats)), dim3(256),
+                     (size_t)kLeafVecCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, d_in_pos_.p, K_, C_,
+                     d_param_vec_.p + ns);
+  check_launch("vectorize");
+  PCM_HIP(hipMemcpyAsync(out, d_param_vec_.p, (size_t)n * sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
 }
 
 void HcltCircuit::update_parameters(const float* in, int64_t n) {
   if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
                          (long long)size(0));
-  std::vector<float> lt;
-  fetch(lt, d_logtheta_.p, d_logtheta_.n, stream);
+  if (!in) fail(PCM_ERR_ARG, "parameter vector is null");
   const int64_t ns = (int64_t)sum_param_src_.size();
-  for (int64_t i = 0; i < ns; ++i) lt[sum_param_src_[i]] = in[i];
-  std::vector<float> lf((size_t)V_ * C_ * K_);
-  const float* o = in + ns;
-  for (size_t q = 0; q < input_order_.size(); ++q) {
-    const int v = input_order_[q] / K_, j = input_order_[q] % K_;
-    for (int c = 0; c < C_; ++c) lf[((size_t)v * C_ + c) * K_ + j] = o[q * C_ + c];
-  }
-  PCM_HIP(hipMemcpyAsync(d_logtheta_.p, lt.data(), lt.size() * sizeof(float), hipMemcpyHostToDevice, stream));
-  PCM_HIP(hipMemcpyAsync(d_leaf_.p, lf.data(), lf.size() * sizeof(float), hipMemcpyHostToDevice, stream));
-  PCM_HIP(hipStreamSynchronize(stream));
+  d_param_vec_.ensure((size_t)n);
+  PCM_HIP(hipMemcpyAsync(d_param_vec_.p, in, (size_t)n * sizeof(float), hipMemcpyHostToDevice, stream));
+  if (ns > 0)
+    hipLaunchKernelGGL(hclt_params_scatter_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
+                       d_sum_param_src_.p, d_param_vec_.p, d_logtheta_.p);
+  hipLaunchKernelGGL(hclt_leaf_vector_kernel<false>, dim3(V_, ceil_div(C_, kLeafVecCats)), dim3(256),
+                     (size_t)kLeafVecCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, d_in_pos_.p, K_, C_,
+                     d_param_vec_.p + ns);
+  check_launch("update_parameters");
+  PCM_HIP(hipStreamSynchronize(stream));   // the caller's vector is free again
   rebuild_w();
   general_stale_ = true;
 }

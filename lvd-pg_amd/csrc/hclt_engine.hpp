@@ -208,6 +208,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int32_t> d_sample_passes_;   // the sampler's levels from the root in records of 64 {node, parent} pairs
   int sample_passes_ = 0;
   DevBuf<int64_t> d_sum_param_src_;
+  DevBuf<int32_t> d_in_pos_;   // input node (v, j) -> its position among the input nodes of the parameter vector
+  DevBuf<float> d_param_vec_;  // a parameter vector on its way to or from the host
   int cap_slices_ = 0;
   bool have_flows_ = false;
   // soft evidence on the block kernels (single head, K <= 64)

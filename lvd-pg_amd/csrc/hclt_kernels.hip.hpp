@@ -677,6 +677,47 @@ __device__ __forceinline__ void put_w(float* Wf, float* Wb, int k, int j, float 
   Wb[(((j / 16) * KT + k / 16) * 64 + ((k % 16) / 4) * 16 + j % 16) * 4 + k % 4] = w;
 }
 
+// Parameter vector <-> block form (src/misc.jl:5-135 on the block layout): sum parameters are
+// gathered / scattered through their positions in logtheta; the leaf tables [V][C][K] turn into
+// the input nodes' runs of C values (node (v, j) at in_pos[v*K + j] * C) through LDS, 64
+// categories of one variable per workgroup, so both sides move whole rows.
+__global__ void hclt_params_gather_kernel(int64_t ns, const int64_t* __restrict__ src, const float* __restrict__ logtheta,
+                                          float* __restrict__ vec) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < ns) vec[i] = logtheta[src[i]];
+}
+
+__global__ void hclt_params_scatter_kernel(int64_t ns, const int64_t* __restrict__ src, const float* __restrict__ vec,
+                                           float* __restrict__ logtheta) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < ns) logtheta[src[i]] = vec[i];
+}
+
+constexpr int kLeafVecCats = 64;
+
+template <bool kToVector>
+__global__ __launch_bounds__(256) void hclt_leaf_vector_kernel(float* __restrict__ leaf, const int32_t* __restrict__ in_pos,
+                                                               int K, int C, float* __restrict__ vec) {
+  extern __shared__ float turn[];   // [kLeafVecCats][K + 1]
+  const int v = blockIdx.x, c0 = blockIdx.y * kLeafVecCats, nc = min(kLeafVecCats, C - c0);
+  float* rows = leaf + ((size_t)v * C + c0) * K;
+  if (kToVector) {
+    for (int i = threadIdx.x; i < nc * K; i += 256) turn[(i / K) * (K + 1) + i % K] = rows[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < nc * K; i += 256) {
+      const int j = i / nc, cc = i % nc;
+      vec[(size_t)in_pos[v * K + j] * C + c0 + cc] = turn[cc * (K + 1) + j];
+    }
+  } else {
+    for (int i = threadIdx.x; i < nc * K; i += 256) {
+      const int j = i / nc, cc = i % nc;
+      turn[cc * (K + 1) + j] = vec[(size_t)in_pos[v * K + j] * C + c0 + cc];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < nc * K; i += 256) rows[i] = turn[(i / K) * (K + 1) + i % K];
+  }
+}
+
 // Wf / Wb from the log-parameters (after parameters were set from outside).
 template <int K>
 __global__ void hclt_rebuild_w_kernel(const float* __restrict__ logtheta, float* __restrict__ Wf,
