@@ -1143,7 +1143,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     run_forward(d, d_ll_heads_.p);
     heads_forward(d, d_head_mask, nullptr, d_ll, true, rate);
     const size_t root_tile = (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
-    const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_) * sizeof(float);
+    const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_ + (size_t)kHeadWaves * 16) * sizeof(float);
     PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,
                                                stream, d.O + root_tile, d_head_wf_.p, d_head_wb_.p, head_logp(), H_, Hp_,
                                                d.B, d_head_mask, d.R + root_tile, head_aggr(), d_flow_shift_.p));

@@ -125,10 +125,11 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
     const float* __restrict__ O_root, const float* __restrict__ hwf, const float* __restrict__ hwb,
     const float* __restrict__ head_logp, int H, int Hp, int B, const float* __restrict__ mask, float* __restrict__ R_root,
     float* __restrict__ head_aggr, int* __restrict__ flow_shift) {
-  extern __shared__ float lds[];   // R [16][Hp] | E [16][K] | partial T tiles [waves][16*K]
+  extern __shared__ float lds[];   // R [16][Hp] | E [16][K] | partial T tiles [waves][16*K] | mask totals [waves][16]
   float* Rl = lds;
   float* El = Rl + 16 * Hp;
   float* Tl = El + 16 * K;
+  float* Fl = Tl + kHeadWaves * 16 * K;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x;
   const int b = lane & 15, g = lane >> 4, col = slice * kSlice + b;
   Tile<K> e;
@@ -140,6 +141,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
       for (int i = 0; i < 4; ++i) El[b * K + kt * 16 + 4 * g + i] = e.v[kt][i];
   Tile<K> t;
   tile_zero<K>(t);
+  float ftot = 0.f;   // this lane's share of its example's total mask
   for (int ht = wave; ht < Hp / 16; ht += kHeadWaves) {
     const v4f s = heads_contract_f<K>(hwf, ht, lane, e);
     v4f r;
@@ -147,6 +149,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
     for (int i = 0; i < 4; ++i) {
       const int h = ht * 16 + 4 * g + i;
       const float f = (h < H && col < B) ? mask[(size_t)h * B + col] : 0.f;
+      ftot += fmaxf(f, 0.f);
       r[i] = (f > 0.f && s[i] > 0.f) ? f / s[i] : 0.f;
       Rl[b * Hp + h] = r[i];
     }
@@ -162,6 +165,9 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
   v4f* tl = reinterpret_cast<v4f*>(Tl) + (size_t)wave * (K / 16) * 64;
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt) tl[kt * 64 + lane] = t.v[kt];
+  ftot += __shfl_xor(ftot, 16);
+  ftot += __shfl_xor(ftot, 32);
+  if (lane < 16) Fl[wave * 16 + lane] = ftot;
   __syncthreads();
   if (wave == 0) {
     v4f* dst = reinterpret_cast<v4f*>(R_root + (size_t)slice * kSlice * K);
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
   // bound on the flow of one example, as a power of two: total mask <= 2^shift
   if (threadIdx.x < 16 && col < B) {
     float tot = 0.f;
-    for (int h = 0; h < H; ++h) tot += fmaxf(mask[(size_t)h * B + col], 0.f);
+    for (int w2 = 0; w2 < kHeadWaves; ++w2) tot += Fl[w2 * 16 + b];
     int ex = 0;
     frexpf(tot, &ex);
     if (ex > 0) atomicMax(flow_shift, ex);
