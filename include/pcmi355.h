@@ -205,7 +205,8 @@ int pcm_kld_backward_dev(pcm_circuit* p, pcm_circuit* q, float* d_grad_p, float*
  * (:45) and has no counterpart taking a noise tensor.  d_node_noise is
  * [batch][pcm_sample_noise_size()] (HCLT: [batch][inner tree nodes in bottom-up
  * order][K], indexed by the hidden state chosen; general: one float per sum parameter),
- * d_leaf_noise is [batch][num_vars][num_cats], d_out [batch][num_vars] uint8.
+ * d_leaf_noise is [batch][num_vars][num_cats], d_out [batch][num_vars] uint8.  Both noise
+ * pointers must be 16-byte aligned (PCM_ERR_ARG otherwise).
  */
 int64_t pcm_sample_noise_size(const pcm_circuit* c);
 int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_noise,
@@ -219,7 +220,8 @@ int pcm_sample(pcm_circuit* c, const float* d_node_noise, const float* d_leaf_no
  * [batch][num_vars][num_cats]: every variable's top-down probabilities times its input
  * nodes' distributions (:262-284).  On an HCLT the sum nodes of one tree node share their
  * noise column per hidden state; compile the circuit with pcm_circuit_create for one
- * independent draw per sum edge.
+ * independent draw per sum edge.  On an HCLT with block kernels d_node_noise and d_out must be
+ * 16-byte aligned (PCM_ERR_ARG otherwise).
  */
 int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature, int32_t batch,
                     float* d_out);

@@ -1173,6 +1173,8 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
   if (!block_ || !(temperature >= kSoftMinTemperature)) return false;
   if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
+  if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_out)) & 15)
+    fail(PCM_ERR_ARG, "noise and output pointers must be 16-byte aligned (rows move as 16-byte words)");
   if (d_soft_tabs_.n == 0) {
     // parent of every inner node | per variable the node whose probabilities reach its leaf |
     // inner nodes by depth | level offsets

@@ -411,3 +411,25 @@ def test_prealloc_wrappers_run_the_queries_row_by_row(gpu, oracle):
     noisy = W.gumbel_sample_with_prealloc(bpc, p1, temperature=0.5, generator=torch.Generator(device="cuda").manual_seed(3))
     np.testing.assert_allclose(noisy.sum(-1), 1.0, rtol=1e-4)
     W.gumbel_sample_free_mem()
+
+
+def test_misaligned_noise_is_refused(gpu, oracle):
+    """The block samplers read noise rows as 16-byte words: a pointer that is not 16-byte
+    aligned is an argument error, not a launch."""
+    torch, P = gpu
+    from helpers import make_hclt, block_theta
+    V, K, C, B = 6, 16, 8, 5
+    parent, theta, leaf, _ = make_hclt(V, K, C, 3)
+    h = P.hclt_from_clt(parent, C, K)
+    h.set_params(block_theta(parent, K, theta), leaf)
+    need = int(P._lib.lib.pcm_sample_noise_size(h.handle))
+    flat = torch.zeros(B * need + 4, device="cuda")
+    leafn = torch.zeros((B, V, C), device="cuda")
+    shifted = flat[1:1 + B * need].view(B, need)            # contiguous, 4 bytes past an aligned address
+    assert shifted.data_ptr() % 16 != 0
+    with pytest.raises(P.PcmError):
+        P.sample(h, shifted, leafn)
+    with pytest.raises(P.PcmError):
+        P.gumbel_sample(h, B, temperature=0.7, node_noise=shifted)
+    aligned = flat[:B * need].view(B, need)
+    assert P.sample(h, aligned, leafn).shape == (B, V)
