@@ -1215,8 +1215,13 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
     hipLaunchKernelGGL(hclt_soft_walk_kernel<KK>, dim3(ns), dim3(soft_walk_waves(KK) * 64), 0, stream, Af, Ab, parent_of, order,
                        level_ptr, soft_levels_, d_node_noise, n_inner_, batch, ns, inv_t, d_R_.p);
     const int nchunks = ceil_div(C_, kSoftLeafCats);
-    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, dim3(V_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4)), dim3(256), 0,
-                       stream, d_leaf_.p, state_node, d_R_.p, V_, C_, batch, ns, nchunks, d_out);
+    const int use_rows = (C_ & 3) == 0 ? 1 : 0;   // rows of whole 16-byte words leave through an LDS pad
+    const dim3 lgrid(V_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4));
+    const size_t pad_bytes = use_rows ? (size_t)4 * kSlice * (kSoftLeafCats + 4) * sizeof(float) : 0;   // 65 KB
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_soft_leaves_kernel<KK>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)pad_bytes));
+    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, lgrid, dim3(256), pad_bytes, stream, d_leaf_.p, state_node, d_R_.p, V_,
+                       C_, batch, ns, nchunks, use_rows, d_out);
   });
   check_launch("hclt_sample_soft");
   PCM_HIP(hipStreamSynchronize(stream));
