@@ -15,11 +15,11 @@
  * Pinned by tests/test_oracle_pinning.py: brute-force latent enumeration on tiny HCLTs,
  * closed forms quoted from the reference's own tests, finite-difference checks of the
  * flows (= dLL/dlogtheta) and of the KL gradient, exact M-step properties, statistics
- * of exact samples.
- * PARITY UNPINNED: the two leaf lines of orc_kld_backward in their as-written form
- * (analytic == 0), which are not the analytic derivative and which no test or fixture
- * of the reference exercises; they are restated by reading
- * nodes/fixable_categorical_dist.jl:215-221 only.
+ * of exact samples, the closed form theta^(1/T) / sum theta^(1/T) and the cold limit of the
+ * relaxed sampler.  The two leaf lines of orc_kld_backward in their as-written form
+ * (analytic == 0; nodes/fixable_categorical_dist.jl:219, not the analytic derivative) are
+ * pinned through their fixed ratio to the finite-difference-checked analytic form and by a
+ * literal worked by hand.
  */
 #include <math.h>
 #include <stdint.h>

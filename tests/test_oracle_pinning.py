@@ -411,6 +411,47 @@ def test_kld_gradient_by_finite_differences():
             assert abs(fd - want) < 1e-6 * max(1, abs(want)), (i, which)
 
 
+def test_kld_backward_leaf_lines_as_written():
+    """src/nodes/fixable_categorical_dist.jl:219 (norm_params = false) returns, per category,
+    grad1 = g * (p1 - p2 + 1) and grad2 = g * exp(p1 - p2) -- not the analytic derivatives
+    g * exp(p1) * (p1 - p2 + 1) and -g * exp(p1), which central differences pin above.  The two
+    forms differ by a known factor each: written1 * exp(p1) = analytic1 and
+    written2 * exp(p2) = -analytic2.  Plus one literal worked by hand on the three-variable
+    fixture: a leaf under the branch of weight 0.2 receives node gradient 0.2, so a category
+    with p1 = log 0.1 against p2 = log 0.2 gets 0.2 * (1 - log 2) and 0.2 * 0.5."""
+    rng = np.random.default_rng(21)
+    root = random_dag(4, 3, rng, width=2)
+    f1 = O.bits_compile(root, 3, 4)
+    f2 = f1.copy()
+    f2.update_parameters((f1.vectorize_parameters() + rng.normal(0, 0.3, len(f1.vectorize_parameters()))).astype(np.float32))
+    for dbl in (True, False):
+        _, ek = O.kld(f1, f2, double=dbl)
+        _, _, _, a1, a2 = O.kld_backward(f1, f2, ek, analytic=True, double=dbl)
+        _, _, _, w1, w2 = O.kld_backward(f1, f2, ek, analytic=False, double=dbl)
+        tol = 1e-12 if dbl else 1e-5
+        assert np.abs(a1).max() > 1e-3 and np.abs(a2).max() > 1e-3
+        np.testing.assert_allclose(w1 * np.exp(f1.leaf_logp.astype(np.float64)), a1, rtol=tol, atol=tol * 1e-3)
+        np.testing.assert_allclose(w2 * np.exp(f2.leaf_logp.astype(np.float64)), -a2, rtol=tol, atol=tol * 1e-3)
+    # literal on the fixture of test/helpers/simple_circuits.jl:4-14
+    fc, pars = _three_var_pair(2)
+    g1c, g2c = fc.copy(), fc.copy()
+    p1, p2 = pars.copy(), pars.copy()
+    p1[:2] = p2[:2] = np.log(np.float32([0.2, 0.8]))
+    p1[2:7] = np.log(np.float32([0.1, 0.2, 0.3, 0.2, 0.2]))      # first input node: variable 0 of branch 1
+    p2[2:7] = np.log(np.float32([0.2, 0.1, 0.3, 0.3, 0.1]))
+    g1c.update_parameters(p1)
+    g2c.update_parameters(p2)
+    _, ek = O.kld(g1c, g2c)
+    grads, _, _, w1, w2 = O.kld_backward(g1c, g2c, ek)
+    first = int(g1c.input_nodes()[0])
+    np.testing.assert_allclose(grads[first], 0.2, rtol=1e-6)
+    off = g1c.in_off[first]
+    np.testing.assert_allclose(w1[off:off + 5], 0.2 * (1 + np.log([0.5, 2.0, 1.0, 2 / 3, 2.0])), rtol=1e-5)
+    np.testing.assert_allclose(w2[off:off + 5], 0.2 * np.array([0.5, 2.0, 1.0, 2 / 3, 2.0]), rtol=1e-5)
+    np.testing.assert_allclose(w1[off], 0.2 * (1 - np.log(2)), rtol=1e-5)
+    np.testing.assert_allclose(w2[off], 0.1, rtol=1e-5)
+
+
 # ------------------------------------------------------------------------------------
 # sampling
 # ------------------------------------------------------------------------------------
@@ -464,6 +505,91 @@ def test_soft_sampling_invariants():
     np.testing.assert_allclose(out.sum(axis=1), 1.0, rtol=1e-6)
     for ids in fc.meta["sum_node"].values():
         assert abs(td[ids].sum() - 1) < 1e-9
+
+
+@pytest.mark.parametrize("T", [0.5, 2.0])
+def test_soft_sampling_temperature_closed_form(T):
+    """src/queries/sample.jl:47-51: an edge's weight is exp((logp + g)/T) over the sum node's
+    total.  Without noise a single sum node over m leaves therefore hands leaf i the share
+    theta_i^(1/T) / sum_j theta_j^(1/T) (a product, or T in place of 1/T, gives another number)."""
+    C = 3
+    w = np.array([0.5, 0.3, 0.15, 0.05])
+    rng = np.random.default_rng(31)
+    lps = [log_dirichlet(rng, C) for _ in w]
+    fc = O.bits_compile(O.summate(*[O.input_node(0, lp) for lp in lps], logps=np.log(w).astype(np.float32)), C, 1)
+    want = w ** (1 / T) / (w ** (1 / T)).sum()
+    for dbl, tol in ((True, 1e-6), (False, 1e-5)):
+        td, out = O.gumbel_soft(fc, None, T, double=dbl)
+        np.testing.assert_allclose(td[:4], want, rtol=tol)
+        np.testing.assert_allclose(out[0], sum(want[i] * np.exp(lps[i].astype(np.float64)) for i in range(4)), rtol=tol)
+    # with noise: the same closed form on the tilted weights theta_i * exp(g_i)
+    g = _gumbel(rng, 4)
+    tilt = (w * np.exp(g)) ** (1 / T)
+    td, _ = O.gumbel_soft(fc, g, T, double=True)
+    np.testing.assert_allclose(td[:4], tilt / tilt.sum(), rtol=1e-6)
+
+
+@pytest.mark.parametrize("T", [0.3, 1.7])
+def test_soft_sampling_is_a_softmax_per_sum_node(T):
+    """Every sum node shares its top-down probability among its edges as
+    scipy.special.softmax((logp + g)/T); products pass theirs on to prime and sub; an input node's
+    share goes to its variable weighted by its distribution (src/queries/sample.jl:105-140, :262-284).
+    Recomputed here node by node with scipy on a DAG with shared sub-circuits."""
+    from scipy.special import softmax
+    rng = np.random.default_rng(32)
+    V, C = 5, 3
+    fc = O.bits_compile(random_dag(V, C, rng, width=3), C, V)
+    g = _gumbel(rng, fc.n_edges)
+    td, out = O.gumbel_soft(fc, g, T, double=True)
+    want = np.zeros(fc.n_nodes)
+    want[-1] = 1.0
+    want_out = np.zeros((V, C))
+    for n in range(fc.n_nodes - 1, -1, -1):
+        e0, e1 = fc.edge_ptr[n], fc.edge_ptr[n + 1]
+        if fc.type[n] == O.INPUT:
+            want_out[fc.in_var[n]] += want[n] * np.exp(fc.leaf_logp[fc.in_off[n]:fc.in_off[n] + C].astype(np.float64))
+            continue
+        share = softmax((fc.logp[e0:e1].astype(np.float64) + g[e0:e1]) / T) if fc.type[n] == O.SUM else np.ones(e1 - e0)
+        for e, s in zip(range(e0, e1), share):
+            want[fc.prime[e]] += want[n] * s
+            if fc.sub[e] >= 0:
+                want[fc.sub[e]] += want[n] * s
+    np.testing.assert_allclose(td, want, rtol=1e-9, atol=1e-15)
+    np.testing.assert_allclose(out, want_out, rtol=1e-9)
+
+
+def test_soft_sampling_cold_limit_is_the_gumbel_max_sample():
+    """As T -> 0 the relaxed sampler concentrates on the edge maximising logp + g, i.e. on what
+    orc_sample (pinned by the statistics of its draws above) picks from the same noise.  With
+    leaves that put all mass on one category the soft output is then the one-hot of the sample."""
+    rng = np.random.default_rng(33)
+    V, C, T = 5, 4, 0.01
+    fc = O.bits_compile(random_dag(V, C, rng, width=3), C, V)
+    for n in fc.input_nodes():                      # deterministic leaves
+        lp = np.full(C, -80.0, np.float32)
+        lp[rng.integers(C)] = 0.0
+        fc.leaf_logp[fc.in_off[n]:fc.in_off[n] + C] = lp
+    checked = 0
+    for trial in range(40):
+        g = _gumbel(rng, fc.n_edges)
+        # leave out draws whose visited sum nodes do not separate their two best edges by 0.2
+        # (exp(-0.2/T) = 2e-9 is what the runner-up keeps at this temperature)
+        hard = O.sample(fc, g[None, :], np.zeros((1, V, C)), double=True)[0]
+        td, out = O.gumbel_soft(fc, g, T, double=True)
+        gaps = []
+        for n in np.nonzero(fc.type == O.SUM)[0]:
+            if td[n] < 0.5:
+                continue
+            s = np.sort(fc.logp[fc.edge_ptr[n]:fc.edge_ptr[n + 1]].astype(np.float64) + g[fc.edge_ptr[n]:fc.edge_ptr[n + 1]])
+            if len(s) > 1:
+                gaps.append(s[-1] - s[-2])
+        if min(gaps) < 0.2:
+            continue
+        onehot = np.zeros((V, C))
+        onehot[np.arange(V), hard] = 1.0
+        assert np.abs(out - onehot).max() < 1e-6, trial
+        checked += 1
+    assert checked >= 10
 
 
 # ------------------------------------------------------------------------------------
