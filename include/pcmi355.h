@@ -248,7 +248,7 @@ int pcm_flows_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, i
  *
  * pcm_pairwise_mi: `pairwise_MI_chunked` (src/utils/information.jl:97-141 with the marginals of
  * :43-95): mutual information of every pair of variables of a device-resident uint8 data set
- * (element strides as in pcm_loglikelihoods, at most 65535 examples), counts smoothed with
+ * (element strides as in pcm_loglikelihoods; any number of examples in one call), counts smoothed with
  * pseudocount/C per category and pseudocount/C^2 per cell.  d_mi: device, [num_vars][num_vars],
  * symmetric, diagonal included.  Synchronous on `stream` (NULL: the default stream).
  *

@@ -14,8 +14,11 @@
 //   f(c) = (xlogx(p(c)) - xlogx(p(0))) / c,   M_u = (1/Z) sum_e la[u][x_eu],   L_u = sum_a la[u][a]
 // (each non-empty cell's term is shared out among its c examples; the empty cells' terms are the
 // closed-form remainder), so a pair costs three passes over its N examples against a C x C table
-// of 16-bit counters in LDS -- count, look up f, clear -- and no pass over the table itself.
+// of counters in LDS -- count, look up f, clear -- and no pass over the table itself.  Up to 65535
+// examples the counters are 16 bits wide and the whole table fits; beyond, they are 32 bits wide
+// and the table is walked in bands of rows.
 #include "common.hpp"
+#include "chow_liu.hpp"
 #include "stage_kernel.hip.hpp"
 
 #include <algorithm>
@@ -29,24 +32,23 @@ static void check_launch_c(const char* what) {
   if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
 }
 
-// Single marginals of one variable per workgroup:
-//   la[v][a] = log((count + pc/C)/Z),  stat[v] = {M_v, L_v}
-__global__ __launch_bounds__(256) void mi_single_kernel(const uint8_t* __restrict__ xb, int N, int Np, int C, float pc,
-                                                        float* __restrict__ la, double* __restrict__ stat) {
+// Single marginals of one variable per workgroup: with la[a] = log((count_a + pc/C)/Z),
+//   stat[v] = {M_v, L_v}
+__global__ __launch_bounds__(256) void mi_single_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int C, float pc,
+                                                        double* __restrict__ stat) {
   __shared__ unsigned cnt[256];
   __shared__ double red[256];
   const int v = blockIdx.x, t = threadIdx.x;
   cnt[t] = 0u;
   __syncthreads();
   const uint8_t* row = xb + (size_t)v * Np;
-  for (int b = t; b < N; b += 256) atomicAdd(&cnt[row[b]], 1u);
+  for (int64_t b = t; b < N; b += 256) atomicAdd(&cnt[row[b]], 1u);
   __syncthreads();
   const double Z = (double)N + (double)pc;
   double l = 0.0, m = 0.0;
   if (t < C) {
     const double p = ((double)cnt[t] + (double)pc / C) / Z;
     const double lg = p > 0.0 ? log(p) : -INFINITY;
-    la[(size_t)v * C + t] = (float)lg;
     l = lg;                                        // -inf if a category is empty and pc = 0: only used with pc > 0
     m = cnt[t] ? (double)cnt[t] * lg / Z : 0.0;
   }
@@ -63,7 +65,7 @@ __global__ __launch_bounds__(256) void mi_single_kernel(const uint8_t* __restric
 
 // f(c) for c = 0 .. N (f(0) unused).
 __global__ void mi_table_kernel(int N, int C, float pc, double* __restrict__ f) {
-  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c > N) return;
   const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
   const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
@@ -73,9 +75,40 @@ __global__ void mi_table_kernel(int N, int C, float pc, double* __restrict__ f) 
 
 constexpr int kMiThreads = 1024;
 
+// Calls fn(a, b) for every example of a pair of staged rows; thread t owns examples 4t .. 4t+3
+// (+ 4096 per further round).
+template <typename F>
+__device__ __forceinline__ void mi_each_example(const uint8_t* __restrict__ xu, const uint8_t* __restrict__ xv, int N, int t,
+                                                F&& fn) {
+  for (int64_t b4 = 4 * (int64_t)t; b4 < N; b4 += 4 * kMiThreads) {
+    const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (b4 + i < N) fn((int)((wu >> (8 * i)) & 0xffu), (int)((wv >> (8 * i)) & 0xffu));
+  }
+}
+
+// Sum of acc over the workgroup, then the closed-form remainder; thread 0 writes both halves of the matrix.
+__device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, int u, int v, int V, int C, double p0, double x0,
+                                               const double* __restrict__ stat, float* __restrict__ mi) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
+  if ((t & 63) == 0) red[t >> 6] = acc;
+  __syncthreads();
+  if (t == 0) {
+    double tot = 0.0;
+    for (int w = 0; w < kMiThreads / 64; ++w) tot += red[w];
+    double val = tot - stat[2 * u] - stat[2 * v] + (double)C * C * x0;
+    if (p0 > 0.0) val -= p0 * C * (stat[2 * u + 1] + stat[2 * v + 1]);
+    mi[(size_t)u * V + v] = (float)val;
+    mi[(size_t)v * V + u] = (float)val;
+  }
+  __syncthreads();
+}
+
 // Pairs (u <= v) in row-major order of the upper triangle, dealt round-robin to persistent
-// workgroups.  Thread t owns examples 4t .. 4t+3 (+ 4096 per further round).
-__global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int Np, int V, int C,
+// workgroups.  At most 65535 examples: a cell's count fits 16 bits, two cells per LDS word.
+__global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V, int C,
                                                              float pc, const double* __restrict__ f,
                                                              const double* __restrict__ stat, float* __restrict__ mi) {
   extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 doubles
@@ -96,88 +129,130 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
     const uint8_t* xu = xb + (size_t)u * Np;
     const uint8_t* xv = xb + (size_t)v * Np;
     double acc = 0.0;
-    // the three passes keep their keys in registers when the batch fits one round
-    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
-      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (b4 + i < N) {
-          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
-          atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
-        }
-    }
+    mi_each_example(xu, xv, N, t, [&](int a, int b) {
+      const int key = a * C + b;
+      atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
+    });
     __syncthreads();
-    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
-      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (b4 + i < N) {
-          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
-          acc += f[(cells[key >> 1] >> (16 * (key & 1))) & 0xffffu];
-        }
-    }
+    mi_each_example(xu, xv, N, t, [&](int a, int b) {
+      const int key = a * C + b;
+      acc += f[(cells[key >> 1] >> (16 * (key & 1))) & 0xffffu];
+    });
     __syncthreads();
-    for (int b4 = 4 * t; b4 < N; b4 += 4 * kMiThreads) {
-      const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (b4 + i < N) {
-          const int key = (int)((wu >> (8 * i)) & 0xffu) * C + (int)((wv >> (8 * i)) & 0xffu);
-          cells[key >> 1] = 0u;
-        }
-    }
-    // sum over the workgroup
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
-    if ((t & 63) == 0) red[t >> 6] = acc;
-    __syncthreads();
-    if (t == 0) {
-      double tot = 0.0;
-      for (int w = 0; w < kMiThreads / 64; ++w) tot += red[w];
-      double val = tot - stat[2 * u] - stat[2 * v] + (double)C * C * x0;
-      if (p0 > 0.0) val -= p0 * C * (stat[2 * u + 1] + stat[2 * v + 1]);
-      mi[(size_t)u * V + v] = (float)val;
-      mi[(size_t)v * V + u] = (float)val;
-    }
-    __syncthreads();
+    mi_each_example(xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
+    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, stat, mi);
   }
 }
 
-void pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t n_examples, int num_vars,
-                 int num_cats, float pseudocount, float* d_mi, hipStream_t stream) {
+// The same for any number of examples: 32-bit cells.  A C x C table of them can exceed the LDS, so
+// the categories of u are cut into bands of `band` rows and the three passes run once per band over
+// the examples whose u-category falls into it.
+__global__ __launch_bounds__(kMiThreads) void mi_pair_wide_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V,
+                                                                  int C, int band, float pc, const double* __restrict__ f,
+                                                                  const double* __restrict__ stat, float* __restrict__ mi) {
+  extern __shared__ unsigned cells[];   // band*C counters | 16 doubles
+  const int t = threadIdx.x;
+  const int words = band * C;
+  double* red = reinterpret_cast<double*>(cells + ((words + 1) & ~1));
+  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;
+  __syncthreads();
+  const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
+  const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
+  const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
+  int u = 0;
+  int64_t row0 = 0;
+  for (int64_t p = blockIdx.x; p < n_pairs; p += gridDim.x) {
+    while (p >= row0 + (V - u)) { row0 += V - u; ++u; }
+    const int v = u + (int)(p - row0);
+    const uint8_t* xu = xb + (size_t)u * Np;
+    const uint8_t* xv = xb + (size_t)v * Np;
+    double acc = 0.0;
+    for (int a0 = 0; a0 < C; a0 += band) {
+      mi_each_example(xu, xv, N, t, [&](int a, int b) {
+        if ((unsigned)(a - a0) < (unsigned)band) atomicAdd(&cells[(a - a0) * C + b], 1u);
+      });
+      __syncthreads();
+      mi_each_example(xu, xv, N, t, [&](int a, int b) {
+        if ((unsigned)(a - a0) < (unsigned)band) acc += f[cells[(a - a0) * C + b]];
+      });
+      __syncthreads();
+      mi_each_example(xu, xv, N, t, [&](int a, int b) {
+        if ((unsigned)(a - a0) < (unsigned)band) cells[(a - a0) * C + b] = 0u;
+      });
+      __syncthreads();
+    }
+    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, stat, mi);
+  }
+}
+
+MiShape mi_check(const uint8_t* d_data, int64_t n_examples, int num_vars, int num_cats, float pseudocount, const float* d_mi) {
   if (!d_data || !d_mi) fail(PCM_ERR_ARG, "data or output pointer is null");
-  if (n_examples < 1 || n_examples > 65535)
-    fail(PCM_ERR_UNSUPPORTED, "pairwise MI counts cells in 16 bits: 1..65535 examples per call, got %lld", (long long)n_examples);
+  if (n_examples < 1 || n_examples > 2147483584LL)
+    fail(PCM_ERR_ARG, "pairwise MI takes 1..2147483584 examples per call, got %lld", (long long)n_examples);
   if (num_vars < 1) fail(PCM_ERR_SHAPE, "num_vars must be positive, got %d", num_vars);
   if (num_cats < 1 || num_cats > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", num_cats);
   if (pseudocount < 0.f) fail(PCM_ERR_ARG, "pseudocount must not be negative");
-  const int N = (int)n_examples, Np = ceil_div(N, 64) * 64, V = num_vars, C = num_cats;
-  DevBuf<uint8_t> xb;
-  DevBuf<float> la;
-  DevBuf<double> stat, f;
-  xb.alloc((size_t)V * Np);
-  la.alloc((size_t)V * C);
-  stat.alloc((size_t)2 * V);
-  f.alloc((size_t)N + 1);
-  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Np, 64), ceil_div(V, 64)), dim3(256), 0, stream, d_data, stride_ex,
-                     stride_var, (const int32_t*)nullptr, N, Np, V, C, xb.p);
-  hipLaunchKernelGGL(mi_single_kernel, dim3(V), dim3(256), 0, stream, xb.p, N, Np, C, pseudocount, la.p, stat.p);
-  hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div(N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, f.p);
-  const int words = (C * C + 1) / 2;
-  const size_t lds = ((size_t)((words + 1) & ~1)) * 4 + (kMiThreads / 64) * sizeof(double);
+  MiShape s;
+  s.N = (int)n_examples;
+  s.V = num_vars;
+  s.C = num_cats;
+  s.Np = (n_examples + 63) / 64 * 64;
+  return s;
+}
+
+// Queues staging, marginals, the count table and the pair kernel on `stream`; allocates nothing.
+void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, const MiShape& sh, float pseudocount,
+               const MiScratch& w, float* d_mi, hipStream_t stream) {
+  const int N = sh.N, V = sh.V, C = sh.C;
   int dev = 0, cus = 0, max_lds = 0;
   PCM_HIP(hipGetDevice(&dev));
   PCM_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
   PCM_HIP(hipDeviceGetAttribute(&max_lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+  const size_t red_bytes = (kMiThreads / 64) * sizeof(double);
+  const bool narrow = N <= 65535;
+  int band = C;
+  size_t lds;
+  if (narrow) {
+    const int words = (C * C + 1) / 2;
+    lds = ((size_t)((words + 1) & ~1)) * 4 + red_bytes;
+  } else {
+    const size_t budget = std::min<size_t>((size_t)max_lds, 160 * 1024) - red_bytes - 8;
+    band = (int)std::min<size_t>((size_t)C, budget / ((size_t)C * 4));
+    if (band < 1) fail(PCM_ERR_UNSUPPORTED, "one row of the pair table does not fit %d bytes of LDS", max_lds);
+    band = ceil_div(C, ceil_div(C, band));         // equal bands
+    lds = ((size_t)((band * C + 1) & ~1)) * 4 + red_bytes;
+  }
   if (lds > (size_t)max_lds) fail(PCM_ERR_UNSUPPORTED, "pair table needs %zu bytes of LDS, device offers %d", lds, max_lds);
-  PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              (int)lds));
+  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(sh.Np, 64), ceil_div(V, 64)), dim3(256), 0, stream, d_data, stride_ex,
+                     stride_var, (const int32_t*)nullptr, N, sh.Np, V, C, w.xb);
+  hipLaunchKernelGGL(mi_single_kernel, dim3(V), dim3(256), 0, stream, w.xb, N, sh.Np, C, pseudocount, w.stat);
+  hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div((int64_t)N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, w.f);
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
   const int per_cu = std::max<int>(1, (int)(std::min<size_t>((size_t)max_lds, 160 * 1024) / lds));
   const int grid = (int)std::min<int64_t>(n_pairs, (int64_t)cus * std::min(per_cu, 2));
-  hipLaunchKernelGGL(mi_pair_kernel, dim3(grid), dim3(kMiThreads), lds, stream, xb.p, N, Np, V, C, pseudocount, f.p, stat.p,
-                     d_mi);
+  if (narrow) {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds));
+    hipLaunchKernelGGL(mi_pair_kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.f,
+                       w.stat, d_mi);
+  } else {
+    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_wide_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(mi_pair_wide_kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, band,
+                       pseudocount, w.f, w.stat, d_mi);
+  }
   check_launch_c("pairwise_mi");
+}
+
+void pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t n_examples, int num_vars,
+                 int num_cats, float pseudocount, float* d_mi, hipStream_t stream) {
+  const MiShape sh = mi_check(d_data, n_examples, num_vars, num_cats, pseudocount, d_mi);
+  DevBuf<uint8_t> xb;
+  DevBuf<double> stat, f;
+  xb.alloc((size_t)sh.V * sh.Np);
+  stat.alloc((size_t)2 * sh.V);
+  f.alloc((size_t)sh.N + 1);
+  mi_launch(d_data, stride_ex, stride_var, sh, pseudocount, MiScratch{xb.p, stat.p, f.p}, d_mi, stream);
   PCM_HIP(hipStreamSynchronize(stream));   // the scratch arrays die with this call
 }
 

@@ -9,8 +9,9 @@ from .circuits import hclt_from_clt
 def pairwise_MI(data, num_cats=None, pseudocount=0.1):
     """`pairwise_MI_chunked(data; num_cats, pseudocount)` (src/utils/information.jl:97-141):
     mutual information of every pair of variables of a uint8 device tensor [N, V]; returns a
-    float32 device tensor [V, V] (symmetric, diagonal included).  No chunking is needed: a
-    pair's table never leaves the workgroup that counts it."""
+    float32 device tensor [V, V] (symmetric, diagonal included).  Any number of examples in one
+    call: a pair's table never leaves the workgroup that counts it (16-bit cells up to 65535
+    examples, 32-bit cells walked in bands of rows beyond)."""
     if not (isinstance(data, torch.Tensor) and data.is_cuda and data.dtype == torch.uint8 and data.dim() == 2):
         raise ValueError("data must be a 2-D uint8 tensor on the GPU (examples x variables)")
     n, v = data.shape
