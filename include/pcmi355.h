@@ -261,6 +261,20 @@ int pcm_pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var
 int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent);
 
 /*
+ * pcm_pairwise_mi without any allocation.  No counterpart in the reference: it is for callers that
+ * cannot call hipMalloc (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * it).  Same arguments, kernels and results as pcm_pairwise_mi; the staging buffer and the two
+ * tables the kernels need live in a fixed 16.6 MiB array of the library's code object, held by every
+ * GPU the library runs on until the process ends.  Limits (PCM_ERR_UNSUPPORTED beyond them):
+ * num_examples <= 65535, num_vars <= 4096, num_vars * ceil64(num_examples) <= 16 MiB (e.g. 4096
+ * examples of 3072 variables).  The work is queued on `stream` and the call does NOT wait for it.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls queued on one stream do not.
+ */
+int pcm_pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
+                           int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream);
+
+/*
  * Adam ascent step on the sum parameters followed by per-sum-node normalisation
  * (src/sgd/adam.jl:63-86, :88-127, :318-319).  d_grad, d_params (unnormalised
  * log-parameters), d_m, d_v are device vectors in parameter-vector order over the sum

@@ -4,7 +4,7 @@ import subprocess
 import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["api.hip", "hclt_engine.hip", "hclt_queries.hip", "hclt_kld.hip", "hclt_wide.hip", "chow_liu.hip", "sparse_engine.hip"]
+SOURCES = ["api.hip", "hclt_engine.hip", "hclt_queries.hip", "hclt_kld.hip", "hclt_wide.hip", "chow_liu.hip", "pairwise_mi_static.hip", "sparse_engine.hip"]
 OUT = os.path.join(HERE, "libpcmi355.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
          # packed-fp32 code generation is switched off for every device function

@@ -226,6 +226,14 @@ int pcm_pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var
   });
 }
 
+int pcm_pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
+                           int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream) {
+  return guarded([&] {
+    pcm::pairwise_mi_static(d_data, stride_ex, stride_var, num_examples, num_vars, num_cats, pseudocount, d_mi,
+                            static_cast<hipStream_t>(stream));
+  });
+}
+
 int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent) {
   return guarded([&] { pcm::chow_liu_tree(mi, num_vars, clt_parent); });
 }

@@ -52,6 +52,7 @@ _SIGS = {
     "pcm_loglikelihoods_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, vp],
     "pcm_flows_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, c_f32, vp, vp],
     "pcm_pairwise_mi": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],
+    "pcm_pairwise_mi_static": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],
     "pcm_chow_liu_tree": [vp, c_i32, vp],
     "pcm_set_timing": [H, c_i32],
     "pcm_get_timing": [H, vp, c_i32],
