@@ -228,7 +228,9 @@ void HcltCircuit::build_schedules() {
   // lean schedule rows (see hclt_walk_lean.hip.hpp) from the padded items of a walk, or none
   // if some node has more operands than the lean kernels hold
   const size_t leaf_stride = (size_t)C_ * K_ * sizeof(float);
-  auto make_lean = [&](const std::vector<StepItem>& sched, bool forward, int stride, DevBuf<int32_t>& dst) -> bool {
+  // (backward: ratio_slot[n] is the LDS slot in which node n finds its ratio tile, left there by its parent)
+  auto make_lean = [&](const std::vector<StepItem>& sched, bool forward, int stride, DevBuf<int32_t>& dst,
+                       const std::vector<int32_t>* ratio_slot = nullptr) -> bool {
     if (K_ > 32 || lds_slots_ > 255 || (size_t)V_ * leaf_stride >= ((size_t)1 << 31)) return false;
     std::vector<int32_t> f((size_t)kLeanFields * kWalkWaves * stride, 0);
     for (int s = 0; s < stride; ++s)
@@ -239,7 +241,7 @@ void HcltCircuit::build_schedules() {
         put(kLA1, -1); put(kLA2, -1); put(kLA3, -1);
         if (n < 0) {   // idle: trash tile, trash slot, block and leaf rows of node / variable 0
           put(kLNode, n_inner_);
-          put(kLSlots, forward ? (int32_t)(0xffffff00u | (uint32_t)trash_slot) : (trash_slot | trash_slot << 8));
+          put(kLSlots, (int32_t)(0xffffff00u | (uint32_t)trash_slot));
           continue;
         }
         put(kLW, (int32_t)((size_t)n * K_ * K_ * sizeof(float)));
@@ -257,12 +259,16 @@ void HcltCircuit::build_schedules() {
           }
           put(kLSlots, (int32_t)slots);
         } else {
-          if (lc[n].size() + ic[n].size() > 3 || it.in_slot < 0 || (it.flags & kItemSpillOut)) return false;
+          if (lc[n].size() + ic[n].size() > 3) return false;
           int q = 0;
-          for (int c : ic[n]) put(kLA1 + q++, c << 3);
+          uint32_t slots = (uint32_t)(par[n] < 0 ? trash_slot : (*ratio_slot)[n]) | 0xffffff00u;
+          for (int c : ic[n]) {
+            slots = (slots & ~(0xffu << (8 * (q + 1)))) | ((uint32_t)(*ratio_slot)[c] << (8 * (q + 1)));
+            put(kLA1 + q++, c << 3);
+          }
           for (size_t i = 0; i < lc[n].size(); ++i)
             put(kLA1 + q++, (int32_t)((size_t)lc[n][i] * leaf_stride) | 1 | (int32_t)((i + 1) << 1));
-          put(kLSlots, it.out_slot | it.in_slot << 8);
+          put(kLSlots, (int32_t)slots);
         }
       }
     dst.upload(f);
@@ -403,8 +409,30 @@ void HcltCircuit::build_schedules() {
       }
     }
     n_bwd_steps_ = (int)sched.size() / kWalkWaves;
+    // The lean backward walk hands every inner child its own tile: a slot per (parent, inner child) pair, taken
+    // in the parent's step and free again from the step after the child's.
+    std::vector<int32_t> ratio_slot(n_inner_, -1);
+    bool slots_ok = true;
+    {
+      std::vector<int32_t> fs;
+      for (int sl = trash_slot - 1; sl >= 0; --sl) fs.push_back(sl);
+      for (int st = 0; st < n_bwd_steps_ && slots_ok; ++st) {
+        std::vector<int32_t> freed;
+        for (int w = 0; w < kWalkWaves && slots_ok; ++w) {
+          const int n = sched[(size_t)st * kWalkWaves + w].node;
+          if (n < 0) continue;
+          if (par[n] >= 0) freed.push_back(ratio_slot[n]);
+          for (int c : ic[n]) {
+            if (fs.empty()) { slots_ok = false; break; }
+            ratio_slot[c] = fs.back();
+            fs.pop_back();
+          }
+        }
+        fs.insert(fs.end(), freed.begin(), freed.end());
+      }
+    }
     make_fields(sched, pre, false, bwd_stride_, d_bwd_fields_);
-    bwd_lean_ = !bwd_spill_ && make_lean(sched, false, bwd_stride_, d_bwd_lean_);
+    bwd_lean_ = slots_ok && make_lean(sched, false, bwd_stride_, d_bwd_lean_, &ratio_slot);
     d_bwd_sched_.upload(sched);
   }
   // ---- statistics: the static operands of every node ------------------------------------
@@ -440,8 +468,14 @@ void HcltCircuit::build_schedules() {
         q.hvar[q.n_hist++] = lc[n][i];
       }
     }
+    {   // its LDS: two histograms if they fit, else one (or the parked edge-flow blocks, if larger) | per-wave pads
+      const size_t hist = 2 * (size_t)C_ * K_, park = (size_t)kStatLeanWaves * K_ * K_, pads = (size_t)kStatLeanWaves * kSlice * K_;
+      stat_lean_hists_ = (std::max(2 * hist, park) + pads) * 4 <= (size_t)max_lds_ ? 2 : 1;
+      if ((std::max(hist, park) + pads) * 4 > (size_t)max_lds_) stat_lean_ = false;
+    }
     if (stat_lean_) d_stat_lean_.upload(sn);
   }
+  lean_ = fwd_lean_ && bwd_lean_ && stat_lean_;
   if (ext.empty()) ext.push_back(0);
   d_ext_ops_.upload(ext);
   if (getenv("PCM_VERBOSE"))
@@ -650,7 +684,7 @@ int64_t HcltCircuit::size(int what) const {
     case 11: return (int64_t)V_ * K_;
     case 12: return H_;
     case 13: return 0;
-    case 14: return wide_walk_ ? 3 : !block_ ? 0 : (fwd_lean_ && bwd_lean_ && stat_lean_) ? 1 : 2;
+    case 14: return wide_walk_ ? 3 : !block_ ? 0 : lean_ ? 1 : 2;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -860,7 +894,7 @@ void HcltCircuit::ensure_batch(int batch) {
     d_wide_es_.alloc((size_t)n_inner_ * tile);
     d_xb_.alloc((size_t)V_ * ns * kSlice);
     d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
-    d_xn_.zero();
+    d_xn_.zero(stream);
     cap_slices_ = ns;
     return;
   }
@@ -871,9 +905,10 @@ void HcltCircuit::ensure_batch(int batch) {
     d_wide_rs_.alloc((size_t)n_inner_ * tile);
     d_wide_es_.alloc((size_t)n_inner_ * tile);
   }
+  if (lean_) d_M_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
   d_xb_.alloc((size_t)V_ * ns * kSlice);
   d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
-  d_xn_.zero();
+  d_xn_.zero(stream);
   cap_slices_ = ns;
 }
 
@@ -891,6 +926,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.O = d_O_.p;
   d.R = d_R_.p;
   d.G = d_G_.p;
+  d.M = d_M_.p;
   d.ext_ops = d_ext_ops_.p;
   d.B = batch;
   d.nslices = ceil_div(batch, kSlice);
@@ -927,7 +963,7 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
   };
   // the lean kernels address every array with 32-bit offsets from one descriptor
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
-  if (fwd_lean_ && small && !force_general_walks_) {
+  if (lean_ && small && !force_general_walks_) {
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
@@ -951,7 +987,7 @@ void HcltCircuit::run_backward(const HcltDev& d) {
                        bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
-  if (bwd_lean_ && small && !force_general_walks_) {
+  if (lean_ && small && !force_general_walks_) {
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
       hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_lean_.p, bwd_stride_,
@@ -980,17 +1016,18 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   const size_t hist = 2 * (size_t)C_ * (K_ + 1);                    // words per histogram (two limbs)
-  if (stat_lean_ && !force_general_walks_) {
-    // LDS: one histogram (or the parked edge-flow blocks, whichever is larger) | per-wave pads
+  const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
+  if (lean_ && small && !force_general_walks_) {
+    // LDS: the histograms of a pass (or the parked edge-flow blocks, whichever is larger) | per-wave pads
     const size_t park = (size_t)kStatLeanWaves * K_ * K_;
-    const size_t hw = (std::max(hist, park) + 3) & ~(size_t)3;
-    const size_t lds = (hw + (size_t)kStatLeanWaves * kSlice * (K_ + 16)) * 4;
-    if (lds <= (size_t)max_lds_) {
+    const size_t hw = std::max((size_t)stat_lean_hists_ * 2 * C_ * K_, park);
+    const size_t lds = (hw + (size_t)kStatLeanWaves * kSlice * K_) * 4;
+    {
       PCM_DISPATCH_LEAN_K(K_, {
         PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_lean_kernel<KK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(n_inner_), dim3(kStatLeanWaves * 64), lds, stream, d,
-                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, limb,
+                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
                            H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
       });
       check_launch("hclt_stats_lean");

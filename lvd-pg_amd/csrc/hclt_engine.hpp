@@ -101,6 +101,7 @@ struct HcltDev {
   float* O;               // [n_inner][nslices][16*K] node values, tile-native layout
   float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
+  float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (lean kernels; row n_inner: idle waves)
   int32_t B, Bp, nslices, C, n_inner, V;
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
   uint32_t leaf_slice;    // 0; soft evidence: the "leaf table" holds one row per example ([V][Bp][K], the
@@ -191,7 +192,10 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int32_t> d_child_inner_, d_child_leaf_;
   DevBuf<StepItem> d_fwd_sched_, d_bwd_sched_, d_stat_items_;
   DevBuf<int32_t> d_fwd_fields_, d_bwd_fields_, d_fwd_lean_, d_bwd_lean_;
-  bool fwd_lean_ = false, bwd_lean_ = false, stat_lean_ = false;   // the lean kernels can run this tree
+  bool fwd_lean_ = false, bwd_lean_ = false, stat_lean_ = false;   // each lean kernel could run this tree ...
+  bool lean_ = false;   // ... and all three do (they share the stored row maxima, so it is all or none)
+  DevBuf<float> d_M_;
+  int stat_lean_hists_ = 1;   // histograms the lean statistics kernel holds in LDS per pass
   DevBuf<StatNode> d_stat_lean_;
   int fwd_stride_ = 0, bwd_stride_ = 0;
   DevBuf<uint32_t> d_ext_ops_;

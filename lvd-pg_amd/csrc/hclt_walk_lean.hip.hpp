@@ -26,13 +26,14 @@ namespace pcm {
 //   kLW     byte offset of the node's parameter block
 //   kLA0    byte offset of the node's own leaf rows (variable * leaf_stride)
 //   kLA1..3 forward: leaf children's rows (-1: none; their categories are bytes 1..3 of the
-//           packed word).  backward: children, -1: none, leaf child: row offset | 1 | category
-//           byte << 1, inner child: node index << 3 (its value tile)
-//   kLNode  node index (value / flow tile, packed-category row); idle waves: n_inner, the
-//           trash tile (its category row is out of range and reads as zero)
-//   kLSlots forward: out slot | child slots << 8, 16, 24 (0xff: none); backward: out slot |
-//           slot of the parent's flow tile << 8
-//   kLFlags bit 0: root
+//           packed word).  backward: children, inner ones first, -1: none, leaf child: row
+//           offset | 1 | category byte << 1, inner child: node index << 3 (its value tile)
+//   kLNode  node index (value / flow tile, packed-category row, row of maxima); idle waves:
+//           n_inner, the trash tile (its category row is out of range and reads as zero)
+//   kLSlots forward: out slot | child slots << 8, 16, 24 (0xff: none); backward: slot holding
+//           this node's ratio tile | slots of the inner children's ratio tiles << 8, 16, 24
+//           (0xff: that child is a leaf or absent)
+//   kLFlags bit 0: root; bit 1: root of a multi-head circuit
 enum { kLW = 0, kLA0, kLA1, kLA2, kLA3, kLNode, kLSlots, kLFlags, kLeanFields };
 
 constexpr int kLeanChunk = 62;   // steps per refill: 64 lanes minus two steps of look-ahead
@@ -115,6 +116,11 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
   const __amdgpu_buffer_rsrc_t rX =
       make_rsrc(d.xn + (size_t)slice * kSlice, (uint32_t)d.n_inner * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
   const int xrow = d.Bp * 4;
+  // the row maxima M[node][example] go out beside the value tiles: the backward walk and the statistics
+  // kernel scale by exactly these numbers (lanes 16..63 hold copies: their stores fall outside the buffer)
+  const __amdgpu_buffer_rsrc_t rM =
+      make_rsrc(d.M + (size_t)slice * kSlice, (uint32_t)(d.n_inner + 1) * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
+  const uint32_t vm = lane < 16 ? vx : 0x7ffffff0u;
 
   LeanChunk sc;
   lean_refill(fields, stride, wave, lane, 0, sc);
@@ -137,6 +143,8 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
   Tile<K> o_prev;   // the value tile of the previous step, stored at the top of the next one
   tile_zero<K>(o_prev);
   int store_prev = d.n_inner * (int)d.tile_stride;
+  float m_prev = 0.f;
+  int mrow_prev = d.n_inner * xrow;
 
   // the schedule is consumed in chunks of kLeanChunk steps (a chunk's registers also serve
   // the two steps of look-ahead past its end)
@@ -148,6 +156,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     if (a3 >= 0) tile_add<K>(z, P3);
     // the previous step's value tile goes out now
     lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_prev), rM, (int)vm, mrow_prev, kStreamStore);
     // (2) request the leaf rows of step s+1 and the categories of step s+2
     {
       // (the categories first: everything that later waits for a leaf row then covers them)
@@ -181,6 +190,8 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);   // the block of step s+2, same registers
     o_prev = o;
     store_prev = lean_get(sc, kLNode, s) * (int)d.tile_stride;
+    m_prev = m;
+    mrow_prev = lean_get(sc, kLNode, s) * xrow;
     lds_tile_store<K>(lds, (int)(slots & 0xffu), lane, o);
     if (lean_get(sc, kLFlags, s) & 1) ll = o.v[0][0];
     lean_barrier();
@@ -198,12 +209,21 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     }
   }
   lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+  __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_prev), rM, (int)vm, mrow_prev, kStreamStore);
   if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
 }
 
 // ---- backward -----------------------------------------------------------------------------
-// kHeads: multi-head circuit, whose head kernel has left the root's ratio tile in memory (a
-// build of its own: the extra load in the root branch costs the single-head walk 5%).
+// What travels down the tree through LDS is not the flow of a child's sum nodes but already their
+// ratio tile R_c = F_c / S_c, built by the parent: with t = W_v^T R_v, F_c = G_v = exp(Z_v - M_v) .* t
+// and S_c = exp(O_c - M_c),
+//   R_c[j] = t[j] * exp((Z_v[j] - O_c[j]) + (M_c - M_v)),
+// where Z_v - O_c is the sum of v's OTHER operands (own leaf row, leaf children, further inner
+// children): the child's own values cancel, so a node never reads its own value tile, and the
+// exponent is formed from small numbers (M_c - M_v is exact when the two lie within a factor of
+// two).  M are the row maxima the forward walk stored.  A state the child gives probability zero
+// (O_c = -inf) has flow 0 and keeps ratio 0.  A node without inner children only stores its tile.
+// kHeads: multi-head circuit, whose head kernel has left the root's ratio tile in memory.
 template <int K, bool kHeads>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps) {
@@ -221,78 +241,126 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
   const __amdgpu_buffer_rsrc_t rL = make_rsrc(d.leaf, (uint32_t)d.V * d.leaf_stride);
   const __amdgpu_buffer_rsrc_t rX =
       make_rsrc(d.xn + (size_t)slice * kSlice, (uint32_t)d.n_inner * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
+  const __amdgpu_buffer_rsrc_t rM =
+      make_rsrc(d.M + (size_t)slice * kSlice, (uint32_t)(d.n_inner + 1) * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
   const int xrow = d.Bp * 4;
 
-  // a child operand: value tile of an inner child, or leaf row of a leaf child
-  auto child_load = [&](int c, uint32_t xpack, Tile<K>& t) {
-    if (c & 1) lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), c & ~7, t);
-    else lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride, t);
+  // a child operand: value tile (and row maxima) of an inner child, or leaf row of a leaf child
+  auto child_load = [&](int c, uint32_t xpack, Tile<K>& t, float& mc) {
+    if (c & 1) {
+      lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), c & ~7, t);
+    } else {
+      lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride, t);
+      mc = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, (c >> 3) * xrow, 0));
+    }
   };
+  auto is_inner = [](int c) { return c >= 0 && !(c & 1); };
 
   LeanChunk sc;
   lean_refill(fields, stride, wave, lane, 0, sc);
-  Tile<K> P0, OV, C1, C2, C3;
+  Tile<K> P0, C1, C2, C3;
   WTile<K> wA, wB;
   uint32_t xs;
   int c1, c2, c3;
+  float mv, m1 = 0.f, m2 = 0.f, m3 = 0.f;
   {
     const uint32_t x0 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0);
     xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 1) * xrow, 0);
+    mv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0));
     lean_row_load<K>(rL, lean_row_off<K>(x0, 0, vleaf), lean_get(sc, kLA0, 0), P0);
-    lean_tile_load<K>(rO, vtile, lean_get(sc, kLNode, 0) * (int)d.tile_stride, OV);
     c1 = lean_get(sc, kLA1, 0); c2 = lean_get(sc, kLA2, 0); c3 = lean_get(sc, kLA3, 0);
-    if (c1 >= 0) child_load(c1, x0, C1);
-    if (c2 >= 0) child_load(c2, x0, C2);
-    if (c3 >= 0) child_load(c3, x0, C3);
-    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 0), wA);
-    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
+    if (c1 >= 0) child_load(c1, x0, C1, m1);
+    if (c2 >= 0) child_load(c2, x0, C2, m2);
+    if (c3 >= 0) child_load(c3, x0, C3, m3);
+    // (a node without inner children has no use for its parameter block)
+    if (is_inner(c1)) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 0), wA);
+    if (is_inner(lean_get(sc, kLA1, 1))) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
   }
 
-  auto step = [&](const int s, WTile<K>& w) {
-    // (1) E_v (unnormalised) and the factor 1/S_v = exp(m - O_v) from the landed operands
-    Tile<K> e = P0;
-    if (c1 >= 0) tile_add<K>(e, C1);
-    if (c2 >= 0) tile_add<K>(e, C2);
-    if (c3 >= 0) tile_add<K>(e, C3);
-    const float m = tile_rowmax<K>(e);
-    Tile<K> sinv;
+  // exponent tile of inner child `own` among the landed operands: the other operands plus M_c - M_v,
+  // in base-2 units; -inf where the child's own value is -inf
+  auto exponent = [&](const Tile<K>& own, float mc, bool has_a, const Tile<K>& a, bool has_b, const Tile<K>& b, Tile<K>& x) {
+    const float dm = (mc - mv) * kLog2e;
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)   // capped: a state (or a whole example) of probability zero has flow 0, not 0 * inf
-        sinv.v[kt][i] = fminf(__builtin_amdgcn_exp2f(fmaf(OV.v[kt][i], -kLog2e, m * kLog2e)), kFlowRatioCap);
+      for (int i = 0; i < 4; ++i) {
+        float rest = P0.v[kt][i];
+        if (has_a) rest += a.v[kt][i];
+        if (has_b) rest += b.v[kt][i];
+        x.v[kt][i] = own.v[kt][i] == -INFINITY ? -INFINITY : fmaf(rest, kLog2e, dm);
+      }
+  };
+
+  auto step = [&](const int s, WTile<K>& w) {
+    // (1) from the landed operands: the exponent tiles of the inner children (they come first).  The first
+    // stays in registers; a second and third wait in the LDS slots their ratio tiles will take.
+    const bool in1 = is_inner(c1), in2 = is_inner(c2), in3 = is_inner(c3);
+    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
+    Tile<K> X1;
+    if (in1) exponent(C1, m1, c2 >= 0, C2, c3 >= 0, C3, X1);
+    if (in2) {
+      Tile<K> x;
+      exponent(C2, m2, true, C1, c3 >= 0, C3, x);
+      lds_tile_store<K>(lds, (int)((slots >> 16) & 0xffu), lane, x);
+    }
+    if (in3) {
+      Tile<K> x;
+      exponent(C3, m3, true, C1, true, C2, x);
+      lds_tile_store<K>(lds, (int)((slots >> 24) & 0xffu), lane, x);
+    }
+    const float mroot = mv;
     // (2) request the operands of step s+1 and the categories of step s+2
     {
       const uint32_t xc = xs;
       xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, s + 2) * xrow, 0);
+      mv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, lean_get(sc, kLNode, s + 1) * xrow, 0));
       lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), lean_get(sc, kLA0, s + 1), P0);
-      lean_tile_load<K>(rO, vtile, lean_get(sc, kLNode, s + 1) * (int)d.tile_stride, OV);
       c1 = lean_get(sc, kLA1, s + 1); c2 = lean_get(sc, kLA2, s + 1); c3 = lean_get(sc, kLA3, s + 1);
-      if (c1 >= 0) child_load(c1, xc, C1);
-      if (c2 >= 0) child_load(c2, xc, C2);
-      if (c3 >= 0) child_load(c3, xc, C3);
+      if (c1 >= 0) child_load(c1, xc, C1, m1);
+      if (c2 >= 0) child_load(c2, xc, C2, m2);
+      if (c3 >= 0) child_load(c3, xc, C3, m3);
     }
-    // (3) R_v = F_v / S_v, G_v = E_v .* (R_v W_v)
-    tile_exp_sub<K>(e, m);
-    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
-    Tile<K> r, t;
-    lds_tile_load<K>(lds, (int)((slots >> 8) & 0xffu), lane, r);
-#pragma unroll
-    for (int kt = 0; kt < K / 16; ++kt) r.v[kt] *= sinv.v[kt];
+    // (3) this node's ratio tile: left in LDS by the parent
+    Tile<K> r;
+    lds_tile_load<K>(lds, (int)(slots & 0xffu), lane, r);
     const int fl = lean_get(sc, kLFlags, s);
     if (kHeads && (fl & 2)) {   // multi-head circuit: the head kernel has left the root's ratio tile in memory
       lean_tile_load<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
-    } else if (fl & 1) {   // flow 1 into the single root sum node of every live example
-      const float r00 = (lane < 16 && bcol < d.B) ? sinv.v[0][0] : 0.f;
+    } else if (fl & 1) {   // flow 1 into the single root sum node of every live example: R = 1 / S = exp(M - O)
+      const float o00 = __builtin_bit_cast(
+          float, __builtin_amdgcn_raw_buffer_load_b32(rO, (int)vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, 0));
+      const float r00 = (lane < 16 && bcol < d.B)
+                            ? fminf(__builtin_amdgcn_exp2f(fmaf(o00, -kLog2e, mroot * kLog2e)), kFlowRatioCap) : 0.f;
       tile_zero<K>(r);
       r.v[0][0] = r00;
     }
     lean_tile_store<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
-    contract<K>(w, r, t);
-    lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);
+    // (4) the inner children's ratio tiles
+    if (in1) {
+      Tile<K> t;
+      contract<K>(w, r, t);
+      auto emit = [&](const Tile<K>& x, uint32_t slot) {
+        Tile<K> rc;
 #pragma unroll
-    for (int kt = 0; kt < K / 16; ++kt) t.v[kt] *= e.v[kt];
-    lds_tile_store<K>(lds, (int)(slots & 0xffu), lane, t);
+        for (int kt = 0; kt < K / 16; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) rc.v[kt][i] = t.v[kt][i] * fminf(__builtin_amdgcn_exp2f(x.v[kt][i]), kFlowRatioCap);
+        lds_tile_store<K>(lds, (int)slot, lane, rc);
+      };
+      emit(X1, (slots >> 8) & 0xffu);
+      if (in2) {
+        Tile<K> x;
+        lds_tile_load<K>(lds, (int)((slots >> 16) & 0xffu), lane, x);
+        emit(x, (slots >> 16) & 0xffu);
+      }
+      if (in3) {
+        Tile<K> x;
+        lds_tile_load<K>(lds, (int)((slots >> 24) & 0xffu), lane, x);
+        emit(x, (slots >> 24) & 0xffu);
+      }
+    }
+    if (is_inner(lean_get(sc, kLA1, s + 2))) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);
     lean_barrier();
   };
   for (int base = 0; base < n_steps; base += kLeanChunk) {
@@ -311,18 +379,22 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
 // with at most three children, written like the lean walks: per-operand descriptors built once
 // (the node is fixed, only the slice moves), typed operands behind scalar branches, every
 // register reloaded right after its last use, the waves' partial edge-flow blocks combined by
-// a plain LDS sum.  A node with leaf children runs one pass over the batch per variable it has
-// to histogram (the LDS holds one histogram): pass 0 does all the arithmetic and leaves the
-// child-flow tiles G where it read R from; the passes of the leaf children re-read G only.
+// a plain LDS sum.  The LDS holds up to `nh_pass` histograms (two where they fit: a node's own
+// variable and its first leaf child then need one pass over the batch).  Pass 0 does all the
+// arithmetic; a node with more variables than that leaves the child-flow tiles G where it read R
+// from, and further passes re-read G only.
+//
+// LDS layouts, both without padding so that two histograms of 256 x 32 cells and sixteen pads fill
+// 160 KB exactly: histogram cell (category x, state j) sits in word x*K + (j ^ (x % K)) of its limb
+// (equal states of different categories spread over the banks); a wave's 16 x K transposition pad
+// rotates row r by 8*r floats (column reads of four rows then cover every bank twice).
 constexpr int kStatLeanWaves = 16;
 
 template <int K>
 __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     HcltDev d, const StatNode* __restrict__ nodes, float* __restrict__ edge_aggr, float* __restrict__ leaf_flow,
-    float rate, int hist_words, int limb, const int* __restrict__ flow_shift) {
+    float rate, int hist_words, int nh_pass, int limb, const int* __restrict__ flow_shift) {
   constexpr int KT = K / 16;
-  constexpr int LD = K + 16;   // row stride of the pad: conflict-free column reads
-  constexpr int HS = K + 1;    // row stride of a histogram: spreads equal states over banks
   extern __shared__ float smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -331,9 +403,9 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
   const StatNode* __restrict__ np = nodes + n;   // fields are read where needed (a local copy indexed by the pass would live in scratch)
   const int own_var = np->var, n_hist = np->n_hist;
   const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)g * 16, vx = (uint32_t)b * 4;
-  const int hist_sz = d.C * HS;
+  const int hist_sz = d.C * K;           // words per limb; a histogram is two limbs
   unsigned* hist = reinterpret_cast<unsigned*>(smem);
-  float* pad = smem + hist_words + (size_t)wave * (kSlice * LD);
+  float* pad = smem + hist_words + (size_t)wave * (kSlice * K);
   // flows lie in [0, 2^shift]: 1 per example in a single-head circuit, the largest total head
   // mask of an example (found on the device by the head kernel) in a multi-head one
   const int shift = flow_shift ? __builtin_amdgcn_readfirstlane(*flow_shift) : 0;
@@ -341,6 +413,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 
   const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + (size_t)n * d.tile_stride, d.tile_stride);
   const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);
+  const __amdgpu_buffer_rsrc_t rM = make_rsrc(d.M + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);   // row maxima of the forward walk
   const __amdgpu_buffer_rsrc_t rL0 = make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)own_var * d.leaf_stride, d.leaf_stride);
   auto child_rsrc = [&](int c) {
     return (c & 1) ? make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)(c >> 3) * d.leaf_stride, d.leaf_stride)
@@ -361,10 +434,11 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 #pragma unroll
     for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  // fixed-point limbs of this lane's K/4 flows (clamped to [0, 2^shift]) into row x of the histogram
-  auto histogram = [&](const Tile<K>& t, uint32_t xpack, int sel) {
+  // fixed-point limbs of this lane's K/4 flows (clamped to [0, 2^shift]) into row x of histogram h
+  auto histogram = [&](const Tile<K>& t, uint32_t xpack, int sel, int h) {
     const uint32_t x = (xpack >> (8 * sel)) & 0xffu;
-    unsigned* hrow = hist + x * HS + 4 * g;
+    unsigned* hrow = hist + (size_t)h * 2 * hist_sz + x * K;
+    const uint32_t sw = x & (K - 1);
 #pragma unroll
     for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -372,24 +446,34 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
         const float v = __builtin_amdgcn_fmed3f(t.v[kt][i] * scale_in, 0.f, scale);
         const unsigned hi = (unsigned)v;
         const unsigned lo = (unsigned)(__builtin_amdgcn_fractf(v) * scale);
-        __hip_atomic_fetch_add(&hrow[kt * 16 + i], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        __hip_atomic_fetch_add(&hrow[hist_sz + kt * 16 + i], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        const uint32_t col = (uint32_t)(kt * 16 + 4 * g + i) ^ sw;
+        __hip_atomic_fetch_add(&hrow[col], hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        __hip_atomic_fetch_add(&hrow[hist_sz + col], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
   };
+  // pad positions: this lane's float4 of example row b (states kt*16 + 4g ..), and the element
+  // (example 4q + g, state kt*16 + b) of the transposed read
+  auto pad_w = [&](int kt) { return b * K + ((kt * 16 + 4 * g + 8 * b) & (K - 1)); };
+  auto pad_r = [&](int q, int kt) { return (4 * q + g) * K + ((kt * 16 + b + 8 * g) & (K - 1)); };
 
   const int last = d.nslices - 1;
-  for (int pass = 0; pass < n_hist; ++pass) {
-    for (int i = threadIdx.x; i < 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
+  const int n_pass = (n_hist + nh_pass - 1) / nh_pass;
+  for (int pass = 0; pass < n_pass; ++pass) {
+    const int h0 = pass * nh_pass, nh = min(nh_pass, n_hist - h0);   // this pass fills histograms of variables h0 .. h0+nh-1
+    for (int i = threadIdx.x; i < nh * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
     __syncthreads();
     if (pass == 0) {
     // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
     // repeated loads), categories of the second
     Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
     uint32_t xc, xn;
+    float mc, mn;            // the slices' row maxima, requested like their categories
     {
       const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
       xc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sa * (kSlice * 4), 0);
       xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sb * (kSlice * 4), 0);
+      mc = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, sa * (kSlice * 4), 0));
+      mn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, sb * (kSlice * 4), 0));
       const uint32_t so = (uint32_t)sa * (kSlice * K * 4);
       lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
       if (c1 >= 0) child_load(rC1, c1, xc, so, C1);
@@ -411,11 +495,13 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
       }
       xc = xn;
       xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
+      const float m = mc;   // the scale the backward walk built R with
+      mc = mn;
+      mn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, s2 * (kSlice * 4), 0));
       lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
       if (c1 >= 0) child_load(rC1, c1, xc, so1, C1);
       if (c2 >= 0) child_load(rC2, c2, xc, so1, C2);
       // (2) E, the edge flows, then G = E .* (R W)
-      const float m = tile_rowmax<K>(e);
       tile_exp_sub<K>(e, m);
       {
         // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
@@ -423,19 +509,19 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
         // accesses execute in order, so the pad needs no barrier between its phases.
         float ra[4][KT];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = R.v[kt];
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = R.v[kt];
 #pragma unroll
         for (int q = 0; q < 4; ++q)
 #pragma unroll
-          for (int kt = 0; kt < KT; ++kt) ra[q][kt] = pad[(4 * q + g) * LD + kt * 16 + b];
+          for (int kt = 0; kt < KT; ++kt) ra[q][kt] = pad[pad_r(q, kt)];
         __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[b * LD + kt * 16 + 4 * g]) = e.v[kt];
+        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = e.v[kt];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float eb[KT];
 #pragma unroll
-          for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[(4 * q + g) * LD + jt * 16 + b];
+          for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[pad_r(q, jt)];
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
@@ -449,18 +535,21 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 #pragma unroll
       for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
       lean_tile_load<K>(rR, vtile, (int)so1, R);   // next slice's ratios, after the last use of these
-      if (n_hist > 1) {
-        // the later passes (one per leaf child) only need G: it replaces the tile of R just consumed
+      if (n_pass > 1) {
+        // the later passes only need G: it replaces the tile of R just consumed
 #pragma unroll
         for (int kt = 0; kt < KT; ++kt)
           __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), rR, (int)(vtile + kt * 1024),
                                                  (int)((uint32_t)s0 * (kSlice * K * 4)), 0);
       }
-      // (3) histogram
-      if (s0 * kSlice + b < d.B) histogram(t, xh, 0);
+      // (3) histograms: the node's own variable, and its first leaf child if the LDS holds two
+      if (s0 * kSlice + b < d.B) {
+        histogram(t, xh, 0, 0);
+        if (nh > 1) histogram(t, xh, 1, 1);
+      }
     }
     } else {
-      // leaf child `pass`: G comes back from where pass 0 left it; only the categories differ
+      // further leaf children: G comes back from where pass 0 left it; only the categories differ
       Tile<K> T;
       uint32_t xc, xn;
       {
@@ -474,19 +563,26 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
         const uint32_t xh = xc;
         xc = xn;
         xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
-        if (s0 * kSlice + b < d.B) histogram(T, xh, pass);
+        if (s0 * kSlice + b < d.B) {
+          histogram(T, xh, h0, 0);
+          if (nh > 1) histogram(T, xh, h0 + 1, 1);
+        }
         lean_tile_load<K>(rR, vtile, (int)((uint32_t)s1 * (kSlice * K * 4)), T);
       }
     }
     __syncthreads();
     {
       const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
-      float* dst = leaf_flow + (size_t)np->hvar[pass] * d.C * K;
-      for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
-        const int c = i / K, j = i % K;
-        const float val = (float)hist[c * HS + j] * hi_inv + (float)hist[hist_sz + c * HS + j] * lo_inv;
-        const float old = rate != 0.f ? rate * dst[i] : 0.f;
-        dst[i] = old + val;
+      for (int h = 0; h < nh; ++h) {
+        float* dst = leaf_flow + (size_t)np->hvar[h0 + h] * d.C * K;
+        const unsigned* hh = hist + (size_t)h * 2 * hist_sz;
+        for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
+          const int c = i / K, j = i % K;
+          const int cell = c * K + (j ^ (c & (K - 1)));
+          const float val = (float)hh[cell] * hi_inv + (float)hh[hist_sz + cell] * lo_inv;
+          const float old = rate != 0.f ? rate * dst[i] : 0.f;
+          dst[i] = old + val;
+        }
       }
     }
     __syncthreads();
