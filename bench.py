@@ -25,20 +25,21 @@ KERNEL_NAMES = {"forward": "hclt_forward_lean_kernel<%d>", "backward": "hclt_bac
 
 def algorithmic_bytes(n_int, V, K, C, B):
     """Bytes the algorithm has to move per launch, per kernel.  A node-value or flow vector
-    is K*4 bytes per (tree node, example); the whole step needs six of them per tree node:
-    the value vector written and read as a child going up, read again as a child and as a
-    parent going down, the flow vector written once and read once.  They are booked where
-    this implementation's kernels touch them: forward 2 (value written, value read as a
-    child), backward 3 (value as child, value as parent, flow written), statistics 1 (flow
-    read).  Each kernel also reads the batch (V*B bytes), the sum parameters (4 bytes per
+    is K*4 bytes per (tree node, example); the whole step is priced at six of them per tree
+    node (value written and read as a child going up, read twice going down, flow written
+    once and read once).  They are booked where this implementation's kernels touch them, two
+    per kernel: forward (value written, value read as a child -- served from LDS), backward
+    (children's values read, ratio vector written: a node's own value is not read going
+    down), statistics (ratio vector read, children's values read to rebuild the edge
+    weights).  Each kernel also reads the batch (V*B bytes), the sum parameters (4 bytes per
     edge) and the leaf tables (4*V*K*C); statistics additionally writes both accumulators."""
     vec = K * 4 * B
     n_sum_edges = (n_int - 1) * K * K + K
     theta = 4 * n_sum_edges
     leaf = 4 * V * K * C
     fwd = n_int * 2 * vec + V * B + theta + leaf
-    bwd = n_int * 3 * vec + V * B + theta + leaf
-    stats = n_int * 1 * vec + V * B + 2 * theta + 2 * leaf
+    bwd = n_int * 2 * vec + V * B + theta + leaf
+    stats = n_int * 2 * vec + V * B + 2 * theta + 2 * leaf
     return dict(forward=fwd, backward=bwd, statistics=stats,
                 step=n_int * 6 * vec + V * B + 3 * theta + 5 * leaf)
 
