@@ -78,11 +78,22 @@ def test_full_batch_step_properties_and_oracle_subset(c3, oracle):
     rel = lambda a, b: (np.abs(np.exp(np.asarray(a, np.float64)) - np.exp(b)) / np.exp(b)).max()
     e_gpu = max(rel(th[v][:b.shape[0]], b) for v, b in th64.items())
     e_f32 = max(rel(th32[v], b) for v, b in th64.items())
-    print(f"sum parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}")
+    e_gpu32 = max(rel(th[v][:b.shape[0]], th32[v].astype(np.float64)) for v, b in th64.items())
+    print(f"sum parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}, "
+          f"library vs float32 oracle {e_gpu32:.2e}")
     assert e_gpu < max(PARAM_RTOL, 2 * e_f32)
+    # against the float32 oracle -- the reference's own arithmetic -- the two float32 results may be
+    # apart by the sum of their distances from the exact one and no more
+    assert e_gpu32 < max(PARAM_RTOL, e_gpu + e_f32)
     e_gpu, e_f32 = rel(lf_new, lf64), rel(lf32, lf64)
-    print(f"leaf parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}")
+    e_gpu32 = rel(lf_new, lf32.astype(np.float64))
+    print(f"leaf parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}, "
+          f"library vs float32 oracle {e_gpu32:.2e}")
     assert e_gpu < max(PARAM_RTOL, 2 * e_f32)
+    assert e_gpu32 < max(PARAM_RTOL, e_gpu + e_f32)
+    # the per-example log-likelihoods of the step against the float32 oracle, at the bar itself
+    ll32 = O.forward(fc, cfg["data"][:sub])[-1]
+    assert (np.abs(llb.cpu().numpy() - ll32) / np.abs(ll32)).max() < LL_RTOL
     # (log-values near the root are ~ -14000, where one float32 ulp is 1e-3: a sizeable share of
     # the flows carries that error in any float32 implementation)
     frac = lambda a: (np.abs(np.exp(np.asarray(a, np.float64)) - np.exp(lf64)) / np.exp(lf64) > PARAM_RTOL).mean()
@@ -120,6 +131,33 @@ def test_kld_on_the_benchmark_circuit(c3, oracle):
     n_sum = bpc.num_inner_params()
     # the gradient with respect to q's sum log-parameters is -g * p1 <= 0
     assert (g2[:n_sum] <= 0).all()
+    # both gradient vectors, all 27.7 M entries, against the float64 oracle at the tolerance of the
+    # small circuits (1e-4 of the largest entry).  The oracle works on the direct flat form, whose
+    # numbering is its own: a third circuit whose parameters are their own block coordinates tells
+    # where every block entry sits in the parameter vector.
+    V, K, C = cfg["V"], cfg["K"], cfg["C"]
+    ids = P.hclt_from_clt(cfg["parent"], C, K)
+    ch, root = O.clt_children(cfg["parent"])
+    inner = [v for v in range(V) if ch[v]]
+    code = np.zeros((V, K, K), np.float32)
+    for r, v in enumerate(inner):
+        code[v] = (r * K * K + np.arange(K * K)).reshape(K, K)
+    leaf_code = np.broadcast_to((np.arange(V * K, dtype=np.float32)).reshape(V, K, 1), (V, K, C))
+    ids.set_params(code, np.ascontiguousarray(leaf_code))
+    where = P.vectorize_parameters(ids)
+    sum_at = where[:n_sum].astype(np.int64)                      # -> inner rank * K*K + k*K + j
+    leaf_at = where[n_sum::C].astype(np.int64)                   # -> v*K + j of every input node, in vector order
+    assert len(np.unique(sum_at)) == n_sum and len(np.unique(leaf_at)) == V * K
+    _, ek = O.kld(f1, f2, double=True)
+    _, eg1, eg2, lg1, lg2 = O.kld_backward(f1, f2, ek, double=True)
+    for got_vec, eg, lg in ((g1, eg1, lg1), (g2, eg2, lg2)):
+        blocks = np.zeros((len(inner), K, K))
+        for r, v in enumerate(inner):
+            nk = len(f1.meta["sum_node"][v])
+            e0 = f1.meta["edge_of"][v]
+            blocks[r, :nk] = eg[e0:e0 + nk * K].reshape(nk, K)
+        want_vec = np.concatenate([blocks.reshape(-1)[sum_at], lg.reshape(V * K, C)[leaf_at].reshape(-1)])
+        assert np.abs(got_vec - want_vec).max() < 1e-4 * np.abs(want_vec).max()
 
 
 def test_sampling_on_the_benchmark_circuit(c3, oracle):

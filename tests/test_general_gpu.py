@@ -272,6 +272,94 @@ def test_config_patch_circuit_with_128_heads_and_top_hclt(gpu, oracle):
     assert lls[2] > lls[1] > lls[0]
 
 
+def test_patch_circuit_on_the_block_engine_at_its_real_shape(gpu, oracle):
+    """The patch circuit of the patch-clustered configuration as the benchmark runs it: built from its
+    tree with pcm_hclt_create_multihead (body on the walk kernels, 128 heads in the head kernels), 192
+    variables, K = 32, 256 categories, batch 1024.  Against the layered engine on the equivalent
+    description over the whole batch (per-head values, mixtures and EM updates under a one-hot and a soft
+    head mask) and against the oracle on a subset."""
+    torch, P = gpu
+    O = oracle
+    import sys
+    from pcmi355 import workloads
+    from pcmi355._lib import lib, check
+    from helpers import multihead_hclt, rel_err
+    sys.setrecursionlimit(20000)
+    V, K, C, H, B = 192, 32, 256, 128, 1024
+    rng = np.random.default_rng(1004)
+    data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
+    parent = workloads.chow_liu_parent(data)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    gen = _compile(P, heads, V, C, heads=H)
+    blk = P.multihead_hclt_from_clt(parent, C, K, H)
+    assert blk.size("walk_kernels") in (1, 2)
+    pv = P.vectorize_parameters(gen)
+    P.update_parameters(blk, pv)
+    np.testing.assert_array_equal(P.vectorize_parameters(blk), pv)
+    d = torch.from_numpy(data).cuda()
+    ll_g = P.loglikelihoods(gen, d).cpu().numpy()
+    ll_b = P.loglikelihoods(blk, d).cpu().numpy()
+    assert ll_b.shape == (B, H) and rel_err(ll_b, ll_g).max() < LL_RTOL
+    sub = 24
+    fc = O.bits_compile(O.summate(*heads), C, V)
+    root_ids = (blk.table("heads") - 1).astype(np.int64)
+    mars = O.forward(fc, data[:sub])
+    assert rel_err(ll_b[:sub], mars[root_ids].T).max() < LL_RTOL
+    cluster = rng.integers(0, H, size=B)
+    for soft in (False, True):
+        mask = np.zeros((B, H), np.float32)
+        mask[np.arange(B), cluster] = 1.0
+        if soft:
+            mask = (mask + rng.random((B, H)).astype(np.float32) * (rng.random((B, H)) < 0.1)).astype(np.float32)
+        hm = torch.from_numpy(mask).cuda()
+        P.update_parameters(gen, pv)
+        P.update_parameters(blk, pv)
+        mix_g = P.probs_flows_circuit(gen, d, head_mask=hm).cpu().numpy()
+        mix_b = P.probs_flows_circuit(blk, d, head_mask=hm).cpu().numpy()
+        assert rel_err(mix_b, mix_g).max() < LL_RTOL
+        with np.errstate(divide="ignore"):
+            want = np.logaddexp.reduce(mars[root_ids].astype(np.float64) + np.log(mask[:sub].T.astype(np.float64)), axis=0) \
+                - np.log(mask[:sub].sum(axis=1, dtype=np.float64))
+        assert rel_err(mix_b[:sub], want).max() < LL_RTOL
+        check(lib.pcm_em_update(gen.handle, 0.1, 0.9))
+        check(lib.pcm_em_update(blk.handle, 0.1, 0.9))
+        a, b = np.exp(P.vectorize_parameters(gen).astype(np.float64)), np.exp(P.vectorize_parameters(blk).astype(np.float64))
+        assert (np.abs(a - b) / np.maximum(a, 1e-6)).max() < 2e-4          # two float32 engines, as in the random-shape test
+    # the same EM step on the subset against the oracle (one-hot mask)
+    P.update_parameters(blk, pv)
+    mask = np.zeros((sub, H), np.float32)
+    mask[np.arange(sub), cluster[:sub]] = 1.0
+    P.probs_flows_circuit(blk, d[:sub].contiguous(), head_mask=torch.from_numpy(mask).cuda())
+    check(lib.pcm_em_update(blk.handle, 0.1, 0.9))
+    skip = (fc.edge_parent() == fc.n_nodes - 1).astype(np.uint8)
+
+    def oracle_step(double):
+        m = O.forward(fc, data[:sub], double=double)
+        fl, ea = O.backward(fc, m, skip=skip, root_ids=root_ids.astype(np.int32), root_flow=np.ascontiguousarray(mask.T),
+                            double=double)
+        lf = O.input_flows(fc, data[:sub], fl, double=double)
+        logp_new, leaf_new = O.em_update(fc, ea, lf, 0.1, 0.9, double=double)
+        ref = fc.copy()
+        ref.logp, ref.leaf_logp = logp_new, leaf_new
+        return np.exp(ref.vectorize_parameters().astype(np.float64)) if not double else \
+            np.exp(np.concatenate([logp_new[ref.sum_param_edges()]] +
+                                  [leaf_new[ref.in_off[n]:ref.in_off[n] + C] for n in ref.input_nodes()]))
+
+    want64, want32 = oracle_step(True), oracle_step(False)
+    n_real = len(pv)
+    # (the oracle's circuit has the fake root's H edges as extra sum parameters at the end of the sum block)
+    ns = blk.num_inner_params()
+    got = np.exp(P.vectorize_parameters(blk).astype(np.float64))
+    # 24 examples leave most edges little more than their pseudocount share, and the body is 60 levels deep:
+    # where the float32 oracle (the reference's arithmetic) cannot hold 1e-4 against float64, the library
+    # may be as far from the exact result as twice the float32 oracle is
+    for lo_g, hi_g, lo_w, hi_w in ((0, ns, 0, ns), (ns, n_real, len(want64) - (n_real - ns), len(want64))):
+        e_gpu = rel_err(got[lo_g:hi_g], want64[lo_w:hi_w]).max()
+        e_f32 = rel_err(want32[lo_w:hi_w], want64[lo_w:hi_w]).max()
+        print(f"patch circuit, block engine vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}")
+        assert e_gpu < max(PARAM_RTOL, 2 * e_f32)
+
+
 def test_hclt_general_form_matches_block_engine(gpu, oracle):
     """The same HCLT through both engines: LL, parameter vector after an EM step."""
     torch, P = gpu
