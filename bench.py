@@ -188,14 +188,34 @@ def secondary(args):
         soft_out = torch.empty((B, V, C), device="cuda")
         t_soft = _timed(torch, lambda: check(lib.pcm_sample_soft(p.handle, node_noise.data_ptr(), 0.5, B, soft_out.data_ptr())),
                         max(1, args.steps // 4), 1)
-        del soft_out
+        del soft_out, node_noise, leaf_noise
+        # the same queries on a matrix of 64 parameter rows (one parameter vector per example, as the
+        # variational models call them): rows of p's parameters against rows of q's
+        R = 64
+        n_par = p.num_parameters()
+        pv = torch.from_numpy(P.vectorize_parameters(p)).cuda()
+        qv = torch.from_numpy(P.vectorize_parameters(q)).cuda()
+        m1 = pv.repeat(R, 1)
+        m2 = qv.repeat(R, 1)
+        m1 += 0.01 * torch.randn((R, 1), device="cuda", generator=gen)      # rows differ (values only matter for the clock)
+        klr = P.kld(p, m1, m2)
+        t_kld_rows = _timed(torch, lambda: P.kld(p, m1, m2), max(1, args.steps // 4), 1)
+        t_grad_rows = _timed(torch, lambda: P.kld_backward(p, m1, m2), max(1, args.steps // 4), 1)
+        soft_rows = None
+        t_soft_rows = _timed(torch, lambda: P.gumbel_sample_rows(p, m1, temperature=1.0), max(1, args.steps // 4), 1)
+        rows_bytes = {"kld_rows": 2 * 4 * R * n_par, "kld_backward_rows": 5 * 4 * R * n_par}
+        del m1, m2, klr
         dt = t_samp
         algo = 4 * B * (n_inner * K + V * C)                           # the noise tensors, read once
         out.update(metric="samples/sec Gumbel-max from supplied noise, 3072-var HCLT K=32",
                    value=B / t_samp, unit="samples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B},
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
-                               "sample": t_samp * 1e3, "gumbel_sample_relaxed_T0.5": t_soft * 1e3})
+                               "sample": t_samp * 1e3, "gumbel_sample_relaxed_T0.5": t_soft * 1e3,
+                               "kld_rows_R64": t_kld_rows * 1e3, "kld_backward_rows_R64": t_grad_rows * 1e3,
+                               "gumbel_sample_rows_R64_no_gumbel": t_soft_rows * 1e3},
+                   rows_gbs={"kld_rows_R64": rows_bytes["kld_rows"] / t_kld_rows / 1e9,
+                             "kld_backward_rows_R64": rows_bytes["kld_backward_rows"] / t_grad_rows / 1e9})
     elif args.workload == "c4_patch_x8_streams":
         # eight independent patch circuits (C4 has 64), each queued on one of four streams: the layered engine's
         # per-layer launches are small, so circuits overlap on the device

@@ -227,6 +227,35 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
                     float* d_out);
 
 /*
+ * The same three queries on a MATRIX of parameter rows -- one structure, `rows` parameter vectors, all
+ * rows in one pass -- as the reference's own signatures have them: `kld(mbpc, params1, params2;
+ * norm_params)` (src/queries/kld.jl:164-206), `kld_backward(mbpc, params1, params2; norm_params,
+ * grad_wrt_logparams = true)` (:593-649) and `gumbel_sample(mbpc, params, num_vars, par_buffer_size;
+ * temperature, no_gumbel, norm_params)` (src/queries/sample.jl:338-383), called with one row per example
+ * by src/utils/cuda_preallocation.jl:47-78, :189-203.  The circuit gives the structure only; its own
+ * parameters are not read.  Element (row r, parameter i) of a matrix is at d_x[r * stride_row + i *
+ * stride_param], parameters in pcm_vectorize_parameters order; Julia's column-major [rows, n] array is
+ * (1, rows), a row-major tensor (n, 1).  Unit stride along the parameters is the layout the kernels work
+ * in; anything else is re-laid-out on the way in and out.  norm_params != 0: the LEAF parameters are
+ * probabilities, not log-probabilities (src/nodes/fixable_categorical_dist.jl:182-186, :216-217;
+ * sample.jl:265-268); sum parameters are log-parameters either way, as in the reference.
+ *
+ * pcm_kld_rows: d_klds [rows] (device) receives klds[:, end].
+ * pcm_kld_backward_rows: d_grads1 / d_grads2 (device, the strides of the parameter matrices) receive the
+ * gradients with respect to the rows of params1 / params2; d_klds may be NULL.
+ * pcm_gumbel_sample_rows: d_noise is [rows][num sum parameters] (dense, one draw per sum edge) or NULL for
+ * no_gumbel = true; d_out [rows][num_vars][num_cats].
+ * All three queue their work on the circuit's stream and do not wait for it.  At most 65535 rows per call.
+ */
+int pcm_kld_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row, int64_t stride_param,
+                 int32_t rows, int32_t norm_params, float* d_klds);
+int pcm_kld_backward_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row,
+                          int64_t stride_param, int32_t rows, int32_t norm_params, float* d_grads1, float* d_grads2,
+                          float* d_klds);
+int pcm_gumbel_sample_rows(pcm_circuit* c, const float* d_params, int64_t stride_row, int64_t stride_param, int32_t rows,
+                           const float* d_noise, float temperature, int32_t norm_params, float* d_out);
+
+/*
  * Soft evidence: the same two queries with a three-dimensional data argument, as the reference
  * dispatches on `data isa CuArray{Float32,3}` (`init_mar!_with_reg_cat_kernel`
  * src/regularization/reg_likelihood.jl:51-91, `input_flows_circuit_with_reg_cat_kernel`

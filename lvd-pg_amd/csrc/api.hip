@@ -203,6 +203,27 @@ int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d
   return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });
 }
 
+int pcm_kld_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row, int64_t stride_param,
+                 int32_t rows, int32_t norm_params, float* d_klds) {
+  return guarded([&] { need(c)->kld_rows(d_params1, d_params2, stride_row, stride_param, rows, norm_params != 0, d_klds); });
+}
+
+int pcm_kld_backward_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row,
+                          int64_t stride_param, int32_t rows, int32_t norm_params, float* d_grads1, float* d_grads2,
+                          float* d_klds) {
+  return guarded([&] {
+    need(c)->kld_backward_rows(d_params1, d_params2, stride_row, stride_param, rows, norm_params != 0, d_grads1, d_grads2,
+                               d_klds);
+  });
+}
+
+int pcm_gumbel_sample_rows(pcm_circuit* c, const float* d_params, int64_t stride_row, int64_t stride_param, int32_t rows,
+                           const float* d_noise, float temperature, int32_t norm_params, float* d_out) {
+  return guarded([&] {
+    need(c)->gumbel_sample_rows(d_params, stride_row, stride_param, rows, d_noise, temperature, norm_params != 0, d_out);
+  });
+}
+
 int pcm_loglikelihoods_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var,
                             int64_t stride_cat, const int32_t* d_example_ids, int32_t batch, float* d_ll) {
   return guarded([&] {

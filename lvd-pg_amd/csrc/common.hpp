@@ -121,4 +121,11 @@ struct pcm_circuit {
   virtual void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) = 0;
   virtual void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
                          float b1, float b2, float eps, int t) = 0;
+  // queries on a matrix of parameter rows (element strides sr, sp), all rows in one pass
+  virtual void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                        float* d_out) = 0;
+  virtual void kld_backward_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows,
+                                 bool norm_params, float* d_g1, float* d_g2, float* d_klds) = 0;
+  virtual void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                  float temperature, bool norm_params, float* d_out) = 0;
 };

@@ -151,6 +151,19 @@ class HcltCircuit : public pcm_circuit {
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
                  float b2, float eps, int t) override;
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
+  // parameter-row queries run on the circuit's general form (its structure; the rows bring the parameters)
+  void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                float* d_out) override {
+    general_structure()->kld_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_out);
+  }
+  void kld_backward_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                         float* d_g1, float* d_g2, float* d_klds) override {
+    general_structure()->kld_backward_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_g1, d_g2, d_klds);
+  }
+  void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                          float temperature, bool norm_params, float* d_out) override {
+    general_structure()->gumbel_sample_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params, d_out);
+  }
 
   bool sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out);
   void set_block_params(const float* theta, const float* leaf);
@@ -233,6 +246,7 @@ class HcltCircuit : public pcm_circuit {
   std::unique_ptr<SparseCircuit> general_; // built on first use by the KL / sampling / Adam queries
   bool general_stale_ = true;
   SparseCircuit* general();
+  SparseCircuit* general_structure();   // the same object without bringing its parameters up to date
   // KL recursion on the block form
   DevBuf<int32_t> d_kl_up_, d_kl_down_;   // chain steps (KlItem records) bottom-up / top-down
   DevBuf<int32_t> d_kl_tabs_;             // parent of every inner node | h-giving node of every variable | input-node positions

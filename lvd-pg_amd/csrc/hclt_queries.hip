@@ -301,6 +301,15 @@ SparseCircuit* HcltCircuit::general() {
   return general_.get();
 }
 
+SparseCircuit* HcltCircuit::general_structure() {
+  if (!general_) {
+    general_.reset(new SparseCircuit(flat_));
+    general_stale_ = true;
+  }
+  general_->stream = stream;
+  return general_.get();
+}
+
 void HcltCircuit::pull_from_general() {
   std::vector<float> p((size_t)size(0));
   general_->vectorize(p.data(), (int64_t)p.size());

@@ -7,6 +7,8 @@
 // its result once -- no atomics on node values or flows.
 #pragma once
 
+#include <memory>
+
 #include "common.hpp"
 
 namespace pcm {
@@ -44,7 +46,7 @@ FlatCircuit flatten_dag(int32_t num_nodes, const uint8_t* node_type, const int32
 class SparseCircuit : public pcm_circuit {
  public:
   explicit SparseCircuit(FlatCircuit fc);
-  ~SparseCircuit() override {}
+  ~SparseCircuit() override;
 
   int64_t size(int what) const override;
   void index_table(int which, int64_t* out, int64_t n) const override;
@@ -65,6 +67,13 @@ class SparseCircuit : public pcm_circuit {
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
   void sample_soft_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
                               float temperature, int32_t batch, float* d_out);
+  void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                float* d_out) override;
+  void kld_backward_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                         float* d_g1, float* d_g2, float* d_klds) override;
+  void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                          float temperature, bool norm_params, float* d_out) override;
+  struct RowsState;   // tables and scratch of the parameter-row queries (param_rows.hip)
 
   void get_node_values(float* mars, float* flows, int64_t n);
   void get_aggregates(float* edge_aggr, int64_t n_edges, float* leaf_flow, int64_t n_leaf);
@@ -105,6 +114,9 @@ class SparseCircuit : public pcm_circuit {
   int flow_batch_ = 0;   // examples whose node flows d_flows_ holds (0: none)
   DevBuf<float> d_node_sums_;
 
+  std::shared_ptr<RowsState> rows_;   // (shared_ptr: the type is complete only in param_rows.hip)
+  RowsState& rows_state();
+  void kld_rows_forward(const float* p1, const float* p2, int rows, bool norm, bool with_edges);
   void ensure_batch(int batch);
   void ensure_var_tables();
   void run_forward(const BatchRef* b, const SoftRef* s);

@@ -198,29 +198,97 @@ def update_parameters(bpc, params):
     check(lib.pcm_update_parameters(bpc.handle, np_ptr(p), c_i64(len(p))))
 
 
-def kld(bpc_p, bpc_q):
-    """`kld(mbpc, params1, params2)` (src/queries/kld.jl:177-206), one parameter row:
-    the two parameter sets are the two circuits' own parameters."""
-    out = np.zeros(1, np.float32)
-    check(lib.pcm_kld(bpc_p.handle, bpc_q.handle, np_ptr(out)))
-    return float(out[0])
+def _rows_on_device(x, n, what):
+    """A parameter matrix [rows, n] as a float32 GPU tensor (host arrays are uploaded); returns
+    (tensor, was_host)."""
+    host = not isinstance(x, torch.Tensor)
+    t = torch.as_tensor(np.ascontiguousarray(x, np.float32) if host else x)
+    if t.dim() != 2 or t.shape[1] != n:
+        raise ValueError(f"{what} must be [rows, {n}], got {tuple(t.shape)}")
+    if t.dtype != torch.float32:
+        t = t.float()
+    return (t.cuda() if not t.is_cuda else t), host
 
 
-def kld_backward(bpc_p, bpc_q, device=False):
-    """`kld_backward(mbpc, params1, params2; grad_wrt_logparams = true)`
-    (src/queries/kld.jl:593-649) -> (grads1, grads2) in parameter-vector order: host numpy
-    vectors like the reference, or with device=True float32 tensors on the GPU (what
-    adam_step takes)."""
-    n = bpc_p.num_parameters()
-    if device:
-        g1 = torch.empty(n, dtype=torch.float32, device="cuda")
-        g2 = torch.empty(n, dtype=torch.float32, device="cuda")
-        check(lib.pcm_kld_backward_dev(bpc_p.handle, bpc_q.handle, g1.data_ptr(), g2.data_ptr(), c_i64(n)))
+def kld(mbpc, params1, params2=None, *, norm_params=False):
+    """`kld(mbpc, params1, params2; norm_params)` (src/queries/kld.jl:164-206): KL(row r of params1
+    || row r of params2) for every row of the two [rows, num_parameters] matrices (host arrays
+    or GPU tensors, any strides), all rows in one pass; returns `klds[:, end]` as a host vector
+    (GPU tensor for GPU input).  With norm_params the leaf parameters are probabilities.
+    Called with a second circuit instead, `kld(bpc_p, bpc_q)`, it takes the two circuits' own
+    parameters as the single row and returns a float."""
+    if params2 is None:
+        out = np.zeros(1, np.float32)
+        check(lib.pcm_kld(mbpc.handle, params1.handle, np_ptr(out)))
+        return float(out[0])
+    n = mbpc.num_parameters()
+    p1, host = _rows_on_device(params1, n, "params1")
+    p2, _ = _rows_on_device(params2, n, "params2")
+    if p2.shape[0] == 1 and p1.shape[0] > 1:
+        p2 = p2.expand(p1.shape[0], n).contiguous()
+    if p2.shape != p1.shape or p2.stride() != p1.stride():
+        p1, p2 = p1.contiguous(), p2.contiguous()
+    if p1.shape != p2.shape:
+        raise ValueError("params1 and params2 must have the same shape")
+    out = torch.empty(p1.shape[0], dtype=torch.float32, device=p1.device)
+    check(lib.pcm_kld_rows(mbpc.handle, p1.data_ptr(), p2.data_ptr(), p1.stride(0), p1.stride(1), p1.shape[0],
+                           int(bool(norm_params)), out.data_ptr()))
+    return out.cpu().numpy() if host else out
+
+
+def kld_backward(mbpc, params1, params2=None, *, device=False, norm_params=False, grad_wrt_logparams=True):
+    """`kld_backward(mbpc, params1, params2; norm_params, grad_wrt_logparams = true)`
+    (src/queries/kld.jl:593-649) -> (grads1, grads2), matrices shaped like the parameter
+    matrices, all rows in one pass.  Called with a second circuit instead it differentiates
+    the single row of the two circuits' own parameters: host vectors, or with device=True GPU
+    tensors (what adam_step takes)."""
+    if not grad_wrt_logparams:
+        raise NotImplementedError("grad_wrt_logparams = false: the reference's kernel for it is empty (kld.jl:322-331)")
+    n = mbpc.num_parameters()
+    if params2 is None:
+        bpc_q = params1
+        if device:
+            g1 = torch.empty(n, dtype=torch.float32, device="cuda")
+            g2 = torch.empty(n, dtype=torch.float32, device="cuda")
+            check(lib.pcm_kld_backward_dev(mbpc.handle, bpc_q.handle, g1.data_ptr(), g2.data_ptr(), c_i64(n)))
+            return g1, g2
+        g1 = np.empty(n, np.float32)
+        g2 = np.empty(n, np.float32)
+        check(lib.pcm_kld_backward(mbpc.handle, bpc_q.handle, np_ptr(g1), np_ptr(g2), c_i64(n)))
         return g1, g2
-    g1 = np.empty(n, np.float32)
-    g2 = np.empty(n, np.float32)
-    check(lib.pcm_kld_backward(bpc_p.handle, bpc_q.handle, np_ptr(g1), np_ptr(g2), c_i64(n)))
-    return g1, g2
+    p1, host = _rows_on_device(params1, n, "params1")
+    p2, _ = _rows_on_device(params2, n, "params2")
+    if p2.shape[0] == 1 and p1.shape[0] > 1:
+        p2 = p2.expand(p1.shape[0], n).contiguous()
+    if p2.shape != p1.shape or p2.stride() != p1.stride():
+        p1, p2 = p1.contiguous(), p2.contiguous()
+    if p1.shape != p2.shape:
+        raise ValueError("params1 and params2 must have the same shape")
+    g1, g2 = torch.empty_strided(p1.shape, p1.stride(), dtype=torch.float32, device=p1.device), \
+        torch.empty_strided(p1.shape, p1.stride(), dtype=torch.float32, device=p1.device)
+    check(lib.pcm_kld_backward_rows(mbpc.handle, p1.data_ptr(), p2.data_ptr(), p1.stride(0), p1.stride(1), p1.shape[0],
+                                    int(bool(norm_params)), g1.data_ptr(), g2.data_ptr(), None))
+    return (g1.cpu().numpy(), g2.cpu().numpy()) if host else (g1, g2)
+
+
+def gumbel_sample_rows(mbpc, params, *, temperature, noise=None, norm_params=False):
+    """`gumbel_sample(mbpc, params, num_vars, par_buffer_size; temperature, no_gumbel, norm_params)`
+    (src/queries/sample.jl:338-383) for a [rows, num_parameters] matrix: one relaxed top-down
+    pass per row, all rows at once.  noise: [rows, num sum parameters] Gumbel draws (one per sum
+    edge, as the reference draws them in its kernel, :45), or None for no_gumbel = true.
+    Returns the soft assignment [rows, V, C] (host array for host input, else GPU tensor)."""
+    n = mbpc.num_parameters()
+    p, host = _rows_on_device(params, n, "params")
+    ns = mbpc.num_inner_params()
+    if noise is not None:
+        noise, _ = _rows_on_device(noise, ns, "noise")
+        noise = noise.contiguous()
+        if noise.shape[0] != p.shape[0]:
+            raise ValueError("noise must have one row per parameter row")
+    out = torch.empty((p.shape[0], mbpc.size("variables"), mbpc.size("categories")), dtype=torch.float32, device=p.device)
+    check(lib.pcm_gumbel_sample_rows(mbpc.handle, p.data_ptr(), p.stride(0), p.stride(1), p.shape[0], _dev_ptr(noise),
+                                     float(temperature), int(bool(norm_params)), out.data_ptr()))
+    return out.cpu().numpy() if host else out
 
 
 def sample(bpc, node_noise, leaf_noise):

@@ -286,17 +286,22 @@ void orc_em_update(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
  *   edges  : queries/kld.jl:95-107 -- kld = klds[prime] (+ klds[sub]); for a sum edge
  *            kld = exp(p1) * (kld + p1 - p2); a parent adds up its edges (:113-128).
  * klds is [n_nodes]; edge_klds [n_edges] (may be NULL).
+ * norm_params != 0: the LEAF arrays hold probabilities instead of log-probabilities and the
+ * leaf term is nodes/fixable_categorical_dist.jl:182-186,
+ *            kld = sum_c p1_c * (log(p1_c + 1e-8) - log(p2_c + 1e-8));
+ * the sum edges are in log space either way (queries/kld.jl:103-107 has no such switch).
  */
 void orc_kld(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
              const int32_t* prime, const int32_t* sub, const REAL* logp1,
              const REAL* logp2, const int64_t* in_off, int C, const REAL* leaf1,
-             const REAL* leaf2, REAL* klds, REAL* edge_klds) {
+             const REAL* leaf2, REAL* klds, REAL* edge_klds, int norm_params) {
   for (int n = 0; n < n_nodes; ++n) {
     if (type[n] == NODE_INPUT) {
       REAL k = 0;
       for (int i = 0; i < C; ++i) {
         REAL a = leaf1[in_off[n] + i], b = leaf2[in_off[n] + i];
-        k += (REAL)exp((double)a) * (a - b);
+        if (norm_params) k += a * ((REAL)log((double)(a + (REAL)1e-8)) - (REAL)log((double)(b + (REAL)1e-8)));
+        else k += (REAL)exp((double)a) * (a - b);
       }
       klds[n] = k;
       continue;
@@ -325,6 +330,9 @@ void orc_kld(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
  * If analytic != 0 the leaf lines use the true derivatives
  *   grad1_c = g * exp(p1_c) * (p1_c - p2_c + 1), grad2_c = -g * exp(p1_c)
  * (used only to pin the recursion against finite differences).
+ * analytic == 2: the leaf arrays hold probabilities (norm_params = true) and the leaf lines are
+ * those of nodes/fixable_categorical_dist.jl:216-217, as written:
+ *   grad1_c = g * (log(p1_c + 1e-8) - log(p2_c + 1e-8) + 1), grad2_c = g * p1_c / (p2_c + 1e-8).
  */
 void orc_kld_backward(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
                       const int32_t* prime, const int32_t* sub, const REAL* logp1,
@@ -340,7 +348,10 @@ void orc_kld_backward(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
     if (type[n] == NODE_INPUT) {
       for (int i = 0; i < C; ++i) {
         REAL a = leaf1[in_off[n] + i], b = leaf2[in_off[n] + i];
-        if (analytic) {
+        if (analytic == 2) {
+          leaf_g1[in_off[n] + i] = g * ((REAL)log((double)(a + (REAL)1e-8)) - (REAL)log((double)(b + (REAL)1e-8)) + 1);
+          leaf_g2[in_off[n] + i] = g * a / (b + (REAL)1e-8);
+        } else if (analytic) {
           leaf_g1[in_off[n] + i] = g * (REAL)exp((double)a) * (a - b + 1);
           leaf_g2[in_off[n] + i] = -g * (REAL)exp((double)a);
         } else {
@@ -433,19 +444,21 @@ void orc_sample(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
  * sum node), :105-140 (td_prob[child] += td_prob[parent] * w / group_sum; products pass
  * td_prob on to prime and sub) and the categorical leaf step :262-284
  * (out[var][c] += td_prob * exp(leaf_logp[c])).  g may be NULL (no_gumbel = true).
+ * norm_params != 0: the leaf array holds probabilities and is added without the exp (:265-268).
  */
 void orc_gumbel_soft(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
                      const int32_t* prime, const int32_t* sub, const REAL* logp,
                      const int32_t* in_var, const int64_t* in_off, int C,
                      const REAL* leaf_logp, const REAL* g, REAL temperature, int64_t V,
-                     REAL* td, REAL* out) {
+                     REAL* td, REAL* out, int norm_params) {
   memset(td, 0, sizeof(REAL) * (size_t)n_nodes);
   memset(out, 0, sizeof(REAL) * (size_t)(V * C));
   td[n_nodes - 1] = 1;
   for (int n = n_nodes - 1; n >= 0; --n) {
     if (type[n] == NODE_INPUT) {
       for (int c = 0; c < C; ++c)
-        out[(int64_t)in_var[n] * C + c] += td[n] * (REAL)exp((double)leaf_logp[in_off[n] + c]);
+        out[(int64_t)in_var[n] * C + c] +=
+            td[n] * (norm_params ? leaf_logp[in_off[n] + c] : (REAL)exp((double)leaf_logp[in_off[n] + c]));
       continue;
     }
     int e0 = edge_ptr[n], e1 = edge_ptr[n + 1];

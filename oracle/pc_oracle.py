@@ -267,18 +267,20 @@ def em_step(fc, data, idx, pseudocount, inertia, double=False):
     return mars[-1].copy(), logp, leaf, ea, lf
 
 
-def kld(fc1, fc2, double=False):
+def kld(fc1, fc2, double=False, norm_params=False):
+    """norm_params: the circuits' leaf arrays hold probabilities (sum edges stay in log space)."""
     R = _real(double)
     klds = np.empty(fc1.n_nodes, dtype=R)
     ek = np.empty(fc1.n_edges, dtype=R)
     a = [np.ascontiguousarray(x, R) for x in (fc1.logp, fc2.logp, fc1.leaf_logp, fc2.leaf_logp)]
     lib(double).orc_kld(ctypes.c_int(fc1.n_nodes), _p(fc1.type), _p(fc1.edge_ptr), _p(fc1.prime),
                         _p(fc1.sub), _p(a[0]), _p(a[1]), _p(fc1.in_off), ctypes.c_int(fc1.C),
-                        _p(a[2]), _p(a[3]), _p(klds), _p(ek))
+                        _p(a[2]), _p(a[3]), _p(klds), _p(ek), ctypes.c_int(int(norm_params)))
     return klds, ek
 
 
-def kld_backward(fc1, fc2, edge_klds, analytic=False, double=False):
+def kld_backward(fc1, fc2, edge_klds, analytic=False, double=False, norm_params=False):
+    """norm_params: leaf arrays hold probabilities, leaf lines of fixable_categorical_dist.jl:216-217."""
     R = _real(double)
     a = [np.ascontiguousarray(x, R) for x in (fc1.logp, fc2.logp, fc1.leaf_logp, fc2.leaf_logp, edge_klds)]
     grads = np.empty(fc1.n_nodes, dtype=R)
@@ -289,7 +291,7 @@ def kld_backward(fc1, fc2, edge_klds, analytic=False, double=False):
     lib(double).orc_kld_backward(ctypes.c_int(fc1.n_nodes), _p(fc1.type), _p(fc1.edge_ptr), _p(fc1.prime),
                                  _p(fc1.sub), _p(a[0]), _p(a[1]), _p(fc1.in_off), ctypes.c_int(fc1.C),
                                  _p(a[2]), _p(a[3]), _p(a[4]), _p(grads), _p(eg1), _p(eg2), _p(lg1), _p(lg2),
-                                 ctypes.c_int(int(analytic)))
+                                 ctypes.c_int(2 if norm_params else int(analytic)))
     return grads, eg1, eg2, lg1, lg2
 
 
@@ -309,7 +311,7 @@ def sample(fc, edge_noise, leaf_noise, noise_slot=None, double=False):
     return out
 
 
-def gumbel_soft(fc, g, temperature, double=False):
+def gumbel_soft(fc, g, temperature, double=False, norm_params=False):
     R = _real(double)
     td = np.empty(fc.n_nodes, dtype=R)
     out = np.empty((fc.V, fc.C), dtype=R)
@@ -318,7 +320,8 @@ def gumbel_soft(fc, g, temperature, double=False):
     lib(double).orc_gumbel_soft(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(fc.prime),
                                 _p(fc.sub), _p(np.ascontiguousarray(fc.logp, R)), _p(fc.in_var),
                                 _p(fc.in_off), ctypes.c_int(fc.C), _p(np.ascontiguousarray(fc.leaf_logp, R)),
-                                _p(gg), rc(temperature), ctypes.c_int64(fc.V), _p(td), _p(out))
+                                _p(gg), rc(temperature), ctypes.c_int64(fc.V), _p(td), _p(out),
+                                ctypes.c_int(int(norm_params)))
     return td, out
 
 

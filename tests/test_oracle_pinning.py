@@ -452,6 +452,48 @@ def test_kld_backward_leaf_lines_as_written():
     np.testing.assert_allclose(w2[off], 0.1, rtol=1e-5)
 
 
+def test_probability_valued_leaf_parameters():
+    """norm_params = true: leaf parameters are probabilities (src/nodes/fixable_categorical_dist.jl:182-186,
+    :216-217; src/queries/sample.jl:265-268), sum edges stay in log space.  The KL equals the
+    log-parameter form on the logarithms and scipy's entropy leaf by leaf; grad1 as written IS the
+    derivative with respect to p1 (central differences), grad2 as written is minus the derivative
+    with respect to p2; the relaxed sampler's output equals the log-parameter form's."""
+    from scipy.stats import entropy
+    rng = np.random.default_rng(41)
+    root = random_dag(4, 3, rng, width=2)
+    f1 = O.bits_compile(root, 3, 4)
+    f2 = f1.copy()
+    f2.update_parameters((f1.vectorize_parameters() + rng.normal(0, 0.3, len(f1.vectorize_parameters()))).astype(np.float32))
+    f2.leaf_logp = np.log(np.exp(f2.leaf_logp.reshape(-1, 3)) / np.exp(f2.leaf_logp.reshape(-1, 3)).sum(1, keepdims=True)).reshape(-1)
+    n1, n2 = f1.copy(), f2.copy()
+    for a, b in ((n1, f1), (n2, f2)):
+        a.logp = b.logp.astype(np.float64)
+        a.leaf_logp = np.exp(b.leaf_logp.astype(np.float64))
+    want, _ = O.kld(f1, f2, double=True)
+    got, ek = O.kld(n1, n2, double=True, norm_params=True)
+    np.testing.assert_allclose(got[-1], want[-1], rtol=1e-6)            # the 1e-8 inside the logarithms
+    for n in f1.input_nodes():
+        o = f1.in_off[n]
+        # (scipy renormalises its arguments; float32 draws add up to 1 within 1e-7)
+        np.testing.assert_allclose(got[n], entropy(n1.leaf_logp[o:o + 3], n2.leaf_logp[o:o + 3]), rtol=1e-5, atol=1e-6)
+    _, _, _, w1, w2 = O.kld_backward(n1, n2, ek, double=True, norm_params=True)
+    h = 1e-7
+    for i in range(len(n1.leaf_logp)):
+        for which, wantg in ((0, w1[i]), (1, -w2[i])):
+            a, b = n1.copy(), n2.copy()
+            t = (a, b)[which]
+            t.leaf_logp = t.leaf_logp.copy()
+            t.leaf_logp[i] += h
+            up = O.kld(a, b, double=True, norm_params=True)[0][-1]
+            t.leaf_logp[i] -= 2 * h
+            fd = (up - O.kld(a, b, double=True, norm_params=True)[0][-1]) / (2 * h)
+            assert abs(fd - wantg) < 1e-5 * max(1, abs(wantg)), (i, which)
+    g = _gumbel(rng, f1.n_edges)
+    _, out_log = O.gumbel_soft(f1, g, 0.7, double=True)
+    _, out_prob = O.gumbel_soft(n1, g, 0.7, double=True, norm_params=True)
+    np.testing.assert_allclose(out_prob, out_log, rtol=1e-6)
+
+
 # ------------------------------------------------------------------------------------
 # sampling
 # ------------------------------------------------------------------------------------

@@ -360,10 +360,101 @@ def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
             np.testing.assert_allclose(cold[b], want, rtol=1e-3, atol=1e-6)
 
 
-def test_prealloc_wrappers_run_the_queries_row_by_row(gpu, oracle):
+def _row_oracle(O, fc, row, n_sum, norm):
+    """The oracle circuit whose parameters are one row of a parameter matrix (with norm the leaf
+    part of the row holds probabilities, which the oracle's leaf array then holds as they are)."""
+    f = fc.copy()
+    f.logp = f.logp.astype(np.float64)
+    f.leaf_logp = f.leaf_logp.astype(np.float64)
+    f.update_parameters(row.astype(np.float64))
+    return f
+
+
+@pytest.mark.parametrize("kind,R,norm", [("hclt", 1, False), ("hclt", 7, True), ("hclt", 64, False), ("dag", 7, False),
+                                         ("dag", 64, True), ("hclt64", 5, True)])
+def test_parameter_row_queries_match_oracle(gpu, oracle, kind, R, norm):
+    """`kld`, `kld_backward` and `gumbel_sample` on a matrix of parameter rows (src/queries/kld.jl:164-206,
+    :593-649, src/queries/sample.jl:338-383), all rows in one pass, log-parameters and probability-valued
+    leaves (norm_params), row-major and column-major matrices: every row against the oracle on that row's
+    parameters.  Tolerances: 1e-4 of the KL, 1e-4 of the largest gradient entry, 1e-4 on the soft samples."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, random_dag, log_dirichlet
+    rng = np.random.default_rng(100 + R)
+    if kind.startswith("hclt"):
+        V, K, C = (9, 64, 5) if kind == "hclt64" else (13, 16, 6)
+        parent, theta, leaf, _ = make_hclt(V, K, C, 61)
+        bpc = P.hclt_from_clt(parent, C, K)
+        fc = O.bits_compile(O.hclt_dag(parent, K, C, theta, leaf), C, V)
+    else:
+        V, C = 8, 5
+        root = random_dag(V, C, rng, width=3)
+        bpc = _compile(P, root, V, C)
+        fc = O.bits_compile(root, C, V)
+    n, ns = bpc.num_parameters(), bpc.num_inner_params()
+    sizes = bpc.table("pargroup_sizes")
+
+    def draw_rows():
+        rows = np.empty((R, n), np.float32)
+        for r in range(R):
+            pos = 0
+            for sz in sizes:
+                rows[r, pos:pos + sz] = log_dirichlet(rng, sz) if sz > 1 else 0.0
+                pos += sz
+            lf = np.exp(np.stack([log_dirichlet(rng, C) for _ in range((n - ns) // C)]))
+            rows[r, ns:] = (lf if norm else np.log(lf)).reshape(-1)
+        return rows
+
+    p1, p2 = draw_rows(), draw_rows()
+    want_kl, want_g1, want_g2 = [], [], []
+    for r in range(R):
+        f1, f2 = _row_oracle(O, fc, p1[r], ns, norm), _row_oracle(O, fc, p2[r], ns, norm)
+        klds, ek = O.kld(f1, f2, double=True, norm_params=norm)
+        _, eg1, eg2, lg1, lg2 = O.kld_backward(f1, f2, ek, double=True, norm_params=norm)
+        want_kl.append(klds[-1])
+        want_g1.append(_grads_in_param_order(fc, eg1, lg1))
+        want_g2.append(_grads_in_param_order(fc, eg2, lg2))
+    want_kl, want_g1, want_g2 = np.array(want_kl), np.stack(want_g1), np.stack(want_g2)
+    # host matrices (row-major on the device)
+    got = P.kld(bpc, p1, p2, norm_params=norm)
+    assert got.shape == (R,) and np.abs(got - want_kl).max() < KLD_RTOL * np.abs(want_kl).max()
+    g1, g2 = P.kld_backward(bpc, p1, p2, norm_params=norm)
+    assert g1.shape == (R, n)
+    assert np.abs(g1 - want_g1).max() < GRAD_RTOL * np.abs(want_g1).max()
+    assert np.abs(g2 - want_g2).max() < GRAD_RTOL * np.abs(want_g2).max()
+    # column-major device matrices, as Julia holds [rows, n]: same numbers, gradients come back in that layout
+    t1 = torch.from_numpy(np.ascontiguousarray(p1.T)).cuda().t()
+    t2 = torch.from_numpy(np.ascontiguousarray(p2.T)).cuda().t()
+    assert R == 1 or t1.stride() == (1, R)
+    np.testing.assert_array_equal(P.kld(bpc, t1, t2, norm_params=norm).cpu().numpy(), got)
+    c1, c2 = P.kld_backward(bpc, t1, t2, norm_params=norm)
+    assert R == 1 or c1.stride() == (1, R)
+    np.testing.assert_array_equal(c1.cpu().numpy(), g1)
+    np.testing.assert_array_equal(c2.cpu().numpy(), g2)
+    # relaxed samples: one draw of noise per row and sum edge
+    for T, with_noise in ((1.0, False), (0.6, True)):
+        noise = _gumbel(rng, (R, ns)) if with_noise else None
+        soft = P.gumbel_sample_rows(bpc, p1, temperature=T, noise=noise, norm_params=norm)
+        assert soft.shape == (R, V, C)
+        pe = fc.sum_param_edges()
+        for r in range(0, R, max(1, R // 5)):
+            f1 = _row_oracle(O, fc, p1[r], ns, norm)
+            g = None
+            if with_noise:
+                g = np.zeros(fc.n_edges)
+                g[pe] = noise[r]
+            _, want = O.gumbel_soft(f1, g, T, double=True, norm_params=norm)
+            np.testing.assert_allclose(soft[r], want, rtol=1e-4, atol=1e-7)
+    # the circuit lends its structure only: its own parameters were not read or touched
+    with pytest.raises(P.PcmError):
+        P._lib.check(P._lib.lib.pcm_kld_rows(bpc.handle, None, None, n, 1, R, 0, None))
+
+
+def test_prealloc_wrappers_run_all_rows_at_once(gpu, oracle):
     """`kld_with_prealloc`, `kld_backward_with_prealloc`, `gumbel_sample_with_prealloc`
-    (src/utils/cuda_preallocation.jl:47-78,189-203) with one parameter vector per example,
-    against the single-vector queries and the oracle."""
+    (src/utils/cuda_preallocation.jl:47-78,189-203) with one parameter vector per example and the
+    arguments src/models/pc_vae.py:81-92 passes (norm_params = True for the sampler, a repeated prior
+    for the KL), against the single-vector queries and the oracle."""
     torch, P = gpu
     O = oracle
     from helpers import make_hclt, block_theta
@@ -395,8 +486,8 @@ def test_prealloc_wrappers_run_the_queries_row_by_row(gpu, oracle):
     P.update_parameters(bpc, p1[1])
     e1, e2 = P.kld_backward(bpc, q)
     P.update_parameters(bpc, base)
-    np.testing.assert_allclose(g1[1], e1, rtol=1e-6, atol=1e-7)
-    np.testing.assert_allclose(g2[1], e2, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(g1[1], e1, rtol=1e-4, atol=1e-6)              # two engines: block chains / lane groups
+    np.testing.assert_allclose(g2[1], e2, rtol=1e-4, atol=1e-6)
     with pytest.raises(ValueError):
         W.kld_with_prealloc(bpc, p1[:2], prior)                                # not the preallocated number of rows
     W.kld_free_mem()
@@ -407,10 +498,21 @@ def test_prealloc_wrappers_run_the_queries_row_by_row(gpu, oracle):
     P.update_parameters(bpc, p1[2])
     direct = P.gumbel_sample(bpc, 1, temperature=1.0)[0].cpu().numpy()
     P.update_parameters(bpc, base)
-    np.testing.assert_allclose(soft[2, :, :C], direct, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(soft[2, :, :C], direct, rtol=1e-4, atol=1e-7)
     noisy = W.gumbel_sample_with_prealloc(bpc, p1, temperature=0.5, generator=torch.Generator(device="cuda").manual_seed(3))
     np.testing.assert_allclose(noisy.sum(-1), 1.0, rtol=1e-4)
+    # what pc_vae.py:81-86 asks for: probability-valued leaves, no noise
+    ns = bpc.num_inner_params()
+    probs = p1.copy()
+    probs[:, ns:] = np.exp(p1[:, ns:])
+    as_vae = W.gumbel_sample_with_prealloc(bpc, probs, temperature=1.0, norm_params=True, no_gumbel=True)
+    np.testing.assert_allclose(as_vae, soft, rtol=1e-5, atol=1e-7)
     W.gumbel_sample_free_mem()
+    # pc_vae.py:88-92: the prior repeated for every row
+    W.kld_preallocation(bpc, num_examples=R)
+    np.testing.assert_allclose(W.kld_with_prealloc(bpc, p1, np.repeat(prior, R, axis=0)), klds, rtol=1e-6)
+    W.kld_free_mem()
+    np.testing.assert_array_equal(P.vectorize_parameters(bpc), base)
 
 
 def test_misaligned_noise_is_refused(gpu, oracle):
