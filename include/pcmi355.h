@@ -312,6 +312,22 @@ int pcm_pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t str
 int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d_m, float* d_v,
                   float lr, float beta1, float beta2, float eps, int32_t t);
 
+/*
+ * The `adam` trainer's step from the flows of a batch (src/sgd/adam.jl:244-344), after pcm_flows with rate 0:
+ * pcm_flow_gradients: d_grad [num sum parameters] (device, parameter-vector order) receives
+ *   edge_aggr / batch_size - exp(logp) * (sum of the sum node's edge_aggr / batch_size)
+ * (`edge_aggr ./= batch_size` :310, `compute_gradients` :27-61), the gradient of the mean log-likelihood with
+ * respect to the unnormalised log-parameters.
+ * pcm_adam_flow_step: that gradient, then the sum-parameter step of pcm_adam_step (:318-325, :63-127), and --
+ * if d_leaf_params is not NULL -- `update_input_node_params_adam` (:218-242) on the three device arrays
+ * [num input parameters] that stand for the reference's auxiliary heap (a copy of the leaf log-parameters that
+ * takes the steps, and its two moments): g = flow + exp(logp) * node_flow as the source writes it.  Like the
+ * source, it never writes the stepped leaf values back into the circuit.
+ */
+int pcm_flow_gradients(pcm_circuit* c, int32_t batch_size, float* d_grad);
+int pcm_adam_flow_step(pcm_circuit* c, int32_t batch_size, float* d_params, float* d_m, float* d_v, float* d_leaf_params,
+                       float* d_leaf_m, float* d_leaf_v, float lr, float beta1, float beta2, float eps, int32_t t);
+
 /* ---- instrumentation ----------------------------------------------------------- */
 
 /* Per-kernel timing, the role of `debug = true` -> `CUDA.@time` around each launch

@@ -1,4 +1,5 @@
 // C ABI of pcmi355: argument checks, exception -> status translation.
+#include <algorithm>
 #include <new>
 
 #include "common.hpp"
@@ -201,6 +202,25 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
 int pcm_adam_step(pcm_circuit* c, const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
                   float b1, float b2, float eps, int32_t t) {
   return guarded([&] { need(c)->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t); });
+}
+
+int pcm_flow_gradients(pcm_circuit* c, int32_t batch_size, float* d_grad) {
+  return guarded([&] { need(c)->flow_gradients(batch_size, d_grad); });
+}
+
+int pcm_adam_flow_step(pcm_circuit* c, int32_t batch_size, float* d_params, float* d_m, float* d_v, float* d_leaf_params,
+                       float* d_leaf_m, float* d_leaf_v, float lr, float b1, float b2, float eps, int32_t t) {
+  return guarded([&] {
+    if (!d_params || !d_m || !d_v) pcm::fail(PCM_ERR_ARG, "null optimiser array");
+    const int64_t ns = need(c)->size(1);
+    // the gradient takes the place the reference gives it: edge_aggr itself (src/sgd/adam.jl:305-319)
+    pcm::DevBuf<float> grad;
+    grad.alloc((size_t)std::max<int64_t>(ns, 1));
+    c->flow_gradients(batch_size, grad.p);
+    if (d_leaf_params) c->leaf_adam(d_leaf_params, d_leaf_m, d_leaf_v, lr, b1, b2, eps, t);   // reads the leaves before the sum step, as :319-325
+    c->adam_step(grad.p, d_params, d_m, d_v, lr, b1, b2, eps, t);
+    PCM_HIP(hipStreamSynchronize(c->stream));
+  });
 }
 
 int pcm_kld_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row, int64_t stride_param,

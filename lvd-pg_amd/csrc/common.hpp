@@ -121,6 +121,10 @@ struct pcm_circuit {
   virtual void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) = 0;
   virtual void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr,
                          float b1, float b2, float eps, int t) = 0;
+  // gradient of the mean log-likelihood w.r.t. the unnormalised sum log-parameters, from the accumulated edge flows
+  virtual void flow_gradients(int32_t batch_size, float* d_grad) = 0;
+  // Adam on the input nodes' auxiliary parameter copy, from the accumulated leaf flows
+  virtual void leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) = 0;
   // queries on a matrix of parameter rows (element strides sr, sp), all rows in one pass
   virtual void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
                         float* d_out) = 0;

@@ -151,6 +151,8 @@ class HcltCircuit : public pcm_circuit {
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
                  float b2, float eps, int t) override;
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
+  void flow_gradients(int32_t batch_size, float* d_grad) override;
+  void leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) override;
   // parameter-row queries run on the circuit's general form (its structure; the rows bring the parameters)
   void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
                 float* d_out) override {
@@ -227,6 +229,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int64_t> d_sum_param_src_;
   DevBuf<int32_t> d_in_pos_;   // input node (v, j) -> its position among the input nodes of the parameter vector
   DevBuf<float> d_param_vec_;  // a parameter vector on its way to or from the host
+  DevBuf<float> d_row_sum_;    // Adam from flows: per-sum-node / per-input-node flow totals
+  DevBuf<int32_t> d_input_order_;   // i-th input node of the parameter vector -> v*K + j
   int cap_slices_ = 0;
   bool have_flows_ = false;
   // soft evidence on the block kernels (single head, K <= 64)

@@ -309,7 +309,94 @@ __global__ __launch_bounds__(256) void hclt_adam_kernel(int64_t ns, const float*
   if (live) logtheta[src[i]] = p - logf(s);
 }
 
+// Adam from flows (src/sgd/adam.jl:305-311, :27-61): gradient of the mean log-likelihood with respect to the
+// unnormalised log-parameters, edge flows / batch size minus exp(theta) times their sum over the sum node.  A sum
+// node is a row of K entries of the block arrays: first the row sums (a wave per row), then one thread per parameter.
+__global__ __launch_bounds__(256) void hclt_row_sum_kernel(const float* __restrict__ edge_aggr, int64_t rows, int K,
+                                                           float* __restrict__ row_sum) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (r >= rows) return;
+  float s = 0.f;
+  for (int j = lane; j < K; j += 64) s += edge_aggr[r * K + j];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+  if (lane == 0) row_sum[r] = s;
+}
+
+__global__ void hclt_flow_grad_kernel(int64_t ns, const int64_t* __restrict__ src, const float* __restrict__ edge_aggr,
+                                      const float* __restrict__ logtheta, const float* __restrict__ row_sum, int K,
+                                      float inv_batch, float* __restrict__ grad) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= ns) return;
+  const int64_t at = src[i];
+  grad[i] = (edge_aggr[at] - expf(logtheta[at]) * row_sum[at / K]) * inv_batch;
+}
+
+// Adam on the input nodes (src/sgd/adam.jl:218-242), one thread per leaf parameter in parameter order: node (v, j)
+// at position q has its C values at q * C; the tables are [V][C][K].  g = flow + exp(logp) * node flow, as the
+// source has it; the steps go to the auxiliary copy, the circuit's leaves are not written.
+__global__ __launch_bounds__(256) void hclt_leaf_node_flow_kernel(const float* __restrict__ leaf_flow, int C, int K,
+                                                                  float* __restrict__ node_flow) {
+  const int v = blockIdx.x;
+  for (int j = threadIdx.x; j < K; j += blockDim.x) {
+    float s = 0.f;
+    for (int c = 0; c < C; ++c) s += leaf_flow[((size_t)v * C + c) * K + j];
+    node_flow[(size_t)v * K + j] = s;
+  }
+}
+
+__global__ __launch_bounds__(256) void hclt_leaf_adam_kernel(int64_t n_leaf, const int32_t* __restrict__ input_order, int C,
+                                                             int K, const float* __restrict__ leaf,
+                                                             const float* __restrict__ leaf_flow,
+                                                             const float* __restrict__ node_flow, float* __restrict__ aux_p,
+                                                             float* __restrict__ aux_m, float* __restrict__ aux_v, float lr,
+                                                             float b1, float b2, float eps, float c1, float c2) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_leaf) return;
+  const int vj = input_order[i / C], c = (int)(i % C);
+  const int v = vj / K, j = vj % K;
+  const size_t at = ((size_t)v * C + c) * K + j;
+  const float g = leaf_flow[at] + expf(leaf[at]) * node_flow[vj];
+  const float m = b1 * aux_m[i] + (1.f - b1) * g, vv = b2 * aux_v[i] + (1.f - b2) * g * g;
+  aux_m[i] = m;
+  aux_v[i] = vv;
+  aux_p[i] += lr * ((m / c1) / (sqrtf(vv / c2) + eps));
+}
+
 // ---- host --------------------------------------------------------------------------------
+
+void HcltCircuit::flow_gradients(int32_t batch_size, float* d_grad) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
+  if (flows_in_general_ || (!block_ && !wide_)) return general_->flow_gradients(batch_size, d_grad);
+  if (!d_grad) fail(PCM_ERR_ARG, "gradient pointer is null");
+  if (batch_size < 1) fail(PCM_ERR_ARG, "batch size must be positive, got %d", batch_size);
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  const int64_t rows = (int64_t)n_inner_ * K_ + H_;
+  d_row_sum_.ensure((size_t)rows);
+  hipLaunchKernelGGL(hclt_row_sum_kernel, dim3((unsigned)ceil_div(rows, 4)), dim3(256), 0, stream, d_edge_aggr_.p, rows, K_,
+                     d_row_sum_.p);
+  hipLaunchKernelGGL(hclt_flow_grad_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns, d_sum_param_src_.p,
+                     d_edge_aggr_.p, d_logtheta_.p, d_row_sum_.p, K_, 1.f / (float)batch_size, d_grad);
+  check_launch_k("hclt_flow_grad");
+}
+
+void HcltCircuit::leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
+  if (flows_in_general_ || (!block_ && !wide_)) return general_->leaf_adam(d_aux_p, d_aux_m, d_aux_v, lr, b1, b2, eps, t);
+  if (!d_aux_p || !d_aux_m || !d_aux_v) fail(PCM_ERR_ARG, "null optimiser array");
+  if (t < 1) fail(PCM_ERR_ARG, "step count must start at 1, got %d", t);
+  if (d_input_order_.n == 0) d_input_order_.upload(input_order_, stream);
+  d_row_sum_.ensure((size_t)V_ * K_);
+  hipLaunchKernelGGL(hclt_leaf_node_flow_kernel, dim3(V_), dim3(std::min(256, ceil_div(K_, 64) * 64)), 0, stream,
+                     d_leaf_flow_.p, C_, K_, d_row_sum_.p);
+  const int64_t n_leaf = (int64_t)V_ * K_ * C_;
+  const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
+  hipLaunchKernelGGL(hclt_leaf_adam_kernel, dim3((unsigned)ceil_div(n_leaf, 256)), dim3(256), 0, stream, n_leaf,
+                     d_input_order_.p, C_, K_, d_leaf_.p, d_leaf_flow_.p, d_row_sum_.p, d_aux_p, d_aux_m, d_aux_v, lr, b1, b2,
+                     eps, c1, c2);
+  check_launch_k("hclt_leaf_adam");
+}
 
 HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "KL of multi-head circuits is not defined");

@@ -1456,4 +1456,68 @@ void SparseCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, 
   check_launch("sparse_adam");
 }
 
+
+// ---- Adam from flows ------------------------------------------------------------------------
+// src/sgd/adam.jl:305-311 and :27-61: edge flows / batch size minus exp(logp) times their sum over the sum node,
+// one thread per normalisation group, written in parameter order.
+__global__ void sparse_flow_grad_kernel(int n_groups, const int32_t* __restrict__ group_ptr,
+                                        const int32_t* __restrict__ param2edge, const float* __restrict__ edge_aggr,
+                                        const float* __restrict__ logp, float inv_batch, float* __restrict__ grad) {
+  const int gi = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gi >= n_groups) return;
+  const int p0 = group_ptr[gi], p1 = group_ptr[gi + 1];
+  float s = 0.f;
+  for (int p = p0; p < p1; ++p) s += edge_aggr[param2edge[p]] * inv_batch;
+  for (int p = p0; p < p1; ++p) {
+    const int e = param2edge[p];
+    grad[p] = edge_aggr[e] * inv_batch - expf(logp[e]) * s;
+  }
+}
+
+// src/sgd/adam.jl:218-242, a wave per input node: g = flow + exp(logp) * node flow (as the source has it); the
+// steps go to the auxiliary copy, never into the circuit.
+__global__ __launch_bounds__(256) void sparse_leaf_adam_kernel(int64_t n_inputs, int C, const float* __restrict__ leaf,
+                                                               const float* __restrict__ leaf_flow, float* __restrict__ aux_p,
+                                                               float* __restrict__ aux_m, float* __restrict__ aux_v, float lr,
+                                                               float b1, float b2, float eps, float c1, float c2) {
+  const int lane = threadIdx.x & 63;
+  const int64_t q = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (q >= n_inputs) return;
+  const float* fl = leaf_flow + q * C;
+  float node_flow = 0.f;
+  for (int c = lane; c < C; c += 64) node_flow += fl[c];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) node_flow += __shfl_xor(node_flow, o);
+  for (int c = lane; c < C; c += 64) {
+    const int64_t i = q * C + c;
+    const float g = fl[c] + expf(leaf[i]) * node_flow;
+    const float m = b1 * aux_m[i] + (1.f - b1) * g, v = b2 * aux_v[i] + (1.f - b2) * g * g;
+    aux_m[i] = m;
+    aux_v[i] = v;
+    aux_p[i] += lr * ((m / c1) / (sqrtf(v / c2) + eps));
+  }
+}
+
+void SparseCircuit::flow_gradients(int32_t batch_size, float* d_grad) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
+  if (!d_grad) fail(PCM_ERR_ARG, "gradient pointer is null");
+  if (batch_size < 1) fail(PCM_ERR_ARG, "batch size must be positive, got %d", batch_size);
+  const int ng = (int)fc_.pargroup_sizes.size();
+  if (!ng) return;
+  hipLaunchKernelGGL(sparse_flow_grad_kernel, dim3(ceil_div(ng, 128)), dim3(128), 0, stream, ng, d_group_ptr_.p,
+                     d_param2edge_.p, d_edge_aggr_.p, d_logp_.p, 1.f / (float)batch_size, d_grad);
+  check_launch("sparse_flow_grad");
+}
+
+void SparseCircuit::leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) {
+  if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
+  if (!d_aux_p || !d_aux_m || !d_aux_v) fail(PCM_ERR_ARG, "null optimiser array");
+  if (t < 1) fail(PCM_ERR_ARG, "step count must start at 1, got %d", t);
+  const int64_t ni = (int64_t)fc_.input_nodes.size();
+  const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
+  hipLaunchKernelGGL(sparse_leaf_adam_kernel, dim3((unsigned)ceil_div(ni, 4)), dim3(256), 0, stream, ni, fc_.num_cats,
+                     d_leaf_.p, d_leaf_flow_.p, d_aux_p, d_aux_m, d_aux_v, lr, b1, b2, eps, c1, c2);
+  check_launch("sparse_leaf_adam");
+}
+
 }  // namespace pcm

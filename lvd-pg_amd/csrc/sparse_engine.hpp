@@ -65,6 +65,8 @@ class SparseCircuit : public pcm_circuit {
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1, float b2,
                  float eps, int t) override;
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
+  void flow_gradients(int32_t batch_size, float* d_grad) override;
+  void leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) override;
   void sample_soft_with_slots(const float* d_node_noise, const int32_t* d_noise_slot, int64_t noise_stride,
                               float temperature, int32_t batch, float* d_out);
   void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,

@@ -49,6 +49,8 @@ _SIGS = {
     "pcm_sample": [H, vp, vp, c_i32, vp],
     "pcm_sample_soft": [H, vp, ctypes.c_float, c_i32, vp],
     "pcm_adam_step": [H, vp, vp, vp, vp, c_f32, c_f32, c_f32, c_f32, c_i32],
+    "pcm_flow_gradients": [H, c_i32, vp],
+    "pcm_adam_flow_step": [H, c_i32, vp, vp, vp, vp, vp, vp, c_f32, c_f32, c_f32, c_f32, c_i32],
     "pcm_kld_rows": [H, vp, vp, c_i64, c_i64, c_i32, c_i32, vp],
     "pcm_kld_backward_rows": [H, vp, vp, c_i64, c_i64, c_i32, c_i32, vp, vp, vp],
     "pcm_gumbel_sample_rows": [H, vp, c_i64, c_i64, c_i32, vp, c_f32, c_i32, vp],

@@ -140,6 +140,7 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
     lls = []
     ll = torch.empty(batch_size, dtype=torch.float32, device=data.device)
     hm_t = None if head_mask is None else head_mask.to(device=data.device, dtype=torch.float32)
+    fresh = True     # the reference clears edge_aggr and the input nodes' flows before its loop (:243-244)
     for _ in range(num_epochs):
         if shuffle == "each_epoch":
             do_shuffle()
@@ -148,7 +149,8 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
             if shuffle == "each_batch":
                 do_shuffle()
             ids = perm[bi * batch_size:(bi + 1) * batch_size]
-            rate = 0.0 if flow_memory == 0 else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
+            rate = 0.0 if (flow_memory == 0 or fresh) else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
+            fresh = False
             if hm_t is None and not _is_soft(data):
                 check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
                                       batch_size, rate, float(pseudocount), float(param_inertia), ll.data_ptr()))
@@ -331,6 +333,57 @@ def adam_step(bpc, grad, params, m, v, *, lr, beta1=0.9, beta2=0.999, eps=1e-8, 
     update of the unnormalised sum parameters, per-node normalisation into the circuit."""
     check(lib.pcm_adam_step(bpc.handle, grad.data_ptr(), params.data_ptr(), m.data_ptr(), v.data_ptr(),
                             float(lr), float(beta1), float(beta2), float(eps), int(t)))
+
+
+def flow_gradients(bpc, batch_size):
+    """`edge_aggr ./= batch_size; compute_gradients(bpc, edge_aggr, node_aggr)` (src/sgd/adam.jl:310-311,
+    :27-61) on the flows the circuit holds: the gradient of the mean log-likelihood with respect to the
+    unnormalised sum log-parameters, a GPU vector in parameter order."""
+    g = torch.empty(bpc.num_inner_params(), dtype=torch.float32, device="cuda")
+    check(lib.pcm_flow_gradients(bpc.handle, int(batch_size), g.data_ptr()))
+    return g
+
+
+def adam(bpc, data, num_epochs, *, batch_size, lr, beta1=0.9, beta2=0.999, eps=1e-8, verbose=False, generator=None,
+         shuffle=True, state=None):
+    """`adam(bpc, data, num_epochs; batch_size, lr, beta1, beta2, eps)` (src/sgd/adam.jl:244-344): per batch the
+    flows, the gradient from them, Adam on the unnormalised sum log-parameters with per-node renormalisation
+    into the circuit, and the input nodes' Adam on an auxiliary copy of their parameters (which, as in the
+    source, never flows back into the circuit).  Returns the per-epoch mean log-likelihoods.  `state`, if given,
+    is a dict that receives the optimiser arrays (params, m, v, leaf_params, leaf_m, leaf_v, opt_count)."""
+    _check_data(bpc, data)
+    n = data.shape[0]
+    if batch_size > n:
+        raise ValueError("batch_size must not exceed the number of examples")    # adam.jl:258
+    num_batches = n // batch_size
+    dev = data.device
+    ns, nl = bpc.num_inner_params(), bpc.num_input_params()
+    pv = torch.from_numpy(vectorize_parameters(bpc)).to(dev)
+    params = pv[:ns].clone()                  # copy_parameters_to_vec (:150-172)
+    leaf_params = pv[ns:].clone()             # copy_input_parameters_to_heap (:174-203)
+    m, v = torch.zeros_like(params), torch.zeros_like(params)
+    leaf_m, leaf_v = torch.zeros_like(leaf_params), torch.zeros_like(leaf_params)
+    ll = torch.empty(batch_size, dtype=torch.float32, device=dev)
+    perm = torch.arange(n, dtype=torch.int32, device=dev)
+    lls, opt_count = [], 0
+    for epoch in range(num_epochs):
+        if shuffle:
+            perm = torch.randperm(n, generator=generator).to(device=dev, dtype=torch.int32)
+        acc = torch.zeros((), dtype=torch.float64, device=dev)
+        for bi in range(num_batches):
+            opt_count += 1
+            ids = perm[bi * batch_size:(bi + 1) * batch_size]
+            _flows(bpc, data, ids.data_ptr(), batch_size, 0.0, None, ll.data_ptr())
+            acc += ll.sum(dtype=torch.float64)
+            check(lib.pcm_adam_flow_step(bpc.handle, batch_size, params.data_ptr(), m.data_ptr(), v.data_ptr(),
+                                         leaf_params.data_ptr(), leaf_m.data_ptr(), leaf_v.data_ptr(), float(lr),
+                                         float(beta1), float(beta2), float(eps), opt_count))
+        lls.append(float(acc.item()) / batch_size / num_batches)
+        if verbose:
+            print(f"Adam epoch {epoch + 1}; train LL {lls[-1]}")
+    if state is not None:
+        state.update(params=params, m=m, v=v, leaf_params=leaf_params, leaf_m=leaf_m, leaf_v=leaf_v, opt_count=opt_count)
+    return lls
 
 
 def patch_level_evidence(mhbpcs, patches, batch_size=256):

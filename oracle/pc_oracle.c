@@ -509,6 +509,56 @@ void orc_adam_step(int64_t n, REAL* params, const REAL* grad, REAL* m, REAL* v, 
   }
 }
 
+/*
+ * Gradient of the mean log-likelihood with respect to the unnormalised log-parameters of the sum
+ * edges, from the accumulated edge flows: sgd/adam.jl:305-311 (edge_aggr ./= batch_size) and :27-61
+ * (`compute_gradients`: node_aggr[parent] = sum of the parent's edge flows, then
+ * edge_aggr[e] -= exp(logp_e) * node_aggr[parent]).  Product edges are left as they are.
+ * edge_aggr is [n_edges] in CSR order and is overwritten with the gradient.
+ */
+void orc_flow_gradients(int n_nodes, const uint8_t* type, const int32_t* edge_ptr, const REAL* logp,
+                        REAL* edge_aggr, REAL batch_size) {
+  for (int n = 0; n < n_nodes; ++n) {
+    if (type[n] != NODE_SUM) continue;
+    REAL node_aggr = 0;
+    for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
+      edge_aggr[e] /= batch_size;
+      node_aggr += edge_aggr[e];
+    }
+    for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e)
+      edge_aggr[e] -= (REAL)exp((double)logp[e]) * node_aggr;
+  }
+}
+
+/*
+ * Adam on the input nodes as sgd/adam.jl:218-242 writes it (`update_params_adam` of a categorical
+ * leaf), one call per input node with its C log-probabilities `lp` (read only: the source never
+ * writes the stepped values back into the circuit), its C flows, and its slice of the auxiliary
+ * heap: aux_p (a copy of the parameters that takes the steps), aux_m, aux_v.
+ *   node_flow = sum_i flow_i;  g_i = flow_i + exp(lp_i) * node_flow   (the sign is the source's)
+ *   m = b1*m + (1-b1)*g;  v = b2*v + (1-b2)*g^2;  aux_p += lr * (m/(1-b1^t)) / (sqrt(v/(1-b2^t)) + eps)
+ */
+void orc_leaf_adam(int64_t n_inputs, int C, const REAL* leaf_logp, const REAL* leaf_flow, REAL* aux_p,
+                   REAL* aux_m, REAL* aux_v, REAL lr, REAL b1, REAL b2, REAL eps, int t) {
+  REAL c1 = (REAL)1 - (REAL)pow((double)b1, (double)t);
+  REAL c2 = (REAL)1 - (REAL)pow((double)b2, (double)t);
+  for (int64_t q = 0; q < n_inputs; ++q) {
+    const REAL* lp = leaf_logp + q * C;
+    const REAL* fl = leaf_flow + q * C;
+    REAL node_flow = 0;
+    for (int i = 0; i < C; ++i) node_flow += fl[i];
+    for (int i = 0; i < C; ++i) {
+      REAL p = (REAL)exp((double)lp[i]);
+      REAL g = fl[i] + p * node_flow;
+      REAL m = b1 * aux_m[q * C + i] + ((REAL)1 - b1) * g;
+      REAL v = b2 * aux_v[q * C + i] + ((REAL)1 - b2) * g * g;
+      aux_m[q * C + i] = m;
+      aux_v[q * C + i] = v;
+      aux_p[q * C + i] += lr * ((m / c1) / ((REAL)sqrt((double)(v / c2)) + eps));
+    }
+  }
+}
+
 int orc_real_size(void) { return (int)sizeof(REAL); }
 int orc_max_threads(void) {
 #if defined(_OPENMP)

@@ -332,6 +332,27 @@ def adam_step(params, grad, m, v, lr, b1, b2, eps, t, group_ptr, logp_out, doubl
                               rc(b2), rc(eps), ctypes.c_int(t), ctypes.c_int(len(gp) - 1), _p(gp), _p(logp_out))
 
 
+def flow_gradients(fc, edge_aggr, batch_size, double=False):
+    """sgd/adam.jl:27-61, 305-311: gradient of the mean LL w.r.t. unnormalised sum log-parameters,
+    [n_edges] in CSR order (product edges keep their flow)."""
+    R = _real(double)
+    g = np.ascontiguousarray(edge_aggr, R).copy()
+    rc = ctypes.c_double if double else ctypes.c_float
+    lib(double).orc_flow_gradients(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr),
+                                   _p(np.ascontiguousarray(fc.logp, R)), _p(g), rc(batch_size))
+    return g
+
+
+def leaf_adam(fc, leaf_flow, aux_p, aux_m, aux_v, lr, b1, b2, eps, t, double=False):
+    """sgd/adam.jl:218-242 on every input node, in the order of fc.leaf_logp; the aux arrays are
+    updated in place, the circuit's leaves are not."""
+    R = _real(double)
+    rc = ctypes.c_double if double else ctypes.c_float
+    lib(double).orc_leaf_adam(ctypes.c_int64(len(fc.leaf_logp) // fc.C), ctypes.c_int(fc.C),
+                              _p(np.ascontiguousarray(fc.leaf_logp, R)), _p(np.ascontiguousarray(leaf_flow, R)),
+                              _p(aux_p), _p(aux_m), _p(aux_v), rc(lr), rc(b1), rc(b2), rc(eps), ctypes.c_int(t))
+
+
 # ----------------------------------------------------------------------------------
 # circuit DAGs and their flattening (small circuits)
 # ----------------------------------------------------------------------------------

@@ -535,3 +535,89 @@ def test_misaligned_noise_is_refused(gpu, oracle):
         P.gumbel_sample(h, B, temperature=0.7, node_noise=shifted)
     aligned = flat[:B * need].view(B, need)
     assert P.sample(h, aligned, leafn).shape == (B, V)
+
+
+@pytest.mark.parametrize("kind", ["hclt16", "hclt64", "hclt128", "hclt8", "dag"])
+def test_adam_from_flows_matches_oracle(gpu, oracle, kind):
+    """`compute_gradients` and the `adam` loop's step (src/sgd/adam.jl:27-61, :218-242, :305-325) on the block
+    engines (lean / general walks, wide blocks), on a hidden size without block kernels and on a DAG: the
+    gradient vector, then three steps of the sum parameters' and the input nodes' optimiser state, against
+    the oracle.  Tolerance 1e-4 (gradient: of its largest entry)."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, random_dag, correlated_data
+    from pcmi355._lib import lib, check
+    rng = np.random.default_rng(7)
+    B = 50
+    if kind == "dag":
+        V, C = 7, 5
+        root = random_dag(V, C, rng, width=3)
+        bpc = _compile(P, root, V, C)
+        fc = O.bits_compile(root, C, V)
+        data = rng.integers(0, C, (B, V)).astype(np.uint8)
+    else:
+        K = int(kind[4:])
+        V, C = 9, 6
+        parent, theta, leaf, _ = make_hclt(V, K, C, 17)
+        bpc = P.hclt_from_clt(parent, C, K)
+        bpc.set_params(block_theta(parent, K, theta), leaf)
+        fc = O.bits_compile(O.hclt_dag(parent, K, C, theta, leaf), C, V)
+        data = correlated_data(B, V, C, 18, parent)
+    np.testing.assert_allclose(P.vectorize_parameters(bpc), fc.vectorize_parameters(), atol=1e-6)
+    d = torch.from_numpy(data).cuda()
+    ns, nl = bpc.num_inner_params(), bpc.num_input_params()
+    pe = fc.sum_param_edges()
+    sizes = bpc.table("pargroup_sizes")
+    gp = np.concatenate([[0], np.cumsum(sizes)])
+    # optimiser state on both sides
+    params = fc.logp[pe].astype(np.float32).copy()
+    m, v = np.zeros(ns, np.float32), np.zeros(ns, np.float32)
+    aux_p = fc.leaf_logp.astype(np.float32).copy()      # the oracle keeps leaves in input-node order = parameter order
+    aux_m, aux_v = np.zeros(nl, np.float32), np.zeros(nl, np.float32)
+    dp, dm, dv = (torch.from_numpy(x.copy()).cuda() for x in (params, m, v))
+    lp, lm, lv = (torch.from_numpy(x.copy()).cuda() for x in (aux_p, aux_m, aux_v))
+    lr = 2e-2
+    leaves_before = P.vectorize_parameters(bpc)[ns:].copy()
+    for t in range(1, 4):
+        P.probs_flows_circuit(bpc, d)
+        mars = O.forward(fc, data)
+        flows, ea = O.backward(fc, mars)
+        lf = O.input_flows(fc, data, flows)
+        want_grad = O.flow_gradients(fc, ea, B)[pe]
+        got_grad = P.flow_gradients(bpc, B).cpu().numpy()
+        assert np.abs(got_grad - want_grad).max() < 1e-4 * np.abs(want_grad).max()
+        check(lib.pcm_adam_flow_step(bpc.handle, B, dp.data_ptr(), dm.data_ptr(), dv.data_ptr(), lp.data_ptr(), lm.data_ptr(),
+                                     lv.data_ptr(), lr, 0.9, 0.999, 1e-8, t))
+        O.leaf_adam(fc, lf, aux_p, aux_m, aux_v, lr, 0.9, 0.999, 1e-8, t)
+        logp_new = fc.logp[pe].astype(np.float32).copy()
+        O.adam_step(params, want_grad.astype(np.float32), m, v, lr, 0.9, 0.999, 1e-8, t, gp, logp_new)
+        fc.logp = fc.logp.copy()
+        fc.logp[pe] = logp_new
+        np.testing.assert_allclose(dp.cpu().numpy(), params, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(lp.cpu().numpy(), aux_p, rtol=1e-4, atol=1e-5)
+        np.testing.assert_allclose(lm.cpu().numpy(), aux_m, rtol=1e-4, atol=1e-6)
+        got = P.vectorize_parameters(bpc)
+        # (m / sqrt(v) carries the gradient's 1e-4 over to parameters whose gradient is near zero: 5e-4 here)
+        np.testing.assert_allclose(np.exp(got[:ns]), np.exp(logp_new), rtol=5e-4)
+        np.testing.assert_array_equal(got[ns:], leaves_before)        # the source never writes the leaves back
+
+
+def test_em_then_adam_raises_the_likelihood(gpu):
+    """The sequence of test/sgd/adam_tests.jl:16-24 on the small single-channel configuration (64 variables,
+    K = 16, 256 categories, 1024 examples): mini-batch EM epochs, then Adam epochs on the same data; every
+    phase raises the training log-likelihood and the Adam phase ends above where EM left off."""
+    torch, P = gpu
+    from pcmi355 import workloads
+    cfg = workloads.make_config("c1_hclt64_k16")
+    bpc = P.hclt_from_clt(cfg["parent"], cfg["C"], cfg["K"])
+    bpc.set_params(cfg["theta"], cfg["leaf"])
+    d = torch.from_numpy(cfg["data"]).cuda()
+    g = torch.Generator().manual_seed(1)
+    em = P.mini_batch_em(bpc, d, 5, batch_size=256, pseudocount=0.1, param_inertia=0.1, param_inertia_end=0.9, generator=g)
+    assert em[-1] > em[0]
+    st = {}
+    lls = P.adam(bpc, d, 6, batch_size=256, lr=1e-2, generator=g, state=st)
+    assert len(lls) == 6 and st["opt_count"] == 24
+    assert lls[-1] > lls[0] and lls[-1] > em[-1]
+    final = float(P.loglikelihoods(bpc, d).mean().item())
+    assert final > em[-1]
