@@ -88,6 +88,17 @@ def _timed(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) / steps
 
 
+def _patch_heads(P, parent, K, C, H, rng):
+    """A patch circuit as the progressive-growing experiments build it: one HCLT body and H head
+    sum nodes over the K products under its root (exps/progressive_growing/parallel_PG.jl:214-225),
+    parameters drawn as `init_parameters(perturbation = 0.4)` draws them."""
+    from pcmi355 import nodes as N
+    body = P.hclt_pc(parent, C, K)
+    heads = [N.summate(list(body.inputs)) for _ in range(H)]
+    N.init_parameters(heads, perturbation=0.4, rng=rng)
+    return heads
+
+
 def secondary(args):
     """The other configurations (not the headline; same JSON shape).  c2: wide block kernels,
     priced against the fp32 matrix peak.  c4: layered engine, whose byte count is its own minimum:
@@ -124,22 +135,14 @@ def secondary(args):
         print(json.dumps(out))
         return
     elif args.workload in ("c4_patch_multihead", "c4_patch_multihead_block"):
-        sys.path.insert(0, os.path.join(ROOT, "tests"))
-        sys.path.insert(0, os.path.join(ROOT, "oracle"))
-        sys.setrecursionlimit(20000)
-        from helpers import multihead_hclt, describe_dag      # DAG builders shared with the tests
         V, K, C, H, B = 192, 32, 256, 128, 1024
         data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
         parent = workloads.chow_liu_parent(data)
-        heads, _ = multihead_hclt(parent, K, C, H, rng)
-        g = describe_dag(heads)
-        bpc = P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"],
-                                g["input_logp"], V, C, H)
-        engine = "layered engine"
-        if args.workload.endswith("_block"):      # the same circuit and parameters on the block engine
-            blk = P.multihead_hclt_from_clt(parent, C, K, H)
-            P.update_parameters(blk, P.vectorize_parameters(bpc))
-            bpc, engine = blk, "block engine"
+        if args.workload.endswith("_block"):      # the same circuit on the block engine
+            bpc, engine = P.multihead_hclt_from_clt(parent, C, K, H), "block engine"
+            bpc.set_params(*workloads.init_params(parent, K, C, 1104, kind="dirichlet"))     # heads stay uniform
+        else:
+            bpc, engine = P.CuMultiHeadBitsProbCircuit(_patch_heads(P, parent, K, C, H, rng), V), "layered engine"
         mask = np.zeros((B, H), np.float32)
         mask[np.arange(B), rng.integers(0, H, size=B)] = 1.0
         d = torch.from_numpy(data).cuda()
@@ -219,17 +222,11 @@ def secondary(args):
     elif args.workload == "c4_patch_x8_streams":
         # eight independent patch circuits (C4 has 64), each queued on one of four streams: the layered engine's
         # per-layer launches are small, so circuits overlap on the device
-        sys.path.insert(0, os.path.join(ROOT, "tests"))
-        sys.path.insert(0, os.path.join(ROOT, "oracle"))
-        sys.setrecursionlimit(20000)
-        from helpers import multihead_hclt, describe_dag
         V, K, C, H, B, NC, NS = 192, 32, 256, 128, 1024, 8, 4
         data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
         parent = workloads.chow_liu_parent(data)
-        heads, _ = multihead_hclt(parent, K, C, H, rng)
-        g = describe_dag(heads)
-        circs = [P.compile_circuit(g["node_type"], g["child_ptr"], g["child_idx"], g["sum_logp"], g["input_var"],
-                                   g["input_logp"], V, C, H) for _ in range(NC)]
+        heads = _patch_heads(P, parent, K, C, H, rng)
+        circs = [P.CuMultiHeadBitsProbCircuit(heads, V) for _ in range(NC)]
         mask = np.zeros((B, H), np.float32)
         mask[np.arange(B), rng.integers(0, H, size=B)] = 1.0
         d = torch.from_numpy(data).cuda()
@@ -354,6 +351,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c3_hclt3072_k32")
+    ap.add_argument("--tree", choices=("chow_liu", "gaussian"), default="chow_liu",
+                    help="chow_liu: learned by the library from 32768 training images; gaussian: host stand-in")
     ap.add_argument("--cpu-sample", type=int, default=4096)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
@@ -376,7 +375,9 @@ def main():
     if args.workload not in workloads.CONFIGS:
         return secondary(args)
 
-    cfg = workloads.make_config(args.workload)
+    # the tree is learned as the reference learns it: pairwise mutual information of a training set and its
+    # maximum spanning tree, both by the library (pcm_pairwise_mi, pcm_chow_liu_tree)
+    cfg = workloads.make_config(args.workload, tree=args.tree)
     stats = workloads.tree_stats(cfg["parent"])
     V, K, C, B = cfg["V"], cfg["K"], cfg["C"], cfg["B"]
     bpc = pcmi355.hclt_from_clt(cfg["parent"], C, K)
@@ -426,7 +427,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
-                   "tree_inner_nodes": stats["n_inner"], "tree_depth": stats["depth"]},
+                   "tree": args.tree, "tree_inner_nodes": stats["n_inner"], "tree_depth": stats["depth"],
+                   "tree_max_children": stats["max_children"]},
         "roofline": {"bound": "hbm", "kernel": KERNEL_NAMES[dominant] % K, "achieved": achieved,
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": measured_traffic(args.workload, dominant)},

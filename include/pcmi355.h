@@ -82,7 +82,9 @@ int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_
                        const float* input_logp, int32_t num_vars, int32_t num_cats,
                        int32_t num_heads, pcm_circuit** out);
 
-/* Releases the circuit and all device memory it owns. */
+/* Releases the circuit and all device memory it owns.  The library keeps a table of the handles it
+ * has given out: every entry point answers PCM_ERR_ARG, without touching the pointer, for a handle
+ * that is null, was freed before or was not created by this library. */
 int pcm_free(pcm_circuit* c);
 
 /* Queue this circuit's work on the given hipStream_t (NULL = null stream). */

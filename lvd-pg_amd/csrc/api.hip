@@ -1,6 +1,8 @@
 // C ABI of pcmi355: argument checks, exception -> status translation.
 #include <algorithm>
+#include <mutex>
 #include <new>
+#include <unordered_set>
 
 #include "common.hpp"
 #include "hclt_engine.hpp"
@@ -26,8 +28,27 @@ int guarded(F&& f) {
   }
 }
 
+// Every handle the library has given out and not yet freed.  A call with any other pointer (freed
+// twice, never created here) is turned down before it is dereferenced.
+std::mutex g_handles_mu;
+std::unordered_set<const pcm_circuit*> g_handles;
+
+void adopt(pcm_circuit* c) {
+  std::lock_guard<std::mutex> lock(g_handles_mu);
+  g_handles.insert(c);
+}
+
 pcm_circuit* need(pcm_circuit* c) {
   if (!c) pcm::fail(PCM_ERR_ARG, "circuit handle is null");
+  std::lock_guard<std::mutex> lock(g_handles_mu);
+  if (!g_handles.count(c)) pcm::fail(PCM_ERR_ARG, "not a live circuit handle (already freed, or not created by this library)");
+  return c;
+}
+
+pcm_circuit* release(pcm_circuit* c) {
+  if (!c) pcm::fail(PCM_ERR_ARG, "circuit handle is null");
+  std::lock_guard<std::mutex> lock(g_handles_mu);
+  if (!g_handles.erase(c)) pcm::fail(PCM_ERR_ARG, "not a live circuit handle (already freed, or not created by this library)");
   return c;
 }
 
@@ -52,7 +73,7 @@ int pcm_hclt_create(const int32_t* clt_parent, int32_t num_vars, int32_t num_hid
   return guarded([&] {
     if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
     *out = nullptr;
-    *out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats);
+    adopt(*out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats));
   });
 }
 
@@ -62,7 +83,7 @@ int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32
     if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
     *out = nullptr;
     if (num_heads < 1) pcm::fail(PCM_ERR_SHAPE, "num_heads must be positive, got %d", num_heads);
-    *out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats, num_heads);
+    adopt(*out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats, num_heads));
   });
 }
 
@@ -73,13 +94,13 @@ int pcm_circuit_create(int32_t num_nodes, const uint8_t* node_type, const int32_
   return guarded([&] {
     if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
     *out = nullptr;
-    *out = new pcm::SparseCircuit(pcm::flatten_dag(num_nodes, node_type, child_ptr, child_idx, sum_logp, input_var,
-                                                   input_logp, num_vars, num_cats, num_heads));
+    adopt(*out = new pcm::SparseCircuit(pcm::flatten_dag(num_nodes, node_type, child_ptr, child_idx, sum_logp, input_var,
+                                                         input_logp, num_vars, num_cats, num_heads)));
   });
 }
 
 int pcm_free(pcm_circuit* c) {
-  return guarded([&] { delete need(c); });
+  return guarded([&] { delete release(c); });
 }
 
 int pcm_set_stream(pcm_circuit* c, void* s) {

@@ -68,10 +68,27 @@ struct DevBuf {
       PCM_HIP(hipStreamSynchronize(s));
     }
   }
+  // On a stream of the caller's the clear is queued like any other work; without one (set-up code) it has
+  // finished when the call returns, so work queued later on any stream finds the memory cleared.
   void zero(hipStream_t s = nullptr) {
-    if (n) PCM_HIP(hipMemsetAsync(p, 0, n * sizeof(T), s));
+    if (!n) return;
+    PCM_HIP(hipMemsetAsync(p, 0, n * sizeof(T), s));
+    if (!s) PCM_HIP(hipStreamSynchronize(nullptr));
   }
 };
+
+// dst[i] += w(i) * (part[0][i] + part[1][i] + ...), the parts added in their order; w(i) = exp(logw[i]) or 1.
+// Kernels that share one sum out among workgroups leave their parts in rows of `part` and this kernel
+// puts them together: no atomics, the same bits on every run.
+template <bool kExpWeight>
+__global__ void sum_parts_kernel(const float* __restrict__ part, int n_parts, int64_t n, const float* __restrict__ logw,
+                                 float* __restrict__ dst) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float s = 0.f;
+  for (int q = 0; q < n_parts; ++q) s += part[(size_t)q * n + i];
+  dst[i] += kExpWeight ? __expf(logw[i]) * s : s;
+}
 
 // A batch of soft evidence: log-evidence per (example, variable, category) with element strides.
 struct SoftRef {

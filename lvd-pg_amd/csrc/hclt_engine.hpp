@@ -229,6 +229,7 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<int64_t> d_sum_param_src_;
   DevBuf<int32_t> d_in_pos_;   // input node (v, j) -> its position among the input nodes of the parameter vector
   DevBuf<float> d_param_vec_;  // a parameter vector on its way to or from the host
+  DevBuf<float> d_part_;       // rows of partial sums (head statistics per slice, soft leaf counts per split)
   DevBuf<float> d_row_sum_;    // Adam from flows: per-sum-node / per-input-node flow totals
   DevBuf<int32_t> d_input_order_;   // i-th input node of the parameter vector -> v*K + j
   int cap_slices_ = 0;

@@ -124,7 +124,7 @@ template <int K>
 __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
     const float* __restrict__ O_root, const float* __restrict__ hwf, const float* __restrict__ hwb,
     const float* __restrict__ head_logp, int H, int Hp, int B, const float* __restrict__ mask, float* __restrict__ R_root,
-    float* __restrict__ head_aggr, int* __restrict__ flow_shift) {
+    float* __restrict__ head_part, int* __restrict__ flow_shift) {
   extern __shared__ float lds[];   // R [16][Hp] | E [16][K] | partial T tiles [waves][16*K] | mask totals [waves][16]
   float* Rl = lds;
   float* El = Rl + 16 * Hp;
@@ -187,13 +187,15 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
     frexpf(tot, &ex);
     if (ex > 0) atomicMax(flow_shift, ex);
   }
-  // head statistics of this slice
+  // head statistics of this slice, without the head weight: row `slice` of head_part [slices][H * K], which
+  // sum_parts_kernel adds up in slice order and weights
+  float* part = head_part + (size_t)slice * H * K;
   for (int o = threadIdx.x; o < H * K; o += blockDim.x) {
     const int h = o / K, j = o % K;
     float a = 0.f;
 #pragma unroll
     for (int bb = 0; bb < 16; ++bb) a += Rl[bb * Hp + h] * El[bb * K + j];
-    if (a != 0.f) atomicAdd(&head_aggr[o], __expf(head_logp[o]) * a);
+    part[o] = a;
   }
 }
 

@@ -154,7 +154,8 @@ __global__ void hclt_soft_scale_kernel(float* __restrict__ p, int64_t n, float r
 }
 
 // leaf_flow[v][c][k] += P[c,k] * sum_b E[b,c] Gs[b,k] over the examples of split blockIdx.z;
-// grid (ceil(C / 64), V, splits), 256 threads.
+// grid (ceil(C / 64), V, splits), 256 threads.  With one split the sum goes straight into leaf_flow; with
+// several, split z leaves its share in row z of part_all [splits][V * C * K] for sum_parts_kernel.
 // G: the child-flow tiles the statistics pass left behind; g_node[v]: the tree node whose tile
 // carries the flow of variable v's leaves (its own node, or its parent's).
 // LDS: E tile [64 examples][68] | Gs [64 examples][K + 4].  Wave w contracts categories
@@ -166,8 +167,9 @@ __global__ __launch_bounds__(256) void hclt_soft_leafflow_kernel(SoftRef s, cons
                                                                  const float* __restrict__ LV, const float* __restrict__ M,
                                                                  const float* __restrict__ G, const int32_t* __restrict__ g_node,
                                                                  int C, int B, int Bp, size_t node_floats, int split_examples,
-                                                                 float* __restrict__ leaf_flow) {
+                                                                 float* __restrict__ leaf_flow, float* __restrict__ part_all) {
   constexpr int KT = K / 16, ELD = kEvCats + 4, LDG = K + 4;
+  float* part = part_all ? part_all + (size_t)blockIdx.z * gridDim.y * C * K : nullptr;
   __shared__ __align__(16) float Et[kEvExamples * ELD];
   __shared__ __align__(16) float Gs[kEvExamples * LDG];
   __shared__ int any_slow;
@@ -275,7 +277,8 @@ __global__ __launch_bounds__(256) void hclt_soft_leafflow_kernel(SoftRef s, cons
     for (int kt = 0; kt < KT; ++kt) {
       const size_t o = ((size_t)v * C + c) * K + kt * 16 + r;
       const float add = __expf(leaf[o]) * acc[kt][i] + accD[kt][i];
-      if (add != 0.f) atomicAdd(&leaf_flow[o], add);
+      if (part) part[o] = add;       // this workgroup is the only writer of the cell either way
+      else leaf_flow[o] += add;
     }
   }
 }

@@ -351,7 +351,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 template <int U, int EX>
 __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const int (&bb)[EX], const bool (&live)[EX],
-                                             float (&acc)[EX], float* __restrict__ edge_aggr) {
+                                             float (&acc)[EX], float* __restrict__ edge_part) {
   float fl[U][EX], ex[U][EX];
   int ies[U];
 #pragma unroll
@@ -384,9 +384,9 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
       acc[x] += ef;
       part += ef;
     }
-    if (!(ies[u] & 1) && edge_aggr) {
+    if (!(ies[u] & 1) && edge_part) {
       const float tot = wave_sum(part);
-      if ((threadIdx.x & 63) == 0) atomicAdd(&edge_aggr[ies[u] >> 1], tot);
+      if ((threadIdx.x & 63) == 0) edge_part[ies[u] >> 1] = tot;   // this wave is the only writer of the cell
     }
   }
 }
@@ -395,18 +395,20 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
 // flows of the node's incoming edges, src/queries/flow.jl:49-60: edge_flow = flows[parent]
 // (product edge) or flows[parent] * exp(mars[prime] + logp (+ mars[sub]) - mars[parent]) (sum
 // edge).  Each edge's flow is summed over the batch where the node is the edge's prime
-// (:73-81): over the thread's examples, then over the wave, then one atomic.
+// (:73-81): over the thread's examples, then over the wave; the wave's sum goes to row blockIdx.y of
+// edge_part ([gridDim.y][n_edges]), whose rows a later kernel adds up in order.
 template <int EX, int kLayerWaves>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
                                                                            const int32_t* __restrict__ seed_of,
                                                                            const float* __restrict__ seed,
-                                                                           float* __restrict__ edge_aggr,
+                                                                           float* __restrict__ edge_part_all, int64_t n_edges,
                                                                            const int32_t* __restrict__ alias_ptr,
                                                                            const int32_t* __restrict__ alias_list) {
   __shared__ float xa[kLayerWaves][EX][64];
   const int n = d.order[n0 + blockIdx.x];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int b0 = blockIdx.y * (64 * EX) + lane;
+  float* edge_part = edge_part_all ? edge_part_all + (size_t)blockIdx.y * n_edges : nullptr;
   int bb[EX];
   bool live[EX];
   float acc[EX];
@@ -424,10 +426,10 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
   int c0 = my0;
-  for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_aggr);
-  for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_aggr);
-  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_aggr);
-  for (; c0 < my1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_aggr);
+  for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_part);
+  for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_part);
+  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_part);
+  for (; c0 < my1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
 #pragma unroll
     for (int x = 0; x < EX; ++x) xa[wave][x][lane] = acc[x];
@@ -459,19 +461,35 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
 
 // Leaf counters, src/nodes/fixable_categorical_dist.jl:121-130: an input node's flow goes to the
 // counter of the example's category.  One workgroup per input node over the whole batch: the
-// node owns its C counters, so they are summed in LDS and added to memory without atomics.
+// node owns its C counters.  They are summed in LDS as 64-bit fixed-point integers, scaled so that
+// the node's largest flow times the batch size still fits: integer sums do not depend on the order
+// the lanes arrive in, so the counters come out the same on every run.
 __global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, const int32_t* __restrict__ input_nodes,
                                                                float* __restrict__ leaf_flow) {
-  __shared__ float hist[256];
+  __shared__ unsigned long long hist[256];
+  __shared__ float wave_max[4];
   const int n = input_nodes[blockIdx.x];
-  for (int c = threadIdx.x; c < d.C; c += blockDim.x) hist[c] = 0.f;
-  __syncthreads();
+  for (int c = threadIdx.x; c < d.C; c += blockDim.x) hist[c] = 0ull;
   const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
   const float* fr = d.flows + (size_t)n * d.Bp;
-  for (int b = threadIdx.x; b < d.B; b += blockDim.x) atomicAdd(&hist[xr[b]], fr[b]);
+  float mx = 0.f;
+  for (int b = threadIdx.x; b < d.B; b += blockDim.x) mx = fmaxf(mx, fr[b]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  if (!(mx > 0.f)) return;                       // no flow reached this node (uniform over the workgroup)
+  int ex = 0;
+  frexpf(mx, &ex);                               // every flow < 2^ex
+  const int shift = 62 - (32 - __clz(d.B)) - ex; // flow * 2^shift < 2^62 / batch
+  for (int b = threadIdx.x; b < d.B; b += blockDim.x) {
+    const float f = fr[b];
+    if (f > 0.f) atomicAdd(&hist[xr[b]], (unsigned long long)ldexpf(f, shift));
+  }
   __syncthreads();
   float* dst = leaf_flow + d.in_off[n];
-  for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += hist[c];
+  for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += ldexpf((float)hist[c], -shift);
 }
 
 // Soft evidence, per variable.  All input nodes of a variable read the same evidence, so a
@@ -1183,16 +1201,27 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     db.in_logp = d_in_logp_.p;
   }
   db.order = d_bwd_order_.p;   // the layers without the input nodes whose rows other nodes write
+  // edge flows summed over the batch: one row of partial sums per 64 examples, cleared first (an edge that
+  // no wave visits must read as zero), added into the accumulators in row order after the walk
+  const int n_parts = Bp / 64;
+  if (ne) {
+    d_edge_part_.ensure((size_t)n_parts * ne);
+    hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)n_parts * ne, 256)), dim3(256), 0, stream, d_edge_part_.p,
+                       (int64_t)n_parts * ne, 0.f);
+  }
   for (int l = n_layers_ - 1; l >= 0; --l) {
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     if (cnt == 0) continue;
     if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
       hipLaunchKernelGGL((sparse_backward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, db, n0,
-                         d_heads_.p, d_head_mask, d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
+                         d_heads_.p, d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
     else
       hipLaunchKernelGGL((sparse_backward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
-                         d_head_mask, d_edge_aggr_.p, d_alias_ptr_.p, d_alias_list_.p);
+                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
   }
+  if (ne)
+    hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 256)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,
+                       (const float*)nullptr, d_edge_aggr_.p);
   if (!fc_.input_nodes.empty()) {
     if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);
     if (soft)

@@ -104,7 +104,7 @@ class SparseCircuit : public pcm_circuit {
   // incoming edges per node (down direction)
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
   DevBuf<int4> d_in_rec_;
-  DevBuf<float> d_in_logp_;
+  DevBuf<float> d_in_logp_, d_edge_part_;
   DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads

@@ -2,11 +2,13 @@
 images, a Chow-Liu tree over them, and seeded parameter draws.  Host-side numpy; this is
 benchmark input preparation, not part of the timed path.
 
-The tree stands in for `learn_chow_liu_tree(data; pseudocount = 0.1)` +
-`clt_edges2graphs` (src/structures/hclts.jl:17-18, both in un-vendored packages): pairwise
-mutual information is taken from the Gaussian closed form -0.5*log(1 - rho^2) of the pixel
-correlations rather than from 256 x 256 contingency tables, the maximum spanning tree is
-exact, and the root is the tree's centre.
+Two trees: `make_config(name, tree="chow_liu")` learns it as the reference does
+(`learn_chow_liu_tree(data; pseudocount = 0.1)` + `clt_edges2graphs`, src/structures/hclts.jl:17-18)
+with the library's own pairwise mutual information and spanning tree, on a training set of
+TRAIN_EXAMPLES images of which the batch is the head; it needs the GPU.  `tree="gaussian"` (the
+default, host only) takes the mutual information from the Gaussian closed form
+-0.5*log(1 - rho^2) of the pixel correlations of the batch; the maximum spanning tree is exact and
+the root is the tree's centre.
 """
 import numpy as np
 
@@ -117,9 +119,22 @@ CONFIGS = {
 }
 
 
-def make_config(name):
+TRAIN_EXAMPLES = 32768      # images the Chow-Liu tree of tree="chow_liu" is learned from
+
+
+def make_config(name, tree="gaussian"):
     h, w, ch, K, C, B, ls, seed = CONFIGS[name]
-    data = grf_images(B, h, w, ch, ls, 0.8, seed)
-    parent = chow_liu_parent(data)
+    if tree == "chow_liu":
+        import torch
+        from .structures import learn_chow_liu_tree
+        train = grf_images(TRAIN_EXAMPLES, h, w, ch, ls, 0.8, seed)
+        parent = learn_chow_liu_tree(torch.from_numpy(train).cuda(), C, 0.1)
+        data = np.ascontiguousarray(train[:B])
+        del train
+    elif tree == "gaussian":
+        data = grf_images(B, h, w, ch, ls, 0.8, seed)
+        parent = chow_liu_parent(data)
+    else:
+        raise ValueError("tree: 'gaussian' or 'chow_liu'")
     theta, leaf = init_params(parent, K, C, seed + 100)
     return dict(name=name, data=data, parent=parent, theta=theta, leaf=leaf, K=K, C=C, B=B, V=h * w * ch)

@@ -59,7 +59,14 @@ def test_version_and_error_reporting_without_a_gpu(cdll):
     cdll.pcm_size.restype = ctypes.c_int64
     assert cdll.pcm_size(None, 0) < 0
     assert cdll.pcm_em_update(None, ctypes.c_float(0.1), ctypes.c_float(0.9)) == -1
-    assert cdll.pcm_free(None) in (0, -1)
+    assert cdll.pcm_free(None) == -1
+    # a pointer the library never gave out is turned down without being touched
+    stray = ctypes.create_string_buffer(64)
+    h = ctypes.cast(stray, ctypes.c_void_p)
+    assert cdll.pcm_size(h, 0) < 0
+    assert cdll.pcm_em_update(h, ctypes.c_float(0.1), ctypes.c_float(0.9)) == -1
+    assert cdll.pcm_free(h) == -1 and b"live" in cdll.pcm_last_error()
+    assert stray.raw == bytes(64)
     # structure learning and soft evidence: argument errors come back as status codes
     i64, f32 = ctypes.c_int64, ctypes.c_float
     assert cdll.pcm_pairwise_mi(None, i64(1), i64(1), i64(10), 3, 4, f32(0.1), None, None) == -1

@@ -404,3 +404,40 @@ def test_error_paths(gpu):
         L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.9))
     with pytest.raises(ValueError):      # wrong number of variables
         P.loglikelihoods(bpc, torch.zeros((4, 2), dtype=torch.uint8, device="cuda"))
+
+
+def test_statistics_are_the_same_bits_on_every_run(gpu, oracle):
+    """No floating-point atomics anywhere on the path: the accumulated edge and leaf statistics of a batch
+    are identical, bit for bit, however often the pass is repeated -- layered engine with heads, block
+    engine with heads, and the block engine on soft evidence."""
+    torch, P = gpu
+    from helpers import multihead_hclt
+    rng = np.random.default_rng(11)
+    V, K, C, H, B = 24, 16, 32, 12, 700
+    parent = np.array([-1] + [int(rng.integers(0, v)) for v in range(1, V)], np.int32)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    data = torch.from_numpy(rng.integers(0, C, size=(B, V)).astype(np.uint8)).cuda()
+    mask = torch.from_numpy(rng.dirichlet(np.ones(H), size=B).astype(np.float32)).cuda()
+    layered = _compile(P, heads, V, C, H)
+    block = P.multihead_hclt_from_clt(parent, C, K, H)
+    P.update_parameters(block, P.vectorize_parameters(layered))
+    soft = P.hclt_from_clt(parent, C, K)
+    ev = torch.from_numpy((rng.normal(-30, 3, (B, V, 1)) + rng.gumbel(0, 2, (B, V, C))).astype(np.float32)).cuda()
+
+    from pcmi355._lib import lib, check
+
+    def stats(c, x, hm):
+        P.update_parameters(c, start[id(c)])
+        P.probs_flows_circuit(c, x, head_mask=hm)
+        agg = c.get_aggregates() if c is layered else c.get_flows()
+        check(lib.pcm_em_update(c.handle, 0.1, 0.9))            # the head statistics show in the updated parameters
+        return (*agg, P.vectorize_parameters(c))
+
+    start = {id(c): P.vectorize_parameters(c) for c in (layered, block, soft)}
+    for c, x, hm in ((layered, data, mask), (block, data, mask), (soft, ev, None)):
+        first = stats(c, x, hm)
+        for _ in range(4):
+            again = stats(c, x, hm)
+            for a, b in zip(first, again):
+                assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+        assert all(np.isfinite(a).all() for a in first) and first[0].sum() > 0 and first[1].sum() > 0

@@ -110,6 +110,22 @@ def test_degenerate_inputs(gpu, oracle):
                                  param_inertia=0.5)
 
 
+def test_a_freed_handle_is_refused(gpu):
+    """The C ABI keeps a table of live handles: a second free, or any call on a freed handle, comes
+    back as an argument error instead of touching freed memory."""
+    import ctypes
+    torch, P = gpu
+    from pcmi355._lib import lib
+    par = (ctypes.c_int32 * 3)(-1, 0, 0)
+    h = ctypes.c_void_p()
+    assert lib.pcm_hclt_create(par, 3, 16, 8, ctypes.byref(h)) == 0
+    assert lib.pcm_size(h, 0) > 0
+    assert lib.pcm_free(h) == 0
+    assert lib.pcm_free(h) == -1
+    assert lib.pcm_size(h, 0) < 0
+    assert lib.pcm_em_update(h, ctypes.c_float(0.1), ctypes.c_float(0.9)) == -1
+
+
 @pytest.mark.parametrize("K", [16, 32, 64, 128, 8])
 def test_examples_of_probability_zero_carry_no_flow(gpu, oracle, K):
     """A leaf that forbids a category makes the examples showing it impossible: their value is
