@@ -647,20 +647,23 @@ __global__ __launch_bounds__(kStatWaves * 64) void hclt_stats_kernel(
     __syncthreads();
   }
 
-  // combine the waves' partial A through LDS, scale by W, write the node's block once
-  // (floating-point LDS atomics: K*K per wave per node, negligible)
+  // combine the waves' partial A through LDS, scale by W, write the node's block once.  A wave's lanes hold
+  // every cell of the block exactly once, so the waves add their blocks in turn, wave 0 first: plain
+  // read-modify-writes in a fixed order, the same sum on every run
   float* abuf = smem;
   for (int i = threadIdx.x; i < K * K; i += blockDim.x) abuf[i] = 0.f;
   __syncthreads();
+  for (int turn = 0; turn < (int)(blockDim.x >> 6); ++turn) {
+    if (turn == (int)(threadIdx.x >> 6)) {
 #pragma unroll
-  for (int kt = 0; kt < KT; ++kt)
+      for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-    for (int jt = 0; jt < KT; ++jt)
+        for (int jt = 0; jt < KT; ++jt)
 #pragma unroll
-      for (int v = 0; v < 4; ++v)
-        __hip_atomic_fetch_add(&abuf[(kt * 16 + 4 * g + v) * K + jt * 16 + b], accA[kt][jt][v],
-                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  __syncthreads();
+          for (int v = 0; v < 4; ++v) abuf[(kt * 16 + 4 * g + v) * K + jt * 16 + b] += accA[kt][jt][v];
+    }
+    __syncthreads();
+  }
   float* dst = edge_aggr + (size_t)n * K * K;
   const float* lt = d.logtheta + (size_t)n * K * K;
   for (int i = threadIdx.x; i < K * K; i += blockDim.x) {
