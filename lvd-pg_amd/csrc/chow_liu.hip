@@ -223,8 +223,7 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
     lds = ((size_t)((band * C + 1) & ~1)) * 4 + red_bytes;
   }
   if (lds > (size_t)max_lds) fail(PCM_ERR_UNSUPPORTED, "pair table needs %zu bytes of LDS, device offers %d", lds, max_lds);
-  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(sh.Np, 64), ceil_div(V, 64)), dim3(256), 0, stream, d_data, stride_ex,
-                     stride_var, (const int32_t*)nullptr, N, sh.Np, V, C, w.xb);
+  pcm_stage(d_data, stride_ex, stride_var, nullptr, N, sh.Np, V, C, w.xb, stream);
   hipLaunchKernelGGL(mi_single_kernel, dim3(V), dim3(256), 0, stream, w.xb, N, sh.Np, C, pseudocount, w.stat);
   hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div((int64_t)N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, w.f);
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;

@@ -945,10 +945,9 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
   ensure_batch(b.batch);
   const int Bp = ceil_div(b.batch, kSlice) * kSlice;
-  hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(V_, 64)), dim3(256), 0, stream,
-                     b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p);
+  pcm_stage(b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p, stream);
   check_launch("stage_batch");
-  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
+  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 1024), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
   check_launch("pack_x");
 }
@@ -1082,7 +1081,7 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
   if ((size_t)d.Bp * K_ * 4 >= ((size_t)1 << 31)) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", s.batch);
   const int64_t nx = (int64_t)V_ * d.Bp;
   hipLaunchKernelGGL(hclt_soft_x_kernel, dim3(ceil_div(nx, 256)), dim3(256), 0, stream, d_xb_.p, nx);
-  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(d.Bp, 256), n_inner_), dim3(256), 0, stream, d_nodes_.p,
+  hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(d.Bp, 1024), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, d.Bp, d_xn_.p);
   check_launch("soft pack_x");
   const int Bp64 = ceil_div(d.Bp, kEvExamples) * kEvExamples;
@@ -1321,9 +1320,17 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4)), dim3(256), 0, stream, head_logp(), head_aggr(), H_, Hp_,
                        K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
   }
-  // few variables: more category groups per workgroup, for the latency of the two passes
-  hipLaunchKernelGGL(hclt_leaf_update_kernel, dim3(V_, ceil_div(K_, 32)), dim3(V_ * ceil_div(K_, 32) < 1024 ? 1024 : 256), 0,
-                     stream, d_leaf_.p, d_leaf_flow_.p, C_, K_, pseudocount, inertia);
+  // 32 category groups per workgroup; a thread holds its group's share of the categories (8 of 256)
+  {
+    const int threads = 1024, cats = ceil_div(C_, threads / 32);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, dim3(V_, ceil_div(K_, 32)), dim3(threads), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
+                         pseudocount, inertia);
+    };
+    if (cats <= 8) launch(&hclt_leaf_update_kernel<8>);
+    else if (cats <= 16) launch(&hclt_leaf_update_kernel<16>);
+    else launch(&hclt_leaf_update_kernel<32>);
+  }
   check_launch("leaf_update");
   general_stale_ = true;
 }

@@ -769,9 +769,12 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
 }
 
 // Leaf update (the reference's per-input-node update with missing_flow = 0), one workgroup
-// per (variable, run of 32 hidden states): thread (category group cg, hidden state j) first
-// sums the flows of its categories, the groups are combined through LDS, then every thread
-// rewrites its categories.  Consecutive threads touch consecutive addresses in both passes.
+// per (variable, run of 32 hidden states): thread (category group cg, hidden state j) holds the
+// flows and parameters of its categories (every kCats-th one) in registers -- all of its requests
+// are in flight at once, and nothing is read twice -- sums its flows, the groups are combined
+// through LDS, then every thread rewrites its categories.  Consecutive threads touch consecutive
+// addresses.  blockDim.x * kCats >= 32 * C.
+template <int kCats>
 __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restrict__ leaf,
                                                                const float* __restrict__ leaf_flow, int C, int K,
                                                                float pseudocount, float inertia) {
@@ -782,35 +785,51 @@ __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restric
   const bool valid = j < K;
   float* lp = leaf + (size_t)u * C * K;
   const float* fl = leaf_flow + (size_t)u * C * K;
+  float f[kCats], p[kCats];
+#pragma unroll
+  for (int q = 0; q < kCats; ++q) {
+    const int c = cg + q * ncg;
+    const bool in = valid && c < C;
+    f[q] = in ? fl[(size_t)c * K + j] : 0.f;
+    p[q] = in ? lp[(size_t)c * K + j] : 0.f;
+  }
   float s = 0.f;
-  if (valid)
-    for (int c = cg; c < C; c += ncg) s += fl[(size_t)c * K + j];
+#pragma unroll
+  for (int q = 0; q < kCats; ++q) s += f[q];
   part[threadIdx.x] = s;
   __syncthreads();
   if (!valid) return;
   float node_flow = pseudocount;
   for (int q = 0; q < ncg; ++q) node_flow += part[q * 32 + jl];
-  const float cat_pc = pseudocount / (float)C;
-  for (int c = cg; c < C; c += ncg) {
-    const size_t i = (size_t)c * K + j;
-    const float oldv = inertia * expf(lp[i]);
-    const float newv = (1.f - inertia) * (fl[i] + cat_pc) / node_flow;
-    lp[i] = logf(oldv + newv);
+  const float cat_pc = pseudocount / (float)C, scale = (1.f - inertia) / node_flow;
+#pragma unroll
+  for (int q = 0; q < kCats; ++q) {
+    const int c = cg + q * ncg;
+    if (c < C) lp[(size_t)c * K + j] = __logf(inertia * __expf(p[q]) + (f[q] + cat_pc) * scale);
   }
 }
 
 // xn[node][example] = categories of the node's own variable (byte 0) and of its first three
-// leaf children (bytes 1..3), so that a wave fetches all of them with one request.
+// leaf children (bytes 1..3), so that a wave fetches all of them with one request.  A thread makes
+// the words of four examples (Bp is a multiple of 16): one word of four categories in per variable,
+// one request of four words out.
 __global__ void hclt_pack_x_kernel(const HcltNode* __restrict__ nodes, const int32_t* __restrict__ child_leaf,
                                    const uint8_t* __restrict__ xb, int n_inner, int Bp,
                                    uint32_t* __restrict__ xn) {
-  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = 4 * (blockIdx.x * blockDim.x + threadIdx.x);
   const int n = blockIdx.y;
   if (b >= Bp) return;
   const HcltNode nd = nodes[n];
-  uint32_t v = xb[(size_t)nd.var * Bp + b];
-  for (int i = 0; i < nd.lc_cnt && i < 3; ++i) v |= (uint32_t)xb[(size_t)child_leaf[nd.lc_off + i] * Bp + b] << (8 * (i + 1));
-  xn[(size_t)n * Bp + b] = v;
+  uint32_t in[4] = {*reinterpret_cast<const uint32_t*>(xb + (size_t)nd.var * Bp + b), 0u, 0u, 0u};
+  for (int i = 0; i < nd.lc_cnt && i < 3; ++i)
+    in[i + 1] = *reinterpret_cast<const uint32_t*>(xb + (size_t)child_leaf[nd.lc_off + i] * Bp + b);
+  uint4 out;
+  uint32_t* o = &out.x;
+#pragma unroll
+  for (int e = 0; e < 4; ++e)
+    o[e] = ((in[0] >> (8 * e)) & 0xffu) | ((in[1] >> (8 * e)) & 0xffu) << 8 | ((in[2] >> (8 * e)) & 0xffu) << 16 |
+           ((in[3] >> (8 * e)) & 0xffu) << 24;
+  *reinterpret_cast<uint4*>(xn + (size_t)n * Bp + b) = out;
 }
 
 }  // namespace pcm

@@ -1121,8 +1121,7 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
   d_visit_.ensure((size_t)std::max<int64_t>((int64_t)fc_.num_vars, fc_.n_nodes()) * Bp);
   uint8_t* xb = d_visit_.p;
   if (b) {
-    hipLaunchKernelGGL(pcm_stage_kernel, dim3(ceil_div(Bp, 64), ceil_div(fc_.num_vars, 64)), dim3(256), 0, stream,
-                       b->d_data, b->stride_ex, b->stride_var, b->d_idx, batch, Bp, fc_.num_vars, fc_.num_cats, xb);
+    pcm_stage(b->d_data, b->stride_ex, b->stride_var, b->d_idx, batch, Bp, fc_.num_vars, fc_.num_cats, xb, stream);
     check_launch("stage_batch");
   }
   SparseDev d = SPARSE_DEV(batch, Bp, xb);
