@@ -247,7 +247,16 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
  * gradients with respect to the rows of params1 / params2; d_klds may be NULL.
  * pcm_gumbel_sample_rows: d_noise is [rows][num sum parameters] (dense, one draw per sum edge) or NULL for
  * no_gumbel = true; d_out [rows][num_vars][num_cats].
- * All three queue their work on the circuit's stream and do not wait for it.  At most 65535 rows per call.
+ * pcm_gumbel_sample_backward_rows: the reverse pass of pcm_gumbel_sample_rows, `gumbel_sample_backward(mbpc,
+ * params, input_aggr_params, input_aggr_grads, temperature; norm_params, grad_wrt_logparams)`
+ * (src/queries/sample.jl:389-650; src/utils/cuda_preallocation.jl:205-218).  d_out_grads [rows][num_vars][num_cats]
+ * is the gradient of a loss with respect to the soft output; d_param_grads (the strides of the parameter matrix)
+ * receives its gradient with respect to every parameter, for the same d_params, d_noise and temperature as the
+ * forward call (the top-down probabilities are rebuilt, nothing is kept between the two calls).  Sum parameters:
+ * with respect to the log-parameter, or divided by the edge's share of its node when grad_wrt_logparams == 0
+ * (:466-469).  Leaf parameters: with respect to the PROBABILITY of the category, whatever norm_params says, as
+ * the source writes it (:560-570).
+ * All of these queue their work on the circuit's stream and do not wait for it.  At most 65535 rows per call.
  */
 int pcm_kld_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row, int64_t stride_param,
                  int32_t rows, int32_t norm_params, float* d_klds);
@@ -256,6 +265,9 @@ int pcm_kld_backward_rows(pcm_circuit* c, const float* d_params1, const float* d
                           float* d_klds);
 int pcm_gumbel_sample_rows(pcm_circuit* c, const float* d_params, int64_t stride_row, int64_t stride_param, int32_t rows,
                            const float* d_noise, float temperature, int32_t norm_params, float* d_out);
+int pcm_gumbel_sample_backward_rows(pcm_circuit* c, const float* d_params, int64_t stride_row, int64_t stride_param,
+                                    int32_t rows, const float* d_noise, float temperature, int32_t norm_params,
+                                    int32_t grad_wrt_logparams, const float* d_out_grads, float* d_param_grads);
 
 /*
  * Soft evidence: the same two queries with a three-dimensional data argument, as the reference

@@ -265,6 +265,15 @@ int pcm_gumbel_sample_rows(pcm_circuit* c, const float* d_params, int64_t stride
   });
 }
 
+int pcm_gumbel_sample_backward_rows(pcm_circuit* c, const float* d_params, int64_t stride_row, int64_t stride_param,
+                                    int32_t rows, const float* d_noise, float temperature, int32_t norm_params,
+                                    int32_t grad_wrt_logparams, const float* d_out_grads, float* d_param_grads) {
+  return guarded([&] {
+    need(c)->gumbel_sample_backward_rows(d_params, stride_row, stride_param, rows, d_noise, temperature, norm_params != 0,
+                                         grad_wrt_logparams != 0, d_out_grads, d_param_grads);
+  });
+}
+
 int pcm_loglikelihoods_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var,
                             int64_t stride_cat, const int32_t* d_example_ids, int32_t batch, float* d_ll) {
   return guarded([&] {

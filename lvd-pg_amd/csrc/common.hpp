@@ -149,4 +149,7 @@ struct pcm_circuit {
                                  bool norm_params, float* d_g1, float* d_g2, float* d_klds) = 0;
   virtual void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                   float temperature, bool norm_params, float* d_out) = 0;
+  virtual void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                           float temperature, bool norm_params, bool grad_wrt_logparams,
+                                           const float* d_out_grad, float* d_grads) = 0;
 };

@@ -166,6 +166,12 @@ class HcltCircuit : public pcm_circuit {
                           float temperature, bool norm_params, float* d_out) override {
     general_structure()->gumbel_sample_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params, d_out);
   }
+  void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                   float temperature, bool norm_params, bool grad_wrt_logparams, const float* d_out_grad,
+                                   float* d_grads) override {
+    general_structure()->gumbel_sample_backward_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params,
+                                                     grad_wrt_logparams, d_out_grad, d_grads);
+  }
 
   bool sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out);
   void set_block_params(const float* theta, const float* leaf);

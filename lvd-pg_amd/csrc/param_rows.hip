@@ -32,7 +32,7 @@ void check_launch_r(const char* what) {
 
 struct RowsDev {
   const uint8_t* type;
-  const int32_t *order, *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_ptr, *in_edge, *e2p, *p2e, *input_nodes;
+  const int32_t *order, *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_ptr, *in_edge, *e2p, *p2e, *input_nodes, *in_var;
   int64_t n_nodes, n_edges, n_sum, n_par;
   int32_t C, n_inputs;
 };
@@ -281,6 +281,83 @@ __global__ __launch_bounds__(256) void rows_soft_leaf_kernel(RowsDev d, const in
   }
 }
 
+// ---- relaxed sampling, reverse pass --------------------------------------------------------------------
+// Input nodes, a wave per (input node, row): gumbel_input_sample_up_kernel, sample.jl:531-598.  The leaf part
+// of the gradient matrix is the gradient with respect to the PROBABILITY of the category (og * td), with
+// probability-valued parameters or not, as the source writes it (:560-570); the node's own gradient is the
+// output gradient weighted by its distribution.
+template <bool kNorm>
+__global__ __launch_bounds__(256) void rows_soft_back_leaf_kernel(RowsDev d, int V, const float* __restrict__ P,
+                                                                  const float* __restrict__ td, const float* __restrict__ og,
+                                                                  float* __restrict__ grads, float* __restrict__ G) {
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int r = blockIdx.y;
+  if (i >= d.n_inputs) return;
+  const int node = d.input_nodes[i];
+  const size_t at = (size_t)r * d.n_par + d.n_sum + (size_t)i * d.C;
+  const float* o = og + ((size_t)r * V + d.in_var[node]) * d.C;
+  const float t = td[(size_t)r * d.n_nodes + node];
+  float acc = 0.f;
+  for (int c = lane; c < d.C; c += 64) {
+    const float x = P[at + c], oc = o[c];
+    G[at + c] = oc * t;
+    acc += (kNorm ? x : expf(x)) * oc;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (lane == 0) grads[(size_t)r * d.n_nodes + node] = acc;
+}
+
+// One layer of inner nodes, children first, a lane group per (node, row): gumbel_params_up_layer_kernel,
+// sample.jl:391-480.  A sum node's edges share the node's probability as w = softmax((logp + g) / T); the
+// gradient passes through that softmax: edge gradient (child_grad * td - sum_e' child_grad' * td * w') * w / T
+// (without the last w when the gradient is wanted per probability, :466-469).  The group owns the node, so
+// the two sums are lane reductions: nothing is accumulated in memory.
+__global__ __launch_bounds__(kGroup * kGroupsPerBlock) void rows_soft_back_up_kernel(
+    RowsDev d, int n0, int n1, const float* __restrict__ P, const float* __restrict__ noise, float inv_t,
+    const float* __restrict__ emax, const float* __restrict__ esum, const float* __restrict__ td, int wrt_log,
+    float* __restrict__ grads, float* __restrict__ G) {
+  const int l = threadIdx.x % kGroup;
+  const int i = n0 + blockIdx.x * kGroupsPerBlock + threadIdx.x / kGroup;
+  const int r = blockIdx.y;
+  if (i >= n1) return;
+  const int n = d.order[i];
+  const bool issum = d.type[n] == kSum;
+  const float* p = P + (size_t)r * d.n_par;
+  const float* g = noise ? noise + (size_t)r * d.n_sum : nullptr;
+  float* gr = grads + (size_t)r * d.n_nodes;
+  const float t = td[(size_t)r * d.n_nodes + n];
+  const float em = issum ? emax[(size_t)r * d.n_nodes + n] : 0.f, es = issum ? esum[(size_t)r * d.n_nodes + n] : 1.f;
+  float acc = 0.f, cum = 0.f;
+  for (int e = d.node_e0[n] + l; e < d.node_e1[n]; e += kGroup) {
+    float child = gr[d.e_prime[e]];
+    const int s = d.e_sub[e];
+    if (s >= 0) child += gr[s];
+    if (issum) {
+      const int pid = d.e2p[e];
+      const float w = expf((p[pid] + (g ? g[pid] : 0.f)) * inv_t - em) / es;
+      cum += child * t * w;
+      child *= w;
+    }
+    acc += child;
+  }
+  acc = group_sum(acc);
+  if (issum) {
+    cum = group_sum(cum);
+    float* out = G + (size_t)r * d.n_par;
+    for (int e = d.node_e0[n] + l; e < d.node_e1[n]; e += kGroup) {
+      float child = gr[d.e_prime[e]];
+      const int s = d.e_sub[e];
+      if (s >= 0) child += gr[s];
+      const int pid = d.e2p[e];
+      const float w = expf((p[pid] + (g ? g[pid] : 0.f)) * inv_t - em) / es;
+      out[pid] = (child * t - cum) * (wrt_log ? w : 1.f) * inv_t;
+    }
+  }
+  if (l == 0) gr[n] = acc;
+}
+
 }  // namespace
 
 // ---- host -------------------------------------------------------------------------------------------
@@ -288,7 +365,7 @@ __global__ __launch_bounds__(256) void rows_soft_leaf_kernel(RowsDev d, const in
 struct SparseCircuit::RowsState {
   DevBuf<int32_t> e2p, input_nodes, var_ptr, var_inputs;
   DevBuf<float> pk1, pk2, pg1, pg2;        // matrices re-laid out to unit parameter stride
-  DevBuf<float> node_a, node_b, node_c, edge_a;   // [rows][n_nodes] x 3, [rows][n_edges]
+  DevBuf<float> node_a, node_b, node_c, node_d, edge_a;   // [rows][n_nodes] x 4, [rows][n_edges]
 };
 
 SparseCircuit::~SparseCircuit() {}
@@ -296,9 +373,10 @@ SparseCircuit::~SparseCircuit() {}
 static RowsDev rows_dev(const SparseCircuit& c, const FlatCircuit& fc, const SparseCircuit::RowsState& st,
                         const uint8_t* type, const int32_t* order, const int32_t* e0, const int32_t* e1, const int32_t* ep,
                         const int32_t* epr, const int32_t* es, const int32_t* in_ptr, const int32_t* in_edge,
-                        const int32_t* p2e) {
+                        const int32_t* p2e, const int32_t* in_var) {
   (void)c;
   RowsDev d;
+  d.in_var = in_var;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
   d.in_ptr = in_ptr; d.in_edge = in_edge; d.e2p = st.e2p.p; d.p2e = p2e; d.input_nodes = st.input_nodes.p;
   d.n_nodes = fc.n_nodes(); d.n_edges = fc.n_edges(); d.n_sum = (int64_t)fc.param2edge.size();
@@ -328,7 +406,7 @@ SparseCircuit::RowsState& SparseCircuit::rows_state() {
 
 #define ROWS_DEV(st)                                                                                              \
   rows_dev(*this, fc_, st, d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, \
-           d_in_ptr_.p, d_in_edge_.p, d_param2edge_.p)
+           d_in_ptr_.p, d_in_edge_.p, d_param2edge_.p, d_in_var_.p)
 
 namespace {
 void check_rows_args(const SparseCircuit& c, const FlatCircuit& fc, const void* p, int64_t sr, int64_t sp, int rows) {
@@ -422,6 +500,22 @@ void SparseCircuit::kld_backward_rows(const float* d_p1, const float* d_p2, int6
   check_launch_r("rows_kld_backward");
 }
 
+// emax / esum / td of every node and row (node_a, node_b, node_c): the top-down half both directions share
+void SparseCircuit::soft_rows_down(const float* p, int rows, const float* d_noise, float inv_t) {
+  RowsState& st = rows_state();
+  const RowsDev d = ROWS_DEV(st);
+  st.node_a.ensure((size_t)rows * d.n_nodes);
+  st.node_b.ensure((size_t)rows * d.n_nodes);
+  st.node_c.ensure((size_t)rows * d.n_nodes);
+  hipLaunchKernelGGL(rows_soft_norm_kernel, dim3((unsigned)ceil_div(d.n_nodes, kGroupsPerBlock), rows),
+                     dim3(kGroup * kGroupsPerBlock), 0, stream, d, p, d_noise, inv_t, st.node_a.p, st.node_b.p);
+  for (int l = n_layers_ - 1; l >= 0; --l) {
+    const int n0 = layer_node0_[l], n1 = layer_node0_[l + 1];
+    hipLaunchKernelGGL(rows_soft_down_kernel, dim3(ceil_div(n1 - n0, kGroupsPerBlock), rows), dim3(kGroup * kGroupsPerBlock), 0,
+                       stream, d, n0, n1, p, d_noise, inv_t, st.node_a.p, st.node_b.p, st.node_c.p);
+  }
+}
+
 void SparseCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                        float temperature, bool norm, float* d_out) {
   check_rows_args(*this, fc_, d_params, sr, sp, rows);
@@ -430,18 +524,8 @@ void SparseCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_
   RowsState& st = rows_state();
   const int64_t n = size(0);
   const float* p = packed_in(d_params, sr, sp, rows, n, st.pk1, stream);
+  soft_rows_down(p, rows, d_noise, 1.f / temperature);
   const RowsDev d = ROWS_DEV(st);
-  st.node_a.ensure((size_t)rows * d.n_nodes);
-  st.node_b.ensure((size_t)rows * d.n_nodes);
-  st.node_c.ensure((size_t)rows * d.n_nodes);
-  const float inv_t = 1.f / temperature;
-  hipLaunchKernelGGL(rows_soft_norm_kernel, dim3((unsigned)ceil_div(d.n_nodes, kGroupsPerBlock), rows),
-                     dim3(kGroup * kGroupsPerBlock), 0, stream, d, p, d_noise, inv_t, st.node_a.p, st.node_b.p);
-  for (int l = n_layers_ - 1; l >= 0; --l) {
-    const int n0 = layer_node0_[l], n1 = layer_node0_[l + 1];
-    hipLaunchKernelGGL(rows_soft_down_kernel, dim3(ceil_div(n1 - n0, kGroupsPerBlock), rows), dim3(kGroup * kGroupsPerBlock), 0,
-                       stream, d, n0, n1, p, d_noise, inv_t, st.node_a.p, st.node_b.p, st.node_c.p);
-  }
   const dim3 lgrid(fc_.num_vars, rows);
   const int threads = std::min(256, ceil_div(fc_.num_cats, 64) * 64);
   if (norm) hipLaunchKernelGGL(rows_soft_leaf_kernel<true>, lgrid, dim3(threads), 0, stream, d, st.var_ptr.p, st.var_inputs.p,
@@ -449,6 +533,42 @@ void SparseCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_
   else hipLaunchKernelGGL(rows_soft_leaf_kernel<false>, lgrid, dim3(threads), 0, stream, d, st.var_ptr.p, st.var_inputs.p,
                           fc_.num_vars, p, st.node_c.p, d_out);
   check_launch_r("rows_gumbel_sample");
+}
+
+void SparseCircuit::gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                                float temperature, bool norm, bool wrt_log, const float* d_out_grad,
+                                                float* d_grads) {
+  check_rows_args(*this, fc_, d_params, sr, sp, rows);
+  if (!d_out_grad || !d_grads) fail(PCM_ERR_ARG, "gradient pointer is null");
+  if (!(temperature > 0.f)) fail(PCM_ERR_ARG, "temperature must be positive");
+  RowsState& st = rows_state();
+  const int64_t n = size(0);
+  const float* p = packed_in(d_params, sr, sp, rows, n, st.pk1, stream);
+  const float inv_t = 1.f / temperature;
+  soft_rows_down(p, rows, d_noise, inv_t);
+  const RowsDev d = ROWS_DEV(st);
+  st.node_d.ensure((size_t)rows * d.n_nodes);
+  const bool direct = sp == 1 && sr == n;
+  float* g = d_grads;
+  if (!direct) {
+    st.pg1.ensure((size_t)rows * n);
+    g = st.pg1.p;
+  }
+  const dim3 lgrid(ceil_div(d.n_inputs, 4), rows);
+  if (norm) hipLaunchKernelGGL(rows_soft_back_leaf_kernel<true>, lgrid, dim3(256), 0, stream, d, fc_.num_vars, p, st.node_c.p,
+                               d_out_grad, st.node_d.p, g);
+  else hipLaunchKernelGGL(rows_soft_back_leaf_kernel<false>, lgrid, dim3(256), 0, stream, d, fc_.num_vars, p, st.node_c.p,
+                          d_out_grad, st.node_d.p, g);
+  for (int l = 1; l < n_layers_; ++l) {
+    const int n0 = layer_node0_[l], n1 = layer_node0_[l + 1];
+    hipLaunchKernelGGL(rows_soft_back_up_kernel, dim3(ceil_div(n1 - n0, kGroupsPerBlock), rows), dim3(kGroup * kGroupsPerBlock), 0,
+                       stream, d, n0, n1, p, d_noise, inv_t, st.node_a.p, st.node_b.p, st.node_c.p, wrt_log ? 1 : 0, st.node_d.p, g);
+  }
+  if (!direct) {
+    const dim3 tgrid((unsigned)ceil_div(n, 32), ceil_div(rows, 32));
+    hipLaunchKernelGGL(rows_relayout_kernel<false>, tgrid, dim3(256), 0, stream, g, d_grads, sr, sp, rows, n);
+  }
+  check_launch_r("rows_gumbel_sample_backward");
 }
 
 }  // namespace pcm

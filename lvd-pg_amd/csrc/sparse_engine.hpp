@@ -75,6 +75,10 @@ class SparseCircuit : public pcm_circuit {
                          float* d_g1, float* d_g2, float* d_klds) override;
   void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                           float temperature, bool norm_params, float* d_out) override;
+  void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                   float temperature, bool norm_params, bool grad_wrt_logparams, const float* d_out_grad,
+                                   float* d_grads) override;
+  void soft_rows_down(const float* p, int rows, const float* d_noise, float inv_t);
   struct RowsState;   // tables and scratch of the parameter-row queries (param_rows.hip)
 
   void get_node_values(float* mars, float* flows, int64_t n);

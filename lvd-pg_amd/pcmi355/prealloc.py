@@ -11,7 +11,7 @@ parameters are neither read nor changed.  Host arrays in, host arrays out, as th
 import numpy as np
 import torch
 
-from .queries import kld, kld_backward, gumbel_sample_rows, _rows_on_device
+from .queries import kld, kld_backward, gumbel_sample_rows, gumbel_sample_backward_rows, _rows_on_device
 
 _state = {}
 
@@ -56,11 +56,12 @@ def kld_backward_with_prealloc(mbpc, *, norm_params=False, grad_wrt_logparams=Tr
 
 def gumbel_sample_preallocation(mbpc, *, num_examples, num_vars, par_buffer_size, allocate_for_grad=False,
                                 allocate_for_target=False):
-    if allocate_for_grad or allocate_for_target:
-        raise NotImplementedError("the reverse pass of the relaxed sampler is not built")
+    if allocate_for_target:
+        raise NotImplementedError("gumbel_sample_target_with_prealloc (parameter targets) is not built")
     if num_vars != mbpc.size("variables") or par_buffer_size < mbpc.size("categories"):
         raise ValueError("num_vars / par_buffer_size do not fit the circuit")
-    _state["sample"] = dict(num_examples=int(num_examples), num_vars=int(num_vars), width=int(par_buffer_size), mbpc=mbpc)
+    _state["sample"] = dict(num_examples=int(num_examples), num_vars=int(num_vars), width=int(par_buffer_size), mbpc=mbpc,
+                            grad=bool(allocate_for_grad), last=None)
 
 
 def gumbel_sample_free_mem(allocate_for_grad=False, allocate_for_target=False):
@@ -85,7 +86,29 @@ def gumbel_sample_with_prealloc(mbpc, params, *, temperature, no_gumbel=False, n
         u = torch.rand((p.shape[0], mbpc.num_inner_params()), device=p.device, generator=generator)
         noise = -torch.log(-torch.log(u * (1.0 - 1e-6) + 1e-6))
     soft = gumbel_sample_rows(mbpc, p, temperature=temperature, noise=noise, norm_params=norm_params)
+    st["last"] = (p, noise)                      # the reverse pass runs on the same parameters and draws
     C = mbpc.size("categories")
     out = np.zeros((p.shape[0], st["num_vars"], st["width"]), np.float32)
     out[:, :, :C] = soft.cpu().numpy()
     return out
+
+
+def gumbel_sample_backward_with_prealloc(mbpc, input_aggr_grads, *, temperature, norm_params=False, grad_wrt_logparams=True):
+    """`gumbel_sample_backward_with_prealloc(mbpc, input_aggr_grads; temperature, norm_params,
+    grad_wrt_logparams)` (:205-218): gradients with respect to the parameter rows of the last
+    `gumbel_sample_with_prealloc` call, given the gradients [num_examples, num_vars, par_buffer_size] with
+    respect to what it returned; a host matrix [num_examples, num_parameters]."""
+    st = _state.get("sample")
+    if st is None or st["mbpc"] is not mbpc or st["last"] is None:
+        raise RuntimeError("call gumbel_sample_with_prealloc first")
+    if not st["grad"]:
+        raise RuntimeError("gumbel_sample_preallocation was called without allocate_for_grad")
+    p, noise = st["last"]
+    og = np.asarray(input_aggr_grads, np.float32)
+    if og.shape != (p.shape[0], st["num_vars"], st["width"]):
+        raise ValueError(f"input_aggr_grads must be {(p.shape[0], st['num_vars'], st['width'])}, got {og.shape}")
+    C = mbpc.size("categories")
+    g = gumbel_sample_backward_rows(mbpc, p, torch.from_numpy(np.ascontiguousarray(og[:, :, :C])).to(p.device),
+                                    temperature=temperature, noise=noise, norm_params=norm_params,
+                                    grad_wrt_logparams=grad_wrt_logparams)
+    return g.cpu().numpy()

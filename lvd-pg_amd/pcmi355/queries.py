@@ -293,6 +293,32 @@ def gumbel_sample_rows(mbpc, params, *, temperature, noise=None, norm_params=Fal
     return out.cpu().numpy() if host else out
 
 
+def gumbel_sample_backward_rows(mbpc, params, out_grads, *, temperature, noise=None, norm_params=False,
+                                grad_wrt_logparams=True):
+    """`gumbel_sample_backward(mbpc, params, input_aggr_params, input_aggr_grads, temperature; norm_params,
+    grad_wrt_logparams)` (src/queries/sample.jl:620-692): gradients of a loss with respect to every row of
+    `params`, given its gradients `out_grads` [rows, V, C] with respect to the soft assignment that
+    `gumbel_sample_rows` returned for the same params, noise and temperature.  Leaf entries are gradients
+    per probability of the category, as the source writes them (:560-570).  Returns [rows, num_parameters]
+    (host array for host input, else GPU tensor with the strides of `params`)."""
+    n = mbpc.num_parameters()
+    p, host = _rows_on_device(params, n, "params")
+    rows = p.shape[0]
+    if noise is not None:
+        noise, _ = _rows_on_device(noise, mbpc.num_inner_params(), "noise")
+        noise = noise.contiguous()
+        if noise.shape[0] != rows:
+            raise ValueError("noise must have one row per parameter row")
+    og = torch.as_tensor(out_grads, dtype=torch.float32, device=p.device).contiguous()
+    if tuple(og.shape) != (rows, mbpc.size("variables"), mbpc.size("categories")):
+        raise ValueError("out_grads must be [rows, num_vars, num_cats]")
+    g = torch.empty_strided(p.shape, p.stride(), dtype=torch.float32, device=p.device)
+    check(lib.pcm_gumbel_sample_backward_rows(mbpc.handle, p.data_ptr(), p.stride(0), p.stride(1), rows, _dev_ptr(noise),
+                                              float(temperature), int(bool(norm_params)), int(bool(grad_wrt_logparams)),
+                                              og.data_ptr(), g.data_ptr()))
+    return g.cpu().numpy() if host else g
+
+
 def sample(bpc, node_noise, leaf_noise):
     """Gumbel-max samples from supplied noise (temperature -> 0 limit of `gumbel_sample`,
     src/queries/sample.jl:338-383).  node_noise [B, sample_noise_size], leaf_noise

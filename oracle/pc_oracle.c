@@ -477,6 +477,70 @@ void orc_gumbel_soft(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
 }
 
 /*
+ * Reverse pass of the relaxed sampler, VariationalJuice.jl/src/queries/sample.jl:389-650
+ * (gumbel_input_sample_up_kernel :531-598, gumbel_params_up_layer_kernel :391-480,
+ * gumbel_sample_backward :620-640), one example.  og[var][c]: gradient of the loss with
+ * respect to the soft output of orc_gumbel_soft; td: the top-down probabilities that
+ * call left behind.  Nodes are walked children first.
+ *   input node (:560-570)  leaf_grad[c] = og[var][c] * td[node]  -- with respect to the
+ *       PROBABILITY of category c, with or without norm_params, as the source writes it;
+ *       grads[node] = sum_c prob(c) * og[var][c]
+ *   sum edge (:421-436)    w = exp((logp + g)/T) / cum;  param_grad = child_grad * td[parent];
+ *       cum_grad += param_grad * w;  grads[parent] += child_grad * w
+ *       then (:463-470)    edge_grad = (param_grad - cum_grad) * w / T   (grad_wrt_logparams)
+ *                                     (param_grad - cum_grad) / T       (otherwise)
+ *   product edge           grads[parent] += child_grad
+ * with child_grad = grads[prime] (+ grads[sub]).  Product edges get edge_grad 0.
+ */
+void orc_gumbel_soft_backward(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
+                              const int32_t* prime, const int32_t* sub, const REAL* logp,
+                              const int32_t* in_var, const int64_t* in_off, int C,
+                              const REAL* leaf_logp, const REAL* g, REAL temperature,
+                              const REAL* td, const REAL* og, int norm_params,
+                              int grad_wrt_logparams, REAL* grads, REAL* edge_grad,
+                              REAL* leaf_grad) {
+  for (int n = 0; n < n_nodes; ++n) {
+    if (type[n] == NODE_INPUT) {
+      REAL acc = 0;
+      for (int c = 0; c < C; ++c) {
+        REAL o = og[(int64_t)in_var[n] * C + c], x = leaf_logp[in_off[n] + c];
+        leaf_grad[in_off[n] + c] = o * td[n];
+        acc += (norm_params ? x : (REAL)exp((double)x)) * o;
+      }
+      grads[n] = acc;
+      continue;
+    }
+    int e0 = edge_ptr[n], e1 = edge_ptr[n + 1];
+    REAL acc = 0;
+    if (type[n] != NODE_SUM) {
+      for (int e = e0; e < e1; ++e) {
+        acc += grads[prime[e]] + (sub[e] >= 0 ? grads[sub[e]] : 0);
+        edge_grad[e] = 0;
+      }
+      grads[n] = acc;
+      continue;
+    }
+    REAL cum = 0, cum_grad = 0;
+    for (int e = e0; e < e1; ++e)
+      cum += (REAL)exp((double)((logp[e] + (g ? g[e] : 0)) / temperature));
+    for (int e = e0; e < e1; ++e) {
+      REAL w = (REAL)exp((double)((logp[e] + (g ? g[e] : 0)) / temperature)) / cum;
+      REAL child = grads[prime[e]] + (sub[e] >= 0 ? grads[sub[e]] : 0);
+      REAL pg = child * td[n];
+      edge_grad[e] = pg;
+      cum_grad += pg * w;
+      acc += child * w;
+    }
+    for (int e = e0; e < e1; ++e) {
+      REAL w = (REAL)exp((double)((logp[e] + (g ? g[e] : 0)) / temperature)) / cum;
+      edge_grad[e] = grad_wrt_logparams ? (edge_grad[e] - cum_grad) * w / temperature
+                                        : (edge_grad[e] - cum_grad) / temperature;
+    }
+    grads[n] = acc;
+  }
+}
+
+/*
  * Adam ascent step on unnormalised log-parameters, then per-sum-node normalisation
  * into the circuit's log-parameters, as the reference's training loop does it:
  *   sgd/adam.jl:318-319  m = b1*m + (1-b1)*g ; v = b2*v + (1-b2)*g^2

@@ -325,6 +325,25 @@ def gumbel_soft(fc, g, temperature, double=False, norm_params=False):
     return td, out
 
 
+def gumbel_soft_backward(fc, g, temperature, out_grad, double=False, norm_params=False, grad_wrt_logparams=True):
+    """Reverse pass of `gumbel_soft` (sample.jl:389-650): returns (edge_grad [n_edges] in CSR order,
+    leaf_grad [n_leaf_params]) for the gradient `out_grad` [V, C] of a loss w.r.t. the soft output."""
+    R = _real(double)
+    td, _ = gumbel_soft(fc, g, temperature, double, norm_params)
+    gg = None if g is None else np.ascontiguousarray(g, R)
+    og = np.ascontiguousarray(out_grad, R)
+    grads = np.zeros(fc.n_nodes, R)
+    eg = np.zeros(fc.n_edges, R)
+    lg = np.zeros(len(fc.leaf_logp), R)
+    rc = ctypes.c_double if double else ctypes.c_float
+    lib(double).orc_gumbel_soft_backward(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(fc.prime),
+                                         _p(fc.sub), _p(np.ascontiguousarray(fc.logp, R)), _p(fc.in_var),
+                                         _p(fc.in_off), ctypes.c_int(fc.C), _p(np.ascontiguousarray(fc.leaf_logp, R)),
+                                         _p(gg), rc(temperature), _p(td), _p(og), ctypes.c_int(int(norm_params)),
+                                         ctypes.c_int(int(grad_wrt_logparams)), _p(grads), _p(eg), _p(lg))
+    return eg, lg
+
+
 def adam_step(params, grad, m, v, lr, b1, b2, eps, t, group_ptr, logp_out, double=False):
     rc = ctypes.c_double if double else ctypes.c_float
     gp = np.ascontiguousarray(group_ptr, np.int64)

@@ -634,6 +634,85 @@ def test_soft_sampling_cold_limit_is_the_gumbel_max_sample():
     assert checked >= 10
 
 
+@pytest.mark.parametrize("T,noise", [(1.0, False), (0.6, True), (1.8, True)])
+def test_soft_sampling_reverse_pass_is_the_derivative_of_the_soft_output(T, noise):
+    """src/queries/sample.jl:389-650.  For a loss L = sum(out * G) the reverse pass must return dL/d(log
+    parameter) on the sum edges, and on the leaves dL/d(probability of the category), i.e. the log-parameter
+    derivative divided by that probability (the source leaves the factor p out, :566).  Checked against
+    float64 central differences of orc_gumbel_soft, itself pinned above, on a DAG with shared sub-circuits;
+    a wrong sign, a missing 1/T, a dropped normaliser term or td taken from the wrong end each fail it."""
+    rng = np.random.default_rng(41)
+    V, C = 5, 3
+    fc = O.bits_compile(random_dag(V, C, rng, width=3), C, V)
+    g = _gumbel(rng, fc.n_edges) if noise else None
+    G = rng.normal(size=(V, C))
+    eg, lg = O.gumbel_soft_backward(fc, g, T, G, double=True)
+
+    def loss():
+        return float((O.gumbel_soft(fc, g, T, double=True)[1] * G).sum())
+
+    h = 1e-5
+    logp0, leaf0 = fc.logp.copy(), fc.leaf_logp.copy()
+    fc.logp = logp0.astype(np.float64)
+    fc.leaf_logp = leaf0.astype(np.float64)
+    sum_edges = np.nonzero(fc.type[fc.edge_parent()] == O.SUM)[0]
+    for e in rng.choice(sum_edges, size=min(25, len(sum_edges)), replace=False):
+        keep = fc.logp[e]
+        fc.logp[e] = keep + h
+        up = loss()
+        fc.logp[e] = keep - h
+        dn = loss()
+        fc.logp[e] = keep
+        assert abs(eg[e] - (up - dn) / (2 * h)) < 1e-6 * max(1.0, abs(eg[e])), e
+    assert np.all(eg[fc.type[fc.edge_parent()] != O.SUM] == 0)
+    for i in rng.choice(len(fc.leaf_logp), size=25, replace=False):
+        keep = fc.leaf_logp[i]
+        fc.leaf_logp[i] = keep + h
+        up = loss()
+        fc.leaf_logp[i] = keep - h
+        dn = loss()
+        fc.leaf_logp[i] = keep
+        assert abs(lg[i] * np.exp(keep) - (up - dn) / (2 * h)) < 1e-6 * max(1.0, abs(lg[i])), i
+    # grad_wrt_logparams = false drops the factor w = softmax weight of the edge (:466-469)
+    eg_p, _ = O.gumbel_soft_backward(fc, g, T, G, double=True, grad_wrt_logparams=False)
+    td, _ = O.gumbel_soft(fc, g, T, double=True)
+    par = fc.edge_parent()
+    for n in np.nonzero(fc.type == O.SUM)[0]:
+        e0, e1 = fc.edge_ptr[n], fc.edge_ptr[n + 1]
+        z = (fc.logp[e0:e1] + (g[e0:e1] if noise else 0.0)) / T
+        w = np.exp(z - z.max())
+        w /= w.sum()
+        np.testing.assert_allclose(eg_p[e0:e1] * w, eg[e0:e1], rtol=1e-9, atol=1e-14)
+    # probability-valued leaves (norm_params): the leaf gradient is then the plain derivative
+    fc.leaf_logp = np.exp(fc.leaf_logp)
+    _, lgn = O.gumbel_soft_backward(fc, g, T, G, double=True, norm_params=True)
+    for i in rng.choice(len(fc.leaf_logp), size=15, replace=False):
+        keep = fc.leaf_logp[i]
+        vals = []
+        for d in (h, -h):
+            fc.leaf_logp[i] = keep + d
+            vals.append(float((O.gumbel_soft(fc, g, T, double=True, norm_params=True)[1] * G).sum()))
+        fc.leaf_logp[i] = keep
+        assert abs(lgn[i] - (vals[0] - vals[1]) / (2 * h)) < 1e-6 * max(1.0, abs(lgn[i])), i
+    fc.logp, fc.leaf_logp = logp0, leaf0
+
+
+def test_soft_sampling_reverse_pass_single_sum_node_closed_form():
+    """One sum node over m leaves, no noise: out = sum_i w_i p_i with w = softmax(logp / T), so
+    dL/dlogp_i = w_i (a_i - sum_j w_j a_j) / T with a_i = <p_i, G>  (softmax derivative, worked by hand)."""
+    rng = np.random.default_rng(42)
+    C, T = 4, 0.7
+    w = np.array([0.4, 0.3, 0.2, 0.1])
+    lps = [log_dirichlet(rng, C) for _ in w]
+    fc = O.bits_compile(O.summate(*[O.input_node(0, lp) for lp in lps], logps=np.log(w).astype(np.float32)), C, 1)
+    G = rng.normal(size=(1, C))
+    eg, lg = O.gumbel_soft_backward(fc, None, T, G, double=True)
+    sm = w ** (1 / T) / (w ** (1 / T)).sum()
+    a = np.array([(np.exp(lp.astype(np.float64)) * G[0]).sum() for lp in lps])
+    np.testing.assert_allclose(eg, sm * (a - (sm * a).sum()) / T, rtol=1e-6)
+    np.testing.assert_allclose(lg.reshape(4, C), sm[:, None] * G, rtol=1e-6)
+
+
 # ------------------------------------------------------------------------------------
 # Adam
 # ------------------------------------------------------------------------------------

@@ -445,6 +445,27 @@ def test_parameter_row_queries_match_oracle(gpu, oracle, kind, R, norm):
                 g[pe] = noise[r]
             _, want = O.gumbel_soft(f1, g, T, double=True, norm_params=norm)
             np.testing.assert_allclose(soft[r], want, rtol=1e-4, atol=1e-7)
+        # and back (src/queries/sample.jl:389-650): gradients of sum(soft * G) w.r.t. every parameter row,
+        # per log-parameter and per probability (grad_wrt_logparams), row- and column-major
+        G = rng.normal(size=(R, V, C)).astype(np.float32)
+        for wrt_log in (True, False):
+            back = P.gumbel_sample_backward_rows(bpc, p1, G, temperature=T, noise=noise, norm_params=norm,
+                                                 grad_wrt_logparams=wrt_log)
+            assert back.shape == (R, n)
+            for r in range(0, R, max(1, R // 5)):
+                f1 = _row_oracle(O, fc, p1[r], ns, norm)
+                g = None
+                if with_noise:
+                    g = np.zeros(fc.n_edges)
+                    g[pe] = noise[r]
+                eg, lg = O.gumbel_soft_backward(f1, g, T, G[r], double=True, norm_params=norm, grad_wrt_logparams=wrt_log)
+                want = _grads_in_param_order(fc, eg, lg)
+                assert np.abs(back[r] - want).max() < GRAD_RTOL * np.abs(want).max(), (T, wrt_log, r)
+        tb = P.gumbel_sample_backward_rows(bpc, t1, torch.from_numpy(G).cuda(), temperature=T,
+                                           noise=None if noise is None else torch.from_numpy(noise).cuda(), norm_params=norm,
+                                           grad_wrt_logparams=False)
+        assert R == 1 or tb.stride() == (1, R)
+        np.testing.assert_array_equal(tb.cpu().numpy(), back)
     # the circuit lends its structure only: its own parameters were not read or touched
     with pytest.raises(P.PcmError):
         P._lib.check(P._lib.lib.pcm_kld_rows(bpc.handle, None, None, n, 1, R, 0, None))
@@ -507,6 +528,24 @@ def test_prealloc_wrappers_run_all_rows_at_once(gpu, oracle):
     probs[:, ns:] = np.exp(p1[:, ns:])
     as_vae = W.gumbel_sample_with_prealloc(bpc, probs, temperature=1.0, norm_params=True, no_gumbel=True)
     np.testing.assert_allclose(as_vae, soft, rtol=1e-5, atol=1e-7)
+    with pytest.raises(RuntimeError):                                          # allocate_for_grad was not asked for
+        W.gumbel_sample_backward_with_prealloc(bpc, np.zeros((R, V, C + 2), np.float32), temperature=1.0)
+    W.gumbel_sample_free_mem()
+    # the reverse pass through the wrappers (src/utils/cuda_preallocation.jl:205-218): central differences of
+    # sum(soft * G) in float32 along a few sum parameters of row 1
+    W.gumbel_sample_preallocation(bpc, num_examples=R, num_vars=V, par_buffer_size=C + 2, allocate_for_grad=True)
+    G = np.random.default_rng(5).normal(size=(R, V, C + 2)).astype(np.float32)
+    W.gumbel_sample_with_prealloc(bpc, probs, temperature=0.8, norm_params=True, no_gumbel=True)
+    back = W.gumbel_sample_backward_with_prealloc(bpc, G, temperature=0.8, norm_params=True)
+    assert back.shape == probs.shape
+    for i in (0, 7, ns - 3):
+        vals = []
+        for h in (1e-2, -1e-2):
+            q = probs.copy()
+            q[1, i] += h
+            vals.append(float((W.gumbel_sample_with_prealloc(bpc, q, temperature=0.8, norm_params=True, no_gumbel=True)[1] * G[1]).sum()))
+        fd = (vals[0] - vals[1]) / 2e-2
+        assert abs(back[1, i] - fd) < 2e-3 * max(1.0, abs(fd)), (i, back[1, i], fd)
     W.gumbel_sample_free_mem()
     # pc_vae.py:88-92: the prior repeated for every row
     W.kld_preallocation(bpc, num_examples=R)
