@@ -150,11 +150,16 @@ void HcltCircuit::build_structure() {
 // steps).  The host also places every produced tile into one of the LDS slots, for as long
 // as a later step still reads it.
 void HcltCircuit::build_schedules() {
+  if (!walk_err_) {
+    PCM_HIP(hipHostMalloc((void**)&walk_err_, sizeof(int), hipHostMallocMapped));
+    *walk_err_ = 0;
+  }
   int dev_id = 0;
   PCM_HIP(hipGetDevice(&dev_id));
   PCM_HIP(hipDeviceGetAttribute(&max_lds_, hipDeviceAttributeMaxSharedMemoryPerBlock, dev_id));
   const int tile_bytes = kSlice * K_ * (int)sizeof(float);
-  lds_slots_ = std::min(max_lds_ / tile_bytes, (1 << (31 - kSlotShift)) - 2);
+  // (the lean walks keep one state word per slot behind the slots)
+  lds_slots_ = std::min((max_lds_ - kLeanFlagWords * 4) / tile_bytes, (1 << (31 - kSlotShift)) - 2);
   if (lds_slots_ < 3) fail(PCM_ERR_UNSUPPORTED, "device offers %d bytes of LDS, a value tile needs %d", max_lds_, tile_bytes);
   const int trash_slot = lds_slots_ - 1;          // idle waves and childless nodes write here
 
@@ -233,6 +238,35 @@ void HcltCircuit::build_schedules() {
                        const std::vector<int32_t>* ratio_slot = nullptr) -> bool {
     if (K_ > 32 || lds_slots_ > 255 || (size_t)V_ * leaf_stride >= ((size_t)1 << 31)) return false;
     std::vector<int32_t> f((size_t)kLeanFields * kWalkWaves * stride, 0);
+    // how often each slot has been filled so far: a step's reads see the fills of earlier steps only, so the
+    // readers of a step are numbered before its writers
+    std::vector<int32_t> fills(256, 0);
+    for (int s = 0; s < stride; ++s) {
+      for (int pass = 0; pass < 2; ++pass)
+        for (int w = 0; w < kWalkWaves; ++w) {
+          const StepItem& it = sched[(size_t)s * kWalkWaves + w];
+          if (it.node < 0) continue;
+          int32_t& turns = f[((size_t)kLTurns * kWalkWaves + w) * stride + s];
+          if (!forward) {   // a node reads the slot its parent filled and fills one per inner child
+            const int n = it.node;
+            if (pass == 0) {
+              if (par[n] >= 0) turns |= (fills[(*ratio_slot)[n]] - 1) & 0x7f;
+            } else {
+              int q = 0;
+              for (int c : ic[n]) turns |= (fills[(*ratio_slot)[c]]++ & 0x7f) << (8 * ++q);
+            }
+            continue;
+          }
+          if (pass == 0) {
+            for (int c = 0; c < it.n_l; ++c) {
+              const int sl = (int)(it.l[c] >> kSlotShift) - 1;
+              if (sl >= 0) turns |= ((fills[sl] - 1) & 0x7f) << (8 * (c + 1));
+            }
+          } else if (it.out_slot != trash_slot) {
+            turns |= fills[it.out_slot]++ & 0x7f;
+          }
+        }
+    }
     for (int s = 0; s < stride; ++s)
       for (int w = 0; w < kWalkWaves; ++w) {
         const StepItem& it = sched[(size_t)s * kWalkWaves + w];
@@ -927,6 +961,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.R = d_R_.p;
   d.G = d_G_.p;
   d.M = d_M_.p;
+  d.err = walk_err_;
   d.ext_ops = d_ext_ops_.p;
   d.B = batch;
   d.nslices = ceil_div(batch, kSlice);
@@ -941,6 +976,7 @@ HcltDev HcltCircuit::dev(int batch) const {
 }
 
 void HcltCircuit::stage_batch(const BatchRef& b) {
+  check_walks();
   if (!b.d_data) fail(PCM_ERR_ARG, "data pointer is null");
   if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
   ensure_batch(b.batch);
@@ -963,11 +999,12 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
   // the lean kernels address every array with 32-bit offsets from one descriptor
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
   if (lean_ && small && !force_general_walks_) {
+    const size_t lean_lds = lds + kLeanFlagWords * 4;   // the slots' state words sit behind the slots
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      hipLaunchKernelGGL(hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d,
-                         d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll);
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
+      hipLaunchKernelGGL(hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, stream, d,
+                         d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
     });
   } else {
     PCM_DISPATCH_K(K_, {
@@ -987,10 +1024,11 @@ void HcltCircuit::run_backward(const HcltDev& d) {
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
   if (lean_ && small && !force_general_walks_) {
+    const size_t lean_lds = lds + kLeanFlagWords * 4;
     auto launch_lean = [&](auto kernel) {
-      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_lean_.p, bwd_stride_,
-                         n_bwd_steps_);
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
+      hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, stream, d, d_bwd_lean_.p, bwd_stride_,
+                         n_bwd_steps_, lds_slots_);
     };
     PCM_DISPATCH_LEAN_K(K_, {
       if (H_ > 0) launch_lean(&hclt_backward_lean_kernel<KK, true>); else launch_lean(&hclt_backward_lean_kernel<KK, false>);
@@ -1277,6 +1315,16 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
 
 HcltCircuit::~HcltCircuit() {
   for (hipEvent_t e : ev_) (void)hipEventDestroy(e);
+  if (walk_err_) (void)hipHostFree(walk_err_);
+}
+
+// A walk kernel whose wave ran out of polls waiting for a tile has raised the word (its results are
+// void); seen here at the next call that looks.
+void HcltCircuit::check_walks() {
+  if (walk_err_ && *walk_err_) {
+    *walk_err_ = 0;
+    fail(PCM_ERR_HIP, "a tree-walk kernel gave up waiting for a tile of an earlier step; the results of that pass are void");
+  }
 }
 
 hipEvent_t* HcltCircuit::ev_set() {

@@ -102,6 +102,7 @@ struct HcltDev {
   float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (lean kernels; row n_inner: idle waves)
+  int* err;               // host-visible word a walk kernel sets when a wave gave up waiting for a tile
   int32_t B, Bp, nslices, C, n_inner, V;
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
   uint32_t leaf_slice;    // 0; soft evidence: the "leaf table" holds one row per example ([V][Bp][K], the
@@ -216,6 +217,8 @@ class HcltCircuit : public pcm_circuit {
   bool fwd_lean_ = false, bwd_lean_ = false, stat_lean_ = false;   // each lean kernel could run this tree ...
   bool lean_ = false;   // ... and all three do (they share the stored row maxima, so it is all or none)
   DevBuf<float> d_M_;
+  int* walk_err_ = nullptr;    // pinned host word the walk kernels raise (HcltDev::err); checked by check_walks()
+  void check_walks();
   int stat_lean_hists_ = 1;   // histograms the lean statistics kernel holds in LDS per pass
   DevBuf<StatNode> d_stat_lean_;
   int fwd_stride_ = 0, bwd_stride_ = 0;

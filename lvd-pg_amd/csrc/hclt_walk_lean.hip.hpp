@@ -34,7 +34,11 @@ namespace pcm {
 //           this node's ratio tile | slots of the inner children's ratio tiles << 8, 16, 24
 //           (0xff: that child is a leaf or absent)
 //   kLFlags bit 0: root; bit 1: root of a multi-head circuit
-enum { kLW = 0, kLA0, kLA1, kLA2, kLA3, kLNode, kLSlots, kLFlags, kLeanFields };
+//   kLTurns which use of its slot a tile is, modulo 128, in the byte layout of kLSlots: a slot passes through
+//           the states 2t (free for its t-th tile), 2t + 1 (that tile is there), 2t + 2 (read, free again)
+enum { kLW = 0, kLA0, kLA1, kLA2, kLA3, kLNode, kLSlots, kLFlags, kLTurns, kLeanFields };
+constexpr int kLeanFlagWords = 256;        // one state word per LDS slot, behind the slots
+constexpr int kLeanSpinLimit = 1 << 22;    // polls before a wave gives up on a tile (never reached by a sound schedule)
 
 constexpr int kLeanChunk = 62;   // steps per refill: 64 lanes minus two steps of look-ahead
 
@@ -92,20 +96,42 @@ __device__ __forceinline__ uint32_t lean_row_off(uint32_t xpack, int sel, uint32
   return ((xpack >> (8 * sel)) & 0xffu) * (K * 4) + vleaf;
 }
 
-__device__ __forceinline__ void lean_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
+// Waits until the slot's state word reads `want`.  The walks have no barrier between steps: a wave goes on as
+// soon as the tiles it needs are there, and hands its own tile on by advancing the slot's state.  Every wait is
+// for a tile of an earlier step of the host's schedule, and every wave works through its steps in order, so the
+// earliest unfinished step can always proceed.  The wait is bounded all the same: a wave that runs out of polls
+// raises *err and carries on, so the kernel ends whatever the schedule holds.
+__device__ __forceinline__ void lean_wait(const unsigned* state, unsigned want, int* err) {
+  int polls = 0;
+  while (__builtin_amdgcn_readfirstlane(
+             (int)__hip_atomic_load(state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != (int)want) {
+    if (++polls > kLeanSpinLimit) {
+      if ((threadIdx.x & 63) == 0) __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      break;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Advances a slot's state once everything this wave did to the slot's tile before is in LDS order (a wave's
+// LDS accesses execute in the order they were issued; the fence keeps the compiler to that order too).
+__device__ __forceinline__ void lean_post(unsigned* state, unsigned value) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __hip_atomic_store(state, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
 // ---- forward ------------------------------------------------------------------------------
 template <int K>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
-    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps, float* __restrict__ ll_out) {
+    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps, float* __restrict__ ll_out, int n_slots) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slice = blockIdx.x;
+  unsigned* state = reinterpret_cast<unsigned*>(lds + (size_t)n_slots * (kSlice * K));
+  for (int i = threadIdx.x; i < kLeanFlagWords; i += blockDim.x) state[i] = 0u;
+  __syncthreads();
   const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)(lane >> 4) * 16, vx = (uint32_t)(lane & 15) * 4;
   const int bcol = slice * kSlice + (lane & 15);
   const uint32_t slice_bytes = (uint32_t)slice * (kSlice * K * 4);
@@ -169,14 +195,16 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
       if (a3 >= 0) lean_row_load<K>(rL, lean_row_off<K>(xc, 3, vleaf), a3, P3);
     }
     // (3) children from LDS, logsumexp through the matrix cores
-    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
+    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s), turns = (uint32_t)lean_get(sc, kLTurns, s);
 #pragma unroll
     for (int c = 1; c <= 3; ++c) {
-      const uint32_t sl = (slots >> (8 * c)) & 0xffu;
+      const uint32_t sl = (slots >> (8 * c)) & 0xffu, tn = (turns >> (8 * c)) & 0x7fu;
       if (sl != 0xffu) {
+        lean_wait(state + sl, (2 * tn + 1) & 0xffu, d.err);
         Tile<K> t;
         lds_tile_load<K>(lds, (int)sl, lane, t);
         tile_add<K>(z, t);
+        lean_post(state + sl, (2 * tn + 2) & 0xffu);   // read: the slot may take its next tile
       }
     }
     const float m = tile_rowmax<K>(z);
@@ -192,9 +220,15 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     store_prev = lean_get(sc, kLNode, s) * (int)d.tile_stride;
     m_prev = m;
     mrow_prev = lean_get(sc, kLNode, s) * xrow;
-    lds_tile_store<K>(lds, (int)(slots & 0xffu), lane, o);
+    {
+      // idle steps and the root write the trash slot, which nobody reads: no hand-over there
+      const uint32_t so = slots & 0xffu, tn = turns & 0x7fu;
+      const bool handed = so != (uint32_t)(n_slots - 1);
+      if (handed) lean_wait(state + so, (2 * tn) & 0xffu, d.err);
+      lds_tile_store<K>(lds, (int)so, lane, o);
+      if (handed) lean_post(state + so, (2 * tn + 1) & 0xffu);
+    }
     if (lean_get(sc, kLFlags, s) & 1) ll = o.v[0][0];
-    lean_barrier();
   };
   // The schedule is consumed in chunks of kLeanChunk steps (a chunk's registers also serve the
   // two steps of look-ahead past its end), two steps per trip: the parameter blocks alternate
@@ -226,11 +260,14 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
 // kHeads: multi-head circuit, whose head kernel has left the root's ratio tile in memory.
 template <int K, bool kHeads>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
-    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps) {
+    HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps, int n_slots) {
   extern __shared__ float lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int slice = blockIdx.x;
+  unsigned* state = reinterpret_cast<unsigned*>(lds + (size_t)n_slots * (kSlice * K));
+  for (int i = threadIdx.x; i < kLeanFlagWords; i += blockDim.x) state[i] = 0u;
+  __syncthreads();
   const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)(lane >> 4) * 16, vx = (uint32_t)(lane & 15) * 4;
   const int bcol = slice * kSlice + (lane & 15);
   const uint32_t slice_bytes = (uint32_t)slice * (kSlice * K * 4);
@@ -296,7 +333,12 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     // (1) from the landed operands: the exponent tiles of the inner children (they come first).  The first
     // stays in registers; a second and third wait in the LDS slots their ratio tiles will take.
     const bool in1 = is_inner(c1), in2 = is_inner(c2), in3 = is_inner(c3);
-    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s);
+    const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s), turns = (uint32_t)lean_get(sc, kLTurns, s);
+    {   // the children's slots are this wave's from here (scratch first, their ratio tiles at the end)
+      if (in1) lean_wait(state + ((slots >> 8) & 0xffu), (2 * ((turns >> 8) & 0x7fu)) & 0xffu, d.err);
+      if (in2) lean_wait(state + ((slots >> 16) & 0xffu), (2 * ((turns >> 16) & 0x7fu)) & 0xffu, d.err);
+      if (in3) lean_wait(state + ((slots >> 24) & 0xffu), (2 * ((turns >> 24) & 0x7fu)) & 0xffu, d.err);
+    }
     Tile<K> X1;
     if (in1) exponent(C1, m1, c2 >= 0, C2, c3 >= 0, C3, X1);
     if (in2) {
@@ -321,9 +363,12 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
       if (c2 >= 0) child_load(c2, xc, C2, m2);
       if (c3 >= 0) child_load(c3, xc, C3, m3);
     }
-    // (3) this node's ratio tile: left in LDS by the parent
+    // (3) this node's ratio tile: left in LDS by the parent (the root and idle steps read the trash slot)
     Tile<K> r;
+    const bool handed = (slots & 0xffu) != (uint32_t)(n_slots - 1);
+    if (handed) lean_wait(state + (slots & 0xffu), (2 * (turns & 0x7fu) + 1) & 0xffu, d.err);
     lds_tile_load<K>(lds, (int)(slots & 0xffu), lane, r);
+    if (handed) lean_post(state + (slots & 0xffu), (2 * (turns & 0x7fu) + 2) & 0xffu);
     const int fl = lean_get(sc, kLFlags, s);
     if (kHeads && (fl & 2)) {   // multi-head circuit: the head kernel has left the root's ratio tile in memory
       lean_tile_load<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
@@ -359,9 +404,13 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
         lds_tile_load<K>(lds, (int)((slots >> 24) & 0xffu), lane, x);
         emit(x, (slots >> 24) & 0xffu);
       }
+      {
+        lean_post(state + ((slots >> 8) & 0xffu), (2 * ((turns >> 8) & 0x7fu) + 1) & 0xffu);
+        if (in2) lean_post(state + ((slots >> 16) & 0xffu), (2 * ((turns >> 16) & 0x7fu) + 1) & 0xffu);
+        if (in3) lean_post(state + ((slots >> 24) & 0xffu), (2 * ((turns >> 24) & 0x7fu) + 1) & 0xffu);
+      }
     }
     if (is_inner(lean_get(sc, kLA1, s + 2))) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);
-    lean_barrier();
   };
   for (int base = 0; base < n_steps; base += kLeanChunk) {
     if (base) lean_refill(fields, stride, wave, lane, base, sc);
