@@ -1357,17 +1357,8 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     pull_from_general();
     return;
   }
-  PCM_DISPATCH_PARAM_K(K_, {
-    constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
-    hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,
-                       stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia,
-                       H_ > 0 ? 1 : 0);
-  });
-  check_launch("theta_update");
-  if (H_ > 0) {
-    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4)), dim3(256), 0, stream, head_logp(), head_aggr(), H_, Hp_,
-                       K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
-  }
+  // the leaf tables first, the parameter blocks last: what the next forward walk reads most often is then
+  // what the caches saw last (the blocks are read by every workgroup, a leaf table row by sixteen examples)
   // 32 category groups per workgroup; a thread holds its group's share of the categories (8 of 256)
   {
     const int threads = 1024, cats = ceil_div(C_, threads / 32);
@@ -1380,6 +1371,17 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     else launch(&hclt_leaf_update_kernel<32>);
   }
   check_launch("leaf_update");
+  PCM_DISPATCH_PARAM_K(K_, {
+    constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
+    hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,
+                       stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia,
+                       H_ > 0 ? 1 : 0);
+  });
+  check_launch("theta_update");
+  if (H_ > 0) {
+    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4)), dim3(256), 0, stream, head_logp(), head_aggr(), H_, Hp_,
+                       K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
+  }
   general_stale_ = true;
 }
 

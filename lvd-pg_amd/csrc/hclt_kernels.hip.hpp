@@ -35,6 +35,8 @@ typedef float v4f __attribute__((ext_vector_type(4)));
 // 3072-variable benchmark this alone takes 20 % off the forward kernel (the default policy
 // makes every store burst wait on L2 allocation).
 constexpr int kStreamStore = 1 | 2 | 16;
+constexpr int kStreamLoad = 2;   // value and ratio tiles are read once per kernel: non-temporal, so that they do not push the
+                                 // parameter blocks and leaf tables (read by every workgroup) out of the caches
 
 constexpr int kStatWaves = 12;   // waves per workgroup in the statistics kernel (168 registers each)
 
@@ -790,7 +792,7 @@ __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restric
   for (int q = 0; q < kCats; ++q) {
     const int c = cg + q * ncg;
     const bool in = valid && c < C;
-    f[q] = in ? fl[(size_t)c * K + j] : 0.f;
+    f[q] = in ? __builtin_nontemporal_load(&fl[(size_t)c * K + j]) : 0.f;   // read once; the parameters are what should stay cached
     p[q] = in ? lp[(size_t)c * K + j] : 0.f;
   }
   float s = 0.f;

@@ -73,14 +73,20 @@ template <int K>
 __device__ __forceinline__ void lean_tile_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, Tile<K>& t) {
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
-    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * 1024), soff, 0));
+    t.v[kt] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(r, (int)(voff + kt * 1024), soff, kStreamLoad));
 }
 
-template <int K>
+#ifndef PCM_ST_O
+#define PCM_ST_O kStreamStore
+#endif
+#ifndef PCM_ST_R
+#define PCM_ST_R kStreamStore
+#endif
+template <int K, int kAux = kStreamStore>
 __device__ __forceinline__ void lean_tile_store(__amdgpu_buffer_rsrc_t r, uint32_t voff, int soff, const Tile<K>& t) {
 #pragma unroll
   for (int kt = 0; kt < K / 16; ++kt)
-    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(voff + kt * 1024), soff, kStreamStore);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), r, (int)(voff + kt * 1024), soff, kAux);
 }
 
 template <int K>
@@ -181,7 +187,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     if (a2 >= 0) tile_add<K>(z, P2);
     if (a3 >= 0) tile_add<K>(z, P3);
     // the previous step's value tile goes out now
-    lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+    lean_tile_store<K, PCM_ST_O>(rO, vtile, store_prev, o_prev);
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_prev), rM, (int)vm, mrow_prev, kStreamStore);
     // (2) request the leaf rows of step s+1 and the categories of step s+2
     {
@@ -242,7 +248,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
       step(s + 1, wB);
     }
   }
-  lean_tile_store<K>(rO, vtile, store_prev, o_prev);
+  lean_tile_store<K, PCM_ST_O>(rO, vtile, store_prev, o_prev);
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_prev), rM, (int)vm, mrow_prev, kStreamStore);
   if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
 }
@@ -380,7 +386,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
       tile_zero<K>(r);
       r.v[0][0] = r00;
     }
-    lean_tile_store<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
+    lean_tile_store<K, PCM_ST_R>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
     // (4) the inner children's ratio tiles
     if (in1) {
       Tile<K> t;
