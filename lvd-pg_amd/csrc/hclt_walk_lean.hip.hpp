@@ -636,7 +636,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
           const int cell = c * K + (j ^ (c & (K - 1)));
           const float val = (float)hh[cell] * hi_inv + (float)hh[hist_sz + cell] * lo_inv;
           const float old = rate != 0.f ? rate * dst[i] : 0.f;
-          dst[i] = old + val;
+          __builtin_nontemporal_store(old + val, &dst[i]);   // read once more, by the update
         }
       }
     }
