@@ -77,17 +77,25 @@ struct DevBuf {
   }
 };
 
-// dst[i] += w(i) * (part[0][i] + part[1][i] + ...), the parts added in their order; w(i) = exp(logw[i]) or 1.
-// Kernels that share one sum out among workgroups leave their parts in rows of `part` and this kernel
-// puts them together: no atomics, the same bits on every run.
+// dst[i] += w(i) * (part[0][i] + part[1][i] + ...); w(i) = exp(logw[i]) or 1.  Kernels that share one sum out
+// among workgroups leave their parts in rows of `part` and this kernel puts them together: no atomics, the same
+// bits on every run.  A workgroup takes 64 elements; its four waves each add up every fourth row in order, and
+// the four subtotals are added in order too (the order is fixed, just not row after row).
 template <bool kExpWeight>
-__global__ void sum_parts_kernel(const float* __restrict__ part, int n_parts, int64_t n, const float* __restrict__ logw,
-                                 float* __restrict__ dst) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
+__global__ __launch_bounds__(256) void sum_parts_kernel(const float* __restrict__ part, int n_parts, int64_t n,
+                                                        const float* __restrict__ logw, float* __restrict__ dst) {
+  __shared__ float sub[4][64];
+  const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int64_t i = (int64_t)blockIdx.x * 64 + lane;
   float s = 0.f;
-  for (int q = 0; q < n_parts; ++q) s += part[(size_t)q * n + i];
-  dst[i] += kExpWeight ? __expf(logw[i]) * s : s;
+  if (i < n)
+    for (int q = g; q < n_parts; q += 4) s += part[(size_t)q * n + i];
+  sub[g][lane] = s;
+  __syncthreads();
+  if (g == 0 && i < n) {
+    s = ((sub[0][lane] + sub[1][lane]) + sub[2][lane]) + sub[3][lane];
+    dst[i] += kExpWeight ? __expf(logw[i]) * s : s;
+  }
 }
 
 // A batch of soft evidence: log-evidence per (example, variable, category) with element strides.

@@ -1178,11 +1178,11 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
     }
     const int Bp64 = ceil_div(d.Bp, kEvExamples) * kEvExamples;
     // old statistics times the flow memory rate first; then the batch's counts.  Small tables are split over the
-    // examples (in chunks of 64) until about 2048 workgroups run; the splits' shares are added in order afterwards
+    // examples (in chunks of 64) until about 512 workgroups run; the splits' shares are added in order afterwards
     const int64_t n_leaf = (int64_t)V_ * C_ * K_;
     hipLaunchKernelGGL(hclt_soft_scale_kernel, dim3(ceil_div(n_leaf, 256)), dim3(256), 0, stream, d_leaf_flow_.p, n_leaf, rate);
     const int chunks = ceil_div(s.batch, kEvExamples);
-    const int want = std::max(1, ceil_div(2048, (int64_t)V_ * ceil_div(C_, kEvCats)));
+    const int want = std::max(1, ceil_div(512, (int64_t)V_ * ceil_div(C_, kEvCats)));
     const int split = ceil_div(chunks, std::min(chunks, want)) * kEvExamples;      // examples per split
     const int n_split = ceil_div(s.batch, split);
     if (n_split > 1) d_part_.ensure((size_t)n_split * n_leaf);
@@ -1191,7 +1191,7 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
                                           d_soft_gnode_.p, C_, s.batch, Bp64, (size_t)d.nslices * kSlice * K_, split,
                                           d_leaf_flow_.p, n_split > 1 ? d_part_.p : (float*)nullptr));
     if (n_split > 1)
-      hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(n_leaf, 256)), dim3(256), 0, stream, d_part_.p, n_split, n_leaf,
+      hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(n_leaf, 64)), dim3(256), 0, stream, d_part_.p, n_split, n_leaf,
                          (const float*)nullptr, d_leaf_flow_.p);
     check_launch("soft_leafflow");
     have_flows_ = true;
@@ -1230,7 +1230,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,
                                                stream, d.O + root_tile, d_head_wf_.p, d_head_wb_.p, head_logp(), H_, Hp_,
                                                d.B, d_head_mask, d.R + root_tile, d_part_.p, d_flow_shift_.p));
-    hipLaunchKernelGGL(sum_parts_kernel<true>, dim3(ceil_div((int64_t)H_ * K_, 256)), dim3(256), 0, stream, d_part_.p, d.nslices,
+    hipLaunchKernelGGL(sum_parts_kernel<true>, dim3(ceil_div((int64_t)H_ * K_, 64)), dim3(256), 0, stream, d_part_.p, d.nslices,
                        (int64_t)H_ * K_, head_logp(), head_aggr());
     check_launch("heads_backward");
     run_backward(d);

@@ -1219,7 +1219,7 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
                          d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
   }
   if (ne)
-    hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 256)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,
+    hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 64)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,
                        (const float*)nullptr, d_edge_aggr_.p);
   if (!fc_.input_nodes.empty()) {
     if (d_input_nodes_.n == 0) d_input_nodes_.upload(fc_.input_nodes, stream);
