@@ -109,19 +109,42 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
     return ll
 
 
+def soft_reg_evidence(rows, num_cats, soft_reg, soft_reg_width):
+    """The categorical batch `rows` [B, V] (uint8) as the log-evidence [B, V, C] under which a leaf's value is
+    the reference's `soft_loglikelihood` (src/regularization/reg_likelihood.jl:4-14):
+    log((1 - soft_reg) * p[x] + soft_reg * mean(p[c] for c in the window)), the window being
+    c_start = max(0, x - width ÷ 2) .. min(c_start + width - 1, C - 1)."""
+    x = rows.long().unsqueeze(-1)
+    c = torch.arange(num_cats, device=rows.device).view(1, 1, -1)
+    c_start = (x - int(soft_reg_width) // 2).clamp_(min=0)
+    c_end = (c_start + int(soft_reg_width) - 1).clamp_(max=num_cats - 1)
+    w = ((c >= c_start) & (c <= c_end)).float() * (float(soft_reg) / (c_end - c_start + 1).float())
+    w += (c == x).float() * (1.0 - float(soft_reg))
+    return torch.log(w)
+
+
 def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
                            ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
                            shuffle="each_epoch", verbose=False, generator=None, head_mask=None, eval_dataset=None,
                            eval_interval=0):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
-    of per-epoch mean log-likelihoods.  soft_reg and ent_reg must be 0 (the reference's
-    entropy regulariser is commented out at :294-296).  `data` may be 3-D float32 soft evidence,
-    as for the top-level circuits of exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl.
-    With `verbose`, every `eval_interval` epochs the mean log-likelihood of `eval_dataset` is printed
-    beside the training one (:308-327)."""
-    if soft_reg != 0.0 or ent_reg != 0.0:
-        raise NotImplementedError("soft_reg / ent_reg other than 0 are not supported")
+    of per-epoch mean log-likelihoods.  ent_reg must be 0 (the reference's entropy regulariser is
+    commented out at :294-296).  `data` may be 3-D float32 soft evidence, as for the top-level circuits of
+    exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl.  With `verbose`, every `eval_interval` epochs the
+    mean log-likelihood of `eval_dataset` is printed beside the training one (:308-327).
+
+    soft_reg > 0 on categorical data (reg_likelihood.jl:4-14, reg_flow.jl:3-22): every batch is turned into
+    the soft evidence that gives the leaves the reference's smoothed value (`soft_reg_evidence`) and runs
+    through the soft-evidence kernels.  Likelihoods are the reference's; the leaf flows are the derivative of
+    that value -- (1 - s) p[x] / base for the observed category and s / n * p[c] / base over the window, the
+    form of `soft_flow_params` (src/nodes/fixable_categorical_dist.jl:141-160) -- whereas `soft_flow` as
+    written (reg_flow.jl:12-17) puts log-probabilities where these probabilities stand."""
+    if ent_reg != 0.0:
+        raise NotImplementedError("ent_reg other than 0 is not supported (commented out in the reference)")
     _check_data(bpc, data)
+    smooth = soft_reg != 0.0 and not _is_soft(data)
+    if smooth and not 0.0 < soft_reg < 1.0:
+        raise ValueError("soft_reg must lie in [0, 1)")
     n = data.shape[0]
     if batch_size > n:
         raise ValueError("batch_size must not exceed the number of examples")   # reg_em.jl:219
@@ -151,7 +174,12 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
             ids = perm[bi * batch_size:(bi + 1) * batch_size]
             rate = 0.0 if (flow_memory == 0 or fresh) else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
             fresh = False
-            if hm_t is None and not _is_soft(data):
+            if smooth:
+                ev = soft_reg_evidence(data[ids.long()], bpc.size("categories"), soft_reg, soft_reg_width)
+                hm = None if hm_t is None else hm_t[ids.long()].t().contiguous()
+                _flows(bpc, ev, None, batch_size, rate, _dev_ptr(hm), ll.data_ptr())
+                check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
+            elif hm_t is None and not _is_soft(data):
                 check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
                                       batch_size, rate, float(pseudocount), float(param_inertia), ll.data_ptr()))
             else:

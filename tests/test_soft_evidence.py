@@ -202,3 +202,80 @@ def test_top_level_circuit_shape(gpu):
     assert np.abs(ll[:24] - want).max() < LL_RTOL * np.abs(want).max()
     lls = P.mini_batch_em_with_reg(bpc, d, 3, batch_size=256, pseudocount=0.1, param_inertia=0.9, shuffle="none")
     assert lls[-1] > lls[0]
+
+
+def _soft_ll_as_written(logp, x, s, width):
+    """`soft_loglikelihood` of src/regularization/reg_likelihood.jl:4-14, line by line."""
+    C = len(logp)
+    c_start = max(0, x - width // 2)
+    c_end = min(c_start + width - 1, C - 1)
+    sp = sum(np.exp(logp[c]) for c in range(c_start, c_end + 1)) / (c_end - c_start + 1)
+    return np.logaddexp(logp[x] + np.log(1 - s), np.log(sp) + np.log(s))
+
+
+@pytest.mark.parametrize("C,width", [(7, 3), (7, 5), (4, 7), (9, 1)])
+def test_soft_reg_is_soft_evidence(C, width):
+    """soft_reg smoothing of categorical data (reg_likelihood.jl:4-14) is the soft evidence
+    `soft_reg_evidence` builds: for every observed category, also at both ends of the range where the window
+    is cut, log sum_c exp(ev[c]) p[c] equals the reference's leaf value worked out line by line; and the leaf
+    flows of that evidence are the shares (1 - s) p[x] / base and s / n p[c] / base of `soft_flow_params`
+    (src/nodes/fixable_categorical_dist.jl:141-160)."""
+    import sys
+    import torch
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "lvd-pg_amd"))
+    from pcmi355.queries import soft_reg_evidence
+    rng = np.random.default_rng(C * 10 + width)
+    s = 0.07
+    logp = np.log(rng.dirichlet(np.ones(C)))
+    rows = torch.arange(C, dtype=torch.uint8).view(C, 1)              # one variable, every category once
+    ev = soft_reg_evidence(rows, C, s, width).numpy()[:, 0, :].astype(np.float64)
+    for x in range(C):
+        got = np.log(np.exp(ev[x] + logp).sum())
+        assert abs(got - _soft_ll_as_written(logp, x, s, width)) < 1e-6
+        c_start = max(0, x - width // 2)
+        c_end = min(c_start + width - 1, C - 1)
+        n = c_end - c_start + 1
+        base = (1 - s) * np.exp(logp[x]) + s * np.exp(logp[c_start:c_end + 1]).sum() / n
+        want = np.zeros(C)
+        want[x] += (1 - s) * np.exp(logp[x]) / base
+        want[c_start:c_end + 1] += s / n * np.exp(logp[c_start:c_end + 1]) / base
+        share = np.exp(ev[x] + logp - got)
+        np.testing.assert_allclose(share, want, rtol=1e-6, atol=1e-12)
+
+
+@pytest.mark.gpu
+def test_em_with_soft_reg_matches_oracle(gpu):
+    """mini_batch_em_with_reg(...; soft_reg = 0.02, soft_reg_width = 5) as test/regularization/reg_em_tests.jl:20-21
+    calls it: the likelihoods and the parameters after two batches against the oracle's EM on the evidence
+    worked out line by line from reg_likelihood.jl:4-14."""
+    torch, P = gpu
+    V, K, C, B, s, width = 8, 16, 11, 48, 0.02, 5
+    parent, theta, leaf, fc = make_hclt(V, K, C, 77)
+    rng = np.random.default_rng(7)
+    data = rng.integers(0, C, size=(2 * B, V)).astype(np.uint8)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    lls = P.mini_batch_em_with_reg(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=0.01, soft_reg=s,
+                                   soft_reg_width=width, param_inertia=0.9, shuffle="none")
+    want_ll = []
+    for b0 in (0, B):
+        ev = np.full((B, V, C), -np.inf)
+        for i in range(B):
+            for v in range(V):
+                x = int(data[b0 + i, v])
+                c_start = max(0, x - width // 2)
+                c_end = min(c_start + width - 1, C - 1)
+                ev[i, v, c_start:c_end + 1] = np.log(s / (c_end - c_start + 1))
+                ev[i, v, x] = np.log(np.exp(ev[i, v, x]) + 1 - s)
+        mars = O.forward_soft(fc, ev.astype(np.float32), double=True)
+        want_ll.append(mars[-1].mean())
+        fl, ea = O.backward(fc, mars, double=True)
+        counts = O.input_flows_soft(fc, ev.astype(np.float32), mars, fl, double=True)
+        new_logp, new_leaf = O.em_update(fc, ea, counts, 0.01, 0.9, double=True)
+        fc.logp, fc.leaf_logp = new_logp.astype(np.float32), new_leaf.astype(np.float32)
+    assert abs(lls[0] - np.mean(want_ll)) < 1e-5 * abs(np.mean(want_ll))
+    _, leaf_after = bpc.get_params()
+    assert np.abs(np.exp(leaf_after) - np.exp(fc.leaf_logp.reshape(V, K, C))).max() < 5e-4 * np.exp(fc.leaf_logp).max()
+    with pytest.raises(NotImplementedError):
+        P.mini_batch_em_with_reg(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=0.01, ent_reg=0.1,
+                                 param_inertia=0.9)
