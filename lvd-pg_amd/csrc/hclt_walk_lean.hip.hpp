@@ -513,6 +513,15 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
 
   const int last = d.nslices - 1;
   const int n_pass = (n_hist + nh_pass - 1) / nh_pass;
+  // categories and row maxima of the wave's first two slices: requested before the histograms are cleared, so
+  // that the leaf rows that depend on them can go out right behind the barrier
+  const uint32_t x_first = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, min(wave, last) * (kSlice * 4), 0);
+  const uint32_t x_second =
+      (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, min(wave + kStatLeanWaves, last) * (kSlice * 4), 0);
+  const float m_first =
+      __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, min(wave, last) * (kSlice * 4), 0));
+  const float m_second = __builtin_bit_cast(
+      float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, min(wave + kStatLeanWaves, last) * (kSlice * 4), 0));
   for (int pass = 0; pass < n_pass; ++pass) {
     const int h0 = pass * nh_pass, nh = min(nh_pass, n_hist - h0);   // this pass fills histograms of variables h0 .. h0+nh-1
     for (int i = threadIdx.x; i < nh * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
@@ -521,14 +530,10 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
     // repeated loads), categories of the second
     Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
-    uint32_t xc, xn;
-    float mc, mn;            // the slices' row maxima, requested like their categories
+    uint32_t xc = x_first, xn = x_second;
+    float mc = m_first, mn = m_second;   // the slices' row maxima, requested like their categories
     {
-      const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
-      xc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sa * (kSlice * 4), 0);
-      xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sb * (kSlice * 4), 0);
-      mc = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, sa * (kSlice * 4), 0));
-      mn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, sb * (kSlice * 4), 0));
+      const int sa = min(wave, last);
       const uint32_t so = (uint32_t)sa * (kSlice * K * 4);
       lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
       if (c1 >= 0) child_load(rC1, c1, xc, so, C1);
@@ -643,16 +648,19 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     __syncthreads();
   }
 
-  // combine the waves' partial blocks: every wave parks its accumulators in LDS (the histogram
-  // area is free now), then each thread adds up the waves' copies of its elements
+  // combine the waves' partial blocks: every wave parks its accumulators in LDS (the histogram area is free
+  // now), then each thread adds up the waves' copies of its elements in wave order.  The edge weight of an
+  // element is already in the lane that holds it -- the block as the backward contraction's operand has
+  // element (k, j) where the accumulator tile has it -- so the partial sums are parked weighted and the
+  // parameters are not read again.
   v4f* park = reinterpret_cast<v4f*>(smem);
 #pragma unroll
   for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
-    for (int jt = 0; jt < KT; ++jt) park[((size_t)wave * KT * KT + kt * KT + jt) * 64 + lane] = accA[kt][jt];
+    for (int jt = 0; jt < KT; ++jt)
+      park[((size_t)wave * KT * KT + kt * KT + jt) * 64 + lane] = accA[kt][jt] * w.a[jt * KT + kt];
   __syncthreads();
   float* dst = edge_aggr + (size_t)n * K * K;
-  const float* lt = d.logtheta + (size_t)n * K * K;
   for (int q = threadIdx.x; q < KT * KT * 64; q += blockDim.x) {
     v4f sum = park[q];
     for (int wv = 1; wv < kStatLeanWaves; ++wv) sum += park[(size_t)wv * KT * KT * 64 + q];
@@ -661,7 +669,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     for (int v = 0; v < 4; ++v) {
       const int idx = (kt * 16 + 4 * (l >> 4) + v) * K + jt * 16 + (l & 15);
       const float old = rate != 0.f ? rate * dst[idx] : 0.f;
-      dst[idx] = old + __expf(lt[idx]) * sum[v];
+      dst[idx] = old + sum[v];
     }
   }
 }
