@@ -157,6 +157,7 @@ void HcltCircuit::build_schedules() {
   int dev_id = 0;
   PCM_HIP(hipGetDevice(&dev_id));
   PCM_HIP(hipDeviceGetAttribute(&max_lds_, hipDeviceAttributeMaxSharedMemoryPerBlock, dev_id));
+  PCM_HIP(hipDeviceGetAttribute(&n_cus_, hipDeviceAttributeMultiprocessorCount, dev_id));
   const int tile_bytes = kSlice * K_ * (int)sizeof(float);
   // (the lean walks keep one state word per slot behind the slots)
   lds_slots_ = std::min((max_lds_ - kLeanFlagWords * 4) / tile_bytes, (1 << (31 - kSlotShift)) - 2);
@@ -507,7 +508,10 @@ void HcltCircuit::build_schedules() {
       stat_lean_hists_ = (std::max(2 * hist, park) + pads) * 4 <= (size_t)max_lds_ ? 2 : 1;
       if ((std::max(hist, park) + pads) * 4 > (size_t)max_lds_) stat_lean_ = false;
     }
-    if (stat_lean_) d_stat_lean_.upload(sn);
+    if (stat_lean_) {
+      d_stat_lean_.upload(sn);
+      d_stat_claim_.upload(std::vector<uint32_t>(1, 0u));
+    }
   }
   lean_ = fwd_lean_ && bwd_lean_ && stat_lean_;
   if (ext.empty()) ext.push_back(0);
@@ -1063,9 +1067,10 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
       PCM_DISPATCH_LEAN_K(K_, {
         PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_lean_kernel<KK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-        hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(n_inner_), dim3(kStatLeanWaves * 64), lds, stream, d,
-                           d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
-                           H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
+        // one workgroup fills a compute unit; they draw nodes from d_stat_claim_, which every launch leaves at zero
+        hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(std::min(n_inner_, n_cus_)), dim3(kStatLeanWaves * 64), lds,
+                           stream, d, d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
+                           H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
       });
       check_launch("hclt_stats_lean");
       if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));

@@ -201,7 +201,7 @@ class HcltCircuit : public pcm_circuit {
   bool wide_ = false;   // the hidden size has the wide block kernels (likelihoods, flows, EM); neither: layered engine
   std::vector<int32_t> parent_, inner_of_var_, var_of_inner_, height_, depth_;
   std::vector<std::vector<int32_t>> children_;
-  int n_fwd_steps_ = 0, n_bwd_steps_ = 0, lds_slots_ = 0, max_lds_ = 0;
+  int n_fwd_steps_ = 0, n_bwd_steps_ = 0, lds_slots_ = 0, max_lds_ = 0, n_cus_ = 1;
   bool fwd_spill_ = false, bwd_spill_ = false;
   // parameter-vector order (reference numbering, see build_param_order)
   std::vector<int64_t> sum_param_src_;   // param i -> index into logtheta [n_inner][K][K]
@@ -221,6 +221,7 @@ class HcltCircuit : public pcm_circuit {
   void check_walks();
   int stat_lean_hists_ = 1;   // histograms the lean statistics kernel holds in LDS per pass
   DevBuf<StatNode> d_stat_lean_;
+  DevBuf<uint32_t> d_stat_claim_;   // the statistics workgroups draw their nodes from this counter; zero between launches
   int fwd_stride_ = 0, bwd_stride_ = 0;
   DevBuf<uint32_t> d_ext_ops_;
   DevBuf<float> d_leaf_, d_logtheta_, d_Wf_, d_Wb_, d_edge_aggr_, d_leaf_flow_, d_O_, d_R_, d_G_;

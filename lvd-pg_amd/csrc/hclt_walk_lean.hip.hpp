@@ -429,65 +429,102 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
 }
 
 // ---- statistics -----------------------------------------------------------------------------
-// Same job as hclt_stats_kernel (one workgroup per tree node, all slices; edge flows summed
+// Same job as hclt_stats_kernel (a workgroup takes a tree node over all slices; edge flows summed
 // over the batch with the matrix cores, leaf histograms with integer LDS atomics), for nodes
-// with at most three children, written like the lean walks: per-operand descriptors built once
-// (the node is fixed, only the slice moves), typed operands behind scalar branches, every
-// register reloaded right after its last use, the waves' partial edge-flow blocks combined by
-// a plain LDS sum.  The LDS holds up to `nh_pass` histograms (two where they fit: a node's own
-// variable and its first leaf child then need one pass over the batch).  Pass 0 does all the
-// arithmetic; a node with more variables than that leaves the child-flow tiles G where it read R
-// from, and further passes re-read G only.
+// with at most three children, written like the lean walks: one descriptor per array, a node's
+// byte offsets as scalars, typed operands behind scalar branches, every register reloaded right
+// after its last use, the waves' partial edge-flow blocks combined by a plain LDS sum.  The LDS
+// holds up to `nh_pass` histograms (two where they fit: a node's own variable and its first leaf
+// child then need one pass over the batch).  Pass 0 does all the arithmetic; a node with more
+// variables than that leaves the child-flow tiles G where it read R from, and further passes
+// re-read G only.
+//
+// The workgroups are persistent: one per compute unit, each working through nodes it claims from a
+// counter in memory (the first two by its index), and a wave's stream of slices runs on from one
+// node into the next: in its last two slices of a node the requests it sends ahead are the first
+// operands of the next node, so that they land while the histograms are written out and the
+// partial blocks are combined.  A node that needs several passes, and a batch of fewer than
+// 32 slices, ends the stream: the node after it starts with requests of its own.
 //
 // LDS layouts, both without padding so that two histograms of 256 x 32 cells and sixteen pads fill
 // 160 KB exactly: histogram cell (category x, state j) sits in word x*K + (j ^ (x % K)) of its limb
 // (equal states of different categories spread over the banks); a wave's 16 x K transposition pad
-// rotates row r by 8*r floats (column reads of four rows then cover every bank twice).
+// rotates row r by 8*r floats (column reads of four rows then cover every bank twice).  The
+// histogram area is all zero whenever a node begins: whoever reads a cell out clears it.
 constexpr int kStatLeanWaves = 16;
+
+// A node's scalars as the statistics kernel uses them.
+struct StatRef {
+  int tile_off;      // byte offset of the node's tiles in the value and ratio arrays
+  int x_off;         // ... of its row of packed categories (and of row maxima)
+  int leaf_off;      // ... of its own variable's leaf table
+  int w_off;         // ... of its parameter block
+  int c1, c2, c3;    // children as in StatNode
+  int n_hist;
+};
+
+__device__ __forceinline__ StatRef stat_ref(const HcltDev& d, const StatNode* __restrict__ nodes, int n, int kk4) {
+  const StatNode* __restrict__ np = nodes + n;
+  StatRef r;
+  r.tile_off = n * (int)d.tile_stride;
+  r.x_off = n * d.Bp * 4;
+  r.leaf_off = np->var * (int)d.leaf_stride;
+  r.w_off = n * kk4;
+  r.c1 = np->c[0];
+  r.c2 = np->c[1];
+  r.c3 = np->c[2];
+  r.n_hist = np->n_hist;
+  return r;
+}
+
+// Next node of a workgroup (-1: none left).  Tickets count from the third node of every workgroup; each
+// workgroup draws until its first miss, so a launch hands out n_nodes - gridDim.x tickets in all, and whoever
+// draws the last one puts the counter back to zero for the next launch.
+__device__ __forceinline__ int stat_claim(unsigned* counter, int n_nodes) {
+  const unsigned t = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (t + 1u == (unsigned)n_nodes - gridDim.x) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned n = 2u * gridDim.x + t;
+  return n < (unsigned)n_nodes ? (int)n : -1;
+}
 
 template <int K>
 __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     HcltDev d, const StatNode* __restrict__ nodes, float* __restrict__ edge_aggr, float* __restrict__ leaf_flow,
-    float rate, int hist_words, int nh_pass, int limb, const int* __restrict__ flow_shift) {
+    float rate, int hist_words, int nh_pass, int limb, const int* __restrict__ flow_shift, unsigned* __restrict__ counter,
+    int n_nodes) {
   constexpr int KT = K / 16;
   extern __shared__ float smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int b = lane & 15, g = lane >> 4;
-  const int n = blockIdx.x;
-  const StatNode* __restrict__ np = nodes + n;   // fields are read where needed (a local copy indexed by the pass would live in scratch)
-  const int own_var = np->var, n_hist = np->n_hist;
   const uint32_t vtile = (uint32_t)lane * 16, vleaf = (uint32_t)g * 16, vx = (uint32_t)b * 4;
   const int hist_sz = d.C * K;           // words per limb; a histogram is two limbs
   unsigned* hist = reinterpret_cast<unsigned*>(smem);
   float* pad = smem + hist_words + (size_t)wave * (kSlice * K);
+  int* claim_word = reinterpret_cast<int*>(smem + hist_words);   // wave 0's pad, which is idle between two nodes
   // flows lie in [0, 2^shift]: 1 per example in a single-head circuit, the largest total head
   // mask of an example (found on the device by the head kernel) in a multi-head one
   const int shift = flow_shift ? __builtin_amdgcn_readfirstlane(*flow_shift) : 0;
   const float scale = __builtin_ldexpf(1.f, limb), scale_in = __builtin_ldexpf(1.f, limb - shift);
+  const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
 
-  const __amdgpu_buffer_rsrc_t rR = make_rsrc(reinterpret_cast<const char*>(d.R) + (size_t)n * d.tile_stride, d.tile_stride);
-  const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);
-  const __amdgpu_buffer_rsrc_t rM = make_rsrc(d.M + (size_t)n * d.Bp, (uint32_t)d.Bp * 4u);   // row maxima of the forward walk
-  const __amdgpu_buffer_rsrc_t rL0 = make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)own_var * d.leaf_stride, d.leaf_stride);
-  auto child_rsrc = [&](int c) {
-    return (c & 1) ? make_rsrc(reinterpret_cast<const char*>(d.leaf) + (size_t)(c >> 3) * d.leaf_stride, d.leaf_stride)
-                   : make_rsrc(reinterpret_cast<const char*>(d.O) + (size_t)(max(c, 0) >> 3) * d.tile_stride, d.tile_stride);
+  const uint32_t tiles_bytes = (uint32_t)(d.n_inner + 1) * d.tile_stride;
+  const __amdgpu_buffer_rsrc_t rR = make_rsrc(d.R, tiles_bytes);
+  const __amdgpu_buffer_rsrc_t rO = make_rsrc(d.O, tiles_bytes);
+  const __amdgpu_buffer_rsrc_t rL = make_rsrc(d.leaf, (uint32_t)d.V * d.leaf_stride);
+  const __amdgpu_buffer_rsrc_t rX = make_rsrc(d.xn, (uint32_t)d.n_inner * (uint32_t)d.Bp * 4u);
+  const __amdgpu_buffer_rsrc_t rM = make_rsrc(d.M, (uint32_t)(d.n_inner + 1) * (uint32_t)d.Bp * 4u);   // row maxima of the forward walk
+  const __amdgpu_buffer_rsrc_t rW = make_rsrc(d.Wb, (uint32_t)d.n_inner * (K * K * 4));
+  auto child_load = [&](int c, uint32_t xpack, int slice_off, Tile<K>& t) {
+    if (c & 1) lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), (c >> 3) * (int)d.leaf_stride, t);
+    else lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride + slice_off, t);
   };
-  const int c1 = np->c[0], c2 = np->c[1], c3 = np->c[2];
-  const __amdgpu_buffer_rsrc_t rC1 = child_rsrc(c1), rC2 = child_rsrc(c2), rC3 = child_rsrc(c3);
-  auto child_load = [&](__amdgpu_buffer_rsrc_t r, int c, uint32_t xpack, uint32_t slice_off, Tile<K>& t) {
-    if (c & 1) lean_row_load<K>(r, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), 0, t);
-    else lean_tile_load<K>(r, vtile, (int)slice_off, t);
+  auto load_x = [&](const StatRef& r, int s) {
+    return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, r.x_off + s * (kSlice * 4), 0);
   };
-
-  WTile<K> w;
-  lean_w_load<K>(make_rsrc(d.Wb + (size_t)n * K * K, K * K * 4u), vtile, 0, w);
-  v4f accA[KT][KT];
-#pragma unroll
-  for (int a = 0; a < KT; ++a)
-#pragma unroll
-    for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
+  auto load_m = [&](const StatRef& r, int s) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, r.x_off + s * (kSlice * 4), 0));
+  };
 
   // fixed-point limbs of this lane's K/4 flows (clamped to [0, 2^shift]) into row x of histogram h
   auto histogram = [&](const Tile<K>& t, uint32_t xpack, int sel, int h) {
@@ -506,171 +543,221 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
         __hip_atomic_fetch_add(&hrow[hist_sz + col], lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       }
   };
+  // a pass's histograms out to memory; every cell read is cleared for whoever uses the area next
+  auto flush = [&](const StatNode* __restrict__ np, int h0, int nh) {
+    for (int h = 0; h < nh; ++h) {
+      float* dst = leaf_flow + (size_t)np->hvar[h0 + h] * d.C * K;
+      unsigned* hh = hist + (size_t)h * 2 * hist_sz;
+      for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
+        const int c = i / K, j = i % K;
+        const int cell = c * K + (j ^ (c & (K - 1)));
+        const float val = (float)hh[cell] * hi_inv + (float)hh[hist_sz + cell] * lo_inv;
+        hh[cell] = 0u;
+        hh[hist_sz + cell] = 0u;
+        const float old = rate != 0.f ? rate * dst[i] : 0.f;
+        __builtin_nontemporal_store(old + val, &dst[i]);   // read once more, by the update
+      }
+    }
+  };
   // pad positions: this lane's float4 of example row b (states kt*16 + 4g ..), and the element
   // (example 4q + g, state kt*16 + b) of the transposed read
   auto pad_w = [&](int kt) { return b * K + ((kt * 16 + 4 * g + 8 * b) & (K - 1)); };
   auto pad_r = [&](int q, int kt) { return (4 * q + g) * K + ((kt * 16 + b + 8 * g) & (K - 1)); };
 
   const int last = d.nslices - 1;
-  const int n_pass = (n_hist + nh_pass - 1) / nh_pass;
+  const bool stream_on = d.nslices >= 2 * kStatLeanWaves;   // every wave then has two slices of a node at least
+  const int n_it = (d.nslices - wave + kStatLeanWaves - 1) / kStatLeanWaves;   // this wave's slices of a node
+  constexpr int kTileBytes = kSlice * K * 4;
+
+  int cur = blockIdx.x;
+  int nxt = cur + (int)gridDim.x < n_nodes ? cur + (int)gridDim.x : -1;
+  StatRef A = stat_ref(d, nodes, cur, K * K * 4);
+  // loop-carried requests: operands of the wave's next slice, categories and row maxima of the one after
+  Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
+  uint32_t xc, xn;
+  float mc, mn;
+  WTile<K> w;
   // categories and row maxima of the wave's first two slices: requested before the histograms are cleared, so
   // that the leaf rows that depend on them can go out right behind the barrier
-  const uint32_t x_first = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, min(wave, last) * (kSlice * 4), 0);
-  const uint32_t x_second =
-      (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, min(wave + kStatLeanWaves, last) * (kSlice * 4), 0);
-  const float m_first =
-      __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, min(wave, last) * (kSlice * 4), 0));
-  const float m_second = __builtin_bit_cast(
-      float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, min(wave + kStatLeanWaves, last) * (kSlice * 4), 0));
-  for (int pass = 0; pass < n_pass; ++pass) {
-    const int h0 = pass * nh_pass, nh = min(nh_pass, n_hist - h0);   // this pass fills histograms of variables h0 .. h0+nh-1
-    for (int i = threadIdx.x; i < nh * 2 * hist_sz; i += blockDim.x) hist[i] = 0u;
-    __syncthreads();
-    if (pass == 0) {
-    // prologue: operands of the wave's first slice (slices past the end are clamped: harmless
-    // repeated loads), categories of the second
-    Tile<K> P0, R, C1, C2;   // (a third child is rare: it is fetched at the point of use)
-    uint32_t xc = x_first, xn = x_second;
-    float mc = m_first, mn = m_second;   // the slices' row maxima, requested like their categories
-    {
-      const int sa = min(wave, last);
-      const uint32_t so = (uint32_t)sa * (kSlice * K * 4);
-      lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
-      if (c1 >= 0) child_load(rC1, c1, xc, so, C1);
-      if (c2 >= 0) child_load(rC2, c2, xc, so, C2);
-      lean_tile_load<K>(rR, vtile, (int)so, R);
+  xc = load_x(A, min(wave, last));
+  xn = load_x(A, min(wave + kStatLeanWaves, last));
+  mc = load_m(A, min(wave, last));
+  mn = load_m(A, min(wave + kStatLeanWaves, last));
+  lean_w_load<K>(rW, vtile, A.w_off, w);
+  for (int i = threadIdx.x; i < hist_words; i += blockDim.x) hist[i] = 0u;
+  __syncthreads();
+  bool warm = false;   // the first slice's operands of `cur` are on their way already
+
+  while (true) {
+    const StatNode* __restrict__ np = nodes + cur;
+    const StatRef B = stat_ref(d, nodes, max(nxt, 0), K * K * 4);
+    const int n_pass = (A.n_hist + nh_pass - 1) / nh_pass;
+    const bool cross = stream_on && nxt >= 0 && n_pass == 1;   // this wave's stream runs on into `nxt`
+    if (!warm) {
+      // operands of the wave's first slice (slices past the end are clamped: harmless repeated loads)
+      const int so = min(wave, last) * kTileBytes;
+      lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), A.leaf_off, P0);
+      if (A.c1 >= 0) child_load(A.c1, xc, so, C1);
+      if (A.c2 >= 0) child_load(A.c2, xc, so, C2);
+      lean_tile_load<K>(rR, vtile, A.tile_off + so, R);
     }
-    for (int s0 = wave; s0 < d.nslices; s0 += kStatLeanWaves) {
-      const int s1 = min(s0 + kStatLeanWaves, last), s2 = min(s0 + 2 * kStatLeanWaves, last);
-      const uint32_t so1 = (uint32_t)s1 * (kSlice * K * 4);
-      // (1) E (unnormalised) from the landed operands; request the next slice's
-      Tile<K> e = P0;
-      if (c1 >= 0) tile_add<K>(e, C1);
-      if (c2 >= 0) tile_add<K>(e, C2);
-      const uint32_t xh = xc;   // categories of the slice computed now
-      if (c3 >= 0) {
-        Tile<K> t3;
-        child_load(rC3, c3, xh, (uint32_t)s0 * (kSlice * K * 4), t3);
-        tile_add<K>(e, t3);
-      }
-      xc = xn;
-      xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
-      const float m = mc;   // the scale the backward walk built R with
-      mc = mn;
-      mn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, s2 * (kSlice * 4), 0));
-      lean_row_load<K>(rL0, lean_row_off<K>(xc, 0, vleaf), 0, P0);
-      if (c1 >= 0) child_load(rC1, c1, xc, so1, C1);
-      if (c2 >= 0) child_load(rC2, c2, xc, so1, C2);
-      // (2) E, the edge flows, then G = E .* (R W)
-      tile_exp_sub<K>(e, m);
-      {
-        // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
-        // go through the wave's pad to reach the [state][example] operand layout.  A wave's LDS
-        // accesses execute in order, so the pad needs no barrier between its phases.
-        float ra[4][KT];
+    v4f accA[KT][KT];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = R.v[kt];
+    for (int a = 0; a < KT; ++a)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
+      for (int c = 0; c < KT; ++c) accA[a][c] = v4f{0.f, 0.f, 0.f, 0.f};
+
+    {
+      const int nh = min(nh_pass, A.n_hist);   // pass 0 fills the histograms of the first nh variables
+      for (int it = 0; it < n_it; ++it) {
+        const int s0 = wave + it * kStatLeanWaves;
+        // where the requests of this turn go: the next slice of this node, or the first of the next node
+        const bool over1 = it + 1 >= n_it, over2 = it + 2 >= n_it;
+        const bool x1 = cross && over1, x2 = cross && over2;
+        const int s1 = x1 ? wave : min(s0 + kStatLeanWaves, last);
+        const int s2 = x2 ? wave + (it + 2 - n_it) * kStatLeanWaves : min(s0 + 2 * kStatLeanWaves, last);
+        const int t_tile = x1 ? B.tile_off : A.tile_off, t_leaf = x1 ? B.leaf_off : A.leaf_off;
+        const int t_c1 = x1 ? B.c1 : A.c1, t_c2 = x1 ? B.c2 : A.c2;
+        const int t_x = x2 ? B.x_off : A.x_off;
+        const int so1 = s1 * kTileBytes;
+        // (1) E (unnormalised) from the landed operands; request the next slice's
+        Tile<K> e = P0;
+        if (A.c1 >= 0) tile_add<K>(e, C1);
+        if (A.c2 >= 0) tile_add<K>(e, C2);
+        const uint32_t xh = xc;   // categories of the slice computed now
+        if (A.c3 >= 0) {
+          Tile<K> t3;
+          child_load(A.c3, xh, s0 * kTileBytes, t3);
+          tile_add<K>(e, t3);
+        }
+        xc = xn;
+        xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, t_x + s2 * (kSlice * 4), 0);
+        const float m = mc;   // the scale the backward walk built R with
+        mc = mn;
+        mn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, t_x + s2 * (kSlice * 4), 0));
+        lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), t_leaf, P0);
+        if (t_c1 >= 0) child_load(t_c1, xc, so1, C1);
+        if (t_c2 >= 0) child_load(t_c2, xc, so1, C2);
+        // (2) E, the edge flows, then G = E .* (R W)
+        tile_exp_sub<K>(e, m);
+        {
+          // A += R^T E over the 16 examples of the tile (contraction over examples): both operands
+          // go through the wave's pad to reach the [state][example] operand layout.  A wave's LDS
+          // accesses execute in order, so the pad needs no barrier between its phases.
+          float ra[4][KT];
 #pragma unroll
-          for (int kt = 0; kt < KT; ++kt) ra[q][kt] = pad[pad_r(q, kt)];
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+          for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = R.v[kt];
 #pragma unroll
-        for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = e.v[kt];
+          for (int q = 0; q < 4; ++q)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float eb[KT];
+            for (int kt = 0; kt < KT; ++kt) ra[q][kt] = pad[pad_r(q, kt)];
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
 #pragma unroll
-          for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[pad_r(q, jt)];
+          for (int kt = 0; kt < KT; ++kt) *reinterpret_cast<v4f*>(&pad[pad_w(kt)]) = e.v[kt];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float eb[KT];
+#pragma unroll
+            for (int jt = 0; jt < KT; ++jt) eb[jt] = pad[pad_r(q, jt)];
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+              for (int jt = 0; jt < KT; ++jt)
+                accA[kt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[q][kt], eb[jt], accA[kt][jt], 0, 0, 0);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        }
+        Tile<K> t;
+        contract<K>(w, R, t);
+#pragma unroll
+        for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
+        lean_tile_load<K>(rR, vtile, t_tile + so1, R);   // next slice's ratios, after the last use of these
+        if (n_pass > 1) {
+          // the later passes only need G: it replaces the tile of R just consumed
 #pragma unroll
           for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-            for (int jt = 0; jt < KT; ++jt)
-              accA[kt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(ra[q][kt], eb[jt], accA[kt][jt], 0, 0, 0);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), rR, (int)(vtile + kt * 1024),
+                                                   A.tile_off + s0 * kTileBytes, 0);
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        // (3) histograms: the node's own variable, and its first leaf child if the LDS holds two
+        if (s0 * kSlice + b < d.B) {
+          histogram(t, xh, 0, 0);
+          if (nh > 1) histogram(t, xh, 1, 1);
+        }
       }
-      Tile<K> t;
-      contract<K>(w, R, t);
-#pragma unroll
-      for (int kt = 0; kt < KT; ++kt) t.v[kt] *= e.v[kt];
-      lean_tile_load<K>(rR, vtile, (int)so1, R);   // next slice's ratios, after the last use of these
-      if (n_pass > 1) {
-        // the later passes only need G: it replaces the tile of R just consumed
-#pragma unroll
-        for (int kt = 0; kt < KT; ++kt)
-          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, t.v[kt]), rR, (int)(vtile + kt * 1024),
-                                                 (int)((uint32_t)s0 * (kSlice * K * 4)), 0);
-      }
-      // (3) histograms: the node's own variable, and its first leaf child if the LDS holds two
-      if (s0 * kSlice + b < d.B) {
-        histogram(t, xh, 0, 0);
-        if (nh > 1) histogram(t, xh, 1, 1);
-      }
+      __syncthreads();
+      // the node after next is drawn while the histograms go out
+      if (threadIdx.x == 0) *claim_word = nxt >= 0 ? stat_claim(counter, n_nodes) : -1;
+      flush(np, 0, nh);
+      __syncthreads();
     }
-    } else {
+    const int nxt2 = __builtin_amdgcn_readfirstlane(*claim_word);
+    for (int pass = 1; pass < n_pass; ++pass) {
       // further leaf children: G comes back from where pass 0 left it; only the categories differ
+      const int h0 = pass * nh_pass, nh = min(nh_pass, A.n_hist - h0);
       Tile<K> T;
-      uint32_t xc, xn;
-      {
-        const int sa = min(wave, last), sb = min(wave + kStatLeanWaves, last);
-        xc = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sa * (kSlice * 4), 0);
-        xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, sb * (kSlice * 4), 0);
-        lean_tile_load<K>(rR, vtile, (int)((uint32_t)sa * (kSlice * K * 4)), T);
-      }
+      uint32_t yc = load_x(A, min(wave, last)), yn = load_x(A, min(wave + kStatLeanWaves, last));
+      lean_tile_load<K>(rR, vtile, A.tile_off + min(wave, last) * kTileBytes, T);
       for (int s0 = wave; s0 < d.nslices; s0 += kStatLeanWaves) {
         const int s1 = min(s0 + kStatLeanWaves, last), s2 = min(s0 + 2 * kStatLeanWaves, last);
-        const uint32_t xh = xc;
-        xc = xn;
-        xn = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, s2 * (kSlice * 4), 0);
+        const uint32_t xh = yc;
+        yc = yn;
+        yn = load_x(A, s2);
         if (s0 * kSlice + b < d.B) {
           histogram(T, xh, h0, 0);
           if (nh > 1) histogram(T, xh, h0 + 1, 1);
         }
-        lean_tile_load<K>(rR, vtile, (int)((uint32_t)s1 * (kSlice * K * 4)), T);
+        lean_tile_load<K>(rR, vtile, A.tile_off + s1 * kTileBytes, T);
       }
+      __syncthreads();
+      flush(np, h0, nh);
+      __syncthreads();
     }
+
+    // combine the waves' partial blocks: every wave parks its accumulators in LDS (the histogram area is free
+    // now), then each thread adds up the waves' copies of its elements in wave order.  The edge weight of an
+    // element is already in the lane that holds it -- the block as the backward contraction's operand has
+    // element (k, j) where the accumulator tile has it -- so the partial sums are parked weighted and the
+    // parameters are not read again.
+    v4f* park = reinterpret_cast<v4f*>(smem);
+#pragma unroll
+    for (int kt = 0; kt < KT; ++kt)
+#pragma unroll
+      for (int jt = 0; jt < KT; ++jt)
+        park[((size_t)wave * KT * KT + kt * KT + jt) * 64 + lane] = accA[kt][jt] * w.a[jt * KT + kt];
+    if (nxt >= 0) lean_w_load<K>(rW, vtile, B.w_off, w);   // the next node's block, into the registers just freed
     __syncthreads();
     {
-      const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
-      for (int h = 0; h < nh; ++h) {
-        float* dst = leaf_flow + (size_t)np->hvar[h0 + h] * d.C * K;
-        const unsigned* hh = hist + (size_t)h * 2 * hist_sz;
-        for (int i = threadIdx.x; i < d.C * K; i += blockDim.x) {
-          const int c = i / K, j = i % K;
-          const int cell = c * K + (j ^ (c & (K - 1)));
-          const float val = (float)hh[cell] * hi_inv + (float)hh[hist_sz + cell] * lo_inv;
-          const float old = rate != 0.f ? rate * dst[i] : 0.f;
-          __builtin_nontemporal_store(old + val, &dst[i]);   // read once more, by the update
+      float* dst = edge_aggr + (size_t)cur * K * K;
+      float* parkf = smem;
+      for (int t = threadIdx.x; t < K * K; t += blockDim.x) {   // one element a thread: (tile q, component v)
+        const int q = t >> 2, v = t & 3;
+        float sum = parkf[t];
+        parkf[t] = 0.f;
+#pragma unroll
+        for (int wv = 1; wv < kStatLeanWaves; ++wv) {
+          sum += parkf[wv * (K * K) + t];
+          parkf[wv * (K * K) + t] = 0.f;
         }
+        const int kt = q / (KT * 64), jt = (q / 64) % KT, l = q % 64;
+        const int idx = (kt * 16 + 4 * (l >> 4) + v) * K + jt * 16 + (l & 15);
+        const float old = rate != 0.f ? rate * dst[idx] : 0.f;
+        dst[idx] = old + sum;
       }
     }
-    __syncthreads();
-  }
-
-  // combine the waves' partial blocks: every wave parks its accumulators in LDS (the histogram area is free
-  // now), then each thread adds up the waves' copies of its elements in wave order.  The edge weight of an
-  // element is already in the lane that holds it -- the block as the backward contraction's operand has
-  // element (k, j) where the accumulator tile has it -- so the partial sums are parked weighted and the
-  // parameters are not read again.
-  v4f* park = reinterpret_cast<v4f*>(smem);
-#pragma unroll
-  for (int kt = 0; kt < KT; ++kt)
-#pragma unroll
-    for (int jt = 0; jt < KT; ++jt)
-      park[((size_t)wave * KT * KT + kt * KT + jt) * 64 + lane] = accA[kt][jt] * w.a[jt * KT + kt];
-  __syncthreads();
-  float* dst = edge_aggr + (size_t)n * K * K;
-  for (int q = threadIdx.x; q < KT * KT * 64; q += blockDim.x) {
-    v4f sum = park[q];
-    for (int wv = 1; wv < kStatLeanWaves; ++wv) sum += park[(size_t)wv * KT * KT * 64 + q];
-    const int kt = q / (KT * 64), jt = (q / 64) % KT, l = q % 64;
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-      const int idx = (kt * 16 + 4 * (l >> 4) + v) * K + jt * 16 + (l & 15);
-      const float old = rate != 0.f ? rate * dst[idx] : 0.f;
-      dst[idx] = old + sum[v];
+    if (nxt < 0) break;
+    if (!cross) {
+      // the stream ended with this node: first categories and row maxima of the next one
+      xc = load_x(B, min(wave, last));
+      xn = load_x(B, min(wave + kStatLeanWaves, last));
+      mc = load_m(B, min(wave, last));
+      mn = load_m(B, min(wave + kStatLeanWaves, last));
     }
+    __syncthreads();   // the area is clear again before anyone counts into it
+    warm = cross;
+    cur = nxt;
+    nxt = nxt2;
+    A = B;
   }
 }
 
