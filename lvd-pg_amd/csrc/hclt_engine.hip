@@ -786,7 +786,7 @@ void HcltCircuit::rebuild_heads() {
 // head values from the root tile the forward walk has left (identity block: the root's Z)
 void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow,
                                 float rate) {
-  const float* o_root = d.O + (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
+  const float* o_root = d.O + (size_t)inner_of_var_[root_] * (d.tile_stride / 4);
   PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), 0, stream,
                                              o_root, d_head_wf_.p, H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix,
                                              flows_follow ? head_aggr() : (float*)nullptr, rate, d_flow_shift_.p));
@@ -924,7 +924,7 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
 void HcltCircuit::ensure_batch(int batch) {
   const int ns = ceil_div(batch, kSlice);
   if (ns <= cap_slices_) return;
-  const size_t tile = (size_t)ns * kSlice * K_;
+  const size_t tile = tile_floats(ns);
   if (wide_) {
     d_O_.alloc((size_t)n_inner_ * tile);
     d_G_.alloc((size_t)n_inner_ * tile);
@@ -975,7 +975,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.V = V_;
   d.leaf_stride = (uint32_t)C_ * K_ * 4;
   d.leaf_slice = 0;
-  d.tile_stride = (uint32_t)d.nslices * kSlice * K_ * 4;
+  d.tile_stride = (uint32_t)(tile_floats(d.nslices) * 4);
   return d;
 }
 
@@ -1193,7 +1193,7 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
     if (n_split > 1) d_part_.ensure((size_t)n_split * n_leaf);
     PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_soft_leafflow_kernel<KK>, dim3(ceil_div(C_, kEvCats), V_, n_split),
                                           dim3(256), 0, stream, s, d_leaf_.p, d_soft_lv_.p, d_soft_m_.p, g_tiles,
-                                          d_soft_gnode_.p, C_, s.batch, Bp64, (size_t)d.nslices * kSlice * K_, split,
+                                          d_soft_gnode_.p, C_, s.batch, Bp64, (size_t)d.tile_stride / 4, split,
                                           d_leaf_flow_.p, n_split > 1 ? d_part_.p : (float*)nullptr));
     if (n_split > 1)
       hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(n_leaf, 64)), dim3(256), 0, stream, d_part_.p, n_split, n_leaf,
@@ -1229,7 +1229,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     d_ll_heads_.ensure((size_t)b.batch);
     run_forward(d, d_ll_heads_.p);
     heads_forward(d, d_head_mask, nullptr, d_ll, true, rate);
-    const size_t root_tile = (size_t)inner_of_var_[root_] * d.nslices * kSlice * K_;
+    const size_t root_tile = (size_t)inner_of_var_[root_] * (d.tile_stride / 4);
     const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_ + (size_t)kHeadWaves * 16) * sizeof(float);
     d_part_.ensure((size_t)d.nslices * H_ * K_);
     PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,

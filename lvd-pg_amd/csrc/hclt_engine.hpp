@@ -107,7 +107,7 @@ struct HcltDev {
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
   uint32_t leaf_slice;    // 0; soft evidence: the "leaf table" holds one row per example ([V][Bp][K], the
                           // categories are the example's rank in its slice) and a slice's rows start this many bytes on
-  uint32_t tile_stride;   // bytes per node in O / R / G (nslices*16*K*4)
+  uint32_t tile_stride;   // bytes per node in O / R / G: its slices' tiles, plus one unused tile where that makes the count odd
 };
 
 #define PCM_DISPATCH_K(K_, ...)                         \
@@ -219,6 +219,10 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_M_;
   int* walk_err_ = nullptr;    // pinned host word the walk kernels raise (HcltDev::err); checked by check_walks()
   void check_walks();
+  // Floats per node in the tile arrays.  The walk engines keep an odd number of tiles per node: with a power
+  // of two (a batch of 4096), the tiles that one step reads from different nodes at equal slice offsets fell on
+  // the same memory channels (the backward walk ran 4 % slower).  The wide kernels index by slice count.
+  size_t tile_floats(int ns) const { return (size_t)((wide_ || wide_walk_) ? ns : (ns | 1)) * kSlice * K_; }
   int stat_lean_hists_ = 1;   // histograms the lean statistics kernel holds in LDS per pass
   DevBuf<StatNode> d_stat_lean_;
   DevBuf<uint32_t> d_stat_claim_;   // the statistics workgroups draw their nodes from this counter; zero between launches
