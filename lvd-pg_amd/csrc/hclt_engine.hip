@@ -1,5 +1,7 @@
 // Host side of the dense-block HCLT engine: structure, schedules, parameter order,
 // launches.
+#include <hip/hip_ext.h>
+
 #include "hclt_engine.hpp"
 
 #include <algorithm>
@@ -21,6 +23,19 @@ namespace pcm {
     case 32: { constexpr int KK = 32; __VA_ARGS__; break; } \
     default: fail(PCM_ERR_STATE, "no lean walk kernel for hidden size %d", K_); \
   }
+
+// A launch of one of the three timed phases (0 forward, 1 backward, 2 statistics).  With timing on, the phase's
+// start / stop events ride on the kernel's own dispatch: events recorded between the kernels of a step are
+// packets of their own that keep the next kernel waiting (measured: about 6 us each).
+#define PCM_LAUNCH_PHASE(phase, kernel, grid, block, lds, ...)                                                       \
+  do {                                                                                                               \
+    if (timing) {                                                                                                    \
+      hipEvent_t* ev__ = ev_set() + 2 * (phase);                                                                     \
+      hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)(lds), stream, ev__[0], ev__[1], 0, __VA_ARGS__);        \
+    } else {                                                                                                         \
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                             \
+    }                                                                                                                \
+  } while (0)
 
 static void check_launch(const char* what) {
   hipError_t e = hipGetLastError();
@@ -993,12 +1008,11 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
 }
 
 void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
   const size_t lds = (size_t)lds_slots_ * kSlice * K_ * sizeof(float);
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_fwd_fields_.p,
-                       fwd_stride_, d_fwd_sched_.p, n_fwd_steps_, d_ll);
+    PCM_LAUNCH_PHASE(0, kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, d, d_fwd_fields_.p, fwd_stride_,
+                     d_fwd_sched_.p, n_fwd_steps_, d_ll);
   };
   // the lean kernels address every array with 32-bit offsets from one descriptor
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
@@ -1007,8 +1021,8 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      hipLaunchKernelGGL(hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, stream, d,
-                         d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
+      PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, d,
+                       d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
     });
   } else {
     PCM_DISPATCH_K(K_, {
@@ -1016,23 +1030,22 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
     });
   }
   check_launch("hclt_forward");
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
 
 void HcltCircuit::run_backward(const HcltDev& d) {
   const size_t lds = (size_t)lds_slots_ * kSlice * K_ * sizeof(float);
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, stream, d, d_bwd_fields_.p,
-                       bwd_stride_, d_bwd_sched_.p, n_bwd_steps_);
+    PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lds, d, d_bwd_fields_.p, bwd_stride_,
+                     d_bwd_sched_.p, n_bwd_steps_);
   };
   const bool small = (size_t)(n_inner_ + 1) * d.tile_stride < ((size_t)1 << 31);
   if (lean_ && small && !force_general_walks_) {
     const size_t lean_lds = lds + kLeanFlagWords * 4;
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      hipLaunchKernelGGL(kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, stream, d, d_bwd_lean_.p, bwd_stride_,
-                         n_bwd_steps_, lds_slots_);
+      PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, d, d_bwd_lean_.p, bwd_stride_,
+                       n_bwd_steps_, lds_slots_);
     };
     PCM_DISPATCH_LEAN_K(K_, {
       if (H_ > 0) launch_lean(&hclt_backward_lean_kernel<KK, true>); else launch_lean(&hclt_backward_lean_kernel<KK, false>);
@@ -1047,7 +1060,6 @@ void HcltCircuit::run_backward(const HcltDev& d) {
     });
   }
   check_launch("hclt_backward");
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
@@ -1068,12 +1080,11 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
         PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_stats_lean_kernel<KK>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         // one workgroup fills a compute unit; they draw nodes from d_stat_claim_, which every launch leaves at zero
-        hipLaunchKernelGGL(hclt_stats_lean_kernel<KK>, dim3(std::min(n_inner_, n_cus_)), dim3(kStatLeanWaves * 64), lds,
-                           stream, d, d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
-                           H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
+        PCM_LAUNCH_PHASE(2, hclt_stats_lean_kernel<KK>, dim3(std::min(n_inner_, n_cus_)), dim3(kStatLeanWaves * 64), lds,
+                         d, d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
+                         H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
       });
       check_launch("hclt_stats_lean");
-      if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
       return;
     }
   }
@@ -1087,14 +1098,13 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
     fail(PCM_ERR_UNSUPPORTED, "statistics kernel needs %zu bytes of LDS, device offers %d", lds, max_lds_);
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, stream, d, d_stat_items_.p, d_edge_aggr_.p,
-                       d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
+    PCM_LAUNCH_PHASE(2, kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, d, d_stat_items_.p, d_edge_aggr_.p,
+                     d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   };
   PCM_DISPATCH_K(K_, {
     if (d.leaf_slice != 0) launch(&hclt_stats_kernel<KK, true>); else launch(&hclt_stats_kernel<KK, false>);
   });
   check_launch("hclt_stats");
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
 }
 
 void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
@@ -1334,10 +1344,10 @@ void HcltCircuit::check_walks() {
 
 hipEvent_t* HcltCircuit::ev_set() {
   if (ev_.empty()) {
-    ev_.resize((size_t)kTimingRing * 4, nullptr);
+    ev_.resize((size_t)kTimingRing * 6, nullptr);
     for (auto& e : ev_) PCM_HIP(hipEventCreate(&e));
   }
-  return ev_.data() + (size_t)(n_timed_ % kTimingRing) * 4;
+  return ev_.data() + (size_t)(n_timed_ % kTimingRing) * 6;
 }
 
 void HcltCircuit::read_timing(float* ms, int n) {
@@ -1348,7 +1358,7 @@ void HcltCircuit::read_timing(float* ms, int n) {
   for (int s = 0; s < cnt; ++s)
     for (int i = 0; i < std::min(n, 3); ++i) {
       float t = 0.f;
-      PCM_HIP(hipEventElapsedTime(&t, ev_[(size_t)s * 4 + i], ev_[(size_t)s * 4 + i + 1]));
+      PCM_HIP(hipEventElapsedTime(&t, ev_[(size_t)s * 6 + 2 * i], ev_[(size_t)s * 6 + 2 * i + 1]));
       ms[i] += t / cnt;
     }
   n_timed_ = 0;

@@ -256,7 +256,7 @@ class HcltCircuit : public pcm_circuit {
   bool force_general_walks_ = false;
   bool wide_walk_ = false;            // forward / backward / statistics run on the node-at-a-time wide kernels
   bool flows_in_general_ = false;   // the last flows were computed by the layered engine (soft evidence)
-  std::vector<hipEvent_t> ev_;   // kTimingRing sets of 4 events
+  std::vector<hipEvent_t> ev_;   // kTimingRing sets of 6 events: start and stop of the forward, backward, statistics phase
   int n_timed_ = 0;
   hipEvent_t* ev_set();
 

@@ -17,6 +17,8 @@
 //   O[k] = m + log(sum_j W[k,j] E[j])                              forward
 //   R[k] = F[k] / exp(O[k] - m),  G[j] = E[j] * sum_k W[k,j] R[k]   backward (F = parent's G, root: e_0)
 //   edge_aggr[k,j] += W[k,j] * sum_b R[b,k] E[b,j];  leaf_flow[u][x_b,u][j] += G[b,j]
+#include <hip/hip_ext.h>
+
 #include "hclt_engine.hpp"
 
 #include <hip/hip_runtime.h>
@@ -552,14 +554,14 @@ void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
   if (d_wide_ops_.n == 0) build_wide_tables();
   if ((size_t)V_ * d.leaf_stride >= ((size_t)1 << 31) || (size_t)n_inner_ * d.tile_stride >= ((size_t)1 << 31))
     fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call of the wide kernels", d.B);
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[0], stream));
   const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
   const int ops_in_lds = ops_bytes <= 32768;
-  PCM_DISPATCH_WIDE_K(K_, hipLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
-                                             ops_in_lds ? ops_bytes : 0, stream, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p,
-                                             d_ll));
+  // with timing on, a phase's start / stop events ride on its kernels' own dispatches
+  hipEvent_t* ev = timing ? ev_set() : nullptr;
+  PCM_DISPATCH_WIDE_K(K_, hipExtLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
+                                                (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, ev ? ev[0] : nullptr,
+                                                ev ? ev[1] : nullptr, 0, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_ll));
   check_launch_w("hclt_wide_forward");
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[1], stream));
 }
 
 // soft: the evidence is soft, the caller shares out the leaf flows from the G tiles itself
@@ -573,23 +575,24 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   while ((1 << bits) < d.Bp) ++bits;
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
+  hipEvent_t* ev = timing ? ev_set() : nullptr;
   PCM_DISPATCH_WIDE_K(K_, {
     const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
     const int ops_in_lds = ops_bytes <= 32768;
-    hipLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
-                       ops_in_lds ? ops_bytes : 0, stream, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_G_.p, d_wide_rs_.p,
-                       d_wide_es_.p);
+    hipExtLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
+                          (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, ev ? ev[2] : nullptr, ev ? ev[3] : nullptr, 0, d,
+                          d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_G_.p, d_wide_rs_.p, d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
-    if (timing) PCM_HIP(hipEventRecord(ev_set()[2], stream));
-    hipLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream, d,
-                       d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p, rate);
+    // statistics: the edge kernel starts the phase, the leaf kernel (absent with soft evidence) ends it
+    hipExtLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream,
+                          ev ? ev[4] : nullptr, ev && soft ? ev[5] : nullptr, 0, d, d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p,
+                          rate);
   });
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
   if (!soft)
-    hipLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), lds, stream, d, d_G_.p,
-                     d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
+    hipExtLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), (uint32_t)lds, stream, nullptr,
+                          ev ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
   check_launch_w("hclt_wide_stats");
-  if (timing) PCM_HIP(hipEventRecord(ev_set()[3], stream));
 }
 
 }  // namespace pcm

@@ -159,6 +159,29 @@ def test_config1_shape(gpu, oracle):
     _compare_step(gpu, oracle, 64, 16, 256, 1024, seed=11)
 
 
+@pytest.mark.parametrize("K", [32, 128])
+def test_kernel_timing_does_not_change_results(gpu, oracle, K):
+    """pcm_set_timing / pcm_get_timing: the three phases report a positive time each, the flows of a timed call are
+    the bits of an untimed one, and a second read without a call in between reports nothing."""
+    torch, P = gpu
+    from helpers import make_hclt, correlated_data, block_theta
+    parent, theta, leaf, _ = make_hclt(20, K, 16, 5)
+    data = torch.from_numpy(correlated_data(200, 20, 16, 6, parent)).cuda()
+    bpc = P.hclt_from_clt(parent, 16, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    ll0 = P.probs_flows_circuit(bpc, data).cpu().numpy()
+    ea0, lf0 = bpc.get_flows()
+    bpc.set_timing(True)
+    for _ in range(3):
+        ll1 = P.probs_flows_circuit(bpc, data).cpu().numpy()
+    ms = bpc.get_timing()
+    assert all(0.0 < ms[k] < 50.0 for k in ("forward", "backward", "statistics")), ms
+    ea1, lf1 = bpc.get_flows()
+    assert np.array_equal(ll0, ll1) and np.array_equal(lf0, lf1) and np.array_equal(ea0, ea1)
+    assert all(v == 0.0 for v in bpc.get_timing().values())
+    bpc.set_timing(False)
+
+
 @pytest.mark.parametrize("tree", [None, [-1, 0, 0], [-1, 0, 1, 1], [-1, 0, 0, 0, 0], [1, -1, 1, 2, 2, 0, 0, 3],
                                   [-1, 0, 0, 2, 2, 2, 4, 1, 6, 3, 9]])
 def test_param_vector_roundtrip(gpu, oracle, tree):
