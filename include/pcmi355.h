@@ -345,11 +345,14 @@ int pcm_adam_flow_step(pcm_circuit* c, int32_t batch_size, float* d_params, floa
 /* ---- instrumentation ----------------------------------------------------------- */
 
 /* Per-kernel timing, the role of `debug = true` -> `CUDA.@time` around each launch
- * (src/queries/likelihood.jl:86-92, src/queries/flow.jl:127-133).  When on, pcm_flows
- * brackets its forward / backward / statistics launches with events on the circuit's
- * stream (no synchronisation); pcm_get_timing synchronises and returns the mean
- * milliseconds over the calls since the previous read of each
- * (n <= 4 values: forward, backward, statistics, reserved). */
+ * (src/queries/likelihood.jl:86-92, src/queries/flow.jl:127-133).  When on, the
+ * forward / backward / statistics launches of pcm_flows carry a start and a stop event
+ * on their own dispatches (nothing is put between the kernels, nothing synchronises);
+ * pcm_get_timing synchronises and returns the mean milliseconds over the calls since
+ * the previous read of each (n <= 4 values: forward, backward, statistics, reserved).
+ * `on`: 0 off, 1 all three phases, otherwise a mask of phases (2 forward, 4 backward,
+ * 8 statistics): a timed dispatch costs a few microseconds, so a measurement of one
+ * kernel inside a throughput run times that kernel only; phases not timed read 0. */
 int pcm_set_timing(pcm_circuit* c, int32_t on);
 int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n);
 

@@ -310,7 +310,10 @@ int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent) {
 }
 
 int pcm_set_timing(pcm_circuit* c, int32_t on) {
-  return guarded([&] { need_hclt(c)->timing = on != 0; });
+  return guarded([&] {
+    if (on < 0 || on > 15) pcm::fail(PCM_ERR_ARG, "timing mode %d outside 0..15", on);
+    need_hclt(c)->set_timing(on == 1 ? 7 : on >> 1);
+  });
 }
 int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n) {
   return guarded([&] {

@@ -29,7 +29,7 @@ namespace pcm {
 // packets of their own that keep the next kernel waiting (measured: about 6 us each).
 #define PCM_LAUNCH_PHASE(phase, kernel, grid, block, lds, ...)                                                       \
   do {                                                                                                               \
-    if (timing) {                                                                                                    \
+    if (timing & (1 << (phase))) {                                                                                   \
       hipEvent_t* ev__ = ev_set() + 2 * (phase);                                                                     \
       hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)(lds), stream, ev__[0], ev__[1], 0, __VA_ARGS__);        \
     } else {                                                                                                         \
@@ -1357,6 +1357,7 @@ void HcltCircuit::read_timing(float* ms, int n) {
   PCM_HIP(hipStreamSynchronize(stream));
   for (int s = 0; s < cnt; ++s)
     for (int i = 0; i < std::min(n, 3); ++i) {
+      if (!(timing & (1 << i))) continue;
       float t = 0.f;
       PCM_HIP(hipEventElapsedTime(&t, ev_[(size_t)s * 6 + 2 * i], ev_[(size_t)s * 6 + 2 * i + 1]));
       ms[i] += t / cnt;

@@ -179,11 +179,15 @@ class HcltCircuit : public pcm_circuit {
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 
-  // Kernel timing: when on, pcm_flows brackets its forward / backward / statistics launches
-  // with events on the circuit's stream (no synchronisation); read_timing synchronises and
+  // Kernel timing: the launches of the phases in the mask (bit 0 forward, 1 backward, 2 statistics) carry a
+  // start and a stop event on their own dispatch (no synchronisation); read_timing synchronises and
   // averages the calls recorded since the previous read (at most kTimingRing of them).
   static constexpr int kTimingRing = 64;
-  bool timing = false;
+  int timing = 0;
+  void set_timing(int mask) {
+    timing = mask;
+    n_timed_ = 0;
+  }
   void read_timing(float* ms, int n);
 
  private:

@@ -557,7 +557,7 @@ void HcltCircuit::wide_forward(const HcltDev& d, float* d_ll) {
   const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
   const int ops_in_lds = ops_bytes <= 32768;
   // with timing on, a phase's start / stop events ride on its kernels' own dispatches
-  hipEvent_t* ev = timing ? ev_set() : nullptr;
+  hipEvent_t* ev = (timing & 1) ? ev_set() : nullptr;
   PCM_DISPATCH_WIDE_K(K_, hipExtLaunchKernelGGL(hclt_wide_forward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
                                                 (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, ev ? ev[0] : nullptr,
                                                 ev ? ev[1] : nullptr, 0, d, d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_ll));
@@ -576,22 +576,23 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   const int limb = std::min(24, 32 - bits);
   if (limb < 12) fail(PCM_ERR_UNSUPPORTED, "batch of %d examples is too large for one call", d.B);
   hipEvent_t* ev = timing ? ev_set() : nullptr;
+  const bool t_bwd = timing & 2, t_stat = timing & 4;
   PCM_DISPATCH_WIDE_K(K_, {
     const size_t ops_bytes = (size_t)n_inner_ * sizeof(WideOps);
     const int ops_in_lds = ops_bytes <= 32768;
     hipExtLaunchKernelGGL(hclt_wide_backward_kernel<KK>, dim3(d.nslices), dim3(wide_walk_waves<KK>() * 64),
-                          (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, ev ? ev[2] : nullptr, ev ? ev[3] : nullptr, 0, d,
+                          (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, t_bwd ? ev[2] : nullptr, t_bwd ? ev[3] : nullptr, 0, d,
                           d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_G_.p, d_wide_rs_.p, d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
     // statistics: the edge kernel starts the phase, the leaf kernel (absent with soft evidence) ends it
     hipExtLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream,
-                          ev ? ev[4] : nullptr, ev && soft ? ev[5] : nullptr, 0, d, d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p,
+                          t_stat ? ev[4] : nullptr, t_stat && soft ? ev[5] : nullptr, 0, d, d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p,
                           rate);
   });
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
   if (!soft)
     hipExtLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), (uint32_t)lds, stream, nullptr,
-                          ev ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
+                          t_stat ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
   check_launch_w("hclt_wide_stats");
 }
 

@@ -121,6 +121,8 @@ class HcltCircuit(BitsCircuit):
         return ea, lf
 
     def set_timing(self, on):
+        """0 / False: off; 1 / True: the forward, backward and statistics kernels of every flows call carry timing
+        events; 2, 4, 8 (or a sum of them): only the forward / backward / statistics kernel does."""
         check(lib.pcm_set_timing(self.handle, int(on)))
 
     def get_timing(self):

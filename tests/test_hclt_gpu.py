@@ -179,6 +179,10 @@ def test_kernel_timing_does_not_change_results(gpu, oracle, K):
     ea1, lf1 = bpc.get_flows()
     assert np.array_equal(ll0, ll1) and np.array_equal(lf0, lf1) and np.array_equal(ea0, ea1)
     assert all(v == 0.0 for v in bpc.get_timing().values())
+    bpc.set_timing(8)   # the statistics kernel only
+    P.probs_flows_circuit(bpc, data)
+    ms = bpc.get_timing()
+    assert ms["forward"] == 0.0 and ms["backward"] == 0.0 and 0.0 < ms["statistics"] < 50.0, ms
     bpc.set_timing(False)
 
 
