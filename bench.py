@@ -249,49 +249,85 @@ def secondary(args):
                    value=NC * B / dt, unit="examples/s",
                    config={"workload": args.workload, "circuits": NC, "streams": NS, "num_vars": V, "hidden": K,
                            "categories": C, "heads": H, "batch": B})
-    elif args.workload == "c4_full":
+    elif args.workload in ("c4_full", "c4_full_handles"):
         # C4 as a whole: 64 x 64 x 3 images cut into 64 patches of 8 x 8 x 3; one 192-variable K = 32 circuit with 128
-        # cluster heads per patch (block engine, 32 streams) and the K = 64 top-level HCLT over the 64 cluster ids
+        # cluster heads per patch and the K = 64 top-level HCLT over the 64 cluster ids.  c4_full: the 64 patch
+        # circuits as ONE forest handle over the 12288 pixels (one launch per kernel for all of them);
+        # c4_full_handles: a handle per patch circuit, queued on 32 streams.
         V, K, C, H, B, NP, NS = 192, 32, 256, 128, 1024, 64, 32
         img = workloads.grf_images(B, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(B, 3, 64, 64)
-        patches = [np.ascontiguousarray(img[:, :, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8]).reshape(B, V)
-                   for p in range(NP)]
+        pixel = np.arange(3 * 64 * 64).reshape(3, 64, 64)
+        pvars = [pixel[:, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8].reshape(V) for p in range(NP)]
+        flat = np.ascontiguousarray(img.reshape(B, -1))
         cluster = rng.integers(0, H, size=(B, NP)).astype(np.uint8)          # seeded uniform cluster ids
-        circs, datas, masks = [], [], []
-        for p in range(NP):
-            parent = workloads.chow_liu_parent(patches[p])
-            c = P.multihead_hclt_from_clt(parent, C, K, H)
-            th, lf = workloads.init_params(parent, K, C, 2000 + p, kind="dirichlet")
-            c.set_params(th, lf)                                             # heads stay uniform
-            circs.append(c)
-            datas.append(torch.from_numpy(patches[p]).cuda())
-            m = np.zeros((H, B), np.float32)
-            m[cluster[:, p], np.arange(B)] = 1.0
-            masks.append(torch.from_numpy(m).cuda())
+        parents = [workloads.chow_liu_parent(np.ascontiguousarray(flat[:, pv])) for pv in pvars]
+        params = [workloads.init_params(parents[p], K, C, 2000 + p, kind="dirichlet") for p in range(NP)]
         tparent = workloads.chow_liu_parent(cluster)
         top = P.hclt_from_clt(tparent, H, 64)
         top.set_params(*workloads.init_params(tparent, 64, H, 2100, kind="dirichlet"))
         dtop = torch.from_numpy(cluster).cuda()
-        lls = [torch.empty(B, device="cuda") for _ in range(NP + 1)]
-        streams = [torch.cuda.Stream() for _ in range(NS)]
-        torch.cuda.synchronize()
-        for i, c in enumerate(circs):
-            check(lib.pcm_set_stream(c.handle, streams[i % NS].cuda_stream))
-        check(lib.pcm_set_stream(top.handle, streams[0].cuda_stream))
+        ll_top = torch.empty(B, device="cuda")
+        n_int = [int((np.bincount(par[par >= 0], minlength=V) > 0).sum()) for par in parents]
+        if args.workload == "c4_full":
+            fparent = np.empty(NP * V, np.int32)
+            theta = np.empty((NP * V, K, K), np.float32)
+            leaf = np.empty((NP * V, K, C), np.float32)
+            for pv, par, (th, lf) in zip(pvars, parents, params):
+                fparent[pv] = np.where(par < 0, -1, pv[np.maximum(par, 0)])
+                theta[pv], leaf[pv] = th, lf
+            forest = P.hclt_forest_from_clts(fparent, C, K, H)               # heads stay uniform
+            forest.set_params(theta, leaf)
+            roots = [int(pv[np.flatnonzero(par < 0)[0]]) for pv, par in zip(pvars, parents)]
+            mask = np.zeros((NP, H, B), np.float32)
+            for t, p in enumerate(np.argsort(roots)):                        # trees are numbered by their root's variable
+                mask[t, cluster[:, p], np.arange(B)] = 1.0
+            dmask = torch.from_numpy(mask).cuda()
+            d = torch.from_numpy(flat).cuda()
+            ll = torch.empty((NP, B), device="cuda")
+            streams = [torch.cuda.Stream() for _ in range(2)]
+            torch.cuda.synchronize()
+            check(lib.pcm_set_stream(forest.handle, streams[0].cuda_stream))
+            check(lib.pcm_set_stream(top.handle, streams[1].cuda_stream))
 
-        def step():
-            for c, d, hm, ll in zip(circs, datas, masks, lls):
-                check(lib.pcm_flows(c.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(), ll.data_ptr()))
-                check(lib.pcm_em_update(c.handle, 0.1, 0.9))
-            check(lib.pcm_em_step(top.handle, dtop.data_ptr(), dtop.stride(0), dtop.stride(1), None, B, 0.0, 0.1, 0.9,
-                                  lls[NP].data_ptr()))
+            def step():
+                check(lib.pcm_flows(forest.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, dmask.data_ptr(),
+                                    ll.data_ptr()))
+                check(lib.pcm_em_update(forest.handle, 0.1, 0.9))
+                check(lib.pcm_em_step(top.handle, dtop.data_ptr(), dtop.stride(0), dtop.stride(1), None, B, 0.0, 0.1, 0.9,
+                                      ll_top.data_ptr()))
+            how = "one forest handle"
+        else:
+            circs, datas, masks = [], [], []
+            for p in range(NP):
+                c = P.multihead_hclt_from_clt(parents[p], C, K, H)
+                c.set_params(*params[p])                                     # heads stay uniform
+                circs.append(c)
+                datas.append(torch.from_numpy(np.ascontiguousarray(flat[:, pvars[p]])).cuda())
+                m = np.zeros((H, B), np.float32)
+                m[cluster[:, p], np.arange(B)] = 1.0
+                masks.append(torch.from_numpy(m).cuda())
+            lls = [torch.empty(B, device="cuda") for _ in range(NP)]
+            streams = [torch.cuda.Stream() for _ in range(NS)]
+            torch.cuda.synchronize()
+            for i, c in enumerate(circs):
+                check(lib.pcm_set_stream(c.handle, streams[i % NS].cuda_stream))
+            check(lib.pcm_set_stream(top.handle, streams[0].cuda_stream))
+
+            def step():
+                for c, d, hm, ll in zip(circs, datas, masks, lls):
+                    check(lib.pcm_flows(c.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(),
+                                        ll.data_ptr()))
+                    check(lib.pcm_em_update(c.handle, 0.1, 0.9))
+                check(lib.pcm_em_step(top.handle, dtop.data_ptr(), dtop.stride(0), dtop.stride(1), None, B, 0.0, 0.1, 0.9,
+                                      ll_top.data_ptr()))
+            how = "%d handles on %d streams" % (NP, NS)
         dt = _timed(torch, step, args.steps, args.warmup)
-        algo = sum(algorithmic_bytes(c.size("inner_tree_nodes"), V, K, C, B)["step"] + 2 * 4 * H * B for c in circs) \
+        algo = sum(algorithmic_bytes(n, V, K, C, B)["step"] + 2 * 4 * H * B for n in n_int) \
             + algorithmic_bytes(top.size("inner_tree_nodes"), NP, 64, H, B)["step"]
         out.update(metric="images/sec fwd+bwd+EM, 12288-variable patch-clustered circuit: 64 patch circuits (192 vars, K=32, "
-                          "128 heads) on 32 streams + top HCLT (64 vars, K=64)",
+                          "128 heads; %s) + top HCLT (64 vars, K=64)" % how,
                    value=B / dt, unit="examples/s",
-                   config={"workload": args.workload, "patch_circuits": NP, "streams": NS, "num_vars": NP * V, "hidden": K,
+                   config={"workload": args.workload, "patch_circuits": NP, "num_vars": NP * V, "hidden": K,
                            "top_hidden": 64, "categories": C, "heads": H, "batch": B})
     elif args.workload == "c4_top_soft":
         # the top-level circuit of C4: 64 patch variables, 128 cluster categories, K = 64, trained on soft evidence

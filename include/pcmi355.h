@@ -64,6 +64,35 @@ int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32
                               int32_t num_heads, pcm_circuit** out);
 
 /*
+ * Many multi-head HCLTs over one batch as ONE handle: the 64 patch circuits of
+ * exps/progressive_growing/parallel_PG.jl:214-225, each of which the reference trains with its own
+ * `mini_batch_em_for_multihead_pc` call (src-jl/multi_head_pc/em.jl:1-99) on its own columns of the same
+ * images.  clt_parent is a forest over the num_vars variables of the batch: every -1 entry roots a tree
+ * (trees are numbered by their root's variable index), every tree has at least two variables and gets
+ * num_heads heads.  The handle is a container for running them together -- one launch per kernel for
+ * all trees, the walks' sixteen waves filled with nodes of different trees -- and computes per tree the
+ * bits a handle of pcm_hclt_create_multihead over that tree's variables (numbered in the same relative
+ * order: a node's children are added up in variable order) would:
+ *   pcm_loglikelihoods  d_ll_out [num_trees][num_heads][batch]
+ *   pcm_flows           d_head_mask [num_trees][num_heads][batch], d_ll_out [num_trees][batch]
+ *   pcm_em_update, pcm_em_step (mask as pcm_flows), pcm_set_stream, pcm_set_timing
+ *   pcm_hclt_set_params / get_params / get_flows  (per-variable blocks: rows of trees stay apart)
+ *   pcm_hclt_set_heads / get_heads, pcm_size
+ * Everything a single circuit defines beyond that (parameter vector and index tables, KL, sampling, soft
+ * evidence, Adam) returns PCM_ERR_UNSUPPORTED: move a tree's blocks and heads to a handle of its own for those.
+ * Needs num_hidden_cats 16 or 32 and trees the lean walk kernels take (at most three children per tree
+ * node), PCM_ERR_UNSUPPORTED otherwise.
+ */
+int pcm_hclt_create_forest(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
+                           int32_t num_heads, pcm_circuit** out);
+
+/* Head log-parameters of a multi-head HCLT or a forest, [num_trees][num_heads][num_hidden_cats] on the host:
+ * the `params` of the head sum nodes (src-jl/multi_head_pc/bit_circuit.jl:14-56 keeps them in the heads'
+ * edges), row h of a tree being the head that row h of its head mask seeds. */
+int pcm_hclt_set_heads(pcm_circuit* c, const float* heads);
+int pcm_hclt_get_heads(pcm_circuit* c, float* heads);
+
+/*
  * Compile a general circuit given as a DAG in topological order (children before
  * parents, root last), the flat form a binding obtains by walking a `ProbCircuit`:
  * replaces `CuMetaBitsProbCircuit(pc)` (src/bits_circuit.jl:39) and, with num_heads > 0,
@@ -98,7 +127,8 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
  * HCLT), 8 inner tree nodes (HCLT), 9 up layers, 10 parameter groups, 11 input nodes,
  * 12 heads (0 for a single-root circuit), 13 nodes of the description the circuit was
  * built from (0 for an HCLT built from its tree), 14 which kernels run likelihoods and flows:
- * 0 per-layer kernels, 1 lean tree walks, 2 general tree walks, 3 wide block kernels. */
+ * 0 per-layer kernels, 1 lean tree walks, 2 general tree walks, 3 wide block kernels, 15 trees (1 unless
+ * the handle is a forest). */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.

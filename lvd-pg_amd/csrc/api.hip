@@ -134,6 +134,23 @@ int pcm_update_parameters(pcm_circuit* c, const float* p, int64_t n) {
   });
 }
 
+int pcm_hclt_create_forest(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
+                           int32_t num_heads, pcm_circuit** out) {
+  return guarded([&] {
+    if (!out) pcm::fail(PCM_ERR_ARG, "out is null");
+    *out = nullptr;
+    if (num_heads < 1) pcm::fail(PCM_ERR_SHAPE, "num_heads must be positive, got %d", num_heads);
+    adopt(*out = new pcm::HcltCircuit(clt_parent, num_vars, num_hidden_cats, num_cats, num_heads, true));
+  });
+}
+
+int pcm_hclt_set_heads(pcm_circuit* c, const float* heads) {
+  return guarded([&] { need_hclt(c)->set_heads(heads); });
+}
+int pcm_hclt_get_heads(pcm_circuit* c, float* heads) {
+  return guarded([&] { need_hclt(c)->get_heads(heads); });
+}
+
 int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf) {
   return guarded([&] { need_hclt(c)->set_block_params(theta, leaf); });
 }

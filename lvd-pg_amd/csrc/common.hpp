@@ -87,6 +87,10 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(const float* __restrict_
   __shared__ float sub[4][64];
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int64_t i = (int64_t)blockIdx.x * 64 + lane;
+  // blockIdx.y: one of several independent sums laid out one behind the other (the trees of a forest)
+  part += (size_t)blockIdx.y * n_parts * n;
+  dst += (size_t)blockIdx.y * n;
+  if (kExpWeight) logw += (size_t)blockIdx.y * n;
   float s = 0.f;
   if (i < n)
     for (int q = g; q < n_parts; q += 4) s += part[(size_t)q * n + i];

@@ -42,8 +42,10 @@ static void check_launch(const char* what) {
   if (e != hipSuccess) fail(PCM_ERR_HIP, "launch of %s failed: %s", what, hipGetErrorString(e));
 }
 
-HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads) : V_(V), K_(K), C_(C) {
+HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads, bool forest)
+    : V_(V), K_(K), C_(C), forest_(forest) {
   if (num_heads < 0 || num_heads > 4096) fail(PCM_ERR_SHAPE, "num_heads must be in 0..4096, got %d", num_heads);
+  if (forest && num_heads < 1) fail(PCM_ERR_SHAPE, "the trees of a forest are multi-head circuits: num_heads must be positive");
   H_ = num_heads;
   Hp_ = ceil_div(num_heads, 16) * 16;
   if (!parent) fail(PCM_ERR_ARG, "clt_parent is null");
@@ -55,6 +57,8 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   wide_ = K == 128;
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
+  Vu_ = V;
+  if (forest_) split_wide_nodes();
   build_structure();
   // K = 64: a parameter block and its prefetched successor do not fit the 128 registers a wave of the 16-wave
   // walk kernels has, so those kernels spill (6 us per step); the node-at-a-time wide kernels take about
@@ -62,21 +66,27 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   wide_walk_ = wide_ || (K == 64 && (double)n_inner_ * kWideNodeUs < (double)(n_fwd_steps_ + n_bwd_steps_) * 0.5 * kWalk64StepUs);
   if (H_ > 0 && !(block_ && K <= 32))
     fail(PCM_ERR_UNSUPPORTED, "multi-head block kernels need K = 16 or 32; compile this circuit with pcm_circuit_create");
-  build_param_order();
+  if (forest_ && !lean_)
+    fail(PCM_ERR_UNSUPPORTED, "a forest needs trees the lean walk kernels take (at most three children per node, "
+                              "every tile in LDS); use one handle per tree");
+  if (!forest_) build_param_order();
 
   // uniform parameters
-  std::vector<float> theta((size_t)V_ * K_ * K_, -std::log((float)K_));
-  std::vector<float> leaf((size_t)V_ * K_ * C_, -std::log((float)C_));
+  std::vector<float> theta((size_t)Vu_ * K_ * K_, -std::log((float)K_));
+  std::vector<float> leaf((size_t)Vu_ * K_ * C_, -std::log((float)C_));
   d_leaf_.alloc((size_t)V_ * C_ * K_);
-  d_logtheta_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)H_ * K_);   // the head rows sit behind the blocks
+  d_logtheta_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)T_ * H_ * K_);   // the head rows sit behind the blocks
   d_Wf_.alloc((size_t)n_inner_ * K_ * K_);
   d_Wb_.alloc((size_t)n_inner_ * K_ * K_);
-  d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)H_ * K_);
+  d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)T_ * H_ * K_);
   if (H_ > 0) {
-    d_head_wf_.alloc((size_t)Hp_ * K_);
+    d_head_wf_.alloc((size_t)T_ * Hp_ * K_);
     d_flow_shift_.alloc(1);
-    d_head_wb_.alloc((size_t)Hp_ * K_);
-    std::vector<float> hl((size_t)H_ * K_, -std::log((float)K_));
+    d_head_wb_.alloc((size_t)T_ * Hp_ * K_);
+    std::vector<int32_t> rn;
+    for (int r : roots_) rn.push_back(inner_of_var_[r]);
+    d_root_node_.upload(rn);
+    std::vector<float> hl((size_t)T_ * H_ * K_, -std::log((float)K_));
     PCM_HIP(hipMemcpy(head_logp(), hl.data(), hl.size() * sizeof(float), hipMemcpyHostToDevice));
   }
   d_leaf_flow_.alloc((size_t)V_ * C_ * K_);
@@ -85,14 +95,43 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   set_block_params(theta.data(), leaf.data());
 }
 
+// The lean walk kernels hold three children per tree node.  A forest meets that by construction: a node with
+// more children hands the last two or three of them to an auxiliary node below it, a tree node over a variable
+// of its own that nobody observes (variables Vu_ .. V_-1: one category with probability 1, so its leaf row adds
+// nothing) with the identity as its block (so its sum nodes ARE its products: the value of the K products
+// the children form goes up unchanged, the flow goes down unchanged).  The update kernels leave the auxiliary
+// blocks and leaf rows alone, and the caller's arrays never show them.  It is the same circuit: a product of
+// five factors written as a product of three, one of which is a product of three.
+void HcltCircuit::split_wide_nodes() {
+  for (int v = 0; v < Vu_; ++v)
+    if (parent_[v] >= Vu_ || parent_[v] == v) fail(PCM_ERR_SHAPE, "clt_parent[%d] = %d is out of range", v, parent_[v]);
+  std::vector<std::vector<int32_t>> ch(Vu_);
+  for (int v = 0; v < Vu_; ++v)
+    if (parent_[v] >= 0) ch[parent_[v]].push_back(v);
+  for (int v = 0; v < Vu_; ++v) {
+    std::vector<int32_t> c = ch[v];
+    while (c.size() > 3) {
+      const size_t take = std::min<size_t>(3, c.size() - 2);
+      const int u = (int)parent_.size();
+      parent_.push_back(v);
+      for (size_t i = c.size() - take; i < c.size(); ++i) parent_[c[i]] = u;
+      c.resize(c.size() - take);
+      c.push_back(u);
+    }
+  }
+  V_ = (int)parent_.size();
+}
+
 void HcltCircuit::build_structure() {
   children_.assign(V_, {});
   root_ = -1;
+  roots_.clear();
   for (int v = 0; v < V_; ++v) {
     int p = parent_[v];
     if (p < 0) {
-      if (root_ >= 0) fail(PCM_ERR_SHAPE, "clt_parent has more than one root (%d and %d)", root_, v);
-      root_ = v;
+      if (root_ >= 0 && !forest_) fail(PCM_ERR_SHAPE, "clt_parent has more than one root (%d and %d)", root_, v);
+      if (root_ < 0) root_ = v;
+      roots_.push_back(v);
     } else {
       if (p >= V_ || p == v) fail(PCM_ERR_SHAPE, "clt_parent[%d] = %d is out of range", v, p);
       children_[p].push_back(v);
@@ -103,22 +142,26 @@ void HcltCircuit::build_structure() {
   std::vector<int32_t> order;
   order.reserve(V_);
   std::vector<std::pair<int32_t, int32_t>> st;
-  st.push_back({root_, 0});
   depth_.assign(V_, -1);
-  depth_[root_] = 0;
-  while (!st.empty()) {
-    auto& top = st.back();
-    int v = top.first;
-    if (top.second < (int)children_[v].size()) {
-      int c = children_[v][top.second++];
-      depth_[c] = depth_[v] + 1;
-      st.push_back({c, 0});
-    } else {
-      order.push_back(v);
-      st.pop_back();
+  T_ = (int)roots_.size();
+  for (int r : roots_) {   // tree after tree
+    if (children_[r].empty()) fail(PCM_ERR_SHAPE, "variable %d is a tree of its own: a tree needs at least 2 variables", r);
+    st.push_back({r, 0});
+    depth_[r] = 0;
+    while (!st.empty()) {
+      auto& top = st.back();
+      int v = top.first;
+      if (top.second < (int)children_[v].size()) {
+        int c = children_[v][top.second++];
+        depth_[c] = depth_[v] + 1;
+        st.push_back({c, 0});
+      } else {
+        order.push_back(v);
+        st.pop_back();
+      }
     }
   }
-  if ((int)order.size() != V_) fail(PCM_ERR_SHAPE, "clt_parent is not a tree: %d of %d variables reach the root",
+  if ((int)order.size() != V_) fail(PCM_ERR_SHAPE, "clt_parent is not a tree: %d of %d variables reach a root",
                                     (int)order.size(), V_);
   inner_of_var_.assign(V_, -1);
   var_of_inner_.clear();
@@ -132,6 +175,12 @@ void HcltCircuit::build_structure() {
     height_[v] = h + 1;
   }
   n_inner_ = (int)var_of_inner_.size();
+  // post-order goes tree after tree: a node's tree is the number of roots before it
+  tree_of_inner_.assign(n_inner_, 0);
+  for (int n = 0, t = 0; n < n_inner_; ++n) {
+    tree_of_inner_[n] = t;
+    if (parent_[var_of_inner_[n]] < 0) ++t;
+  }
 
   std::vector<HcltNode> nodes(n_inner_);
   std::vector<int32_t> ci, cl;
@@ -140,7 +189,7 @@ void HcltCircuit::build_structure() {
     HcltNode& nd = nodes[n];
     nd.var = v;
     nd.parent = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
-    nd.is_root = v == root_;
+    nd.is_root = parent_[v] < 0 || v >= Vu_;   // (the sum-edge update skips identity blocks: heads' roots, auxiliary nodes)
     nd.ic_off = (int)ci.size();
     nd.lc_off = (int)cl.size();
     for (int c : children_[v]) {
@@ -250,10 +299,12 @@ void HcltCircuit::build_schedules() {
   // if some node has more operands than the lean kernels hold
   const size_t leaf_stride = (size_t)C_ * K_ * sizeof(float);
   // (backward: ratio_slot[n] is the LDS slot in which node n finds its ratio tile, left there by its parent)
-  auto make_lean = [&](const std::vector<StepItem>& sched, bool forward, int stride, DevBuf<int32_t>& dst,
+  auto make_lean = [&](const std::vector<StepItem>& sched, bool forward, int stride, std::vector<int32_t>& dst,
                        const std::vector<int32_t>* ratio_slot = nullptr) -> bool {
     if (K_ > 32 || lds_slots_ > 255 || (size_t)V_ * leaf_stride >= ((size_t)1 << 31)) return false;
-    std::vector<int32_t> f((size_t)kLeanFields * kWalkWaves * stride, 0);
+    const size_t f0 = dst.size();   // (the rows of a further group of trees go behind those of the groups before)
+    dst.resize(f0 + (size_t)kLeanFields * kWalkWaves * stride, 0);
+    int32_t* f = dst.data() + f0;
     // how often each slot has been filled so far: a step's reads see the fills of earlier steps only, so the
     // readers of a step are numbered before its writers
     std::vector<int32_t> fills(256, 0);
@@ -321,26 +372,48 @@ void HcltCircuit::build_schedules() {
           put(kLSlots, (int32_t)slots);
         }
       }
-    dst.upload(f);
     return true;
   };
   auto depth_of = [&](int n) { return depth_[var_of_inner_[n]]; };
 
-  // ---- forward -----------------------------------------------------------------------
+  // A forest's trees are walked in groups side by side (blockIdx.y of the walk kernels): each group of whole trees
+  // has a schedule of its own, so that a batch too small to fill the device with its slices (1024 examples are 64
+  // workgroups) still does.  Groups are node ranges (post-order goes tree after tree) of about equal size.
+  std::vector<std::pair<int, int>> groups;
   {
+    const int G = forest_ ? std::max(1, std::min(4, T_ / 8)) : 1;
+    int n0 = 0;
+    for (int g = 0; g < G && n0 < n_inner_; ++g) {
+      // up to the end of the tree in which this group's share of the nodes is reached
+      const int want = (int)((int64_t)n_inner_ * (g + 1) / G);
+      int n1 = std::max(n0 + 1, want);
+      while (n1 < n_inner_ && tree_of_inner_[n1] == tree_of_inner_[n1 - 1]) ++n1;
+      if (g == G - 1) n1 = n_inner_;
+      groups.push_back({n0, n1});
+      n0 = n1;
+    }
+  }
+  n_groups_ = (int)groups.size();
+
+  // ---- forward -----------------------------------------------------------------------
+  auto schedule_forward = [&](int g0, int g1, std::vector<StepItem>& sched, std::vector<PreItem>& pre) {
     std::vector<int32_t> pending(n_inner_), slot(n_inner_, -1), free_slots;
     for (int s = trash_slot - 1; s >= 0; --s) free_slots.push_back(s);
-    auto cmp = [&](int a, int b) {   // max-heap: deeper first, then lower id (post-order)
+    // max-heap: deeper first, then lower id (post-order).  In a forest the earlier tree goes first whatever the
+    // depth: the trees then pass through the waves one behind the other, a few at a time, and the tiles that wait
+    // for a parent in LDS are those of a few trees instead of all.
+    auto cmp = [&](int a, int b) {
+      if (tree_of_inner_[a] != tree_of_inner_[b]) return tree_of_inner_[a] > tree_of_inner_[b];
       return depth_of(a) != depth_of(b) ? depth_of(a) < depth_of(b) : a > b;
     };
+    // ... and a node without inner children, which fills a slot and frees none, only starts while more than a
+    // step's worth of slots is free (or nothing else can run)
+    const int producer_reserve = T_ > 1 ? kWalkWaves : 0;
     std::vector<int32_t> ready;
-    for (int n = 0; n < n_inner_; ++n) { pending[n] = (int)ic[n].size(); if (!pending[n]) ready.push_back(n); }
+    for (int n = g0; n < g1; ++n) { pending[n] = (int)ic[n].size(); if (!pending[n]) ready.push_back(n); }
     std::make_heap(ready.begin(), ready.end(), cmp);
-    std::vector<StepItem> sched;
-    std::vector<PreItem> pre;
-    fwd_spill_ = false;
     int done = 0;
-    while (done < n_inner_) {
+    while (done < g1 - g0) {
       // nodes whose flow tile needs an LDS slot wait while none is free (their turn comes
       // when children of earlier nodes have drained); only if nothing else is ready does a
       // tile go through HBM instead
@@ -350,13 +423,23 @@ void HcltCircuit::build_schedules() {
         std::pop_heap(ready.begin(), ready.end(), cmp);
         const int n = ready.back();
         ready.pop_back();
-        if (!ic[n].empty()) {
+        if (T_ > 1) {
+          if (par[n] >= 0) {
+            if (slots_left <= (ic[n].empty() ? producer_reserve : 0)) { deferred.push_back(n); continue; }
+            --slots_left;
+          }
+        } else if (!ic[n].empty()) {
           if (slots_left == 0) { deferred.push_back(n); continue; }
           --slots_left;
         }
         step.push_back(n);
       }
-      if (step.empty() && !deferred.empty()) { step.push_back(deferred.back()); deferred.pop_back(); }
+      if (step.empty() && !deferred.empty()) {
+        // nothing fits: the first of the waiting nodes in heap order (a forest) / the last (one tree) goes anyway
+        const size_t pick = T_ > 1 ? 0 : deferred.size() - 1;
+        step.push_back(deferred[pick]);
+        deferred.erase(deferred.begin() + (std::ptrdiff_t)pick);
+      }
       for (int n : deferred) { ready.push_back(n); std::push_heap(ready.begin(), ready.end(), cmp); }
       if (step.empty()) fail(PCM_ERR_SHAPE, "forward schedule stalled (tree is inconsistent)");
       for (int w = 0; w < kWalkWaves; ++w) {
@@ -392,26 +475,43 @@ void HcltCircuit::build_schedules() {
         ++done;
       }
     }
-    n_fwd_steps_ = (int)sched.size() / kWalkWaves;
-    make_fields(sched, pre, true, fwd_stride_, d_fwd_fields_);
-    fwd_lean_ = !fwd_spill_ && make_lean(sched, true, fwd_stride_, d_fwd_lean_);
-    d_fwd_sched_.upload(sched);
+  };
+  auto pad_steps = [&](std::vector<StepItem>& sched, std::vector<PreItem>& pre, int steps) {
+    while ((int)sched.size() < steps * kWalkWaves) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); }
+  };
+  {
+    fwd_spill_ = false;
+    std::vector<std::vector<StepItem>> sched(n_groups_);
+    std::vector<std::vector<PreItem>> pre(n_groups_);
+    n_fwd_steps_ = 0;
+    for (int g = 0; g < n_groups_; ++g) {
+      schedule_forward(groups[g].first, groups[g].second, sched[g], pre[g]);
+      n_fwd_steps_ = std::max(n_fwd_steps_, (int)sched[g].size() / kWalkWaves);
+    }
+    std::vector<int32_t> lean_rows;
+    fwd_lean_ = !fwd_spill_;
+    for (int g = 0; g < n_groups_; ++g) {
+      pad_steps(sched[g], pre[g], n_fwd_steps_);   // the shorter groups idle at the end
+      if (g == 0) make_fields(sched[g], pre[g], true, fwd_stride_, d_fwd_fields_);
+      else pad_steps(sched[g], pre[g], fwd_stride_);
+      fwd_lean_ = fwd_lean_ && make_lean(sched[g], true, fwd_stride_, lean_rows);
+    }
+    if (fwd_lean_) d_fwd_lean_.upload(lean_rows);
+    d_fwd_sched_.upload(sched[0]);
   }
   // ---- backward ----------------------------------------------------------------------
   // Oldest-ready first (ties: longest chain below first): a parent's flow tile then leaves
   // its LDS slot a few steps after it was produced, so the number of live tiles stays near
   // the width of the tree instead of growing with every postponed short subtree.
-  {
+  auto schedule_backward = [&](int g0, int g1, std::vector<StepItem>& sched, std::vector<PreItem>& pre) {
     std::vector<int32_t> remaining(n_inner_), slot(n_inner_, -1), ready_at(n_inner_, 0), free_slots;
     for (int s = trash_slot - 1; s >= 0; --s) free_slots.push_back(s);
     std::vector<int32_t> ready;
-    for (int n = 0; n < n_inner_; ++n) { remaining[n] = (int)ic[n].size(); if (par[n] < 0) ready.push_back(n); }
-    std::vector<StepItem> sched;
-    std::vector<PreItem> pre;
-    bwd_spill_ = false;
-    int done = 0, step_no = 0;
-    while (done < n_inner_) {
+    for (int n = g0; n < g1; ++n) { remaining[n] = (int)ic[n].size(); if (par[n] < 0) ready.push_back(n); }
+    int done = 0, step_no = 0, ratio_live = 0;
+    while (done < g1 - g0) {
       std::sort(ready.begin(), ready.end(), [&](int a, int b) {
+        if (tree_of_inner_[a] != tree_of_inner_[b]) return tree_of_inner_[a] < tree_of_inner_[b];   // a forest: tree after tree
         if (ready_at[a] != ready_at[b]) return ready_at[a] < ready_at[b];
         return hin[a] != hin[b] ? hin[a] > hin[b] : a > b;
       });
@@ -420,9 +520,15 @@ void HcltCircuit::build_schedules() {
       std::vector<int32_t> step, rest;
       int slots_left = (int)free_slots.size();
       for (int n : ready) {
-        if ((int)step.size() < kWalkWaves && (ic[n].empty() || slots_left > 0)) {
+        // a forest also counts the ratio tiles of the lean walk while it schedules (one per inner child, from the
+        // parent's step to the end of the child's): a node only runs if its children's tiles fit, and a new tree
+        // only starts while half the slots are free, so that the trees under way can finish
+        const int need = (int)ic[n].size();
+        const bool ratio_ok = T_ == 1 || ratio_live + need <= (par[n] < 0 ? trash_slot / 2 : trash_slot);
+        if ((int)step.size() < kWalkWaves && (ic[n].empty() || slots_left > 0) && ratio_ok) {
           step.push_back(n);
           if (!ic[n].empty()) --slots_left;
+          ratio_live += need;
         } else {
           rest.push_back(n);
         }
@@ -453,20 +559,32 @@ void HcltCircuit::build_schedules() {
       }
       ++step_no;
       for (int n : step) {
+        if (par[n] >= 0) --ratio_live;
         if (par[n] >= 0 && --remaining[par[n]] == 0 && slot[par[n]] >= 0) free_slots.push_back(slot[par[n]]);
         for (int c : ic[n]) { ready.push_back(c); ready_at[c] = step_no; }
         ++done;
       }
     }
-    n_bwd_steps_ = (int)sched.size() / kWalkWaves;
+  };
+  {
+    bwd_spill_ = false;
+    std::vector<std::vector<StepItem>> scheds(n_groups_);
+    std::vector<std::vector<PreItem>> pres(n_groups_);
+    n_bwd_steps_ = 0;
+    for (int g = 0; g < n_groups_; ++g) {
+      schedule_backward(groups[g].first, groups[g].second, scheds[g], pres[g]);
+      n_bwd_steps_ = std::max(n_bwd_steps_, (int)scheds[g].size() / kWalkWaves);
+    }
     // The lean backward walk hands every inner child its own tile: a slot per (parent, inner child) pair, taken
     // in the parent's step and free again from the step after the child's.
     std::vector<int32_t> ratio_slot(n_inner_, -1);
     bool slots_ok = true;
-    {
+    for (int g = 0; g < n_groups_; ++g) {
+      const std::vector<StepItem>& sched = scheds[g];
+      const int g_steps = (int)sched.size() / kWalkWaves;
       std::vector<int32_t> fs;
       for (int sl = trash_slot - 1; sl >= 0; --sl) fs.push_back(sl);
-      for (int st = 0; st < n_bwd_steps_ && slots_ok; ++st) {
+      for (int st = 0; st < g_steps && slots_ok; ++st) {
         std::vector<int32_t> freed;
         for (int w = 0; w < kWalkWaves && slots_ok; ++w) {
           const int n = sched[(size_t)st * kWalkWaves + w].node;
@@ -481,9 +599,16 @@ void HcltCircuit::build_schedules() {
         fs.insert(fs.end(), freed.begin(), freed.end());
       }
     }
-    make_fields(sched, pre, false, bwd_stride_, d_bwd_fields_);
-    bwd_lean_ = slots_ok && make_lean(sched, false, bwd_stride_, d_bwd_lean_, &ratio_slot);
-    d_bwd_sched_.upload(sched);
+    std::vector<int32_t> lean_rows;
+    bwd_lean_ = slots_ok;
+    for (int g = 0; g < n_groups_; ++g) {
+      pad_steps(scheds[g], pres[g], n_bwd_steps_);
+      if (g == 0) make_fields(scheds[g], pres[g], false, bwd_stride_, d_bwd_fields_);
+      else pad_steps(scheds[g], pres[g], bwd_stride_);
+      bwd_lean_ = bwd_lean_ && make_lean(scheds[g], false, bwd_stride_, lean_rows, &ratio_slot);
+    }
+    if (bwd_lean_) d_bwd_lean_.upload(lean_rows);
+    d_bwd_sched_.upload(scheds[0]);
   }
   // ---- statistics: the static operands of every node ------------------------------------
   {
@@ -532,9 +657,10 @@ void HcltCircuit::build_schedules() {
   if (ext.empty()) ext.push_back(0);
   d_ext_ops_.upload(ext);
   if (getenv("PCM_VERBOSE"))
-    fprintf(stderr, "[pcmi355] hclt V=%d K=%d C=%d inner=%d: forward %d steps%s%s, backward %d steps%s%s, %d LDS slots\n",
-            V_, K_, C_, n_inner_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", fwd_lean_ ? " (lean)" : "", n_bwd_steps_,
-            bwd_spill_ ? " (spills)" : "", bwd_lean_ ? " (lean)" : "", lds_slots_);
+    fprintf(stderr, "[pcmi355] hclt V=%d K=%d C=%d inner=%d trees=%d groups=%d: forward %d steps%s%s, backward %d steps%s%s, statistics%s, "
+            "%d LDS slots\n",
+            V_, K_, C_, n_inner_, T_, n_groups_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", fwd_lean_ ? " (lean)" : "", n_bwd_steps_,
+            bwd_spill_ ? " (spills)" : "", bwd_lean_ ? " (lean)" : "", stat_lean_ ? " (lean)" : "", lds_slots_);
 }
 
 // Numbering the reference would give this circuit.  Nodes are created in depth-first
@@ -728,7 +854,7 @@ int64_t HcltCircuit::size(int what) const {
     case 2: return n_nodes_;
     case 3: return n_edges_;
     case 4: return (int64_t)V_ * K_ * C_;
-    case 5: return V_;
+    case 5: return Vu_;
     case 6: return C_;
     case 7: return K_;
     case 8: return n_inner_;
@@ -738,11 +864,13 @@ int64_t HcltCircuit::size(int what) const {
     case 12: return H_;
     case 13: return 0;
     case 14: return wide_walk_ ? 3 : !block_ ? 0 : lean_ ? 1 : 2;
+    case 15: return T_;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
 
 void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
+  no_forest("an index table");
   auto copy = [&](const std::vector<int64_t>& v) {
     if ((int64_t)v.size() != n) fail(PCM_ERR_ARG, "index table %d has %lld entries, caller gave %lld",
                                      which, (long long)v.size(), (long long)n);
@@ -793,17 +921,17 @@ void HcltCircuit::rebuild_w() {
 
 void HcltCircuit::rebuild_heads() {
   if (H_ == 0) return;
-  hipLaunchKernelGGL(hclt_heads_rebuild_kernel, dim3(ceil_div((int64_t)Hp_ * K_, 256)), dim3(256), 0, stream, head_logp(), H_,
-                     Hp_, K_, d_head_wf_.p, d_head_wb_.p);
+  hipLaunchKernelGGL(hclt_heads_rebuild_kernel, dim3(ceil_div((int64_t)Hp_ * K_, 256), T_), dim3(256), 0, stream, head_logp(),
+                     H_, Hp_, K_, d_head_wf_.p, d_head_wb_.p);
   check_launch("rebuild_heads");
 }
 
 // head values from the root tile the forward walk has left (identity block: the root's Z)
 void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow,
                                 float rate) {
-  const float* o_root = d.O + (size_t)inner_of_var_[root_] * (d.tile_stride / 4);
-  PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), 0, stream,
-                                             o_root, d_head_wf_.p, H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix,
+  PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices, T_), dim3(kHeadWaves * 64), 0,
+                                             stream, d.O, d_root_node_.p, (int64_t)(d.tile_stride / 4), d_head_wf_.p, H_, Hp_,
+                                             d.B, d_mask, d_ll_heads, d_ll_mix,
                                              flows_follow ? head_aggr() : (float*)nullptr, rate, d_flow_shift_.p));
   check_launch("heads_forward");
 }
@@ -813,10 +941,14 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
   if (theta) {
     std::vector<float> lt((size_t)n_inner_ * K * K);
     for (int n = 0; n < n_inner_; ++n) {
-      const float* src = theta + (size_t)var_of_inner_[n] * K * K;
       float* dst = lt.data() + (size_t)n * K * K;
+      if (var_of_inner_[n] >= Vu_) {   // auxiliary node: identity
+        for (int i = 0; i < K * K; ++i) dst[i] = (i / K == i % K) ? 0.f : -INFINITY;
+        continue;
+      }
+      const float* src = theta + (size_t)var_of_inner_[n] * K * K;
       std::copy(src, src + (size_t)K * K, dst);
-      if (var_of_inner_[n] == root_) {
+      if (parent_[var_of_inner_[n]] < 0) {
         if (H_ > 0) {   // multi-head: identity block, the heads have their own rows
           for (int i = 0; i < K * K; ++i) dst[i] = (i / K == i % K) ? 0.f : -INFINITY;
         } else {
@@ -830,13 +962,29 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
   }
   general_stale_ = true;
   if (leaf) {
-    std::vector<float> t((size_t)V_ * C * K);
-    for (int v = 0; v < V_; ++v)
+    std::vector<float> t((size_t)V_ * C * K, 0.f);   // (auxiliary variables: log 1 whatever the category)
+    for (int v = 0; v < Vu_; ++v)
       for (int j = 0; j < K; ++j)
         for (int c = 0; c < C; ++c) t[((size_t)v * C + c) * K + j] = leaf[((size_t)v * K + j) * C + c];
     PCM_HIP(hipMemcpyAsync(d_leaf_.p, t.data(), t.size() * sizeof(float), hipMemcpyHostToDevice, stream));
     PCM_HIP(hipStreamSynchronize(stream));
   }
+}
+
+void HcltCircuit::set_heads(const float* heads) {
+  if (H_ == 0) fail(PCM_ERR_STATE, "a single-head circuit has no head parameters");
+  if (!heads) fail(PCM_ERR_ARG, "head parameters are null");
+  PCM_HIP(hipMemcpyAsync(head_logp(), heads, (size_t)T_ * H_ * K_ * sizeof(float), hipMemcpyHostToDevice, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
+  rebuild_heads();
+  general_stale_ = true;
+}
+
+void HcltCircuit::get_heads(float* heads) {
+  if (H_ == 0) fail(PCM_ERR_STATE, "a single-head circuit has no head parameters");
+  if (!heads) fail(PCM_ERR_ARG, "head parameters are null");
+  PCM_HIP(hipMemcpyAsync(heads, head_logp(), (size_t)T_ * H_ * K_ * sizeof(float), hipMemcpyDeviceToHost, stream));
+  PCM_HIP(hipStreamSynchronize(stream));
 }
 
 static void fetch(std::vector<float>& h, const float* d, size_t n, hipStream_t s) {
@@ -850,14 +998,15 @@ void HcltCircuit::get_block_params(float* theta, float* leaf) {
   std::vector<float> h;
   if (theta) {
     fetch(h, d_logtheta_.p, d_logtheta_.n, stream);
-    std::fill(theta, theta + (size_t)V_ * K * K, 0.f);
+    std::fill(theta, theta + (size_t)Vu_ * K * K, 0.f);
     for (int n = 0; n < n_inner_; ++n)
-      std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
-                theta + (size_t)var_of_inner_[n] * K * K);
+      if (var_of_inner_[n] < Vu_)
+        std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
+                  theta + (size_t)var_of_inner_[n] * K * K);
   }
   if (leaf) {
     fetch(h, d_leaf_.p, d_leaf_.n, stream);
-    for (int v = 0; v < V_; ++v)
+    for (int v = 0; v < Vu_; ++v)
       for (int j = 0; j < K; ++j)
         for (int c = 0; c < C; ++c) leaf[((size_t)v * K + j) * C + c] = h[((size_t)v * C + c) * K + j];
   }
@@ -885,20 +1034,22 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
   }
   if (edge_aggr) {
     fetch(h, d_edge_aggr_.p, d_edge_aggr_.n, stream);
-    std::fill(edge_aggr, edge_aggr + (size_t)V_ * K * K, 0.f);
+    std::fill(edge_aggr, edge_aggr + (size_t)Vu_ * K * K, 0.f);
     for (int n = 0; n < n_inner_; ++n)
-      std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
-                edge_aggr + (size_t)var_of_inner_[n] * K * K);
+      if (var_of_inner_[n] < Vu_)
+        std::copy(h.begin() + (size_t)n * K * K, h.begin() + (size_t)(n + 1) * K * K,
+                  edge_aggr + (size_t)var_of_inner_[n] * K * K);
   }
   if (leaf_flow) {
     fetch(h, d_leaf_flow_.p, d_leaf_flow_.n, stream);
-    for (int v = 0; v < V_; ++v)
+    for (int v = 0; v < Vu_; ++v)
       for (int j = 0; j < K; ++j)
         for (int c = 0; c < C; ++c) leaf_flow[((size_t)v * K + j) * C + c] = h[((size_t)v * C + c) * K + j];
   }
 }
 
 void HcltCircuit::vectorize(float* out, int64_t n) {
+  no_forest("the parameter vector");
   if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
                          (long long)size(0));
   if (!out) fail(PCM_ERR_ARG, "parameter vector is null");
@@ -916,6 +1067,7 @@ void HcltCircuit::vectorize(float* out, int64_t n) {
 }
 
 void HcltCircuit::update_parameters(const float* in, int64_t n) {
+  no_forest("the parameter vector");
   if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
                          (long long)size(0));
   if (!in) fail(PCM_ERR_ARG, "parameter vector is null");
@@ -960,6 +1112,7 @@ void HcltCircuit::ensure_batch(int batch) {
   }
   if (lean_) d_M_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
   d_xb_.alloc((size_t)V_ * ns * kSlice);
+  if (V_ > Vu_) d_xb_.zero(stream);   // the category of an auxiliary variable is always 0
   d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
   d_xn_.zero(stream);
   cap_slices_ = ns;
@@ -1000,7 +1153,7 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   if (b.batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", b.batch);
   ensure_batch(b.batch);
   const int Bp = ceil_div(b.batch, kSlice) * kSlice;
-  pcm_stage(b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, V_, C_, d_xb_.p, stream);
+  pcm_stage(b.d_data, b.stride_ex, b.stride_var, b.d_idx, b.batch, Bp, Vu_, C_, d_xb_.p, stream);   // (auxiliary rows stay 0)
   check_launch("stage_batch");
   hipLaunchKernelGGL(hclt_pack_x_kernel, dim3(ceil_div(Bp, 1024), n_inner_), dim3(256), 0, stream, d_nodes_.p,
                      d_child_leaf_.p, d_xb_.p, n_inner_, Bp, d_xn_.p);
@@ -1021,7 +1174,7 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, d,
+      PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d,
                        d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
     });
   } else {
@@ -1044,7 +1197,7 @@ void HcltCircuit::run_backward(const HcltDev& d) {
     const size_t lean_lds = lds + kLeanFlagWords * 4;
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices), dim3(kWalkWaves * 64), lean_lds, d, d_bwd_lean_.p, bwd_stride_,
+      PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d, d_bwd_lean_.p, bwd_stride_,
                        n_bwd_steps_, lds_slots_);
     };
     PCM_DISPATCH_LEAN_K(K_, {
@@ -1156,6 +1309,7 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
 }
 
 void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
+  no_forest("soft evidence");
   if (!soft_block_ok()) return general()->loglikelihoods_soft(s, d_ll);
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   const HcltDev d = soft_stage(s);
@@ -1166,6 +1320,7 @@ void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 }
 
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
+  no_forest("soft evidence");
   if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (soft_block_ok()) {
     if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
@@ -1239,14 +1394,13 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     d_ll_heads_.ensure((size_t)b.batch);
     run_forward(d, d_ll_heads_.p);
     heads_forward(d, d_head_mask, nullptr, d_ll, true, rate);
-    const size_t root_tile = (size_t)inner_of_var_[root_] * (d.tile_stride / 4);
     const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_ + (size_t)kHeadWaves * 16) * sizeof(float);
-    d_part_.ensure((size_t)d.nslices * H_ * K_);
-    PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices), dim3(kHeadWaves * 64), lds,
-                                               stream, d.O + root_tile, d_head_wf_.p, d_head_wb_.p, head_logp(), H_, Hp_,
-                                               d.B, d_head_mask, d.R + root_tile, d_part_.p, d_flow_shift_.p));
-    hipLaunchKernelGGL(sum_parts_kernel<true>, dim3(ceil_div((int64_t)H_ * K_, 64)), dim3(256), 0, stream, d_part_.p, d.nslices,
-                       (int64_t)H_ * K_, head_logp(), head_aggr());
+    d_part_.ensure((size_t)T_ * d.nslices * H_ * K_);
+    PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_backward_kernel<KK>, dim3(d.nslices, T_), dim3(kHeadWaves * 64), lds,
+                                               stream, d.O, d.R, d_root_node_.p, (int64_t)(d.tile_stride / 4), d_head_wf_.p,
+                                               d_head_wb_.p, H_, Hp_, d.B, d_head_mask, d_part_.p, d_flow_shift_.p));
+    hipLaunchKernelGGL(sum_parts_kernel<true>, dim3(ceil_div((int64_t)H_ * K_, 64), T_), dim3(256), 0, stream, d_part_.p,
+                       d.nslices, (int64_t)H_ * K_, head_logp(), head_aggr());
     check_launch("heads_backward");
     run_backward(d);
     run_stats(d, rate);
@@ -1379,7 +1533,7 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
   {
     const int threads = 1024, cats = ceil_div(C_, threads / 32);
     auto launch = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, dim3(V_, ceil_div(K_, 32)), dim3(threads), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
+      hipLaunchKernelGGL(kernel, dim3(Vu_, ceil_div(K_, 32)), dim3(threads), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
                          pseudocount, inertia);
     };
     if (cats <= 8) launch(&hclt_leaf_update_kernel<8>);
@@ -1395,8 +1549,8 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
   });
   check_launch("theta_update");
   if (H_ > 0) {
-    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4)), dim3(256), 0, stream, head_logp(), head_aggr(), H_, Hp_,
-                       K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
+    hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4), T_), dim3(256), 0, stream, head_logp(), head_aggr(), H_,
+                       Hp_, K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
   }
   general_stale_ = true;
 }

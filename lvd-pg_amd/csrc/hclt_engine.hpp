@@ -130,8 +130,10 @@ struct HcltDev {
 
 class HcltCircuit : public pcm_circuit {
  public:
-  // num_heads > 0: a multi-head circuit, num_heads sum nodes over the root's K products instead of one
-  HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads = 0);
+  // num_heads > 0: a multi-head circuit, num_heads sum nodes over the root's K products instead of one.
+  // forest: `parent` may hold several roots; every tree is a multi-head circuit of its own over the same batch
+  // (num_heads heads each), and the handle runs flows and EM for all of them with one launch per kernel.
+  HcltCircuit(const int32_t* parent, int V, int K, int C, int num_heads = 0, bool forest = false);
   ~HcltCircuit() override;
 
   int64_t size(int what) const override;
@@ -176,6 +178,10 @@ class HcltCircuit : public pcm_circuit {
 
   bool sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out);
   void set_block_params(const float* theta, const float* leaf);
+  // head log-parameters [trees][H][K] (host); a tree's heads are in the order of its head mask rows
+  void set_heads(const float* heads);
+  void get_heads(float* heads);
+  int num_trees() const { return T_; }
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 
@@ -192,11 +198,23 @@ class HcltCircuit : public pcm_circuit {
 
  private:
   int V_, K_, C_, n_inner_, root_;
+  int Vu_ = 0;                     // the caller's variables; V_ - Vu_ auxiliary ones behind them (forests only)
+  void split_wide_nodes();
+  bool forest_ = false;
+  int T_ = 1;                      // trees (1 unless a forest)
+  int n_groups_ = 1;               // groups of trees the walk kernels take side by side (blockIdx.y)
+  std::vector<int32_t> roots_;     // root variable of every tree, in variable order
+  std::vector<int32_t> tree_of_inner_;   // tree of every inner node
+  DevBuf<int32_t> d_root_node_;    // ... their nodes
+  // what only a single circuit defines (parameter vector order, the general form and the queries on it)
+  void no_forest(const char* what) const {
+    if (forest_) fail(PCM_ERR_UNSUPPORTED, "%s is not defined for a forest handle: use one handle per tree", what);
+  }
   int H_ = 0, Hp_ = 0;             // heads, and heads rounded up to whole operand tiles
   DevBuf<float> d_head_wf_, d_head_wb_;   // head block [Hp][K] in the two operand layouts
   DevBuf<int> d_flow_shift_;              // ceil(log2) of the largest flow one example carried in the last flow pass
   DevBuf<float> d_ll_heads_;       // scratch: the walk's own root output, per-head values
-  float* head_logp() { return d_logtheta_.p + (size_t)n_inner_ * K_ * K_; }   // [H][K], behind the blocks
+  float* head_logp() { return d_logtheta_.p + (size_t)n_inner_ * K_ * K_; }   // [trees][H][K], behind the blocks
   float* head_aggr() { return d_edge_aggr_.p + (size_t)n_inner_ * K_ * K_; }
   void rebuild_heads();
   void heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow = false,

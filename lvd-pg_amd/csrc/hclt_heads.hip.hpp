@@ -17,6 +17,10 @@
 // Head blocks are [Hp][K] (Hp = H rounded up to 16, padding rows zero) in the two MFMA
 // A-operand layouts: hwf: rows = heads, contraction over states; hwb: rows = states,
 // contraction over heads.
+//
+// A forest (several trees over one batch, H heads each) runs the same kernels with the tree in
+// blockIdx.y: every per-tree array is [tree][...], the root tiles are found through `root_node`
+// (each tree's root node, whose tiles start `tile_floats` floats per node into the value / ratio arrays).
 #pragma once
 
 #include "hclt_kernels.hip.hpp"
@@ -37,6 +41,9 @@ __global__ void hclt_heads_rebuild_kernel(const float* __restrict__ head_logp, i
                                           float* __restrict__ hwb) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= Hp * K) return;
+  head_logp += (size_t)blockIdx.y * H * K;
+  hwf += (size_t)blockIdx.y * Hp * K;
+  hwb += (size_t)blockIdx.y * Hp * K;
   const int h = i / K, j = i % K;
   const float w = h < H ? __expf(head_logp[(size_t)h * K + j]) : 0.f;
   hwf[head_wf_at(h, j, K)] = w;
@@ -71,7 +78,9 @@ __device__ __forceinline__ v4f heads_contract_f(const float* __restrict__ hwf, i
 // Per-head log-likelihoods [H][B] and/or the mask-weighted mixture
 //   logsumexp_h(ll_h + log mask_h) - log sum_h mask_h   (src-jl/multi_head_pc/likelihood.jl:3-12).
 template <int K>
-__global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(const float* __restrict__ O_root,
+__global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(const float* __restrict__ O,
+                                                                             const int32_t* __restrict__ root_node,
+                                                                             int64_t tile_floats,
                                                                              const float* __restrict__ hwf, int H, int Hp,
                                                                              int B, const float* __restrict__ mask,
                                                                              float* __restrict__ ll_heads,
@@ -79,7 +88,13 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
                                                                              float* __restrict__ head_aggr, float rate,
                                                                              int* __restrict__ flow_shift) {
   __shared__ float pm[kHeadWaves * 4][16], ps[kHeadWaves * 4][16], pt[kHeadWaves * 4][16];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x, tree = blockIdx.y;
+  const float* __restrict__ O_root = O + (size_t)root_node[tree] * tile_floats;
+  hwf += (size_t)tree * Hp * K;
+  if (mask) mask += (size_t)tree * H * B;
+  if (ll_heads) ll_heads += (size_t)tree * H * B;
+  if (ll_mix) ll_mix += (size_t)tree * B;
+  if (head_aggr) head_aggr += (size_t)tree * H * K;
   if (head_aggr) {   // ahead of a flow pass: previous head statistics times the flow memory rate, flow bound cleared
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < H * K; i += gridDim.x * blockDim.x)
       head_aggr[i] = rate != 0.f ? head_aggr[i] * rate : 0.f;
@@ -122,15 +137,20 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
 // Head flows (src-jl/multi_head_pc/flow.jl:141-176: head h of example b starts with flow mask[h][b]).
 template <int K>
 __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
-    const float* __restrict__ O_root, const float* __restrict__ hwf, const float* __restrict__ hwb,
-    const float* __restrict__ head_logp, int H, int Hp, int B, const float* __restrict__ mask, float* __restrict__ R_root,
+    const float* __restrict__ O, float* __restrict__ R, const int32_t* __restrict__ root_node, int64_t tile_floats,
+    const float* __restrict__ hwf, const float* __restrict__ hwb, int H, int Hp, int B, const float* __restrict__ mask,
     float* __restrict__ head_part, int* __restrict__ flow_shift) {
   extern __shared__ float lds[];   // R [16][Hp] | E [16][K] | partial T tiles [waves][16*K] | mask totals [waves][16]
   float* Rl = lds;
   float* El = Rl + 16 * Hp;
   float* Tl = El + 16 * K;
   float* Fl = Tl + kHeadWaves * 16 * K;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x, tree = blockIdx.y;
+  const float* __restrict__ O_root = O + (size_t)root_node[tree] * tile_floats;
+  float* __restrict__ R_root = R + (size_t)root_node[tree] * tile_floats;
+  hwf += (size_t)tree * Hp * K;
+  hwb += (size_t)tree * Hp * K;
+  mask += (size_t)tree * H * B;
   const int b = lane & 15, g = lane >> 4, col = slice * kSlice + b;
   Tile<K> e;
   heads_load_e<K>(O_root, slice, lane, e);
@@ -189,7 +209,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
   }
   // head statistics of this slice, without the head weight: row `slice` of head_part [slices][H * K], which
   // sum_parts_kernel adds up in slice order and weights
-  float* part = head_part + (size_t)slice * H * K;
+  float* part = head_part + ((size_t)tree * gridDim.x + slice) * H * K;
   for (int o = threadIdx.x; o < H * K; o += blockDim.x) {
     const int h = o / K, j = o % K;
     float a = 0.f;
@@ -199,7 +219,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
   }
 }
 
-// add_pseudocount / aggr_node_flows / update_params for the head sum nodes (one wave per head);
+// add_pseudocount / aggr_node_flows / update_params for the head sum nodes (one wave per head; blockIdx.y: tree);
 // also refreshes the two operand layouts (their padding rows stay zero)
 __global__ __launch_bounds__(256) void hclt_heads_update_kernel(float* __restrict__ head_logp, float* __restrict__ head_aggr,
                                                                 int H, int Hp, int K, float pseudocount, float inertia,
@@ -207,6 +227,10 @@ __global__ __launch_bounds__(256) void hclt_heads_update_kernel(float* __restric
   const int lane = threadIdx.x & 63;
   const int h = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (h >= H) return;
+  head_logp += (size_t)blockIdx.y * H * K;
+  head_aggr += (size_t)blockIdx.y * H * K;
+  hwf += (size_t)blockIdx.y * Hp * K;
+  hwb += (size_t)blockIdx.y * Hp * K;
   float* a = head_aggr + (size_t)h * K;
   float* lt = head_logp + (size_t)h * K;
   const float share = pseudocount / (float)K;

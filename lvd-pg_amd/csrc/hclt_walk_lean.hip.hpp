@@ -154,6 +154,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
       make_rsrc(d.M + (size_t)slice * kSlice, (uint32_t)(d.n_inner + 1) * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
   const uint32_t vm = lane < 16 ? vx : 0x7ffffff0u;
 
+  fields += (size_t)blockIdx.y * (kLeanFields * kWalkWaves) * stride;   // a forest's groups of trees: a schedule each
   LeanChunk sc;
   lean_refill(fields, stride, wave, lane, 0, sc);
   Tile<K> P0, P1, P2, P3;
@@ -299,6 +300,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
   };
   auto is_inner = [](int c) { return c >= 0 && !(c & 1); };
 
+  fields += (size_t)blockIdx.y * (kLeanFields * kWalkWaves) * stride;   // a forest's groups of trees: a schedule each
   LeanChunk sc;
   lean_refill(fields, stride, wave, lane, 0, sc);
   Tile<K> P0, C1, C2, C3;

@@ -1015,6 +1015,7 @@ int64_t SparseCircuit::size(int what) const {
     case 12: return fc_.num_heads;
     case 13: return (int64_t)fc_.desc_node.size();
     case 14: return 0;
+    case 15: return 1;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }

@@ -5,12 +5,13 @@ the host side is Python; names, argument meaning and error behaviour follow the 
 functions cited in each docstring (paths relative to VariationalJuice.jl/).  Device
 memory and streams come from torch; everything numeric happens in the HIP library.
 """
-from .circuits import (BitsCircuit, HcltCircuit, hclt_from_clt, multihead_hclt_from_clt, compile_circuit,  # noqa: F401
+from .circuits import (BitsCircuit, HcltCircuit, HcltForest, hclt_from_clt, multihead_hclt_from_clt,  # noqa: F401
+                       hclt_forest_from_clts, compile_circuit,
                        compile_multihead, CuBitsProbCircuit, CuMultiHeadBitsProbCircuit, node_maps, write_back_parameters)
 from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample, gumbel_sample_rows, gumbel_sample_backward_rows,
-                      patch_level_evidence, flow_gradients, adam, soft_reg_evidence)
+                      patch_level_evidence, flow_gradients, adam, soft_reg_evidence, forest_loglikelihoods, forest_flows)
 from .structures import (pairwise_MI, chow_liu_tree, learn_chow_liu_tree, hclt, clt_edges2parent, hclt_pc,  # noqa: F401
                          customized_hclt, joined_hclt, joined_hclt_from_clts, group_vars_by_grid, group_vars_by_cgrid)
 from .transformations import prune_pc, grow_heads_by_flows, aggregate_edge_flows, aggregate_node_flows  # noqa: F401

@@ -7,7 +7,7 @@ from ._lib import lib, check, np_ptr, H, c_i64
 
 _SIZE = dict(parameters=0, sum_parameters=1, nodes=2, edges=3, input_parameters=4, variables=5,
              categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11, heads=12,
-             description_nodes=13, walk_kernels=14)
+             description_nodes=13, walk_kernels=14, trees=15)
 _TABLE = dict(edge2param=(0, "edges"), param2edge=(1, "sum_parameters"), param2group=(2, "sum_parameters"),
               pargroup_sizes=(3, "groups"), innode2ncumparam=(4, "input_nodes"), layer_ends=(5, "layers"),
               edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"), heads=(9, "heads"),
@@ -129,6 +129,58 @@ class HcltCircuit(BitsCircuit):
         ms = np.zeros(4, np.float32)
         check(lib.pcm_get_timing(self.handle, np_ptr(ms), 4))
         return dict(forward=float(ms[0]), backward=float(ms[1]), statistics=float(ms[2]))
+
+
+class HcltForest(HcltCircuit):
+    """Many multi-head HCLTs over the same batch behind one handle (`pcm_hclt_create_forest`): the patch circuits
+    of exps/progressive_growing/parallel_PG.jl:214-225, trained together instead of one
+    `mini_batch_em_for_multihead_pc` call each.  Tree t is the t-th root of `clt_parent` in variable order."""
+
+    @property
+    def num_trees(self):
+        return self.size("trees")
+
+    def tree_of_var(self):
+        """[num_vars] index of the tree every variable belongs to."""
+        par = self.clt_parent
+        roots = np.flatnonzero(par < 0)
+        tree = np.full(len(par), -1, np.int64)
+        tree[roots] = np.arange(len(roots))
+        pending = np.flatnonzero(tree < 0)
+        while len(pending):
+            tree[pending] = tree[par[pending]]
+            pending = pending[tree[pending] < 0]
+        return tree
+
+
+def _set_heads(self, heads):
+    """Head log-parameters [num_trees, num_heads, K] ([num_heads, K] for a single multi-head circuit)."""
+    h = np.ascontiguousarray(heads, dtype=np.float32)
+    assert h.size == self.size("trees") * self.num_heads * self.num_hidden_cats, h.shape
+    check(lib.pcm_hclt_set_heads(self.handle, np_ptr(h)))
+
+
+def _get_heads(self):
+    T = self.size("trees")
+    h = np.empty((T, self.num_heads, self.num_hidden_cats), np.float32)
+    check(lib.pcm_hclt_get_heads(self.handle, np_ptr(h)))
+    return h if isinstance(self, HcltForest) else h[0]
+
+
+HcltCircuit.set_heads = _set_heads
+HcltCircuit.get_heads = _get_heads
+
+
+def hclt_forest_from_clts(clt_parent, num_cats, num_hidden_cats, num_heads):
+    """A forest handle: `clt_parent` over all variables of the batch, one -1 entry per tree; every tree becomes a
+    multi-head HCLT with `num_heads` heads (see HcltForest)."""
+    par = np.ascontiguousarray(clt_parent, dtype=np.int32)
+    h = H()
+    check(lib.pcm_hclt_create_forest(np_ptr(par), len(par), int(num_hidden_cats), int(num_cats), int(num_heads),
+                                     ctypes.byref(h)))
+    c = HcltForest(h, par, int(num_cats), int(num_hidden_cats))
+    c.num_heads = int(num_heads)
+    return c
 
 
 def multihead_hclt_from_clt(clt_parent, num_cats, num_hidden_cats, num_heads):

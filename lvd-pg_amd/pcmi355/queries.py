@@ -109,6 +109,34 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
     return ll
 
 
+def forest_loglikelihoods(forest, data, example_ids=None):
+    """Per-head log-likelihoods of every tree of a forest handle for one batch, [trees, heads, examples]: what
+    `loglikelihoods(mhbpc, data)` (src-jl/multi_head_pc/likelihood.jl:37-71) gives per patch circuit, transposed."""
+    _check_data(forest, data)
+    ids = _ids(example_ids, data.device)
+    b = data.shape[0] if ids is None else len(ids)
+    out = torch.empty((forest.size("trees"), forest.num_heads, b), dtype=torch.float32, device=data.device)
+    if b:
+        _forward(forest, data, data.data_ptr(), _dev_ptr(ids), b, out.data_ptr())
+    return out
+
+
+def forest_flows(forest, data, head_mask, example_ids=None, rate=0.0):
+    """`probs_flows_circuit` of every tree of a forest handle for one batch.  head_mask: [trees, heads, examples of
+    the batch] (src-jl/multi_head_pc/flow.jl:141-176 per tree); returns the mask-weighted log-likelihoods
+    [trees, examples]."""
+    _check_data(forest, data)
+    ids = _ids(example_ids, data.device)
+    b = data.shape[0] if ids is None else len(ids)
+    T, Hn = forest.size("trees"), forest.num_heads
+    hm = head_mask.to(device=data.device, dtype=torch.float32).contiguous()
+    if tuple(hm.shape) != (T, Hn, b):
+        raise ValueError(f"head_mask is {tuple(hm.shape)}, the forest needs {(T, Hn, b)}")
+    ll = torch.empty((T, b), dtype=torch.float32, device=data.device)
+    _flows(forest, data, _dev_ptr(ids), b, rate, hm.data_ptr(), ll.data_ptr())
+    return ll
+
+
 def soft_reg_evidence(rows, num_cats, soft_reg, soft_reg_width):
     """The categorical batch `rows` [B, V] (uint8) as the log-evidence [B, V, C] under which a leaf's value is
     the reference's `soft_loglikelihood` (src/regularization/reg_likelihood.jl:4-14):

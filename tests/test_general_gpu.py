@@ -441,3 +441,79 @@ def test_statistics_are_the_same_bits_on_every_run(gpu, oracle):
             for a, b in zip(first, again):
                 assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert all(np.isfinite(a).all() for a in first) and first[0].sum() > 0 and first[1].sum() > 0
+
+
+def test_forest_of_patch_circuits_at_their_real_shape(gpu, oracle):
+    """Sixteen patch circuits of the patch-clustered configuration (8 x 8 x 3 patches of 64 x 64 x 3 images: 192
+    variables, K = 32, 256 categories, 128 heads, batch 1024) as one forest handle over the image's pixels, against a
+    handle per patch (the path the test above pins to the layered engine and the oracle): per-head values, mixtures,
+    flows and the EM update under a one-hot and a soft head mask.  Some of the sixteen Chow-Liu trees have nodes with
+    four children, which the forest splits; two groups of trees walk side by side."""
+    torch, P = gpu
+    from pcmi355 import workloads
+    from pcmi355._lib import lib, check
+    from helpers import rel_err
+    V, K, C, H, B, NP = 192, 32, 256, 128, 1024, 16
+    rng = np.random.default_rng(1004)
+    img = workloads.grf_images(B, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(B, 3, 64, 64)
+    flat = np.ascontiguousarray(img.reshape(B, -1))
+    pixel = np.arange(3 * 64 * 64).reshape(3, 64, 64)
+    pvars = [pixel[:, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8].reshape(V) for p in range(NP)]
+    used = np.sort(np.concatenate(pvars))                       # the forest's variables: the pixels of these patches
+    col = np.full(flat.shape[1], -1, np.int64)
+    col[used] = np.arange(len(used))
+    parents = [workloads.chow_liu_parent(np.ascontiguousarray(flat[:, pv])) for pv in pvars]
+    assert max(np.bincount(par[par >= 0]).max() for par in parents) > 3
+    fparent = np.empty(len(used), np.int32)
+    theta = np.empty((len(used), K, K), np.float32)
+    leaf = np.empty((len(used), K, C), np.float32)
+    heads = np.log(rng.dirichlet(np.ones(K), size=(NP, H))).astype(np.float32)
+    singles = []
+    for p, (pv, par) in enumerate(zip(pvars, parents)):
+        th, lf = workloads.init_params(par, K, C, 2000 + p, kind="dirichlet")
+        fparent[col[pv]] = np.where(par < 0, -1, col[pv][np.maximum(par, 0)])
+        theta[col[pv]], leaf[col[pv]] = th, lf
+        c = P.multihead_hclt_from_clt(par, C, K, H)
+        c.set_params(th, lf)
+        singles.append((c, torch.from_numpy(np.ascontiguousarray(flat[:, pv])).cuda()))
+    order = np.argsort([col[pv][np.flatnonzero(par < 0)[0]] for pv, par in zip(pvars, parents)])   # tree t = patch order[t]
+    forest = P.hclt_forest_from_clts(fparent, C, K, H)
+    assert forest.num_trees == NP and forest.size("walk_kernels") == 1 and forest.size("variables") == len(used)
+    forest.set_params(theta, leaf)
+    forest.set_heads(heads[order])
+    for p, (c, _) in enumerate(singles):
+        c.set_heads(heads[p])
+    d = torch.from_numpy(np.ascontiguousarray(flat[:, used])).cuda()
+    ll_f = P.forest_loglikelihoods(forest, d).cpu().numpy()
+    for t, p in enumerate(order):
+        c, dp = singles[p]
+        assert rel_err(ll_f[t].T, P.loglikelihoods(c, dp).cpu().numpy()).max() < 1e-5, f"patch {p}"
+    cluster = rng.integers(0, H, size=(NP, B))
+    for soft in (False, True):
+        mask = np.zeros((NP, H, B), np.float32)
+        for p in range(NP):
+            mask[p, cluster[p], np.arange(B)] = 1.0
+        if soft:
+            mask = (mask + rng.random(mask.shape).astype(np.float32) * (rng.random(mask.shape) < 0.1)).astype(np.float32)
+        mix_f = P.forest_flows(forest, d, torch.from_numpy(mask[order]).cuda()).cpu().numpy()
+        ea_f, lf_f = forest.get_flows()
+        check(lib.pcm_em_update(forest.handle, 0.1, 0.9))
+        th_f, leaf_f = forest.get_params()
+        heads_f = forest.get_heads()
+        worst = 0.0
+        for t, p in enumerate(order):
+            c, dp = singles[p]
+            mix = P.probs_flows_circuit(c, dp, head_mask=torch.from_numpy(mask[p].T.copy()).cuda()).cpu().numpy()
+            assert rel_err(mix_f[t], mix).max() < 1e-5, f"patch {p} mixture"
+            ea, lf = c.get_flows()
+            gv = col[pvars[p]]
+            assert np.abs(ea_f[gv] - ea).max() < FLOW_RTOL * ea.max() and np.abs(lf_f[gv] - lf).max() < FLOW_RTOL * lf.max()
+            check(lib.pcm_em_update(c.handle, 0.1, 0.9))
+            th, lp = c.get_params()
+            inner = np.flatnonzero(np.bincount(parents[p][parents[p] >= 0], minlength=V) > 0)
+            inner = inner[parents[p][inner] >= 0]                # (the root's block is the identity in both)
+            for a, b in ((th_f[gv][inner], th[inner]), (leaf_f[gv], lp), (heads_f[t], c.get_heads())):
+                worst = max(worst, float((np.abs(np.exp(a.astype(np.float64)) - np.exp(b.astype(np.float64)))
+                                          / np.maximum(np.exp(b.astype(np.float64)), 1e-6)).max()))
+        print(f"forest vs one handle per patch, {'soft' if soft else 'one-hot'} mask: parameters differ by {worst:.2e}")
+        assert worst < 2e-4

@@ -417,3 +417,104 @@ def test_random_shapes_block_engine_against_layered_engine(gpu, oracle, seed):
         P.mini_batch_em(c, data, 1, batch_size=B, pseudocount=0.1, param_inertia=0.3)
     pa, pg = np.exp(P.vectorize_parameters(a)), np.exp(P.vectorize_parameters(g))
     assert np.max(np.abs(pa - pg) / np.maximum(pg, 1e-6)) < 2e-4
+
+
+def _forest_case(P, O, rng, T, Vt, K, C, H, max_children=3):
+    """T random trees over interleaved variables of one batch."""
+    from helpers import block_theta
+    V = sum(Vt)
+    owner = rng.permutation(np.repeat(np.arange(T), Vt))           # tree of every global variable
+    gvars = [np.flatnonzero(owner == t) for t in range(T)]          # a tree's variables keep their relative order: the
+    # children of a node are added up in variable order, so only then are the sums the same bits
+    parent = np.full(V, -2, np.int32)
+    trees = []
+    for t in range(T):
+        par_t = O.random_tree(Vt[t], rng, max_children)
+        theta_t = np.log(rng.dirichlet(np.ones(K), size=(Vt[t], K))).astype(np.float32)
+        leaf_t = np.log(rng.dirichlet(np.ones(C), size=(Vt[t], K))).astype(np.float32)
+        heads_t = np.log(rng.dirichlet(np.ones(K), size=H)).astype(np.float32)
+        trees.append((par_t, theta_t, leaf_t, heads_t))
+        for v in range(Vt[t]):
+            parent[gvars[t][v]] = -1 if par_t[v] < 0 else gvars[t][par_t[v]]
+    # trees are numbered by their root's variable index
+    order = np.argsort([gvars[t][np.flatnonzero(trees[t][0] < 0)[0]] for t in range(T)])
+    return V, parent, [gvars[t] for t in order], [trees[t] for t in order]
+
+
+@pytest.mark.parametrize("T,Vt,K,C,H,B,wide", [(3, [5, 9, 2], 16, 6, 4, 40, 3), (5, [12, 7, 20, 3, 9], 32, 256, 128, 100, 3),
+                                               (16, [24] * 16, 32, 17, 40, 256, 3), (6, [30, 9, 14, 40, 8, 21], 32, 9, 7, 90, 7),
+                                               (2, [8, 7], 16, 5, 3, 33, 6)])
+def test_forest_handle_gives_the_bits_of_one_handle_per_tree(gpu, oracle, T, Vt, K, C, H, B, wide):
+    """pcm_hclt_create_forest: per tree, likelihoods, flows and the EM update are those of a multi-head handle over
+    that tree's variables (parallel_PG.jl:214-225 runs one such circuit per patch).  With at most three children per
+    tree node both run the same kernels and agree to the bit; nodes with more children are split inside a forest
+    (auxiliary identity nodes) and walked by the general kernels in a handle of their own: same circuit, rounding apart."""
+    torch, P = gpu
+    from pcmi355._lib import lib, check
+    rng = np.random.default_rng(T * 1000 + K)
+    V, parent, gvars, trees = _forest_case(P, oracle, rng, T, Vt, K, C, H, max_children=wide)
+    if wide > 3:
+        assert max(np.bincount(t[0][t[0] >= 0]).max() for t in trees) > 3
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+    forest = P.hclt_forest_from_clts(parent, C, K, H)
+    assert forest.num_trees == T and forest.size("walk_kernels") == 1
+    theta = np.zeros((V, K, K), np.float32)
+    leaf = np.zeros((V, K, C), np.float32)
+    for gv, (par_t, theta_t, leaf_t, _) in zip(gvars, trees):
+        theta[gv], leaf[gv] = theta_t, leaf_t
+    forest.set_params(theta, leaf)
+    forest.set_heads(np.stack([t[3] for t in trees]))
+    np.testing.assert_array_equal(forest.get_heads(), np.stack([t[3] for t in trees]))
+    singles = []
+    for gv, (par_t, theta_t, leaf_t, heads_t) in zip(gvars, trees):
+        c = P.multihead_hclt_from_clt(par_t, C, K, H)
+        c.set_params(theta_t, leaf_t)
+        c.set_heads(heads_t)
+        singles.append((c, torch.from_numpy(np.ascontiguousarray(data[:, gv])).cuda()))
+    ll_f = P.forest_loglikelihoods(forest, d).cpu().numpy()
+    for t, (c, dt) in enumerate(singles):
+        if wide <= 3:
+            np.testing.assert_array_equal(ll_f[t].T, P.loglikelihoods(c, dt).cpu().numpy(), err_msg=f"tree {t}")
+        else:
+            np.testing.assert_allclose(ll_f[t].T, P.loglikelihoods(c, dt).cpu().numpy(), rtol=2e-6, err_msg=f"tree {t}")
+    for soft in (False, True):
+        mask = np.zeros((T, H, B), np.float32)
+        for t in range(T):
+            mask[t, rng.integers(0, H, B), np.arange(B)] = 1.0
+        if soft:   # the trees share one bound on an example's total mask, so their fixed-point grids may differ
+            mask = (mask + rng.random((T, H, B)).astype(np.float32) * (rng.random((T, H, B)) < 0.3)).astype(np.float32)
+        rate = 0.25 if soft else 0.0
+        mix_f = P.forest_flows(forest, d, torch.from_numpy(mask).cuda(), rate=rate).cpu().numpy()
+        ea_f, lf_f = forest.get_flows()
+        check(lib.pcm_em_update(forest.handle, 0.1, 0.7))
+        th_f, leaf_f = forest.get_params()
+        heads_f = forest.get_heads()
+        for t, (c, dt) in enumerate(singles):
+            mix = P.probs_flows_circuit(c, dt, head_mask=torch.from_numpy(mask[t].T.copy()).cuda(), rate=rate).cpu().numpy()
+            ea, lf = c.get_flows()
+            check(lib.pcm_em_update(c.handle, 0.1, 0.7))
+            th, lp = c.get_params()
+            exact = not soft and wide <= 3
+            cmp = np.testing.assert_array_equal if exact else (
+                lambda a, b, err_msg="": np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-6 * max(1.0, float(np.abs(b).max())), err_msg=err_msg))
+            cmp(mix_f[t], mix, err_msg=f"tree {t} mixture")
+            cmp(ea_f[gvars[t]], ea, err_msg=f"tree {t} edge flows")
+            cmp(lf_f[gvars[t]], lf, err_msg=f"tree {t} leaf flows")
+            cmp(th_f[gvars[t]], th, err_msg=f"tree {t} sum parameters")
+            cmp(leaf_f[gvars[t]], lp, err_msg=f"tree {t} leaf parameters")
+            cmp(heads_f[t], c.get_heads(), err_msg=f"tree {t} heads")
+
+
+def test_forest_handle_refuses_what_only_one_circuit_defines(gpu, oracle):
+    torch, P = gpu
+    parent = np.array([-1, 0, 0, -1, 3], np.int32)
+    forest = P.hclt_forest_from_clts(parent, 4, 16, 2)
+    with pytest.raises(P.PcmError, match="forest"):
+        P.vectorize_parameters(forest)
+    with pytest.raises(P.PcmError, match="forest"):
+        forest.table("edge2param")
+    with pytest.raises(P.PcmError, match="tree of its own"):
+        P.hclt_forest_from_clts(np.array([-1, 0, -1], np.int32), 4, 16, 2)
+    with pytest.raises(P.PcmError, match="more than one root"):
+        P.multihead_hclt_from_clt(parent, 4, 16, 2)
