@@ -75,7 +75,7 @@ int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32
  * order: a node's children are added up in variable order) would:
  *   pcm_loglikelihoods  d_ll_out [num_trees][num_heads][batch]
  *   pcm_flows           d_head_mask [num_trees][num_heads][batch], d_ll_out [num_trees][batch]
- *   pcm_em_update, pcm_em_step (mask as pcm_flows), pcm_set_stream, pcm_set_timing
+ *   pcm_em_update, pcm_set_stream, pcm_set_timing  (pcm_em_step has no head mask: not for multi-head circuits)
  *   pcm_hclt_set_params / get_params / get_flows  (per-variable blocks: rows of trees stay apart)
  *   pcm_hclt_set_heads / get_heads, pcm_size
  * Everything a single circuit defines beyond that (parameter vector and index tables, KL, sampling, soft

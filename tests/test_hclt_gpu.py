@@ -506,6 +506,54 @@ def test_forest_handle_gives_the_bits_of_one_handle_per_tree(gpu, oracle, T, Vt,
             cmp(heads_f[t], c.get_heads(), err_msg=f"tree {t} heads")
 
 
+def test_forest_handle_with_example_ids_and_flow_memory(gpu, oracle):
+    """Flows and EM update of a forest with example ids and flow memory, two batches in a row, against one handle per
+    tree."""
+    torch, P = gpu
+    from pcmi355._lib import lib, check
+    T, Vt, K, C, H, N = 9, [11, 6, 14, 9, 5, 17, 8, 12, 7], 16, 12, 5, 150
+    rng = np.random.default_rng(77)
+    V, parent, gvars, trees = _forest_case(P, oracle, rng, T, Vt, K, C, H)
+    data = rng.integers(0, C, size=(N, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+    forest = P.hclt_forest_from_clts(parent, C, K, H)
+    theta = np.zeros((V, K, K), np.float32)
+    leaf = np.zeros((V, K, C), np.float32)
+    for gv, (par_t, theta_t, leaf_t, _) in zip(gvars, trees):
+        theta[gv], leaf[gv] = theta_t, leaf_t
+    forest.set_params(theta, leaf)
+    forest.set_heads(np.stack([t[3] for t in trees]))
+    singles = []
+    for gv, (par_t, theta_t, leaf_t, heads_t) in zip(gvars, trees):
+        c = P.multihead_hclt_from_clt(par_t, C, K, H)
+        c.set_params(theta_t, leaf_t)
+        c.set_heads(heads_t)
+        singles.append((c, torch.from_numpy(np.ascontiguousarray(data[:, gv])).cuda()))
+    for it, (B, rate) in enumerate([(70, 0.0), (45, 0.6)]):
+        ids = torch.from_numpy(rng.choice(N, size=B, replace=False).astype(np.int32)).cuda()
+        mask = np.zeros((T, H, B), np.float32)
+        for t in range(T):
+            mask[t, rng.integers(0, H, B), np.arange(B)] = 1.0
+        hm = torch.from_numpy(mask).cuda()
+        ll = torch.empty((T, B), device="cuda")
+        check(lib.pcm_flows(forest.handle, d.data_ptr(), d.stride(0), d.stride(1), ids.data_ptr(), B, rate, hm.data_ptr(),
+                            ll.data_ptr()))
+        check(lib.pcm_em_update(forest.handle, 0.1, 0.8))
+        th_f, leaf_f = forest.get_params()
+        heads_f = forest.get_heads()
+        for t, (c, dt) in enumerate(singles):
+            hm_t = torch.from_numpy(np.ascontiguousarray(mask[t])).cuda()
+            ll_t = torch.empty(B, device="cuda")
+            check(lib.pcm_flows(c.handle, dt.data_ptr(), dt.stride(0), dt.stride(1), ids.data_ptr(), B, rate, hm_t.data_ptr(),
+                                ll_t.data_ptr()))
+            check(lib.pcm_em_update(c.handle, 0.1, 0.8))
+            th, lp = c.get_params()
+            np.testing.assert_array_equal(ll[t].cpu().numpy(), ll_t.cpu().numpy(), err_msg=f"batch {it} tree {t}")
+            np.testing.assert_array_equal(th_f[gvars[t]], th, err_msg=f"batch {it} tree {t}")
+            np.testing.assert_array_equal(leaf_f[gvars[t]], lp, err_msg=f"batch {it} tree {t}")
+            np.testing.assert_array_equal(heads_f[t], c.get_heads(), err_msg=f"batch {it} tree {t}")
+
+
 def test_forest_handle_refuses_what_only_one_circuit_defines(gpu, oracle):
     torch, P = gpu
     parent = np.array([-1, 0, 0, -1, 3], np.int32)
