@@ -11,7 +11,8 @@ from .circuits import (BitsCircuit, HcltCircuit, HcltForest, hclt_from_clt, mult
 from .queries import (loglikelihoods, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample, gumbel_sample_rows, gumbel_sample_backward_rows,
-                      patch_level_evidence, flow_gradients, adam, soft_reg_evidence, forest_loglikelihoods, forest_flows)
+                      patch_level_evidence, flow_gradients, adam, soft_reg_evidence, forest_loglikelihoods, forest_flows,
+                      mini_batch_em_for_forest)
 from .structures import (pairwise_MI, chow_liu_tree, learn_chow_liu_tree, hclt, clt_edges2parent, hclt_pc,  # noqa: F401
                          customized_hclt, joined_hclt, joined_hclt_from_clts, group_vars_by_grid, group_vars_by_cgrid)
 from .transformations import prune_pc, grow_heads_by_flows, aggregate_edge_flows, aggregate_node_flows  # noqa: F401

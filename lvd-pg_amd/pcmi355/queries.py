@@ -241,6 +241,53 @@ def mini_batch_em_for_multihead_pc(mhbpc, data, head_mask, num_epochs, **kw):
     return mini_batch_em_with_reg(mhbpc, data, num_epochs, head_mask=head_mask, **kw)
 
 
+def mini_batch_em_for_forest(forest, data, head_masks, num_epochs, *, batch_size, pseudocount, param_inertia,
+                             param_inertia_end=None, flow_memory=0.0, shuffle="each_epoch", generator=None):
+    """The loop over patch circuits of exps/progressive_growing/parallel_PG.jl:214-225 -- one
+    `mini_batch_em_for_multihead_pc` (src-jl/multi_head_pc/em.jl:1-99) per circuit -- as one loop over a forest handle:
+    every batch is one `pcm_flows` + `pcm_em_update` for all trees, with the batch order, inertia schedule and flow
+    memory of `mini_batch_em_with_reg`.  head_masks: [trees, examples, heads], a tree's slice being the `head_mask`
+    the reference passes for that circuit.  Returns the per-epoch mean log-likelihoods, [epochs, trees]."""
+    _check_data(forest, data)
+    n, T = data.shape[0], forest.size("trees")
+    if batch_size > n:
+        raise ValueError("batch_size must not exceed the number of examples")
+    hm_t = head_masks.to(device=data.device, dtype=torch.float32)
+    if tuple(hm_t.shape) != (T, n, forest.num_heads):
+        raise ValueError(f"head_masks is {tuple(hm_t.shape)}, the forest needs {(T, n, forest.num_heads)}")
+    num_batches = n // batch_size
+    if param_inertia_end is None:
+        param_inertia_end = param_inertia
+    d_inertia = (param_inertia_end - param_inertia) / num_epochs
+    perm = torch.arange(n, dtype=torch.int32, device=data.device)
+
+    def do_shuffle():
+        nonlocal perm
+        perm = torch.randperm(n, generator=generator).to(device=data.device, dtype=torch.int32)
+
+    if shuffle == "once":
+        do_shuffle()
+    lls, fresh = [], True
+    ll = torch.empty((T, batch_size), dtype=torch.float32, device=data.device)
+    for _ in range(num_epochs):
+        if shuffle == "each_epoch":
+            do_shuffle()
+        acc = torch.zeros(T, dtype=torch.float64, device=data.device)
+        for bi in range(num_batches):
+            if shuffle == "each_batch":
+                do_shuffle()
+            ids = perm[bi * batch_size:(bi + 1) * batch_size]
+            rate = 0.0 if (flow_memory == 0 or fresh) else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
+            fresh = False
+            hm = hm_t[:, ids.long()].transpose(1, 2).contiguous()   # [trees, heads, batch]
+            _flows(forest, data, ids.data_ptr(), batch_size, rate, hm.data_ptr(), ll.data_ptr())
+            check(lib.pcm_em_update(forest.handle, float(pseudocount), float(param_inertia)))
+            acc += ll.sum(dim=1, dtype=torch.float64)
+        lls.append((acc / batch_size / num_batches).cpu().numpy())
+        param_inertia += d_inertia
+    return np.stack(lls)
+
+
 def vectorize_parameters(bpc):
     """`vectorize_parameters(mbpc)` (src/misc.jl:33-40) -> host float32 vector."""
     out = np.empty(bpc.num_parameters(), np.float32)

@@ -554,6 +554,38 @@ def test_forest_handle_with_example_ids_and_flow_memory(gpu, oracle):
             np.testing.assert_array_equal(heads_f[t], c.get_heads(), err_msg=f"batch {it} tree {t}")
 
 
+def test_em_driver_of_a_forest_follows_the_driver_of_every_tree(gpu, oracle):
+    """mini_batch_em_for_forest against mini_batch_em_for_multihead_pc on a handle per tree: three epochs in the
+    given order of examples, rising inertia, flow memory."""
+    torch, P = gpu
+    T, Vt, K, C, H, N = 4, [9, 13, 6, 10], 16, 8, 6, 96
+    rng = np.random.default_rng(5)
+    V, parent, gvars, trees = _forest_case(P, oracle, rng, T, Vt, K, C, H)
+    data = rng.integers(0, C, size=(N, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+    masks = np.zeros((T, N, H), np.float32)
+    for t in range(T):
+        masks[t, np.arange(N), rng.integers(0, H, N)] = 1.0
+    forest = P.hclt_forest_from_clts(parent, C, K, H)
+    theta = np.zeros((V, K, K), np.float32)
+    leaf = np.zeros((V, K, C), np.float32)
+    for gv, (par_t, theta_t, leaf_t, _) in zip(gvars, trees):
+        theta[gv], leaf[gv] = theta_t, leaf_t
+    forest.set_params(theta, leaf)
+    forest.set_heads(np.stack([t[3] for t in trees]))
+    kw = dict(batch_size=32, pseudocount=0.1, param_inertia=0.8, param_inertia_end=0.95, flow_memory=200.0, shuffle="none")
+    lls_f = P.mini_batch_em_for_forest(forest, d, torch.from_numpy(masks), 3, **kw)
+    assert lls_f.shape == (3, T) and (lls_f[2] > lls_f[0]).all()
+    for t, (gv, (par_t, theta_t, leaf_t, heads_t)) in enumerate(zip(gvars, trees)):
+        c = P.multihead_hclt_from_clt(par_t, C, K, H)
+        c.set_params(theta_t, leaf_t)
+        c.set_heads(heads_t)
+        dt = torch.from_numpy(np.ascontiguousarray(data[:, gv])).cuda()
+        lls = P.mini_batch_em_for_multihead_pc(c, dt, torch.from_numpy(masks[t]).cuda(), 3, **kw)
+        np.testing.assert_allclose(lls_f[:, t], lls, rtol=1e-12)
+        np.testing.assert_array_equal(forest.get_heads()[t], c.get_heads())
+
+
 def test_forest_handle_refuses_what_only_one_circuit_defines(gpu, oracle):
     torch, P = gpu
     parent = np.array([-1, 0, 0, -1, 3], np.int32)
