@@ -77,13 +77,15 @@ struct DevBuf {
   }
 };
 
-// dst[i] += w(i) * (part[0][i] + part[1][i] + ...); w(i) = exp(logw[i]) or 1.  Kernels that share one sum out
+// dst[i] = keep * dst[i] + w(i) * (part[0][i] + part[1][i] + ...); w(i) = exp(logw[i]) or 1; keep < 0 stands for
+// keep = 1 (plain accumulation), keep = 0 never reads dst.  Kernels that share one sum out
 // among workgroups leave their parts in rows of `part` and this kernel puts them together: no atomics, the same
 // bits on every run.  A workgroup takes 64 elements; its four waves each add up every fourth row in order, and
 // the four subtotals are added in order too (the order is fixed, just not row after row).
 template <bool kExpWeight>
 __global__ __launch_bounds__(256) void sum_parts_kernel(const float* __restrict__ part, int n_parts, int64_t n,
-                                                        const float* __restrict__ logw, float* __restrict__ dst) {
+                                                        const float* __restrict__ logw, float* __restrict__ dst,
+                                                        float keep = -1.f) {
   __shared__ float sub[4][64];
   const int lane = threadIdx.x & 63, g = threadIdx.x >> 6;
   const int64_t i = (int64_t)blockIdx.x * 64 + lane;
@@ -98,7 +100,8 @@ __global__ __launch_bounds__(256) void sum_parts_kernel(const float* __restrict_
   __syncthreads();
   if (g == 0 && i < n) {
     s = ((sub[0][lane] + sub[1][lane]) + sub[2][lane]) + sub[3][lane];
-    dst[i] += kExpWeight ? __expf(logw[i]) * s : s;
+    const float old = keep < 0.f ? dst[i] : keep != 0.f ? keep * dst[i] : 0.f;
+    dst[i] = old + (kExpWeight ? __expf(logw[i]) * s : s);
   }
 }
 

@@ -405,73 +405,74 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
   }
 }
 
-// Edge statistics: workgroup (node n, row tile kt) contracts R^T E over all examples.
+// Edge statistics: R^T E over all examples.  Workgroup (node n, split p of the slices); its four waves share the
+// rows of the block out (K / 64 row tiles each, all columns), so every wave keeps its accumulators to itself, the
+// E tile of a slice is read from memory once per workgroup (the four waves' requests meet in L1) and serves
+// K / 16 x K / 16 matrix instructions per wave.  (With a workgroup per row tile, as before, every row tile read
+// all of E again: 0.5 GB of L2 traffic on C2, which bound the kernel at 77 us.)  The splits' shares go to rows
+// of `part` [splits][n_inner * K * K]; sum_parts_kernel adds them in order and weights them.
+constexpr int kWideEdgeSplits = 8;
 template <int K>
-__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_edge_kernel(HcltDev d, const float* __restrict__ RS,
-                                                                         const float* __restrict__ ES,
-                                                                         float* __restrict__ edge_aggr, float rate) {
-  constexpr int KT = K / 16;
-  __shared__ v4f red[kWideWaves][KT][64];
+__device__ __forceinline__ void wide_edge_block(const HcltDev& d, const float* __restrict__ RS, const float* __restrict__ ES,
+                                                float* __restrict__ part, int n, int split, int n_splits) {
+  constexpr int KT = K / 16, RT = KT / kWideWaves;
+  static_assert(RT >= 1, "a wave takes at least one row tile");
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int n = blockIdx.x, kt = blockIdx.y;
-  v4f acc[KT];
+  const int per = (d.nslices + n_splits - 1) / n_splits;
+  const int s_begin = split * per, s_end = min(s_begin + per, d.nslices);
+  v4f acc[RT][KT];
 #pragma unroll
-  for (int jt = 0; jt < KT; ++jt) acc[jt] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt) acc[rt][jt] = v4f{0.f, 0.f, 0.f, 0.f};
   const v4f* rs = reinterpret_cast<const v4f*>(RS + (size_t)n * d.nslices * kSlice * K);
   const v4f* es = reinterpret_cast<const v4f*>(ES + (size_t)n * d.nslices * kSlice * K);
-  v4f a, e[KT];
-  if (wave < d.nslices) {
-    a = rs[((size_t)wave * KT + kt) * 64 + lane];
+  v4f a[RT], e[KT];
+  auto request = [&](int s) {
 #pragma unroll
-    for (int jt = 0; jt < KT; ++jt) e[jt] = es[((size_t)wave * KT + jt) * 64 + lane];
-  }
-  for (int s = wave; s < d.nslices; s += kWideWaves) {
-    const v4f a0 = a;
-    v4f e0[KT];
+    for (int rt = 0; rt < RT; ++rt) a[rt] = rs[((size_t)s * KT + wave * RT + rt) * 64 + lane];
+#pragma unroll
+    for (int jt = 0; jt < KT; ++jt) e[jt] = es[((size_t)s * KT + jt) * 64 + lane];
+  };
+  if (s_begin < s_end) request(s_begin);
+  for (int s = s_begin; s < s_end; ++s) {
+    v4f a0[RT], e0[KT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) a0[rt] = a[rt];
 #pragma unroll
     for (int jt = 0; jt < KT; ++jt) e0[jt] = e[jt];
-    const int sn = s + kWideWaves;
-    if (sn < d.nslices) {
-      a = rs[((size_t)sn * KT + kt) * 64 + lane];
+    if (s + 1 < s_end) request(s + 1);
 #pragma unroll
-      for (int jt = 0; jt < KT; ++jt) e[jt] = es[((size_t)sn * KT + jt) * 64 + lane];
-    }
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int jt = 0; jt < KT; ++jt)
+          acc[rt][jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[rt][t], e0[jt][t], acc[rt][jt], 0, 0, 0);
+  }
+  float* out = part + ((size_t)split * d.n_inner + n) * K * K;
+  const int g = lane >> 4, j0 = lane & 15;
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
     for (int jt = 0; jt < KT; ++jt)
 #pragma unroll
-      for (int t = 0; t < 4; ++t) acc[jt] = __builtin_amdgcn_mfma_f32_16x16x4f32(a0[t], e0[jt][t], acc[jt], 0, 0, 0);
-  }
-#pragma unroll
-  for (int jt = 0; jt < KT; ++jt) red[wave][jt][lane] = acc[jt];
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < KT * 64; idx += blockDim.x) {
-    const int jt = idx >> 6, l = idx & 63;
-    v4f sum = red[0][jt][l];
-#pragma unroll
-    for (int w = 1; w < kWideWaves; ++w) sum += red[w][jt][l];
-    const int g = l >> 4, j = jt * 16 + (l & 15);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const size_t at = ((size_t)n * K + kt * 16 + 4 * g + i) * K + j;
-      const float old = rate != 0.f ? rate * edge_aggr[at] : 0.f;
-      edge_aggr[at] = old + __expf(d.logtheta[at]) * sum[i];
-    }
-  }
+      for (int i = 0; i < 4; ++i)
+        out[(size_t)((wave * RT + rt) * 16 + 4 * g + i) * K + jt * 16 + j0] = acc[rt][jt][i];
 }
 
 // Leaf histograms: workgroup (variable u, state tile kt) adds, for every example, the 16 flows
 // of the tile to row x_b of a [C][16] table in LDS, as two-limb fixed-point integers (integer
 // LDS atomics are more than ten times cheaper than floating-point ones here and make the sum
 // independent of the order of arrival); flows are in [0, 1].
-__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev d, const float* __restrict__ G,
-                                                                         const int32_t* __restrict__ state_node, int K,
-                                                                         float* __restrict__ leaf_flow, float rate,
-                                                                         int limb) {
+__device__ __forceinline__ void wide_leaf_block(const HcltDev& d, const float* __restrict__ G,
+                                                const int32_t* __restrict__ state_node, int K,
+                                                float* __restrict__ leaf_flow, float rate, int limb, int u, int kt) {
   extern __shared__ unsigned hist[];   // [2][C][17]
   constexpr int HS = 17;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int b = lane & 15, g = lane >> 4;
-  const int u = blockIdx.x, kt = blockIdx.y, KT = K / 16;
+  const int KT = K / 16;
   const int n = state_node[u];
   const int hw = d.C * HS;
   for (int i = threadIdx.x; i < 2 * hw; i += blockDim.x) hist[i] = 0u;
@@ -502,6 +503,20 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev
     const float old = rate != 0.f ? rate * leaf_flow[at] : 0.f;
     leaf_flow[at] = old + val;
   }
+}
+
+template <int K>
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_edge_kernel(HcltDev d, const float* __restrict__ RS,
+                                                                         const float* __restrict__ ES,
+                                                                         float* __restrict__ part) {
+  wide_edge_block<K>(d, RS, ES, part, blockIdx.x, blockIdx.y, gridDim.y);
+}
+
+__global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev d, const float* __restrict__ G,
+                                                                         const int32_t* __restrict__ state_node, int K,
+                                                                         float* __restrict__ leaf_flow, float rate,
+                                                                         int limb) {
+  wide_leaf_block(d, G, state_node, K, leaf_flow, rate, limb, blockIdx.x, blockIdx.y);
 }
 
 // ---- host --------------------------------------------------------------------------------
@@ -584,10 +599,17 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
                           (uint32_t)(ops_in_lds ? ops_bytes : 0), stream, t_bwd ? ev[2] : nullptr, t_bwd ? ev[3] : nullptr, 0, d,
                           d_wide_ops_.p, ops_in_lds, d_wide_extra_.p, d_G_.p, d_wide_rs_.p, d_wide_es_.p);
     check_launch_w("hclt_wide_backward");
-    // statistics: the edge kernel starts the phase, the leaf kernel (absent with soft evidence) ends it
-    hipExtLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, KK / 16), dim3(kWideWaves * 64), 0, stream,
-                          t_stat ? ev[4] : nullptr, t_stat && soft ? ev[5] : nullptr, 0, d, d_wide_rs_.p, d_wide_es_.p, d_edge_aggr_.p,
-                          rate);
+    // statistics: the edge blocks by splits of the slices, the splits' sum, and (unless the evidence is soft) the leaf
+    // histograms.  (Edge blocks and histograms as two halves of one launch ran slower than one after the other: 357
+    // against 320 us per step on C2.)
+    const int splits = std::min(kWideEdgeSplits, d.nslices);
+    const int64_t n_edge = (int64_t)n_inner_ * KK * KK;
+    d_part_.ensure((size_t)splits * n_edge);
+    hipExtLaunchKernelGGL(hclt_wide_edge_kernel<KK>, dim3(n_inner_, splits), dim3(kWideWaves * 64), 0, stream,
+                          t_stat ? ev[4] : nullptr, nullptr, 0, d, d_wide_rs_.p, d_wide_es_.p, d_part_.p);
+    hipExtLaunchKernelGGL(sum_parts_kernel<true>, dim3(ceil_div(n_edge, 64)), dim3(256), 0, stream, nullptr,
+                          t_stat && soft ? ev[5] : nullptr, 0, (const float*)d_part_.p, splits, n_edge,
+                          (const float*)d_logtheta_.p, d_edge_aggr_.p, rate);
   });
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
   if (!soft)
