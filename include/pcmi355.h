@@ -86,6 +86,20 @@ int pcm_hclt_create_multihead(const int32_t* clt_parent, int32_t num_vars, int32
 int pcm_hclt_create_forest(const int32_t* clt_parent, int32_t num_vars, int32_t num_hidden_cats, int32_t num_cats,
                            int32_t num_heads, pcm_circuit** out);
 
+/*
+ * Missing values.  The reference's data may hold `missing` where a variable was not observed: the leaf then
+ * counts as probability 1 (src/regularization/reg_likelihood.jl:40-47, :76-83), its flow goes to the input node's
+ * `missing_flow`, and the update spreads that flow over the categories as the leaf's own distribution
+ * (src/nodes/fixable_categorical_dist.jl:223-248).  uint8 data has no such value, so a circuit that is to see
+ * missing values is created with one category more than the data has, and this call (HCLT, forest and multi-head
+ * HCLT handles on the block kernels; on != 0) declares that last category, num_cats - 1, the marker: a binding
+ * writes it where the reference has `missing`.  The marker's row of every leaf table is pinned to log-probability
+ * 0 and left out of the normalisation, the pseudocount is shared by the num_cats - 1 real categories, and the
+ * marker's row of the leaf statistics (pcm_hclt_get_flows) is the missing_flow.  Likelihoods, flows and EM
+ * are defined on such a circuit; KL, sampling, soft evidence and Adam return PCM_ERR_UNSUPPORTED.
+ */
+int pcm_set_missing_category(pcm_circuit* c, int32_t on);
+
 /* Head log-parameters of a multi-head HCLT or a forest, [num_trees][num_heads][num_hidden_cats] on the host:
  * the `params` of the head sum nodes (src-jl/multi_head_pc/bit_circuit.jl:14-56 keeps them in the heads'
  * edges), row h of a tree being the head that row h of its head mask seeds. */

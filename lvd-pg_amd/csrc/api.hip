@@ -151,6 +151,10 @@ int pcm_hclt_get_heads(pcm_circuit* c, float* heads) {
   return guarded([&] { need_hclt(c)->get_heads(heads); });
 }
 
+int pcm_set_missing_category(pcm_circuit* c, int32_t on) {
+  return guarded([&] { need_hclt(c)->set_missing_category(on != 0); });
+}
+
 int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf) {
   return guarded([&] { need_hclt(c)->set_block_params(theta, leaf); });
 }

@@ -968,7 +968,26 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
         for (int c = 0; c < C; ++c) t[((size_t)v * C + c) * K + j] = leaf[((size_t)v * K + j) * C + c];
     PCM_HIP(hipMemcpyAsync(d_leaf_.p, t.data(), t.size() * sizeof(float), hipMemcpyHostToDevice, stream));
     PCM_HIP(hipStreamSynchronize(stream));
+    pin_missing_marker();
   }
+}
+
+// The marker of a missing value is a table row like the categories', with log-probability 0 for every hidden state:
+// a missing observation then multiplies every leaf by 1 (src/regularization/reg_likelihood.jl:40-47), its flow
+// collects in the marker's row of the leaf statistics, and no walk or statistics kernel knows about it.
+void HcltCircuit::pin_missing_marker() {
+  if (!missing_) return;
+  PCM_HIP(hipMemset2DAsync(d_leaf_.p + (size_t)(C_ - 1) * K_, (size_t)C_ * K_ * sizeof(float), 0, (size_t)K_ * sizeof(float),
+                           (size_t)V_, stream));
+  general_stale_ = true;
+}
+
+void HcltCircuit::set_missing_category(bool on) {
+  if (on && !(block_ || wide_))
+    fail(PCM_ERR_UNSUPPORTED, "a missing-value category needs the block kernels (K = 16, 32, 64 or 128)");
+  if (on && C_ < 2) fail(PCM_ERR_SHAPE, "a circuit with a missing-value category needs at least one real category");
+  missing_ = on;
+  pin_missing_marker();
 }
 
 void HcltCircuit::set_heads(const float* heads) {
@@ -1084,6 +1103,7 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
   PCM_HIP(hipStreamSynchronize(stream));   // the caller's vector is free again
   rebuild_w();
   general_stale_ = true;
+  pin_missing_marker();
 }
 
 // ---- batches ------------------------------------------------------------------------
@@ -1310,6 +1330,7 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
 
 void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
   no_forest("soft evidence");
+  no_missing("soft evidence");
   if (!soft_block_ok()) return general()->loglikelihoods_soft(s, d_ll);
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   const HcltDev d = soft_stage(s);
@@ -1321,6 +1342,7 @@ void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
   no_forest("soft evidence");
+  no_missing("soft evidence");
   if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (soft_block_ok()) {
     if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
@@ -1534,7 +1556,7 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     const int threads = 1024, cats = ceil_div(C_, threads / 32);
     auto launch = [&](auto kernel) {
       hipLaunchKernelGGL(kernel, dim3(Vu_, ceil_div(K_, 32)), dim3(threads), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
-                         pseudocount, inertia);
+                         pseudocount, inertia, missing_ ? 1 : 0);
     };
     if (cats <= 8) launch(&hclt_leaf_update_kernel<8>);
     else if (cats <= 16) launch(&hclt_leaf_update_kernel<16>);

@@ -182,6 +182,8 @@ class HcltCircuit : public pcm_circuit {
   void set_heads(const float* heads);
   void get_heads(float* heads);
   int num_trees() const { return T_; }
+  // The last of the num_cats categories becomes the marker of a missing value (see pin_missing_marker).
+  void set_missing_category(bool on);
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 
@@ -207,6 +209,13 @@ class HcltCircuit : public pcm_circuit {
   std::vector<int32_t> tree_of_inner_;   // tree of every inner node
   DevBuf<int32_t> d_root_node_;    // ... their nodes
   // what only a single circuit defines (parameter vector order, the general form and the queries on it)
+  bool missing_ = false;           // the last category is the marker of a missing value
+  void pin_missing_marker();
+  void no_missing(const char* what) const {
+    if (missing_)
+      fail(PCM_ERR_UNSUPPORTED, "%s is not defined for a circuit with a missing-value category (likelihoods, flows and EM are)",
+           what);
+  }
   void no_forest(const char* what) const {
     if (forest_) fail(PCM_ERR_UNSUPPORTED, "%s is not defined for a forest handle: use one handle per tree", what);
   }

@@ -776,11 +776,15 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
 // are in flight at once, and nothing is read twice -- sums its flows, the groups are combined
 // through LDS, then every thread rewrites its categories.  Consecutive threads touch consecutive
 // addresses.  blockDim.x * kCats >= 32 * C.
+// missing != 0: row C - 1 is not a category but the marker of a missing value: its flow is the reference's
+// missing_flow (src/nodes/fixable_categorical_dist.jl:233-241: a missing value spreads over the categories as the
+// leaf's own distribution), its log-probability stays 0, and the pseudocount is shared by the C - 1 real categories.
 template <int kCats>
 __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restrict__ leaf,
                                                                const float* __restrict__ leaf_flow, int C, int K,
-                                                               float pseudocount, float inertia) {
+                                                               float pseudocount, float inertia, int missing) {
   __shared__ float part[1024];
+  __shared__ float miss[32];
   const int u = blockIdx.x;
   const int jl = threadIdx.x & 31, cg = threadIdx.x >> 5, ncg = blockDim.x >> 5;
   const int j = blockIdx.y * 32 + jl;
@@ -797,17 +801,23 @@ __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restric
   }
   float s = 0.f;
 #pragma unroll
-  for (int q = 0; q < kCats; ++q) s += f[q];
+  for (int q = 0; q < kCats; ++q) {
+    s += f[q];
+    if (missing && cg + q * ncg == C - 1) miss[jl] = f[q];
+  }
   part[threadIdx.x] = s;
   __syncthreads();
   if (!valid) return;
-  float node_flow = pseudocount;
+  float node_flow = pseudocount;   // (the marker's flow is part of the sum, as the reference adds missing_flow)
   for (int q = 0; q < ncg; ++q) node_flow += part[q * 32 + jl];
-  const float cat_pc = pseudocount / (float)C, scale = (1.f - inertia) / node_flow;
+  const int n_real = missing ? C - 1 : C;
+  const float missing_flow = missing ? miss[jl] : 0.f;
+  const float cat_pc = pseudocount / (float)n_real, scale = (1.f - inertia) / node_flow;
 #pragma unroll
   for (int q = 0; q < kCats; ++q) {
     const int c = cg + q * ncg;
-    if (c < C) lp[(size_t)c * K + j] = __logf(inertia * __expf(p[q]) + (f[q] + cat_pc) * scale);
+    const float oldp = __expf(p[q]);
+    if (c < n_real) lp[(size_t)c * K + j] = __logf(inertia * oldp + (f[q] + cat_pc + missing_flow * oldp) * scale);
   }
 }
 

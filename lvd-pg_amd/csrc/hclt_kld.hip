@@ -368,6 +368,7 @@ __global__ __launch_bounds__(256) void hclt_leaf_adam_kernel(int64_t n_leaf, con
 
 void HcltCircuit::flow_gradients(int32_t batch_size, float* d_grad) {
   no_forest("this query");
+  no_missing("this query");
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   if (flows_in_general_ || (!block_ && !wide_)) return general_->flow_gradients(batch_size, d_grad);
   if (!d_grad) fail(PCM_ERR_ARG, "gradient pointer is null");
@@ -384,6 +385,7 @@ void HcltCircuit::flow_gradients(int32_t batch_size, float* d_grad) {
 
 void HcltCircuit::leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) {
   no_forest("Adam");
+  no_missing("Adam");
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   if (flows_in_general_ || (!block_ && !wide_)) return general_->leaf_adam(d_aux_p, d_aux_m, d_aux_v, lr, b1, b2, eps, t);
   if (!d_aux_p || !d_aux_m || !d_aux_v) fail(PCM_ERR_ARG, "null optimiser array");
@@ -402,6 +404,7 @@ void HcltCircuit::leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, floa
 
 HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
   no_forest("this query");
+  no_missing("this query");
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "KL of multi-head circuits is not defined");
   auto* o = dynamic_cast<HcltCircuit*>(q);
   if (!o) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
@@ -412,6 +415,7 @@ HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
 
 void HcltCircuit::build_kld_tables() {
   no_forest("this query");
+  no_missing("this query");
   if (d_kl_up_.n) return;
   const int W = kl_waves(K_), D = kl_ahead(K_);
   std::vector<int32_t> pos((size_t)2 * n_inner_, 0);
@@ -579,6 +583,7 @@ void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) 
 void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
                             float b2, float eps, int t) {
   no_forest("Adam");
+  no_missing("Adam");
   if (!block_) {
     general()->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t);
     PCM_HIP(hipStreamSynchronize(stream));

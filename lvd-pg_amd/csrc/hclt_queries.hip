@@ -287,6 +287,7 @@ __global__ void hclt_leaf_kc_kernel(const float* __restrict__ leaf, float* __res
 
 SparseCircuit* HcltCircuit::general() {
   no_forest("this query");
+  no_missing("this query");
   if (!general_) {
     general_.reset(new SparseCircuit(flat_));
     general_->stream = stream;
@@ -304,6 +305,7 @@ SparseCircuit* HcltCircuit::general() {
 
 SparseCircuit* HcltCircuit::general_structure() {
   no_forest("this query");
+  no_missing("this query");
   if (!general_) {
     general_.reset(new SparseCircuit(flat_));
     general_stale_ = true;
@@ -321,6 +323,7 @@ void HcltCircuit::pull_from_general() {
 
 void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch, uint8_t* d_out) {
   no_forest("this query");
+  no_missing("this query");
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
   if (!d_node_noise || !d_leaf_noise || !d_out) fail(PCM_ERR_ARG, "null noise or output pointer");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
@@ -397,6 +400,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
 
 void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
   no_forest("this query");
+  no_missing("this query");
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "sampling from a multi-head circuit needs a head choice");
   if (sample_soft_block(d_node_noise, temperature, batch, d_out)) return;
   SparseCircuit* g = general();

@@ -120,6 +120,13 @@ class HcltCircuit(BitsCircuit):
         check(lib.pcm_hclt_get_flows(self.handle, np_ptr(ea), np_ptr(lf)))
         return ea, lf
 
+    def set_missing_category(self, on=True):
+        """Declares the last category (num_cats - 1) the marker of a missing value: data carry it where the
+        reference's data hold `missing` (src/regularization/reg_likelihood.jl:40-47); the leaf then counts as
+        probability 1 and the update treats the marker's flow as `missing_flow`
+        (src/nodes/fixable_categorical_dist.jl:223-248).  Create the circuit with one category more than the data has."""
+        check(lib.pcm_set_missing_category(self.handle, int(bool(on))))
+
     def set_timing(self, on):
         """0 / False: off; 1 / True: the forward, backward and statistics kernels of every flows call carry timing
         events; 2, 4, 8 (or a sum of them): only the forward / backward / statistics kernel does."""

@@ -241,12 +241,12 @@ void orc_input_flows_soft(int n_nodes, const uint8_t* type, const int32_t* in_va
  *   update_params   : logp = log(inertia*exp(logp) + (1-inertia)*edge_aggr/node_aggr),
  *                     skipped for a sum node with a single edge
  *                     (pretrain/mini_batch_warmup.jl:54-70)
- *   leaf update     : nodes/fixable_categorical_dist.jl:223-248 with missing_flow = 0.
+ *   leaf update     : nodes/fixable_categorical_dist.jl:223-248 (missing_flow = 0 unless `missing`).
  * edge_aggr is modified in place (the pseudocount stays in it, as in the reference).
  */
 void orc_em_update(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
                    REAL* logp, REAL* edge_aggr, const int64_t* in_off, int C,
-                   REAL* leaf_logp, const REAL* leaf_flow, REAL pseudocount, REAL inertia) {
+                   REAL* leaf_logp, const REAL* leaf_flow, REAL pseudocount, REAL inertia, int missing) {
   for (int n = 0; n < n_nodes; ++n) {
     if (type[n] == NODE_SUM) {
       int e0 = edge_ptr[n], e1 = edge_ptr[n + 1];
@@ -265,14 +265,18 @@ void orc_em_update(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
     } else if (type[n] == NODE_INPUT) {
       REAL* lp = leaf_logp + in_off[n];
       const REAL* fl = leaf_flow + in_off[n];
+      /* missing != 0: the last of the C table rows is not a category but the marker of a missing value
+       * (log-probability 0, never updated); its flow is the reference's missing_flow (:233-241) */
+      const int num_cats = missing ? C - 1 : C;
+      const REAL missing_flow = missing ? fl[C - 1] : (REAL)0;
       REAL node_flow = 0;
-      REAL cat_pc = pseudocount / (REAL)C;
-      for (int i = 0; i < C; ++i) node_flow += fl[i];
-      node_flow += pseudocount;
-      for (int i = 0; i < C; ++i) {
+      REAL cat_pc = pseudocount / (REAL)num_cats;
+      for (int i = 0; i < num_cats; ++i) node_flow += fl[i];
+      node_flow += missing_flow + pseudocount;
+      for (int i = 0; i < num_cats; ++i) {
         REAL oldp = (REAL)exp((double)lp[i]);
         REAL oldv = inertia * oldp;
-        REAL newv = ((REAL)1 - inertia) * (fl[i] + cat_pc) / node_flow;
+        REAL newv = ((REAL)1 - inertia) * (fl[i] + cat_pc + missing_flow * oldp) / node_flow;
         lp[i] = (REAL)log((double)(oldv + newv));
       }
     }

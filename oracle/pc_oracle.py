@@ -52,8 +52,8 @@ def lib(double=False):
     key = "64" if double else "32"
     if key not in _libs:
         path = os.path.join(HERE, f"liborc{key}.so")
-        if not os.path.exists(path):
-            build()
+        if not os.path.exists(path) or os.path.getmtime(path) < os.path.getmtime(os.path.join(HERE, "pc_oracle.c")):
+            build()   # absent, or older than its source
         _libs[key] = ctypes.CDLL(path)
         assert _libs[key].orc_real_size() == (8 if double else 4)
     return _libs[key]
@@ -243,8 +243,10 @@ def input_flows_soft(fc, ev, mars, flows, leaf_flow=None, double=False):
     return leaf_flow
 
 
-def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False):
-    """Updates fc.logp / fc.leaf_logp in place (float circuits only when double=False)."""
+def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False, missing=False):
+    """Returns the updated (logp, leaf_logp).  missing: the last row of every leaf table marks a missing value
+    (log-probability 0; data carry category C - 1 where the reference has `missing`), and the flow it collected
+    is the `missing_flow` of nodes/fixable_categorical_dist.jl:233-241."""
     R = _real(double)
     logp = np.ascontiguousarray(fc.logp, dtype=R).copy()
     leaf = np.ascontiguousarray(fc.leaf_logp, dtype=R).copy()
@@ -253,7 +255,7 @@ def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False):
     rc = ctypes.c_double if double else ctypes.c_float
     lib(double).orc_em_update(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(logp), _p(ea),
                               _p(fc.in_off), ctypes.c_int(fc.C), _p(leaf), _p(lf),
-                              rc(pseudocount), rc(inertia))
+                              rc(pseudocount), rc(inertia), ctypes.c_int(int(bool(missing))))
     return logp, leaf
 
 

@@ -598,3 +598,72 @@ def test_forest_handle_refuses_what_only_one_circuit_defines(gpu, oracle):
         P.hclt_forest_from_clts(np.array([-1, 0, -1], np.int32), 4, 16, 2)
     with pytest.raises(P.PcmError, match="more than one root"):
         P.multihead_hclt_from_clt(parent, 4, 16, 2)
+
+
+@pytest.mark.parametrize("V,K,C,B,heads", [(9, 16, 6, 70, 0), (14, 32, 256, 100, 0), (6, 128, 9, 48, 0), (11, 64, 5, 33, 0),
+                                           (8, 32, 7, 50, 3)])
+def test_missing_values_as_a_marker_category(gpu, oracle, V, K, C, B, heads):
+    """pcm_set_missing_category: the last category marks a missing value (src/regularization/reg_likelihood.jl:40-47,
+    src/nodes/fixable_categorical_dist.jl:223-248).  Likelihoods, flows (the marker's row = missing_flow) and the EM
+    update against the oracle, whose treatment of the marker is pinned by enumeration of completions."""
+    torch, P = gpu
+    O = oracle
+    from helpers import block_theta, rel_err
+    from pcmi355._lib import lib, check
+    rng = np.random.default_rng(V * K + C)
+    parent = O.random_tree(V, rng, 3)
+    theta, leaf = O.random_hclt_params(parent, K, C - 1, rng, "dirichlet")
+    leaf = np.concatenate([leaf, np.zeros((V, K, 1), np.float32)], axis=2)          # the marker's row: log 1
+    data = rng.integers(0, C - 1, size=(B, V)).astype(np.uint8)
+    data[rng.random((B, V)) < 0.25] = C - 1
+    data[0] = C - 1                                                                  # an example with nothing observed
+    d = torch.from_numpy(data).cuda()
+    if heads:
+        bpc = P.multihead_hclt_from_clt(parent, C, K, heads)
+        head_logp = np.log(rng.dirichlet(np.ones(K), size=heads)).astype(np.float32)
+        bpc.set_heads(head_logp)
+    else:
+        bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_missing_category()
+    noisy = leaf.copy()
+    noisy[:, :, C - 1] = -3.0                                                        # whatever the caller puts there
+    bpc.set_params(block_theta(parent, K, theta), noisy)
+    assert (bpc.get_params()[1][:, :, C - 1] == 0).all()
+    fc = O.hclt_flat(parent, K, C, theta, leaf)
+    if heads:
+        # the oracle's single root row stands for head 0: give it that head's parameters over the root's products
+        mask = np.zeros((B, heads), np.float32)
+        mask[:, 0] = 1.0
+        th0 = {v: t.copy() for v, t in theta.items()}
+        root = int(np.flatnonzero(parent < 0)[0])
+        th0[root] = np.vstack([head_logp[0][None, :], theta[root][1:]]) if theta[root].shape[0] > 1 else head_logp[0][None, :]
+        fc = O.hclt_flat(parent, K, C, th0, leaf)
+        ll = P.probs_flows_circuit(bpc, d, head_mask=torch.from_numpy(mask).cuda()).cpu().numpy()
+    else:
+        ll = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    mars = O.forward(fc, data)
+    assert rel_err(ll[1:], mars[-1][1:]).max() < LL_RTOL
+    assert abs(ll[0]) < 1e-4 and abs(mars[-1][0]) < 1e-4                             # nothing observed: probability 1
+    if heads:
+        return                                                                       # (flows of the body as below)
+    flows, ea = O.backward(fc, mars)
+    lf_ref = O.input_flows(fc, data, flows).reshape(V, K, C)
+    _, lf = bpc.get_flows()
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * max(lf_ref.max(), 1e-3)
+    np.testing.assert_allclose(lf.sum(axis=(1, 2)), B, rtol=1e-4)                    # marker's row included
+    logp_new, leaf_new = O.em_update(fc, ea, lf_ref.reshape(-1), 0.1, 0.9, missing=True)
+    check(lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+    new = fc.copy()
+    new.logp, new.leaf_logp = logp_new, leaf_new
+    th_ref, leaf_ref = O.hclt_block_params(new)
+    th, lp = bpc.get_params()
+    for v, blk in th_ref.items():
+        assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < PARAM_RTOL
+    assert rel_err(np.exp(lp), np.exp(leaf_ref)).max() < PARAM_RTOL
+    assert (lp[:, :, C - 1] == 0).all()
+    np.testing.assert_allclose(np.exp(lp[:, :, :C - 1]).sum(axis=2), 1.0, rtol=1e-5)
+    # a second step keeps going up; what only complete data define is refused
+    ll2 = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    assert ll2.mean() > ll.mean()
+    with pytest.raises(P.PcmError, match="missing-value"):
+        P.kld(bpc, bpc)

@@ -801,3 +801,77 @@ def test_leaf_adam_as_the_source_writes_it():
     np.testing.assert_allclose(aux_p, before + 1e-2 * g / (np.abs(g) + 1e-8), rtol=1e-9)
     assert np.array_equal(fc.leaf_logp, before)
     np.testing.assert_allclose(g[0], 1.0 + 0.1 * 4.0)          # the literal: flow 1, p 0.1, node flow 4
+
+
+# ---- missing values --------------------------------------------------------------------------------
+
+def _marker_case(seed=3, V=4, K=2, C_real=3, N=6):
+    """A small HCLT twice: over the C_real categories, and with one table row more, pinned to log 1, whose
+    category (C_real) marks a missing value in the data."""
+    rng = np.random.default_rng(seed)
+    parent = O.random_tree(V, rng, 3)
+    theta, leaf = O.random_hclt_params(parent, K, C_real, rng, "dirichlet")
+    real = O.hclt_flat(parent, K, C_real, theta, leaf)
+    leaf_m = np.concatenate([leaf, np.zeros((V, K, 1), leaf.dtype)], axis=2)
+    marked = O.hclt_flat(parent, K, C_real + 1, theta, leaf_m)
+    data = rng.integers(0, C_real, size=(N, V)).astype(np.uint8)
+    hole = rng.random((N, V)) < 0.35
+    hole[0] = False                                   # one complete example
+    hole[1] = True
+    hole[1, 0] = False                                # one with a single observed variable
+    data_m = np.where(hole, C_real, data).astype(np.uint8)
+    return real, marked, data_m, hole, C_real
+
+
+def _completions(row, hole_row, C_real):
+    """Every way of filling the holes of one example."""
+    holes = np.flatnonzero(hole_row)
+    for fill in itertools.product(range(C_real), repeat=len(holes)):
+        x = row.copy()
+        x[holes] = fill
+        yield x
+
+
+def test_missing_marker_marginalises_the_variable():
+    """A table row of log-probability 0 for the marker makes the leaf count as 1
+    (src/regularization/reg_likelihood.jl:40-47): the likelihood of an example with holes is then the sum of the
+    likelihoods of all its completions."""
+    real, marked, data_m, hole, C_real = _marker_case()
+    ll = O.forward(marked, data_m, double=True)[-1]
+    for b in range(len(data_m)):
+        comp = np.array(list(_completions(data_m[b], hole[b], C_real)), np.uint8)
+        want = logsumexp(O.forward(real, comp, double=True)[-1])
+        assert abs(ll[b] - want) < 1e-6, b        # (the float32 parameters sum to 1 to seven digits only)
+
+
+def test_missing_flow_update_is_the_m_step_on_expected_counts():
+    """The update with missing_flow (src/nodes/fixable_categorical_dist.jl:223-248) is the EM step for
+    incomplete data: the same numbers as the ordinary update applied to the flows of all completions of
+    every example, each weighted by its posterior probability given what was observed."""
+    real, marked, data_m, hole, C_real = _marker_case()
+    pc, inertia = 0.3, 0.6
+    mars = O.forward(marked, data_m, double=True)
+    flows, ea = O.backward(marked, mars, double=True)
+    lf = O.input_flows(marked, data_m, flows, double=True)
+    logp_m, leaf_m = O.em_update(marked, ea, lf, pc, inertia, double=True, missing=True)
+    # expected complete-data statistics by enumeration, on the circuit without the marker
+    ea_x = np.zeros(real.n_edges)
+    lf_x = np.zeros(len(real.leaf_logp))
+    for b in range(len(data_m)):
+        comp = np.array(list(_completions(data_m[b], hole[b], C_real)), np.uint8)
+        m = O.forward(real, comp, double=True)
+        w = np.exp(m[-1] - logsumexp(m[-1]))                     # posterior of every completion
+        fl, _ = O.backward(real, m, double=True)
+        for i in range(len(comp)):
+            _, ea_i = O.backward(real, m[:, i:i + 1].copy(), double=True)
+            lf_i = O.input_flows(real, comp[i:i + 1], fl[:, i:i + 1].copy(), double=True)
+            ea_x += w[i] * ea_i
+            lf_x += w[i] * lf_i
+    logp_x, leaf_x = O.em_update(real, ea_x, lf_x, pc, inertia, double=True)
+    # (to seven digits: the float32 parameters the circuits start from are normalised no better)
+    np.testing.assert_allclose(logp_m, logp_x, rtol=1e-7, atol=1e-7)
+    C = C_real + 1
+    got = leaf_m.reshape(-1, C)
+    np.testing.assert_allclose(got[:, :C_real], leaf_x.reshape(-1, C_real), rtol=1e-7, atol=1e-7)
+    assert (got[:, C_real] == 0).all()                           # the marker's row stays log 1
+    np.testing.assert_allclose(np.exp(got[:, :C_real]).sum(axis=1), 1.0, rtol=1e-6)
