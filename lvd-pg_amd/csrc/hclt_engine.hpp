@@ -250,6 +250,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_M_;
   int* walk_err_ = nullptr;    // pinned host word the walk kernels raise (HcltDev::err); checked by check_walks()
   void check_walks();
+  int walk_chunk(int batch) const;
+  static BatchRef chunk_of(const BatchRef& b, int off, int chunk);
   // Floats per node in the tile arrays.  The walk engines keep an odd number of tiles per node: with a power
   // of two (a batch of 4096), the tiles that one step reads from different nodes at equal slice offsets fell on
   // the same memory channels (the backward walk ran 4 % slower).  The wide kernels index by slice count.

@@ -92,6 +92,29 @@ def test_ragged_batch_and_example_ids(gpu, oracle):
     _compare_step(gpu, oracle, 10, 32, 11, 37, seed=7, idx=idx, N=200)
 
 
+@pytest.mark.parametrize("K", [16, 32])
+def test_batches_larger_than_the_device_go_through_in_chunks(gpu, oracle, K):
+    """More examples than one 16-example workgroup per compute unit (4096 on 256 units): likelihoods, flows and the
+    EM update of the whole batch, contiguous and through example ids, with flow memory on the second call."""
+    torch, P = gpu
+    import pcmi355._lib as L
+    _compare_step(gpu, oracle, 6, K, 5, 9000, seed=21)
+    rng = np.random.default_rng(3)
+    idx = rng.permutation(12000)[:8200].astype(np.int32)
+    bpc = _compare_step(gpu, oracle, 5, K, 7, 8200, seed=22, idx=idx, N=12000)
+    # flow memory: a second, smaller batch on top of 0.5 x the first equals the two halves of it added by hand
+    from helpers import correlated_data
+    data = torch.from_numpy(correlated_data(12000, 5, 7, 23, bpc.clt_parent)).cuda()
+    P.probs_flows_circuit(bpc, data[:8200].contiguous())
+    ea1, lf1 = bpc.get_flows()
+    P.probs_flows_circuit(bpc, data[8200:].contiguous(), rate=0.5)
+    ea2, lf2 = bpc.get_flows()
+    P.probs_flows_circuit(bpc, data[8200:].contiguous())
+    ea3, lf3 = bpc.get_flows()
+    np.testing.assert_allclose(lf2, 0.5 * lf1 + lf3, rtol=1e-5, atol=1e-4)
+    np.testing.assert_allclose(ea2, 0.5 * ea1 + ea3, rtol=1e-5, atol=1e-4)
+
+
 def test_degenerate_inputs(gpu, oracle):
     """No examples, one example, the smallest tree; a tree of one variable has no sum node and is refused."""
     torch, P = gpu
