@@ -408,6 +408,8 @@ HcltCircuit* HcltCircuit::same_tree(pcm_circuit* q) {
   if (H_ > 0) fail(PCM_ERR_UNSUPPORTED, "KL of multi-head circuits is not defined");
   auto* o = dynamic_cast<HcltCircuit*>(q);
   if (!o) fail(PCM_ERR_ARG, "the two circuits of a KL query must be of the same kind");
+  o->no_forest("this query");
+  o->no_missing("this query");
   if (o->K_ != K_ || o->C_ != C_ || o->H_ != H_ || o->parent_ != parent_)
     fail(PCM_ERR_SHAPE, "the two circuits of a KL query must share one structure");
   return o;

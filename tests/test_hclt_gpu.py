@@ -617,6 +617,26 @@ def test_forest_handle_refuses_what_only_one_circuit_defines(gpu, oracle):
         P.vectorize_parameters(forest)
     with pytest.raises(P.PcmError, match="forest"):
         forest.table("edge2param")
+    data = torch.zeros((8, 5), dtype=torch.uint8, device="cuda")
+    noise = torch.zeros((8, 64), device="cuda")
+    other = P.hclt_from_clt(np.array([-1, 0, 0], np.int32), 4, 16)
+    marked = P.hclt_from_clt(np.array([-1, 0, 0], np.int32), 4, 16)
+    marked.set_missing_category()
+    for bad, what in ((forest, "forest"), (marked, "missing-value")):
+        for call in (lambda: P.kld(bad, bad), lambda: P.kld(other, bad) if bad is marked else P.kld(bad, bad),
+                     lambda: P.kld_backward(bad, bad),
+                     lambda: P.sample(bad, noise, torch.zeros((8, 5, 4), device="cuda")),
+                     lambda: P.gumbel_sample(bad, 8, temperature=1.0),
+                     lambda: P.flow_gradients(bad, 8),
+                     lambda: P.loglikelihoods(bad, torch.zeros((8, bad.num_vars, 4), device="cuda")),
+                     lambda: P.kld(bad, np.zeros((2, 10), np.float32), np.zeros((2, 10), np.float32))):
+            with pytest.raises((P.PcmError, ValueError)) as e:
+                call()
+            assert what in str(e.value) or isinstance(e.value, ValueError), str(e.value)
+    with pytest.raises(P.PcmError, match="head_mask"):      # pcm_em_step carries no head mask
+        from pcmi355._lib import lib, check
+        check(lib.pcm_em_step(forest.handle, data.data_ptr(), data.stride(0), data.stride(1), None, 8, 0.0, 0.1, 0.9,
+                              torch.empty(16, device="cuda").data_ptr()))
     with pytest.raises(P.PcmError, match="tree of its own"):
         P.hclt_forest_from_clts(np.array([-1, 0, -1], np.int32), 4, 16, 2)
     with pytest.raises(P.PcmError, match="more than one root"):
