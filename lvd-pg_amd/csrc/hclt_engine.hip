@@ -58,7 +58,9 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   if (C < 1 || C > 256) fail(PCM_ERR_SHAPE, "num_cats must be in 1..256 (uint8 data), got %d", C);
   parent_.assign(parent, parent + V);
   Vu_ = V;
-  if (forest_) split_wide_nodes();
+  // (single circuits too, where the lean kernels exist: otherwise one node with four children would put the whole
+  // circuit on the general walk kernels, 1.4 x slower on the 3072-variable tree)
+  if (forest_ || K == 16 || K == 32) split_wide_nodes();
   build_structure();
   // K = 64: a parameter block and its prefetched successor do not fit the 128 registers a wave of the 16-wave
   // walk kernels has, so those kernels spill (6 us per step); the node-at-a-time wide kernels take about
@@ -105,7 +107,8 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
 void HcltCircuit::split_wide_nodes() {
   for (int v = 0; v < Vu_; ++v)
     if (parent_[v] >= Vu_ || parent_[v] == v) fail(PCM_ERR_SHAPE, "clt_parent[%d] = %d is out of range", v, parent_[v]);
-  std::vector<std::vector<int32_t>> ch(Vu_);
+  std::vector<std::vector<int32_t>>& ch = uchildren_;
+  ch.assign(Vu_, {});
   for (int v = 0; v < Vu_; ++v)
     if (parent_[v] >= 0) ch[parent_[v]].push_back(v);
   for (int v = 0; v < Vu_; ++v) {
@@ -175,6 +178,10 @@ void HcltCircuit::build_structure() {
     height_[v] = h + 1;
   }
   n_inner_ = (int)var_of_inner_.size();
+  user_index_.assign(n_inner_, -1);
+  n_user_inner_ = 0;
+  for (int n = 0; n < n_inner_; ++n)
+    if (var_of_inner_[n] < Vu_) user_index_[n] = n_user_inner_++;
   // post-order goes tree after tree: a node's tree is the number of roots before it
   tree_of_inner_.assign(n_inner_, 0);
   for (int n = 0, t = 0; n < n_inner_; ++n) {
@@ -189,7 +196,7 @@ void HcltCircuit::build_structure() {
     HcltNode& nd = nodes[n];
     nd.var = v;
     nd.parent = parent_[v] < 0 ? -1 : inner_of_var_[parent_[v]];
-    nd.is_root = parent_[v] < 0 || v >= Vu_;   // (the sum-edge update skips identity blocks: heads' roots, auxiliary nodes)
+    nd.is_root = v >= Vu_ ? 2 : parent_[v] < 0;   // (2: an auxiliary node, whose identity block no update touches)
     nd.ic_off = (int)ci.size();
     nd.lc_off = (int)cl.size();
     for (int c : children_[v]) {
@@ -673,6 +680,9 @@ void HcltCircuit::build_schedules() {
 // part; src/bits_circuit.jl:46-70 for the tables).
 void HcltCircuit::build_param_order() {
   const int K = K_;
+  // the caller's tree: auxiliary nodes (split_wide_nodes) are no part of the circuit the reference would number
+  const std::vector<std::vector<int32_t>>& children_ = V_ > Vu_ ? uchildren_ : this->children_;
+  const int V_ = Vu_;
   std::vector<int64_t> sum_id((size_t)V_ * K, -1), mul_id((size_t)V_ * K, -1), in_id((size_t)V_ * K, -1);
   std::vector<int64_t> rprod_id(K, -1);
   int64_t next = 0;
@@ -728,6 +738,7 @@ void HcltCircuit::build_param_order() {
   std::vector<int> mlayer(V_, 0);
   for (int n = 0; n < n_inner_; ++n) {
     int v = var_of_inner_[n];
+    if (v >= Vu_) continue;
     int lc = 0;
     for (int c : children_[v]) lc = std::max(lc, vlayer[c]);
     if (children_[v].size() > 1) { mlayer[v] = lc + 1; lc = lc + 1; }
@@ -738,6 +749,7 @@ void HcltCircuit::build_param_order() {
   std::vector<Rec> recs;
   for (int n = 0; n < n_inner_; ++n) {
     int v = var_of_inner_[n];
+    if (v >= Vu_) continue;
     if (children_[v].size() > 1)
       for (int j = 0; j < K; ++j) recs.push_back({mlayer[v], mul_id[(size_t)v * K + j], 0, v, j});
     int nk = v == root_ ? (H_ > 0 ? 0 : 1) : K;
@@ -820,6 +832,7 @@ void HcltCircuit::build_param_order() {
   }
   for (int n = 0; n < n_inner_; ++n) {
     const int v = var_of_inner_[n];
+    if (v >= Vu_) continue;
     for (int k = 0; k < K; ++k) {
       if (mul_id[(size_t)v * K + k] >= 0) { flat_.type[mul_id[(size_t)v * K + k]] = kMul; flat_.layer[mul_id[(size_t)v * K + k]] = mlayer[v]; }
       if (sum_id[(size_t)v * K + k] >= 0) { flat_.type[sum_id[(size_t)v * K + k]] = kSum; flat_.layer[sum_id[(size_t)v * K + k]] = vlayer[v]; }
@@ -841,7 +854,7 @@ void HcltCircuit::build_param_order() {
     flat_.e_logp.push_back(0.f);
     if (edge2param_[ed]) {
       const int64_t src = sum_param_src_[edge2param_[ed] - 1];
-      if (src < (int64_t)n_inner_ * K * K) noise_slot_[ed] = (int32_t)((src / ((int64_t)K * K)) * K + src % K);
+      if (src < (int64_t)n_inner_ * K * K) noise_slot_[ed] = (int32_t)(user_index_[src / ((int64_t)K * K)] * K + src % K);
     }
   }
   flat_.finish();
@@ -849,18 +862,18 @@ void HcltCircuit::build_param_order() {
 
 int64_t HcltCircuit::size(int what) const {
   switch (what) {
-    case 0: return (int64_t)sum_param_src_.size() + (int64_t)V_ * K_ * C_;
+    case 0: return (int64_t)sum_param_src_.size() + (int64_t)Vu_ * K_ * C_;
     case 1: return (int64_t)sum_param_src_.size();
     case 2: return n_nodes_;
     case 3: return n_edges_;
-    case 4: return (int64_t)V_ * K_ * C_;
+    case 4: return (int64_t)Vu_ * K_ * C_;
     case 5: return Vu_;
     case 6: return C_;
     case 7: return K_;
-    case 8: return n_inner_;
+    case 8: return n_user_inner_;
     case 9: return (int64_t)layer_ends_.size();
     case 10: return (int64_t)sum_group_size_.size();
-    case 11: return (int64_t)V_ * K_;
+    case 11: return (int64_t)Vu_ * K_;
     case 12: return H_;
     case 13: return 0;
     case 14: return wide_walk_ ? 3 : !block_ ? 0 : lean_ ? 1 : 2;
@@ -891,7 +904,7 @@ void HcltCircuit::index_table(int which, int64_t* out, int64_t n) const {
     }
     case 3: copy(std::vector<int64_t>(sum_group_size_.begin(), sum_group_size_.end())); break;
     case 4: {
-      std::vector<int64_t> cum((size_t)V_ * K_);
+      std::vector<int64_t> cum((size_t)Vu_ * K_);
       for (size_t i = 0; i < cum.size(); ++i) cum[i] = (int64_t)(i + 1) * C_;
       copy(cum); break;
     }
@@ -1036,10 +1049,10 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
   const int K = K_, C = C_;
   std::vector<float> h;
   if (flows_in_general_ || (!block_ && !wide_)) {   // from the layered engine's accumulators: up-edge / input-node order -> blocks
-    std::vector<float> ea((size_t)n_edges_), lf((size_t)V_ * K * C);
+    std::vector<float> ea((size_t)n_edges_), lf((size_t)Vu_ * K * C);
     general_->get_aggregates(ea.data(), n_edges_, lf.data(), (int64_t)lf.size());
     if (edge_aggr) {
-      std::fill(edge_aggr, edge_aggr + (size_t)V_ * K * K, 0.f);
+      std::fill(edge_aggr, edge_aggr + (size_t)Vu_ * K * K, 0.f);
       for (int64_t e = 0; e < n_edges_; ++e)
         if (edge2param_[e]) {
           const int64_t src = sum_param_src_[edge2param_[e] - 1];
@@ -1077,7 +1090,7 @@ void HcltCircuit::vectorize(float* out, int64_t n) {
   if (ns > 0)
     hipLaunchKernelGGL(hclt_params_gather_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
                        d_sum_param_src_.p, d_logtheta_.p, d_param_vec_.p);
-  hipLaunchKernelGGL(hclt_leaf_vector_kernel<true>, dim3(V_, ceil_div(C_, kLeafVecCats)), dim3(256),
+  hipLaunchKernelGGL(hclt_leaf_vector_kernel<true>, dim3(Vu_, ceil_div(C_, kLeafVecCats)), dim3(256),
                      (size_t)kLeafVecCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, d_in_pos_.p, K_, C_,
                      d_param_vec_.p + ns);
   check_launch("vectorize");
@@ -1096,7 +1109,7 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
   if (ns > 0)
     hipLaunchKernelGGL(hclt_params_scatter_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
                        d_sum_param_src_.p, d_param_vec_.p, d_logtheta_.p);
-  hipLaunchKernelGGL(hclt_leaf_vector_kernel<false>, dim3(V_, ceil_div(C_, kLeafVecCats)), dim3(256),
+  hipLaunchKernelGGL(hclt_leaf_vector_kernel<false>, dim3(Vu_, ceil_div(C_, kLeafVecCats)), dim3(256),
                      (size_t)kLeafVecCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, d_in_pos_.p, K_, C_,
                      d_param_vec_.p + ns);
   check_launch("update_parameters");
@@ -1473,7 +1486,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
 
 // Relaxed sampling on the block form; false: this hidden size / temperature goes to the layered engine.
 bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
-  if (!block_ || !(temperature >= kSoftMinTemperature)) return false;
+  if (!block_queries() || !(temperature >= kSoftMinTemperature)) return false;
   if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_out)) & 15)

@@ -148,7 +148,7 @@ class HcltCircuit : public pcm_circuit {
   void kld(pcm_circuit* q, float* out) override;
   void kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) override;
   void kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) override;
-  int64_t sample_noise_size() const override { return (int64_t)n_inner_ * K_; }
+  int64_t sample_noise_size() const override { return (int64_t)n_user_inner_ * K_; }
   void sample(const float* d_node_noise, const float* d_leaf_noise, int32_t batch,
               uint8_t* d_out) override;
   void adam_step(const float* d_grad, float* d_params, float* d_m, float* d_v, float lr, float b1,
@@ -202,11 +202,19 @@ class HcltCircuit : public pcm_circuit {
   int V_, K_, C_, n_inner_, root_;
   int Vu_ = 0;                     // the caller's variables; V_ - Vu_ auxiliary ones behind them (forests only)
   void split_wide_nodes();
+  std::vector<std::vector<int32_t>> uchildren_;   // the caller's tree (children of every variable) where nodes were split
+  // KL, sampling and soft evidence on the block form walk the tree as the kernels see it; with auxiliary nodes in it
+  // those queries take the general form of the caller's circuit instead
+  bool block_queries() const { return block_ && V_ == Vu_; }
   bool forest_ = false;
   int T_ = 1;                      // trees (1 unless a forest)
   int n_groups_ = 1;               // groups of trees the walk kernels take side by side (blockIdx.y)
   std::vector<int32_t> roots_;     // root variable of every tree, in variable order
   std::vector<int32_t> tree_of_inner_;   // tree of every inner node
+  // inner nodes of the caller's tree, and every node's index among them (auxiliary nodes keep the post-order of the
+  // caller's nodes as it would be without them): the sampling noise is indexed by this
+  int n_user_inner_ = 0;
+  std::vector<int32_t> user_index_;
   DevBuf<int32_t> d_root_node_;    // ... their nodes
   // what only a single circuit defines (parameter vector order, the general form and the queries on it)
   bool missing_ = false;           // the last category is the marker of a missing value
@@ -282,7 +290,7 @@ class HcltCircuit : public pcm_circuit {
   int cap_slices_ = 0;
   bool have_flows_ = false;
   // soft evidence on the block kernels (single head, K <= 64)
-  bool soft_block_ok() const { return block_ && !wide_ && H_ == 0; }
+  bool soft_block_ok() const { return block_queries() && !wide_ && H_ == 0; }
   HcltDev soft_stage(const SoftRef& s);
   DevBuf<float> d_soft_lv_, d_soft_m_;   // value table [V][Bp][K] and largest evidence [V][Bp] of the batch
   DevBuf<int32_t> d_soft_gnode_;

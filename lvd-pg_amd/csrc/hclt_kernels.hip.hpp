@@ -746,7 +746,8 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
   const int row = blockIdx.x * RPB + threadIdx.x / G, l = threadIdx.x % G;
   if (row >= n_inner * K) return;
   const int n = row / K, k = row % K;
-  if (nodes[n].is_root && (k > 0 || skip_root)) return;   // multi-head circuits keep an identity block at the root
+  // a root keeps one sum node (row 0), or none under heads (identity block); an auxiliary node (is_root 2) is all identity
+  if (nodes[n].is_root && (k > 0 || skip_root || nodes[n].is_root == 2)) return;
   float* a = edge_aggr + (size_t)row * K;
   float* lt = logtheta + (size_t)row * K;
   const float share = pseudocount / (float)K;

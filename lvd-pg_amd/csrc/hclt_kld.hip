@@ -394,7 +394,7 @@ void HcltCircuit::leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, floa
   d_row_sum_.ensure((size_t)V_ * K_);
   hipLaunchKernelGGL(hclt_leaf_node_flow_kernel, dim3(V_), dim3(std::min(256, ceil_div(K_, 64) * 64)), 0, stream,
                      d_leaf_flow_.p, C_, K_, d_row_sum_.p);
-  const int64_t n_leaf = (int64_t)V_ * K_ * C_;
+  const int64_t n_leaf = (int64_t)Vu_ * K_ * C_;   // (the caller's variables: auxiliary ones have no parameters)
   const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
   hipLaunchKernelGGL(hclt_leaf_adam_kernel, dim3((unsigned)ceil_div(n_leaf, 256)), dim3(256), 0, stream, n_leaf,
                      d_input_order_.p, C_, K_, d_leaf_.p, d_leaf_flow_.p, d_row_sum_.p, d_aux_p, d_aux_m, d_aux_v, lr, b1, b2,
@@ -535,7 +535,7 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
 
 void HcltCircuit::kld(pcm_circuit* q, float* out) {
   HcltCircuit* o = same_tree(q);
-  if (!block_) {
+  if (!block_queries()) {
     general()->kld(o->general(), out);
     return;
   }
@@ -547,7 +547,7 @@ void HcltCircuit::kld(pcm_circuit* q, float* out) {
 
 void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
   HcltCircuit* o = same_tree(q);
-  if (!block_) {
+  if (!block_queries()) {
     general()->kld_backward_dev(o->general(), d_gp, d_gq, n);
     return;
   }
@@ -568,7 +568,7 @@ void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int
 
 void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) {
   HcltCircuit* o = same_tree(q);
-  if (!block_) {
+  if (!block_queries()) {
     general()->kld_backward(o->general(), gp, gq, n);
     return;
   }

@@ -329,7 +329,8 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_leaf_noise)) & 15)
     fail(PCM_ERR_ARG, "noise pointers must be 16-byte aligned (rows are read as 16-byte words)");
-  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0;   // rows of whole 16-byte words, states in a byte
+  // rows of whole 16-byte words, states in a byte; the tree as the caller gave it (no auxiliary nodes)
+  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0 && V_ == Vu_;
   const int stride = (n_inner_ + 15) & ~15;   // bytes of one example's states in LDS
   const size_t st_bytes = (size_t)4 * stride;
   if (!rows_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler

@@ -71,15 +71,17 @@ def test_em_step_on_wide_trees(gpu, oracle, tree):
 
 
 def test_every_walk_kernel_family_is_exercised(gpu, oracle):
-    """Which kernels a circuit gets: lean walks (K <= 32, at most three children per node), general
-    walks (more children; K = 64 on bushy trees), wide block kernels (K = 128; K = 64 on small
-    trees), per-layer kernels (other hidden sizes) -- and the bushy K = 64 case against the oracle."""
+    """Which kernels a circuit gets: lean walks (K <= 32; a node with more than three children is split for them),
+    general walks (K = 64 on bushy trees), wide block kernels (K = 128; K = 64 on small trees), per-layer kernels
+    (other hidden sizes) -- and the bushy K = 64 case against the oracle."""
     torch, P = gpu
     rng = np.random.default_rng(1)
     kind = lambda parent, K: P.hclt_from_clt(np.asarray(parent, np.int32), 4, K).size("walk_kernels")
     chain = [-1] + list(range(9))
-    assert kind(chain, 32) == 1 and kind([-1, 0, 0, 0, 0, 0], 16) == 2 and kind(chain, 128) == 3 and kind(chain, 8) == 0
-    assert kind(chain, 64) == 3
+    assert kind(chain, 32) == 1 and kind([-1, 0, 0, 0, 0, 0], 16) == 1 and kind(chain, 128) == 3 and kind(chain, 8) == 0
+    assert kind(chain, 64) == 3 and kind([-1, 0, 0, 0, 0, 0], 64) == 3
+    star = P.hclt_from_clt(np.array([-1, 0, 0, 0, 0, 0], np.int32), 4, 16)       # what the caller sees is the caller's tree
+    assert star.size("variables") == 6 and star.size("inner_tree_nodes") == 1 and star.size("input_nodes") == 6 * 16
     bushy = oracle.random_tree(600, rng, 3)
     assert kind(bushy, 64) == 2
     bpc = _compare_step(gpu, oracle, 600, 64, 4, 16, seed=5, tree=list(bushy))
@@ -469,9 +471,8 @@ def _forest_case(P, O, rng, T, Vt, K, C, H, max_children=3):
                                                (2, [8, 7], 16, 5, 3, 33, 6)])
 def test_forest_handle_gives_the_bits_of_one_handle_per_tree(gpu, oracle, T, Vt, K, C, H, B, wide):
     """pcm_hclt_create_forest: per tree, likelihoods, flows and the EM update are those of a multi-head handle over
-    that tree's variables (parallel_PG.jl:214-225 runs one such circuit per patch).  With at most three children per
-    tree node both run the same kernels and agree to the bit; nodes with more children are split inside a forest
-    (auxiliary identity nodes) and walked by the general kernels in a handle of their own: same circuit, rounding apart."""
+    that tree's variables (parallel_PG.jl:214-225 runs one such circuit per patch), to the bit where the trees have at
+    most three children per node and within rounding where nodes are split."""
     torch, P = gpu
     from pcmi355._lib import lib, check
     rng = np.random.default_rng(T * 1000 + K)

@@ -187,7 +187,9 @@ def test_sampling_bit_exact_random_dag(gpu, oracle, V, C, width, B, seed):
 
 @pytest.mark.parametrize("V,K,C,B,tree", [
     (7, 16, 8, 130, None), (12, 32, 256, 64, None), (10, 64, 5, 70, None), (9, 4, 6, 50, None), (6, 2, 3, 40, None),
-    (141, 8, 3, 33, [-1] + [0] * 70 + list(range(1, 71)))])      # a level of more than 64 tree nodes
+    (141, 8, 3, 33, [-1] + [0] * 70 + list(range(1, 71))),       # a level of more than 64 tree nodes
+    (13, 16, 6, 50, [-1, 0, 1, 1, 1, 1, 2, 3, 0, 8, 8, 8, 8]),   # four children twice: split for the walks, the noise
+    (11, 32, 5, 40, [-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5])])        # stays indexed by the caller's tree nodes
 def test_sampling_bit_exact_hclt(gpu, oracle, V, K, C, B, tree):
     torch, P = gpu
     O = oracle
@@ -326,9 +328,11 @@ def test_relaxed_sampling_matches_oracle(gpu, oracle, temperature):
     # HCLT: the K sum nodes of a tree node share the noise column of each hidden state.  Block
     # sizes run on the block form (two matrix contractions per tree node and 16 examples), other
     # sizes on the layered engine.
-    for Vh, K, Ch, Bh in ((6, 16, 4, 3), (11, 32, 256, 37), (9, 64, 10, 16), (5, 8, 4, 3),
-                          (7, 16, 200, 20), (6, 32, 20, 33)):       # category tiles left out past C; a partial tile of whole words
-        parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23 + K)
+    star = np.array([-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5], np.int32)    # five non-leaf children: split for the walks
+    for Vh, K, Ch, Bh, tree in ((6, 16, 4, 3, None), (11, 32, 256, 37, None), (9, 64, 10, 16, None), (5, 8, 4, 3, None),
+                                (7, 16, 200, 20, None), (6, 32, 20, 33, None),   # category tiles left out past C; a partial tile of whole words
+                                (11, 16, 5, 9, star)):
+        parent, theta, leaf, flat = make_hclt(Vh, K, Ch, 23 + K, parent=tree)
         h = P.hclt_from_clt(parent, Ch, K)
         h.set_params(block_theta(parent, K, theta), leaf)
         ch, _ = O.clt_children(parent)
@@ -576,7 +580,7 @@ def test_misaligned_noise_is_refused(gpu, oracle):
     assert P.sample(h, aligned, leafn).shape == (B, V)
 
 
-@pytest.mark.parametrize("kind", ["hclt16", "hclt64", "hclt128", "hclt8", "dag"])
+@pytest.mark.parametrize("kind", ["hclt16", "hclt64", "hclt128", "hclt8", "dag", "star32"])
 def test_adam_from_flows_matches_oracle(gpu, oracle, kind):
     """`compute_gradients` and the `adam` loop's step (src/sgd/adam.jl:27-61, :218-242, :305-325) on the block
     engines (lean / general walks, wide blocks), on a hidden size without block kernels and on a DAG: the
@@ -597,7 +601,10 @@ def test_adam_from_flows_matches_oracle(gpu, oracle, kind):
     else:
         K = int(kind[4:])
         V, C = 9, 6
-        parent, theta, leaf, _ = make_hclt(V, K, C, 17)
+        # star: a root with five non-leaf children, which the walk kernels split
+        tree = np.array([-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5], np.int32) if kind.startswith("star") else None
+        V = V if tree is None else len(tree)
+        parent, theta, leaf, _ = make_hclt(V, K, C, 17, parent=tree)
         bpc = P.hclt_from_clt(parent, C, K)
         bpc.set_params(block_theta(parent, K, theta), leaf)
         fc = O.bits_compile(O.hclt_dag(parent, K, C, theta, leaf), C, V)

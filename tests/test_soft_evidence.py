@@ -87,10 +87,11 @@ LL_RTOL, FLOW_RTOL = 1e-5, 1e-4
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("V,K,C,B", [(7, 16, 5, 70), (9, 64, 128, 33), (6, 8, 4, 64), (5, 128, 6, 20)])
-def test_hclt_soft_evidence_matches_oracle(gpu, V, K, C, B):
+@pytest.mark.parametrize("V,K,C,B,tree", [(7, 16, 5, 70, None), (9, 64, 128, 33, None), (6, 8, 4, 64, None), (5, 128, 6, 20, None),
+                                          (11, 16, 6, 40, [-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5])])   # a node the walks split
+def test_hclt_soft_evidence_matches_oracle(gpu, V, K, C, B, tree):
     torch, P = gpu
-    parent, theta, leaf, fc = make_hclt(V, K, C, 50 + V)
+    parent, theta, leaf, fc = make_hclt(V, K, C, 50 + V, parent=None if tree is None else np.array(tree, np.int32))
     rng = np.random.default_rng(V)
     ev = rng.normal(0, 2, (B, V, C)).astype(np.float32)
     ev[rng.random((B, V, C)) < 0.1] = -np.inf                # impossible categories
