@@ -1485,8 +1485,21 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
 }
 
 // Relaxed sampling on the block form; false: this hidden size / temperature goes to the layered engine.
+const float* HcltCircuit::kernel_noise(const float* d_node_noise, int32_t batch) {
+  if (V_ == Vu_ || !d_node_noise) return d_node_noise;
+  if (K_ % 4) fail(PCM_ERR_STATE, "noise rows of %d floats do not move as 16-byte words", K_);
+  if (d_user_index_.n == 0) d_user_index_.upload(user_index_, stream);
+  const int64_t total = (int64_t)batch * n_inner_ * (K_ / 4);
+  d_noise_x_.ensure((size_t)total * 4);
+  hipLaunchKernelGGL(hclt_expand_noise_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, stream,
+                     reinterpret_cast<const float4*>(d_node_noise), d_user_index_.p, n_inner_, n_user_inner_, K_ / 4, total,
+                     reinterpret_cast<float4*>(d_noise_x_.p));
+  check_launch("expand_noise");
+  return d_noise_x_.p;
+}
+
 bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {
-  if (!block_queries() || !(temperature >= kSoftMinTemperature)) return false;
+  if (!block_ || !(temperature >= kSoftMinTemperature)) return false;
   if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_out)) & 15)
@@ -1529,14 +1542,14 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
     hipLaunchKernelGGL(hclt_soft_w_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, 128)), dim3(128), 0, stream, d_logtheta_.p,
                        inv_t, n_inner_, Af, Ab);
     hipLaunchKernelGGL(hclt_soft_walk_kernel<KK>, dim3(ns), dim3(soft_walk_waves(KK) * 64), 0, stream, Af, Ab, parent_of, order,
-                       level_ptr, soft_levels_, d_node_noise, n_inner_, batch, ns, inv_t, d_R_.p);
+                       level_ptr, soft_levels_, kernel_noise(d_node_noise, batch), n_inner_, batch, ns, inv_t, d_R_.p);
     const int nchunks = ceil_div(C_, kSoftLeafCats);
     const int use_rows = (C_ & 3) == 0 ? 1 : 0;   // rows of whole 16-byte words leave through an LDS pad
-    const dim3 lgrid(V_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4));
+    const dim3 lgrid(Vu_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4));   // (the caller's variables)
     const size_t pad_bytes = use_rows ? (size_t)4 * kSlice * (kSoftLeafCats + 4) * sizeof(float) : 0;   // 65 KB
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_soft_leaves_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)pad_bytes));
-    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, lgrid, dim3(256), pad_bytes, stream, d_leaf_.p, state_node, d_R_.p, V_,
+    hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, lgrid, dim3(256), pad_bytes, stream, d_leaf_.p, state_node, d_R_.p, Vu_,
                        C_, batch, ns, nchunks, use_rows, d_out);
   });
   check_launch("hclt_sample_soft");

@@ -203,8 +203,8 @@ class HcltCircuit : public pcm_circuit {
   int Vu_ = 0;                     // the caller's variables; V_ - Vu_ auxiliary ones behind them (forests only)
   void split_wide_nodes();
   std::vector<std::vector<int32_t>> uchildren_;   // the caller's tree (children of every variable) where nodes were split
-  // KL, sampling and soft evidence on the block form walk the tree as the kernels see it; with auxiliary nodes in it
-  // those queries take the general form of the caller's circuit instead
+  // soft evidence on the block form reads evidence per variable of the stored tree; with auxiliary nodes in it
+  // that query takes the general form of the caller's circuit instead
   bool block_queries() const { return block_ && V_ == Vu_; }
   bool forest_ = false;
   int T_ = 1;                      // trees (1 unless a forest)
@@ -215,6 +215,10 @@ class HcltCircuit : public pcm_circuit {
   // caller's nodes as it would be without them): the sampling noise is indexed by this
   int n_user_inner_ = 0;
   std::vector<int32_t> user_index_;
+  DevBuf<int32_t> d_user_index_;
+  DevBuf<float> d_noise_x_;
+  // the sampling noise as the block kernels index it: the caller's array, or a copy with room for the auxiliary nodes
+  const float* kernel_noise(const float* d_node_noise, int32_t batch);
   DevBuf<int32_t> d_root_node_;    // ... their nodes
   // what only a single circuit defines (parameter vector order, the general form and the queries on it)
   bool missing_ = false;           // the last category is the marker of a missing value

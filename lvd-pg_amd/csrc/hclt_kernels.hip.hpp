@@ -822,6 +822,21 @@ __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restric
   }
 }
 
+// Sampling noise comes indexed by the caller's tree nodes; where nodes were split, the kernels' nodes include the
+// auxiliary ones: dst[b][n][:] = src[b][user_index[n]][:], zero for an auxiliary node (whose identity block leaves no
+// choice to the noise).
+__global__ void hclt_expand_noise_kernel(const float4* __restrict__ src, const int32_t* __restrict__ user_index, int n_inner,
+                                         int n_user, int K4, int64_t total, float4* __restrict__ dst) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int q = (int)(i % K4);
+  const int64_t r = i / K4;
+  const int n = (int)(r % n_inner);
+  const int64_t b = r / n_inner;
+  const int u = user_index[n];
+  dst[i] = u >= 0 ? src[(b * n_user + u) * K4 + q] : make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 // xn[node][example] = categories of the node's own variable (byte 0) and of its first three
 // leaf children (bytes 1..3), so that a wave fetches all of them with one request.  A thread makes
 // the words of four examples (Bp is a multiple of 16): one word of four categories in per variable,

@@ -535,7 +535,7 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
 
 void HcltCircuit::kld(pcm_circuit* q, float* out) {
   HcltCircuit* o = same_tree(q);
-  if (!block_queries()) {
+  if (!block_) {
     general()->kld(o->general(), out);
     return;
   }
@@ -547,7 +547,7 @@ void HcltCircuit::kld(pcm_circuit* q, float* out) {
 
 void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int64_t n) {
   HcltCircuit* o = same_tree(q);
-  if (!block_queries()) {
+  if (!block_) {
     general()->kld_backward_dev(o->general(), d_gp, d_gq, n);
     return;
   }
@@ -560,7 +560,8 @@ void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int
   const int64_t ns = (int64_t)sum_param_src_.size();
   hipLaunchKernelGGL(hclt_kld_edge_grad_kernel, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns, K_,
                      d_sum_param_src_.p, d_kl_tabs_.p, d_logtheta_.p, o->d_logtheta_.p, z, h, d_gp, d_gq);
-  hipLaunchKernelGGL(hclt_kld_leaf_grad_kernel, dim3(V_, ceil_div(C_, kLeafGradCats)), dim3(256),
+  // (the caller's variables: an auxiliary one has no parameters to differentiate)
+  hipLaunchKernelGGL(hclt_kld_leaf_grad_kernel, dim3(Vu_, ceil_div(C_, kLeafGradCats)), dim3(256),
                      2 * kLeafGradCats * (K_ + 1) * sizeof(float), stream, d_leaf_.p, o->d_leaf_.p, d_kl_tabs_.p + n_inner_,
                      d_kl_tabs_.p + n_inner_ + V_, h, K_, C_, d_gp + ns, d_gq + ns);
   check_launch_k("hclt_kld_backward");
@@ -568,7 +569,7 @@ void HcltCircuit::kld_backward_dev(pcm_circuit* q, float* d_gp, float* d_gq, int
 
 void HcltCircuit::kld_backward(pcm_circuit* q, float* gp, float* gq, int64_t n) {
   HcltCircuit* o = same_tree(q);
-  if (!block_queries()) {
+  if (!block_) {
     general()->kld_backward(o->general(), gp, gq, n);
     return;
   }

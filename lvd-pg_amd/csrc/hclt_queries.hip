@@ -329,8 +329,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_leaf_noise)) & 15)
     fail(PCM_ERR_ARG, "noise pointers must be 16-byte aligned (rows are read as 16-byte words)");
-  // rows of whole 16-byte words, states in a byte; the tree as the caller gave it (no auxiliary nodes)
-  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0 && V_ == Vu_;
+  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0;   // rows of whole 16-byte words, states in a byte
   const int stride = (n_inner_ + 15) & ~15;   // bytes of one example's states in LDS
   const size_t st_bytes = (size_t)4 * stride;
   if (!rows_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
@@ -371,8 +370,8 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   d_state_.ensure((size_t)batch * n_inner_);
   auto node_states = [&](auto kernel) {
     hipLaunchKernelGGL(kernel, dim3(ceil_div(batch, 4)), dim3(256), st_bytes, stream, d_logtheta_.p,
-                       reinterpret_cast<const int2*>(d_sample_passes_.p), sample_passes_, d_node_noise, n_inner_, stride, batch,
-                       d_state_.p);
+                       reinterpret_cast<const int2*>(d_sample_passes_.p), sample_passes_, kernel_noise(d_node_noise, batch),
+                       n_inner_, stride, batch, d_state_.p);
   };
   switch (K_) {
     case 4: node_states(&hclt_sample_states_node_kernel<4>); break;
@@ -384,16 +383,17 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   // the variable's table in LDS when 64 KB hold it and its rows are whole 16-byte words
   const size_t lds = (size_t)K_ * (C_ + 4) * sizeof(float) + kLeafExamples;
   if ((C_ & 3) == 0 && (K_ & 3) == 0 && lds <= (size_t)64 * 1024) {
-    hipLaunchKernelGGL(hclt_sample_leaves_lds_kernel, dim3(V_, ceil_div(batch, kLeafExamples)), dim3(kLeafWaves * 64), lds,
-                       stream, d_leaf_.p, d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch,
+    // (leaves: the caller's variables, which come first; the auxiliary ones have nothing to draw)
+    hipLaunchKernelGGL(hclt_sample_leaves_lds_kernel, dim3(Vu_, ceil_div(batch, kLeafExamples)), dim3(kLeafWaves * 64), lds,
+                       stream, d_leaf_.p, d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, Vu_, K_, C_, n_inner_, batch,
                        d_out);
   } else {
     d_leaf_kc_.ensure((size_t)V_ * K_ * C_);
     const int64_t tot = (int64_t)V_ * K_ * C_;
     hipLaunchKernelGGL(hclt_leaf_kc_kernel, dim3((unsigned)ceil_div(tot, 256)), dim3(256), 0, stream, d_leaf_.p, d_leaf_kc_.p,
                        V_, K_, C_);
-    hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(V_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
-                       d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, V_, K_, C_, n_inner_, batch, d_out);
+    hipLaunchKernelGGL(hclt_sample_leaves_kernel, dim3(batch, ceil_div(Vu_, 4 * kVarsPerWave)), dim3(256), 0, stream, d_leaf_kc_.p,
+                       d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, Vu_, K_, C_, n_inner_, batch, d_out);
   }
   check_launch_q("hclt_sample");
   PCM_HIP(hipStreamSynchronize(stream));
