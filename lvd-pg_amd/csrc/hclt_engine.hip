@@ -640,6 +640,7 @@ void HcltCircuit::build_schedules() {
       std::memset(&q, 0, sizeof q);
       if (ic[n].size() + lc[n].size() > 3) { stat_lean_ = false; break; }
       q.var = var_of_inner_[n];
+      q.node = n;
       q.c[0] = q.c[1] = q.c[2] = -1;
       int k = 0;
       for (int c : ic[n]) q.c[k++] = c << 3;
@@ -656,6 +657,15 @@ void HcltCircuit::build_schedules() {
       if ((std::max(hist, park) + pads) * 4 > (size_t)max_lds_) stat_lean_ = false;
     }
     if (stat_lean_) {
+      // The workgroups draw the records in this order, and the kernel ends when the last drawn node is done: the
+      // costliest nodes (passes over the batch, then histograms, then operands) go first, so that what is left for
+      // the end are the short ones.
+      const int nh_pass = stat_lean_hists_;
+      auto cost = [&](const StatNode& q) {
+        const int children = (q.c[0] >= 0) + (q.c[1] >= 0) + (q.c[2] >= 0);
+        return ((q.n_hist + nh_pass - 1) / nh_pass) * 100 + std::min(q.n_hist, nh_pass) * 10 + children;
+      };
+      std::stable_sort(sn.begin(), sn.end(), [&](const StatNode& a, const StatNode& b) { return cost(a) > cost(b); });
       d_stat_lean_.upload(sn);
       d_stat_claim_.upload(std::vector<uint32_t>(1, 0u));
     }

@@ -75,7 +75,8 @@ struct StatNode {
   int32_t c[3];       // children: -1 none, leaf child: variable << 3 | 1 | category byte << 1, inner child: node << 3
   int32_t n_hist;     // variables to histogram: own + leaf children
   int32_t hvar[4];    // ... their ids; entry i uses category byte i
-  int32_t pad[7];
+  int32_t node;       // the node's index (the records are in the order the workgroups draw them: costliest first)
+  int32_t pad[6];
 };
 static_assert(sizeof(StatNode) == 64, "StatNode is read with scalar loads");
 

@@ -457,6 +457,7 @@ constexpr int kStatLeanWaves = 16;
 
 // A node's scalars as the statistics kernel uses them.
 struct StatRef {
+  int node;          // the node's index
   int tile_off;      // byte offset of the node's tiles in the value and ratio arrays
   int x_off;         // ... of its row of packed categories (and of row maxima)
   int leaf_off;      // ... of its own variable's leaf table
@@ -465,9 +466,11 @@ struct StatRef {
   int n_hist;
 };
 
-__device__ __forceinline__ StatRef stat_ref(const HcltDev& d, const StatNode* __restrict__ nodes, int n, int kk4) {
-  const StatNode* __restrict__ np = nodes + n;
+__device__ __forceinline__ StatRef stat_ref(const HcltDev& d, const StatNode* __restrict__ nodes, int pos, int kk4) {
+  const StatNode* __restrict__ np = nodes + pos;
+  const int n = np->node;
   StatRef r;
+  r.node = n;
   r.tile_off = n * (int)d.tile_stride;
   r.x_off = n * d.Bp * 4;
   r.leaf_off = np->var * (int)d.leaf_stride;
@@ -730,7 +733,7 @@ __global__ __launch_bounds__(kStatLeanWaves * 64) void hclt_stats_lean_kernel(
     if (nxt >= 0) lean_w_load<K>(rW, vtile, B.w_off, w);   // the next node's block, into the registers just freed
     __syncthreads();
     {
-      float* dst = edge_aggr + (size_t)cur * K * K;
+      float* dst = edge_aggr + (size_t)A.node * K * K;
       float* parkf = smem;
       for (int t = threadIdx.x; t < K * K; t += blockDim.x) {   // one element a thread: (tile q, component v)
         const int q = t >> 2, v = t & 3;
