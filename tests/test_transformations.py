@@ -431,6 +431,26 @@ def test_write_back_parameters_after_em(gpu, oracle):
     np.testing.assert_allclose(ll, np.stack([va[id(r)] for r in after], 1), rtol=2e-5)
     vb = D.values(before, data)
     assert np.abs(np.stack([vb[id(r)] for r in before], 1) - ll).max() > 1e-3    # the parameters did move
+
+
+@pytest.mark.gpu
+def test_trained_heads_through_a_jpc_file(gpu, oracle, tmp_path):
+    """write_mhpc / read_mhpc (src-jl/multi_head_pc/io.jl:2-9) around a trained circuit: the heads read back
+    compile to a circuit with the same likelihoods, to the bit."""
+    torch, P = gpu
+    rng = np.random.default_rng(15)
+    heads, data, mask = _heads_and_data(oracle, rng, B=96)
+    pcs, _ = from_oracle_dag(heads)
+    bpc = P.CuMultiHeadBitsProbCircuit(pcs)
+    d, hm = torch.from_numpy(data).cuda(), torch.from_numpy(mask).cuda()
+    P.mini_batch_em_for_multihead_pc(bpc, d, hm, 1, batch_size=48, pseudocount=0.1, param_inertia=0.5, shuffle="none")
+    P.write_back_parameters(bpc)
+    path = tmp_path / "heads.jpc.gz"
+    P.write_mhpc(path, pcs)
+    back = P.read_mhpc(path)
+    assert len(back) == len(pcs)
+    bpc2 = P.CuMultiHeadBitsProbCircuit(back)
+    np.testing.assert_array_equal(P.loglikelihoods(bpc2, d).cpu().numpy(), P.loglikelihoods(bpc, d).cpu().numpy())
     again = P.CuMultiHeadBitsProbCircuit(pcs)
     np.testing.assert_array_equal(P.vectorize_parameters(again), P.vectorize_parameters(bpc))
 
