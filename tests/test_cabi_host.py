@@ -87,6 +87,36 @@ def test_python_mirror_binds_every_symbol():
         assert hasattr(L.lib, n), n
 
 
+def test_julia_bindings_follow_the_header_and_the_ctypes_table():
+    """lvd-pg_amd/julia/LibPCMI355.jl is what gen_bindings.py writes from the header, binds every entry point, and
+    its argument types are the ones the ctypes table of the Python mirror uses (two independent readings of the
+    header)."""
+    import importlib.util
+    import pcmi355._lib as L
+    jdir = os.path.join(ROOT, "lvd-pg_amd", "julia")
+    spec = importlib.util.spec_from_file_location("gen_bindings", os.path.join(jdir, "gen_bindings.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    text = open(os.path.join(jdir, "LibPCMI355.jl")).read()
+    assert text == gen.render(open(HEADER).read()), "run python lvd-pg_amd/julia/gen_bindings.py"
+    bound = dict(re.findall(r"ccall\(\(:(pcm_[a-z0-9_]+), libpcmi355\), \w+, \(([^)]*)\)", text))
+    assert sorted(bound) == declared_symbols()
+
+    def kind(t):
+        if t in (ctypes.c_int32, ctypes.c_int):
+            return "Int32"
+        if t is ctypes.c_int64:
+            return "Int64"
+        if t is ctypes.c_float:
+            return "Float32"
+        return "Ptr"
+    for name in declared_symbols():
+        argtypes = getattr(L.lib, name).argtypes or []
+        jl = [t.strip() for t in bound[name].split(",") if t.strip()]
+        jl = ["Ptr" if t.startswith("Ptr{") else "Int32" if t == "Cint" else t for t in jl]
+        assert jl == [kind(t) for t in argtypes], name
+
+
 def test_workload_builders():
     from pcmi355 import workloads as W
     a = W.grf_images(64, 8, 8, 3, 2.0, 0.8, seed=5)
