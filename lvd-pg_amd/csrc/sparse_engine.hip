@@ -261,10 +261,15 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int 
 // kLayerWaves waves share a node's edges: the kernels are chains of dependent memory round
 // trips, so a layer too small to fill the machine finishes sooner when a node's chain is cut in
 // four; layers with plenty of (node, 64 examples) pairs give each pair one wave.
+// kMaxRun = 4 leaves out the runs of 32 and 16: a layer whose nodes have few edges then runs in a third of the
+// registers, i.e. with three times the waves in flight to hide its round trips, and with EX = 4 a wave's index
+// fetches (node, edge range, edge records) serve 256 examples instead of 64.
 constexpr int kSplitWaves = 4;
 constexpr int kSplitBelow = 1024;   // (node, 64 examples) pairs in a layer below which its nodes are split
+constexpr int kNarrowDegree = 8;    // a layer whose nodes have at most this many edges takes the kMaxRun = 4 kernels
+constexpr int kManyPairs = 16384;   // (node, 64 examples) pairs from which a narrow layer takes four examples per lane
 
-template <int EX, int kLayerWaves>
+template <int EX, int kLayerWaves, int kMaxRun = 32>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(SparseDev d, int n0) {
   __shared__ float xm[kLayerWaves][EX][64], xs[kLayerWaves][EX][64];
   const int n = d.order[n0 + blockIdx.x];
@@ -293,8 +298,10 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
 #pragma unroll
     for (int x = 0; x < EX; ++x) { m[x] = issum ? -INFINITY : 0.f; sum[x] = issum ? 0.f : 1.f; }
     int c0 = my0;
-    for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX>(d, issum, c0, bb, m, sum);
-    for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX>(d, issum, c0, bb, m, sum);
+    if constexpr (kMaxRun >= 32)
+      for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX>(d, issum, c0, bb, m, sum);
+    if constexpr (kMaxRun >= 16)
+      for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX>(d, issum, c0, bb, m, sum);
     for (; c0 + 4 <= my1; c0 += 4) forward_run<4, EX>(d, issum, c0, bb, m, sum);
     for (; c0 < my1; ++c0) forward_run<1, EX>(d, issum, c0, bb, m, sum);
     if (e1 - e0 > per) {   // more than one share is in use (uniform over the workgroup)
@@ -397,7 +404,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
 // edge).  Each edge's flow is summed over the batch where the node is the edge's prime
 // (:73-81): over the thread's examples, then over the wave; the wave's sum goes to row blockIdx.y of
 // edge_part ([gridDim.y][n_edges]), whose rows a later kernel adds up in order.
-template <int EX, int kLayerWaves>
+template <int EX, int kLayerWaves, int kMaxRun = 32>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
                                                                            const int32_t* __restrict__ seed_of,
                                                                            const float* __restrict__ seed,
@@ -426,8 +433,10 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
   int c0 = my0;
-  for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_part);
-  for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_part);
+  if constexpr (kMaxRun >= 32)
+    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_part);
+  if constexpr (kMaxRun >= 16)
+    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_part);
   for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_part);
   for (; c0 < my1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
@@ -919,6 +928,11 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   layer_node0_.assign(n_layers_ + 1, 0);
   for (int64_t i = 0; i < nn; ++i) layer_node0_[fc_.layer[order[i]] + 1]++;
   for (int l = 0; l < n_layers_; ++l) layer_node0_[l + 1] += layer_node0_[l];
+  layer_max_children_.assign(n_layers_, 0);
+  for (int l = 0; l < n_layers_; ++l)
+    for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i)
+      if (fc_.type[order[i]] != kInput)
+        layer_max_children_[l] = std::max(layer_max_children_[l], (int)(fc_.node_e1[order[i]] - fc_.node_e0[order[i]]));
   // incoming edges per node: entry = edge << 1 | as_sub
   std::vector<int32_t> in_ptr(nn + 1, 0), in_edge;
   for (int64_t e = 0; e < ne; ++e) { in_ptr[fc_.e_prime[e] + 1]++; if (fc_.e_sub[e] >= 0) in_ptr[fc_.e_sub[e] + 1]++; }
@@ -981,9 +995,13 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   if (alias_list.empty()) alias_list.push_back(0);
   std::vector<int32_t> bwd_order;
   bwd_layer0_.assign(n_layers_ + 1, 0);
+  bwd_layer_max_in_.assign(n_layers_, 0);
   for (int l = 0; l < n_layers_; ++l) {
     for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i)
-      if (alias_of[order[i]] < 0) bwd_order.push_back(order[i]);
+      if (alias_of[order[i]] < 0) {
+        bwd_order.push_back(order[i]);
+        bwd_layer_max_in_[l] = std::max(bwd_layer_max_in_[l], (int)(in_ptr[order[i] + 1] - in_ptr[order[i]]));
+      }
     bwd_layer0_[l + 1] = (int)bwd_order.size();
   }
   d_alias_ptr_.upload(alias_ptr);
@@ -1134,10 +1152,15 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
   }
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
-    if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
+    const int64_t pairs = (int64_t)cnt * (Bp / 64);
+    if (pairs < kSplitBelow)
       hipLaunchKernelGGL((sparse_forward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, d, n0);
-    else
+    else if (layer_max_children_[l] > kNarrowDegree)
       hipLaunchKernelGGL((sparse_forward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
+    else if (pairs < kManyPairs)
+      hipLaunchKernelGGL((sparse_forward_kernel<1, 1, 4>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
+    else
+      hipLaunchKernelGGL((sparse_forward_kernel<4, 1, 4>), dim3(cnt, ceil_div(Bp, 256)), dim3(64), 0, stream, d, n0);
   }
   check_launch("sparse_forward");
   last_batch_ = batch;
@@ -1212,11 +1235,18 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
   for (int l = n_layers_ - 1; l >= 0; --l) {
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     if (cnt == 0) continue;
-    if ((int64_t)cnt * (Bp / 64) < kSplitBelow)
+    const int64_t pairs = (int64_t)cnt * (Bp / 64);
+    if (pairs < kSplitBelow)
       hipLaunchKernelGGL((sparse_backward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, db, n0,
                          d_heads_.p, d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
-    else
+    else if (bwd_layer_max_in_[l] > kNarrowDegree)
       hipLaunchKernelGGL((sparse_backward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
+                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
+    else if (pairs < kManyPairs)
+      hipLaunchKernelGGL((sparse_backward_kernel<1, 1, 4>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
+                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
+    else   // (the rows of partial edge sums beyond a quarter stay as cleared)
+      hipLaunchKernelGGL((sparse_backward_kernel<4, 1, 4>), dim3(cnt, ceil_div(Bp, 256)), dim3(64), 0, stream, db, n0, d_heads_.p,
                          d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
   }
   if (ne)

@@ -111,6 +111,7 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_in_logp_, d_edge_part_;
   DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
+  std::vector<int> layer_max_children_, bwd_layer_max_in_;   // per layer: most edges of a node going up / coming in
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;

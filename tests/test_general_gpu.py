@@ -105,6 +105,14 @@ def test_random_dag_em_step(gpu, oracle, V, C, width, seed):
     _check_em_step(gpu, oracle, root, V, C, 96, seed=seed + 50)
 
 
+def test_random_dag_em_step_on_a_large_batch(gpu, oracle):
+    """Layers of many nodes with few edges each take the layer kernels with four examples per lane
+    (at least 16384 (node, 64 examples) pairs): 96 input nodes and 16000 examples."""
+    from helpers import random_dag
+    root = random_dag(12, 5, np.random.default_rng(21), width=8)
+    _check_em_step(gpu, oracle, root, 12, 5, 16000, seed=77)
+
+
 def test_example_ids_and_flow_memory(gpu, oracle):
     """Batches picked by example ids; accumulators scaled by `rate` before a batch
     (src/regularization/reg_em.jl:276-284)."""
