@@ -203,6 +203,7 @@ struct SparseDev {
   float* mars;               // [n_nodes][Bp]
   float* flows;
   int32_t B, Bp, C;
+  int64_t n_nodes;
 };
 
 // ProbabilisticCircuits.jl logsumexp(x, y) as used by src/queries/likelihood.jl:101-102.
@@ -222,20 +223,51 @@ __device__ __forceinline__ float keep_bits(float x, unsigned keep) {
   return __builtin_bit_cast(float, __builtin_bit_cast(unsigned, x) & keep);
 }
 
-template <int U, int EX>
-__device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int c0, const int (&bb)[EX],
-                                            float (&m)[EX], float (&sum)[EX]) {
+
+// A value every lane of the wave holds alike, moved to a scalar register: what is computed from it (row
+// addresses, edge ranges, branch conditions) is then scalar work, and a row access becomes scalar base + lane
+// offset.  Without it the layer kernels keep a copy of every index and 64-bit address per lane and run out of
+// registers: 2 waves per SIMD with 32 edges in flight.
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ float uni(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, v)));
+}
+
+// The rows of the value and flow arrays, addressed the way the layer kernels need them: one descriptor per
+// array in scalar registers, the row as a scalar byte offset, the example as the lane's byte offset -- a row
+// costs one scalar register instead of a 64-bit address.  kBuf = false (arrays of 4 GiB or more, beyond a
+// descriptor's range) keeps plain pointers.
+template <bool kBuf>
+struct Rows {
+  const float* base;
+  __amdgpu_buffer_rsrc_t rsrc;
+  int row_bytes;
+  __device__ __forceinline__ Rows(const float* p, int64_t n_rows, int Bp) : base(p), row_bytes(Bp * 4) {
+    if constexpr (kBuf)
+      rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p), 0, (int)(uint32_t)(n_rows * Bp * 4), 0x00020000);
+  }
+  // value of example b (a lane's own) in row `row` (wave-uniform)
+  __device__ __forceinline__ float at(int row, int b) const {
+    if constexpr (kBuf)
+      return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, b * 4, row * row_bytes, 0));
+    else
+      return base[(size_t)row * (row_bytes >> 2) + b];
+  }
+};
+
+template <int U, int EX, bool kBuf>
+__device__ __forceinline__ void forward_run(const SparseDev& d, const Rows<kBuf>& mars, bool issum, int c0,
+                                            const int (&bb)[EX], float (&m)[EX], float (&sum)[EX]) {
   float child[U][EX];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int e = c0 + u;
-    const float* pr = d.mars + (size_t)d.e_prime[e] * d.Bp;
-    const int s = d.e_sub[e];
-    const float* sr = d.mars + (size_t)max(s, 0) * d.Bp;
+    const int pr = uni(d.e_prime[e]);
+    const int s = uni(d.e_sub[e]);
     const unsigned has_sub = s >= 0 ? ~0u : 0u;
-    const float lp = d.logp[e];   // 0 on product edges
+    const float lp = uni(d.logp[e]);   // 0 on product edges
 #pragma unroll
-    for (int x = 0; x < EX; ++x) child[u][x] = pr[bb[x]] + keep_bits(sr[bb[x]], has_sub) + lp;
+    for (int x = 0; x < EX; ++x) child[u][x] = mars.at(pr, bb[x]) + keep_bits(mars.at(max(s, 0), bb[x]), has_sub) + lp;
   }
 #pragma unroll
   for (int u = 0; u < U; ++u)
@@ -261,49 +293,61 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, bool issum, int 
 // kLayerWaves waves share a node's edges: the kernels are chains of dependent memory round
 // trips, so a layer too small to fill the machine finishes sooner when a node's chain is cut in
 // four; layers with plenty of (node, 64 examples) pairs give each pair one wave.
-// kMaxRun = 4 leaves out the runs of 32 and 16: a layer whose nodes have few edges then runs in a third of the
-// registers, i.e. with three times the waves in flight to hide its round trips, and with EX = 4 a wave's index
-// fetches (node, edge range, edge records) serve 256 examples instead of 64.
+// Which build of the two layer kernels a layer takes (measured on a 192-variable, K = 32, 128-head circuit at
+// 1024 examples, 1.31 -> 0.72 ms per EM step together with the scalar indices and buffer-addressed rows above):
+//   * nodes with at most kNarrowDegree edges: runs of 4 only (a third of the registers, three times the waves in
+//     flight), from kManyPairs (node, 64 examples) pairs on with four examples per lane, so that a wave's index
+//     fetches (node, edge range, edge records) serve 256 examples;
+//   * otherwise, below kSplitBelow pairs: kSplitWaves waves share a node's edges (the layer cannot fill the
+//     device with one wave per pair, and a wave's chain of round trips gets shorter);
+//   * otherwise one wave per pair, runs of up to kWideRun edges requested at once (16: seven waves per SIMD;
+//     32 halves the waves and is slower, 8 leaves too few requests in flight).
 constexpr int kSplitWaves = 4;
-constexpr int kSplitBelow = 1024;   // (node, 64 examples) pairs in a layer below which its nodes are split
+constexpr int kSplitRun = 16;       // longest run in the kernels that split a node over kSplitWaves waves
+constexpr int kSplitBelow = 8192;   // (node, 64 examples) pairs in a layer below which its nodes are split
 constexpr int kNarrowDegree = 8;    // a layer whose nodes have at most this many edges takes the kMaxRun = 4 kernels
+constexpr int kWideRun = 16;        // longest run of edges requested at once in the one-wave kernels
 constexpr int kManyPairs = 16384;   // (node, 64 examples) pairs from which a narrow layer takes four examples per lane
 
-template <int EX, int kLayerWaves, int kMaxRun = 32>
+template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(SparseDev d, int n0) {
   __shared__ float xm[kLayerWaves][EX][64], xs[kLayerWaves][EX][64];
-  const int n = d.order[n0 + blockIdx.x];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = uni(d.order[n0 + blockIdx.x]);
+  const int lane = threadIdx.x & 63, wave = uni((int)(threadIdx.x >> 6));
   const int b0 = blockIdx.y * (64 * EX) + lane;
   int bb[EX];
 #pragma unroll
   for (int x = 0; x < EX; ++x) bb[x] = min(b0 + 64 * x, d.Bp - 1);
   float m[EX], sum[EX];
-  if (d.type[n] == kInput) {
+  const int type = uni((int)d.type[n]);
+  if (type == kInput) {
     if (wave) return;
     if (d.ev) return;   // soft evidence: sparse_soft_input_kernel has filled the input rows
     {
-      const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
+      const uint8_t* xr = d.xb + (size_t)uni(d.in_var[n]) * d.Bp;
+      const int64_t off = d.in_off[n];
+      const float* row = d.leaf + (((int64_t)uni((int)(off >> 32)) << 32) | (uint32_t)uni((int)off));
 #pragma unroll
-      for (int x = 0; x < EX; ++x) { m[x] = d.leaf[d.in_off[n] + xr[bb[x]]]; sum[x] = 1.f; }
+      for (int x = 0; x < EX; ++x) { m[x] = row[xr[bb[x]]]; sum[x] = 1.f; }
     }
   } else {
     // the node's edges in kLayerWaves contiguous shares, one per wave; a share is folded as a
     // running maximum and a sum of exponentials (products: a plain sum), the shares are then
     // combined through LDS by the first wave
-    const bool issum = d.type[n] == kSum;
-    const int e0 = d.node_e0[n], e1 = d.node_e1[n];
+    const bool issum = type == kSum;
+    const int e0 = uni(d.node_e0[n]), e1 = uni(d.node_e1[n]);
     const int per = (e1 - e0 + kLayerWaves - 1) / kLayerWaves;
     const int my0 = min(e0 + wave * per, e1), my1 = min(my0 + per, e1);
 #pragma unroll
     for (int x = 0; x < EX; ++x) { m[x] = issum ? -INFINITY : 0.f; sum[x] = issum ? 0.f : 1.f; }
+    const Rows<kBuf> mars(d.mars, d.n_nodes, d.Bp);
     int c0 = my0;
     if constexpr (kMaxRun >= 32)
-      for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX>(d, issum, c0, bb, m, sum);
+      for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     if constexpr (kMaxRun >= 16)
-      for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX>(d, issum, c0, bb, m, sum);
-    for (; c0 + 4 <= my1; c0 += 4) forward_run<4, EX>(d, issum, c0, bb, m, sum);
-    for (; c0 < my1; ++c0) forward_run<1, EX>(d, issum, c0, bb, m, sum);
+      for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
+    for (; c0 + 4 <= my1; c0 += 4) forward_run<4, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
+    for (; c0 < my1; ++c0) forward_run<1, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     if (e1 - e0 > per) {   // more than one share is in use (uniform over the workgroup)
 #pragma unroll
       for (int x = 0; x < EX; ++x) { xm[wave][x][lane] = m[x]; xs[wave][x][lane] = sum[x]; }
@@ -356,28 +400,26 @@ __device__ __forceinline__ float wave_sum(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
 }
 
-template <int U, int EX>
-__device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const int (&bb)[EX], const bool (&live)[EX],
-                                             float (&acc)[EX], float* __restrict__ edge_part) {
+template <int U, int EX, bool kBuf>
+__device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf>& mars, const Rows<kBuf>& flows, int c0,
+                                             const int (&bb)[EX], const bool (&live)[EX], float (&acc)[EX],
+                                             float* __restrict__ edge_part) {
   float fl[U][EX], ex[U][EX];
   int ies[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int4 rec = d.in_rec[c0 + u];   // one scalar record per edge instead of a chain of four index fetches
-    ies[u] = rec.x;
-    const bool issum = rec.y >= 0;
-    const int p = issum ? rec.y : ~rec.y;
-    const int s = rec.w;
-    const float* fr = d.flows + (size_t)p * d.Bp;
-    const float* mp = d.mars + (size_t)p * d.Bp;
-    const float* pr = d.mars + (size_t)rec.z * d.Bp;
-    const float* sr = d.mars + (size_t)max(s, 0) * d.Bp;
-    const float lp = d.in_logp[c0 + u];
+    const int4 rec = d.in_rec[c0 + u];   // one record per edge instead of a chain of four index fetches
+    ies[u] = uni(rec.x);
+    const int ry = uni(rec.y);
+    const bool issum = ry >= 0;
+    const int p = issum ? ry : ~ry;
+    const int s = uni(rec.w), pr = uni(rec.z);
+    const float lp = uni(d.in_logp[c0 + u]);
     const unsigned has_sub = s >= 0 ? ~0u : 0u, sum_edge = issum ? ~0u : 0u;
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
-      fl[u][x] = fr[bb[x]];
-      ex[u][x] = keep_bits(pr[bb[x]] + lp + keep_bits(sr[bb[x]], has_sub) - mp[bb[x]], sum_edge);
+      fl[u][x] = flows.at(p, bb[x]);
+      ex[u][x] = keep_bits(mars.at(pr, bb[x]) + lp + keep_bits(mars.at(max(s, 0), bb[x]), has_sub) - mars.at(p, bb[x]), sum_edge);
     }
   }
 #pragma unroll
@@ -404,7 +446,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, int c0, const i
 // edge).  Each edge's flow is summed over the batch where the node is the edge's prime
 // (:73-81): over the thread's examples, then over the wave; the wave's sum goes to row blockIdx.y of
 // edge_part ([gridDim.y][n_edges]), whose rows a later kernel adds up in order.
-template <int EX, int kLayerWaves, int kMaxRun = 32>
+template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
                                                                            const int32_t* __restrict__ seed_of,
                                                                            const float* __restrict__ seed,
@@ -412,14 +454,14 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
                                                                            const int32_t* __restrict__ alias_ptr,
                                                                            const int32_t* __restrict__ alias_list) {
   __shared__ float xa[kLayerWaves][EX][64];
-  const int n = d.order[n0 + blockIdx.x];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = uni(d.order[n0 + blockIdx.x]);
+  const int lane = threadIdx.x & 63, wave = uni((int)(threadIdx.x >> 6));
   const int b0 = blockIdx.y * (64 * EX) + lane;
   float* edge_part = edge_part_all ? edge_part_all + (size_t)blockIdx.y * n_edges : nullptr;
   int bb[EX];
   bool live[EX];
   float acc[EX];
-  const int sd = seed_of[n];
+  const int sd = uni(seed_of[n]);
 #pragma unroll
   for (int x = 0; x < EX; ++x) {
     const int b = b0 + 64 * x;
@@ -429,16 +471,17 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
     if (sd >= 0 && wave == 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
   }
   // the node's incoming edges in kLayerWaves contiguous shares, one per wave
-  const int i0 = d.in_ptr[n], i1 = d.in_ptr[n + 1];
+  const int i0 = uni(d.in_ptr[n]), i1 = uni(d.in_ptr[n + 1]);
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
+  const Rows<kBuf> mars(d.mars, d.n_nodes, d.Bp), flows(d.flows, d.n_nodes, d.Bp);
   int c0 = my0;
   if constexpr (kMaxRun >= 32)
-    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX>(d, c0, bb, live, acc, edge_part);
+    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   if constexpr (kMaxRun >= 16)
-    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX>(d, c0, bb, live, acc, edge_part);
-  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX>(d, c0, bb, live, acc, edge_part);
-  for (; c0 < my1; ++c0) backward_run<1, EX>(d, c0, bb, live, acc, edge_part);
+    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+  for (; c0 < my1; ++c0) backward_run<1, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
 #pragma unroll
     for (int x = 0; x < EX; ++x) xa[wave][x][lane] = acc[x];
@@ -458,8 +501,8 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   }
   // input nodes that receive exactly this node's edge flows (the other factor of the same
   // two-child products) are not computed again: their rows are copies
-  for (int q = alias_ptr[n]; q < alias_ptr[n + 1]; ++q) {
-    const int t = alias_list[q];
+  for (int q = uni(alias_ptr[n]), q1 = uni(alias_ptr[n + 1]); q < q1; ++q) {
+    const int t = uni(alias_list[q]);
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
       const int b = b0 + 64 * x;
@@ -1102,18 +1145,27 @@ void SparseCircuit::ensure_batch(int batch) {
 static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32_t* e0, const int32_t* e1,
                           const int32_t* ep, const int32_t* epr, const int32_t* es, const int32_t* in_var,
                           const int32_t* in_ptr, const int32_t* in_edge, const int4* in_rec, const int64_t* in_off, const float* logp,
-                          const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C) {
+                          const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C, int64_t n_nodes) {
   SparseDev d;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
   d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off;
   d.ev = nullptr; d.ev_se = d.ev_sv = d.ev_sc = 0; d.ev_idx = nullptr; d.logp = logp; d.leaf = leaf;
-  d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C;
+  d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C; d.n_nodes = n_nodes;
   return d;
 }
 
+// a layer kernel with rows through buffer descriptors where the value / flow arrays are within a descriptor's 4 GiB
+#define PCM_LAYER_LAUNCH(kernel, EX_, W_, RUN_, grid, ...)                                                      \
+  do {                                                                                                          \
+    if ((int64_t)fc_.n_nodes() * Bp * 4 < ((int64_t)1 << 32))                                                   \
+      hipLaunchKernelGGL((kernel<EX_, W_, RUN_, true>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);         \
+    else                                                                                                        \
+      hipLaunchKernelGGL((kernel<EX_, W_, RUN_, false>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);        \
+  } while (0)
+
 #define SPARSE_DEV(B_, Bp_, xb_) \
   make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
-           d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats)
+           d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats, fc_.n_nodes())
 
 // input nodes grouped by variable
 void SparseCircuit::ensure_var_tables() {
@@ -1153,14 +1205,14 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
-    if (pairs < kSplitBelow)
-      hipLaunchKernelGGL((sparse_forward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, d, n0);
-    else if (layer_max_children_[l] > kNarrowDegree)
-      hipLaunchKernelGGL((sparse_forward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
-    else if (pairs < kManyPairs)
-      hipLaunchKernelGGL((sparse_forward_kernel<1, 1, 4>), dim3(cnt, Bp / 64), dim3(64), 0, stream, d, n0);
-    else
-      hipLaunchKernelGGL((sparse_forward_kernel<4, 1, 4>), dim3(cnt, ceil_div(Bp, 256)), dim3(64), 0, stream, d, n0);
+    if (layer_max_children_[l] <= kNarrowDegree) {
+      if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), d, n0);
+      else PCM_LAYER_LAUNCH(sparse_forward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), d, n0);
+    } else if (pairs < kSplitBelow) {
+      PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, kSplitWaves, kSplitRun, dim3(cnt, Bp / 64), d, n0);
+    } else {
+      PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, 1, kWideRun, dim3(cnt, Bp / 64), d, n0);
+    }
   }
   check_launch("sparse_forward");
   last_batch_ = batch;
@@ -1236,18 +1288,17 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
-    if (pairs < kSplitBelow)
-      hipLaunchKernelGGL((sparse_backward_kernel<1, kSplitWaves>), dim3(cnt, Bp / 64), dim3(kSplitWaves * 64), 0, stream, db, n0,
-                         d_heads_.p, d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
-    else if (bwd_layer_max_in_[l] > kNarrowDegree)
-      hipLaunchKernelGGL((sparse_backward_kernel<1, 1>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
-                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
-    else if (pairs < kManyPairs)
-      hipLaunchKernelGGL((sparse_backward_kernel<1, 1, 4>), dim3(cnt, Bp / 64), dim3(64), 0, stream, db, n0, d_heads_.p,
-                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
-    else   // (the rows of partial edge sums beyond a quarter stay as cleared)
-      hipLaunchKernelGGL((sparse_backward_kernel<4, 1, 4>), dim3(cnt, ceil_div(Bp, 256)), dim3(64), 0, stream, db, n0, d_heads_.p,
-                         d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p);
+#define PCM_BWD_ARGS db, n0, d_heads_.p, d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p
+    if (bwd_layer_max_in_[l] <= kNarrowDegree) {
+      if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
+      else   // (the rows of partial edge sums beyond a quarter stay as cleared)
+        PCM_LAYER_LAUNCH(sparse_backward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), PCM_BWD_ARGS);
+    } else if (pairs < kSplitBelow) {
+      PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, kSplitWaves, kSplitRun, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
+    } else {
+      PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, kWideRun, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
+    }
+#undef PCM_BWD_ARGS
   }
   if (ne)
     hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 64)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,
