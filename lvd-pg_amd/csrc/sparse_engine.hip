@@ -190,6 +190,9 @@ void FlatCircuit::finish() {
 struct SparseDev {
   const uint8_t* type;
   const int32_t* order;      // node ids sorted by layer
+  const int4* fwd_rec;       // per position of `order`: {node, type, first up edge, end of up edges}
+  const int4* bwd_rec;       // per position of the backward order: {node, seed index or -1, first in-edge, end of in-edges}
+  const int2* bwd_alias;     // ... and its range in the alias list
   const int32_t *node_e0, *node_e1, *e_parent, *e_prime, *e_sub, *in_var, *in_ptr, *in_edge;
   const int4* in_rec;        // per incoming edge: {edge << 1 | role, parent (~parent: product), prime, sub}
   const float* in_logp;      // ... and the edge's log-parameter, gathered before every backward pass
@@ -312,14 +315,15 @@ constexpr int kManyPairs = 16384;   // (node, 64 examples) pairs from which a na
 template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(SparseDev d, int n0) {
   __shared__ float xm[kLayerWaves][EX][64], xs[kLayerWaves][EX][64];
-  const int n = uni(d.order[n0 + blockIdx.x]);
+  const int4 rec = d.fwd_rec[n0 + blockIdx.x];   // one fetch instead of order -> type, edge range
+  const int n = uni(rec.x);
   const int lane = threadIdx.x & 63, wave = uni((int)(threadIdx.x >> 6));
   const int b0 = blockIdx.y * (64 * EX) + lane;
   int bb[EX];
 #pragma unroll
   for (int x = 0; x < EX; ++x) bb[x] = min(b0 + 64 * x, d.Bp - 1);
   float m[EX], sum[EX];
-  const int type = uni((int)d.type[n]);
+  const int type = uni(rec.y);
   if (type == kInput) {
     if (wave) return;
     if (d.ev) return;   // soft evidence: sparse_soft_input_kernel has filled the input rows
@@ -335,7 +339,7 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
     // running maximum and a sum of exponentials (products: a plain sum), the shares are then
     // combined through LDS by the first wave
     const bool issum = type == kSum;
-    const int e0 = uni(d.node_e0[n]), e1 = uni(d.node_e1[n]);
+    const int e0 = uni(rec.z), e1 = uni(rec.w);
     const int per = (e1 - e0 + kLayerWaves - 1) / kLayerWaves;
     const int my0 = min(e0 + wave * per, e1), my1 = min(my0 + per, e1);
 #pragma unroll
@@ -448,20 +452,20 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
 // edge_part ([gridDim.y][n_edges]), whose rows a later kernel adds up in order.
 template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
-                                                                           const int32_t* __restrict__ seed_of,
                                                                            const float* __restrict__ seed,
                                                                            float* __restrict__ edge_part_all, int64_t n_edges,
-                                                                           const int32_t* __restrict__ alias_ptr,
                                                                            const int32_t* __restrict__ alias_list) {
   __shared__ float xa[kLayerWaves][EX][64];
-  const int n = uni(d.order[n0 + blockIdx.x]);
+  const int4 rec = d.bwd_rec[n0 + blockIdx.x];   // one fetch instead of order -> seed, in-edge range
+  const int2 arec = d.bwd_alias[n0 + blockIdx.x];
+  const int n = uni(rec.x);
   const int lane = threadIdx.x & 63, wave = uni((int)(threadIdx.x >> 6));
   const int b0 = blockIdx.y * (64 * EX) + lane;
   float* edge_part = edge_part_all ? edge_part_all + (size_t)blockIdx.y * n_edges : nullptr;
   int bb[EX];
   bool live[EX];
   float acc[EX];
-  const int sd = uni(seed_of[n]);
+  const int sd = uni(rec.y);
 #pragma unroll
   for (int x = 0; x < EX; ++x) {
     const int b = b0 + 64 * x;
@@ -471,7 +475,7 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
     if (sd >= 0 && wave == 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
   }
   // the node's incoming edges in kLayerWaves contiguous shares, one per wave
-  const int i0 = uni(d.in_ptr[n]), i1 = uni(d.in_ptr[n + 1]);
+  const int i0 = uni(rec.z), i1 = uni(rec.w);
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
   const Rows<kBuf> mars(d.mars, d.n_nodes, d.Bp), flows(d.flows, d.n_nodes, d.Bp);
@@ -501,7 +505,7 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   }
   // input nodes that receive exactly this node's edge flows (the other factor of the same
   // two-child products) are not computed again: their rows are copies
-  for (int q = uni(alias_ptr[n]), q1 = uni(alias_ptr[n + 1]); q < q1; ++q) {
+  for (int q = uni(arec.x), q1 = uni(arec.y); q < q1; ++q) {
     const int t = uni(alias_list[q]);
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
@@ -997,6 +1001,14 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   d_in_rec_.upload(in_rec);
   d_type_.upload(fc_.type);
   d_order_.upload(order);
+  {
+    std::vector<int4> fr(nn);
+    for (int64_t i = 0; i < nn; ++i) {
+      const int32_t n = order[i];
+      fr[i] = int4{n, (int)fc_.type[n], fc_.node_e0[n], fc_.node_e1[n]};
+    }
+    d_fwd_rec_.upload(fr);
+  }
   d_node_e0_.upload(fc_.node_e0); d_node_e1_.upload(fc_.node_e1);
   auto up = [&](DevBuf<int32_t>& dst, std::vector<int32_t> v) { if (v.empty()) v.push_back(0); dst.upload(v); };
   up(d_e_parent_, fc_.e_parent); up(d_e_prime_, fc_.e_prime); up(d_e_sub_, fc_.e_sub);
@@ -1050,6 +1062,17 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   d_alias_ptr_.upload(alias_ptr);
   d_alias_list_.upload(alias_list);
   d_bwd_order_.upload(bwd_order);
+  {
+    std::vector<int4> br(std::max<size_t>(bwd_order.size(), 1), int4{0, -1, 0, 0});
+    std::vector<int2> ar(br.size(), int2{0, 0});
+    for (size_t i = 0; i < bwd_order.size(); ++i) {
+      const int32_t n = bwd_order[i];
+      br[i] = int4{n, seed_of[n], in_ptr[n], in_ptr[n + 1]};
+      ar[i] = int2{alias_ptr[n], alias_ptr[n + 1]};
+    }
+    d_bwd_rec_.upload(br);
+    d_bwd_alias_.upload(ar);
+  }
   // normalisation groups over the sum parameters
   std::vector<int32_t> gp(1, 0), p2e;
   for (int64_t s : fc_.pargroup_sizes) gp.push_back(gp.back() + (int32_t)s);
@@ -1145,8 +1168,10 @@ void SparseCircuit::ensure_batch(int batch) {
 static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32_t* e0, const int32_t* e1,
                           const int32_t* ep, const int32_t* epr, const int32_t* es, const int32_t* in_var,
                           const int32_t* in_ptr, const int32_t* in_edge, const int4* in_rec, const int64_t* in_off, const float* logp,
-                          const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C, int64_t n_nodes) {
+                          const float* leaf, const uint8_t* xb, float* mars, float* flows, int B, int Bp, int C, int64_t n_nodes,
+                          const int4* fwd_rec, const int4* bwd_rec, const int2* bwd_alias) {
   SparseDev d;
+  d.fwd_rec = fwd_rec; d.bwd_rec = bwd_rec; d.bwd_alias = bwd_alias;
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
   d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off;
   d.ev = nullptr; d.ev_se = d.ev_sv = d.ev_sc = 0; d.ev_idx = nullptr; d.logp = logp; d.leaf = leaf;
@@ -1165,7 +1190,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
 
 #define SPARSE_DEV(B_, Bp_, xb_) \
   make_dev(d_type_.p, d_order_.p, d_node_e0_.p, d_node_e1_.p, d_e_parent_.p, d_e_prime_.p, d_e_sub_.p, d_in_var_.p, \
-           d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats, fc_.n_nodes())
+           d_in_ptr_.p, d_in_edge_.p, d_in_rec_.p, d_in_off_.p, d_logp_.p, d_leaf_.p, xb_, d_mars_.p, d_flows_.p, B_, Bp_, fc_.num_cats, fc_.n_nodes(), d_fwd_rec_.p, d_bwd_rec_.p, d_bwd_alias_.p)
 
 // input nodes grouped by variable
 void SparseCircuit::ensure_var_tables() {
@@ -1288,7 +1313,7 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
-#define PCM_BWD_ARGS db, n0, d_heads_.p, d_head_mask, d_edge_part_.p, ne, d_alias_ptr_.p, d_alias_list_.p
+#define PCM_BWD_ARGS db, n0, d_head_mask, d_edge_part_.p, ne, d_alias_list_.p
     if (bwd_layer_max_in_[l] <= kNarrowDegree) {
       if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
       else   // (the rows of partial edge sums beyond a quarter stay as cleared)

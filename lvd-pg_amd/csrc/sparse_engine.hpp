@@ -111,6 +111,8 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<float> d_in_logp_, d_edge_part_;
   DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
+  DevBuf<int4> d_fwd_rec_, d_bwd_rec_;   // per position of the forward / backward order: node and its ranges in one record
+  DevBuf<int2> d_bwd_alias_;
   std::vector<int> layer_max_children_, bwd_layer_max_in_;   // per layer: most edges of a node going up / coming in
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
   DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
