@@ -1023,7 +1023,6 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   std::vector<int32_t> seed_of(nn, -1);
   if (fc_.heads.empty()) seed_of[nn - 1] = 0;
   else for (size_t h = 0; h < fc_.heads.size(); ++h) seed_of[fc_.heads[h]] = (int32_t)h;
-  d_heads_.upload(seed_of);
   if (!fc_.heads.empty()) d_head_nodes_.upload(fc_.heads);
   // An input node that is the second factor of two-child products and sees exactly the edges its
   // first factor (the prime) sees gets the same flow as the prime: it is dropped from the backward
@@ -1059,7 +1058,6 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
       }
     bwd_layer0_[l + 1] = (int)bwd_order.size();
   }
-  d_alias_ptr_.upload(alias_ptr);
   d_alias_list_.upload(alias_list);
   d_bwd_order_.upload(bwd_order);
   {

@@ -109,13 +109,13 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<int32_t> d_in_ptr_, d_in_edge_;
   DevBuf<int4> d_in_rec_;
   DevBuf<float> d_in_logp_, d_edge_part_;
-  DevBuf<int32_t> d_input_nodes_, d_alias_ptr_, d_alias_list_, d_bwd_order_;
+  DevBuf<int32_t> d_input_nodes_, d_alias_list_, d_bwd_order_;
   std::vector<int> bwd_layer0_;
   DevBuf<int4> d_fwd_rec_, d_bwd_rec_;   // per position of the forward / backward order: node and its ranges in one record
   DevBuf<int2> d_bwd_alias_;
   std::vector<int> layer_max_children_, bwd_layer_max_in_;   // per layer: most edges of a node going up / coming in
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
-  DevBuf<int32_t> d_heads_, d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
+  DevBuf<int32_t> d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;
   DevBuf<float> d_g1_, d_g2_, d_l1_, d_l2_;   // KL gradients in edge / leaf order
   int cap_batch_ = 0, last_batch_ = 0, max_var_nodes_ = 1;
