@@ -386,9 +386,8 @@ void HcltCircuit::build_schedules() {
   // A forest's trees are walked in groups side by side (blockIdx.y of the walk kernels): each group of whole trees
   // has a schedule of its own, so that a batch too small to fill the device with its slices (1024 examples are 64
   // workgroups) still does.  Groups are node ranges (post-order goes tree after tree) of about equal size.
-  std::vector<std::pair<int, int>> groups;
-  {
-    const int G = forest_ ? std::max(1, std::min(4, T_ / 8)) : 1;
+  auto make_groups = [&](int G) {
+    std::vector<std::pair<int, int>> gr;
     int n0 = 0;
     for (int g = 0; g < G && n0 < n_inner_; ++g) {
       // up to the end of the tree in which this group's share of the nodes is reached
@@ -396,10 +395,12 @@ void HcltCircuit::build_schedules() {
       int n1 = std::max(n0 + 1, want);
       while (n1 < n_inner_ && tree_of_inner_[n1] == tree_of_inner_[n1 - 1]) ++n1;
       if (g == G - 1) n1 = n_inner_;
-      groups.push_back({n0, n1});
+      gr.push_back({n0, n1});
       n0 = n1;
     }
-  }
+    return gr;
+  };
+  const std::vector<std::pair<int, int>> groups = make_groups(forest_ ? std::max(1, std::min(4, T_ / 8)) : 1);
   n_groups_ = (int)groups.size();
 
   // ---- forward -----------------------------------------------------------------------
@@ -482,6 +483,28 @@ void HcltCircuit::build_schedules() {
         ++done;
       }
     }
+  };
+  // The lean backward walk hands every inner child its own tile: a slot per (parent, inner child) pair, taken
+  // in the parent's step and free again from the step after the child's.  False if the slots run out.
+  auto assign_ratio_slots = [&](const std::vector<StepItem>& sched, std::vector<int32_t>& ratio_slot) {
+    const int g_steps = (int)sched.size() / kWalkWaves;
+    std::vector<int32_t> fs;
+    for (int sl = trash_slot - 1; sl >= 0; --sl) fs.push_back(sl);
+    for (int st = 0; st < g_steps; ++st) {
+      std::vector<int32_t> freed;
+      for (int w = 0; w < kWalkWaves; ++w) {
+        const int n = sched[(size_t)st * kWalkWaves + w].node;
+        if (n < 0) continue;
+        if (par[n] >= 0) freed.push_back(ratio_slot[n]);
+        for (int c : ic[n]) {
+          if (fs.empty()) return false;
+          ratio_slot[c] = fs.back();
+          fs.pop_back();
+        }
+      }
+      fs.insert(fs.end(), freed.begin(), freed.end());
+    }
+    return true;
   };
   auto pad_steps = [&](std::vector<StepItem>& sched, std::vector<PreItem>& pre, int steps) {
     while ((int)sched.size() < steps * kWalkWaves) { sched.push_back(blank(-1)); pre.push_back(blank_pre(-1)); }
@@ -582,30 +605,9 @@ void HcltCircuit::build_schedules() {
       schedule_backward(groups[g].first, groups[g].second, scheds[g], pres[g]);
       n_bwd_steps_ = std::max(n_bwd_steps_, (int)scheds[g].size() / kWalkWaves);
     }
-    // The lean backward walk hands every inner child its own tile: a slot per (parent, inner child) pair, taken
-    // in the parent's step and free again from the step after the child's.
     std::vector<int32_t> ratio_slot(n_inner_, -1);
     bool slots_ok = true;
-    for (int g = 0; g < n_groups_; ++g) {
-      const std::vector<StepItem>& sched = scheds[g];
-      const int g_steps = (int)sched.size() / kWalkWaves;
-      std::vector<int32_t> fs;
-      for (int sl = trash_slot - 1; sl >= 0; --sl) fs.push_back(sl);
-      for (int st = 0; st < g_steps && slots_ok; ++st) {
-        std::vector<int32_t> freed;
-        for (int w = 0; w < kWalkWaves && slots_ok; ++w) {
-          const int n = sched[(size_t)st * kWalkWaves + w].node;
-          if (n < 0) continue;
-          if (par[n] >= 0) freed.push_back(ratio_slot[n]);
-          for (int c : ic[n]) {
-            if (fs.empty()) { slots_ok = false; break; }
-            ratio_slot[c] = fs.back();
-            fs.pop_back();
-          }
-        }
-        fs.insert(fs.end(), freed.begin(), freed.end());
-      }
-    }
+    for (int g = 0; g < n_groups_ && slots_ok; ++g) slots_ok = assign_ratio_slots(scheds[g], ratio_slot);
     std::vector<int32_t> lean_rows;
     bwd_lean_ = slots_ok;
     for (int g = 0; g < n_groups_; ++g) {
@@ -616,6 +618,62 @@ void HcltCircuit::build_schedules() {
     }
     if (bwd_lean_) d_bwd_lean_.upload(lean_rows);
     d_bwd_sched_.upload(scheds[0]);
+  }
+  // ---- a forest's finer plans --------------------------------------------------------------
+  // The same walks with two and four times as many, smaller groups of trees, for batches whose slices times the
+  // groups above leave most of the device idle (256 examples are 16 slices): the walk then takes the plan with
+  // the most groups that still gives every workgroup a compute unit of its own.  A tree's arithmetic does not
+  // depend on the group it is walked in, so the results are the same bits under every plan.
+  fine_plans_.clear();
+  if (forest_ && fwd_lean_ && bwd_lean_) {
+    const bool keep_fwd_spill = fwd_spill_, keep_bwd_spill = bwd_spill_;
+    for (int G = 2 * n_groups_; G <= 4 * n_groups_ && G <= T_ / 4; G *= 2) {
+      const std::vector<std::pair<int, int>> gr = make_groups(G);
+      if ((int)gr.size() <= (fine_plans_.empty() ? n_groups_ : fine_plans_.back()->n_groups)) break;
+      std::unique_ptr<LeanPlan> plan(new LeanPlan);
+      plan->n_groups = (int)gr.size();
+      bool ok = true;
+      std::vector<int32_t> rows;
+      {
+        fwd_spill_ = false;
+        std::vector<std::vector<StepItem>> sched(gr.size());
+        std::vector<std::vector<PreItem>> pre(gr.size());
+        for (size_t g = 0; g < gr.size(); ++g) {
+          schedule_forward(gr[g].first, gr[g].second, sched[g], pre[g]);
+          plan->n_fwd_steps = std::max(plan->n_fwd_steps, (int)sched[g].size() / kWalkWaves);
+        }
+        ok = !fwd_spill_;
+        plan->fwd_stride = plan->n_fwd_steps + 64;
+        for (size_t g = 0; g < gr.size() && ok; ++g) {
+          pad_steps(sched[g], pre[g], plan->fwd_stride);
+          ok = make_lean(sched[g], true, plan->fwd_stride, rows);
+        }
+        if (ok) plan->fwd.upload(rows);
+      }
+      if (ok) {
+        bwd_spill_ = false;
+        std::vector<std::vector<StepItem>> sched(gr.size());
+        std::vector<std::vector<PreItem>> pre(gr.size());
+        for (size_t g = 0; g < gr.size(); ++g) {
+          schedule_backward(gr[g].first, gr[g].second, sched[g], pre[g]);
+          plan->n_bwd_steps = std::max(plan->n_bwd_steps, (int)sched[g].size() / kWalkWaves);
+        }
+        ok = !bwd_spill_;
+        std::vector<int32_t> ratio_slot(n_inner_, -1);
+        for (size_t g = 0; g < gr.size() && ok; ++g) ok = assign_ratio_slots(sched[g], ratio_slot);
+        plan->bwd_stride = plan->n_bwd_steps + 64;
+        rows.clear();
+        for (size_t g = 0; g < gr.size() && ok; ++g) {
+          pad_steps(sched[g], pre[g], plan->bwd_stride);
+          ok = make_lean(sched[g], false, plan->bwd_stride, rows, &ratio_slot);
+        }
+        if (ok) plan->bwd.upload(rows);
+      }
+      if (!ok) break;
+      fine_plans_.push_back(std::move(plan));
+    }
+    fwd_spill_ = keep_fwd_spill;
+    bwd_spill_ = keep_bwd_spill;
   }
   // ---- statistics: the static operands of every node ------------------------------------
   {
@@ -678,6 +736,10 @@ void HcltCircuit::build_schedules() {
             "%d LDS slots\n",
             V_, K_, C_, n_inner_, T_, n_groups_, n_fwd_steps_, fwd_spill_ ? " (spills)" : "", fwd_lean_ ? " (lean)" : "", n_bwd_steps_,
             bwd_spill_ ? " (spills)" : "", bwd_lean_ ? " (lean)" : "", stat_lean_ ? " (lean)" : "", lds_slots_);
+  if (getenv("PCM_VERBOSE"))
+    for (const auto& p : fine_plans_)
+      fprintf(stderr, "[pcmi355]   finer plan: %d groups, forward %d steps, backward %d steps\n", p->n_groups, p->n_fwd_steps,
+              p->n_bwd_steps);
 }
 
 // Numbering the reference would give this circuit.  Nodes are created in depth-first
@@ -1221,6 +1283,15 @@ void HcltCircuit::stage_batch(const BatchRef& b) {
   check_launch("pack_x");
 }
 
+// The finer plan a batch of `nslices` slices walks a forest with, or null for the plan of the constructor: the
+// most groups whose workgroups still get a compute unit each.
+const HcltCircuit::LeanPlan* HcltCircuit::fine_plan(int nslices) const {
+  const LeanPlan* best = nullptr;
+  for (const auto& p : fine_plans_)
+    if ((int64_t)nslices * p->n_groups <= n_cus_) best = p.get();
+  return best;
+}
+
 void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
   const size_t lds = (size_t)lds_slots_ * kSlice * K_ * sizeof(float);
   auto launch = [&](auto kernel) {
@@ -1235,8 +1306,13 @@ void HcltCircuit::run_forward(const HcltDev& d, float* d_ll) {
     PCM_DISPATCH_LEAN_K(K_, {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_forward_lean_kernel<KK>),
                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d,
-                       d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
+      const LeanPlan* fp = fine_plan(d.nslices);
+      if (fp)
+        PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices, fp->n_groups), dim3(kWalkWaves * 64), lean_lds, d,
+                         fp->fwd.p, fp->fwd_stride, fp->n_fwd_steps, d_ll, lds_slots_);
+      else
+        PCM_LAUNCH_PHASE(0, hclt_forward_lean_kernel<KK>, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d,
+                         d_fwd_lean_.p, fwd_stride_, n_fwd_steps_, d_ll, lds_slots_);
     });
   } else {
     PCM_DISPATCH_K(K_, {
@@ -1258,8 +1334,13 @@ void HcltCircuit::run_backward(const HcltDev& d) {
     const size_t lean_lds = lds + kLeanFlagWords * 4;
     auto launch_lean = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lean_lds));
-      PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d, d_bwd_lean_.p, bwd_stride_,
-                       n_bwd_steps_, lds_slots_);
+      const LeanPlan* fp = fine_plan(d.nslices);
+      if (fp)
+        PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices, fp->n_groups), dim3(kWalkWaves * 64), lean_lds, d, fp->bwd.p,
+                         fp->bwd_stride, fp->n_bwd_steps, lds_slots_);
+      else
+        PCM_LAUNCH_PHASE(1, kernel, dim3(d.nslices, n_groups_), dim3(kWalkWaves * 64), lean_lds, d, d_bwd_lean_.p, bwd_stride_,
+                         n_bwd_steps_, lds_slots_);
     };
     PCM_DISPATCH_LEAN_K(K_, {
       if (H_ > 0) launch_lean(&hclt_backward_lean_kernel<KK, true>); else launch_lean(&hclt_backward_lean_kernel<KK, false>);

@@ -210,6 +210,13 @@ class HcltCircuit : public pcm_circuit {
   bool forest_ = false;
   int T_ = 1;                      // trees (1 unless a forest)
   int n_groups_ = 1;               // groups of trees the walk kernels take side by side (blockIdx.y)
+  // a forest's walk schedules with more, smaller groups of trees, for batches whose slices do not fill the device
+  struct LeanPlan {
+    int n_groups = 1, n_fwd_steps = 0, fwd_stride = 0, n_bwd_steps = 0, bwd_stride = 0;
+    DevBuf<int32_t> fwd, bwd;
+  };
+  std::vector<std::unique_ptr<LeanPlan>> fine_plans_;
+  const LeanPlan* fine_plan(int nslices) const;
   std::vector<int32_t> roots_;     // root variable of every tree, in variable order
   std::vector<int32_t> tree_of_inner_;   // tree of every inner node
   // inner nodes of the caller's tree, and every node's index among them (auxiliary nodes keep the post-order of the
