@@ -304,12 +304,15 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, const Rows<kBuf>
 //   * otherwise, below kSplitBelow pairs: kSplitWaves waves share a node's edges (the layer cannot fill the
 //     device with one wave per pair, and a wave's chain of round trips gets shorter);
 //   * otherwise one wave per pair, runs of up to kWideRun edges requested at once (16: seven waves per SIMD;
-//     32 halves the waves and is slower, 8 leaves too few requests in flight).
+//     32 halves the waves and is slower, 8 leaves too few requests in flight); from kSaturated pairs on, where the
+//     device is full whatever the shape of a wave, two examples per lane and runs of 8, which halves the index
+//     work per example (16 circuits of that kind compiled as one: 5.47 -> 5.17 ms per step).
 constexpr int kSplitWaves = 4;
 constexpr int kSplitRun = 16;       // longest run in the kernels that split a node over kSplitWaves waves
 constexpr int kSplitBelow = 8192;   // (node, 64 examples) pairs in a layer below which its nodes are split
 constexpr int kNarrowDegree = 8;    // a layer whose nodes have at most this many edges takes the kMaxRun = 4 kernels
 constexpr int kWideRun = 16;        // longest run of edges requested at once in the one-wave kernels
+constexpr int kSaturated = 32768;   // pairs from which a many-edged layer takes two examples per lane and runs of 8
 constexpr int kManyPairs = 16384;   // (node, 64 examples) pairs from which a narrow layer takes four examples per lane
 
 template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
@@ -350,6 +353,8 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
       for (; c0 + 32 <= my1; c0 += 32) forward_run<32, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     if constexpr (kMaxRun >= 16)
       for (; c0 + 16 <= my1; c0 += 16) forward_run<16, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
+    if constexpr (kMaxRun == 8)
+      for (; c0 + 8 <= my1; c0 += 8) forward_run<8, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     for (; c0 + 4 <= my1; c0 += 4) forward_run<4, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     for (; c0 < my1; ++c0) forward_run<1, EX, kBuf>(d, mars, issum, c0, bb, m, sum);
     if (e1 - e0 > per) {   // more than one share is in use (uniform over the workgroup)
@@ -404,6 +409,56 @@ __device__ __forceinline__ float wave_sum(float v) {
          __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
 }
 
+// The sums over the wave of U values at once (a run's edge flows): each of the first log2(U) pairings of lanes
+// (lane ^ 32, lane ^ 16, mirror of 16, mirror of 8) adds partners and halves the values a lane carries -- one
+// partner keeps the lower half of the values, the other the upper half -- and the remaining pairings add without
+// halving, as wave_sum does.  Afterwards lane l holds the total of value (l >> kShift) & (U - 1), kShift =
+// 6 - log2(U): about 40 instructions for 16 sums where one wave_sum per edge takes 190.
+template <int U>
+struct EdgeTotals {
+  static_assert(U == 16 || U == 8 || U == 4, "runs of 16, 8 or 4 edges");
+  static constexpr int kShift = U == 16 ? 2 : U == 8 ? 3 : 4;
+  template <int CTRL>
+  static __device__ __forceinline__ float dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+  }
+  // lanes with `upper` keep b's sum over the pair, the others a's; CTRL names the pairing inside a row of 16
+  template <int CTRL>
+  static __device__ __forceinline__ float halve(float a, float b, bool upper) {
+    const float keep = upper ? b : a, send = upper ? a : b;
+    return keep + dpp<CTRL>(send);
+  }
+  static __device__ __forceinline__ float run(float (&v)[U], int lane) {
+    float w8[U / 2];
+#pragma unroll
+    for (int i = 0; i < U / 2; ++i) {   // lane ^ 32
+      const auto r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(int, v[i]), __builtin_bit_cast(int, v[i + U / 2]), false, false);
+      w8[i] = __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+    }
+    float w4[U / 4];
+#pragma unroll
+    for (int i = 0; i < U / 4; ++i) {   // lane ^ 16
+      const auto r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(int, w8[i]), __builtin_bit_cast(int, w8[i + U / 4]), false, false);
+      w4[i] = __builtin_bit_cast(float, (int)r[0]) + __builtin_bit_cast(float, (int)r[1]);
+    }
+    float t;
+    if constexpr (U == 16) {
+      const float a = halve<0x140>(w4[0], w4[2], lane & 8), b = halve<0x140>(w4[1], w4[3], lane & 8);   // row_mirror
+      t = halve<0x141>(a, b, lane & 4);                                                                  // row_half_mirror
+    } else if constexpr (U == 8) {
+      t = halve<0x140>(w4[0], w4[1], lane & 8);
+      t += dpp<0x141>(t);
+    } else {
+      t = w4[0];
+      t += dpp<0x140>(t);
+      t += dpp<0x141>(t);
+    }
+    t += dpp<0x4E>(t);   // quad_perm [2,3,0,1]
+    t += dpp<0xB1>(t);   // quad_perm [1,0,3,2]
+    return t;
+  }
+};
+
 template <int U, int EX, bool kBuf>
 __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf>& mars, const Rows<kBuf>& flows, int c0,
                                              const int (&bb)[EX], const bool (&live)[EX], float (&acc)[EX],
@@ -426,21 +481,33 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
       ex[u][x] = keep_bits(mars.at(pr, bb[x]) + lp + keep_bits(mars.at(max(s, 0), bb[x]), has_sub) - mars.at(p, bb[x]), sum_edge);
     }
   }
+  float part[U];
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    float part = 0.f;
+    part[u] = 0.f;
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
       float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * expf(ex[u][x]);   // product edges carry exponent 0
       // no flow stays no flow where the parent's value is -inf (an example of probability zero: -inf - -inf)
       if (!live[x] || ex[u][x] != ex[u][x]) ef = 0.f;
       acc[x] += ef;
-      part += ef;
+      part[u] += ef;
     }
-    if (!(ies[u] & 1) && edge_part) {
-      const float tot = wave_sum(part);
-      if ((threadIdx.x & 63) == 0) edge_part[ies[u] >> 1] = tot;   // this wave is the only writer of the cell
-    }
+  }
+  if (!edge_part) return;
+  if constexpr (U >= 4 && U <= 16) {
+    // all the run's sums at once; lane l ends up with the total of edge (l >> kShift) % U, whose record it reads itself
+    const int lane = threadIdx.x & 63;
+    const int mine = d.in_rec[c0 + ((lane >> EdgeTotals<U>::kShift) & (U - 1))].x;
+    const float tot = EdgeTotals<U>::run(part, lane);
+    if (!(lane & ((1 << EdgeTotals<U>::kShift) - 1)) && !(mine & 1)) edge_part[mine >> 1] = tot;   // this wave is the only writer of the cell
+  } else {
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (!(ies[u] & 1)) {
+        const float tot = wave_sum(part[u]);
+        if ((threadIdx.x & 63) == 0) edge_part[ies[u] >> 1] = tot;
+      }
   }
 }
 
@@ -484,6 +551,8 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
     for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   if constexpr (kMaxRun >= 16)
     for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+  if constexpr (kMaxRun == 8)
+    for (; c0 + 8 <= my1; c0 += 8) backward_run<8, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   for (; c0 < my1; ++c0) backward_run<1, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
@@ -1233,8 +1302,10 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
       else PCM_LAYER_LAUNCH(sparse_forward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), d, n0);
     } else if (pairs < kSplitBelow) {
       PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, kSplitWaves, kSplitRun, dim3(cnt, Bp / 64), d, n0);
-    } else {
+    } else if (pairs < kSaturated) {
       PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, 1, kWideRun, dim3(cnt, Bp / 64), d, n0);
+    } else {
+      PCM_LAYER_LAUNCH(sparse_forward_kernel, 2, 1, 8, dim3(cnt, ceil_div(Bp, 128)), d, n0);
     }
   }
   check_launch("sparse_forward");
@@ -1318,8 +1389,10 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
         PCM_LAYER_LAUNCH(sparse_backward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), PCM_BWD_ARGS);
     } else if (pairs < kSplitBelow) {
       PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, kSplitWaves, kSplitRun, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
-    } else {
+    } else if (pairs < kSaturated) {
       PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, kWideRun, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
+    } else {
+      PCM_LAYER_LAUNCH(sparse_backward_kernel, 2, 1, 8, dim3(cnt, ceil_div(Bp, 128)), PCM_BWD_ARGS);
     }
 #undef PCM_BWD_ARGS
   }

@@ -113,6 +113,35 @@ def test_random_dag_em_step_on_a_large_batch(gpu, oracle):
     _check_em_step(gpu, oracle, root, 12, 5, 16000, seed=77)
 
 
+def test_layered_engine_on_a_batch_that_saturates_the_device(gpu, oracle):
+    """Layers of many-edged nodes with at least 32768 (node, 64 examples) pairs take two examples per lane: an HCLT
+    with K = 32 compiled as a general circuit, 8192 examples, against the block engine on the same tree and
+    parameters (itself checked against the oracle elsewhere) and against the oracle on the head of the batch."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, describe_dag, rel_err
+    V, K, C, B = 30, 32, 16, 8192
+    rng = np.random.default_rng(31)
+    parent = np.full(V, -1, np.int32)
+    for v in range(1, V):
+        parent[v] = rng.integers(max(0, v - 4), v)
+    parent, theta, leaf, fc = make_hclt(V, K, C, 31, parent=parent)
+    a = P.hclt_from_clt(parent, C, K)
+    a.set_params(block_theta(parent, K, theta), leaf)
+    d = describe_dag([O.hclt_dag(parent, K, C, theta, leaf)])
+    g = P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"], d["input_logp"], V, C)
+    np.testing.assert_allclose(P.vectorize_parameters(a), P.vectorize_parameters(g), atol=1e-6)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    dd = torch.from_numpy(data).cuda()
+    la, lg = P.loglikelihoods(a, dd).cpu().numpy(), P.loglikelihoods(g, dd).cpu().numpy()
+    assert rel_err(lg, la).max() < LL_RTOL
+    assert rel_err(lg[:64], O.forward(fc, data[:64])[-1]).max() < LL_RTOL
+    for c in (a, g):
+        P.mini_batch_em(c, dd, 1, batch_size=B, pseudocount=0.1, param_inertia=0.3)
+    pa, pg = P.vectorize_parameters(a), P.vectorize_parameters(g)
+    assert rel_err(np.exp(pg), np.exp(pa)).max() < PARAM_RTOL
+
+
 def test_example_ids_and_flow_memory(gpu, oracle):
     """Batches picked by example ids; accumulators scaled by `rate` before a batch
     (src/regularization/reg_em.jl:276-284)."""
