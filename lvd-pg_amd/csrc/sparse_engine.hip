@@ -238,8 +238,8 @@ __device__ __forceinline__ float uni(float v) {
 
 // The rows of the value and flow arrays, addressed the way the layer kernels need them: one descriptor per
 // array in scalar registers, the row as a scalar byte offset, the example as the lane's byte offset -- a row
-// costs one scalar register instead of a 64-bit address.  kBuf = false (arrays of 4 GiB or more, beyond a
-// descriptor's range) keeps plain pointers.
+// costs one scalar register instead of a 64-bit address.  kBuf = false (arrays of 2 GiB or more, beyond a
+// signed 32-bit row offset) keeps plain pointers.
 template <bool kBuf>
 struct Rows {
   const float* base;
@@ -1246,10 +1246,11 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
   return d;
 }
 
-// a layer kernel with rows through buffer descriptors where the value / flow arrays are within a descriptor's 4 GiB
+// a layer kernel with rows through buffer descriptors where the value / flow arrays stay below 2 GiB (row offsets are
+// signed 32-bit scalars)
 #define PCM_LAYER_LAUNCH(kernel, EX_, W_, RUN_, grid, ...)                                                      \
   do {                                                                                                          \
-    if ((int64_t)fc_.n_nodes() * Bp * 4 < ((int64_t)1 << 32))                                                   \
+    if ((int64_t)fc_.n_nodes() * Bp * 4 < ((int64_t)1 << 31))                                                   \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, true>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);         \
     else                                                                                                        \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, false>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);        \
