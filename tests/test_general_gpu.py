@@ -142,6 +142,44 @@ def test_layered_engine_on_a_batch_that_saturates_the_device(gpu, oracle):
     assert rel_err(np.exp(pg), np.exp(pa)).max() < PARAM_RTOL
 
 
+def test_layered_engine_with_value_arrays_beyond_two_gigabytes(gpu, oracle):
+    """From 2 GiB of node values on, the layer kernels address rows through pointers instead of buffer descriptors:
+    a circuit of about 7900 nodes (K = 32 HCLT over 128 variables) on 73728 examples, 96 copies of 768 distinct ones.  The
+    likelihood of a copy is that of its original in a 768-example batch (the descriptor path) and the same bits in
+    every copy, and with no
+    pseudocount the EM update of the large batch is the update of the small one up to rounding."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, describe_dag, rel_err
+    V, K, C, base, copies = 128, 32, 6, 768, 96
+    rng = np.random.default_rng(41)
+    parent = np.full(V, -1, np.int32)
+    for v in range(1, V):
+        parent[v] = rng.integers(max(0, v - 3), v)
+    parent, theta, leaf, fc = make_hclt(V, K, C, 41, parent=parent)
+    d = describe_dag([O.hclt_dag(parent, K, C, theta, leaf)])
+
+    def compiled():
+        return P.compile_circuit(d["node_type"], d["child_ptr"], d["child_idx"], d["sum_logp"], d["input_var"],
+                                 d["input_logp"], V, C)
+    small, large = compiled(), compiled()
+    assert small.num_nodes() * base * 4 < 2 ** 31 <= large.num_nodes() * base * copies * 4
+    data = rng.integers(0, C, size=(base, V)).astype(np.uint8)
+    ds = torch.from_numpy(data).cuda()
+    dl = torch.from_numpy(np.tile(data, (copies, 1))).cuda()
+    ll_s = P.loglikelihoods(small, ds).cpu().numpy()
+    assert rel_err(ll_s[:32], O.forward(fc, data[:32])[-1]).max() < LL_RTOL
+    ll_l = P.loglikelihoods(large, dl).cpu().numpy().reshape(copies, base)
+    # (which build of the layer kernels a layer takes depends on the batch, and they fold a node's edges in
+    # different groupings: equal to rounding, not to the bit)
+    np.testing.assert_allclose(ll_l, np.broadcast_to(ll_s, (copies, base)), rtol=2e-6)
+    np.testing.assert_array_equal(ll_l, np.broadcast_to(ll_l[0], (copies, base)))   # a copy is a copy
+    P.mini_batch_em(small, ds, 1, batch_size=base, pseudocount=0.0, param_inertia=0.0)
+    P.mini_batch_em(large, dl, 1, batch_size=base * copies, pseudocount=0.0, param_inertia=0.0)
+    ps, pl = np.exp(P.vectorize_parameters(small)), np.exp(P.vectorize_parameters(large))
+    assert np.abs(pl - ps).max() < 2e-5
+
+
 def test_example_ids_and_flow_memory(gpu, oracle):
     """Batches picked by example ids; accumulators scaled by `rate` before a batch
     (src/regularization/reg_em.jl:276-284)."""
