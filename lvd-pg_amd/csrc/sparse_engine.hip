@@ -272,20 +272,27 @@ __device__ __forceinline__ void forward_run(const SparseDev& d, const Rows<kBuf>
 #pragma unroll
     for (int x = 0; x < EX; ++x) child[u][x] = mars.at(pr, bb[x]) + keep_bits(mars.at(max(s, 0), bb[x]), has_sub) + lp;
   }
+  // a run is folded in two passes: its maximum first, then one exponential per edge relative to the larger of
+  // that and the maximum so far (the sum so far is rescaled once per run)
 #pragma unroll
-  for (int u = 0; u < U; ++u)
+  for (int x = 0; x < EX; ++x) {
+    if (!issum) {
 #pragma unroll
-    for (int x = 0; x < EX; ++x) {
-      const float c = child[u][x];
-      if (!issum) {
-        m[x] += c;
-      } else if (c > m[x]) {
-        sum[x] = sum[x] * __expf(m[x] - c) + 1.f;
-        m[x] = c;
-      } else if (c != -INFINITY) {
-        sum[x] += __expf(c - m[x]);
+      for (int u = 0; u < U; ++u) m[x] += child[u][x];
+    } else {
+      float mr = child[0][x];
+#pragma unroll
+      for (int u = 1; u < U; ++u) mr = fmaxf(mr, child[u][x]);
+      const float mn = fmaxf(m[x], mr);
+      if (mn != -INFINITY) {
+        float s = sum[x] * __expf(m[x] - mn);
+#pragma unroll
+        for (int u = 0; u < U; ++u) s += __expf(child[u][x] - mn);
+        sum[x] = s;
+        m[x] = mn;
       }
     }
+  }
 }
 
 // Forward, one layer: a workgroup takes one node of the layer and 64 * EX examples (lane t:
