@@ -494,7 +494,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
     part[u] = 0.f;
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
-      float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * expf(ex[u][x]);   // product edges carry exponent 0
+      float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * __expf(ex[u][x]);   // product edges carry exponent 0
       // no flow stays no flow where the parent's value is -inf (an example of probability zero: -inf - -inf)
       if (!live[x] || ex[u][x] != ex[u][x]) ef = 0.f;
       acc[x] += ef;
