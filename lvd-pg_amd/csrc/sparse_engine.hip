@@ -468,8 +468,9 @@ struct EdgeTotals {
 
 template <int U, int EX, bool kBuf>
 __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf>& mars, const Rows<kBuf>& flows, int c0,
-                                             const int (&bb)[EX], const bool (&live)[EX], float (&acc)[EX],
+                                             const int (&bb)[EX], const unsigned (&alive)[EX], float (&acc)[EX],
                                              float* __restrict__ edge_part) {
+  const int zrow = (int)d.n_nodes;
   float fl[U][EX], ex[U][EX];
   int ies[U];
 #pragma unroll
@@ -479,13 +480,13 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
     const int ry = uni(rec.y);
     const bool issum = ry >= 0;
     const int p = issum ? ry : ~ry;
-    const int s = uni(rec.w), pr = uni(rec.z);
-    const float lp = uni(d.in_logp[c0 + u]);
-    const unsigned has_sub = s >= 0 ? ~0u : 0u, sum_edge = issum ? ~0u : 0u;
+    const int s = uni(rec.w), pr = uni(rec.z);    // (the row of zeros where the edge has no such operand)
+    const int mrow = issum ? p : zrow;
+    const float lp = uni(d.in_logp[c0 + u]);      // 0 on product edges
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
-      fl[u][x] = flows.at(p, bb[x]);
-      ex[u][x] = keep_bits(mars.at(pr, bb[x]) + lp + keep_bits(mars.at(max(s, 0), bb[x]), has_sub) - mars.at(p, bb[x]), sum_edge);
+      fl[u][x] = keep_bits(flows.at(p, bb[x]), alive[x]);   // a lane past the padded batch repeats its last example
+      ex[u][x] = mars.at(pr, bb[x]) + lp + mars.at(s, bb[x]) - mars.at(mrow, bb[x]);
     }
   }
   float part[U];
@@ -494,9 +495,11 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
     part[u] = 0.f;
 #pragma unroll
     for (int x = 0; x < EX; ++x) {
-      float ef = ex[u][x] == 0.f ? fl[u][x] : fl[u][x] * __expf(ex[u][x]);   // product edges carry exponent 0
+      // (product edges carry exponent 0 and exp2(0) is 1; lanes between the batch and its padding carry flow 0
+      // from the seeds on)
+      float ef = fl[u][x] * __expf(ex[u][x]);
       // no flow stays no flow where the parent's value is -inf (an example of probability zero: -inf - -inf)
-      if (!live[x] || ex[u][x] != ex[u][x]) ef = 0.f;
+      if (ex[u][x] != ex[u][x]) ef = 0.f;
       acc[x] += ef;
       part[u] += ef;
     }
@@ -538,30 +541,32 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   float* edge_part = edge_part_all ? edge_part_all + (size_t)blockIdx.y * n_edges : nullptr;
   int bb[EX];
   bool live[EX];
+  unsigned alive[EX];   // all ones for the lanes inside the padded batch
   float acc[EX];
   const int sd = uni(rec.y);
 #pragma unroll
   for (int x = 0; x < EX; ++x) {
     const int b = b0 + 64 * x;
     live[x] = b < d.B;
+    alive[x] = b < d.Bp ? ~0u : 0u;
     bb[x] = min(b, d.Bp - 1);
     acc[x] = 0.f;
-    if (sd >= 0 && wave == 0) acc[x] = seed ? seed[(size_t)sd * d.B + min(b, d.B - 1)] : 1.f;
+    if (sd >= 0 && wave == 0 && live[x]) acc[x] = seed ? seed[(size_t)sd * d.B + b] : 1.f;   // no flow past the batch
   }
   // the node's incoming edges in kLayerWaves contiguous shares, one per wave
   const int i0 = uni(rec.z), i1 = uni(rec.w);
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
-  const Rows<kBuf> mars(d.mars, d.n_nodes, d.Bp), flows(d.flows, d.n_nodes, d.Bp);
+  const Rows<kBuf> mars(d.mars, d.n_nodes + 1, d.Bp), flows(d.flows, d.n_nodes, d.Bp);
   int c0 = my0;
   if constexpr (kMaxRun >= 32)
-    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if constexpr (kMaxRun >= 16)
-    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if constexpr (kMaxRun == 8)
-    for (; c0 + 8 <= my1; c0 += 8) backward_run<8, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
-  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
-  for (; c0 < my1; ++c0) backward_run<1, EX, kBuf>(d, mars, flows, c0, bb, live, acc, edge_part);
+    for (; c0 + 8 <= my1; c0 += 8) backward_run<8, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
+  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
+  for (; c0 < my1; ++c0) backward_run<1, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
 #pragma unroll
     for (int x = 0; x < EX; ++x) xa[wave][x][lane] = acc[x];
@@ -1072,7 +1077,12 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   std::vector<int4> in_rec(in_edge.size());
   for (size_t i = 0; i < in_edge.size() && ne; ++i) {
     const int32_t e = in_edge[i] >> 1, p = fc_.e_parent[e];
-    in_rec[i] = int4{in_edge[i], fc_.type[p] == kSum ? p : ~p, fc_.e_prime[e], fc_.e_sub[e]};
+    // operands an edge does not have name the row of zeros behind the last node's: the flow through a product
+    // edge is its parent's (exponent 0 - 0 + 0 - 0), a sum edge without a second child adds 0
+    const bool sum_edge = fc_.type[p] == kSum;
+    const int32_t zrow = (int32_t)nn;
+    in_rec[i] = int4{in_edge[i], sum_edge ? p : ~p, sum_edge ? fc_.e_prime[e] : zrow,
+                     sum_edge && fc_.e_sub[e] >= 0 ? fc_.e_sub[e] : zrow};
   }
   d_in_rec_.upload(in_rec);
   d_type_.upload(fc_.type);
@@ -1234,7 +1244,7 @@ void SparseCircuit::update_parameters(const float* in, int64_t n) {
 void SparseCircuit::ensure_batch(int batch) {
   if (batch <= cap_batch_) return;
   const int Bp = ceil_div(batch, 64) * 64;
-  d_mars_.alloc((size_t)fc_.n_nodes() * Bp);
+  d_mars_.alloc((size_t)(fc_.n_nodes() + 1) * Bp);   // one more row, of zeros: the operand an edge does not have
   d_flows_.alloc((size_t)fc_.n_nodes() * Bp);
   cap_batch_ = Bp;
 }
@@ -1257,7 +1267,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
 // signed 32-bit scalars)
 #define PCM_LAYER_LAUNCH(kernel, EX_, W_, RUN_, grid, ...)                                                      \
   do {                                                                                                          \
-    if ((int64_t)fc_.n_nodes() * Bp * 4 < ((int64_t)1 << 31))                                                   \
+    if ((int64_t)(fc_.n_nodes() + 1) * Bp * 4 < ((int64_t)1 << 31))                                             \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, true>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);         \
     else                                                                                                        \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, false>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);        \
@@ -1296,6 +1306,9 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
     check_launch("stage_batch");
   }
   SparseDev d = SPARSE_DEV(batch, Bp, xb);
+  // the row of zeros sits behind the last node's row at this batch's row length (a smaller batch than the
+  // arrays were sized for finds old values there)
+  PCM_HIP(hipMemsetAsync(d_mars_.p + (size_t)fc_.n_nodes() * Bp, 0, (size_t)Bp * sizeof(float), stream));
   if (s) {
     d.ev = s->d_ev; d.ev_se = s->stride_ex; d.ev_sv = s->stride_var; d.ev_sc = s->stride_cat; d.ev_idx = s->d_idx;
     ensure_var_tables();
