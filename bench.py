@@ -256,6 +256,40 @@ def secondary(args):
                    value=NC * B / dt, unit="examples/s",
                    config={"workload": args.workload, "circuits": NC, "streams": NS, "num_vars": V, "hidden": K,
                            "categories": C, "heads": H, "batch": B})
+    elif args.workload == "c4_patch_x16_as_one":
+        # sixteen patch circuits over sixteen blocks of 192 variables compiled as ONE multi-head circuit (2048 heads):
+        # every layer launch then carries the nodes of all sixteen, which is the layered engine with the device full
+        from pcmi355 import nodes as N
+        V, K, C, H, B, NC = 192, 32, 256, 128, 1024, 16
+        data = workloads.grf_images(B, 8, 8, 3, 3.0, 0.8, seed=1004)
+        parent = workloads.chow_liu_parent(data)
+        heads = []
+        for c in range(NC):
+            hs = _patch_heads(P, parent, K, C, H, rng)
+            for n in N.linearize(hs):
+                if n.kind == N.INPUT:
+                    n.var += c * V
+            heads += hs
+        bpc = P.CuMultiHeadBitsProbCircuit(heads, NC * V)
+        mask = np.zeros((NC * H, B), np.float32)
+        for c in range(NC):
+            mask[c * H + rng.integers(0, H, size=B), np.arange(B)] = 1.0
+        d = torch.from_numpy(np.tile(data, (1, NC))).cuda()
+        hm = torch.from_numpy(mask).cuda()
+        ll = torch.empty(B, device="cuda")
+
+        def step():
+            check(lib.pcm_flows(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, hm.data_ptr(), ll.data_ptr()))
+            check(lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+        dt = _timed(torch, step, args.steps, args.warmup)
+        nn, ne = bpc.num_nodes(), bpc.num_edges()
+        algo = B * (8 * nn + 24 * ne)
+        note = REQUESTED_NOTE
+        out.update(metric="examples/sec fwd+bwd+EM over 16 192-var K=32 128-head patch circuits compiled as one circuit "
+                          "(layered engine); an example counts once per circuit",
+                   value=NC * B / dt, unit="examples/s",
+                   config={"workload": args.workload, "circuits": NC, "num_vars": V, "hidden": K, "categories": C,
+                           "heads": H, "batch": B, "nodes": nn, "edges": ne})
     elif args.workload in ("c4_full", "c4_full_handles"):
         # C4 as a whole: 64 x 64 x 3 images cut into 64 patches of 8 x 8 x 3; one 192-variable K = 32 circuit with 128
         # cluster heads per patch and the K = 64 top-level HCLT over the 64 cluster ids.  c4_full: the 64 patch
