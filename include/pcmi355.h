@@ -197,11 +197,16 @@ int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex,
  * (src/regularization/reg_flow.jl:276-282) == `probs_flows_circuit`
  * (src/queries/flow.jl:228-234).  The circuit's edge_aggr and leaf flow accumulators are
  * first scaled by `rate` (0 clears them; src/regularization/reg_em.jl:276-284) and then
- * receive this batch.  d_head_mask (multi-head circuits only, else NULL) is
+ * receive this batch.  d_head_mask (multi-head circuits, else NULL) is
  * [num_heads][batch] and seeds the head flows (src-jl/multi_head_pc/flow.jl:141-176);
  * d_ll_out then receives `batch` floats, the mask-weighted mixture
  * logsumexp_h(mars[head_h] + log mask_h) - log sum_h mask_h
  * (src-jl/multi_head_pc/likelihood.jl:3-12).
+ * Per-example weights (the `weights` of reg_flow.jl:38-39,190-191, which multiply an example's edge and
+ * leaf flows): every flow is linear in the flow its example starts with, so for a multi-head circuit they
+ * are a factor of the mask's column, and a single-root circuit made by pcm_circuit_create takes them as a
+ * mask [1][batch]; d_ll_out is not weighted.  Single-head circuits of pcm_hclt_create take no mask
+ * (PCM_ERR_UNSUPPORTED).
  */
 int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
               const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask,

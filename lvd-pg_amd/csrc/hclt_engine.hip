@@ -1469,7 +1469,9 @@ void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
   no_forest("soft evidence");
   no_missing("soft evidence");
-  if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (H_ == 0 && d_head_mask)
+    fail(PCM_ERR_UNSUPPORTED, "per-example weights (a mask for a single-head circuit) need a circuit compiled with "
+                              "pcm_circuit_create or a multi-head circuit");
   if (soft_block_ok()) {
     if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
     if (flows_in_general_ && rate != 0.f) fail(PCM_ERR_STATE, "flow memory cannot carry over from the layered engine");
@@ -1525,7 +1527,9 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
 }
 
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
-  if (H_ == 0 && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  if (H_ == 0 && d_head_mask)
+    fail(PCM_ERR_UNSUPPORTED, "per-example weights (a mask for a single-head circuit) need a circuit compiled with "
+                              "pcm_circuit_create or a multi-head circuit");
   if (H_ > 0 && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (flows_in_general_ && rate != 0.f && (block_ || wide_))

@@ -1361,7 +1361,8 @@ void SparseCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 
 void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (fc_.heads.empty() && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
+  // (a circuit with one root takes the mask as [1][batch]: the flow each example starts with at the root, i.e. the
+  // per-example weights of reg_flow.jl:38-39,190-191 -- every flow is linear in it)
   if (!fc_.heads.empty() && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   run_forward(&b, nullptr);
   run_flows(b.batch, nullptr, rate, d_head_mask, d_ll);
@@ -1369,7 +1370,6 @@ void SparseCircuit::flows(const BatchRef& b, float rate, const float* d_head_mas
 
 void SparseCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
-  if (fc_.heads.empty() && d_head_mask) fail(PCM_ERR_ARG, "head_mask given for a single-head circuit");
   if (!fc_.heads.empty() && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   run_forward(nullptr, &s);
   run_flows(s.batch, &s, rate, d_head_mask, d_ll);

@@ -90,11 +90,12 @@ def multihead_loglikelihoods(mhbpc, data, head_mask, batch_size=None, example_id
     return torch.logsumexp(per_head + torch.log(hm), dim=1) - torch.log(hm.sum(dim=1))
 
 
-def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
+def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None, weights=None):
     """`probs_flows_circuit` (src/queries/flow.jl:228-234) /
     `probs_flows_circuit_with_reg` with soft_reg = 0 (src/regularization/reg_flow.jl:276-282):
     forward, backward and leaf flows for one batch; the aggregates stay in the circuit.
-    Returns the batch's log-likelihoods (`mars[:, end]`)."""
+    Returns the batch's log-likelihoods (`mars[:, end]`).  `weights` (one per example of `data`) multiply the
+    examples' edge and leaf flows (reg_flow.jl:38-39,190-191), see `mini_batch_em_with_reg`."""
     _check_data(bpc, data)
     ids = _ids(example_ids, data.device)
     b = data.shape[0] if ids is None else len(ids)
@@ -104,7 +105,13 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None):
         hm = head_mask.to(device=data.device, dtype=torch.float32)
         if ids is not None:
             hm = hm[ids.long()]
-        hm = hm.t().contiguous()   # [heads, batch]
+    if weights is not None:
+        w = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
+        if ids is not None:
+            w = w[ids.long()]
+        hm = w[:, None] if hm is None else hm * w[:, None]
+    if hm is not None:
+        hm = hm.t().contiguous()   # [heads (or 1), batch]
     _flows(bpc, data, _dev_ptr(ids), b, rate, _dev_ptr(hm), ll.data_ptr())
     return ll
 
@@ -154,12 +161,19 @@ def soft_reg_evidence(rows, num_cats, soft_reg, soft_reg_width):
 def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
                            ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
                            shuffle="each_epoch", verbose=False, generator=None, head_mask=None, eval_dataset=None,
-                           eval_interval=0):
+                           eval_interval=0, weights=None, eval_weights=None):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
     of per-epoch mean log-likelihoods.  ent_reg must be 0 (the reference's entropy regulariser is
     commented out at :294-296).  `data` may be 3-D float32 soft evidence, as for the top-level circuits of
     exps/LVD_for_imagenet/src/train_PG_top_level_pcs.jl.  With `verbose`, every `eval_interval` epochs the
     mean log-likelihood of `eval_dataset` is printed beside the training one (:308-327).
+
+    `weights` (one per example of `data`, reg_em.jl:212,220) multiply an example's edge and leaf flows
+    (reg_flow.jl:38-39,190-191); flows being linear in the flow an example starts with, they go in as that
+    starting flow: a factor of the head mask for multi-head circuits, a one-row mask for single-root circuits
+    compiled with `CuBitsProbCircuit`.  Single-head circuits of `hclt_from_clt` do not take them.  The returned
+    training likelihoods are unweighted as in the reference (:302); `eval_weights` weight the mean of the
+    evaluation set (`weighted_ll`, :191-196).
 
     soft_reg > 0 on categorical data (reg_likelihood.jl:4-14, reg_flow.jl:3-22): every batch is turned into
     the soft evidence that gives the leaves the reference's smoothed value (`soft_reg_evidence`) and runs
@@ -191,6 +205,22 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
     lls = []
     ll = torch.empty(batch_size, dtype=torch.float32, device=data.device)
     hm_t = None if head_mask is None else head_mask.to(device=data.device, dtype=torch.float32)
+    w_t = None
+    if weights is not None:
+        w_t = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
+        if w_t.shape != (n,):
+            raise ValueError(f"weights is {tuple(w_t.shape)}, the data has {n} examples")   # reg_em.jl:220
+
+    def batch_mask(ids):
+        # [heads (or 1), batch]: the head mask of the batch, times the examples' weights
+        if hm_t is None and w_t is None:
+            return None
+        if hm_t is None:
+            return w_t[ids.long()][None, :].contiguous()
+        hm = hm_t[ids.long()]
+        if w_t is not None:
+            hm = hm * w_t[ids.long()][:, None]
+        return hm.t().contiguous()
     fresh = True     # the reference clears edge_aggr and the input nodes' flows before its loop (:243-244)
     for _ in range(num_epochs):
         if shuffle == "each_epoch":
@@ -204,14 +234,14 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
             fresh = False
             if smooth:
                 ev = soft_reg_evidence(data[ids.long()], bpc.size("categories"), soft_reg, soft_reg_width)
-                hm = None if hm_t is None else hm_t[ids.long()].t().contiguous()
+                hm = batch_mask(ids)
                 _flows(bpc, ev, None, batch_size, rate, _dev_ptr(hm), ll.data_ptr())
                 check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
-            elif hm_t is None and not _is_soft(data):
+            elif hm_t is None and w_t is None and not _is_soft(data):
                 check(lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(),
                                       batch_size, rate, float(pseudocount), float(param_inertia), ll.data_ptr()))
             else:
-                hm = None if hm_t is None else hm_t[ids.long()].t().contiguous()
+                hm = batch_mask(ids)
                 _flows(bpc, data, ids.data_ptr(), batch_size, rate, _dev_ptr(hm), ll.data_ptr())
                 check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
             acc += ll.sum(dtype=torch.float64)
@@ -220,7 +250,12 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
         if verbose:
             epoch = len(lls)
             if eval_dataset is not None and eval_interval > 0 and epoch % eval_interval == 0 and hm_t is None:
-                test_ll = float(loglikelihoods(bpc, eval_dataset, batch_size=min(batch_size, eval_dataset.shape[0])).mean().item())
+                tl = loglikelihoods(bpc, eval_dataset, batch_size=min(batch_size, eval_dataset.shape[0]))
+                if eval_weights is None:
+                    test_ll = float(tl.mean().item())
+                else:
+                    ew = torch.as_tensor(eval_weights).to(device=tl.device, dtype=torch.float32)
+                    test_ll = float(((tl * ew).sum() / ew.sum()).item())
                 print(f"Mini-batch EM epoch {epoch}/{num_epochs}: train LL {lls[-1]} - test LL {test_ll}")
             else:
                 print(f"Mini-batch EM epoch {epoch}/{num_epochs}; train LL {lls[-1]}")

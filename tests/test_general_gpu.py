@@ -180,6 +180,59 @@ def test_layered_engine_with_value_arrays_beyond_two_gigabytes(gpu, oracle):
     assert np.abs(pl - ps).max() < 2e-5
 
 
+def test_per_example_weights(gpu, oracle):
+    """`weights` of probs_flows_circuit_with_reg / mini_batch_em_with_reg (reg_flow.jl:38-39,190-191: an example's
+    edge and leaf flows times its weight), as the flow the example starts with at the root: a single-root circuit
+    of the layered engine against the oracle seeded with the weights, the driver against the same loop written
+    out, and the refusal of single-head block circuits."""
+    torch, P = gpu
+    O = oracle
+    import pcmi355._lib as L
+    from helpers import random_dag
+    V, C, B = 8, 4, 150
+    rng = np.random.default_rng(61)
+    root = random_dag(V, C, rng, width=3)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, [root], V, C)
+    order = fc.up_order()
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    w = rng.uniform(0.0, 3.0, size=B).astype(np.float32)
+    w[::7] = 0.0
+    d = torch.from_numpy(data).cuda()
+    ll = P.probs_flows_circuit(bpc, d, weights=w).cpu().numpy()
+    mars = O.forward(fc, data)
+    assert np.abs(ll - mars[-1]).max() < LL_RTOL * np.abs(mars[-1]).max()      # likelihoods are not weighted
+    flows, ea_ref = O.backward(fc, mars, root_ids=np.array([fc.n_nodes - 1], np.int32), root_flow=w[None, :])
+    lf_ref = O.input_flows(fc, data, flows)
+    ea, lf = bpc.get_aggregates()
+    assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * max(ea_ref.max(), 1.0)
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * max(lf_ref.max(), 1.0)
+    # weights of one are no weights
+    P.probs_flows_circuit(bpc, d, weights=np.ones(B, np.float32))
+    ea1, lf1 = bpc.get_aggregates()
+    P.probs_flows_circuit(bpc, d)
+    ea0, lf0 = bpc.get_aggregates()
+    np.testing.assert_array_equal(ea1, ea0)
+    np.testing.assert_array_equal(lf1, lf0)
+    # the driver: two circuits, one through mini_batch_em_with_reg(weights=...), one through the loop written out
+    a, b = _compile(P, [root], V, C), _compile(P, [root], V, C)
+    lls = P.mini_batch_em_with_reg(a, d, 2, batch_size=50, pseudocount=0.1, param_inertia=0.4, shuffle="none", weights=w)
+    for _ in range(2):
+        for s0 in range(0, B, 50):
+            ids = np.arange(s0, s0 + 50, dtype=np.int32)
+            P.probs_flows_circuit(b, d, example_ids=ids, weights=w)
+            L.check(L.lib.pcm_em_update(b.handle, 0.1, 0.4))
+    np.testing.assert_array_equal(P.vectorize_parameters(a), P.vectorize_parameters(b))
+    assert len(lls) == 2 and lls[1] > lls[0]
+    with pytest.raises(ValueError):
+        P.mini_batch_em_with_reg(a, d, 1, batch_size=50, pseudocount=0.1, param_inertia=0.4, weights=w[:10])
+    # a single-head circuit on the block kernels takes no mask
+    h = P.hclt_from_clt(np.array([-1, 0, 0, 1], np.int32), C, 16)
+    with pytest.raises(P.PcmError) as e:
+        P.probs_flows_circuit(h, d[:, :4].contiguous(), weights=w)
+    assert e.value.status == -3 and "weights" in str(e.value)   # PCM_ERR_UNSUPPORTED
+
+
 def test_example_ids_and_flow_memory(gpu, oracle):
     """Batches picked by example ids; accumulators scaled by `rate` before a batch
     (src/regularization/reg_em.jl:276-284)."""
