@@ -83,7 +83,6 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
   d_edge_aggr_.alloc((size_t)n_inner_ * K_ * K_ + (size_t)T_ * H_ * K_);
   if (H_ > 0) {
     d_head_wf_.alloc((size_t)T_ * Hp_ * K_);
-    d_flow_shift_.alloc(1);
     d_head_wb_.alloc((size_t)T_ * Hp_ * K_);
     std::vector<int32_t> rn;
     for (int r : roots_) rn.push_back(inner_of_var_[r]);
@@ -91,6 +90,7 @@ HcltCircuit::HcltCircuit(const int32_t* parent, int V, int K, int C, int num_hea
     std::vector<float> hl((size_t)T_ * H_ * K_, -std::log((float)K_));
     PCM_HIP(hipMemcpy(head_logp(), hl.data(), hl.size() * sizeof(float), hipMemcpyHostToDevice));
   }
+  d_flow_shift_.alloc(1);
   d_leaf_flow_.alloc((size_t)V_ * C_ * K_);
   d_edge_aggr_.zero();
   d_leaf_flow_.zero();
@@ -1239,6 +1239,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.G = d_G_.p;
   d.M = d_M_.p;
   d.err = walk_err_;
+  d.w = nullptr;
   d.ext_ops = d_ext_ops_.p;
   d.B = batch;
   d.nslices = ceil_div(batch, kSlice);
@@ -1377,7 +1378,7 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
         // one workgroup fills a compute unit; they draw nodes from d_stat_claim_, which every launch leaves at zero
         PCM_LAUNCH_PHASE(2, hclt_stats_lean_kernel<KK>, dim3(std::min(n_inner_, n_cus_)), dim3(kStatLeanWaves * 64), lds,
                          d, d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
-                         H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
+                         (H_ > 0 || d.w) ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
       });
       check_launch("hclt_stats_lean");
       return;
@@ -1394,7 +1395,7 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     PCM_LAUNCH_PHASE(2, kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, d, d_stat_items_.p, d_edge_aggr_.p,
-                     d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, H_ > 0 ? (const int*)d_flow_shift_.p : (const int*)nullptr);
+                     d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, (H_ > 0 || d.w) ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   };
   PCM_DISPATCH_K(K_, {
     if (d.leaf_slice != 0) launch(&hclt_stats_kernel<KK, true>); else launch(&hclt_stats_kernel<KK, false>);
@@ -1469,10 +1470,8 @@ void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
   no_forest("soft evidence");
   no_missing("soft evidence");
-  if (H_ == 0 && d_head_mask)
-    fail(PCM_ERR_UNSUPPORTED, "per-example weights (a mask for a single-head circuit) need a circuit compiled with "
-                              "pcm_circuit_create or a multi-head circuit");
-  if (soft_block_ok()) {
+  // (per-example weights on soft evidence -- a mask for a single-head circuit -- go to the layered engine)
+  if (soft_block_ok() && !(H_ == 0 && d_head_mask)) {
     if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
     if (flows_in_general_ && rate != 0.f) fail(PCM_ERR_STATE, "flow memory cannot carry over from the layered engine");
     const HcltDev d = soft_stage(s);
@@ -1527,26 +1526,35 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
 }
 
 void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask, float* d_ll) {
-  if (H_ == 0 && d_head_mask)
-    fail(PCM_ERR_UNSUPPORTED, "per-example weights (a mask for a single-head circuit) need a circuit compiled with "
-                              "pcm_circuit_create or a multi-head circuit");
+  // a single-head circuit takes the mask as [1][batch]: the flow every example starts with at the root, i.e. the
+  // per-example weights of reg_flow.jl:38-39,190-191 (every flow is linear in it)
+  const float* weights = H_ == 0 ? d_head_mask : nullptr;
+  if (weights && wide_walk_)
+    fail(PCM_ERR_UNSUPPORTED, "per-example weights are not available on the wide block kernels (K = 128, small trees at "
+                              "K = 64); compile this circuit with pcm_circuit_create");
   if (H_ > 0 && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from soft-evidence batches to categorical batches");
   flows_in_general_ = false;
   if (!block_ && !wide_) {
-    general()->flows(b, rate, nullptr, d_ll);
+    general()->flows(b, rate, weights, d_ll);
     have_flows_ = true;
     return;
   }
   if (const int chunk = walk_chunk(b.batch)) {
     // the accumulators take the first chunk scaled by `rate` and the others on top
-    for (int off = 0; off < b.batch; off += chunk) flows(chunk_of(b, off, chunk), off == 0 ? rate : 1.f, nullptr, d_ll + off);
+    for (int off = 0; off < b.batch; off += chunk)
+      flows(chunk_of(b, off, chunk), off == 0 ? rate : 1.f, weights ? weights + off : nullptr, d_ll + off);
     return;
   }
   stage_batch(b);
   HcltDev d = dev(b.batch);
+  d.w = weights;
+  if (weights) {   // bound on the flow of one example, as a power of two, for the statistics' fixed-point counters
+    hipLaunchKernelGGL(hclt_weight_shift_kernel, dim3(1), dim3(256), 0, stream, weights, b.batch, d_flow_shift_.p);
+    check_launch("weight_shift");
+  }
   if (H_ > 0) {
     d_ll_heads_.ensure((size_t)b.batch);
     run_forward(d, d_ll_heads_.p);

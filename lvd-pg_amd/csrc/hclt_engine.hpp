@@ -104,6 +104,7 @@ struct HcltDev {
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (lean kernels; row n_inner: idle waves)
   int* err;               // host-visible word a walk kernel sets when a wave gave up waiting for a tile
+  const float* w;         // [B] flow every example starts with at a single root (per-example weights), or null: 1
   int32_t B, Bp, nslices, C, n_inner, V;
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
   uint32_t leaf_slice;    // 0; soft evidence: the "leaf table" holds one row per example ([V][Bp][K], the

@@ -38,6 +38,23 @@ constexpr int kStreamStore = 1 | 2 | 16;
 constexpr int kStreamLoad = 2;   // value and ratio tiles are read once per kernel: non-temporal, so that they do not push the
                                  // parameter blocks and leaf tables (read by every workgroup) out of the caches
 
+// ceil(log2) of the largest per-example weight, at least 0: the bound on one example's flow that the statistics
+// kernels' fixed-point counters are scaled by (heads_backward leaves the same bound for a head mask).
+__global__ __launch_bounds__(256) void hclt_weight_shift_kernel(const float* __restrict__ w, int B, int* __restrict__ shift) {
+  __shared__ int best;
+  if (threadIdx.x == 0) best = 0;
+  __syncthreads();
+  int mine = 0;
+  for (int b = threadIdx.x; b < B; b += blockDim.x) {
+    int ex = 0;
+    if (frexpf(fmaxf(w[b], 0.f), &ex) == 0.5f) --ex;   // w <= 2^ex (a power of two is its own bound)
+    mine = max(mine, ex);
+  }
+  atomicMax(&best, mine);
+  __syncthreads();
+  if (threadIdx.x == 0) *shift = best;
+}
+
 constexpr int kStatWaves = 12;   // waves per workgroup in the statistics kernel (168 registers each)
 
 template <int K>
@@ -461,7 +478,9 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
         tile_load<K>(d.R, node, d.tile_stride, lo.tile, r);
       } else {        // flow 1 into the single root sum node of every live example
         tile_zero<K>(r);
-        r.v[0][0] = (lane < 16 && bcol < d.B) ? fminf(__builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e), kFlowRatioCap) : 0.f;
+        const bool live = lane < 16 && bcol < d.B;
+        const float wgt = (d.w && live) ? d.w[bcol] : 1.f;   // per-example weights: the flow the example starts with
+        r.v[0][0] = live ? wgt * fminf(__builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e), kFlowRatioCap) : 0.f;
       }
     }
     tile_store<K>(d.R, node, d.tile_stride, lo.tile, r);

@@ -383,8 +383,9 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     } else if (fl & 1) {   // flow 1 into the single root sum node of every live example: R = 1 / S = exp(M - O)
       const float o00 = __builtin_bit_cast(
           float, __builtin_amdgcn_raw_buffer_load_b32(rO, (int)vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, 0));
-      const float r00 = (lane < 16 && bcol < d.B)
-                            ? fminf(__builtin_amdgcn_exp2f(fmaf(o00, -kLog2e, mroot * kLog2e)), kFlowRatioCap) : 0.f;
+      const bool live = lane < 16 && bcol < d.B;
+      const float wgt = (d.w && live) ? d.w[bcol] : 1.f;   // per-example weights: the flow the example starts with
+      const float r00 = live ? wgt * fminf(__builtin_amdgcn_exp2f(fmaf(o00, -kLog2e, mroot * kLog2e)), kFlowRatioCap) : 0.f;
       tile_zero<K>(r);
       r.v[0][0] = r00;
     }

@@ -226,8 +226,8 @@ def test_per_example_weights(gpu, oracle):
     assert len(lls) == 2 and lls[1] > lls[0]
     with pytest.raises(ValueError):
         P.mini_batch_em_with_reg(a, d, 1, batch_size=50, pseudocount=0.1, param_inertia=0.4, weights=w[:10])
-    # a single-head circuit on the block kernels takes no mask
-    h = P.hclt_from_clt(np.array([-1, 0, 0, 1], np.int32), C, 16)
+    # the wide block kernels take no mask
+    h = P.hclt_from_clt(np.array([-1, 0, 0, 1], np.int32), C, 128)
     with pytest.raises(P.PcmError) as e:
         P.probs_flows_circuit(h, d[:, :4].contiguous(), weights=w)
     assert e.value.status == -3 and "weights" in str(e.value)   # PCM_ERR_UNSUPPORTED

@@ -711,3 +711,60 @@ def test_missing_values_as_a_marker_category(gpu, oracle, V, K, C, B, heads):
     assert ll2.mean() > ll.mean()
     with pytest.raises(P.PcmError, match="missing-value"):
         P.kld(bpc, bpc)
+
+
+@pytest.mark.parametrize("V,K,C,B,bushy", [(9, 16, 5, 70, False), (40, 32, 256, 300, False), (600, 64, 4, 40, True)])
+def test_per_example_weights_on_single_head_block_circuits(gpu, oracle, V, K, C, B, bushy):
+    """`weights` of probs_flows_circuit_with_reg (reg_flow.jl:38-39,190-191) on the walk kernels: the flow an example
+    starts with at the root.  Edge and leaf statistics against the oracle seeded with the weights (some of them
+    zero, some above one: the fixed-point counters scale by their bound), likelihoods unweighted; on the lean
+    kernels (K = 16, 32) and on the general walk kernels (K = 64 on a bushy tree)."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta
+    rng = np.random.default_rng(V * 100 + K)
+    if bushy:
+        parent = np.asarray(O.random_tree(V, rng, 3), np.int32)
+    else:
+        parent = np.full(V, -1, np.int32)
+        for v in range(1, V):
+            parent[v] = rng.integers(max(0, v - 3), v)
+    parent, theta, leaf, fc = make_hclt(V, K, C, V + K, parent=parent)
+    c = P.hclt_from_clt(parent, C, K)
+    c.set_params(block_theta(parent, K, theta), leaf)
+    assert c.size("walk_kernels") == (2 if bushy else 1)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    w = rng.uniform(0.0, 5.0, size=B).astype(np.float32)
+    w[::5] = 0.0
+    d = torch.from_numpy(data).cuda()
+    ll = P.probs_flows_circuit(c, d, weights=w).cpu().numpy()
+    mars = O.forward(fc, data)
+    assert np.abs(ll - mars[-1]).max() < 1e-4 * np.abs(mars[-1]).max()
+    flows, ea_ref = O.backward(fc, mars, root_ids=np.array([fc.n_nodes - 1], np.int32), root_flow=w[None, :])
+    lf_ref = O.input_flows(fc, data, flows).reshape(V, K, C)
+    ea, lf = c.get_flows()
+    for v, blk in O.hclt_block_aggr(fc, ea_ref).items():
+        nk = blk.shape[0]
+        assert np.abs(ea[v][:nk] - blk).max() < 2e-4 * max(blk.max(), 1e-3), f"edge_aggr block {v}"
+    assert np.abs(lf - lf_ref).max() < 2e-4 * max(lf_ref.max(), 1e-3)
+    np.testing.assert_allclose(lf.sum(axis=(1, 2)), w.sum(), rtol=1e-4)   # every example passes every variable with its weight
+    ref = fc.copy()
+    ref.logp, ref.leaf_logp = O.em_update(fc, ea_ref, lf_ref.reshape(-1), 0.1, 0.9)
+    th_ref, leaf_ref = O.hclt_block_params(ref)
+    import pcmi355._lib as L
+    from helpers import rel_err
+    L.check(L.lib.pcm_em_update(c.handle, 0.1, 0.9))
+    th, lf_new = c.get_params()
+    tol = 3e-4 if bushy else 1e-4   # (600 variables deep in float32 on both sides: rounding, not method)
+    for v, blk in th_ref.items():
+        nk = blk.shape[0]
+        assert rel_err(np.exp(th[v][:nk]), np.exp(blk)).max() < tol, f"theta block {v}"
+    assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < tol
+    # unit weights are no weights, to the bit
+    c.set_params(block_theta(parent, K, theta), leaf)
+    P.probs_flows_circuit(c, d, weights=np.ones(B, np.float32))
+    a1 = c.get_flows()
+    P.probs_flows_circuit(c, d)
+    a0 = c.get_flows()
+    for x, y in zip(a1, a0):
+        np.testing.assert_array_equal(x, y)
