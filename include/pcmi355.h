@@ -205,8 +205,7 @@ int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex,
  * Per-example weights (the `weights` of reg_flow.jl:38-39,190-191, which multiply an example's edge and
  * leaf flows): every flow is linear in the flow its example starts with, so for a multi-head circuit they
  * are a factor of the mask's column, and a single-root circuit (pcm_circuit_create without heads,
- * pcm_hclt_create) takes them as a mask [1][batch]; d_ll_out is not weighted.  Not on the wide block kernels
- * (pcm_hclt_create with K = 128, or K = 64 on a small tree: PCM_ERR_UNSUPPORTED).
+ * pcm_hclt_create) takes them as a mask [1][batch]; d_ll_out is not weighted.
  */
 int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
               const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask,

@@ -1529,9 +1529,6 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   // a single-head circuit takes the mask as [1][batch]: the flow every example starts with at the root, i.e. the
   // per-example weights of reg_flow.jl:38-39,190-191 (every flow is linear in it)
   const float* weights = H_ == 0 ? d_head_mask : nullptr;
-  if (weights && wide_walk_)
-    fail(PCM_ERR_UNSUPPORTED, "per-example weights are not available on the wide block kernels (K = 128, small trees at "
-                              "K = 64); compile this circuit with pcm_circuit_create");
   if (H_ > 0 && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
   if (flows_in_general_ && rate != 0.f && (block_ || wide_))

@@ -354,7 +354,8 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
     for (int q = 0; q < Q; ++q) {
       const int kt = wave * Q + q;
       v4f fq;
-      if (on.parent < 0) fq = v4f{kt == 0 && g == 0 && live ? 1.f : 0.f, 0.f, 0.f, 0.f};
+      if (on.parent < 0)   // the root: the flow the example starts with (1, or its weight) in state 0
+        fq = v4f{kt == 0 && g == 0 && live ? (d.w ? d.w[col] : 1.f) : 0.f, 0.f, 0.f, 0.f};
       else if (on.parent == n + 1) fq = prev_g[q];
       else fq = f[q];
       v4f r;
@@ -464,10 +465,11 @@ __device__ __forceinline__ void wide_edge_block(const HcltDev& d, const float* _
 // Leaf histograms: workgroup (variable u, state tile kt) adds, for every example, the 16 flows
 // of the tile to row x_b of a [C][16] table in LDS, as two-limb fixed-point integers (integer
 // LDS atomics are more than ten times cheaper than floating-point ones here and make the sum
-// independent of the order of arrival); flows are in [0, 1].
+// independent of the order of arrival); flows are in [0, 1], or in [0, 2^shift] under per-example weights.
 __device__ __forceinline__ void wide_leaf_block(const HcltDev& d, const float* __restrict__ G,
                                                 const int32_t* __restrict__ state_node, int K,
-                                                float* __restrict__ leaf_flow, float rate, int limb, int u, int kt) {
+                                                float* __restrict__ leaf_flow, float rate, int limb,
+                                                const int* __restrict__ flow_shift, int u, int kt) {
   extern __shared__ unsigned hist[];   // [2][C][17]
   constexpr int HS = 17;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -477,7 +479,9 @@ __device__ __forceinline__ void wide_leaf_block(const HcltDev& d, const float* _
   const int hw = d.C * HS;
   for (int i = threadIdx.x; i < 2 * hw; i += blockDim.x) hist[i] = 0u;
   __syncthreads();
-  const float scale = __builtin_ldexpf(1.f, limb);
+  // (with per-example weights a flow is at most 2^shift, the bound the host left: counted in units of that)
+  const int shift = flow_shift ? __builtin_amdgcn_readfirstlane(*flow_shift) : 0;
+  const float scale = __builtin_ldexpf(1.f, limb), unit_inv = __builtin_ldexpf(1.f, -shift);
   const v4f* gt = reinterpret_cast<const v4f*>(G + (size_t)n * d.nslices * kSlice * K);
   for (int s = wave; s < d.nslices; s += kWideWaves) {
     const int col = s * kSlice + b;
@@ -486,7 +490,7 @@ __device__ __forceinline__ void wide_leaf_block(const HcltDev& d, const float* _
     if (col < d.B) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float v = fminf(fmaxf(f[i], 0.f), 1.f) * scale;
+        const float v = fminf(fmaxf(f[i] * unit_inv, 0.f), 1.f) * scale;
         const float fl = floorf(v);
         __hip_atomic_fetch_add(&hist[x * HS + 4 * g + i], (unsigned)fl, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         __hip_atomic_fetch_add(&hist[hw + x * HS + 4 * g + i], (unsigned)((v - fl) * scale), __ATOMIC_RELAXED,
@@ -495,7 +499,7 @@ __device__ __forceinline__ void wide_leaf_block(const HcltDev& d, const float* _
     }
   }
   __syncthreads();
-  const float hi_inv = __builtin_ldexpf(1.f, -limb), lo_inv = __builtin_ldexpf(1.f, -2 * limb);
+  const float hi_inv = __builtin_ldexpf(1.f, shift - limb), lo_inv = __builtin_ldexpf(1.f, shift - 2 * limb);
   for (int i = threadIdx.x; i < d.C * 16; i += blockDim.x) {
     const int c = i >> 4, jj = i & 15;
     const float val = (float)hist[c * HS + jj] * hi_inv + (float)hist[hw + c * HS + jj] * lo_inv;
@@ -515,8 +519,8 @@ __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_edge_kernel(HcltDev
 __global__ __launch_bounds__(kWideWaves * 64) void hclt_wide_leaf_kernel(HcltDev d, const float* __restrict__ G,
                                                                          const int32_t* __restrict__ state_node, int K,
                                                                          float* __restrict__ leaf_flow, float rate,
-                                                                         int limb) {
-  wide_leaf_block(d, G, state_node, K, leaf_flow, rate, limb, blockIdx.x, blockIdx.y);
+                                                                         int limb, const int* __restrict__ flow_shift) {
+  wide_leaf_block(d, G, state_node, K, leaf_flow, rate, limb, flow_shift, blockIdx.x, blockIdx.y);
 }
 
 // ---- host --------------------------------------------------------------------------------
@@ -614,7 +618,8 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
   if (!soft)
     hipExtLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideWaves * 64), (uint32_t)lds, stream, nullptr,
-                          t_stat ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb);
+                          t_stat ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb,
+                          d.w ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   check_launch_w("hclt_wide_stats");
 }
 

@@ -170,8 +170,7 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
 
     `weights` (one per example of `data`, reg_em.jl:212,220) multiply an example's edge and leaf flows
     (reg_flow.jl:38-39,190-191); flows being linear in the flow an example starts with, they go in as that
-    starting flow: a factor of the head mask for multi-head circuits, a one-row mask for single-root circuits
-    (not on the wide block kernels: `hclt_from_clt` with K = 128, or K = 64 on a small tree).  The returned
+    starting flow: a factor of the head mask for multi-head circuits, a one-row mask for single-root circuits.  The returned
     training likelihoods are unweighted as in the reference (:302); `eval_weights` weight the mean of the
     evaluation set (`weighted_ll`, :191-196).
 

@@ -184,7 +184,7 @@ def test_per_example_weights(gpu, oracle):
     """`weights` of probs_flows_circuit_with_reg / mini_batch_em_with_reg (reg_flow.jl:38-39,190-191: an example's
     edge and leaf flows times its weight), as the flow the example starts with at the root: a single-root circuit
     of the layered engine against the oracle seeded with the weights, the driver against the same loop written
-    out, and the refusal of single-head block circuits."""
+    out."""
     torch, P = gpu
     O = oracle
     import pcmi355._lib as L
@@ -226,11 +226,6 @@ def test_per_example_weights(gpu, oracle):
     assert len(lls) == 2 and lls[1] > lls[0]
     with pytest.raises(ValueError):
         P.mini_batch_em_with_reg(a, d, 1, batch_size=50, pseudocount=0.1, param_inertia=0.4, weights=w[:10])
-    # the wide block kernels take no mask
-    h = P.hclt_from_clt(np.array([-1, 0, 0, 1], np.int32), C, 128)
-    with pytest.raises(P.PcmError) as e:
-        P.probs_flows_circuit(h, d[:, :4].contiguous(), weights=w)
-    assert e.value.status == -3 and "weights" in str(e.value)   # PCM_ERR_UNSUPPORTED
 
 
 def test_example_ids_and_flow_memory(gpu, oracle):

@@ -713,12 +713,14 @@ def test_missing_values_as_a_marker_category(gpu, oracle, V, K, C, B, heads):
         P.kld(bpc, bpc)
 
 
-@pytest.mark.parametrize("V,K,C,B,bushy", [(9, 16, 5, 70, False), (40, 32, 256, 300, False), (600, 64, 4, 40, True)])
+@pytest.mark.parametrize("V,K,C,B,bushy", [(9, 16, 5, 70, False), (40, 32, 256, 300, False), (600, 64, 4, 40, True),
+                                            (11, 128, 9, 50, False), (8, 64, 256, 33, False)])
 def test_per_example_weights_on_single_head_block_circuits(gpu, oracle, V, K, C, B, bushy):
     """`weights` of probs_flows_circuit_with_reg (reg_flow.jl:38-39,190-191) on the walk kernels: the flow an example
     starts with at the root.  Edge and leaf statistics against the oracle seeded with the weights (some of them
     zero, some above one: the fixed-point counters scale by their bound), likelihoods unweighted; on the lean
-    kernels (K = 16, 32) and on the general walk kernels (K = 64 on a bushy tree)."""
+    kernels (K = 16, 32), the general walk kernels (K = 64 on a bushy tree) and the wide kernels (K = 128, K = 64 on
+    a small tree)."""
     torch, P = gpu
     O = oracle
     from helpers import make_hclt, block_theta
@@ -732,7 +734,7 @@ def test_per_example_weights_on_single_head_block_circuits(gpu, oracle, V, K, C,
     parent, theta, leaf, fc = make_hclt(V, K, C, V + K, parent=parent)
     c = P.hclt_from_clt(parent, C, K)
     c.set_params(block_theta(parent, K, theta), leaf)
-    assert c.size("walk_kernels") == (2 if bushy else 1)
+    assert c.size("walk_kernels") == (2 if bushy else 3 if K >= 64 else 1)
     data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
     w = rng.uniform(0.0, 5.0, size=B).astype(np.float32)
     w[::5] = 0.0
