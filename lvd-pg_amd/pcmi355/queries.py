@@ -276,12 +276,14 @@ def mini_batch_em_for_multihead_pc(mhbpc, data, head_mask, num_epochs, **kw):
 
 
 def mini_batch_em_for_forest(forest, data, head_masks, num_epochs, *, batch_size, pseudocount, param_inertia,
-                             param_inertia_end=None, flow_memory=0.0, shuffle="each_epoch", generator=None):
+                             param_inertia_end=None, flow_memory=0.0, shuffle="each_epoch", generator=None,
+                             weights=None):
     """The loop over patch circuits of exps/progressive_growing/parallel_PG.jl:214-225 -- one
     `mini_batch_em_for_multihead_pc` (src-jl/multi_head_pc/em.jl:1-99) per circuit -- as one loop over a forest handle:
     every batch is one `pcm_flows` + `pcm_em_update` for all trees, with the batch order, inertia schedule and flow
     memory of `mini_batch_em_with_reg`.  head_masks: [trees, examples, heads], a tree's slice being the `head_mask`
-    the reference passes for that circuit.  Returns the per-epoch mean log-likelihoods, [epochs, trees]."""
+    the reference passes for that circuit; `weights` (one per example, em.jl:5,20) multiply an example's flows in
+    every tree, as a factor of its masks.  Returns the per-epoch mean log-likelihoods, [epochs, trees]."""
     _check_data(forest, data)
     n, T = data.shape[0], forest.size("trees")
     if batch_size > n:
@@ -289,6 +291,11 @@ def mini_batch_em_for_forest(forest, data, head_masks, num_epochs, *, batch_size
     hm_t = head_masks.to(device=data.device, dtype=torch.float32)
     if tuple(hm_t.shape) != (T, n, forest.num_heads):
         raise ValueError(f"head_masks is {tuple(hm_t.shape)}, the forest needs {(T, n, forest.num_heads)}")
+    if weights is not None:
+        w_t = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
+        if w_t.shape != (n,):
+            raise ValueError(f"weights is {tuple(w_t.shape)}, the data has {n} examples")
+        hm_t = hm_t * w_t[None, :, None]
     num_batches = n // batch_size
     if param_inertia_end is None:
         param_inertia_end = param_inertia

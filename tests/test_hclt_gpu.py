@@ -770,3 +770,33 @@ def test_per_example_weights_on_single_head_block_circuits(gpu, oracle, V, K, C,
     a0 = c.get_flows()
     for x, y in zip(a1, a0):
         np.testing.assert_array_equal(x, y)
+
+
+def test_forest_driver_with_per_example_weights(gpu, oracle):
+    """`weights` of the multi-head EM driver (src-jl/multi_head_pc/em.jl:5,20,72) over a forest: the same as masks
+    that carry the weights, to the bit, and different from the unweighted run."""
+    torch, P = gpu
+    rng = np.random.default_rng(77)
+    T, Vt, K, C, H, B = 3, [6, 9, 4], 16, 5, 4, 96
+    V, parent, gvars, trees = _forest_case(P, oracle, rng, T, Vt, K, C, H)
+    data = torch.from_numpy(rng.integers(0, C, size=(B, V)).astype(np.uint8)).cuda()
+    masks = torch.from_numpy(rng.random((T, B, H)).astype(np.float32)).cuda()
+    w = torch.from_numpy(rng.uniform(0.0, 4.0, size=B).astype(np.float32)).cuda()
+
+    def run(m, weights):
+        f = P.hclt_forest_from_clts(parent, C, K, H)
+        theta = np.zeros((V, K, K), np.float32)
+        leaf = np.zeros((V, K, C), np.float32)
+        for gv, (par_t, theta_t, leaf_t, _) in zip(gvars, trees):
+            theta[gv], leaf[gv] = theta_t, leaf_t
+        f.set_params(theta, leaf)
+        f.set_heads(np.stack([t[3] for t in trees]))
+        P.mini_batch_em_for_forest(f, data, m, 2, batch_size=48, pseudocount=0.1, param_inertia=0.5, shuffle="none",
+                                   weights=weights)
+        return f.get_params() + (f.get_heads(),)
+    a = run(masks, w)
+    b = run(masks * w[None, :, None], None)
+    c = run(masks, None)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    assert np.abs(np.exp(a[1]) - np.exp(c[1])).max() > 1e-3   # (leaf tables)
