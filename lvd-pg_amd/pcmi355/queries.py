@@ -161,7 +161,7 @@ def soft_reg_evidence(rows, num_cats, soft_reg, soft_reg_width):
 def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
                            ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
                            shuffle="each_epoch", verbose=False, generator=None, head_mask=None, eval_dataset=None,
-                           eval_interval=0, weights=None, eval_weights=None):
+                           eval_interval=0, weights=None, eval_weights=None, init_clear_mem=True):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
     of per-epoch mean log-likelihoods.  ent_reg must be 0 (the reference's entropy regulariser is
     commented out at :294-296).  `data` may be 3-D float32 soft evidence, as for the top-level circuits of
@@ -172,7 +172,9 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
     (reg_flow.jl:38-39,190-191); flows being linear in the flow an example starts with, they go in as that
     starting flow: a factor of the head mask for multi-head circuits, a one-row mask for single-root circuits.  The returned
     training likelihoods are unweighted as in the reference (:302); `eval_weights` weight the mean of the
-    evaluation set (`weighted_ll`, :191-196).
+    evaluation set (`weighted_ll`, :191-196).  `init_clear_mem = False` (src-jl/multi_head_pc/em.jl:6,28-31) keeps
+    the flows the circuit holds from an earlier call as the flow memory of the first batch; the circuit owns its
+    accumulators, so this is the reference's `edge_aggr_mem` given and not cleared.
 
     soft_reg > 0 on categorical data (reg_likelihood.jl:4-14, reg_flow.jl:3-22): every batch is turned into
     the soft evidence that gives the leaves the reference's smoothed value (`soft_reg_evidence`) and runs
@@ -220,7 +222,7 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
         if w_t is not None:
             hm = hm * w_t[ids.long()][:, None]
         return hm.t().contiguous()
-    fresh = True     # the reference clears edge_aggr and the input nodes' flows before its loop (:243-244)
+    fresh = bool(init_clear_mem)   # the reference clears edge_aggr and the input nodes' flows before its loop (:243-244)
     for _ in range(num_epochs):
         if shuffle == "each_epoch":
             do_shuffle()

@@ -228,6 +228,25 @@ def test_per_example_weights(gpu, oracle):
         P.mini_batch_em_with_reg(a, d, 1, batch_size=50, pseudocount=0.1, param_inertia=0.4, weights=w[:10])
 
 
+def test_driver_called_again_without_clearing_its_flow_memory(gpu, oracle):
+    """`init_clear_mem = false` (src-jl/multi_head_pc/em.jl:6,28-31): two calls of one epoch, the second keeping the
+    accumulators, are one call of two epochs; with the default the second call starts from cleared ones."""
+    torch, P = gpu
+    from helpers import random_dag
+    V, C, B = 7, 4, 120
+    rng = np.random.default_rng(71)
+    root = random_dag(V, C, rng, width=3)
+    d = torch.from_numpy(rng.integers(0, C, size=(B, V)).astype(np.uint8)).cuda()
+    kw = dict(batch_size=40, pseudocount=0.1, param_inertia=0.6, flow_memory=150.0, shuffle="none")
+    one, two, cleared = (_compile(P, [root], V, C) for _ in range(3))
+    P.mini_batch_em_with_reg(one, d, 2, **kw)
+    for c, keep in ((two, False), (cleared, True)):
+        P.mini_batch_em_with_reg(c, d, 1, **kw)
+        P.mini_batch_em_with_reg(c, d, 1, init_clear_mem=keep, **kw)
+    np.testing.assert_array_equal(P.vectorize_parameters(two), P.vectorize_parameters(one))
+    assert np.abs(P.vectorize_parameters(cleared) - P.vectorize_parameters(one)).max() > 1e-6
+
+
 def test_example_ids_and_flow_memory(gpu, oracle):
     """Batches picked by example ids; accumulators scaled by `rate` before a batch
     (src/regularization/reg_em.jl:276-284)."""
