@@ -41,12 +41,38 @@ def learn_chow_liu_tree(data, num_cats=None, pseudocount=0.1):
     return chow_liu_tree(pairwise_MI(data, num_cats, pseudocount))
 
 
-def hclt(data, num_hidden_cats, num_cats=None, pseudocount=0.1):
-    """`hclt(data, num_hidden_cats; num_cats, pseudocount)` (src/structures/hclts.jl:7-24) with
-    one variable per group: Chow-Liu tree of the data, then the hidden Chow-Liu tree circuit."""
+def hclt(data, num_hidden_cats, variable_groups=None, num_cats=None, pseudocount=0.1, get_leaves=False):
+    """`hclt(data, num_hidden_cats, variable_groups; num_cats, pseudocount)` (src/structures/hclts.jl:7-24): the
+    Chow-Liu tree of the groups' first variables, then the hidden Chow-Liu tree circuit over the groups.  Without
+    groups (one variable per tree node) the circuit is built on the block kernels (`hclt_from_clt`); with groups
+    it is the DAG of `hclt_pc`, to be compiled with `CuBitsProbCircuit` (with `get_leaves` also the tree nodes'
+    leaf circuits, as `hclt_from_clt(...; get_leaves = true)` returns them)."""
     if num_cats is None:
         num_cats = int(data.max().item()) + 1
-    return hclt_from_clt(learn_chow_liu_tree(data, num_cats, pseudocount), int(num_cats), int(num_hidden_cats))
+    if variable_groups is None:
+        return hclt_from_clt(learn_chow_liu_tree(data, num_cats, pseudocount), int(num_cats), int(num_hidden_cats))
+    firsts = [int(g[0]) for g in variable_groups]
+    mapped = data[:, firsts].contiguous()            # mapped_data[:, idx] = data[:, variable_groups[idx][1]] (:14)
+    clt = learn_chow_liu_tree(mapped, num_cats, pseudocount)
+    return hclt_pc(clt, int(num_cats), int(num_hidden_cats), variable_groups, get_leaves=get_leaves)
+
+
+def hclt_for_colored_images(data, nc, height, width, num_hidden_cats, num_cats=None, pseudocount=0.1, mode="red_only",
+                            patch_size=2):
+    """`hclt_for_colored_images` (src/structures/hclts.jl:26-98): an HCLT over patch_size x patch_size groups of the
+    pixels of one channel ("red_only", "green_only", "blue_only": the channel's plane of the [N, nc * height * width]
+    data) or of all channels of a patch ("cat_channels").  Returns (circuit, leaves) as the reference does."""
+    plane = height * width
+    if mode in ("red_only", "green_only", "blue_only"):
+        offset = {"red_only": 0, "green_only": plane, "blue_only": 2 * plane}[mode]
+        groups = group_vars_by_grid(height, width, 1, patch_h=patch_size, patch_w=patch_size, global_offset=offset)
+    elif mode == "cat_channels":
+        groups = group_vars_by_cgrid(height, width, nc, patch_h=patch_size, patch_w=patch_size, global_offset=0)
+    else:
+        raise ValueError("Not implemented")           # hclts.jl:94
+    if num_cats is None:
+        num_cats = int(data.max().item()) + 1
+    return hclt(data, num_hidden_cats, groups, num_cats=num_cats, pseudocount=pseudocount, get_leaves=True)
 
 
 # ---- trees ---------------------------------------------------------------------------------
@@ -147,7 +173,7 @@ def group_vars_by_cgrid(height, width, cdepth, patch_h=2, patch_w=2, global_offs
 
 # ---- circuits as DAGs ------------------------------------------------------------------------
 
-def hclt_pc(clt_parent, num_cats, num_hidden_cats, variable_groups=None):
+def hclt_pc(clt_parent, num_cats, num_hidden_cats, variable_groups=None, get_leaves=False):
     """`hclt_from_clt(clt, num_cats, num_hidden_cats, variable_groups; input_type = Categorical)`
     (src/structures/hclts.jl:100-145) as a DAG of `pcmi355.nodes`: tree node i stands for the
     observed variables `variable_groups[i][1]` (default: variable i alone), whose joint leaf is
@@ -174,7 +200,7 @@ def hclt_pc(clt_parent, num_cats, num_hidden_cats, variable_groups=None):
         cc = [circuits[c] for c in ch[v]]
         cc = [N.summate(N.multiply([c[j] for c in cc])) for j in range(K)] if len(cc) > 1 else cc[0]
         circuits[v] = [N.summate([N.multiply(cc[j], leaves[v][j]) for j in range(K)]) for _ in range(K)]
-    return circuits[root][0]
+    return (circuits[root][0], leaves) if get_leaves else circuits[root][0]
 
 
 def customized_hclt(clt, num_hidden_cats, get_leaf_pcs, get_edge_params=None, parameterize_leaf_edge=True,

@@ -132,6 +132,40 @@ def test_learned_tree_and_hclt(gpu):
 
 
 @pytest.mark.gpu
+def test_hclt_over_variable_groups_and_for_colored_images(gpu):
+    """`hclt(data, K, variable_groups)` and `hclt_for_colored_images` (src/structures/hclts.jl:7-98): the tree is
+    learned on the groups' first variables, a tree node's leaf is the product of one categorical per variable of
+    its group; the circuit is the one `hclt_pc` builds from that tree, it covers exactly the grouped variables,
+    and it trains."""
+    torch, P = gpu
+    from pcmi355 import nodes as N
+    nc, h, w, K, C, n = 3, 4, 4, 4, 6, 600
+    x = _data(n, nc * h * w, C, 23)
+    d = torch.from_numpy(x).cuda()
+    for mode, offset in (("red_only", 0), ("green_only", h * w), ("blue_only", 2 * h * w), ("cat_channels", None)):
+        pc, leaves = P.hclt_for_colored_images(d, nc, h, w, K, num_cats=C, mode=mode, patch_size=2)
+        groups = (P.group_vars_by_cgrid(h, w, nc, 2, 2, 0) if offset is None else P.group_vars_by_grid(h, w, 1, 2, 2, offset))
+        assert len(leaves) == len(groups) == 4 and all(len(l) == K for l in leaves)
+        want_vars = sorted(v for g in groups for v in g[1])
+        assert N.variables(pc) == want_vars and len(want_vars) == (4 * nc if offset is None else 4) * 4
+        firsts = [g[0] for g in groups]
+        clt = P.learn_chow_liu_tree(d[:, firsts].contiguous(), C, 0.1)
+        same, _ = N.describe(P.hclt_pc(clt, C, K, groups))
+        got, _ = N.describe(pc)
+        for k in same:
+            np.testing.assert_array_equal(got[k], same[k], err_msg=f"{mode} {k}")
+        for i, g in enumerate(groups):                          # a leaf circuit: sum over the product of its group's inputs
+            prod = leaves[i][0].inputs[0]
+            assert [c.var for c in prod.inputs] == list(g[1])
+    with pytest.raises(ValueError):
+        P.hclt_for_colored_images(d, nc, h, w, K, num_cats=C, mode="grey")
+    N.init_parameters(pc, perturbation=0.4, rng=np.random.default_rng(1))
+    bpc = P.CuBitsProbCircuit(pc, nc * h * w)
+    lls = P.mini_batch_em_with_reg(bpc, d, 3, batch_size=200, pseudocount=0.1, param_inertia=0.9, shuffle="none")
+    assert lls[-1] > lls[0]
+
+
+@pytest.mark.gpu
 def test_pairwise_mi_full_size_properties(gpu):
     """4096 examples x 512 variables x 256 categories: symmetry, MI(x, x) = smoothed entropy
     identity against the oracle on a few pairs, duplicated column gives the same row."""
