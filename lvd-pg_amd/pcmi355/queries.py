@@ -90,6 +90,30 @@ def multihead_loglikelihoods(mhbpc, data, head_mask, batch_size=None, example_id
     return torch.logsumexp(per_head + torch.log(hm), dim=1) - torch.log(hm.sum(dim=1))
 
 
+def loglikelihood(bpc, data, weights=None, batch_size=None, head_mask=None):
+    """`loglikelihood_probcat(bpc, data, weights; batch_size)` (src/regularization/reg_likelihood.jl:164-173) and
+    `weighted_ll` (src/regularization/reg_em.jl:191-197): the mean of the per-example log-likelihoods, weighted by
+    `weights` (one per example) when given: sum(ll * w) / sum(w).  With `head_mask` the per-example values are the
+    multi-head mixture's (`multihead_loglikelihoods`).  Returns a Python float; the sum runs in float64 on the device."""
+    if head_mask is not None:
+        lls = multihead_loglikelihoods(bpc, data, head_mask, batch_size=batch_size)
+    else:
+        lls = loglikelihoods(bpc, data, batch_size=batch_size)
+    if lls.dim() != 1:
+        raise ValueError("a multi-head circuit needs a head_mask to have one log-likelihood per example")
+    if weights is None:
+        return float(lls.sum(dtype=torch.float64).item()) / max(lls.numel(), 1)
+    w = torch.as_tensor(weights).to(device=lls.device, dtype=torch.float64)
+    if w.shape != lls.shape:
+        raise ValueError(f"{w.numel()} weights for {lls.numel()} examples")
+    return float(((lls.double() * w).sum() / w.sum()).item())
+
+
+loglikelihoods_probcat = loglikelihoods        # reg_likelihood.jl:139-162: the same pass, the reference's other name
+loglikelihood_probcat = loglikelihood          # reg_likelihood.jl:164-173
+weighted_ll = loglikelihood                    # reg_em.jl:191-197
+
+
 def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None, weights=None):
     """`probs_flows_circuit` (src/queries/flow.jl:228-234) /
     `probs_flows_circuit_with_reg` with soft_reg = 0 (src/regularization/reg_flow.jl:276-282):
@@ -251,12 +275,7 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
         if verbose:
             epoch = len(lls)
             if eval_dataset is not None and eval_interval > 0 and epoch % eval_interval == 0 and hm_t is None:
-                tl = loglikelihoods(bpc, eval_dataset, batch_size=min(batch_size, eval_dataset.shape[0]))
-                if eval_weights is None:
-                    test_ll = float(tl.mean().item())
-                else:
-                    ew = torch.as_tensor(eval_weights).to(device=tl.device, dtype=torch.float32)
-                    test_ll = float(((tl * ew).sum() / ew.sum()).item())
+                test_ll = loglikelihood(bpc, eval_dataset, eval_weights, batch_size=min(batch_size, eval_dataset.shape[0]))
                 print(f"Mini-batch EM epoch {epoch}/{num_epochs}: train LL {lls[-1]} - test LL {test_ll}")
             else:
                 print(f"Mini-batch EM epoch {epoch}/{num_epochs}; train LL {lls[-1]}")

@@ -207,6 +207,9 @@ def test_per_example_weights(gpu, oracle):
     ea, lf = bpc.get_aggregates()
     assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * max(ea_ref.max(), 1.0)
     assert np.abs(lf - lf_ref).max() < FLOW_RTOL * max(lf_ref.max(), 1.0)
+    # the weighted mean of the data set's log-likelihoods, with chunks that do not divide the data set
+    assert abs(P.loglikelihood(bpc, d, w, batch_size=64) - (mars[-1].astype(np.float64) * w).sum() / w.astype(np.float64).sum()) < 1e-5
+    assert abs(P.loglikelihood(bpc, d) - mars[-1].astype(np.float64).mean()) < 1e-5
     # weights of one are no weights
     P.probs_flows_circuit(bpc, d, weights=np.ones(B, np.float32))
     ea1, lf1 = bpc.get_aggregates()
@@ -297,6 +300,15 @@ def test_multihead_closed_forms(gpu, oracle):
     per_head = P.loglikelihoods(bpc, data).cpu().numpy()
     assert per_head.shape == (2, 2)
     np.testing.assert_allclose([per_head[0, 0], per_head[1, 1]], want, rtol=1e-5)
+
+    # the means over the data set (reg_likelihood.jl:164-173, reg_em.jl:191-197), against the closed forms above
+    assert abs(P.loglikelihood(bpc, data, head_mask=head_mask) - np.mean(want)) < 1e-5
+    assert abs(P.weighted_ll(bpc, data, np.float32([3.0, 1.0]), head_mask=head_mask) - (3 * want[0] + want[1]) / 4) < 1e-5
+    assert P.loglikelihood_probcat is P.loglikelihood and P.loglikelihoods_probcat is P.loglikelihoods
+    with pytest.raises(ValueError, match="head_mask"):
+        P.loglikelihood(bpc, data)
+    with pytest.raises(ValueError, match="3 weights for 2 examples"):
+        P.loglikelihood(bpc, data, np.ones(3, np.float32), head_mask=head_mask)
 
     ll = P.probs_flows_circuit(bpc, data, head_mask=head_mask).cpu().numpy()
     np.testing.assert_allclose(ll, want, rtol=1e-5)
