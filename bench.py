@@ -118,10 +118,8 @@ def secondary(args):
     out = {"n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic", "cpu_baseline": None}
     if args.workload == "c2_hclt48_k128":
-        V, K, C, B = 48, 128, 256, 4096
-        data = workloads.grf_images(B, 4, 4, 3, 2.0, 0.8, seed=1002)
-        parent = workloads.chow_liu_parent(data)
-        theta, leaf = workloads.init_params(parent, K, C, 1102, kind="dirichlet")
+        c2 = workloads.c2_config()
+        V, K, C, B, data, parent, theta, leaf = (c2[k] for k in ("V", "K", "C", "B", "data", "parent", "theta", "leaf"))
         bpc = P.hclt_from_clt(parent, C, K)
         bpc.set_params(theta, leaf)
         d = torch.from_numpy(data).cuda()
@@ -295,34 +293,18 @@ def secondary(args):
         # cluster heads per patch and the K = 64 top-level HCLT over the 64 cluster ids.  c4_full: the 64 patch
         # circuits as ONE forest handle over the 12288 pixels (one launch per kernel for all of them);
         # c4_full_handles: a handle per patch circuit, queued on 32 streams.
-        V, K, C, H, B, NP, NS = 192, 32, 256, 128, 1024, 64, 32
-        img = workloads.grf_images(B, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(B, 3, 64, 64)
-        pixel = np.arange(3 * 64 * 64).reshape(3, 64, 64)
-        pvars = [pixel[:, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8].reshape(V) for p in range(NP)]
-        flat = np.ascontiguousarray(img.reshape(B, -1))
-        cluster = rng.integers(0, H, size=(B, NP)).astype(np.uint8)          # seeded uniform cluster ids
-        parents = [workloads.chow_liu_parent(np.ascontiguousarray(flat[:, pv])) for pv in pvars]
-        params = [workloads.init_params(parents[p], K, C, 2000 + p, kind="dirichlet") for p in range(NP)]
-        tparent = workloads.chow_liu_parent(cluster)
-        top = P.hclt_from_clt(tparent, H, 64)
-        top.set_params(*workloads.init_params(tparent, 64, H, 2100, kind="dirichlet"))
+        c4 = workloads.c4_config()
+        V, K, C, H, B, NP, NS = c4["V"], c4["K"], c4["C"], c4["H"], c4["B"], c4["patches"], 32
+        flat, cluster, pvars, parents, params = c4["data"], c4["cluster"], c4["pvars"], c4["parents"], c4["params"]
+        top = P.hclt_from_clt(c4["top_parent"], H, 64)
+        top.set_params(*c4["top_params"])
         dtop = torch.from_numpy(cluster).cuda()
         ll_top = torch.empty(B, device="cuda")
         n_int = [int((np.bincount(par[par >= 0], minlength=V) > 0).sum()) for par in parents]
         if args.workload == "c4_full":
-            fparent = np.empty(NP * V, np.int32)
-            theta = np.empty((NP * V, K, K), np.float32)
-            leaf = np.empty((NP * V, K, C), np.float32)
-            for pv, par, (th, lf) in zip(pvars, parents, params):
-                fparent[pv] = np.where(par < 0, -1, pv[np.maximum(par, 0)])
-                theta[pv], leaf[pv] = th, lf
-            forest = P.hclt_forest_from_clts(fparent, C, K, H)               # heads stay uniform
-            forest.set_params(theta, leaf)
-            roots = [int(pv[np.flatnonzero(par < 0)[0]]) for pv, par in zip(pvars, parents)]
-            mask = np.zeros((NP, H, B), np.float32)
-            for t, p in enumerate(np.argsort(roots)):                        # trees are numbered by their root's variable
-                mask[t, cluster[:, p], np.arange(B)] = 1.0
-            dmask = torch.from_numpy(mask).cuda()
+            forest = P.hclt_forest_from_clts(c4["fparent"], C, K, H)         # heads stay uniform
+            forest.set_params(c4["theta"], c4["leaf"])
+            dmask = torch.from_numpy(c4["mask"]).cuda()
             d = torch.from_numpy(flat).cuda()
             ll = torch.empty((NP, B), device="cuda")
             streams = [torch.cuda.Stream() for _ in range(2)]

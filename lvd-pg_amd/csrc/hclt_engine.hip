@@ -1015,8 +1015,8 @@ void HcltCircuit::rebuild_heads() {
 void HcltCircuit::heads_forward(const HcltDev& d, const float* d_mask, float* d_ll_heads, float* d_ll_mix, bool flows_follow,
                                 float rate) {
   PCM_DISPATCH_LEAN_K(K_, hipLaunchKernelGGL(hclt_heads_forward_kernel<KK>, dim3(d.nslices, T_), dim3(kHeadWaves * 64), 0,
-                                             stream, d.O, d_root_node_.p, (int64_t)(d.tile_stride / 4), d_head_wf_.p, H_, Hp_,
-                                             d.B, d_mask, d_ll_heads, d_ll_mix,
+                                             stream, d.O, d.M, d.Bp, d_root_node_.p, (int64_t)(d.tile_stride / 4), d_head_wf_.p,
+                                             H_, Hp_, d.B, d_mask, d_ll_heads, d_ll_mix,
                                              flows_follow ? head_aggr() : (float*)nullptr, rate, d_flow_shift_.p));
   check_launch("heads_forward");
 }
@@ -1215,7 +1215,7 @@ void HcltCircuit::ensure_batch(int batch) {
     d_wide_rs_.alloc((size_t)n_inner_ * tile);
     d_wide_es_.alloc((size_t)n_inner_ * tile);
   }
-  if (lean_) d_M_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
+  d_M_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);   // row maxima of the forward walk
   d_xb_.alloc((size_t)V_ * ns * kSlice);
   if (V_ > Vu_) d_xb_.zero(stream);   // the category of an auxiliary variable is always 0
   d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
@@ -1413,9 +1413,8 @@ void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
   stage_batch(b);
   if (wide_walk_) return wide_forward(dev(b.batch), d_ll);
   if (H_ > 0) {   // per-head values [H][batch]
-    d_ll_heads_.ensure((size_t)b.batch);
     const HcltDev d = dev(b.batch);
-    run_forward(d, d_ll_heads_.p);
+    run_forward(d, nullptr);   // (the head kernel reads the root tiles and the row maxima)
     heads_forward(d, nullptr, d_ll, nullptr);
     return;
   }
@@ -1553,8 +1552,7 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
     check_launch("weight_shift");
   }
   if (H_ > 0) {
-    d_ll_heads_.ensure((size_t)b.batch);
-    run_forward(d, d_ll_heads_.p);
+    run_forward(d, nullptr);
     heads_forward(d, d_head_mask, nullptr, d_ll, true, rate);
     const size_t lds = ((size_t)16 * Hp_ + 16 * K_ + (size_t)kHeadWaves * 16 * K_ + (size_t)kHeadWaves * 16) * sizeof(float);
     d_part_.ensure((size_t)T_ * d.nslices * H_ * K_);

@@ -243,7 +243,6 @@ class HcltCircuit : public pcm_circuit {
   int H_ = 0, Hp_ = 0;             // heads, and heads rounded up to whole operand tiles
   DevBuf<float> d_head_wf_, d_head_wb_;   // head block [Hp][K] in the two operand layouts
   DevBuf<int> d_flow_shift_;              // ceil(log2) of the largest flow one example carried in the last flow pass
-  DevBuf<float> d_ll_heads_;       // scratch: the walk's own root output, per-head values
   float* head_logp() { return d_logtheta_.p + (size_t)n_inner_ * K_ * K_; }   // [trees][H][K], behind the blocks
   float* head_aggr() { return d_edge_aggr_.p + (size_t)n_inner_ * K_ * K_; }
   void rebuild_heads();

@@ -3,10 +3,11 @@
 // `pcs` sharing one body; likelihood.jl:3-18, flow.jl:141-176).
 //
 // The body runs through the ordinary walk kernels with the root's parameter block set to the
-// identity, which makes the root tile O_root[b,k] the root's Z[b,k] and turns the root step of
+// identity, which makes the root tile O_root[b,k] the root's Z[b,k] (less the row maxima of the tree's
+// nodes, which the walk keeps apart: `base` below is their sum) and turns the root step of
 // the backward walk into G_root = E .* R_root for whatever R_root it is handed.  Two small
 // kernels per pass do the heads, one workgroup per 16-example slice:
-//   forward   ll[h][b] = m + log sum_j Wh[h,j] E[b,j],  E = exp(Z - m)   (+ the mask-weighted mixture)
+//   forward   ll[h][b] = base + m + log sum_j Wh[h,j] E[b,j],  E = exp(Z - m)   (+ the mask-weighted mixture)
 //   backward  R[b,h] = mask[h][b] / S[b,h],  T[b,j] = sum_h Wh[h,j] R[b,h]  -> stored as R_root;
 //             head_aggr[h,j] += Wh[h,j] * sum_b R[b,h] E[b,j]
 // The statistics kernel then finds R_root = T like any other node's ratio tile and histograms
@@ -79,6 +80,7 @@ __device__ __forceinline__ v4f heads_contract_f(const float* __restrict__ hwf, i
 //   logsumexp_h(ll_h + log mask_h) - log sum_h mask_h   (src-jl/multi_head_pc/likelihood.jl:3-12).
 template <int K>
 __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(const float* __restrict__ O,
+                                                                             const float* __restrict__ M, int Bp,
                                                                              const int32_t* __restrict__ root_node,
                                                                              int64_t tile_floats,
                                                                              const float* __restrict__ hwf, int H, int Hp,
@@ -88,6 +90,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
                                                                              float* __restrict__ head_aggr, float rate,
                                                                              int* __restrict__ flow_shift) {
   __shared__ float pm[kHeadWaves * 4][16], ps[kHeadWaves * 4][16], pt[kHeadWaves * 4][16];
+  __shared__ double pb[kHeadWaves * 4][16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, slice = blockIdx.x, tree = blockIdx.y;
   const float* __restrict__ O_root = O + (size_t)root_node[tree] * tile_floats;
   hwf += (size_t)tree * Hp * K;
@@ -101,6 +104,19 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
     if (blockIdx.x == 0 && threadIdx.x == 0) *flow_shift = 0;
   }
   const int b = lane & 15, g = lane >> 4, col = slice * kSlice + b;
+  // base: the row maxima of the tree's nodes (post-order goes tree after tree: the nodes after the root before
+  // up to this tree's root), every sixteenth node per group of lanes, the groups' sums added in order
+  double base;
+  {
+    const int n_lo = tree > 0 ? root_node[tree - 1] + 1 : 0, n_hi = root_node[tree];
+    double acc = 0.0;
+    for (int n = n_lo + wave * 4 + g; n <= n_hi; n += kHeadWaves * 4) acc += (double)M[(size_t)n * Bp + col];
+    pb[wave * 4 + g][b] = acc;
+    __syncthreads();
+    base = 0.0;
+#pragma unroll
+    for (int q = 0; q < kHeadWaves * 4; ++q) base += pb[q][b];
+  }
   Tile<K> e;
   const float m = heads_load_e<K>(O_root, slice, lane, e);
   float mx = -INFINITY, sm = 0.f, tot = 0.f;   // running mixture over this lane's heads
@@ -110,7 +126,7 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_forward_kernel(con
     for (int i = 0; i < 4; ++i) {
       const int h = ht * 16 + 4 * g + i;
       if (h >= H || col >= B) continue;
-      const float val = m + __logf(s[i]);
+      const float val = (float)(base + (double)(m + __logf(s[i])));
       if (ll_heads) ll_heads[(size_t)h * B + col] = val;
       if (mask) {
         const float mk = mask[(size_t)h * B + col];

@@ -335,9 +335,11 @@ __device__ __forceinline__ PreRegs sched_pre(const SchedChunk& c, int step) {
 // empty buffer descriptors), so the waits the compiler places count exactly the requests
 // that must have landed and never the ones just issued.
 //
-// ---- forward: O_v = m + log(E W^T), E = exp(Z - m) ------------------------------------
+// ---- forward: O'_v = log(E W^T), E = exp(Z' - m) ---------------------------------------
 // Static operands: the node's own leaf row and its leaf children's rows.  Dependencies:
 // the value tiles of its inner children, read from their LDS slots (kSpill: or from HBM).
+// The tiles hold log S only; the row maxima m_v go to d.M (when it is there) and their sum over all
+// nodes is added to the root's tile value for the log-likelihood: see hclt_forward_lean_kernel.
 template <int K, bool kSpill>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
     HcltDev d, const int32_t* __restrict__ fields, int stride, const StepItem* __restrict__ sched,
@@ -363,6 +365,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
     xs = xpack_load(d, q1.wnode, bcol);
   }
   float ll = 0.f;
+  double msum = 0.0;
 
   for (int s = 0; s < n_steps; ++s) {
     if (s - sc.base >= 61) sched_refill(fields, stride, wave, lane, s, sc);
@@ -403,18 +406,32 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_kernel(
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o.v[kt][i] = fmaf(__builtin_amdgcn_logf(o.v[kt][i]), kLn2, m);
+      for (int i = 0; i < 4; ++i) o.v[kt][i] = __builtin_amdgcn_logf(o.v[kt][i]) * kLn2;
     tile_store<K>(d.O, node, d.tile_stride, lo.tile, o);
     lds_tile_store<K>(lds, out_slot, lane, o);
+    if (node >= 0) {   // (idle waves have no node)
+      msum += (double)m;
+      if (d.M && lane < 16) d.M[(size_t)node * d.Bp + bcol] = m;
+    }
     if (flags & kItemRoot) ll = o.v[0][0];
     step_barrier<kSpill>();
   }
-  if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
+  if (!ll_out) return;
+  // the waves' sums of row maxima, added in wave order (the last step's barrier has freed the slots)
+  double* part = reinterpret_cast<double*>(lds);
+  if (lane < 16) part[wave * 16 + lane] = msum;
+  __syncthreads();
+  if (wave == 0 && lane < 16 && bcol < d.B) {   // the root is item 0 of the last step
+    double tot = 0.0;
+#pragma unroll
+    for (int w = 0; w < kWalkWaves; ++w) tot += part[w * 16 + lane];
+    ll_out[bcol] = (float)(tot + (double)ll);
+  }
 }
 
 // ---- backward: R_v = F_v / S_v, G_v = E_v .* (R_v W_v) ----------------------------------
 // Static operands: own leaf row, children's value tiles, leaf children's rows (-> E_v), and
-// the node's own value tile O_v (-> S_v = exp(O_v - m)).  Dependency: F_v = G_parent from
+// the node's own value tile O'_v (-> S_v = exp(O'_v)).  Dependency: F_v = G_parent from
 // its LDS slot.  R_v goes to HBM for the statistics kernel, G_v to an LDS slot for the
 // children (kSpill: to HBM when no slot was free).
 // kHeads: multi-head circuit; the head kernel has left the root's ratio tile in memory.
@@ -472,7 +489,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i)   // capped: a state (or a whole example) of probability zero has flow 0, not 0 * inf
-        r.v[kt][i] *= fminf(__builtin_amdgcn_exp2f(fmaf(ov.v[kt][i], -kLog2e, m * kLog2e)), kFlowRatioCap);
+        r.v[kt][i] *= fminf(__builtin_amdgcn_exp2f(ov.v[kt][i] * -kLog2e), kFlowRatioCap);
     if (flags & kItemRoot) {
       if (kHeads) {   // the heads' flows, already divided by their sums
         tile_load<K>(d.R, node, d.tile_stride, lo.tile, r);
@@ -480,7 +497,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_kernel(
         tile_zero<K>(r);
         const bool live = lane < 16 && bcol < d.B;
         const float wgt = (d.w && live) ? d.w[bcol] : 1.f;   // per-example weights: the flow the example starts with
-        r.v[0][0] = live ? wgt * fminf(__builtin_amdgcn_exp2f((m - ov.v[0][0]) * kLog2e), kFlowRatioCap) : 0.f;
+        r.v[0][0] = live ? wgt * fminf(__builtin_amdgcn_exp2f(ov.v[0][0] * -kLog2e), kFlowRatioCap) : 0.f;
       }
     }
     tile_store<K>(d.R, node, d.tile_stride, lo.tile, r);

@@ -128,6 +128,13 @@ __device__ __forceinline__ void lean_post(unsigned* state, unsigned value) {
 }
 
 // ---- forward ------------------------------------------------------------------------------
+// A node's value is kept in two parts: the tile holds O'_v[k] = log S_v[k] = log sum_j W[k,j] exp(Z'_v[j] - m_v), numbers
+// of order one, and the row of maxima holds m_v = max_j Z'_v[j], where Z'_v is the sum of the node's leaf rows and of its
+// inner children's TILES (not of their full values).  The full value is O'_v[k] plus the maxima of all nodes of the
+// subtree, a number that grows with the size of the subtree and is the same for all K states: nothing below needs it
+// but the log-likelihood at the root.  Stored as one float32 it would cost every state of a 3000-variable circuit
+// (values near -14000) an absolute error of 1e-3, which is a relative error of 1e-3 on every flow; in two parts the
+// flows keep float32's relative accuracy at any depth.
 template <int K>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     HcltDev d, const int32_t* __restrict__ fields, int stride, int n_steps, float* __restrict__ ll_out, int n_slots) {
@@ -173,6 +180,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
   }
   float ll = 0.f;
+  double msum = 0.0;   // sum of the row maxima of this wave's nodes: the part of the log-likelihood the tiles leave out
   Tile<K> o_prev;   // the value tile of the previous step, stored at the top of the next one
   tile_zero<K>(o_prev);
   int store_prev = d.n_inner * (int)d.tile_stride;
@@ -221,12 +229,14 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o.v[kt][i] = fmaf(__builtin_amdgcn_logf(o.v[kt][i]), kLn2, m);
+      for (int i = 0; i < 4; ++i) o.v[kt][i] = __builtin_amdgcn_logf(o.v[kt][i]) * kLn2;
     lean_w_load<K>(rW, vtile, lean_get(sc, kLW, s + 2), w);   // the block of step s+2, same registers
     o_prev = o;
-    store_prev = lean_get(sc, kLNode, s) * (int)d.tile_stride;
+    const int node = lean_get(sc, kLNode, s);
+    store_prev = node * (int)d.tile_stride;
     m_prev = m;
-    mrow_prev = lean_get(sc, kLNode, s) * xrow;
+    mrow_prev = node * xrow;
+    if (node != d.n_inner) msum += (double)m;   // (idle steps work on the trash tile)
     {
       // idle steps and the root write the trash slot, which nobody reads: no hand-over there
       const uint32_t so = slots & 0xffu, tn = turns & 0x7fu;
@@ -251,19 +261,31 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
   }
   lean_tile_store<K, PCM_ST_O>(rO, vtile, store_prev, o_prev);
   __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, m_prev), rM, (int)vm, mrow_prev, kStreamStore);
-  if (ll_out && wave == 0 && lane < 16 && bcol < d.B) ll_out[bcol] = ll;   // the root is item 0 of the last step
+  // log-likelihood of a single-root circuit: the root's (scaled) value plus the row maxima of all nodes, the
+  // waves' sums added in wave order (a multi-head circuit's head kernel adds up the stored maxima per tree)
+  if (!ll_out) return;
+  __syncthreads();   // every wave is through its steps: the slots are free
+  double* part = reinterpret_cast<double*>(lds);
+  if (lane < 16) part[wave * 16 + lane] = msum;
+  __syncthreads();
+  if (wave == 0 && lane < 16 && bcol < d.B) {   // the root is item 0 of the last step
+    double tot = 0.0;
+#pragma unroll
+    for (int w = 0; w < kWalkWaves; ++w) tot += part[w * 16 + lane];
+    ll_out[bcol] = (float)(tot + (double)ll);
+  }
 }
 
 // ---- backward -----------------------------------------------------------------------------
 // What travels down the tree through LDS is not the flow of a child's sum nodes but already their
-// ratio tile R_c = F_c / S_c, built by the parent: with t = W_v^T R_v, F_c = G_v = exp(Z_v - M_v) .* t
-// and S_c = exp(O_c - M_c),
-//   R_c[j] = t[j] * exp((Z_v[j] - O_c[j]) + (M_c - M_v)),
-// where Z_v - O_c is the sum of v's OTHER operands (own leaf row, leaf children, further inner
-// children): the child's own values cancel, so a node never reads its own value tile, and the
-// exponent is formed from small numbers (M_c - M_v is exact when the two lie within a factor of
-// two).  M are the row maxima the forward walk stored.  A state the child gives probability zero
-// (O_c = -inf) has flow 0 and keeps ratio 0.  A node without inner children only stores its tile.
+// ratio tile R_c = F_c / S_c, built by the parent: with t = W_v^T R_v, F_c = G_v = exp(Z'_v - m_v) .* t
+// and S_c = exp(O'_c) (the tiles hold log S, see the forward walk),
+//   R_c[j] = t[j] * exp((Z'_v[j] - O'_c[j]) - m_v),
+// where Z'_v - O'_c is the sum of v's OTHER operands (own leaf row, leaf children, further inner
+// children's tiles): the child's own values cancel, so a node never reads its own value tile, and the
+// exponent is formed from small numbers.  m_v are the row maxima the forward walk stored.  A state the
+// child gives probability zero (O'_c = -inf) has flow 0 and keeps ratio 0.  A node without inner children
+// only stores its tile.
 // kHeads: multi-head circuit, whose head kernel has left the root's ratio tile in memory.
 template <int K, bool kHeads>
 __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
@@ -289,14 +311,10 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
       make_rsrc(d.M + (size_t)slice * kSlice, (uint32_t)(d.n_inner + 1) * (uint32_t)d.Bp * 4u - (uint32_t)slice * (kSlice * 4));
   const int xrow = d.Bp * 4;
 
-  // a child operand: value tile (and row maxima) of an inner child, or leaf row of a leaf child
-  auto child_load = [&](int c, uint32_t xpack, Tile<K>& t, float& mc) {
-    if (c & 1) {
-      lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), c & ~7, t);
-    } else {
-      lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride, t);
-      mc = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, (c >> 3) * xrow, 0));
-    }
+  // a child operand: value tile of an inner child, or leaf row of a leaf child
+  auto child_load = [&](int c, uint32_t xpack, Tile<K>& t) {
+    if (c & 1) lean_row_load<K>(rL, lean_row_off<K>(xpack, (c >> 1) & 3, vleaf), c & ~7, t);
+    else lean_tile_load<K>(rO, vtile, (c >> 3) * (int)d.tile_stride, t);
   };
   auto is_inner = [](int c) { return c >= 0 && !(c & 1); };
 
@@ -307,25 +325,25 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
   WTile<K> wA, wB;
   uint32_t xs;
   int c1, c2, c3;
-  float mv, m1 = 0.f, m2 = 0.f, m3 = 0.f;
+  float mv;
   {
     const uint32_t x0 = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0);
     xs = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rX, (int)vx, lean_get(sc, kLNode, 1) * xrow, 0);
     mv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, lean_get(sc, kLNode, 0) * xrow, 0));
     lean_row_load<K>(rL, lean_row_off<K>(x0, 0, vleaf), lean_get(sc, kLA0, 0), P0);
     c1 = lean_get(sc, kLA1, 0); c2 = lean_get(sc, kLA2, 0); c3 = lean_get(sc, kLA3, 0);
-    if (c1 >= 0) child_load(c1, x0, C1, m1);
-    if (c2 >= 0) child_load(c2, x0, C2, m2);
-    if (c3 >= 0) child_load(c3, x0, C3, m3);
+    if (c1 >= 0) child_load(c1, x0, C1);
+    if (c2 >= 0) child_load(c2, x0, C2);
+    if (c3 >= 0) child_load(c3, x0, C3);
     // (a node without inner children has no use for its parameter block)
     if (is_inner(c1)) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 0), wA);
     if (is_inner(lean_get(sc, kLA1, 1))) lean_w_load<K>(rW, vtile, lean_get(sc, kLW, 1), wB);
   }
 
-  // exponent tile of inner child `own` among the landed operands: the other operands plus M_c - M_v,
+  // exponent tile of inner child `own` among the landed operands: the other operands minus m_v,
   // in base-2 units; -inf where the child's own value is -inf
-  auto exponent = [&](const Tile<K>& own, float mc, bool has_a, const Tile<K>& a, bool has_b, const Tile<K>& b, Tile<K>& x) {
-    const float dm = (mc - mv) * kLog2e;
+  auto exponent = [&](const Tile<K>& own, bool has_a, const Tile<K>& a, bool has_b, const Tile<K>& b, Tile<K>& x) {
+    const float dm = -mv * kLog2e;
 #pragma unroll
     for (int kt = 0; kt < K / 16; ++kt)
 #pragma unroll
@@ -348,18 +366,17 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
       if (in3) lean_wait(state + ((slots >> 24) & 0xffu), (2 * ((turns >> 24) & 0x7fu)) & 0xffu, d.err);
     }
     Tile<K> X1;
-    if (in1) exponent(C1, m1, c2 >= 0, C2, c3 >= 0, C3, X1);
+    if (in1) exponent(C1, c2 >= 0, C2, c3 >= 0, C3, X1);
     if (in2) {
       Tile<K> x;
-      exponent(C2, m2, true, C1, c3 >= 0, C3, x);
+      exponent(C2, true, C1, c3 >= 0, C3, x);
       lds_tile_store<K>(lds, (int)((slots >> 16) & 0xffu), lane, x);
     }
     if (in3) {
       Tile<K> x;
-      exponent(C3, m3, true, C1, true, C2, x);
+      exponent(C3, true, C1, true, C2, x);
       lds_tile_store<K>(lds, (int)((slots >> 24) & 0xffu), lane, x);
     }
-    const float mroot = mv;
     // (2) request the operands of step s+1 and the categories of step s+2
     {
       const uint32_t xc = xs;
@@ -367,9 +384,9 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
       mv = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rM, (int)vx, lean_get(sc, kLNode, s + 1) * xrow, 0));
       lean_row_load<K>(rL, lean_row_off<K>(xc, 0, vleaf), lean_get(sc, kLA0, s + 1), P0);
       c1 = lean_get(sc, kLA1, s + 1); c2 = lean_get(sc, kLA2, s + 1); c3 = lean_get(sc, kLA3, s + 1);
-      if (c1 >= 0) child_load(c1, xc, C1, m1);
-      if (c2 >= 0) child_load(c2, xc, C2, m2);
-      if (c3 >= 0) child_load(c3, xc, C3, m3);
+      if (c1 >= 0) child_load(c1, xc, C1);
+      if (c2 >= 0) child_load(c2, xc, C2);
+      if (c3 >= 0) child_load(c3, xc, C3);
     }
     // (3) this node's ratio tile: left in LDS by the parent (the root and idle steps read the trash slot)
     Tile<K> r;
@@ -380,12 +397,12 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     const int fl = lean_get(sc, kLFlags, s);
     if (kHeads && (fl & 2)) {   // multi-head circuit: the head kernel has left the root's ratio tile in memory
       lean_tile_load<K>(rR, vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, r);
-    } else if (fl & 1) {   // flow 1 into the single root sum node of every live example: R = 1 / S = exp(M - O)
+    } else if (fl & 1) {   // flow 1 into the single root sum node of every live example: R = 1 / S = exp(-O')
       const float o00 = __builtin_bit_cast(
           float, __builtin_amdgcn_raw_buffer_load_b32(rO, (int)vtile, lean_get(sc, kLNode, s) * (int)d.tile_stride, 0));
       const bool live = lane < 16 && bcol < d.B;
       const float wgt = (d.w && live) ? d.w[bcol] : 1.f;   // per-example weights: the flow the example starts with
-      const float r00 = live ? wgt * fminf(__builtin_amdgcn_exp2f(fmaf(o00, -kLog2e, mroot * kLog2e)), kFlowRatioCap) : 0.f;
+      const float r00 = live ? wgt * fminf(__builtin_amdgcn_exp2f(o00 * -kLog2e), kFlowRatioCap) : 0.f;
       tile_zero<K>(r);
       r.v[0][0] = r00;
     }

@@ -13,9 +13,11 @@
 //
 // Algebra per tree node (reference: src/queries/likelihood.jl:4-68, src/queries/flow.jl:8-106,
 // :165-195 on the K^2 sum edges of src/structures/hclts.jl:133):
-//   Z = leaf rows + children's values, m = max_j Z, E = exp(Z - m)
-//   O[k] = m + log(sum_j W[k,j] E[j])                              forward
-//   R[k] = F[k] / exp(O[k] - m),  G[j] = E[j] * sum_k W[k,j] R[k]   backward (F = parent's G, root: e_0)
+//   Z = leaf rows + children's tiles, m = max_j Z, E = exp(Z - m)
+//   O[k] = log(sum_j W[k,j] E[j])                                  forward: the tiles hold log S, numbers of order one;
+//                                                                  a node's full value is O[k] plus the maxima m of its
+//                                                                  whole subtree, which only the log-likelihood needs
+//   R[k] = F[k] / exp(O[k]),  G[j] = E[j] * sum_k W[k,j] R[k]       backward (F = parent's G, root: e_0)
 //   edge_aggr[k,j] += W[k,j] * sum_b R[b,k] E[b,j];  leaf_flow[u][x_b,u][j] += G[b,j]
 #include <hip/hip_ext.h>
 
@@ -238,6 +240,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_k
   request(0, d.xn[col]);
 #pragma unroll
   for (int q = 0; q < Q; ++q) prev_o[q] = v4f{0.f, 0.f, 0.f, 0.f};
+  double msum = 0.0;   // row maxima of all nodes so far: what the tiles leave out of the root's value
   for (int n = 0; n < d.n_inner; ++n) {
     const WideOps on = on_next;
     v4f z[Q], w[Q][KT];
@@ -257,6 +260,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_k
     if (on.fwd_extra_cnt) wide_extras<K>(d, extra, on.fwd_extra_off, on.fwd_extra_cnt, s, lane, wave, z);
     v4f e[KT];
     const float m = wide_e_from_z<K>(z, lane, wave, L, e);
+    msum += (double)m;
     v4f* out = reinterpret_cast<v4f*>(d.O + ((size_t)n * d.nslices + s) * kSlice * K);
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -270,10 +274,10 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_forward_k
       const v4f acc = (part[0] + part[1]) + (part[2] + part[3]);
       v4f o;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) o[i] = m + __logf(acc[i]);
+      for (int i = 0; i < 4; ++i) o[i] = __logf(acc[i]);
       out[(wave * Q + q) * 64 + lane] = o;
       prev_o[q] = o;
-      if (on.is_root && wave == 0 && q == 0 && g == 0 && col < d.B) ll[col] = o[0];
+      if (on.is_root && wave == 0 && q == 0 && g == 0 && col < d.B) ll[col] = (float)(msum + (double)o[0]);
     }
     // no barrier here: a wave reads from memory only what it wrote itself, and the next node's LDS
     // writes sit behind its own barriers
@@ -348,7 +352,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
     request(max(n - 1, 0), xcur);   // past the last node: a repeat of its requests, never used
     if (on.bwd_extra_cnt) wide_extras<K>(d, extra, on.bwd_extra_off, on.bwd_extra_cnt, s, lane, wave, z);
     v4f e[KT];
-    const float m = wide_e_from_z<K>(z, lane, wave, L, e);
+    wide_e_from_z<K>(z, lane, wave, L, e);
     const size_t tile = ((size_t)n * d.nslices + s) * kSlice * K;
 #pragma unroll
     for (int q = 0; q < Q; ++q) {
@@ -361,7 +365,7 @@ __global__ __launch_bounds__(wide_walk_waves<K>() * 64) void hclt_wide_backward_
       v4f r;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float sc = __expf(o[q][i] - m);
+        const float sc = __expf(o[q][i]);
         r[i] = (sc > 0.f && fq[i] > 0.f) ? fq[i] / sc : 0.f;
       }
       L.r[kt][lane] = r;

@@ -138,3 +138,47 @@ def make_config(name, tree="gaussian"):
         raise ValueError("tree: 'gaussian' or 'chow_liu'")
     theta, leaf = init_params(parent, K, C, seed + 100)
     return dict(name=name, data=data, parent=parent, theta=theta, leaf=leaf, K=K, C=C, B=B, V=h * w * ch)
+
+
+def c2_config():
+    """The K = 128 configuration: 48 variables (one 4x4x3 patch, 256 categories), Dirichlet(1) parameters, batch
+    4096 of smoothed-random-field patches with channel correlation 0.8."""
+    V, K, C, B = 48, 128, 256, 4096
+    data = grf_images(B, 4, 4, 3, 2.0, 0.8, seed=1002)
+    parent = chow_liu_parent(data)
+    theta, leaf = init_params(parent, K, C, 1102, kind="dirichlet")
+    return dict(name="c2_hclt48_k128", data=data, parent=parent, theta=theta, leaf=leaf, K=K, C=C, B=B, V=V)
+
+
+def c4_config(batch=1024):
+    """The patch-clustered configuration: 64 x 64 x 3 images cut into 64 patches of 8 x 8 x 3; one 192-variable
+    K = 32 circuit with 128 cluster heads per patch, all of them as one forest over the 12288 pixels, seeded
+    uniform cluster ids per (image, patch), and the K = 64 top-level tree over the 64 cluster ids.
+    Returns the per-patch pieces (`pvars`, `parents`, `params`) and the forest's arrays: `fparent` (64 roots),
+    `theta`, `leaf` indexed by pixel, `mask` [trees][heads][batch] one-hot in the forest's tree order (trees are
+    numbered by their root's variable), `tree_patch[t]` = the patch tree t covers."""
+    V, K, C, H, NP = 192, 32, 256, 128, 64
+    rng = np.random.default_rng(0)
+    img = grf_images(batch, 64, 64, 3, 3.0, 0.8, seed=1004).reshape(batch, 3, 64, 64)
+    pixel = np.arange(3 * 64 * 64).reshape(3, 64, 64)
+    pvars = [pixel[:, 8 * (p // 8):8 * (p // 8) + 8, 8 * (p % 8):8 * (p % 8) + 8].reshape(V) for p in range(NP)]
+    flat = np.ascontiguousarray(img.reshape(batch, -1))
+    cluster = rng.integers(0, H, size=(batch, NP)).astype(np.uint8)
+    parents = [chow_liu_parent(np.ascontiguousarray(flat[:, pv])) for pv in pvars]
+    params = [init_params(parents[p], K, C, 2000 + p, kind="dirichlet") for p in range(NP)]
+    nv = flat.shape[1]
+    fparent = np.empty(nv, np.int32)
+    theta = np.zeros((nv, K, K), np.float32)
+    leaf = np.zeros((nv, K, C), np.float32)
+    for pv, par, (th, lf) in zip(pvars, parents, params):
+        fparent[pv] = np.where(par < 0, -1, pv[np.maximum(par, 0)])
+        theta[pv], leaf[pv] = th, lf
+    roots = [int(pv[np.flatnonzero(par < 0)[0]]) for pv, par in zip(pvars, parents)]
+    tree_patch = np.argsort(roots)
+    mask = np.zeros((NP, H, batch), np.float32)
+    for t, p in enumerate(tree_patch):
+        mask[t, cluster[:, p], np.arange(batch)] = 1.0
+    tparent = chow_liu_parent(cluster)
+    return dict(V=V, K=K, C=C, H=H, B=batch, patches=NP, data=flat, cluster=cluster, pvars=pvars, parents=parents,
+                params=params, fparent=fparent, theta=theta, leaf=leaf, mask=mask, tree_patch=tree_patch,
+                top_parent=tparent, top_params=init_params(tparent, 64, H, 2100, kind="dirichlet"))

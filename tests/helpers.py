@@ -39,9 +39,9 @@ def correlated_data(N, V, C, seed, parent=None):
     return x.astype(np.uint8)
 
 
-def oracle_em_reference(fc, data, idx, pseudocount, inertia):
+def oracle_em_reference(fc, data, idx, pseudocount, inertia, double=False):
     """One EM step on the oracle; returns LL, theta blocks, leaf [V,K,C], edge_aggr blocks, leaf flows."""
-    ll, logp, leaf, ea, lf = O.em_step(fc, data, idx, pseudocount, inertia)
+    ll, logp, leaf, ea, lf = O.em_step(fc, data, idx, pseudocount, inertia, double=double)
     K, C, V = fc.meta["K"], fc.C, fc.V
     new = fc.copy()
     new.logp = logp
@@ -54,6 +54,35 @@ def rel_err(a, b, floor=1e-30):
     a = np.asarray(a, np.float64)
     b = np.asarray(b, np.float64)
     return np.abs(a - b) / np.maximum(np.abs(b), floor)
+
+
+def three_way(got, exact, single):
+    """Worst relative distances, as probabilities, between three sets of log-parameters: (library vs float64
+    oracle, float32 oracle vs float64 oracle, library vs float32 oracle).  Each argument is (theta blocks by
+    tree node -- the library's as a dense array --, leaf tables)."""
+    def rel(a, b):
+        a, b = np.exp(np.asarray(a, np.float64)), np.exp(np.asarray(b, np.float64))
+        return float((np.abs(a - b) / b).max())
+    (th, lf), (th64, lf64), (th32, lf32) = got, exact, single
+    sums = (max(rel(th[v][:b.shape[0]], b) for v, b in th64.items()),
+            max(rel(th32[v], b) for v, b in th64.items()),
+            max(rel(th[v][:b.shape[0]], th32[v]) for v, b in th64.items()))
+    leaves = (rel(lf, lf64), rel(lf32, lf64), rel(lf, lf32))
+    return sums, leaves
+
+
+def assert_three_way(got, exact, single, bar, label=""):
+    """The library must be within `bar` of the exact (float64) result, whatever the float32 oracle -- the
+    reference's arithmetic, whose log-values lose absolute precision with the depth of the circuit -- manages, and
+    where the two float32 results are further apart than `bar`, the float32 oracle's own error must account for
+    it (the distances obey the triangle inequality up to the different denominators)."""
+    sums, leaves = three_way(got, exact, single)
+    print(f"\n{label}: sum parameters library/f64 {sums[0]:.2e} f32/f64 {sums[1]:.2e} library/f32 {sums[2]:.2e}; "
+          f"leaf parameters {leaves[0]:.2e} {leaves[1]:.2e} {leaves[2]:.2e}")
+    for e_gpu, e_f32, e_gpu32 in (sums, leaves):
+        assert e_gpu < bar, (label, sums, leaves)
+        assert e_gpu32 < max(bar, 1.01 * (e_gpu + e_f32)), (label, sums, leaves)
+    return sums, leaves
 
 
 def describe_dag(roots):

@@ -58,11 +58,11 @@ def test_full_batch_step_properties_and_oracle_subset(c3, oracle):
     llb = torch.empty(sub, device="cuda")
     L.check(L.lib.pcm_em_step(bpc.handle, data.data_ptr(), data.stride(0), data.stride(1), ids.data_ptr(), sub, 0.0,
                               0.1, 0.9, llb.data_ptr()))
-    # At this depth (114 tree levels, sub-circuit log-values of several thousand) float32 log-space
-    # arithmetic itself is only good to ~1e-3 relative on the smallest flows: the float32 oracle,
-    # i.e. the reference's arithmetic, misses the float64 result by that much on a few of the
-    # 27 M parameters.  The library must be within 1e-4 of the float64 result or, where float32
-    # cannot be, no further from it than twice the float32 oracle is.
+    # At this depth (132 tree levels, sub-circuit log-values of several thousand) float32 log-values, the reference's
+    # arithmetic, are only good to ~1e-3 absolute, which is a relative error of 1e-3 on the smallest flows: the
+    # float32 oracle misses the float64 result by 2.5e-3 on a few of the 27 M parameters.  The library keeps node
+    # values in two parts (order-one tiles + per-example maxima) and must be within 1e-4 of the float64 result;
+    # what separates it from the float32 oracle must be that oracle's own error.
     ids_np = np.arange(sub, dtype=np.int32)
     _, logp64, leaf64, _, _ = O.em_step(fc, cfg["data"], ids_np, 0.1, 0.9, double=True)
     _, logp32, leaf32, _, _ = O.em_step(fc, cfg["data"], ids_np, 0.1, 0.9)
@@ -73,33 +73,13 @@ def test_full_batch_step_properties_and_oracle_subset(c3, oracle):
         new.logp, new.leaf_logp = logp, leaf
         return O.hclt_block_params(new)
 
+    from helpers import assert_three_way
     th64, lf64 = blocks(logp64, leaf64)
     th32, lf32 = blocks(logp32, leaf32)
-    rel = lambda a, b: (np.abs(np.exp(np.asarray(a, np.float64)) - np.exp(b)) / np.exp(b)).max()
-    e_gpu = max(rel(th[v][:b.shape[0]], b) for v, b in th64.items())
-    e_f32 = max(rel(th32[v], b) for v, b in th64.items())
-    e_gpu32 = max(rel(th[v][:b.shape[0]], th32[v].astype(np.float64)) for v, b in th64.items())
-    print(f"sum parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}, "
-          f"library vs float32 oracle {e_gpu32:.2e}")
-    assert e_gpu < max(PARAM_RTOL, 2 * e_f32)
-    # against the float32 oracle -- the reference's own arithmetic -- the two float32 results may be
-    # apart by the sum of their distances from the exact one and no more
-    assert e_gpu32 < max(PARAM_RTOL, e_gpu + e_f32)
-    e_gpu, e_f32 = rel(lf_new, lf64), rel(lf32, lf64)
-    e_gpu32 = rel(lf_new, lf32.astype(np.float64))
-    print(f"leaf parameters: library vs float64 {e_gpu:.2e}, float32 oracle vs float64 {e_f32:.2e}, "
-          f"library vs float32 oracle {e_gpu32:.2e}")
-    assert e_gpu < max(PARAM_RTOL, 2 * e_f32)
-    assert e_gpu32 < max(PARAM_RTOL, e_gpu + e_f32)
+    assert_three_way((th, lf_new), (th64, lf64), (th32, lf32), PARAM_RTOL, "3072 variables, 96 examples")
     # the per-example log-likelihoods of the step against the float32 oracle, at the bar itself
     ll32 = O.forward(fc, cfg["data"][:sub])[-1]
     assert (np.abs(llb.cpu().numpy() - ll32) / np.abs(ll32)).max() < LL_RTOL
-    # (log-values near the root are ~ -14000, where one float32 ulp is 1e-3: a sizeable share of
-    # the flows carries that error in any float32 implementation)
-    frac = lambda a: (np.abs(np.exp(np.asarray(a, np.float64)) - np.exp(lf64)) / np.exp(lf64) > PARAM_RTOL).mean()
-    f_gpu, f_f32 = frac(lf_new), frac(lf32)
-    print(f"share of leaf parameters off by more than 1e-4: library {f_gpu:.3f}, float32 oracle {f_f32:.3f}")
-    assert f_gpu < 1.5 * f_f32 + 1e-4
     bpc.set_params(cfg["theta"], cfg["leaf"])
 
 
@@ -227,3 +207,132 @@ def test_kl_gradient_feeds_an_adam_step_on_the_benchmark_circuit(c3, oracle):
     # divergence must come out unchanged, which checks the normalisation at full size)
     after = P.kld(bpc, q)
     assert abs(after - before) < 1e-5 * before
+
+
+def test_c2_em_step_at_its_real_shape(oracle):
+    """The K = 128 configuration at its real shape (48 variables, 256 categories, batch 4096, wide block kernels):
+    one EM step on the first 128 examples against the oracle -- log-likelihoods, `edge_aggr`, leaf flows and the
+    updated parameters in the order of reg_em.jl:276-299 -- and on the whole batch the flow every example sends
+    through every variable and every tree node."""
+    import torch
+    import pcmi355 as P
+    import pcmi355._lib as L
+    from pcmi355 import workloads
+    from helpers import rel_err, assert_three_way
+    O = oracle
+    c2 = workloads.c2_config()
+    V, K, C, B, data, parent = (c2[k] for k in ("V", "K", "C", "B", "data", "parent"))
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(c2["theta"], c2["leaf"])
+    assert bpc.size("walk_kernels") == 3
+    ch, _ = O.clt_children(parent)
+    fc = O.hclt_flat(parent, K, C, {v: c2["theta"][v] for v in range(V) if ch[v]}, c2["leaf"])
+    d = torch.from_numpy(data).cuda()
+    sub = 128
+    ids = np.arange(sub, dtype=np.int32)
+    ll_ref, logp, leaf_new, ea_ref, lf_ref = O.em_step(fc, data, ids, 0.1, 0.9)
+    ll = P.probs_flows_circuit(bpc, d[:sub].contiguous()).cpu().numpy()
+    assert rel_err(ll, ll_ref).max() < LL_RTOL
+    ea, lf = bpc.get_flows()
+    for v, blk in O.hclt_block_aggr(fc, ea_ref).items():
+        nk = blk.shape[0]
+        assert np.abs(ea[v][:nk] - blk).max() < 2e-4 * max(blk.max(), 1e-3), f"edge_aggr block {v}"
+    lf_ref = lf_ref.reshape(V, K, C)
+    assert np.abs(lf - lf_ref).max() < 2e-4 * max(lf_ref.max(), 1e-3)
+    L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.9))
+    th, lp = bpc.get_params()
+    # updated parameters, three-way: with Dirichlet(1) parameters and 128 hidden states most leaf counts of 128
+    # examples are tiny, and float32 flows (the reference's type) are themselves a little over 1e-4 from exact there
+    def blocks(lg, lf_):
+        new = fc.copy()
+        new.logp, new.leaf_logp = lg, lf_
+        return O.hclt_block_params(new)
+    _, logp64, leaf64, _, _ = O.em_step(fc, data, ids, 0.1, 0.9, double=True)
+    assert_three_way((th, lp), blocks(logp64, leaf64), blocks(logp, leaf_new), PARAM_RTOL, "C2, 128 examples")
+    # the whole batch
+    bpc.set_params(c2["theta"], c2["leaf"])
+    ll_all = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    np.testing.assert_array_equal(ll_all[:sub], ll)
+    ea, lf = bpc.get_flows()
+    np.testing.assert_allclose(lf.sum(axis=(1, 2)), B, rtol=1e-4)
+    inner = np.array([v for v in range(V) if ch[v]])
+    np.testing.assert_allclose(ea[inner].sum(axis=(1, 2)), B, rtol=1e-4)
+    assert (ea >= 0).all() and (lf >= 0).all()
+
+
+def test_c4_forest_as_the_benchmark_builds_it(oracle):
+    """The patch layer of the patch-clustered configuration exactly as `bench.py --workload c4_full` runs it: 64
+    patch circuits (192 variables, K = 32, 128 cluster heads) as one forest handle over the 12288 pixels, four walk
+    groups, one-hot cluster masks, batch 1024.  On the whole batch: every example sends one unit of flow through
+    every variable, every tree node and the heads of every tree; four sampled trees give the bits of a handle of
+    their own (likelihoods, flows, updated parameters, heads), and one of them matches the oracle on a subset."""
+    import torch
+    import pcmi355 as P
+    from pcmi355 import workloads
+    from pcmi355._lib import lib, check
+    from helpers import rel_err
+    O = oracle
+    c4 = workloads.c4_config()
+    V, K, C, H, B, NP = c4["V"], c4["K"], c4["C"], c4["H"], c4["B"], c4["patches"]
+    forest = P.hclt_forest_from_clts(c4["fparent"], C, K, H)
+    forest.set_params(c4["theta"], c4["leaf"])
+    rng = np.random.default_rng(5)
+    heads = np.log(rng.dirichlet(np.ones(K), size=(NP, H))).astype(np.float32)     # tree order
+    forest.set_heads(heads)
+    assert forest.num_trees == NP and forest.size("walk_kernels") == 1
+    d = torch.from_numpy(c4["data"]).cuda()
+    dmask = torch.from_numpy(c4["mask"]).cuda()
+    mix_f = P.forest_flows(forest, d, dmask).cpu().numpy()
+    assert mix_f.shape == (NP, B) and np.isfinite(mix_f).all()
+    ea_f, lf_f = forest.get_flows()
+    assert (ea_f >= 0).all() and (lf_f >= 0).all()
+    np.testing.assert_allclose(lf_f.sum(axis=(1, 2)), B, rtol=1e-4)                 # every variable of every tree
+    fparent = c4["fparent"]
+    has_child = np.bincount(fparent[fparent >= 0], minlength=len(fparent)) > 0
+    inner_not_root = has_child & (fparent >= 0)
+    np.testing.assert_allclose(ea_f[inner_not_root].sum(axis=(1, 2)), B, rtol=1e-4)
+    check(lib.pcm_em_update(forest.handle, 0.1, 0.9))
+    th_f, leaf_f = forest.get_params()
+    heads_f = forest.get_heads()
+    np.testing.assert_allclose(np.exp(heads_f.astype(np.float64)).sum(-1), 1.0, rtol=1e-5)
+    np.testing.assert_allclose(np.exp(leaf_f.astype(np.float64)).sum(-1), 1.0, rtol=1e-4)
+    sampled = [0, 21, 42, 63]
+    for t in sampled:
+        p = int(c4["tree_patch"][t])
+        pv, par = c4["pvars"][p], c4["parents"][p]
+        c = P.multihead_hclt_from_clt(par, C, K, H)
+        c.set_params(*c4["params"][p])
+        c.set_heads(heads[t])
+        dp = torch.from_numpy(np.ascontiguousarray(c4["data"][:, pv])).cuda()
+        mix = P.probs_flows_circuit(c, dp, head_mask=torch.from_numpy(c4["mask"][t].T.copy()).cuda()).cpu().numpy()
+        ea, lf = c.get_flows()
+        check(lib.pcm_em_update(c.handle, 0.1, 0.9))
+        th, lp = c.get_params()
+        split = np.bincount(par[par >= 0]).max() > 3       # to the bit, or within rounding where a node is split
+        cmp = np.testing.assert_array_equal if not split else (
+            lambda a, b, err_msg="": np.testing.assert_allclose(a, b, rtol=2e-5, atol=2e-6 * max(1.0, float(np.abs(b).max())),
+                                                                 err_msg=err_msg))
+        cmp(mix_f[t], mix, err_msg=f"tree {t} mixture")
+        cmp(ea_f[pv], ea, err_msg=f"tree {t} edge flows (split={split})")
+        cmp(lf_f[pv], lf, err_msg=f"tree {t} leaf flows")
+        cmp(th_f[pv], th, err_msg=f"tree {t} sum parameters")
+        cmp(leaf_f[pv], lp, err_msg=f"tree {t} leaf parameters")
+        cmp(heads_f[t], c.get_heads(), err_msg=f"tree {t} heads")
+    # one tree against the oracle on a subset: the mixture likelihood under the one-hot mask is the
+    # chosen head's value
+    t = 21
+    p = int(c4["tree_patch"][t])
+    pv, par = c4["pvars"][p], c4["parents"][p]
+    th0, lf0 = c4["params"][p]
+    ch, root = O.clt_children(par)
+    sub = 24
+    heads_dag = []
+    body = O.hclt_dag(par, K, C, {v: th0[v] for v in range(V) if ch[v]}, lf0)
+    for h in range(H):
+        heads_dag.append(O.summate(*body.children, logps=heads[t][h]))
+    fc = O.bits_compile(O.summate(*heads_dag), C, V)
+    mars = O.forward(fc, np.ascontiguousarray(c4["data"][:sub, pv]))
+    n_heads_first = fc.n_nodes - 1 - H
+    cl = c4["cluster"][:sub, p].astype(np.int64)
+    want = mars[n_heads_first + cl, np.arange(sub)]
+    assert rel_err(mix_f[t][:sub], want).max() < LL_RTOL

@@ -24,14 +24,18 @@ def _compare_step(gpu, oracle, V, K, C, B, seed, idx=None, N=None, tree=None):
     N = N or B
     data = correlated_data(N, V, C, seed + 1, parent)
     ids = np.arange(B, dtype=np.int32) if idx is None else idx
-    ll_ref, th_ref, leaf_ref, ea_ref, lf_ref = oracle_em_reference(fc, data, ids, 0.1, 0.9)
+    # statistics and updated parameters against the float64 oracle: the exact result of the reference's
+    # formulas (its own float32 arithmetic, the float32 oracle, loses up to 1e-4 on trees a few hundred
+    # variables deep; test_deep_trees_three_way); log-likelihoods against both
+    ll_ref, th_ref, leaf_ref, ea_ref, lf_ref = oracle_em_reference(fc, data, ids, 0.1, 0.9, double=True)
+    ll32 = oracle.forward(fc, data, ids)[-1]
 
     bpc = P.hclt_from_clt(parent, C, K)
     bpc.set_params(block_theta(parent, K, theta), leaf)
     d = torch.from_numpy(data).cuda()
     ll = P.loglikelihoods(bpc, d, example_ids=None if idx is None else idx)
     ll = ll.cpu().numpy()
-    assert rel_err(ll, ll_ref).max() < LL_RTOL
+    assert rel_err(ll, ll_ref).max() < LL_RTOL and rel_err(ll, ll32).max() < LL_RTOL
 
     ll2 = P.probs_flows_circuit(bpc, d, example_ids=None if idx is None else idx).cpu().numpy()
     assert np.array_equal(ll, ll2)
@@ -800,3 +804,69 @@ def test_forest_driver_with_per_example_weights(gpu, oracle):
     for x, y in zip(a, b):
         np.testing.assert_array_equal(x, y)
     assert np.abs(np.exp(a[1]) - np.exp(c[1])).max() > 1e-3   # (leaf tables)
+
+
+def _deep_tree(rng, V, chain):
+    """A tree that is mostly one long chain (every node hangs on its predecessor with probability `chain`,
+    else on one of the six before it): hundreds of levels deep at a few hundred variables."""
+    parent = np.full(V, -1, np.int32)
+    for v in range(1, V):
+        parent[v] = v - 1 if rng.random() < chain else rng.integers(max(0, v - 6), v)
+    return parent
+
+
+@pytest.mark.parametrize("V,K,C,B,chain,weighted", [(128, 16, 33, 96, 0.8, False), (128, 32, 255, 120, 0.8, True),
+                                                    (200, 32, 256, 150, 0.8, False), (200, 16, 255, 300, 0.5, True),
+                                                    (263, 32, 33, 200, 0.8, False), (263, 16, 256, 260, 0.9, True),
+                                                    (263, 32, 256, 64, 0.0, False)])
+def test_deep_trees_three_way(gpu, oracle, V, K, C, B, chain, weighted):
+    """Trees of 128-263 variables, 80-200 levels deep, one EM step (pseudocount 0.1, inertia 0.3 so that the
+    statistics dominate the new parameters), with and without per-example weights.  At these depths the reference's
+    float32 log-values (several hundred to a thousand nats, one ulp = 6e-5) make its own flows good to a few 1e-4
+    only, so the comparison is three-way: library vs float64 oracle, float32 oracle (the reference's arithmetic)
+    vs float64 oracle, library vs float32 oracle.  The library keeps a node's value as a tile of order-one numbers
+    plus per-example scalars and must meet the 1e-4 bar against the exact result at every depth; its distance to
+    the float32 oracle must be the float32 oracle's own error."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, block_theta, assert_three_way
+    rng = np.random.default_rng(V * 1000 + K * 10 + C)
+    parent = _deep_tree(rng, V, chain)
+    parent, theta, leaf, fc = make_hclt(V, K, C, V + K + C, parent=parent)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    w = None
+    if weighted:
+        w = rng.uniform(0.0, 5.0, size=B).astype(np.float32)
+        w[::3] = 0.0
+    pc, inertia = 0.1, 0.3
+    c = P.hclt_from_clt(parent, C, K)
+    c.set_params(block_theta(parent, K, theta), leaf)
+    assert c.size("walk_kernels") == 1
+    d = torch.from_numpy(data).cuda()
+    ll = P.probs_flows_circuit(c, d, weights=w).cpu().numpy()
+    import pcmi355._lib as L
+    L.check(L.lib.pcm_em_update(c.handle, pc, inertia))
+    th, lf_new = c.get_params()
+
+    def oracle_step(double):
+        mars = O.forward(fc, data, double=double)
+        root_flow = None if w is None else w[None, :].astype(np.float64 if double else np.float32)
+        flows, ea = O.backward(fc, mars, root_ids=np.array([fc.n_nodes - 1], np.int32),
+                               root_flow=np.ones((1, B)) if root_flow is None else root_flow, double=double)
+        lfl = O.input_flows(fc, data, flows, double=double)
+        new = fc.copy()
+        new.logp, new.leaf_logp = O.em_update(fc, ea, lfl, pc, inertia, double=double)
+        return mars[-1], O.hclt_block_params(new)
+
+    ll64, (th64, lf64) = oracle_step(True)
+    ll32, (th32, lf32) = oracle_step(False)
+    assert (np.abs(ll - ll32) / np.abs(ll32)).max() < LL_RTOL
+    assert (np.abs(ll - ll64) / np.abs(ll64)).max() < LL_RTOL
+    depth = 0
+    for v in range(V):
+        n, u = 0, v
+        while parent[u] >= 0:
+            u, n = parent[u], n + 1
+        depth = max(depth, n)
+    assert_three_way((th, lf_new), (th64, lf64), (th32, lf32), PARAM_RTOL,
+                     f"V={V} K={K} C={C} B={B} depth={depth} weighted={weighted}")
