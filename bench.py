@@ -32,16 +32,18 @@ def algorithmic_bytes(n_int, V, K, C, B):
     is K*4 bytes per (tree node, example); the whole step is priced at six of them per tree
     node (value written and read as a child going up, read twice going down, flow written
     once and read once).  They are booked where this implementation's kernels touch them, two
-    per kernel: forward (value written, value read as a child -- served from LDS), backward
+    per kernel: forward (value written, value read as a child), backward
     (children's values read, ratio vector written: a node's own value is not read going
     down), statistics (ratio vector read, children's values read to rebuild the edge
-    weights).  Each kernel also reads the batch (V*B bytes), the sum parameters (4 bytes per
+    weights).  The forward walk's second vector, the value read as a child, never leaves LDS in this
+    implementation, so that kernel's own roofline entry counts the ONE vector that reaches HBM (the step's
+    total keeps all six).  Each kernel also reads the batch (V*B bytes), the sum parameters (4 bytes per
     edge) and the leaf tables (4*V*K*C); statistics additionally writes both accumulators."""
     vec = K * 4 * B
     n_sum_edges = (n_int - 1) * K * K + K
     theta = 4 * n_sum_edges
     leaf = 4 * V * K * C
-    fwd = n_int * 2 * vec + V * B + theta + leaf
+    fwd = n_int * 1 * vec + V * B + theta + leaf
     bwd = n_int * 2 * vec + V * B + theta + leaf
     stats = n_int * 2 * vec + V * B + 2 * theta + 2 * leaf
     return dict(forward=fwd, backward=bwd, statistics=stats,
@@ -464,9 +466,10 @@ def main():
     for _ in range(args.warmup):
         step()
     # A timed dispatch costs a few microseconds, so the timed steps carry events on the dominant kernel only;
-    # which one that is comes from five steps with all three timed, before the clock starts.
+    # which one that is comes from twenty steps with all three timed, before the clock starts, and is confirmed
+    # afterwards: the two longest kernels are within a few per cent of each other.
     bpc.set_timing(1)
-    for _ in range(5):
+    for _ in range(20):
         step()
     probe_ms = bpc.get_timing()
     dominant = max(probe_ms, key=probe_ms.get)
@@ -479,10 +482,20 @@ def main():
     dt = time.perf_counter() - t0
     dominant_ms = bpc.get_timing()[dominant]   # mean over the timed steps, events on the kernel's own dispatch
     bpc.set_timing(1)
-    for _ in range(10):                        # the other two kernels, for the record: ten further steps
+    for _ in range(20):                        # the other two kernels, for the record: twenty further steps
         step()
     kernel_ms = bpc.get_timing()
     kernel_ms[dominant] = dominant_ms
+    longest = max(kernel_ms, key=kernel_ms.get)
+    if longest != dominant:
+        # the probe picked the second-longest kernel: the longest one is timed alone over as many steps as the
+        # timed region had (same state of the device, clock not running) and is the one reported
+        bpc.set_timing(PHASE_MASK[longest])
+        for _ in range(args.steps):
+            step()
+        kernel_ms[longest] = bpc.get_timing()[longest]
+        if kernel_ms[longest] >= kernel_ms[dominant]:
+            dominant = longest
     bpc.set_timing(0)
     ll_first = ll[:args.cpu_sample].cpu().numpy()
 

@@ -205,7 +205,8 @@ int pcm_loglikelihoods(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex,
  * Per-example weights (the `weights` of reg_flow.jl:38-39,190-191, which multiply an example's edge and
  * leaf flows): every flow is linear in the flow its example starts with, so for a multi-head circuit they
  * are a factor of the mask's column, and a single-root circuit (pcm_circuit_create without heads,
- * pcm_hclt_create) takes them as a mask [1][batch]; d_ll_out is not weighted.
+ * pcm_hclt_create) takes them as a mask [1][batch]; d_ll_out is not weighted.  Masks and weights must be
+ * finite and >= 0: the library does not look at them on the host (they are device memory), a binding does.
  */
 int pcm_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
               const int32_t* d_example_ids, int32_t batch, float rate, const float* d_head_mask,
@@ -360,7 +361,9 @@ int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent);
  * num_examples <= 65535, num_vars <= 4096, num_vars * ceil64(num_examples) <= 16 MiB (e.g. 4096
  * examples of 3072 variables).  The work is queued on `stream` and the call does NOT wait for it.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
- * threads) race; calls queued on one stream do not.
+ * threads) race; calls queued on one stream do not.  The first call on a device resolves the array's
+ * address (hipGetSymbolAddress) and raises the kernels' LDS limit: make it before any stream capture
+ * begins; later calls only query a device attribute and launch.
  */
 int pcm_pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t num_examples,
                            int32_t num_vars, int32_t num_cats, float pseudocount, float* d_mi, void* stream);

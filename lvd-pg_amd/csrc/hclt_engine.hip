@@ -12,6 +12,7 @@
 #include "hclt_walk_lean.hip.hpp"
 #include "hclt_soft_sample.hip.hpp"
 #include "hclt_heads.hip.hpp"
+#include "lean_schedule_check.hpp"
 #include "hclt_soft_evidence.hip.hpp"
 
 namespace pcm {
@@ -224,6 +225,7 @@ void HcltCircuit::build_schedules() {
   if (!walk_err_) {
     PCM_HIP(hipHostMalloc((void**)&walk_err_, sizeof(int), hipHostMallocMapped));
     *walk_err_ = 0;
+    d_walk_void_.upload(std::vector<int32_t>(1, 0));
   }
   int dev_id = 0;
   PCM_HIP(hipGetDevice(&dev_id));
@@ -379,6 +381,13 @@ void HcltCircuit::build_schedules() {
           put(kLSlots, (int32_t)slots);
         }
       }
+    // the waits and posts of all waves, replayed: a schedule on which a wave would wait for ever is refused here
+    static_assert(kLeanCheckA1 == kLA1 && kLeanCheckSlots == kLSlots && kLeanCheckTurns == kLTurns &&
+                  kLeanCheckFields == kLeanFields && kLeanCheckWaves == kWalkWaves, "lean_schedule_check.hpp follows the lean field rows");
+    const int stuck = lean_schedule_stuck_at(f, stride, stride, forward, trash_slot);
+    if (stuck >= 0)
+      fail(PCM_ERR_STATE, "%s walk schedule is unsound: wave %d would wait for ever in step %d", forward ? "forward" : "backward",
+           stuck % kWalkWaves, stuck / kWalkWaves);
     return true;
   };
   auto depth_of = [&](int n) { return depth_[var_of_inner_[n]]; };
@@ -1088,7 +1097,7 @@ void HcltCircuit::get_heads(float* heads) {
   if (H_ == 0) fail(PCM_ERR_STATE, "a single-head circuit has no head parameters");
   if (!heads) fail(PCM_ERR_ARG, "head parameters are null");
   PCM_HIP(hipMemcpyAsync(heads, head_logp(), (size_t)T_ * H_ * K_ * sizeof(float), hipMemcpyDeviceToHost, stream));
-  PCM_HIP(hipStreamSynchronize(stream));
+  sync_checked();
 }
 
 static void fetch(std::vector<float>& h, const float* d, size_t n, hipStream_t s) {
@@ -1098,6 +1107,7 @@ static void fetch(std::vector<float>& h, const float* d, size_t n, hipStream_t s
 }
 
 void HcltCircuit::get_block_params(float* theta, float* leaf) {
+  sync_checked();   // (a void pass is reported before anything that came after it is handed out)
   const int K = K_, C = C_;
   std::vector<float> h;
   if (theta) {
@@ -1117,6 +1127,7 @@ void HcltCircuit::get_block_params(float* theta, float* leaf) {
 }
 
 void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
+  sync_checked();
   if (!have_flows_) fail(PCM_ERR_STATE, "no flows have been computed on this circuit yet");
   const int K = K_, C = C_;
   std::vector<float> h;
@@ -1154,6 +1165,7 @@ void HcltCircuit::get_block_flows(float* edge_aggr, float* leaf_flow) {
 
 void HcltCircuit::vectorize(float* out, int64_t n) {
   no_forest("the parameter vector");
+  sync_checked();
   if (n != size(0)) fail(PCM_ERR_ARG, "parameter vector has %lld entries, circuit has %lld", (long long)n,
                          (long long)size(0));
   if (!out) fail(PCM_ERR_ARG, "parameter vector is null");
@@ -1239,6 +1251,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.G = d_G_.p;
   d.M = d_M_.p;
   d.err = walk_err_;
+  d.err_dev = d_walk_void_.p;
   d.w = nullptr;
   d.ext_ops = d_ext_ops_.p;
   d.B = batch;
@@ -1662,11 +1675,24 @@ HcltCircuit::~HcltCircuit() {
 
 // A walk kernel whose wave ran out of polls waiting for a tile has raised the word (its results are
 // void); seen here at the next call that looks.
+// The same kernel raises a word in device memory, which the update kernels look at: they leave the parameters
+// alone after a void pass, whether or not the host has looked in between (pcm_em_step queues flows and update
+// without waiting).  Reporting also puts the device word and the statistics kernel's node counter back to zero
+// (a launch that followed a void walk may have ended before all its tickets were drawn).
 void HcltCircuit::check_walks() {
   if (walk_err_ && *walk_err_) {
+    (void)hipStreamSynchronize(stream);
     *walk_err_ = 0;
+    if (d_walk_void_.p) (void)hipMemsetAsync(d_walk_void_.p, 0, sizeof(int32_t), stream);
+    if (d_stat_claim_.p) (void)hipMemsetAsync(d_stat_claim_.p, 0, sizeof(uint32_t), stream);
+    have_flows_ = false;
     fail(PCM_ERR_HIP, "a tree-walk kernel gave up waiting for a tile of an earlier step; the results of that pass are void");
   }
+}
+
+void HcltCircuit::sync_checked() {
+  PCM_HIP(hipStreamSynchronize(stream));
+  check_walks();
 }
 
 hipEvent_t* HcltCircuit::ev_set() {
@@ -1681,7 +1707,7 @@ void HcltCircuit::read_timing(float* ms, int n) {
   for (int i = 0; i < n; ++i) ms[i] = 0.f;
   const int cnt = std::min(n_timed_, (int)kTimingRing);
   if (cnt == 0) return;
-  PCM_HIP(hipStreamSynchronize(stream));
+  sync_checked();
   for (int s = 0; s < cnt; ++s)
     for (int i = 0; i < std::min(n, 3); ++i) {
       if (!(timing & (1 << i))) continue;
@@ -1693,6 +1719,7 @@ void HcltCircuit::read_timing(float* ms, int n) {
 }
 
 void HcltCircuit::em_update(float pseudocount, float inertia) {
+  check_walks();   // (a pass already known to be void is reported before its statistics are used)
   if (!have_flows_) fail(PCM_ERR_STATE, "pcm_em_update called before any pcm_flows");
   if (flows_in_general_ || (!block_ && !wide_)) {
     general_->em_update(pseudocount, inertia);
@@ -1707,7 +1734,7 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     const int threads = 1024, cats = ceil_div(C_, threads / 32);
     auto launch = [&](auto kernel) {
       hipLaunchKernelGGL(kernel, dim3(Vu_, ceil_div(K_, 32)), dim3(threads), 0, stream, d_leaf_.p, d_leaf_flow_.p, C_, K_,
-                         pseudocount, inertia, missing_ ? 1 : 0);
+                         pseudocount, inertia, missing_ ? 1 : 0, (const int32_t*)d_walk_void_.p);
     };
     if (cats <= 8) launch(&hclt_leaf_update_kernel<8>);
     else if (cats <= 16) launch(&hclt_leaf_update_kernel<16>);
@@ -1718,12 +1745,12 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
     hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,
                        stream, d_nodes_.p, d_logtheta_.p, d_Wf_.p, d_Wb_.p, d_edge_aggr_.p, n_inner_, pseudocount, inertia,
-                       H_ > 0 ? 1 : 0);
+                       H_ > 0 ? 1 : 0, (const int32_t*)d_walk_void_.p);
   });
   check_launch("theta_update");
   if (H_ > 0) {
     hipLaunchKernelGGL(hclt_heads_update_kernel, dim3(ceil_div(H_, 4), T_), dim3(256), 0, stream, head_logp(), head_aggr(), H_,
-                       Hp_, K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p);
+                       Hp_, K_, pseudocount, inertia, d_head_wf_.p, d_head_wb_.p, (const int32_t*)d_walk_void_.p);
   }
   general_stale_ = true;
 }

@@ -104,6 +104,7 @@ struct HcltDev {
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
   float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (lean kernels; row n_inner: idle waves)
   int* err;               // host-visible word a walk kernel sets when a wave gave up waiting for a tile
+  int* err_dev;           // the same in device memory: the update kernels skip their work after such a pass
   const float* w;         // [B] flow every example starts with at a single root (per-example weights), or null: 1
   int32_t B, Bp, nslices, C, n_inner, V;
   uint32_t leaf_stride;   // bytes per variable in the leaf table (C*K*4)
@@ -270,6 +271,8 @@ class HcltCircuit : public pcm_circuit {
   DevBuf<float> d_M_;
   int* walk_err_ = nullptr;    // pinned host word the walk kernels raise (HcltDev::err); checked by check_walks()
   void check_walks();
+  void sync_checked();   // waits for the stream, then check_walks()
+  DevBuf<int32_t> d_walk_void_;   // device copy of the word: non-zero after a void pass, read by the update kernels
   int walk_chunk(int batch) const;
   static BatchRef chunk_of(const BatchRef& b, int off, int chunk);
   // Floats per node in the tile arrays.  The walk engines keep an odd number of tiles per node: with a power

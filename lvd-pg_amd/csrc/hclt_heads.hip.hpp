@@ -239,10 +239,12 @@ __global__ __launch_bounds__(kHeadWaves * 64) void hclt_heads_backward_kernel(
 // also refreshes the two operand layouts (their padding rows stay zero)
 __global__ __launch_bounds__(256) void hclt_heads_update_kernel(float* __restrict__ head_logp, float* __restrict__ head_aggr,
                                                                 int H, int Hp, int K, float pseudocount, float inertia,
-                                                                float* __restrict__ hwf, float* __restrict__ hwb) {
+                                                                float* __restrict__ hwf, float* __restrict__ hwb,
+                                                                const int32_t* __restrict__ void_pass) {
   const int lane = threadIdx.x & 63;
   const int h = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (h >= H) return;
+  if (void_pass && *void_pass) return;
   head_logp += (size_t)blockIdx.y * H * K;
   head_aggr += (size_t)blockIdx.y * H * K;
   hwf += (size_t)blockIdx.y * Hp * K;

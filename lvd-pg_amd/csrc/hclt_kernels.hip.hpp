@@ -47,7 +47,10 @@ __global__ __launch_bounds__(256) void hclt_weight_shift_kernel(const float* __r
   int mine = 0;
   for (int b = threadIdx.x; b < B; b += blockDim.x) {
     int ex = 0;
-    if (frexpf(fmaxf(w[b], 0.f), &ex) == 0.5f) --ex;   // w <= 2^ex (a power of two is its own bound)
+    // (weights must be finite and >= 0: a binding checks that; what is not counts as the largest float here,
+    // so that the scale stays defined whatever arrives)
+    const float wb = w[b] >= 0.f ? fminf(w[b], 3.0e38f) : (w[b] < 0.f ? 0.f : 3.0e38f);
+    if (frexpf(wb, &ex) == 0.5f) --ex;   // w <= 2^ex (a power of two is its own bound)
     mine = max(mine, ex);
   }
   atomicMax(&best, mine);
@@ -777,10 +780,11 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
                                                                 float* __restrict__ logtheta, float* __restrict__ Wf,
                                                                 float* __restrict__ Wb, float* __restrict__ edge_aggr,
                                                                 int n_inner, float pseudocount, float inertia,
-                                                                int skip_root) {
+                                                                int skip_root, const int32_t* __restrict__ void_pass) {
   constexpr int G = K < 64 ? K : 64, E = K / G, RPB = 256 / G;
   const int row = blockIdx.x * RPB + threadIdx.x / G, l = threadIdx.x % G;
   if (row >= n_inner * K) return;
+  if (void_pass && *void_pass) return;   // a walk of this pass gave up: its statistics must not reach the parameters
   const int n = row / K, k = row % K;
   // a root keeps one sum node (row 0), or none under heads (identity block); an auxiliary node (is_root 2) is all identity
   if (nodes[n].is_root && (k > 0 || skip_root || nodes[n].is_root == 2)) return;
@@ -819,9 +823,11 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
 template <int kCats>
 __global__ __launch_bounds__(1024) void hclt_leaf_update_kernel(float* __restrict__ leaf,
                                                                const float* __restrict__ leaf_flow, int C, int K,
-                                                               float pseudocount, float inertia, int missing) {
+                                                               float pseudocount, float inertia, int missing,
+                                                               const int32_t* __restrict__ void_pass) {
   __shared__ float part[1024];
   __shared__ float miss[32];
+  if (void_pass && *void_pass) return;   // (uniform: every thread reads the same word)
   const int u = blockIdx.x;
   const int jl = threadIdx.x & 31, cg = threadIdx.x >> 5, ncg = blockDim.x >> 5;
   const int j = blockIdx.y * 32 + jl;

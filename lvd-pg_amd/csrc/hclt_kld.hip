@@ -535,6 +535,8 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
 
 void HcltCircuit::kld(pcm_circuit* q, float* out) {
   HcltCircuit* o = same_tree(q);
+  check_walks();
+  o->check_walks();
   if (!block_) {
     general()->kld(o->general(), out);
     return;

@@ -396,7 +396,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
                        d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, Vu_, K_, C_, n_inner_, batch, d_out);
   }
   check_launch_q("hclt_sample");
-  PCM_HIP(hipStreamSynchronize(stream));
+  sync_checked();
 }
 
 void HcltCircuit::sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) {

@@ -107,12 +107,15 @@ __device__ __forceinline__ uint32_t lean_row_off(uint32_t xpack, int sel, uint32
 // for a tile of an earlier step of the host's schedule, and every wave works through its steps in order, so the
 // earliest unfinished step can always proceed.  The wait is bounded all the same: a wave that runs out of polls
 // raises *err and carries on, so the kernel ends whatever the schedule holds.
-__device__ __forceinline__ void lean_wait(const unsigned* state, unsigned want, int* err) {
+__device__ __forceinline__ void lean_wait(const unsigned* state, unsigned want, const HcltDev& d) {
   int polls = 0;
   while (__builtin_amdgcn_readfirstlane(
              (int)__hip_atomic_load(state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP)) != (int)want) {
     if (++polls > kLeanSpinLimit) {
-      if ((threadIdx.x & 63) == 0) __hip_atomic_store(err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+      if ((threadIdx.x & 63) == 0) {
+        __hip_atomic_store(d.err, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        __hip_atomic_store(d.err_dev, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
       break;
     }
     __builtin_amdgcn_s_sleep(1);
@@ -215,7 +218,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
     for (int c = 1; c <= 3; ++c) {
       const uint32_t sl = (slots >> (8 * c)) & 0xffu, tn = (turns >> (8 * c)) & 0x7fu;
       if (sl != 0xffu) {
-        lean_wait(state + sl, (2 * tn + 1) & 0xffu, d.err);
+        lean_wait(state + sl, (2 * tn + 1) & 0xffu, d);
         Tile<K> t;
         lds_tile_load<K>(lds, (int)sl, lane, t);
         tile_add<K>(z, t);
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_forward_lean_kernel(
       // idle steps and the root write the trash slot, which nobody reads: no hand-over there
       const uint32_t so = slots & 0xffu, tn = turns & 0x7fu;
       const bool handed = so != (uint32_t)(n_slots - 1);
-      if (handed) lean_wait(state + so, (2 * tn) & 0xffu, d.err);
+      if (handed) lean_wait(state + so, (2 * tn) & 0xffu, d);
       lds_tile_store<K>(lds, (int)so, lane, o);
       if (handed) lean_post(state + so, (2 * tn + 1) & 0xffu);
     }
@@ -361,9 +364,9 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     const bool in1 = is_inner(c1), in2 = is_inner(c2), in3 = is_inner(c3);
     const uint32_t slots = (uint32_t)lean_get(sc, kLSlots, s), turns = (uint32_t)lean_get(sc, kLTurns, s);
     {   // the children's slots are this wave's from here (scratch first, their ratio tiles at the end)
-      if (in1) lean_wait(state + ((slots >> 8) & 0xffu), (2 * ((turns >> 8) & 0x7fu)) & 0xffu, d.err);
-      if (in2) lean_wait(state + ((slots >> 16) & 0xffu), (2 * ((turns >> 16) & 0x7fu)) & 0xffu, d.err);
-      if (in3) lean_wait(state + ((slots >> 24) & 0xffu), (2 * ((turns >> 24) & 0x7fu)) & 0xffu, d.err);
+      if (in1) lean_wait(state + ((slots >> 8) & 0xffu), (2 * ((turns >> 8) & 0x7fu)) & 0xffu, d);
+      if (in2) lean_wait(state + ((slots >> 16) & 0xffu), (2 * ((turns >> 16) & 0x7fu)) & 0xffu, d);
+      if (in3) lean_wait(state + ((slots >> 24) & 0xffu), (2 * ((turns >> 24) & 0x7fu)) & 0xffu, d);
     }
     Tile<K> X1;
     if (in1) exponent(C1, c2 >= 0, C2, c3 >= 0, C3, X1);
@@ -391,7 +394,7 @@ __global__ __launch_bounds__(kWalkWaves * 64) void hclt_backward_lean_kernel(
     // (3) this node's ratio tile: left in LDS by the parent (the root and idle steps read the trash slot)
     Tile<K> r;
     const bool handed = (slots & 0xffu) != (uint32_t)(n_slots - 1);
-    if (handed) lean_wait(state + (slots & 0xffu), (2 * (turns & 0x7fu) + 1) & 0xffu, d.err);
+    if (handed) lean_wait(state + (slots & 0xffu), (2 * (turns & 0x7fu) + 1) & 0xffu, d);
     lds_tile_load<K>(lds, (int)(slots & 0xffu), lane, r);
     if (handed) lean_post(state + (slots & 0xffu), (2 * (turns & 0x7fu) + 2) & 0xffu);
     const int fl = lean_get(sc, kLFlags, s);

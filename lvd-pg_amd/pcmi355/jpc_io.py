@@ -29,6 +29,8 @@ grammar and by reading them back, not against files the reference wrote.
 import gzip
 import io as _io
 
+import re
+
 import numpy as np
 
 from . import nodes as N
@@ -91,12 +93,19 @@ def write_jpc(file, pc):
             f.close()
 
 
+_JULIA_F32 = re.compile(r"^[-+]?(\d+\.?\d*|\.\d+)f[-+]?\d+$")
+
+
 def _logp(tok, where):
+    """A log-probability token.  Besides what Python's float() reads, the spellings Julia prints for a Float32:
+    an `f` exponent (`-1.0f-5`) and `-Inf32` (ProbabilisticCircuits.jl keeps parameters as Float32)."""
     t = tok.lower()
-    if t in ("-inf", "-infinity"):
+    if t in ("-inf", "-infinity", "-inf32", "-inf16"):
         return -np.inf
+    if _JULIA_F32.match(t):
+        t = t.replace("f", "e")
     try:
-        return float(tok)
+        return float(t)
     except ValueError:
         raise ValueError(f"{where}: '{tok}' is not a log-probability") from None
 

@@ -111,7 +111,25 @@ def loglikelihood(bpc, data, weights=None, batch_size=None, head_mask=None):
 
 loglikelihoods_probcat = loglikelihoods        # reg_likelihood.jl:139-162: the same pass, the reference's other name
 loglikelihood_probcat = loglikelihood          # reg_likelihood.jl:164-173
-weighted_ll = loglikelihood                    # reg_em.jl:191-197
+
+
+def weighted_ll(bpc, data, weights=None, batch_size=None):
+    """`weighted_ll` (src/regularization/reg_em.jl:191-197): without weights the per-example log-likelihoods (a
+    device vector, as `loglikelihoods_probcat` returns them), with weights the scalar sum(ll * w) / sum(w)."""
+    if weights is None:
+        return loglikelihoods(bpc, data, batch_size=batch_size)
+    return loglikelihood(bpc, data, weights, batch_size=batch_size)
+
+
+def _check_weights(weights, n, device):
+    """Per-example weights as a float32 device vector: one per example, finite and not negative (a negative
+    weight would give edge and leaf statistics of different signs, a non-finite one has no fixed-point scale)."""
+    w = torch.as_tensor(weights).to(device=device, dtype=torch.float32)
+    if w.shape != (n,):
+        raise ValueError(f"weights is {tuple(w.shape)}, the data has {n} examples")   # reg_em.jl:220
+    if not bool((torch.isfinite(w) & (w >= 0)).all()):
+        raise ValueError("weights must be finite and >= 0")
+    return w
 
 
 def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None, weights=None):
@@ -130,7 +148,7 @@ def probs_flows_circuit(bpc, data, example_ids=None, rate=0.0, head_mask=None, w
         if ids is not None:
             hm = hm[ids.long()]
     if weights is not None:
-        w = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
+        w = _check_weights(weights, data.shape[0], data.device)
         if ids is not None:
             w = w[ids.long()]
         hm = w[:, None] if hm is None else hm * w[:, None]
@@ -232,9 +250,7 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
     hm_t = None if head_mask is None else head_mask.to(device=data.device, dtype=torch.float32)
     w_t = None
     if weights is not None:
-        w_t = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
-        if w_t.shape != (n,):
-            raise ValueError(f"weights is {tuple(w_t.shape)}, the data has {n} examples")   # reg_em.jl:220
+        w_t = _check_weights(weights, n, data.device)
 
     def batch_mask(ids):
         # [heads (or 1), batch]: the head mask of the batch, times the examples' weights
@@ -313,10 +329,7 @@ def mini_batch_em_for_forest(forest, data, head_masks, num_epochs, *, batch_size
     if tuple(hm_t.shape) != (T, n, forest.num_heads):
         raise ValueError(f"head_masks is {tuple(hm_t.shape)}, the forest needs {(T, n, forest.num_heads)}")
     if weights is not None:
-        w_t = torch.as_tensor(weights).to(device=data.device, dtype=torch.float32)
-        if w_t.shape != (n,):
-            raise ValueError(f"weights is {tuple(w_t.shape)}, the data has {n} examples")
-        hm_t = hm_t * w_t[None, :, None]
+        hm_t = hm_t * _check_weights(weights, n, data.device)[None, :, None]
     num_batches = n // batch_size
     if param_inertia_end is None:
         param_inertia_end = param_inertia

@@ -57,6 +57,18 @@ def test_a_file_written_out_by_hand_from_the_grammar():
     assert abs(np.exp(val[id(root)]) - p) < 1e-7
 
 
+def test_log_parameters_in_julia_float32_spelling():
+    """Julia prints a Float32 with an `f` exponent and its infinities as `Inf32`; a file written by the reference
+    may hold both (ProbabilisticCircuits.jl keeps parameters as Float32)."""
+    text = "c a file with Float32 tokens\njpc 4\nC 0 0 1 -1.0f-5 -Inf32 -2.5f0\nC 1 0 1 -Inf -11.512925f0 -1f1\nP 2 0 1 0\nS 3 0 2 2 -6.9077554f-1 2 -0.6955f0\n"
+    root = read_jpc(io.StringIO(text))
+    np.testing.assert_array_equal(root.params, np.float32([-0.69077554, -0.6955]))
+    leaf = root.inputs[0].inputs[0]
+    np.testing.assert_array_equal(leaf.logps, np.float32([-1.0e-5, -np.inf, -2.5]))
+    with pytest.raises(ValueError, match="not a log-probability"):
+        read_jpc(io.StringIO("jpc 1\nC 0 0 1 -1.0g-5 0.0\n"))
+
+
 def test_literals_read_as_categoricals_over_two_values():
     root = read_jpc(io.StringIO("jpc 3\nL 0 0 2\nL 1 0 -1\nP 2 0 2 0 1\n"))
     pos, neg = root.inputs

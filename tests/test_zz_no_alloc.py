@@ -49,6 +49,31 @@ def test_static_entry_point_matches_the_allocating_one_twice(gpu):
 
 
 @pytest.mark.gpu
+def test_static_entry_point_allocates_nothing_and_takes_any_stream(gpu):
+    """After one warm-up call (the first call on a device resolves the array's address), further calls leave the
+    device's free memory as it was -- hipMemGetInfo, with torch's caching allocator idle --, and a call queued on a
+    stream of the caller's gives the same bits as one on the default stream."""
+    torch, P = gpu
+    from pcmi355._lib import lib, check
+    x = _data(2000, 24, 64, 11)
+    d = torch.from_numpy(x).cuda()
+    n, v = x.shape
+    out0 = torch.zeros((v, v), dtype=torch.float32, device="cuda")
+    out1 = torch.zeros((v, v), dtype=torch.float32, device="cuda")
+    side = torch.cuda.Stream()
+    check(lib.pcm_pairwise_mi_static(d.data_ptr(), d.stride(0), d.stride(1), n, v, 64, 0.1, out0.data_ptr(), None))   # warm-up
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(3):
+        check(lib.pcm_pairwise_mi_static(d.data_ptr(), d.stride(0), d.stride(1), n, v, 64, 0.1, out0.data_ptr(), None))
+    torch.cuda.synchronize()
+    check(lib.pcm_pairwise_mi_static(d.data_ptr(), d.stride(0), d.stride(1), n, v, 64, 0.1, out1.data_ptr(), side.cuda_stream))
+    side.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    assert torch.equal(out0, out1)
+
+
+@pytest.mark.gpu
 def test_static_entry_point_rejects_what_its_array_cannot_hold(gpu):
     torch, P = gpu
     from pcmi355._lib import lib
