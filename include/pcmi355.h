@@ -319,6 +319,34 @@ int pcm_gumbel_sample_backward_rows(pcm_circuit* c, const float* d_params, int64
                                     int32_t grad_wrt_logparams, const float* d_out_grads, float* d_param_grads);
 
 /*
+ * Per-example normalised flows: `per_sample_normalized_flows(mbpc, data; batch_size)` (src/queries/flow.jl:417-464)
+ * for one batch, what `normalized_flows_with_prealloc` (src/utils/cuda_preallocation.jl:292-308, called by
+ * src/models/pc_vae.py:77) starts from.  A forward and a backward pass that leave the circuit's accumulators alone;
+ * row r of d_out (element (r, i) at d_out[r * stride_row + i * stride_param], parameters in
+ * pcm_vectorize_parameters order; Julia's [batch, n] array: 1, batch) belongs to example r of the batch:
+ *   sum parameters (`map_flows_kernel`, flow.jl:496-528):  log(f / (g + 1e-8) + 1e-8), f the example's flow over the
+ *     edge and g its flow over all edges of the same sum node (the edge's posterior share, guarded as the source does);
+ *   input parameters (`map_input_flows_kernel`, :549-593): log(f_c / sum_c f_c) of the node's per-example edge flows,
+ *     which hold the node's flow in one slot: 0 there, -inf in the other slots, NaN (0/0) in all of them where the
+ *     node has no flow.  as_written != 0 places the flow as `get_edge_flow` does
+ *     (src/nodes/fixable_categorical_dist.jl:162-176: it compares the 0-based category x with the 1-based parameter
+ *     index, so the flow of category x sits in the slot of category x - 1 and category 0 fills no slot: NaN);
+ *     as_written == 0 places it in the slot of the observed category (src/conditional_pc/flow.jl:244).
+ * Single-root circuits (PCM_ERR_UNSUPPORTED with heads or for a forest); an HCLT handle answers on its general form.
+ * Queued on the circuit's stream; the call does not wait for it.
+ *
+ * pcm_normalize_params_rows: `normalize_params(mbpc, params; undo)` (src/misc.jl:448-498) in place on a matrix of
+ * parameter rows (the circuit gives the structure only): undo == 0: an input node's entries become exp(entry) / their
+ * sum (probabilities, :364-378) and a sum node's entries logp - log(sum of exp(logp)) (:403-446); undo != 0: input
+ * entries p > 0 become log(p + 1e-6) (:380-393), the sum parameters are normalised as before.
+ */
+int pcm_normalized_flows(pcm_circuit* c, const uint8_t* d_data, int64_t stride_ex, int64_t stride_var,
+                         const int32_t* d_example_ids, int32_t batch, int32_t as_written, float* d_out, int64_t stride_row,
+                         int64_t stride_param);
+int pcm_normalize_params_rows(pcm_circuit* c, float* d_params, int64_t stride_row, int64_t stride_param, int32_t rows,
+                              int32_t undo);
+
+/*
  * Soft evidence: the same two queries with a three-dimensional data argument, as the reference
  * dispatches on `data isa CuArray{Float32,3}` (`init_mar!_with_reg_cat_kernel`
  * src/regularization/reg_likelihood.jl:51-91, `input_flows_circuit_with_reg_cat_kernel`

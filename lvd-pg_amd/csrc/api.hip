@@ -295,6 +295,18 @@ int pcm_gumbel_sample_backward_rows(pcm_circuit* c, const float* d_params, int64
   });
 }
 
+int pcm_normalized_flows(pcm_circuit* c, const uint8_t* d_data, int64_t se, int64_t sv, const int32_t* idx, int32_t batch,
+                         int32_t as_written, float* d_out, int64_t stride_row, int64_t stride_param) {
+  return guarded([&] {
+    need(c)->normalized_flows(batch_ref(d_data, se, sv, idx, batch), d_out, stride_row, stride_param, as_written != 0);
+  });
+}
+
+int pcm_normalize_params_rows(pcm_circuit* c, float* d_params, int64_t stride_row, int64_t stride_param, int32_t rows,
+                              int32_t undo) {
+  return guarded([&] { need(c)->normalize_params_rows(d_params, stride_row, stride_param, rows, undo != 0); });
+}
+
 int pcm_loglikelihoods_soft(pcm_circuit* c, const float* d_evidence, int64_t stride_ex, int64_t stride_var,
                             int64_t stride_cat, const int32_t* d_example_ids, int32_t batch, float* d_ll) {
   return guarded([&] {

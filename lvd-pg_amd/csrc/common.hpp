@@ -167,4 +167,7 @@ struct pcm_circuit {
   virtual void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                            float temperature, bool norm_params, bool grad_wrt_logparams,
                                            const float* d_out_grad, float* d_grads) = 0;
+  // per-example normalised flows [batch][parameters] (element strides sr, sp); normalize_params on parameter rows
+  virtual void normalized_flows(const pcm::BatchRef& b, float* d_out, int64_t sr, int64_t sp, bool as_written) = 0;
+  virtual void normalize_params_rows(float* d_params, int64_t sr, int64_t sp, int32_t rows, bool undo) = 0;
 };

@@ -179,6 +179,14 @@ class HcltCircuit : public pcm_circuit {
                                                      grad_wrt_logparams, d_out_grad, d_grads);
   }
 
+  // (both on the general form: the first with the circuit's own parameters, the second on the rows alone)
+  void normalized_flows(const BatchRef& b, float* d_out, int64_t sr, int64_t sp, bool as_written) override {
+    general()->normalized_flows(b, d_out, sr, sp, as_written);
+  }
+  void normalize_params_rows(float* d_params, int64_t sr, int64_t sp, int32_t rows, bool undo) override {
+    general_structure()->normalize_params_rows(d_params, sr, sp, rows, undo);
+  }
+
   bool sample_soft_block(const float* d_node_noise, float temperature, int32_t batch, float* d_out);
   void set_block_params(const float* theta, const float* leaf);
   // head log-parameters [trees][H][K] (host); a tree's heads are in the order of its head mask rows

@@ -1375,12 +1375,15 @@ void SparseCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head
   run_flows(s.batch, &s, rate, d_head_mask, d_ll);
 }
 
-void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll) {
+// accumulate = false: node flows only (d_flows_), the circuit's accumulators and d_ll are left alone
+void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll, bool accumulate) {
   const int Bp = ceil_div(batch, 64) * 64;
   const int64_t ne = fc_.n_edges();
-  hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div(std::max<int64_t>(ne, 1), 256)), dim3(256), 0, stream, d_edge_aggr_.p, ne, rate);
-  hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)fc_.leaf_logp.size(), 256)), dim3(256), 0, stream,
-                     d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
+  if (accumulate) {
+    hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div(std::max<int64_t>(ne, 1), 256)), dim3(256), 0, stream, d_edge_aggr_.p, ne, rate);
+    hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)fc_.leaf_logp.size(), 256)), dim3(256), 0, stream,
+                       d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
+  }
   SparseDev d = SPARSE_DEV(batch, Bp, d_visit_.p);
   if (soft) { d.ev = soft->d_ev; d.ev_se = soft->stride_ex; d.ev_sv = soft->stride_var; d.ev_sc = soft->stride_cat; d.ev_idx = soft->d_idx; }
   SparseDev db = d;
@@ -1416,6 +1419,11 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
       PCM_LAYER_LAUNCH(sparse_backward_kernel, 2, 1, 8, dim3(cnt, ceil_div(Bp, 128)), PCM_BWD_ARGS);
     }
 #undef PCM_BWD_ARGS
+  }
+  if (!accumulate) {
+    check_launch("sparse_backward");
+    flow_batch_ = last_batch_;
+    return;
   }
   if (ne)
     hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 64)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,

@@ -78,6 +78,8 @@ class SparseCircuit : public pcm_circuit {
   void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                    float temperature, bool norm_params, bool grad_wrt_logparams, const float* d_out_grad,
                                    float* d_grads) override;
+  void normalized_flows(const BatchRef& b, float* d_out, int64_t sr, int64_t sp, bool as_written) override;
+  void normalize_params_rows(float* d_params, int64_t sr, int64_t sp, int32_t rows, bool undo) override;
   void soft_rows_down(const float* p, int rows, const float* d_noise, float inv_t);
   struct RowsState;   // tables and scratch of the parameter-row queries (param_rows.hip)
 
@@ -130,7 +132,7 @@ class SparseCircuit : public pcm_circuit {
   void ensure_var_tables();
   void run_forward(const BatchRef* b, const SoftRef* s);
   void write_ll(int batch, float* d_ll);
-  void run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll);
+  void run_flows(int batch, const SoftRef* soft, float rate, const float* d_head_mask, float* d_ll, bool accumulate = true);
 };
 
 }  // namespace pcm

@@ -78,6 +78,10 @@ pcm_gumbel_sample_rows(c, d_params, stride_row, stride_param, rows, d_noise, tem
     ccall((:pcm_gumbel_sample_rows, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64, Int64, Int32, Ptr{Float32}, Float32, Int32, Ptr{Float32}), c, d_params, stride_row, stride_param, rows, d_noise, temperature, norm_params, d_out)
 pcm_gumbel_sample_backward_rows(c, d_params, stride_row, stride_param, rows, d_noise, temperature, norm_params, grad_wrt_logparams, d_out_grads, d_param_grads) =
     ccall((:pcm_gumbel_sample_backward_rows, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64, Int64, Int32, Ptr{Float32}, Float32, Int32, Int32, Ptr{Float32}, Ptr{Float32}), c, d_params, stride_row, stride_param, rows, d_noise, temperature, norm_params, grad_wrt_logparams, d_out_grads, d_param_grads)
+pcm_normalized_flows(c, d_data, stride_ex, stride_var, d_example_ids, batch, as_written, d_out, stride_row, stride_param) =
+    ccall((:pcm_normalized_flows, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{UInt8}, Int64, Int64, Ptr{Int32}, Int32, Int32, Ptr{Float32}, Int64, Int64), c, d_data, stride_ex, stride_var, d_example_ids, batch, as_written, d_out, stride_row, stride_param)
+pcm_normalize_params_rows(c, d_params, stride_row, stride_param, rows, undo) =
+    ccall((:pcm_normalize_params_rows, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64, Int64, Int32, Int32), c, d_params, stride_row, stride_param, rows, undo)
 pcm_loglikelihoods_soft(c, d_evidence, stride_ex, stride_var, stride_cat, d_example_ids, batch, d_ll) =
     ccall((:pcm_loglikelihoods_soft, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64, Int64, Int64, Ptr{Int32}, Int32, Ptr{Float32}), c, d_evidence, stride_ex, stride_var, stride_cat, d_example_ids, batch, d_ll)
 pcm_flows_soft(c, d_evidence, stride_ex, stride_var, stride_cat, d_example_ids, batch, rate, d_head_mask, d_ll) =

@@ -13,7 +13,7 @@ from .queries import (loglikelihoods, loglikelihood, loglikelihoods_probcat, log
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample, gumbel_sample_rows, gumbel_sample_backward_rows,
                       patch_level_evidence, flow_gradients, adam, soft_reg_evidence, forest_loglikelihoods, forest_flows,
-                      mini_batch_em_for_forest)
+                      mini_batch_em_for_forest, per_sample_normalized_flows, normalize_params, map_pc_parameters)
 from .structures import (pairwise_MI, chow_liu_tree, learn_chow_liu_tree, hclt, hclt_for_colored_images, clt_edges2parent, hclt_pc,  # noqa: F401
                          customized_hclt, joined_hclt, joined_hclt_from_clts, group_vars_by_grid, group_vars_by_cgrid)
 from .transformations import prune_pc, grow_heads_by_flows, aggregate_edge_flows, aggregate_node_flows  # noqa: F401

@@ -59,6 +59,8 @@ _SIGS = {
     "pcm_kld_backward_rows": [H, vp, vp, c_i64, c_i64, c_i32, c_i32, vp, vp, vp],
     "pcm_gumbel_sample_rows": [H, vp, c_i64, c_i64, c_i32, vp, c_f32, c_i32, vp],
     "pcm_gumbel_sample_backward_rows": [H, vp, c_i64, c_i64, c_i32, vp, c_f32, c_i32, c_i32, vp, vp],
+    "pcm_normalized_flows": [H, vp, c_i64, c_i64, vp, c_i32, c_i32, vp, c_i64, c_i64],
+    "pcm_normalize_params_rows": [H, vp, c_i64, c_i64, c_i32, c_i32],
     "pcm_loglikelihoods_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, vp],
     "pcm_flows_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, c_f32, vp, vp],
     "pcm_pairwise_mi": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],

@@ -11,7 +11,8 @@ parameters are neither read nor changed.  Host arrays in, host arrays out, as th
 import numpy as np
 import torch
 
-from .queries import kld, kld_backward, gumbel_sample_rows, gumbel_sample_backward_rows, _rows_on_device
+from .queries import (kld, kld_backward, gumbel_sample_rows, gumbel_sample_backward_rows, _rows_on_device,
+                      per_sample_normalized_flows, map_pc_parameters, normalize_params)
 
 _state = {}
 
@@ -112,3 +113,33 @@ def gumbel_sample_backward_with_prealloc(mbpc, input_aggr_grads, *, temperature,
                                     temperature=temperature, noise=noise, norm_params=norm_params,
                                     grad_wrt_logparams=grad_wrt_logparams)
     return g.cpu().numpy()
+
+
+def normalized_flows_preallocation(mbpc_xz, mbpc_z, *, num_examples, num_vars, mbpc_mapping):
+    """`normalized_flows_preallocation` (:236-263): records the shapes and the parameter mapping (ids of mbpc_z,
+    ids of mbpc_xz; 1-based)."""
+    _state["nflows"] = dict(num_examples=int(num_examples), num_vars=int(num_vars), xz=mbpc_xz, z=mbpc_z,
+                            mapping=(np.asarray(mbpc_mapping[0], np.int64), np.asarray(mbpc_mapping[1], np.int64)))
+
+
+def normalized_flows_free_mem():
+    _state.pop("nflows", None)
+
+
+def normalized_flows_with_prealloc(mbpc_xz, mbpc_z, data):
+    """`normalized_flows_with_prealloc(mbpc_xz, mbpc_z, data)` (:292-308), the first call of
+    src/models/pc_vae.py:77: the per-example normalised flows of the joint circuit over (x, z), the columns of the
+    matched sum parameters copied into a parameter matrix of the circuit over z, clamped to [-20, 0], and
+    normalised (`normalize_params`: the leaves of mbpc_z become probabilities, its sum parameters normalised
+    log-parameters).  Host matrix [num_examples, num_parameters(mbpc_z)]."""
+    st = _state.get("nflows")
+    if st is None or st["xz"] is not mbpc_xz or st["z"] is not mbpc_z:
+        raise RuntimeError("call normalized_flows_preallocation(mbpc_xz, mbpc_z; ...) first")
+    data = np.asarray(data)
+    if data.shape != (st["num_examples"], st["num_vars"]):
+        raise ValueError(f"preallocated for {(st['num_examples'], st['num_vars'])}, got {data.shape}")
+    d = torch.from_numpy(np.ascontiguousarray(data, np.uint8)).cuda()
+    xz = per_sample_normalized_flows(mbpc_xz, d, batch_size=data.shape[0])
+    z = map_pc_parameters(mbpc_z, mbpc_xz, xz, param_mapping=st["mapping"])
+    z.clamp_(-20.0, 0.0)
+    return normalize_params(mbpc_z, z).cpu().numpy()

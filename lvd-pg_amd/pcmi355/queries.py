@@ -113,12 +113,15 @@ loglikelihoods_probcat = loglikelihoods        # reg_likelihood.jl:139-162: the 
 loglikelihood_probcat = loglikelihood          # reg_likelihood.jl:164-173
 
 
-def weighted_ll(bpc, data, weights=None, batch_size=None):
+def weighted_ll(bpc, data, weights=None, batch_size=None, head_mask=None):
     """`weighted_ll` (src/regularization/reg_em.jl:191-197): without weights the per-example log-likelihoods (a
-    device vector, as `loglikelihoods_probcat` returns them), with weights the scalar sum(ll * w) / sum(w)."""
+    device vector, as `loglikelihoods_probcat` returns them), with weights the scalar sum(ll * w) / sum(w).  With
+    `head_mask` the per-example values are the multi-head mixture's."""
     if weights is None:
+        if head_mask is not None:
+            return multihead_loglikelihoods(bpc, data, head_mask, batch_size=batch_size)
         return loglikelihoods(bpc, data, batch_size=batch_size)
-    return loglikelihood(bpc, data, weights, batch_size=batch_size)
+    return loglikelihood(bpc, data, weights, batch_size=batch_size, head_mask=head_mask)
 
 
 def _check_weights(weights, n, device):
@@ -388,6 +391,60 @@ def _rows_on_device(x, n, what):
     if t.dtype != torch.float32:
         t = t.float()
     return (t.cuda() if not t.is_cuda else t), host
+
+
+def per_sample_normalized_flows(mbpc, data, *, batch_size=None, as_written=True, out=None):
+    """`per_sample_normalized_flows(mbpc, data; batch_size)` (src/queries/flow.jl:417-464): for every example the
+    vector, in parameter order, of its flows normalised per sum node and per input node --
+    log(f / (g + 1e-8) + 1e-8) for a sum parameter (`map_flows_kernel`, :496-528) and log(f_c / sum_c f_c) for an
+    input parameter (`map_input_flows_kernel`, :549-593).  The circuit's accumulators are not touched.  `data` is a
+    uint8 GPU tensor or host array [examples, variables]; returns [examples, num_parameters] float32, a host array
+    for host data (the reference returns `Array(normalized_flows)`), a GPU tensor otherwise or when `out` (a float32
+    GPU tensor of that shape, any strides) is given.
+    as_written: the input node's flow lands where `get_edge_flow` (src/nodes/fixable_categorical_dist.jl:162-176) puts
+    it, which compares the 0-based category with the 1-based parameter index: category x fills the slot of category
+    x - 1 and category 0 none (its node's entries are NaN).  False: the slot of the observed category."""
+    host = not isinstance(data, torch.Tensor)
+    d = torch.as_tensor(np.ascontiguousarray(data, np.uint8)).cuda() if host else data
+    _check_data(mbpc, d)
+    n, npar = d.shape[0], mbpc.num_parameters()
+    if out is None:
+        out = torch.empty((n, npar), dtype=torch.float32, device=d.device)
+    elif tuple(out.shape) != (n, npar) or out.dtype != torch.float32 or not out.is_cuda:
+        raise ValueError(f"out must be a float32 GPU tensor of shape {(n, npar)}")
+    batch_size = n if batch_size is None else int(batch_size)
+    for s in range(0, n, max(batch_size, 1)):
+        part = d[s:s + batch_size]
+        o = out[s:s + batch_size]
+        check(lib.pcm_normalized_flows(mbpc.handle, part.data_ptr(), part.stride(0), part.stride(1), None, part.shape[0],
+                                       int(bool(as_written)), o.data_ptr(), o.stride(0), o.stride(1)))
+    return out.cpu().numpy() if host else out
+
+
+def normalize_params(mbpc, params, *, undo=False):
+    """`normalize_params(mbpc, params; undo)` (src/misc.jl:448-498) on a matrix [rows, num_parameters]: input
+    entries -> exp(entry) / sum over the node (probabilities; undo: p > 0 -> log(p + 1e-6)), sum parameters ->
+    logp - log(sum over the node of exp(logp)).  A GPU tensor is changed in place and returned; a host array comes
+    back as a new host array (the reference returns `Array(params)`)."""
+    p, host = _rows_on_device(params, mbpc.num_parameters(), "params")
+    check(lib.pcm_normalize_params_rows(mbpc.handle, p.data_ptr(), p.stride(0), p.stride(1), p.shape[0], int(bool(undo))))
+    return p.cpu().numpy() if host else p
+
+
+def map_pc_parameters(mbpc1, mbpc2, params2, *, param_mapping, params1=None):
+    """`map_pc_parameters(mbpc1, mbpc2, params1, params2; param_mapping)` (src/utils/map_params.jl:12-45, kernel
+    :128-146): params1[:, ids1[i]] = params2[:, ids2[i]] for the matched parameter pairs `param_mapping = (ids1,
+    ids2)`, 1-based as `compute_mbpc_mapping` (:47-126) gives them; unmatched columns of params1 keep what they
+    held (zeros for a new matrix, as :7).  GPU tensors in and out."""
+    ids1, ids2 = (torch.as_tensor(np.asarray(x, np.int64) - 1) for x in param_mapping)
+    p2, _ = _rows_on_device(params2, mbpc2.num_parameters(), "params2")
+    if params1 is None:
+        params1 = torch.zeros((p2.shape[0], mbpc1.num_parameters()), dtype=torch.float32, device=p2.device)
+    if ids1.numel() and (int(ids1.max()) >= params1.shape[1] or int(ids2.max()) >= p2.shape[1] or int(ids1.min()) < 0
+                         or int(ids2.min()) < 0):
+        raise ValueError("param_mapping names parameters the circuits do not have")
+    params1[:, ids1.to(p2.device)] = p2[:, ids2.to(p2.device)]
+    return params1
 
 
 def kld(mbpc, params1, params2=None, *, norm_params=False):

@@ -269,6 +269,84 @@ def em_step(fc, data, idx, pseudocount, inertia, double=False):
     return mars[-1].copy(), logp, leaf, ea, lf
 
 
+def edge_flows(fc, mars, flows):
+    """Per-example flows of the sum parameters, [n_sum_params, B] in parameter-vector order (the reference's
+    `edge_flows[ex, edge]`, src/queries/flow.jl:49-60, :70-71): flow of the parent times
+    exp(value of the edge's children + logp - value of the parent); 0 where the parent has no flow."""
+    pe = fc.sum_param_edges()
+    par = fc.edge_parent()[pe]
+    R = mars.dtype
+    em = mars[fc.prime[pe]] + fc.logp[pe].astype(R)[:, None]
+    sub = fc.sub[pe]
+    has = sub >= 0
+    em[has] += mars[sub[has]]
+    with np.errstate(invalid="ignore", over="ignore"):
+        ef = flows[par] * np.exp(em - mars[par])
+    ef[~(flows[par] > 0)] = 0
+    return ef.astype(R), par
+
+
+def normalized_flows(fc, data, idx=None, double=False, as_written=True):
+    """`per_sample_normalized_flows(mbpc, data; batch_size)` (src/queries/flow.jl:417-464) -> [B, n_params] in
+    parameter-vector order.  Sum parameters as `map_flows_kernel` writes them (:496-528): with f the edge flow
+    and g the sum of the flows of the sum node's edges, log(f / (g + 1e-8) + 1e-8) (`par_groups` starts at 1e-8,
+    :535).  Input parameters as `map_input_flows_kernel` (:549-593): log(f_c / sum_c f_c) of the node's
+    per-example edge flows (`input_flows_circuit_kernel` :165-195), which hold the node's flow in ONE slot and 0
+    elsewhere -- so the entries are 0 in that slot and -inf in the others, NaN (0/0) throughout where the node has
+    no flow.  Which slot: `get_edge_flow` (src/nodes/fixable_categorical_dist.jl:162-176) compares the 0-based
+    category with the 1-based parameter index, so as written the flow of category x sits in the slot of category
+    x - 1 and category 0 leaves every slot empty (the test of test/queries/flow_tests.jl:54-64 has data value 1 in
+    slot 1); as_written = False puts it in the slot of category x (what src/conditional_pc/flow.jl:244 does)."""
+    R = _real(double)
+    data = np.ascontiguousarray(data, dtype=np.uint8)
+    idx = np.arange(data.shape[0], dtype=np.int32) if idx is None else np.ascontiguousarray(idx, np.int32)
+    B = len(idx)
+    mars = forward(fc, data, idx, double)
+    flows, _ = backward(fc, mars, double=double)
+    ef, par = edge_flows(fc, mars, flows)
+    _, inv = np.unique(par, return_inverse=True)
+    g = np.full((inv.max() + 1 if len(inv) else 0, B), 1e-8, dtype=R)
+    np.add.at(g, inv, ef)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        sums = np.log(ef / g[inv] + R(1e-8))
+        leaves = []
+        for n in fc.input_nodes():
+            x = data[idx, fc.in_var[n]].astype(np.int64)
+            slot = x - 1 if as_written else x
+            f = np.zeros((fc.C, B), dtype=R)
+            ok = slot >= 0
+            f[slot[ok], np.nonzero(ok)[0]] = flows[n][ok]
+            leaves.append(np.log(f / f.sum(axis=0, keepdims=True)))
+    return np.concatenate([sums] + leaves, axis=0).T.astype(R)
+
+
+def normalize_params(fc, params, undo=False, double=False):
+    """`normalize_params(mbpc, params; undo)` (src/misc.jl:448-498) on rows [R, n_params] of parameter vectors.
+    undo = False: every input node's C entries become exp(entry) / sum of them (`normalize_params_step`,
+    :364-378: log-parameters -> probabilities) and every sum parameter logp - log(sum over its node of exp(logp))
+    (`preprocess_inner_params_kernel`, :403-446).  undo = True: input entries p > 0 become log(p + 1e-6), others
+    stay (`undo_normalize_params_step`, :380-393); the sum parameters go through the same normalisation."""
+    R = _real(double)
+    p = np.array(params, dtype=R, ndmin=2)
+    pe = fc.sum_param_edges()
+    ns = len(pe)
+    par = fc.edge_parent()[pe]
+    nin = len(fc.input_nodes())
+    leaf = p[:, ns:].reshape(p.shape[0], nin, fc.C)
+    with np.errstate(divide="ignore", invalid="ignore", over="ignore"):
+        if not undo:
+            e = np.exp(leaf)
+            leaf[...] = e / e.sum(axis=2, keepdims=True)
+        else:
+            leaf[...] = np.where(leaf > 0, np.log(leaf + R(1e-6)), leaf)
+        if ns:
+            _, inv = np.unique(par, return_inverse=True)
+            cum = np.zeros((p.shape[0], inv.max() + 1), dtype=R)
+            np.add.at(cum.T, inv, np.exp(p[:, :ns]).T)
+            p[:, :ns] -= np.log(cum[:, inv])
+    return p
+
+
 def kld(fc1, fc2, double=False, norm_params=False):
     """norm_params: the circuits' leaf arrays hold probabilities (sum edges stay in log space)."""
     R = _real(double)

@@ -146,8 +146,9 @@ def test_workload_builders():
 
 
 def test_algorithmic_bytes_formula():
-    """Per-kernel bookings add up to the step formula: 6 vectors of K floats per (inner tree
-    node, example), the batch once, the sum parameters three times, the leaf tables five."""
+    """The step formula: 6 vectors of K floats per (inner tree node, example), the batch once, the sum parameters
+    three times, the leaf tables five.  Per kernel: two vectors each for the backward walk and the statistics, ONE
+    for the forward walk (its second vector, the value read as a child, never leaves LDS and is not HBM traffic)."""
     import importlib.util
     spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
     bench = importlib.util.module_from_spec(spec)
@@ -156,7 +157,8 @@ def test_algorithmic_bytes_formula():
     ab = bench.algorithmic_bytes(n_int, V, K, C, B)
     edges = (n_int - 1) * K * K + K
     assert ab["step"] == n_int * 6 * K * 4 * B + V * B + 3 * 4 * edges + 5 * 4 * V * K * C
-    assert ab["forward"] == n_int * 2 * K * 4 * B + V * B + 4 * edges + 4 * V * K * C
+    assert ab["forward"] == n_int * 1 * K * 4 * B + V * B + 4 * edges + 4 * V * K * C
+    assert ab["backward"] == n_int * 2 * K * 4 * B + V * B + 4 * edges + 4 * V * K * C
 
 
 def test_describe_dag_is_topological():

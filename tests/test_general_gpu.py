@@ -307,6 +307,7 @@ def test_multihead_closed_forms(gpu, oracle):
     assert P.loglikelihood_probcat is P.loglikelihood and P.loglikelihoods_probcat is P.loglikelihoods
     # weighted_ll without weights: the per-example vector, as reg_em.jl:191-197 returns it (here: one row per head)
     np.testing.assert_array_equal(P.weighted_ll(bpc, data).cpu().numpy(), per_head)
+    np.testing.assert_array_equal(P.weighted_ll(bpc, data, head_mask=head_mask).cpu().numpy(), lls)
     for bad in ([1.0, -0.5], [np.inf, 1.0], [np.nan, 1.0]):
         with pytest.raises(ValueError, match="finite and >= 0"):
             P.probs_flows_circuit(bpc, data, head_mask=head_mask, weights=np.float32(bad))

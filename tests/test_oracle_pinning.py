@@ -875,3 +875,145 @@ def test_missing_flow_update_is_the_m_step_on_expected_counts():
     np.testing.assert_allclose(got[:, :C_real], leaf_x.reshape(-1, C_real), rtol=1e-7, atol=1e-7)
     assert (got[:, C_real] == 0).all()                           # the marker's row stays log 1
     np.testing.assert_allclose(np.exp(got[:, :C_real]).sum(axis=1), 1.0, rtol=1e-6)
+
+
+# ------------------------------------------------------------------------------------
+# per-example normalised flows (src/queries/flow.jl:417-593) and normalize_params (src/misc.jl:448-498)
+# ------------------------------------------------------------------------------------
+
+def _hclt_joint(parent, K, theta, leaf, x):
+    """log of the joint of x and every assignment of the inner tree nodes' hidden states, as a dict
+    states -> log-probability (the terms of brute_force_hclt_ll)."""
+    ch, root = O.clt_children(parent)
+    inner = [v for v in range(len(parent)) if ch[v]]
+    out = {}
+    for states in itertools.product(range(K), repeat=len(inner)):
+        j = dict(zip(inner, states))
+        lp = 0.0
+        for v in inner:
+            jp = 0 if v == root else j[parent[v]]
+            lp += float(theta[v][jp, j[v]]) + float(leaf[v, j[v], x[v]])
+            for c in ch[v]:
+                if not ch[c]:
+                    lp += float(leaf[c, j[v], x[c]])
+        out[states] = lp
+    return inner, out
+
+
+@pytest.mark.parametrize("tree,K,C", [([-1, 0, 1, 1], 3, 2), ([1, -1, 1, 0, 0, 0], 2, 3), ([-1, 0, 1, 2, 3], 2, 3)])
+def test_normalized_flows_are_posteriors_of_the_hidden_states(tree, K, C):
+    """A sum parameter's normalised flow is the posterior of its child's hidden state given its own node's (the
+    parent tree node's state) and the example: exp(entry of (v, k, j)) = P(z_v = j | z_parent(v) = k, x), summed
+    out of the joint over all hidden-state assignments in float64; and the entries of a sum node add up to 1."""
+    parent = np.array(tree, np.int32)
+    V = len(parent)
+    rng = np.random.default_rng(V + K)
+    theta, leaf = O.random_hclt_params(parent, K, C, rng)
+    fc = O.hclt_flat(parent, K, C, theta, leaf)
+    data = rng.integers(0, C, size=(5, V)).astype(np.uint8)
+    nf = O.normalized_flows(fc, data, double=True)
+    pe = fc.sum_param_edges()
+    pos_of_edge = {int(e): i for i, e in enumerate(pe)}
+    ch, root = O.clt_children(parent)
+    for b, x in enumerate(data):
+        inner, joint = _hclt_joint(parent, K, theta, leaf, x)
+        at = {v: i for i, v in enumerate(inner)}
+        for v in inner:
+            nk = len(fc.meta["sum_node"][v])
+            for k in range(nk):
+                num = np.full(K, -np.inf)
+                for states, lp in joint.items():
+                    if v != root and states[at[parent[v]]] != k:
+                        continue
+                    num[states[at[v]]] = np.logaddexp(num[states[at[v]]], lp)
+                post = np.exp(num - logsumexp(num))
+                got = np.array([nf[b, pos_of_edge[fc.meta["edge_of"][v] + k * K + j]] for j in range(K)])
+                np.testing.assert_allclose(np.exp(got), post, rtol=1e-5, atol=1e-7)
+                assert abs(np.exp(got).sum() - 1) < 1e-5
+
+
+def test_normalized_flows_are_derivatives_of_the_parent_value():
+    """On a DAG with shared sub-circuits: edge flow / node flow = d(log-value of the sum node) / d(logp of the
+    edge), by central differences in float64, for every sum parameter whose node has flow."""
+    fc = O.bits_compile(random_dag(5, 3, np.random.default_rng(8), width=3), 3, 5)
+    fc.logp = fc.logp.astype(np.float64)
+    fc.leaf_logp = fc.leaf_logp.astype(np.float64)
+    data = np.random.default_rng(9).integers(0, 3, size=(4, 5)).astype(np.uint8)
+    nf = O.normalized_flows(fc, data, double=True)
+    mars = O.forward(fc, data, double=True)
+    flows, _ = O.backward(fc, mars, double=True)
+    pe = fc.sum_param_edges()
+    par = fc.edge_parent()
+    h = 1e-6
+    seen = 0
+    for i, e in enumerate(pe):
+        g = fc.copy()
+        g.logp[e] += h
+        up = O.forward(g, data, double=True)[par[e]]
+        g.logp[e] -= 2 * h
+        fd = (up - O.forward(g, data, double=True)[par[e]]) / (2 * h)
+        live = flows[par[e]] > 1e-3
+        seen += int(live.sum())
+        np.testing.assert_allclose(np.exp(nf[live, i]), fd[live], rtol=1e-5, atol=1e-7)
+    assert seen > 20
+
+
+def test_normalized_flows_guards_and_input_slots_as_written():
+    """The 1e-8 guards of map_flows (flow.jl:525, :535) on a sum node that no flow reaches: log(0 / 1e-8 + 1e-8);
+    and the input entries as written: the node's flow in the slot get_edge_flow picks, the literal of
+    test/queries/flow_tests.jl:54-64 (data value 1 -> slot 1 of 5, i.e. the first), -inf elsewhere, NaN throughout
+    where nothing lands (category 0) -- against the corrected placement with as_written = False."""
+    C = 5
+    lp = lambda: np.log(np.full(C, 1.0 / C, np.float32))
+    dead = O.summate(O.input_node(1, lp()), O.input_node(1, lp()), logps=np.log(np.float32([0.3, 0.7])))
+    root = O.summate(O.multiply(O.input_node(0, lp()), O.input_node(1, lp())),
+                     O.multiply(O.input_node(0, lp()), dead), logps=np.float32([0.0, -np.inf]))
+    fc = O.bits_compile(root, C, 2)
+    data = np.array([[1, 2], [0, 4]], np.uint8)
+    for dbl in (False, True):
+        nf = O.normalized_flows(fc, data, double=dbl)
+        pe = fc.sum_param_edges()
+        par = fc.edge_parent()[pe]
+        dead_rows = np.nonzero(par != fc.n_nodes - 1)[0]
+        assert len(dead_rows) == 2
+        np.testing.assert_allclose(nf[:, dead_rows], np.log(1e-8), rtol=1e-6)
+        top = np.nonzero(par == fc.n_nodes - 1)[0]
+        np.testing.assert_allclose(nf[:, top[0]], np.log(1.0 / (1 + 1e-8) + 1e-8), atol=1e-7)
+        np.testing.assert_allclose(nf[:, top[1]], np.log(1e-8), rtol=1e-6)
+    nf = O.normalized_flows(fc, data, double=True)
+    ns = len(fc.sum_param_edges())
+    inputs = fc.input_nodes()
+    first_var0 = [i for i, n in enumerate(inputs) if fc.in_var[n] == 0][0]     # an input node of variable 0 that has flow
+    blk = nf[:, ns + first_var0 * C: ns + (first_var0 + 1) * C]
+    with np.errstate(invalid="ignore"):
+        assert blk[0].tolist() == [0.0, -np.inf, -np.inf, -np.inf, -np.inf]        # value 1: the first slot
+    assert np.isnan(blk[1]).all()                                                  # value 0: no slot, 0 / 0
+    fixed = O.normalized_flows(fc, data, double=True, as_written=False)
+    blk = fixed[:, ns + first_var0 * C: ns + (first_var0 + 1) * C]
+    assert blk[0].tolist() == [-np.inf, 0.0, -np.inf, -np.inf, -np.inf]
+    assert blk[1].tolist() == [0.0, -np.inf, -np.inf, -np.inf, -np.inf]
+    np.testing.assert_array_equal(fixed[:, :ns], nf[:, :ns])
+
+
+def test_normalize_params_against_scipy():
+    """normalize_params (src/misc.jl:448-498): input entries -> scipy's softmax per input node, sum parameters ->
+    scipy's log_softmax per sum node; undo: log(p + 1e-6) where p > 0 (:380-393)."""
+    from scipy.special import softmax, log_softmax
+    fc = O.bits_compile(random_dag(4, 3, np.random.default_rng(2), width=3), 3, 4)
+    rng = np.random.default_rng(3)
+    n = len(fc.vectorize_parameters())
+    p = rng.normal(0, 2, size=(3, n)).astype(np.float32)
+    got = O.normalize_params(fc, p, double=True)
+    pe = fc.sum_param_edges()
+    ns = len(pe)
+    par = fc.edge_parent()[pe]
+    for node in np.unique(par):
+        cols = np.nonzero(par == node)[0]
+        assert (np.diff(cols) == 1).all()                       # a sum node's parameters sit side by side
+        np.testing.assert_allclose(got[:, cols], log_softmax(p[:, cols].astype(np.float64), axis=1), rtol=1e-6, atol=1e-9)
+    nin = len(fc.input_nodes())
+    np.testing.assert_allclose(got[:, ns:].reshape(3, nin, 3), softmax(p[:, ns:].astype(np.float64).reshape(3, nin, 3), axis=2),
+                               rtol=1e-6)
+    back = O.normalize_params(fc, got, undo=True, double=True)
+    np.testing.assert_allclose(back[:, ns:], np.log(got[:, ns:] + 1e-6), rtol=1e-6)
+    np.testing.assert_allclose(back[:, :ns], got[:, :ns], atol=1e-6)     # already normalised: unchanged
