@@ -1214,6 +1214,7 @@ void HcltCircuit::ensure_batch(int batch) {
     d_G_.alloc((size_t)n_inner_ * tile);
     d_wide_rs_.alloc((size_t)n_inner_ * tile);
     d_wide_es_.alloc((size_t)n_inner_ * tile);
+    d_M_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
     d_xb_.alloc((size_t)V_ * ns * kSlice);
     d_xn_.alloc((size_t)(n_inner_ + 1) * ns * kSlice);
     d_xn_.zero(stream);

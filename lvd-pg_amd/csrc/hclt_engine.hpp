@@ -80,12 +80,15 @@ struct StatNode {
 };
 static_assert(sizeof(StatNode) == 64, "StatNode is read with scalar loads");
 
-// Per tree node, what the wide walk kernels request a node ahead (hclt_wide.hip).
-struct WideOps {
-  uint32_t fwd[6], bwd[6];   // 0: none; leaf row: bit 31 | category selector << 24 | variable; value tile: bit 30 | node
-  int32_t fwd_extra_off, fwd_extra_cnt, bwd_extra_off, bwd_extra_cnt;   // operands fetched at the point of use
-  int32_t parent, is_root, prev_child, pad;   // prev_child: node - 1 is a child (its tile is still in registers going up)
+// One slot of a wide walk's schedule: what one of the two groups of waves does in one step (hclt_wide.hip).
+struct WideSlot {
+  uint32_t op[6];      // operands requested a slot ahead.  0: none; leaf row: bit 31 | category selector << 24 | variable; value tile: bit 30 | node
+  int32_t node;        // -1: the group idles this step
+  int32_t parent;      // the parent's node, -1 at the root
+  int32_t flags;       // bit 0: the root; bit 1: the tile of the group's previous slot is an operand (still in registers)
+  int32_t extra_off, extra_cnt;   // operands fetched at the point of use
 };
+constexpr int kWideRoot = 1, kWidePrev = 2;
 
 // Everything the kernels need, passed by value.
 struct HcltDev {
@@ -102,7 +105,7 @@ struct HcltDev {
   float* O;               // [n_inner][nslices][16*K] node values, tile-native layout
   float* R;               // [n_inner][nslices][16*K] flow / value ratios of the sum nodes
   float* G;               // child-flow tiles that found no LDS slot (same layout), or null
-  float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (lean kernels; row n_inner: idle waves)
+  float* M;               // [n_inner + 1][Bp] row maxima of the forward walk (row n_inner: idle waves of the lean kernels)
   int* err;               // host-visible word a walk kernel sets when a wave gave up waiting for a tile
   int* err_dev;           // the same in device memory: the update kernels skip their work after such a pass
   const float* w;         // [B] flow every example starts with at a single root (per-example weights), or null: 1
@@ -355,7 +358,8 @@ class HcltCircuit : public pcm_circuit {
   // wide block kernels
   DevBuf<float> d_wide_rs_, d_wide_es_;   // R and E of every node in the operand layout of the statistics contraction
   DevBuf<int32_t> d_wide_state_node_;     // per variable: the inner node whose flow tile feeds its leaf histogram
-  DevBuf<WideOps> d_wide_ops_;
+  DevBuf<WideSlot> d_wide_fwd_, d_wide_bwd_;   // [steps][2 groups]
+  int wide_steps_f_ = 0, wide_steps_b_ = 0;
   DevBuf<uint32_t> d_wide_extra_;
   void build_wide_tables();
   void wide_forward(const HcltDev& d, float* d_ll);
