@@ -378,6 +378,31 @@ def secondary(args):
                    value=B / dt, unit="examples/s",
                    config={"workload": args.workload, "num_vars": V, "hidden": K, "categories": C, "batch": B,
                            "nodes": nn, "edges": ne})
+    elif args.workload == "hbm_stream_mix":
+        # What the device's memory gives a kernel that only streams (pcm_stream_probe: 16 bytes per lane and
+        # access, non-temporal, like the walks' tile traffic), per mix of reads and writes.  A "step" is one launch
+        # of the backward walk's mix, 4 reads : 3 writes; the other mixes are listed beside it.
+        lanes = 20 << 20                                    # 336 MB per stream
+        src = torch.zeros(6 * lanes * 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty(3 * lanes * 4, dtype=torch.float32, device="cuda")
+        stream = torch.cuda.current_stream().cuda_stream
+        rates = {}
+        for name, (r, w) in {"read_only": (1, 0), "write_only": (0, 1), "1r_1w": (1, 1), "backward_4r_3w": (4, 3),
+                             "forward_1r_3w": (1, 3), "statistics_6r_1w": (6, 1)}.items():
+            best = 0.0
+            for grid in (1024, 2048, 8192):
+                t = _timed(torch, lambda: check(lib.pcm_stream_probe(src.data_ptr(), dst.data_ptr(), lanes, r, w, grid, stream)),
+                           max(3, args.steps // 5), 2)
+                best = max(best, lanes * 16.0 * (r + w) / t / 1e9)
+            rates[name] = best
+        dt = _timed(torch, lambda: check(lib.pcm_stream_probe(src.data_ptr(), dst.data_ptr(), lanes, 4, 3, 2048, stream)),
+                    args.steps, args.warmup)
+        algo = lanes * 16.0 * 7
+        out["dtype"] = "bytes"
+        out.update(metric="GB/s of a plain streaming kernel, 4 reads : 3 writes of 16 B per lane, non-temporal",
+                   value=algo / dt / 1e9, unit="GB/s",
+                   config={"workload": args.workload, "bytes_per_stream": lanes * 16, "grid": 2048, "threads": 256},
+                   mixes_gbs=rates)
     elif args.workload == "chow_liu_c3":
         cfg = workloads.make_config("c3_hclt3072_k32")
         V, C, B = cfg["V"], cfg["C"], cfg["B"]

@@ -435,6 +435,14 @@ int pcm_adam_flow_step(pcm_circuit* c, int32_t batch_size, float* d_params, floa
 int pcm_set_timing(pcm_circuit* c, int32_t on);
 int pcm_get_timing(pcm_circuit* c, float* ms, int32_t n);
 
+/* A plain streaming kernel, for bench.py's `hbm_stream_mix` workload: no counterpart in the reference, a
+ * measuring instrument.  One launch reads `reads` streams of `lanes` x 16 bytes from d_src (laid out one after
+ * the other) and writes `writes` such streams to d_dst, every access 16 bytes per lane and non-temporal, on a
+ * grid of `grid` workgroups of 256 threads; (reads, writes) is one of (1,0) (0,1) (1,1) (4,3) (1,3) (6,1) --
+ * the last three are the mixes of the backward walk, the forward walk and the statistics kernel of the EM step.
+ * Queued on `stream`, not waited for.  With writes = 0, d_dst still needs 16 valid bytes. */
+int pcm_stream_probe(const void* d_src, void* d_dst, int64_t lanes, int32_t reads, int32_t writes, int32_t grid, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

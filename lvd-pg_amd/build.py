@@ -9,7 +9,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["api.hip", "hclt_engine.hip", "hclt_queries.hip", "hclt_kld.hip", "hclt_wide.hip", "chow_liu.hip",
-           "pairwise_mi_static.hip", "sparse_engine.hip", "param_rows.hip", "flow_rows.hip"]
+           "pairwise_mi_static.hip", "sparse_engine.hip", "param_rows.hip", "flow_rows.hip", "stream_probe.hip"]
 OUT = os.path.join(HERE, "libpcmi355.so")
 OBJ_DIR = os.path.join(HERE, "build")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

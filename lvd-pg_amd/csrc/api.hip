@@ -342,6 +342,10 @@ int pcm_chow_liu_tree(const float* mi, int32_t num_vars, int32_t* clt_parent) {
   return guarded([&] { pcm::chow_liu_tree(mi, num_vars, clt_parent); });
 }
 
+int pcm_stream_probe(const void* d_src, void* d_dst, int64_t lanes, int32_t reads, int32_t writes, int32_t grid, void* stream) {
+  return guarded([&] { pcm::stream_probe(d_src, d_dst, lanes, reads, writes, grid, static_cast<hipStream_t>(stream)); });
+}
+
 int pcm_set_timing(pcm_circuit* c, int32_t on) {
   return guarded([&] {
     if (on < 0 || on > 15) pcm::fail(PCM_ERR_ARG, "timing mode %d outside 0..15", on);

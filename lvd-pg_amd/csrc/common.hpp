@@ -125,6 +125,7 @@ struct BatchRef {
 // structure learning (chow_liu.hip)
 void pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t n_examples, int num_vars,
                  int num_cats, float pseudocount, float* d_mi, hipStream_t stream);
+void stream_probe(const void* d_src, void* d_dst, int64_t lanes, int reads, int writes, int grid, hipStream_t stream);
 void pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, int64_t n_examples, int num_vars,
                         int num_cats, float pseudocount, float* d_mi, hipStream_t stream);
 void chow_liu_tree(const float* mi, int num_vars, int32_t* parent_out);

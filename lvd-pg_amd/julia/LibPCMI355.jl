@@ -102,5 +102,7 @@ pcm_set_timing(c, on) =
     ccall((:pcm_set_timing, libpcmi355), Cint, (Ptr{Cvoid}, Int32), c, on)
 pcm_get_timing(c, ms, n) =
     ccall((:pcm_get_timing, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int32), c, ms, n)
+pcm_stream_probe(d_src, d_dst, lanes, reads, writes, grid, stream) =
+    ccall((:pcm_stream_probe, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Cvoid}, Int64, Int32, Int32, Int32, Ptr{Cvoid}), d_src, d_dst, lanes, reads, writes, grid, stream)
 
 end # module

@@ -61,6 +61,7 @@ _SIGS = {
     "pcm_gumbel_sample_backward_rows": [H, vp, c_i64, c_i64, c_i32, vp, c_f32, c_i32, c_i32, vp, vp],
     "pcm_normalized_flows": [H, vp, c_i64, c_i64, vp, c_i32, c_i32, vp, c_i64, c_i64],
     "pcm_normalize_params_rows": [H, vp, c_i64, c_i64, c_i32, c_i32],
+    "pcm_stream_probe": [vp, vp, c_i64, c_i32, c_i32, c_i32, vp],
     "pcm_loglikelihoods_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, vp],
     "pcm_flows_soft": [H, vp, c_i64, c_i64, c_i64, vp, c_i32, c_f32, vp, vp],
     "pcm_pairwise_mi": [vp, c_i64, c_i64, c_i64, c_i32, c_i32, c_f32, vp, vp],
