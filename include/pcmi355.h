@@ -100,6 +100,23 @@ int pcm_hclt_create_forest(const int32_t* clt_parent, int32_t num_vars, int32_t 
  */
 int pcm_set_missing_category(pcm_circuit* c, int32_t on);
 
+/*
+ * `soft_reg`, `soft_reg_width` of mini_batch_em_with_reg / probs_flows_circuit_with_reg
+ * (src/regularization/reg_em.jl:208-213, reg_flow.jl:276-282) for HCLT handles on the block kernels: from this call
+ * on, categorical batches (pcm_loglikelihoods, pcm_flows, pcm_em_step) see every leaf at the smoothed value
+ * soft_loglikelihood = log((1 - soft_reg) p[x] + soft_reg mean(p[c], c in the window of x))
+ * (src/regularization/reg_likelihood.jl:4-14; window: c_start = max(0, x - width / 2), c_end = min(c_start + width - 1,
+ * num_cats - 1)), and an example's leaf flow is shared out over x and its window as soft_flow does
+ * (reg_flow.jl:3-22).  as_written != 0: the shares as that source line computes them, with the heap's
+ * LOG-probabilities where probabilities are meant -- (1 - s) logp[x] F / base and s / n logp[c] F / base with
+ * base = (1 - s) logp[x] + s mean(p) -- for parity with the reference as it runs; as_written == 0: the derivative of
+ * the smoothed value, the same lines with probabilities (the form of soft_flow_params,
+ * src/nodes/fixable_categorical_dist.jl:141-160).  soft_reg = 0 switches the smoothing off.  Inner flows and
+ * likelihoods do not depend on as_written.  PCM_ERR_UNSUPPORTED for hidden sizes without block kernels and circuits with
+ * a missing-value category (those smooth through the soft-evidence entry points).
+ */
+int pcm_set_soft_reg(pcm_circuit* c, float soft_reg, int32_t soft_reg_width, int32_t as_written);
+
 /* Head log-parameters of a multi-head HCLT or a forest, [num_trees][num_heads][num_hidden_cats] on the host:
  * the `params` of the head sum nodes (src-jl/multi_head_pc/bit_circuit.jl:14-56 keeps them in the heads'
  * edges), row h of a tree being the head that row h of its head mask seeds. */

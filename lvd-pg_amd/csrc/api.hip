@@ -155,6 +155,10 @@ int pcm_set_missing_category(pcm_circuit* c, int32_t on) {
   return guarded([&] { need_hclt(c)->set_missing_category(on != 0); });
 }
 
+int pcm_set_soft_reg(pcm_circuit* c, float soft_reg, int32_t soft_reg_width, int32_t as_written) {
+  return guarded([&] { need_hclt(c)->set_soft_reg(soft_reg, soft_reg_width, as_written != 0); });
+}
+
 int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf) {
   return guarded([&] { need_hclt(c)->set_block_params(theta, leaf); });
 }

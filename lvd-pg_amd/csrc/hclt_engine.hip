@@ -1062,7 +1062,7 @@ void HcltCircuit::set_block_params(const float* theta, const float* leaf) {
         for (int c = 0; c < C; ++c) t[((size_t)v * C + c) * K + j] = leaf[((size_t)v * K + j) * C + c];
     PCM_HIP(hipMemcpyAsync(d_leaf_.p, t.data(), t.size() * sizeof(float), hipMemcpyHostToDevice, stream));
     PCM_HIP(hipStreamSynchronize(stream));
-    pin_missing_marker();
+    leaf_changed();
   }
 }
 
@@ -1080,8 +1080,45 @@ void HcltCircuit::set_missing_category(bool on) {
   if (on && !(block_ || wide_))
     fail(PCM_ERR_UNSUPPORTED, "a missing-value category needs the block kernels (K = 16, 32, 64 or 128)");
   if (on && C_ < 2) fail(PCM_ERR_SHAPE, "a circuit with a missing-value category needs at least one real category");
+  if (on && soft_reg_ > 0.f) fail(PCM_ERR_UNSUPPORTED, "soft_reg smoothing and a missing-value category together");
   missing_ = on;
   pin_missing_marker();
+}
+
+void HcltCircuit::leaf_changed() {
+  pin_missing_marker();
+  if (soft_reg_ > 0.f) {
+    const int64_t total = (int64_t)V_ * C_ * K_;
+    hipLaunchKernelGGL(hclt_leaf_smooth_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, stream, d_leaf_.p,
+                       d_leaf_smooth_.p, total, C_, K_, soft_reg_, soft_width_);
+    check_launch("leaf_smooth");
+  }
+}
+
+void HcltCircuit::set_soft_reg(float soft_reg, int width, bool as_written) {
+  if (!(soft_reg >= 0.f && soft_reg < 1.f)) fail(PCM_ERR_ARG, "soft_reg must lie in [0, 1), got %g", (double)soft_reg);
+  if (width < 1) fail(PCM_ERR_ARG, "soft_reg_width must be at least 1, got %d", width);
+  if (soft_reg > 0.f) {
+    if (!(block_ || wide_)) fail(PCM_ERR_UNSUPPORTED, "soft_reg smoothing in the kernels needs the block kernels (K = 16, 32, 64 or 128)");
+    if (missing_) fail(PCM_ERR_UNSUPPORTED, "soft_reg smoothing and a missing-value category together");
+    if (flows_in_general_) fail(PCM_ERR_STATE, "the flows of this circuit are held by the layered engine");
+    d_leaf_smooth_.ensure((size_t)V_ * C_ * K_);
+    d_leaf_hist_.ensure((size_t)V_ * C_ * K_);
+  }
+  soft_reg_ = soft_reg;
+  soft_width_ = width;
+  soft_written_ = as_written;
+  leaf_changed();
+}
+
+// the statistics kernels have left the histogram by shown category in d_leaf_hist_
+void HcltCircuit::soft_reg_counts(float rate) {
+  if (!(soft_reg_ > 0.f)) return;
+  const int64_t total = (int64_t)V_ * C_ * K_;
+  hipLaunchKernelGGL(hclt_soft_counts_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, stream, d_leaf_.p,
+                     d_leaf_smooth_.p, d_leaf_hist_.p, d_leaf_flow_.p, total, C_, K_, soft_reg_, soft_width_, rate,
+                     soft_written_ ? 1 : 0);
+  check_launch("soft_counts");
 }
 
 void HcltCircuit::set_heads(const float* heads) {
@@ -1200,7 +1237,7 @@ void HcltCircuit::update_parameters(const float* in, int64_t n) {
   PCM_HIP(hipStreamSynchronize(stream));   // the caller's vector is free again
   rebuild_w();
   general_stale_ = true;
-  pin_missing_marker();
+  leaf_changed();
 }
 
 // ---- batches ------------------------------------------------------------------------
@@ -1241,7 +1278,7 @@ HcltDev HcltCircuit::dev(int batch) const {
   d.nodes = d_nodes_.p;
   d.child_inner = d_child_inner_.p;
   d.child_leaf = d_child_leaf_.p;
-  d.leaf = d_leaf_.p;
+  d.leaf = soft_reg_ > 0.f ? d_leaf_smooth_.p : d_leaf_.p;   // (the smoothed table: categorical batches under soft_reg)
   d.logtheta = d_logtheta_.p;
   d.Wf = d_Wf_.p;
   d.Wb = d_Wb_.p;
@@ -1373,6 +1410,7 @@ void HcltCircuit::run_backward(const HcltDev& d) {
 }
 
 void HcltCircuit::run_stats(const HcltDev& d, float rate) {
+  if (soft_reg_ > 0.f) PCM_HIP(hipMemsetAsync(d_leaf_hist_.p, 0, d_leaf_hist_.n * sizeof(float), stream));   // (the kernels add to rate x what is there)
   // fixed-point split of the flows: limb sums over the padded batch must stay below 2^32
   int bits = 0;
   while ((1 << bits) < d.Bp) ++bits;
@@ -1391,10 +1429,11 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
         // one workgroup fills a compute unit; they draw nodes from d_stat_claim_, which every launch leaves at zero
         PCM_LAUNCH_PHASE(2, hclt_stats_lean_kernel<KK>, dim3(std::min(n_inner_, n_cus_)), dim3(kStatLeanWaves * 64), lds,
-                         d, d_stat_lean_.p, d_edge_aggr_.p, d_leaf_flow_.p, rate, (int)hw, stat_lean_hists_, limb,
+                         d, d_stat_lean_.p, d_edge_aggr_.p, stats_leaf_out(), rate, (int)hw, stat_lean_hists_, limb,
                          (H_ > 0 || d.w) ? (const int*)d_flow_shift_.p : (const int*)nullptr, d_stat_claim_.p, n_inner_);
       });
       check_launch("hclt_stats_lean");
+      soft_reg_counts(rate);
       return;
     }
   }
@@ -1409,12 +1448,13 @@ void HcltCircuit::run_stats(const HcltDev& d, float rate) {
   auto launch = [&](auto kernel) {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     PCM_LAUNCH_PHASE(2, kernel, dim3(n_inner_), dim3(kStatWaves * 64), lds, d, d_stat_items_.p, d_edge_aggr_.p,
-                     d_leaf_flow_.p, rate, nh, (int)hist_words(nh), limb, (H_ > 0 || d.w) ? (const int*)d_flow_shift_.p : (const int*)nullptr);
+                     stats_leaf_out(), rate, nh, (int)hist_words(nh), limb, (H_ > 0 || d.w) ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   };
   PCM_DISPATCH_K(K_, {
     if (d.leaf_slice != 0) launch(&hclt_stats_kernel<KK, true>); else launch(&hclt_stats_kernel<KK, false>);
   });
   check_launch("hclt_stats");
+  soft_reg_counts(rate);
 }
 
 void HcltCircuit::loglikelihoods(const BatchRef& b, float* d_ll) {
@@ -1469,6 +1509,7 @@ HcltDev HcltCircuit::soft_stage(const SoftRef& s) {
 }
 
 void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
+  if (soft_reg_ > 0.f) fail(PCM_ERR_STATE, "soft_reg smoothing is for categorical batches; switch it off for soft evidence");
   no_forest("soft evidence");
   no_missing("soft evidence");
   if (!soft_block_ok()) return general()->loglikelihoods_soft(s, d_ll);
@@ -1481,6 +1522,7 @@ void HcltCircuit::loglikelihoods_soft(const SoftRef& s, float* d_ll) {
 }
 
 void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_mask, float* d_ll) {
+  if (soft_reg_ > 0.f) fail(PCM_ERR_STATE, "soft_reg smoothing is for categorical batches; switch it off for soft evidence");
   no_forest("soft evidence");
   no_missing("soft evidence");
   // (per-example weights on soft evidence -- a mask for a single-head circuit -- go to the layered engine)
@@ -1742,6 +1784,7 @@ void HcltCircuit::em_update(float pseudocount, float inertia) {
     else launch(&hclt_leaf_update_kernel<32>);
   }
   check_launch("leaf_update");
+  leaf_changed();   // (the smoothed table of soft_reg follows the leaf table)
   PCM_DISPATCH_PARAM_K(K_, {
     constexpr int rows_per_block = 256 / (KK < 64 ? KK : 64);
     hipLaunchKernelGGL(hclt_theta_update_kernel<KK>, dim3(ceil_div((int64_t)n_inner_ * K_, rows_per_block)), dim3(256), 0,

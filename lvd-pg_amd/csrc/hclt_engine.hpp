@@ -198,6 +198,9 @@ class HcltCircuit : public pcm_circuit {
   int num_trees() const { return T_; }
   // The last of the num_cats categories becomes the marker of a missing value (see pin_missing_marker).
   void set_missing_category(bool on);
+  // soft_reg > 0: categorical batches are smoothed as reg_likelihood.jl:4-14 has it; as_written: leaf statistics as
+  // reg_flow.jl:12-17 computes them (log-probabilities in the shares) instead of the derivative of the smoothed value
+  void set_soft_reg(float soft_reg, int width, bool as_written);
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 
@@ -244,6 +247,15 @@ class HcltCircuit : public pcm_circuit {
   // what only a single circuit defines (parameter vector order, the general form and the queries on it)
   bool missing_ = false;           // the last category is the marker of a missing value
   void pin_missing_marker();
+  // soft_reg smoothing of categorical data on the block kernels (see hclt_leaf_smooth_kernel)
+  float soft_reg_ = 0.f;
+  int soft_width_ = 1;
+  bool soft_written_ = false;
+  DevBuf<float> d_leaf_smooth_, d_leaf_hist_;
+  void leaf_changed();                          // after anything that rewrites the leaf table
+  float* stats_leaf_out() { return soft_reg_ > 0.f ? d_leaf_hist_.p : d_leaf_flow_.p; }
+  float stats_leaf_rate(float rate) const { return soft_reg_ > 0.f ? 0.f : rate; }
+  void soft_reg_counts(float rate);             // histogram by shown category -> leaf statistics
   void no_missing(const char* what) const {
     if (missing_)
       fail(PCM_ERR_UNSUPPORTED, "%s is not defined for a circuit with a missing-value category (likelihoods, flows and EM are)",

@@ -811,6 +811,70 @@ __global__ __launch_bounds__(256) void hclt_theta_update_kernel(const HcltNode* 
   }
 }
 
+// ---- soft_reg: smoothing of categorical data (src/regularization/reg_likelihood.jl:4-14, reg_flow.jl:3-22) ----------
+// The smoothed value of a leaf depends on the example only through its category x:
+//   soft_loglikelihood = log((1 - s) p[x] + s * mean(p[c], c in the window of x)),
+//   window: c_start = max(0, x - width / 2) .. c_end = min(c_start + width - 1, C - 1),
+// so it is a table of the shape of the leaf table itself, and the walks and the statistics kernel run on it as they
+// run on the leaf table, on the categories as they are.  The statistics then hold, per leaf and category x, the flow
+// of the examples that SHOWED x; soft_flow shares such an example's flow out over x and its window, which is a
+// banded linear map of that histogram, applied by hclt_soft_counts_kernel.
+__device__ __forceinline__ void soft_window(int x, int width, int C, int& c0, int& c1) {
+  c0 = max(0, x - width / 2);
+  c1 = min(c0 + width - 1, C - 1);
+}
+
+// smooth[v][x][k] from leaf[v][c][k]; thread = (v, x, k), k fastest
+__global__ __launch_bounds__(256) void hclt_leaf_smooth_kernel(const float* __restrict__ leaf, float* __restrict__ smooth,
+                                                               int64_t total, int C, int K, float s, int width) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int k = (int)(i % K), x = (int)((i / K) % C);
+  const float* row = leaf + (i / ((int64_t)C * K)) * (int64_t)C * K + k;
+  int c0, c1;
+  soft_window(x, width, C, c0, c1);
+  float sp = 0.f;
+  for (int c = c0; c <= c1; ++c) sp += __expf(row[(int64_t)c * K]);
+  sp /= (float)(c1 - c0 + 1);
+  // PCs.logsumexp(logp + log(1 - s), log(sp) + log(s)), written on the probabilities
+  smooth[i] = __logf((1.f - s) * __expf(row[(int64_t)x * K]) + s * sp);
+}
+
+// leaf_flow[v][c][k] = rate * leaf_flow[v][c][k] + sum over the categories x whose window holds c (or x = c) of
+//   hist[v][x][k] * ((x == c) (1 - s) q[x] + (c in window(x)) s / n(x) q[c]) / base(x),
+// where hist is the statistics' histogram by shown category.  soft_flow as the source has it (reg_flow.jl:12-17) takes
+// q = the heap entries, i.e. LOG-probabilities, and base = (1 - s) logp[x] + s mean(p[window]) (as_written != 0);
+// the derivative of the smoothed value -- the form of soft_flow_params, src/nodes/fixable_categorical_dist.jl:141-160 --
+// takes q = p and base = (1 - s) p[x] + s mean(p[window]) = exp(smooth[x]).
+__global__ __launch_bounds__(256) void hclt_soft_counts_kernel(const float* __restrict__ leaf, const float* __restrict__ smooth,
+                                                               const float* __restrict__ hist, float* __restrict__ leaf_flow,
+                                                               int64_t total, int C, int K, float s, int width, float rate,
+                                                               int as_written) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int k = (int)(i % K), c = (int)((i / K) % C);
+  const int64_t base_v = (i / ((int64_t)C * K)) * (int64_t)C * K + k;
+  const float lc = leaf[base_v + (int64_t)c * K];
+  const float qc = as_written ? lc : __expf(lc);
+  float acc = 0.f;
+  // x - width / 2 <= c (or c_start = 0) and c <= c_start + width - 1: x within [c - width, c + width / 2]
+  for (int x = max(0, c - width); x <= min(C - 1, c + width / 2); ++x) {
+    int c0, c1;
+    soft_window(x, width, C, c0, c1);
+    const bool in_window = c >= c0 && c <= c1;
+    if (!in_window && x != c) continue;
+    const float h = hist[base_v + (int64_t)x * K];
+    if (h == 0.f) continue;
+    const float lx = leaf[base_v + (int64_t)x * K], bs = __expf(smooth[base_v + (int64_t)x * K]);
+    const float base = as_written ? (1.f - s) * lx + (bs - (1.f - s) * __expf(lx)) : bs;
+    float coef = 0.f;
+    if (x == c) coef += (1.f - s) * qc;
+    if (in_window) coef += s / (float)(c1 - c0 + 1) * qc;
+    acc += h * coef / base;
+  }
+  leaf_flow[i] = (rate != 0.f ? rate * leaf_flow[i] : 0.f) + acc;
+}
+
 // Leaf update (the reference's per-input-node update with missing_flow = 0), one workgroup
 // per (variable, run of 32 hidden states): thread (category group cg, hidden state j) holds the
 // flows and parameters of its categories (every kCats-th one) in registers -- all of its requests

@@ -714,11 +714,13 @@ void HcltCircuit::wide_backward_stats(const HcltDev& d, float rate, bool soft) {
                           (const float*)d_logtheta_.p, d_edge_aggr_.p, rate);
   });
   const size_t lds = 2 * (size_t)C_ * 17 * sizeof(unsigned);
+  if (!soft && soft_reg_ > 0.f) PCM_HIP(hipMemsetAsync(d_leaf_hist_.p, 0, d_leaf_hist_.n * sizeof(float), stream));   // (the kernel adds to rate x what is there)
   if (!soft)
     hipExtLaunchKernelGGL(hclt_wide_leaf_kernel, dim3(V_, K_ / 16), dim3(kWideLeafWaves * 64), (uint32_t)lds, stream, nullptr,
-                          t_stat ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, d_leaf_flow_.p, rate, limb,
+                          t_stat ? ev[5] : nullptr, 0, d, d_G_.p, d_wide_state_node_.p, K_, stats_leaf_out(), rate, limb,
                           d.w ? (const int*)d_flow_shift_.p : (const int*)nullptr);
   check_launch_w("hclt_wide_stats");
+  if (!soft) soft_reg_counts(rate);
 }
 
 }  // namespace pcm

@@ -20,6 +20,8 @@ pcm_hclt_create_forest(clt_parent, num_vars, num_hidden_cats, num_cats, num_head
     ccall((:pcm_hclt_create_forest, libpcmi355), Cint, (Ptr{Int32}, Int32, Int32, Int32, Int32, Ptr{Ptr{Cvoid}}), clt_parent, num_vars, num_hidden_cats, num_cats, num_heads, out)
 pcm_set_missing_category(c, on) =
     ccall((:pcm_set_missing_category, libpcmi355), Cint, (Ptr{Cvoid}, Int32), c, on)
+pcm_set_soft_reg(c, soft_reg, soft_reg_width, as_written) =
+    ccall((:pcm_set_soft_reg, libpcmi355), Cint, (Ptr{Cvoid}, Float32, Int32, Int32), c, soft_reg, soft_reg_width, as_written)
 pcm_hclt_set_heads(c, heads) =
     ccall((:pcm_hclt_set_heads, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}), c, heads)
 pcm_hclt_get_heads(c, heads) =

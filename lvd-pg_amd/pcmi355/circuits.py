@@ -120,6 +120,12 @@ class HcltCircuit(BitsCircuit):
         check(lib.pcm_hclt_get_flows(self.handle, np_ptr(ea), np_ptr(lf)))
         return ea, lf
 
+    def set_soft_reg(self, soft_reg, soft_reg_width=1, as_written=False):
+        """`soft_reg` / `soft_reg_width` smoothing of categorical batches inside the block kernels
+        (src/regularization/reg_likelihood.jl:4-14, reg_flow.jl:3-22); `as_written`: leaf statistics as `soft_flow`
+        computes them.  0 switches it off.  `mini_batch_em_with_reg` sets and clears it around its loop."""
+        check(lib.pcm_set_soft_reg(self.handle, float(soft_reg), int(soft_reg_width), int(bool(as_written))))
+
     def set_missing_category(self, on=True):
         """Declares the last category (num_cats - 1) the marker of a missing value: data carry it where the
         reference's data hold `missing` (src/regularization/reg_likelihood.jl:40-47); the leaf then counts as

@@ -206,7 +206,8 @@ def soft_reg_evidence(rows, num_cats, soft_reg, soft_reg_width):
 def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1,
                            ent_reg=0.0, param_inertia, param_inertia_end=None, flow_memory=0.0,
                            shuffle="each_epoch", verbose=False, generator=None, head_mask=None, eval_dataset=None,
-                           eval_interval=0, weights=None, eval_weights=None, init_clear_mem=True):
+                           eval_interval=0, weights=None, eval_weights=None, init_clear_mem=True, soft_flow="derivative",
+                           soft_reg_route=None):
     """`mini_batch_em_with_reg` (src/regularization/reg_em.jl:208-336).  Returns the list
     of per-epoch mean log-likelihoods.  ent_reg must be 0 (the reference's entropy regulariser is
     commented out at :294-296).  `data` may be 3-D float32 soft evidence, as for the top-level circuits of
@@ -221,18 +222,46 @@ def mini_batch_em_with_reg(bpc, data, num_epochs, *, batch_size, pseudocount, so
     the flows the circuit holds from an earlier call as the flow memory of the first batch; the circuit owns its
     accumulators, so this is the reference's `edge_aggr_mem` given and not cleared.
 
-    soft_reg > 0 on categorical data (reg_likelihood.jl:4-14, reg_flow.jl:3-22): every batch is turned into
-    the soft evidence that gives the leaves the reference's smoothed value (`soft_reg_evidence`) and runs
-    through the soft-evidence kernels.  Likelihoods are the reference's; the leaf flows are the derivative of
-    that value -- (1 - s) p[x] / base for the observed category and s / n * p[c] / base over the window, the
-    form of `soft_flow_params` (src/nodes/fixable_categorical_dist.jl:141-160) -- whereas `soft_flow` as
-    written (reg_flow.jl:12-17) puts log-probabilities where these probabilities stand."""
+    soft_reg > 0 on categorical data (reg_likelihood.jl:4-14, reg_flow.jl:3-22).  HCLT handles on the block kernels
+    smooth inside the kernels (`pcm_set_soft_reg`: the leaves' smoothed values are a table of the shape of the leaf
+    table, the walks run on the categories as they are); every other circuit has each batch turned into the soft
+    evidence that gives the leaves the same value (`soft_reg_evidence`) and runs through the soft-evidence kernels
+    (`soft_reg_route` = "kernels" / "evidence" insists on one of the two).  Likelihoods and inner flows are the
+    reference's either way.  `soft_flow`: "derivative" shares a leaf's flow out as (1 - s) p[x] / base for the observed
+    category and s / n * p[c] / base over the window -- the derivative of the smoothed value, the form of
+    `soft_flow_params` (src/nodes/fixable_categorical_dist.jl:141-160); "as_written" as `soft_flow` itself computes it
+    (reg_flow.jl:12-17), with log-probabilities where these probabilities stand: what the reference's own runs with
+    soft_reg > 0 accumulate.  "as_written" needs the kernel route."""
     if ent_reg != 0.0:
         raise NotImplementedError("ent_reg other than 0 is not supported (commented out in the reference)")
     _check_data(bpc, data)
     smooth = soft_reg != 0.0 and not _is_soft(data)
     if smooth and not 0.0 < soft_reg < 1.0:
         raise ValueError("soft_reg must lie in [0, 1)")
+    if soft_flow not in ("derivative", "as_written"):
+        raise ValueError("soft_flow is 'derivative' or 'as_written'")
+    in_kernels = False
+    if smooth and soft_reg_route != "evidence":
+        rc = lib.pcm_set_soft_reg(bpc.handle, float(soft_reg), int(soft_reg_width), int(soft_flow == "as_written"))
+        in_kernels = rc == 0
+        if not in_kernels and (soft_reg_route == "kernels" or soft_flow == "as_written"):
+            check(rc)
+    if smooth and not in_kernels and soft_flow == "as_written":
+        raise NotImplementedError("soft_flow = 'as_written' needs the kernel route (an HCLT handle on the block kernels)")
+    try:
+        return _em_loop(bpc, data, num_epochs, batch_size, pseudocount, soft_reg, soft_reg_width, param_inertia,
+                        param_inertia_end, flow_memory, shuffle, verbose, generator, head_mask, eval_dataset, eval_interval,
+                        weights, eval_weights, init_clear_mem, smooth and not in_kernels)
+    finally:
+        if in_kernels:
+            check(lib.pcm_set_soft_reg(bpc.handle, 0.0, 1, 0))
+
+
+def _em_loop(bpc, data, num_epochs, batch_size, pseudocount, soft_reg, soft_reg_width, param_inertia, param_inertia_end,
+             flow_memory, shuffle, verbose, generator, head_mask, eval_dataset, eval_interval, weights, eval_weights,
+             init_clear_mem, smooth):
+    """The batch loop of `mini_batch_em_with_reg` (src/regularization/reg_em.jl:236-336); `smooth`: soft_reg through
+    the soft-evidence entry points."""
     n = data.shape[0]
     if batch_size > n:
         raise ValueError("batch_size must not exceed the number of examples")   # reg_em.jl:219

@@ -243,6 +243,36 @@ def input_flows_soft(fc, ev, mars, flows, leaf_flow=None, double=False):
     return leaf_flow
 
 
+def soft_flow_counts(fc, data, flows, soft_reg, soft_reg_width, as_written=True, leaf_flow=None, double=False):
+    """`soft_flow` over a batch (src/regularization/reg_flow.jl:3-22, called per input node and example by
+    input_flows_circuit_with_reg_kernel, :24-48): an input node's flow goes to the observed category and to the
+    categories of its window.  as_written: the lines as they stand, with the heap's entries -- LOG-probabilities -- in
+    the shares and in the first term of `base`; otherwise the same lines on probabilities, i.e. the derivative of
+    `soft_loglikelihood` (reg_likelihood.jl:4-14).  data [B, V] categories, flows [n_nodes, B]; returns the counts in
+    the layout of fc.leaf_logp.  Plain loops: small cases only."""
+    R = _real(double)
+    leaf = np.asarray(fc.leaf_logp, dtype=R)
+    out = np.zeros(len(leaf), dtype=R) if leaf_flow is None else leaf_flow
+    s, C = R(soft_reg), fc.C
+    for n in range(fc.n_nodes):
+        if fc.type[n] != 0:
+            continue
+        v, off = int(fc.in_var[n]), int(fc.in_off[n])
+        heap = leaf[off:off + C]
+        for b in range(data.shape[0]):
+            value = int(data[b, v])
+            node_flow = R(flows[n, b])
+            c_start = max(0, value - soft_reg_width // 2)
+            c_end = min(c_start + soft_reg_width - 1, C - 1)
+            sp = np.exp(heap[c_start:c_end + 1]).sum(dtype=R) / R(c_end - c_start + 1)
+            q = heap if as_written else np.exp(heap)
+            base = (R(1) - s) * q[value] + s * sp
+            out[off + value] += (R(1) - s) * q[value] * node_flow / base
+            for c in range(c_start, c_end + 1):
+                out[off + c] += s / R(c_end - c_start + 1) * q[c] * node_flow / base
+    return out
+
+
 def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False, missing=False):
     """Returns the updated (logp, leaf_logp).  missing: the last row of every leaf table marks a missing value
     (log-probability 0; data carry category C - 1 where the reference has `missing`), and the flow it collected

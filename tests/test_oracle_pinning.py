@@ -1017,3 +1017,58 @@ def test_normalize_params_against_scipy():
     back = O.normalize_params(fc, got, undo=True, double=True)
     np.testing.assert_allclose(back[:, ns:], np.log(got[:, ns:] + 1e-6), rtol=1e-6)
     np.testing.assert_allclose(back[:, :ns], got[:, :ns], atol=1e-6)     # already normalised: unchanged
+
+
+# ---- soft_flow: the leaf statistics under soft_reg (src/regularization/reg_flow.jl:3-22) ----------------------
+
+def test_soft_flow_as_written_by_hand():
+    """One leaf, worked by hand from the source lines.  p = (0.5, 0.3, 0.2), x = 1, soft_reg = 0.1, width 3, node flow 2:
+    window 0..2, sp = 1/3, base = 0.9 ln 0.3 + 0.1 / 3 = -1.08357552 + 0.03333333 = -1.05024219;
+    counts[1] = (0.9 ln 0.3 + (0.1 / 3) ln 0.3) * 2 / base = -2.2474159 / -1.05024219 = 2.139903,
+    counts[0] = (0.1 / 3) ln 0.5 * 2 / base = -0.04620981 / -1.05024219 = 0.0439992,
+    counts[2] = (0.1 / 3) ln 0.2 * 2 / base = -0.1072959 / -1.05024219 = 0.1021630.
+    Then a window cut by the end of the range: p = (0.1, 0.2, 0.3, 0.4), x = 3: c_start = 2, c_end = min(4, 3) = 3, n = 2,
+    sp = 0.35, base = 0.9 ln 0.4 + 0.035 = -0.78966166: counts = (0, 0, 0.05 ln 0.3 * 2 / base, 0.95 ln 0.4 * 2 / base)
+    = (0, 0, 0.1524669, 2.2046814).  With probabilities in place of the logarithms (as_written = False) the shares of
+    a leaf add up to its flow; as written they do not."""
+    from types import SimpleNamespace
+
+    def leaf(p):
+        return SimpleNamespace(n_nodes=1, type=np.array([O.INPUT], np.uint8), in_var=np.array([0], np.int32),
+                               in_off=np.array([0], np.int64), leaf_logp=np.log(np.array(p)), C=len(p))
+    flows = np.array([[2.0]])
+    got = O.soft_flow_counts(leaf([0.5, 0.3, 0.2]), np.array([[1]]), flows, 0.1, 3, as_written=True, double=True)
+    np.testing.assert_allclose(got, [0.0439992, 2.139903, 0.1021630], rtol=2e-6)
+    got = O.soft_flow_counts(leaf([0.1, 0.2, 0.3, 0.4]), np.array([[3]]), flows, 0.1, 3, as_written=True, double=True)
+    np.testing.assert_allclose(got, [0.0, 0.0, 0.1524669, 2.2046814], rtol=2e-6, atol=1e-12)
+    assert abs(got.sum() - 2.0) > 0.1
+    der = O.soft_flow_counts(leaf([0.1, 0.2, 0.3, 0.4]), np.array([[3]]), flows, 0.1, 3, as_written=False, double=True)
+    assert abs(der.sum() - 2.0) < 1e-12
+    np.testing.assert_allclose(der, [0, 0, 0.05 * 0.3 * 2 / (0.9 * 0.4 + 0.035), 0.95 * 0.4 * 2 / (0.9 * 0.4 + 0.035)], rtol=1e-12)
+
+
+def test_soft_flow_derivative_form_is_the_soft_evidence_flow():
+    """With probabilities where the source has heap entries, soft_flow is the leaf flow of the soft evidence that gives
+    the leaves the smoothed value -- `orc_input_flows_soft`, pinned by central differences in tests/test_soft_evidence.py
+    -- on a whole HCLT, windows cut at both ends included."""
+    V, K, C, B, s, width = 6, 3, 7, 9, 0.15, 4
+    parent, theta, leaf, fc = make_hclt(V, K, C, 5)
+    rng = np.random.default_rng(3)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    data[0, :] = 0
+    data[1, :] = C - 1
+    ev = np.full((B, V, C), -np.inf)
+    for b in range(B):
+        for v in range(V):
+            x = int(data[b, v])
+            c0 = max(0, x - width // 2)
+            c1 = min(c0 + width - 1, C - 1)
+            ev[b, v, c0:c1 + 1] = np.log(s / (c1 - c0 + 1))
+            ev[b, v, x] = np.log(np.exp(ev[b, v, x]) + 1 - s)
+    mars = O.forward_soft(fc, ev, double=True)
+    fl, _ = O.backward(fc, mars, double=True)
+    want = O.input_flows_soft(fc, ev, mars, fl, double=True)
+    got = O.soft_flow_counts(fc, data, fl, s, width, as_written=False, double=True)
+    np.testing.assert_allclose(got, want, rtol=1e-9, atol=1e-12)
+    written = O.soft_flow_counts(fc, data, fl, s, width, as_written=True, double=True)
+    assert np.abs(written - want).max() > 1e-3        # the two forms are not the same numbers

@@ -280,3 +280,100 @@ def test_em_with_soft_reg_matches_oracle(gpu):
     with pytest.raises(NotImplementedError):
         P.mini_batch_em_with_reg(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=0.01, ent_reg=0.1,
                                  param_inertia=0.9)
+
+
+def _soft_reg_oracle_step(fc, batch, s, width, pseudocount, inertia, as_written):
+    """One batch of mini_batch_em_with_reg with soft_reg on the float64 oracle: values and inner flows from the evidence
+    worked out line by line, leaf statistics from `soft_flow` (reg_flow.jl:3-22) in the form asked for."""
+    B, V = batch.shape
+    C = fc.C
+    ev = np.full((B, V, C), -np.inf)
+    for i in range(B):
+        for v in range(V):
+            x = int(batch[i, v])
+            c0 = max(0, x - width // 2)
+            c1 = min(c0 + width - 1, C - 1)
+            ev[i, v, c0:c1 + 1] = np.log(s / (c1 - c0 + 1))
+            ev[i, v, x] = np.log(np.exp(ev[i, v, x]) + 1 - s)
+    mars = O.forward_soft(fc, ev, double=True)
+    fl, ea = O.backward(fc, mars, double=True)
+    counts = O.soft_flow_counts(fc, batch, fl, s, width, as_written=as_written, double=True)
+    new_logp, new_leaf = O.em_update(fc, ea, counts, pseudocount, inertia, double=True)
+    return mars[-1], ea, counts, new_logp, new_leaf
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("K,V,max_children,form", [(16, 9, 3, "as_written"), (16, 9, 3, "derivative"), (32, 12, 5, "as_written"),
+                                                   (64, 7, 5, "as_written"), (128, 6, 3, "as_written"), (128, 6, 3, "derivative")])
+def test_soft_reg_in_the_kernels_matches_oracle(gpu, K, V, max_children, form):
+    """soft_reg smoothing inside the block kernels (pcm_set_soft_reg): likelihoods, sum-edge statistics and the leaf
+    statistics in both forms -- `soft_flow` as written (reg_flow.jl:12-17, pinned by a hand-worked literal) and the
+    derivative of the smoothed value -- and the parameters after two batches, against the float64 oracle; on the lean
+    walks (K = 16), a tree whose wide nodes are split (K = 32, five children), the general statistics kernel (K = 64)
+    and the wide kernels (K = 128).  Flow memory carries the first batch's statistics into the second."""
+    torch, P = gpu
+    from pcmi355._lib import lib, check
+    C, B, s, width, pc, inertia = 13, 40, 0.05, 5, 0.02, 0.8
+    parent, theta, leaf, fc = make_hclt(V, K, C, 31 + K, max_children=max_children)
+    rng = np.random.default_rng(K)
+    data = rng.integers(0, C, size=(2 * B, V)).astype(np.uint8)
+    data[0, :] = 0
+    data[1, :] = C - 1
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    d = torch.from_numpy(data).cuda()
+    ll = torch.empty(B, device="cuda")
+    print(f"soft_reg in kernels: K={K} V={V} form={form}", flush=True)
+    check(lib.pcm_set_soft_reg(bpc.handle, s, width, int(form == "as_written")))
+    # one batch: statistics against the oracle's
+    check(lib.pcm_flows(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, None, ll.data_ptr()))
+    want_ll, want_ea, want_counts, _, _ = _soft_reg_oracle_step(fc, data[:B], s, width, pc, inertia, form == "as_written")
+    np.testing.assert_allclose(ll.cpu().numpy(), want_ll, rtol=1e-5, atol=1e-5)
+    _, leaf_flow = bpc.get_flows()                                         # [V, K, C]
+    want = want_counts.reshape(V, K, C)
+    assert np.abs(leaf_flow - want).max() < 2e-5 * np.abs(want).max(), np.abs(leaf_flow - want).max()
+    check(lib.pcm_set_soft_reg(bpc.handle, 0.0, 1, 0))
+    # the driver: two batches with flow memory, parameters against the oracle's
+    lls = P.mini_batch_em_with_reg(bpc, d, 1, batch_size=B, pseudocount=pc, soft_reg=s, soft_reg_width=width,
+                                   param_inertia=inertia, shuffle="none", flow_memory=0.0, soft_flow=form, soft_reg_route="kernels")
+    want_lls = []
+    for b0 in (0, B):
+        wl, _, _, new_logp, new_leaf = _soft_reg_oracle_step(fc, data[b0:b0 + B], s, width, pc, inertia, form == "as_written")
+        want_lls.append(wl.mean())
+        fc.logp, fc.leaf_logp = new_logp.astype(np.float32), new_leaf.astype(np.float32)
+    assert abs(lls[0] - np.mean(want_lls)) < 1e-5 * abs(np.mean(want_lls))
+    _, leaf_after = bpc.get_params()
+    want_leaf = fc.leaf_logp.reshape(V, K, C)
+    assert np.abs(np.exp(leaf_after) - np.exp(want_leaf)).max() < 1e-4 * np.exp(want_leaf).max()
+    # the smoothing is off again: plain likelihoods
+    plain = P.loglikelihoods(bpc, d[:B]).cpu().numpy()
+    mars = O.forward(fc, data[:B], double=True)
+    np.testing.assert_allclose(plain, mars[-1], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_soft_reg_routes_agree_and_as_written_needs_the_kernels(gpu):
+    """The kernel route and the soft-evidence route of mini_batch_em_with_reg(soft_reg > 0) train the same parameters
+    (derivative form); a circuit without block kernels takes the evidence route by itself and refuses `as_written`."""
+    torch, P = gpu
+    V, K, C, B, s, width = 8, 16, 11, 48, 0.02, 5
+    parent, theta, leaf, fc = make_hclt(V, K, C, 77)
+    data = torch.from_numpy(np.random.default_rng(7).integers(0, C, size=(2 * B, V)).astype(np.uint8)).cuda()
+    out = []
+    for route in ("kernels", "evidence"):
+        bpc = P.hclt_from_clt(parent, C, K)
+        bpc.set_params(block_theta(parent, K, theta), leaf)
+        lls = P.mini_batch_em_with_reg(bpc, data, 2, batch_size=B, pseudocount=0.01, soft_reg=s, soft_reg_width=width,
+                                       param_inertia=0.9, shuffle="none", soft_reg_route=route)
+        out.append((lls, bpc.get_params()))
+    np.testing.assert_allclose(out[0][0], out[1][0], rtol=1e-5)
+    np.testing.assert_allclose(np.exp(out[0][1][1]), np.exp(out[1][1][1]), rtol=2e-4, atol=1e-7)
+    np.testing.assert_allclose(np.exp(out[0][1][0]), np.exp(out[1][1][0]), rtol=2e-4, atol=1e-7)
+    parent5, theta5, leaf5, _ = make_hclt(6, 5, C, 3)
+    odd = P.hclt_from_clt(parent5, C, 5)                                   # K = 5: no block kernels
+    odd.set_params(block_theta(parent5, 5, theta5), leaf5)
+    P.mini_batch_em_with_reg(odd, data[:, :6].contiguous(), 1, batch_size=B, pseudocount=0.01, soft_reg=s, soft_reg_width=width,
+                             param_inertia=0.9, shuffle="none")
+    with pytest.raises(Exception):
+        P.mini_batch_em_with_reg(odd, data[:, :6].contiguous(), 1, batch_size=B, pseudocount=0.01, soft_reg=s,
+                                 soft_reg_width=width, param_inertia=0.9, shuffle="none", soft_flow="as_written")
