@@ -9,7 +9,7 @@ from .circuits import (BitsCircuit, HcltCircuit, HcltForest, hclt_from_clt, mult
                        hclt_forest_from_clts, compile_circuit,
                        compile_multihead, CuBitsProbCircuit, CuMultiHeadBitsProbCircuit, node_maps, write_back_parameters)
 from .queries import (loglikelihoods, loglikelihood, loglikelihoods_probcat, loglikelihood_probcat, weighted_ll,
-                      probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em,  # noqa: F401
+                      probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em, mini_batch_em_beta,  # noqa: F401
                       vectorize_parameters, update_parameters, kld, kld_backward, sample, adam_step,
                       mini_batch_em_for_multihead_pc, multihead_loglikelihoods, gumbel_sample, gumbel_sample_rows, gumbel_sample_backward_rows,
                       patch_level_evidence, flow_gradients, adam, soft_reg_evidence, forest_loglikelihoods, forest_flows,

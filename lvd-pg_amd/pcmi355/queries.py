@@ -330,6 +330,86 @@ def _em_loop(bpc, data, num_epochs, batch_size, pseudocount, soft_reg, soft_reg_
     return lls
 
 
+def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_reg=0.0, soft_reg_width=1, param_inertia,
+                       param_inertia_end=None, flow_memory=0.0, flow_memory_end=None, shuffle="each_epoch",
+                       update_interval=1, fscale=1.0, verbose=False, generator=None, eval_dataset=None, eval_interval=0,
+                       soft_flow="derivative"):
+    """`mini_batch_em_beta` (src-jl/learning/em.jl:289-409): the EM loop whose statistics collect over
+    `update_interval` batches before the parameters move, with a schedule for the flow memory as well as for the
+    inertia.  As the source has it: the accumulators are cleared at the start of every epoch; at a batch with
+    `batch_id % update_interval == 1` (1-based) they are cleared again (flow_memory = 0) or scaled by
+    max(0, 1 - (batch_size + pseudocount) / flow_memory); every batch adds its flows; after a batch with
+    `batch_id % update_interval == 0` the parameters are updated.  (With update_interval = 1 the first condition never
+    holds, so the statistics of an epoch pile up while the parameters move after every batch -- kept as written.)
+    `fscale` other than 1 (flows of the tempered posterior, src-jl/learning/flow.jl:120-370) is not built; soft_reg > 0
+    needs an HCLT handle on the block kernels (`pcm_set_soft_reg`).
+    Returns the per-epoch mean log-likelihoods."""
+    if fscale != 1.0:
+        raise NotImplementedError("fscale other than 1 (tempered flows, src-jl/learning/flow.jl:120-370) is not built")
+    _check_data(bpc, data)
+    if pseudocount < 0 or not 0 <= param_inertia <= 1:
+        raise ValueError("pseudocount >= 0 and 0 <= param_inertia <= 1")                        # em.jl:299-300
+    param_inertia_end = param_inertia if param_inertia_end is None else param_inertia_end
+    flow_memory_end = flow_memory if flow_memory_end is None else flow_memory_end
+    if not param_inertia <= param_inertia_end <= 1 or not 0 <= flow_memory <= flow_memory_end:
+        raise ValueError("param_inertia <= param_inertia_end <= 1 and 0 <= flow_memory <= flow_memory_end")   # :301-303
+    if shuffle not in ("once", "each_epoch", "each_batch", "none"):
+        raise ValueError("shuffle is once, each_epoch or each_batch")
+    if update_interval < 1:
+        raise ValueError("update_interval must be at least 1")
+    n = data.shape[0]
+    if batch_size > n:
+        raise ValueError("batch_size must not exceed the number of examples")
+    num_batches = n // batch_size
+    smooth = soft_reg != 0.0
+    if smooth:
+        check(lib.pcm_set_soft_reg(bpc.handle, float(soft_reg), int(soft_reg_width), int(soft_flow == "as_written")))
+    perm = torch.arange(n, dtype=torch.int32, device=data.device)
+
+    def do_shuffle():
+        nonlocal perm
+        perm = torch.randperm(n, generator=generator).to(device=data.device, dtype=torch.int32)
+
+    d_inertia = (param_inertia_end - param_inertia) / num_epochs
+    d_memory = (flow_memory_end - flow_memory) / num_epochs
+    ll = torch.empty(batch_size, dtype=torch.float32, device=data.device)
+    lls = []
+    try:
+        if shuffle == "once":
+            do_shuffle()
+        for epoch in range(1, num_epochs + 1):
+            if shuffle == "each_epoch":
+                do_shuffle()
+            acc = torch.zeros((), dtype=torch.float64, device=data.device)
+            cleared = True                                                                      # em.jl:344-345
+            for batch_id in range(1, num_batches + 1):
+                if shuffle == "each_batch":
+                    do_shuffle()
+                rate = 1.0
+                if batch_id % update_interval == 1:                                             # :354-363
+                    rate = 0.0 if flow_memory == 0 else max(0.0, 1.0 - (batch_size + pseudocount) / flow_memory)
+                if cleared:
+                    rate, cleared = 0.0, False
+                ids = perm[(batch_id - 1) * batch_size:batch_id * batch_size]
+                _flows(bpc, data, ids.data_ptr(), batch_size, rate, None, ll.data_ptr())
+                acc += ll.sum(dtype=torch.float64)
+                if batch_id % update_interval == 0:                                             # :373-379
+                    check(lib.pcm_em_update(bpc.handle, float(pseudocount), float(param_inertia)))
+            lls.append(float(acc.item()) / batch_size / num_batches)
+            param_inertia += d_inertia
+            flow_memory += d_memory
+            if verbose:
+                if eval_dataset is not None and eval_interval > 0 and epoch % eval_interval == 0:
+                    test_ll = loglikelihood(bpc, eval_dataset, batch_size=min(batch_size, eval_dataset.shape[0]))
+                    print(f"Mini-batch EM epoch {epoch}/{num_epochs}: train LL {lls[-1]} - test LL {test_ll}")
+                else:
+                    print(f"Mini-batch EM epoch {epoch}/{num_epochs}; train LL {lls[-1]}")
+    finally:
+        if smooth:
+            check(lib.pcm_set_soft_reg(bpc.handle, 0.0, 1, 0))
+    return lls
+
+
 def mini_batch_em(bpc, data, num_epochs, *, batch_size, pseudocount, param_inertia, param_inertia_end=None,
                   flow_memory=0.0, shuffle="each_epoch", **kw):
     """`PCs.mini_batch_em` as called by test/sgd/adam_tests.jl:20: the same loop without

@@ -273,10 +273,12 @@ def soft_flow_counts(fc, data, flows, soft_reg, soft_reg_width, as_written=True,
     return out
 
 
-def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False, missing=False):
+def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False, missing=False, return_aggr=False):
     """Returns the updated (logp, leaf_logp).  missing: the last row of every leaf table marks a missing value
     (log-probability 0; data carry category C - 1 where the reference has `missing`), and the flow it collected
-    is the `missing_flow` of nodes/fixable_categorical_dist.jl:233-241."""
+    is the `missing_flow` of nodes/fixable_categorical_dist.jl:233-241.  return_aggr: also the edge statistics as the
+    update leaves them -- `add_pseudocount` works in place (src/regularization/reg_em.jl:292), so under a flow memory
+    the pseudocount of one update is part of what the next batch decays."""
     R = _real(double)
     logp = np.ascontiguousarray(fc.logp, dtype=R).copy()
     leaf = np.ascontiguousarray(fc.leaf_logp, dtype=R).copy()
@@ -286,6 +288,8 @@ def em_update(fc, edge_aggr, leaf_flow, pseudocount, inertia, double=False, miss
     lib(double).orc_em_update(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(logp), _p(ea),
                               _p(fc.in_off), ctypes.c_int(fc.C), _p(leaf), _p(lf),
                               rc(pseudocount), rc(inertia), ctypes.c_int(int(bool(missing))))
+    if return_aggr:
+        return logp, leaf, ea
     return logp, leaf
 
 

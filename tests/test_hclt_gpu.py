@@ -870,3 +870,51 @@ def test_deep_trees_three_way(gpu, oracle, V, K, C, B, chain, weighted):
         depth = max(depth, n)
     assert_three_way((th, lf_new), (th64, lf64), (th32, lf32), PARAM_RTOL,
                      f"V={V} K={K} C={C} B={B} depth={depth} weighted={weighted}")
+
+
+@pytest.mark.parametrize("update_interval,flow_memory", [(2, 0.0), (3, 400.0), (1, 0.0)])
+def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update_interval, flow_memory):
+    """`mini_batch_em_beta` (src-jl/learning/em.jl:289-409): statistics collect over `update_interval` batches, are
+    cleared (or decayed by the flow memory) at a batch with batch_id % update_interval == 1, and the parameters move
+    after a batch with batch_id % update_interval == 0 -- replayed on the float64 oracle batch by batch, including the
+    source's behaviour at update_interval = 1 (the clearing condition never holds, the statistics of an epoch pile up)."""
+    torch, P = gpu
+    from helpers import make_hclt, correlated_data, block_theta, rel_err
+    V, K, C, B, nb, pc, inertia = 10, 16, 12, 64, 6, 0.1, 0.7
+    parent, theta, leaf, fc = make_hclt(V, K, C, 5)
+    data = correlated_data(B * nb, V, C, 6, parent)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    lls = P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 2, batch_size=B, pseudocount=pc, param_inertia=inertia,
+                               param_inertia_end=0.9, flow_memory=flow_memory, flow_memory_end=flow_memory * 2,
+                               shuffle="none", update_interval=update_interval)
+    cur, want, inr, fm = fc.copy(), [], inertia, flow_memory
+    for epoch in range(2):
+        ea = lf = None
+        tot = 0.0
+        for batch_id in range(1, nb + 1):
+            idx = np.arange((batch_id - 1) * B, batch_id * B, dtype=np.int32)
+            if ea is not None and batch_id % update_interval == 1:
+                rate = 0.0 if fm == 0 else max(0.0, 1.0 - (B + pc) / fm)
+                ea, lf = ea * rate, lf * rate
+            mars = oracle.forward(cur, data, idx, True)
+            flows, ea_b = oracle.backward(cur, mars, double=True)
+            lf_b = oracle.input_flows(cur, data, flows, idx, double=True)
+            ea = ea_b if ea is None else ea + ea_b
+            lf = lf_b if lf is None else lf + lf_b
+            tot += mars[-1].sum()
+            if batch_id % update_interval == 0:
+                logp, new_leaf, ea = oracle.em_update(cur, ea, lf, pc, inr, True, return_aggr=True)   # (the pseudocount stays in)
+                cur = cur.copy()
+                cur.logp, cur.leaf_logp = logp.astype(np.float32), new_leaf.astype(np.float32)
+        want.append(tot / B / nb)
+        inr += (0.9 - inertia) / 2
+        fm += flow_memory / 2
+    assert np.abs(np.array(lls) - np.array(want)).max() < 2e-5 * abs(want[0])
+    th_ref, leaf_ref = oracle.hclt_block_params(cur)
+    th, lf_new = bpc.get_params()
+    for v, blk in th_ref.items():
+        assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
+    assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
+    with pytest.raises(NotImplementedError):
+        P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia, fscale=2.0)
