@@ -447,6 +447,9 @@ def main():
                     help="chow_liu: learned by the library from 32768 training images; gaussian: host stand-in")
     ap.add_argument("--cpu-sample", type=int, default=4096)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--constant-categories", action="store_true",
+                    help="ablation for the byte counters: every example shows category 0 everywhere after the tree is "
+                         "built, so each leaf table is read at one row (what the leaf rows cost in fetches)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MiB",
                     help="also launch one plain device copy of this many MiB before the timed region "
                          "(a known-size kernel to scale hardware byte counters against)")
@@ -475,6 +478,8 @@ def main():
     bpc = pcmi355.hclt_from_clt(cfg["parent"], C, K)
     bpc.set_params(cfg["theta"], cfg["leaf"])
     data = torch.from_numpy(cfg["data"]).cuda()
+    if args.constant_categories:
+        data.zero_()
     ll = torch.empty(B, dtype=torch.float32, device="cuda")
 
     def step():
