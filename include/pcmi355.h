@@ -159,7 +159,10 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
  * 12 heads (0 for a single-root circuit), 13 nodes of the description the circuit was
  * built from (0 for an HCLT built from its tree), 14 which kernels run likelihoods and flows:
  * 0 per-layer kernels, 1 lean tree walks, 2 general tree walks, 3 wide block kernels, 15 trees (1 unless
- * the handle is a forest). */
+ * the handle is a forest), 16 dense groups of a pcm_circuit_create circuit: sets of sum nodes of one layer with one
+ * and the same list of children, which run as blocks on the matrix cores instead of edge by edge (0 for an HCLT
+ * handle, and for every circuit created while PCMI355_DENSE_GROUPS=0 is in the environment: a switch for comparisons,
+ * results agree to rounding), 17 nodes whose values the per-layer kernels compute (the others are the groups'). */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.

@@ -959,6 +959,8 @@ int64_t HcltCircuit::size(int what) const {
     case 13: return 0;
     case 14: return wide_walk_ ? 3 : !block_ ? 0 : lean_ ? 1 : 2;
     case 15: return T_;
+    case 16: return 0;
+    case 17: return 0;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }

@@ -3,8 +3,11 @@
 
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <numeric>
+#include <tuple>
 #include <type_traits>
+#include <unordered_map>
 
 #include "stage_kernel.hip.hpp"
 
@@ -187,6 +190,10 @@ void FlatCircuit::finish() {
 // kernels
 // ---------------------------------------------------------------------------------------
 
+}  // namespace pcm
+#include "sparse_groups.hip.hpp"
+namespace pcm {
+
 struct SparseDev {
   const uint8_t* type;
   const int32_t* order;      // node ids sorted by layer
@@ -207,6 +214,7 @@ struct SparseDev {
   float* flows;
   int32_t B, Bp, C;
   int64_t n_nodes;
+  int64_t n_flow_rows;       // node rows of the flow array + the rows dense groups hand their children
 };
 
 // ProbabilisticCircuits.jl logsumexp(x, y) as used by src/queries/likelihood.jl:101-102.
@@ -557,7 +565,7 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   const int i0 = uni(rec.z), i1 = uni(rec.w);
   const int per = (i1 - i0 + kLayerWaves - 1) / kLayerWaves;
   const int my0 = min(i0 + wave * per, i1), my1 = min(my0 + per, i1);
-  const Rows<kBuf> mars(d.mars, d.n_nodes + 1, d.Bp), flows(d.flows, d.n_nodes, d.Bp);
+  const Rows<kBuf> mars(d.mars, d.n_nodes + 1, d.Bp), flows(d.flows, d.n_flow_rows, d.Bp);
   int c0 = my0;
   if constexpr (kMaxRun >= 32)
     for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
@@ -745,10 +753,13 @@ __global__ __launch_bounds__(256) void sparse_leaf_flow_soft_kernel(SparseDev d,
     }
 }
 
+// (a record that names a dense group's row behind the node rows is not an edge: its flow is taken as it is)
 __global__ void sparse_gather_in_logp_kernel(const int4* __restrict__ in_rec, const float* __restrict__ logp, int64_t n,
-                                             float* __restrict__ in_logp) {
+                                             int64_t n_nodes, float* __restrict__ in_logp) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < n) in_logp[i] = logp[in_rec[i].x >> 1];
+  if (i >= n) return;
+  const int4 r = in_rec[i];
+  in_logp[i] = (r.y < 0 && (int64_t)~r.y >= n_nodes) ? 0.f : logp[r.x >> 1];
 }
 
 __global__ void sparse_scale_kernel(float* p, int64_t n, float rate) {
@@ -1041,9 +1052,245 @@ __global__ __launch_bounds__(64 * kMixGroups) void sparse_head_mixture_kernel(co
   out[b] = M + logf(S) - logf(T);
 }
 
+// Edge flows of product edges whose child takes its flow from a group's kernel instead of a layer's: the edge's flow
+// is its parent's, summed over each block of 64 examples into the block's row of partial sums.  One wave per
+// (edge, block).
+__global__ __launch_bounds__(256) void sparse_product_edge_kernel(const int2* __restrict__ pairs, int n_pairs,
+                                                                  const float* __restrict__ flows, int Bp,
+                                                                  float* __restrict__ edge_part, int64_t n_edges) {
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (i >= n_pairs) return;
+  const int2 pe = pairs[i];
+  const float tot = wave_sum(flows[(size_t)pe.y * Bp + (size_t)blockIdx.y * 64 + lane]);
+  if (lane == 0) edge_part[(size_t)blockIdx.y * n_edges + pe.x] = tot;
+}
+
 // ---------------------------------------------------------------------------------------
 // host
 // ---------------------------------------------------------------------------------------
+
+// Dense groups: sum nodes of one layer over one and the same set of (prime, sub) children (each may list them in an
+// order of its own), at least kGroupMinSide sums over at least kGroupMinSide children and at most kGroupMaxSide of
+// either (more sums: several groups over the same children).  group_of[node] = group or -1; edge_slot[edge] = the
+// child's number among all groups' children (its "slot") for the edges of a group's first sum, -1 for all others.
+// PCMI355_DENSE_GROUPS=0 in the environment keeps every node on the layer kernels (for comparisons).
+constexpr int kGroupMinSide = 4, kGroupMinEdges = 64, kGroupMaxSide = 128;
+static_assert(sizeof(GroupRec) == 2 * sizeof(int4), "a group's record is uploaded as two int4");
+
+void SparseCircuit::build_groups(std::vector<int32_t>& group_of, std::vector<int32_t>& edge_slot) {
+  const int64_t nn = fc_.n_nodes();
+  const char* env = std::getenv("PCMI355_DENSE_GROUPS");
+  std::vector<int32_t> g_node, g_edge, g_prime;
+  struct Found { int layer; std::vector<int32_t> nodes; };
+  std::vector<Found> found;
+  // a sum's edges ordered by (prime, sub): the order of a group's children
+  auto sorted_edges = [&](int32_t n) {
+    std::vector<int32_t> es(fc_.node_e1[n] - fc_.node_e0[n]);
+    for (size_t i = 0; i < es.size(); ++i) es[i] = fc_.node_e0[n] + (int32_t)i;
+    std::sort(es.begin(), es.end(), [&](int32_t a, int32_t b) {
+      return std::make_tuple(fc_.e_prime[a], fc_.e_sub[a], a) < std::make_tuple(fc_.e_prime[b], fc_.e_sub[b], b);
+    });
+    return es;
+  };
+  if (!(env && env[0] == '0')) {
+    // candidates by (layer, number of children, hash of the children), then compared child by child
+    std::unordered_map<uint64_t, std::vector<int32_t>> buckets;
+    for (int64_t n = 0; n < nn; ++n) {
+      const int c = fc_.node_e1[n] - fc_.node_e0[n];
+      if (fc_.type[n] != kSum || c < kGroupMinSide || c > kGroupMaxSide) continue;
+      uint64_t h = 1469598103934665603ull ^ (uint64_t)fc_.layer[n];
+      for (int32_t e : sorted_edges((int32_t)n)) {
+        h = (h ^ (uint64_t)(uint32_t)fc_.e_prime[e]) * 1099511628211ull;
+        h = (h ^ (uint64_t)(uint32_t)fc_.e_sub[e]) * 1099511628211ull;
+      }
+      buckets[h].push_back((int32_t)n);
+    }
+    auto same_children = [&](int32_t a, int32_t b) {
+      if (fc_.layer[a] != fc_.layer[b] || fc_.node_e1[b] - fc_.node_e0[b] != fc_.node_e1[a] - fc_.node_e0[a]) return false;
+      const std::vector<int32_t> ea = sorted_edges(a), eb = sorted_edges(b);
+      for (size_t i = 0; i < ea.size(); ++i)
+        if (fc_.e_prime[ea[i]] != fc_.e_prime[eb[i]] || fc_.e_sub[ea[i]] != fc_.e_sub[eb[i]]) return false;
+      return true;
+    };
+    std::vector<uint64_t> keys;
+    for (auto& kv : buckets) keys.push_back(kv.first);
+    std::sort(keys.begin(), keys.end());   // (an order that does not depend on the hash table's)
+    for (uint64_t k : keys) {
+      std::vector<int32_t>& cand = buckets[k];   // ascending node ids
+      std::vector<char> used(cand.size(), 0);
+      for (size_t i = 0; i < cand.size(); ++i) {
+        if (used[i]) continue;
+        std::vector<int32_t> members{cand[i]};
+        for (size_t j = i + 1; j < cand.size(); ++j)
+          if (!used[j] && same_children(cand[i], cand[j])) { members.push_back(cand[j]); used[j] = 1; }
+        const int c = fc_.node_e1[cand[i]] - fc_.node_e0[cand[i]];
+        for (size_t m0 = 0; m0 < members.size(); m0 += kGroupMaxSide) {
+          const size_t g = std::min<size_t>(kGroupMaxSide, members.size() - m0);
+          if ((int)g < kGroupMinSide || (int64_t)g * c < kGroupMinEdges) continue;
+          found.push_back(Found{fc_.layer[cand[i]], std::vector<int32_t>(members.begin() + m0, members.begin() + m0 + g)});
+        }
+      }
+    }
+  }
+  auto tiles = [](int x) { int t = 1; while (t * 16 < x) t *= 2; return t; };   // 16-row tiles, a power of two of them
+  std::sort(found.begin(), found.end(), [&](const Found& a, const Found& b) {
+    const int ca = fc_.node_e1[a.nodes[0]] - fc_.node_e0[a.nodes[0]], cb = fc_.node_e1[b.nodes[0]] - fc_.node_e0[b.nodes[0]];
+    const auto ka = std::make_tuple(a.layer, tiles((int)a.nodes.size()), tiles(ca), a.nodes[0]);
+    const auto kb = std::make_tuple(b.layer, tiles((int)b.nodes.size()), tiles(cb), b.nodes[0]);
+    return ka < kb;
+  });
+  for (size_t gi = 0; gi < found.size(); ++gi)
+    for (int32_t n : found[gi].nodes) group_of[n] = (int32_t)gi;
+  // A product of at most three factors that only groups use, as the prime of a child, is computed by those groups
+  // (every one of them writes its value; the values are the same).
+  grp_expanded_.assign(nn, 0);
+  if (!found.empty()) {
+    std::vector<char> used_by_group(nn, 0), used_otherwise(nn, 0);
+    for (int64_t e = 0; e < fc_.n_edges(); ++e) {
+      const int32_t p = fc_.e_parent[e], pr = fc_.e_prime[e], sb = fc_.e_sub[e];
+      (group_of[p] >= 0 ? used_by_group : used_otherwise)[pr] = 1;
+      if (sb >= 0) used_otherwise[sb] = 1;
+    }
+    for (int32_t hd : fc_.heads) used_otherwise[hd] = 1;
+    used_otherwise[nn - 1] = 1;
+    for (int64_t n = 0; n < nn; ++n) {
+      if (fc_.type[n] != kMul || !used_by_group[n] || used_otherwise[n]) continue;
+      int factors = 0;
+      for (int e = fc_.node_e0[n]; e < fc_.node_e1[n]; ++e) factors += 1 + (fc_.e_sub[e] >= 0);
+      grp_expanded_[n] = factors <= 3;
+    }
+  }
+  // the device tables, padded to the tiles: Gp entries of sums and Cp of children per group, Gp x Cp of W
+  std::vector<int4> g_rows, dev_recs;
+  std::vector<int32_t> g_own, elem, shape_gt, shape_ct;
+  group_launches_.clear();
+  group_stat_launches_.clear();
+  grp_pslot_h_.clear();
+  const int32_t zrow = (int32_t)nn;
+  int32_t n_slots = 0;
+  for (size_t gi = 0; gi < found.size(); ++gi) {
+    const Found& f = found[gi];
+    const std::vector<int32_t> first = sorted_edges(f.nodes[0]);
+    const int32_t c = (int32_t)first.size(), gn = (int32_t)f.nodes.size();
+    const int gt = tiles(gn), ct = tiles(c);
+    shape_gt.push_back(gt);
+    shape_ct.push_back(ct);
+    const int32_t pnode0 = (int32_t)g_node.size(), pslot0 = (int32_t)g_rows.size();
+    const int64_t pw0 = (int64_t)elem.size();
+    dev_recs.push_back(int4{gn, c, pnode0, pslot0});
+    dev_recs.push_back(int4{(int32_t)(pw0 & 0xffffffff), (int32_t)(pw0 >> 32), gt, ct});
+    elem.insert(elem.end(), (size_t)gt * 16 * ct * 16, (int32_t)gi);
+    for (int i = 0; i < gt * 16; ++i) {
+      g_node.push_back(i < gn ? f.nodes[i] : -1);
+      std::vector<int32_t> es;
+      if (i < gn) es = sorted_edges(f.nodes[i]);
+      for (int k = 0; k < ct * 16; ++k) g_edge.push_back(i < gn && k < c ? es[k] : -1);
+    }
+    for (int i = 0; i < ct * 16; ++i) {
+      if (i >= c) { g_rows.push_back(int4{zrow, zrow, zrow, zrow}); g_own.push_back(-2); continue; }
+      const int32_t pr = fc_.e_prime[first[i]], sb = fc_.e_sub[first[i]];
+      edge_slot[first[i]] = n_slots + i;
+      g_prime.push_back(pr);
+      grp_pslot_h_.push_back(pslot0 + i);
+      int32_t r[3] = {pr, zrow, zrow};   // (the row of zeros)
+      if (grp_expanded_[pr]) {
+        int k = 0;
+        for (int e = fc_.node_e0[pr]; e < fc_.node_e1[pr]; ++e) {
+          r[k++] = fc_.e_prime[e];
+          if (fc_.e_sub[e] >= 0) r[k++] = fc_.e_sub[e];
+        }
+      }
+      g_rows.push_back(int4{r[0], r[1], r[2], sb >= 0 ? sb : zrow});
+      g_own.push_back(grp_expanded_[pr] ? pr : -1);
+    }
+    n_slots += c;
+    if (!group_launches_.empty() && group_launches_.back().layer == f.layer && group_launches_.back().gt == gt &&
+        group_launches_.back().ct == ct)
+      group_launches_.back().count++;
+    else
+      group_launches_.push_back(GroupLaunch{f.layer, (int)gi, 1, gt, ct, pnode0, pslot0, pw0});
+  }
+  n_group_slots_ = n_slots;
+  n_groups_ = (int64_t)found.size();
+  grp_prime_h_ = g_prime;
+  if (found.empty()) return;
+  {   // the groups by shape, for the launches that take all layers at once
+    std::vector<int32_t> by_shape(found.size());
+    for (size_t gi = 0; gi < found.size(); ++gi) by_shape[gi] = (int32_t)gi;
+    auto shape = [&](int32_t gi) { return std::make_pair(shape_gt[gi], shape_ct[gi]); };
+    std::stable_sort(by_shape.begin(), by_shape.end(), [&](int32_t a, int32_t b) { return shape(a) < shape(b); });
+    for (size_t i = 0; i < by_shape.size(); ++i) {
+      const auto s = shape(by_shape[i]);
+      if (!group_stat_launches_.empty() && group_stat_launches_.back().gt == s.first && group_stat_launches_.back().ct == s.second)
+        group_stat_launches_.back().count++;
+      else
+        group_stat_launches_.push_back(GroupLaunch{-1, (int)i, 1, s.first, s.second, 0, 0, 0});
+    }
+    d_grp_order_.upload(by_shape);
+  }
+  n_group_elems_ = (int64_t)elem.size();
+  d_grp_elem_.upload(elem);
+  d_grp_wf_.alloc(elem.size());
+  d_grp_wb_.alloc(elem.size());
+  d_grp_rec_.upload(dev_recs);
+  d_grp_node_.upload(g_node);
+  d_grp_edge_.upload(g_edge);
+  d_grp_rows_.upload(g_rows);
+  d_grp_own_.upload(g_own);
+}
+
+#define PCM_GROUP_DEV(g, batch_, bp_)                                                                                 \
+  GroupDev g{};                                                                                                      \
+  g.rec = reinterpret_cast<const GroupRec*>(d_grp_rec_.p);                                                           \
+  g.node = d_grp_node_.p; g.edge = d_grp_edge_.p;   g.rows = d_grp_rows_.p; g.own = d_grp_own_.p;                    \
+  g.copies = d_grp_copies_.p; g.order = d_grp_order_.p; g.wf = d_grp_wf_.p; g.wb = d_grp_wb_.p; g.m = d_grp_m_.p;       \
+  g.logp = d_logp_.p; g.mars = d_mars_.p; g.flows = d_flows_.p; g.edge_part = d_edge_part_.p;                        \
+  g.n_nodes = fc_.n_nodes(); g.n_edges = fc_.n_edges(); g.B = batch_; g.Bp = bp_
+
+// exp of the groups' log-parameters, before a forward pass
+void SparseCircuit::refresh_group_w() {
+  if (n_group_elems_ == 0) return;
+  PCM_GROUP_DEV(g, 0, 0);
+  hipLaunchKernelGGL(sparse_group_w_kernel, dim3((unsigned)ceil_div(n_group_elems_, 256)), dim3(256), 0, stream, g, d_grp_elem_.p,
+                     n_group_elems_);
+}
+
+// the group kernels of one layer: what = 0 values going up, 1 the children's rows going down; what = 2: the edge
+// flows of every group, after the backward pass
+void SparseCircuit::launch_groups(int layer, int what, int Bp, int batch) {
+  if (group_launches_.empty()) return;
+  PCM_GROUP_DEV(g, batch, Bp);
+  for (const GroupLaunch& L : what == 2 ? group_stat_launches_ : group_launches_) {
+    if (what != 2 && L.layer != layer) continue;
+    const size_t lds = what == 2 ? group_lds_floats(L.gt * 16, L.ct * 16) * sizeof(float) : 0;
+    const dim3 grid(L.count, what == 2 ? Bp / 64 : Bp / 16), block(what == 2 ? 256 : 64);
+    const GroupBase base{L.group0, L.pnode0, L.pslot0, L.pw0};
+    auto run = [&](auto kernel, auto arg) {
+      if (lds > 48 * 1024)
+        PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(kernel, grid, block, lds, stream, g, arg);
+    };
+#define PCM_GROUP_CT(GT_, CT_)                                                     \
+    if (what == 0) run(&sparse_group_forward_kernel<GT_, CT_>, base);              \
+    else if (what == 1) run(&sparse_group_backward_kernel<GT_, CT_>, base);        \
+    else run(&sparse_group_stats_kernel<GT_, CT_>, L.group0);
+#define PCM_GROUP_GT(GT_)                                                          \
+    switch (L.ct) {                                                                \
+      case 1: PCM_GROUP_CT(GT_, 1) break;                                          \
+      case 2: PCM_GROUP_CT(GT_, 2) break;                                          \
+      case 4: PCM_GROUP_CT(GT_, 4) break;                                          \
+      default: PCM_GROUP_CT(GT_, 8) break;                                         \
+    }
+    switch (L.gt) {
+      case 1: PCM_GROUP_GT(1) break;
+      case 2: PCM_GROUP_GT(2) break;
+      case 4: PCM_GROUP_GT(4) break;
+      default: PCM_GROUP_GT(8) break;
+    }
+#undef PCM_GROUP_GT
+#undef PCM_GROUP_CT
+  }
+}
 
 SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   const int64_t nn = fc_.n_nodes(), ne = fc_.n_edges();
@@ -1056,11 +1303,6 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   layer_node0_.assign(n_layers_ + 1, 0);
   for (int64_t i = 0; i < nn; ++i) layer_node0_[fc_.layer[order[i]] + 1]++;
   for (int l = 0; l < n_layers_; ++l) layer_node0_[l + 1] += layer_node0_[l];
-  layer_max_children_.assign(n_layers_, 0);
-  for (int l = 0; l < n_layers_; ++l)
-    for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i)
-      if (fc_.type[order[i]] != kInput)
-        layer_max_children_[l] = std::max(layer_max_children_[l], (int)(fc_.node_e1[order[i]] - fc_.node_e0[order[i]]));
   // incoming edges per node: entry = edge << 1 | as_sub
   std::vector<int32_t> in_ptr(nn + 1, 0), in_edge;
   for (int64_t e = 0; e < ne; ++e) { in_ptr[fc_.e_prime[e] + 1]++; if (fc_.e_sub[e] >= 0) in_ptr[fc_.e_sub[e] + 1]++; }
@@ -1074,25 +1316,100 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
     }
   }
   if (in_edge.empty()) in_edge.push_back(0);
-  std::vector<int4> in_rec(in_edge.size());
-  for (size_t i = 0; i < in_edge.size() && ne; ++i) {
-    const int32_t e = in_edge[i] >> 1, p = fc_.e_parent[e];
+  // dense groups: their sums' edges leave the records of the backward pass, one record per (group, child) takes
+  // their place in the child's list (at the place of the first of them)
+  std::vector<int32_t> group_of(nn, -1), edge_slot(std::max<int64_t>(ne, 1), -1);
+  build_groups(group_of, edge_slot);
+  // the backward pass's records per node, in the order of the edges: {edge << 1 | role, parent (~parent: product),
+  // prime, sub} or, for a group's row, {slot << 1 | 1, ~(n_nodes + slot), row of zeros, row of zeros}: read like the
+  // flow of a product parent, never written to the edge sums (odd first word)
+  struct Entry { int4 rec; int32_t key; uint8_t role; };   // key: edge, or -1 - slot; role 1: the node is the sub
+  std::vector<std::vector<Entry>> in_list(nn);
+  const int32_t zrow = (int32_t)nn;
+  for (int64_t e = 0; e < ne; ++e) {
+    const int32_t p = fc_.e_parent[e], pr = fc_.e_prime[e], sb = fc_.e_sub[e];
+    if (group_of[p] >= 0) {
+      const int32_t slot = edge_slot[e];
+      if (slot < 0) continue;   // (one record per child: from the edges of the group's first sum)
+      const int4 rec{(slot << 1) | 1, ~(int32_t)(nn + slot), zrow, zrow};
+      in_list[pr].push_back(Entry{rec, -1 - slot, 0});
+      if (sb >= 0) in_list[sb].push_back(Entry{rec, -1 - slot, 1});
+      continue;
+    }
     // operands an edge does not have name the row of zeros behind the last node's: the flow through a product
     // edge is its parent's (exponent 0 - 0 + 0 - 0), a sum edge without a second child adds 0
     const bool sum_edge = fc_.type[p] == kSum;
-    const int32_t zrow = (int32_t)nn;
-    in_rec[i] = int4{in_edge[i], sum_edge ? p : ~p, sum_edge ? fc_.e_prime[e] : zrow,
-                     sum_edge && fc_.e_sub[e] >= 0 ? fc_.e_sub[e] : zrow};
+    const int4 rec{(int32_t)(e << 1), sum_edge ? p : ~p, sum_edge ? pr : zrow, sum_edge && sb >= 0 ? sb : zrow};
+    in_list[pr].push_back(Entry{rec, (int32_t)e, 0});
+    if (sb >= 0) in_list[sb].push_back(Entry{int4{rec.x | 1, rec.y, rec.z, rec.w}, (int32_t)e, 1});
   }
+  // A node that a single group row reaches, and nothing else, has that row as its flow, and so has a node whose only
+  // parent is such a product: the group's kernel writes their rows (up to kGroupCopies per child) and they leave the
+  // backward layers (in an HCLT: every product, every sum below the root's and every leaf).  The row itself is kept
+  // only where a node that stays in the layers reads it.
+  std::vector<char> copied(nn, 0);
+  if (n_group_slots_) {
+    std::vector<char> is_seed(nn, 0);
+    if (fc_.heads.empty()) is_seed[nn - 1] = 1;
+    else for (int32_t hd : fc_.heads) is_seed[hd] = 1;
+    std::vector<int32_t> slot_of(nn, -1);
+    std::vector<std::vector<int32_t>> rows_of((size_t)n_group_slots_);
+    for (int64_t i = nn - 1; i >= 0; --i) {   // parents before children
+      const int32_t n = order[i];
+      if (in_list[n].size() != 1 || is_seed[n]) continue;
+      const Entry& en = in_list[n][0];
+      int32_t slot = -1;
+      if (en.key < 0) slot = -1 - en.key;
+      else if (fc_.type[fc_.e_parent[en.key]] == kMul && copied[fc_.e_parent[en.key]]) slot = slot_of[fc_.e_parent[en.key]];
+      if (slot < 0 || (int)rows_of[slot].size() >= kGroupCopies - 1) continue;
+      slot_of[n] = slot;
+      copied[n] = 1;
+      rows_of[slot].push_back(n);
+    }
+    for (int64_t n = 0; n < nn; ++n) {
+      if (copied[n]) continue;
+      for (const Entry& en : in_list[n])
+        if (en.key < 0 && (rows_of[-1 - en.key].empty() || rows_of[-1 - en.key][0] != (int32_t)(nn + (-1 - en.key))))
+          rows_of[-1 - en.key].insert(rows_of[-1 - en.key].begin(), (int32_t)(nn + (-1 - en.key)));
+    }
+    std::vector<int4> copies(2 * d_grp_rows_.n, int4{-1, -1, -1, -1});   // (by entry of the padded per-child tables)
+    for (int64_t s = 0; s < n_group_slots_; ++s) {
+      int32_t r[kGroupCopies];
+      for (int k = 0; k < kGroupCopies; ++k) r[k] = k < (int)rows_of[s].size() ? rows_of[s][k] : -1;
+      copies[2 * (size_t)grp_pslot_h_[s]] = int4{r[0], r[1], r[2], r[3]};
+      copies[2 * (size_t)grp_pslot_h_[s] + 1] = int4{r[4], r[5], r[6], r[7]};
+    }
+    d_grp_copies_.upload(copies);
+    // the product edges that no layer kernel sums any more (it is the wave of an edge's prime that does)
+    std::vector<int2> pe;
+    for (int64_t n = 0; n < nn; ++n)
+      if (copied[n] && in_list[n][0].key >= 0 && in_list[n][0].role == 0) pe.push_back(int2{in_list[n][0].key, fc_.e_parent[in_list[n][0].key]});
+    n_group_product_edges_ = (int)pe.size();
+    if (!pe.empty()) d_grp_product_edges_.upload(pe);
+  }
+  std::vector<int32_t> rec_ptr(nn + 1, 0);
+  for (int64_t n = 0; n < nn; ++n) rec_ptr[n + 1] = rec_ptr[n] + (int32_t)in_list[n].size();
+  std::vector<int4> in_rec(std::max<size_t>(rec_ptr[nn], 1), int4{0, 0, 0, 0});
+  for (int64_t n = 0; n < nn; ++n)
+    for (size_t q = 0; q < in_list[n].size(); ++q) in_rec[rec_ptr[n] + q] = in_list[n][q].rec;
   d_in_rec_.upload(in_rec);
   d_type_.upload(fc_.type);
   d_order_.upload(order);
-  {
-    std::vector<int4> fr(nn);
-    for (int64_t i = 0; i < nn; ++i) {
-      const int32_t n = order[i];
-      fr[i] = int4{n, (int)fc_.type[n], fc_.node_e0[n], fc_.node_e1[n]};
+  {   // the forward layers: the nodes that no group's kernel computes
+    std::vector<int4> fr;
+    fwd_layer0_.assign(n_layers_ + 1, 0);
+    layer_max_children_.assign(n_layers_, 0);
+    for (int l = 0; l < n_layers_; ++l) {
+      for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i) {
+        const int32_t n = order[i];
+        if (group_of[n] >= 0 || grp_expanded_[n]) continue;
+        fr.push_back(int4{n, (int)fc_.type[n], fc_.node_e0[n], fc_.node_e1[n]});
+        if (fc_.type[n] != kInput) layer_max_children_[l] = std::max(layer_max_children_[l], (int)(fc_.node_e1[n] - fc_.node_e0[n]));
+      }
+      fwd_layer0_[l + 1] = (int)fr.size();
     }
+    n_layer_nodes_ = (int64_t)fr.size();
+    if (fr.empty()) fr.push_back(int4{0, 0, 0, 0});
     d_fwd_rec_.upload(fr);
   }
   d_node_e0_.upload(fc_.node_e0); d_node_e1_.upload(fc_.node_e1);
@@ -1115,13 +1432,14 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   // layers and the prime's wave writes its row too (in an HCLT: every leaf).
   std::vector<int32_t> alias_of(nn, -1);
   for (int64_t b = 0; b < nn && ne; ++b) {
-    const int i0 = in_ptr[b], i1 = in_ptr[b + 1];
-    if (fc_.type[b] != kInput || seed_of[b] >= 0 || i0 == i1 || !(in_edge[i0] & 1)) continue;
-    const int32_t a = fc_.e_prime[in_edge[i0] >> 1];
-    if (a == b || in_ptr[a + 1] - in_ptr[a] != i1 - i0) continue;
+    const auto& lb = in_list[b];
+    if (fc_.type[b] != kInput || seed_of[b] >= 0 || lb.empty() || !lb[0].role || copied[b]) continue;
+    // the prime beside which b stands in its first record
+    const int32_t a = lb[0].key >= 0 ? fc_.e_prime[lb[0].key] : grp_prime_h_[-1 - lb[0].key];
+    if (a == b || copied[a] || in_list[a].size() != lb.size()) continue;
     bool same = true;
-    for (int q = 0; q < i1 - i0 && same; ++q)
-      same = (in_edge[i0 + q] & 1) && in_edge[in_ptr[a] + q] == (in_edge[i0 + q] & ~1);
+    for (size_t q = 0; q < lb.size() && same; ++q)
+      same = lb[q].role == 1 && in_list[a][q].role == 0 && in_list[a][q].key == lb[q].key;
     if (same) alias_of[b] = a;
   }
   std::vector<int32_t> alias_ptr(nn + 1, 0), alias_list;
@@ -1138,9 +1456,9 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
   bwd_layer_max_in_.assign(n_layers_, 0);
   for (int l = 0; l < n_layers_; ++l) {
     for (int i = layer_node0_[l]; i < layer_node0_[l + 1]; ++i)
-      if (alias_of[order[i]] < 0) {
+      if (alias_of[order[i]] < 0 && !copied[order[i]]) {
         bwd_order.push_back(order[i]);
-        bwd_layer_max_in_[l] = std::max(bwd_layer_max_in_[l], (int)(in_ptr[order[i] + 1] - in_ptr[order[i]]));
+        bwd_layer_max_in_[l] = std::max(bwd_layer_max_in_[l], (int)(rec_ptr[order[i] + 1] - rec_ptr[order[i]]));
       }
     bwd_layer0_[l + 1] = (int)bwd_order.size();
   }
@@ -1151,7 +1469,7 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
     std::vector<int2> ar(br.size(), int2{0, 0});
     for (size_t i = 0; i < bwd_order.size(); ++i) {
       const int32_t n = bwd_order[i];
-      br[i] = int4{n, seed_of[n], in_ptr[n], in_ptr[n + 1]};
+      br[i] = int4{n, seed_of[n], rec_ptr[n], rec_ptr[n + 1]};
       ar[i] = int2{alias_ptr[n], alias_ptr[n + 1]};
     }
     d_bwd_rec_.upload(br);
@@ -1184,6 +1502,8 @@ int64_t SparseCircuit::size(int what) const {
     case 13: return (int64_t)fc_.desc_node.size();
     case 14: return 0;
     case 15: return 1;
+    case 16: return n_groups_;
+    case 17: return n_layer_nodes_;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -1245,7 +1565,7 @@ void SparseCircuit::ensure_batch(int batch) {
   if (batch <= cap_batch_) return;
   const int Bp = ceil_div(batch, 64) * 64;
   d_mars_.alloc((size_t)(fc_.n_nodes() + 1) * Bp);   // one more row, of zeros: the operand an edge does not have
-  d_flows_.alloc((size_t)fc_.n_nodes() * Bp);
+  d_flows_.alloc((size_t)n_flow_rows() * Bp);
   cap_batch_ = Bp;
 }
 
@@ -1259,7 +1579,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
   d.type = type; d.order = order; d.node_e0 = e0; d.node_e1 = e1; d.e_parent = ep; d.e_prime = epr; d.e_sub = es;
   d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off;
   d.ev = nullptr; d.ev_se = d.ev_sv = d.ev_sc = 0; d.ev_idx = nullptr; d.logp = logp; d.leaf = leaf;
-  d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C; d.n_nodes = n_nodes;
+  d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C; d.n_nodes = n_nodes; d.n_flow_rows = n_nodes;
   return d;
 }
 
@@ -1267,7 +1587,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
 // signed 32-bit scalars)
 #define PCM_LAYER_LAUNCH(kernel, EX_, W_, RUN_, grid, ...)                                                      \
   do {                                                                                                          \
-    if ((int64_t)(fc_.n_nodes() + 1) * Bp * 4 < ((int64_t)1 << 31))                                             \
+    if ((int64_t)(n_flow_rows() + 1) * Bp * 4 < ((int64_t)1 << 31))                                             \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, true>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);         \
     else                                                                                                        \
       hipLaunchKernelGGL((kernel<EX_, W_, RUN_, false>), grid, dim3((W_) * 64), 0, stream, __VA_ARGS__);        \
@@ -1315,8 +1635,12 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
     hipLaunchKernelGGL(sparse_soft_input_kernel, dim3(fc_.num_vars, Bp / kSoftTile), dim3(256), 0, stream, d, d_var_ptr_.p,
                        d_var_nodes_.p);
   }
+  refresh_group_w();
+  if (n_groups_) d_grp_m_.ensure((size_t)n_groups_ * Bp);
   for (int l = 0; l < n_layers_; ++l) {
-    const int n0 = layer_node0_[l], cnt = layer_node0_[l + 1] - n0;
+    const int n0 = fwd_layer0_[l], cnt = fwd_layer0_[l + 1] - n0;
+    launch_groups(l, 0, Bp, batch);
+    if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
     if (layer_max_children_[l] <= kNarrowDegree) {
       if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), d, n0);
@@ -1385,12 +1709,13 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
                        d_leaf_flow_.p, (int64_t)fc_.leaf_logp.size(), rate);
   }
   SparseDev d = SPARSE_DEV(batch, Bp, d_visit_.p);
+  d.n_flow_rows = n_flow_rows();
   if (soft) { d.ev = soft->d_ev; d.ev_se = soft->stride_ex; d.ev_sv = soft->stride_var; d.ev_sc = soft->stride_cat; d.ev_idx = soft->d_idx; }
   SparseDev db = d;
   if (ne) {
     d_in_logp_.ensure(d_in_rec_.n);
     hipLaunchKernelGGL(sparse_gather_in_logp_kernel, dim3(ceil_div((int64_t)d_in_rec_.n, 256)), dim3(256), 0, stream,
-                       d_in_rec_.p, d_logp_.p, (int64_t)d_in_rec_.n, d_in_logp_.p);
+                       d_in_rec_.p, d_logp_.p, (int64_t)d_in_rec_.n, fc_.n_nodes(), d_in_logp_.p);
     db.in_logp = d_in_logp_.p;
   }
   db.order = d_bwd_order_.p;   // the layers without the input nodes whose rows other nodes write
@@ -1404,10 +1729,10 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
   }
   for (int l = n_layers_ - 1; l >= 0; --l) {
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
-    if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
 #define PCM_BWD_ARGS db, n0, d_head_mask, d_edge_part_.p, ne, d_alias_list_.p
-    if (bwd_layer_max_in_[l] <= kNarrowDegree) {
+    if (cnt == 0) {   // (every node of the layer takes its flow from a group's row)
+    } else if (bwd_layer_max_in_[l] <= kNarrowDegree) {
       if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
       else   // (the rows of partial edge sums beyond a quarter stay as cleared)
         PCM_LAYER_LAUNCH(sparse_backward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), PCM_BWD_ARGS);
@@ -1419,12 +1744,17 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
       PCM_LAYER_LAUNCH(sparse_backward_kernel, 2, 1, 8, dim3(cnt, ceil_div(Bp, 128)), PCM_BWD_ARGS);
     }
 #undef PCM_BWD_ARGS
+    launch_groups(l, 1, Bp, batch);   // the layer's sums have their flows: on to their children's rows
   }
   if (!accumulate) {
     check_launch("sparse_backward");
     flow_batch_ = last_batch_;
     return;
   }
+  launch_groups(-1, 2, Bp, batch);   // the groups' edge flows, into the same rows of partial sums
+  if (n_group_product_edges_)
+    hipLaunchKernelGGL(sparse_product_edge_kernel, dim3(ceil_div(n_group_product_edges_, 4), Bp / 64), dim3(256), 0, stream,
+                       d_grp_product_edges_.p, n_group_product_edges_, d_flows_.p, Bp, d_edge_part_.p, ne);
   if (ne)
     hipLaunchKernelGGL(sum_parts_kernel<false>, dim3(ceil_div(ne, 64)), dim3(256), 0, stream, d_edge_part_.p, n_parts, ne,
                        (const float*)nullptr, d_edge_aggr_.p);

@@ -116,6 +116,25 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<int4> d_fwd_rec_, d_bwd_rec_;   // per position of the forward / backward order: node and its ranges in one record
   DevBuf<int2> d_bwd_alias_;
   std::vector<int> layer_max_children_, bwd_layer_max_in_;   // per layer: most edges of a node going up / coming in
+  // dense groups (sparse_groups.hip.hpp): sum nodes of a layer that share one list of children
+  struct GroupLaunch { int layer, group0, count, gt, ct; int32_t pnode0, pslot0; int64_t pw0; };
+  std::vector<GroupLaunch> group_launches_;   // per (layer, shape), sorted by layer: ranges of groups
+  std::vector<GroupLaunch> group_stat_launches_;   // per shape: ranges of d_grp_order_ (layer and bases unused)
+  std::vector<int> fwd_layer0_;               // ranges of d_fwd_rec_ per layer: the nodes no group computes
+  int64_t n_layer_nodes_ = 0;                 // nodes whose values the layer kernels compute (the others: the groups')
+  int64_t n_group_slots_ = 0, n_groups_ = 0, n_group_elems_ = 0;   // children of all groups; groups; padded W entries
+  DevBuf<int32_t> d_grp_node_, d_grp_edge_, d_grp_own_, d_grp_elem_, d_grp_order_;
+  DevBuf<int4> d_grp_rec_, d_grp_rows_, d_grp_copies_;   // (a group's record is two int4)
+  DevBuf<float> d_grp_wf_, d_grp_wb_, d_grp_m_;
+  DevBuf<int2> d_grp_product_edges_;          // {edge, parent}: product edges into nodes a group's kernel writes
+  int n_group_product_edges_ = 0;
+  std::vector<int32_t> grp_pslot_h_;          // host: where a slot's entry sits in the padded per-child tables
+  std::vector<int32_t> grp_prime_h_;          // host copy: the prime of every slot
+  std::vector<char> grp_expanded_;            // per node: a product that the groups using it compute themselves
+  void refresh_group_w();
+  void build_groups(std::vector<int32_t>& group_of, std::vector<int32_t>& edge_slot);
+  void launch_groups(int layer, int what, int Bp, int batch);   // what: 0 forward, 1 backward (one layer), 2 edge flows (all layers)
+  int64_t n_flow_rows() const { return fc_.n_nodes() + n_group_slots_; }
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
   DevBuf<int32_t> d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;
   DevBuf<uint8_t> d_visit_;

@@ -579,6 +579,7 @@ def test_statistics_are_the_same_bits_on_every_run(gpu, oracle):
     data = torch.from_numpy(rng.integers(0, C, size=(B, V)).astype(np.uint8)).cuda()
     mask = torch.from_numpy(rng.dirichlet(np.ones(H), size=B).astype(np.float32)).cuda()
     layered = _compile(P, heads, V, C, H)
+    assert layered.size("dense_groups") == len(set(parent[1:].tolist()))    # every inner tree node's sums (the root's: the heads) run as blocks
     block = P.multihead_hclt_from_clt(parent, C, K, H)
     P.update_parameters(block, P.vectorize_parameters(layered))
     soft = P.hclt_from_clt(parent, C, K)
@@ -601,6 +602,147 @@ def test_statistics_are_the_same_bits_on_every_run(gpu, oracle):
             for a, b in zip(first, again):
                 assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
         assert all(np.isfinite(a).all() for a in first) and first[0].sum() > 0 and first[1].sum() > 0
+
+
+def _with_and_without_groups(P, heads, V, C):
+    """The circuit compiled twice: sums with one list of children as blocks on the matrix cores, and (the switch the
+    library reads when a circuit is created) every sum edge by edge on the layer kernels."""
+    import os
+    grouped = _compile(P, heads, V, C, len(heads))
+    os.environ["PCMI355_DENSE_GROUPS"] = "0"
+    try:
+        plain = _compile(P, heads, V, C, len(heads))
+    finally:
+        del os.environ["PCMI355_DENSE_GROUPS"]
+    assert plain.size("dense_groups") == 0 and plain.size("layer_nodes") == plain.num_nodes()
+    return grouped, plain
+
+
+def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
+    """Values, flows, statistics and updated parameters of a multi-head circuit whose dense groups run on the block
+    kernels, against the oracle and against the same circuit on the layer kernels alone."""
+    torch, P = gpu
+    from helpers import rel_err
+    import pcmi355._lib as L
+    rng = np.random.default_rng(seed)
+    H = len(heads)
+    grouped, plain = _with_and_without_groups(P, heads, V, C)
+    assert grouped.size("dense_groups") >= min_groups
+    assert grouped.size("layer_nodes") < grouped.num_nodes()
+    fc = O.bits_compile(O.summate(*heads), C, V)
+    n_real = fc.n_nodes - 1
+    assert grouped.num_nodes() == n_real
+    start = P.vectorize_parameters(grouped)
+    assert np.array_equal(start, P.vectorize_parameters(plain))
+    root_ids = (grouped.table("heads") - 1).astype(np.int32)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    mask = rng.random((B, H)).astype(np.float32) + 0.05
+    mask[::5, 0] = 0.0
+    d, hm = torch.from_numpy(data).cuda(), torch.from_numpy(mask).cuda()
+    mars_ref = O.forward(fc, data)
+    skip = (fc.edge_parent() == fc.n_nodes - 1).astype(np.uint8)
+    flows_ref, ea_ref = O.backward(fc, mars_ref, skip=skip, root_ids=root_ids, root_flow=np.ascontiguousarray(mask.T))
+    lf_ref = O.input_flows(fc, data, flows_ref)
+    order = fc.up_order()
+    order = order[fc.edge_parent()[order] != fc.n_nodes - 1]
+    got = []
+    for bpc in (grouped, plain):
+        per_head = P.loglikelihoods(bpc, d).cpu().numpy()
+        assert rel_err(per_head, mars_ref[root_ids].T).max() < LL_RTOL
+        ll = P.probs_flows_circuit(bpc, d, head_mask=hm).cpu().numpy()
+        mars, flows = bpc.get_node_values(B)
+        finite = np.isfinite(mars_ref[:n_real])
+        assert np.array_equal(np.isfinite(mars), finite)
+        assert np.abs(mars[finite] - mars_ref[:n_real][finite]).max() < LL_RTOL * np.abs(mars_ref[:n_real][finite]).max()
+        assert np.abs(flows - flows_ref[:n_real]).max() < FLOW_RTOL
+        ea, lf = bpc.get_aggregates()
+        assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
+        assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
+        L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.7))
+        got.append((ll, mars, flows, ea, lf, P.vectorize_parameters(bpc)))
+    for a, b in zip(*got):                                   # the two paths round differently, no more
+        fa, fb = np.isfinite(a), np.isfinite(b)
+        assert np.array_equal(fa, fb)
+        assert np.abs(a[fa] - b[fb]).max() <= 2e-4 * max(np.abs(b[fb]).max(), 1.0)
+    # a smaller batch afterwards finds the arrays of the larger one (rows of 64 examples, the last one partly filled)
+    small = d[: B // 3]
+    for bpc in (grouped, plain):
+        P.update_parameters(bpc, start)
+    a, b = (P.loglikelihoods(bpc, small).cpu().numpy() for bpc in (grouped, plain))
+    assert rel_err(a, mars_ref[root_ids][:, : B // 3].T).max() < LL_RTOL and rel_err(a, b).max() < LL_RTOL
+    return grouped, fc
+
+
+@pytest.mark.parametrize("V,K,C,H,B,max_children,seed", [(20, 8, 5, 9, 150, 5, 31), (9, 32, 4, 40, 64, 2, 32),
+                                                         (33, 12, 3, 6, 333, 3, 33)])
+def test_dense_groups_of_a_multihead_hclt(gpu, oracle, V, K, C, H, B, max_children, seed):
+    """An HCLT's K sums per tree node and the heads over the root's products are groups; products of up to three
+    children are taken apart by the groups above them, those of more stay nodes of a layer."""
+    from helpers import multihead_hclt
+    rng = np.random.default_rng(seed)
+    parent = np.full(V, -1, np.int32)
+    n_children = np.zeros(V, int)
+    for v in range(1, V):
+        free = [u for u in range(v) if n_children[u] < max_children]
+        parent[v] = free[int(rng.integers(0, len(free)))] if v > max_children + 1 else 0   # the root takes max_children + 1
+        n_children[parent[v]] += 1
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    inner = len(set(parent[1:].tolist()))                    # (the K sums of an inner tree node; the root's are the heads)
+    grouped, _ = _check_grouped_multihead(gpu, oracle, heads, V, C, B, seed, min_groups=inner)
+    assert grouped.size("dense_groups") == inner
+    if max_children <= 3:
+        # nothing but the inputs and the product of the root's children is left to the layer kernels going up
+        assert grouped.size("layer_nodes") == grouped.size("input_nodes") + K
+
+
+def test_dense_groups_after_pruning_and_growing(gpu, oracle):
+    """prune_pc takes edges out of some of a group's sums (their lists of children differ from then on) and
+    grow_heads_by_flows doubles sums and products: what is left of the groups, and the new ones, still compute what
+    the oracle does."""
+    torch, P = gpu
+    from helpers import multihead_hclt, from_oracle_dag, to_oracle_dag
+    rng = np.random.default_rng(41)
+    V, K, C, H, B = 8, 12, 4, 8, 200
+    parent = np.array([-1, 0, 0, 1, 1, 2, 5, 5], np.int32)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    pcs, _ = from_oracle_dag(heads)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    mask = rng.dirichlet(np.ones(H), size=B).astype(np.float32)
+    d, hm = torch.from_numpy(data).cuda(), torch.from_numpy(mask).cuda()
+    for threshold in (1e-4, 3e-4, 1e-3, 3e-3):               # the first that takes some edges, and not too many
+        pruned = P.prune_pc(pcs, d, hm, batch_size=100, prune_threshold=threshold)
+        if P.nodes.num_edges(pruned) < P.nodes.num_edges(pcs):
+            break
+    assert P.nodes.num_edges(pruned) < P.nodes.num_edges(pcs)
+    po, _ = to_oracle_dag(pruned)
+    _check_grouped_multihead(gpu, oracle, po, V, C, 90, 42, min_groups=1)
+    grown = P.grow_heads_by_flows(pcs, d, hm, batch_size=100, sigma=0.1, node_selection_args={"grow_frac": 0.5},
+                                  rng=np.random.default_rng(3))
+    go, _ = to_oracle_dag(grown)
+    assert len(go) > H
+    # (a split sum and its copy share their products, which then are nodes; an unsplit sum's are folded into its
+    # edges: the sums of one tree node fall into several sets of children, of which those with four sums are groups)
+    _check_grouped_multihead(gpu, oracle, go, V, C, 90, 43, min_groups=1)
+
+
+def test_dense_groups_beside_ordinary_edges(gpu, oracle):
+    """A group whose children other sums use too (their rows of flow are added to what those sums send), beside a
+    group whose products nothing else uses (taken apart, written by the group), under one root."""
+    O = oracle
+    from helpers import log_dirichlet
+    rng = np.random.default_rng(51)
+    C, G, J = 5, 6, 12
+    leaf = lambda v: O.input_node(v, log_dirichlet(rng, C))
+    p = [O.multiply(leaf(0), leaf(1)) for _ in range(J)]
+    q = [O.multiply(leaf(2), leaf(3)) for _ in range(J)]
+    s = [O.summate(*p, logps=log_dirichlet(rng, J)) for _ in range(G)]
+    t = O.summate(*p[:3], logps=log_dirichlet(rng, 3))
+    t2 = O.summate(*p[2:9], logps=log_dirichlet(rng, 7))
+    u = [O.summate(*q, logps=log_dirichlet(rng, J)) for _ in range(G)]
+    tops = [O.multiply(s[i], u[i]) for i in range(G)] + [O.multiply(t, u[0]), O.multiply(t2, u[3])]
+    heads = [O.summate(*tops, logps=log_dirichlet(rng, len(tops))) for _ in range(2)]
+    grouped, _ = _check_grouped_multihead(gpu, oracle, heads, 4, C, 130, 52, min_groups=2)
+    assert grouped.size("dense_groups") == 2
 
 
 def test_forest_of_patch_circuits_at_their_real_shape(gpu, oracle):
