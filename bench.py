@@ -19,7 +19,8 @@ sys.path.insert(0, os.path.join(ROOT, "lvd-pg_amd"))
 
 HBM_PEAK_GBS = 8000.0   # MI355X HBM3E, published
 # the layered engine's byte count is what its kernels ask the caches for, not what must cross the HBM interface
-REQUESTED_NOTE = ("bytes requested by the layer kernels: 8 per (node, example) + 24 per (edge, example); at this size most "
+REQUESTED_NOTE = ("bytes the circuit asks for edge by edge: 8 per (node, example) + 24 per (edge, example), a measure of the "
+                  "work; sums that run as dense groups read a child's row once per group, and at this size most requests "
                   "are served by L2 and the last-level cache, so frac is not a fraction of HBM traffic")
 # kernels the benchmark circuit runs (three children per node at most, K = 32: the lean set)
 PHASE_MASK = {"forward": 2, "backward": 4, "statistics": 8}   # pcm_set_timing: time that phase's kernel only

@@ -293,14 +293,24 @@ __global__ __launch_bounds__(256) void sparse_group_stats_kernel(GroupDev d, int
       if (c < Cp) E[c * kGroupPad + b] = x[q] > -INFINITY ? __expf(x[q] - mb) : 0.f;
     }
   }
-  for (int g = part; g < Gp; g += 4) {
-    float rv = 0.f;
-    if (g < r.G) {
-      const int64_t n = d.node[r.pnode0 + g];
-      const float f = d.flows[n * d.Bp + b0 + b], v = d.mars[n * d.Bp + b0 + b];
-      if (f > 0.f && v > -INFINITY) rv = f * __expf(mb - v);
+  for (int gb = part; gb < Gp; gb += 32) {   // (eight sums' rows requested before the first is used, as above)
+    float f[8], v[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int g = gb + 4 * q;
+      f[q] = 0.f;
+      v[q] = 0.f;
+      if (g < r.G) {
+        const int64_t n = guni(d.node[r.pnode0 + g]);
+        f[q] = d.flows[n * d.Bp + b0 + b];
+        v[q] = d.mars[n * d.Bp + b0 + b];
+      }
     }
-    R[g * kGroupPad + b] = rv;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int g = gb + 4 * q;
+      if (g < Gp) R[g * kGroupPad + b] = (f[q] > 0.f && v[q] > -INFINITY) ? f[q] * __expf(mb - v[q]) : 0.f;
+    }
   }
   __syncthreads();
   const int lane = t & 63, wave = t >> 6;
