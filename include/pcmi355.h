@@ -117,6 +117,20 @@ int pcm_set_missing_category(pcm_circuit* c, int32_t on);
  */
 int pcm_set_soft_reg(pcm_circuit* c, float soft_reg, int32_t soft_reg_width, int32_t as_written);
 
+/*
+ * `fscale` of mini_batch_em_beta (VariationalJuice.jl/src-jl/learning/em.jl:289-296, scaled_probs_flows_circuit
+ * flow.jl:367-373): from this call on, pcm_flows / pcm_flows_soft / pcm_em_step hand every sum node's flow to its
+ * edges in shares proportional to (posterior share)^(1 / fscale) -- scale_flows_kernel flow.jl:120-175 computes the
+ * sum of those per node, reg_layer_down_kernel :204-300 the edge flows -- instead of the posterior shares themselves;
+ * likelihoods, per-example normalised flows and every other query are not touched.  fscale = 1 (the default) is the
+ * ordinary pass.  Any handle but a forest or a circuit with a missing-value category (PCM_ERR_UNSUPPORTED); HCLT
+ * handles run these passes on their layered form (kernels per layer, dense groups on the matrix cores), with the
+ * statistics and the flow memory held there until pcm_em_update.  Per-example weights / head masks scale the
+ * flows as always (the reference's tempered pass reads its `weights` argument only at the input nodes).
+ * PCM_ERR_ARG unless fscale is positive and finite.
+ */
+int pcm_set_flow_scale(pcm_circuit* c, float fscale);
+
 /* Head log-parameters of a multi-head HCLT or a forest, [num_trees][num_heads][num_hidden_cats] on the host:
  * the `params` of the head sum nodes (src-jl/multi_head_pc/bit_circuit.jl:14-56 keeps them in the heads'
  * edges), row h of a tree being the head that row h of its head mask seeds. */

@@ -159,6 +159,15 @@ int pcm_set_soft_reg(pcm_circuit* c, float soft_reg, int32_t soft_reg_width, int
   return guarded([&] { need_hclt(c)->set_soft_reg(soft_reg, soft_reg_width, as_written != 0); });
 }
 
+int pcm_set_flow_scale(pcm_circuit* c, float fscale) {
+  return guarded([&] {
+    pcm_circuit* h = need(c);
+    if (!(fscale > 0.f) || !std::isfinite(fscale)) pcm::fail(PCM_ERR_ARG, "fscale must be positive and finite, got %g", (double)fscale);
+    if (auto* hc = dynamic_cast<pcm::HcltCircuit*>(h)) hc->check_flow_scale(fscale);
+    h->flow_scale = fscale;
+  });
+}
+
 int pcm_hclt_set_params(pcm_circuit* c, const float* theta, const float* leaf) {
   return guarded([&] { need_hclt(c)->set_block_params(theta, leaf); });
 }

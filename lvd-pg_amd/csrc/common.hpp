@@ -135,6 +135,9 @@ void chow_liu_tree(const float* mi, int num_vars, int32_t* parent_out);
 // The opaque handle of the C ABI.
 struct pcm_circuit {
   hipStream_t stream = nullptr;
+  // fscale of mini_batch_em_beta (src-jl/learning/em.jl:293, flow.jl:120-370): flows that feed the accumulators hand
+  // a sum node's flow down in shares proportional to (posterior share)^(1 / flow_scale); 1: the ordinary flows
+  float flow_scale = 1.f;
   virtual ~pcm_circuit() {}
   virtual int64_t size(int what) const = 0;
   virtual void index_table(int which, int64_t* out, int64_t n) const = 0;

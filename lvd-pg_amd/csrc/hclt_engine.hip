@@ -1528,7 +1528,7 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
   no_forest("soft evidence");
   no_missing("soft evidence");
   // (per-example weights on soft evidence -- a mask for a single-head circuit -- go to the layered engine)
-  if (soft_block_ok() && !(H_ == 0 && d_head_mask)) {
+  if (soft_block_ok() && !(H_ == 0 && d_head_mask) && flow_scale == 1.f) {   // (tempered flows: the layered engine)
     if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
     if (flows_in_general_ && rate != 0.f) fail(PCM_ERR_STATE, "flow memory cannot carry over from the layered engine");
     const HcltDev d = soft_stage(s);
@@ -1577,6 +1577,7 @@ void HcltCircuit::flows_soft(const SoftRef& s, float rate, const float* d_head_m
   }
   if (have_flows_ && !flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from categorical batches to soft-evidence batches");
+  general()->flow_scale = flow_scale;
   general()->flows_soft(s, rate, d_head_mask, d_ll);
   have_flows_ = true;
   flows_in_general_ = true;
@@ -1588,10 +1589,24 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   const float* weights = H_ == 0 ? d_head_mask : nullptr;
   if (H_ > 0 && !d_head_mask) fail(PCM_ERR_ARG, "a multi-head circuit needs a head_mask for its flows");
   if (!d_ll) fail(PCM_ERR_ARG, "output pointer is null");
+  if (flow_scale != 1.f && (block_ || wide_)) {
+    // tempered flows (fscale of mini_batch_em_beta) are the layered engine's: the block kernels keep S, not the sum of
+    // the shares to the power 1 / fscale
+    if (soft_reg_ > 0.f) fail(PCM_ERR_UNSUPPORTED, "tempered flows with soft_reg in the kernels: give the smoothed batch as soft evidence");
+    if (have_flows_ && !flows_in_general_ && rate != 0.f)
+      fail(PCM_ERR_STATE, "flow memory cannot carry over from ordinary flows on the block kernels to tempered flows");
+    SparseCircuit* g = general();
+    g->flow_scale = flow_scale;
+    g->flows(b, rate, d_head_mask, d_ll);
+    have_flows_ = true;
+    flows_in_general_ = true;
+    return;
+  }
   if (flows_in_general_ && rate != 0.f && (block_ || wide_))
     fail(PCM_ERR_STATE, "flow memory cannot carry over from soft-evidence batches to categorical batches");
   flows_in_general_ = false;
   if (!block_ && !wide_) {
+    general()->flow_scale = flow_scale;
     general()->flows(b, rate, weights, d_ll);
     have_flows_ = true;
     return;

@@ -201,6 +201,12 @@ class HcltCircuit : public pcm_circuit {
   // soft_reg > 0: categorical batches are smoothed as reg_likelihood.jl:4-14 has it; as_written: leaf statistics as
   // reg_flow.jl:12-17 computes them (log-probabilities in the shares) instead of the derivative of the smoothed value
   void set_soft_reg(float soft_reg, int width, bool as_written);
+  // tempered flows run on the circuit's layered form: not for forests and circuits with a missing-value category
+  void check_flow_scale(float fscale) {
+    if (fscale == 1.f) return;
+    no_forest("tempered flows");
+    no_missing("tempered flows");
+  }
   void get_block_params(float* theta, float* leaf);
   void get_block_flows(float* edge_aggr, float* leaf_flow);
 

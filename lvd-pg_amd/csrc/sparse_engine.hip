@@ -215,6 +215,8 @@ struct SparseDev {
   int32_t B, Bp, C;
   int64_t n_nodes;
   int64_t n_flow_rows;       // node rows of the flow array + the rows dense groups hand their children
+  const float* norm;         // tempered flows: [n_nodes + 1][Bp], log of a sum node's sum over its edges of share^(1 / fscale); 0 elsewhere
+  float inv_f;               // ... and 1 / fscale
 };
 
 // ProbabilisticCircuits.jl logsumexp(x, y) as used by src/queries/likelihood.jl:101-102.
@@ -474,7 +476,7 @@ struct EdgeTotals {
   }
 };
 
-template <int U, int EX, bool kBuf>
+template <int U, int EX, bool kBuf, bool kTempered = false>
 __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf>& mars, const Rows<kBuf>& flows, int c0,
                                              const int (&bb)[EX], const unsigned (&alive)[EX], float (&acc)[EX],
                                              float* __restrict__ edge_part) {
@@ -495,6 +497,8 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
     for (int x = 0; x < EX; ++x) {
       fl[u][x] = keep_bits(flows.at(p, bb[x]), alive[x]);   // a lane past the padded batch repeats its last example
       ex[u][x] = mars.at(pr, bb[x]) + lp + mars.at(s, bb[x]) - mars.at(mrow, bb[x]);
+      // tempered (src-jl/learning/flow.jl:259-262): the share to the power 1 / fscale over the node's sum of those
+      if constexpr (kTempered) ex[u][x] = ex[u][x] * d.inv_f - d.norm[(size_t)mrow * d.Bp + bb[x]];
     }
   }
   float part[U];
@@ -535,7 +539,7 @@ __device__ __forceinline__ void backward_run(const SparseDev& d, const Rows<kBuf
 // edge).  Each edge's flow is summed over the batch where the node is the edge's prime
 // (:73-81): over the thread's examples, then over the wave; the wave's sum goes to row blockIdx.y of
 // edge_part ([gridDim.y][n_edges]), whose rows a later kernel adds up in order.
-template <int EX, int kLayerWaves, int kMaxRun, bool kBuf>
+template <int EX, int kLayerWaves, int kMaxRun, bool kBuf, bool kTempered = false>
 __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(SparseDev d, int n0,
                                                                            const float* __restrict__ seed,
                                                                            float* __restrict__ edge_part_all, int64_t n_edges,
@@ -568,13 +572,13 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
   const Rows<kBuf> mars(d.mars, d.n_nodes + 1, d.Bp), flows(d.flows, d.n_flow_rows, d.Bp);
   int c0 = my0;
   if constexpr (kMaxRun >= 32)
-    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
+    for (; c0 + 32 <= my1; c0 += 32) backward_run<32, EX, kBuf, kTempered>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if constexpr (kMaxRun >= 16)
-    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
+    for (; c0 + 16 <= my1; c0 += 16) backward_run<16, EX, kBuf, kTempered>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if constexpr (kMaxRun == 8)
-    for (; c0 + 8 <= my1; c0 += 8) backward_run<8, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
-  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
-  for (; c0 < my1; ++c0) backward_run<1, EX, kBuf>(d, mars, flows, c0, bb, alive, acc, edge_part);
+    for (; c0 + 8 <= my1; c0 += 8) backward_run<8, EX, kBuf, kTempered>(d, mars, flows, c0, bb, alive, acc, edge_part);
+  for (; c0 + 4 <= my1; c0 += 4) backward_run<4, EX, kBuf, kTempered>(d, mars, flows, c0, bb, alive, acc, edge_part);
+  for (; c0 < my1; ++c0) backward_run<1, EX, kBuf, kTempered>(d, mars, flows, c0, bb, alive, acc, edge_part);
   if (i1 - i0 > per) {   // more than one share is in use (uniform over the workgroup)
 #pragma unroll
     for (int x = 0; x < EX; ++x) xa[wave][x][lane] = acc[x];
@@ -1052,6 +1056,30 @@ __global__ __launch_bounds__(64 * kMixGroups) void sparse_head_mixture_kernel(co
   out[b] = M + logf(S) - logf(T);
 }
 
+// Tempered flows, scale_flows_kernel of src-jl/learning/flow.jl:120-175: per sum node and example the logarithm of the
+// sum over the node's edges of exp((value of the edge's children + log-parameter - value of the node) / fscale); 0 for
+// every other node and for the row of zeros behind the last node.  thread = (node, example)
+__global__ __launch_bounds__(256) void sparse_tempered_norm_kernel(SparseDev d, float* __restrict__ norm) {
+  const int64_t n = blockIdx.x;
+  const int b = blockIdx.y * 256 + threadIdx.x;
+  if (b >= d.Bp) return;
+  float out = 0.f;
+  if (n < d.n_nodes && d.type[n] == kSum) {
+    const float v = d.mars[n * d.Bp + b];
+    float mx = -INFINITY, s = 0.f;
+    for (int e = d.node_e0[n]; e < d.node_e1[n]; ++e) {
+      float t = d.mars[(int64_t)d.e_prime[e] * d.Bp + b] + d.logp[e];
+      if (d.e_sub[e] >= 0) t += d.mars[(int64_t)d.e_sub[e] * d.Bp + b];
+      t = (t - v) * d.inv_f;
+      if (!(t > -INFINITY)) continue;   // (also an example of probability zero: -inf - -inf)
+      if (t > mx) { s = s * __expf(mx - t) + 1.f; mx = t; }
+      else s += __expf(t - mx);
+    }
+    if (s > 0.f) out = mx + __logf(s);
+  }
+  norm[n * d.Bp + b] = out;
+}
+
 // Edge flows of product edges whose child takes its flow from a group's kernel instead of a layer's: the edge's flow
 // is its parent's, summed over each block of 64 examples into the block's row of partial sums.  One wave per
 // (edge, block).
@@ -1245,21 +1273,24 @@ void SparseCircuit::build_groups(std::vector<int32_t>& group_of, std::vector<int
   g.node = d_grp_node_.p; g.edge = d_grp_edge_.p;   g.rows = d_grp_rows_.p; g.own = d_grp_own_.p;                    \
   g.copies = d_grp_copies_.p; g.order = d_grp_order_.p; g.wf = d_grp_wf_.p; g.wb = d_grp_wb_.p; g.m = d_grp_m_.p;       \
   g.logp = d_logp_.p; g.mars = d_mars_.p; g.flows = d_flows_.p; g.edge_part = d_edge_part_.p;                        \
-  g.n_nodes = fc_.n_nodes(); g.n_edges = fc_.n_edges(); g.B = batch_; g.Bp = bp_
+  g.n_nodes = fc_.n_nodes(); g.n_edges = fc_.n_edges(); g.B = batch_; g.Bp = bp_;                                   \
+  g.inv_f = 1.f; g.norm = d_mars_.p; g.norm_row = fc_.n_nodes()   /* (not tempered: the row of zeros for every sum) */
 
 // exp of the groups' log-parameters, before a forward pass
-void SparseCircuit::refresh_group_w() {
+void SparseCircuit::refresh_group_w(float inv_f) {
   if (n_group_elems_ == 0) return;
   PCM_GROUP_DEV(g, 0, 0);
+  g.inv_f = inv_f;
   hipLaunchKernelGGL(sparse_group_w_kernel, dim3((unsigned)ceil_div(n_group_elems_, 256)), dim3(256), 0, stream, g, d_grp_elem_.p,
                      n_group_elems_);
 }
 
 // the group kernels of one layer: what = 0 values going up, 1 the children's rows going down; what = 2: the edge
 // flows of every group, after the backward pass
-void SparseCircuit::launch_groups(int layer, int what, int Bp, int batch) {
+void SparseCircuit::launch_groups(int layer, int what, int Bp, int batch, bool tempered) {
   if (group_launches_.empty()) return;
   PCM_GROUP_DEV(g, batch, Bp);
+  if (tempered) { g.inv_f = 1.f / flow_scale; g.norm = d_norm_.p; g.norm_row = -1; }
   for (const GroupLaunch& L : what == 2 ? group_stat_launches_ : group_launches_) {
     if (what != 2 && L.layer != layer) continue;
     const size_t lds = what == 2 ? group_lds_floats(L.gt * 16, L.ct * 16) * sizeof(float) : 0;
@@ -1580,6 +1611,7 @@ static SparseDev make_dev(const uint8_t* type, const int32_t* order, const int32
   d.in_var = in_var; d.in_ptr = in_ptr; d.in_edge = in_edge; d.in_rec = in_rec; d.in_logp = nullptr; d.in_off = in_off;
   d.ev = nullptr; d.ev_se = d.ev_sv = d.ev_sc = 0; d.ev_idx = nullptr; d.logp = logp; d.leaf = leaf;
   d.xb = xb; d.mars = mars; d.flows = flows; d.B = B; d.Bp = Bp; d.C = C; d.n_nodes = n_nodes; d.n_flow_rows = n_nodes;
+  d.norm = nullptr; d.inv_f = 1.f;
   return d;
 }
 
@@ -1719,6 +1751,15 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     db.in_logp = d_in_logp_.p;
   }
   db.order = d_bwd_order_.p;   // the layers without the input nodes whose rows other nodes write
+  const bool tempered = accumulate && flow_scale != 1.f;
+  if (tempered) {
+    d_norm_.ensure((size_t)(fc_.n_nodes() + 1) * Bp);
+    db.inv_f = 1.f / flow_scale;
+    db.norm = d_norm_.p;
+    hipLaunchKernelGGL(sparse_tempered_norm_kernel, dim3((unsigned)(fc_.n_nodes() + 1), ceil_div(Bp, 256)), dim3(256), 0, stream, db,
+                       d_norm_.p);
+    refresh_group_w(db.inv_f);   // W^(1 / fscale) for this pass; the next forward pass puts W back
+  }
   // edge flows summed over the batch: one row of partial sums per 64 examples, cleared first (an edge that
   // no wave visits must read as zero), added into the accumulators in row order after the walk
   const int n_parts = Bp / 64;
@@ -1732,6 +1773,8 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
 #define PCM_BWD_ARGS db, n0, d_head_mask, d_edge_part_.p, ne, d_alias_list_.p
     if (cnt == 0) {   // (every node of the layer takes its flow from a group's row)
+    } else if (tempered) {
+      hipLaunchKernelGGL((sparse_backward_kernel<1, 1, 16, false, true>), dim3(cnt, Bp / 64), dim3(64), 0, stream, PCM_BWD_ARGS);
     } else if (bwd_layer_max_in_[l] <= kNarrowDegree) {
       if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_backward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), PCM_BWD_ARGS);
       else   // (the rows of partial edge sums beyond a quarter stay as cleared)
@@ -1744,14 +1787,15 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
       PCM_LAYER_LAUNCH(sparse_backward_kernel, 2, 1, 8, dim3(cnt, ceil_div(Bp, 128)), PCM_BWD_ARGS);
     }
 #undef PCM_BWD_ARGS
-    launch_groups(l, 1, Bp, batch);   // the layer's sums have their flows: on to their children's rows
+    launch_groups(l, 1, Bp, batch, tempered);   // the layer's sums have their flows: on to their children's rows
   }
   if (!accumulate) {
     check_launch("sparse_backward");
     flow_batch_ = last_batch_;
     return;
   }
-  launch_groups(-1, 2, Bp, batch);   // the groups' edge flows, into the same rows of partial sums
+  launch_groups(-1, 2, Bp, batch, tempered);   // the groups' edge flows, into the same rows of partial sums
+  if (tempered) refresh_group_w();   // (W itself again, for whatever reads the tables next)
   if (n_group_product_edges_)
     hipLaunchKernelGGL(sparse_product_edge_kernel, dim3(ceil_div(n_group_product_edges_, 4), Bp / 64), dim3(256), 0, stream,
                        d_grp_product_edges_.p, n_group_product_edges_, d_flows_.p, Bp, d_edge_part_.p, ne);

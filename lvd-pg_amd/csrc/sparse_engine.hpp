@@ -126,14 +126,15 @@ class SparseCircuit : public pcm_circuit {
   DevBuf<int32_t> d_grp_node_, d_grp_edge_, d_grp_own_, d_grp_elem_, d_grp_order_;
   DevBuf<int4> d_grp_rec_, d_grp_rows_, d_grp_copies_;   // (a group's record is two int4)
   DevBuf<float> d_grp_wf_, d_grp_wb_, d_grp_m_;
+  DevBuf<float> d_norm_;                      // tempered flows: [n_nodes + 1][Bp], see sparse_tempered_norm_kernel
   DevBuf<int2> d_grp_product_edges_;          // {edge, parent}: product edges into nodes a group's kernel writes
   int n_group_product_edges_ = 0;
   std::vector<int32_t> grp_pslot_h_;          // host: where a slot's entry sits in the padded per-child tables
   std::vector<int32_t> grp_prime_h_;          // host copy: the prime of every slot
   std::vector<char> grp_expanded_;            // per node: a product that the groups using it compute themselves
-  void refresh_group_w();
+  void refresh_group_w(float inv_f = 1.f);    // W = exp(log-parameter * inv_f): 1 / fscale for a tempered backward pass
   void build_groups(std::vector<int32_t>& group_of, std::vector<int32_t>& edge_slot);
-  void launch_groups(int layer, int what, int Bp, int batch);   // what: 0 forward, 1 backward (one layer), 2 edge flows (all layers)
+  void launch_groups(int layer, int what, int Bp, int batch, bool tempered = false);   // what: 0 forward, 1 backward (one layer), 2 edge flows (all layers)
   int64_t n_flow_rows() const { return fc_.n_nodes() + n_group_slots_; }
   DevBuf<int32_t> d_head_nodes_;   // node ids of the heads
   DevBuf<int32_t> d_group_ptr_, d_param2edge_, d_var_ptr_, d_var_nodes_;

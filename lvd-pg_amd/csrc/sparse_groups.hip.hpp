@@ -9,6 +9,7 @@
 //   S[g] = sum_c W[g,c] E[c],  value of sum g = m + log S[g]                       (forward; W = exp(log-parameters))
 //   R[g] = flow of sum g / S[g],  flow into child c = E[c] * sum_g W[g,c] R[g]      (backward)
 //   edge flow (g, c) summed over the batch = W[g,c] * sum_b R[b,g] E[b,c]
+// (tempered flows, fscale != 1: going down W, E and the shares of R to the power 1 / fscale, R over the tempered sum)
 // with the three contractions on v_mfma_f32_16x16x4_f32: C exponentials per example instead of G * C.  The two that
 // sit in the chain of layers are one wave per (group, 16 examples) with everything in registers; the edge flows, which
 // nothing waits for, are one launch per shape of group after the pass.
@@ -60,6 +61,11 @@ struct GroupDev {
   float* edge_part;       // [Bp / 64][n_edges]
   int64_t n_nodes, n_edges;
   int32_t B, Bp;
+  // tempered flows (fscale of mini_batch_em_beta): shares to the power inv_f = 1 / fscale, normalised again by the
+  // sums' rows of `norm` (row norm_row for every sum if it is >= 0: the row of zeros of a pass that is not tempered)
+  float inv_f;
+  const float* norm;
+  int64_t norm_row;
 };
 
 // where the kernels of one launch find their groups' entries: group = group0 + block, entries at base + block * stride
@@ -89,7 +95,7 @@ __global__ __launch_bounds__(256) void sparse_group_w_kernel(GroupDev d, const i
   const int64_t local = i - r.pw0;
   const int g = (int)(local / (16 * r.ct)), c = (int)(local % (16 * r.ct));
   const int e = d.edge[i];
-  const float w = e >= 0 ? __expf(d.logp[e]) : 0.f;
+  const float w = e >= 0 ? __expf(d.logp[e] * d.inv_f) : 0.f;
   const_cast<float*>(d.wf)[r.pw0 + group_wf_index(g, c, r.ct)] = w;
   const_cast<float*>(d.wb)[r.pw0 + group_wb_index(g, c, r.gt)] = w;
 }
@@ -219,7 +225,7 @@ __global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, G
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float xv = group_x(d, rw[s][i], col);
-      e[s][i] = xv > -INFINITY ? __expf(xv - mb) : 0.f;
+      e[s][i] = xv > -INFINITY ? __expf((xv - mb) * d.inv_f) : 0.f;
     }
   };
   if constexpr (kPre) {
@@ -231,7 +237,8 @@ __global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, G
   for (int k = 0; k < NG; ++k) {   // R = F / S = F * exp(m - value): no flow stays no flow where the value is -inf
     const int64_t n = nd[k] < 0 ? 0 : nd[k];
     const float f = d.flows[n * d.Bp + col], v = d.mars[n * d.Bp + col];
-    rv[k] = (nd[k] >= 0 && f > 0.f && v > -INFINITY) ? f * __expf(mb - v) : 0.f;
+    const float nv = d.norm[(d.norm_row >= 0 ? d.norm_row : n) * d.Bp + col];
+    rv[k] = (nd[k] >= 0 && f > 0.f && v > -INFINITY) ? f * __expf((mb - v) * d.inv_f - nv) : 0.f;
   }
   if constexpr (kPre) {
 #pragma unroll
@@ -290,26 +297,28 @@ __global__ __launch_bounds__(256) void sparse_group_stats_kernel(GroupDev d, int
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int c = cb + 4 * q;
-      if (c < Cp) E[c * kGroupPad + b] = x[q] > -INFINITY ? __expf(x[q] - mb) : 0.f;
+      if (c < Cp) E[c * kGroupPad + b] = x[q] > -INFINITY ? __expf((x[q] - mb) * d.inv_f) : 0.f;
     }
   }
   for (int gb = part; gb < Gp; gb += 32) {   // (eight sums' rows requested before the first is used, as above)
-    float f[8], v[8];
+    float f[8], v[8], nv[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int g = gb + 4 * q;
       f[q] = 0.f;
       v[q] = 0.f;
+      nv[q] = 0.f;
       if (g < r.G) {
         const int64_t n = guni(d.node[r.pnode0 + g]);
         f[q] = d.flows[n * d.Bp + b0 + b];
         v[q] = d.mars[n * d.Bp + b0 + b];
+        nv[q] = d.norm[(d.norm_row >= 0 ? d.norm_row : n) * d.Bp + b0 + b];
       }
     }
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int g = gb + 4 * q;
-      if (g < Gp) R[g * kGroupPad + b] = (f[q] > 0.f && v[q] > -INFINITY) ? f[q] * __expf(mb - v[q]) : 0.f;
+      if (g < Gp) R[g * kGroupPad + b] = (f[q] > 0.f && v[q] > -INFINITY) ? f[q] * __expf((mb - v[q]) * d.inv_f - nv[q]) : 0.f;
     }
   }
   __syncthreads();

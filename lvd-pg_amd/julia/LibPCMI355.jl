@@ -22,6 +22,8 @@ pcm_set_missing_category(c, on) =
     ccall((:pcm_set_missing_category, libpcmi355), Cint, (Ptr{Cvoid}, Int32), c, on)
 pcm_set_soft_reg(c, soft_reg, soft_reg_width, as_written) =
     ccall((:pcm_set_soft_reg, libpcmi355), Cint, (Ptr{Cvoid}, Float32, Int32, Int32), c, soft_reg, soft_reg_width, as_written)
+pcm_set_flow_scale(c, fscale) =
+    ccall((:pcm_set_flow_scale, libpcmi355), Cint, (Ptr{Cvoid}, Float32), c, fscale)
 pcm_hclt_set_heads(c, heads) =
     ccall((:pcm_hclt_set_heads, libpcmi355), Cint, (Ptr{Cvoid}, Ptr{Float32}), c, heads)
 pcm_hclt_get_heads(c, heads) =

@@ -17,7 +17,7 @@ using .LibPCMI355
 using Random
 
 export DeviceArray, to_device, to_host, Circuit, hclt, hclt_from_clt, compile_circuit, num_parameters,
-       loglikelihoods, loglikelihood, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em_for_multihead_pc,
+       loglikelihoods, loglikelihood, probs_flows_circuit, mini_batch_em_with_reg, mini_batch_em_beta, mini_batch_em_for_multihead_pc,
        vectorize_parameters, update_parameters, kld, kld_backward, gumbel_sample, gumbel_sample_backward,
        per_sample_normalized_flows, normalize_params, pairwise_MI, learn_chow_liu_tree
 
@@ -224,15 +224,17 @@ end
 
 "`mini_batch_em_with_reg(bpc, data, num_epochs; batch_size, pseudocount, soft_reg, soft_reg_width, ent_reg,
 param_inertia, param_inertia_end, flow_memory, shuffle, verbose)` (src/regularization/reg_em.jl:208-336): the mean
-log-likelihood of every epoch.  `soft_reg` > 0 and `ent_reg` > 0 are refused here (the Python host builds the
-smoothed evidence for the former; the reference has the latter commented out, reg_em.jl:294-296)."
+log-likelihood of every epoch.  `soft_reg` > 0 is set on the handle for the length of the loop (`pcm_set_soft_reg`:
+HCLT handles on the block kernels; `soft_flow_as_written` picks the leaf statistics of reg_flow.jl:12-17 as they
+stand); `ent_reg` > 0 is refused (the reference has it commented out, reg_em.jl:294-296)."
 function mini_batch_em_with_reg(c::Circuit, data, num_epochs::Integer; batch_size::Integer, pseudocount,
                                 soft_reg = 0.0, soft_reg_width = 1, ent_reg = 0.0,
                                 param_inertia, param_inertia_end = param_inertia, flow_memory = 0,
-                                shuffle = :each_epoch, verbose = true, rng = Random.default_rng())
+                                shuffle = :each_epoch, verbose = true, rng = Random.default_rng(),
+                                soft_flow_as_written::Bool = true)
     @assert pseudocount >= 0
-    soft_reg == 0 || throw(ArgumentError("soft_reg > 0: build the evidence with soft_reg_evidence and call the soft entry points"))
     ent_reg == 0 || throw(ArgumentError("ent_reg is not part of this path"))
+    soft_reg == 0 || check(LibPCMI355.pcm_set_soft_reg(c.h, Float32(soft_reg), Int32(soft_reg_width), Int32(soft_flow_as_written)))
     n = size(data, 1)
     @assert batch_size <= n
     num_batches = n ÷ batch_size                                            # reg_em.jl:216
@@ -260,6 +262,75 @@ function mini_batch_em_with_reg(c::Circuit, data, num_epochs::Integer; batch_siz
         verbose && println("epoch ", epoch, ": train LL ", log_likelihoods[end])
         inertia += Float32(delta)                                           # reg_em.jl:307
     end
+    soft_reg == 0 || check(LibPCMI355.pcm_set_soft_reg(c.h, 0f0, Int32(1), Int32(0)))
+    log_likelihoods
+end
+
+"`mini_batch_em_beta(bpc, data, num_epochs; batch_size, pseudocount, soft_reg, soft_reg_width, param_inertia,
+param_inertia_end, flow_memory, flow_memory_end, shuffle, update_interval, fscale, verbose)`
+(VariationalJuice.jl/src-jl/learning/em.jl:289-409): statistics collect over `update_interval` batches -- cleared at the
+start of an epoch, cleared or decayed by the flow memory at a batch with batch_id % update_interval == 1, every batch
+adds its flows, the parameters move after a batch with batch_id % update_interval == 0 -- with schedules for the
+inertia and the flow memory.  `fscale` other than 1: the flows of the tempered posterior (`pcm_set_flow_scale`)."
+function mini_batch_em_beta(c::Circuit, data, num_epochs::Integer; batch_size::Integer, pseudocount,
+                            soft_reg = 0.0, soft_reg_width = 1, param_inertia, param_inertia_end = param_inertia,
+                            flow_memory = 0, flow_memory_end = flow_memory, shuffle = :each_epoch,
+                            update_interval::Integer = 1, fscale = 1.0, verbose = true, rng = Random.default_rng(),
+                            soft_flow_as_written::Bool = true)
+    @assert pseudocount >= 0
+    @assert 0 <= param_inertia <= 1
+    @assert param_inertia <= param_inertia_end <= 1
+    @assert 0 <= flow_memory <= flow_memory_end                            # em.jl:299-303
+    @assert update_interval >= 1
+    n = size(data, 1)
+    @assert batch_size <= n
+    num_batches = n ÷ batch_size
+    soft_reg == 0 || check(LibPCMI355.pcm_set_soft_reg(c.h, Float32(soft_reg), Int32(soft_reg_width), Int32(soft_flow_as_written)))
+    fscale == 1 || check(LibPCMI355.pcm_set_flow_scale(c.h, Float32(fscale)))
+    ids_host = Vector{Int32}(undef, n)
+    ids_host .= Int32.(0:n-1)
+    shuffle == :once && shuffle!(rng, ids_host)
+    ids = to_device(ids_host)
+    lls = DeviceArray{Float32}(batch_size)
+    log_likelihoods = Float32[]
+    delta = (param_inertia_end - param_inertia) / num_epochs
+    delta_memory = (flow_memory_end - flow_memory) / num_epochs
+    inertia = Float32(param_inertia)
+    memory = Float64(flow_memory)
+    for epoch in 1:num_epochs
+        if shuffle == :each_epoch
+            shuffle!(rng, ids_host)
+            ids = to_device(ids_host)
+        end
+        total = 0.0
+        cleared = true                                                      # em.jl:344-345
+        for batch_id in 1:num_batches
+            if shuffle == :each_batch
+                shuffle!(rng, ids_host)
+                ids = to_device(ids_host)
+            end
+            rate = 1f0
+            if batch_id % update_interval == 1                              # em.jl:354-363
+                rate = memory == 0 ? 0f0 : max(0f0, 1f0 - Float32((batch_size + pseudocount) / memory))
+            end
+            if cleared
+                rate = 0f0
+                cleared = false
+            end
+            check(LibPCMI355.pcm_flows(c.h, device_pointer(data), 1, n, device_pointer(ids, (batch_id - 1) * batch_size),
+                                       batch_size, rate, device_pointer(nothing), device_pointer(lls)))
+            total += sum(to_host(lls))
+            if batch_id % update_interval == 0                              # em.jl:373-379
+                check(LibPCMI355.pcm_em_update(c.h, Float32(pseudocount), inertia))
+            end
+        end
+        push!(log_likelihoods, Float32(total / (num_batches * batch_size)))
+        verbose && println("epoch ", epoch, ": train LL ", log_likelihoods[end])
+        inertia += Float32(delta)
+        memory += delta_memory
+    end
+    soft_reg == 0 || check(LibPCMI355.pcm_set_soft_reg(c.h, 0f0, Int32(1), Int32(0)))
+    fscale == 1 || check(LibPCMI355.pcm_set_flow_scale(c.h, 1f0))
     log_likelihoods
 end
 

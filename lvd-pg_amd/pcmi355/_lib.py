@@ -30,6 +30,7 @@ _SIGS = {
     "pcm_hclt_create_forest": [vp, c_i32, c_i32, c_i32, c_i32, ctypes.POINTER(H)],
     "pcm_set_missing_category": [H, c_i32],
     "pcm_set_soft_reg": [H, c_f32, c_i32, c_i32],
+    "pcm_set_flow_scale": [H, c_f32],
     "pcm_hclt_set_heads": [H, vp],
     "pcm_hclt_get_heads": [H, vp],
     "pcm_circuit_create": [c_i32, vp, vp, vp, vp, vp, vp, c_i32, c_i32, c_i32, ctypes.POINTER(H)],

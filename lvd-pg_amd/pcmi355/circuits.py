@@ -38,6 +38,11 @@ class BitsCircuit:
             check(-1)
         return int(r)
 
+    def set_flow_scale(self, fscale):
+        """`fscale` of `mini_batch_em_beta` (src-jl/learning/em.jl:293, flow.jl:120-373): flows that feed the statistics
+        hand a sum node's flow down in shares proportional to (posterior share)^(1 / fscale).  1 switches it off."""
+        check(lib.pcm_set_flow_scale(self.handle, float(fscale)))
+
     # src/bits_circuit.jl:119-131
     def num_parameters(self):
         return self.size("parameters")

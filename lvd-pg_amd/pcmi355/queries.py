@@ -341,11 +341,16 @@ def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_r
     max(0, 1 - (batch_size + pseudocount) / flow_memory); every batch adds its flows; after a batch with
     `batch_id % update_interval == 0` the parameters are updated.  (With update_interval = 1 the first condition never
     holds, so the statistics of an epoch pile up while the parameters move after every batch -- kept as written.)
-    `fscale` other than 1 (flows of the tempered posterior, src-jl/learning/flow.jl:120-370) is not built; soft_reg > 0
-    needs an HCLT handle on the block kernels (`pcm_set_soft_reg`).
+    `fscale` other than 1: the flows of the tempered posterior (`scaled_probs_flows_circuit`,
+    src-jl/learning/flow.jl:120-373), set on the handle for the length of the loop (`pcm_set_flow_scale`; an HCLT handle
+    runs them on its layered form).  soft_reg > 0 needs an HCLT handle on the block kernels (`pcm_set_soft_reg`) and,
+    for now, fscale = 1.
     Returns the per-epoch mean log-likelihoods."""
-    if fscale != 1.0:
-        raise NotImplementedError("fscale other than 1 (tempered flows, src-jl/learning/flow.jl:120-370) is not built")
+    if fscale != 1.0 and soft_reg != 0.0:
+        raise NotImplementedError("soft_reg together with fscale other than 1: the smoothing runs in the block kernels, "
+                                  "the tempered flows on the layered engine")
+    if not (fscale > 0 and np.isfinite(fscale)):
+        raise ValueError("fscale must be positive and finite")
     _check_data(bpc, data)
     if pseudocount < 0 or not 0 <= param_inertia <= 1:
         raise ValueError("pseudocount >= 0 and 0 <= param_inertia <= 1")                        # em.jl:299-300
@@ -364,6 +369,8 @@ def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_r
     smooth = soft_reg != 0.0
     if smooth:
         check(lib.pcm_set_soft_reg(bpc.handle, float(soft_reg), int(soft_reg_width), int(soft_flow == "as_written")))
+    if fscale != 1.0:
+        check(lib.pcm_set_flow_scale(bpc.handle, float(fscale)))
     perm = torch.arange(n, dtype=torch.int32, device=data.device)
 
     def do_shuffle():
@@ -407,6 +414,8 @@ def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_r
     finally:
         if smooth:
             check(lib.pcm_set_soft_reg(bpc.handle, 0.0, 1, 0))
+        if fscale != 1.0:
+            check(lib.pcm_set_flow_scale(bpc.handle, 1.0))
     return lls
 
 

@@ -162,6 +162,70 @@ void orc_backward(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
 }
 
 /*
+ * Tempered flows of mini_batch_em_beta (fscale), VariationalJuice.jl/src-jl/learning/flow.jl:
+ *   :120-175 scale_flows_kernel -- per sum node and example the logsumexp over its edges of
+ *            (child - parent) / fscale, folded pairwise in edge order (the node-owned path, flows_buf = acc);
+ *   :204-300 reg_layer_down_kernel -- edge flow = flows[parent] * exp((child - parent) / fscale - that logsumexp)
+ *            for a sum edge, flows[parent] for a product edge; children and edge_aggr as in orc_backward.
+ * The root's flow (flows[:, end] = 1, :344) or root_flow as in orc_backward.
+ */
+void orc_backward_scaled(int n_nodes, const uint8_t* type, const int32_t* edge_ptr,
+                         const int32_t* prime, const int32_t* sub, const REAL* logp,
+                         const uint8_t* skip, const REAL* mars, int B, REAL* flows,
+                         REAL* edge_aggr, int n_roots, const int32_t* root_ids,
+                         const REAL* root_flow, REAL fscale) {
+  int n_edges = edge_ptr[n_nodes];
+  double* aggr = (double*)calloc((size_t)n_edges, sizeof(double));
+  REAL* norm = (REAL*)malloc((size_t)B * sizeof(REAL));
+  for (int64_t i = 0; i < (int64_t)n_nodes * B; ++i) flows[i] = 0;
+  if (n_roots == 0) {
+    for (int b = 0; b < B; ++b) flows[(int64_t)(n_nodes - 1) * B + b] = 1;
+  } else {
+    for (int h = 0; h < n_roots; ++h)
+      for (int b = 0; b < B; ++b) flows[(int64_t)root_ids[h] * B + b] = root_flow[(int64_t)h * B + b];
+  }
+  for (int n = n_nodes - 1; n >= 0; --n) {
+    if (type[n] == NODE_INPUT) continue;
+    int issum = type[n] == NODE_SUM;
+    if (issum)
+      for (int b = 0; b < B; ++b) {
+        int first = 1;
+        REAL acc = 0;
+        for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
+          if (skip && skip[e]) continue;
+          REAL child = mars[(int64_t)prime[e] * B + b] + logp[e];
+          if (sub[e] >= 0) child += mars[(int64_t)sub[e] * B + b];
+          REAL d = (child - mars[(int64_t)n * B + b]) / fscale;
+          acc = first ? d : lse2f(acc, d);
+          first = 0;
+        }
+        norm[b] = acc;
+      }
+    for (int e = edge_ptr[n]; e < edge_ptr[n + 1]; ++e) {
+      if (skip && skip[e]) continue;
+      double s = 0;
+      for (int b = 0; b < B; ++b) {
+        REAL ef = flows[(int64_t)n * B + b];
+        if (issum) {
+          REAL child = mars[(int64_t)prime[e] * B + b] + logp[e];
+          if (sub[e] >= 0) child += mars[(int64_t)sub[e] * B + b];
+          REAL d = (child - mars[(int64_t)n * B + b]) / fscale - norm[b];
+          ef = ef * (sizeof(REAL) == 4 ? (REAL)expf((float)d) : (REAL)exp((double)d));
+        }
+        flows[(int64_t)prime[e] * B + b] += ef;
+        if (sub[e] >= 0) flows[(int64_t)sub[e] * B + b] += ef;
+        s += ef;
+      }
+      aggr[e] += s;
+    }
+  }
+  if (edge_aggr)
+    for (int e = 0; e < n_edges; ++e) edge_aggr[e] += (REAL)aggr[e];
+  free(norm);
+  free(aggr);
+}
+
+/*
  * Leaf sufficient statistics: queries/flow.jl:165-195 with the categorical `flow`
  * of nodes/fixable_categorical_dist.jl:121-130: counts[node][value] += flows[b, node].
  * leaf_flow has the same indexing as leaf_logp (in_off[n] + category).

@@ -188,7 +188,10 @@ def forward(fc, data, idx=None, double=False):
     return mars
 
 
-def backward(fc, mars, edge_aggr=None, skip=None, root_ids=None, root_flow=None, double=False):
+def backward(fc, mars, edge_aggr=None, skip=None, root_ids=None, root_flow=None, double=False, fscale=1.0):
+    """Node flows and (added to edge_aggr) edge flows summed over the batch.  fscale != 1: the tempered flows of
+    `mini_batch_em_beta` (src-jl/learning/flow.jl:120-175, :204-300): every sum node's shares raised to 1 / fscale
+    and normalised again."""
     R = _real(double)
     B = mars.shape[1]
     flows = np.empty((fc.n_nodes, B), dtype=R)
@@ -198,6 +201,12 @@ def backward(fc, mars, edge_aggr=None, skip=None, root_ids=None, root_flow=None,
     nr = 0 if root_ids is None else len(root_ids)
     rid = None if root_ids is None else np.ascontiguousarray(root_ids, np.int32)
     rfl = None if root_flow is None else np.ascontiguousarray(root_flow, R)
+    if fscale != 1.0:
+        lib(double).orc_backward_scaled(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(fc.prime),
+                                        _p(fc.sub), _p(logp), _p(skip), _p(np.ascontiguousarray(mars, R)),
+                                        ctypes.c_int(B), _p(flows), _p(edge_aggr), ctypes.c_int(nr), _p(rid), _p(rfl),
+                                        (ctypes.c_double if double else ctypes.c_float)(fscale))
+        return flows, edge_aggr
     lib(double).orc_backward(ctypes.c_int(fc.n_nodes), _p(fc.type), _p(fc.edge_ptr), _p(fc.prime),
                              _p(fc.sub), _p(logp), _p(skip), _p(np.ascontiguousarray(mars, R)),
                              ctypes.c_int(B), _p(flows), _p(edge_aggr), ctypes.c_int(nr), _p(rid), _p(rfl))

@@ -745,6 +745,102 @@ def test_dense_groups_beside_ordinary_edges(gpu, oracle):
     assert grouped.size("dense_groups") == 2
 
 
+@pytest.mark.parametrize("fscale", [0.5, 2.5])
+def test_tempered_flows_match_the_oracle(gpu, oracle, fscale):
+    """`fscale` of mini_batch_em_beta (src-jl/learning/flow.jl:120-373, `pcm_set_flow_scale`): node flows, edge and leaf
+    statistics of the tempered pass on a random DAG (layer kernels), on a multi-head HCLT whose sums run as dense
+    groups (and the same circuit without them), and on an HCLT handle of the block engine, which hands such passes to
+    its layered form; likelihoods are not touched and fscale = 1 afterwards is the ordinary pass again."""
+    torch, P = gpu
+    O = oracle
+    import pcmi355._lib as L
+    from helpers import random_dag, multihead_hclt, make_hclt, block_theta, correlated_data, rel_err
+    rng = np.random.default_rng(61)
+    # (1) a single-root DAG
+    V, C, B = 6, 4, 90
+    root = random_dag(V, C, rng, width=3)
+    fc = O.bits_compile(root, C, V)
+    bpc = _compile(P, [root], V, C)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    d = torch.from_numpy(data).cuda()
+    order = fc.up_order()
+    mars_ref = O.forward(fc, data)
+    plain_ll = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    plain_ea, _ = bpc.get_aggregates()
+    bpc.set_flow_scale(fscale)
+    ll = P.probs_flows_circuit(bpc, d).cpu().numpy()
+    assert np.array_equal(ll, plain_ll)
+    flows_ref, ea_ref = O.backward(fc, mars_ref, fscale=fscale)
+    lf_ref = O.input_flows(fc, data, flows_ref)
+    _, flows = bpc.get_node_values(B)
+    ea, lf = bpc.get_aggregates()
+    assert np.abs(flows - flows_ref).max() < FLOW_RTOL
+    assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
+    assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
+    assert np.abs(ea - plain_ea).max() > 1e-2 * ea_ref.max()           # (and it is not the ordinary pass)
+    with pytest.raises(L.PcmError):
+        bpc.set_flow_scale(0.0)
+    bpc.set_flow_scale(1.0)
+    P.probs_flows_circuit(bpc, d)
+    assert np.array_equal(bpc.get_aggregates()[0], plain_ea)
+
+    # (2) dense groups, heads, a soft head mask
+    V, K, C, H, B = 12, 8, 5, 9, 150
+    parent = np.array([-1] + [int(rng.integers(max(0, v - 3), v)) for v in range(1, V)], np.int32)
+    heads, _ = multihead_hclt(parent, K, C, H, rng)
+    grouped, plain = _with_and_without_groups(P, heads, V, C)
+    assert grouped.size("dense_groups") > 0
+    fc = O.bits_compile(O.summate(*heads), C, V)
+    n_real = fc.n_nodes - 1
+    root_ids = (grouped.table("heads") - 1).astype(np.int32)
+    data = rng.integers(0, C, size=(B, V)).astype(np.uint8)
+    mask = rng.random((B, H)).astype(np.float32) + 0.05
+    d, hm = torch.from_numpy(data).cuda(), torch.from_numpy(mask).cuda()
+    mars_ref = O.forward(fc, data)
+    skip = (fc.edge_parent() == fc.n_nodes - 1).astype(np.uint8)
+    flows_ref, ea_ref = O.backward(fc, mars_ref, skip=skip, root_ids=root_ids, root_flow=np.ascontiguousarray(mask.T),
+                                   fscale=fscale)
+    lf_ref = O.input_flows(fc, data, flows_ref)
+    order = fc.up_order()
+    order = order[fc.edge_parent()[order] != fc.n_nodes - 1]
+    for c in (grouped, plain):
+        c.set_flow_scale(fscale)
+        P.probs_flows_circuit(c, d, head_mask=hm)
+        _, flows = c.get_node_values(B)
+        ea, lf = c.get_aggregates()
+        assert np.abs(flows - flows_ref[:n_real]).max() < FLOW_RTOL
+        assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
+        assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
+
+    # (3) an HCLT handle of the block engine: EM step with tempered flows, then an ordinary one
+    V, K, C, B = 11, 16, 7, 200
+    parent, theta, leaf, fc = make_hclt(V, K, C, 62)
+    data = correlated_data(B, V, C, 63, parent)
+    d = torch.from_numpy(data).cuda()
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    cur = fc
+    for f in (fscale, 1.0):
+        bpc.set_flow_scale(f)
+        ll = torch.empty(B, device="cuda")
+        L.check(L.lib.pcm_em_step(bpc.handle, d.data_ptr(), d.stride(0), d.stride(1), None, B, 0.0, 0.1, 0.8, ll.data_ptr()))
+        mars = O.forward(cur, data, double=True)
+        assert rel_err(ll.cpu().numpy(), mars[-1]).max() < LL_RTOL
+        flows, ea = O.backward(cur, mars, double=True, fscale=f)
+        lf = O.input_flows(cur, data, flows, double=True)
+        logp, new_leaf = O.em_update(cur, ea, lf, 0.1, 0.8, True)
+        cur = cur.copy()
+        cur.logp, cur.leaf_logp = logp.astype(np.float32), new_leaf.astype(np.float32)
+        th_ref, leaf_ref = O.hclt_block_params(cur)
+        th, lf_new = bpc.get_params()
+        for v, blk in th_ref.items():
+            assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
+        assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
+    forest = P.hclt_forest_from_clts(np.array([-1, 0, -1, 2], np.int32), 4, 16, 2)
+    with pytest.raises(L.PcmError):               # (a forest has no layered form)
+        forest.set_flow_scale(2.0)
+
+
 def test_forest_of_patch_circuits_at_their_real_shape(gpu, oracle):
     """Sixteen patch circuits of the patch-clustered configuration (8 x 8 x 3 patches of 64 x 64 x 3 images: 192
     variables, K = 32, 256 categories, 128 heads, batch 1024) as one forest handle over the image's pixels, against a

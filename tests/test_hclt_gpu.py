@@ -872,12 +872,15 @@ def test_deep_trees_three_way(gpu, oracle, V, K, C, B, chain, weighted):
                      f"V={V} K={K} C={C} B={B} depth={depth} weighted={weighted}")
 
 
-@pytest.mark.parametrize("update_interval,flow_memory", [(2, 0.0), (3, 400.0), (1, 0.0)])
-def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update_interval, flow_memory):
+@pytest.mark.parametrize("update_interval,flow_memory,fscale", [(2, 0.0, 1.0), (3, 400.0, 1.0), (1, 0.0, 1.0), (2, 300.0, 2.0),
+                                                                (1, 0.0, 0.6)])
+def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update_interval, flow_memory, fscale):
     """`mini_batch_em_beta` (src-jl/learning/em.jl:289-409): statistics collect over `update_interval` batches, are
     cleared (or decayed by the flow memory) at a batch with batch_id % update_interval == 1, and the parameters move
     after a batch with batch_id % update_interval == 0 -- replayed on the float64 oracle batch by batch, including the
-    source's behaviour at update_interval = 1 (the clearing condition never holds, the statistics of an epoch pile up)."""
+    source's behaviour at update_interval = 1 (the clearing condition never holds, the statistics of an epoch pile up).
+    fscale != 1: the flows of the tempered posterior (src-jl/learning/flow.jl:120-373), which an HCLT handle runs on
+    its layered form."""
     torch, P = gpu
     from helpers import make_hclt, correlated_data, block_theta, rel_err
     V, K, C, B, nb, pc, inertia = 10, 16, 12, 64, 6, 0.1, 0.7
@@ -887,7 +890,7 @@ def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update
     bpc.set_params(block_theta(parent, K, theta), leaf)
     lls = P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 2, batch_size=B, pseudocount=pc, param_inertia=inertia,
                                param_inertia_end=0.9, flow_memory=flow_memory, flow_memory_end=flow_memory * 2,
-                               shuffle="none", update_interval=update_interval)
+                               shuffle="none", update_interval=update_interval, fscale=fscale)
     cur, want, inr, fm = fc.copy(), [], inertia, flow_memory
     for epoch in range(2):
         ea = lf = None
@@ -898,7 +901,7 @@ def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update
                 rate = 0.0 if fm == 0 else max(0.0, 1.0 - (B + pc) / fm)
                 ea, lf = ea * rate, lf * rate
             mars = oracle.forward(cur, data, idx, True)
-            flows, ea_b = oracle.backward(cur, mars, double=True)
+            flows, ea_b = oracle.backward(cur, mars, double=True, fscale=fscale)
             lf_b = oracle.input_flows(cur, data, flows, idx, double=True)
             ea = ea_b if ea is None else ea + ea_b
             lf = lf_b if lf is None else lf + lf_b
@@ -916,5 +919,9 @@ def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update
     for v, blk in th_ref.items():
         assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
     assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
-    with pytest.raises(NotImplementedError):
-        P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia, fscale=2.0)
+    with pytest.raises(NotImplementedError):      # the smoothing is the block kernels', the tempered flows the layered engine's
+        P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia, fscale=2.0,
+                             soft_reg=0.01, soft_reg_width=3)
+    # the loop leaves the handle as it found it: an ordinary step afterwards runs on the block kernels again
+    ll = P.probs_flows_circuit(bpc, torch.from_numpy(data[:B]).cuda()).cpu().numpy()
+    assert rel_err(ll, oracle.forward(cur, data[:B], double=True)[-1]).max() < 1e-4

@@ -56,7 +56,7 @@ def test_host_module_blocks_are_balanced_and_has_the_reference_interface():
     ends = len(re.findall(r"(?<![\w.:])end(?![\w!])", src))
     assert opens == ends, (opens, ends)
     assert src.count("(") == src.count(")") and src.count("[") == src.count("]")
-    for name in ("loglikelihoods", "loglikelihood", "probs_flows_circuit", "mini_batch_em_with_reg",
+    for name in ("loglikelihoods", "loglikelihood", "probs_flows_circuit", "mini_batch_em_with_reg", "mini_batch_em_beta",
                  "mini_batch_em_for_multihead_pc", "vectorize_parameters", "update_parameters", "kld", "kld_backward",
                  "gumbel_sample", "gumbel_sample_backward", "per_sample_normalized_flows", "normalize_params", "hclt",
                  "hclt_from_clt", "pairwise_MI", "learn_chow_liu_tree", "num_parameters"):
@@ -66,5 +66,11 @@ def test_host_module_blocks_are_balanced_and_has_the_reference_interface():
     sig = sig[:sig.index(")\n")]
     for kw in ("batch_size", "pseudocount", "soft_reg", "soft_reg_width", "ent_reg", "param_inertia", "param_inertia_end",
                "flow_memory", "shuffle", "verbose"):
+        assert re.search(rf"\b{kw}\b", sig), kw
+    # ... and of the interval driver (VariationalJuice.jl/src-jl/learning/em.jl:289-296)
+    sig = src[src.index("function mini_batch_em_beta("):]
+    sig = sig[:sig.index(")\n")]
+    for kw in ("batch_size", "pseudocount", "soft_reg", "soft_reg_width", "param_inertia", "param_inertia_end", "flow_memory",
+               "flow_memory_end", "shuffle", "update_interval", "fscale", "verbose"):
         assert re.search(rf"\b{kw}\b", sig), kw
     assert "CUDA" not in src and "AMDGPU" not in src

@@ -233,6 +233,51 @@ def test_flow_invariants():
     np.testing.assert_allclose(lf.reshape(8, -1).sum(axis=1), 30.0, rtol=1e-4)
 
 
+def test_tempered_flows_by_hand_and_in_their_limits():
+    """fscale of mini_batch_em_beta (src-jl/learning/flow.jl:120-175, :204-300): a sum node hands its flow down in
+    shares proportional to (posterior share)^(1 / fscale).  One sum node over two leaves by hand; fscale = 1 is the
+    ordinary pass; a very large fscale splits evenly; whatever the scale a sum's edge flows add up to its flow and a
+    product hands its flow on unchanged."""
+    C = 3
+    pa, pb = np.array([0.5, 0.25, 0.25], np.float32), np.array([0.1, 0.1, 0.8], np.float32)
+    root = O.summate(O.input_node(0, np.log(pa)), O.input_node(0, np.log(pb)), logps=np.log(np.float32([0.2, 0.8])))
+    fc = O.bits_compile(root, C, 1)
+    data = np.array([[0], [2]], np.uint8)
+    mars = O.forward(fc, data, double=True)
+    flows, ea = O.backward(fc, mars, double=True, fscale=2.0)
+    # example 0: terms 0.2 * 0.5 = 0.1 and 0.8 * 0.1 = 0.08 -> square roots 0.31623, 0.28284 -> shares 0.52786, 0.47214
+    # example 1: terms 0.2 * 0.25 = 0.05 and 0.8 * 0.8 = 0.64 -> 0.22361, 0.8 -> shares 0.218450, 0.781550
+    np.testing.assert_allclose(flows[0], [0.527864, 0.218450], rtol=2e-6)
+    np.testing.assert_allclose(flows[1], [0.472136, 0.781550], rtol=2e-6)
+    np.testing.assert_allclose(ea, [0.527864 + 0.218450, 0.472136 + 0.781550], rtol=2e-6)
+
+    parent, theta, leaf, fc = make_hclt(9, 4, 5, 25)
+    data = correlated_data(20, 9, 5, 26, parent)
+    mars = O.forward(fc, data, double=True)
+    plain, ea_plain = O.backward(fc, mars, double=True)
+    one, ea_one = O.backward(fc, mars, double=True, fscale=1.0 + 1e-12)      # through the tempered code
+    np.testing.assert_allclose(one, plain, rtol=1e-9, atol=1e-300)
+    np.testing.assert_allclose(ea_one, ea_plain, rtol=1e-9)
+    for fscale in (0.5, 3.0, 1e9):
+        flows, ea = O.backward(fc, mars, double=True, fscale=fscale)
+        par = fc.edge_parent()
+        for n in np.nonzero(fc.type != O.INPUT)[0]:
+            es = np.arange(fc.edge_ptr[n], fc.edge_ptr[n + 1])
+            if fc.type[n] == O.SUM:
+                np.testing.assert_allclose(ea[es].sum(), flows[n].sum(), rtol=1e-9)
+                if fscale == 1e9:
+                    np.testing.assert_allclose(ea[es], flows[n].sum() / len(es), rtol=1e-6)
+            else:
+                np.testing.assert_allclose(ea[es], flows[n].sum(), rtol=1e-9)
+        np.testing.assert_allclose(flows[fc.type == O.INPUT].reshape(9, -1, 20).sum(axis=1), 1.0, rtol=1e-9)
+    # sharper than the posterior: fscale < 1 moves flow towards the larger share
+    sharp, _ = O.backward(fc, mars, double=True, fscale=0.5)
+    top = fc.meta["sum_node"][int(np.nonzero(np.asarray(parent) < 0)[0][0])]
+    es = np.arange(fc.edge_ptr[top[0]], fc.edge_ptr[top[0] + 1])
+    kids = fc.prime[es]
+    assert (sharp[kids].max(axis=0) >= plain[kids].max(axis=0) - 1e-12).all()
+
+
 # ------------------------------------------------------------------------------------
 # EM update
 # ------------------------------------------------------------------------------------
