@@ -628,7 +628,7 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
     H = len(heads)
     grouped, plain = _with_and_without_groups(P, heads, V, C)
     assert grouped.size("dense_groups") >= min_groups
-    assert grouped.size("layer_nodes") < grouped.num_nodes()
+    assert grouped.size("layer_nodes") < grouped.num_nodes() or grouped.size("dense_groups") == 0
     fc = O.bits_compile(O.summate(*heads), C, V)
     n_real = fc.n_nodes - 1
     assert grouped.num_nodes() == n_real
@@ -654,7 +654,7 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
         finite = np.isfinite(mars_ref[:n_real])
         assert np.array_equal(np.isfinite(mars), finite)
         assert np.abs(mars[finite] - mars_ref[:n_real][finite]).max() < LL_RTOL * np.abs(mars_ref[:n_real][finite]).max()
-        assert np.abs(flows - flows_ref[:n_real]).max() < FLOW_RTOL
+        assert np.abs(flows - flows_ref[:n_real]).max() < FLOW_RTOL * max(flows_ref.max(), 1.0)   # (an example's flow: the sum of its mask)
         ea, lf = bpc.get_aggregates()
         assert np.abs(ea - ea_ref[order]).max() < FLOW_RTOL * ea_ref.max()
         assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
