@@ -162,15 +162,15 @@ class HcltCircuit : public pcm_circuit {
   void sample_soft(const float* d_node_noise, float temperature, int32_t batch, float* d_out) override;
   void flow_gradients(int32_t batch_size, float* d_grad) override;
   void leaf_adam(float* d_aux_p, float* d_aux_m, float* d_aux_v, float lr, float b1, float b2, float eps, int t) override;
-  // parameter-row queries run on the circuit's general form (its structure; the rows bring the parameters)
+  // Parameter-row queries: the KL recursion and its gradient on the block form with the row as a grid dimension
+  // (hclt_kld.hip) for single-root circuits with block kernels; everything else on the circuit's general form (its
+  // structure; the rows bring the parameters).
   void kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
-                float* d_out) override {
-    general_structure()->kld_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_out);
-  }
+                float* d_out) override;
   void kld_backward_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
-                         float* d_g1, float* d_g2, float* d_klds) override {
-    general_structure()->kld_backward_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_g1, d_g2, d_klds);
-  }
+                         float* d_g1, float* d_g2, float* d_klds) override;
+  void kld_rows_block(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm, float* d_klds,
+                      float* d_g1, float* d_g2);
   void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                           float temperature, bool norm_params, float* d_out) override {
     general_structure()->gumbel_sample_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params, d_out);
@@ -353,6 +353,8 @@ class HcltCircuit : public pcm_circuit {
   SparseCircuit* general_structure();   // the same object without bringing its parameters up to date
   // KL recursion on the block form
   DevBuf<int32_t> d_kl_up_, d_kl_down_;   // chain steps (KlItem records) bottom-up / top-down
+  DevBuf<int32_t> d_blk2par_;             // entry of the [n_inner][K][K] blocks -> parameter (-1: no such edge), for the row queries
+  DevBuf<float> d_rows_scratch_, d_rows_pk1_, d_rows_pk2_, d_rows_pg1_, d_rows_pg2_;   // row queries: per-row arrays; re-laid-out matrices
   DevBuf<int32_t> d_kl_tabs_;             // parent of every inner node | h-giving node of every variable | input-node positions
   DevBuf<int32_t> d_kl_pos_;              // chain slot of every inner node: upward | downward
   DevBuf<float> d_kl_leaf_, d_kl_vec_, d_kl_par_;

@@ -129,6 +129,12 @@ __global__ __launch_bounds__(256) void hclt_kld_base_kernel(const HcltNode* __re
   }
 }
 
+// Distances in floats between the arrays of consecutive rows when the chains run on a matrix of parameter rows (one
+// pair of chains per row, blockIdx.y); all zero for the circuit's own parameters.
+struct KlRowStrides {
+  size_t pu, pd, vec, out, ring_up, ring_down;
+};
+
 // The two chains.  Workgroup 0 walks up (KL_v, Z_v), workgroup 1 walks down (h_v); launched
 // with one workgroup when only the divergence is wanted.  A step is kl_waves(K) independent
 // nodes (same level).  The vectors a step reads were left in the ring by earlier steps of the
@@ -143,12 +149,19 @@ __global__ __launch_bounds__(kl_waves(K) * 64) void hclt_kld_chain_kernel(
     const KlItem* __restrict__ up_items, int up_steps, const KlItem* __restrict__ down_items, int down_steps,
     const int32_t* __restrict__ ext, const float* __restrict__ pu, const float* __restrict__ base,
     const float* __restrict__ ell, const float* __restrict__ pd, int ring_mask, float* ring_up, float* ring_down,
-    float* __restrict__ klv, float* __restrict__ z, float* __restrict__ h) {
+    float* __restrict__ klv, float* __restrict__ z, float* __restrict__ h, KlRowStrides rs) {
   constexpr int PARTS = 64 / K, JP = K / PARTS, Q = JP / 4, W = kl_waves(K), D = kl_ahead(K);
   extern __shared__ float lds_ring[];   // kLds: [ring_mask + 1][K]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane % K, part = lane / K;
   const bool up = blockIdx.x == 0;
+  {   // a row of a parameter matrix per blockIdx.y: its operands, constants and results sit rs.* floats further on
+    const size_t row = blockIdx.y;
+    pu += row * rs.pu; pd += row * rs.pd; base += row * rs.vec; ell += row * rs.vec;
+    klv += row * rs.out; z += row * rs.out; h += row * rs.out;
+    if (ring_up) ring_up += row * rs.ring_up;
+    if (ring_down) ring_down += row * rs.ring_down;
+  }
   const int steps = up ? up_steps : down_steps;
   const int4* __restrict__ items = reinterpret_cast<const int4*>(up ? up_items : down_items);
   const float4* __restrict__ par = reinterpret_cast<const float4*>(up ? pu : pd);
@@ -525,7 +538,7 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
       hipLaunchKernelGGL(kernel, dim3(with_down ? 2 : 1), dim3(kl_waves(KK) * 64), lds, stream,
                          reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
                          reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
-                         kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h);
+                         kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, KlRowStrides{0, 0, 0, 0, 0, 0});
     };
     if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
     else chain(&hclt_kld_chain_kernel<KK, false>, 0);
@@ -606,6 +619,309 @@ void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, fl
   rebuild_w();
   general_stale_ = true;
   PCM_HIP(hipStreamSynchronize(stream));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// The same recursion on a MATRIX of parameter rows (`kld(mbpc, params1[R, n], params2[R, n])` src/queries/kld.jl:164-206,
+// `kld_backward` :593-649, reached from src/utils/cuda_preallocation.jl:47-78 with one row per example): every row is a
+// pair of circuits of this structure, and nothing couples two rows, so the block-form pipeline above runs with the row
+// as a second grid dimension -- the leaf terms straight from the rows (a wave per (input node, row), 16-byte loads: nine
+// tenths of the bytes of a query), the per-node operands gathered from the rows through a block-entry -> parameter
+// table, one pair of chains per row, and the gradients written in parameter order where they belong.  Against the
+// per-layer kernels of the general form (one launch per layer and a lane group per (node, row)) this is six launches.
+// ---------------------------------------------------------------------------------------------------------
+
+constexpr float kRowsNormEps = 1e-8f;   // leaf parameters that are probabilities: fixable_categorical_dist.jl:182-186
+
+template <bool kNorm>
+__device__ __forceinline__ float rows_leaf_term(float x, float y) {
+  return kNorm ? x * (logf(x + kRowsNormEps) - logf(y + kRowsNormEps)) : expf(x) * (x - y);
+}
+
+// kl_leaf[row][v * K + j] of input node i = (v, j): a wave takes four input nodes of one row
+template <bool kNorm, bool kVec>
+__global__ __launch_bounds__(256) void hclt_rows_leaf_kl_kernel(const float* __restrict__ P1, const float* __restrict__ P2,
+                                                                size_t n_par, size_t ns, int C, int n_inputs,
+                                                                const int32_t* __restrict__ input_order, size_t vk,
+                                                                float* __restrict__ kl_leaf) {
+  const int lane = threadIdx.x & 63;
+  const int i0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 4;
+  const size_t row = blockIdx.y;
+  if (i0 >= n_inputs) return;
+  const float* a = P1 + row * n_par + ns + (size_t)i0 * C;
+  const float* b = P2 + row * n_par + ns + (size_t)i0 * C;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (kVec) {
+    for (int c4 = lane; c4 < C / 4; c4 += 64) {
+      float4 x[4], y[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int iu = min(i0 + u, n_inputs - 1) - i0;   // (past the last node: the last node again, not added)
+        x[u] = reinterpret_cast<const float4*>(a + (size_t)iu * C)[c4];
+        y[u] = reinterpret_cast<const float4*>(b + (size_t)iu * C)[c4];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        acc[u] += (rows_leaf_term<kNorm>(x[u].x, y[u].x) + rows_leaf_term<kNorm>(x[u].y, y[u].y)) +
+                  (rows_leaf_term<kNorm>(x[u].z, y[u].z) + rows_leaf_term<kNorm>(x[u].w, y[u].w));
+    }
+  } else {
+    for (int c = lane; c < C; c += 64)
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int iu = min(i0 + u, n_inputs - 1) - i0;
+        acc[u] += rows_leaf_term<kNorm>(a[(size_t)iu * C + c], b[(size_t)iu * C + c]);
+      }
+  }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) acc[u] += __shfl_xor(acc[u], o);
+    if (lane == 0 && i0 + u < n_inputs) kl_leaf[row * vk + input_order[i0 + u]] = acc[u];
+  }
+}
+
+// hclt_kld_base_kernel for (tree node, row): theta through blk2par (entry of the [n_inner][K][K] blocks -> parameter,
+// -1: an edge that is not there, the root's rows past the first)
+template <int K>
+__global__ __launch_bounds__(256) void hclt_rows_base_kernel(const HcltNode* __restrict__ nodes,
+                                                             const int32_t* __restrict__ child_leaf,
+                                                             const int32_t* __restrict__ pos, int n_inner,
+                                                             const int32_t* __restrict__ blk2par,
+                                                             const float* __restrict__ P1, const float* __restrict__ P2,
+                                                             size_t n_par, const float* __restrict__ kl_leaf, size_t vk,
+                                                             float* __restrict__ ell, float* __restrict__ base,
+                                                             float* __restrict__ pu, float* __restrict__ pd, KlRowStrides rs) {
+  __shared__ float tile[K][K + 1];
+  __shared__ float l[K];
+  const int n = blockIdx.x, t = threadIdx.x;
+  const size_t row = blockIdx.y;
+  const HcltNode nd = nodes[n];
+  const size_t su = (size_t)pos[n], sd = (size_t)pos[n_inner + n];
+  const float* p1 = P1 + row * n_par;
+  const float* p2 = P2 + row * n_par;
+  kl_leaf += row * vk;
+  ell += row * rs.vec;
+  base += row * rs.vec;
+  if (t < K) {
+    float s = kl_leaf[(size_t)nd.var * K + t];
+    for (int q = 0; q < nd.lc_cnt; ++q) s += kl_leaf[(size_t)child_leaf[nd.lc_off + q] * K + t];
+    l[t] = s;
+    ell[su * K + t] = s;
+  }
+  __syncthreads();
+  const int j = t % K;
+  for (int k = t / K; k < K; k += 256 / K) {
+    const int idx = blk2par[((size_t)n * K + k) * K + j];
+    const float x = idx >= 0 ? p1[idx] : -INFINITY, y = idx >= 0 ? p2[idx] : 0.f;
+    const float p = expf(x);
+    tile[k][j] = p;
+    float term = p > 0.f ? p * (x - y + l[j]) : 0.f;
+#pragma unroll
+    for (int o = K / 2; o > 0; o >>= 1) term += __shfl_xor(term, o, K);
+    if (j == 0) base[su * K + k] = term;
+  }
+  __syncthreads();
+  constexpr int JP = K * K / 64;
+  float* pur = pu + row * rs.pu + su * K * K;
+  float* pdr = pd ? pd + row * rs.pd + sd * K * K : nullptr;
+  for (int w = t; w < K * K; w += 256) {
+    const int e = w & 3, lane = (w >> 2) & 63, i4 = w >> 8;
+    const int rw = (lane / K) * JP + i4 * 4 + e, col = lane % K;
+    pur[w] = tile[col][rw];
+    if (pdr) pdr[w] = tile[rw][col];
+  }
+}
+
+__global__ void hclt_rows_take_kernel(const float* __restrict__ klv, size_t nk, size_t at, int rows, float* __restrict__ out) {
+  const int r = blockIdx.x * blockDim.x + threadIdx.x;
+  if (r < rows) out[r] = klv[(size_t)r * nk + at];
+}
+
+// hclt_kld_edge_grad_kernel on rows: the parameters are the rows' own entries.  A thread takes one parameter through
+// kEdgeGradRows rows, so its place in the blocks is looked up once.
+constexpr int kEdgeGradRows = 8;
+
+__global__ void hclt_rows_edge_grad_kernel(int64_t ns, int K, const int64_t* __restrict__ src,
+                                           const int32_t* __restrict__ parent_of, const float* __restrict__ P1,
+                                           const float* __restrict__ P2, size_t n_par, const float* __restrict__ z,
+                                           const float* __restrict__ h, size_t nk, int rows, float* __restrict__ G1,
+                                           float* __restrict__ G2) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= ns) return;
+  const int64_t s = src[i];
+  const int j = (int)(s % K), k = (int)((s / K) % K);
+  const int n = (int)(s / ((int64_t)K * K));
+  const int par = parent_of[n];
+  const size_t zat = (size_t)n * K + j, hat = par < 0 ? 0 : (size_t)par * K + k;
+  const int r0 = blockIdx.y * kEdgeGradRows;
+  float a[kEdgeGradRows], b[kEdgeGradRows], zz[kEdgeGradRows], g[kEdgeGradRows];
+#pragma unroll
+  for (int q = 0; q < kEdgeGradRows; ++q) {
+    const size_t row = (size_t)min(r0 + q, rows - 1);
+    a[q] = P1[row * n_par + i];
+    b[q] = P2[row * n_par + i];
+    zz[q] = z[row * nk + zat];
+    g[q] = h[row * nk + hat];
+  }
+#pragma unroll
+  for (int q = 0; q < kEdgeGradRows; ++q) {
+    if (r0 + q >= rows) break;
+    const size_t row = (size_t)(r0 + q);
+    const float gg = par < 0 ? 1.f : g[q], p1 = expf(a[q]);
+    G1[row * n_par + i] = gg * (p1 * (zz[q] + a[q] - b[q]) + p1);
+    G2[row * n_par + i] = -gg * p1;
+  }
+}
+
+// gradients of the leaf parameters, as the source writes them (src/queries/kld.jl:528-535,
+// src/nodes/fixable_categorical_dist.jl:216-219): a thread takes four consecutive categories of one input node
+template <bool kNorm>
+__global__ __launch_bounds__(256) void hclt_rows_leaf_grad_kernel(const float* __restrict__ P1, const float* __restrict__ P2,
+                                                                  size_t n_par, size_t ns, int C, int K, int64_t n_leaf4,
+                                                                  const int32_t* __restrict__ input_order,
+                                                                  const int32_t* __restrict__ state_node,
+                                                                  const float* __restrict__ h, size_t nk,
+                                                                  float* __restrict__ G1, float* __restrict__ G2) {
+  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t row = blockIdx.y;
+  if (q >= n_leaf4) return;
+  const int64_t at = q * 4;
+  const int vj = input_order[at / C];
+  const float g = h[row * nk + (size_t)state_node[vj / K] * K + vj % K];
+  const size_t off = row * n_par + ns + at;
+  const float4 a = *reinterpret_cast<const float4*>(P1 + off), b = *reinterpret_cast<const float4*>(P2 + off);
+  auto d1 = [&](float x, float y) { return kNorm ? g * (logf(x + kRowsNormEps) - logf(y + kRowsNormEps) + 1.f) : g * (x - y + 1.f); };
+  auto d2 = [&](float x, float y) { return kNorm ? g * x / (y + kRowsNormEps) : g * expf(x - y); };
+  *reinterpret_cast<float4*>(G1 + off) = make_float4(d1(a.x, b.x), d1(a.y, b.y), d1(a.z, b.z), d1(a.w, b.w));
+  *reinterpret_cast<float4*>(G2 + off) = make_float4(d2(a.x, b.x), d2(a.y, b.y), d2(a.z, b.z), d2(a.w, b.w));
+}
+
+// KL of every row (d_klds, may be null with gradients) and, with d_g1 / d_g2, its gradients in the layout of the inputs
+void HcltCircuit::kld_rows_block(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm,
+                                 float* d_klds, float* d_g1, float* d_g2) {
+  const bool with_down = d_g1 != nullptr;
+  build_kld_tables();
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  const int64_t n = size(0);
+  if (d_blk2par_.n == 0) {
+    std::vector<int32_t> b2p((size_t)n_inner_ * K_ * K_, -1);
+    for (int64_t i = 0; i < ns; ++i) b2p[(size_t)sum_param_src_[i]] = (int32_t)i;
+    d_blk2par_.upload(b2p, stream);
+  }
+  if (d_input_order_.n == 0) d_input_order_.upload(input_order_, stream);
+  const float* p1 = rows_packed_in(d_p1, sr, sp, rows, n, d_rows_pk1_, stream);
+  const float* p2 = rows_packed_in(d_p2, sr, sp, rows, n, d_rows_pk2_, stream);
+  const bool direct = sp == 1 && sr == n;
+  float* g1 = d_g1;
+  float* g2 = d_g2;
+  if (with_down && !direct) {
+    d_rows_pg1_.ensure((size_t)rows * n);
+    d_rows_pg2_.ensure((size_t)rows * n);
+    g1 = d_rows_pg1_.p;
+    g2 = d_rows_pg2_.p;
+  }
+  const int W = kl_waves(K_), D = kl_ahead(K_);
+  const size_t nk = (size_t)n_inner_ * K_, vk = (size_t)V_ * K_;
+  const size_t su = (size_t)(kl_up_steps_ + D) * W, sd = (size_t)(kl_down_steps_ + D) * W, sm = std::max(su, sd);
+  KlRowStrides rs;
+  rs.pu = su * K_ * K_;
+  rs.pd = with_down ? sd * K_ * K_ : 0;
+  rs.vec = sm * K_;
+  rs.out = nk;
+  rs.ring_up = kl_ring_slots_ ? 0 : su * K_;
+  rs.ring_down = kl_ring_slots_ ? 0 : sd * K_;
+  const size_t per_row = vk + 2 * rs.vec + rs.pu + rs.pd + 3 * nk + rs.ring_up + rs.ring_down;
+  // rows at a time: what keeps the scratch arrays within 8 GB
+  const int chunk = (int)std::max<size_t>(1, std::min<size_t>((size_t)rows, ((size_t)2 << 30) / per_row));
+  d_rows_scratch_.ensure((size_t)chunk * per_row);
+  float* kl_leaf = d_rows_scratch_.p;
+  float* ell = kl_leaf + (size_t)chunk * vk;
+  float* base = ell + (size_t)chunk * rs.vec;
+  float* pu = base + (size_t)chunk * rs.vec;
+  float* pd = with_down ? pu + (size_t)chunk * rs.pu : nullptr;
+  float* klv = pu + (size_t)chunk * (rs.pu + rs.pd);
+  float* z = klv + (size_t)chunk * nk;
+  float* h = z + (size_t)chunk * nk;
+  float* ring_up = kl_ring_slots_ ? nullptr : h + (size_t)chunk * nk;
+  float* ring_down = kl_ring_slots_ ? nullptr : ring_up + (size_t)chunk * rs.ring_up;
+  // (klv, z and h of a row sit nk apart per row, not behind one another: rs.out strides each of them)
+  const int n_inputs = (int)input_order_.size();
+  const bool vec = C_ % 4 == 0 && n % 4 == 0 && ns % 4 == 0 && ((reinterpret_cast<uintptr_t>(p1) | reinterpret_cast<uintptr_t>(p2)) & 15) == 0;
+  const bool vec_g = vec && (!with_down || ((reinterpret_cast<uintptr_t>(g1) | reinterpret_cast<uintptr_t>(g2)) & 15) == 0);
+  if (with_down && !vec_g) fail(PCM_ERR_UNSUPPORTED, "row gradients on the block kernels need 16-byte aligned matrices and a category count divisible by 4");
+  const size_t root_at = (size_t)inner_of_var_[root_] * K_;
+  for (int r0 = 0; r0 < rows; r0 += chunk) {
+    const int rc = std::min(chunk, rows - r0);
+    const float* q1 = p1 + (size_t)r0 * n;
+    const float* q2 = p2 + (size_t)r0 * n;
+    const dim3 lgrid(ceil_div(n_inputs, 16), rc);
+    auto leaf = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, lgrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, n_inputs, d_input_order_.p, vk, kl_leaf);
+    };
+    if (norm) { if (vec) leaf(&hclt_rows_leaf_kl_kernel<true, true>); else leaf(&hclt_rows_leaf_kl_kernel<true, false>); }
+    else { if (vec) leaf(&hclt_rows_leaf_kl_kernel<false, true>); else leaf(&hclt_rows_leaf_kl_kernel<false, false>); }
+    PCM_DISPATCH_K(K_, {
+      hipLaunchKernelGGL(hclt_rows_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
+                         d_kl_pos_.p, n_inner_, d_blk2par_.p, q1, q2, (size_t)n, kl_leaf, vk, ell, base, pu, pd, rs);
+      auto chain = [&](auto kernel, size_t lds) {
+        hipLaunchKernelGGL(kernel, dim3(with_down ? 2 : 1, rc), dim3(kl_waves(KK) * 64), lds, stream,
+                           reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                           reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
+                           kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, rs);
+      };
+      if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
+      else chain(&hclt_kld_chain_kernel<KK, false>, 0);
+    });
+    if (d_klds)
+      hipLaunchKernelGGL(hclt_rows_take_kernel, dim3(ceil_div(rc, 256)), dim3(256), 0, stream, klv, nk, root_at, rc, d_klds + r0);
+    if (with_down) {
+      float* o1 = g1 + (size_t)r0 * n;
+      float* o2 = g2 + (size_t)r0 * n;
+      hipLaunchKernelGGL(hclt_rows_edge_grad_kernel, dim3((unsigned)ceil_div(ns, 256), ceil_div(rc, kEdgeGradRows)), dim3(256), 0,
+                         stream, ns, K_, d_sum_param_src_.p, d_kl_tabs_.p, q1, q2, (size_t)n, z, h, nk, rc, o1, o2);
+      const int64_t n_leaf4 = (int64_t)n_inputs * C_ / 4;
+      const dim3 ggrid((unsigned)ceil_div(n_leaf4, 256), rc);
+      if (norm)
+        hipLaunchKernelGGL(hclt_rows_leaf_grad_kernel<true>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
+                           n_leaf4, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, o1, o2);
+      else
+        hipLaunchKernelGGL(hclt_rows_leaf_grad_kernel<false>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
+                           n_leaf4, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, o1, o2);
+    }
+  }
+  if (with_down && !direct) {
+    rows_unpack_out(g1, d_g1, sr, sp, rows, n, stream);
+    rows_unpack_out(g2, d_g2, sr, sp, rows, n, stream);
+  }
+  check_launch_k("hclt_kld_rows");
+}
+
+static void check_rows_block_args(const void* p1, const void* p2, int64_t sr, int64_t sp, int rows) {
+  if (!p1 || !p2) fail(PCM_ERR_ARG, "parameter matrix is null");
+  if (rows < 1) fail(PCM_ERR_ARG, "need at least one parameter row, got %d", rows);
+  if (rows > 65535) fail(PCM_ERR_UNSUPPORTED, "at most 65535 parameter rows per call, got %d", rows);
+  if (sr == 0 || sp == 0) fail(PCM_ERR_ARG, "parameter matrix strides must not be zero");
+}
+
+void HcltCircuit::kld_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                           float* d_out) {
+  if (!block_queries() || H_ > 0 || missing_) return general_structure()->kld_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_out);
+  check_rows_block_args(d_p1, d_p2, sr, sp, rows);
+  if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
+  kld_rows_block(d_p1, d_p2, sr, sp, rows, norm_params, d_out, nullptr, nullptr);
+}
+
+void HcltCircuit::kld_backward_rows(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm_params,
+                                    float* d_g1, float* d_g2, float* d_klds) {
+  const bool aligned = C_ % 4 == 0 && size(0) % 4 == 0 && (int64_t)sum_param_src_.size() % 4 == 0 &&
+                       ((reinterpret_cast<uintptr_t>(d_p1) | reinterpret_cast<uintptr_t>(d_p2) | reinterpret_cast<uintptr_t>(d_g1) |
+                         reinterpret_cast<uintptr_t>(d_g2)) & 15) == 0;
+  if (!block_queries() || H_ > 0 || missing_ || !aligned)
+    return general_structure()->kld_backward_rows(d_p1, d_p2, sr, sp, rows, norm_params, d_g1, d_g2, d_klds);
+  check_rows_block_args(d_p1, d_p2, sr, sp, rows);
+  if (!d_g1 || !d_g2) fail(PCM_ERR_ARG, "parameter or gradient matrix is null");
+  kld_rows_block(d_p1, d_p2, sr, sp, rows, norm_params, d_klds, d_g1, d_g2);
 }
 
 }  // namespace pcm

@@ -418,15 +418,25 @@ void check_rows_args(const SparseCircuit& c, const FlatCircuit& fc, const void* 
   if (sr == 0 || sp == 0) fail(PCM_ERR_ARG, "parameter matrix strides must not be zero");
 }
 
-// the matrix with unit stride along the parameters: itself, or a re-laid-out copy in `tmp`
 const float* packed_in(const float* m, int64_t sr, int64_t sp, int rows, int64_t n, DevBuf<float>& tmp, hipStream_t s) {
+  return rows_packed_in(m, sr, sp, rows, n, tmp, s);
+}
+}  // namespace
+
+// the matrix with unit stride along the parameters: itself, or a re-laid-out copy in `tmp`
+const float* rows_packed_in(const float* m, int64_t sr, int64_t sp, int rows, int64_t n, DevBuf<float>& tmp, hipStream_t s) {
   if (sp == 1 && sr == n) return m;
   tmp.ensure((size_t)rows * n);
   hipLaunchKernelGGL(rows_relayout_kernel<true>, dim3((unsigned)ceil_div(n, 32), ceil_div(rows, 32)), dim3(256), 0, s, tmp.p,
                      const_cast<float*>(m), sr, sp, rows, n);
   return tmp.p;
 }
-}  // namespace
+
+// ... and back: a packed [rows][n] result into the caller's matrix
+void rows_unpack_out(float* packed, float* m, int64_t sr, int64_t sp, int rows, int64_t n, hipStream_t s) {
+  hipLaunchKernelGGL(rows_relayout_kernel<false>, dim3((unsigned)ceil_div(n, 32), ceil_div(rows, 32)), dim3(256), 0, s, packed, m,
+                     sr, sp, rows, n);
+}
 
 // klds [rows] on the device; with_edges keeps what the reverse pass needs
 void SparseCircuit::kld_rows_forward(const float* p1, const float* p2, int rows, bool norm, bool with_edges) {

@@ -43,6 +43,11 @@ FlatCircuit flatten_dag(int32_t num_nodes, const uint8_t* node_type, const int32
                         const int32_t* child_idx, const float* sum_logp, const int32_t* input_var,
                         const float* input_logp, int32_t num_vars, int32_t num_cats, int32_t num_heads);
 
+// Matrices of parameter rows arrive with element strides; the row kernels want unit stride along the parameters
+// (param_rows.hip): the matrix itself, or a re-laid-out copy in `tmp`; and a packed result back into a strided matrix.
+const float* rows_packed_in(const float* m, int64_t sr, int64_t sp, int rows, int64_t n, DevBuf<float>& tmp, hipStream_t s);
+void rows_unpack_out(float* packed, float* m, int64_t sr, int64_t sp, int rows, int64_t n, hipStream_t s);
+
 class SparseCircuit : public pcm_circuit {
  public:
   explicit SparseCircuit(FlatCircuit fc);

@@ -375,7 +375,8 @@ def _row_oracle(O, fc, row, n_sum, norm):
 
 
 @pytest.mark.parametrize("kind,R,norm", [("hclt", 1, False), ("hclt", 7, True), ("hclt", 64, False), ("dag", 7, False),
-                                         ("dag", 64, True), ("hclt64", 5, True)])
+                                         ("dag", 64, True), ("hclt64", 5, True), ("hclt_c8", 7, False), ("hclt_c8", 33, True),
+                                         ("hclt32_c12", 5, False), ("hclt64_c4", 3, True)])
 def test_parameter_row_queries_match_oracle(gpu, oracle, kind, R, norm):
     """`kld`, `kld_backward` and `gumbel_sample` on a matrix of parameter rows (src/queries/kld.jl:164-206,
     :593-649, src/queries/sample.jl:338-383), all rows in one pass, log-parameters and probability-valued
@@ -386,7 +387,9 @@ def test_parameter_row_queries_match_oracle(gpu, oracle, kind, R, norm):
     from helpers import make_hclt, block_theta, random_dag, log_dirichlet
     rng = np.random.default_rng(100 + R)
     if kind.startswith("hclt"):
-        V, K, C = (9, 64, 5) if kind == "hclt64" else (13, 16, 6)
+        # (category counts divisible by 4: the KL gradient of the rows also runs on the block kernels)
+        V, K, C = {"hclt64": (9, 64, 5), "hclt": (13, 16, 6), "hclt_c8": (13, 16, 8), "hclt32_c12": (21, 32, 12),
+                   "hclt64_c4": (7, 64, 4)}[kind]
         parent, theta, leaf, _ = make_hclt(V, K, C, 61)
         bpc = P.hclt_from_clt(parent, C, K)
         fc = O.bits_compile(O.hclt_dag(parent, K, C, theta, leaf), C, V)
