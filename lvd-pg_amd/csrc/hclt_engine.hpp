@@ -172,9 +172,7 @@ class HcltCircuit : public pcm_circuit {
   void kld_rows_block(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm, float* d_klds,
                       float* d_g1, float* d_g2);
   void gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
-                          float temperature, bool norm_params, float* d_out) override {
-    general_structure()->gumbel_sample_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params, d_out);
-  }
+                          float temperature, bool norm_params, float* d_out) override;
   void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                    float temperature, bool norm_params, bool grad_wrt_logparams, const float* d_out_grad,
                                    float* d_grads) override {

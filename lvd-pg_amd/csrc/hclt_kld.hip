@@ -133,6 +133,7 @@ __global__ __launch_bounds__(256) void hclt_kld_base_kernel(const HcltNode* __re
 // pair of chains per row, blockIdx.y); all zero for the circuit's own parameters.
 struct KlRowStrides {
   size_t pu, pd, vec, out, ring_up, ring_down;
+  int down_only;   // 1: the launch has one workgroup per row and it walks down (the relaxed sampler on rows)
 };
 
 // The two chains.  Workgroup 0 walks up (KL_v, Z_v), workgroup 1 walks down (h_v); launched
@@ -154,7 +155,7 @@ __global__ __launch_bounds__(kl_waves(K) * 64) void hclt_kld_chain_kernel(
   extern __shared__ float lds_ring[];   // kLds: [ring_mask + 1][K]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane % K, part = lane / K;
-  const bool up = blockIdx.x == 0;
+  const bool up = blockIdx.x == 0 && !rs.down_only;
   {   // a row of a parameter matrix per blockIdx.y: its operands, constants and results sit rs.* floats further on
     const size_t row = blockIdx.y;
     pu += row * rs.pu; pd += row * rs.pd; base += row * rs.vec; ell += row * rs.vec;
@@ -538,7 +539,7 @@ void HcltCircuit::kld_device(HcltCircuit* q, bool with_down) {
       hipLaunchKernelGGL(kernel, dim3(with_down ? 2 : 1), dim3(kl_waves(KK) * 64), lds, stream,
                          reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
                          reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
-                         kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, KlRowStrides{0, 0, 0, 0, 0, 0});
+                         kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, KlRowStrides{0, 0, 0, 0, 0, 0, 0});
     };
     if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
     else chain(&hclt_kld_chain_kernel<KK, false>, 0);
@@ -831,6 +832,7 @@ void HcltCircuit::kld_rows_block(const float* d_p1, const float* d_p2, int64_t s
   rs.out = nk;
   rs.ring_up = kl_ring_slots_ ? 0 : su * K_;
   rs.ring_down = kl_ring_slots_ ? 0 : sd * K_;
+  rs.down_only = 0;
   const size_t per_row = vk + 2 * rs.vec + rs.pu + rs.pd + 3 * nk + rs.ring_up + rs.ring_down;
   // rows at a time: what keeps the scratch arrays within 8 GB
   const int chunk = (int)std::max<size_t>(1, std::min<size_t>((size_t)rows, ((size_t)2 << 30) / per_row));
@@ -895,6 +897,145 @@ void HcltCircuit::kld_rows_block(const float* d_p1, const float* d_p2, int64_t s
     rows_unpack_out(g2, d_g2, sr, sp, rows, n, stream);
   }
   check_launch_k("hclt_kld_rows");
+}
+
+// ---- the relaxed sampler on parameter rows (`gumbel_sample(mbpc, params[R, n], ...)`, src/queries/sample.jl:338-383) ----
+// A sum node hands its top-down probability to its edges in shares softmax((logp + g) / T) over the node (sample.jl:37-51,
+// :105-140), a product passes it on, an input node adds td * its distribution to out[variable] (:262-284).  On the block
+// form that is the downward chain above with the softmax weights as operand: per (tree node, row) the K x K weights,
+// one chain per row, then per (variable, row) the mixture of the variable's K leaf distributions.
+
+// pd[sd]: operand (row k, column j) = softmax_j((theta[k,j] + g[k,j]) / T); noise in parameter order like the rows (null: none)
+template <int K>
+__global__ __launch_bounds__(256) void hclt_rows_soft_base_kernel(const int32_t* __restrict__ pos, int n_inner,
+                                                                  const int32_t* __restrict__ blk2par,
+                                                                  const float* __restrict__ P, size_t n_par,
+                                                                  const float* __restrict__ noise, size_t ns, float inv_t,
+                                                                  float* __restrict__ pd, KlRowStrides rs) {
+  __shared__ float tile[K][K + 1];
+  const int n = blockIdx.x, t = threadIdx.x;
+  const size_t row = blockIdx.y;
+  const size_t sd = (size_t)pos[n_inner + n];
+  const float* p = P + row * n_par;
+  const float* g = noise ? noise + row * ns : nullptr;
+  const int j = t % K;
+  for (int k = t / K; k < K; k += 256 / K) {
+    const int idx = blk2par[((size_t)n * K + k) * K + j];
+    float x = -INFINITY;
+    if (idx >= 0) x = (p[idx] + (g ? g[idx] : 0.f)) * inv_t;
+    float m = x;
+#pragma unroll
+    for (int o = K / 2; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, K));
+    const float e = x > -INFINITY ? expf(x - m) : 0.f;
+    float sum = e;
+#pragma unroll
+    for (int o = K / 2; o > 0; o >>= 1) sum += __shfl_xor(sum, o, K);
+    tile[k][j] = sum > 0.f ? e / sum : 0.f;
+  }
+  __syncthreads();
+  constexpr int JP = K * K / 64;
+  float* pdr = pd + row * rs.pd + sd * K * K;
+  for (int w = t; w < K * K; w += 256) {
+    const int e = w & 3, lane = (w >> 2) & 63, i4 = w >> 8;
+    const int rw = (lane / K) * JP + i4 * 4 + e, col = lane % K;
+    pdr[w] = tile[rw][col];
+  }
+}
+
+// out[row][v][c] = sum_j h[state node of v][j] * distribution of input node (v, j) at c
+template <bool kNorm>
+__global__ __launch_bounds__(256) void hclt_rows_soft_leaf_kernel(const float* __restrict__ P, size_t n_par, size_t ns, int C, int K,
+                                                                  int V, const int32_t* __restrict__ state_node,
+                                                                  const int32_t* __restrict__ in_pos, const float* __restrict__ h,
+                                                                  size_t nk, float* __restrict__ out) {
+  __shared__ float td[64];
+  __shared__ int at[64];
+  const int v = blockIdx.x;
+  const size_t row = blockIdx.y;
+  if ((int)threadIdx.x < K) {
+    td[threadIdx.x] = h[row * nk + (size_t)state_node[v] * K + threadIdx.x];
+    at[threadIdx.x] = in_pos[(size_t)v * K + threadIdx.x];
+  }
+  __syncthreads();
+  const float* p = P + row * n_par + ns;
+  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    float acc = 0.f;
+    for (int j0 = 0; j0 < K; j0 += 8) {   // eight rows requested before the first is used
+      float x[8];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) x[q] = p[(size_t)at[j0 + q] * C + c];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc += td[j0 + q] * (kNorm ? x[q] : expf(x[q]));
+    }
+    out[(row * V + v) * C + c] = acc;
+  }
+}
+
+void HcltCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                     float temperature, bool norm_params, float* d_out) {
+  if (!block_queries() || H_ > 0 || missing_)
+    return general_structure()->gumbel_sample_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params, d_out);
+  if (!d_params) fail(PCM_ERR_ARG, "parameter matrix is null");
+  if (rows < 1) fail(PCM_ERR_ARG, "need at least one parameter row, got %d", rows);
+  if (rows > 65535) fail(PCM_ERR_UNSUPPORTED, "at most 65535 parameter rows per call, got %d", rows);
+  if (sr == 0 || sp == 0) fail(PCM_ERR_ARG, "parameter matrix strides must not be zero");
+  if (!d_out) fail(PCM_ERR_ARG, "output pointer is null");
+  if (!(temperature > 0.f)) fail(PCM_ERR_ARG, "temperature must be positive");
+  build_kld_tables();
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  const int64_t n = size(0);
+  if (d_blk2par_.n == 0) {
+    std::vector<int32_t> b2p((size_t)n_inner_ * K_ * K_, -1);
+    for (int64_t i = 0; i < ns; ++i) b2p[(size_t)sum_param_src_[i]] = (int32_t)i;
+    d_blk2par_.upload(b2p, stream);
+  }
+  const float* p = rows_packed_in(d_params, sr, sp, rows, n, d_rows_pk1_, stream);
+  const int W = kl_waves(K_), D = kl_ahead(K_);
+  const size_t nk = (size_t)n_inner_ * K_;
+  const size_t su = (size_t)(kl_up_steps_ + D) * W, sd = (size_t)(kl_down_steps_ + D) * W, sm = std::max(su, sd);
+  KlRowStrides rs;
+  rs.pu = 0;               // (a chain that walks down reads no upward operand; the constants it requests are not used)
+  rs.pd = sd * K_ * K_;
+  rs.vec = sm * K_;
+  rs.out = nk;
+  rs.ring_up = 0;
+  rs.ring_down = kl_ring_slots_ ? 0 : sd * K_;
+  rs.down_only = 1;
+  const size_t per_row = rs.pd + rs.vec + nk + rs.ring_down;
+  const int chunk = (int)std::max<size_t>(1, std::min<size_t>((size_t)rows, ((size_t)2 << 30) / per_row));
+  d_rows_scratch_.ensure((size_t)chunk * per_row + su * K_ * K_);
+  float* pd = d_rows_scratch_.p;
+  float* vec = pd + (size_t)chunk * rs.pd;
+  float* h = vec + (size_t)chunk * rs.vec;
+  float* ring_down = kl_ring_slots_ ? nullptr : h + (size_t)chunk * nk;
+  float* pu = d_rows_scratch_.p + (size_t)chunk * per_row;   // never used, but named by the kernel's requests
+  const float inv_t = 1.f / temperature;
+  for (int r0 = 0; r0 < rows; r0 += chunk) {
+    const int rc = std::min(chunk, rows - r0);
+    const float* q = p + (size_t)r0 * n;
+    const float* g = d_noise ? d_noise + (size_t)r0 * ns : nullptr;
+    PCM_DISPATCH_K(K_, {
+      hipLaunchKernelGGL(hclt_rows_soft_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_kl_pos_.p, n_inner_,
+                         d_blk2par_.p, q, (size_t)n, g, (size_t)ns, inv_t, pd, rs);
+      auto chain = [&](auto kernel, size_t lds) {
+        hipLaunchKernelGGL(kernel, dim3(1, rc), dim3(kl_waves(KK) * 64), lds, stream,
+                           reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                           reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, vec, vec, pd,
+                           kl_ring_slots_ - 1, (float*)nullptr, ring_down, h, h, h, rs);
+      };
+      if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
+      else chain(&hclt_kld_chain_kernel<KK, false>, 0);
+    });
+    float* out = d_out + (size_t)r0 * Vu_ * C_;
+    const dim3 lgrid(Vu_, rc);
+    if (norm_params)
+      hipLaunchKernelGGL(hclt_rows_soft_leaf_kernel<true>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
+                         d_kl_tabs_.p + n_inner_, d_kl_tabs_.p + n_inner_ + V_, h, nk, out);
+    else
+      hipLaunchKernelGGL(hclt_rows_soft_leaf_kernel<false>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
+                         d_kl_tabs_.p + n_inner_, d_kl_tabs_.p + n_inner_ + V_, h, nk, out);
+  }
+  check_launch_k("hclt_gumbel_sample_rows");
 }
 
 static void check_rows_block_args(const void* p1, const void* p2, int64_t sr, int64_t sp, int rows) {
