@@ -214,6 +214,9 @@ def secondary(args):
         t_grad_rows = _timed(torch, lambda: P.kld_backward(p, m1, m2), max(1, args.steps // 4), 1)
         soft_rows = None
         t_soft_rows = _timed(torch, lambda: P.gumbel_sample_rows(p, m1, temperature=1.0), max(1, args.steps // 4), 1)
+        og = torch.randn((R, V, C), device="cuda", generator=gen)
+        t_soft_back_rows = _timed(torch, lambda: P.gumbel_sample_backward_rows(p, m1, og, temperature=1.0), max(1, args.steps // 4), 1)
+        del og
         rows_bytes = {"kld_rows": 2 * 4 * R * n_par, "kld_backward_rows": 5 * 4 * R * n_par}
         del m1, m2, klr
         dt = t_samp
@@ -224,7 +227,8 @@ def secondary(args):
                    queries_ms={"kld": t_kld * 1e3, "kld_backward_dev": t_grad * 1e3, "adam_step": t_adam * 1e3,
                                "sample": t_samp * 1e3, "gumbel_sample_relaxed_T0.5": t_soft * 1e3,
                                "kld_rows_R64": t_kld_rows * 1e3, "kld_backward_rows_R64": t_grad_rows * 1e3,
-                               "gumbel_sample_rows_R64_no_gumbel": t_soft_rows * 1e3},
+                               "gumbel_sample_rows_R64_no_gumbel": t_soft_rows * 1e3,
+                               "gumbel_sample_backward_rows_R64_no_gumbel": t_soft_back_rows * 1e3},
                    rows_gbs={"kld_rows_R64": rows_bytes["kld_rows"] / t_kld_rows / 1e9,
                              "kld_backward_rows_R64": rows_bytes["kld_backward_rows"] / t_grad_rows / 1e9})
     elif args.workload == "c4_patch_x8_streams":

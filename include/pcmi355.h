@@ -340,10 +340,9 @@ int pcm_sample_soft(pcm_circuit* c, const float* d_node_noise, float temperature
  * (:466-469).  Leaf parameters: with respect to the PROBABILITY of the category, whatever norm_params says, as
  * the source writes it (:560-570).
  * All of these queue their work on the circuit's stream and do not wait for it.  At most 65535 rows per call.
- * pcm_kld_rows, pcm_kld_backward_rows and pcm_gumbel_sample_rows of a single-root HCLT handle with block kernels (hidden
- * size 16, 32 or 64) run on the block form, the row as a grid dimension (fastest with 16-byte aligned matrices and a
- * category count divisible by 4: otherwise the KL gradient takes the per-layer kernels of the general form, which every
- * other circuit and pcm_gumbel_sample_backward_rows use).
+ * On a single-root HCLT handle with block kernels (hidden size 16, 32 or 64) the four of them run on the block form, the
+ * row as a grid dimension (fastest with 16-byte aligned matrices and a category count divisible by 4: otherwise the
+ * two gradients take the per-layer kernels of the general form, which every other circuit uses).
  */
 int pcm_kld_rows(pcm_circuit* c, const float* d_params1, const float* d_params2, int64_t stride_row, int64_t stride_param,
                  int32_t rows, int32_t norm_params, float* d_klds);

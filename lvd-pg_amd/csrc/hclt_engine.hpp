@@ -175,10 +175,7 @@ class HcltCircuit : public pcm_circuit {
                           float temperature, bool norm_params, float* d_out) override;
   void gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
                                    float temperature, bool norm_params, bool grad_wrt_logparams, const float* d_out_grad,
-                                   float* d_grads) override {
-    general_structure()->gumbel_sample_backward_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params,
-                                                     grad_wrt_logparams, d_out_grad, d_grads);
-  }
+                                   float* d_grads) override;
 
   // (both on the general form: the first with the circuit's own parameters, the second on the rows alone)
   void normalized_flows(const BatchRef& b, float* d_out, int64_t sr, int64_t sp, bool as_written) override {

@@ -911,11 +911,11 @@ __global__ __launch_bounds__(256) void hclt_rows_soft_base_kernel(const int32_t*
                                                                   const int32_t* __restrict__ blk2par,
                                                                   const float* __restrict__ P, size_t n_par,
                                                                   const float* __restrict__ noise, size_t ns, float inv_t,
-                                                                  float* __restrict__ pd, KlRowStrides rs) {
+                                                                  float* __restrict__ pd, float* __restrict__ pu, KlRowStrides rs) {
   __shared__ float tile[K][K + 1];
   const int n = blockIdx.x, t = threadIdx.x;
   const size_t row = blockIdx.y;
-  const size_t sd = (size_t)pos[n_inner + n];
+  const size_t sd = (size_t)pos[n_inner + n], su = (size_t)pos[n];
   const float* p = P + row * n_par;
   const float* g = noise ? noise + row * ns : nullptr;
   const int j = t % K;
@@ -935,10 +935,115 @@ __global__ __launch_bounds__(256) void hclt_rows_soft_base_kernel(const int32_t*
   __syncthreads();
   constexpr int JP = K * K / 64;
   float* pdr = pd + row * rs.pd + sd * K * K;
+  float* pur = pu ? pu + row * rs.pu + su * K * K : nullptr;   // (the reverse pass walks up with the same weights)
   for (int w = t; w < K * K; w += 256) {
     const int e = w & 3, lane = (w >> 2) & 63, i4 = w >> 8;
     const int rw = (lane / K) * JP + i4 * 4 + e, col = lane % K;
     pdr[w] = tile[rw][col];
+    if (pur) pur[w] = tile[col][rw];
+  }
+}
+
+// where entry (row rw, column col) of a K x K operand sits in its slot (the layout the chains read, see above)
+template <int K>
+__device__ __forceinline__ int kl_operand_word(int rw, int col) {
+  constexpr int JP = K * K / 64;
+  const int part = rw / JP, i = rw % JP;
+  return (((i >> 2) * 64) + part * K + col) * 4 + (i & 3);
+}
+
+// Reverse pass, input nodes (gumbel_input_sample_up_kernel, sample.jl:531-598): the gradient of a leaf parameter is
+// og[v][c] * td(v, j) -- per PROBABILITY of the category, with probability-valued parameters or not, as the source writes
+// it (:560-570) -- and the node's own gradient sum_c p(c) * og[v][c] goes to leaf_grad[row][v * K + j].  A wave per
+// input node and row, 16-byte accesses.
+template <bool kNorm>
+__global__ __launch_bounds__(256) void hclt_rows_soft_back_leaf_kernel(const float* __restrict__ P, size_t n_par, size_t ns, int C,
+                                                                       int K, int V, int n_inputs,
+                                                                       const int32_t* __restrict__ input_order,
+                                                                       const int32_t* __restrict__ state_node,
+                                                                       const float* __restrict__ h, size_t nk,
+                                                                       const float* __restrict__ og, size_t vk,
+                                                                       float* __restrict__ leaf_grad, float* __restrict__ G) {
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const size_t row = blockIdx.y;
+  if (i >= n_inputs) return;
+  const int vj = input_order[i], v = vj / K;
+  const float t = h[row * nk + (size_t)state_node[v] * K + vj % K];
+  const size_t at = row * n_par + ns + (size_t)i * C;
+  const float4* p = reinterpret_cast<const float4*>(P + at);
+  const float4* o = reinterpret_cast<const float4*>(og + (row * V + v) * C);
+  float4* g = reinterpret_cast<float4*>(G + at);
+  float acc = 0.f;
+  for (int c4 = lane; c4 < C / 4; c4 += 64) {
+    const float4 x = p[c4], oc = o[c4];
+    g[c4] = make_float4(oc.x * t, oc.y * t, oc.z * t, oc.w * t);
+    acc += kNorm ? (x.x * oc.x + x.y * oc.y) + (x.z * oc.z + x.w * oc.w)
+                 : (expf(x.x) * oc.x + expf(x.y) * oc.y) + (expf(x.z) * oc.z + expf(x.w) * oc.w);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+  if (lane == 0) leaf_grad[row * vk + vj] = acc;
+}
+
+// Reverse pass, what the upward chain starts from, per (tree node, row): ell[su][j] = the gradients of the leaves that
+// are factors of product j, base[su][k] = sum_j w[k,j] * ell[j] with the weights read back from the downward operand
+template <int K>
+__global__ __launch_bounds__(256) void hclt_rows_soft_base2_kernel(const HcltNode* __restrict__ nodes,
+                                                                   const int32_t* __restrict__ child_leaf,
+                                                                   const int32_t* __restrict__ pos, int n_inner,
+                                                                   const float* __restrict__ leaf_grad, size_t vk,
+                                                                   const float* __restrict__ pd, float* __restrict__ ell,
+                                                                   float* __restrict__ base, KlRowStrides rs) {
+  __shared__ float l[K];
+  const int n = blockIdx.x, t = threadIdx.x;
+  const size_t row = blockIdx.y;
+  const HcltNode nd = nodes[n];
+  const size_t su = (size_t)pos[n], sd = (size_t)pos[n_inner + n];
+  leaf_grad += row * vk;
+  ell += row * rs.vec;
+  base += row * rs.vec;
+  if (t < K) {
+    float s = leaf_grad[(size_t)nd.var * K + t];
+    for (int q = 0; q < nd.lc_cnt; ++q) s += leaf_grad[(size_t)child_leaf[nd.lc_off + q] * K + t];
+    l[t] = s;
+    ell[su * K + t] = s;
+  }
+  __syncthreads();
+  const float* w = pd + row * rs.pd + sd * K * K;
+  const int j = t % K;
+  for (int k = t / K; k < K; k += 256 / K) {
+    float term = w[kl_operand_word<K>(k, j)] * l[j];
+#pragma unroll
+    for (int o = K / 2; o > 0; o >>= 1) term += __shfl_xor(term, o, K);
+    if (j == 0) base[su * K + k] = term;
+  }
+}
+
+// Reverse pass, sum parameters (gumbel_params_up_layer_kernel, sample.jl:391-480): edge (k, j) of tree node n gets
+// td(S_n[k]) * (Z_n[j] - grad(S_n[k])) * w[k,j] / T, without the w when the gradient is wanted per probability (:466-469).
+template <int K>
+__global__ void hclt_rows_soft_edge_grad_kernel(int64_t ns, const int64_t* __restrict__ src, const int32_t* __restrict__ parent_of,
+                                                const int32_t* __restrict__ pos, int n_inner, const float* __restrict__ pd,
+                                                const float* __restrict__ z, const float* __restrict__ klv,
+                                                const float* __restrict__ h, size_t nk, KlRowStrides rs, float inv_t, int wrt_log,
+                                                int rows, size_t n_par, float* __restrict__ G) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= ns) return;
+  const int64_t s = src[i];
+  const int j = (int)(s % K), k = (int)((s / K) % K);
+  const int n = (int)(s / ((int64_t)K * K));
+  const int par = parent_of[n];
+  const size_t wat = (size_t)pos[n_inner + n] * K * K + kl_operand_word<K>(k, j);
+  const size_t zat = (size_t)n * K + j, kat = (size_t)n * K + k, hat = par < 0 ? 0 : (size_t)par * K + k;
+  const int r0 = blockIdx.y * kEdgeGradRows;
+#pragma unroll
+  for (int q = 0; q < kEdgeGradRows; ++q) {
+    if (r0 + q >= rows) break;
+    const size_t row = (size_t)(r0 + q);
+    const float t = par < 0 ? 1.f : h[row * nk + hat];
+    const float w = wrt_log ? pd[row * rs.pd + wat] : 1.f;
+    G[row * n_par + i] = t * (z[row * nk + zat] - klv[row * nk + kat]) * w * inv_t;
   }
 }
 
@@ -1016,7 +1121,7 @@ void HcltCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_t 
     const float* g = d_noise ? d_noise + (size_t)r0 * ns : nullptr;
     PCM_DISPATCH_K(K_, {
       hipLaunchKernelGGL(hclt_rows_soft_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_kl_pos_.p, n_inner_,
-                         d_blk2par_.p, q, (size_t)n, g, (size_t)ns, inv_t, pd, rs);
+                         d_blk2par_.p, q, (size_t)n, g, (size_t)ns, inv_t, pd, (float*)nullptr, rs);
       auto chain = [&](auto kernel, size_t lds) {
         hipLaunchKernelGGL(kernel, dim3(1, rc), dim3(kl_waves(KK) * 64), lds, stream,
                            reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
@@ -1036,6 +1141,104 @@ void HcltCircuit::gumbel_sample_rows(const float* d_params, int64_t sr, int64_t 
                          d_kl_tabs_.p + n_inner_, d_kl_tabs_.p + n_inner_ + V_, h, nk, out);
   }
   check_launch_k("hclt_gumbel_sample_rows");
+}
+
+void HcltCircuit::gumbel_sample_backward_rows(const float* d_params, int64_t sr, int64_t sp, int32_t rows, const float* d_noise,
+                                              float temperature, bool norm_params, bool grad_wrt_logparams,
+                                              const float* d_out_grad, float* d_grads) {
+  const int64_t ns = (int64_t)sum_param_src_.size();
+  const int64_t n = size(0);
+  const bool direct = sp == 1 && sr == n;
+  // 16-byte rows on every side: the leaf kernel moves four categories at a time
+  const bool aligned = C_ % 4 == 0 && n % 4 == 0 && ns % 4 == 0 && (reinterpret_cast<uintptr_t>(d_out_grad) & 15) == 0 &&
+                       (!direct || ((reinterpret_cast<uintptr_t>(d_params) | reinterpret_cast<uintptr_t>(d_grads)) & 15) == 0);
+  if (!block_queries() || H_ > 0 || missing_ || !aligned)
+    return general_structure()->gumbel_sample_backward_rows(d_params, sr, sp, rows, d_noise, temperature, norm_params,
+                                                            grad_wrt_logparams, d_out_grad, d_grads);
+  if (!d_params) fail(PCM_ERR_ARG, "parameter matrix is null");
+  if (rows < 1) fail(PCM_ERR_ARG, "need at least one parameter row, got %d", rows);
+  if (rows > 65535) fail(PCM_ERR_UNSUPPORTED, "at most 65535 parameter rows per call, got %d", rows);
+  if (sr == 0 || sp == 0) fail(PCM_ERR_ARG, "parameter matrix strides must not be zero");
+  if (!d_out_grad || !d_grads) fail(PCM_ERR_ARG, "gradient pointer is null");
+  if (!(temperature > 0.f)) fail(PCM_ERR_ARG, "temperature must be positive");
+  build_kld_tables();
+  if (d_blk2par_.n == 0) {
+    std::vector<int32_t> b2p((size_t)n_inner_ * K_ * K_, -1);
+    for (int64_t i = 0; i < ns; ++i) b2p[(size_t)sum_param_src_[i]] = (int32_t)i;
+    d_blk2par_.upload(b2p, stream);
+  }
+  if (d_input_order_.n == 0) d_input_order_.upload(input_order_, stream);
+  const float* p = rows_packed_in(d_params, sr, sp, rows, n, d_rows_pk1_, stream);
+  float* gout = d_grads;
+  if (!direct) {
+    d_rows_pg1_.ensure((size_t)rows * n);
+    gout = d_rows_pg1_.p;
+  }
+  const int W = kl_waves(K_), D = kl_ahead(K_);
+  const size_t nk = (size_t)n_inner_ * K_, vk = (size_t)V_ * K_;
+  const size_t su = (size_t)(kl_up_steps_ + D) * W, sd = (size_t)(kl_down_steps_ + D) * W, sm = std::max(su, sd);
+  KlRowStrides rs;
+  rs.pu = su * K_ * K_;
+  rs.pd = sd * K_ * K_;
+  rs.vec = sm * K_;
+  rs.out = nk;
+  rs.ring_up = kl_ring_slots_ ? 0 : su * K_;
+  rs.ring_down = kl_ring_slots_ ? 0 : sd * K_;
+  rs.down_only = 0;
+  const size_t per_row = rs.pu + rs.pd + 2 * rs.vec + 3 * nk + vk + rs.ring_up + rs.ring_down;
+  const int chunk = (int)std::max<size_t>(1, std::min<size_t>((size_t)rows, ((size_t)2 << 30) / per_row));
+  d_rows_scratch_.ensure((size_t)chunk * per_row);
+  float* pd = d_rows_scratch_.p;
+  float* pu = pd + (size_t)chunk * rs.pd;
+  float* ell = pu + (size_t)chunk * rs.pu;
+  float* base = ell + (size_t)chunk * rs.vec;
+  float* h = base + (size_t)chunk * rs.vec;
+  float* klv = h + (size_t)chunk * nk;
+  float* z = klv + (size_t)chunk * nk;
+  float* leaf_grad = z + (size_t)chunk * nk;
+  float* ring_up = kl_ring_slots_ ? nullptr : leaf_grad + (size_t)chunk * vk;
+  float* ring_down = kl_ring_slots_ ? nullptr : ring_up + (size_t)chunk * rs.ring_up;
+  const float inv_t = 1.f / temperature;
+  const int n_inputs = (int)input_order_.size();
+  for (int r0 = 0; r0 < rows; r0 += chunk) {
+    const int rc = std::min(chunk, rows - r0);
+    const float* q = p + (size_t)r0 * n;
+    const float* g = d_noise ? d_noise + (size_t)r0 * ns : nullptr;
+    const float* og = d_out_grad + (size_t)r0 * Vu_ * C_;
+    float* out = gout + (size_t)r0 * n;
+    PCM_DISPATCH_K(K_, {
+      auto chain = [&](int down_only) {
+        KlRowStrides r2 = rs;
+        r2.down_only = down_only;
+        auto launch = [&](auto kernel, size_t lds) {
+          hipLaunchKernelGGL(kernel, dim3(1, rc), dim3(kl_waves(KK) * 64), lds, stream,
+                             reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                             reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
+                             kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, r2);
+        };
+        if (kl_ring_slots_) launch(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
+        else launch(&hclt_kld_chain_kernel<KK, false>, 0);
+      };
+      hipLaunchKernelGGL(hclt_rows_soft_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_kl_pos_.p, n_inner_,
+                         d_blk2par_.p, q, (size_t)n, g, (size_t)ns, inv_t, pd, pu, rs);
+      chain(1);   // the top-down probabilities
+      const dim3 lgrid(ceil_div(n_inputs, 4), rc);
+      if (norm_params)
+        hipLaunchKernelGGL(hclt_rows_soft_back_leaf_kernel<true>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
+                           n_inputs, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, og, vk, leaf_grad, out);
+      else
+        hipLaunchKernelGGL(hclt_rows_soft_back_leaf_kernel<false>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
+                           n_inputs, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, og, vk, leaf_grad, out);
+      hipLaunchKernelGGL(hclt_rows_soft_base2_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
+                         d_kl_pos_.p, n_inner_, leaf_grad, vk, pd, ell, base, rs);
+      chain(0);   // the gradients of the sum nodes, bottom-up
+      hipLaunchKernelGGL(hclt_rows_soft_edge_grad_kernel<KK>, dim3((unsigned)ceil_div(ns, 256), ceil_div(rc, kEdgeGradRows)),
+                         dim3(256), 0, stream, ns, d_sum_param_src_.p, d_kl_tabs_.p, d_kl_pos_.p, n_inner_, pd, z, klv, h, nk, rs,
+                         inv_t, grad_wrt_logparams ? 1 : 0, rc, (size_t)n, out);
+    });
+  }
+  if (!direct) rows_unpack_out(gout, d_grads, sr, sp, rows, n, stream);
+  check_launch_k("hclt_gumbel_sample_backward_rows");
 }
 
 static void check_rows_block_args(const void* p1, const void* p2, int64_t sr, int64_t sp, int rows) {
