@@ -670,3 +670,56 @@ def test_em_then_adam_raises_the_likelihood(gpu):
     assert lls[-1] > lls[0] and lls[-1] > em[-1]
     final = float(P.loglikelihoods(bpc, d).mean().item())
     assert final > em[-1]
+
+
+@pytest.mark.parametrize("shape", ["random", "wide_levels"])
+def test_row_queries_on_the_block_form_agree_with_the_layer_kernels(gpu, oracle, shape):
+    """The four row queries of an HCLT handle (block form, the row as a grid dimension) against the same circuit
+    compiled from its DAG (per-layer kernels of the general form; same parameter order): a random tree with up to five
+    children per node, and a complete binary tree of twelve levels, whose widest level (1024 tree nodes) no longer
+    fits the chains' ring of vectors in LDS -- the ring is then in device memory, one per row."""
+    torch, P = gpu
+    O = oracle
+    from helpers import make_hclt, log_dirichlet
+    rng = np.random.default_rng(77)
+    if shape == "random":
+        V, K, C, R = 57, 32, 12, 9
+        parent, theta, leaf, _ = make_hclt(V, K, C, 78, max_children=5)
+    else:
+        V, K, C, R = 4095, 16, 4, 3
+        parent = np.array([-1] + [(v - 1) // 2 for v in range(1, V)], np.int32)
+        parent, theta, leaf, _ = make_hclt(V, K, C, 79, parent=parent)
+    blk = P.hclt_from_clt(parent, C, K)
+    gen = _compile(P, O.hclt_dag(parent, K, C, theta, leaf), V, C)
+    n, ns = blk.num_parameters(), blk.num_inner_params()
+    assert n == gen.num_parameters() and np.array_equal(blk.table("param2edge"), gen.table("param2edge"))
+    sizes = blk.table("pargroup_sizes")
+
+    def draw(norm):
+        rows = np.empty((R, n), np.float32)
+        for r in range(R):
+            pos = 0
+            for sz in sizes:
+                rows[r, pos:pos + sz] = log_dirichlet(rng, sz) if sz > 1 else 0.0
+                pos += sz
+            lf = np.exp(np.stack([log_dirichlet(rng, C) for _ in range((n - ns) // C)]))
+            rows[r, ns:] = (lf if norm else np.log(lf)).reshape(-1)
+        return torch.from_numpy(rows).cuda()
+
+    def close(a, b, what):
+        a, b = a.cpu().numpy(), b.cpu().numpy()
+        assert np.abs(a - b).max() < 1e-4 * np.abs(b).max(), what
+
+    for norm in (False, True):
+        p1, p2 = draw(norm), draw(norm)
+        noise = torch.from_numpy(_gumbel(rng, (R, ns))).cuda()
+        G = torch.from_numpy(rng.normal(size=(R, V, C)).astype(np.float32)).cuda()
+        close(P.kld(blk, p1, p2, norm_params=norm), P.kld(gen, p1, p2, norm_params=norm), "kld")
+        a, b = P.kld_backward(blk, p1, p2, norm_params=norm), P.kld_backward(gen, p1, p2, norm_params=norm)
+        close(a[0], b[0], "kld gradient 1")
+        close(a[1], b[1], "kld gradient 2")
+        kw = dict(temperature=0.7, noise=noise, norm_params=norm)
+        close(P.gumbel_sample_rows(blk, p1, **kw), P.gumbel_sample_rows(gen, p1, **kw), "relaxed samples")
+        for wrt_log in (True, False):
+            close(P.gumbel_sample_backward_rows(blk, p1, G, grad_wrt_logparams=wrt_log, **kw),
+                  P.gumbel_sample_backward_rows(gen, p1, G, grad_wrt_logparams=wrt_log, **kw), "reverse pass")
