@@ -437,6 +437,8 @@ def secondary(args):
                        "unit": "GB/s", "frac": ach / HBM_PEAK_GBS, "traffic": None}
     if note:
         out["roofline"]["note"] = note
+        if note is REQUESTED_NOTE:   # a count of requests, most of them served by caches: no fraction of the HBM rate
+            out["roofline"]["frac"] = None
     print(json.dumps(out))
 
 

@@ -176,7 +176,10 @@ int pcm_set_stream(pcm_circuit* c, void* hip_stream);
  * the handle is a forest), 16 dense groups of a pcm_circuit_create circuit: sets of sum nodes of one layer with one
  * and the same list of children, which run as blocks on the matrix cores instead of edge by edge (0 for an HCLT
  * handle, and for every circuit created while PCMI355_DENSE_GROUPS=0 is in the environment: a switch for comparisons,
- * results agree to rounding), 17 nodes whose values the per-layer kernels compute (the others are the groups'). */
+ * results agree to rounding), 17 nodes whose values the per-layer kernels compute (the others are the groups'), 18 layers
+ * of groups that go inside walk launches: runs of consecutive layers that hold groups of one shape and nothing else take
+ * one launch per direction where their groups are few (PCMI355_GROUP_WALK=0 at creation: a launch per layer, the same
+ * bits). */
 int64_t pcm_size(const pcm_circuit* c, int32_t what);
 
 /* Index tables of src/bits_circuit.jl:9-36, 1-based as the reference holds them.

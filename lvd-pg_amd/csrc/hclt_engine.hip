@@ -961,6 +961,7 @@ int64_t HcltCircuit::size(int what) const {
     case 15: return T_;
     case 16: return 0;
     case 17: return 0;
+    case 18: return 0;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }

@@ -1272,6 +1272,7 @@ void SparseCircuit::build_groups(std::vector<int32_t>& group_of, std::vector<int
   g.rec = reinterpret_cast<const GroupRec*>(d_grp_rec_.p);                                                           \
   g.node = d_grp_node_.p; g.edge = d_grp_edge_.p;   g.rows = d_grp_rows_.p; g.own = d_grp_own_.p;                    \
   g.copies = d_grp_copies_.p; g.order = d_grp_order_.p; g.wf = d_grp_wf_.p; g.wb = d_grp_wb_.p; g.m = d_grp_m_.p;       \
+  g.xm = d_grp_xm_.p;                                                                                                \
   g.logp = d_logp_.p; g.mars = d_mars_.p; g.flows = d_flows_.p; g.edge_part = d_edge_part_.p;                        \
   g.n_nodes = fc_.n_nodes(); g.n_edges = fc_.n_edges(); g.B = batch_; g.Bp = bp_;                                   \
   g.inv_f = 1.f; g.norm = d_mars_.p; g.norm_row = fc_.n_nodes()   /* (not tempered: the row of zeros for every sum) */
@@ -1283,6 +1284,88 @@ void SparseCircuit::refresh_group_w(float inv_f) {
   g.inv_f = inv_f;
   hipLaunchKernelGGL(sparse_group_w_kernel, dim3((unsigned)ceil_div(n_group_elems_, 256)), dim3(256), 0, stream, g, d_grp_elem_.p,
                      n_group_elems_);
+}
+
+// Runs of consecutive layers that hold groups of one shape and no node of the layer kernels: one walk launch each
+// (sparse_group_walk_kernel) instead of a launch per layer, where a layer's groups are few.  Going up and going down have
+// runs of their own: a node the layer kernels compute going up may take its flow from a group's kernel going down.
+// PCMI355_GROUP_WALK=0 in the environment when the circuit is created keeps the launch per layer (for comparisons).
+void SparseCircuit::build_group_runs() {
+  group_runs_fwd_.clear();
+  group_runs_bwd_.clear();
+  n_walk_levels_ = 0;
+  const char* env = std::getenv("PCMI355_GROUP_WALK");
+  if (group_launches_.empty() || (env && env[0] == '0')) return;
+  std::vector<int2> levels;
+  auto collect = [&](const std::vector<int>& layer0, std::vector<GroupRun>& runs) {
+    // per layer: the one launch of its groups (-1: none, -2: several shapes)
+    std::vector<int> of_layer(n_layers_, -1);
+    for (size_t i = 0; i < group_launches_.size(); ++i) {
+      int& slot = of_layer[group_launches_[i].layer];
+      slot = slot == -1 ? (int)i : -2;
+    }
+    GroupRun cur{};
+    bool open = false;
+    auto close = [&]() {
+      if (open && cur.n_levels >= 2) runs.push_back(cur);
+      open = false;
+    };
+    for (int l = 0; l < n_layers_; ++l) {
+      const bool plain_nodes = layer0[l + 1] - layer0[l] > 0;
+      if (plain_nodes || of_layer[l] == -2) { close(); continue; }
+      if (of_layer[l] == -1) continue;   // (an empty layer: nothing to launch, nothing to wait for)
+      const GroupLaunch& L = group_launches_[of_layer[l]];
+      const bool shape_walks = L.gt == L.ct && (L.gt == 1 || L.gt == 2 || L.gt == 4);   // the shapes the walk kernels are built for
+      if (!shape_walks) { close(); continue; }
+      if (open && (cur.gt != L.gt || cur.ct != L.ct || cur.group0 + cur.n_groups != L.group0)) close();
+      if (!open) {
+        cur = GroupRun{l, l, L.gt, L.ct, L.group0, 0, L.pnode0, L.pslot0, L.pw0, (int)levels.size(), 0, 0};
+        open = true;
+      }
+      levels.push_back(int2{L.group0 - cur.group0, L.count});
+      cur.layer_last = l;
+      cur.n_groups += L.count;
+      cur.n_levels++;
+      cur.max_count = std::max(cur.max_count, L.count);
+    }
+    close();
+  };
+  collect(fwd_layer0_, group_runs_fwd_);
+  collect(bwd_layer0_, group_runs_bwd_);
+  // the walk going down takes a run's layers from the last to the first
+  for (GroupRun& r : group_runs_bwd_) std::reverse(levels.begin() + r.level0, levels.begin() + r.level0 + r.n_levels);
+  for (const GroupRun& r : group_runs_fwd_) n_walk_levels_ += r.n_levels;
+  if (!levels.empty()) d_grp_levels_.upload(levels);
+}
+
+// a run goes as one walk launch if its layers' groups are few: each slice of 16 examples is one workgroup whose waves
+// share a layer's groups, so a layer of many groups is better off spread over the device by a launch of its own
+static bool run_walks(int max_count, int Bp) {
+  return max_count <= 32 && (int64_t)max_count * (Bp / 16) <= 4096;
+}
+
+bool SparseCircuit::launch_group_walk(const GroupRun& r, bool forward, int Bp, int batch, bool tempered) {
+  if (!run_walks(r.max_count, Bp)) return false;
+  PCM_GROUP_DEV(g, batch, Bp);
+  if (tempered) { g.inv_f = 1.f / flow_scale; g.norm = d_norm_.p; g.norm_row = -1; }
+  GroupWalk w;
+  w.levels = d_grp_levels_.p + r.level0;
+  w.n_levels = r.n_levels;
+  w.base = GroupBase{r.group0, r.pnode0, r.pslot0, r.pw0};
+  const dim3 grid(Bp / 16);
+  // waves per workgroup: as many as the kernel's registers allow (going down a 32 x 32 group takes 128 and more)
+#define PCM_WALK(GT_, WVF_, WVB_)                                                                                              \
+  do {                                                                                                                         \
+    if (forward) hipLaunchKernelGGL((sparse_group_walk_kernel<GT_, GT_, WVF_, true>), grid, dim3(WVF_ * 64), 0, stream, g, w);  \
+    else hipLaunchKernelGGL((sparse_group_walk_kernel<GT_, GT_, WVB_, false>), grid, dim3(WVB_ * 64), 0, stream, g, w);         \
+  } while (0)
+  switch (r.gt) {
+    case 1: PCM_WALK(1, 16, 16); break;
+    case 2: PCM_WALK(2, 16, 8); break;
+    default: PCM_WALK(4, 4, 4); break;
+  }
+#undef PCM_WALK
+  return true;
 }
 
 // the group kernels of one layer: what = 0 values going up, 1 the children's rows going down; what = 2: the edge
@@ -1506,6 +1589,7 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
     d_bwd_rec_.upload(br);
     d_bwd_alias_.upload(ar);
   }
+  build_group_runs();
   // normalisation groups over the sum parameters
   std::vector<int32_t> gp(1, 0), p2e;
   for (int64_t s : fc_.pargroup_sizes) gp.push_back(gp.back() + (int32_t)s);
@@ -1535,6 +1619,7 @@ int64_t SparseCircuit::size(int what) const {
     case 15: return 1;
     case 16: return n_groups_;
     case 17: return n_layer_nodes_;
+    case 18: return n_walk_levels_;
     default: fail(PCM_ERR_ARG, "unknown size selector %d", what);
   }
 }
@@ -1668,9 +1753,19 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
                        d_var_nodes_.p);
   }
   refresh_group_w();
-  if (n_groups_) d_grp_m_.ensure((size_t)n_groups_ * Bp);
+  if (n_groups_) {
+    d_grp_m_.ensure((size_t)n_groups_ * Bp);
+    d_grp_xm_.ensure(d_grp_rows_.n * (size_t)Bp);
+  }
+  size_t next_run = 0;
   for (int l = 0; l < n_layers_; ++l) {
     const int n0 = fwd_layer0_[l], cnt = fwd_layer0_[l + 1] - n0;
+    while (next_run < group_runs_fwd_.size() && group_runs_fwd_[next_run].layer_first < l) ++next_run;
+    if (next_run < group_runs_fwd_.size() && group_runs_fwd_[next_run].layer_first == l &&
+        launch_group_walk(group_runs_fwd_[next_run], true, Bp, batch, false)) {
+      l = group_runs_fwd_[next_run].layer_last;   // the run's layers hold nothing but these groups
+      continue;
+    }
     launch_groups(l, 0, Bp, batch);
     if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
@@ -1768,7 +1863,14 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
     hipLaunchKernelGGL(sparse_scale_kernel, dim3(ceil_div((int64_t)n_parts * ne, 256)), dim3(256), 0, stream, d_edge_part_.p,
                        (int64_t)n_parts * ne, 0.f);
   }
+  int next_run = (int)group_runs_bwd_.size() - 1;
   for (int l = n_layers_ - 1; l >= 0; --l) {
+    while (next_run >= 0 && group_runs_bwd_[next_run].layer_last > l) --next_run;
+    if (next_run >= 0 && group_runs_bwd_[next_run].layer_last == l &&
+        launch_group_walk(group_runs_bwd_[next_run], false, Bp, batch, tempered)) {
+      l = group_runs_bwd_[next_run].layer_first;   // (the loop's --l moves on below the run)
+      continue;
+    }
     const int n0 = bwd_layer0_[l], cnt = bwd_layer0_[l + 1] - n0;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
 #define PCM_BWD_ARGS db, n0, d_head_mask, d_edge_part_.p, ne, d_alias_list_.p

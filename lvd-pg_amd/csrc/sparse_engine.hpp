@@ -124,13 +124,20 @@ class SparseCircuit : public pcm_circuit {
   // dense groups (sparse_groups.hip.hpp): sum nodes of a layer that share one list of children
   struct GroupLaunch { int layer, group0, count, gt, ct; int32_t pnode0, pslot0; int64_t pw0; };
   std::vector<GroupLaunch> group_launches_;   // per (layer, shape), sorted by layer: ranges of groups
+  // runs of layers of groups that go as one walk launch (sparse_group_walk_kernel); level0: the run's layers in d_grp_levels_
+  struct GroupRun { int layer_first, layer_last, gt, ct, group0, n_groups; int32_t pnode0, pslot0; int64_t pw0; int level0, n_levels, max_count; };
+  std::vector<GroupRun> group_runs_fwd_, group_runs_bwd_;
+  DevBuf<int2> d_grp_levels_;
+  int64_t n_walk_levels_ = 0;                 // layers of groups inside forward runs
+  void build_group_runs();
+  bool launch_group_walk(const GroupRun& r, bool forward, int Bp, int batch, bool tempered);
   std::vector<GroupLaunch> group_stat_launches_;   // per shape: ranges of d_grp_order_ (layer and bases unused)
   std::vector<int> fwd_layer0_;               // ranges of d_fwd_rec_ per layer: the nodes no group computes
   int64_t n_layer_nodes_ = 0;                 // nodes whose values the layer kernels compute (the others: the groups')
   int64_t n_group_slots_ = 0, n_groups_ = 0, n_group_elems_ = 0;   // children of all groups; groups; padded W entries
   DevBuf<int32_t> d_grp_node_, d_grp_edge_, d_grp_own_, d_grp_elem_, d_grp_order_;
   DevBuf<int4> d_grp_rec_, d_grp_rows_, d_grp_copies_;   // (a group's record is two int4)
-  DevBuf<float> d_grp_wf_, d_grp_wb_, d_grp_m_;
+  DevBuf<float> d_grp_wf_, d_grp_wb_, d_grp_m_, d_grp_xm_;
   DevBuf<float> d_norm_;                      // tempered flows: [n_nodes + 1][Bp], see sparse_tempered_norm_kernel
   DevBuf<int2> d_grp_product_edges_;          // {edge, parent}: product edges into nodes a group's kernel writes
   int n_group_product_edges_ = 0;

@@ -55,6 +55,7 @@ struct GroupDev {
   const float* wf;        // W in the order the forward kernel's lanes take it: [gt][q][lane] = W[16 gt + lo][4 q + hi]
   const float* wb;        // ... and the backward kernel's: [ct][k][lane] = W[4 k + hi][16 ct + lo]
   float* m;               // [groups][Bp]: the maximum the forward kernel took out, per example
+  float* xm;              // [child entries][Bp]: X - m as the forward kernel formed it (-inf: an impossible child), for the way down
   const float* logp;
   float* mars;
   float* flows;           // [n_nodes + slots][Bp]
@@ -128,12 +129,12 @@ __device__ __forceinline__ float group_max4(float v) {
 // before anything of it is used and no branch around a load: a layer's launch lasts as long as its longest chain of
 // requests.  The maximum goes to d.m for the backward kernels.
 template <int GT, int CT>
-__global__ __launch_bounds__(64) void sparse_group_forward_kernel(GroupDev d, GroupBase base) {
+__device__ __forceinline__ void group_forward_body(const GroupDev& d, const GroupBase& base, int bx, int lane, int slice) {
   constexpr int NK = CT * 4, Gp = GT * 16, Cp = CT * 16;
   constexpr bool kPre = GT * NK <= 64;   // W in registers before the rows arrive
-  const int bx = blockIdx.x, group = base.group0 + bx;
-  const int lane = threadIdx.x, lo = lane & 15, hi = lane >> 4;
-  const int64_t col = (int64_t)blockIdx.y * 16 + lo;
+  const int group = base.group0 + bx;
+  const int lo = lane & 15, hi = lane >> 4;
+  const int64_t col = (int64_t)slice * 16 + lo;
   const int4* rows = d.rows + base.pslot0 + (int64_t)bx * Cp;
   const int32_t* owns = d.own + base.pslot0 + (int64_t)bx * Cp;
   const int32_t* node = d.node + base.pnode0 + (int64_t)bx * Gp;
@@ -149,11 +150,9 @@ __global__ __launch_bounds__(64) void sparse_group_forward_kernel(GroupDev d, Gr
 #pragma unroll
       for (int q = 0; q < NK; ++q) a[gt][q] = wg[(gt * NK + q) * 64];
   }
-  int nd[GT][4];
+  int4 nd4[GT];   // (the four sums of a lane's output rows are neighbours in the table: one request per tile)
 #pragma unroll
-  for (int gt = 0; gt < GT; ++gt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) nd[gt][i] = node[gt * 16 + 4 * hi + i];
+  for (int gt = 0; gt < GT; ++gt) nd4[gt] = *reinterpret_cast<const int4*>(node + gt * 16 + 4 * hi);
   float x[NK], pv[NK];
 #pragma unroll
   for (int q = 0; q < NK; ++q) {
@@ -167,10 +166,13 @@ __global__ __launch_bounds__(64) void sparse_group_forward_kernel(GroupDev d, Gr
   for (int q = 1; q < NK; ++q) mx = fmaxf(mx, x[q]);
   mx = group_max4(mx);
   if (!(mx > -INFINITY)) mx = 0.f;   // every child impossible: E = 0, the sums come out as -inf
+  float* xm = d.xm + (base.pslot0 + (int64_t)bx * Cp) * d.Bp + col;
 #pragma unroll
   for (int q = 0; q < NK; ++q) {
     if (own[q] >= 0) d.mars[(int64_t)own[q] * d.Bp + col] = pv[q];
-    x[q] = x[q] > -INFINITY ? __expf(x[q] - mx) : 0.f;
+    const float xs = x[q] - mx;   // (-inf stays -inf)
+    xm[(int64_t)(4 * q + hi) * d.Bp] = xs;
+    x[q] = x[q] > -INFINITY ? __expf(xs) : 0.f;
   }
   if (hi == 0) d.m[(int64_t)group * d.Bp + col] = mx;
 #pragma unroll
@@ -183,24 +185,30 @@ __global__ __launch_bounds__(64) void sparse_group_forward_kernel(GroupDev d, Gr
       else av = wg[(gt * NK + q) * 64];
       acc = __builtin_amdgcn_mfma_f32_16x16x4f32(av, x[q], acc, 0, 0, 0);
     }
+    const int nd[4] = {nd4[gt].x, nd4[gt].y, nd4[gt].z, nd4[gt].w};
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (nd[gt][i] >= 0) d.mars[(int64_t)nd[gt][i] * d.Bp + col] = mx + __logf(acc[i]);
+      if (nd[i] >= 0) d.mars[(int64_t)nd[i] * d.Bp + col] = mx + __logf(acc[i]);
   }
+}
+
+template <int GT, int CT>
+__global__ __launch_bounds__(64) void sparse_group_forward_kernel(GroupDev d, GroupBase base) {
+  group_forward_body<GT, CT>(d, base, blockIdx.x, threadIdx.x, blockIdx.y);
 }
 
 // Backward, per layer: the rows the group hands its children, E[c] * sum_g W[g,c] R[g].  One wave per (group, 16
 // examples) as going up: R of the sums g = 4 k + hi is the B operand of k-step k as it is loaded.  The same two
 // rounds of requests where the registers hold a group's W and row numbers (kPre); 16 children at a time otherwise.
 template <int GT, int CT>
-__global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, GroupBase base) {
+__device__ __forceinline__ void group_backward_body(const GroupDev& d, const GroupBase& base, int bx, int lane, int slice) {
   constexpr int NG = GT * 4, Gp = GT * 16, Cp = CT * 16;
   constexpr bool kPre = CT <= 2 && GT * CT <= 16;
   constexpr int CL = kPre ? CT : 1;
-  const int bx = blockIdx.x, group = base.group0 + bx;
-  const int lane = threadIdx.x, lo = lane & 15, hi = lane >> 4;
-  const int64_t col = (int64_t)blockIdx.y * 16 + lo;
-  const int4* rows = d.rows + base.pslot0 + (int64_t)bx * Cp;
+  const int group = base.group0 + bx;
+  const int lo = lane & 15, hi = lane >> 4;
+  const int64_t col = (int64_t)slice * 16 + lo;
+  const float* xm = d.xm + (base.pslot0 + (int64_t)bx * Cp) * d.Bp + col;
   const int4* copies = d.copies + 2 * (base.pslot0 + (int64_t)bx * Cp);
   const int32_t* node = d.node + base.pnode0 + (int64_t)bx * Gp;
   const float* wg = d.wb + base.pw0 + (int64_t)bx * Gp * Cp + lane;
@@ -208,52 +216,59 @@ __global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, G
   int nd[NG];
 #pragma unroll
   for (int k = 0; k < NG; ++k) nd[k] = node[4 * k + hi];
-  int4 rw[CL][4], cpa[CL][4], cpb[CL][4];
+  int4 cpa[CL][4], cpb[CL][4];
   float a[CL][NG], e[CL][4];
   auto numbers = [&](int ct, int s) {   // row numbers and W for the children 16 ct + 4 hi + i
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int c = ct * 16 + 4 * hi + i;
-      rw[s][i] = rows[c];
       cpa[s][i] = copies[2 * c];
       cpb[s][i] = copies[2 * c + 1];
     }
 #pragma unroll
     for (int k = 0; k < NG; ++k) a[s][k] = wg[(ct * NG + k) * 64];
   };
-  auto values = [&](int s) {   // (a child that is not there: W = 0 and no row to write, whatever E comes out as)
+  auto values = [&](int ct, int s) {   // X - m as the forward kernel left it (a child that is not there: -inf)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float xv = group_x(d, rw[s][i], col);
-      e[s][i] = xv > -INFINITY ? __expf((xv - mb) * d.inv_f) : 0.f;
-    }
+    for (int i = 0; i < 4; ++i) e[s][i] = xm[(int64_t)(ct * 16 + 4 * hi + i) * d.Bp];
   };
   if constexpr (kPre) {
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) numbers(ct, ct);
   }
   float rv[NG];
+  {   // R = F / S = F * exp(m - value): no flow stays no flow where the value is -inf.  (All rows requested, then used:
+      // written as one loop the compiler waits for every sum's rows in turn.)
+    float f[NG], v[NG], nv[NG];
 #pragma unroll
-  for (int k = 0; k < NG; ++k) {   // R = F / S = F * exp(m - value): no flow stays no flow where the value is -inf
-    const int64_t n = nd[k] < 0 ? 0 : nd[k];
-    const float f = d.flows[n * d.Bp + col], v = d.mars[n * d.Bp + col];
-    const float nv = d.norm[(d.norm_row >= 0 ? d.norm_row : n) * d.Bp + col];
-    rv[k] = (nd[k] >= 0 && f > 0.f && v > -INFINITY) ? f * __expf((mb - v) * d.inv_f - nv) : 0.f;
+    for (int k = 0; k < NG; ++k) {
+      const int64_t n = nd[k] < 0 ? 0 : nd[k];
+      f[k] = d.flows[n * d.Bp + col];
+      v[k] = d.mars[n * d.Bp + col];
+      nv[k] = 0.f;
+    }
+    if (d.norm_row < 0) {   // tempered flows only (the same for every lane: a branch around requests, none around a wait)
+#pragma unroll
+      for (int k = 0; k < NG; ++k) nv[k] = d.norm[(nd[k] < 0 ? 0 : (int64_t)nd[k]) * d.Bp + col];
+    }
+#pragma unroll
+    for (int k = 0; k < NG; ++k)
+      rv[k] = (nd[k] >= 0 && f[k] > 0.f && v[k] > -INFINITY) ? f[k] * __expf((mb - v[k]) * d.inv_f - nv[k]) : 0.f;
   }
   if constexpr (kPre) {
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) values(ct);
+    for (int ct = 0; ct < CT; ++ct) values(ct, ct);
   }
 #pragma unroll
   for (int ct = 0; ct < CT; ++ct) {
     const int s = kPre ? ct : 0;
-    if constexpr (!kPre) { numbers(ct, 0); values(0); }
+    if constexpr (!kPre) { numbers(ct, 0); values(ct, 0); }
     g4f acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int k = 0; k < NG; ++k) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s][k], rv[k], acc, 0, 0, 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float f = e[s][i] * acc[i];
+      const float f = (e[s][i] > -INFINITY ? __expf(e[s][i] * d.inv_f) : 0.f) * acc[i];
       const int4 p = cpa[s][i], q = cpb[s][i];
       if (p.x >= 0) d.flows[(int64_t)p.x * d.Bp + col] = f;
       if (p.y >= 0) d.flows[(int64_t)p.y * d.Bp + col] = f;
@@ -264,6 +279,37 @@ __global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, G
       if (q.z >= 0) d.flows[(int64_t)q.z * d.Bp + col] = f;
       if (q.w >= 0) d.flows[(int64_t)q.w * d.Bp + col] = f;
     }
+  }
+}
+
+template <int GT, int CT>
+__global__ __launch_bounds__(64) void sparse_group_backward_kernel(GroupDev d, GroupBase base) {
+  group_backward_body<GT, CT>(d, base, blockIdx.x, threadIdx.x, blockIdx.y);
+}
+
+// Walks: several consecutive layers of groups in ONE launch.  A launch that depends on the one before costs 4 to 5 us
+// however little it does, and a circuit over a tree has as many layers of groups as the tree has levels; but everything
+// a group reads and writes for 16 examples is read and written for those 16 examples only.  So a workgroup takes one
+// slice of 16 examples through all the layers of a run (layers that hold groups of one shape and nothing else): a layer's
+// groups dealt to its waves, a barrier between layers.  What a layer stores the next one reads through the same compute
+// unit's cache, which the waves of a workgroup share: the barrier's wait for the stores is all the ordering it needs.
+// Used where a layer's groups would not fill the device anyway (the host decides).
+struct GroupWalk {
+  const int2* levels;   // per layer of the run, in the order of the walk: {its first group, counted from the run's first; groups}
+  int n_levels;
+  GroupBase base;       // of the run's first group (the tables are padded: group i's entries are i strides further on)
+};
+
+template <int GT, int CT, int WV, bool kForward>
+__global__ __launch_bounds__(WV * 64) void sparse_group_walk_kernel(GroupDev d, GroupWalk w) {
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  for (int l = 0; l < w.n_levels; ++l) {
+    const int2 lv = w.levels[l];
+    for (int i = wave; i < lv.y; i += WV) {
+      if constexpr (kForward) group_forward_body<GT, CT>(d, w.base, lv.x + i, lane, blockIdx.x);
+      else group_backward_body<GT, CT>(d, w.base, lv.x + i, lane, blockIdx.x);
+    }
+    __syncthreads();
   }
 }
 
@@ -288,16 +334,12 @@ __global__ __launch_bounds__(256) void sparse_group_stats_kernel(GroupDev d, int
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int c = cb + 4 * q;
-      x[q] = -INFINITY;
-      if (c < r.C) {
-        const int4 v = d.rows[r.pslot0 + c];
-        x[q] = group_x(d, int4{guni(v.x), guni(v.y), guni(v.z), guni(v.w)}, b0 + b);
-      }
+      x[q] = c < Cp ? d.xm[(int64_t)(r.pslot0 + c) * d.Bp + b0 + b] : -INFINITY;
     }
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
       const int c = cb + 4 * q;
-      if (c < Cp) E[c * kGroupPad + b] = x[q] > -INFINITY ? __expf((x[q] - mb) * d.inv_f) : 0.f;
+      if (c < Cp) E[c * kGroupPad + b] = x[q] > -INFINITY ? __expf(x[q] * d.inv_f) : 0.f;
     }
   }
   for (int gb = part; gb < Gp; gb += 32) {   // (eight sums' rows requested before the first is used, as above)

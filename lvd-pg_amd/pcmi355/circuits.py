@@ -7,7 +7,7 @@ from ._lib import lib, check, np_ptr, H, c_i64
 
 _SIZE = dict(parameters=0, sum_parameters=1, nodes=2, edges=3, input_parameters=4, variables=5,
              categories=6, hidden_categories=7, inner_tree_nodes=8, layers=9, groups=10, input_nodes=11, heads=12,
-             description_nodes=13, walk_kernels=14, trees=15, dense_groups=16, layer_nodes=17)
+             description_nodes=13, walk_kernels=14, trees=15, dense_groups=16, layer_nodes=17, walk_levels=18)
 _TABLE = dict(edge2param=(0, "edges"), param2edge=(1, "sum_parameters"), param2group=(2, "sum_parameters"),
               pargroup_sizes=(3, "groups"), innode2ncumparam=(4, "input_nodes"), layer_ends=(5, "layers"),
               edge_parent=(6, "edges"), edge_prime=(7, "edges"), edge_sub=(8, "edges"), heads=(9, "heads"),

@@ -618,6 +618,18 @@ def _with_and_without_groups(P, heads, V, C):
     return grouped, plain
 
 
+def _without_group_walks(P, heads, V, C):
+    """... and with its groups, but a launch per layer where runs of layers would go as one walk launch."""
+    import os
+    os.environ["PCMI355_GROUP_WALK"] = "0"
+    try:
+        c = _compile(P, heads, V, C, len(heads))
+    finally:
+        del os.environ["PCMI355_GROUP_WALK"]
+    assert c.size("walk_levels") == 0
+    return c
+
+
 def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
     """Values, flows, statistics and updated parameters of a multi-head circuit whose dense groups run on the block
     kernels, against the oracle and against the same circuit on the layer kernels alone."""
@@ -646,7 +658,9 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
     order = fc.up_order()
     order = order[fc.edge_parent()[order] != fc.n_nodes - 1]
     got = []
-    for bpc in (grouped, plain):
+    layered = _without_group_walks(P, heads, V, C)
+    assert layered.size("dense_groups") == grouped.size("dense_groups")
+    for bpc in (grouped, plain, layered):
         per_head = P.loglikelihoods(bpc, d).cpu().numpy()
         assert rel_err(per_head, mars_ref[root_ids].T).max() < LL_RTOL
         ll = P.probs_flows_circuit(bpc, d, head_mask=hm).cpu().numpy()
@@ -660,10 +674,11 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
         assert np.abs(lf - lf_ref).max() < FLOW_RTOL * lf_ref.max()
         L.check(L.lib.pcm_em_update(bpc.handle, 0.1, 0.7))
         got.append((ll, mars, flows, ea, lf, P.vectorize_parameters(bpc)))
-    for a, b in zip(*got):                                   # the two paths round differently, no more
+    for a, b, c in zip(*got):                                # the two paths round differently, no more
         fa, fb = np.isfinite(a), np.isfinite(b)
         assert np.array_equal(fa, fb)
         assert np.abs(a[fa] - b[fb]).max() <= 2e-4 * max(np.abs(b[fb]).max(), 1.0)
+        assert np.array_equal(a.view(np.uint32), c.view(np.uint32))   # a walk and a launch per layer: the same arithmetic
     # a smaller batch afterwards finds the arrays of the larger one (rows of 64 examples, the last one partly filled)
     small = d[: B // 3]
     for bpc in (grouped, plain):
@@ -674,7 +689,8 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
 
 
 @pytest.mark.parametrize("V,K,C,H,B,max_children,seed", [(20, 8, 5, 9, 150, 5, 31), (9, 32, 4, 40, 64, 2, 32),
-                                                         (33, 12, 3, 6, 333, 3, 33)])
+                                                         (33, 12, 3, 6, 333, 3, 33), (40, 16, 4, 7, 100, 3, 34),
+                                                         (12, 64, 3, 5, 50, 2, 35)])
 def test_dense_groups_of_a_multihead_hclt(gpu, oracle, V, K, C, H, B, max_children, seed):
     """An HCLT's K sums per tree node and the heads over the root's products are groups; products of up to three
     children are taken apart by the groups above them, those of more stay nodes of a layer."""
@@ -690,6 +706,9 @@ def test_dense_groups_of_a_multihead_hclt(gpu, oracle, V, K, C, H, B, max_childr
     inner = len(set(parent[1:].tolist()))                    # (the K sums of an inner tree node; the root's are the heads)
     grouped, _ = _check_grouped_multihead(gpu, oracle, heads, V, C, B, seed, min_groups=inner)
     assert grouped.size("dense_groups") == inner
+    if max_children <= 3 and K in (16, 32, 64):
+        # every level of the tree below the root's is a layer of K x K groups and nothing else: one walk launch
+        assert grouped.size("walk_levels") >= 2
     if max_children <= 3:
         # nothing but the inputs and the product of the root's children is left to the layer kernels going up
         assert grouped.size("layer_nodes") == grouped.size("input_nodes") + K
