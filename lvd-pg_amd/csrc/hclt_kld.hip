@@ -693,6 +693,9 @@ __global__ __launch_bounds__(256) void hclt_rows_base_kernel(const HcltNode* __r
                                                              size_t n_par, const float* __restrict__ kl_leaf, size_t vk,
                                                              float* __restrict__ ell, float* __restrict__ base,
                                                              float* __restrict__ pu, float* __restrict__ pd, KlRowStrides rs) {
+  // (kl_leaf null: the leaf terms are not known yet -- the gradient's downward chain runs before the one pass over the
+  // leaf parameters -- and base gets the node's own part sum_j p (x - y) only; hclt_rows_soft_base2_kernel adds
+  // sum_j p * ell[j] from the operand afterwards)
   __shared__ float tile[K][K + 1];
   __shared__ float l[K];
   const int n = blockIdx.x, t = threadIdx.x;
@@ -701,14 +704,17 @@ __global__ __launch_bounds__(256) void hclt_rows_base_kernel(const HcltNode* __r
   const size_t su = (size_t)pos[n], sd = (size_t)pos[n_inner + n];
   const float* p1 = P1 + row * n_par;
   const float* p2 = P2 + row * n_par;
-  kl_leaf += row * vk;
   ell += row * rs.vec;
   base += row * rs.vec;
   if (t < K) {
-    float s = kl_leaf[(size_t)nd.var * K + t];
-    for (int q = 0; q < nd.lc_cnt; ++q) s += kl_leaf[(size_t)child_leaf[nd.lc_off + q] * K + t];
+    float s = 0.f;
+    if (kl_leaf) {
+      kl_leaf += row * vk;
+      s = kl_leaf[(size_t)nd.var * K + t];
+      for (int q = 0; q < nd.lc_cnt; ++q) s += kl_leaf[(size_t)child_leaf[nd.lc_off + q] * K + t];
+      ell[su * K + t] = s;
+    }
     l[t] = s;
-    ell[su * K + t] = s;
   }
   __syncthreads();
   const int j = t % K;
@@ -775,28 +781,50 @@ __global__ void hclt_rows_edge_grad_kernel(int64_t ns, int K, const int64_t* __r
   }
 }
 
-// gradients of the leaf parameters, as the source writes them (src/queries/kld.jl:528-535,
-// src/nodes/fixable_categorical_dist.jl:216-219): a thread takes four consecutive categories of one input node
+// The two leaf passes of the gradient in one: the leaf terms of the divergence (hclt_rows_leaf_kl_kernel) and the
+// gradients of the leaf parameters (src/queries/kld.jl:528-535, src/nodes/fixable_categorical_dist.jl:216-219) read
+// the same two runs of C values per input node, and
+// the gradient's weight h comes from the DOWNWARD chain, which needs only the parameters -- so it can run first and
+// the leaf parameters, nine tenths of a row, cross the memory bus once.  L lanes (a power of two, at most 64) per
+// (input node, row): 64 where C >= 256, fewer for short category lists so that no lane idles.
 template <bool kNorm>
-__global__ __launch_bounds__(256) void hclt_rows_leaf_grad_kernel(const float* __restrict__ P1, const float* __restrict__ P2,
-                                                                  size_t n_par, size_t ns, int C, int K, int64_t n_leaf4,
-                                                                  const int32_t* __restrict__ input_order,
-                                                                  const int32_t* __restrict__ state_node,
-                                                                  const float* __restrict__ h, size_t nk,
-                                                                  float* __restrict__ G1, float* __restrict__ G2) {
-  const int64_t q = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void hclt_rows_leaf_kl_grad_kernel(const float* __restrict__ P1, const float* __restrict__ P2,
+                                                                     size_t n_par, size_t ns, int C, int K, int n_inputs, int L,
+                                                                     const int32_t* __restrict__ input_order,
+                                                                     const int32_t* __restrict__ state_node,
+                                                                     const float* __restrict__ h, size_t nk, size_t vk,
+                                                                     float* __restrict__ kl_leaf, float* __restrict__ G1,
+                                                                     float* __restrict__ G2) {
+  const int lane = threadIdx.x % L;
+  const int i = (blockIdx.x * 256 + threadIdx.x) / L;
   const size_t row = blockIdx.y;
-  if (q >= n_leaf4) return;
-  const int64_t at = q * 4;
-  const int vj = input_order[at / C];
+  if (i >= n_inputs) return;
+  const int vj = input_order[i];
   const float g = h[row * nk + (size_t)state_node[vj / K] * K + vj % K];
-  const size_t off = row * n_par + ns + at;
-  const float4 a = *reinterpret_cast<const float4*>(P1 + off), b = *reinterpret_cast<const float4*>(P2 + off);
+  const size_t at = row * n_par + ns + (size_t)i * C;
+  const float4* a4 = reinterpret_cast<const float4*>(P1 + at);
+  const float4* b4 = reinterpret_cast<const float4*>(P2 + at);
+  float4* g1 = reinterpret_cast<float4*>(G1 + at);
+  float4* g2 = reinterpret_cast<float4*>(G2 + at);
   auto d1 = [&](float x, float y) { return kNorm ? g * (logf(x + kRowsNormEps) - logf(y + kRowsNormEps) + 1.f) : g * (x - y + 1.f); };
   auto d2 = [&](float x, float y) { return kNorm ? g * x / (y + kRowsNormEps) : g * expf(x - y); };
-  *reinterpret_cast<float4*>(G1 + off) = make_float4(d1(a.x, b.x), d1(a.y, b.y), d1(a.z, b.z), d1(a.w, b.w));
-  *reinterpret_cast<float4*>(G2 + off) = make_float4(d2(a.x, b.x), d2(a.y, b.y), d2(a.z, b.z), d2(a.w, b.w));
+  float acc = 0.f;
+  for (int c4 = lane; c4 < C / 4; c4 += L) {
+    const float4 a = a4[c4], b = b4[c4];
+    g1[c4] = make_float4(d1(a.x, b.x), d1(a.y, b.y), d1(a.z, b.z), d1(a.w, b.w));
+    g2[c4] = make_float4(d2(a.x, b.x), d2(a.y, b.y), d2(a.z, b.z), d2(a.w, b.w));
+    acc += (rows_leaf_term<kNorm>(a.x, b.x) + rows_leaf_term<kNorm>(a.y, b.y)) +
+           (rows_leaf_term<kNorm>(a.z, b.z) + rows_leaf_term<kNorm>(a.w, b.w));
+  }
+  for (int o = L / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o);   // (the L lanes of a node leave or stay together)
+  if (lane == 0) kl_leaf[row * vk + vj] = acc;
 }
+
+template <int K>
+__global__ void hclt_rows_soft_base2_kernel(const HcltNode* __restrict__ nodes, const int32_t* __restrict__ child_leaf,
+                                            const int32_t* __restrict__ pos, int n_inner, const float* __restrict__ leaf_grad,
+                                            size_t vk, const float* __restrict__ pd, float* __restrict__ ell,
+                                            float* __restrict__ base, KlRowStrides rs, int add);
 
 // KL of every row (d_klds, may be null with gradients) and, with d_g1 / d_g2, its gradients in the layout of the inputs
 void HcltCircuit::kld_rows_block(const float* d_p1, const float* d_p2, int64_t sr, int64_t sp, int32_t rows, bool norm,
@@ -857,40 +885,58 @@ void HcltCircuit::kld_rows_block(const float* d_p1, const float* d_p2, int64_t s
     const int rc = std::min(chunk, rows - r0);
     const float* q1 = p1 + (size_t)r0 * n;
     const float* q2 = p2 + (size_t)r0 * n;
-    const dim3 lgrid(ceil_div(n_inputs, 16), rc);
-    auto leaf = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, lgrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, n_inputs, d_input_order_.p, vk, kl_leaf);
+    auto chain = [&](int down_only) {   // one workgroup per row, up the tree or down it
+      KlRowStrides r2 = rs;
+      r2.down_only = down_only;
+      PCM_DISPATCH_K(K_, {
+        auto launch = [&](auto kernel, size_t lds) {
+          hipLaunchKernelGGL(kernel, dim3(1, rc), dim3(kl_waves(KK) * 64), lds, stream,
+                             reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
+                             reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
+                             kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, r2);
+        };
+        if (kl_ring_slots_) launch(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
+        else launch(&hclt_kld_chain_kernel<KK, false>, 0);
+      });
     };
-    if (norm) { if (vec) leaf(&hclt_rows_leaf_kl_kernel<true, true>); else leaf(&hclt_rows_leaf_kl_kernel<true, false>); }
-    else { if (vec) leaf(&hclt_rows_leaf_kl_kernel<false, true>); else leaf(&hclt_rows_leaf_kl_kernel<false, false>); }
-    PCM_DISPATCH_K(K_, {
-      hipLaunchKernelGGL(hclt_rows_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
-                         d_kl_pos_.p, n_inner_, d_blk2par_.p, q1, q2, (size_t)n, kl_leaf, vk, ell, base, pu, pd, rs);
-      auto chain = [&](auto kernel, size_t lds) {
-        hipLaunchKernelGGL(kernel, dim3(with_down ? 2 : 1, rc), dim3(kl_waves(KK) * 64), lds, stream,
-                           reinterpret_cast<const KlItem*>(d_kl_up_.p), kl_up_steps_,
-                           reinterpret_cast<const KlItem*>(d_kl_down_.p), kl_down_steps_, d_kl_ext_.p, pu, base, ell, pd,
-                           kl_ring_slots_ - 1, ring_up, ring_down, klv, z, h, rs);
+    auto base_pass = [&](const float* leaf_terms, float* up, float* down) {
+      PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_rows_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p,
+                                            d_child_leaf_.p, d_kl_pos_.p, n_inner_, d_blk2par_.p, q1, q2, (size_t)n, leaf_terms,
+                                            vk, ell, base, up, down, rs));
+    };
+    if (!with_down) {
+      const dim3 lgrid(ceil_div(n_inputs, 16), rc);
+      auto leaf = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, lgrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, n_inputs, d_input_order_.p, vk, kl_leaf);
       };
-      if (kl_ring_slots_) chain(&hclt_kld_chain_kernel<KK, true>, (size_t)kl_ring_slots_ * KK * sizeof(float));
-      else chain(&hclt_kld_chain_kernel<KK, false>, 0);
-    });
-    if (d_klds)
-      hipLaunchKernelGGL(hclt_rows_take_kernel, dim3(ceil_div(rc, 256)), dim3(256), 0, stream, klv, nk, root_at, rc, d_klds + r0);
-    if (with_down) {
+      if (norm) { if (vec) leaf(&hclt_rows_leaf_kl_kernel<true, true>); else leaf(&hclt_rows_leaf_kl_kernel<true, false>); }
+      else { if (vec) leaf(&hclt_rows_leaf_kl_kernel<false, true>); else leaf(&hclt_rows_leaf_kl_kernel<false, false>); }
+      base_pass(kl_leaf, pu, nullptr);
+      chain(0);
+    } else {
+      // the operands, the downward chain (it needs nothing but the parameters), ONE pass over the leaf parameters for the
+      // leaf terms and the leaf gradients, then the constants of the upward chain, that chain, the sum parameters
       float* o1 = g1 + (size_t)r0 * n;
       float* o2 = g2 + (size_t)r0 * n;
+      base_pass(nullptr, pu, pd);
+      chain(1);
+      int L = 1;
+      while (L < 64 && L * 4 < C_) L *= 2;
+      const dim3 ggrid((unsigned)ceil_div((int64_t)n_inputs * L, 256), rc);
+      if (norm)
+        hipLaunchKernelGGL(hclt_rows_leaf_kl_grad_kernel<true>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
+                           n_inputs, L, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, vk, kl_leaf, o1, o2);
+      else
+        hipLaunchKernelGGL(hclt_rows_leaf_kl_grad_kernel<false>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
+                           n_inputs, L, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, vk, kl_leaf, o1, o2);
+      PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_rows_soft_base2_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p,
+                                            d_child_leaf_.p, d_kl_pos_.p, n_inner_, kl_leaf, vk, pd, ell, base, rs, 1));
+      chain(0);
       hipLaunchKernelGGL(hclt_rows_edge_grad_kernel, dim3((unsigned)ceil_div(ns, 256), ceil_div(rc, kEdgeGradRows)), dim3(256), 0,
                          stream, ns, K_, d_sum_param_src_.p, d_kl_tabs_.p, q1, q2, (size_t)n, z, h, nk, rc, o1, o2);
-      const int64_t n_leaf4 = (int64_t)n_inputs * C_ / 4;
-      const dim3 ggrid((unsigned)ceil_div(n_leaf4, 256), rc);
-      if (norm)
-        hipLaunchKernelGGL(hclt_rows_leaf_grad_kernel<true>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
-                           n_leaf4, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, o1, o2);
-      else
-        hipLaunchKernelGGL(hclt_rows_leaf_grad_kernel<false>, ggrid, dim3(256), 0, stream, q1, q2, (size_t)n, (size_t)ns, C_, K_,
-                           n_leaf4, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, o1, o2);
     }
+    if (d_klds)
+      hipLaunchKernelGGL(hclt_rows_take_kernel, dim3(ceil_div(rc, 256)), dim3(256), 0, stream, klv, nk, root_at, rc, d_klds + r0);
   }
   if (with_down && !direct) {
     rows_unpack_out(g1, d_g1, sr, sp, rows, n, stream);
@@ -955,7 +1001,7 @@ __device__ __forceinline__ int kl_operand_word(int rw, int col) {
 // Reverse pass, input nodes (gumbel_input_sample_up_kernel, sample.jl:531-598): the gradient of a leaf parameter is
 // og[v][c] * td(v, j) -- per PROBABILITY of the category, with probability-valued parameters or not, as the source writes
 // it (:560-570) -- and the node's own gradient sum_c p(c) * og[v][c] goes to leaf_grad[row][v * K + j].  A wave per
-// input node and row, 16-byte accesses.
+// two input nodes and row, 16-byte accesses.
 template <bool kNorm>
 __global__ __launch_bounds__(256) void hclt_rows_soft_back_leaf_kernel(const float* __restrict__ P, size_t n_par, size_t ns, int C,
                                                                        int K, int V, int n_inputs,
@@ -965,36 +1011,54 @@ __global__ __launch_bounds__(256) void hclt_rows_soft_back_leaf_kernel(const flo
                                                                        const float* __restrict__ og, size_t vk,
                                                                        float* __restrict__ leaf_grad, float* __restrict__ G) {
   const int lane = threadIdx.x & 63;
-  const int i = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int i0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * 2;   // two nodes per wave: both nodes' loads leave before either is used
   const size_t row = blockIdx.y;
-  if (i >= n_inputs) return;
-  const int vj = input_order[i], v = vj / K;
-  const float t = h[row * nk + (size_t)state_node[v] * K + vj % K];
-  const size_t at = row * n_par + ns + (size_t)i * C;
-  const float4* p = reinterpret_cast<const float4*>(P + at);
-  const float4* o = reinterpret_cast<const float4*>(og + (row * V + v) * C);
-  float4* g = reinterpret_cast<float4*>(G + at);
-  float acc = 0.f;
-  for (int c4 = lane; c4 < C / 4; c4 += 64) {
-    const float4 x = p[c4], oc = o[c4];
-    g[c4] = make_float4(oc.x * t, oc.y * t, oc.z * t, oc.w * t);
-    acc += kNorm ? (x.x * oc.x + x.y * oc.y) + (x.z * oc.z + x.w * oc.w)
+  if (i0 >= n_inputs) return;
+  const bool two = i0 + 1 < n_inputs;
+  const int vj0 = input_order[i0], vj1 = input_order[two ? i0 + 1 : i0];
+  const int v0 = vj0 / K, v1 = vj1 / K;
+  const float t0 = h[row * nk + (size_t)state_node[v0] * K + vj0 % K];
+  const float t1 = h[row * nk + (size_t)state_node[v1] * K + vj1 % K];
+  const size_t at = row * n_par + ns + (size_t)i0 * C;
+  const float4* p0 = reinterpret_cast<const float4*>(P + at);
+  const float4* p1 = reinterpret_cast<const float4*>(P + at + (two ? C : 0));
+  const float4* o0 = reinterpret_cast<const float4*>(og + (row * V + v0) * C);
+  const float4* o1 = reinterpret_cast<const float4*>(og + (row * V + v1) * C);
+  float4* g0 = reinterpret_cast<float4*>(G + at);
+  float4* g1 = reinterpret_cast<float4*>(G + at + C);
+  auto dot = [&](const float4& x, const float4& oc) {
+    return kNorm ? (x.x * oc.x + x.y * oc.y) + (x.z * oc.z + x.w * oc.w)
                  : (expf(x.x) * oc.x + expf(x.y) * oc.y) + (expf(x.z) * oc.z + expf(x.w) * oc.w);
+  };
+  float acc0 = 0.f, acc1 = 0.f;
+  for (int c4 = lane; c4 < C / 4; c4 += 64) {
+    const float4 x0 = p0[c4], x1 = p1[c4], oc0 = o0[c4], oc1 = o1[c4];
+    g0[c4] = make_float4(oc0.x * t0, oc0.y * t0, oc0.z * t0, oc0.w * t0);
+    if (two) g1[c4] = make_float4(oc1.x * t1, oc1.y * t1, oc1.z * t1, oc1.w * t1);
+    acc0 += dot(x0, oc0);
+    acc1 += dot(x1, oc1);
   }
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-  if (lane == 0) leaf_grad[row * vk + vj] = acc;
+  for (int off = 32; off > 0; off >>= 1) {
+    acc0 += __shfl_xor(acc0, off);
+    acc1 += __shfl_xor(acc1, off);
+  }
+  if (lane == 0) {
+    leaf_grad[row * vk + vj0] = acc0;
+    if (two) leaf_grad[row * vk + vj1] = acc1;
+  }
 }
 
 // Reverse pass, what the upward chain starts from, per (tree node, row): ell[su][j] = the gradients of the leaves that
 // are factors of product j, base[su][k] = sum_j w[k,j] * ell[j] with the weights read back from the downward operand
+// (add: on top of what base holds -- the KL gradient on rows, whose base starts as the node's own part)
 template <int K>
 __global__ __launch_bounds__(256) void hclt_rows_soft_base2_kernel(const HcltNode* __restrict__ nodes,
                                                                    const int32_t* __restrict__ child_leaf,
                                                                    const int32_t* __restrict__ pos, int n_inner,
                                                                    const float* __restrict__ leaf_grad, size_t vk,
                                                                    const float* __restrict__ pd, float* __restrict__ ell,
-                                                                   float* __restrict__ base, KlRowStrides rs) {
+                                                                   float* __restrict__ base, KlRowStrides rs, int add) {
   __shared__ float l[K];
   const int n = blockIdx.x, t = threadIdx.x;
   const size_t row = blockIdx.y;
@@ -1016,7 +1080,7 @@ __global__ __launch_bounds__(256) void hclt_rows_soft_base2_kernel(const HcltNod
     float term = w[kl_operand_word<K>(k, j)] * l[j];
 #pragma unroll
     for (int o = K / 2; o > 0; o >>= 1) term += __shfl_xor(term, o, K);
-    if (j == 0) base[su * K + k] = term;
+    if (j == 0) base[su * K + k] = add ? base[su * K + k] + term : term;
   }
 }
 
@@ -1222,7 +1286,7 @@ void HcltCircuit::gumbel_sample_backward_rows(const float* d_params, int64_t sr,
       hipLaunchKernelGGL(hclt_rows_soft_base_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_kl_pos_.p, n_inner_,
                          d_blk2par_.p, q, (size_t)n, g, (size_t)ns, inv_t, pd, pu, rs);
       chain(1);   // the top-down probabilities
-      const dim3 lgrid(ceil_div(n_inputs, 4), rc);
+      const dim3 lgrid(ceil_div(n_inputs, 8), rc);
       if (norm_params)
         hipLaunchKernelGGL(hclt_rows_soft_back_leaf_kernel<true>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
                            n_inputs, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, og, vk, leaf_grad, out);
@@ -1230,7 +1294,7 @@ void HcltCircuit::gumbel_sample_backward_rows(const float* d_params, int64_t sr,
         hipLaunchKernelGGL(hclt_rows_soft_back_leaf_kernel<false>, lgrid, dim3(256), 0, stream, q, (size_t)n, (size_t)ns, C_, K_, Vu_,
                            n_inputs, d_input_order_.p, d_kl_tabs_.p + n_inner_, h, nk, og, vk, leaf_grad, out);
       hipLaunchKernelGGL(hclt_rows_soft_base2_kernel<KK>, dim3(n_inner_, rc), dim3(256), 0, stream, d_nodes_.p, d_child_leaf_.p,
-                         d_kl_pos_.p, n_inner_, leaf_grad, vk, pd, ell, base, rs);
+                         d_kl_pos_.p, n_inner_, leaf_grad, vk, pd, ell, base, rs, 0);
       chain(0);   // the gradients of the sum nodes, bottom-up
       hipLaunchKernelGGL(hclt_rows_soft_edge_grad_kernel<KK>, dim3((unsigned)ceil_div(ns, 256), ceil_div(rc, kEdgeGradRows)),
                          dim3(256), 0, stream, ns, d_sum_param_src_.p, d_kl_tabs_.p, d_kl_pos_.p, n_inner_, pd, z, klv, h, nk, rs,
