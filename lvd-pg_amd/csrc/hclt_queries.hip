@@ -136,6 +136,56 @@ __global__ __launch_bounds__(256) void hclt_sample_states_node_kernel(const floa
   for (int i = lane; i < n_inner; i += 64) states[(size_t)b * n_inner + i] = mine[i];
 }
 
+// (value, category) of one lane against another's: the larger value, the lower category among equal values; a lane
+// that has seen nothing carries category 0x7fffffff
+__device__ __forceinline__ void argmax_take(float& bv, int& bx, float ov, int oi) {
+  if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
+}
+
+// The maxima of N examples over a wave as one butterfly: at the first log2(N) steps the two halves of a group of lanes
+// swap half of the examples they still carry, the remaining steps reduce the one example a group of 64 / N lanes is
+// left with.  Afterwards bv[0], bx[0] of lane l belong to example l / (64 / N).  2 (N - 1) + 2 log2(64 / N) cross-lane
+// moves instead of 12 N; the moves go through the LDS unit, which in these kernels also serves the table rows.
+template <int N>
+__device__ __forceinline__ void argmax_deal(float (&bv)[N], int (&bx)[N], int lane) {
+  static_assert(N == 2 || N == 4 || N == 8, "N examples on 64 lanes");
+  int o = 32;
+#pragma unroll
+  for (int n = N; n > 1; n >>= 1, o >>= 1) {
+    const bool up = lane & o;
+#pragma unroll
+    for (int i = 0; i < n / 2; ++i) {
+      float kv = up ? bv[n / 2 + i] : bv[i];
+      int ki = up ? bx[n / 2 + i] : bx[i];
+      const float sv = up ? bv[i] : bv[n / 2 + i];
+      const int si = up ? bx[i] : bx[n / 2 + i];
+      argmax_take(kv, ki, __shfl_xor(sv, o), __shfl_xor(si, o));
+      bv[i] = kv;
+      bx[i] = ki;
+    }
+  }
+#pragma unroll
+  for (int r = 64 / N / 2; r > 0; r >>= 1) argmax_take(bv[0], bx[0], __shfl_xor(bv[0], r), __shfl_xor(bx[0], r));
+}
+
+// N = 4 written out (the category kernel with the table in LDS): the same moves, but the kernel around it comes out 8 %
+// faster than with the loops above (2.71 against 2.96 ms at 4096 samples of a 3072-variable circuit).
+template <>
+__device__ __forceinline__ void argmax_deal<4>(float (&best)[4], int (&bi)[4], int lane) {
+  const bool hb = lane & 32, qb = lane & 16;
+  float k0 = hb ? best[2] : best[0], k1 = hb ? best[3] : best[1];
+  int i0 = hb ? bi[2] : bi[0], i1 = hb ? bi[3] : bi[1];
+  argmax_take(k0, i0, __shfl_xor(hb ? best[0] : best[2], 32), __shfl_xor(hb ? bi[0] : bi[2], 32));
+  argmax_take(k1, i1, __shfl_xor(hb ? best[1] : best[3], 32), __shfl_xor(hb ? bi[1] : bi[3], 32));
+  float bv = qb ? k1 : k0;
+  int bx = qb ? i1 : i0;
+  argmax_take(bv, bx, __shfl_xor(qb ? k0 : k1, 16), __shfl_xor(qb ? i0 : i1, 16));
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) argmax_take(bv, bx, __shfl_xor(bv, o), __shfl_xor(bx, o));
+  best[0] = bv;
+  bi[0] = bx;
+}
+
 // Categories.  A wave takes kVarsPerWave consecutive variables of one example, 64 lanes x 4
 // categories each (more categories: further rounds), requests all their rows first and then
 // reduces them one by one: per variable the wave keeps the largest value and, among equal
@@ -193,18 +243,9 @@ __global__ __launch_bounds__(256) void hclt_sample_leaves_kernel(const float* __
       for (int i = 0; i < 4; ++i)
         if (c0 + i < C && (x[q][i] > best[q] || bi[q] == 0x7fffffff)) { best[q] = x[q][i]; bi[q] = c0 + i; }
   }
-#pragma unroll
-  for (int q = 0; q < kVarsPerWave; ++q) {
-    float bv = best[q];
-    int bx = bi[q];
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o);
-      const int oi = __shfl_xor(bx, o);
-      if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
-    }
-    if (lane == 0 && v0 + q < V) out[(size_t)b * V + v0 + q] = (uint8_t)bx;
-  }
+  argmax_deal<kVarsPerWave>(best, bi, lane);
+  const int q = lane / (64 / kVarsPerWave);   // the variable this group of lanes is left with
+  if (lane % (64 / kVarsPerWave) == 0 && v0 + q < V) out[(size_t)b * V + v0 + q] = (uint8_t)bi[0];
 }
 
 // Categories with the leaf table in LDS.  A workgroup takes one variable and kLeafExamples
@@ -262,18 +303,10 @@ __global__ __launch_bounds__(kLeafWaves * 64) void hclt_sample_leaves_lds_kernel
           if (x[i] > best[u] || bi[u] == 0x7fffffff) { best[u] = x[i]; bi[u] = c0 + i; }
       }
     }
-#pragma unroll
-    for (int u = 0; u < kLeafUnroll; ++u) {
-      float bv = best[u];
-      int bx = bi[u];
-#pragma unroll
-      for (int o = 32; o > 0; o >>= 1) {
-        const float ov = __shfl_xor(bv, o);
-        const int oi = __shfl_xor(bx, o);
-        if (oi != 0x7fffffff && (bx == 0x7fffffff || ov > bv || (ov == bv && oi < bx))) { bv = ov; bx = oi; }
-      }
-      if (lane == 0 && e0 + u < nb) out[(size_t)(b0 + e0 + u) * V + v] = (uint8_t)bx;
-    }
+    argmax_deal<kLeafUnroll>(best, bi, lane);
+    const int bx = bi[0];
+    const int u = lane / (64 / kLeafUnroll);   // the example this group of lanes is left with
+    if (lane % (64 / kLeafUnroll) == 0 && e0 + u < nb) out[(size_t)(b0 + e0 + u) * V + v] = (uint8_t)bx;
   }
 }
 
