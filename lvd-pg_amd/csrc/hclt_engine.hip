@@ -1717,12 +1717,13 @@ bool HcltCircuit::sample_soft_block(const float* d_node_noise, float temperature
                        level_ptr, soft_levels_, kernel_noise(d_node_noise, batch), n_inner_, batch, ns, inv_t, d_R_.p);
     const int nchunks = ceil_div(C_, kSoftLeafCats);
     const int use_rows = (C_ & 3) == 0 ? 1 : 0;   // rows of whole 16-byte words leave through an LDS pad
-    const dim3 lgrid(Vu_, ceil_div(nchunks * ceil_div(ns, kSoftLeafSlices), 4));   // (the caller's variables)
+    const int run_slices = soft_leaf_run_slices((int64_t)Vu_ * nchunks, ns);
+    const dim3 lgrid(Vu_, ceil_div(nchunks * ceil_div(ns, run_slices), 4));   // (the caller's variables)
     const size_t pad_bytes = use_rows ? (size_t)4 * kSlice * (kSoftLeafCats + 4) * sizeof(float) : 0;   // 65 KB
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_soft_leaves_kernel<KK>),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)pad_bytes));
     hipLaunchKernelGGL(hclt_soft_leaves_kernel<KK>, lgrid, dim3(256), pad_bytes, stream, d_leaf_.p, state_node, d_R_.p, Vu_,
-                       C_, batch, ns, nchunks, use_rows, d_out);
+                       C_, batch, ns, nchunks, run_slices, use_rows, d_out);
   });
   check_launch("hclt_sample_soft");
   PCM_HIP(hipStreamSynchronize(stream));

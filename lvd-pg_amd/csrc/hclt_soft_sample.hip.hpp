@@ -96,31 +96,40 @@ __global__ __launch_bounds__(soft_walk_waves(K) * 64) void hclt_soft_walk_kernel
 // out[b][u][:] = p_{v(u)}[b][:] * exp(leaf[u]): a [B x K] by [K x C] product per variable, on
 // the matrix cores with categories as rows and the 16 examples of a slice as columns.  A wave
 // keeps exp(leaf[u]) of kSoftLeafCats categories as A operands in registers for a run of
-// kSoftLeafSlices slices; a slice's probabilities arrive in the tile layout the walk wrote them
+// run_slices slices; a slice's probabilities arrive in the tile layout the walk wrote them
 // in, which is the B operand layout: with k-step (kt, i) standing for the states
 // kt*16 + 4g + i, g = 0..3, component i of a lane's 16-byte word at kt is its B value and
 // component i of the word at leaf[u][c][kt*16 + 4g] its A value.  A lane of the result holds
 // four consecutive categories of one example.  With rows of whole 16-byte words (use_rows) the
 // tiles of a slice are turned in a wave-private LDS pad and leave as one contiguous,
 // non-temporal run of C floats per example (a quarter faster than 16-byte stores four lanes
-// side by side, which is what other category counts get).  Write-bound: the output is
-// batch x V x C floats.
-constexpr int kSoftLeafSlices = 8;   // slices of 16 examples per work item
+// side by side, which is what other category counts get).  The output is batch x V x C floats; with the stores taken
+// out the kernel still takes two thirds of its time (the matrix instructions alone 2.0 ms of 3.5 at 4096 examples of a
+// 3072-variable circuit, against 1.3 ms at the data sheet's rate), and issuing a slice's rows between the matrix
+// instructions of the next slice instead of behind its own gained 1 %.
+// Slices of 16 examples per work item: every item loads and exponentiates its 32 KB of table rows again, so long runs
+// are cheaper (4096 examples of the 3072-variable circuit: 3.55 ms with runs of 8, 3.1 with runs of 64) as long as the
+// items still fill the device several times over.
+inline int soft_leaf_run_slices(int64_t items_per_slice_run, int nslices) {
+  for (int run = 64; run > 8; run /= 2)
+    if (items_per_slice_run * ((nslices + run - 1) / run) >= 12288) return run;
+  return 8;
+}
 constexpr int kSoftLeafCats = 256;   // categories per work item
 
 template <int K>
 __global__ __launch_bounds__(256) void hclt_soft_leaves_kernel(const float* __restrict__ leaf,
                                                                const int32_t* __restrict__ state_node,
                                                                const float* __restrict__ P, int V, int C, int batch,
-                                                               int nslices, int nchunks, int use_rows, float* __restrict__ out) {
+                                                               int nslices, int nchunks, int run_slices, int use_rows, float* __restrict__ out) {
   constexpr int KT = K / 16, CT = kSoftLeafCats / 16;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int u = blockIdx.x;
   const int item = blockIdx.y * 4 + wave;
   const int chunk = item % nchunks, run = item / nchunks;
-  const int s_first = run * kSoftLeafSlices;
+  const int s_first = run * run_slices;
   if (s_first >= nslices) return;
-  const int s_end = min(s_first + kSoftLeafSlices, nslices);
+  const int s_end = min(s_first + run_slices, nslices);
   const int g = lane >> 4, bb = lane & 15;
   const int cbase = chunk * kSoftLeafCats;
   v4f a[CT][KT];
