@@ -127,6 +127,10 @@ int pcm_set_soft_reg(pcm_circuit* c, float soft_reg, int32_t soft_reg_width, int
  * handles run these passes on their layered form (kernels per layer, dense groups on the matrix cores), with the
  * statistics and the flow memory held there until pcm_em_update.  Per-example weights / head masks scale the
  * flows as always (the reference's tempered pass reads its `weights` argument only at the input nodes).
+ * Together with pcm_set_soft_reg (mini_batch_em_beta passes both on, em.jl:366-368): the layered form has no smoothed
+ * leaf table, so the library turns every categorical batch into the soft evidence that gives the leaves the smoothed
+ * values (batch x num_vars x num_cats floats of device memory) and runs the tempered soft-evidence pass on it; the leaf
+ * flows are those of as_written == 0, and as_written != 0 makes such a pass fail with PCM_ERR_UNSUPPORTED.
  * PCM_ERR_ARG unless fscale is positive and finite.
  */
 int pcm_set_flow_scale(pcm_circuit* c, float fscale);

@@ -1593,12 +1593,26 @@ void HcltCircuit::flows(const BatchRef& b, float rate, const float* d_head_mask,
   if (flow_scale != 1.f && (block_ || wide_)) {
     // tempered flows (fscale of mini_batch_em_beta) are the layered engine's: the block kernels keep S, not the sum of
     // the shares to the power 1 / fscale
-    if (soft_reg_ > 0.f) fail(PCM_ERR_UNSUPPORTED, "tempered flows with soft_reg in the kernels: give the smoothed batch as soft evidence");
+    if (soft_reg_ > 0.f && soft_written_)
+      fail(PCM_ERR_UNSUPPORTED, "tempered flows with the leaf flows of soft_reg as the source writes them: that form is the block kernels'");
     if (have_flows_ && !flows_in_general_ && rate != 0.f)
       fail(PCM_ERR_STATE, "flow memory cannot carry over from ordinary flows on the block kernels to tempered flows");
     SparseCircuit* g = general();
     g->flow_scale = flow_scale;
-    g->flows(b, rate, d_head_mask, d_ll);
+    if (soft_reg_ > 0.f) {
+      // soft_reg and fscale together (scaled_probs_flows_circuit, src-jl/learning/flow.jl:366-372): the layered form
+      // has no smoothed leaf table, it takes the batch as the soft evidence that gives its leaves the smoothed values
+      no_forest("soft_reg with tempered flows");
+      const int64_t total = (int64_t)b.batch * Vu_ * C_;
+      d_soft_reg_ev_.ensure((size_t)total);
+      hipLaunchKernelGGL(hclt_soft_reg_evidence_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, stream, b, Vu_, C_,
+                         soft_reg_, soft_width_, d_soft_reg_ev_.p);
+      check_launch("soft_reg_evidence");
+      const SoftRef ev{d_soft_reg_ev_.p, (int64_t)Vu_ * C_, C_, 1, nullptr, b.batch};
+      g->flows_soft(ev, rate, d_head_mask, d_ll);
+    } else {
+      g->flows(b, rate, d_head_mask, d_ll);
+    }
     have_flows_ = true;
     flows_in_general_ = true;
     return;

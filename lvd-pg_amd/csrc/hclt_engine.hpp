@@ -253,6 +253,7 @@ class HcltCircuit : public pcm_circuit {
   int soft_width_ = 1;
   bool soft_written_ = false;
   DevBuf<float> d_leaf_smooth_, d_leaf_hist_;
+  DevBuf<float> d_soft_reg_ev_;                 // a smoothed batch as soft evidence, for tempered flows on the layered form
   void leaf_changed();                          // after anything that rewrites the leaf table
   float* stats_leaf_out() { return soft_reg_ > 0.f ? d_leaf_hist_.p : d_leaf_flow_.p; }
   float stats_leaf_rate(float rate) const { return soft_reg_ > 0.f ? 0.f : rate; }

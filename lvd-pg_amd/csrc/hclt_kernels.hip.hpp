@@ -840,6 +840,25 @@ __global__ __launch_bounds__(256) void hclt_leaf_smooth_kernel(const float* __re
   smooth[i] = __logf((1.f - s) * __expf(row[(int64_t)x * K]) + s * sp);
 }
 
+// The same smoothing as soft evidence, for the engine without a smoothed leaf table (tempered flows of a smoothed
+// batch run on the layered form): ev[b][v][c] = log((c == x) (1 - s) + (c in window(x)) s / n(x)), x the category example
+// b shows at variable v -- under it a leaf's value is soft_loglikelihood and the share of its flow that category c
+// gets is that of the derivative form below.  Thread = (b, v, c), c fastest.
+__global__ __launch_bounds__(256) void hclt_soft_reg_evidence_kernel(BatchRef b, int V, int C, float s, int width,
+                                                                    float* __restrict__ ev) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (int64_t)b.batch * V * C) return;
+  const int c = (int)(i % C), v = (int)((i / C) % V);
+  const int64_t e = i / ((int64_t)C * V);
+  const int64_t ex = b.d_idx ? b.d_idx[e] : e;
+  const int x = b.d_data[ex * b.stride_ex + (int64_t)v * b.stride_var];
+  int c0, c1;
+  soft_window(x, width, C, c0, c1);
+  float w = c >= c0 && c <= c1 ? s / (float)(c1 - c0 + 1) : 0.f;
+  if (c == x) w += 1.f - s;
+  ev[i] = __logf(w);   // (-inf outside the window)
+}
+
 // leaf_flow[v][c][k] = rate * leaf_flow[v][c][k] + sum over the categories x whose window holds c (or x = c) of
 //   hist[v][x][k] * ((x == c) (1 - s) q[x] + (c in window(x)) s / n(x) q[c]) / base(x),
 // where hist is the statistics' histogram by shown category.  soft_flow as the source has it (reg_flow.jl:12-17) takes

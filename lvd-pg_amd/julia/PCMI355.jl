@@ -271,7 +271,8 @@ param_inertia_end, flow_memory, flow_memory_end, shuffle, update_interval, fscal
 (VariationalJuice.jl/src-jl/learning/em.jl:289-409): statistics collect over `update_interval` batches -- cleared at the
 start of an epoch, cleared or decayed by the flow memory at a batch with batch_id % update_interval == 1, every batch
 adds its flows, the parameters move after a batch with batch_id % update_interval == 0 -- with schedules for the
-inertia and the flow memory.  `fscale` other than 1: the flows of the tempered posterior (`pcm_set_flow_scale`)."
+inertia and the flow memory.  `fscale` other than 1: the flows of the tempered posterior (`pcm_set_flow_scale`); together
+with `soft_reg` the library smooths through soft evidence and needs `soft_flow_as_written = false`."
 function mini_batch_em_beta(c::Circuit, data, num_epochs::Integer; batch_size::Integer, pseudocount,
                             soft_reg = 0.0, soft_reg_width = 1, param_inertia, param_inertia_end = param_inertia,
                             flow_memory = 0, flow_memory_end = flow_memory, shuffle = :each_epoch,

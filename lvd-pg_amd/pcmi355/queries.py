@@ -343,12 +343,14 @@ def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_r
     holds, so the statistics of an epoch pile up while the parameters move after every batch -- kept as written.)
     `fscale` other than 1: the flows of the tempered posterior (`scaled_probs_flows_circuit`,
     src-jl/learning/flow.jl:120-373), set on the handle for the length of the loop (`pcm_set_flow_scale`; an HCLT handle
-    runs them on its layered form).  soft_reg > 0 needs an HCLT handle on the block kernels (`pcm_set_soft_reg`) and,
-    for now, fscale = 1.
+    runs them on its layered form).  soft_reg > 0 with fscale = 1 needs an HCLT handle on the block kernels
+    (`pcm_set_soft_reg`); with fscale other than 1 the library turns every batch into the soft evidence that gives the
+    leaves the smoothed values, with tempered flows above them and the leaf flows in their "derivative" form --
+    `soft_flow = "as_written"` is the block kernels' and raises NotImplementedError there.
     Returns the per-epoch mean log-likelihoods."""
-    if fscale != 1.0 and soft_reg != 0.0:
-        raise NotImplementedError("soft_reg together with fscale other than 1: the smoothing runs in the block kernels, "
-                                  "the tempered flows on the layered engine")
+    if fscale != 1.0 and soft_reg != 0.0 and soft_flow == "as_written":
+        raise NotImplementedError("soft_flow = 'as_written' together with fscale other than 1: that form of the leaf flows "
+                                  "runs in the block kernels, the tempered flows on the layered engine")
     if not (fscale > 0 and np.isfinite(fscale)):
         raise ValueError("fscale must be positive and finite")
     _check_data(bpc, data)
@@ -367,6 +369,8 @@ def mini_batch_em_beta(bpc, data, num_epochs, *, batch_size, pseudocount, soft_r
         raise ValueError("batch_size must not exceed the number of examples")
     num_batches = n // batch_size
     smooth = soft_reg != 0.0
+    if smooth and not 0.0 < soft_reg < 1.0:
+        raise ValueError("soft_reg must lie in [0, 1)")
     if smooth:
         check(lib.pcm_set_soft_reg(bpc.handle, float(soft_reg), int(soft_reg_width), int(soft_flow == "as_written")))
     if fscale != 1.0:

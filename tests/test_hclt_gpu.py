@@ -919,9 +919,6 @@ def test_em_beta_driver_collects_statistics_over_an_interval(gpu, oracle, update
     for v, blk in th_ref.items():
         assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
     assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
-    with pytest.raises(NotImplementedError):      # the smoothing is the block kernels', the tempered flows the layered engine's
-        P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia, fscale=2.0,
-                             soft_reg=0.01, soft_reg_width=3)
     # the loop leaves the handle as it found it: an ordinary step afterwards runs on the block kernels again
     ll = P.probs_flows_circuit(bpc, torch.from_numpy(data[:B]).cuda()).cpu().numpy()
     assert rel_err(ll, oracle.forward(cur, data[:B], double=True)[-1]).max() < 1e-4

@@ -377,3 +377,63 @@ def test_soft_reg_routes_agree_and_as_written_needs_the_kernels(gpu):
     with pytest.raises(Exception):
         P.mini_batch_em_with_reg(odd, data[:, :6].contiguous(), 1, batch_size=B, pseudocount=0.01, soft_reg=s,
                                  soft_reg_width=width, param_inertia=0.9, shuffle="none", soft_flow="as_written")
+
+
+def _soft_reg_evidence_rows(batch, C, s, width):
+    """The log-evidence of a categorical batch under soft_reg (reg_likelihood.jl:4-14), category by category."""
+    B, V = batch.shape
+    ev = np.full((B, V, C), -np.inf)
+    for i in range(B):
+        for v in range(V):
+            x = int(batch[i, v])
+            c0 = max(0, x - width // 2)
+            c1 = min(c0 + width - 1, C - 1)
+            ev[i, v, c0:c1 + 1] = np.log(s / (c1 - c0 + 1))
+            ev[i, v, x] = np.log(np.exp(ev[i, v, x]) + 1 - s)
+    return ev
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fscale,update_interval", [(2.0, 2), (0.7, 1)])
+def test_em_beta_with_soft_reg_and_tempered_flows_matches_oracle(gpu, fscale, update_interval):
+    """`mini_batch_em_beta(...; soft_reg, soft_reg_width, fscale)` with both at once (src-jl/learning/em.jl:366-368 ->
+    flow.jl:366-372): the leaves take their smoothed values on the way up, the inner flows are those of the tempered
+    posterior, the leaves share their flow out as `soft_flow_params` does -- replayed on the float64 oracle batch by
+    batch.  `soft_flow = "as_written"` is the block kernels' form and is refused beside fscale != 1."""
+    torch, P = gpu
+    from helpers import correlated_data, rel_err
+    V, K, C, B, nb, pc, inertia, s, width = 9, 16, 12, 48, 4, 0.1, 0.8, 0.05, 3
+    parent, theta, leaf, fc = make_hclt(V, K, C, 21)
+    data = correlated_data(B * nb, V, C, 22, parent)
+    bpc = P.hclt_from_clt(parent, C, K)
+    bpc.set_params(block_theta(parent, K, theta), leaf)
+    lls = P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia,
+                               shuffle="none", update_interval=update_interval, fscale=fscale, soft_reg=s,
+                               soft_reg_width=width)
+    cur, ea, lf, tot = fc.copy(), None, None, 0.0
+    for batch_id in range(1, nb + 1):
+        batch = data[(batch_id - 1) * B:batch_id * B]
+        if ea is not None and batch_id % update_interval == 1:
+            ea, lf = ea * 0.0, lf * 0.0                                     # flow_memory = 0
+        mars = O.forward_soft(cur, _soft_reg_evidence_rows(batch, C, s, width), double=True)
+        flows, ea_b = O.backward(cur, mars, double=True, fscale=fscale)
+        lf_b = O.soft_flow_counts(cur, batch, flows, s, width, as_written=False, double=True)
+        ea = ea_b if ea is None else ea + ea_b
+        lf = lf_b if lf is None else lf + lf_b
+        tot += mars[-1].sum()
+        if batch_id % update_interval == 0:
+            logp, new_leaf, ea = O.em_update(cur, ea, lf, pc, inertia, True, return_aggr=True)
+            cur = cur.copy()
+            cur.logp, cur.leaf_logp = logp.astype(np.float32), new_leaf.astype(np.float32)
+    assert abs(lls[0] - tot / B / nb) < 2e-5 * abs(tot / B / nb)
+    th_ref, leaf_ref = O.hclt_block_params(cur)
+    th, lf_new = bpc.get_params()
+    for v, blk in th_ref.items():
+        assert rel_err(np.exp(th[v][:blk.shape[0]]), np.exp(blk)).max() < 5e-4
+    assert rel_err(np.exp(lf_new), np.exp(leaf_ref)).max() < 5e-4
+    with pytest.raises(NotImplementedError):
+        P.mini_batch_em_beta(bpc, torch.from_numpy(data).cuda(), 1, batch_size=B, pseudocount=pc, param_inertia=inertia,
+                             fscale=fscale, soft_reg=s, soft_reg_width=width, soft_flow="as_written")
+    # the loop leaves the handle as it found it: an ordinary pass afterwards runs on the block kernels again
+    ll = P.probs_flows_circuit(bpc, torch.from_numpy(data[:B]).cuda()).cpu().numpy()
+    assert rel_err(ll, O.forward(cur, data[:B], double=True)[-1]).max() < 1e-4
