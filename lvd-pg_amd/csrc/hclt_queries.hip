@@ -100,7 +100,7 @@ __global__ __launch_bounds__(256) void hclt_sample_states_node_kernel(const floa
       rec1 = rec2;
     }
   } else {
-    // K = 64: a row is scanned in two rounds of 32 values, its noise requested with it
+    // K = 64, 128: a row is scanned in rounds of 32 values, its noise requested with it
   int2 rec = passes_tab[lane];
     for (int ps = 0; ps < passes; ++ps) {
       const int n = rec.x, par = rec.y;
@@ -362,7 +362,7 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
   if (batch < 1) fail(PCM_ERR_ARG, "batch must be positive, got %d", batch);
   if ((reinterpret_cast<uintptr_t>(d_node_noise) | reinterpret_cast<uintptr_t>(d_leaf_noise)) & 15)
     fail(PCM_ERR_ARG, "noise pointers must be 16-byte aligned (rows are read as 16-byte words)");
-  const bool rows_fit = K_ >= 4 && K_ <= 64 && (K_ & (K_ - 1)) == 0;   // rows of whole 16-byte words, states in a byte
+  const bool rows_fit = K_ >= 4 && K_ <= 128 && (K_ & (K_ - 1)) == 0;   // rows of whole 16-byte words, states in a byte
   const int stride = (n_inner_ + 15) & ~15;   // bytes of one example's states in LDS
   const size_t st_bytes = (size_t)4 * stride;
   if (!rows_fit || st_bytes > (size_t)64 * 1024) {   // other hidden sizes: the layered engine's sampler
@@ -411,7 +411,8 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     case 8: node_states(&hclt_sample_states_node_kernel<8>); break;
     case 16: node_states(&hclt_sample_states_node_kernel<16>); break;
     case 32: node_states(&hclt_sample_states_node_kernel<32>); break;
-    default: node_states(&hclt_sample_states_node_kernel<64>); break;
+    case 64: node_states(&hclt_sample_states_node_kernel<64>); break;
+    default: node_states(&hclt_sample_states_node_kernel<128>); break;
   }
   // the variable's table in LDS when 64 KB hold it and its rows are whole 16-byte words
   const size_t lds = (size_t)K_ * (C_ + 4) * sizeof(float) + kLeafExamples;
