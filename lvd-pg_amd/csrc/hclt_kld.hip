@@ -318,8 +318,19 @@ __global__ __launch_bounds__(256) void hclt_adam_kernel(int64_t ns, const float*
     params[i] = p;
   }
   float s = expf(p);
+  if constexpr (K <= 64) {
 #pragma unroll
-  for (int o = K / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, K);
+    for (int o = K / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, K);
+  } else {   // K = 128: a group is two neighbouring waves of the workgroup
+    static_assert(K == 128, "a normalisation group is at most two waves");
+    __shared__ float half[4];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) s += __shfl_xor(s, o);
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) half[wave] = s;
+    __syncthreads();
+    s = half[wave & ~1] + half[wave | 1];
+  }
   if (live) logtheta[src[i]] = p - logf(s);
 }
 
@@ -603,7 +614,7 @@ void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, fl
                             float b2, float eps, int t) {
   no_forest("Adam");
   no_missing("Adam");
-  if (!block_) {
+  if (!block_ && !wide_) {
     general()->adam_step(d_grad, d_params, d_m, d_v, lr, b1, b2, eps, t);
     PCM_HIP(hipStreamSynchronize(stream));
     pull_from_general();
@@ -613,9 +624,13 @@ void HcltCircuit::adam_step(const float* d_grad, float* d_params, float* d_m, fl
   if (t < 1) fail(PCM_ERR_ARG, "step count must start at 1, got %d", t);
   const int64_t ns = (int64_t)sum_param_src_.size();
   const float c1 = 1.f - std::pow(b1, (float)t), c2 = 1.f - std::pow(b2, (float)t);
-  PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_adam_kernel<KK>, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
-                                        d_grad, d_params, d_m, d_v, lr, b1, b2, eps, c1, c2, d_sum_param_src_.p,
-                                        d_logtheta_.p));
+  if (wide_)
+    hipLaunchKernelGGL(hclt_adam_kernel<128>, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns, d_grad, d_params, d_m,
+                       d_v, lr, b1, b2, eps, c1, c2, d_sum_param_src_.p, d_logtheta_.p);
+  else
+    PCM_DISPATCH_K(K_, hipLaunchKernelGGL(hclt_adam_kernel<KK>, dim3((unsigned)ceil_div(ns, 256)), dim3(256), 0, stream, ns,
+                                          d_grad, d_params, d_m, d_v, lr, b1, b2, eps, c1, c2, d_sum_param_src_.p,
+                                          d_logtheta_.p));
   check_launch_k("hclt_adam");
   rebuild_w();
   general_stale_ = true;

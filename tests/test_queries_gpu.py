@@ -244,7 +244,7 @@ def test_adam_step_matches_oracle(gpu, oracle):
     from helpers import make_hclt, block_theta, random_dag, rel_err
     V, C = 6, 5
     hcs = []
-    for K in (16, 32, 64, 8):
+    for K in (16, 32, 64, 128, 8):
         parent, theta, leaf, fc = make_hclt(V, K, C, 41)
         hc = P.hclt_from_clt(parent, C, K)
         hc.set_params(block_theta(parent, K, theta), leaf)
