@@ -414,9 +414,12 @@ void HcltCircuit::sample(const float* d_node_noise, const float* d_leaf_noise, i
     case 64: node_states(&hclt_sample_states_node_kernel<64>); break;
     default: node_states(&hclt_sample_states_node_kernel<128>); break;
   }
-  // the variable's table in LDS when 64 KB hold it and its rows are whole 16-byte words
+  // the variable's table in LDS when the 160 KB of a compute unit hold it and its rows are whole 16-byte words
   const size_t lds = (size_t)K_ * (C_ + 4) * sizeof(float) + kLeafExamples;
-  if ((C_ & 3) == 0 && (K_ & 3) == 0 && lds <= (size_t)64 * 1024) {
+  if ((C_ & 3) == 0 && (K_ & 3) == 0 && lds <= (size_t)160 * 1024) {
+    if (lds > (size_t)64 * 1024)
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&hclt_sample_leaves_lds_kernel),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     // (leaves: the caller's variables, which come first; the auxiliary ones have nothing to draw)
     hipLaunchKernelGGL(hclt_sample_leaves_lds_kernel, dim3(Vu_, ceil_div(batch, kLeafExamples)), dim3(kLeafWaves * 64), lds,
                        stream, d_leaf_.p, d_sample_tabs_.p + n_inner_, d_state_.p, d_leaf_noise, Vu_, K_, C_, n_inner_, batch,

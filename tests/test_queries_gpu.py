@@ -188,7 +188,8 @@ def test_sampling_bit_exact_random_dag(gpu, oracle, V, C, width, B, seed):
 @pytest.mark.parametrize("V,K,C,B,tree", [
     (7, 16, 8, 130, None), (12, 32, 256, 64, None), (10, 64, 5, 70, None), (9, 4, 6, 50, None), (6, 2, 3, 40, None),
     (6, 16, 36, 1030, None),                                     # three blocks of examples, the last one ragged
-    (7, 128, 8, 45, None), (5, 128, 128, 20, None),              # K = 128: block sampler, leaf table in LDS or not
+    (7, 128, 8, 45, None), (5, 128, 128, 20, None),              # K = 128: block sampler; 6 KB and 68 KB of leaf table in LDS
+    (5, 64, 256, 70, None), (3, 128, 252, 30, None),             # 67 KB and 131 KB
     (141, 8, 3, 33, [-1] + [0] * 70 + list(range(1, 71))),       # a level of more than 64 tree nodes
     (13, 16, 6, 50, [-1, 0, 1, 1, 1, 1, 2, 3, 0, 8, 8, 8, 8]),   # four children twice: split for the walks, the noise
     (11, 32, 5, 40, [-1, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5])])        # stays indexed by the caller's tree nodes
