@@ -407,6 +407,31 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_forward_kernel(Sparse
     if (b0 + 64 * x < d.Bp) d.mars[(size_t)n * d.Bp + b0 + 64 * x] = sum[x] == 1.f ? m[x] : m[x] + __logf(sum[x]);
 }
 
+// The input layer on categorical data when it holds thousands of nodes: a wave takes one input node through the whole
+// batch, four examples a lane and request (a packed word of categories, four table entries, one 16-byte store) and
+// four requests in flight, instead of the layer kernel's one wave per (node, 256 examples) with its three dependent
+// round trips each (sixteen 192-variable K = 32 circuits as one, 1024 examples: 196 -> 135 us).
+__global__ __launch_bounds__(256) void sparse_input_kernel(SparseDev d, int n0, int cnt) {
+  const int lane = threadIdx.x & 63;
+  const int i = blockIdx.x * 4 + (int)(threadIdx.x >> 6);
+  if (i >= cnt) return;
+  const int n = uni(d.fwd_rec[n0 + i].x);
+  const uchar4* xr4 = reinterpret_cast<const uchar4*>(d.xb + (size_t)uni(d.in_var[n]) * d.Bp);
+  const int64_t off = d.in_off[n];
+  const float* row = d.leaf + (((int64_t)uni((int)(off >> 32)) << 32) | (uint32_t)uni((int)off));
+  float4* out = reinterpret_cast<float4*>(d.mars + (size_t)n * d.Bp);
+  const int n4 = d.Bp / 4;   // (rows are padded to 64 examples, the padding holds categories like any other)
+  constexpr int U = 4;
+  for (int q0 = lane; q0 < n4; q0 += 64 * U) {
+    uchar4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) x[u] = xr4[min(q0 + 64 * u, n4 - 1)];
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+      if (q0 + 64 * u < n4) out[q0 + 64 * u] = make_float4(row[x[u].x], row[x[u].y], row[x[u].z], row[x[u].w]);
+  }
+}
+
 // Sum over the 64 lanes of a wave, valid in every lane: butterflies inside rows of 16 lanes
 // with data-parallel-primitive moves (lane ^ 1, lane ^ 2, mirror of 8, mirror of 16), then the
 // four row sums through scalar registers.
@@ -609,36 +634,78 @@ __global__ __launch_bounds__(kLayerWaves * 64) void sparse_backward_kernel(Spars
 }
 
 // Leaf counters, src/nodes/fixable_categorical_dist.jl:121-130: an input node's flow goes to the
-// counter of the example's category.  One workgroup per input node over the whole batch: the
-// node owns its C counters.  They are summed in LDS as 64-bit fixed-point integers, scaled so that
-// the node's largest flow times the batch size still fits: integer sums do not depend on the order
-// the lanes arrive in, so the counters come out the same on every run.
+// counter of the example's category.  NT threads per input node over the whole batch -- a workgroup (NT = 256) where
+// there are few nodes, a wave (NT = 64, four nodes per workgroup and no workgroup barrier: a wave's LDS operations
+// execute in order) where there are thousands and a node's 1024 examples are four per thread: the node owns its C
+// counters.  They are summed in LDS as 64-bit fixed-point integers, scaled so that the node's largest flow times the
+// batch size still fits: integer sums do not depend on the order the lanes arrive in, so the counters come out the
+// same on every run and under either NT.
+template <int NT>
 __global__ __launch_bounds__(256) void sparse_leaf_flow_kernel(SparseDev d, const int32_t* __restrict__ input_nodes,
-                                                               float* __restrict__ leaf_flow) {
-  __shared__ unsigned long long hist[256];
+                                                               int n_input_nodes, float* __restrict__ leaf_flow) {
+  constexpr int G = 256 / NT;   // nodes per workgroup
+  __shared__ unsigned long long hist_all[G][256];
   __shared__ float wave_max[4];
-  const int n = input_nodes[blockIdx.x];
-  for (int c = threadIdx.x; c < d.C; c += blockDim.x) hist[c] = 0ull;
+  const int grp = threadIdx.x / NT, t = threadIdx.x % NT;
+  const int at = blockIdx.x * G + grp;
+  if (at >= n_input_nodes) return;   // (NT = 64: a whole wave; NT = 256: never)
+  unsigned long long* hist = hist_all[grp];
+  const int n = input_nodes[at];
+  for (int c = t; c < d.C; c += NT) hist[c] = 0ull;
   const uint8_t* xr = d.xb + (size_t)d.in_var[n] * d.Bp;
   const float* fr = d.flows + (size_t)n * d.Bp;
+  // (rows are padded to whole 16-byte words; four words requested before the first is used: a loop of single
+  // dependent loads made this kernel wait out sixteen memory latencies per node and pass)
+  constexpr int U = 4;
+  const float4* fr4 = reinterpret_cast<const float4*>(fr);
+  const uchar4* xr4 = reinterpret_cast<const uchar4*>(xr);
+  const int n4 = d.Bp / 4;
   float mx = 0.f;
-  for (int b = threadIdx.x; b < d.B; b += blockDim.x) mx = fmaxf(mx, fr[b]);
+  for (int q0 = t; q0 < n4; q0 += NT * U) {
+    float4 f[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) f[u] = fr4[min(q0 + u * NT, n4 - 1)];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int b0 = (q0 + u * NT) * 4;   // (past the batch: not counted)
+      if (b0 < d.B) mx = fmaxf(mx, f[u].x);
+      if (b0 + 1 < d.B) mx = fmaxf(mx, f[u].y);
+      if (b0 + 2 < d.B) mx = fmaxf(mx, f[u].z);
+      if (b0 + 3 < d.B) mx = fmaxf(mx, f[u].w);
+    }
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-  if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
-  __syncthreads();
-  mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-  if (!(mx > 0.f)) return;                       // no flow reached this node (uniform over the workgroup)
+  if constexpr (NT == 256) {
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  }
+  if (!(mx > 0.f)) return;                       // no flow reached this node (uniform over the node's threads)
   int ex = 0;
   frexpf(mx, &ex);                               // every flow < 2^ex
   const int shift = 62 - (32 - __clz(d.B)) - ex; // flow * 2^shift < 2^62 / batch
-  for (int b = threadIdx.x; b < d.B; b += blockDim.x) {
-    const float f = fr[b];
-    if (f > 0.f) atomicAdd(&hist[xr[b]], (unsigned long long)ldexpf(f, shift));
+  for (int q0 = t; q0 < n4; q0 += NT * U) {
+    float4 f[U];
+    uchar4 x[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      f[u] = fr4[min(q0 + u * NT, n4 - 1)];
+      x[u] = xr4[min(q0 + u * NT, n4 - 1)];
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int b0 = (q0 + u * NT) * 4;
+      if (b0 < d.B && f[u].x > 0.f) atomicAdd(&hist[x[u].x], (unsigned long long)ldexpf(f[u].x, shift));
+      if (b0 + 1 < d.B && f[u].y > 0.f) atomicAdd(&hist[x[u].y], (unsigned long long)ldexpf(f[u].y, shift));
+      if (b0 + 2 < d.B && f[u].z > 0.f) atomicAdd(&hist[x[u].z], (unsigned long long)ldexpf(f[u].z, shift));
+      if (b0 + 3 < d.B && f[u].w > 0.f) atomicAdd(&hist[x[u].w], (unsigned long long)ldexpf(f[u].w, shift));
+    }
   }
-  __syncthreads();
+  if constexpr (NT == 256) __syncthreads();
+  else __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
   float* dst = leaf_flow + d.in_off[n];
-  for (int c = threadIdx.x; c < d.C; c += blockDim.x) dst[c] += ldexpf((float)hist[c], -shift);
+  for (int c = t; c < d.C; c += NT) dst[c] += ldexpf((float)hist[c], -shift);
 }
 
 // Soft evidence, per variable.  All input nodes of a variable read the same evidence, so a
@@ -794,10 +861,27 @@ __global__ __launch_bounds__(256) void sparse_update_kernel(SparseDev d, int n_n
   } else if (type == kInput) {
     float* lp = leaf + d.in_off[n];
     const float* fl = leaf_flow + d.in_off[n];
+    const float cat_pc = pseudocount / (float)d.C;
+    if ((d.C & 3) == 0 && d.C <= 256) {
+      // a node's row as one 16-byte word per lane, the parameters requested together with the flows: the loops below
+      // are a chain of a dozen dependent round trips per node, and a circuit has a hundred thousand of these nodes
+      const int c = 4 * lane;
+      float4 f = make_float4(0.f, 0.f, 0.f, 0.f), l = f;
+      if (c < d.C) {
+        f = *reinterpret_cast<const float4*>(fl + c);
+        l = *reinterpret_cast<const float4*>(lp + c);
+      }
+      const float node_flow = wave_sum((f.x + f.y) + (f.z + f.w)) + pseudocount;
+      if (c < d.C)
+        *reinterpret_cast<float4*>(lp + c) = make_float4(logf(inertia * expf(l.x) + (1.f - inertia) * (f.x + cat_pc) / node_flow),
+                                                         logf(inertia * expf(l.y) + (1.f - inertia) * (f.y + cat_pc) / node_flow),
+                                                         logf(inertia * expf(l.z) + (1.f - inertia) * (f.z + cat_pc) / node_flow),
+                                                         logf(inertia * expf(l.w) + (1.f - inertia) * (f.w + cat_pc) / node_flow));
+      return;
+    }
     float node_flow = 0.f;
     for (int c = lane; c < d.C; c += 64) node_flow += fl[c];
     node_flow = wave_sum(node_flow) + pseudocount;
-    const float cat_pc = pseudocount / (float)d.C;
     for (int c = lane; c < d.C; c += 64)
       lp[c] = logf(inertia * expf(lp[c]) + (1.f - inertia) * (fl[c] + cat_pc) / node_flow);
   }
@@ -1039,12 +1123,23 @@ __global__ __launch_bounds__(64 * kMixGroups) void sparse_head_mixture_kernel(co
   const int b = blockIdx.x * 64 + lane;
   float mx = -INFINITY, sm = 0.f, tot = 0.f;
   if (b < B)
-    for (int h = g; h < n_heads; h += kMixGroups) {
-      const float m = mask[(size_t)h * B + b];
-      const float t = mars[(size_t)heads[h] * Bp + b] + logf(m);
-      tot += m;
-      if (t > mx) { sm = sm * expf(mx - t) + 1.f; mx = t; }
-      else if (t > -INFINITY) sm += expf(t - mx);
+    for (int h0 = g; h0 < n_heads; h0 += kMixGroups * 4) {   // four heads' requests before the first is folded in
+      float m4[4], v4[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int h = min(h0 + u * kMixGroups, n_heads - 1);
+        m4[u] = mask[(size_t)h * B + b];
+        v4[u] = mars[(size_t)heads[h] * Bp + b];
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (h0 + u * kMixGroups >= n_heads) break;
+        const float m = m4[u];
+        const float t = v4[u] + logf(m);
+        tot += m;
+        if (t > mx) { sm = sm * expf(mx - t) + 1.f; mx = t; }
+        else if (t > -INFINITY) sm += expf(t - mx);
+      }
     }
   pm[g][lane] = mx; ps[g][lane] = sm; pt[g][lane] = tot;
   __syncthreads();
@@ -1518,6 +1613,7 @@ SparseCircuit::SparseCircuit(FlatCircuit fc) : fc_(std::move(fc)) {
         const int32_t n = order[i];
         if (group_of[n] >= 0 || grp_expanded_[n]) continue;
         fr.push_back(int4{n, (int)fc_.type[n], fc_.node_e0[n], fc_.node_e1[n]});
+        if (l == 0 && fc_.type[n] != kInput) layer0_inputs_only_ = false;
         if (fc_.type[n] != kInput) layer_max_children_[l] = std::max(layer_max_children_[l], (int)(fc_.node_e1[n] - fc_.node_e0[n]));
       }
       fwd_layer0_[l + 1] = (int)fr.size();
@@ -1769,6 +1865,10 @@ void SparseCircuit::run_forward(const BatchRef* b, const SoftRef* s) {
     launch_groups(l, 0, Bp, batch);
     if (cnt == 0) continue;
     const int64_t pairs = (int64_t)cnt * (Bp / 64);
+    if (l == 0 && layer0_inputs_only_ && cnt >= 4096) {
+      if (!s) hipLaunchKernelGGL(sparse_input_kernel, dim3(ceil_div(cnt, 4)), dim3(256), 0, stream, d, n0, cnt);
+      continue;   // (soft evidence: sparse_soft_input_kernel has filled the input rows)
+    }
     if (layer_max_children_[l] <= kNarrowDegree) {
       if (pairs < kManyPairs) PCM_LAYER_LAUNCH(sparse_forward_kernel, 1, 1, 4, dim3(cnt, Bp / 64), d, n0);
       else PCM_LAYER_LAUNCH(sparse_forward_kernel, 4, 1, 4, dim3(cnt, ceil_div(Bp, 256)), d, n0);
@@ -1911,8 +2011,15 @@ void SparseCircuit::run_flows(int batch, const SoftRef* soft, float rate, const 
                          dim3(fc_.num_vars, ceil_div(fc_.num_cats, kSoftTile), ceil_div(max_var_nodes_, 4 * kFlowNodes)), dim3(256), 0,
                          stream, d, d_var_ptr_.p, d_var_nodes_.p, d_leaf_flow_.p);
     else
-      hipLaunchKernelGGL(sparse_leaf_flow_kernel, dim3((unsigned)fc_.input_nodes.size()), dim3(256), 0, stream, d,
-                         d_input_nodes_.p, d_leaf_flow_.p);
+    {
+      const int n_in = (int)fc_.input_nodes.size();
+      if (n_in >= 4096 && batch <= 16384)   // (a wave per node: enough nodes to fill the device four to a workgroup)
+        hipLaunchKernelGGL(sparse_leaf_flow_kernel<64>, dim3((unsigned)ceil_div(n_in, 4)), dim3(256), 0, stream, d,
+                           d_input_nodes_.p, n_in, d_leaf_flow_.p);
+      else
+        hipLaunchKernelGGL(sparse_leaf_flow_kernel<256>, dim3((unsigned)n_in), dim3(256), 0, stream, d, d_input_nodes_.p, n_in,
+                           d_leaf_flow_.p);
+    }
   }
   check_launch("sparse_backward");
   if (fc_.heads.empty()) {

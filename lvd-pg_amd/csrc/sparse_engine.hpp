@@ -133,6 +133,7 @@ class SparseCircuit : public pcm_circuit {
   bool launch_group_walk(const GroupRun& r, bool forward, int Bp, int batch, bool tempered);
   std::vector<GroupLaunch> group_stat_launches_;   // per shape: ranges of d_grp_order_ (layer and bases unused)
   std::vector<int> fwd_layer0_;               // ranges of d_fwd_rec_ per layer: the nodes no group computes
+  bool layer0_inputs_only_ = true;            // the first layer holds input nodes and nothing else
   int64_t n_layer_nodes_ = 0;                 // nodes whose values the layer kernels compute (the others: the groups')
   int64_t n_group_slots_ = 0, n_groups_ = 0, n_group_elems_ = 0;   // children of all groups; groups; padded W entries
   DevBuf<int32_t> d_grp_node_, d_grp_edge_, d_grp_own_, d_grp_elem_, d_grp_order_;

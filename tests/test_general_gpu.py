@@ -690,7 +690,8 @@ def _check_grouped_multihead(gpu, O, heads, V, C, B, seed, min_groups):
 
 @pytest.mark.parametrize("V,K,C,H,B,max_children,seed", [(20, 8, 5, 9, 150, 5, 31), (9, 32, 4, 40, 64, 2, 32),
                                                          (33, 12, 3, 6, 333, 3, 33), (40, 16, 4, 7, 100, 3, 34),
-                                                         (12, 64, 3, 5, 50, 2, 35)])
+                                                         (12, 64, 3, 5, 50, 2, 35),
+                                                         (130, 32, 4, 6, 101, 3, 36)])   # 4160 input nodes: a wave per node
 def test_dense_groups_of_a_multihead_hclt(gpu, oracle, V, K, C, H, B, max_children, seed):
     """An HCLT's K sums per tree node and the heads over the root's products are groups; products of up to three
     children are taken apart by the groups above them, those of more stay nodes of a layer."""
