@@ -88,9 +88,31 @@ __device__ __forceinline__ void mi_each_example(const uint8_t* __restrict__ xu, 
   }
 }
 
-// Sum of acc over the workgroup, then the closed-form remainder; thread 0 writes both halves of the matrix.
+// The same with the words of the thread's first four examples already in registers (w0u, w0v): a pair's three passes
+// read them once, and the next pair's are requested while this pair's passes run -- a persistent workgroup owns its
+// compute unit (the table fills the LDS), so nothing else hides the latency of its rows.
+template <typename F>
+__device__ __forceinline__ void mi_each_example_from(uint32_t w0u, uint32_t w0v, const uint8_t* __restrict__ xu,
+                                                     const uint8_t* __restrict__ xv, int N, int t, F&& fn) {
+  uint32_t wu = w0u, wv = w0v;
+  for (int64_t b4 = 4 * (int64_t)t; b4 < N; b4 += 4 * kMiThreads) {
+    if (b4 != 4 * (int64_t)t) {
+      wu = *reinterpret_cast<const uint32_t*>(xu + b4);
+      wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (b4 + i < N) fn((int)((wu >> (8 * i)) & 0xffu), (int)((wv >> (8 * i)) & 0xffu));
+  }
+}
+
+// Sum of acc over the workgroup, then the closed-form remainder; thread 0 writes both halves of the matrix.  su, sv: the
+// two variables' constants (M, L), read when the pair began -- read here they kept the whole workgroup waiting for
+// thread 0's trip to memory.  No barrier behind thread 0: whoever writes `red` next has passed a barrier that thread 0
+// reaches only after this.
+struct MiStat { double m, l; };
 __device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, int u, int v, int V, int C, double p0, double x0,
-                                               const double* __restrict__ stat, float* __restrict__ mi) {
+                                               MiStat su, MiStat sv, float* __restrict__ mi) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
   if ((t & 63) == 0) red[t >> 6] = acc;
@@ -98,49 +120,69 @@ __device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, i
   if (t == 0) {
     double tot = 0.0;
     for (int w = 0; w < kMiThreads / 64; ++w) tot += red[w];
-    double val = tot - stat[2 * u] - stat[2 * v] + (double)C * C * x0;
-    if (p0 > 0.0) val -= p0 * C * (stat[2 * u + 1] + stat[2 * v + 1]);
+    double val = tot - su.m - sv.m + (double)C * C * x0;
+    if (p0 > 0.0) val -= p0 * C * (su.l + sv.l);
     mi[(size_t)u * V + v] = (float)val;
     mi[(size_t)v * V + u] = (float)val;
   }
-  __syncthreads();
 }
 
 // Pairs (u <= v) in row-major order of the upper triangle, dealt round-robin to persistent
 // workgroups.  At most 65535 examples: a cell's count fits 16 bits, two cells per LDS word.
 __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V, int C,
-                                                             float pc, const double* __restrict__ f,
+                                                             float pc, const double* __restrict__ f, int f_lds,
                                                              const double* __restrict__ stat, float* __restrict__ mi) {
-  extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 doubles
+  extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 doubles | the first f_lds entries of f
   const int t = threadIdx.x;
   const int words = (C * C + 1) / 2;
   double* red = reinterpret_cast<double*>(cells + ((words + 1) & ~1));
-  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;
+  double* fl = red + kMiThreads / 64;   // what the LDS has left holds the table over counts from its start: a lookup per
+  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;   // example is then no trip to memory (counts past it are rare)
+  for (int i = t; i < f_lds; i += kMiThreads) fl[i] = f[i];
   __syncthreads();
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
   const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
   const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
   // row u of the triangle starts at pair u*V - u*(u-1)/2
-  int u = 0;
-  int64_t row0 = 0;
+  int u = 0, un = 0;          // rows of this pair and of the workgroup's next one
+  int64_t row0 = 0, rown = 0;
+  const int64_t first = 4 * (int64_t)min(t, (N - 1) / 4);   // (the rows are padded to whole words past N)
+  uint32_t cu = 0u, cv = 0u;
+  if ((int64_t)blockIdx.x < n_pairs) {
+    while ((int64_t)blockIdx.x >= rown + (V - un)) { rown += V - un; ++un; }
+    cu = *reinterpret_cast<const uint32_t*>(xb + (size_t)un * Np + first);
+    cv = *reinterpret_cast<const uint32_t*>(xb + (size_t)(un + (int)(blockIdx.x - rown)) * Np + first);
+  }
   for (int64_t p = blockIdx.x; p < n_pairs; p += gridDim.x) {
     while (p >= row0 + (V - u)) { row0 += V - u; ++u; }
     const int v = u + (int)(p - row0);
     const uint8_t* xu = xb + (size_t)u * Np;
     const uint8_t* xv = xb + (size_t)v * Np;
+    const MiStat su{stat[2 * u], stat[2 * u + 1]}, sv{stat[2 * v], stat[2 * v + 1]};
     double acc = 0.0;
-    mi_each_example(xu, xv, N, t, [&](int a, int b) {
+    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) {
       const int key = a * C + b;
       atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
     });
+    // the next pair's first words, on their way while this pair is looked up and cleared
+    uint32_t nu = 0u, nv = 0u;
+    const int64_t pn = p + gridDim.x;
+    if (pn < n_pairs) {
+      while (pn >= rown + (V - un)) { rown += V - un; ++un; }
+      nu = *reinterpret_cast<const uint32_t*>(xb + (size_t)un * Np + first);
+      nv = *reinterpret_cast<const uint32_t*>(xb + (size_t)(un + (int)(pn - rown)) * Np + first);
+    }
     __syncthreads();
-    mi_each_example(xu, xv, N, t, [&](int a, int b) {
+    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) {
       const int key = a * C + b;
-      acc += f[(cells[key >> 1] >> (16 * (key & 1))) & 0xffffu];
+      const int cnt = (int)((cells[key >> 1] >> (16 * (key & 1))) & 0xffffu);
+      acc += cnt < f_lds ? fl[cnt] : f[cnt];
     });
     __syncthreads();
-    mi_each_example(xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
-    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, stat, mi);
+    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
+    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, su, sv, mi);
+    cu = nu;
+    cv = nv;
   }
 }
 
@@ -166,6 +208,7 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_wide_kernel(const uint8_t*
     const int v = u + (int)(p - row0);
     const uint8_t* xu = xb + (size_t)u * Np;
     const uint8_t* xv = xb + (size_t)v * Np;
+    const MiStat su{stat[2 * u], stat[2 * u + 1]}, sv{stat[2 * v], stat[2 * v + 1]};
     double acc = 0.0;
     for (int a0 = 0; a0 < C; a0 += band) {
       mi_each_example(xu, xv, N, t, [&](int a, int b) {
@@ -181,7 +224,7 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_wide_kernel(const uint8_t*
       });
       __syncthreads();
     }
-    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, stat, mi);
+    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, su, sv, mi);
   }
 }
 
@@ -212,9 +255,14 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
   const bool narrow = N <= 65535;
   int band = C;
   size_t lds;
+  int f_lds = 0;
   if (narrow) {
     const int words = (C * C + 1) / 2;
     lds = ((size_t)((words + 1) & ~1)) * 4 + red_bytes;
+    // the rest of the LDS -- of half of it where two workgroups fit a compute unit -- holds the start of the f table
+    const size_t whole = std::min<size_t>((size_t)max_lds, 160 * 1024), share = lds <= whole / 4 ? whole / 2 : whole;
+    f_lds = (int)std::min<size_t>((size_t)N + 1, (share - lds) / sizeof(double));
+    lds += (size_t)f_lds * sizeof(double);
   } else {
     const size_t budget = std::min<size_t>((size_t)max_lds, 160 * 1024) - red_bytes - 8;
     band = (int)std::min<size_t>((size_t)C, budget / ((size_t)C * 4));
@@ -233,7 +281,7 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)lds));
     hipLaunchKernelGGL(mi_pair_kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.f,
-                       w.stat, d_mi);
+                       f_lds, w.stat, d_mi);
   } else {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_wide_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
