@@ -88,18 +88,40 @@ __device__ __forceinline__ void mi_each_example(const uint8_t* __restrict__ xu, 
   }
 }
 
-// The same with the words of the thread's first four examples already in registers (w0u, w0v): a pair's three passes
-// read them once, and the next pair's are requested while this pair's passes run -- a persistent workgroup owns its
-// compute unit (the table fills the LDS), so nothing else hides the latency of its rows.
-template <typename F>
-__device__ __forceinline__ void mi_each_example_from(uint32_t w0u, uint32_t w0v, const uint8_t* __restrict__ xu,
-                                                     const uint8_t* __restrict__ xv, int N, int t, F&& fn) {
-  uint32_t wu = w0u, wv = w0v;
-  for (int64_t b4 = 4 * (int64_t)t; b4 < N; b4 += 4 * kMiThreads) {
-    if (b4 != 4 * (int64_t)t) {
-      wu = *reinterpret_cast<const uint32_t*>(xu + b4);
-      wv = *reinterpret_cast<const uint32_t*>(xv + b4);
+// The same with the words of the thread's first R rounds already in registers (R = 1, 2, 4 or 8: the host picks the
+// smallest that covers the examples; rounds are masked, not branched around): a pair's three passes read them
+// once, all of them requested before the first is used (a loop of a load and its use per round waits out one memory
+// latency per round and pass), and the next pair's are requested while this pair's passes run -- a persistent workgroup
+// owns its compute unit (the table fills the LDS), so nothing else hides the latency of its rows.
+template <int R>
+struct MiWords { uint32_t u[R], v[R]; };
+
+template <int R>
+__device__ __forceinline__ void mi_load_words(const uint8_t* __restrict__ xu, const uint8_t* __restrict__ xv, int N, int t,
+                                              MiWords<R>& w) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t b4 = 4 * (int64_t)t + (int64_t)r * 4 * kMiThreads;
+    w.u[r] = w.v[r] = 0u;
+    if (b4 < N) {   // (the rows are padded to whole words past N)
+      w.u[r] = *reinterpret_cast<const uint32_t*>(xu + b4);
+      w.v[r] = *reinterpret_cast<const uint32_t*>(xv + b4);
     }
+  }
+}
+
+template <int R, typename F>
+__device__ __forceinline__ void mi_each_example_from(const MiWords<R>& w, const uint8_t* __restrict__ xu,
+                                                     const uint8_t* __restrict__ xv, int N, int t, F&& fn) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int64_t b4 = 4 * (int64_t)t + (int64_t)r * 4 * kMiThreads;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (b4 + i < N) fn((int)((w.u[r] >> (8 * i)) & 0xffu), (int)((w.v[r] >> (8 * i)) & 0xffu));
+  }
+  for (int64_t b4 = 4 * (int64_t)t + (int64_t)R * 4 * kMiThreads; b4 < N; b4 += 4 * kMiThreads) {
+    const uint32_t wu = *reinterpret_cast<const uint32_t*>(xu + b4), wv = *reinterpret_cast<const uint32_t*>(xv + b4);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
       if (b4 + i < N) fn((int)((wu >> (8 * i)) & 0xffu), (int)((wv >> (8 * i)) & 0xffu));
@@ -129,6 +151,7 @@ __device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, i
 
 // Pairs (u <= v) in row-major order of the upper triangle, dealt round-robin to persistent
 // workgroups.  At most 65535 examples: a cell's count fits 16 bits, two cells per LDS word.
+template <int R>
 __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V, int C,
                                                              float pc, const double* __restrict__ f, int f_lds,
                                                              const double* __restrict__ stat, float* __restrict__ mi) {
@@ -146,12 +169,10 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
   // row u of the triangle starts at pair u*V - u*(u-1)/2
   int u = 0, un = 0;          // rows of this pair and of the workgroup's next one
   int64_t row0 = 0, rown = 0;
-  const int64_t first = 4 * (int64_t)min(t, (N - 1) / 4);   // (the rows are padded to whole words past N)
-  uint32_t cu = 0u, cv = 0u;
+  MiWords<R> cur, nxt;
   if ((int64_t)blockIdx.x < n_pairs) {
     while ((int64_t)blockIdx.x >= rown + (V - un)) { rown += V - un; ++un; }
-    cu = *reinterpret_cast<const uint32_t*>(xb + (size_t)un * Np + first);
-    cv = *reinterpret_cast<const uint32_t*>(xb + (size_t)(un + (int)(blockIdx.x - rown)) * Np + first);
+    mi_load_words(xb + (size_t)un * Np, xb + (size_t)(un + (int)(blockIdx.x - rown)) * Np, N, t, cur);
   }
   for (int64_t p = blockIdx.x; p < n_pairs; p += gridDim.x) {
     while (p >= row0 + (V - u)) { row0 += V - u; ++u; }
@@ -160,29 +181,26 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
     const uint8_t* xv = xb + (size_t)v * Np;
     const MiStat su{stat[2 * u], stat[2 * u + 1]}, sv{stat[2 * v], stat[2 * v + 1]};
     double acc = 0.0;
-    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) {
+    mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) {
       const int key = a * C + b;
       atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
     });
-    // the next pair's first words, on their way while this pair is looked up and cleared
-    uint32_t nu = 0u, nv = 0u;
+    // the next pair's words, on their way while this pair is looked up and cleared
     const int64_t pn = p + gridDim.x;
     if (pn < n_pairs) {
       while (pn >= rown + (V - un)) { rown += V - un; ++un; }
-      nu = *reinterpret_cast<const uint32_t*>(xb + (size_t)un * Np + first);
-      nv = *reinterpret_cast<const uint32_t*>(xb + (size_t)(un + (int)(pn - rown)) * Np + first);
+      mi_load_words(xb + (size_t)un * Np, xb + (size_t)(un + (int)(pn - rown)) * Np, N, t, nxt);
     }
     __syncthreads();
-    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) {
+    mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) {
       const int key = a * C + b;
       const int cnt = (int)((cells[key >> 1] >> (16 * (key & 1))) & 0xffffu);
       acc += cnt < f_lds ? fl[cnt] : f[cnt];
     });
     __syncthreads();
-    mi_each_example_from(cu, cv, xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
+    mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
     mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, su, sv, mi);
-    cu = nu;
-    cv = nv;
+    cur = nxt;
   }
 }
 
@@ -278,10 +296,16 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
   const int per_cu = std::max<int>(1, (int)(std::min<size_t>((size_t)max_lds, 160 * 1024) / lds));
   const int grid = (int)std::min<int64_t>(n_pairs, (int64_t)cus * std::min(per_cu, 2));
   if (narrow) {
-    PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds));
-    hipLaunchKernelGGL(mi_pair_kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.f,
-                       f_lds, w.stat, d_mi);
+    auto pairs = [&](auto kernel) {
+      PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.f, f_lds, w.stat,
+                         d_mi);
+    };
+    // rounds of 4 * kMiThreads examples whose words a thread keeps in registers
+    if (N <= 4 * kMiThreads) pairs(&mi_pair_kernel<1>);
+    else if (N <= 8 * kMiThreads) pairs(&mi_pair_kernel<2>);
+    else if (N <= 16 * kMiThreads) pairs(&mi_pair_kernel<4>);
+    else pairs(&mi_pair_kernel<8>);
   } else {
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_wide_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

@@ -101,7 +101,7 @@ def gpu():
 @pytest.mark.gpu
 @pytest.mark.parametrize("N,V,C,pc", [(300, 7, 5, 0.1), (1000, 9, 16, 0.0), (4097, 6, 256, 0.1), (64, 3, 2, 1.0),
                                       (5000, 4, 200, 0.1), (65535, 3, 256, 0.1), (65536, 3, 256, 0.1), (70001, 4, 256, 0.1),
-                                      (140000, 3, 7, 0.0), (66000, 3, 200, 0.1)])
+                                      (140000, 3, 7, 0.0), (66000, 3, 200, 0.1), (12000, 5, 64, 0.1), (30000, 3, 256, 0.1)])
 def test_pairwise_mi_matches_oracle(gpu, N, V, C, pc):
     """Tolerance: 1e-4 of the largest entry (float32 output of float64 sums).  Beyond 65535 examples
     the cells are counted in 32 bits, band by band of the first variable's categories (two bands at
