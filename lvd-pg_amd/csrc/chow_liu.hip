@@ -10,11 +10,11 @@
 // The reference fills a dense [V][V][C][C] table with float atomics and reduces it on the host.
 // Here a pair never leaves the workgroup.  With c(a,b) the count of a cell, s = pc/C^2,
 // p(c) = (c + s)/Z, la[u][a] = log P_u[a]:
-//   MI[u,v] = sum over examples e of f(c(cell of e))  -  M_u - M_v  +  C^2 * xlogx(p(0))  -  p(0) * C * (L_u + L_v)
-//   f(c) = (xlogx(p(c)) - xlogx(p(0))) / c,   M_u = (1/Z) sum_e la[u][x_eu],   L_u = sum_a la[u][a]
-// (each non-empty cell's term is shared out among its c examples; the empty cells' terms are the
-// closed-form remainder), so a pair costs three passes over its N examples against a C x C table
-// of counters in LDS -- count, look up f, clear -- and no pass over the table itself.  Up to 65535
+//   MI[u,v] = sum over non-empty cells of g(c(cell))  -  M_u - M_v  +  C^2 * xlogx(p(0))  -  p(0) * C * (L_u + L_v)
+//   g(c) = xlogx(p(c)) - xlogx(p(0)),   M_u = (1/Z) sum_e la[u][x_eu],   L_u = sum_a la[u][a]
+// (the empty cells' terms are the closed-form remainder), so a pair costs two passes over its N examples against a
+// C x C table of counters in LDS -- count; then every example takes its cell's count away with it, and the one that
+// finds a count there adds the cell's term -- and no pass over the table itself.  Up to 65535
 // examples the counters are 16 bits wide and the whole table fits; beyond, they are 32 bits wide
 // and the table is walked in bands of rows.
 #include "common.hpp"
@@ -63,14 +63,17 @@ __global__ __launch_bounds__(256) void mi_single_kernel(const uint8_t* __restric
   if (t == 0) { stat[2 * v] = M; stat[2 * v + 1] = red[0]; }
 }
 
-// f(c) for c = 0 .. N (f(0) unused).
-__global__ void mi_table_kernel(int N, int C, float pc, double* __restrict__ f) {
+// g(c) = xlogx(p(c)) - xlogx(p(0)) for c = 0 .. N, the term of a cell that holds c examples, as a fixed-point integer of
+// kMiFrac fractional bits: |g| < 0.37, a pair adds at most N < 2^17 of them into 64 bits, and integer sums do not
+// depend on which thread adds which term (2^-44 per term is far below the float the sum ends as).
+constexpr int kMiFrac = 44;
+__global__ void mi_table_kernel(int N, int C, float pc, long long* __restrict__ g) {
   const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c > N) return;
   const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
   const double p0 = s / Z, x0 = p0 > 0.0 ? p0 * log(p0) : 0.0;
   const double p = ((double)c + s) / Z;
-  f[c] = c ? (p * log(p) - x0) / (double)c : 0.0;
+  g[c] = c ? llrint(ldexp(p * log(p) - x0, kMiFrac)) : 0ll;
 }
 
 constexpr int kMiThreads = 1024;
@@ -133,15 +136,16 @@ __device__ __forceinline__ void mi_each_example_from(const MiWords<R>& w, const 
 // thread 0's trip to memory.  No barrier behind thread 0: whoever writes `red` next has passed a barrier that thread 0
 // reaches only after this.
 struct MiStat { double m, l; };
-__device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, int u, int v, int V, int C, double p0, double x0,
-                                               MiStat su, MiStat sv, float* __restrict__ mi) {
+__device__ __forceinline__ void mi_finish_pair(long long acc, long long* red, int t, int u, int v, int V, int C, double p0,
+                                               double x0, MiStat su, MiStat sv, float* __restrict__ mi) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o);
   if ((t & 63) == 0) red[t >> 6] = acc;
   __syncthreads();
   if (t == 0) {
-    double tot = 0.0;
-    for (int w = 0; w < kMiThreads / 64; ++w) tot += red[w];
+    long long sum = 0;
+    for (int w = 0; w < kMiThreads / 64; ++w) sum += red[w];
+    const double tot = ldexp((double)sum, -kMiFrac);
     double val = tot - su.m - sv.m + (double)C * C * x0;
     if (p0 > 0.0) val -= p0 * C * (su.l + sv.l);
     mi[(size_t)u * V + v] = (float)val;
@@ -153,15 +157,15 @@ __device__ __forceinline__ void mi_finish_pair(double acc, double* red, int t, i
 // workgroups.  At most 65535 examples: a cell's count fits 16 bits, two cells per LDS word.
 template <int R>
 __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V, int C,
-                                                             float pc, const double* __restrict__ f, int f_lds,
+                                                             float pc, const long long* __restrict__ g, int g_lds,
                                                              const double* __restrict__ stat, float* __restrict__ mi) {
-  extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 doubles | the first f_lds entries of f
+  extern __shared__ unsigned cells[];   // C*C 16-bit counters, two per word | 16 sums | the first g_lds entries of g
   const int t = threadIdx.x;
   const int words = (C * C + 1) / 2;
-  double* red = reinterpret_cast<double*>(cells + ((words + 1) & ~1));
-  double* fl = red + kMiThreads / 64;   // what the LDS has left holds the table over counts from its start: a lookup per
-  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;   // example is then no trip to memory (counts past it are rare)
-  for (int i = t; i < f_lds; i += kMiThreads) fl[i] = f[i];
+  long long* red = reinterpret_cast<long long*>(cells + ((words + 1) & ~1));
+  long long* gl = red + kMiThreads / 64;   // what the LDS has left holds the table over counts from its start: a lookup
+  for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;   // is then no trip to memory (counts past it are rare)
+  for (int i = t; i < g_lds; i += kMiThreads) gl[i] = g[i];
   __syncthreads();
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
   const double Z = (double)N + (double)pc, s = (double)pc / ((double)C * C);
@@ -180,7 +184,7 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
     const uint8_t* xu = xb + (size_t)u * Np;
     const uint8_t* xv = xb + (size_t)v * Np;
     const MiStat su{stat[2 * u], stat[2 * u + 1]}, sv{stat[2 * v], stat[2 * v + 1]};
-    double acc = 0.0;
+    long long acc = 0;
     mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) {
       const int key = a * C + b;
       atomicAdd(&cells[key >> 1], 1u << (16 * (key & 1)));
@@ -192,14 +196,14 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
       mi_load_words(xb + (size_t)un * Np, xb + (size_t)(un + (int)(pn - rown)) * Np, N, t, nxt);
     }
     __syncthreads();
+    // look up and clear in one: the first of a cell's examples to come takes the cell's count with it and adds the
+    // cell's term, the others find it empty (the sums are integers: who adds what does not show in the result)
     mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) {
-      const int key = a * C + b;
-      const int cnt = (int)((cells[key >> 1] >> (16 * (key & 1))) & 0xffffu);
-      acc += cnt < f_lds ? fl[cnt] : f[cnt];
+      const int key = a * C + b, sh = 16 * (key & 1);
+      const int cnt = (int)((atomicAnd(&cells[key >> 1], ~(0xffffu << sh)) >> sh) & 0xffffu);
+      if (cnt) acc += cnt < g_lds ? gl[cnt] : g[cnt];
     });
-    __syncthreads();
-    mi_each_example_from(cur, xu, xv, N, t, [&](int a, int b) { cells[(a * C + b) >> 1] = 0u; });
-    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, su, sv, mi);
+    mi_finish_pair(acc, red, t, u, v, V, C, p0, x0, su, sv, mi);   // (its barrier also ends the clearing)
     cur = nxt;
   }
 }
@@ -208,12 +212,12 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_kernel(const uint8_t* __re
 // the categories of u are cut into bands of `band` rows and the three passes run once per band over
 // the examples whose u-category falls into it.
 __global__ __launch_bounds__(kMiThreads) void mi_pair_wide_kernel(const uint8_t* __restrict__ xb, int N, int64_t Np, int V,
-                                                                  int C, int band, float pc, const double* __restrict__ f,
+                                                                  int C, int band, float pc, const long long* __restrict__ g,
                                                                   const double* __restrict__ stat, float* __restrict__ mi) {
-  extern __shared__ unsigned cells[];   // band*C counters | 16 doubles
+  extern __shared__ unsigned cells[];   // band*C counters | 16 sums
   const int t = threadIdx.x;
   const int words = band * C;
-  double* red = reinterpret_cast<double*>(cells + ((words + 1) & ~1));
+  long long* red = reinterpret_cast<long long*>(cells + ((words + 1) & ~1));
   for (int i = t; i < words; i += kMiThreads) cells[i] = 0u;
   __syncthreads();
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
@@ -227,18 +231,17 @@ __global__ __launch_bounds__(kMiThreads) void mi_pair_wide_kernel(const uint8_t*
     const uint8_t* xu = xb + (size_t)u * Np;
     const uint8_t* xv = xb + (size_t)v * Np;
     const MiStat su{stat[2 * u], stat[2 * u + 1]}, sv{stat[2 * v], stat[2 * v + 1]};
-    double acc = 0.0;
+    long long acc = 0;
     for (int a0 = 0; a0 < C; a0 += band) {
       mi_each_example(xu, xv, N, t, [&](int a, int b) {
         if ((unsigned)(a - a0) < (unsigned)band) atomicAdd(&cells[(a - a0) * C + b], 1u);
       });
       __syncthreads();
-      mi_each_example(xu, xv, N, t, [&](int a, int b) {
-        if ((unsigned)(a - a0) < (unsigned)band) acc += f[cells[(a - a0) * C + b]];
-      });
-      __syncthreads();
-      mi_each_example(xu, xv, N, t, [&](int a, int b) {
-        if ((unsigned)(a - a0) < (unsigned)band) cells[(a - a0) * C + b] = 0u;
+      mi_each_example(xu, xv, N, t, [&](int a, int b) {   // look up and clear in one, as above
+        if ((unsigned)(a - a0) < (unsigned)band) {
+          const unsigned cnt = atomicExch(&cells[(a - a0) * C + b], 0u);
+          if (cnt) acc += g[cnt];
+        }
       });
       __syncthreads();
     }
@@ -273,14 +276,14 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
   const bool narrow = N <= 65535;
   int band = C;
   size_t lds;
-  int f_lds = 0;
+  int g_lds = 0;
   if (narrow) {
     const int words = (C * C + 1) / 2;
     lds = ((size_t)((words + 1) & ~1)) * 4 + red_bytes;
-    // the rest of the LDS -- of half of it where two workgroups fit a compute unit -- holds the start of the f table
+    // the rest of the LDS -- of half of it where two workgroups fit a compute unit -- holds the start of the g table
     const size_t whole = std::min<size_t>((size_t)max_lds, 160 * 1024), share = lds <= whole / 4 ? whole / 2 : whole;
-    f_lds = (int)std::min<size_t>((size_t)N + 1, (share - lds) / sizeof(double));
-    lds += (size_t)f_lds * sizeof(double);
+    g_lds = (int)std::min<size_t>((size_t)N + 1, (share - lds) / sizeof(double));
+    lds += (size_t)g_lds * sizeof(long long);
   } else {
     const size_t budget = std::min<size_t>((size_t)max_lds, 160 * 1024) - red_bytes - 8;
     band = (int)std::min<size_t>((size_t)C, budget / ((size_t)C * 4));
@@ -291,14 +294,14 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
   if (lds > (size_t)max_lds) fail(PCM_ERR_UNSUPPORTED, "pair table needs %zu bytes of LDS, device offers %d", lds, max_lds);
   pcm_stage(d_data, stride_ex, stride_var, nullptr, N, sh.Np, V, C, w.xb, stream);
   hipLaunchKernelGGL(mi_single_kernel, dim3(V), dim3(256), 0, stream, w.xb, N, sh.Np, C, pseudocount, w.stat);
-  hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div((int64_t)N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, w.f);
+  hipLaunchKernelGGL(mi_table_kernel, dim3(ceil_div((int64_t)N + 1, 256)), dim3(256), 0, stream, N, C, pseudocount, w.g);
   const int64_t n_pairs = (int64_t)V * (V + 1) / 2;
   const int per_cu = std::max<int>(1, (int)(std::min<size_t>((size_t)max_lds, 160 * 1024) / lds));
   const int grid = (int)std::min<int64_t>(n_pairs, (int64_t)cus * std::min(per_cu, 2));
   if (narrow) {
     auto pairs = [&](auto kernel) {
       PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.f, f_lds, w.stat,
+      hipLaunchKernelGGL(kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, pseudocount, w.g, g_lds, w.stat,
                          d_mi);
     };
     // rounds of 4 * kMiThreads examples whose words a thread keeps in registers
@@ -310,7 +313,7 @@ void mi_launch(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, con
     PCM_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&mi_pair_wide_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     hipLaunchKernelGGL(mi_pair_wide_kernel, dim3(grid), dim3(kMiThreads), lds, stream, w.xb, N, sh.Np, V, C, band,
-                       pseudocount, w.f, w.stat, d_mi);
+                       pseudocount, w.g, w.stat, d_mi);
   }
   check_launch_c("pairwise_mi");
 }
@@ -319,11 +322,12 @@ void pairwise_mi(const uint8_t* d_data, int64_t stride_ex, int64_t stride_var, i
                  int num_cats, float pseudocount, float* d_mi, hipStream_t stream) {
   const MiShape sh = mi_check(d_data, n_examples, num_vars, num_cats, pseudocount, d_mi);
   DevBuf<uint8_t> xb;
-  DevBuf<double> stat, f;
+  DevBuf<double> stat;
+  DevBuf<long long> g;
   xb.alloc((size_t)sh.V * sh.Np);
   stat.alloc((size_t)2 * sh.V);
-  f.alloc((size_t)sh.N + 1);
-  mi_launch(d_data, stride_ex, stride_var, sh, pseudocount, MiScratch{xb.p, stat.p, f.p}, d_mi, stream);
+  g.alloc((size_t)sh.N + 1);
+  mi_launch(d_data, stride_ex, stride_var, sh, pseudocount, MiScratch{xb.p, stat.p, g.p}, d_mi, stream);
   PCM_HIP(hipStreamSynchronize(stream));   // the scratch arrays die with this call
 }
 

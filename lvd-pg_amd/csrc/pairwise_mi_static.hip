@@ -54,7 +54,7 @@ void pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride
          "(use pcm_pairwise_mi)", (size_t)sh.V * (size_t)sh.Np, kMiStaticStage);
   unsigned char* base = mi_static_scratch();
   // every byte the kernels read from the array is written earlier in the same call: nothing to clear
-  const MiScratch w{base, reinterpret_cast<double*>(base + kMiStaticStatOff), reinterpret_cast<double*>(base + kMiStaticFOff)};
+  const MiScratch w{base, reinterpret_cast<double*>(base + kMiStaticStatOff), reinterpret_cast<long long*>(base + kMiStaticFOff)};
   mi_launch(d_data, stride_ex, stride_var, sh, pseudocount, w, d_mi, stream);
 }
 
