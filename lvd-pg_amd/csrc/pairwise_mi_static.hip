@@ -8,13 +8,13 @@
 namespace pcm {
 
 // Its working memory is one array in the code object, so every device the library runs on holds
-// kMiStaticBytes of it until the process ends.  Layout: staged categories | stat | f.
+// kMiStaticBytes of it until the process ends.  Layout: staged categories | stat | g.
 constexpr size_t kMiStaticStage = 16u << 20;                      // num_vars * ceil64(num_examples) bytes
 constexpr int kMiStaticVars = 4096;                                // stat: 2 doubles per variable
-constexpr int kMiStaticExamples = 65535;                           // f: one double per count
+constexpr int kMiStaticExamples = 65535;                           // g: one 64-bit integer per count
 constexpr size_t kMiStaticStatOff = kMiStaticStage;
-constexpr size_t kMiStaticFOff = kMiStaticStatOff + (size_t)kMiStaticVars * 2 * sizeof(double);
-constexpr size_t kMiStaticBytes = kMiStaticFOff + ((size_t)kMiStaticExamples + 1) * sizeof(double);
+constexpr size_t kMiStaticGOff = kMiStaticStatOff + (size_t)kMiStaticVars * 2 * sizeof(double);
+constexpr size_t kMiStaticBytes = kMiStaticGOff + ((size_t)kMiStaticExamples + 1) * sizeof(long long);
 
 static __device__ __align__(256) unsigned char scratch[kMiStaticBytes];
 
@@ -54,7 +54,7 @@ void pairwise_mi_static(const uint8_t* d_data, int64_t stride_ex, int64_t stride
          "(use pcm_pairwise_mi)", (size_t)sh.V * (size_t)sh.Np, kMiStaticStage);
   unsigned char* base = mi_static_scratch();
   // every byte the kernels read from the array is written earlier in the same call: nothing to clear
-  const MiScratch w{base, reinterpret_cast<double*>(base + kMiStaticStatOff), reinterpret_cast<long long*>(base + kMiStaticFOff)};
+  const MiScratch w{base, reinterpret_cast<double*>(base + kMiStaticStatOff), reinterpret_cast<long long*>(base + kMiStaticGOff)};
   mi_launch(d_data, stride_ex, stride_var, sh, pseudocount, w, d_mi, stream);
 }
 
